@@ -1,0 +1,1084 @@
+// CPU oracle: the reference's Numerics::Exact arithmetic restated in C++.
+//
+// TEST INFRASTRUCTURE ONLY: parity checker and timed CPU baseline. The device
+// library never links, loads or calls this file.
+//
+// Build: g++ -O3 -ffp-contract=off -fno-fast-math (no contraction, no
+// reassociation), so every sum below keeps the order it is written in.
+//
+// Pinning (reference vectors that hold each function bit for bit unless a
+// tolerance is given):
+//   linear fwd/bwd, gemm      ojas-cpu/tests/exact_golden.rs:206-242 (36 digests)
+//   muon f32                  exact_golden.rs:243-250 (8 digests)
+//   muon bf16                 ojas-oracle/fixtures/tiny/muon_step_bf16.safetensors (tolerance)
+//   sdpa fwd/lse/bwd          exact_golden.rs:251-265 (15 digests); window and
+//                             GQA: brute-force softmax in the tests
+//   rms fwd/bwd, rope         exact_golden.rs:266-270; rms_norm_f64.json
+//   ce grad                   exact_golden.rs:272 (digest); ce loss: libm ln, tolerance
+//                             against ojas-cuda/tests/fixtures/goldens/ce_rows_c*.npy
+//   adamw exact               exact_golden.rs:273-275; adamw_100 fixtures (tolerance)
+//   adamw fast (f32)          ojas-cpu/tests/adamw_lerp_oracle.rs rows
+//   exp_exact                 ojas-core/src/exp_exact_pins.txt (2162 pairs) + edges
+//   erf / gelu                ojas-core/src/erf_exact.rs:86-140 known-answer tables
+//   embedding fwd/bwd         ojas-cuda goldens embed_*.npy; gather is a bit copy
+//   bf16 rounding             integer rule autocast.rs:70-96, value table in the tests
+//   argmax / topk             brute force in the tests
+//   gpt step (graph A)        parity unpinned by the reference (no fixture holds this
+//                             graph); pinned by f64 central differences in the tests
+#include "ojas_exact.h"
+
+#include <algorithm>
+#include <atomic>
+#include <cmath>
+#include <cstring>
+#include <functional>
+#include <limits>
+#include <thread>
+#include <vector>
+
+namespace {
+
+int g_threads = 1;
+
+// Splits [0, n) into contiguous chunks, one per worker. Outputs only; no
+// reduction is ever split (ojas-cpu/src/lib.rs:9-16).
+void parallel_for(size_t n, size_t min_chunk, const std::function<void(size_t, size_t)>& body) {
+  size_t workers = static_cast<size_t>(std::max(1, g_threads));
+  if (min_chunk == 0) min_chunk = 1;
+  workers = std::min(workers, std::max<size_t>(1, n / min_chunk));
+  if (workers <= 1 || n == 0) {
+    body(0, n);
+    return;
+  }
+  std::vector<std::thread> pool;
+  size_t per = (n + workers - 1) / workers;
+  for (size_t w = 0; w < workers; ++w) {
+    size_t lo = w * per, hi = std::min(n, lo + per);
+    if (lo >= hi) break;
+    pool.emplace_back([=, &body] { body(lo, hi); });
+  }
+  for (auto& t : pool) t.join();
+}
+
+inline uint32_t bits_of(float x) {
+  uint32_t b;
+  std::memcpy(&b, &x, 4);
+  return b;
+}
+inline float float_of(uint32_t b) {
+  float x;
+  std::memcpy(&x, &b, 4);
+  return x;
+}
+inline double double_of(uint64_t b) {
+  double x;
+  std::memcpy(&x, &b, 8);
+  return x;
+}
+inline bool finite32(float x) { return (bits_of(x) & 0x7fffffffu) < 0x7f800000u; }
+
+bool all_finite(const float* x, size_t n) {
+  uint32_t top = 0;
+  for (size_t i = 0; i < n; ++i) top = std::max(top, bits_of(x[i]) & 0x7fffffffu);
+  return top < 0x7f800000u;
+}
+
+// ---- exp_exact (ojas-core/src/exp_exact.rs:8-73) ----
+const uint64_t kExp2Bits[256][2] = {
+#include "exp2_j256.inc"
+};
+const double kRoundF64 = 6755399441055744.0;  // 1.5 * 2^52
+const double kInvLn2_256 = double_of(0x40771547652b82feull);
+const double kLn2_256Hi = double_of(0x3f662e42fefa0000ull);
+const double kLn2_256Lo = double_of(0x3cfcf79abc9e3b3aull);
+
+inline double exp_in_range_f64(double xd) {
+  double kf = (xd * kInvLn2_256 + kRoundF64) - kRoundF64;
+  int64_t k = static_cast<int64_t>(kf);
+  double r = (xd - kf * kLn2_256Hi) - kf * kLn2_256Lo;
+  double t_hi = double_of(kExp2Bits[k & 255][0]);
+  double t_lo = double_of(kExp2Bits[k & 255][1]);
+  double p = r + r * r * (0.5 + r * (1.0 / 6.0 + r * (1.0 / 24.0)));
+  double y = t_hi + (t_hi * p + t_lo);
+  return y * double_of(static_cast<uint64_t>((k >> 8) + 1023) << 52);
+}
+
+inline double exp_exact_wide(float x) {
+  if (x != x) return static_cast<double>(x);
+  if (x > 89.0f) return std::numeric_limits<double>::infinity();
+  if (x < -104.0f) return 0.0;
+  return exp_in_range_f64(static_cast<double>(x));
+}
+inline float exp_exact(float x) { return static_cast<float>(exp_exact_wide(x)); }
+
+// ln of a positive normal f64 (exp_exact.rs:141-160).
+double ln_wide(double x) {
+  uint64_t b;
+  std::memcpy(&b, &x, 8);
+  int64_t e = static_cast<int64_t>((b >> 52) & 0x7ff) - 1023;
+  double m = double_of((b & 0x000fffffffffffffull) | (1023ull << 52));
+  if (m > 1.4142135623730951) {
+    m *= 0.5;
+    e += 1;
+  }
+  double z = (m - 1.0) / (m + 1.0);
+  double z2 = z * z;
+  double series = 0.0;
+  for (int k = 11; k >= 0; --k) series = series * z2 + 1.0 / static_cast<double>(2 * k + 1);
+  double ef = static_cast<double>(e);
+  const double hi = double_of(0x3fe62e42fee00000ull), lo = double_of(0x3dea39ef35793c76ull);
+  return ef * hi + (ef * lo + 2.0 * z * series);
+}
+
+float log_sum_exp_exact(float max, float sum) {
+  if (!(finite32(max) && finite32(sum) && sum > 0.0f)) return std::numeric_limits<float>::quiet_NaN();
+  return static_cast<float>(static_cast<double>(max) + ln_wide(static_cast<double>(sum)));
+}
+
+float log1p_exact(float xf) {
+  if (!(xf >= 0.0f && xf <= 1.0f)) return std::numeric_limits<float>::quiet_NaN();
+  double x = xf;
+  double z = x / (2.0 + x);
+  double z2 = z * z;
+  double term = z, sum = 0.0;
+  for (int k = 0; k < 24; ++k) {
+    sum += term / static_cast<double>(2 * k + 1);
+    term *= z2;
+  }
+  return static_cast<float>(2.0 * sum);
+}
+
+// ---- erf / GELU (ojas-core/src/erf_exact.rs:29-110, gelu_tanh.rs:27-68) ----
+double erf_f64(double z) {
+  if (z != z) return z;
+  double a = std::fabs(z);
+  if (a >= 6.0) return std::copysign(1.0, z);
+  double two_a2 = 2.0 * a * a;
+  double term = a, sum = a, denom = 3.0;
+  for (int i = 0; i < 400; ++i) {
+    if (term <= sum * 1e-17) break;
+    term = term * two_a2 / denom;
+    sum += term;
+    denom += 2.0;
+  }
+  const double frac_2_sqrt_pi = 1.1283791670955126;
+  double value = std::min(frac_2_sqrt_pi * exp_in_range_f64(-(a * a)) * sum, 1.0);
+  return std::copysign(value, z);
+}
+double exp_neg(double h) {
+  if (h <= 104.0) return exp_in_range_f64(-h);
+  if (h <= 208.0) return exp_in_range_f64(-104.0) * exp_in_range_f64(104.0 - h);
+  return 0.0;
+}
+const double kFrac1Sqrt2 = 0.7071067811865476;
+float gelu_erf(float x) {
+  double xd = x;
+  return static_cast<float>(0.5 * xd * (1.0 + erf_f64(xd * kFrac1Sqrt2)));
+}
+float gelu_erf_backward(float x, float dy) {
+  if (x != x) return std::numeric_limits<float>::quiet_NaN();
+  double xd = x;
+  double cdf = 0.5 * (1.0 + erf_f64(xd * kFrac1Sqrt2));
+  double pdf = 0.3989422804014327 * exp_neg(0.5 * xd * xd);
+  return static_cast<float>(static_cast<double>(dy) * (cdf + xd * pdf));
+}
+const double kSqrt2OverPi = 0.7978845608028654;
+const double kCubic = 0.044715;
+inline void sigmoid_pair(double u, double* s, double* slope) {
+  double e = exp_neg(std::fabs(u));
+  double denom = 1.0 + e;
+  *s = u >= 0.0 ? 1.0 / denom : e / denom;
+  *slope = e / (denom * denom);
+}
+inline double sigmoid_arg(double x) { return 2.0 * kSqrt2OverPi * (x + kCubic * x * x * x); }
+float gelu_tanh(float x) {
+  if (x != x) return std::numeric_limits<float>::quiet_NaN();
+  double xd = x, s, slope;
+  sigmoid_pair(sigmoid_arg(xd), &s, &slope);
+  return static_cast<float>(xd * s);
+}
+float gelu_tanh_backward(float x, float dy) {
+  if (x != x) return std::numeric_limits<float>::quiet_NaN();
+  double xd = x, s, slope;
+  sigmoid_pair(sigmoid_arg(xd), &s, &slope);
+  double du = 2.0 * kSqrt2OverPi * (1.0 + 3.0 * kCubic * xd * xd);
+  return static_cast<float>(static_cast<double>(dy) * (s + xd * slope * du));
+}
+
+// ---- bf16 (ojas-core/src/autocast.rs:66-101) ----
+inline uint16_t f32_to_bf16(float v) {
+  uint32_t b = bits_of(v);
+  if (v != v) return static_cast<uint16_t>((b >> 16) | 0x0040u);
+  uint32_t round = 0x7fffu + ((b >> 16) & 1u);
+  return static_cast<uint16_t>((b + round) >> 16);
+}
+inline float round_bf16(float v) { return float_of(static_cast<uint32_t>(f32_to_bf16(v)) << 16); }
+
+// ---- GEMM (ojas-cpu/src/gemm.rs:1-41,1063-1081): every output is
+// ((0 + a0*b0) + a1*b1) + ... for k ascending, two roundings per step. ----
+void gemm(const float* a, size_t a_rs, size_t a_cs, const float* b, size_t b_rs, size_t b_cs,
+          float* c, size_t m, size_t k, size_t n, bool accumulate) {
+  // B is packed k-major so the inner loop runs over independent outputs.
+  std::vector<float> packed;
+  const float* bp = b;
+  if (!(b_cs == 1 && b_rs == n)) {
+    packed.resize(k * n);
+    parallel_for(k, 16, [&](size_t lo, size_t hi) {
+      for (size_t p = lo; p < hi; ++p)
+        for (size_t j = 0; j < n; ++j) packed[p * n + j] = b[p * b_rs + j * b_cs];
+    });
+    bp = packed.data();
+  }
+  parallel_for(m, 1, [&](size_t lo, size_t hi) {
+    for (size_t i = lo; i < hi; ++i) {
+      float* row = c + i * n;
+      if (!accumulate)
+        for (size_t j = 0; j < n; ++j) row[j] = 0.0f;
+      for (size_t p = 0; p < k; ++p) {
+        float s = a[i * a_rs + p * a_cs];
+        const float* br = bp + p * n;
+        for (size_t j = 0; j < n; ++j) row[j] = row[j] + s * br[j];
+      }
+    }
+  });
+}
+
+}  // namespace
+
+extern "C" {
+
+void orc_set_threads(int threads) { g_threads = std::max(1, threads); }
+int orc_get_threads(void) { return g_threads; }
+
+uint64_t orc_splitmix_next(uint64_t* state) {
+  *state += 0x9e3779b97f4a7c15ull;
+  uint64_t z = *state;
+  z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+  z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+  return z ^ (z >> 31);
+}
+void orc_splitmix_vec(uint64_t* state, float* out, size_t n, float scale) {
+  for (size_t i = 0; i < n; ++i) {
+    float mantissa = static_cast<float>(orc_splitmix_next(state) >> 40) / static_cast<float>(1u << 24);
+    out[i] = scale * (2.0f * mantissa - 1.0f);
+  }
+}
+uint64_t orc_splitmix_below(uint64_t* state, uint64_t n) { return orc_splitmix_next(state) % n; }
+uint64_t orc_fnv_f32(const float* values, size_t n) {
+  uint64_t h = 0xcbf29ce484222325ull;
+  for (size_t i = 0; i < n; ++i) {
+    uint32_t b = bits_of(values[i]);
+    for (int s = 0; s < 4; ++s) {
+      h ^= (b >> (8 * s)) & 0xffu;
+      h *= 0x00000100000001b3ull;
+    }
+  }
+  return h;
+}
+
+float orc_exp_exact(float x) { return exp_exact(x); }
+float orc_log_sum_exp_exact(float max, float sum) { return log_sum_exp_exact(max, sum); }
+float orc_log1p_exact(float x) { return log1p_exact(x); }
+double orc_erf_f64(double z) { return erf_f64(z); }
+float orc_gelu_erf(float x) { return gelu_erf(x); }
+float orc_gelu_erf_backward(float x, float dy) { return gelu_erf_backward(x, dy); }
+float orc_gelu_tanh(float x) { return gelu_tanh(x); }
+float orc_gelu_tanh_backward(float x, float dy) { return gelu_tanh_backward(x, dy); }
+// ojas-cpu/src/pointwise.rs:57-65
+float orc_sigmoid_exact(float x) {
+  if (x >= 0.0f) {
+    float z = exp_exact(-x);
+    return 1.0f / (1.0f + z);
+  }
+  float z = exp_exact(x);
+  return z / (1.0f + z);
+}
+uint16_t orc_f32_to_bf16(float x) { return f32_to_bf16(x); }
+float orc_round_bf16(float x) { return round_bf16(x); }
+void orc_exp_exact_vec(const float* x, float* y, size_t n) {
+  for (size_t i = 0; i < n; ++i) y[i] = exp_exact(x[i]);
+}
+void orc_round_bf16_vec(const float* x, float* y, size_t n) {
+  for (size_t i = 0; i < n; ++i) y[i] = round_bf16(x[i]);
+}
+void orc_to_bf16_vec(const float* x, uint16_t* y, size_t n) {
+  for (size_t i = 0; i < n; ++i) y[i] = f32_to_bf16(x[i]);
+}
+void orc_bf16_to_f32_vec(const uint16_t* x, float* y, size_t n) {
+  for (size_t i = 0; i < n; ++i) y[i] = float_of(static_cast<uint32_t>(x[i]) << 16);
+}
+
+// ojas-core/src/backend.rs:244-257
+double orc_pow_u64(double base, uint64_t exp) {
+  double result = 1.0, b = base;
+  while (exp > 0) {
+    if (exp & 1) result *= b;
+    exp >>= 1;
+    if (exp > 0) b *= b;
+  }
+  return result;
+}
+
+// ojas-core/src/backend.rs:277-303
+int orc_clip_scale(float max_norm, float total_norm, float* coef) {
+  if (!finite32(total_norm) || max_norm != max_norm ||
+      max_norm == -std::numeric_limits<float>::infinity())
+    return ORC_NON_FINITE;
+  if (max_norm < 0.0f) return ORC_OUT_OF_RANGE;
+  if (total_norm < 0.0f) return ORC_OUT_OF_RANGE;
+  float c = max_norm / (total_norm + 1e-6f);
+  if (c != c) return ORC_NON_FINITE;
+  *coef = std::min(c, 1.0f);
+  return ORC_OK;
+}
+
+// ojas-core/src/backend.rs:312-432
+int orc_adamw_scalars(double lr, double beta1, double beta2, double eps, double weight_decay,
+                      uint64_t step_before, double words[7], int32_t flags[3]) {
+  const double scalars[5] = {lr, beta1, beta2, eps, weight_decay};
+  for (double s : scalars)
+    if (!std::isfinite(s)) return ORC_NON_FINITE;
+  if (!(beta1 >= 0.0 && beta1 < 1.0 && beta2 >= 0.0 && beta2 < 1.0)) return ORC_OUT_OF_RANGE;
+  if (eps <= 0.0) return ORC_OUT_OF_RANGE;
+  if (lr < 0.0 || weight_decay < 0.0) return ORC_OUT_OF_RANGE;
+  if (step_before == UINT64_MAX) return ORC_OUT_OF_RANGE;
+  uint64_t next = step_before + 1;
+  double bc1 = 1.0 - orc_pow_u64(beta1, next);
+  double bc2 = 1.0 - orc_pow_u64(beta2, next);
+  if (!(std::isfinite(bc1) && std::isfinite(bc2) && bc1 > 0.0 && bc2 > 0.0)) return ORC_OUT_OF_RANGE;
+  double one_minus_b1 = 1.0 - beta1;
+  words[0] = 1.0 - lr * weight_decay;
+  words[1] = one_minus_b1;
+  words[2] = beta2;
+  words[3] = 1.0 - beta2;
+  words[4] = lr / bc1;
+  words[5] = std::sqrt(bc2);
+  words[6] = eps;
+  flags[0] = weight_decay != 0.0;
+  flags[1] = one_minus_b1 < 0.5;
+  flags[2] = static_cast<float>(one_minus_b1) < 0.5f;
+  return ORC_OK;
+}
+
+int orc_gemm(const float* a, size_t a_rs, size_t a_cs, const float* b, size_t b_rs, size_t b_cs,
+             float* c, size_t m, size_t k, size_t n, int accumulate) {
+  gemm(a, a_rs, a_cs, b, b_rs, b_cs, c, m, k, n, accumulate != 0);
+  return ORC_OK;
+}
+
+// ojas-cpu/src/linalg.rs:69-89: y = x . W^T
+int orc_linear_forward(const float* x, const float* w, float* y, size_t rows, size_t kin,
+                       size_t nout) {
+  if (!all_finite(x, rows * kin) || !all_finite(w, nout * kin)) return ORC_NON_FINITE;
+  gemm(x, kin, 1, w, 1, kin, y, rows, kin, nout, false);
+  return all_finite(y, rows * nout) ? ORC_OK : ORC_NON_FINITE;
+}
+
+// ojas-cpu/src/linalg.rs:105-184: gx = g . W (sum over out), gw = g^T . x (sum over rows)
+int orc_linear_backward(const float* x, const float* w, const float* gy, float* gx, float* gw,
+                        size_t rows, size_t kin, size_t nout) {
+  if (gx) gemm(gy, nout, 1, w, kin, 1, gx, rows, nout, kin, false);
+  if (gw) gemm(gy, 1, nout, x, kin, 1, gw, nout, rows, kin, false);
+  if (gx && !all_finite(gx, rows * kin)) return ORC_NON_FINITE;
+  if (gw && !all_finite(gw, nout * kin)) return ORC_NON_FINITE;
+  return ORC_OK;
+}
+
+// ---- attention ----
+namespace {
+struct SdpaDims {
+  size_t batch, heads, kv_heads, time, dim, window;
+  float scale;
+  size_t rep() const { return (kv_heads == 0 || kv_heads == heads) ? 1 : heads / kv_heads; }
+  size_t kv_plane(size_t q_plane) const {
+    return (q_plane / heads) * kv_heads + (q_plane % heads) / rep();
+  }
+  size_t first_key(size_t t) const {
+    if (window == 0) return 0;
+    return (t + 1 > window) ? t + 1 - window : 0;
+  }
+};
+inline float dot_up(const float* a, const float* b, size_t n) {
+  float acc = 0.0f;
+  for (size_t i = 0; i < n; ++i) acc += a[i] * b[i];
+  return acc;
+}
+inline void saxpy_up(float* dst, const float* src, float s, size_t n) {
+  for (size_t i = 0; i < n; ++i) dst[i] += s * src[i];
+}
+}  // namespace
+
+// ojas-cpu/src/attn.rs:176-227 (rows), :262-309 (scores), :350-389 (softmax), :392-427 (mix)
+int orc_causal_sdpa_forward(const float* q, const float* k, const float* v, float* out, float* lse,
+                            size_t batch, size_t heads, size_t kv_heads, size_t time, size_t dim,
+                            size_t window) {
+  if (dim == 0 || heads == 0 || kv_heads == 0 || kv_heads > heads || heads % kv_heads != 0)
+    return ORC_SHAPE;
+  if (window >= time) window = 0;
+  SdpaDims d{batch, heads, kv_heads, time, dim, window,
+             1.0f / std::sqrt(static_cast<float>(static_cast<uint32_t>(dim)))};
+  size_t planes = batch * heads, stride = time * dim;
+  std::atomic<int> status{ORC_OK};
+  parallel_for(planes, 1, [&](size_t lo, size_t hi) {
+    std::vector<float> scores(time), probs(time);
+    for (size_t plane = lo; plane < hi; ++plane) {
+      const float* qh = q + plane * stride;
+      const float* kh = k + d.kv_plane(plane) * stride;
+      const float* vh = v + d.kv_plane(plane) * stride;
+      for (size_t t = 0; t < time; ++t) {
+        size_t j0 = d.first_key(t), j1 = t + 1;
+        for (size_t j = j0; j < j1; ++j) {
+          float s = dot_up(qh + t * dim, kh + j * dim, dim) * d.scale;
+          if (!finite32(s)) {
+            status = ORC_NON_FINITE;
+            return;
+          }
+          scores[j] = s;
+        }
+        float max = -std::numeric_limits<float>::infinity();
+        for (size_t j = j0; j < j1; ++j) max = (scores[j] > max) ? scores[j] : max;
+        float sum = 0.0f;
+        for (size_t j = j0; j < j1; ++j) {
+          float e = exp_exact(scores[j] - max);
+          probs[j] = e;
+          sum += e;
+        }
+        for (size_t j = j0; j < j1; ++j) probs[j] /= sum;
+        if (!(finite32(sum) && sum > 0.0f)) {
+          status = ORC_NON_FINITE;
+          return;
+        }
+        lse[plane * time + t] = log_sum_exp_exact(max, sum);
+        float* o = out + plane * stride + t * dim;
+        for (size_t c = 0; c < dim; ++c) o[c] = 0.0f;
+        for (size_t j = j0; j < j1; ++j) saxpy_up(o, vh + j * dim, probs[j], dim);
+      }
+    }
+  });
+  return status.load();
+}
+
+// ojas-cpu/src/attn.rs:437-597: KV groups are independent; the query heads of
+// a group accumulate into its grad_k / grad_v in ascending head order.
+int orc_causal_sdpa_backward(const float* q, const float* k, const float* v, const float* out,
+                             const float* lse, const float* gy, float* gq, float* gk, float* gv,
+                             size_t batch, size_t heads, size_t kv_heads, size_t time, size_t dim,
+                             size_t window) {
+  if (dim == 0 || heads == 0 || kv_heads == 0 || kv_heads > heads || heads % kv_heads != 0)
+    return ORC_SHAPE;
+  if (window >= time) window = 0;
+  SdpaDims d{batch, heads, kv_heads, time, dim, window,
+             1.0f / std::sqrt(static_cast<float>(static_cast<uint32_t>(dim)))};
+  size_t groups = batch * kv_heads, stride = time * dim, rep = d.rep();
+  std::memset(gq, 0, sizeof(float) * batch * heads * stride);
+  std::memset(gk, 0, sizeof(float) * groups * stride);
+  std::memset(gv, 0, sizeof(float) * groups * stride);
+  std::atomic<int> status{ORC_OK};
+  parallel_for(groups, 1, [&](size_t lo, size_t hi) {
+    std::vector<float> probs(time), dprobs(time);
+    for (size_t group = lo; group < hi; ++group) {
+      const float* kh = k + group * stride;
+      const float* vh = v + group * stride;
+      float* gkh = gk + group * stride;
+      float* gvh = gv + group * stride;
+      for (size_t r = 0; r < rep; ++r) {
+        size_t head = group * rep + r;
+        const float* qh = q + head * stride;
+        const float* oh = out + head * stride;
+        const float* gyh = gy + head * stride;
+        float* gqh = gq + head * stride;
+        for (size_t t = 0; t < time; ++t) {
+          const float* q_row = qh + t * dim;
+          const float* gy_row = gyh + t * dim;
+          size_t j0 = d.first_key(t), j1 = t + 1;
+          float row_lse = lse[head * time + t];
+          float expected = dot_up(gy_row, oh + t * dim, dim);
+          if (!(finite32(row_lse) && finite32(expected))) {
+            status = ORC_NON_FINITE;
+            return;
+          }
+          for (size_t j = j0; j < j1; ++j) {
+            float score = dot_up(q_row, kh + j * dim, dim) * d.scale;
+            if (!finite32(score)) {
+              status = ORC_NON_FINITE;
+              return;
+            }
+            float p = exp_exact(score - row_lse);
+            if (!finite32(p)) {
+              status = ORC_NON_FINITE;
+              return;
+            }
+            probs[j] = p;
+            dprobs[j] = dot_up(gy_row, vh + j * dim, dim);
+          }
+          for (size_t j = j0; j < j1; ++j) {
+            float p = probs[j];
+            float coef = d.scale * (p * (dprobs[j] - expected));
+            saxpy_up(gqh + t * dim, kh + j * dim, coef, dim);
+            saxpy_up(gkh + j * dim, q_row, coef, dim);
+            saxpy_up(gvh + j * dim, gy_row, p, dim);
+          }
+        }
+      }
+    }
+  });
+  return status.load();
+}
+
+// ---- RMSNorm (ojas-cpu/src/norm.rs:24-56,62-127,129-204) ----
+namespace {
+inline bool rstd_of_sum(float sum_sq, size_t dim, float eps, float* rstd) {
+  float mean_sq = sum_sq / static_cast<float>(dim);
+  float denom = mean_sq + eps;
+  if (!(finite32(denom) && denom > 0.0f)) return false;
+  float r = 1.0f / std::sqrt(denom);
+  if (!finite32(r)) return false;
+  *rstd = r;
+  return true;
+}
+}  // namespace
+
+int orc_rms_norm_forward(const float* x, const float* w, float* y, size_t rows, size_t dim,
+                         float eps) {
+  std::atomic<int> status{ORC_OK};
+  parallel_for(rows, 8, [&](size_t lo, size_t hi) {
+    for (size_t r = lo; r < hi; ++r) {
+      const float* src = x + r * dim;
+      float sum_sq = 0.0f;
+      for (size_t c = 0; c < dim; ++c) sum_sq += src[c] * src[c];
+      float rstd;
+      if (!rstd_of_sum(sum_sq, dim, eps, &rstd)) {
+        status = ORC_NON_FINITE;
+        return;
+      }
+      float* dst = y + r * dim;
+      for (size_t c = 0; c < dim; ++c) dst[c] = src[c] * rstd * w[c];
+    }
+  });
+  return status.load();
+}
+
+int orc_rms_norm_backward(const float* x, const float* w, const float* gy, float* gx, float* gw,
+                          size_t rows, size_t dim, float eps) {
+  std::vector<float> rstds(rows);
+  std::atomic<int> status{ORC_OK};
+  float inv_dim = 1.0f / static_cast<float>(dim);
+  parallel_for(rows, 8, [&](size_t lo, size_t hi) {
+    for (size_t r = lo; r < hi; ++r) {
+      const float* src = x + r * dim;
+      const float* g = gy + r * dim;
+      float sum_sq = 0.0f;
+      for (size_t c = 0; c < dim; ++c) sum_sq += src[c] * src[c];
+      float rstd;
+      if (!rstd_of_sum(sum_sq, dim, eps, &rstd)) {
+        status = ORC_NON_FINITE;
+        return;
+      }
+      rstds[r] = rstd;
+      float dot = 0.0f;
+      for (size_t c = 0; c < dim; ++c) dot += (g[c] * w[c]) * (src[c] * rstd);
+      float mean = dot * inv_dim;
+      float* dst = gx + r * dim;
+      for (size_t c = 0; c < dim; ++c) {
+        float dxhat = g[c] * w[c];
+        float xhat = src[c] * rstd;
+        dst[c] = (dxhat - xhat * mean) * rstd;
+      }
+    }
+  });
+  if (status.load() != ORC_OK) return status.load();
+  parallel_for(dim, 16, [&](size_t lo, size_t hi) {
+    for (size_t c = lo; c < hi; ++c) gw[c] = 0.0f;
+    for (size_t r = 0; r < rows; ++r) {
+      float rs = rstds[r];
+      const float* src = x + r * dim;
+      const float* g = gy + r * dim;
+      for (size_t c = lo; c < hi; ++c) gw[c] += g[c] * (src[c] * rs);
+    }
+  });
+  return ORC_OK;
+}
+
+// ---- RoPE (ojas-cpu/src/norm.rs:271-347) ----
+namespace {
+int rope_rows(const float* x, const float* cos, const float* sin, float* y, size_t rows, size_t dim,
+              size_t time, size_t heads, bool forward) {
+  if (dim % 2 != 0) return ORC_SHAPE;
+  size_t half = dim / 2;
+  for (size_t row = 0; row < rows; ++row) {
+    size_t base = (heads == 0) ? row * dim : ((row / heads) % time) * dim;
+    const float* cr = cos + base;
+    const float* sr = sin + base;
+    const float* src = x + row * dim;
+    float* dst = y + row * dim;
+    for (size_t col = 0; col < half; ++col) {
+      float a = src[col], b = src[col + half];
+      float c1 = cr[col], s1 = sr[col], c2 = cr[col + half], s2 = sr[col + half];
+      if (forward) {
+        dst[col] = a * c1 + (-b) * s1;
+        dst[col + half] = b * c2 + a * s2;
+      } else {
+        dst[col] = a * c1 + b * s2;
+        dst[col + half] = -a * s1 + b * c2;
+      }
+    }
+  }
+  return ORC_OK;
+}
+}  // namespace
+int orc_rope_forward(const float* x, const float* cos, const float* sin, float* y, size_t rows,
+                     size_t dim, size_t time, size_t heads) {
+  return rope_rows(x, cos, sin, y, rows, dim, time, heads, true);
+}
+int orc_rope_backward(const float* gy, const float* cos, const float* sin, float* gx, size_t rows,
+                      size_t dim, size_t time, size_t heads) {
+  return rope_rows(gy, cos, sin, gx, rows, dim, time, heads, false);
+}
+
+// ---- cross-entropy (ojas-cpu/src/pointwise.rs:2172-2438) ----
+namespace {
+int ce_valid(const uint32_t* targets, size_t rows, size_t vocab, int has_ignore, uint32_t ignore,
+             uint32_t* valid_out) {
+  uint32_t valid = 0;
+  for (size_t n = 0; n < rows; ++n) {
+    if (has_ignore && targets[n] == ignore) continue;
+    if (static_cast<size_t>(targets[n]) >= vocab) return ORC_OUT_OF_RANGE;
+    valid += 1;
+  }
+  if (valid == 0) return ORC_NON_FINITE;
+  *valid_out = valid;
+  return ORC_OK;
+}
+
+// One row: returns ORC_OK and sets *term (and has_term) or an error.
+int ce_row(const float* row, size_t vocab, uint32_t target, bool ignored, uint32_t valid,
+           float* grad, bool* has_term, float* term) {
+  *has_term = false;
+  if (ignored) return all_finite(row, vocab) ? ORC_OK : ORC_NON_FINITE;
+  float max = -std::numeric_limits<float>::infinity();
+  uint32_t top = 0;
+  for (size_t c = 0; c < vocab; ++c) {
+    if (row[c] > max) max = row[c];
+    top = std::max(top, bits_of(row[c]) & 0x7fffffffu);
+  }
+  if (top >= 0x7f800000u) return ORC_NON_FINITE;
+  size_t cls = target;
+  float picked = row[cls];
+  float sum = 0.0f;
+  for (size_t c = 0; c < vocab; ++c) {
+    float e = exp_exact(row[c] - max);
+    if (!finite32(e)) return ORC_NON_FINITE;
+    if (grad) grad[c] = e;
+    sum += e;
+  }
+  if (!(finite32(sum) && sum > 0.0f)) return ORC_NON_FINITE;
+  // Collapse rule (pointwise.rs:2305-2325): the target holds the whole mass.
+  bool use_other = false;
+  float other = 0.0f;
+  if (picked == max && sum == 1.0f) {
+    for (size_t c = 0; c < vocab; ++c)
+      if (c != cls) other += exp_exact(row[c] - max);
+    use_other = other > 0.0f;
+  }
+  if (grad) {
+    float denom = static_cast<float>(valid);
+    if (use_other) {
+      float dd = 1.0f + other;
+      for (size_t c = 0; c < vocab; ++c) grad[c] = (grad[c] / dd) / denom;
+      grad[cls] = -(other / dd) / denom;
+    } else {
+      for (size_t c = 0; c < vocab; ++c) {
+        float p = grad[c] / sum;
+        grad[c] = p / denom;
+      }
+      grad[cls] -= 1.0f / denom;
+    }
+  }
+  *has_term = true;
+  *term = use_other ? log1p_exact(other) : (max + std::log(sum) - picked);
+  return ORC_OK;
+}
+
+int ce_mean(const float* logits, const uint32_t* targets, size_t rows, size_t vocab, int has_ignore,
+            uint32_t ignore, float* loss, float* grad) {
+  uint32_t valid = 0;
+  int rc = ce_valid(targets, rows, vocab, has_ignore, ignore, &valid);
+  if (rc != ORC_OK) {
+    // A non-finite logit outranks a target refusal (pointwise.rs:2453-2455).
+    if (!all_finite(logits, rows * vocab)) return ORC_NON_FINITE;
+    return rc;
+  }
+  std::vector<float> terms(rows, 0.0f);
+  std::vector<uint8_t> has(rows, 0);
+  std::atomic<int> status{ORC_OK};
+  parallel_for(rows, 4, [&](size_t lo, size_t hi) {
+    for (size_t n = lo; n < hi; ++n) {
+      bool ignored = has_ignore && targets[n] == ignore;
+      float* g = grad ? grad + n * vocab : nullptr;
+      if (g && ignored)
+        for (size_t c = 0; c < vocab; ++c) g[c] = 0.0f;
+      bool ht;
+      float term;
+      int r = ce_row(logits + n * vocab, vocab, targets[n], ignored, valid, ignored ? nullptr : g,
+                     &ht, &term);
+      if (r != ORC_OK) {
+        status = r;
+        return;
+      }
+      has[n] = ht;
+      terms[n] = term;
+    }
+  });
+  if (status.load() != ORC_OK) return status.load();
+  float total = 0.0f;
+  for (size_t n = 0; n < rows; ++n)
+    if (has[n]) total += terms[n];
+  float l = total / static_cast<float>(valid);
+  if (!finite32(l)) return ORC_NON_FINITE;
+  if (loss) *loss = l;
+  return ORC_OK;
+}
+}  // namespace
+
+int orc_cross_entropy_mean_forward(const float* logits, const uint32_t* targets, size_t rows,
+                                   size_t vocab, int has_ignore, uint32_t ignore, float* loss) {
+  return ce_mean(logits, targets, rows, vocab, has_ignore, ignore, loss, nullptr);
+}
+int orc_cross_entropy_mean_backward(const float* logits, const uint32_t* targets, size_t rows,
+                                    size_t vocab, int has_ignore, uint32_t ignore, float* grad) {
+  return ce_mean(logits, targets, rows, vocab, has_ignore, ignore, nullptr, grad);
+}
+
+int orc_linear_cross_entropy_mean(const float* x, const float* w, const uint32_t* targets,
+                                  size_t rows, size_t dim, size_t vocab, int has_ignore,
+                                  uint32_t ignore, float* loss, float* gx, float* gw) {
+  std::vector<float> logits(rows * vocab);
+  int rc = orc_linear_forward(x, w, logits.data(), rows, dim, vocab);
+  if (rc != ORC_OK) return rc;
+  rc = ce_mean(logits.data(), targets, rows, vocab, has_ignore, ignore, loss, nullptr);
+  if (rc != ORC_OK) return rc;
+  if (!gx && !gw) return ORC_OK;
+  std::vector<float> g(rows * vocab);
+  rc = ce_mean(logits.data(), targets, rows, vocab, has_ignore, ignore, nullptr, g.data());
+  if (rc != ORC_OK) return rc;
+  logits.clear();
+  logits.shrink_to_fit();
+  return orc_linear_backward(x, w, g.data(), gx, gw, rows, dim, vocab);
+}
+
+// ---- embedding ----
+int orc_embedding_forward(const float* table, const uint32_t* ids, float* out, size_t tokens,
+                          size_t vocab, size_t dim) {
+  for (size_t n = 0; n < tokens; ++n)
+    if (static_cast<size_t>(ids[n]) >= vocab) return ORC_OUT_OF_RANGE;
+  for (size_t n = 0; n < tokens; ++n)
+    std::memcpy(out + n * dim, table + static_cast<size_t>(ids[n]) * dim, dim * sizeof(float));
+  return ORC_OK;
+}
+int orc_embedding_backward(const uint32_t* ids, const float* grad, float* table_grad, size_t tokens,
+                           size_t vocab, size_t dim) {
+  for (size_t n = 0; n < tokens; ++n)
+    if (static_cast<size_t>(ids[n]) >= vocab) return ORC_OUT_OF_RANGE;
+  std::memset(table_grad, 0, sizeof(float) * vocab * dim);
+  bool finite = true;
+  for (size_t n = 0; n < tokens; ++n) {
+    float* dst = table_grad + static_cast<size_t>(ids[n]) * dim;
+    const float* src = grad + n * dim;
+    for (size_t c = 0; c < dim; ++c) {
+      float s = dst[c] + src[c];
+      finite &= finite32(s);
+      dst[c] = s;
+    }
+  }
+  return finite ? ORC_OK : ORC_NON_FINITE;
+}
+
+// ---- AdamW (ojas-cpu/src/optim.rs:186-257 exact, :302-395 fast; two-pass
+// all-or-nothing :513-621) ----
+int orc_adamw_step(float* p, const float* g, float* m, float* v, size_t n, uint64_t step_before,
+                   double lr, double beta1, double beta2, double eps, double weight_decay,
+                   int exact) {
+  double w[7];
+  int32_t flags[3];
+  int rc = orc_adamw_scalars(lr, beta1, beta2, eps, weight_decay, step_before, w, flags);
+  if (rc != ORC_OK) {
+    if (rc != ORC_NON_FINITE &&
+        !(all_finite(p, n) && all_finite(g, n) && all_finite(m, n) && all_finite(v, n)))
+      return ORC_NON_FINITE;
+    return rc;
+  }
+  const bool decays = flags[0] != 0;
+  std::vector<float> np(n), nm(n), nv(n);
+  std::atomic<int> status{ORC_OK};
+  if (exact) {
+    const double decay = w[0], omb1 = w[1], b2 = w[2], omb2 = w[3], step_size = w[4],
+                 bc2_sqrt = w[5], e = w[6];
+    const double lerp_high = 1.0 - omb1;
+    const bool low = flags[1] != 0;
+    parallel_for(n, 1 << 14, [&](size_t lo, size_t hi) {
+      bool ok = true;
+      for (size_t i = lo; i < hi; ++i) {
+        double gd = g[i], md = m[i], vd = v[i];
+        double m1 = low ? md + omb1 * (gd - md) : gd - (gd - md) * lerp_high;
+        double v1 = b2 * vd + omb2 * gd * gd;
+        double denom = std::sqrt(v1) / bc2_sqrt + e;
+        double delta = (-step_size) * m1 / denom;
+        double q = p[i];
+        if (decays) q *= decay;
+        q += delta;
+        float new_p = (!decays && delta == 0.0) ? p[i] : static_cast<float>(q);
+        float m32 = static_cast<float>(m1), v32 = static_cast<float>(v1);
+        ok &= std::isfinite(m1) && std::isfinite(v1) && std::isfinite(denom) &&
+              std::isfinite(delta) && finite32(new_p) && finite32(m32) && finite32(v32);
+        np[i] = new_p;
+        nm[i] = m32;
+        nv[i] = v32;
+      }
+      if (!ok) status = ORC_NON_FINITE;
+    });
+  } else {
+    const float decay = static_cast<float>(w[0]), omb1 = static_cast<float>(w[1]),
+                b2 = static_cast<float>(w[2]), omb2 = static_cast<float>(w[3]),
+                step_size = static_cast<float>(w[4]), bc2_sqrt = static_cast<float>(w[5]),
+                e = static_cast<float>(w[6]);
+    const float lerp_high = 1.0f - omb1;
+    const bool low = flags[2] != 0;
+    parallel_for(n, 1 << 14, [&](size_t lo, size_t hi) {
+      bool ok = true;
+      for (size_t i = lo; i < hi; ++i) {
+        float gf = g[i], mf = m[i], vf = v[i];
+        float m1 = low ? mf + omb1 * (gf - mf) : gf - (gf - mf) * lerp_high;
+        float v1 = b2 * vf + omb2 * gf * gf;
+        float denom = std::sqrt(v1) / bc2_sqrt + e;
+        float delta = (-step_size) * m1 / denom;
+        float q = p[i];
+        if (decays) q *= decay;
+        q += delta;
+        float new_p = (!decays && delta == 0.0f) ? p[i] : q;
+        ok &= finite32(m1) && finite32(v1) && finite32(denom) && finite32(delta) && finite32(new_p);
+        np[i] = new_p;
+        nm[i] = m1;
+        nv[i] = v1;
+      }
+      if (!ok) status = ORC_NON_FINITE;
+    });
+  }
+  if (status.load() != ORC_OK) return status.load();
+  std::memcpy(p, np.data(), n * sizeof(float));
+  std::memcpy(m, nm.data(), n * sizeof(float));
+  std::memcpy(v, nv.data(), n * sizeof(float));
+  return ORC_OK;
+}
+
+// ---- Muon NS5 (ojas-cpu/src/optim.rs:684-743, :841-985) ----
+namespace {
+void transpose(const float* a, float* out, size_t rows, size_t cols) {
+  for (size_t r = 0; r < rows; ++r)
+    for (size_t c = 0; c < cols; ++c) out[c * rows + r] = a[r * cols + c];
+}
+
+int newton_schulz(std::vector<float>& x, size_t rows, size_t cols, bool bf16) {
+  if (bf16)
+    for (auto& v : x) v = round_bf16(v);
+  // The reference reads a tall 2048x768 update through a transposed view
+  // instead of a copy; its norm sum then walks the same order as the copy's.
+  bool transposed = rows > cols;
+  size_t r = rows, c = cols;
+  if (transposed) {
+    std::vector<float> t(x.size());
+    transpose(x.data(), t.data(), rows, cols);
+    x.swap(t);
+    r = cols;
+    c = rows;
+  }
+  double sum_sq = 0.0;
+  for (float v : x) sum_sq += static_cast<double>(v) * static_cast<double>(v);
+  float norm = static_cast<float>(std::sqrt(sum_sq));
+  const float ns_eps = static_cast<float>(1e-7);
+  float denom = bf16 ? round_bf16(round_bf16(norm) + ns_eps) : norm + ns_eps;
+  if (!(finite32(denom) && denom != 0.0f)) return ORC_NON_FINITE;
+  for (auto& v : x) v /= denom;
+  if (bf16)
+    for (auto& v : x) v = round_bf16(v);
+  const float a = static_cast<float>(3.4445), b_coef = static_cast<float>(-4.7750),
+              c_coef = static_cast<float>(2.0315);
+  std::vector<float> am(r * r), a2(r * r), bx(x.size());
+  for (int it = 0; it < 5; ++it) {
+    // A = X X^T
+    gemm(x.data(), c, 1, x.data(), 1, c, am.data(), r, c, r, false);
+    if (bf16)
+      for (auto& v : am) v = round_bf16(v);
+    gemm(am.data(), r, 1, am.data(), r, 1, a2.data(), r, r, r, false);
+    if (bf16) {
+      for (size_t i = 0; i < a2.size(); ++i)
+        a2[i] = round_bf16(round_bf16(b_coef * am[i]) + round_bf16(c_coef * round_bf16(a2[i])));
+    } else {
+      for (size_t i = 0; i < a2.size(); ++i) a2[i] = b_coef * am[i] + c_coef * a2[i];
+    }
+    gemm(a2.data(), r, 1, x.data(), c, 1, bx.data(), r, r, c, false);
+    if (bf16) {
+      for (size_t i = 0; i < bx.size(); ++i)
+        bx[i] = round_bf16(round_bf16(a * x[i]) + round_bf16(bx[i]));
+    } else {
+      for (size_t i = 0; i < bx.size(); ++i) bx[i] = a * x[i] + bx[i];
+    }
+    if (!all_finite(bx.data(), bx.size())) return ORC_NON_FINITE;
+    x.swap(bx);
+  }
+  if (transposed) {
+    std::vector<float> t(x.size());
+    transpose(x.data(), t.data(), r, c);
+    x.swap(t);
+  }
+  return ORC_OK;
+}
+}  // namespace
+
+int orc_muon_ns5_step(float* p, const float* g, float* m, size_t rows, size_t cols, double lr,
+                      double momentum, double weight_decay, int nesterov, int bf16) {
+  if (!std::isfinite(lr) || !std::isfinite(momentum) || !std::isfinite(weight_decay))
+    return ORC_NON_FINITE;
+  if (lr < 0.0 || momentum < 0.0 || weight_decay < 0.0) return ORC_OUT_OF_RANGE;
+  if (cols == 0 || rows == 0) return ORC_SHAPE;
+  size_t len = rows * cols;
+  if (!(all_finite(p, len) && all_finite(g, len) && all_finite(m, len))) return ORC_NON_FINITE;
+  float mom = static_cast<float>(momentum);
+  std::vector<float> buf(len), update(len);
+  for (size_t i = 0; i < len; ++i) buf[i] = mom * m[i] + g[i];
+  if (!all_finite(buf.data(), len)) return ORC_NON_FINITE;
+  // Nesterov blend and the parameter update are one fused multiply-add per
+  // value, as torch's add(.., alpha=..) is (optim.rs:705-712).
+  if (nesterov)
+    for (size_t i = 0; i < len; ++i) update[i] = std::fmaf(mom, buf[i], g[i]);
+  else
+    update = buf;
+  int rc = newton_schulz(update, rows, cols, bf16 != 0);
+  if (rc != ORC_OK) return rc;
+  double scale = std::sqrt(std::max(static_cast<double>(rows) / static_cast<double>(cols), 1.0));
+  float alpha = static_cast<float>(-lr * scale);
+  bool all_zero = true;
+  for (float v : update) all_zero &= (v == 0.0f);
+  std::vector<float> new_p;
+  if (!(weight_decay == 0.0 && all_zero)) {
+    new_p.resize(len);
+    if (weight_decay != 0.0) {
+      float decay = static_cast<float>(1.0 - lr * weight_decay);
+      for (size_t i = 0; i < len; ++i) new_p[i] = std::fmaf(alpha, update[i], p[i] * decay);
+    } else {
+      for (size_t i = 0; i < len; ++i) new_p[i] = std::fmaf(alpha, update[i], p[i]);
+    }
+    if (!all_finite(new_p.data(), len)) return ORC_NON_FINITE;
+    std::memcpy(p, new_p.data(), len * sizeof(float));
+  }
+  std::memcpy(m, buf.data(), len * sizeof(float));
+  return ORC_OK;
+}
+
+// ojas-cpu/src/backend.rs:770-795, optim.rs:61-101
+int orc_clip_grad_norm(float* const* grads, const size_t* lens, size_t count, float max_norm,
+                       float* norm_out) {
+  double sum_sq = 0.0;
+  for (size_t t = 0; t < count; ++t)
+    for (size_t i = 0; i < lens[t]; ++i) {
+      double v = grads[t][i];
+      sum_sq += v * v;
+    }
+  float norm = static_cast<float>(std::sqrt(sum_sq));
+  if (!finite32(norm)) return ORC_NON_FINITE;
+  float coef;
+  int rc = orc_clip_scale(max_norm, norm, &coef);
+  if (rc != ORC_OK) return rc;
+  if (coef < 1.0f)
+    for (size_t t = 0; t < count; ++t)
+      for (size_t i = 0; i < lens[t]; ++i) grads[t][i] *= coef;
+  *norm_out = norm;
+  return ORC_OK;
+}
+
+// ---- elementwise / layout ----
+int orc_residual_add(const float* x, const float* y, float* out, size_t n) {
+  bool ok = true;
+  for (size_t i = 0; i < n; ++i) {
+    out[i] = x[i] + y[i];
+    ok &= finite32(out[i]);
+  }
+  return ok ? ORC_OK : ORC_NON_FINITE;
+}
+int orc_accumulate_grad(float* acc, const float* g, size_t n) {
+  bool ok = true;
+  for (size_t i = 0; i < n; ++i) ok &= finite32(acc[i] + g[i]);
+  if (!ok) return ORC_NON_FINITE;
+  for (size_t i = 0; i < n; ++i) acc[i] = acc[i] + g[i];
+  return ORC_OK;
+}
+int orc_scale_grad(float* g, float s, size_t n) {
+  for (size_t i = 0; i < n; ++i) g[i] *= s;
+  return all_finite(g, n) ? ORC_OK : ORC_NON_FINITE;
+}
+void orc_gelu_erf_forward_vec(const float* x, float* y, size_t n) {
+  parallel_for(n, 4096, [&](size_t lo, size_t hi) {
+    for (size_t i = lo; i < hi; ++i) y[i] = gelu_erf(x[i]);
+  });
+}
+void orc_gelu_erf_backward_vec(const float* x, const float* gy, float* gx, size_t n) {
+  parallel_for(n, 4096, [&](size_t lo, size_t hi) {
+    for (size_t i = lo; i < hi; ++i) gx[i] = gelu_erf_backward(x[i], gy[i]);
+  });
+}
+void orc_gelu_tanh_forward_vec(const float* x, float* y, size_t n) {
+  parallel_for(n, 4096, [&](size_t lo, size_t hi) {
+    for (size_t i = lo; i < hi; ++i) y[i] = gelu_tanh(x[i]);
+  });
+}
+void orc_gelu_tanh_backward_vec(const float* x, const float* gy, float* gx, size_t n) {
+  parallel_for(n, 4096, [&](size_t lo, size_t hi) {
+    for (size_t i = lo; i < hi; ++i) gx[i] = gelu_tanh_backward(x[i], gy[i]);
+  });
+}
+void orc_permute_0213(const float* x, float* y, size_t d0, size_t d1, size_t d2, size_t d3) {
+  for (size_t a = 0; a < d0; ++a)
+    for (size_t b = 0; b < d1; ++b)
+      for (size_t c = 0; c < d2; ++c)
+        std::memcpy(y + ((a * d2 + c) * d1 + b) * d3, x + ((a * d1 + b) * d2 + c) * d3,
+                    d3 * sizeof(float));
+}
+
+int orc_argmax_rows(const float* x, size_t rows, size_t cols, uint32_t* out) {
+  for (size_t r = 0; r < rows; ++r) {
+    const float* row = x + r * cols;
+    size_t best = 0;
+    for (size_t i = 0; i < cols; ++i) {
+      if (!finite32(row[i])) return ORC_NON_FINITE;
+      if (row[i] > row[best]) best = i;
+    }
+    out[r] = static_cast<uint32_t>(best);
+  }
+  return ORC_OK;
+}
+
+// Order: value descending with +0 == -0, then column ascending
+// (ojas-core/src/backend.rs:184-195: total order on the canonical zero).
+int orc_topk_rows(const float* x, size_t rows, size_t cols, size_t k, uint32_t* idx, float* val) {
+  if (k == 0 || k > cols) return ORC_SHAPE;
+  std::vector<uint32_t> order(cols);
+  for (size_t r = 0; r < rows; ++r) {
+    const float* row = x + r * cols;
+    for (size_t i = 0; i < cols; ++i)
+      if (row[i] != row[i] || row[i] == std::numeric_limits<float>::infinity())
+        return ORC_NON_FINITE;
+    for (size_t i = 0; i < cols; ++i) order[i] = static_cast<uint32_t>(i);
+    auto key = [&](uint32_t i) { return row[i] == 0.0f ? 0.0f : row[i]; };
+    std::stable_sort(order.begin(), order.end(), [&](uint32_t a, uint32_t b) {
+      float ka = key(a), kb = key(b);
+      if (ka != kb) return ka > kb;
+      return a < b;
+    });
+    for (size_t j = 0; j < k; ++j) {
+      idx[r * k + j] = order[j];
+      val[r * k + j] = row[order[j]];
+    }
+  }
+  return ORC_OK;
+}
+
+}  // extern "C"
