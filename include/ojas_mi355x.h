@@ -1,0 +1,240 @@
+/* ojas_mi355x.h: C ABI of the MI355X (gfx950) backend for the nanolab-GPT
+ * training-step op set of ojas.
+ *
+ * The reference has no per-op C ABI: its boundary is the Rust trait
+ * `ojas_core::Backend` (ojas-core/src/backend.rs:2634, method list :2655-2767).
+ * Each entry point below is what a Rust crate implementing that trait binds
+ * for one trait method; the comment on each names the method it serves.
+ *
+ * Conventions
+ *  - Every function returns 0 (OMX_OK) or an omx_status that maps 1:1 onto an
+ *    `OjasError` variant (ojas-core/src/error.rs:18-105). The text of the last
+ *    error of a context is read with omx_last_error.
+ *  - All tensor pointers are DEVICE pointers obtained from omx_alloc (or any
+ *    hipMalloc'd memory of the context's device), contiguous row-major. A view
+ *    with a byte offset is passed as pointer + offset by the caller.
+ *  - Outputs are caller-allocated and fully overwritten. Nothing is freed that
+ *    the library did not allocate.
+ *  - dtype arguments are omx_dtype values. Matmul-class operands may be
+ *    OMX_F32 or OMX_BF16 storage (the reference's bf16 operand slots,
+ *    backend.rs:1003-1031); bf16 storage runs on the bf16 MFMA lane with f32
+ *    accumulation, f32 storage on the f32 MFMA lane.
+ *  - Non-finite detection is deferred (the contract of a device backend,
+ *    ojas-wgpu/src/backend.rs:35-73): an op that meets a NaN/Inf returns
+ *    OMX_OK, raises its bit in the context's device fault word, and the next
+ *    omx_sync / omx_download / omx_clip_grad_norm / omx_read_scalar_f32
+ *    returns OMX_NON_FINITE naming the first faulting op. Optimizer steps
+ *    decide on the device and write nothing when any value is non-finite.
+ *  - A context owns one HIP stream and is not thread-safe.
+ */
+#ifndef OJAS_MI355X_H
+#define OJAS_MI355X_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct omx_ctx omx_ctx;
+
+/* OjasError variants, ojas-core/src/error.rs:18-105. */
+typedef enum {
+  OMX_OK = 0,
+  OMX_SHAPE = 1,
+  OMX_DTYPE = 2,
+  OMX_OUT_OF_RANGE = 3,
+  OMX_NON_FINITE = 4,
+  OMX_UNSUPPORTED_HEAD_DIM = 5,
+  OMX_CAPACITY_EXCEEDED = 6,
+  OMX_POISONED = 7,
+  OMX_DEVICE_LOST = 8,
+  OMX_WAIT_TIMEOUT = 9,
+  OMX_BACKEND = 10,
+  OMX_UNSUPPORTED = 11,
+  OMX_PLACEMENT = 12
+} omx_status;
+
+/* ojas-core/src/dtype.rs:5 (the three the GPT op set uses). */
+typedef enum { OMX_F32 = 0, OMX_BF16 = 1, OMX_U32 = 2 } omx_dtype;
+
+/* ---- context, residency, faults: BackendCore::{upload,download,sync}
+ *      (backend.rs:908-973), Budget (ojas-core/src/budget.rs:19-316) ---- */
+
+/* Opens device `device` with a byte budget for omx_alloc (0 = unlimited).
+ * Failure kinds follow ojas-hip/src/lib.rs:106-122 (no device ->
+ * OMX_DEVICE_LOST, out of memory -> OMX_CAPACITY_EXCEEDED, a device that is
+ * not gfx950 -> OMX_UNSUPPORTED). */
+int32_t omx_open(int32_t device, uint64_t budget_bytes, omx_ctx** out);
+void omx_close(omx_ctx* ctx);
+/* Copies the last error text (NUL-terminated) and returns its length. */
+size_t omx_last_error(omx_ctx* ctx, char* buf, size_t cap);
+/* Name of the device's architecture, e.g. "gfx950". */
+size_t omx_device_name(omx_ctx* ctx, char* buf, size_t cap);
+
+/* Budget: charge before allocating, refuse rather than clamp. */
+int32_t omx_alloc(omx_ctx* ctx, uint64_t bytes, void** out);
+int32_t omx_free(omx_ctx* ctx, void* ptr);
+uint64_t omx_budget_live(omx_ctx* ctx);
+uint64_t omx_budget_peak(omx_ctx* ctx);
+uint64_t omx_budget_limit(omx_ctx* ctx);
+void omx_budget_reset_peak(omx_ctx* ctx);
+
+int32_t omx_upload(omx_ctx* ctx, void* dst, uint64_t dst_offset, const void* host_src,
+                   uint64_t bytes);
+/* Waits for submitted work, reports a deferred fault, then copies. */
+int32_t omx_download(omx_ctx* ctx, void* host_dst, const void* src, uint64_t src_offset,
+                     uint64_t bytes);
+int32_t omx_copy(omx_ctx* ctx, void* dst, const void* src, uint64_t bytes);
+int32_t omx_fill_zero(omx_ctx* ctx, void* dst, uint64_t bytes);
+/* Waits for all submitted work; reports and clears a deferred fault. */
+int32_t omx_sync(omx_ctx* ctx);
+/* The context's HIP stream (hipStream_t), for callers that time with events. */
+void* omx_stream(omx_ctx* ctx);
+
+/* ---- casts: BackendCore::{cast_bf16,to_bf16,to_f32} (backend.rs:975-1090),
+ *      rounding rule ojas-core/src/autocast.rs:66-101 ---- */
+int32_t omx_cast_bf16(omx_ctx* ctx, const void* x_f32, void* y_f32, uint64_t n);
+int32_t omx_to_bf16(omx_ctx* ctx, const void* x_f32, void* y_bf16, uint64_t n);
+int32_t omx_to_f32(omx_ctx* ctx, const void* x_bf16, void* y_f32, uint64_t n);
+
+/* ---- BackendModule::linear_forward (backend.rs:1628):
+ *      y[rows,out] = x[rows,in] . W[out,in]^T ---- */
+int32_t omx_linear_forward(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* w,
+                           int32_t w_dtype, void* y, int32_t y_dtype, uint64_t rows,
+                           uint64_t in_features, uint64_t out_features);
+/* BackendModule::linear_backward (backend.rs:1631): gx = gy.W, gw = gy^T.x.
+ * gx or gw may be NULL (linear_backward_input, backend.rs:1643-1656). */
+int32_t omx_linear_backward(omx_ctx* ctx, const void* x, const void* w, const void* gy,
+                            int32_t operand_dtype, void* gx, int32_t gx_dtype, void* gw,
+                            int32_t gw_dtype, uint64_t rows, uint64_t in_features,
+                            uint64_t out_features);
+/* General product behind the three above and the Newton-Schulz products:
+ * C[m,n] (+)= A.B with A(i,p) at a[i*a_rs + p*a_cs], B(p,j) at b[p*b_rs + j*b_cs]
+ * (element strides; one stride of each operand must be 1). */
+int32_t omx_gemm(omx_ctx* ctx, const void* a, uint64_t a_rs, uint64_t a_cs, const void* b,
+                 uint64_t b_rs, uint64_t b_cs, int32_t operand_dtype, void* c, int32_t c_dtype,
+                 uint64_t m, uint64_t k, uint64_t n, int32_t accumulate);
+
+/* ---- BackendModule::causal_sdpa_forward / _backward (backend.rs:1729-1792).
+ *      q,out,gy,gq: [B,H,T,D]; k,v,gk,gv: [B,Hkv,T,D]; lse: [B,H,T] f32.
+ *      window = 0: every earlier key. scale = 1/sqrt(D) (backend.rs:159). ---- */
+int32_t omx_causal_sdpa_forward(omx_ctx* ctx, const void* q, const void* k, const void* v,
+                                int32_t operand_dtype, void* out, int32_t out_dtype, void* lse,
+                                uint64_t batch, uint64_t heads, uint64_t kv_heads, uint64_t time,
+                                uint64_t head_dim, uint64_t window);
+int32_t omx_causal_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, const void* v,
+                                 const void* out, const void* lse, const void* gy,
+                                 int32_t operand_dtype, void* gq, void* gk, void* gv,
+                                 int32_t grad_dtype, uint64_t batch, uint64_t heads,
+                                 uint64_t kv_heads, uint64_t time, uint64_t head_dim,
+                                 uint64_t window);
+
+/* ---- BackendModule::rms_norm_forward / _backward (backend.rs:1658-1672) ---- */
+int32_t omx_rms_norm_forward(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* w_f32,
+                             void* y, int32_t y_dtype, uint64_t rows, uint64_t dim, float eps);
+int32_t omx_rms_norm_backward(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* w_f32,
+                              const void* gy, int32_t gy_dtype, void* gx, int32_t gx_dtype,
+                              void* gw_f32, uint64_t rows, uint64_t dim, float eps);
+
+/* ---- BackendModule::cross_entropy_mean_forward / _backward
+ *      (backend.rs:2451-2466). loss is one f32 on the device. ---- */
+int32_t omx_cross_entropy_mean_forward(omx_ctx* ctx, const void* logits, int32_t logits_dtype,
+                                       const void* targets_u32, uint64_t rows, uint64_t vocab,
+                                       int32_t has_ignore, uint32_t ignore_index, void* loss_f32);
+int32_t omx_cross_entropy_mean_backward(omx_ctx* ctx, const void* logits, int32_t logits_dtype,
+                                        const void* targets_u32, uint64_t rows, uint64_t vocab,
+                                        int32_t has_ignore, uint32_t ignore_index, void* grad,
+                                        int32_t grad_dtype);
+/* BackendModule::linear_cross_entropy_mean (backend.rs:2493-2524): mean CE of
+ * x.W^T without an [N,V] logits tensor; at most chunk_rows x chunk_cols logits
+ * exist at once (CeChunk, backend.rs:3081). gx / gw may be NULL (CeGrads). */
+int32_t omx_linear_cross_entropy_mean(omx_ctx* ctx, const void* x, const void* w,
+                                      int32_t operand_dtype, const void* targets_u32, uint64_t rows,
+                                      uint64_t dim, uint64_t vocab, int32_t has_ignore,
+                                      uint32_t ignore_index, uint64_t chunk_rows,
+                                      uint64_t chunk_cols, void* loss_f32, void* gx,
+                                      int32_t gx_dtype, void* gw_f32);
+
+/* ---- BackendModule::embedding_forward / _backward (backend.rs:1610-1626).
+ *      The gather is a bit copy; the scatter-add sums each table row's tokens
+ *      in ascending token order (ojas-cpu/src/pointwise.rs:171-215). ---- */
+int32_t omx_embedding_forward(omx_ctx* ctx, const void* table, int32_t table_dtype,
+                              const void* ids_u32, void* out, int32_t out_dtype, uint64_t tokens,
+                              uint64_t vocab, uint64_t dim);
+int32_t omx_embedding_backward(omx_ctx* ctx, const void* ids_u32, const void* grad,
+                               int32_t grad_dtype, void* table_grad_f32, uint64_t tokens,
+                               uint64_t vocab, uint64_t dim);
+
+/* ---- optimizers ---- */
+/* ojas_core::AdamWConfig (backend.rs:494-517). */
+typedef struct {
+  double lr, beta1, beta2, eps, weight_decay;
+} omx_adamw_config;
+/* BackendModule::adamw_step (backend.rs:2468-2478): `step` is the count before
+ * this update. The scalars are formed in f64 on the host
+ * (AdamWScalars, backend.rs:371-477) and the element math is f32 (the Fast
+ * contract, ojas-cpu/src/optim.rs:302-395). param_bf16, when not NULL, also
+ * receives the updated parameter rounded to bf16 (the copy the next step's
+ * bf16 matmuls read). */
+int32_t omx_adamw_step(omx_ctx* ctx, void* param_f32, const void* grad_f32, void* moment1_f32,
+                       void* moment2_f32, uint64_t n, uint64_t step, const omx_adamw_config* config,
+                       void* param_bf16);
+/* ojas_core::MuonNs5Config (backend.rs:548-570). */
+typedef struct {
+  double lr, momentum, weight_decay;
+  int32_t nesterov;
+  int32_t ns5_bf16;
+} omx_muon_config;
+/* BackendModule::muon_ns5_step (backend.rs:2480-2491). */
+int32_t omx_muon_ns5_step(omx_ctx* ctx, void* param_f32, const void* grad_f32, void* momentum_f32,
+                          uint64_t rows, uint64_t cols, const omx_muon_config* config,
+                          void* param_bf16);
+/* Bytes of device scratch omx_muon_ns5_step takes from the budget
+ * (BackendCore::optimizer_scratch_bytes, backend.rs:938-961). */
+uint64_t omx_muon_scratch_bytes(uint64_t rows, uint64_t cols);
+/* BackendFloat::clip_grad_norm (backend.rs:1466-1471): global L2 norm with an
+ * f64 sum of squares, returned on the host; scales in place when the clip
+ * coefficient (clip_scale, backend.rs:277-303) is below 1. A sync point. */
+int32_t omx_clip_grad_norm(omx_ctx* ctx, void* const* grads_f32, const uint64_t* lens,
+                           uint64_t count, float max_norm, float* norm_out);
+
+/* ---- elementwise and layout ---- */
+/* BackendFloat::residual_add_forward (backend.rs:1165-1173). */
+int32_t omx_residual_add(omx_ctx* ctx, const void* x, const void* y, void* out, int32_t dtype,
+                         uint64_t n);
+/* BackendFloat::accumulate_grad / scale_grad (backend.rs:1473-1510). */
+int32_t omx_accumulate_grad(omx_ctx* ctx, void* acc_f32, const void* grad_f32, uint64_t n);
+int32_t omx_scale_grad(omx_ctx* ctx, void* grad_f32, float scale, uint64_t n);
+/* BackendFloat::gelu_erf_* / gelu_tanh_* (backend.rs:1175-1220). tanh_form
+ * selects the tanh approximation. */
+int32_t omx_gelu_forward(omx_ctx* ctx, const void* x, void* y, int32_t dtype, uint64_t n,
+                         int32_t tanh_form);
+int32_t omx_gelu_backward(omx_ctx* ctx, const void* x, const void* gy, void* gx, int32_t dtype,
+                          uint64_t n, int32_t tanh_form);
+/* BackendFloat::permute with axes [0,2,1,3] (backend.rs:1115-1134; the one
+ * permutation the model uses, ojas-model/src/block.rs:25,195-199):
+ * [d0,d1,d2,d3] -> [d0,d2,d1,d3]. */
+int32_t omx_permute_0213(omx_ctx* ctx, const void* x, void* y, int32_t dtype, uint64_t d0,
+                         uint64_t d1, uint64_t d2, uint64_t d3);
+
+/* ---- BackendInt::argmax_rows / topk_rows (backend.rs:1514-1606) ---- */
+int32_t omx_argmax_rows(omx_ctx* ctx, const void* x_f32, uint64_t rows, uint64_t cols,
+                        void* out_u32);
+int32_t omx_topk_rows(omx_ctx* ctx, const void* x_f32, uint64_t rows, uint64_t cols, uint64_t k,
+                      void* values_f32, void* ids_u32);
+
+/* Reads one f32 from the device after a sync (the step's single readback,
+ * ojas-model/src/trainer.rs:1031-1046). */
+int32_t omx_read_scalar_f32(omx_ctx* ctx, const void* src, float* out);
+
+/* Every Backend method outside the GPT op set answers through this: sets the
+ * error text to the op's name and returns OMX_UNSUPPORTED
+ * (unsupported_op, backend.rs:792-797). */
+int32_t omx_unsupported(omx_ctx* ctx, const char* op);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

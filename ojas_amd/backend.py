@@ -1,0 +1,462 @@
+"""`MiBackend`: the host-side mirror of ojas's `Backend` trait over the C ABI.
+
+The reference's boundary is the Rust trait `ojas_core::Backend`
+(ojas-core/src/backend.rs:2634; method list :2655-2767). This module binds
+`libojas_mi355x.so` with ctypes and exposes the same method names, argument
+meaning and error behaviour for the GPT op set; every other trait method
+raises `OjasError(UNSUPPORTED)` (backend.rs:792-797). It holds no arithmetic:
+each method validates nothing itself and forwards to one C entry point.
+
+There is no CPU fallback: constructing `MiBackend` without the built library
+or without a gfx950 device raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from pathlib import Path
+from typing import Optional, Sequence, Tuple
+
+import numpy as np
+
+LIB_PATH = Path(__file__).resolve().parent / "libojas_mi355x.so"
+
+F32, BF16, U32 = 0, 1, 2
+_NP_OF = {F32: np.float32, BF16: np.uint16, U32: np.uint32}
+_SIZE_OF = {F32: 4, BF16: 2, U32: 4}
+
+(OK, SHAPE, DTYPE, OUT_OF_RANGE, NON_FINITE, UNSUPPORTED_HEAD_DIM, CAPACITY_EXCEEDED, POISONED, DEVICE_LOST,
+ WAIT_TIMEOUT, BACKEND, UNSUPPORTED, PLACEMENT) = range(13)
+_STATUS_NAMES = ["Ok", "Shape", "Dtype", "OutOfRange", "NonFinite", "UnsupportedHeadDim", "CapacityExceeded",
+                 "Poisoned", "DeviceLost", "WaitTimeout", "Backend", "Unsupported", "Placement"]
+
+
+class OjasError(RuntimeError):
+    """One `OjasError` variant (ojas-core/src/error.rs:18-105): `code` + detail text."""
+
+    def __init__(self, code: int, detail: str = ""):
+        name = _STATUS_NAMES[code] if 0 <= code < len(_STATUS_NAMES) else str(code)
+        super().__init__(f"{name}: {detail}")
+        self.code = code
+        self.variant = name
+        self.detail = detail
+
+
+class AdamWConfig(C.Structure):
+    """ojas_core::AdamWConfig (backend.rs:494-517)."""
+    _fields_ = [("lr", C.c_double), ("beta1", C.c_double), ("beta2", C.c_double), ("eps", C.c_double),
+                ("weight_decay", C.c_double)]
+
+    @classmethod
+    def nanolab(cls, lr: float, weight_decay: float) -> "AdamWConfig":
+        return cls(lr, 0.9, 0.95, 1e-8, weight_decay)
+
+
+class MuonNs5Config(C.Structure):
+    """ojas_core::MuonNs5Config (backend.rs:548-570)."""
+    _fields_ = [("lr", C.c_double), ("momentum", C.c_double), ("weight_decay", C.c_double), ("nesterov", C.c_int32),
+                ("ns5_bf16", C.c_int32)]
+
+    @classmethod
+    def nanolab_default(cls) -> "MuonNs5Config":
+        return cls(0.025, 0.99, 0.1, 1, 0)
+
+
+def load_library() -> C.CDLL:
+    if not LIB_PATH.exists():
+        raise OjasError(BACKEND, f"{LIB_PATH} is not built; run __graft_entry__.build()")
+    lib = C.CDLL(str(LIB_PATH))
+    lib.omx_last_error.restype = C.c_size_t
+    lib.omx_device_name.restype = C.c_size_t
+    for name in ("omx_budget_live", "omx_budget_peak", "omx_budget_limit", "omx_muon_scratch_bytes"):
+        if hasattr(lib, name):
+            getattr(lib, name).restype = C.c_uint64
+    lib.omx_stream.restype = C.c_void_p
+    return lib
+
+
+class DeviceTensor:
+    """A contiguous device tensor: pointer, shape, dtype. Frees itself on drop
+    (the role of `Arc<dyn DeviceBuffer>` + `Reservation`, tensor.rs:146-163)."""
+
+    def __init__(self, backend: "MiBackend", ptr: int, shape: Tuple[int, ...], dtype: int, owns: bool = True):
+        self.backend, self.ptr, self.shape, self.dtype, self._owns = backend, ptr, tuple(shape), dtype, owns
+
+    @property
+    def numel(self) -> int:
+        return int(np.prod(self.shape)) if self.shape else 1
+
+    @property
+    def nbytes(self) -> int:
+        return self.numel * _SIZE_OF[self.dtype]
+
+    def reshape(self, *shape) -> "DeviceTensor":
+        """Zero-copy view (tensor.rs:1555-1605); the view does not own the memory."""
+        shape = tuple(shape[0]) if len(shape) == 1 and isinstance(shape[0], (tuple, list)) else tuple(shape)
+        if int(np.prod(shape)) != self.numel:
+            raise OjasError(SHAPE, f"reshape {self.shape} -> {shape}")
+        view = DeviceTensor(self.backend, self.ptr, shape, self.dtype, owns=False)
+        view._base = self
+        return view
+
+    def __del__(self):
+        if getattr(self, "_owns", False) and self.ptr and self.backend is not None and self.backend._ctx:
+            self.backend._lib.omx_free(self.backend._ctx, C.c_void_p(self.ptr))
+            self.ptr = 0
+
+
+class MiBackend:
+    """`impl Backend for MiBackend`: BackendId::Hip, Numerics::Fast, bf16 operands accepted."""
+
+    id = "hip"
+    numerics = "fast"
+    bf16_operands = True
+
+    def __init__(self, device: int = 0, budget_bytes: int = 0):
+        self._lib = load_library()
+        ctx = C.c_void_p()
+        rc = self._lib.omx_open(C.c_int32(device), C.c_uint64(budget_bytes), C.byref(ctx))
+        self._ctx = ctx if rc == OK else None
+        if rc != OK:
+            raise OjasError(rc, "omx_open failed (no gfx950 device or runtime error)")
+
+    def close(self):
+        if self._ctx:
+            self._lib.omx_close(self._ctx)
+            self._ctx = None
+
+    # ---- plumbing ----
+    def _check(self, rc: int):
+        if rc != OK:
+            buf = C.create_string_buffer(512)
+            self._lib.omx_last_error(self._ctx, buf, C.c_size_t(512))
+            raise OjasError(rc, buf.value.decode("utf-8", "replace"))
+
+    def device_name(self) -> str:
+        buf = C.create_string_buffer(128)
+        self._lib.omx_device_name(self._ctx, buf, C.c_size_t(128))
+        return buf.value.decode()
+
+    def stream(self) -> int:
+        return int(self._lib.omx_stream(self._ctx) or 0)
+
+    def budget(self):
+        return {"live": int(self._lib.omx_budget_live(self._ctx)), "peak": int(self._lib.omx_budget_peak(self._ctx)),
+                "limit": int(self._lib.omx_budget_limit(self._ctx))}
+
+    def empty(self, shape, dtype: int = F32) -> DeviceTensor:
+        shape = tuple(int(s) for s in (shape if isinstance(shape, (tuple, list)) else (shape,)))
+        n = int(np.prod(shape)) if shape else 1
+        ptr = C.c_void_p()
+        self._check(self._lib.omx_alloc(self._ctx, C.c_uint64(max(n, 1) * _SIZE_OF[dtype]), C.byref(ptr)))
+        return DeviceTensor(self, ptr.value, shape, dtype)
+
+    def zeros(self, shape, dtype: int = F32) -> DeviceTensor:
+        t = self.empty(shape, dtype)
+        self._check(self._lib.omx_fill_zero(self._ctx, C.c_void_p(t.ptr), C.c_uint64(t.nbytes)))
+        return t
+
+    def upload(self, host: np.ndarray, dtype: Optional[int] = None) -> DeviceTensor:
+        """BackendCore::upload (backend.rs:917-936). float32 -> F32, uint32 -> U32,
+        uint16 -> BF16 bits; `dtype=BF16` on a float32 array rounds on the device."""
+        host = np.ascontiguousarray(host)
+        if host.dtype == np.float32:
+            src_dtype = F32
+        elif host.dtype == np.uint32:
+            src_dtype = U32
+        elif host.dtype == np.uint16:
+            src_dtype = BF16
+        else:
+            raise OjasError(DTYPE, f"upload of {host.dtype}")
+        t = self.empty(host.shape, src_dtype)
+        if host.size:
+            self._check(self._lib.omx_upload(self._ctx, C.c_void_p(t.ptr), C.c_uint64(0),
+                                             host.ctypes.data_as(C.c_void_p), C.c_uint64(host.nbytes)))
+        if dtype is not None and dtype != src_dtype:
+            if src_dtype == F32 and dtype == BF16:
+                return self.to_bf16(t)
+            raise OjasError(DTYPE, "upload conversion")
+        return t
+
+    def download(self, t: DeviceTensor) -> np.ndarray:
+        """BackendCore::download (backend.rs:938-961): syncs, reports deferred faults."""
+        out = np.empty(t.shape, dtype=_NP_OF[t.dtype])
+        self._check(self._lib.omx_download(self._ctx, out.ctypes.data_as(C.c_void_p), C.c_void_p(t.ptr),
+                                           C.c_uint64(0), C.c_uint64(t.nbytes)))
+        return out
+
+    def download_f32(self, t: DeviceTensor) -> np.ndarray:
+        """Downloads and widens bf16 storage exactly (bits << 16)."""
+        a = self.download(t)
+        if t.dtype == BF16:
+            return (a.astype(np.uint32) << 16).view(np.float32)
+        return a
+
+    def sync(self):
+        """BackendCore::sync (backend.rs:963-973)."""
+        self._check(self._lib.omx_sync(self._ctx))
+
+    def _p(self, t: Optional[DeviceTensor]):
+        return C.c_void_p(t.ptr) if t is not None else C.c_void_p(None)
+
+    # ---- casts ----
+    def cast_bf16(self, x: DeviceTensor) -> DeviceTensor:
+        y = self.empty(x.shape, F32)
+        self._check(self._lib.omx_cast_bf16(self._ctx, self._p(x), self._p(y), C.c_uint64(x.numel)))
+        return y
+
+    def to_bf16(self, x: DeviceTensor) -> DeviceTensor:
+        y = self.empty(x.shape, BF16)
+        self._check(self._lib.omx_to_bf16(self._ctx, self._p(x), self._p(y), C.c_uint64(x.numel)))
+        return y
+
+    def to_f32(self, x: DeviceTensor) -> DeviceTensor:
+        y = self.empty(x.shape, F32)
+        self._check(self._lib.omx_to_f32(self._ctx, self._p(x), self._p(y), C.c_uint64(x.numel)))
+        return y
+
+    # ---- matmul class ----
+    def linear_forward(self, x: DeviceTensor, w: DeviceTensor, out_dtype: Optional[int] = None) -> DeviceTensor:
+        rows = x.numel // x.shape[-1]
+        kin, nout = x.shape[-1], w.shape[0]
+        if w.shape[-1] != kin or len(w.shape) != 2:
+            raise OjasError(SHAPE, f"linear_forward: input {x.shape} weight {w.shape}")
+        od = F32 if out_dtype is None else out_dtype
+        y = self.empty(x.shape[:-1] + (nout,), od)
+        self._check(self._lib.omx_linear_forward(self._ctx, self._p(x), C.c_int32(x.dtype), self._p(w),
+                                                 C.c_int32(w.dtype), self._p(y), C.c_int32(od), C.c_uint64(rows),
+                                                 C.c_uint64(kin), C.c_uint64(nout)))
+        return y
+
+    def linear_backward(self, x, w, gy, gx_dtype=F32, need_gx=True, need_gw=True):
+        rows = x.numel // x.shape[-1]
+        kin, nout = x.shape[-1], w.shape[0]
+        if not (x.dtype == w.dtype == gy.dtype):
+            raise OjasError(DTYPE, "linear_backward: operands must share a dtype")
+        gx = self.empty(x.shape, gx_dtype) if need_gx else None
+        gw = self.empty(w.shape, F32) if need_gw else None
+        self._check(self._lib.omx_linear_backward(self._ctx, self._p(x), self._p(w), self._p(gy), C.c_int32(x.dtype),
+                                                  self._p(gx), C.c_int32(gx_dtype), self._p(gw), C.c_int32(F32),
+                                                  C.c_uint64(rows), C.c_uint64(kin), C.c_uint64(nout)))
+        return gx, gw
+
+    def linear_backward_input(self, w, gy, in_features=None, gx_dtype=F32):
+        rows = gy.numel // gy.shape[-1]
+        kin, nout = w.shape[1], w.shape[0]
+        gx = self.empty(gy.shape[:-1] + (kin,), gx_dtype)
+        self._check(self._lib.omx_linear_backward(self._ctx, None, self._p(w), self._p(gy), C.c_int32(w.dtype),
+                                                  self._p(gx), C.c_int32(gx_dtype), None, C.c_int32(F32),
+                                                  C.c_uint64(rows), C.c_uint64(kin), C.c_uint64(nout)))
+        return gx
+
+    def gemm(self, a: DeviceTensor, a_strides, b: DeviceTensor, b_strides, m, k, n, out_dtype=F32, c=None):
+        """C[m,n] (+)= A.B with element strides (a_rs, a_cs), (b_rs, b_cs)."""
+        acc = c is not None
+        out = c if acc else self.empty((m, n), out_dtype)
+        self._check(self._lib.omx_gemm(self._ctx, self._p(a), C.c_uint64(a_strides[0]), C.c_uint64(a_strides[1]),
+                                       self._p(b), C.c_uint64(b_strides[0]), C.c_uint64(b_strides[1]),
+                                       C.c_int32(a.dtype), self._p(out), C.c_int32(out.dtype), C.c_uint64(m),
+                                       C.c_uint64(k), C.c_uint64(n), C.c_int32(1 if acc else 0)))
+        return out
+
+    # ---- attention ----
+    def causal_sdpa_forward(self, q, k, v, window: Optional[int] = None, out_dtype: Optional[int] = None):
+        b, h, t, d = q.shape
+        hkv = k.shape[1]
+        if window == 0:
+            raise OjasError(SHAPE, "sdpa window must be at least 1")
+        od = F32 if out_dtype is None else out_dtype
+        out = self.empty(q.shape, od)
+        lse = self.empty((b, h, t), F32)
+        self._check(self._lib.omx_causal_sdpa_forward(self._ctx, self._p(q), self._p(k), self._p(v),
+                                                      C.c_int32(q.dtype), self._p(out), C.c_int32(od), self._p(lse),
+                                                      C.c_uint64(b), C.c_uint64(h), C.c_uint64(hkv), C.c_uint64(t),
+                                                      C.c_uint64(d), C.c_uint64(window or 0)))
+        return out, lse
+
+    def causal_sdpa_backward(self, q, k, v, out, lse, gy, window: Optional[int] = None, grad_dtype=F32):
+        b, h, t, d = q.shape
+        hkv = k.shape[1]
+        if window == 0:
+            raise OjasError(SHAPE, "sdpa window must be at least 1")
+        gq, gk, gv = self.empty(q.shape, grad_dtype), self.empty(k.shape, grad_dtype), self.empty(v.shape, grad_dtype)
+        self._check(self._lib.omx_causal_sdpa_backward(self._ctx, self._p(q), self._p(k), self._p(v), self._p(out),
+                                                       self._p(lse), self._p(gy), C.c_int32(q.dtype), self._p(gq),
+                                                       self._p(gk), self._p(gv), C.c_int32(grad_dtype), C.c_uint64(b),
+                                                       C.c_uint64(h), C.c_uint64(hkv), C.c_uint64(t), C.c_uint64(d),
+                                                       C.c_uint64(window or 0)))
+        return gq, gk, gv
+
+    # ---- norms ----
+    def rms_norm_forward(self, x, w, eps: float = 1e-6, out_dtype: Optional[int] = None):
+        dim = x.shape[-1]
+        rows = x.numel // dim
+        if w.shape != (dim,):
+            raise OjasError(SHAPE, f"rms_norm_forward: weight {w.shape} for dim {dim}")
+        od = x.dtype if out_dtype is None else out_dtype
+        y = self.empty(x.shape, od)
+        self._check(self._lib.omx_rms_norm_forward(self._ctx, self._p(x), C.c_int32(x.dtype), self._p(w), self._p(y),
+                                                   C.c_int32(od), C.c_uint64(rows), C.c_uint64(dim), C.c_float(eps)))
+        return y
+
+    def rms_norm_backward(self, x, w, gy, eps: float = 1e-6):
+        dim = x.shape[-1]
+        rows = x.numel // dim
+        gx = self.empty(x.shape, gy.dtype)
+        gw = self.empty((dim,), F32)
+        self._check(self._lib.omx_rms_norm_backward(self._ctx, self._p(x), C.c_int32(x.dtype), self._p(w),
+                                                    self._p(gy), C.c_int32(gy.dtype), self._p(gx),
+                                                    C.c_int32(gy.dtype), self._p(gw), C.c_uint64(rows),
+                                                    C.c_uint64(dim), C.c_float(eps)))
+        return gx, gw
+
+    # ---- loss ----
+    @staticmethod
+    def _ign(ignore_index):
+        return (C.c_int32(0), C.c_uint32(0)) if ignore_index is None else (C.c_int32(1), C.c_uint32(ignore_index))
+
+    def cross_entropy_mean_forward(self, logits, targets, ignore_index=None):
+        rows, vocab = logits.shape
+        loss = self.empty((1,), F32)
+        hi, iv = self._ign(ignore_index)
+        self._check(self._lib.omx_cross_entropy_mean_forward(self._ctx, self._p(logits), C.c_int32(logits.dtype),
+                                                             self._p(targets), C.c_uint64(rows), C.c_uint64(vocab),
+                                                             hi, iv, self._p(loss)))
+        return loss
+
+    def cross_entropy_mean_backward(self, logits, targets, ignore_index=None, grad_dtype=F32):
+        rows, vocab = logits.shape
+        grad = self.empty(logits.shape, grad_dtype)
+        hi, iv = self._ign(ignore_index)
+        self._check(self._lib.omx_cross_entropy_mean_backward(self._ctx, self._p(logits), C.c_int32(logits.dtype),
+                                                              self._p(targets), C.c_uint64(rows), C.c_uint64(vocab),
+                                                              hi, iv, self._p(grad), C.c_int32(grad_dtype)))
+        return grad
+
+    def linear_cross_entropy_mean(self, x, w, targets, ignore_index=None, chunk=(1024, 8192), grads=(True, True),
+                                  gx_dtype=F32):
+        """Returns (loss, grad_input | None, grad_weight | None); `chunk` is CeChunk(rows, cols)."""
+        rows, dim = x.shape
+        vocab = w.shape[0]
+        if x.dtype != w.dtype:
+            raise OjasError(DTYPE, "linear_cross_entropy_mean: operands must share a dtype")
+        loss = self.empty((1,), F32)
+        gx = self.empty(x.shape, gx_dtype) if grads[0] else None
+        gw = self.empty(w.shape, F32) if grads[1] else None
+        hi, iv = self._ign(ignore_index)
+        self._check(self._lib.omx_linear_cross_entropy_mean(
+            self._ctx, self._p(x), self._p(w), C.c_int32(x.dtype), self._p(targets), C.c_uint64(rows),
+            C.c_uint64(dim), C.c_uint64(vocab), hi, iv, C.c_uint64(chunk[0]), C.c_uint64(chunk[1]), self._p(loss),
+            self._p(gx), C.c_int32(gx_dtype), self._p(gw)))
+        return loss, gx, gw
+
+    # ---- embedding ----
+    def embedding_forward(self, table, ids, out_dtype: Optional[int] = None):
+        vocab, dim = table.shape
+        od = F32 if out_dtype is None else out_dtype
+        out = self.empty(ids.shape + (dim,), od)
+        self._check(self._lib.omx_embedding_forward(self._ctx, self._p(table), C.c_int32(table.dtype), self._p(ids),
+                                                    self._p(out), C.c_int32(od), C.c_uint64(ids.numel),
+                                                    C.c_uint64(vocab), C.c_uint64(dim)))
+        return out
+
+    def embedding_backward(self, ids, grad, vocab: int):
+        dim = grad.shape[-1]
+        out = self.empty((vocab, dim), F32)
+        self._check(self._lib.omx_embedding_backward(self._ctx, self._p(ids), self._p(grad), C.c_int32(grad.dtype),
+                                                     self._p(out), C.c_uint64(ids.numel), C.c_uint64(vocab),
+                                                     C.c_uint64(dim)))
+        return out
+
+    # ---- optimizers (in place) ----
+    def adamw_step(self, param, grad, moment1, moment2, step: int, config: AdamWConfig, param_bf16=None):
+        self._check(self._lib.omx_adamw_step(self._ctx, self._p(param), self._p(grad), self._p(moment1),
+                                             self._p(moment2), C.c_uint64(param.numel), C.c_uint64(step),
+                                             C.byref(config), self._p(param_bf16)))
+
+    def muon_ns5_step(self, param, grad, momentum, config: MuonNs5Config, param_bf16=None):
+        rows, cols = param.shape
+        self._check(self._lib.omx_muon_ns5_step(self._ctx, self._p(param), self._p(grad), self._p(momentum),
+                                                C.c_uint64(rows), C.c_uint64(cols), C.byref(config),
+                                                self._p(param_bf16)))
+
+    def clip_grad_norm(self, grads: Sequence[DeviceTensor], max_norm: float) -> float:
+        n = len(grads)
+        ptrs = (C.c_void_p * max(n, 1))(*[g.ptr for g in grads])
+        lens = (C.c_uint64 * max(n, 1))(*[g.numel for g in grads])
+        norm = C.c_float()
+        self._check(self._lib.omx_clip_grad_norm(self._ctx, ptrs, lens, C.c_uint64(n), C.c_float(max_norm),
+                                                 C.byref(norm)))
+        return float(norm.value)
+
+    # ---- elementwise / layout ----
+    def residual_add_forward(self, x, y):
+        if x.dtype != y.dtype or x.shape != y.shape:
+            raise OjasError(SHAPE, "residual_add_forward: operands differ")
+        out = self.empty(x.shape, x.dtype)
+        self._check(self._lib.omx_residual_add(self._ctx, self._p(x), self._p(y), self._p(out), C.c_int32(x.dtype),
+                                               C.c_uint64(x.numel)))
+        return out
+
+    def accumulate_grad(self, acc, grad):
+        self._check(self._lib.omx_accumulate_grad(self._ctx, self._p(acc), self._p(grad), C.c_uint64(acc.numel)))
+
+    def scale_grad(self, grad, scale: float):
+        self._check(self._lib.omx_scale_grad(self._ctx, self._p(grad), C.c_float(scale), C.c_uint64(grad.numel)))
+
+    def _gelu(self, x, tanh_form):
+        y = self.empty(x.shape, x.dtype)
+        self._check(self._lib.omx_gelu_forward(self._ctx, self._p(x), self._p(y), C.c_int32(x.dtype),
+                                               C.c_uint64(x.numel), C.c_int32(tanh_form)))
+        return y
+
+    def _gelu_bwd(self, x, gy, tanh_form):
+        gx = self.empty(x.shape, x.dtype)
+        self._check(self._lib.omx_gelu_backward(self._ctx, self._p(x), self._p(gy), self._p(gx), C.c_int32(x.dtype),
+                                                C.c_uint64(x.numel), C.c_int32(tanh_form)))
+        return gx
+
+    def gelu_erf_forward(self, x):
+        return self._gelu(x, 0)
+
+    def gelu_erf_backward(self, x, gy):
+        return self._gelu_bwd(x, gy, 0)
+
+    def gelu_tanh_forward(self, x):
+        return self._gelu(x, 1)
+
+    def gelu_tanh_backward(self, x, gy):
+        return self._gelu_bwd(x, gy, 1)
+
+    def permute(self, x, axes):
+        if list(axes) != [0, 2, 1, 3] or len(x.shape) != 4:
+            raise OjasError(UNSUPPORTED, "permute: only axes [0,2,1,3] of a rank-4 tensor")
+        d0, d1, d2, d3 = x.shape
+        y = self.empty((d0, d2, d1, d3), x.dtype)
+        self._check(self._lib.omx_permute_0213(self._ctx, self._p(x), self._p(y), C.c_int32(x.dtype), C.c_uint64(d0),
+                                               C.c_uint64(d1), C.c_uint64(d2), C.c_uint64(d3)))
+        return y
+
+    # ---- integer ops ----
+    def argmax_rows(self, x):
+        rows, cols = x.shape
+        out = self.empty((rows,), U32)
+        self._check(self._lib.omx_argmax_rows(self._ctx, self._p(x), C.c_uint64(rows), C.c_uint64(cols), self._p(out)))
+        return out
+
+    def topk_rows(self, x, k: int):
+        rows, cols = x.shape
+        vals, ids = self.empty((rows, k), F32), self.empty((rows, k), U32)
+        self._check(self._lib.omx_topk_rows(self._ctx, self._p(x), C.c_uint64(rows), C.c_uint64(cols), C.c_uint64(k),
+                                            self._p(vals), self._p(ids)))
+        return vals, ids
+
+    def __getattr__(self, name):
+        # Every other Backend method refuses by name (unsupported_op, backend.rs:792-797).
+        if name.startswith("_"):
+            raise AttributeError(name)
+
+        def refuse(*_a, **_k):
+            self._lib.omx_unsupported(self._ctx, name.encode())
+            raise OjasError(UNSUPPORTED, name)
+
+        return refuse

@@ -1,0 +1,377 @@
+// MFMA GEMM for gfx950: C[M,N] (+)= A[M,K] . B[K,N], f32 accumulation.
+//
+// Serves BackendModule::linear_forward / linear_backward / linear_backward_input
+// (ojas-core/src/backend.rs:1628-1656; CPU reference ojas-cpu/src/linalg.rs:69-210)
+// and the Newton-Schulz products of muon_ns5_step (ojas-cpu/src/optim.rs:841-985).
+//
+// Two lanes share one kernel template:
+//   bf16 storage -> v_mfma_f32_32x32x16_bf16 (8 k-values per lane per issue)
+//   f32 storage  -> v_mfma_f32_32x32x2_f32   (1 k-value per lane per issue)
+// Each product of two bf16 values is exact in f32, so the bf16 lane differs
+// from the CPU Exact chain only in summation order (the Fast contract).
+//
+// Tiling: 128x128 output tile per 256-thread workgroup (4 waves, 2x2, each a
+// 64x64 wave tile = 2x2 MFMA 32x32 blocks), K step of eight 16-byte chunks
+// (64 bf16 / 32 f32), LDS double-buffered with the next K step prefetched into
+// registers while the current one is multiplied. LDS rows are [row][k] with a
+// 16-byte pad (144-byte pitch) so the 16-byte fragment reads of 32 lanes hit
+// distinct banks. An operand whose K index is the slow one in memory
+// ("k-major": gy and x in the weight gradient, W in the input gradient) is
+// loaded with coalesced 16-byte reads along its fast index and transposed in
+// registers on the way into LDS, so the fragment reads are the same for every
+// operand layout.
+#include "omx_common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
+namespace {
+
+constexpr int BM = 128, BN = 128, NT = 256;
+constexpr int PITCH = 144;               // bytes per LDS row: 8 chunks of 16 B + pad
+constexpr int TILE_BYTES = 128 * PITCH;  // one operand tile
+
+struct GemmArgs {
+  const void* a;
+  const void* b;
+  void* c;
+  long lda, ldb, ldc;
+  int M, N, K;
+  int c_bf16, accumulate;
+  int a_vec, b_vec;  // 16-byte loads allowed (alignment of base and leading dimension)
+  int tiles_m, tiles_n;
+  OmxFaultWord* fault;
+  unsigned long long tag;
+};
+
+template <typename T>
+union Chunk {
+  u32x4 v;
+  T e[16 / sizeof(T)];
+};
+
+// Operand stored with K contiguous: element (row, k) at p[row * ld + k].
+// Each thread moves four 16-byte chunks of the 128 x (8 chunk) tile.
+template <typename T>
+__device__ __forceinline__ void load_kcontig(const T* __restrict__ p, long ld, int row0, int rows, int k0, int K,
+                                             bool vec, u32x4 regs[4]) {
+  constexpr int KV = 16 / sizeof(T);
+  const int tid = threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int c = tid + NT * i;
+    int row = c >> 3, kc = c & 7;
+    int gr = row0 + row, gk = k0 + kc * KV;
+    Chunk<T> ch;
+    ch.v = u32x4{0u, 0u, 0u, 0u};
+    if (gr < rows && gk < K) {
+      const T* src = p + static_cast<long>(gr) * ld + gk;
+      if (vec && gk + KV <= K) {
+        ch.v = *reinterpret_cast<const u32x4*>(src);
+      } else {
+#pragma unroll
+        for (int e = 0; e < KV; ++e)
+          if (gk + e < K) ch.e[e] = src[e];
+      }
+    }
+    regs[i] = ch.v;
+  }
+}
+template <typename T>
+__device__ __forceinline__ void store_kcontig(char* lds, const u32x4 regs[4]) {
+  const int tid = threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int c = tid + NT * i;
+    int row = c >> 3, kc = c & 7;
+    *reinterpret_cast<u32x4*>(lds + row * PITCH + kc * 16) = regs[i];
+  }
+}
+
+// Operand stored with K as the slow index: element (row, k) at p[k * ld + row].
+// Each thread loads a 4 (k) x KV (row) block with four 16-byte reads along the
+// row index and stores it transposed: KV LDS writes of four k-values each.
+template <typename T>
+__device__ __forceinline__ void load_kmajor(const T* __restrict__ p, long ld, int row0, int rows, int k0, int K,
+                                            bool vec, u32x4 regs[4]) {
+  constexpr int KV = 16 / sizeof(T);
+  constexpr int MPB = 128 / KV;
+  const int tid = threadIdx.x;
+  const int mb = tid % MPB, kb = tid / MPB;
+  const int gr = row0 + mb * KV;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    int gk = k0 + kb * 4 + r;
+    Chunk<T> ch;
+    ch.v = u32x4{0u, 0u, 0u, 0u};
+    if (gk < K && gr < rows) {
+      const T* src = p + static_cast<long>(gk) * ld + gr;
+      if (vec && gr + KV <= rows) {
+        ch.v = *reinterpret_cast<const u32x4*>(src);
+      } else {
+#pragma unroll
+        for (int e = 0; e < KV; ++e)
+          if (gr + e < rows) ch.e[e] = src[e];
+      }
+    }
+    regs[r] = ch.v;
+  }
+}
+template <typename T>
+__device__ __forceinline__ void store_kmajor(char* lds, const u32x4 regs[4]) {
+  constexpr int KV = 16 / sizeof(T);
+  constexpr int MPB = 128 / KV;
+  const int tid = threadIdx.x;
+  const int mb = tid % MPB, kb = tid / MPB;
+  Chunk<T> in[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) in[r].v = regs[r];
+#pragma unroll
+  for (int mi = 0; mi < KV; ++mi) {
+    T out[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) out[r] = in[r].e[mi];
+    char* dst = lds + (mb * KV + mi) * PITCH + kb * 4 * static_cast<int>(sizeof(T));
+    if constexpr (sizeof(T) == 2) {
+      u32x2 w;
+      w.x = static_cast<unsigned int>(out[0]) | (static_cast<unsigned int>(out[1]) << 16);
+      w.y = static_cast<unsigned int>(out[2]) | (static_cast<unsigned int>(out[3]) << 16);
+      *reinterpret_cast<u32x2*>(dst) = w;
+    } else {
+      u32x4 w;
+      w.x = __float_as_uint(out[0]);
+      w.y = __float_as_uint(out[1]);
+      w.z = __float_as_uint(out[2]);
+      w.w = __float_as_uint(out[3]);
+      *reinterpret_cast<u32x4*>(dst) = w;
+    }
+  }
+}
+
+template <typename T>
+__device__ __forceinline__ void mma_step(const u32x4& af, const u32x4& bf, floatx16& acc) {
+  if constexpr (sizeof(T) == 2) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af), __builtin_bit_cast(bf16x8, bf),
+                                                  acc, 0, 0, 0);
+  } else {
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(af.x), __uint_as_float(bf.x), acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(af.y), __uint_as_float(bf.y), acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(af.z), __uint_as_float(bf.z), acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(af.w), __uint_as_float(bf.w), acc, 0, 0, 0);
+  }
+}
+
+template <typename T, bool A_KM, bool B_KM>
+__global__ __launch_bounds__(NT) void gemm_kernel(GemmArgs g) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  constexpr int KV = 16 / sizeof(T);
+  constexpr int BK = 8 * KV;
+  const T* __restrict__ A = static_cast<const T*>(g.a);
+  const T* __restrict__ B = static_cast<const T*>(g.b);
+
+  // Workgroups are dealt round-robin to the 8 XCDs; give each XCD one
+  // contiguous run of tiles so neighbours share operand rows in its L2.
+  const int total = g.tiles_m * g.tiles_n;
+  int id = blockIdx.x;
+  {
+    const int per = (total + 7) / 8;
+    int xcd = id & 7, local = id >> 3;
+    int mapped = xcd * per + local;
+    // The last XCD's run may be short; ids that fall off the end wrap into
+    // the gaps (a bijection when total is a multiple of 8, otherwise fall
+    // back to the identity order).
+    id = (total % 8 == 0) ? mapped : id;
+  }
+  // Within the run: walk N fastest inside bands of 8 tile rows.
+  const int band = 8;
+  int tiles_per_band = band * g.tiles_n;
+  int band_id = id / tiles_per_band;
+  int first_m = band_id * band;
+  int band_rows = min(band, g.tiles_m - first_m);
+  int in_band = id - band_id * tiles_per_band;
+  const int tile_m = first_m + in_band % band_rows;
+  const int tile_n = in_band / band_rows;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int l32 = lane & 31, lg = lane >> 5;
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  u32x4 ra[4], rb[4];
+  const int ksteps = (g.K + BK - 1) / BK;
+  auto load_tiles = [&](int ks) {
+    int k0 = ks * BK;
+    if constexpr (A_KM) load_kmajor<T>(A, g.lda, m0, g.M, k0, g.K, g.a_vec, ra);
+    else load_kcontig<T>(A, g.lda, m0, g.M, k0, g.K, g.a_vec, ra);
+    if constexpr (B_KM) load_kmajor<T>(B, g.ldb, n0, g.N, k0, g.K, g.b_vec, rb);
+    else load_kcontig<T>(B, g.ldb, n0, g.N, k0, g.K, g.b_vec, rb);
+  };
+  auto store_tiles = [&](int buf) {
+    char* la = smem + buf * 2 * TILE_BYTES;
+    char* lb = la + TILE_BYTES;
+    if constexpr (A_KM) store_kmajor<T>(la, ra);
+    else store_kcontig<T>(la, ra);
+    if constexpr (B_KM) store_kmajor<T>(lb, rb);
+    else store_kcontig<T>(lb, rb);
+  };
+
+  load_tiles(0);
+  store_tiles(0);
+  __syncthreads();
+  for (int ks = 0; ks < ksteps; ++ks) {
+    const int buf = ks & 1;
+    if (ks + 1 < ksteps) load_tiles(ks + 1);
+    const char* la = smem + buf * 2 * TILE_BYTES + (wm * 64 + l32) * PITCH + lg * 16;
+    const char* lb = smem + buf * 2 * TILE_BYTES + TILE_BYTES + (wn * 64 + l32) * PITCH + lg * 16;
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      u32x4 af[2], bf[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        af[t] = *reinterpret_cast<const u32x4*>(la + t * 32 * PITCH + kk * 32);
+        bf[t] = *reinterpret_cast<const u32x4*>(lb + t * 32 * PITCH + kk * 32);
+      }
+#pragma unroll
+      for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < 2; ++tn) mma_step<T>(af[tm], bf[tn], acc[tm][tn]);
+    }
+    if (ks + 1 < ksteps) store_tiles(buf ^ 1);
+    __syncthreads();
+  }
+
+  // Epilogue. Accumulator register v of a 32x32 block holds
+  // row 8*(v/4) + 4*(lane/32) + v%4, column lane%32.
+  bool bad = false;
+#pragma unroll
+  for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+    for (int tn = 0; tn < 2; ++tn) {
+      int col = n0 + wn * 64 + tn * 32 + l32;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        int row = m0 + wm * 64 + tm * 32 + 8 * (v >> 2) + 4 * lg + (v & 3);
+        if (row < g.M && col < g.N) {
+          float val = acc[tm][tn][v];
+          long off = static_cast<long>(row) * g.ldc + col;
+          if (g.c_bf16) {
+            static_cast<unsigned short*>(g.c)[off] = dev_f32_to_bf16_bits(val);
+          } else {
+            float* cp = static_cast<float*>(g.c) + off;
+            if (g.accumulate) val += *cp;
+            *cp = val;
+          }
+          bad |= !dev_finite(val);
+        }
+      }
+    }
+  if (bad) dev_raise_fault(g.fault, g.tag);
+}
+
+template <typename T>
+int32_t launch(omx_ctx* ctx, GemmArgs& g, bool a_km, bool b_km) {
+  int total = g.tiles_m * g.tiles_n;
+  size_t smem = 4 * TILE_BYTES;
+  dim3 grid(total), block(NT);
+  // More than 64 KiB of dynamic LDS has to be granted per kernel, once.
+  static bool granted = false;
+  if (!granted) {
+    OMX_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<T, false, false>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)));
+    OMX_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<T, false, true>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)));
+    OMX_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<T, true, false>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)));
+    OMX_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<T, true, true>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)));
+    granted = true;
+  }
+  if (!a_km && !b_km) hipLaunchKernelGGL((gemm_kernel<T, false, false>), grid, block, smem, ctx->stream, g);
+  else if (!a_km && b_km) hipLaunchKernelGGL((gemm_kernel<T, false, true>), grid, block, smem, ctx->stream, g);
+  else if (a_km && !b_km) hipLaunchKernelGGL((gemm_kernel<T, true, false>), grid, block, smem, ctx->stream, g);
+  else hipLaunchKernelGGL((gemm_kernel<T, true, true>), grid, block, smem, ctx->stream, g);
+  OMX_LAUNCH_CHECK(ctx, "gemm_kernel");
+  return OMX_OK;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace
+
+// Internal entry shared by the linear ops, the fused loss and Muon.
+int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a_rs, uint64_t a_cs, const void* b,
+                      uint64_t b_rs, uint64_t b_cs, int32_t operand_dtype, void* c, int32_t c_dtype, uint64_t ldc,
+                      uint64_t m, uint64_t k, uint64_t n, int32_t accumulate) {
+  const char* op = omx_fault_name(fault_op);
+  if (!a || !b || !c) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  if (!omx_valid_float_dtype(operand_dtype) || !omx_valid_float_dtype(c_dtype))
+    return omx_fail(ctx, OMX_DTYPE, "%s: operands must be f32 or bf16", op);
+  if (m == 0 || n == 0 || k == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
+  if (m > 0x7fffffffull || n > 0x7fffffffull || k > 0x7fffffffull)
+    return omx_fail(ctx, OMX_OUT_OF_RANGE, "%s: axis does not fit in i32", op);
+  if (accumulate && c_dtype != OMX_F32) return omx_fail(ctx, OMX_DTYPE, "%s: accumulation needs an f32 output", op);
+  bool a_km, b_km;
+  long lda, ldb;
+  if (a_cs == 1) {
+    a_km = false;
+    lda = static_cast<long>(a_rs);
+  } else if (a_rs == 1) {
+    a_km = true;
+    lda = static_cast<long>(a_cs);
+  } else {
+    return omx_fail(ctx, OMX_SHAPE, "%s: operand A has no unit stride", op);
+  }
+  if (b_rs == 1) {
+    b_km = false;
+    ldb = static_cast<long>(b_cs);
+  } else if (b_cs == 1) {
+    b_km = true;
+    ldb = static_cast<long>(b_rs);
+  } else {
+    return omx_fail(ctx, OMX_SHAPE, "%s: operand B has no unit stride", op);
+  }
+  const long kv = operand_dtype == OMX_BF16 ? 8 : 4;
+  GemmArgs g;
+  g.a = a;
+  g.b = b;
+  g.c = c;
+  g.lda = lda;
+  g.ldb = ldb;
+  g.ldc = static_cast<long>(ldc);
+  g.M = static_cast<int>(m);
+  g.N = static_cast<int>(n);
+  g.K = static_cast<int>(k);
+  g.c_bf16 = c_dtype == OMX_BF16;
+  g.accumulate = accumulate;
+  g.a_vec = aligned16(a) && (lda % kv == 0);
+  g.b_vec = aligned16(b) && (ldb % kv == 0);
+  g.tiles_m = (g.M + BM - 1) / BM;
+  g.tiles_n = (g.N + BN - 1) / BN;
+  if (static_cast<long>(g.tiles_m) * g.tiles_n > 0x7fffffffl)
+    return omx_fail(ctx, OMX_OUT_OF_RANGE, "%s: too many output tiles", op);
+  g.fault = ctx->fault;
+  g.tag = omx_tag(ctx, fault_op);
+  if (operand_dtype == OMX_BF16) return launch<unsigned short>(ctx, g, a_km, b_km);
+  return launch<float>(ctx, g, a_km, b_km);
+}
+
+extern "C" {
+
+int32_t omx_gemm(omx_ctx* ctx, const void* a, uint64_t a_rs, uint64_t a_cs, const void* b, uint64_t b_rs,
+                 uint64_t b_cs, int32_t operand_dtype, void* c, int32_t c_dtype, uint64_t m, uint64_t k,
+                 uint64_t n, int32_t accumulate) {
+  OMX_REQUIRE_CTX(ctx);
+  return omx_gemm_impl(ctx, F_GEMM, a, a_rs, a_cs, b, b_rs, b_cs, operand_dtype, c, c_dtype, n, m, k, n, accumulate);
+}
+
+}  // extern "C"

@@ -1,0 +1,390 @@
+// Softmax cross-entropy: plain (logits in HBM) and fused with the LM head.
+//
+// Reference semantics:
+//   cross_entropy_mean_forward/backward  ojas-cpu/src/pointwise.rs:2172-2438
+//                                        (trait ojas-core/src/backend.rs:2451-2466)
+//   linear_cross_entropy_mean            ojas-cpu/src/fused_ce.rs:97-158,290-452
+//                                        (trait backend.rs:2493-2524, CeChunk :3081)
+//
+// Per row: loss = max + ln(sum e^(x - max)) - x_t, grad = (softmax - onehot) / valid,
+// ignored rows contribute nothing, an all-ignored batch is NonFinite. The
+// collapse rule (pointwise.rs:2305-2325) is kept: when the target holds the
+// whole mass (x_t == max and the sum rounds to 1), S = sum_{j != t} e^(x_j - x_t)
+// is used instead: loss = log1p(S), grad = e / (1 + S) / valid, target -S / (1 + S) / valid.
+//
+// The row statistics are carried as (max, sum without the target, target
+// logit) so they can be updated one vocabulary tile at a time (online
+// softmax); the fused op therefore never holds more than one
+// chunk_rows x chunk_cols tile of logits.
+#include "omx_common.h"
+
+namespace {
+
+constexpr int CE_THREADS = 256;
+
+struct CeState {
+  float* max;    // running row maximum
+  float* other;  // sum of e^(x - max) over columns other than the target
+  float* picked; // target logit
+};
+
+__device__ __forceinline__ float block_max(float v, float* red) {
+  v = wave_max(v);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  return fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+}
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  return ((red[0] + red[1]) + red[2]) + red[3];
+}
+
+__global__ void ce_count_valid_kernel(const unsigned int* __restrict__ targets, size_t rows, size_t vocab,
+                                      int has_ignore, unsigned int ignore, unsigned int* __restrict__ valid,
+                                      OmxFaultWord* fault, unsigned long long tag) {
+  size_t n = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  bool counts = false;
+  if (n < rows) {
+    unsigned int t = targets[n];
+    if (!(has_ignore && t == ignore)) {
+      if (t >= vocab) dev_raise_range(fault, tag);
+      else counts = true;
+    }
+  }
+  unsigned long long ballot = __ballot(counts);
+  if ((threadIdx.x & 63) == 0 && ballot) atomicAdd(valid, static_cast<unsigned int>(__popcll(ballot)));
+}
+
+// One block per row. Folds the tile's columns [col0, col0 + ncols) into the
+// row's running (max, other, picked). `first` starts the state.
+template <typename T>
+__global__ __launch_bounds__(CE_THREADS) void ce_tile_stats_kernel(const T* __restrict__ tile, size_t ld,
+                                                                   size_t row0, unsigned int col0,
+                                                                   unsigned int ncols,
+                                                                   const unsigned int* __restrict__ targets,
+                                                                   CeState st, int first, OmxFaultWord* fault,
+                                                                   unsigned long long tag) {
+  __shared__ float red[4];
+  const size_t local = blockIdx.x, row = row0 + local;
+  const T* r = tile + local * ld;
+  const unsigned int target = targets[row];
+  float mx = -INFINITY;
+  bool bad = false;
+  for (unsigned int c = threadIdx.x; c < ncols; c += CE_THREADS) {
+    float v = dev_load<T>(r, c);
+    bad |= !dev_finite(v);
+    mx = fmaxf(mx, v);
+  }
+  mx = block_max(mx, red);
+  float old_max = first ? -INFINITY : st.max[row];
+  float new_max = fmaxf(old_max, mx);
+  float sum = 0.0f;
+  for (unsigned int c = threadIdx.x; c < ncols; c += CE_THREADS) {
+    if (col0 + c != target) sum += expf(dev_load<T>(r, c) - new_max);
+  }
+  sum = block_sum(sum, red);
+  if (__syncthreads_or(bad)) {
+    if (threadIdx.x == 0) dev_raise_fault(fault, tag);
+  }
+  if (threadIdx.x == 0) {
+    float other = first ? 0.0f : st.other[row] * expf(old_max - new_max);
+    st.max[row] = new_max;
+    st.other[row] = other + sum;
+    if (target >= col0 && target < col0 + ncols) st.picked[row] = dev_load<T>(r, target - col0);
+  }
+}
+
+// Single block: per-row losses from the final state, summed in a fixed tree
+// order, divided by the valid count.
+__global__ __launch_bounds__(1024) void ce_mean_kernel(CeState st, const unsigned int* __restrict__ targets,
+                                                       size_t rows, int has_ignore, unsigned int ignore,
+                                                       const unsigned int* __restrict__ valid,
+                                                       float* __restrict__ loss, OmxFaultWord* fault,
+                                                       unsigned long long tag) {
+  __shared__ float red[1024];
+  float acc = 0.0f;
+  for (size_t n = threadIdx.x; n < rows; n += 1024) {
+    unsigned int t = targets[n];
+    if (has_ignore && t == ignore) continue;
+    float m = st.max[n], other = st.other[n], p = st.picked[n];
+    float sum = other + expf(p - m);
+    float term;
+    if (p == m && sum == 1.0f && other > 0.0f) term = log1pf(other);
+    else term = m + logf(sum) - p;
+    acc += term;
+  }
+  red[threadIdx.x] = acc;
+  __syncthreads();
+  for (int s = 512; s > 0; s >>= 1) {
+    if (threadIdx.x < s) red[threadIdx.x] += red[threadIdx.x + s];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    unsigned int v = *valid;
+    float l = red[0] / static_cast<float>(v);
+    *loss = l;
+    // An all-ignored batch divides by zero: NonFinite, as on the CPU.
+    if (v == 0 || !dev_finite(l)) dev_raise_fault(fault, tag);
+  }
+}
+
+// One block per row: tile of logits -> tile of gradients (may be in place).
+template <typename TL, typename TG>
+__global__ __launch_bounds__(CE_THREADS) void ce_tile_grad_kernel(const TL* __restrict__ tile, TG* __restrict__ grad,
+                                                                  size_t ld, size_t ld_grad, size_t row0,
+                                                                  unsigned int col0, unsigned int ncols,
+                                                                  const unsigned int* __restrict__ targets,
+                                                                  int has_ignore, unsigned int ignore, CeState st,
+                                                                  const unsigned int* __restrict__ valid) {
+  const size_t local = blockIdx.x, row = row0 + local;
+  const TL* r = tile + local * ld;
+  TG* g = grad + local * ld_grad;
+  const unsigned int target = targets[row];
+  if (has_ignore && target == ignore) {
+    for (unsigned int c = threadIdx.x; c < ncols; c += CE_THREADS) dev_store<TG>(g, c, 0.0f);
+    return;
+  }
+  const float m = st.max[row], other = st.other[row], p = st.picked[row];
+  const float denom = static_cast<float>(*valid);
+  const float sum = other + expf(p - m);
+  const bool collapse = (p == m && sum == 1.0f && other > 0.0f);
+  const float d = collapse ? 1.0f + other : sum;
+  const float target_grad = collapse ? -(other / d) / denom : (expf(p - m) / d) / denom - 1.0f / denom;
+  for (unsigned int c = threadIdx.x; c < ncols; c += CE_THREADS) {
+    float v = (col0 + c == target) ? target_grad : (expf(dev_load<TL>(r, c) - m) / d) / denom;
+    dev_store<TG>(g, c, v);
+  }
+}
+
+template <typename T>
+void launch_stats(omx_ctx* ctx, const void* tile, size_t ld, size_t row0, size_t nrows, unsigned int col0,
+                  unsigned int ncols, const unsigned int* targets, CeState st, int first, unsigned long long tag) {
+  hipLaunchKernelGGL((ce_tile_stats_kernel<T>), dim3(static_cast<unsigned>(nrows)), dim3(CE_THREADS), 0, ctx->stream,
+                     static_cast<const T*>(tile), ld, row0, col0, ncols, targets, st, first, ctx->fault, tag);
+}
+template <typename TL, typename TG>
+void launch_grad(omx_ctx* ctx, const void* tile, void* grad, size_t ld, size_t ld_grad, size_t row0, size_t nrows,
+                 unsigned int col0, unsigned int ncols, const unsigned int* targets, int has_ignore,
+                 unsigned int ignore, CeState st, const unsigned int* valid) {
+  hipLaunchKernelGGL((ce_tile_grad_kernel<TL, TG>), dim3(static_cast<unsigned>(nrows)), dim3(CE_THREADS), 0,
+                     ctx->stream, static_cast<const TL*>(tile), static_cast<TG*>(grad), ld, ld_grad, row0, col0, ncols,
+                     targets, has_ignore, ignore, st, valid);
+}
+
+// State + valid counter carved out of a workspace block.
+struct CeScratch {
+  CeState st;
+  unsigned int* valid;
+};
+inline size_t ce_scratch_bytes(uint64_t rows) { return (3 * rows + 4) * sizeof(float); }
+inline CeScratch carve(void* base, uint64_t rows) {
+  float* f = static_cast<float*>(base);
+  CeScratch s;
+  s.st.max = f;
+  s.st.other = f + rows;
+  s.st.picked = f + 2 * rows;
+  s.valid = reinterpret_cast<unsigned int*>(f + 3 * rows);
+  return s;
+}
+
+int32_t count_valid(omx_ctx* ctx, const unsigned int* targets, uint64_t rows, uint64_t vocab, int has_ignore,
+                    unsigned int ignore, unsigned int* valid, unsigned long long tag) {
+  int32_t rc = omx_fill_zero(ctx, valid, 4);
+  if (rc != OMX_OK) return rc;
+  hipLaunchKernelGGL(ce_count_valid_kernel, dim3(static_cast<unsigned>((rows + 255) / 256)), dim3(256), 0,
+                     ctx->stream, targets, rows, vocab, has_ignore, ignore, valid, ctx->fault, tag);
+  OMX_LAUNCH_CHECK(ctx, "ce_count_valid_kernel");
+  return OMX_OK;
+}
+
+int32_t check_ce_args(omx_ctx* ctx, const char* op, const void* logits, const void* targets, uint64_t rows,
+                      uint64_t vocab, int32_t dtype) {
+  if (!logits || !targets) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  if (!omx_valid_float_dtype(dtype)) return omx_fail(ctx, OMX_DTYPE, "%s: logits must be f32 or bf16", op);
+  if (rows == 0 || vocab == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
+  if (vocab > 0xfffffffeull || rows > 0x7fffffffull)
+    return omx_fail(ctx, OMX_OUT_OF_RANGE, "%s: axis does not fit in u32", op);
+  return OMX_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t omx_cross_entropy_mean_forward(omx_ctx* ctx, const void* logits, int32_t logits_dtype, const void* targets,
+                                       uint64_t rows, uint64_t vocab, int32_t has_ignore, uint32_t ignore_index,
+                                       void* loss) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "cross_entropy_mean_forward";
+  int32_t rc = check_ce_args(ctx, op, logits, targets, rows, vocab, logits_dtype);
+  if (rc != OMX_OK) return rc;
+  if (!loss) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  void* ws = nullptr;
+  rc = omx_workspace(ctx, ce_scratch_bytes(rows), &ws);
+  if (rc != OMX_OK) return rc;
+  CeScratch s = carve(ws, rows);
+  const unsigned int* tg = static_cast<const unsigned int*>(targets);
+  unsigned long long tag = omx_tag(ctx, F_CE_FORWARD);
+  rc = count_valid(ctx, tg, rows, vocab, has_ignore, ignore_index, s.valid, tag);
+  if (rc != OMX_OK) return rc;
+  if (logits_dtype == OMX_F32) launch_stats<float>(ctx, logits, vocab, 0, rows, 0, vocab, tg, s.st, 1, tag);
+  else launch_stats<unsigned short>(ctx, logits, vocab, 0, rows, 0, vocab, tg, s.st, 1, tag);
+  OMX_LAUNCH_CHECK(ctx, "ce_tile_stats_kernel");
+  hipLaunchKernelGGL(ce_mean_kernel, dim3(1), dim3(1024), 0, ctx->stream, s.st, tg, rows, has_ignore, ignore_index,
+                     s.valid, static_cast<float*>(loss), ctx->fault, tag);
+  OMX_LAUNCH_CHECK(ctx, "ce_mean_kernel");
+  return OMX_OK;
+}
+
+int32_t omx_cross_entropy_mean_backward(omx_ctx* ctx, const void* logits, int32_t logits_dtype, const void* targets,
+                                        uint64_t rows, uint64_t vocab, int32_t has_ignore, uint32_t ignore_index,
+                                        void* grad, int32_t grad_dtype) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "cross_entropy_mean_backward";
+  int32_t rc = check_ce_args(ctx, op, logits, targets, rows, vocab, logits_dtype);
+  if (rc != OMX_OK) return rc;
+  if (!grad) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  if (!omx_valid_float_dtype(grad_dtype)) return omx_fail(ctx, OMX_DTYPE, "%s: grad must be f32 or bf16", op);
+  void* ws = nullptr;
+  rc = omx_workspace(ctx, ce_scratch_bytes(rows) + 16, &ws);
+  if (rc != OMX_OK) return rc;
+  CeScratch s = carve(ws, rows);
+  float* loss_scratch = reinterpret_cast<float*>(s.valid + 2);
+  const unsigned int* tg = static_cast<const unsigned int*>(targets);
+  unsigned long long tag = omx_tag(ctx, F_CE_BACKWARD);
+  rc = count_valid(ctx, tg, rows, vocab, has_ignore, ignore_index, s.valid, tag);
+  if (rc != OMX_OK) return rc;
+  if (logits_dtype == OMX_F32) launch_stats<float>(ctx, logits, vocab, 0, rows, 0, vocab, tg, s.st, 1, tag);
+  else launch_stats<unsigned short>(ctx, logits, vocab, 0, rows, 0, vocab, tg, s.st, 1, tag);
+  OMX_LAUNCH_CHECK(ctx, "ce_tile_stats_kernel");
+  // The mean kernel also raises the all-ignored fault, as the forward does.
+  hipLaunchKernelGGL(ce_mean_kernel, dim3(1), dim3(1024), 0, ctx->stream, s.st, tg, rows, has_ignore, ignore_index,
+                     s.valid, loss_scratch, ctx->fault, tag);
+  OMX_LAUNCH_CHECK(ctx, "ce_mean_kernel");
+  if (logits_dtype == OMX_F32 && grad_dtype == OMX_F32)
+    launch_grad<float, float>(ctx, logits, grad, vocab, vocab, 0, rows, 0, vocab, tg, has_ignore, ignore_index, s.st,
+                              s.valid);
+  else if (logits_dtype == OMX_F32)
+    launch_grad<float, unsigned short>(ctx, logits, grad, vocab, vocab, 0, rows, 0, vocab, tg, has_ignore,
+                                       ignore_index, s.st, s.valid);
+  else if (grad_dtype == OMX_F32)
+    launch_grad<unsigned short, float>(ctx, logits, grad, vocab, vocab, 0, rows, 0, vocab, tg, has_ignore,
+                                       ignore_index, s.st, s.valid);
+  else
+    launch_grad<unsigned short, unsigned short>(ctx, logits, grad, vocab, vocab, 0, rows, 0, vocab, tg, has_ignore,
+                                                ignore_index, s.st, s.valid);
+  OMX_LAUNCH_CHECK(ctx, "ce_tile_grad_kernel");
+  return OMX_OK;
+}
+
+int32_t omx_linear_cross_entropy_mean(omx_ctx* ctx, const void* x, const void* w, int32_t operand_dtype,
+                                      const void* targets, uint64_t rows, uint64_t dim, uint64_t vocab,
+                                      int32_t has_ignore, uint32_t ignore_index, uint64_t chunk_rows,
+                                      uint64_t chunk_cols, void* loss, void* gx, int32_t gx_dtype, void* gw) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "linear_cross_entropy_mean";
+  if (!x || !w || !targets || !loss) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  if (!omx_valid_float_dtype(operand_dtype)) return omx_fail(ctx, OMX_DTYPE, "%s: operands must be f32 or bf16", op);
+  if (gx && !omx_valid_float_dtype(gx_dtype)) return omx_fail(ctx, OMX_DTYPE, "%s: grad_input dtype", op);
+  if (rows == 0 || dim == 0 || vocab == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
+  if (chunk_rows == 0 || chunk_cols == 0) return omx_fail(ctx, OMX_SHAPE, "%s: chunk has a zero axis", op);
+  if (vocab > 0xfffffffeull || rows > 0x7fffffffull)
+    return omx_fail(ctx, OMX_OUT_OF_RANGE, "%s: axis does not fit in u32", op);
+  const uint64_t R = chunk_rows < rows ? chunk_rows : rows;
+  // Column tiles start on multiples of 8 so every tile of W stays 16-byte aligned.
+  uint64_t C = chunk_cols < vocab ? chunk_cols : vocab;
+  if (C < vocab && C >= 8) C &= ~7ull;
+  const bool one_tile = C >= vocab;
+  const bool want_grads = gx || gw;
+  const size_t esz = omx_dtype_size(operand_dtype);
+  // Workspace: [tile R x C] [gx accumulator R x dim f32, only with several column tiles] [state].
+  const uint64_t tile_bytes = (R * C * esz + 255) & ~255ull;
+  const uint64_t gxacc_bytes = (gx && !one_tile) ? ((R * dim * 4 + 255) & ~255ull) : 0;
+  void* ws = nullptr;
+  int32_t rc = omx_workspace(ctx, tile_bytes + gxacc_bytes + ce_scratch_bytes(rows), &ws);
+  if (rc != OMX_OK) return rc;
+  char* base = static_cast<char*>(ws);
+  void* tile = base;
+  float* gxacc = reinterpret_cast<float*>(base + tile_bytes);
+  CeScratch s = carve(base + tile_bytes + gxacc_bytes, rows);
+  const unsigned int* tg = static_cast<const unsigned int*>(targets);
+  unsigned long long tag = omx_tag(ctx, F_LINEAR_CE);
+  rc = count_valid(ctx, tg, rows, vocab, has_ignore, ignore_index, s.valid, tag);
+  if (rc != OMX_OK) return rc;
+  const char* xb = static_cast<const char*>(x);
+  const char* wb = static_cast<const char*>(w);
+
+  auto logits_tile = [&](uint64_t r0, uint64_t nr, uint64_t c0, uint64_t nc) -> int32_t {
+    // tile[nr, nc] = x[r0.., :] . W[c0.., :]^T
+    return omx_gemm_impl(ctx, F_LINEAR_CE, xb + r0 * dim * esz, dim, 1, wb + c0 * dim * esz, 1, dim, operand_dtype,
+                         tile, operand_dtype, nc, nr, dim, nc, 0);
+  };
+  for (uint64_t r0 = 0; r0 < rows; r0 += R) {
+    const uint64_t nr = (rows - r0) < R ? (rows - r0) : R;
+    // Pass 1: row statistics over every vocabulary tile.
+    for (uint64_t c0 = 0; c0 < vocab; c0 += C) {
+      const uint64_t nc = (vocab - c0) < C ? (vocab - c0) : C;
+      rc = logits_tile(r0, nr, c0, nc);
+      if (rc != OMX_OK) return rc;
+      if (operand_dtype == OMX_F32)
+        launch_stats<float>(ctx, tile, nc, r0, nr, static_cast<unsigned>(c0), static_cast<unsigned>(nc), tg, s.st,
+                            c0 == 0, tag);
+      else
+        launch_stats<unsigned short>(ctx, tile, nc, r0, nr, static_cast<unsigned>(c0), static_cast<unsigned>(nc), tg,
+                                     s.st, c0 == 0, tag);
+      OMX_LAUNCH_CHECK(ctx, "ce_tile_stats_kernel");
+    }
+    if (!want_grads) continue;
+    // Pass 2: gradient tiles and their two products.
+    for (uint64_t c0 = 0; c0 < vocab; c0 += C) {
+      const uint64_t nc = (vocab - c0) < C ? (vocab - c0) : C;
+      if (!one_tile) {
+        rc = logits_tile(r0, nr, c0, nc);
+        if (rc != OMX_OK) return rc;
+      }
+      if (operand_dtype == OMX_F32)
+        launch_grad<float, float>(ctx, tile, tile, nc, nc, r0, nr, static_cast<unsigned>(c0),
+                                  static_cast<unsigned>(nc), tg, has_ignore, ignore_index, s.st, s.valid);
+      else
+        launch_grad<unsigned short, unsigned short>(ctx, tile, tile, nc, nc, r0, nr, static_cast<unsigned>(c0),
+                                                    static_cast<unsigned>(nc), tg, has_ignore, ignore_index, s.st,
+                                                    s.valid);
+      OMX_LAUNCH_CHECK(ctx, "ce_tile_grad_kernel");
+      if (gx) {
+        // gx[r0.., :] (+)= G[nr, nc] . W[c0.., :]
+        if (one_tile) {
+          rc = omx_gemm_impl(ctx, F_LINEAR_CE, tile, nc, 1, wb + c0 * dim * esz, dim, 1, operand_dtype,
+                             static_cast<char*>(gx) + r0 * dim * omx_dtype_size(gx_dtype), gx_dtype, dim, nr, nc, dim,
+                             0);
+        } else {
+          rc = omx_gemm_impl(ctx, F_LINEAR_CE, tile, nc, 1, wb + c0 * dim * esz, dim, 1, operand_dtype, gxacc,
+                             OMX_F32, dim, nr, nc, dim, c0 != 0);
+        }
+        if (rc != OMX_OK) return rc;
+      }
+      if (gw) {
+        // gw[c0.., :] (+)= G^T[nc, nr] . x[r0.., :]
+        rc = omx_gemm_impl(ctx, F_LINEAR_CE, tile, 1, nc, xb + r0 * dim * esz, dim, 1, operand_dtype,
+                           static_cast<float*>(gw) + c0 * dim, OMX_F32, dim, nc, nr, dim, r0 != 0);
+        if (rc != OMX_OK) return rc;
+      }
+    }
+    if (gx && !one_tile) {
+      rc = omx_convert(ctx, gxacc, OMX_F32, static_cast<char*>(gx) + r0 * dim * omx_dtype_size(gx_dtype), gx_dtype,
+                       nr * dim);
+      if (rc != OMX_OK) return rc;
+    }
+  }
+  hipLaunchKernelGGL(ce_mean_kernel, dim3(1), dim3(1024), 0, ctx->stream, s.st, tg, rows, has_ignore, ignore_index,
+                     s.valid, static_cast<float*>(loss), ctx->fault, tag);
+  OMX_LAUNCH_CHECK(ctx, "ce_mean_kernel");
+  return OMX_OK;
+}
+
+}  // extern "C"

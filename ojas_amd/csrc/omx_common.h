@@ -1,0 +1,168 @@
+// Internal declarations shared by the kernel files of libojas_mi355x.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <string>
+
+#include "ojas_mi355x.h"
+
+// Ops that can raise a deferred non-finite fault, in the order their bits sit
+// in the fault word. The name is what OjasError::NonFinite { op } carries.
+enum OmxFaultOp : uint32_t {
+  F_LINEAR_FORWARD = 0,
+  F_LINEAR_BACKWARD,
+  F_GEMM,
+  F_SDPA_FORWARD,
+  F_SDPA_BACKWARD,
+  F_RMS_FORWARD,
+  F_RMS_BACKWARD,
+  F_CE_FORWARD,
+  F_CE_BACKWARD,
+  F_LINEAR_CE,
+  F_EMBEDDING_FORWARD,
+  F_EMBEDDING_BACKWARD,
+  F_ADAMW,
+  F_MUON,
+  F_CLIP,
+  F_RESIDUAL_ADD,
+  F_ACCUMULATE,
+  F_SCALE_GRAD,
+  F_GELU_FORWARD,
+  F_GELU_BACKWARD,
+  F_ARGMAX,
+  F_TOPK,
+  F_COUNT
+};
+const char* omx_fault_name(uint32_t op);
+
+// Device-side fault record: a bit mask plus the launch sequence number of the
+// first op that faulted (lowest sequence wins), so the error can name it.
+struct OmxFaultWord {
+  unsigned long long mask;
+  unsigned long long first;  // (sequence << 8) | op, ~0 when clear
+};
+
+struct omx_ctx {
+  int device = 0;
+  hipStream_t stream = nullptr;
+  uint64_t budget_limit = 0, budget_live = 0, budget_peak = 0;
+  std::map<void*, uint64_t> allocations;
+  OmxFaultWord* fault = nullptr;  // device
+  OmxFaultWord* fault_host = nullptr;  // pinned
+  uint64_t sequence = 0;
+  std::string last_error;
+  std::string arch;
+  // Scratch the library owns (charged to the budget); grown on demand.
+  void* workspace = nullptr;
+  uint64_t workspace_bytes = 0;
+  int cu_count = 0;
+};
+
+int32_t omx_fail(omx_ctx* ctx, omx_status code, const char* fmt, ...);
+int32_t omx_hip_fail(omx_ctx* ctx, hipError_t err, const char* what);
+// Grows the library workspace to at least `bytes` (budget-charged).
+int32_t omx_workspace(omx_ctx* ctx, uint64_t bytes, void** out);
+// Next launch tag for fault attribution: (sequence << 8) | op.
+inline unsigned long long omx_tag(omx_ctx* ctx, uint32_t op) {
+  return (static_cast<unsigned long long>(++ctx->sequence) << 8) | op;
+}
+
+// C[m,n] (+)= A.B with element strides; `ldc` is C's row pitch in elements.
+int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a_rs, uint64_t a_cs, const void* b,
+                      uint64_t b_rs, uint64_t b_cs, int32_t operand_dtype, void* c, int32_t c_dtype, uint64_t ldc,
+                      uint64_t m, uint64_t k, uint64_t n, int32_t accumulate);
+// Elementwise conversions on the context's stream (no fault reporting).
+int32_t omx_convert(omx_ctx* ctx, const void* src, int32_t src_dtype, void* dst, int32_t dst_dtype, uint64_t n);
+
+#define OMX_HIP(ctx, expr)                                   \
+  do {                                                       \
+    hipError_t e_ = (expr);                                  \
+    if (e_ != hipSuccess) return omx_hip_fail(ctx, e_, #expr); \
+  } while (0)
+
+#define OMX_LAUNCH_CHECK(ctx, what)                               \
+  do {                                                            \
+    hipError_t e_ = hipGetLastError();                            \
+    if (e_ != hipSuccess) return omx_hip_fail(ctx, e_, what);     \
+  } while (0)
+
+#define OMX_REQUIRE_CTX(ctx) \
+  do {                       \
+    if (!(ctx)) return OMX_BACKEND; \
+  } while (0)
+
+// ---- device helpers ----
+typedef __hip_bfloat16 bf16_t;
+
+__device__ __forceinline__ bool dev_finite(float x) {
+  return (__float_as_uint(x) & 0x7fffffffu) < 0x7f800000u;
+}
+
+// Round to nearest even on the dropped 16 bits; NaN keeps sign and payload and
+// sets the quiet bit (ojas-core/src/autocast.rs:70-96).
+__device__ __forceinline__ unsigned short dev_f32_to_bf16_bits(float v) {
+  unsigned int b = __float_as_uint(v);
+  if (v != v) return static_cast<unsigned short>((b >> 16) | 0x0040u);
+  unsigned int round = 0x7fffu + ((b >> 16) & 1u);
+  return static_cast<unsigned short>((b + round) >> 16);
+}
+__device__ __forceinline__ float dev_bf16_bits_to_f32(unsigned short b) {
+  return __uint_as_float(static_cast<unsigned int>(b) << 16);
+}
+__device__ __forceinline__ float dev_round_bf16(float v) {
+  return dev_bf16_bits_to_f32(dev_f32_to_bf16_bits(v));
+}
+
+// The low byte of a tag is the op (bits 0-6) and the fault kind (bit 7:
+// 0 = non-finite value, 1 = index out of range).
+__device__ __forceinline__ void dev_raise_fault(OmxFaultWord* fault, unsigned long long tag) {
+  atomicOr(&fault->mask, 1ull << (tag & 0x3full));
+  atomicMin(&fault->first, tag);
+}
+__device__ __forceinline__ void dev_raise_range(OmxFaultWord* fault, unsigned long long tag) {
+  atomicOr(&fault->mask, 1ull << (tag & 0x3full));
+  atomicMin(&fault->first, tag | 0x80ull);
+}
+
+// Loads element i of a tensor stored as f32 or bf16, widened exactly.
+template <typename T>
+__device__ __forceinline__ float dev_load(const T* p, size_t i);
+template <>
+__device__ __forceinline__ float dev_load<float>(const float* p, size_t i) {
+  return p[i];
+}
+template <>
+__device__ __forceinline__ float dev_load<unsigned short>(const unsigned short* p, size_t i) {
+  return dev_bf16_bits_to_f32(p[i]);
+}
+template <typename T>
+__device__ __forceinline__ void dev_store(T* p, size_t i, float v);
+template <>
+__device__ __forceinline__ void dev_store<float>(float* p, size_t i, float v) {
+  p[i] = v;
+}
+template <>
+__device__ __forceinline__ void dev_store<unsigned short>(unsigned short* p, size_t i, float v) {
+  p[i] = dev_f32_to_bf16_bits(v);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+inline bool omx_valid_float_dtype(int32_t d) { return d == OMX_F32 || d == OMX_BF16; }
+inline size_t omx_dtype_size(int32_t d) { return d == OMX_BF16 ? 2 : 4; }

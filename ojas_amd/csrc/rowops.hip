@@ -1,0 +1,548 @@
+// Row-wise bandwidth-bound kernels: RMSNorm forward/backward, embedding
+// gather / scatter-add, argmax and top-k. One wave (64 lanes) owns one row;
+// reductions are wavefront shuffles; every tensor is read from HBM once.
+//
+// Reference semantics:
+//   rms_norm_*   ojas-cpu/src/norm.rs:24-204   (trait backend.rs:1658-1672)
+//   embedding_*  ojas-cpu/src/pointwise.rs:77-215 (trait backend.rs:1610-1626)
+//   argmax/topk  ojas-core/src/backend.rs:184-195,1514-1606
+#include "omx_common.h"
+
+namespace {
+
+constexpr int ROW_THREADS = 256;  // 4 waves per block, one row per wave at a time
+
+// ---------------------------------------------------------------- RMSNorm
+// PER = ceil(dim / 64): lane l owns columns l, l + 64, ... so a wave's loads
+// are contiguous 64-element runs and the row stays in registers between the
+// sum-of-squares pass and the scaling pass.
+template <typename TX, typename TY, int PER>
+__global__ __launch_bounds__(ROW_THREADS) void rms_fwd_kernel(const TX* __restrict__ x, const float* __restrict__ w,
+                                                              TY* __restrict__ y, size_t rows, int dim, float eps,
+                                                              OmxFaultWord* fault, unsigned long long tag) {
+  const int lane = threadIdx.x & 63;
+  const size_t row = static_cast<size_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const TX* xr = x + row * dim;
+  float xv[PER];
+  float ss = 0.0f;
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    int c = j * 64 + lane;
+    xv[j] = c < dim ? dev_load<TX>(xr, c) : 0.0f;
+    ss += xv[j] * xv[j];
+  }
+  ss = wave_sum(ss);
+  float denom = ss / static_cast<float>(dim) + eps;
+  float rstd = 1.0f / sqrtf(denom);
+  bool bad = !(dev_finite(denom) && denom > 0.0f && dev_finite(rstd));
+  TY* yr = y + row * dim;
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    int c = j * 64 + lane;
+    if (c < dim) {
+      float v = xv[j] * rstd * w[c];
+      bad |= !dev_finite(v);
+      dev_store<TY>(yr, c, v);
+    }
+  }
+  if (bad) dev_raise_fault(fault, tag);
+}
+
+// Backward: gx per row, and per-block partial column sums of g * xhat that a
+// second kernel adds in ascending block order (no atomics, deterministic).
+template <typename TX, typename TG, typename TO, int PER>
+__global__ __launch_bounds__(ROW_THREADS) void rms_bwd_kernel(const TX* __restrict__ x, const float* __restrict__ w,
+                                                              const TG* __restrict__ gy, TO* __restrict__ gx,
+                                                              float* __restrict__ partial, size_t rows, int dim,
+                                                              float eps, int rows_per_block, OmxFaultWord* fault,
+                                                              unsigned long long tag) {
+  extern __shared__ float lds[];  // [4][dim]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const float inv_dim = 1.0f / static_cast<float>(dim);
+  float wv[PER], accw[PER];
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    int c = j * 64 + lane;
+    wv[j] = c < dim ? w[c] : 0.0f;
+    accw[j] = 0.0f;
+  }
+  bool bad = false;
+  const size_t first = static_cast<size_t>(blockIdx.x) * rows_per_block;
+  const size_t last = min(rows, first + rows_per_block);
+  for (size_t row = first + wave; row < last; row += 4) {
+    const TX* xr = x + row * dim;
+    const TG* gr = gy + row * dim;
+    float xv[PER], gv[PER];
+    float ss = 0.0f;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      int c = j * 64 + lane;
+      xv[j] = c < dim ? dev_load<TX>(xr, c) : 0.0f;
+      gv[j] = c < dim ? dev_load<TG>(gr, c) : 0.0f;
+      ss += xv[j] * xv[j];
+    }
+    ss = wave_sum(ss);
+    float denom = ss * inv_dim + eps;
+    float rstd = 1.0f / sqrtf(denom);
+    bad |= !(dev_finite(denom) && denom > 0.0f && dev_finite(rstd));
+    float dot = 0.0f;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) dot += (gv[j] * wv[j]) * (xv[j] * rstd);
+    dot = wave_sum(dot);
+    float mean = dot * inv_dim;
+    TO* gxr = gx + row * dim;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      int c = j * 64 + lane;
+      float xhat = xv[j] * rstd;
+      float v = (gv[j] * wv[j] - xhat * mean) * rstd;
+      accw[j] += gv[j] * xhat;
+      if (c < dim) {
+        bad |= !dev_finite(v);
+        dev_store<TO>(gxr, c, v);
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    int c = j * 64 + lane;
+    if (c < dim) lds[wave * dim + c] = accw[j];
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < dim; c += ROW_THREADS) {
+    float s = ((lds[c] + lds[dim + c]) + lds[2 * dim + c]) + lds[3 * dim + c];
+    partial[static_cast<size_t>(blockIdx.x) * dim + c] = s;
+  }
+  if (bad) dev_raise_fault(fault, tag);
+}
+
+__global__ void column_sum_kernel(const float* __restrict__ partial, float* __restrict__ out, int blocks, int dim,
+                                  OmxFaultWord* fault, unsigned long long tag) {
+  int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= dim) return;
+  float s = 0.0f;
+  for (int b = 0; b < blocks; ++b) s += partial[static_cast<size_t>(b) * dim + c];
+  out[c] = s;
+  if (!dev_finite(s)) dev_raise_fault(fault, tag);
+}
+
+// ---------------------------------------------------------------- embedding
+template <typename TT, typename TO>
+__global__ void embedding_fwd_kernel(const TT* __restrict__ table, const unsigned int* __restrict__ ids,
+                                     TO* __restrict__ out, size_t tokens, size_t vocab, int dim, OmxFaultWord* fault,
+                                     unsigned long long tag) {
+  const int lane = threadIdx.x & 63;
+  const size_t n = static_cast<size_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (n >= tokens) return;
+  size_t id = ids[n];
+  TO* dst = out + n * dim;
+  if (id >= vocab) {
+    // Refused id: the row is zero-filled and the call reports OutOfRange.
+    for (int c = lane; c < dim; c += 64) dev_store<TO>(dst, c, 0.0f);
+    if (lane == 0) dev_raise_range(fault, tag);
+    return;
+  }
+  const TT* src = table + id * dim;
+  if constexpr (sizeof(TT) == sizeof(TO)) {
+    // Same storage: a bit copy (NaN payloads and -0 survive).
+    for (int c = lane; c < dim; c += 64) dst[c] = src[c];
+  } else {
+    for (int c = lane; c < dim; c += 64) dev_store<TO>(dst, c, dev_load<TT>(src, c));
+  }
+}
+
+__global__ void count_ids_kernel(const unsigned int* __restrict__ ids, unsigned int* __restrict__ counts,
+                                 size_t tokens, size_t vocab, OmxFaultWord* fault, unsigned long long tag) {
+  size_t n = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (n >= tokens) return;
+  unsigned int id = ids[n];
+  if (id >= vocab) {
+    dev_raise_range(fault, tag);
+    return;
+  }
+  atomicAdd(&counts[id], 1u);
+}
+
+// Exclusive scan of counts[vocab] into offsets[vocab + 1] and a copy into
+// cursor[vocab]; one 1024-thread block walks the array in 1024-wide strips.
+__global__ __launch_bounds__(1024) void scan_counts_kernel(const unsigned int* __restrict__ counts,
+                                                           unsigned int* __restrict__ offsets,
+                                                           unsigned int* __restrict__ cursor, size_t vocab) {
+  __shared__ unsigned int wave_tot[16];
+  __shared__ unsigned int carry;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (threadIdx.x == 0) carry = 0;
+  __syncthreads();
+  for (size_t base = 0; base < vocab; base += 1024) {
+    size_t i = base + threadIdx.x;
+    unsigned int v = i < vocab ? counts[i] : 0u;
+    unsigned int incl = v;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      unsigned int t = __shfl_up(incl, off, 64);
+      if (lane >= off) incl += t;
+    }
+    if (lane == 63) wave_tot[wave] = incl;
+    __syncthreads();
+    unsigned int before = carry;
+    for (int wv = 0; wv < wave; ++wv) before += wave_tot[wv];
+    unsigned int excl = before + incl - v;
+    if (i < vocab) {
+      offsets[i] = excl;
+      cursor[i] = excl;
+    }
+    __syncthreads();
+    if (threadIdx.x == 1023) carry = excl + v;
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) offsets[vocab] = carry;
+}
+
+__global__ void fill_positions_kernel(const unsigned int* __restrict__ ids, unsigned int* __restrict__ cursor,
+                                      unsigned int* __restrict__ positions, size_t tokens, size_t vocab) {
+  size_t n = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (n >= tokens) return;
+  unsigned int id = ids[n];
+  if (id >= vocab) return;
+  unsigned int slot = atomicAdd(&cursor[id], 1u);
+  positions[slot] = static_cast<unsigned int>(n);
+}
+
+// One wave per table row: zero it, or add its tokens' gradient rows in
+// ascending token order (the order of the CPU scatter, pointwise.rs:196-207),
+// so the f32 sums carry the same bits. The unordered segment is walked by
+// repeated minimum selection.
+template <typename TG>
+__global__ __launch_bounds__(ROW_THREADS) void embedding_bwd_kernel(const unsigned int* __restrict__ offsets,
+                                                                    const unsigned int* __restrict__ positions,
+                                                                    const TG* __restrict__ grad,
+                                                                    float* __restrict__ table_grad, size_t vocab,
+                                                                    int dim, OmxFaultWord* fault,
+                                                                    unsigned long long tag) {
+  const int lane = threadIdx.x & 63;
+  const size_t v = static_cast<size_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (v >= vocab) return;
+  const unsigned int begin = offsets[v], end = offsets[v + 1];
+  float* dst = table_grad + v * dim;
+  if (begin == end) {
+    for (int c = lane; c < dim; c += 64) dst[c] = 0.0f;
+    return;
+  }
+  bool bad = false;
+  for (int c0 = 0; c0 < dim; c0 += 64 * 8) {
+    float acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
+    long last = -1;
+    for (unsigned int step = begin; step < end; ++step) {
+      unsigned int best = 0xffffffffu;
+      for (unsigned int s = begin + lane; s < end; s += 64) {
+        unsigned int p = positions[s];
+        if (static_cast<long>(p) > last && p < best) best = p;
+      }
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) best = min(best, static_cast<unsigned int>(__shfl_xor(best, off, 64)));
+      last = best;
+      const TG* src = grad + static_cast<size_t>(best) * dim;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        int c = c0 + j * 64 + lane;
+        if (c < dim) acc[j] = acc[j] + dev_load<TG>(src, c);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      int c = c0 + j * 64 + lane;
+      if (c < dim) {
+        bad |= !dev_finite(acc[j]);
+        dst[c] = acc[j];
+      }
+    }
+  }
+  if (bad) dev_raise_fault(fault, tag);
+}
+
+// ---------------------------------------------------------------- argmax / top-k
+// Order of rank_logits (backend.rs:184-195): value descending with +0 == -0,
+// then column ascending. `before(a, b)`: a ranks ahead of b.
+__device__ __forceinline__ float rank_key(float v) { return v == 0.0f ? 0.0f : v; }
+__device__ __forceinline__ bool ranks_before(float va, unsigned int ia, float vb, unsigned int ib) {
+  float ka = rank_key(va), kb = rank_key(vb);
+  return ka > kb || (ka == kb && ia < ib);
+}
+
+__global__ void argmax_rows_kernel(const float* __restrict__ x, size_t rows, unsigned int cols,
+                                   unsigned int* __restrict__ out, OmxFaultWord* fault, unsigned long long tag) {
+  const int lane = threadIdx.x & 63;
+  const size_t row = static_cast<size_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const float* r = x + row * cols;
+  // Ties go to the lowest column: strict > within a lane's ascending walk.
+  float best = -INFINITY;
+  unsigned int idx = 0xffffffffu;
+  bool bad = false;
+  for (unsigned int c = lane; c < cols; c += 64) {
+    float v = r[c];
+    bad |= !dev_finite(v);
+    if (idx == 0xffffffffu || v > best) {
+      best = v;
+      idx = c;
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    float ov = __shfl_xor(best, off, 64);
+    unsigned int oi = __shfl_xor(idx, off, 64);
+    if (oi != 0xffffffffu && (idx == 0xffffffffu || ov > best || (ov == best && oi < idx))) {
+      best = ov;
+      idx = oi;
+    }
+  }
+  bad = __any(bad);
+  if (lane == 0) {
+    out[row] = idx;
+    if (bad) dev_raise_fault(fault, tag);
+  }
+}
+
+// k passes over the row; pass j picks the best element ranked after pass
+// j-1's pick. NaN and +inf are refused, -inf sorts last.
+__global__ void topk_rows_kernel(const float* __restrict__ x, size_t rows, unsigned int cols, unsigned int k,
+                                 float* __restrict__ values, unsigned int* __restrict__ ids, OmxFaultWord* fault,
+                                 unsigned long long tag) {
+  const int lane = threadIdx.x & 63;
+  const size_t row = static_cast<size_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const float* r = x + row * cols;
+  bool bad = false;
+  float prev_v = 0.0f;
+  unsigned int prev_i = 0;
+  for (unsigned int j = 0; j < k; ++j) {
+    float best = 0.0f;
+    unsigned int idx = 0xffffffffu;
+    for (unsigned int c = lane; c < cols; c += 64) {
+      float v = r[c];
+      if (j == 0) bad |= (v != v) || v == INFINITY;
+      if (j > 0 && !ranks_before(prev_v, prev_i, v, c)) continue;
+      if (idx == 0xffffffffu || ranks_before(v, c, best, idx)) {
+        best = v;
+        idx = c;
+      }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      float ov = __shfl_xor(best, off, 64);
+      unsigned int oi = __shfl_xor(idx, off, 64);
+      if (oi != 0xffffffffu && (idx == 0xffffffffu || ranks_before(ov, oi, best, idx))) {
+        best = ov;
+        idx = oi;
+      }
+    }
+    prev_v = best;
+    prev_i = idx;
+    if (lane == 0) {
+      values[row * k + j] = best;
+      ids[row * k + j] = idx;
+    }
+  }
+  bad = __any(bad);
+  if (lane == 0 && bad) dev_raise_fault(fault, tag);
+}
+
+inline int per_for_dim(uint64_t dim) {
+  const int options[] = {1, 2, 4, 8, 12, 16, 32, 64, 128};
+  for (int p : options)
+    if (static_cast<uint64_t>(p) * 64 >= dim) return p;
+  return 0;
+}
+
+template <typename TX, typename TY>
+int32_t launch_rms_fwd(omx_ctx* ctx, const void* x, const float* w, void* y, uint64_t rows, uint64_t dim, float eps,
+                       unsigned long long tag) {
+  dim3 grid(static_cast<unsigned>((rows + 3) / 4)), block(ROW_THREADS);
+  int per = per_for_dim(dim);
+#define RMS_FWD(P)                                                                                              \
+  case P:                                                                                                       \
+    hipLaunchKernelGGL((rms_fwd_kernel<TX, TY, P>), grid, block, 0, ctx->stream, static_cast<const TX*>(x), w, \
+                       static_cast<TY*>(y), rows, static_cast<int>(dim), eps, ctx->fault, tag);                 \
+    break;
+  switch (per) {
+    RMS_FWD(1) RMS_FWD(2) RMS_FWD(4) RMS_FWD(8) RMS_FWD(12) RMS_FWD(16) RMS_FWD(32) RMS_FWD(64) RMS_FWD(128)
+    default:
+      return omx_fail(ctx, OMX_UNSUPPORTED, "rms_norm_forward: dim %llu above 8192", (unsigned long long)dim);
+  }
+#undef RMS_FWD
+  OMX_LAUNCH_CHECK(ctx, "rms_fwd_kernel");
+  return OMX_OK;
+}
+
+template <typename TX, typename TG, typename TO>
+int32_t launch_rms_bwd(omx_ctx* ctx, const void* x, const float* w, const void* gy, void* gx, float* gw,
+                       uint64_t rows, uint64_t dim, float eps, unsigned long long tag) {
+  const int rows_per_block = 32;
+  uint64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
+  void* partial = nullptr;
+  int32_t rc = omx_workspace(ctx, blocks * dim * sizeof(float), &partial);
+  if (rc != OMX_OK) return rc;
+  dim3 grid(static_cast<unsigned>(blocks)), block(ROW_THREADS);
+  size_t smem = 4 * dim * sizeof(float);
+  int per = per_for_dim(dim);
+#define RMS_BWD(P)                                                                                                  \
+  case P:                                                                                                           \
+    hipLaunchKernelGGL((rms_bwd_kernel<TX, TG, TO, P>), grid, block, smem, ctx->stream, static_cast<const TX*>(x), \
+                       w, static_cast<const TG*>(gy), static_cast<TO*>(gx), static_cast<float*>(partial), rows,     \
+                       static_cast<int>(dim), eps, rows_per_block, ctx->fault, tag);                                \
+    break;
+  switch (per) {
+    RMS_BWD(1) RMS_BWD(2) RMS_BWD(4) RMS_BWD(8) RMS_BWD(12) RMS_BWD(16) RMS_BWD(32) RMS_BWD(64)
+    default:
+      return omx_fail(ctx, OMX_UNSUPPORTED, "rms_norm_backward: dim %llu above 4096", (unsigned long long)dim);
+  }
+#undef RMS_BWD
+  OMX_LAUNCH_CHECK(ctx, "rms_bwd_kernel");
+  hipLaunchKernelGGL(column_sum_kernel, dim3(static_cast<unsigned>((dim + 255) / 256)), dim3(256), 0, ctx->stream,
+                     static_cast<const float*>(partial), gw, static_cast<int>(blocks), static_cast<int>(dim),
+                     ctx->fault, tag);
+  OMX_LAUNCH_CHECK(ctx, "column_sum_kernel");
+  return OMX_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t omx_rms_norm_forward(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* w, void* y, int32_t y_dtype,
+                             uint64_t rows, uint64_t dim, float eps) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "rms_norm_forward";
+  if (!x || !w || !y) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  if (!omx_valid_float_dtype(x_dtype) || !omx_valid_float_dtype(y_dtype))
+    return omx_fail(ctx, OMX_DTYPE, "%s: dtype must be f32 or bf16", op);
+  if (rows == 0 || dim == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
+  if (!(eps == eps) || eps == INFINITY || eps == -INFINITY) return omx_fail(ctx, OMX_NON_FINITE, "%s", op);
+  unsigned long long tag = omx_tag(ctx, F_RMS_FORWARD);
+  const float* wf = static_cast<const float*>(w);
+  if (x_dtype == OMX_F32 && y_dtype == OMX_F32) return launch_rms_fwd<float, float>(ctx, x, wf, y, rows, dim, eps, tag);
+  if (x_dtype == OMX_F32) return launch_rms_fwd<float, unsigned short>(ctx, x, wf, y, rows, dim, eps, tag);
+  if (y_dtype == OMX_F32) return launch_rms_fwd<unsigned short, float>(ctx, x, wf, y, rows, dim, eps, tag);
+  return launch_rms_fwd<unsigned short, unsigned short>(ctx, x, wf, y, rows, dim, eps, tag);
+}
+
+int32_t omx_rms_norm_backward(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* w, const void* gy,
+                              int32_t gy_dtype, void* gx, int32_t gx_dtype, void* gw, uint64_t rows, uint64_t dim,
+                              float eps) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "rms_norm_backward";
+  if (!x || !w || !gy || !gx || !gw) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  if (!omx_valid_float_dtype(x_dtype) || !omx_valid_float_dtype(gy_dtype) || !omx_valid_float_dtype(gx_dtype))
+    return omx_fail(ctx, OMX_DTYPE, "%s: dtype must be f32 or bf16", op);
+  if (gy_dtype != gx_dtype) return omx_fail(ctx, OMX_DTYPE, "%s: grad dtypes differ", op);
+  if (rows == 0 || dim == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
+  if (!(eps == eps) || eps == INFINITY || eps == -INFINITY) return omx_fail(ctx, OMX_NON_FINITE, "%s", op);
+  unsigned long long tag = omx_tag(ctx, F_RMS_BACKWARD);
+  const float* wf = static_cast<const float*>(w);
+  float* gwf = static_cast<float*>(gw);
+  if (x_dtype == OMX_F32 && gy_dtype == OMX_F32)
+    return launch_rms_bwd<float, float, float>(ctx, x, wf, gy, gx, gwf, rows, dim, eps, tag);
+  if (x_dtype == OMX_BF16 && gy_dtype == OMX_BF16)
+    return launch_rms_bwd<unsigned short, unsigned short, unsigned short>(ctx, x, wf, gy, gx, gwf, rows, dim, eps, tag);
+  if (x_dtype == OMX_F32)
+    return launch_rms_bwd<float, unsigned short, unsigned short>(ctx, x, wf, gy, gx, gwf, rows, dim, eps, tag);
+  return launch_rms_bwd<unsigned short, float, float>(ctx, x, wf, gy, gx, gwf, rows, dim, eps, tag);
+}
+
+int32_t omx_embedding_forward(omx_ctx* ctx, const void* table, int32_t table_dtype, const void* ids, void* out,
+                              int32_t out_dtype, uint64_t tokens, uint64_t vocab, uint64_t dim) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "embedding_forward";
+  if (!table || !ids || !out) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  if (!omx_valid_float_dtype(table_dtype) || !omx_valid_float_dtype(out_dtype))
+    return omx_fail(ctx, OMX_DTYPE, "%s: dtype must be f32 or bf16", op);
+  if (tokens == 0 || vocab == 0 || dim == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
+  if (dim > 0x7fffffffull) return omx_fail(ctx, OMX_OUT_OF_RANGE, "%s: dim does not fit in i32", op);
+  unsigned long long tag = omx_tag(ctx, F_EMBEDDING_FORWARD);
+  dim3 grid(static_cast<unsigned>((tokens + 3) / 4)), block(ROW_THREADS);
+  const unsigned int* idp = static_cast<const unsigned int*>(ids);
+#define EMB_FWD(TT, TO)                                                                                      \
+  hipLaunchKernelGGL((embedding_fwd_kernel<TT, TO>), grid, block, 0, ctx->stream, static_cast<const TT*>(table), \
+                     idp, static_cast<TO*>(out), tokens, vocab, static_cast<int>(dim), ctx->fault, tag)
+  if (table_dtype == OMX_F32 && out_dtype == OMX_F32) EMB_FWD(float, float);
+  else if (table_dtype == OMX_F32) EMB_FWD(float, unsigned short);
+  else if (out_dtype == OMX_F32) EMB_FWD(unsigned short, float);
+  else EMB_FWD(unsigned short, unsigned short);
+#undef EMB_FWD
+  OMX_LAUNCH_CHECK(ctx, "embedding_fwd_kernel");
+  return OMX_OK;
+}
+
+int32_t omx_embedding_backward(omx_ctx* ctx, const void* ids, const void* grad, int32_t grad_dtype, void* table_grad,
+                               uint64_t tokens, uint64_t vocab, uint64_t dim) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "embedding_backward";
+  if (!ids || !grad || !table_grad) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  if (!omx_valid_float_dtype(grad_dtype)) return omx_fail(ctx, OMX_DTYPE, "%s: dtype must be f32 or bf16", op);
+  if (tokens == 0 || vocab == 0 || dim == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
+  if (tokens > 0xfffffffeull || vocab > 0xfffffffeull || dim > 0x7fffffffull)
+    return omx_fail(ctx, OMX_OUT_OF_RANGE, "%s: axis does not fit in u32", op);
+  // Workspace: counts[V], offsets[V+1], cursor[V], positions[N].
+  uint64_t words = vocab + (vocab + 1) + vocab + tokens;
+  void* ws = nullptr;
+  int32_t rc = omx_workspace(ctx, words * 4, &ws);
+  if (rc != OMX_OK) return rc;
+  unsigned int* counts = static_cast<unsigned int*>(ws);
+  unsigned int* offsets = counts + vocab;
+  unsigned int* cursor = offsets + vocab + 1;
+  unsigned int* positions = cursor + vocab;
+  unsigned long long tag = omx_tag(ctx, F_EMBEDDING_BACKWARD);
+  rc = omx_fill_zero(ctx, counts, vocab * 4);
+  if (rc != OMX_OK) return rc;
+  const unsigned int* idp = static_cast<const unsigned int*>(ids);
+  dim3 tgrid(static_cast<unsigned>((tokens + 255) / 256));
+  hipLaunchKernelGGL(count_ids_kernel, tgrid, dim3(256), 0, ctx->stream, idp, counts, tokens, vocab, ctx->fault, tag);
+  OMX_LAUNCH_CHECK(ctx, "count_ids_kernel");
+  hipLaunchKernelGGL(scan_counts_kernel, dim3(1), dim3(1024), 0, ctx->stream, counts, offsets, cursor, vocab);
+  OMX_LAUNCH_CHECK(ctx, "scan_counts_kernel");
+  hipLaunchKernelGGL(fill_positions_kernel, tgrid, dim3(256), 0, ctx->stream, idp, cursor, positions, tokens, vocab);
+  OMX_LAUNCH_CHECK(ctx, "fill_positions_kernel");
+  dim3 vgrid(static_cast<unsigned>((vocab + 3) / 4));
+  if (grad_dtype == OMX_F32)
+    hipLaunchKernelGGL((embedding_bwd_kernel<float>), vgrid, dim3(ROW_THREADS), 0, ctx->stream, offsets, positions,
+                       static_cast<const float*>(grad), static_cast<float*>(table_grad), vocab, static_cast<int>(dim),
+                       ctx->fault, tag);
+  else
+    hipLaunchKernelGGL((embedding_bwd_kernel<unsigned short>), vgrid, dim3(ROW_THREADS), 0, ctx->stream, offsets,
+                       positions, static_cast<const unsigned short*>(grad), static_cast<float*>(table_grad), vocab,
+                       static_cast<int>(dim), ctx->fault, tag);
+  OMX_LAUNCH_CHECK(ctx, "embedding_bwd_kernel");
+  return OMX_OK;
+}
+
+int32_t omx_argmax_rows(omx_ctx* ctx, const void* x, uint64_t rows, uint64_t cols, void* out) {
+  OMX_REQUIRE_CTX(ctx);
+  if (!x || !out) return omx_fail(ctx, OMX_PLACEMENT, "argmax_rows: null device pointer");
+  if (rows == 0 || cols == 0) return omx_fail(ctx, OMX_SHAPE, "argmax_rows: zero-sized axis");
+  if (cols > 0xfffffffeull) return omx_fail(ctx, OMX_OUT_OF_RANGE, "argmax_rows: cols does not fit in u32");
+  hipLaunchKernelGGL(argmax_rows_kernel, dim3(static_cast<unsigned>((rows + 3) / 4)), dim3(ROW_THREADS), 0,
+                     ctx->stream, static_cast<const float*>(x), rows, static_cast<unsigned int>(cols),
+                     static_cast<unsigned int*>(out), ctx->fault, omx_tag(ctx, F_ARGMAX));
+  OMX_LAUNCH_CHECK(ctx, "argmax_rows_kernel");
+  return OMX_OK;
+}
+
+int32_t omx_topk_rows(omx_ctx* ctx, const void* x, uint64_t rows, uint64_t cols, uint64_t k, void* values,
+                      void* ids) {
+  OMX_REQUIRE_CTX(ctx);
+  if (!x || !values || !ids) return omx_fail(ctx, OMX_PLACEMENT, "topk_rows: null device pointer");
+  if (rows == 0 || cols == 0) return omx_fail(ctx, OMX_SHAPE, "topk_rows: zero-sized axis");
+  if (k == 0 || k > cols) return omx_fail(ctx, OMX_SHAPE, "topk_rows: k %llu outside 1..=%llu", (unsigned long long)k,
+                                          (unsigned long long)cols);
+  if (cols > 0xfffffffeull) return omx_fail(ctx, OMX_OUT_OF_RANGE, "topk_rows: cols does not fit in u32");
+  hipLaunchKernelGGL(topk_rows_kernel, dim3(static_cast<unsigned>((rows + 3) / 4)), dim3(ROW_THREADS), 0, ctx->stream,
+                     static_cast<const float*>(x), rows, static_cast<unsigned int>(cols), static_cast<unsigned int>(k),
+                     static_cast<float*>(values), static_cast<unsigned int*>(ids), ctx->fault, omx_tag(ctx, F_TOPK));
+  OMX_LAUNCH_CHECK(ctx, "topk_rows_kernel");
+  return OMX_OK;
+}
+
+}  // extern "C"

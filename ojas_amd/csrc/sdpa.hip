@@ -1,0 +1,398 @@
+// Causal scaled-dot-product attention, forward and backward.
+//
+// Reference semantics: ojas-cpu/src/attn.rs:47-124,176-227 (forward),
+// :437-597 (backward from the saved output and log-sum-exp); trait
+// ojas-core/src/backend.rs:1729-1792. Layout [B, H, T, D]; query t sees keys
+// max(0, t + 1 - window) ..= t; query head h reads KV head h / (H / Hkv);
+// scale = 1 / sqrt(D) formed in f32 (backend.rs:159). lse = max + ln(sum).
+// Backward: P = e^(S - lse), Dr = dO . O, dS = scale * P * (dP - Dr);
+// dQ = dS K, dK = dS^T Q, dV = P^T dO, with the query heads of one KV head
+// summed in ascending head order.
+//
+// Two families of kernels:
+//   * row kernels (this file, first part): one wavefront per query row (or per
+//     key row in the dK/dV pass), any head_dim up to 256, f32 arithmetic. They
+//     serve the f32 tier and every head_dim the MFMA kernels do not cover.
+//   * flash kernels (flash_sdpa.hip): bf16 MFMA tiles for head_dim 64 / 128.
+// Neither forms a T x T matrix; no atomics are used, so results do not depend
+// on scheduling.
+#include "omx_common.h"
+
+int32_t omx_flash_sdpa_forward(omx_ctx* ctx, const void* q, const void* k, const void* v, void* out,
+                               int32_t out_dtype, float* lse, uint64_t batch, uint64_t heads, uint64_t kv_heads,
+                               uint64_t time, uint64_t dim, uint64_t window, float scale, unsigned long long tag);
+int32_t omx_flash_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, const void* v, const void* out,
+                                const float* lse, const void* gy, void* gq, void* gk, void* gv, int32_t grad_dtype,
+                                uint64_t batch, uint64_t heads, uint64_t kv_heads, uint64_t time, uint64_t dim,
+                                uint64_t window, float scale, unsigned long long tag);
+bool omx_flash_sdpa_supports(uint64_t dim, int32_t operand_dtype);
+
+namespace {
+
+constexpr int SD_THREADS = 256;  // 4 waves: 4 rows per block
+constexpr int MAXD = 256;
+
+struct SdpaShape {
+  int batch, heads, kv_heads, time, dim, window, rep;
+  float scale;
+};
+
+__device__ __forceinline__ int first_key(const SdpaShape& s, int t) {
+  return s.window > 0 ? max(0, t + 1 - s.window) : 0;
+}
+__device__ __forceinline__ int last_query(const SdpaShape& s, int j) {
+  // Queries that see key j: j ..= min(T-1, j + window - 1).
+  return s.window > 0 ? min(s.time - 1, j + s.window - 1) : s.time - 1;
+}
+
+// One wave per query row. Lane l scores keys j0 + l of each 64-key block
+// (dot over D from LDS-broadcast q), the block is folded into the running
+// softmax, and lanes then switch to owning output dims for the P.V update.
+template <typename TI, typename TO>
+__global__ __launch_bounds__(SD_THREADS) void sdpa_fwd_rows_kernel(const TI* __restrict__ q, const TI* __restrict__ k,
+                                                                   const TI* __restrict__ v, TO* __restrict__ out,
+                                                                   float* __restrict__ lse, SdpaShape s,
+                                                                   OmxFaultWord* fault, unsigned long long tag) {
+  __shared__ float q_lds[4][MAXD];
+  __shared__ float p_lds[4][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const long row = static_cast<long>(blockIdx.x) * 4 + wave;  // (b*H + h)*T + t
+  const long total = static_cast<long>(s.batch) * s.heads * s.time;
+  if (row >= total) return;
+  const int t = static_cast<int>(row % s.time);
+  const long plane = row / s.time;
+  const int h = static_cast<int>(plane % s.heads), b = static_cast<int>(plane / s.heads);
+  const long kv_plane = static_cast<long>(b) * s.kv_heads + h / s.rep;
+  const TI* qr = q + row * s.dim;
+  const TI* kh = k + kv_plane * s.time * s.dim;
+  const TI* vh = v + kv_plane * s.time * s.dim;
+  const int D = s.dim;
+  for (int d = lane; d < D; d += 64) q_lds[wave][d] = dev_load<TI>(qr, d);
+  constexpr int ND = MAXD / 64;
+  float acc[ND];
+#pragma unroll
+  for (int i = 0; i < ND; ++i) acc[i] = 0.0f;
+  float run_max = -INFINITY, run_sum = 0.0f;
+  bool bad = false;
+  const int j_begin = first_key(s, t), j_end = t + 1;
+  for (int j0 = j_begin; j0 < j_end; j0 += 64) {
+    const int j = j0 + lane;
+    float sc = -INFINITY;
+    if (j < j_end) {
+      const TI* kr = kh + static_cast<long>(j) * D;
+      float dot = 0.0f;
+      for (int d = 0; d < D; ++d) dot += q_lds[wave][d] * dev_load<TI>(kr, d);
+      sc = dot * s.scale;
+      bad |= !dev_finite(sc);
+    }
+    float blk_max = wave_max(sc);
+    float new_max = fmaxf(run_max, blk_max);
+    float p = j < j_end ? expf(sc - new_max) : 0.0f;
+    float blk_sum = wave_sum(p);
+    float rescale = expf(run_max - new_max);  // 0 on the first block (run_max = -inf)
+    run_sum = run_sum * rescale + blk_sum;
+    run_max = new_max;
+    p_lds[wave][lane] = p;
+    // Same-wave LDS traffic: the wave executes in lockstep, a fence orders it.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    const int nk = min(64, j_end - j0);
+#pragma unroll
+    for (int i = 0; i < ND; ++i) {
+      const int d = i * 64 + lane;
+      if (d < D) {
+        float a = acc[i] * rescale;
+        for (int jj = 0; jj < nk; ++jj) a += p_lds[wave][jj] * dev_load<TI>(vh, static_cast<long>(j0 + jj) * D + d);
+        acc[i] = a;
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  bad |= !(dev_finite(run_sum) && run_sum > 0.0f);
+  const float inv = 1.0f / run_sum;
+  TO* orow = out + row * D;
+#pragma unroll
+  for (int i = 0; i < ND; ++i) {
+    const int d = i * 64 + lane;
+    if (d < D) {
+      float o = acc[i] * inv;
+      bad |= !dev_finite(o);
+      dev_store<TO>(orow, d, o);
+    }
+  }
+  if (lane == 0) lse[row] = run_max + logf(run_sum);
+  if (bad) dev_raise_fault(fault, tag);
+}
+
+// Dr[row] = dO[row] . O[row] (f32), one wave per row.
+template <typename TI>
+__global__ __launch_bounds__(SD_THREADS) void sdpa_delta_kernel(const TI* __restrict__ out, const TI* __restrict__ gy,
+                                                                float* __restrict__ delta, long rows, int D) {
+  const int lane = threadIdx.x & 63;
+  const long row = static_cast<long>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  float acc = 0.0f;
+  for (int d = lane; d < D; d += 64) acc += dev_load<TI>(gy, row * D + d) * dev_load<TI>(out, row * D + d);
+  acc = wave_sum(acc);
+  if (lane == 0) delta[row] = acc;
+}
+
+// dQ: one wave per query row, the forward's structure with dS in place of P.
+template <typename TI, typename TO>
+__global__ __launch_bounds__(SD_THREADS) void sdpa_bwd_dq_rows_kernel(
+    const TI* __restrict__ q, const TI* __restrict__ k, const TI* __restrict__ v, const float* __restrict__ lse,
+    const float* __restrict__ delta, const TI* __restrict__ gy, TO* __restrict__ gq, SdpaShape s, OmxFaultWord* fault,
+    unsigned long long tag) {
+  __shared__ float q_lds[4][MAXD];
+  __shared__ float g_lds[4][MAXD];
+  __shared__ float c_lds[4][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const long row = static_cast<long>(blockIdx.x) * 4 + wave;
+  const long total = static_cast<long>(s.batch) * s.heads * s.time;
+  if (row >= total) return;
+  const int t = static_cast<int>(row % s.time);
+  const long plane = row / s.time;
+  const int h = static_cast<int>(plane % s.heads), b = static_cast<int>(plane / s.heads);
+  const long kv_plane = static_cast<long>(b) * s.kv_heads + h / s.rep;
+  const TI* kh = k + kv_plane * s.time * s.dim;
+  const TI* vh = v + kv_plane * s.time * s.dim;
+  const int D = s.dim;
+  for (int d = lane; d < D; d += 64) {
+    q_lds[wave][d] = dev_load<TI>(q, row * D + d);
+    g_lds[wave][d] = dev_load<TI>(gy, row * D + d);
+  }
+  const float row_lse = lse[row], dr = delta[row];
+  bool bad = !(dev_finite(row_lse) && dev_finite(dr));
+  constexpr int ND = MAXD / 64;
+  float acc[ND];
+#pragma unroll
+  for (int i = 0; i < ND; ++i) acc[i] = 0.0f;
+  const int j_begin = first_key(s, t), j_end = t + 1;
+  for (int j0 = j_begin; j0 < j_end; j0 += 64) {
+    const int j = j0 + lane;
+    float coef = 0.0f;
+    if (j < j_end) {
+      const TI* kr = kh + static_cast<long>(j) * D;
+      const TI* vr = vh + static_cast<long>(j) * D;
+      float dot = 0.0f, dp = 0.0f;
+      for (int d = 0; d < D; ++d) {
+        dot += q_lds[wave][d] * dev_load<TI>(kr, d);
+        dp += g_lds[wave][d] * dev_load<TI>(vr, d);
+      }
+      float sc = dot * s.scale;
+      float p = expf(sc - row_lse);
+      bad |= !(dev_finite(sc) && dev_finite(p));
+      coef = s.scale * (p * (dp - dr));
+    }
+    c_lds[wave][lane] = coef;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    const int nk = min(64, j_end - j0);
+#pragma unroll
+    for (int i = 0; i < ND; ++i) {
+      const int d = i * 64 + lane;
+      if (d < D) {
+        float a = acc[i];
+        for (int jj = 0; jj < nk; ++jj) a += c_lds[wave][jj] * dev_load<TI>(kh, static_cast<long>(j0 + jj) * D + d);
+        acc[i] = a;
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+#pragma unroll
+  for (int i = 0; i < ND; ++i) {
+    const int d = i * 64 + lane;
+    if (d < D) {
+      bad |= !dev_finite(acc[i]);
+      dev_store<TO>(gq, row * D + d, acc[i]);
+    }
+  }
+  if (bad) dev_raise_fault(fault, tag);
+}
+
+// dK, dV: one wave per key row of a KV head; walks the query heads of the
+// group in ascending order and, within a head, queries in ascending order.
+template <typename TI, typename TO>
+__global__ __launch_bounds__(SD_THREADS) void sdpa_bwd_dkv_rows_kernel(
+    const TI* __restrict__ q, const TI* __restrict__ k, const TI* __restrict__ v, const float* __restrict__ lse,
+    const float* __restrict__ delta, const TI* __restrict__ gy, TO* __restrict__ gk, TO* __restrict__ gv, SdpaShape s,
+    OmxFaultWord* fault, unsigned long long tag) {
+  __shared__ float k_lds[4][MAXD];
+  __shared__ float v_lds[4][MAXD];
+  __shared__ float c_lds[4][64];
+  __shared__ float p_lds[4][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const long row = static_cast<long>(blockIdx.x) * 4 + wave;  // (b*Hkv + g)*T + j
+  const long total = static_cast<long>(s.batch) * s.kv_heads * s.time;
+  if (row >= total) return;
+  const int j = static_cast<int>(row % s.time);
+  const long kv_plane = row / s.time;
+  const int g = static_cast<int>(kv_plane % s.kv_heads), b = static_cast<int>(kv_plane / s.kv_heads);
+  const int D = s.dim;
+  for (int d = lane; d < D; d += 64) {
+    k_lds[wave][d] = dev_load<TI>(k, row * D + d);
+    v_lds[wave][d] = dev_load<TI>(v, row * D + d);
+  }
+  constexpr int ND = MAXD / 64;
+  float acck[ND], accv[ND];
+#pragma unroll
+  for (int i = 0; i < ND; ++i) acck[i] = accv[i] = 0.0f;
+  bool bad = false;
+  const int t_end = last_query(s, j) + 1;
+  for (int r = 0; r < s.rep; ++r) {
+    const long q_plane = static_cast<long>(b) * s.heads + static_cast<long>(g) * s.rep + r;
+    const TI* qh = q + q_plane * s.time * D;
+    const TI* gh = gy + q_plane * s.time * D;
+    const float* lse_h = lse + q_plane * s.time;
+    const float* del_h = delta + q_plane * s.time;
+    for (int t0 = j; t0 < t_end; t0 += 64) {
+      const int t = t0 + lane;
+      float coef = 0.0f, p = 0.0f;
+      if (t < t_end) {
+        const TI* qr = qh + static_cast<long>(t) * D;
+        const TI* gr = gh + static_cast<long>(t) * D;
+        float dot = 0.0f, dp = 0.0f;
+        for (int d = 0; d < D; ++d) {
+          dot += dev_load<TI>(qr, d) * k_lds[wave][d];
+          dp += dev_load<TI>(gr, d) * v_lds[wave][d];
+        }
+        float sc = dot * s.scale;
+        p = expf(sc - lse_h[t]);
+        bad |= !(dev_finite(sc) && dev_finite(p));
+        coef = s.scale * (p * (dp - del_h[t]));
+      }
+      c_lds[wave][lane] = coef;
+      p_lds[wave][lane] = p;
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      const int nq = min(64, t_end - t0);
+#pragma unroll
+      for (int i = 0; i < ND; ++i) {
+        const int d = i * 64 + lane;
+        if (d < D) {
+          float ak = acck[i], av = accv[i];
+          for (int tt = 0; tt < nq; ++tt) {
+            ak += c_lds[wave][tt] * dev_load<TI>(qh, static_cast<long>(t0 + tt) * D + d);
+            av += p_lds[wave][tt] * dev_load<TI>(gh, static_cast<long>(t0 + tt) * D + d);
+          }
+          acck[i] = ak;
+          accv[i] = av;
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < ND; ++i) {
+    const int d = i * 64 + lane;
+    if (d < D) {
+      bad |= !(dev_finite(acck[i]) && dev_finite(accv[i]));
+      dev_store<TO>(gk, row * D + d, acck[i]);
+      dev_store<TO>(gv, row * D + d, accv[i]);
+    }
+  }
+  if (bad) dev_raise_fault(fault, tag);
+}
+
+int32_t check_shape(omx_ctx* ctx, const char* op, uint64_t batch, uint64_t heads, uint64_t kv_heads, uint64_t time,
+                    uint64_t dim, uint64_t window, SdpaShape* s) {
+  if (batch == 0 || heads == 0 || kv_heads == 0 || time == 0 || dim == 0)
+    return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
+  if (kv_heads > heads || heads % kv_heads != 0)
+    return omx_fail(ctx, OMX_SHAPE, "%s: heads %llu is not a multiple of kv heads %llu", op,
+                    (unsigned long long)heads, (unsigned long long)kv_heads);
+  if (dim > MAXD) return omx_fail(ctx, OMX_UNSUPPORTED_HEAD_DIM, "head_dim %llu limit %d", (unsigned long long)dim, MAXD);
+  if (batch * heads * time > 0x7fffffffull || time > 0x3fffffffull)
+    return omx_fail(ctx, OMX_OUT_OF_RANGE, "%s: B*H*T does not fit in i32", op);
+  s->batch = static_cast<int>(batch);
+  s->heads = static_cast<int>(heads);
+  s->kv_heads = static_cast<int>(kv_heads);
+  s->time = static_cast<int>(time);
+  s->dim = static_cast<int>(dim);
+  // A window of at least T is every earlier key (attn.rs:745).
+  s->window = (window == 0 || window >= time) ? 0 : static_cast<int>(window);
+  s->rep = static_cast<int>(heads / kv_heads);
+  s->scale = 1.0f / sqrtf(static_cast<float>(static_cast<uint32_t>(dim)));
+  return OMX_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t omx_causal_sdpa_forward(omx_ctx* ctx, const void* q, const void* k, const void* v, int32_t operand_dtype,
+                                void* out, int32_t out_dtype, void* lse, uint64_t batch, uint64_t heads,
+                                uint64_t kv_heads, uint64_t time, uint64_t head_dim, uint64_t window) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "causal_sdpa_forward";
+  if (!q || !k || !v || !out || !lse) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  if (!omx_valid_float_dtype(operand_dtype) || !omx_valid_float_dtype(out_dtype))
+    return omx_fail(ctx, OMX_DTYPE, "%s: dtype must be f32 or bf16", op);
+  SdpaShape s;
+  int32_t rc = check_shape(ctx, op, batch, heads, kv_heads, time, head_dim, window, &s);
+  if (rc != OMX_OK) return rc;
+  unsigned long long tag = omx_tag(ctx, F_SDPA_FORWARD);
+  if (omx_flash_sdpa_supports(head_dim, operand_dtype))
+    return omx_flash_sdpa_forward(ctx, q, k, v, out, out_dtype, static_cast<float*>(lse), batch, heads, kv_heads, time,
+                                  head_dim, s.window, s.scale, tag);
+  const long rows = static_cast<long>(batch) * heads * time;
+  dim3 grid(static_cast<unsigned>((rows + 3) / 4)), block(SD_THREADS);
+#define SDPA_FWD(TI, TO)                                                                                          \
+  hipLaunchKernelGGL((sdpa_fwd_rows_kernel<TI, TO>), grid, block, 0, ctx->stream, static_cast<const TI*>(q),      \
+                     static_cast<const TI*>(k), static_cast<const TI*>(v), static_cast<TO*>(out),                 \
+                     static_cast<float*>(lse), s, ctx->fault, tag)
+  if (operand_dtype == OMX_F32 && out_dtype == OMX_F32) SDPA_FWD(float, float);
+  else if (operand_dtype == OMX_F32) SDPA_FWD(float, unsigned short);
+  else if (out_dtype == OMX_F32) SDPA_FWD(unsigned short, float);
+  else SDPA_FWD(unsigned short, unsigned short);
+#undef SDPA_FWD
+  OMX_LAUNCH_CHECK(ctx, "sdpa_fwd_rows_kernel");
+  return OMX_OK;
+}
+
+int32_t omx_causal_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, const void* v, const void* out,
+                                 const void* lse, const void* gy, int32_t operand_dtype, void* gq, void* gk, void* gv,
+                                 int32_t grad_dtype, uint64_t batch, uint64_t heads, uint64_t kv_heads, uint64_t time,
+                                 uint64_t head_dim, uint64_t window) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "causal_sdpa_backward";
+  if (!q || !k || !v || !out || !lse || !gy || !gq || !gk || !gv)
+    return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  if (!omx_valid_float_dtype(operand_dtype) || !omx_valid_float_dtype(grad_dtype))
+    return omx_fail(ctx, OMX_DTYPE, "%s: dtype must be f32 or bf16", op);
+  SdpaShape s;
+  int32_t rc = check_shape(ctx, op, batch, heads, kv_heads, time, head_dim, window, &s);
+  if (rc != OMX_OK) return rc;
+  unsigned long long tag = omx_tag(ctx, F_SDPA_BACKWARD);
+  if (omx_flash_sdpa_supports(head_dim, operand_dtype))
+    return omx_flash_sdpa_backward(ctx, q, k, v, out, static_cast<const float*>(lse), gy, gq, gk, gv, grad_dtype, batch,
+                                   heads, kv_heads, time, head_dim, s.window, s.scale, tag);
+  const long rows = static_cast<long>(batch) * heads * time;
+  const long kv_rows = static_cast<long>(batch) * kv_heads * time;
+  void* ws = nullptr;
+  rc = omx_workspace(ctx, rows * sizeof(float), &ws);
+  if (rc != OMX_OK) return rc;
+  float* delta = static_cast<float*>(ws);
+  dim3 grid(static_cast<unsigned>((rows + 3) / 4)), kv_grid(static_cast<unsigned>((kv_rows + 3) / 4)), block(SD_THREADS);
+  const float* lsef = static_cast<const float*>(lse);
+#define SDPA_BWD(TI, TO)                                                                                              \
+  do {                                                                                                                \
+    hipLaunchKernelGGL((sdpa_delta_kernel<TI>), grid, block, 0, ctx->stream, static_cast<const TI*>(out),             \
+                       static_cast<const TI*>(gy), delta, rows, s.dim);                                               \
+    hipLaunchKernelGGL((sdpa_bwd_dq_rows_kernel<TI, TO>), grid, block, 0, ctx->stream, static_cast<const TI*>(q),     \
+                       static_cast<const TI*>(k), static_cast<const TI*>(v), lsef, delta, static_cast<const TI*>(gy), \
+                       static_cast<TO*>(gq), s, ctx->fault, tag);                                                     \
+    hipLaunchKernelGGL((sdpa_bwd_dkv_rows_kernel<TI, TO>), kv_grid, block, 0, ctx->stream,                            \
+                       static_cast<const TI*>(q), static_cast<const TI*>(k), static_cast<const TI*>(v), lsef, delta,  \
+                       static_cast<const TI*>(gy), static_cast<TO*>(gk), static_cast<TO*>(gv), s, ctx->fault, tag);   \
+  } while (0)
+  if (operand_dtype == OMX_F32 && grad_dtype == OMX_F32) SDPA_BWD(float, float);
+  else if (operand_dtype == OMX_F32) SDPA_BWD(float, unsigned short);
+  else if (grad_dtype == OMX_F32) SDPA_BWD(unsigned short, float);
+  else SDPA_BWD(unsigned short, unsigned short);
+#undef SDPA_BWD
+  OMX_LAUNCH_CHECK(ctx, "sdpa backward row kernels");
+  return OMX_OK;
+}
+
+}  // extern "C"

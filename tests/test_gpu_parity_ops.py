@@ -1,0 +1,437 @@
+"""GPU-vs-oracle parity, one op at a time, through the C ABI.
+
+Template: the reference's GPU-vs-CPU gate (ojas-wgpu/tests/parity.rs:1-6,
+tests/common/mod.rs:11,90-118): every op on shapes that break tiles (1x1,
+primes, 63/64/65, 127/128/129; T = 1, 17, 257) against CPU Exact.
+
+Tolerances (written where used):
+  * integer / bit work (gather, casts, permute, argmax, top-k, embedding
+    scatter-add order): bit-exact;
+  * f32 tier: max|gpu - cpu| <= 1e-5 * max(1, max|cpu|)  (BASELINE "1e-5 relative");
+  * bf16 tier: 2e-2 per element relative to max(1, max|cpu|), inputs rounded to
+    bf16 on both sides so only accumulation order and output rounding differ.
+"""
+import numpy as np
+import pytest
+
+import oracle_api as orc
+
+pytestmark = pytest.mark.gpu
+
+F32_TOL = 1e-5
+BF16_TOL = 2e-2
+
+
+@pytest.fixture(scope="module")
+def be():
+    from ojas_amd.backend import MiBackend
+
+    backend = MiBackend(0)
+    assert backend.device_name().startswith("gfx950")
+    yield backend
+    backend.close()
+
+
+def close(got, want, tol, what=""):
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    assert got.shape == want.shape, (what, got.shape, want.shape)
+    scale = max(1.0, float(np.max(np.abs(want))) if want.size else 1.0)
+    err = float(np.max(np.abs(got - want))) if want.size else 0.0
+    assert np.isfinite(got).all(), f"{what}: non-finite output"
+    assert err <= tol * scale, f"{what}: max err {err:.3e} > {tol:.0e} * {scale:.3e}"
+
+
+def rng_vec(seed, n, scale=1.0):
+    return orc.SplitMix64(seed).vec(n, scale)
+
+
+LINEAR_SHAPES = [(1, 1, 1), (3, 5, 9), (73, 11, 13), (127, 67, 131), (64, 128, 96), (63, 64, 65), (129, 127, 128),
+                 (257, 129, 65), (33, 1000, 17), (200, 300, 520), (256, 256, 768)]
+
+
+@pytest.mark.parametrize("rows,kin,nout", LINEAR_SHAPES)
+def test_linear_f32(be, rows, kin, nout):
+    print(f"linear f32 {rows}x{kin}x{nout}", flush=True)
+    r = orc.SplitMix64(1000 + rows * 7 + kin)
+    x = r.vec(rows * kin, 0.5).reshape(rows, kin)
+    w = r.vec(nout * kin, 0.5).reshape(nout, kin)
+    gy = r.vec(rows * nout, 0.5).reshape(rows, nout)
+    dx, dw, dgy = be.upload(x), be.upload(w), be.upload(gy)
+    y = be.download(be.linear_forward(dx, dw))
+    close(y, orc.linear_forward(x, w), F32_TOL, "linear_forward")
+    gx, gw = be.linear_backward(dx, dw, dgy)
+    ogx, ogw = orc.linear_backward(x, w, gy)
+    close(be.download(gx), ogx, F32_TOL, "linear_backward gx")
+    close(be.download(gw), ogw, F32_TOL, "linear_backward gw")
+    gx_only = be.linear_backward_input(dw, dgy)
+    assert np.array_equal(be.download(gx_only), be.download(gx)), "linear_backward_input bits differ from gx"
+
+
+@pytest.mark.parametrize("rows,kin,nout", LINEAR_SHAPES)
+def test_linear_bf16(be, rows, kin, nout):
+    from ojas_amd.backend import BF16, F32
+
+    print(f"linear bf16 {rows}x{kin}x{nout}", flush=True)
+    r = orc.SplitMix64(2000 + rows * 7 + kin)
+    x = orc.round_bf16(r.vec(rows * kin, 0.5)).reshape(rows, kin)
+    w = orc.round_bf16(r.vec(nout * kin, 0.5)).reshape(nout, kin)
+    gy = orc.round_bf16(r.vec(rows * nout, 0.5)).reshape(rows, nout)
+    dx, dw, dgy = be.upload(x, BF16), be.upload(w, BF16), be.upload(gy, BF16)
+    # f32 output of bf16 operands: exact products, f32 accumulation -> f32-tier tolerance.
+    close(be.download(be.linear_forward(dx, dw)), orc.linear_forward(x, w), F32_TOL, "linear_forward bf16->f32")
+    ybf = be.download_f32(be.linear_forward(dx, dw, out_dtype=BF16))
+    close(ybf, orc.linear_forward(x, w), BF16_TOL, "linear_forward bf16->bf16")
+    gx, gw = be.linear_backward(dx, dw, dgy, gx_dtype=F32)
+    ogx, ogw = orc.linear_backward(x, w, gy)
+    close(be.download(gx), ogx, F32_TOL, "gx")
+    close(be.download(gw), ogw, F32_TOL, "gw")
+
+
+def test_linear_mixed_operands_and_gemm_accumulate(be):
+    from ojas_amd.backend import BF16
+
+    r = orc.SplitMix64(77)
+    x = r.vec(70 * 96, 0.5).reshape(70, 96)
+    w = orc.round_bf16(r.vec(40 * 96, 0.5)).reshape(40, 96)
+    y = be.download(be.linear_forward(be.upload(x), be.upload(w, BF16)))
+    close(y, orc.linear_forward(x, w), F32_TOL, "f32 input, bf16 weight")
+    # gemm_acc: C += A.B continues the stored chain (gemm.rs:365-388).
+    a = r.vec(50 * 30, 0.5).reshape(50, 30)
+    b = r.vec(30 * 20, 0.5).reshape(30, 20)
+    c0 = r.vec(50 * 20, 0.5).reshape(50, 20)
+    dc = be.upload(c0)
+    be.gemm(be.upload(a), (30, 1), be.upload(b), (20, 1), 50, 30, 20, c=dc)
+    close(be.download(dc), orc.gemm(a, b, c0), F32_TOL, "gemm accumulate")
+
+
+@pytest.mark.parametrize("rows,dim", [(1, 1), (5, 64), (300, 256), (17, 63), (9, 65), (130, 768), (4, 1000), (3, 2048)])
+def test_rms_norm_f32(be, rows, dim):
+    print(f"rms {rows}x{dim}", flush=True)
+    r = orc.SplitMix64(400 + rows + dim)
+    x = r.vec(rows * dim, 1.0).reshape(rows, dim)
+    w = (np.float32(1.0) + r.vec(dim, 0.1)).astype(np.float32)
+    gy = r.vec(rows * dim, 1.0).reshape(rows, dim)
+    dx, dw, dgy = be.upload(x), be.upload(w), be.upload(gy)
+    close(be.download(be.rms_norm_forward(dx, dw, 1e-6)), orc.rms_norm_forward(x, w, 1e-6), F32_TOL, "rms fwd")
+    gx, gw = be.rms_norm_backward(dx, dw, dgy, 1e-6)
+    ogx, ogw = orc.rms_norm_backward(x, w, gy, 1e-6)
+    close(be.download(gx), ogx, F32_TOL, "rms gx")
+    close(be.download(gw), ogw, F32_TOL, "rms gw")
+
+
+def test_rms_norm_bf16_storage(be):
+    from ojas_amd.backend import BF16
+
+    rows, dim = 70, 768
+    r = orc.SplitMix64(4242)
+    x = orc.round_bf16(r.vec(rows * dim, 1.0)).reshape(rows, dim)
+    w = (np.float32(1.0) + r.vec(dim, 0.1)).astype(np.float32)
+    gy = orc.round_bf16(r.vec(rows * dim, 1.0)).reshape(rows, dim)
+    y = be.download_f32(be.rms_norm_forward(be.upload(x, BF16), be.upload(w)))
+    close(y, orc.rms_norm_forward(x, w), BF16_TOL, "rms fwd bf16")
+    gx, gw = be.rms_norm_backward(be.upload(x, BF16), be.upload(w), be.upload(gy, BF16))
+    ogx, ogw = orc.rms_norm_backward(x, w, gy)
+    close(be.download_f32(gx), ogx, BF16_TOL, "rms gx bf16")
+    close(be.download(gw), ogw, 1e-4, "rms gw (f32 sums of bf16 inputs)")
+
+
+@pytest.mark.parametrize("tokens,vocab,dim", [(1, 1, 1), (12, 10, 8), (257, 500, 64), (1000, 37, 65), (64, 8192, 256)])
+def test_embedding_is_bit_exact(be, tokens, vocab, dim):
+    print(f"embedding {tokens} {vocab} {dim}", flush=True)
+    r = orc.SplitMix64(31 + tokens)
+    table = r.vec(vocab * dim, 1.0).reshape(vocab, dim)
+    table[0, 0] = -0.0
+    ids = np.array([r.below(vocab) for _ in range(tokens)], dtype=np.uint32)
+    grad = r.vec(tokens * dim, 1.0).reshape(tokens, dim)
+    out = be.download(be.embedding_forward(be.upload(table), be.upload(ids)))
+    assert np.array_equal(out.view(np.uint32), orc.embedding_forward(table, ids).view(np.uint32))
+    # Scatter-add in ascending token order: the same f32 sums, so the same bits.
+    tg = be.download(be.embedding_backward(be.upload(ids), be.upload(grad), vocab))
+    assert np.array_equal(tg.view(np.uint32), orc.embedding_backward(ids, grad, vocab).view(np.uint32))
+
+
+def test_embedding_heavy_collisions_and_bf16_table(be):
+    from ojas_amd.backend import BF16
+
+    tokens, vocab, dim = 700, 3, 96
+    r = orc.SplitMix64(5)
+    ids = np.array([r.below(vocab) for _ in range(tokens)], dtype=np.uint32)
+    grad = r.vec(tokens * dim, 1.0).reshape(tokens, dim)
+    tg = be.download(be.embedding_backward(be.upload(ids), be.upload(grad), vocab))
+    assert np.array_equal(tg.view(np.uint32), orc.embedding_backward(ids, grad, vocab).view(np.uint32))
+    table = orc.round_bf16(r.vec(vocab * dim, 1.0)).reshape(vocab, dim)
+    out = be.download(be.embedding_forward(be.upload(table, BF16), be.upload(ids)))
+    assert np.array_equal(out.view(np.uint32), orc.embedding_forward(table, ids).view(np.uint32))
+
+
+def test_embedding_out_of_range_id_is_reported_at_sync(be):
+    from ojas_amd.backend import OUT_OF_RANGE, OjasError
+
+    table = be.upload(np.ones((4, 8), np.float32))
+    ids = be.upload(np.array([0, 9, 1], np.uint32))
+    be.embedding_forward(table, ids)
+    with pytest.raises(OjasError) as e:
+        be.sync()
+    assert e.value.code == OUT_OF_RANGE and "embedding_forward" in e.value.detail
+    be.sync()  # the fault word was cleared
+
+
+@pytest.mark.parametrize("rows,vocab", [(1, 1), (1, 2), (257, 500), (17, 1023), (5, 8192), (3, 50304)])
+def test_cross_entropy_f32(be, rows, vocab):
+    print(f"ce {rows}x{vocab}", flush=True)
+    r = orc.SplitMix64(600 + rows)
+    logits = r.vec(rows * vocab, 4.0).reshape(rows, vocab)
+    targets = np.array([7 % vocab if i % 11 == 3 else r.below(vocab) for i in range(rows)], dtype=np.uint32)
+    ignore = 7 if vocab > 8 and rows > 4 else None
+    dl, dt = be.upload(logits), be.upload(targets)
+    loss = be.download(be.cross_entropy_mean_forward(dl, dt, ignore))[0]
+    want = orc.cross_entropy_mean_forward(logits, targets, ignore)
+    assert abs(float(loss) - float(want)) <= F32_TOL * max(1.0, abs(float(want)))
+    grad = be.download(be.cross_entropy_mean_backward(dl, dt, ignore))
+    og = orc.cross_entropy_mean_backward(logits, targets, ignore)
+    close(grad, og, F32_TOL, "ce grad")
+    # Invariant: every valid row of the gradient sums to 0 (numerical_invariants.rs T1).
+    assert np.max(np.abs(grad.astype(np.float64).sum(axis=1))) < 1e-6
+
+
+def test_cross_entropy_collapse_row_and_all_ignored(be):
+    from ojas_amd.backend import NON_FINITE, OjasError
+
+    # A planted margin: the target logit dominates by 60, so the plain softmax
+    # gradient of the target rounds to 0 and the collapse rule takes over.
+    rows, vocab = 4, 300
+    r = orc.SplitMix64(9)
+    logits = r.vec(rows * vocab, 1.0).reshape(rows, vocab)
+    targets = np.array([3, 100, 7, 299], np.uint32)
+    logits[1, 100] = 60.0
+    dl, dt = be.upload(logits), be.upload(targets)
+    loss = be.download(be.cross_entropy_mean_forward(dl, dt))[0]
+    want = orc.cross_entropy_mean_forward(logits, targets)
+    assert abs(float(loss) - float(want)) <= F32_TOL * max(1.0, abs(float(want)))
+    grad = be.download(be.cross_entropy_mean_backward(dl, dt))
+    og = orc.cross_entropy_mean_backward(logits, targets)
+    close(grad, og, F32_TOL, "ce grad")
+    assert grad[1, 100] < 0.0, "collapse rule keeps a non-zero target gradient"
+    rel = abs(grad[1, 100] - og[1, 100]) / abs(og[1, 100])
+    assert rel < 1e-4, rel
+    # All rows ignored: NonFinite, reported at the next sync.
+    dt2 = be.upload(np.full(rows, 5, np.uint32))
+    be.cross_entropy_mean_forward(dl, dt2, 5)
+    with pytest.raises(OjasError) as e:
+        be.sync()
+    assert e.value.code == NON_FINITE and "cross_entropy_mean_forward" in e.value.detail
+
+
+@pytest.mark.parametrize("rows,dim,vocab,chunk", [(10, 16, 300, (1024, 8192)), (70, 48, 1000, (32, 256)),
+                                                  (129, 64, 513, (64, 8192)), (33, 24, 97, (7, 40))])
+def test_linear_cross_entropy_matches_composed_path(be, rows, dim, vocab, chunk):
+    print(f"linear_ce {rows} {dim} {vocab} {chunk}", flush=True)
+    r = orc.SplitMix64(800 + rows)
+    x = r.vec(rows * dim, 1.0).reshape(rows, dim)
+    w = r.vec(vocab * dim, 0.3).reshape(vocab, dim)
+    targets = np.array([r.below(vocab) for _ in range(rows)], np.uint32)
+    targets[::5] = 2
+    loss, gx, gw = be.linear_cross_entropy_mean(be.upload(x), be.upload(w), be.upload(targets), 2, chunk)
+    oloss, ogx, ogw = orc.linear_cross_entropy_mean(x, w, targets, 2)
+    assert abs(float(be.download(loss)[0]) - float(oloss)) <= F32_TOL * max(1.0, abs(float(oloss)))
+    close(be.download(gx), ogx, F32_TOL, "fused gx")
+    close(be.download(gw), ogw, F32_TOL, "fused gw")
+    # Loss alone and one gradient alone (CeGrads::EACH).
+    l2, g2, w2 = be.linear_cross_entropy_mean(be.upload(x), be.upload(w), be.upload(targets), 2, chunk, (False, False))
+    assert g2 is None and w2 is None
+    assert abs(float(be.download(l2)[0]) - float(oloss)) <= F32_TOL * max(1.0, abs(float(oloss)))
+    _, g3, w3 = be.linear_cross_entropy_mean(be.upload(x), be.upload(w), be.upload(targets), 2, chunk, (True, False))
+    assert w3 is None
+    close(be.download(g3), ogx, F32_TOL, "fused gx alone")
+
+
+SDPA_SHAPES = [([2, 3, 33, 24], 3, None), ([1, 2, 300, 64], 2, None), ([2, 2, 64, 16], 2, None),
+               ([1, 1, 1, 8], 1, None), ([1, 2, 17, 64], 2, None), ([1, 4, 257, 32], 2, None),
+               ([1, 4, 130, 64], 1, 40), ([2, 2, 65, 128], 2, 7)]
+
+
+@pytest.mark.parametrize("shape,hkv,window", SDPA_SHAPES)
+def test_causal_sdpa_f32(be, shape, hkv, window):
+    print(f"sdpa f32 {shape} hkv {hkv} window {window}", flush=True)
+    b, h, t, d = shape
+    r = orc.SplitMix64(300 + t + d)
+    q = r.vec(b * h * t * d, 0.5).reshape(b, h, t, d)
+    k = r.vec(b * hkv * t * d, 0.5).reshape(b, hkv, t, d)
+    v = r.vec(b * hkv * t * d, 0.5).reshape(b, hkv, t, d)
+    gy = r.vec(b * h * t * d, 0.5).reshape(b, h, t, d)
+    oy, olse = orc.causal_sdpa_forward(q, k, v, window or 0)
+    ogq, ogk, ogv = orc.causal_sdpa_backward(q, k, v, oy, olse, gy, window or 0)
+    dq, dk, dv, dgy = be.upload(q), be.upload(k), be.upload(v), be.upload(gy)
+    y, lse = be.causal_sdpa_forward(dq, dk, dv, window)
+    close(be.download(y), oy, F32_TOL, "sdpa out")
+    close(be.download(lse), olse, F32_TOL, "sdpa lse")
+    gq, gk, gv = be.causal_sdpa_backward(dq, dk, dv, y, lse, dgy, window)
+    close(be.download(gq), ogq, F32_TOL, "sdpa gq")
+    close(be.download(gk), ogk, F32_TOL, "sdpa gk")
+    close(be.download(gv), ogv, F32_TOL, "sdpa gv")
+
+
+def test_adamw_matches_fast_f32_contract_bitwise_and_exact_within_1e6(be):
+    from ojas_amd.backend import AdamWConfig
+
+    n = 100_003
+    r = orc.SplitMix64(700)
+    p, g, m1 = r.vec(n, 1.0), r.vec(n, 0.1), r.vec(n, 0.01)
+    m2 = np.abs(r.vec(n, 0.01))
+    dp, dg, dm1, dm2 = be.upload(p), be.upload(g), be.upload(m1), be.upload(m2)
+    be.adamw_step(dp, dg, dm1, dm2, 9, AdamWConfig.nanolab(3e-3, 0.1))
+    fp, fm1, fm2 = orc.adamw_step(p, g, m1, m2, 9, 3e-3, 0.9, 0.95, 1e-8, 0.1, exact=False)
+    ep, em1, em2 = orc.adamw_step(p, g, m1, m2, 9, 3e-3, 0.9, 0.95, 1e-8, 0.1, exact=True)
+    gp, gm1, gm2 = be.download(dp), be.download(dm1), be.download(dm2)
+    # Same f32 operations in the same order as the CPU Fast contract (optim.rs:302-395).
+    for got, fast, name in ((gp, fp, "p"), (gm1, fm1, "m1"), (gm2, fm2, "m2")):
+        close(got, fast, 2e-7, f"adamw {name} vs Fast")
+    # Fast-vs-Exact gate of the reference: 1e-6 (ojas-cpu/src/lib.rs:57).
+    for got, exact, name in ((gp, ep, "p"), (gm1, em1, "m1"), (gm2, em2, "m2")):
+        close(got, exact, 1e-6, f"adamw {name} vs Exact")
+
+
+def test_adamw_writes_nothing_when_any_value_is_non_finite(be):
+    from ojas_amd.backend import NON_FINITE, AdamWConfig, OjasError
+
+    n = 5000
+    r = orc.SplitMix64(3)
+    p, g, m1 = r.vec(n, 1.0), r.vec(n, 0.1), r.vec(n, 0.01)
+    m2 = np.abs(r.vec(n, 0.01))
+    g[4321] = np.inf
+    dp, dg, dm1, dm2 = be.upload(p), be.upload(g), be.upload(m1), be.upload(m2)
+    be.adamw_step(dp, dg, dm1, dm2, 0, AdamWConfig.nanolab(1e-3, 0.0))
+    with pytest.raises(OjasError) as e:
+        be.sync()
+    assert e.value.code == NON_FINITE and "adamw_step" in e.value.detail
+    assert np.array_equal(be.download(dp), p) and np.array_equal(be.download(dm1), m1)
+    assert np.array_equal(be.download(dm2), m2)
+
+
+def test_adamw_config_refusals(be):
+    from ojas_amd.backend import NON_FINITE, OUT_OF_RANGE, AdamWConfig, OjasError
+
+    t = be.upload(np.ones(8, np.float32))
+    for cfg, code in ((AdamWConfig(1e-3, 1.0, 0.95, 1e-8, 0.0), OUT_OF_RANGE),
+                      (AdamWConfig(-1e-3, 0.9, 0.95, 1e-8, 0.0), OUT_OF_RANGE),
+                      (AdamWConfig(1e-3, 0.9, 0.95, 0.0, 0.0), OUT_OF_RANGE),
+                      (AdamWConfig(float("nan"), 0.9, 0.95, 1e-8, 0.0), NON_FINITE)):
+        with pytest.raises(OjasError) as e:
+            be.adamw_step(t, t, t, t, 0, cfg)
+        assert e.value.code == code
+    with pytest.raises(OjasError) as e:
+        be.adamw_step(t, t, t, t, 2**64 - 1, AdamWConfig.nanolab(1e-3, 0.0))
+    assert e.value.code == OUT_OF_RANGE
+
+
+def test_clip_grad_norm(be):
+    r = orc.SplitMix64(11)
+    grads = [r.vec(n, 1.0) for n in (1, 1000, 70_001, 300_000)]
+    for max_norm in (1.0, 1e9):
+        dg = [be.upload(g) for g in grads]
+        norm = be.clip_grad_norm(dg, max_norm)
+        onorm, oclipped = orc.clip_grad_norm(grads, max_norm)
+        assert abs(norm - float(onorm)) <= 1e-6 * float(onorm)
+        for got, want in zip(dg, oclipped):
+            close(be.download(got), want, 1e-6, "clipped grad")
+    # No clipping leaves the bits alone.
+    dg = [be.upload(g) for g in grads]
+    be.clip_grad_norm(dg, 1e9)
+    for got, want in zip(dg, grads):
+        assert np.array_equal(be.download(got), want)
+
+
+def test_elementwise_ops(be):
+    n = 70_001
+    r = orc.SplitMix64(21)
+    x, y = r.vec(n, 3.0), r.vec(n, 3.0)
+    dx, dy = be.upload(x), be.upload(y)
+    assert np.array_equal(be.download(be.residual_add_forward(dx, dy)), orc.residual_add(x, y))
+    acc = be.upload(x)
+    be.accumulate_grad(acc, dy)
+    assert np.array_equal(be.download(acc), x + y)
+    be.scale_grad(acc, 0.25)
+    assert np.array_equal(be.download(acc), (x + y) * np.float32(0.25))
+    close(be.download(be.gelu_erf_forward(dx)), orc.gelu_erf_forward(x), F32_TOL, "gelu erf")
+    close(be.download(be.gelu_erf_backward(dx, dy)), orc.gelu_erf_backward_vec(x, y), F32_TOL, "gelu erf bwd")
+    close(be.download(be.gelu_tanh_forward(dx)), orc.gelu_tanh_forward(x), F32_TOL, "gelu tanh")
+    close(be.download(be.gelu_tanh_backward(dx, dy)), orc.gelu_tanh_backward_vec(x, y), F32_TOL, "gelu tanh bwd")
+
+
+def test_casts_and_permute_are_bit_exact(be):
+    from ojas_amd.backend import BF16
+
+    r = orc.SplitMix64(55)
+    x = r.vec(10_007, 100.0)
+    special = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1.0 + 2.0**-8, 1.0 + 2.0**-8 + 2.0**-20, 3.3895e38,
+                        -3.4e38, 1e-40], np.float32)
+    nan_payload = np.array([0x7F800001, 0xFFC12345, 0x7FBFFFFF], np.uint32).view(np.float32)
+    x = np.concatenate([x, special, nan_payload]).astype(np.float32)
+    dx = be.upload(x)
+    assert np.array_equal(be.download(be.to_bf16(dx)), orc.to_bf16(x))
+    assert np.array_equal(be.download(be.cast_bf16(dx)).view(np.uint32), orc.round_bf16(x).view(np.uint32))
+    bits = orc.to_bf16(x)
+    assert np.array_equal(be.download(be.to_f32(be.upload(bits))).view(np.uint32), orc.bf16_to_f32(bits).view(np.uint32))
+    for shape in ([2, 3, 5, 7], [1, 64, 4, 64], [2, 17, 3, 16]):
+        a = r.vec(int(np.prod(shape)), 1.0).reshape(shape)
+        got = be.download(be.permute(be.upload(a), [0, 2, 1, 3]))
+        assert np.array_equal(got, orc.permute_0213(a)) and np.array_equal(got, a.transpose(0, 2, 1, 3))
+        gb = be.download(be.permute(be.upload(a, BF16), [0, 2, 1, 3]))
+        assert np.array_equal(gb, orc.to_bf16(a).transpose(0, 2, 1, 3))
+
+
+def test_argmax_and_topk_are_bit_exact(be):
+    from ojas_amd.backend import NON_FINITE, OjasError
+
+    r = orc.SplitMix64(91)
+    for rows, cols, k in ((1, 1, 1), (7, 65, 5), (33, 1000, 50), (4, 50304, 8)):
+        x = np.round(r.vec(rows * cols, 8.0)).reshape(rows, cols).astype(np.float32)  # many ties
+        x[0, 0] = -0.0
+        if cols > 3:
+            x[0, 3] = 0.0
+        dx = be.upload(x)
+        assert np.array_equal(be.download(be.argmax_rows(dx)), orc.argmax_rows(x))
+        xv = x.copy()
+        if cols > 2:
+            xv[-1, 1] = -np.inf  # allowed by top-k, sorts last
+        vals, ids = be.topk_rows(be.upload(xv), k)
+        ov, oi = orc.topk_rows(xv, k)
+        assert np.array_equal(be.download(ids), oi)
+        assert np.array_equal(be.download(vals).view(np.uint32), ov.view(np.uint32))
+    bad = np.ones((2, 9), np.float32)
+    bad[1, 4] = np.nan
+    be.argmax_rows(be.upload(bad))
+    with pytest.raises(OjasError) as e:
+        be.sync()
+    assert e.value.code == NON_FINITE and "argmax_rows" in e.value.detail
+
+
+def test_deferred_non_finite_names_the_first_faulting_op(be):
+    from ojas_amd.backend import NON_FINITE, OjasError
+
+    x = np.ones((4, 8), np.float32)
+    x[2, 3] = np.nan
+    w = np.ones((5, 8), np.float32)
+    dx, dw = be.upload(x), be.upload(w)
+    y = be.linear_forward(dx, dw)            # first fault
+    be.residual_add_forward(y, y)            # second fault, later in recording order
+    with pytest.raises(OjasError) as e:
+        be.download(y)
+    assert e.value.code == NON_FINITE and e.value.detail == "linear_forward"
+
+
+def test_budget_refuses_rather_than_clamps_and_unsupported_ops_name_themselves(be):
+    from ojas_amd.backend import CAPACITY_EXCEEDED, UNSUPPORTED, MiBackend, OjasError
+
+    small = MiBackend(0, budget_bytes=1 << 20)
+    a = small.empty((100_000,))
+    assert small.budget()["live"] == 400_000
+    with pytest.raises(OjasError) as e:
+        small.empty((200_000,))
+    assert e.value.code == CAPACITY_EXCEEDED
+    del a
+    assert small.budget()["live"] == 0 and small.budget()["peak"] == 400_000
+    with pytest.raises(OjasError) as e:
+        small.layer_norm_forward(None, None)
+    assert e.value.code == UNSUPPORTED and "layer_norm_forward" in e.value.detail
+    small.close()
