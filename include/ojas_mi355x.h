@@ -201,9 +201,11 @@ int32_t omx_clip_grad_norm(omx_ctx* ctx, void* const* grads_f32, const uint64_t*
                            uint64_t count, float max_norm, float* norm_out);
 
 /* ---- elementwise and layout ---- */
-/* BackendFloat::residual_add_forward (backend.rs:1165-1173). */
-int32_t omx_residual_add(omx_ctx* ctx, const void* x, const void* y, void* out, int32_t dtype,
-                         uint64_t n);
+/* BackendFloat::residual_add_forward (backend.rs:1165-1173): out = x + y, one
+ * rounding per element. The operands may differ in storage (an f32 residual
+ * stream plus a bf16 branch output). */
+int32_t omx_residual_add(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* y, int32_t y_dtype,
+                         void* out, int32_t out_dtype, uint64_t n);
 /* BackendFloat::accumulate_grad / scale_grad (backend.rs:1473-1510). */
 int32_t omx_accumulate_grad(omx_ctx* ctx, void* acc_f32, const void* grad_f32, uint64_t n);
 int32_t omx_scale_grad(omx_ctx* ctx, void* grad_f32, float scale, uint64_t n);

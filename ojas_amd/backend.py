@@ -389,12 +389,13 @@ class MiBackend:
         return float(norm.value)
 
     # ---- elementwise / layout ----
-    def residual_add_forward(self, x, y):
-        if x.dtype != y.dtype or x.shape != y.shape:
+    def residual_add_forward(self, x, y, out_dtype: Optional[int] = None):
+        if x.shape != y.shape:
             raise OjasError(SHAPE, "residual_add_forward: operands differ")
-        out = self.empty(x.shape, x.dtype)
-        self._check(self._lib.omx_residual_add(self._ctx, self._p(x), self._p(y), self._p(out), C.c_int32(x.dtype),
-                                               C.c_uint64(x.numel)))
+        od = x.dtype if out_dtype is None else out_dtype
+        out = self.empty(x.shape, od)
+        self._check(self._lib.omx_residual_add(self._ctx, self._p(x), C.c_int32(x.dtype), self._p(y),
+                                               C.c_int32(y.dtype), self._p(out), C.c_int32(od), C.c_uint64(x.numel)))
         return out
 
     def accumulate_grad(self, acc, grad):

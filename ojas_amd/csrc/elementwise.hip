@@ -38,14 +38,14 @@ __global__ void fill_zero_kernel(unsigned int* __restrict__ p, size_t words, uns
   if (blockIdx.x == 0 && threadIdx.x < tail_bytes) tail[threadIdx.x] = 0;
 }
 
-template <typename T>
-__global__ void add_kernel(const T* __restrict__ x, const T* __restrict__ y, T* __restrict__ out, size_t n,
+template <typename TX, typename TY, typename TO>
+__global__ void add_kernel(const TX* __restrict__ x, const TY* __restrict__ y, TO* __restrict__ out, size_t n,
                            OmxFaultWord* fault, unsigned long long tag) {
   bool bad = false;
   EW_LOOP(i, n) {
-    float v = dev_load<T>(x, i) + dev_load<T>(y, i);
+    float v = dev_load<TX>(x, i) + dev_load<TY>(y, i);
     bad |= !dev_finite(v);
-    dev_store<T>(out, i, v);
+    dev_store<TO>(out, i, v);
   }
   if (bad) dev_raise_fault(fault, tag);
 }
@@ -195,20 +195,31 @@ int32_t omx_to_f32(omx_ctx* ctx, const void* x, void* y, uint64_t n) {
   return omx_convert(ctx, x, OMX_BF16, y, OMX_F32, n);
 }
 
-int32_t omx_residual_add(omx_ctx* ctx, const void* x, const void* y, void* out, int32_t dtype, uint64_t n) {
+int32_t omx_residual_add(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* y, int32_t y_dtype, void* out,
+                         int32_t out_dtype, uint64_t n) {
   OMX_REQUIRE_CTX(ctx);
   if (!x || !y || !out) return omx_fail(ctx, OMX_PLACEMENT, "residual_add_forward: null device pointer");
-  if (!omx_valid_float_dtype(dtype)) return omx_fail(ctx, OMX_DTYPE, "residual_add_forward: dtype must be f32 or bf16");
+  if (!omx_valid_float_dtype(x_dtype) || !omx_valid_float_dtype(y_dtype) || !omx_valid_float_dtype(out_dtype))
+    return omx_fail(ctx, OMX_DTYPE, "residual_add_forward: dtype must be f32 or bf16");
   if (n == 0) return omx_fail(ctx, OMX_SHAPE, "residual_add_forward: zero-sized axis");
   unsigned long long tag = omx_tag(ctx, F_RESIDUAL_ADD);
-  if (dtype == OMX_F32)
-    hipLaunchKernelGGL((add_kernel<float>), ew_grid(n), dim3(EW_THREADS), 0, ctx->stream,
-                       static_cast<const float*>(x), static_cast<const float*>(y), static_cast<float*>(out), n,
-                       ctx->fault, tag);
-  else
-    hipLaunchKernelGGL((add_kernel<unsigned short>), ew_grid(n), dim3(EW_THREADS), 0, ctx->stream,
-                       static_cast<const unsigned short*>(x), static_cast<const unsigned short*>(y),
-                       static_cast<unsigned short*>(out), n, ctx->fault, tag);
+  dim3 grid = ew_grid(n), block(EW_THREADS);
+#define ADD_K(TX, TY, TO)                                                                                   \
+  hipLaunchKernelGGL((add_kernel<TX, TY, TO>), grid, block, 0, ctx->stream, static_cast<const TX*>(x),      \
+                     static_cast<const TY*>(y), static_cast<TO*>(out), n, ctx->fault, tag)
+  typedef unsigned short h16;
+  const int key = (x_dtype == OMX_BF16 ? 4 : 0) | (y_dtype == OMX_BF16 ? 2 : 0) | (out_dtype == OMX_BF16 ? 1 : 0);
+  switch (key) {
+    case 0: ADD_K(float, float, float); break;
+    case 1: ADD_K(float, float, h16); break;
+    case 2: ADD_K(float, h16, float); break;
+    case 3: ADD_K(float, h16, h16); break;
+    case 4: ADD_K(h16, float, float); break;
+    case 5: ADD_K(h16, float, h16); break;
+    case 6: ADD_K(h16, h16, float); break;
+    default: ADD_K(h16, h16, h16); break;
+  }
+#undef ADD_K
   OMX_LAUNCH_CHECK(ctx, "add_kernel");
   return OMX_OK;
 }

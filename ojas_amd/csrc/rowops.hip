@@ -437,19 +437,23 @@ int32_t omx_rms_norm_backward(omx_ctx* ctx, const void* x, int32_t x_dtype, cons
   if (!x || !w || !gy || !gx || !gw) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
   if (!omx_valid_float_dtype(x_dtype) || !omx_valid_float_dtype(gy_dtype) || !omx_valid_float_dtype(gx_dtype))
     return omx_fail(ctx, OMX_DTYPE, "%s: dtype must be f32 or bf16", op);
-  if (gy_dtype != gx_dtype) return omx_fail(ctx, OMX_DTYPE, "%s: grad dtypes differ", op);
   if (rows == 0 || dim == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
   if (!(eps == eps) || eps == INFINITY || eps == -INFINITY) return omx_fail(ctx, OMX_NON_FINITE, "%s", op);
   unsigned long long tag = omx_tag(ctx, F_RMS_BACKWARD);
   const float* wf = static_cast<const float*>(w);
   float* gwf = static_cast<float*>(gw);
-  if (x_dtype == OMX_F32 && gy_dtype == OMX_F32)
-    return launch_rms_bwd<float, float, float>(ctx, x, wf, gy, gx, gwf, rows, dim, eps, tag);
-  if (x_dtype == OMX_BF16 && gy_dtype == OMX_BF16)
-    return launch_rms_bwd<unsigned short, unsigned short, unsigned short>(ctx, x, wf, gy, gx, gwf, rows, dim, eps, tag);
-  if (x_dtype == OMX_F32)
-    return launch_rms_bwd<float, unsigned short, unsigned short>(ctx, x, wf, gy, gx, gwf, rows, dim, eps, tag);
-  return launch_rms_bwd<unsigned short, float, float>(ctx, x, wf, gy, gx, gwf, rows, dim, eps, tag);
+  typedef unsigned short h16;
+  const int key = (x_dtype == OMX_BF16 ? 4 : 0) | (gy_dtype == OMX_BF16 ? 2 : 0) | (gx_dtype == OMX_BF16 ? 1 : 0);
+  switch (key) {
+    case 0: return launch_rms_bwd<float, float, float>(ctx, x, wf, gy, gx, gwf, rows, dim, eps, tag);
+    case 1: return launch_rms_bwd<float, float, h16>(ctx, x, wf, gy, gx, gwf, rows, dim, eps, tag);
+    case 2: return launch_rms_bwd<float, h16, float>(ctx, x, wf, gy, gx, gwf, rows, dim, eps, tag);
+    case 3: return launch_rms_bwd<float, h16, h16>(ctx, x, wf, gy, gx, gwf, rows, dim, eps, tag);
+    case 4: return launch_rms_bwd<h16, float, float>(ctx, x, wf, gy, gx, gwf, rows, dim, eps, tag);
+    case 5: return launch_rms_bwd<h16, float, h16>(ctx, x, wf, gy, gx, gwf, rows, dim, eps, tag);
+    case 6: return launch_rms_bwd<h16, h16, float>(ctx, x, wf, gy, gx, gwf, rows, dim, eps, tag);
+    default: return launch_rms_bwd<h16, h16, h16>(ctx, x, wf, gy, gx, gwf, rows, dim, eps, tag);
+  }
 }
 
 int32_t omx_embedding_forward(omx_ctx* ctx, const void* table, int32_t table_dtype, const void* ids, void* out,

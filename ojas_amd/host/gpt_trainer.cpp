@@ -1,0 +1,382 @@
+// Host-side training-step driver above the C ABI (see include/ojas_gpt.h).
+//
+// Orchestration only: every tensor operation is one omx_* call, in the order
+// the reference's tape would replay the same graph (forward in program order,
+// backward in reverse with gradient fan-in added later-consumer-first,
+// ojas-autograd/src/tape.rs:2004-2466,2565-2591), then the step of
+// ojas-model/src/trainer.rs:754-1046: clip_grad_norm (sync point), adamw_step,
+// sync + one scalar readback.
+//
+// All buffers are allocated once at creation: parameters, gradients and AdamW
+// moments live in flat f32 arenas (one clip pass and one AdamW pass cover every
+// tensor), the bf16 tier keeps a bf16 mirror of the parameters that AdamW
+// refreshes, and saved activations have one slot per layer.
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <random>
+#include <string>
+#include <vector>
+
+#include "ojas_gpt.h"
+
+namespace {
+
+constexpr uint64_t kAlign = 64;  // elements; keeps every tensor 256-byte aligned in both arenas
+
+struct Slot {
+  uint64_t offset, len;
+};
+
+}  // namespace
+
+struct ogpt {
+  omx_ctx* ctx = nullptr;
+  ogpt_config c{};
+  uint64_t N = 0, P = 0;  // tokens per batch, padded parameter count
+  std::vector<Slot> slots;
+  int32_t AD = OMX_F32;  // activation / operand dtype
+  uint64_t asz = 4;
+  uint64_t steps = 0;
+  uint64_t device_bytes = 0;
+  std::vector<void*> owned;
+
+  float *p32 = nullptr, *g32 = nullptr, *m1 = nullptr, *m2 = nullptr;
+  void* p16 = nullptr;
+  uint32_t *ids = nullptr, *targets = nullptr, *positions = nullptr;
+  float* loss = nullptr;
+
+  // Per-layer saved activations.
+  struct Layer {
+    float *x, *x1;                          // residual stream (f32)
+    void *h1, *q, *k, *v, *a, *ap, *h2, *u, *g;  // AD
+    float* lse;
+  };
+  std::vector<Layer> layers;
+  float* x_final = nullptr;  // residual stream after the last layer
+  void* hf = nullptr;        // final norm output (AD)
+  // Scratch.
+  float *e_tok = nullptr, *e_pos = nullptr;
+  void *t_a = nullptr, *t_b = nullptr;       // [N,d] AD
+  void *gu = nullptr, *gg = nullptr;         // [N,mlp] AD
+  void *gq = nullptr, *gk = nullptr, *gv = nullptr, *ga = nullptr;  // [N,d] AD
+  void* gy16 = nullptr;                      // AD copy of a residual-stream gradient
+  float *gres = nullptr, *gres1 = nullptr, *gt = nullptr, *gh = nullptr;  // [N,d] f32
+  float* g_emb = nullptr;                    // [V,d] f32
+  void* ghf = nullptr;                       // [N,d] AD
+
+  // Parameter views.
+  const void* w(uint64_t i) const {
+    return AD == OMX_BF16 ? static_cast<const void*>(static_cast<const uint16_t*>(p16) + slots[i].offset)
+                          : static_cast<const void*>(p32 + slots[i].offset);
+  }
+  const float* w32(uint64_t i) const { return p32 + slots[i].offset; }
+  float* g(uint64_t i) const { return g32 + slots[i].offset; }
+  uint64_t li(uint64_t l, uint64_t which) const { return 2 + l * 8 + which; }
+  uint64_t nf() const { return 2 + static_cast<uint64_t>(c.layers) * 8; }
+};
+
+namespace {
+
+#define TRY(expr)                    \
+  do {                               \
+    int32_t rc_ = (expr);            \
+    if (rc_ != OMX_OK) return rc_;   \
+  } while (0)
+
+int32_t alloc(ogpt* t, uint64_t bytes, void** out) {
+  TRY(omx_alloc(t->ctx, bytes, out));
+  t->owned.push_back(*out);
+  t->device_bytes += bytes;
+  return OMX_OK;
+}
+template <typename T>
+int32_t alloc_t(ogpt* t, uint64_t count, T** out) {
+  void* p = nullptr;
+  TRY(alloc(t, count * sizeof(T), &p));
+  *out = static_cast<T*>(p);
+  return OMX_OK;
+}
+int32_t alloc_act(ogpt* t, uint64_t count, void** out) { return alloc(t, count * t->asz, out); }
+
+// AD copy of an f32 tensor: the f32 tier aliases it, the bf16 tier rounds it.
+int32_t to_operand(ogpt* t, const float* src, void* scratch, uint64_t n, const void** out) {
+  if (t->AD == OMX_F32) {
+    *out = src;
+    return OMX_OK;
+  }
+  TRY(omx_to_bf16(t->ctx, src, scratch, n));
+  *out = scratch;
+  return OMX_OK;
+}
+
+int32_t forward(ogpt* t) {
+  omx_ctx* ctx = t->ctx;
+  const ogpt_config& c = t->c;
+  const uint64_t N = t->N, d = c.d_model, M = c.mlp, B = c.batch, T = c.ctx, H = c.heads, D = c.head_dim;
+  const int32_t AD = t->AD;
+  const float eps = 1e-6f;
+  TRY(omx_embedding_forward(ctx, t->w32(0), OMX_F32, t->ids, t->e_tok, OMX_F32, N, c.vocab, d));
+  TRY(omx_embedding_forward(ctx, t->w32(1), OMX_F32, t->positions, t->e_pos, OMX_F32, N, T, d));
+  float* x = t->layers.empty() ? t->x_final : t->layers[0].x;
+  TRY(omx_residual_add(ctx, t->e_tok, OMX_F32, t->e_pos, OMX_F32, x, OMX_F32, N * d));
+  for (uint32_t l = 0; l < c.layers; ++l) {
+    ogpt::Layer& A = t->layers[l];
+    float* x_next = (l + 1 < c.layers) ? t->layers[l + 1].x : t->x_final;
+    TRY(omx_rms_norm_forward(ctx, A.x, OMX_F32, t->w32(t->li(l, 0)), A.h1, AD, N, d, eps));
+    TRY(omx_linear_forward(ctx, A.h1, AD, t->w(t->li(l, 1)), AD, t->t_a, AD, N, d, d));
+    TRY(omx_permute_0213(ctx, t->t_a, A.q, AD, B, T, H, D));
+    TRY(omx_linear_forward(ctx, A.h1, AD, t->w(t->li(l, 2)), AD, t->t_a, AD, N, d, d));
+    TRY(omx_permute_0213(ctx, t->t_a, A.k, AD, B, T, H, D));
+    TRY(omx_linear_forward(ctx, A.h1, AD, t->w(t->li(l, 3)), AD, t->t_a, AD, N, d, d));
+    TRY(omx_permute_0213(ctx, t->t_a, A.v, AD, B, T, H, D));
+    TRY(omx_causal_sdpa_forward(ctx, A.q, A.k, A.v, AD, A.a, AD, A.lse, B, H, H, T, D, 0));
+    TRY(omx_permute_0213(ctx, A.a, A.ap, AD, B, H, T, D));
+    TRY(omx_linear_forward(ctx, A.ap, AD, t->w(t->li(l, 4)), AD, t->t_a, AD, N, d, d));
+    TRY(omx_residual_add(ctx, A.x, OMX_F32, t->t_a, AD, A.x1, OMX_F32, N * d));
+    TRY(omx_rms_norm_forward(ctx, A.x1, OMX_F32, t->w32(t->li(l, 5)), A.h2, AD, N, d, eps));
+    TRY(omx_linear_forward(ctx, A.h2, AD, t->w(t->li(l, 6)), AD, A.u, AD, N, d, M));
+    TRY(omx_gelu_forward(ctx, A.u, A.g, AD, N * M, c.gelu_tanh));
+    TRY(omx_linear_forward(ctx, A.g, AD, t->w(t->li(l, 7)), AD, t->t_a, AD, N, M, d));
+    TRY(omx_residual_add(ctx, A.x1, OMX_F32, t->t_a, AD, x_next, OMX_F32, N * d));
+  }
+  TRY(omx_rms_norm_forward(ctx, t->x_final, OMX_F32, t->w32(t->nf()), t->hf, AD, N, d, eps));
+  return OMX_OK;
+}
+
+int32_t backward(ogpt* t) {
+  omx_ctx* ctx = t->ctx;
+  const ogpt_config& c = t->c;
+  const uint64_t N = t->N, d = c.d_model, M = c.mlp, B = c.batch, T = c.ctx, H = c.heads, D = c.head_dim;
+  const int32_t AD = t->AD;
+  const float eps = 1e-6f;
+  // Tied head: loss, grad of the final norm output, and the head's share of the table gradient.
+  // One row block of the whole vocabulary at a time: no logits are recomputed.
+  const uint64_t chunk_rows = N < 4096 ? N : 4096;
+  TRY(omx_linear_cross_entropy_mean(ctx, t->hf, t->w(0), AD, t->targets, N, d, c.vocab, 0, 0, chunk_rows, c.vocab,
+                                    t->loss, t->ghf, AD, t->g(0)));
+  TRY(omx_rms_norm_backward(ctx, t->x_final, OMX_F32, t->w32(t->nf()), t->ghf, AD, t->gres, OMX_F32, t->g(t->nf()), N, d,
+                            eps));
+  for (uint32_t l = c.layers; l-- > 0;) {
+    ogpt::Layer& A = t->layers[l];
+    const void* gy = nullptr;
+    // x_next = x1 + down(gelu(up(norm2(x1))))
+    TRY(to_operand(t, t->gres, t->gy16, N * d, &gy));
+    TRY(omx_linear_backward(ctx, A.g, t->w(t->li(l, 7)), gy, AD, t->gg, AD, t->g(t->li(l, 7)), OMX_F32, N, M, d));
+    TRY(omx_gelu_backward(ctx, A.u, t->gg, t->gu, AD, N * M, c.gelu_tanh));
+    TRY(omx_linear_backward(ctx, A.h2, t->w(t->li(l, 6)), t->gu, AD, t->t_a, AD, t->g(t->li(l, 6)), OMX_F32, N, d, M));
+    TRY(omx_rms_norm_backward(ctx, A.x1, OMX_F32, t->w32(t->li(l, 5)), t->t_a, AD, t->gt, OMX_F32, t->g(t->li(l, 5)), N,
+                              d, eps));
+    // Fan-in at x1: the residual branch arrives first, then the norm branch.
+    TRY(omx_residual_add(ctx, t->gres, OMX_F32, t->gt, OMX_F32, t->gres1, OMX_F32, N * d));
+    // x1 = x + o(attention)
+    TRY(to_operand(t, t->gres1, t->gy16, N * d, &gy));
+    TRY(omx_linear_backward(ctx, A.ap, t->w(t->li(l, 4)), gy, AD, t->t_a, AD, t->g(t->li(l, 4)), OMX_F32, N, d, d));
+    TRY(omx_permute_0213(ctx, t->t_a, t->ga, AD, B, T, H, D));
+    TRY(omx_causal_sdpa_backward(ctx, A.q, A.k, A.v, A.a, A.lse, t->ga, AD, t->gq, t->gk, t->gv, AD, B, H, H, T, D, 0));
+    // h1 feeds q, k, v; their gradients arrive v first, then k, then q.
+    TRY(omx_permute_0213(ctx, t->gv, t->t_a, AD, B, H, T, D));
+    TRY(omx_linear_backward(ctx, A.h1, t->w(t->li(l, 3)), t->t_a, AD, t->t_b, AD, t->g(t->li(l, 3)), OMX_F32, N, d, d));
+    TRY(omx_permute_0213(ctx, t->gk, t->t_a, AD, B, H, T, D));
+    TRY(omx_linear_backward(ctx, A.h1, t->w(t->li(l, 2)), t->t_a, AD, t->ga, AD, t->g(t->li(l, 2)), OMX_F32, N, d, d));
+    TRY(omx_residual_add(ctx, t->t_b, AD, t->ga, AD, t->gh, OMX_F32, N * d));
+    TRY(omx_permute_0213(ctx, t->gq, t->t_a, AD, B, H, T, D));
+    TRY(omx_linear_backward(ctx, A.h1, t->w(t->li(l, 1)), t->t_a, AD, t->ga, AD, t->g(t->li(l, 1)), OMX_F32, N, d, d));
+    TRY(omx_residual_add(ctx, t->gh, OMX_F32, t->ga, AD, t->gh, OMX_F32, N * d));
+    TRY(omx_rms_norm_backward(ctx, A.x, OMX_F32, t->w32(t->li(l, 0)), t->gh, OMX_F32, t->gt, OMX_F32,
+                              t->g(t->li(l, 0)), N, d, eps));
+    TRY(omx_residual_add(ctx, t->gres1, OMX_F32, t->gt, OMX_F32, t->gres, OMX_F32, N * d));
+  }
+  // x0 = tok[ids] + pos[positions]; the tied table adds the embedding's share to the head's.
+  TRY(omx_embedding_backward(ctx, t->positions, t->gres, OMX_F32, t->g(1), N, T, d));
+  TRY(omx_embedding_backward(ctx, t->ids, t->gres, OMX_F32, t->g_emb, N, c.vocab, d));
+  TRY(omx_accumulate_grad(ctx, t->g(0), t->g_emb, static_cast<uint64_t>(c.vocab) * d));
+  return OMX_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t ogpt_create(omx_ctx* ctx, const ogpt_config* config, ogpt** out) {
+  if (!ctx || !config || !out) return OMX_BACKEND;
+  *out = nullptr;
+  const ogpt_config& c = *config;
+  if (c.d_model == 0 || c.heads == 0 || c.head_dim == 0 || c.mlp == 0 || c.ctx == 0 || c.vocab == 0 || c.batch == 0)
+    return OMX_SHAPE;
+  if (static_cast<uint64_t>(c.heads) * c.head_dim != c.d_model) return OMX_SHAPE;
+  ogpt* t = new ogpt();
+  t->ctx = ctx;
+  t->c = c;
+  t->N = static_cast<uint64_t>(c.batch) * c.ctx;
+  t->AD = c.bf16 ? OMX_BF16 : OMX_F32;
+  t->asz = c.bf16 ? 2 : 4;
+  const uint64_t d = c.d_model, M = c.mlp, N = t->N;
+  auto push = [&](uint64_t len) {
+    t->slots.push_back({t->P, len});
+    t->P += (len + kAlign - 1) / kAlign * kAlign;
+  };
+  push(static_cast<uint64_t>(c.vocab) * d);
+  push(static_cast<uint64_t>(c.ctx) * d);
+  for (uint32_t l = 0; l < c.layers; ++l) {
+    push(d);
+    for (int i = 0; i < 4; ++i) push(d * d);
+    push(d);
+    push(M * d);
+    push(d * M);
+  }
+  push(d);
+  auto fail = [&](int32_t rc) {
+    ogpt_destroy(t);
+    return rc;
+  };
+#define CREATE_TRY(expr)                 \
+  do {                                   \
+    int32_t rc_ = (expr);                \
+    if (rc_ != OMX_OK) return fail(rc_); \
+  } while (0)
+  CREATE_TRY(alloc_t(t, t->P, &t->p32));
+  CREATE_TRY(alloc_t(t, t->P, &t->g32));
+  CREATE_TRY(alloc_t(t, t->P, &t->m1));
+  CREATE_TRY(alloc_t(t, t->P, &t->m2));
+  CREATE_TRY(omx_fill_zero(ctx, t->p32, t->P * 4));
+  CREATE_TRY(omx_fill_zero(ctx, t->g32, t->P * 4));
+  CREATE_TRY(omx_fill_zero(ctx, t->m1, t->P * 4));
+  CREATE_TRY(omx_fill_zero(ctx, t->m2, t->P * 4));
+  if (c.bf16) {
+    CREATE_TRY(alloc(t, t->P * 2, &t->p16));
+    CREATE_TRY(omx_fill_zero(ctx, t->p16, t->P * 2));
+  }
+  CREATE_TRY(alloc_t(t, N, &t->ids));
+  CREATE_TRY(alloc_t(t, N, &t->targets));
+  CREATE_TRY(alloc_t(t, N, &t->positions));
+  CREATE_TRY(alloc_t(t, 4, &t->loss));
+  {
+    std::vector<uint32_t> pos(N);
+    for (uint64_t i = 0; i < N; ++i) pos[i] = static_cast<uint32_t>(i % c.ctx);
+    CREATE_TRY(omx_upload(ctx, t->positions, 0, pos.data(), N * 4));
+  }
+  t->layers.resize(c.layers);
+  for (auto& A : t->layers) {
+    CREATE_TRY(alloc_t(t, N * d, &A.x));
+    CREATE_TRY(alloc_t(t, N * d, &A.x1));
+    CREATE_TRY(alloc_act(t, N * d, &A.h1));
+    CREATE_TRY(alloc_act(t, N * d, &A.q));
+    CREATE_TRY(alloc_act(t, N * d, &A.k));
+    CREATE_TRY(alloc_act(t, N * d, &A.v));
+    CREATE_TRY(alloc_act(t, N * d, &A.a));
+    CREATE_TRY(alloc_act(t, N * d, &A.ap));
+    CREATE_TRY(alloc_act(t, N * d, &A.h2));
+    CREATE_TRY(alloc_act(t, N * M, &A.u));
+    CREATE_TRY(alloc_act(t, N * M, &A.g));
+    CREATE_TRY(alloc_t(t, static_cast<uint64_t>(c.batch) * c.heads * c.ctx, &A.lse));
+  }
+  CREATE_TRY(alloc_t(t, N * d, &t->x_final));
+  CREATE_TRY(alloc_act(t, N * d, &t->hf));
+  CREATE_TRY(alloc_t(t, N * d, &t->e_tok));
+  CREATE_TRY(alloc_t(t, N * d, &t->e_pos));
+  CREATE_TRY(alloc_act(t, N * d, &t->t_a));
+  CREATE_TRY(alloc_act(t, N * d, &t->t_b));
+  CREATE_TRY(alloc_act(t, N * M, &t->gu));
+  CREATE_TRY(alloc_act(t, N * M, &t->gg));
+  CREATE_TRY(alloc_act(t, N * d, &t->gq));
+  CREATE_TRY(alloc_act(t, N * d, &t->gk));
+  CREATE_TRY(alloc_act(t, N * d, &t->gv));
+  CREATE_TRY(alloc_act(t, N * d, &t->ga));
+  CREATE_TRY(alloc_act(t, N * d, &t->gy16));
+  CREATE_TRY(alloc_act(t, N * d, &t->ghf));
+  CREATE_TRY(alloc_t(t, N * d, &t->gres));
+  CREATE_TRY(alloc_t(t, N * d, &t->gres1));
+  CREATE_TRY(alloc_t(t, N * d, &t->gt));
+  CREATE_TRY(alloc_t(t, N * d, &t->gh));
+  CREATE_TRY(alloc_t(t, static_cast<uint64_t>(c.vocab) * d, &t->g_emb));
+#undef CREATE_TRY
+  *out = t;
+  return OMX_OK;
+}
+
+void ogpt_destroy(ogpt* t) {
+  if (!t) return;
+  for (void* p : t->owned) omx_free(t->ctx, p);
+  delete t;
+}
+
+uint64_t ogpt_param_count(ogpt* t) { return t ? t->slots.size() : 0; }
+uint64_t ogpt_param_len(ogpt* t, uint64_t index) { return (t && index < t->slots.size()) ? t->slots[index].len : 0; }
+uint64_t ogpt_steps(ogpt* t) { return t ? t->steps : 0; }
+uint64_t ogpt_device_bytes(ogpt* t) { return t ? t->device_bytes : 0; }
+
+int32_t ogpt_set_param(ogpt* t, uint64_t index, const float* host) {
+  if (!t || index >= t->slots.size() || !host) return OMX_SHAPE;
+  const Slot& s = t->slots[index];
+  TRY(omx_upload(t->ctx, t->p32, s.offset * 4, host, s.len * 4));
+  if (t->p16) TRY(omx_to_bf16(t->ctx, t->p32 + s.offset, static_cast<uint16_t*>(t->p16) + s.offset, s.len));
+  return OMX_OK;
+}
+int32_t ogpt_get_param(ogpt* t, uint64_t index, float* host) {
+  if (!t || index >= t->slots.size() || !host) return OMX_SHAPE;
+  const Slot& s = t->slots[index];
+  return omx_download(t->ctx, host, t->p32, s.offset * 4, s.len * 4);
+}
+int32_t ogpt_get_grad(ogpt* t, uint64_t index, float* host) {
+  if (!t || index >= t->slots.size() || !host) return OMX_SHAPE;
+  const Slot& s = t->slots[index];
+  return omx_download(t->ctx, host, t->g32, s.offset * 4, s.len * 4);
+}
+
+int32_t ogpt_init(ogpt* t, uint64_t seed) {
+  if (!t) return OMX_BACKEND;
+  std::mt19937_64 rng(seed);
+  std::normal_distribution<float> normal(0.0f, 0.02f);
+  std::vector<float> host;
+  for (uint64_t i = 0; i < t->slots.size(); ++i) {
+    const Slot& s = t->slots[i];
+    host.resize(s.len);
+    const bool is_norm = s.len == t->c.d_model;
+    for (auto& v : host) v = is_norm ? 1.0f : normal(rng);
+    TRY(ogpt_set_param(t, i, host.data()));
+  }
+  TRY(omx_fill_zero(t->ctx, t->m1, t->P * 4));
+  TRY(omx_fill_zero(t->ctx, t->m2, t->P * 4));
+  t->steps = 0;
+  return omx_sync(t->ctx);
+}
+
+int32_t ogpt_set_batch(ogpt* t, const uint32_t* ids, const uint32_t* targets) {
+  if (!t || !ids || !targets) return OMX_BACKEND;
+  TRY(omx_upload(t->ctx, t->ids, 0, ids, t->N * 4));
+  TRY(omx_upload(t->ctx, t->targets, 0, targets, t->N * 4));
+  return OMX_OK;
+}
+
+int32_t ogpt_loss_and_grads(ogpt* t, float* loss) {
+  if (!t) return OMX_BACKEND;
+  TRY(forward(t));
+  TRY(backward(t));
+  float l = 0.0f;
+  TRY(omx_read_scalar_f32(t->ctx, t->loss, &l));
+  if (loss) *loss = l;
+  return OMX_OK;
+}
+
+int32_t ogpt_step(ogpt* t, const omx_adamw_config* adamw, float grad_clip, float* loss, float* grad_norm) {
+  if (!t || !adamw) return OMX_BACKEND;
+  TRY(forward(t));
+  TRY(backward(t));
+  // Sync point 1: the global gradient norm is a host value (trainer.rs:821-824).
+  void* grads[1] = {t->g32};
+  uint64_t lens[1] = {t->P};
+  float norm = 0.0f;
+  TRY(omx_clip_grad_norm(t->ctx, grads, lens, 1, grad_clip > 0.0f ? grad_clip : INFINITY, &norm));
+  // One AdamW pass over the arena covers every tensor; the bf16 mirror is refreshed in the same pass.
+  TRY(omx_adamw_step(t->ctx, t->p32, t->g32, t->m1, t->m2, t->P, t->steps, adamw, t->p16));
+  // Sync point 2: sync + the step's one readback (trainer.rs:1031-1046).
+  float l = 0.0f;
+  TRY(omx_read_scalar_f32(t->ctx, t->loss, &l));
+  t->steps += 1;
+  if (loss) *loss = l;
+  if (grad_norm) *grad_norm = norm;
+  return OMX_OK;
+}
+
+}  // extern "C"
