@@ -1,0 +1,137 @@
+#!/usr/bin/env python3
+"""Benchmark: train tokens/s of the GPT-124M-shape bf16 AdamW step on one MI355X.
+
+One "step" is one full optimizer step (forward, backward, clip_grad_norm, AdamW,
+loss readback) of the GPT-2-shaped model of BASELINE.json configs[2]
+(12 layers, d_model 768, 12 heads of 64, MLP 3072, ctx 1024, vocab 50304,
+batch 16 = 16384 tokens), bf16 operands with f32 master weights, on synthetic
+tokens that are resident in HBM before the clock starts.
+
+Prints one JSON line. `roofline` covers the dominant kernel, the bf16 MFMA GEMM:
+algorithmic 2*M*N*K FLOPs of its launches divided by their summed duration,
+measured with HIP events on the library's own stream during the timed steps.
+`cpu_baseline` times the CPU oracle (a C++ restatement of the reference's CPU
+Exact arithmetic; the Rust reference cannot be built without cargo) on the
+host cores, on a bounded sample of the same workload.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, vendor figure
+
+
+def cpu_baseline(cfg, threads: int):
+    """Times the oracle on a bounded sample: the same model on a 1 x 256 token batch
+    (forward + backward + clip + AdamW), reported per token."""
+    sys.path.insert(0, str(ROOT / "tests"))
+    import oracle_api as orc
+    from ojas_amd.trainer import GptConfig, synthetic_batch
+
+    sample = GptConfig(cfg.layers, cfg.d_model, cfg.heads, cfg.head_dim, cfg.mlp, 256, cfg.vocab, 1, cfg.gelu_tanh, 0)
+    ocfg = orc.GptConfig(sample.layers, sample.d_model, sample.heads, sample.head_dim, sample.mlp, sample.ctx,
+                         sample.vocab, sample.batch, sample.gelu_tanh)
+    orc.set_threads(threads)
+    rng = np.random.default_rng(0)
+    params = [np.ones(n, np.float32) if n == sample.d_model else rng.normal(0, 0.02, n).astype(np.float32)
+              for n in orc.gpt_param_lens(ocfg)]
+    ids, targets = synthetic_batch(sample, 1)
+    t0 = time.perf_counter()
+    _, grads = orc.gpt_loss_and_grads(ocfg, params, ids.reshape(-1), targets.reshape(-1))
+    _, grads = orc.clip_grad_norm(grads, 1.0)
+    for p, g in zip(params, grads):
+        orc.adamw_step(p, g, np.zeros_like(p), np.zeros_like(p), 0, 3e-4, 0.9, 0.95, 1e-8, 0.1, exact=True)
+    dt = time.perf_counter() - t0
+    tokens = sample.batch * sample.ctx
+    return {"value": tokens / dt, "unit": "tokens/s", "cores": threads, "kind": "port",
+            "sample": f"same 124M-shape model, one step on 1x{sample.ctx} tokens in f32 Exact arithmetic "
+                      f"({dt:.1f} s), scaled per token; C++ restatement of ojas-cpu, not the Rust binary"}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--config", default="gpt124m", choices=["gpt124m", "tiny"])
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).", file=sys.stderr)
+        return 2
+
+    from ojas_amd.backend import AdamWConfig, MiBackend
+    from ojas_amd.trainer import GptTrainer, config_gpt124m_bf16, config_tiny_f32, step_flops, synthetic_batch
+
+    cfg = config_gpt124m_bf16() if args.config == "gpt124m" else config_tiny_f32()
+    be = MiBackend(0)
+    tr = GptTrainer(be, cfg)
+    tr.init(1234)
+    ids, targets = synthetic_batch(cfg, 42)
+    tr.set_batch(ids, targets)
+    adamw = AdamWConfig.nanolab(3e-4, 0.1)
+    losses = []
+    for _ in range(args.warmup):
+        losses.append(tr.step(adamw, 1.0)[0])
+    be.sync()
+    lib = be._lib
+    lib.omx_profile_gemm(be._ctx, C.c_int32(1))
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        losses.append(tr.step(adamw, 1.0)[0])
+    be.sync()
+    dt = time.perf_counter() - t0
+    launches, gemm_ms, gemm_flops = C.c_uint64(), C.c_double(), C.c_double()
+    lib.omx_profile_gemm_report(be._ctx, C.byref(launches), C.byref(gemm_ms), C.byref(gemm_flops))
+    lib.omx_profile_gemm(be._ctx, C.c_int32(0))
+
+    tokens = cfg.batch * cfg.ctx
+    ms_per_step = dt / args.steps * 1e3
+    value = tokens * args.steps / dt
+    flops = step_flops(cfg)
+    achieved = gemm_flops.value / (gemm_ms.value * 1e-3) / 1e12 if gemm_ms.value > 0 else 0.0
+    out = {
+        "metric": "train tokens/s on 1 MI355X (GPT-124M bf16 AdamW step); % bf16 MFMA peak",
+        "value": value,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if cfg.bf16 else "f32",
+        "data": "synthetic",
+        "config": {"workload": "GPT-124M-shape training step (BASELINE configs[2]): L12 d768 H12x64 mlp3072 ctx1024 "
+                               "vocab50304 batch16, bf16 operands, f32 master weights, AdamW lr3e-4 wd0.1, clip 1.0"
+                   if args.config == "gpt124m" else "nanolab-GPT tiny f32 step (BASELINE configs[0])",
+                   "tokens_per_step": tokens, "params": sum(tr.param_lens())},
+        "step_tflops": flops / (ms_per_step * 1e-3) / 1e12,
+        "pct_bf16_mfma_peak": 100.0 * flops / (ms_per_step * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS,
+        "loss_first": losses[0], "loss_last": losses[-1],
+        "roofline": {"bound": "mfma", "kernel": "gemm_kernel (bf16 MFMA, all operand layouts)",
+                     "achieved": achieved, "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / BF16_MFMA_PEAK_TFLOPS, "traffic": None,
+                     "launches": int(launches.value), "avg_launch_us": gemm_ms.value * 1e3 / max(1, launches.value),
+                     "gemm_ms_per_step": gemm_ms.value / args.steps},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(cfg, min(16, os.cpu_count() or 1))
+    tr.close()
+    be.close()
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -231,6 +231,15 @@ int32_t omx_topk_rows(omx_ctx* ctx, const void* x_f32, uint64_t rows, uint64_t c
  * ojas-model/src/trainer.rs:1031-1046). */
 int32_t omx_read_scalar_f32(omx_ctx* ctx, const void* src, float* out);
 
+/* Benchmark instrumentation (no counterpart in the reference, whose benches
+ * time whole ops from the host, bench/README.md:59): while enabled, every
+ * launch of the MFMA GEMM kernel is bracketed by two HIP events on the
+ * context's stream. The report waits for the stream, sums the launches'
+ * durations and their 2*M*N*K FLOPs, and clears the record. */
+int32_t omx_profile_gemm(omx_ctx* ctx, int32_t enable);
+int32_t omx_profile_gemm_report(omx_ctx* ctx, uint64_t* launches, double* total_ms,
+                                double* total_flops);
+
 /* Every Backend method outside the GPT op set answers through this: sets the
  * error text to the op's name and returns OMX_UNSUPPORTED
  * (unsupported_op, backend.rs:792-797). */

@@ -1,15 +1,500 @@
-// bf16 MFMA flash attention for head_dim 64 / 128 (placeholder until the
-// tiled kernels land: every shape currently takes the row kernels).
+// bf16 MFMA flash attention for head_dim 64: causal forward, and the backward
+// as two passes (dK/dV per key block, dQ per query block) that recompute the
+// probabilities from the saved log-sum-exp, so no T x T matrix exists and no
+// atomics are needed (the sums of one output never leave one wavefront).
+//
+// Reference semantics: ojas-cpu/src/attn.rs:176-227 (forward rows), :519-597
+// (backward from saved output and lse); the blocked CPU kernel
+// ojas-cpu/src/attn/flash.rs:1-41 is the Fast-tier precedent for this shape of
+// algorithm (online softmax, delta = sum P dP).
+//
+// Mapping onto v_mfma_f32_32x32x16_bf16 (A: lane (i = l%32, g = l/32) holds
+// A[i][8g..8g+7]; B: lane (j, g) holds B[8g..8g+7][j]; D: lane (j, g), register
+// v holds D[8(v/4) + 4g + v%4][j]):
+//   * scores are formed transposed, S^T = K . Q^T (forward, dQ pass), or plain,
+//     S = Q . K^T (dK/dV pass), so that the index a softmax statistic belongs to
+//     (the query in the first case, nothing per-lane in the second) is the
+//     lane's column and every row reduction stays inside a lane plus one
+//     exchange with lane l^32;
+//   * an accumulator tile is reused directly as the B operand of the next
+//     product (P^T for O^T = V^T P^T, P / dS for dV^T, dK^T, dS^T for dQ^T):
+//     registers 8c..8c+7 of a lane are k-slab c, holding rows
+//     16c + {4g..4g+3, 8+4g..8+4g+3}; the A operand stored transposed in LDS
+//     keeps its k index in the matching order (bits 2 and 3 of the index
+//     swapped), so one 16-byte LDS read fetches exactly those rows.
 #include "omx_common.h"
 
-bool omx_flash_sdpa_supports(uint64_t, int32_t) { return false; }
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-int32_t omx_flash_sdpa_forward(omx_ctx* ctx, const void*, const void*, const void*, void*, int32_t, float*, uint64_t,
-                               uint64_t, uint64_t, uint64_t, uint64_t, uint64_t, float, unsigned long long) {
-  return omx_fail(ctx, OMX_UNSUPPORTED, "flash sdpa forward");
+namespace {
+
+constexpr int FD = 64;              // head dim
+constexpr int FPITCH = 144;         // bytes per LDS row: 64 bf16 + 16 pad
+constexpr int FTILE = 64 * FPITCH;  // a 64-row tile
+constexpr int FT = 256;             // threads per block (4 waves of 32 rows)
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float LN2 = 0.6931471805599453f;
+
+struct FlashShape {
+  int batch, heads, kv_heads, time, window, rep;
+  float scale;
+};
+
+__device__ __forceinline__ int perm16(int k) { return (k & ~12) | ((k & 4) << 1) | ((k & 8) >> 1); }
+
+__device__ __forceinline__ unsigned int pack2(float a, float b) {
+  floatx2 f = {a, b};
+  return __builtin_bit_cast(unsigned int, __builtin_convertvector(f, bf16x2));
 }
-int32_t omx_flash_sdpa_backward(omx_ctx* ctx, const void*, const void*, const void*, const void*, const float*,
-                                const void*, void*, void*, void*, int32_t, uint64_t, uint64_t, uint64_t, uint64_t,
-                                uint64_t, uint64_t, float, unsigned long long) {
-  return omx_fail(ctx, OMX_UNSUPPORTED, "flash sdpa backward");
+__device__ __forceinline__ u32x4 pack8(const floatx16& acc, int c) {
+  u32x4 r;
+  r.x = pack2(acc[8 * c + 0], acc[8 * c + 1]);
+  r.y = pack2(acc[8 * c + 2], acc[8 * c + 3]);
+  r.z = pack2(acc[8 * c + 4], acc[8 * c + 5]);
+  r.w = pack2(acc[8 * c + 6], acc[8 * c + 7]);
+  return r;
+}
+__device__ __forceinline__ floatx16 mfma(const u32x4& a, const u32x4& b, floatx16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
+                                                 0, 0);
+}
+__device__ __forceinline__ floatx16 zero16() {
+  floatx16 z;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) z[v] = 0.0f;
+  return z;
+}
+
+// A 64-row x 64-column bf16 tile starting at row `row0` of a [time, 64] plane.
+// Thread t moves rows 2(t>>3) and 2(t>>3)+1, 16-byte chunk t&7; rows at or
+// past `time` read as zeros.
+__device__ __forceinline__ void tile_load(const unsigned short* __restrict__ plane, int row0, int time, u32x4 r[2]) {
+  const int t = threadIdx.x;
+  const int row = row0 + 2 * (t >> 3), kc = t & 7;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    r[i] = u32x4{0u, 0u, 0u, 0u};
+    if (row + i < time) r[i] = *reinterpret_cast<const u32x4*>(plane + static_cast<long>(row + i) * FD + kc * 8);
+  }
+}
+// [row][d] form.
+__device__ __forceinline__ void tile_store_rows(char* lds, const u32x4 r[2]) {
+  const int t = threadIdx.x;
+  const int row = 2 * (t >> 3), kc = t & 7;
+  *reinterpret_cast<u32x4*>(lds + row * FPITCH + kc * 16) = r[0];
+  *reinterpret_cast<u32x4*>(lds + (row + 1) * FPITCH + kc * 16) = r[1];
+}
+// [d][row'] form, row' = perm16(row): the two rows a thread holds stay adjacent.
+__device__ __forceinline__ void tile_store_transposed(char* lds, const u32x4 r[2]) {
+  const int t = threadIdx.x;
+  const int row = 2 * (t >> 3), kc = t & 7;
+  const int col_bytes = perm16(row) * 2;
+  const unsigned int a[4] = {r[0].x, r[0].y, r[0].z, r[0].w};
+  const unsigned int b[4] = {r[1].x, r[1].y, r[1].z, r[1].w};
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    // Elements 2w and 2w+1 of both rows.
+    unsigned int lo = (a[w] & 0xffffu) | (b[w] << 16);
+    unsigned int hi = (a[w] >> 16) | (b[w] & 0xffff0000u);
+    *reinterpret_cast<unsigned int*>(lds + (kc * 8 + 2 * w) * FPITCH + col_bytes) = lo;
+    *reinterpret_cast<unsigned int*>(lds + (kc * 8 + 2 * w + 1) * FPITCH + col_bytes) = hi;
+  }
+}
+// A operand from a [row][d] tile: rows sub*32 + lane%32, d-slab kk.
+__device__ __forceinline__ u32x4 frag_rows(const char* lds, int sub, int kk, int l32, int lg) {
+  return *reinterpret_cast<const u32x4*>(lds + (sub * 32 + l32) * FPITCH + kk * 32 + lg * 16);
+}
+// A operand from a transposed tile: rows (= d) mt*32 + lane%32, k-slab c of sub-tile sub.
+__device__ __forceinline__ u32x4 frag_transposed(const char* lds, int mt, int sub, int c, int l32, int lg) {
+  return *reinterpret_cast<const u32x4*>(lds + (mt * 32 + l32) * FPITCH + (sub * 32 + c * 16 + lg * 8) * 2);
+}
+// B operand held in registers: the lane's own row of a [time, 64] plane.
+__device__ __forceinline__ void row_frags(const unsigned short* __restrict__ plane, int row, int time, int lg,
+                                          u32x4 f[4]) {
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) {
+    f[kk] = u32x4{0u, 0u, 0u, 0u};
+    if (row < time) f[kk] = *reinterpret_cast<const u32x4*>(plane + static_cast<long>(row) * FD + kk * 16 + lg * 8);
+  }
+}
+// Row index (within a 32-row sub-tile) that accumulator register v of this lane holds.
+__device__ __forceinline__ int acc_row(int v, int lg) { return 8 * (v >> 2) + 4 * lg + (v & 3); }
+
+// Stores a transposed accumulator pair (d x rows) as rows of a [time, 64] plane.
+template <typename TO>
+__device__ __forceinline__ bool store_transposed_acc(TO* __restrict__ plane, int row, int time, int lg,
+                                                     const floatx16 acc[2], float mul) {
+  bool bad = false;
+  if (row >= time) return false;
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      const int d = mt * 32 + 8 * q4 + 4 * lg;
+      float x0 = acc[mt][4 * q4 + 0] * mul, x1 = acc[mt][4 * q4 + 1] * mul, x2 = acc[mt][4 * q4 + 2] * mul,
+            x3 = acc[mt][4 * q4 + 3] * mul;
+      bad |= !(dev_finite(x0) && dev_finite(x1) && dev_finite(x2) && dev_finite(x3));
+      if constexpr (sizeof(TO) == 2) {
+        uint2 w;
+        w.x = pack2(x0, x1);
+        w.y = pack2(x2, x3);
+        *reinterpret_cast<uint2*>(plane + static_cast<long>(row) * FD + d) = w;
+      } else {
+        *reinterpret_cast<float4*>(plane + static_cast<long>(row) * FD + d) = make_float4(x0, x1, x2, x3);
+      }
+    }
+  return bad;
+}
+
+// ------------------------------------------------------------------ forward
+template <typename TO>
+__global__ __launch_bounds__(FT) void flash_fwd_kernel(const unsigned short* __restrict__ q,
+                                                       const unsigned short* __restrict__ k,
+                                                       const unsigned short* __restrict__ v, TO* __restrict__ out,
+                                                       float* __restrict__ lse, FlashShape s, OmxFaultWord* fault,
+                                                       unsigned long long tag) {
+  __shared__ __attribute__((aligned(16))) char smem[2 * FTILE];
+  char* k_rows = smem;
+  char* v_tr = smem + FTILE;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lg = lane >> 5;
+  const int T = s.time;
+  // Late query blocks see the most keys: schedule them first.
+  const int qb = gridDim.x - 1 - blockIdx.x;
+  const long plane = blockIdx.y;
+  const int h = static_cast<int>(plane % s.heads), b = static_cast<int>(plane / s.heads);
+  const long kv_plane = static_cast<long>(b) * s.kv_heads + h / s.rep;
+  const unsigned short* qp = q + plane * T * FD;
+  const unsigned short* kp = k + kv_plane * T * FD;
+  const unsigned short* vp = v + kv_plane * T * FD;
+  const int wave_q0 = qb * 128 + wave * 32;
+  const int q_row = wave_q0 + l32;
+  u32x4 qf[4];
+  row_frags(qp, q_row, T, lg, qf);
+  floatx16 o[2] = {zero16(), zero16()};
+  float m = -INFINITY, lsum = 0.0f;
+  const float scale_log2 = s.scale * LOG2E;
+  const int block_q0 = qb * 128, block_q1 = min(T - 1, qb * 128 + 127);
+  const int kt_first = s.window > 0 ? max(0, block_q0 + 1 - s.window) / 64 : 0;
+  const int kt_last = block_q1 / 64;
+  for (int kt = kt_first; kt <= kt_last; ++kt) {
+    const int key0 = kt * 64;
+    u32x4 rk[2], rv[2];
+    tile_load(kp, key0, T, rk);
+    tile_load(vp, key0, T, rv);
+    __syncthreads();  // the previous tile's reads are done
+    tile_store_rows(k_rows, rk);
+    tile_store_transposed(v_tr, rv);
+    __syncthreads();
+    const bool active = key0 <= wave_q0 + 31 && (s.window == 0 || key0 + 63 + s.window > wave_q0);
+    if (!active) continue;
+    floatx16 sc[2] = {zero16(), zero16()};
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) sc[sub] = mfma(frag_rows(k_rows, sub, kk, l32, lg), qf[kk], sc[sub]);
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+      for (int vv = 0; vv < 16; ++vv) {
+        const int key = key0 + sub * 32 + acc_row(vv, lg);
+        float val = sc[sub][vv] * scale_log2;
+        const bool masked = key > q_row || key >= T || (s.window > 0 && key + s.window <= q_row);
+        val = masked ? -INFINITY : val;
+        sc[sub][vv] = val;
+        tmax = fmaxf(tmax, val);
+      }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float new_m = fmaxf(m, tmax);
+    const float m_safe = new_m == -INFINITY ? 0.0f : new_m;
+    const float alpha = __builtin_amdgcn_exp2f(m - m_safe);
+    float psum = 0.0f;
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+      for (int vv = 0; vv < 16; ++vv) {
+        float p = __builtin_amdgcn_exp2f(sc[sub][vv] - m_safe);
+        sc[sub][vv] = p;
+        psum += p;
+      }
+    psum += __shfl_xor(psum, 32, 64);
+    lsum = lsum * alpha + psum;
+    m = new_m;
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int vv = 0; vv < 16; ++vv) o[mt][vv] *= alpha;
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        const u32x4 pb = pack8(sc[sub], c);
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt) o[mt] = mfma(frag_transposed(v_tr, mt, sub, c, l32, lg), pb, o[mt]);
+      }
+  }
+  bool bad = false;
+  if (q_row < T) {
+    bad |= !(dev_finite(lsum) && lsum > 0.0f);
+    if (lg == 0) lse[plane * T + q_row] = m * LN2 + logf(lsum);
+  }
+  bad |= store_transposed_acc<TO>(out + plane * T * FD, q_row, T, lg, o, 1.0f / lsum);
+  if (bad) dev_raise_fault(fault, tag);
+}
+
+// ------------------------------------------------------------------ backward: dK, dV
+template <typename TO>
+__global__ __launch_bounds__(FT) void flash_bwd_dkv_kernel(
+    const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
+    const float* __restrict__ lse, const float* __restrict__ delta, const unsigned short* __restrict__ gy,
+    TO* __restrict__ gk, TO* __restrict__ gv, FlashShape s, OmxFaultWord* fault, unsigned long long tag) {
+  __shared__ __attribute__((aligned(16))) char smem[4 * FTILE + 2 * 64 * 4];
+  char* q_rows = smem;
+  char* g_rows = smem + FTILE;
+  char* q_tr = smem + 2 * FTILE;
+  char* g_tr = smem + 3 * FTILE;
+  float* lse_s = reinterpret_cast<float*>(smem + 4 * FTILE);
+  float* del_s = lse_s + 64;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lg = lane >> 5;
+  const int T = s.time;
+  const int kb = blockIdx.x;  // early key blocks are seen by the most queries: they come first
+  const long kv_plane = blockIdx.y;
+  const int gidx = static_cast<int>(kv_plane % s.kv_heads), b = static_cast<int>(kv_plane / s.kv_heads);
+  const unsigned short* kp = k + kv_plane * T * FD;
+  const unsigned short* vp = v + kv_plane * T * FD;
+  const int wave_k0 = kb * 128 + wave * 32;
+  const int key_row = wave_k0 + l32;
+  u32x4 kf[4], vf[4];
+  row_frags(kp, key_row, T, lg, kf);
+  row_frags(vp, key_row, T, lg, vf);
+  floatx16 dk[2] = {zero16(), zero16()}, dv[2] = {zero16(), zero16()};
+  const float scale_log2 = s.scale * LOG2E;
+  const int block_k0 = kb * 128, block_k1 = min(T - 1, kb * 128 + 127);
+  const int qt_first = block_k0 / 64;
+  const int qt_last = (s.window > 0 ? min(T - 1, block_k1 + s.window - 1) : T - 1) / 64;
+  bool bad = false;
+  for (int r = 0; r < s.rep; ++r) {
+    const long q_plane = static_cast<long>(b) * s.heads + static_cast<long>(gidx) * s.rep + r;
+    const unsigned short* qp = q + q_plane * T * FD;
+    const unsigned short* gp = gy + q_plane * T * FD;
+    for (int qt = qt_first; qt <= qt_last; ++qt) {
+      const int q0 = qt * 64;
+      u32x4 rq[2], rg[2];
+      tile_load(qp, q0, T, rq);
+      tile_load(gp, q0, T, rg);
+      float row_lse = 0.0f, row_del = 0.0f;
+      if (threadIdx.x < 64 && q0 + static_cast<int>(threadIdx.x) < T) {
+        row_lse = lse[q_plane * T + q0 + threadIdx.x];
+        row_del = delta[q_plane * T + q0 + threadIdx.x];
+        bad |= !(dev_finite(row_lse) && dev_finite(row_del));
+      }
+      __syncthreads();
+      tile_store_rows(q_rows, rq);
+      tile_store_rows(g_rows, rg);
+      tile_store_transposed(q_tr, rq);
+      tile_store_transposed(g_tr, rg);
+      if (threadIdx.x < 64) {
+        lse_s[threadIdx.x] = row_lse * LOG2E;
+        del_s[threadIdx.x] = row_del;
+      }
+      __syncthreads();
+      const bool active = q0 + 63 >= wave_k0 && (s.window == 0 || q0 < wave_k0 + 31 + s.window);
+      if (!active) continue;
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub) {
+        floatx16 sc = zero16(), dp = zero16();
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+          sc = mfma(frag_rows(q_rows, sub, kk, l32, lg), kf[kk], sc);
+          dp = mfma(frag_rows(g_rows, sub, kk, l32, lg), vf[kk], dp);
+        }
+#pragma unroll
+        for (int vv = 0; vv < 16; ++vv) {
+          const int qi_local = sub * 32 + acc_row(vv, lg);
+          const int qi = q0 + qi_local;
+          const bool masked =
+              key_row > qi || qi >= T || key_row >= T || (s.window > 0 && key_row + s.window <= qi);
+          float p = masked ? 0.0f : __builtin_amdgcn_exp2f(sc[vv] * scale_log2 - lse_s[qi_local]);
+          float ds = p * (dp[vv] - del_s[qi_local]) * s.scale;
+          sc[vv] = p;
+          dp[vv] = ds;
+        }
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+          const u32x4 pb = pack8(sc, c), dsb = pack8(dp, c);
+#pragma unroll
+          for (int mt = 0; mt < 2; ++mt) {
+            dv[mt] = mfma(frag_transposed(g_tr, mt, sub, c, l32, lg), pb, dv[mt]);
+            dk[mt] = mfma(frag_transposed(q_tr, mt, sub, c, l32, lg), dsb, dk[mt]);
+          }
+        }
+      }
+    }
+  }
+  bad |= store_transposed_acc<TO>(gk + kv_plane * T * FD, key_row, T, lg, dk, 1.0f);
+  bad |= store_transposed_acc<TO>(gv + kv_plane * T * FD, key_row, T, lg, dv, 1.0f);
+  if (bad) dev_raise_fault(fault, tag);
+}
+
+// ------------------------------------------------------------------ backward: dQ
+template <typename TO>
+__global__ __launch_bounds__(FT) void flash_bwd_dq_kernel(
+    const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
+    const float* __restrict__ lse, const float* __restrict__ delta, const unsigned short* __restrict__ gy,
+    TO* __restrict__ gq, FlashShape s, OmxFaultWord* fault, unsigned long long tag) {
+  __shared__ __attribute__((aligned(16))) char smem[3 * FTILE];
+  char* k_rows = smem;
+  char* v_rows = smem + FTILE;
+  char* k_tr = smem + 2 * FTILE;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lg = lane >> 5;
+  const int T = s.time;
+  const int qb = gridDim.x - 1 - blockIdx.x;
+  const long plane = blockIdx.y;
+  const int h = static_cast<int>(plane % s.heads), b = static_cast<int>(plane / s.heads);
+  const long kv_plane = static_cast<long>(b) * s.kv_heads + h / s.rep;
+  const unsigned short* kp = k + kv_plane * T * FD;
+  const unsigned short* vp = v + kv_plane * T * FD;
+  const int wave_q0 = qb * 128 + wave * 32;
+  const int q_row = wave_q0 + l32;
+  u32x4 qf[4], gf[4];
+  row_frags(q + plane * T * FD, q_row, T, lg, qf);
+  row_frags(gy + plane * T * FD, q_row, T, lg, gf);
+  float row_lse = 0.0f, row_del = 0.0f;
+  bool bad = false;
+  if (q_row < T) {
+    row_lse = lse[plane * T + q_row];
+    row_del = delta[plane * T + q_row];
+    bad |= !(dev_finite(row_lse) && dev_finite(row_del));
+  }
+  row_lse *= LOG2E;
+  floatx16 dq[2] = {zero16(), zero16()};
+  const float scale_log2 = s.scale * LOG2E;
+  const int block_q0 = qb * 128, block_q1 = min(T - 1, qb * 128 + 127);
+  const int kt_first = s.window > 0 ? max(0, block_q0 + 1 - s.window) / 64 : 0;
+  const int kt_last = block_q1 / 64;
+  for (int kt = kt_first; kt <= kt_last; ++kt) {
+    const int key0 = kt * 64;
+    u32x4 rk[2], rv[2];
+    tile_load(kp, key0, T, rk);
+    tile_load(vp, key0, T, rv);
+    __syncthreads();
+    tile_store_rows(k_rows, rk);
+    tile_store_rows(v_rows, rv);
+    tile_store_transposed(k_tr, rk);
+    __syncthreads();
+    const bool active = key0 <= wave_q0 + 31 && (s.window == 0 || key0 + 63 + s.window > wave_q0);
+    if (!active) continue;
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub) {
+      floatx16 sc = zero16(), dp = zero16();
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        sc = mfma(frag_rows(k_rows, sub, kk, l32, lg), qf[kk], sc);
+        dp = mfma(frag_rows(v_rows, sub, kk, l32, lg), gf[kk], dp);
+      }
+#pragma unroll
+      for (int vv = 0; vv < 16; ++vv) {
+        const int key = key0 + sub * 32 + acc_row(vv, lg);
+        const bool masked = key > q_row || key >= T || q_row >= T || (s.window > 0 && key + s.window <= q_row);
+        float p = masked ? 0.0f : __builtin_amdgcn_exp2f(sc[vv] * scale_log2 - row_lse);
+        dp[vv] = p * (dp[vv] - row_del) * s.scale;
+      }
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        const u32x4 dsb = pack8(dp, c);
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt) dq[mt] = mfma(frag_transposed(k_tr, mt, sub, c, l32, lg), dsb, dq[mt]);
+      }
+    }
+  }
+  bad |= store_transposed_acc<TO>(gq + plane * T * FD, q_row, T, lg, dq, 1.0f);
+  if (bad) dev_raise_fault(fault, tag);
+}
+
+// delta[row] = dO[row] . O[row], one wave per row.
+__global__ __launch_bounds__(FT) void flash_delta_kernel(const unsigned short* __restrict__ out,
+                                                         const unsigned short* __restrict__ gy,
+                                                         float* __restrict__ delta, long rows) {
+  const int lane = threadIdx.x & 63;
+  const long row = static_cast<long>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  float acc = dev_bf16_bits_to_f32(gy[row * FD + lane]) * dev_bf16_bits_to_f32(out[row * FD + lane]);
+  acc = wave_sum(acc);
+  if (lane == 0) delta[row] = acc;
+}
+
+FlashShape make_shape(uint64_t batch, uint64_t heads, uint64_t kv_heads, uint64_t time, uint64_t window, float scale) {
+  FlashShape s;
+  s.batch = static_cast<int>(batch);
+  s.heads = static_cast<int>(heads);
+  s.kv_heads = static_cast<int>(kv_heads);
+  s.time = static_cast<int>(time);
+  s.window = static_cast<int>(window);
+  s.rep = static_cast<int>(heads / kv_heads);
+  s.scale = scale;
+  return s;
+}
+
+}  // namespace
+
+bool omx_flash_sdpa_supports(uint64_t dim, int32_t operand_dtype) { return dim == FD && operand_dtype == OMX_BF16; }
+
+int32_t omx_flash_sdpa_forward(omx_ctx* ctx, const void* q, const void* k, const void* v, void* out, int32_t out_dtype,
+                               float* lse, uint64_t batch, uint64_t heads, uint64_t kv_heads, uint64_t time,
+                               uint64_t dim, uint64_t window, float scale, unsigned long long tag) {
+  if (dim != FD) return omx_fail(ctx, OMX_UNSUPPORTED_HEAD_DIM, "head_dim %llu limit %d", (unsigned long long)dim, FD);
+  FlashShape s = make_shape(batch, heads, kv_heads, time, window, scale);
+  dim3 grid(static_cast<unsigned>((time + 127) / 128), static_cast<unsigned>(batch * heads)), block(FT);
+  const unsigned short* qs = static_cast<const unsigned short*>(q);
+  const unsigned short* ks = static_cast<const unsigned short*>(k);
+  const unsigned short* vs = static_cast<const unsigned short*>(v);
+  if (out_dtype == OMX_BF16)
+    hipLaunchKernelGGL((flash_fwd_kernel<unsigned short>), grid, block, 0, ctx->stream, qs, ks, vs,
+                       static_cast<unsigned short*>(out), lse, s, ctx->fault, tag);
+  else
+    hipLaunchKernelGGL((flash_fwd_kernel<float>), grid, block, 0, ctx->stream, qs, ks, vs, static_cast<float*>(out),
+                       lse, s, ctx->fault, tag);
+  OMX_LAUNCH_CHECK(ctx, "flash_fwd_kernel");
+  return OMX_OK;
+}
+
+int32_t omx_flash_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, const void* v, const void* out,
+                                const float* lse, const void* gy, void* gq, void* gk, void* gv, int32_t grad_dtype,
+                                uint64_t batch, uint64_t heads, uint64_t kv_heads, uint64_t time, uint64_t dim,
+                                uint64_t window, float scale, unsigned long long tag) {
+  if (dim != FD) return omx_fail(ctx, OMX_UNSUPPORTED_HEAD_DIM, "head_dim %llu limit %d", (unsigned long long)dim, FD);
+  FlashShape s = make_shape(batch, heads, kv_heads, time, window, scale);
+  const long rows = static_cast<long>(batch * heads * time);
+  void* ws = nullptr;
+  int32_t rc = omx_workspace(ctx, rows * sizeof(float), &ws);
+  if (rc != OMX_OK) return rc;
+  float* delta = static_cast<float*>(ws);
+  const unsigned short* qs = static_cast<const unsigned short*>(q);
+  const unsigned short* ks = static_cast<const unsigned short*>(k);
+  const unsigned short* vs = static_cast<const unsigned short*>(v);
+  const unsigned short* os = static_cast<const unsigned short*>(out);
+  const unsigned short* gs = static_cast<const unsigned short*>(gy);
+  hipLaunchKernelGGL(flash_delta_kernel, dim3(static_cast<unsigned>((rows + 3) / 4)), dim3(FT), 0, ctx->stream, os, gs,
+                     delta, rows);
+  OMX_LAUNCH_CHECK(ctx, "flash_delta_kernel");
+  dim3 block(FT);
+  dim3 kv_grid(static_cast<unsigned>((time + 127) / 128), static_cast<unsigned>(batch * kv_heads));
+  dim3 q_grid(static_cast<unsigned>((time + 127) / 128), static_cast<unsigned>(batch * heads));
+  if (grad_dtype == OMX_BF16) {
+    hipLaunchKernelGGL((flash_bwd_dkv_kernel<unsigned short>), kv_grid, block, 0, ctx->stream, qs, ks, vs, lse, delta,
+                       gs, static_cast<unsigned short*>(gk), static_cast<unsigned short*>(gv), s, ctx->fault, tag);
+    hipLaunchKernelGGL((flash_bwd_dq_kernel<unsigned short>), q_grid, block, 0, ctx->stream, qs, ks, vs, lse, delta,
+                       gs, static_cast<unsigned short*>(gq), s, ctx->fault, tag);
+  } else {
+    hipLaunchKernelGGL((flash_bwd_dkv_kernel<float>), kv_grid, block, 0, ctx->stream, qs, ks, vs, lse, delta, gs,
+                       static_cast<float*>(gk), static_cast<float*>(gv), s, ctx->fault, tag);
+    hipLaunchKernelGGL((flash_bwd_dq_kernel<float>), q_grid, block, 0, ctx->stream, qs, ks, vs, lse, delta, gs,
+                       static_cast<float*>(gq), s, ctx->fault, tag);
+  }
+  OMX_LAUNCH_CHECK(ctx, "flash backward kernels");
+  return OMX_OK;
 }

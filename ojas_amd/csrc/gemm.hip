@@ -361,11 +361,55 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
     return omx_fail(ctx, OMX_OUT_OF_RANGE, "%s: too many output tiles", op);
   g.fault = ctx->fault;
   g.tag = omx_tag(ctx, fault_op);
-  if (operand_dtype == OMX_BF16) return launch<unsigned short>(ctx, g, a_km, b_km);
-  return launch<float>(ctx, g, a_km, b_km);
+  omx_ctx::TimedLaunch timed{};
+  if (ctx->profile_gemm) {
+    auto take = [&](hipEvent_t* e) -> hipError_t {
+      if (!ctx->event_pool.empty()) {
+        *e = ctx->event_pool.back();
+        ctx->event_pool.pop_back();
+        return hipSuccess;
+      }
+      return hipEventCreate(e);
+    };
+    OMX_HIP(ctx, take(&timed.start));
+    OMX_HIP(ctx, take(&timed.stop));
+    timed.flops = 2.0 * static_cast<double>(m) * static_cast<double>(n) * static_cast<double>(k);
+    OMX_HIP(ctx, hipEventRecord(timed.start, ctx->stream));
+  }
+  int32_t rc = operand_dtype == OMX_BF16 ? launch<unsigned short>(ctx, g, a_km, b_km) : launch<float>(ctx, g, a_km, b_km);
+  if (ctx->profile_gemm) {
+    OMX_HIP(ctx, hipEventRecord(timed.stop, ctx->stream));
+    ctx->timed.push_back(timed);
+  }
+  return rc;
 }
 
 extern "C" {
+
+int32_t omx_profile_gemm(omx_ctx* ctx, int32_t enable) {
+  OMX_REQUIRE_CTX(ctx);
+  ctx->profile_gemm = enable != 0;
+  return OMX_OK;
+}
+
+int32_t omx_profile_gemm_report(omx_ctx* ctx, uint64_t* launches, double* total_ms, double* total_flops) {
+  OMX_REQUIRE_CTX(ctx);
+  OMX_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  double ms = 0.0, flops = 0.0;
+  for (auto& t : ctx->timed) {
+    float one = 0.0f;
+    OMX_HIP(ctx, hipEventElapsedTime(&one, t.start, t.stop));
+    ms += one;
+    flops += t.flops;
+    ctx->event_pool.push_back(t.start);
+    ctx->event_pool.push_back(t.stop);
+  }
+  if (launches) *launches = ctx->timed.size();
+  if (total_ms) *total_ms = ms;
+  if (total_flops) *total_flops = flops;
+  ctx->timed.clear();
+  return OMX_OK;
+}
 
 int32_t omx_gemm(omx_ctx* ctx, const void* a, uint64_t a_rs, uint64_t a_cs, const void* b, uint64_t b_rs,
                  uint64_t b_cs, int32_t operand_dtype, void* c, int32_t c_dtype, uint64_t m, uint64_t k,

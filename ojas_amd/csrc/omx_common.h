@@ -10,6 +10,7 @@
 #include <cstring>
 #include <map>
 #include <string>
+#include <vector>
 
 #include "ojas_mi355x.h"
 
@@ -63,6 +64,14 @@ struct omx_ctx {
   void* workspace = nullptr;
   uint64_t workspace_bytes = 0;
   int cu_count = 0;
+  // Optional per-launch timing of the GEMM kernel (benchmark only).
+  bool profile_gemm = false;
+  struct TimedLaunch {
+    hipEvent_t start, stop;
+    double flops;
+  };
+  std::vector<TimedLaunch> timed;
+  std::vector<hipEvent_t> event_pool;
 };
 
 int32_t omx_fail(omx_ctx* ctx, omx_status code, const char* fmt, ...);

@@ -435,3 +435,44 @@ def test_budget_refuses_rather_than_clamps_and_unsupported_ops_name_themselves(b
         small.layer_norm_forward(None, None)
     assert e.value.code == UNSUPPORTED and "layer_norm_forward" in e.value.detail
     small.close()
+
+
+FLASH_SHAPES = [([1, 1, 1, 64], 1, None), ([1, 2, 17, 64], 2, None), ([2, 3, 64, 64], 3, None),
+                ([1, 2, 128, 64], 2, None), ([1, 2, 129, 64], 1, None), ([1, 4, 300, 64], 2, None),
+                ([2, 2, 257, 64], 2, 40), ([1, 2, 200, 64], 2, 1), ([1, 1, 1024, 64], 1, None),
+                ([1, 2, 520, 64], 2, 130)]
+
+
+@pytest.mark.parametrize("shape,hkv,window", FLASH_SHAPES)
+def test_causal_sdpa_bf16_mfma(be, shape, hkv, window):
+    """head_dim 64 with bf16 operands takes the MFMA flash kernels. Inputs are
+    bf16-exact on both sides; the GPU additionally rounds P and dS to bf16 for
+    the second product, so the gate is the bf16 one (2e-2 of the largest value)."""
+    from ojas_amd.backend import BF16, F32
+
+    print(f"sdpa bf16 {shape} hkv {hkv} window {window}", flush=True)
+    b, h, t, d = shape
+    r = orc.SplitMix64(900 + t)
+    mk = lambda n, sh: orc.round_bf16(r.vec(n, 1.0)).reshape(sh)
+    q = mk(b * h * t * d, (b, h, t, d))
+    k = mk(b * hkv * t * d, (b, hkv, t, d))
+    v = mk(b * hkv * t * d, (b, hkv, t, d))
+    gy = mk(b * h * t * d, (b, h, t, d))
+    oy, olse = orc.causal_sdpa_forward(q, k, v, window or 0)
+    dq, dk, dv, dgy = (be.upload(a, BF16) for a in (q, k, v, gy))
+    y32, lse = be.causal_sdpa_forward(dq, dk, dv, window, out_dtype=F32)
+    close(be.download(y32), oy, 1e-2, "flash out (f32 store)")
+    close(be.download(lse), olse, 1e-5, "flash lse")
+    y16, lse16 = be.causal_sdpa_forward(dq, dk, dv, window, out_dtype=BF16)
+    close(be.download_f32(y16), oy, BF16_TOL, "flash out (bf16 store)")
+    # Backward from the oracle's saved output rounded to bf16, as a bf16-tier caller saves it.
+    oy16 = orc.round_bf16(oy)
+    ogq, ogk, ogv = orc.causal_sdpa_backward(q, k, v, oy16, olse, gy, window or 0)
+    gq, gk, gv = be.causal_sdpa_backward(dq, dk, dv, be.upload(oy16, BF16), be.upload(olse), dgy, window, grad_dtype=F32)
+    close(be.download(gq), ogq, BF16_TOL, "flash gq")
+    close(be.download(gk), ogk, BF16_TOL, "flash gk")
+    close(be.download(gv), ogv, BF16_TOL, "flash gv")
+    gq16, gk16, gv16 = be.causal_sdpa_backward(dq, dk, dv, y16, lse16, dgy, window, grad_dtype=BF16)
+    close(be.download_f32(gq16), ogq, BF16_TOL, "flash gq bf16")
+    close(be.download_f32(gk16), ogk, BF16_TOL, "flash gk bf16")
+    close(be.download_f32(gv16), ogv, BF16_TOL, "flash gv bf16")
