@@ -233,21 +233,21 @@ int32_t omx_unsupported(omx_ctx* ctx, const char* op) {
 
 }  // extern "C"
 
-int32_t omx_workspace(omx_ctx* ctx, uint64_t bytes, void** out) {
-  if (bytes <= ctx->workspace_bytes) {
-    *out = ctx->workspace;
+int32_t omx_workspace(omx_ctx* ctx, uint64_t bytes, void** out, int slot) {
+  if (bytes <= ctx->workspace_bytes[slot]) {
+    *out = ctx->workspace[slot];
     return OMX_OK;
   }
-  if (ctx->workspace) {
-    int32_t rc = omx_free(ctx, ctx->workspace);
+  if (ctx->workspace[slot]) {
+    int32_t rc = omx_free(ctx, ctx->workspace[slot]);
     if (rc != OMX_OK) return rc;
-    ctx->workspace = nullptr;
-    ctx->workspace_bytes = 0;
+    ctx->workspace[slot] = nullptr;
+    ctx->workspace_bytes[slot] = 0;
   }
   uint64_t rounded = (bytes + (1ull << 20) - 1) & ~((1ull << 20) - 1);
-  int32_t rc = omx_alloc(ctx, rounded, &ctx->workspace);
+  int32_t rc = omx_alloc(ctx, rounded, &ctx->workspace[slot]);
   if (rc != OMX_OK) return rc;
-  ctx->workspace_bytes = rounded;
-  *out = ctx->workspace;
+  ctx->workspace_bytes[slot] = rounded;
+  *out = ctx->workspace[slot];
   return OMX_OK;
 }

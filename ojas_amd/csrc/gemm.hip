@@ -20,6 +20,8 @@
 // loaded with coalesced 16-byte reads along its fast index and transposed in
 // registers on the way into LDS, so the fragment reads are the same for every
 // operand layout.
+#include <algorithm>
+
 #include "omx_common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -42,6 +44,8 @@ struct GemmArgs {
   int c_bf16, accumulate;
   int a_vec, b_vec;  // 16-byte loads allowed (alignment of base and leading dimension)
   int tiles_m, tiles_n;
+  int splits, ksteps_per_split;  // split-K: each split writes an f32 partial
+  float* partial;                // [splits][M][N] when splits > 1
   OmxFaultWord* fault;
   unsigned long long tag;
 };
@@ -174,7 +178,8 @@ __global__ __launch_bounds__(NT) void gemm_kernel(GemmArgs g) {
   // Workgroups are dealt round-robin to the 8 XCDs; give each XCD one
   // contiguous run of tiles so neighbours share operand rows in its L2.
   const int total = g.tiles_m * g.tiles_n;
-  int id = blockIdx.x;
+  const int split = blockIdx.x / total;
+  int id = blockIdx.x - split * total;
   {
     const int per = (total + 7) / 8;
     int xcd = id & 7, local = id >> 3;
@@ -208,7 +213,9 @@ __global__ __launch_bounds__(NT) void gemm_kernel(GemmArgs g) {
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
   u32x4 ra[4], rb[4];
-  const int ksteps = (g.K + BK - 1) / BK;
+  const int ksteps_all = (g.K + BK - 1) / BK;
+  const int ks_begin = split * g.ksteps_per_split;
+  const int ks_end = min(ksteps_all, ks_begin + g.ksteps_per_split);
   auto load_tiles = [&](int ks) {
     int k0 = ks * BK;
     if constexpr (A_KM) load_kmajor<T>(A, g.lda, m0, g.M, k0, g.K, g.a_vec, ra);
@@ -225,12 +232,12 @@ __global__ __launch_bounds__(NT) void gemm_kernel(GemmArgs g) {
     else store_kcontig<T>(lb, rb);
   };
 
-  load_tiles(0);
+  load_tiles(ks_begin);
   store_tiles(0);
   __syncthreads();
-  for (int ks = 0; ks < ksteps; ++ks) {
-    const int buf = ks & 1;
-    if (ks + 1 < ksteps) load_tiles(ks + 1);
+  for (int ks = ks_begin; ks < ks_end; ++ks) {
+    const int buf = (ks - ks_begin) & 1;
+    if (ks + 1 < ks_end) load_tiles(ks + 1);
     const char* la = smem + buf * 2 * TILE_BYTES + (wm * 64 + l32) * PITCH + lg * 16;
     const char* lb = smem + buf * 2 * TILE_BYTES + TILE_BYTES + (wn * 64 + l32) * PITCH + lg * 16;
 #pragma unroll
@@ -246,8 +253,25 @@ __global__ __launch_bounds__(NT) void gemm_kernel(GemmArgs g) {
 #pragma unroll
         for (int tn = 0; tn < 2; ++tn) mma_step<T>(af[tm], bf[tn], acc[tm][tn]);
     }
-    if (ks + 1 < ksteps) store_tiles(buf ^ 1);
+    if (ks + 1 < ks_end) store_tiles(buf ^ 1);
     __syncthreads();
+  }
+  if (g.splits > 1) {
+    // Partial sums go to the workspace; the reduce kernel adds the splits in
+    // ascending order and applies the output conversion and the fault check.
+    float* part = g.partial + static_cast<long>(split) * g.M * g.N;
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+      for (int tn = 0; tn < 2; ++tn) {
+        int col = n0 + wn * 64 + tn * 32 + l32;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          int row = m0 + wm * 64 + tm * 32 + 8 * (v >> 2) + 4 * lg + (v & 3);
+          if (row < g.M && col < g.N) part[static_cast<long>(row) * g.N + col] = acc[tm][tn][v];
+        }
+      }
+    return;
   }
 
   // Epilogue. Accumulator register v of a 32x32 block holds
@@ -278,9 +302,25 @@ __global__ __launch_bounds__(NT) void gemm_kernel(GemmArgs g) {
   if (bad) dev_raise_fault(g.fault, g.tag);
 }
 
+__global__ void splitk_reduce_kernel(GemmArgs g) {
+  const long total = static_cast<long>(g.M) * g.N;
+  bool bad = false;
+  for (long i = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x; i < total;
+       i += static_cast<long>(gridDim.x) * blockDim.x) {
+    const long row = i / g.N, col = i - row * g.N;
+    const long off = row * g.ldc + col;
+    float acc = g.accumulate ? static_cast<float*>(g.c)[off] : 0.0f;
+    for (int s = 0; s < g.splits; ++s) acc += g.partial[static_cast<long>(s) * total + i];
+    if (g.c_bf16) static_cast<unsigned short*>(g.c)[off] = dev_f32_to_bf16_bits(acc);
+    else static_cast<float*>(g.c)[off] = acc;
+    bad |= !dev_finite(acc);
+  }
+  if (bad) dev_raise_fault(g.fault, g.tag);
+}
+
 template <typename T>
 int32_t launch(omx_ctx* ctx, GemmArgs& g, bool a_km, bool b_km) {
-  int total = g.tiles_m * g.tiles_n;
+  int total = g.tiles_m * g.tiles_n * g.splits;
   size_t smem = 4 * TILE_BYTES;
   dim3 grid(total), block(NT);
   // More than 64 KiB of dynamic LDS has to be granted per kernel, once.
@@ -301,6 +341,12 @@ int32_t launch(omx_ctx* ctx, GemmArgs& g, bool a_km, bool b_km) {
   else if (a_km && !b_km) hipLaunchKernelGGL((gemm_kernel<T, true, false>), grid, block, smem, ctx->stream, g);
   else hipLaunchKernelGGL((gemm_kernel<T, true, true>), grid, block, smem, ctx->stream, g);
   OMX_LAUNCH_CHECK(ctx, "gemm_kernel");
+  if (g.splits > 1) {
+    long elems = static_cast<long>(g.M) * g.N;
+    unsigned blocks = static_cast<unsigned>(std::min<long>((elems + 255) / 256, 4096));
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3(blocks), dim3(256), 0, ctx->stream, g);
+    OMX_LAUNCH_CHECK(ctx, "splitk_reduce_kernel");
+  }
   return OMX_OK;
 }
 
@@ -359,6 +405,28 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
   g.tiles_n = (g.N + BN - 1) / BN;
   if (static_cast<long>(g.tiles_m) * g.tiles_n > 0x7fffffffl)
     return omx_fail(ctx, OMX_OUT_OF_RANGE, "%s: too many output tiles", op);
+  // Few output tiles and a long reduction (the weight gradients: K = tokens):
+  // split K so the grid fills the chip.
+  {
+    const int bk = operand_dtype == OMX_BF16 ? 64 : 32;
+    const int ksteps = (g.K + bk - 1) / bk;
+    const long tiles = static_cast<long>(g.tiles_m) * g.tiles_n;
+    int splits = 1;
+    if (tiles < 256 && ksteps >= 32) {
+      splits = static_cast<int>((512 + tiles - 1) / tiles);
+      if (splits > ksteps / 8) splits = ksteps / 8;
+      if (splits < 1) splits = 1;
+    }
+    g.ksteps_per_split = (ksteps + splits - 1) / splits;
+    g.splits = (ksteps + g.ksteps_per_split - 1) / g.ksteps_per_split;
+    g.partial = nullptr;
+    if (g.splits > 1) {
+      void* ws = nullptr;
+      int32_t wrc = omx_workspace(ctx, static_cast<uint64_t>(g.splits) * m * n * sizeof(float), &ws, 1);
+      if (wrc != OMX_OK) return wrc;
+      g.partial = static_cast<float*>(ws);
+    }
+  }
   g.fault = ctx->fault;
   g.tag = omx_tag(ctx, fault_op);
   omx_ctx::TimedLaunch timed{};

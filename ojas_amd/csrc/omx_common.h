@@ -61,8 +61,10 @@ struct omx_ctx {
   std::string last_error;
   std::string arch;
   // Scratch the library owns (charged to the budget); grown on demand.
-  void* workspace = nullptr;
-  uint64_t workspace_bytes = 0;
+  // Slot 0: per-op scratch. Slot 1: split-K partials of the GEMM (which an op
+  // may call while it holds slot 0).
+  void* workspace[2] = {nullptr, nullptr};
+  uint64_t workspace_bytes[2] = {0, 0};
   int cu_count = 0;
   // Optional per-launch timing of the GEMM kernel (benchmark only).
   bool profile_gemm = false;
@@ -76,8 +78,8 @@ struct omx_ctx {
 
 int32_t omx_fail(omx_ctx* ctx, omx_status code, const char* fmt, ...);
 int32_t omx_hip_fail(omx_ctx* ctx, hipError_t err, const char* what);
-// Grows the library workspace to at least `bytes` (budget-charged).
-int32_t omx_workspace(omx_ctx* ctx, uint64_t bytes, void** out);
+// Grows workspace `slot` to at least `bytes` (budget-charged).
+int32_t omx_workspace(omx_ctx* ctx, uint64_t bytes, void** out, int slot = 0);
 // Next launch tag for fault attribution: (sequence << 8) | op.
 inline unsigned long long omx_tag(omx_ctx* ctx, uint32_t op) {
   return (static_cast<unsigned long long>(++ctx->sequence) << 8) | op;

@@ -117,14 +117,24 @@ __global__ __launch_bounds__(ROW_THREADS) void rms_bwd_kernel(const TX* __restri
   if (bad) dev_raise_fault(fault, tag);
 }
 
-__global__ void column_sum_kernel(const float* __restrict__ partial, float* __restrict__ out, int blocks, int dim,
-                                  OmxFaultWord* fault, unsigned long long tag) {
-  int c = blockIdx.x * blockDim.x + threadIdx.x;
-  if (c >= dim) return;
+// out[c] = sum over blocks of partial[b][c]: 64 columns per workgroup, four
+// row groups that each add their strided share, then a fixed four-way sum.
+__global__ __launch_bounds__(256) void column_sum_kernel(const float* __restrict__ partial, float* __restrict__ out,
+                                                         int blocks, int dim, OmxFaultWord* fault,
+                                                         unsigned long long tag) {
+  __shared__ float red[4][64];
+  const int lane = threadIdx.x & 63, group = threadIdx.x >> 6;
+  const int c = blockIdx.x * 64 + lane;
   float s = 0.0f;
-  for (int b = 0; b < blocks; ++b) s += partial[static_cast<size_t>(b) * dim + c];
-  out[c] = s;
-  if (!dev_finite(s)) dev_raise_fault(fault, tag);
+  if (c < dim)
+    for (int b = group; b < blocks; b += 4) s += partial[static_cast<size_t>(b) * dim + c];
+  red[group][lane] = s;
+  __syncthreads();
+  if (group == 0 && c < dim) {
+    float total = ((red[0][lane] + red[1][lane]) + red[2][lane]) + red[3][lane];
+    out[c] = total;
+    if (!dev_finite(total)) dev_raise_fault(fault, tag);
+  }
 }
 
 // ---------------------------------------------------------------- embedding
@@ -401,7 +411,7 @@ int32_t launch_rms_bwd(omx_ctx* ctx, const void* x, const float* w, const void* 
   }
 #undef RMS_BWD
   OMX_LAUNCH_CHECK(ctx, "rms_bwd_kernel");
-  hipLaunchKernelGGL(column_sum_kernel, dim3(static_cast<unsigned>((dim + 255) / 256)), dim3(256), 0, ctx->stream,
+  hipLaunchKernelGGL(column_sum_kernel, dim3(static_cast<unsigned>((dim + 63) / 64)), dim3(256), 0, ctx->stream,
                      static_cast<const float*>(partial), gw, static_cast<int>(blocks), static_cast<int>(dim),
                      ctx->fault, tag);
   OMX_LAUNCH_CHECK(ctx, "column_sum_kernel");
