@@ -21,6 +21,7 @@
 // registers on the way into LDS, so the fragment reads are the same for every
 // operand layout.
 #include <algorithm>
+#include <cstdlib>
 
 #include "omx_common.h"
 
@@ -31,9 +32,8 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 namespace {
 
-constexpr int BM = 128, BN = 128, NT = 256;
-constexpr int PITCH = 144;               // bytes per LDS row: 8 chunks of 16 B + pad
-constexpr int TILE_BYTES = 128 * PITCH;  // one operand tile
+constexpr int NT = 256;
+constexpr int PITCH = 144;  // bytes per LDS row of a k-contiguous tile: 8 chunks of 16 B + pad
 
 struct GemmArgs {
   const void* a;
@@ -56,15 +56,14 @@ union Chunk {
   T e[16 / sizeof(T)];
 };
 
-// Operand stored with K contiguous: element (row, k) at p[row * ld + k].
-// Each thread moves four 16-byte chunks of the 128 x (8 chunk) tile.
-template <typename T>
+// ---- operand with K contiguous: element (row, k) at p[row * ld + k]; LDS [row][k].
+template <typename T, int ROWS>
 __device__ __forceinline__ void load_kcontig(const T* __restrict__ p, long ld, int row0, int rows, int k0, int K,
-                                             bool vec, u32x4 regs[4]) {
+                                             bool vec, u32x4* regs) {
   constexpr int KV = 16 / sizeof(T);
   const int tid = threadIdx.x;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < ROWS / 32; ++i) {
     int c = tid + NT * i;
     int row = c >> 3, kc = c & 7;
     int gr = row0 + row, gk = k0 + kc * KV;
@@ -83,23 +82,23 @@ __device__ __forceinline__ void load_kcontig(const T* __restrict__ p, long ld, i
     regs[i] = ch.v;
   }
 }
-template <typename T>
-__device__ __forceinline__ void store_kcontig(char* lds, const u32x4 regs[4]) {
+template <int ROWS>
+__device__ __forceinline__ void store_kcontig(char* lds, const u32x4* regs) {
   const int tid = threadIdx.x;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < ROWS / 32; ++i) {
     int c = tid + NT * i;
     int row = c >> 3, kc = c & 7;
     *reinterpret_cast<u32x4*>(lds + row * PITCH + kc * 16) = regs[i];
   }
 }
 
-// Operand stored with K as the slow index: element (row, k) at p[k * ld + row].
-// Each thread loads a 4 (k) x KV (row) block with four 16-byte reads along the
-// row index and stores it transposed: KV LDS writes of four k-values each.
+// ---- f32 operand with K as the slow index: element (row, k) at p[k * ld + row].
+// 128 rows only. Each thread loads a 4 (k) x 4 (row) block with four 16-byte
+// reads along the row index and stores it transposed into the [row][k] layout.
 template <typename T>
 __device__ __forceinline__ void load_kmajor(const T* __restrict__ p, long ld, int row0, int rows, int k0, int K,
-                                            bool vec, u32x4 regs[4]) {
+                                            bool vec, u32x4* regs) {
   constexpr int KV = 16 / sizeof(T);
   constexpr int MPB = 128 / KV;
   const int tid = threadIdx.x;
@@ -124,7 +123,7 @@ __device__ __forceinline__ void load_kmajor(const T* __restrict__ p, long ld, in
   }
 }
 template <typename T>
-__device__ __forceinline__ void store_kmajor(char* lds, const u32x4 regs[4]) {
+__device__ __forceinline__ void store_kmajor(char* lds, const u32x4* regs) {
   constexpr int KV = 16 / sizeof(T);
   constexpr int MPB = 128 / KV;
   const int tid = threadIdx.x;
@@ -154,6 +153,67 @@ __device__ __forceinline__ void store_kmajor(char* lds, const u32x4 regs[4]) {
   }
 }
 
+// ---- bf16 operand with K as the slow index, kept in LDS as it lies in memory:
+// [64 k][ROWS], pitch ROWS * 2 + 32 bytes (consecutive k rows shift by 8 banks,
+// so the four k rows a 16-lane group touches in one transposing read fall on
+// distinct banks). The copy in is plain 16-byte chunks; the MFMA fragment comes
+// out of two ds_read_b64_tr_b16.
+typedef short short4v __attribute__((ext_vector_type(4)));
+
+template <int ROWS>
+__device__ __forceinline__ void load_km16(const unsigned short* __restrict__ p, long ld, int row0, int rows, int k0,
+                                          int K, bool vec, u32x4* regs) {
+  constexpr int CPR = ROWS / 8;  // 16-byte chunks per k row
+  const int tid = threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < ROWS / 32; ++i) {
+    int c = tid + NT * i;
+    int kr = c / CPR, mc = c % CPR;
+    int gk = k0 + kr, gr = row0 + mc * 8;
+    Chunk<unsigned short> ch;
+    ch.v = u32x4{0u, 0u, 0u, 0u};
+    if (gk < K && gr < rows) {
+      const unsigned short* src = p + static_cast<long>(gk) * ld + gr;
+      if (vec && gr + 8 <= rows) {
+        ch.v = *reinterpret_cast<const u32x4*>(src);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (gr + e < rows) ch.e[e] = src[e];
+      }
+    }
+    regs[i] = ch.v;
+  }
+}
+template <int ROWS>
+__device__ __forceinline__ void store_km16(char* lds, const u32x4* regs) {
+  constexpr int CPR = ROWS / 8;
+  constexpr int PITCH_KM = ROWS * 2 + 32;
+  const int tid = threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < ROWS / 32; ++i) {
+    int c = tid + NT * i;
+    int kr = c / CPR, mc = c % CPR;
+    *reinterpret_cast<u32x4*>(lds + kr * PITCH_KM + mc * 16) = regs[i];
+  }
+}
+// Fragment of rows [row_base, row_base + 32) for k slab kk (16 k values): lane
+// (i = lane%32, g = lane/32) receives k = 16kk + 8g + 0..7 of row row_base + i.
+// A transposing read hands lane j of a 16-lane group element j%4 of the 8-byte
+// words that lanes j/4, 4 + j/4, 8 + j/4, 12 + j/4 of the group point at; so
+// lane s points at k row s/4 (+4 for the second read), row block 4(s%4).
+template <int ROWS>
+__device__ __forceinline__ u32x4 frag_km16(const char* tile, int row_base, int kk, int lane) {
+  constexpr int PITCH_KM = ROWS * 2 + 32;
+  const int s = lane & 15, half = (lane >> 4) & 1, g = lane >> 5;
+  const char* p = tile + (kk * 16 + g * 8 + (s >> 2)) * PITCH_KM + (row_base + half * 16 + (s & 3) * 4) * 2;
+  typedef short4v __attribute__((address_space(3))) * lds_ptr;
+  short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
+  short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 4 * PITCH_KM));
+  u32x2 a = __builtin_bit_cast(u32x2, lo), b = __builtin_bit_cast(u32x2, hi);
+  return u32x4{a.x, a.y, b.x, b.y};
+}
+
 template <typename T>
 __device__ __forceinline__ void mma_step(const u32x4& af, const u32x4& bf, floatx16& acc) {
   if constexpr (sizeof(T) == 2) {
@@ -167,11 +227,23 @@ __device__ __forceinline__ void mma_step(const u32x4& af, const u32x4& bf, float
   }
 }
 
-template <typename T, bool A_KM, bool B_KM>
+template <typename T, bool KM, int ROWS>
+constexpr int tile_bytes() {
+  return (KM && sizeof(T) == 2) ? 64 * (ROWS * 2 + 32) : ROWS * PITCH;
+}
+
+// TM x TN MFMA 32x32 blocks per wave; the 4 waves sit 2 x 2, so the workgroup
+// tile is (64 TM) x (64 TN).
+template <typename T, bool A_KM, bool B_KM, int TM, int TN>
 __global__ __launch_bounds__(NT) void gemm_kernel(GemmArgs g) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int KV = 16 / sizeof(T);
   constexpr int BK = 8 * KV;
+  constexpr int BM = 64 * TM, BN = 64 * TN;
+  constexpr bool A_TR = A_KM && sizeof(T) == 2, B_TR = B_KM && sizeof(T) == 2;
+  constexpr int A_BYTES = tile_bytes<T, A_KM, BM>(), B_BYTES = tile_bytes<T, B_KM, BN>();
+  constexpr int STAGE = A_BYTES + B_BYTES;
+  static_assert(sizeof(T) == 2 || (TM == 2 && TN == 2), "the f32 lane uses 128x128 tiles");
   const T* __restrict__ A = static_cast<const T*>(g.a);
   const T* __restrict__ B = static_cast<const T*>(g.b);
 
@@ -180,16 +252,8 @@ __global__ __launch_bounds__(NT) void gemm_kernel(GemmArgs g) {
   const int total = g.tiles_m * g.tiles_n;
   const int split = blockIdx.x / total;
   int id = blockIdx.x - split * total;
-  {
-    const int per = (total + 7) / 8;
-    int xcd = id & 7, local = id >> 3;
-    int mapped = xcd * per + local;
-    // The last XCD's run may be short; ids that fall off the end wrap into
-    // the gaps (a bijection when total is a multiple of 8, otherwise fall
-    // back to the identity order).
-    id = (total % 8 == 0) ? mapped : id;
-  }
-  // Within the run: walk N fastest inside bands of 8 tile rows.
+  if (total % 8 == 0) id = (id & 7) * (total >> 3) + (id >> 3);
+  // Within the run: walk M fastest inside bands of 8 tile rows.
   const int band = 8;
   int tiles_per_band = band * g.tiles_n;
   int band_id = id / tiles_per_band;
@@ -204,32 +268,36 @@ __global__ __launch_bounds__(NT) void gemm_kernel(GemmArgs g) {
   const int wm = wave >> 1, wn = wave & 1;
   const int l32 = lane & 31, lg = lane >> 5;
 
-  floatx16 acc[2][2];
+  floatx16 acc[TM][TN];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  u32x4 ra[4], rb[4];
+  u32x4 ra[BM / 32], rb[BN / 32];
   const int ksteps_all = (g.K + BK - 1) / BK;
   const int ks_begin = split * g.ksteps_per_split;
   const int ks_end = min(ksteps_all, ks_begin + g.ksteps_per_split);
   auto load_tiles = [&](int ks) {
     int k0 = ks * BK;
-    if constexpr (A_KM) load_kmajor<T>(A, g.lda, m0, g.M, k0, g.K, g.a_vec, ra);
-    else load_kcontig<T>(A, g.lda, m0, g.M, k0, g.K, g.a_vec, ra);
-    if constexpr (B_KM) load_kmajor<T>(B, g.ldb, n0, g.N, k0, g.K, g.b_vec, rb);
-    else load_kcontig<T>(B, g.ldb, n0, g.N, k0, g.K, g.b_vec, rb);
+    if constexpr (A_TR) load_km16<BM>(reinterpret_cast<const unsigned short*>(A), g.lda, m0, g.M, k0, g.K, g.a_vec, ra);
+    else if constexpr (A_KM) load_kmajor<T>(A, g.lda, m0, g.M, k0, g.K, g.a_vec, ra);
+    else load_kcontig<T, BM>(A, g.lda, m0, g.M, k0, g.K, g.a_vec, ra);
+    if constexpr (B_TR) load_km16<BN>(reinterpret_cast<const unsigned short*>(B), g.ldb, n0, g.N, k0, g.K, g.b_vec, rb);
+    else if constexpr (B_KM) load_kmajor<T>(B, g.ldb, n0, g.N, k0, g.K, g.b_vec, rb);
+    else load_kcontig<T, BN>(B, g.ldb, n0, g.N, k0, g.K, g.b_vec, rb);
   };
   auto store_tiles = [&](int buf) {
-    char* la = smem + buf * 2 * TILE_BYTES;
-    char* lb = la + TILE_BYTES;
-    if constexpr (A_KM) store_kmajor<T>(la, ra);
-    else store_kcontig<T>(la, ra);
-    if constexpr (B_KM) store_kmajor<T>(lb, rb);
-    else store_kcontig<T>(lb, rb);
+    char* la = smem + buf * STAGE;
+    char* lb = la + A_BYTES;
+    if constexpr (A_TR) store_km16<BM>(la, ra);
+    else if constexpr (A_KM) store_kmajor<T>(la, ra);
+    else store_kcontig<BM>(la, ra);
+    if constexpr (B_TR) store_km16<BN>(lb, rb);
+    else if constexpr (B_KM) store_kmajor<T>(lb, rb);
+    else store_kcontig<BN>(lb, rb);
   };
 
   load_tiles(ks_begin);
@@ -238,53 +306,59 @@ __global__ __launch_bounds__(NT) void gemm_kernel(GemmArgs g) {
   for (int ks = ks_begin; ks < ks_end; ++ks) {
     const int buf = (ks - ks_begin) & 1;
     if (ks + 1 < ks_end) load_tiles(ks + 1);
-    const char* la = smem + buf * 2 * TILE_BYTES + (wm * 64 + l32) * PITCH + lg * 16;
-    const char* lb = smem + buf * 2 * TILE_BYTES + TILE_BYTES + (wn * 64 + l32) * PITCH + lg * 16;
+    const char* ta = smem + buf * STAGE;
+    const char* tb = ta + A_BYTES;
+    const char* la = ta + (wm * 32 * TM + l32) * PITCH + lg * 16;
+    const char* lb = tb + (wn * 32 * TN + l32) * PITCH + lg * 16;
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
-      u32x4 af[2], bf[2];
+      u32x4 af[TM], bf[TN];
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        af[t] = *reinterpret_cast<const u32x4*>(la + t * 32 * PITCH + kk * 32);
-        bf[t] = *reinterpret_cast<const u32x4*>(lb + t * 32 * PITCH + kk * 32);
+      for (int t = 0; t < TM; ++t) {
+        if constexpr (A_TR) af[t] = frag_km16<BM>(ta, wm * 32 * TM + t * 32, kk, lane);
+        else af[t] = *reinterpret_cast<const u32x4*>(la + t * 32 * PITCH + kk * 32);
       }
 #pragma unroll
-      for (int tm = 0; tm < 2; ++tm)
+      for (int t = 0; t < TN; ++t) {
+        if constexpr (B_TR) bf[t] = frag_km16<BN>(tb, wn * 32 * TN + t * 32, kk, lane);
+        else bf[t] = *reinterpret_cast<const u32x4*>(lb + t * 32 * PITCH + kk * 32);
+      }
 #pragma unroll
-        for (int tn = 0; tn < 2; ++tn) mma_step<T>(af[tm], bf[tn], acc[tm][tn]);
+      for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) mma_step<T>(af[tm], bf[tn], acc[tm][tn]);
     }
     if (ks + 1 < ks_end) store_tiles(buf ^ 1);
     __syncthreads();
   }
+
+  // Accumulator register v of a 32x32 block holds row 8*(v/4) + 4*(lane/32) + v%4, column lane%32.
   if (g.splits > 1) {
     // Partial sums go to the workspace; the reduce kernel adds the splits in
     // ascending order and applies the output conversion and the fault check.
     float* part = g.partial + static_cast<long>(split) * g.M * g.N;
 #pragma unroll
-    for (int tm = 0; tm < 2; ++tm)
+    for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
-      for (int tn = 0; tn < 2; ++tn) {
-        int col = n0 + wn * 64 + tn * 32 + l32;
+      for (int tn = 0; tn < TN; ++tn) {
+        int col = n0 + (wn * TN + tn) * 32 + l32;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          int row = m0 + wm * 64 + tm * 32 + 8 * (v >> 2) + 4 * lg + (v & 3);
+          int row = m0 + (wm * TM + tm) * 32 + 8 * (v >> 2) + 4 * lg + (v & 3);
           if (row < g.M && col < g.N) part[static_cast<long>(row) * g.N + col] = acc[tm][tn][v];
         }
       }
     return;
   }
-
-  // Epilogue. Accumulator register v of a 32x32 block holds
-  // row 8*(v/4) + 4*(lane/32) + v%4, column lane%32.
   bool bad = false;
 #pragma unroll
-  for (int tm = 0; tm < 2; ++tm)
+  for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
-    for (int tn = 0; tn < 2; ++tn) {
-      int col = n0 + wn * 64 + tn * 32 + l32;
+    for (int tn = 0; tn < TN; ++tn) {
+      int col = n0 + (wn * TN + tn) * 32 + l32;
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        int row = m0 + wm * 64 + tm * 32 + 8 * (v >> 2) + 4 * lg + (v & 3);
+        int row = m0 + (wm * TM + tm) * 32 + 8 * (v >> 2) + 4 * lg + (v & 3);
         if (row < g.M && col < g.N) {
           float val = acc[tm][tn][v];
           long off = static_cast<long>(row) * g.ldc + col;
@@ -318,29 +392,32 @@ __global__ void splitk_reduce_kernel(GemmArgs g) {
   if (bad) dev_raise_fault(g.fault, g.tag);
 }
 
-template <typename T>
-int32_t launch(omx_ctx* ctx, GemmArgs& g, bool a_km, bool b_km) {
-  int total = g.tiles_m * g.tiles_n * g.splits;
-  size_t smem = 4 * TILE_BYTES;
-  dim3 grid(total), block(NT);
+template <typename T, bool A_KM, bool B_KM, int TM, int TN>
+int32_t launch_one(omx_ctx* ctx, const GemmArgs& g) {
+  constexpr int BM = 64 * TM, BN = 64 * TN;
+  constexpr int smem = 2 * (tile_bytes<T, A_KM, BM>() + tile_bytes<T, B_KM, BN>());
+  auto kernel = &gemm_kernel<T, A_KM, B_KM, TM, TN>;
   // More than 64 KiB of dynamic LDS has to be granted per kernel, once.
   static bool granted = false;
   if (!granted) {
-    OMX_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<T, false, false>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)));
-    OMX_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<T, false, true>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)));
-    OMX_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<T, true, false>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)));
-    OMX_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<T, true, true>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)));
+    OMX_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     smem));
     granted = true;
   }
-  if (!a_km && !b_km) hipLaunchKernelGGL((gemm_kernel<T, false, false>), grid, block, smem, ctx->stream, g);
-  else if (!a_km && b_km) hipLaunchKernelGGL((gemm_kernel<T, false, true>), grid, block, smem, ctx->stream, g);
-  else if (a_km && !b_km) hipLaunchKernelGGL((gemm_kernel<T, true, false>), grid, block, smem, ctx->stream, g);
-  else hipLaunchKernelGGL((gemm_kernel<T, true, true>), grid, block, smem, ctx->stream, g);
+  const int total = g.tiles_m * g.tiles_n * g.splits;
+  hipLaunchKernelGGL(kernel, dim3(total), dim3(NT), smem, ctx->stream, g);
   OMX_LAUNCH_CHECK(ctx, "gemm_kernel");
+  return OMX_OK;
+}
+
+template <typename T, int TM, int TN>
+int32_t launch(omx_ctx* ctx, const GemmArgs& g, bool a_km, bool b_km) {
+  int32_t rc;
+  if (!a_km && !b_km) rc = launch_one<T, false, false, TM, TN>(ctx, g);
+  else if (!a_km && b_km) rc = launch_one<T, false, true, TM, TN>(ctx, g);
+  else if (a_km && !b_km) rc = launch_one<T, true, false, TM, TN>(ctx, g);
+  else rc = launch_one<T, true, true, TM, TN>(ctx, g);
+  if (rc != OMX_OK) return rc;
   if (g.splits > 1) {
     long elems = static_cast<long>(g.M) * g.N;
     unsigned blocks = static_cast<unsigned>(std::min<long>((elems + 255) / 256, 4096));
@@ -401,6 +478,22 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
   g.accumulate = accumulate;
   g.a_vec = aligned16(a) && (lda % kv == 0);
   g.b_vec = aligned16(b) && (ldb % kv == 0);
+  // Tile shape: (64 TM) x (64 TN). The bf16 lane takes the largest tile that
+  // still gives the chip at least a wave of workgroups; f32 uses 128 x 128.
+  int tm = 2, tn = 2;
+  if (operand_dtype == OMX_BF16) {
+    static const int forced = [] {
+      const char* e = getenv("OMX_GEMM_TILE");
+      return e ? atoi(e) : 0;
+    }();
+    if (forced) {
+      tm = forced / 10;
+      tn = forced % 10;
+    }
+    // Measured on MI355X: with one prefetched K step in flight the 128 x 128
+    // tile (two workgroups per CU) beats the larger tiles on every GPT shape.
+  }
+  const int BM = 64 * tm, BN = 64 * tn;
   g.tiles_m = (g.M + BM - 1) / BM;
   g.tiles_n = (g.N + BN - 1) / BN;
   if (static_cast<long>(g.tiles_m) * g.tiles_n > 0x7fffffffl)
@@ -444,7 +537,12 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
     timed.flops = 2.0 * static_cast<double>(m) * static_cast<double>(n) * static_cast<double>(k);
     OMX_HIP(ctx, hipEventRecord(timed.start, ctx->stream));
   }
-  int32_t rc = operand_dtype == OMX_BF16 ? launch<unsigned short>(ctx, g, a_km, b_km) : launch<float>(ctx, g, a_km, b_km);
+  int32_t rc;
+  if (operand_dtype != OMX_BF16) rc = launch<float, 2, 2>(ctx, g, a_km, b_km);
+  else if (tm == 4 && tn == 2) rc = launch<unsigned short, 4, 2>(ctx, g, a_km, b_km);
+  else if (tm == 2 && tn == 4) rc = launch<unsigned short, 2, 4>(ctx, g, a_km, b_km);
+  else if (tm == 4 && tn == 4) rc = launch<unsigned short, 4, 4>(ctx, g, a_km, b_km);
+  else rc = launch<unsigned short, 2, 2>(ctx, g, a_km, b_km);
   if (ctx->profile_gemm) {
     OMX_HIP(ctx, hipEventRecord(timed.stop, ctx->stream));
     ctx->timed.push_back(timed);

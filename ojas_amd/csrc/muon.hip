@@ -1,0 +1,299 @@
+// Muon NS5 step: BackendModule::muon_ns5_step (ojas-core/src/backend.rs:2480-2491,
+// config :548-570). CPU reference: ojas-cpu/src/optim.rs:684-743 (momentum,
+// Nesterov blend, scale, decay, update) and :841-985 (Newton-Schulz).
+//
+//   buf = mom * m + g;  u = nesterov ? fma(mom, buf, g) : buf
+//   X = u / (||u||_F + 1e-7)        (norm from an f64 sum of squares; read as the
+//                                    short-side-first matrix, a stride choice here)
+//   5 x { A = X X^T;  B = b A + c A A;  X = a X + B X }   (a,b,c) = (3.4445, -4.7750, 2.0315)
+//   p = fma(-lr * sqrt(max(1, rows/cols)), X, p * (1 - lr * wd));  m = buf
+//
+// In bf16 mode X, the norm, the sum with the epsilon, the quotient, every GEMM
+// output and every scalar multiple and sum are rounded to bf16 (optim.rs:947-971);
+// the iterate then lives in bf16 storage and the three products run on the
+// bf16 MFMA lane, whose bf16 output store is exactly that rounding.
+//
+// The step is all-or-nothing: a refuse flag raised by any non-finite
+// intermediate keeps the final pass from writing the parameter or the momentum.
+#include <cmath>
+
+#include "omx_common.h"
+
+namespace {
+
+constexpr int MU_THREADS = 256;
+constexpr size_t MU_BLOCK = 1 << 14;  // elements per sum-of-squares partial
+
+struct MuonScalars {
+  float mom, alpha, decay, a, b, c;
+  int nesterov, decays, bf16;
+};
+
+inline unsigned mu_grid(uint64_t n) {
+  uint64_t blocks = (n + MU_THREADS * 4 - 1) / (MU_THREADS * 4);
+  if (blocks > 4096) blocks = 4096;
+  return static_cast<unsigned>(blocks ? blocks : 1);
+}
+
+// buf, the (possibly bf16-rounded) update u, and per-block f64 sums of u^2.
+__global__ __launch_bounds__(MU_THREADS) void muon_momentum_kernel(const float* __restrict__ g,
+                                                                   const float* __restrict__ m,
+                                                                   float* __restrict__ buf, float* __restrict__ u,
+                                                                   double* __restrict__ partial, size_t n,
+                                                                   MuonScalars s, unsigned int* refuse,
+                                                                   OmxFaultWord* fault, unsigned long long tag) {
+  __shared__ double red[MU_THREADS];
+  const size_t begin = static_cast<size_t>(blockIdx.x) * MU_BLOCK, end = min(n, begin + MU_BLOCK);
+  double acc = 0.0;
+  bool bad = false;
+  for (size_t i = begin + threadIdx.x; i < end; i += MU_THREADS) {
+    float gi = g[i];
+    float b = s.mom * m[i] + gi;
+    bad |= !(dev_finite(b) && dev_finite(gi));
+    float upd = s.nesterov ? fmaf(s.mom, b, gi) : b;
+    if (s.bf16) upd = dev_round_bf16(upd);
+    buf[i] = b;
+    u[i] = upd;
+    acc += static_cast<double>(upd) * static_cast<double>(upd);
+  }
+  red[threadIdx.x] = acc;
+  __syncthreads();
+  for (int st = MU_THREADS / 2; st > 0; st >>= 1) {
+    if (threadIdx.x < st) red[threadIdx.x] += red[threadIdx.x + st];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) partial[blockIdx.x] = red[0];
+  if (bad) {
+    atomicOr(refuse, 1u);
+    dev_raise_fault(fault, tag);
+  }
+}
+
+__global__ __launch_bounds__(1024) void muon_norm_kernel(const double* __restrict__ partial, size_t count,
+                                                         float* __restrict__ denom_out, int bf16,
+                                                         unsigned int* refuse, OmxFaultWord* fault,
+                                                         unsigned long long tag) {
+  __shared__ double red[1024];
+  double acc = 0.0;
+  for (size_t i = threadIdx.x; i < count; i += 1024) acc += partial[i];
+  red[threadIdx.x] = acc;
+  __syncthreads();
+  for (int st = 512; st > 0; st >>= 1) {
+    if (threadIdx.x < st) red[threadIdx.x] += red[threadIdx.x + st];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    float norm = static_cast<float>(sqrt(red[0]));
+    const float eps = 1e-7f;
+    float denom = bf16 ? dev_round_bf16(dev_round_bf16(norm) + eps) : norm + eps;
+    *denom_out = denom;
+    if (!(dev_finite(denom) && denom != 0.0f)) {
+      atomicOr(refuse, 1u);
+      dev_raise_fault(fault, tag);
+    }
+  }
+}
+
+template <typename TX>
+__global__ void muon_normalize_kernel(const float* __restrict__ u, const float* __restrict__ denom,
+                                      TX* __restrict__ x, size_t n) {
+  const float d = *denom;
+  for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += static_cast<size_t>(gridDim.x) * blockDim.x)
+    dev_store<TX>(x, i, u[i] / d);  // bf16 storage rounds the quotient
+}
+
+// B = b A + c A2 (in place over A2), with the bf16 roundings of optim.rs:913-921.
+template <typename TX>
+__global__ void muon_combine_b_kernel(const TX* __restrict__ am, TX* __restrict__ a2, size_t n, MuonScalars s) {
+  for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+    float av = dev_load<TX>(am, i), a2v = dev_load<TX>(a2, i);
+    float r;
+    if (s.bf16) r = dev_round_bf16(s.b * av) + dev_round_bf16(s.c * a2v);
+    else r = s.b * av + s.c * a2v;
+    dev_store<TX>(a2, i, r);
+  }
+}
+
+// X_next = a X + BX (in place over BX), finite-checked (optim.rs:950-962).
+template <typename TX>
+__global__ void muon_combine_x_kernel(const TX* __restrict__ x, TX* __restrict__ bx, size_t n, MuonScalars s,
+                                      unsigned int* refuse, OmxFaultWord* fault, unsigned long long tag) {
+  bool bad = false;
+  for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+    float xv = dev_load<TX>(x, i), bxv = dev_load<TX>(bx, i);
+    float r = s.bf16 ? dev_round_bf16(s.a * xv) + bxv : s.a * xv + bxv;
+    if (s.bf16) r = dev_round_bf16(r);
+    bad |= !dev_finite(r);
+    dev_store<TX>(bx, i, r);
+  }
+  if (bad) {
+    atomicOr(refuse, 1u);
+    dev_raise_fault(fault, tag);
+  }
+}
+
+template <typename TX>
+__global__ void muon_check_update_kernel(const float* __restrict__ p, const TX* __restrict__ x, size_t n,
+                                         MuonScalars s, unsigned int* refuse, OmxFaultWord* fault,
+                                         unsigned long long tag) {
+  bool bad = false;
+  for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+    float base = s.decays ? p[i] * s.decay : p[i];
+    bad |= !dev_finite(fmaf(s.alpha, dev_load<TX>(x, i), base));
+  }
+  if (bad) {
+    atomicOr(refuse, 1u);
+    dev_raise_fault(fault, tag);
+  }
+}
+
+template <typename TX>
+__global__ void muon_apply_kernel(float* __restrict__ p, float* __restrict__ m, const float* __restrict__ buf,
+                                  const TX* __restrict__ x, size_t n, MuonScalars s,
+                                  const unsigned int* __restrict__ refuse, unsigned short* __restrict__ p_bf16) {
+  if (*refuse) return;
+  for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+    float base = s.decays ? p[i] * s.decay : p[i];
+    float np = fmaf(s.alpha, dev_load<TX>(x, i), base);
+    p[i] = np;
+    m[i] = buf[i];
+    if (p_bf16) p_bf16[i] = dev_f32_to_bf16_bits(np);
+  }
+}
+
+struct MuonLayout {
+  uint64_t buf, u, x, xn, a, a2, partial, scalars, total;
+};
+MuonLayout muon_layout(uint64_t rows, uint64_t cols) {
+  auto up = [](uint64_t v) { return (v + 255) & ~255ull; };
+  const uint64_t len = rows * cols, r = rows < cols ? rows : cols;
+  MuonLayout L;
+  uint64_t at = 0;
+  L.buf = at;
+  at += up(len * 4);
+  L.u = at;
+  at += up(len * 4);
+  L.x = at;
+  at += up(len * 4);
+  L.xn = at;
+  at += up(len * 4);
+  L.a = at;
+  at += up(r * r * 4);
+  L.a2 = at;
+  at += up(r * r * 4);
+  L.partial = at;
+  at += up(((len + MU_BLOCK - 1) / MU_BLOCK) * 8);
+  L.scalars = at;
+  at += 256;
+  L.total = at;
+  return L;
+}
+
+template <typename TX>
+int32_t run_muon(omx_ctx* ctx, float* p, const float* g, float* m, uint64_t rows, uint64_t cols, MuonScalars s,
+                 unsigned short* p_bf16, char* ws, const MuonLayout& L, unsigned long long tag) {
+  const uint64_t len = rows * cols;
+  const int32_t XD = sizeof(TX) == 2 ? OMX_BF16 : OMX_F32;
+  float* buf = reinterpret_cast<float*>(ws + L.buf);
+  float* u = reinterpret_cast<float*>(ws + L.u);
+  TX* x = reinterpret_cast<TX*>(ws + L.x);
+  TX* xn = reinterpret_cast<TX*>(ws + L.xn);
+  TX* am = reinterpret_cast<TX*>(ws + L.a);
+  TX* a2 = reinterpret_cast<TX*>(ws + L.a2);
+  double* partial = reinterpret_cast<double*>(ws + L.partial);
+  unsigned int* refuse = reinterpret_cast<unsigned int*>(ws + L.scalars);
+  float* denom = reinterpret_cast<float*>(ws + L.scalars + 16);
+  int32_t rc = omx_fill_zero(ctx, refuse, 4);
+  if (rc != OMX_OK) return rc;
+  const unsigned nb = static_cast<unsigned>((len + MU_BLOCK - 1) / MU_BLOCK);
+  hipLaunchKernelGGL(muon_momentum_kernel, dim3(nb), dim3(MU_THREADS), 0, ctx->stream, g, m, buf, u, partial, len, s,
+                     refuse, ctx->fault, tag);
+  hipLaunchKernelGGL(muon_norm_kernel, dim3(1), dim3(1024), 0, ctx->stream, partial, static_cast<size_t>(nb), denom,
+                     s.bf16, refuse, ctx->fault, tag);
+  hipLaunchKernelGGL((muon_normalize_kernel<TX>), dim3(mu_grid(len)), dim3(MU_THREADS), 0, ctx->stream, u, denom, x,
+                     len);
+  OMX_LAUNCH_CHECK(ctx, "muon prologue");
+  const bool tall = rows > cols;
+  const uint64_t r = tall ? cols : rows, c = tall ? rows : cols;
+  for (int it = 0; it < 5; ++it) {
+    // A = X' X'^T with X' the short-side-first reading of X.
+    if (!tall) rc = omx_gemm_impl(ctx, F_MUON, x, cols, 1, x, 1, cols, XD, am, XD, r, r, c, r, 0);
+    else rc = omx_gemm_impl(ctx, F_MUON, x, 1, cols, x, cols, 1, XD, am, XD, r, r, c, r, 0);
+    if (rc != OMX_OK) return rc;
+    rc = omx_gemm_impl(ctx, F_MUON, am, r, 1, am, r, 1, XD, a2, XD, r, r, r, r, 0);
+    if (rc != OMX_OK) return rc;
+    hipLaunchKernelGGL((muon_combine_b_kernel<TX>), dim3(mu_grid(r * r)), dim3(MU_THREADS), 0, ctx->stream, am, a2,
+                       static_cast<size_t>(r * r), s);
+    // BX in X's own physical layout: B X' when wide, X B^T when tall.
+    if (!tall) rc = omx_gemm_impl(ctx, F_MUON, a2, r, 1, x, cols, 1, XD, xn, XD, cols, r, r, c, 0);
+    else rc = omx_gemm_impl(ctx, F_MUON, x, cols, 1, a2, 1, r, XD, xn, XD, cols, rows, cols, cols, 0);
+    if (rc != OMX_OK) return rc;
+    hipLaunchKernelGGL((muon_combine_x_kernel<TX>), dim3(mu_grid(len)), dim3(MU_THREADS), 0, ctx->stream, x, xn, len,
+                       s, refuse, ctx->fault, tag);
+    OMX_LAUNCH_CHECK(ctx, "muon newton-schulz step");
+    TX* t = x;
+    x = xn;
+    xn = t;
+  }
+  hipLaunchKernelGGL((muon_check_update_kernel<TX>), dim3(mu_grid(len)), dim3(MU_THREADS), 0, ctx->stream, p, x, len,
+                     s, refuse, ctx->fault, tag);
+  hipLaunchKernelGGL((muon_apply_kernel<TX>), dim3(mu_grid(len)), dim3(MU_THREADS), 0, ctx->stream, p, m, buf, x, len,
+                     s, refuse, p_bf16);
+  OMX_LAUNCH_CHECK(ctx, "muon apply");
+  return OMX_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+uint64_t omx_muon_scratch_bytes(uint64_t rows, uint64_t cols) {
+  if (rows == 0 || cols == 0) return 0;
+  return muon_layout(rows, cols).total;
+}
+
+int32_t omx_muon_ns5_step(omx_ctx* ctx, void* param, const void* grad, void* momentum, uint64_t rows, uint64_t cols,
+                          const omx_muon_config* c, void* param_bf16) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "muon_ns5_step";
+  if (!param || !grad || !momentum || !c) return omx_fail(ctx, OMX_PLACEMENT, "%s: null pointer", op);
+  if (rows == 0 || cols == 0) return omx_fail(ctx, OMX_SHAPE, "%s: empty tensor", op);
+  if (rows > 0x7fffffffull || cols > 0x7fffffffull) return omx_fail(ctx, OMX_OUT_OF_RANGE, "%s: axis too large", op);
+  // check_muon, ojas-cpu/src/optim.rs:664-681.
+  if (!std::isfinite(c->lr) || !std::isfinite(c->momentum) || !std::isfinite(c->weight_decay))
+    return omx_fail(ctx, OMX_NON_FINITE, "%s", op);
+  if (c->lr < 0.0) return omx_fail(ctx, OMX_OUT_OF_RANGE, "%s: lr %g is negative", op, c->lr);
+  if (c->momentum < 0.0) return omx_fail(ctx, OMX_OUT_OF_RANGE, "%s: momentum %g is negative", op, c->momentum);
+  if (c->weight_decay < 0.0)
+    return omx_fail(ctx, OMX_OUT_OF_RANGE, "%s: weight_decay %g is negative", op, c->weight_decay);
+  MuonScalars s;
+  s.mom = static_cast<float>(c->momentum);
+  const double ratio = static_cast<double>(rows) / static_cast<double>(cols);
+  s.alpha = static_cast<float>(-c->lr * std::sqrt(ratio > 1.0 ? ratio : 1.0));
+  s.decay = static_cast<float>(1.0 - c->lr * c->weight_decay);
+  s.a = static_cast<float>(3.4445);
+  s.b = static_cast<float>(-4.7750);
+  s.c = static_cast<float>(2.0315);
+  s.nesterov = c->nesterov != 0;
+  s.decays = c->weight_decay != 0.0;
+  s.bf16 = c->ns5_bf16 != 0;
+  const MuonLayout L = muon_layout(rows, cols);
+  void* ws = nullptr;
+  int32_t rc = omx_workspace(ctx, L.total, &ws);
+  if (rc != OMX_OK) return rc;
+  unsigned long long tag = omx_tag(ctx, F_MUON);
+  if (s.bf16)
+    return run_muon<unsigned short>(ctx, static_cast<float*>(param), static_cast<const float*>(grad),
+                                    static_cast<float*>(momentum), rows, cols, s,
+                                    static_cast<unsigned short*>(param_bf16), static_cast<char*>(ws), L, tag);
+  return run_muon<float>(ctx, static_cast<float*>(param), static_cast<const float*>(grad),
+                         static_cast<float*>(momentum), rows, cols, s, static_cast<unsigned short*>(param_bf16),
+                         static_cast<char*>(ws), L, tag);
+}
+
+}  // extern "C"
