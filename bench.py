@@ -31,13 +31,13 @@ BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, vendor figure
 
 
 def cpu_baseline(cfg, threads: int):
-    """Times the oracle on a bounded sample: the same model on a 1 x 256 token batch
-    (forward + backward + clip + AdamW), reported per token."""
+    """Times the oracle on a bounded sample: the same model on one 1 x 1024 token
+    sequence (forward + backward + clip + AdamW), reported per token."""
     sys.path.insert(0, str(ROOT / "tests"))
     import oracle_api as orc
     from ojas_amd.trainer import GptConfig, synthetic_batch
 
-    sample = GptConfig(cfg.layers, cfg.d_model, cfg.heads, cfg.head_dim, cfg.mlp, 256, cfg.vocab, 1, cfg.gelu_tanh, 0)
+    sample = GptConfig(cfg.layers, cfg.d_model, cfg.heads, cfg.head_dim, cfg.mlp, min(cfg.ctx, 1024), cfg.vocab, 1, cfg.gelu_tanh, 0)
     ocfg = orc.GptConfig(sample.layers, sample.d_model, sample.heads, sample.head_dim, sample.mlp, sample.ctx,
                          sample.vocab, sample.batch, sample.gelu_tanh)
     orc.set_threads(threads)

@@ -43,6 +43,7 @@ struct GemmArgs {
   int M, N, K;
   int c_bf16, accumulate;
   int a_vec, b_vec;  // 16-byte loads allowed (alignment of base and leading dimension)
+  int c_vec;         // 4-column stores allowed (alignment of C and its row pitch)
   int tiles_m, tiles_n;
   int splits, ksteps_per_split;  // split-K: each split writes an f32 partial
   float* partial;                // [splits][M][N] when splits > 1
@@ -333,46 +334,84 @@ __global__ __launch_bounds__(NT) void gemm_kernel(GemmArgs g) {
   }
 
   // Accumulator register v of a 32x32 block holds row 8*(v/4) + 4*(lane/32) + v%4, column lane%32.
-  if (g.splits > 1) {
-    // Partial sums go to the workspace; the reduce kernel adds the splits in
-    // ascending order and applies the output conversion and the fault check.
-    float* part = g.partial + static_cast<long>(split) * g.M * g.N;
-#pragma unroll
-    for (int tm = 0; tm < TM; ++tm)
-#pragma unroll
-      for (int tn = 0; tn < TN; ++tn) {
-        int col = n0 + (wn * TN + tn) * 32 + l32;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          int row = m0 + (wm * TM + tm) * 32 + 8 * (v >> 2) + 4 * lg + (v & 3);
-          if (row < g.M && col < g.N) part[static_cast<long>(row) * g.N + col] = acc[tm][tn][v];
-        }
-      }
-    return;
-  }
-  bool bad = false;
+  // The tile is staged through LDS (free after the loop's last barrier) so that
+  // global stores are whole 16-byte (f32) / 8-byte (bf16) pieces of a row.
+  constexpr int CP = BN + 4;  // floats per staged row; the pad keeps 16-byte alignment
+  static_assert(BM * CP * 4 <= 2 * STAGE, "the staged output tile must fit in the operand buffers");
+  float* cs = reinterpret_cast<float*>(smem);
 #pragma unroll
   for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) {
-      int col = n0 + (wn * TN + tn) * 32 + l32;
+      const int col = (wn * TN + tn) * 32 + l32;
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        int row = m0 + (wm * TM + tm) * 32 + 8 * (v >> 2) + 4 * lg + (v & 3);
-        if (row < g.M && col < g.N) {
-          float val = acc[tm][tn][v];
-          long off = static_cast<long>(row) * g.ldc + col;
-          if (g.c_bf16) {
-            static_cast<unsigned short*>(g.c)[off] = dev_f32_to_bf16_bits(val);
-          } else {
-            float* cp = static_cast<float*>(g.c) + off;
-            if (g.accumulate) val += *cp;
-            *cp = val;
-          }
-          bad |= !dev_finite(val);
+        const int row = (wm * TM + tm) * 32 + 8 * (v >> 2) + 4 * lg + (v & 3);
+        cs[row * CP + col] = acc[tm][tn][v];
+      }
+    }
+  __syncthreads();
+  constexpr int CPR = BN / 4;  // 4-column pieces per row
+  const bool split_out = g.splits > 1;
+  float* part = split_out ? g.partial + static_cast<long>(split) * g.M * g.N : nullptr;
+  const long ld_out = split_out ? g.N : g.ldc;
+  const bool vec_out = split_out ? (g.N % 4 == 0) : (g.c_vec != 0);
+  bool bad = false;
+  for (int c = threadIdx.x; c < BM * CPR; c += NT) {
+    const int row = c / CPR, cc = (c % CPR) * 4;
+    const int grow = m0 + row, gcol = n0 + cc;
+    if (grow >= g.M || gcol >= g.N) continue;
+    const float4 val = *reinterpret_cast<const float4*>(cs + row * CP + cc);
+    float x[4] = {val.x, val.y, val.z, val.w};
+    const long off = static_cast<long>(grow) * ld_out + gcol;
+    if (split_out) {
+      // Partial sums go to the workspace; the reduce kernel adds the splits in
+      // ascending order and applies the output conversion and the fault check.
+      if (vec_out && gcol + 4 <= g.N) {
+        *reinterpret_cast<float4*>(part + off) = val;
+      } else {
+        for (int e = 0; e < 4 && gcol + e < g.N; ++e) part[off + e] = x[e];
+      }
+      continue;
+    }
+    const bool whole = vec_out && gcol + 4 <= g.N;
+    if (g.c_bf16) {
+      unsigned short* cp = static_cast<unsigned short*>(g.c) + off;
+      if (whole) {
+        uint2 w;
+        w.x = static_cast<unsigned int>(dev_f32_to_bf16_bits(x[0])) |
+              (static_cast<unsigned int>(dev_f32_to_bf16_bits(x[1])) << 16);
+        w.y = static_cast<unsigned int>(dev_f32_to_bf16_bits(x[2])) |
+              (static_cast<unsigned int>(dev_f32_to_bf16_bits(x[3])) << 16);
+        *reinterpret_cast<uint2*>(cp) = w;
+        bad |= !(dev_finite(x[0]) && dev_finite(x[1]) && dev_finite(x[2]) && dev_finite(x[3]));
+      } else {
+        for (int e = 0; e < 4 && gcol + e < g.N; ++e) {
+          cp[e] = dev_f32_to_bf16_bits(x[e]);
+          bad |= !dev_finite(x[e]);
+        }
+      }
+    } else {
+      float* cp = static_cast<float*>(g.c) + off;
+      if (whole) {
+        if (g.accumulate) {
+          const float4 old = *reinterpret_cast<const float4*>(cp);
+          x[0] += old.x;
+          x[1] += old.y;
+          x[2] += old.z;
+          x[3] += old.w;
+        }
+        *reinterpret_cast<float4*>(cp) = make_float4(x[0], x[1], x[2], x[3]);
+        bad |= !(dev_finite(x[0]) && dev_finite(x[1]) && dev_finite(x[2]) && dev_finite(x[3]));
+      } else {
+        for (int e = 0; e < 4 && gcol + e < g.N; ++e) {
+          float y = g.accumulate ? x[e] + cp[e] : x[e];
+          cp[e] = y;
+          bad |= !dev_finite(y);
         }
       }
     }
+  }
   if (bad) dev_raise_fault(g.fault, g.tag);
 }
 
@@ -478,21 +517,11 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
   g.accumulate = accumulate;
   g.a_vec = aligned16(a) && (lda % kv == 0);
   g.b_vec = aligned16(b) && (ldb % kv == 0);
-  // Tile shape: (64 TM) x (64 TN). The bf16 lane takes the largest tile that
-  // still gives the chip at least a wave of workgroups; f32 uses 128 x 128.
-  int tm = 2, tn = 2;
-  if (operand_dtype == OMX_BF16) {
-    static const int forced = [] {
-      const char* e = getenv("OMX_GEMM_TILE");
-      return e ? atoi(e) : 0;
-    }();
-    if (forced) {
-      tm = forced / 10;
-      tn = forced % 10;
-    }
-    // Measured on MI355X: with one prefetched K step in flight the 128 x 128
-    // tile (two workgroups per CU) beats the larger tiles on every GPT shape.
-  }
+  g.c_vec = aligned16(c) && (ldc % 4 == 0);
+  // Tile shape: (64 TM) x (64 TN). Measured on MI355X: with one prefetched K
+  // step in flight the 128 x 128 tile (two workgroups per CU) beats 256 x 128,
+  // 128 x 256 and 256 x 256 on every GPT shape.
+  const int tm = 2, tn = 2;
   const int BM = 64 * tm, BN = 64 * tn;
   g.tiles_m = (g.M + BM - 1) / BM;
   g.tiles_n = (g.N + BN - 1) / BN;
@@ -539,9 +568,6 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
   }
   int32_t rc;
   if (operand_dtype != OMX_BF16) rc = launch<float, 2, 2>(ctx, g, a_km, b_km);
-  else if (tm == 4 && tn == 2) rc = launch<unsigned short, 4, 2>(ctx, g, a_km, b_km);
-  else if (tm == 2 && tn == 4) rc = launch<unsigned short, 2, 4>(ctx, g, a_km, b_km);
-  else if (tm == 4 && tn == 4) rc = launch<unsigned short, 4, 4>(ctx, g, a_km, b_km);
   else rc = launch<unsigned short, 2, 2>(ctx, g, a_km, b_km);
   if (ctx->profile_gemm) {
     OMX_HIP(ctx, hipEventRecord(timed.stop, ctx->stream));
