@@ -231,6 +231,12 @@ int32_t omx_topk_rows(omx_ctx* ctx, const void* x_f32, uint64_t rows, uint64_t c
  * ojas-model/src/trainer.rs:1031-1046). */
 int32_t omx_read_scalar_f32(omx_ctx* ctx, const void* src, float* out);
 
+/* Tuning knobs (no counterpart in the reference). "gemm_dma": 0 = 128x128 GEMM
+ * kernel only, 1 = choose by shape (default), 2 / 3 = force the 256x256 /
+ * 256x128 direct-to-LDS kernel wherever the operands are eligible. Results are
+ * within the same tolerances under every setting. */
+int32_t omx_set_option(omx_ctx* ctx, const char* name, int64_t value);
+
 /* Benchmark instrumentation (no counterpart in the reference, whose benches
  * time whole ops from the host, bench/README.md:59): while enabled, every
  * launch of the MFMA GEMM kernel is bracketed by two HIP events on the

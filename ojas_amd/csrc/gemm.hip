@@ -23,6 +23,7 @@
 #include <algorithm>
 #include <cstdlib>
 
+#include "gemm_args.h"
 #include "omx_common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -34,22 +35,6 @@ namespace {
 
 constexpr int NT = 256;
 constexpr int PITCH = 144;  // bytes per LDS row of a k-contiguous tile: 8 chunks of 16 B + pad
-
-struct GemmArgs {
-  const void* a;
-  const void* b;
-  void* c;
-  long lda, ldb, ldc;
-  int M, N, K;
-  int c_bf16, accumulate;
-  int a_vec, b_vec;  // 16-byte loads allowed (alignment of base and leading dimension)
-  int c_vec;         // 4-column stores allowed (alignment of C and its row pitch)
-  int tiles_m, tiles_n;
-  int splits, ksteps_per_split;  // split-K: each split writes an f32 partial
-  float* partial;                // [splits][M][N] when splits > 1
-  OmxFaultWord* fault;
-  unsigned long long tag;
-};
 
 template <typename T>
 union Chunk {
@@ -352,65 +337,13 @@ __global__ __launch_bounds__(NT) void gemm_kernel(GemmArgs g) {
     }
   __syncthreads();
   constexpr int CPR = BN / 4;  // 4-column pieces per row
-  const bool split_out = g.splits > 1;
-  float* part = split_out ? g.partial + static_cast<long>(split) * g.M * g.N : nullptr;
-  const long ld_out = split_out ? g.N : g.ldc;
-  const bool vec_out = split_out ? (g.N % 4 == 0) : (g.c_vec != 0);
   bool bad = false;
   for (int c = threadIdx.x; c < BM * CPR; c += NT) {
     const int row = c / CPR, cc = (c % CPR) * 4;
     const int grow = m0 + row, gcol = n0 + cc;
     if (grow >= g.M || gcol >= g.N) continue;
     const float4 val = *reinterpret_cast<const float4*>(cs + row * CP + cc);
-    float x[4] = {val.x, val.y, val.z, val.w};
-    const long off = static_cast<long>(grow) * ld_out + gcol;
-    if (split_out) {
-      // Partial sums go to the workspace; the reduce kernel adds the splits in
-      // ascending order and applies the output conversion and the fault check.
-      if (vec_out && gcol + 4 <= g.N) {
-        *reinterpret_cast<float4*>(part + off) = val;
-      } else {
-        for (int e = 0; e < 4 && gcol + e < g.N; ++e) part[off + e] = x[e];
-      }
-      continue;
-    }
-    const bool whole = vec_out && gcol + 4 <= g.N;
-    if (g.c_bf16) {
-      unsigned short* cp = static_cast<unsigned short*>(g.c) + off;
-      if (whole) {
-        uint2 w;
-        w.x = static_cast<unsigned int>(dev_f32_to_bf16_bits(x[0])) |
-              (static_cast<unsigned int>(dev_f32_to_bf16_bits(x[1])) << 16);
-        w.y = static_cast<unsigned int>(dev_f32_to_bf16_bits(x[2])) |
-              (static_cast<unsigned int>(dev_f32_to_bf16_bits(x[3])) << 16);
-        *reinterpret_cast<uint2*>(cp) = w;
-        bad |= !(dev_finite(x[0]) && dev_finite(x[1]) && dev_finite(x[2]) && dev_finite(x[3]));
-      } else {
-        for (int e = 0; e < 4 && gcol + e < g.N; ++e) {
-          cp[e] = dev_f32_to_bf16_bits(x[e]);
-          bad |= !dev_finite(x[e]);
-        }
-      }
-    } else {
-      float* cp = static_cast<float*>(g.c) + off;
-      if (whole) {
-        if (g.accumulate) {
-          const float4 old = *reinterpret_cast<const float4*>(cp);
-          x[0] += old.x;
-          x[1] += old.y;
-          x[2] += old.z;
-          x[3] += old.w;
-        }
-        *reinterpret_cast<float4*>(cp) = make_float4(x[0], x[1], x[2], x[3]);
-        bad |= !(dev_finite(x[0]) && dev_finite(x[1]) && dev_finite(x[2]) && dev_finite(x[3]));
-      } else {
-        for (int e = 0; e < 4 && gcol + e < g.N; ++e) {
-          float y = g.accumulate ? x[e] + cp[e] : x[e];
-          cp[e] = y;
-          bad |= !dev_finite(y);
-        }
-      }
-    }
+    bad |= gemm_store4(g, split, grow, gcol, val.x, val.y, val.z, val.w);
   }
   if (bad) dev_raise_fault(g.fault, g.tag);
 }
@@ -518,11 +451,27 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
   g.a_vec = aligned16(a) && (lda % kv == 0);
   g.b_vec = aligned16(b) && (ldb % kv == 0);
   g.c_vec = aligned16(c) && (ldc % 4 == 0);
-  // Tile shape: (64 TM) x (64 TN). Measured on MI355X: with one prefetched K
-  // step in flight the 128 x 128 tile (two workgroups per CU) beats 256 x 128,
-  // 128 x 256 and 256 x 256 on every GPT shape.
-  const int tm = 2, tn = 2;
-  const int BM = 64 * tm, BN = 64 * tn;
+  // Kernel choice. bf16 shapes whose output fills the chip with 256 x 256 (or
+  // 256 x 128) tiles take the direct-to-LDS kernel; everything else (f32, odd
+  // shapes, small outputs that need split-K) takes the 128 x 128 kernel.
+  int dma_variant = -1;
+  if (operand_dtype == OMX_BF16 && omx_gemm_dma_eligible(g, a_km, b_km)) {
+    const int mode = ctx->gemm_dma_mode;
+    const long t0 = static_cast<long>((g.M + 255) / 256) * ((g.N + 255) / 256);
+    const long t1 = static_cast<long>((g.M + 255) / 256) * ((g.N + 127) / 128);
+    if (mode == 1) {
+      // Measured on the GPT shapes: small outputs (the d x d weight gradients, the
+      // Newton-Schulz squares) stay on the 128 x 128 kernel; a narrow output with a
+      // long reduction fills the chip better with 256 x 128 tiles; the rest takes 256 x 256.
+      if (static_cast<long>(g.M) * g.N <= (1l << 20)) dma_variant = -1;
+      else if (t0 < 256 && g.K >= 2048 && t1 >= 256) dma_variant = 1;
+      else dma_variant = 0;
+    }
+    else if (mode == 2) dma_variant = 0;
+    else if (mode == 3) dma_variant = 1;
+  }
+  int BM = 128, BN = 128;
+  if (dma_variant >= 0) omx_gemm_dma_tile(dma_variant, &BM, &BN);
   g.tiles_m = (g.M + BM - 1) / BM;
   g.tiles_n = (g.N + BN - 1) / BN;
   if (static_cast<long>(g.tiles_m) * g.tiles_n > 0x7fffffffl)
@@ -567,8 +516,19 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
     OMX_HIP(ctx, hipEventRecord(timed.start, ctx->stream));
   }
   int32_t rc;
-  if (operand_dtype != OMX_BF16) rc = launch<float, 2, 2>(ctx, g, a_km, b_km);
-  else rc = launch<unsigned short, 2, 2>(ctx, g, a_km, b_km);
+  if (dma_variant >= 0) {
+    rc = omx_gemm_dma_launch(ctx, g, a_km, b_km, dma_variant);
+    if (rc == OMX_OK && g.splits > 1) {
+      long elems = static_cast<long>(g.M) * g.N;
+      unsigned blocks = static_cast<unsigned>(std::min<long>((elems + 255) / 256, 4096));
+      hipLaunchKernelGGL(splitk_reduce_kernel, dim3(blocks), dim3(256), 0, ctx->stream, g);
+      OMX_LAUNCH_CHECK(ctx, "splitk_reduce_kernel");
+    }
+  } else if (operand_dtype != OMX_BF16) {
+    rc = launch<float, 2, 2>(ctx, g, a_km, b_km);
+  } else {
+    rc = launch<unsigned short, 2, 2>(ctx, g, a_km, b_km);
+  }
   if (ctx->profile_gemm) {
     OMX_HIP(ctx, hipEventRecord(timed.stop, ctx->stream));
     ctx->timed.push_back(timed);
@@ -577,6 +537,16 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
 }
 
 extern "C" {
+
+int32_t omx_set_option(omx_ctx* ctx, const char* name, int64_t value) {
+  OMX_REQUIRE_CTX(ctx);
+  if (name && strcmp(name, "gemm_dma") == 0) {
+    if (value < 0 || value > 3) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: gemm_dma takes 0..3");
+    ctx->gemm_dma_mode = static_cast<int>(value);
+    return OMX_OK;
+  }
+  return omx_fail(ctx, OMX_UNSUPPORTED, "set_option: unknown option %s", name ? name : "(null)");
+}
 
 int32_t omx_profile_gemm(omx_ctx* ctx, int32_t enable) {
   OMX_REQUIRE_CTX(ctx);

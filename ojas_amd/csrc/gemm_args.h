@@ -1,0 +1,85 @@
+// Launch arguments shared by the GEMM kernels (gemm.hip, gemm_dma.hip).
+#pragma once
+
+#include "omx_common.h"
+
+struct GemmArgs {
+  const void* a;
+  const void* b;
+  void* c;
+  long lda, ldb, ldc;
+  int M, N, K;
+  int c_bf16, accumulate;
+  int a_vec, b_vec;  // 16-byte loads allowed (alignment of base and leading dimension)
+  int c_vec;         // 4-column stores allowed (alignment of C and its row pitch)
+  int tiles_m, tiles_n;
+  int splits, ksteps_per_split;  // split-K: each split writes an f32 partial
+  float* partial;                // [splits][M][N] when splits > 1
+  OmxFaultWord* fault;
+  unsigned long long tag;
+};
+
+// Stores four consecutive columns of one output row (row `grow`, columns
+// gcol..gcol+3, clipped to N): a split-K partial, a bf16 result, or an f32
+// result with optional accumulation. Returns true when a stored value is
+// non-finite (partials are checked by the reduce kernel instead).
+__device__ __forceinline__ bool gemm_store4(const GemmArgs& g, int split, int grow, int gcol, float x0, float x1,
+                                            float x2, float x3) {
+  float x[4] = {x0, x1, x2, x3};
+  bool bad = false;
+  if (g.splits > 1) {
+    float* part = g.partial + static_cast<long>(split) * g.M * g.N + static_cast<long>(grow) * g.N + gcol;
+    if ((g.N & 3) == 0 && gcol + 4 <= g.N) {
+      *reinterpret_cast<float4*>(part) = make_float4(x0, x1, x2, x3);
+    } else {
+      for (int e = 0; e < 4 && gcol + e < g.N; ++e) part[e] = x[e];
+    }
+    return false;
+  }
+  const long off = static_cast<long>(grow) * g.ldc + gcol;
+  const bool whole = g.c_vec != 0 && gcol + 4 <= g.N;
+  if (g.c_bf16) {
+    unsigned short* cp = static_cast<unsigned short*>(g.c) + off;
+    if (whole) {
+      uint2 w;
+      w.x = static_cast<unsigned int>(dev_f32_to_bf16_bits(x0)) |
+            (static_cast<unsigned int>(dev_f32_to_bf16_bits(x1)) << 16);
+      w.y = static_cast<unsigned int>(dev_f32_to_bf16_bits(x2)) |
+            (static_cast<unsigned int>(dev_f32_to_bf16_bits(x3)) << 16);
+      *reinterpret_cast<uint2*>(cp) = w;
+      bad = !(dev_finite(x0) && dev_finite(x1) && dev_finite(x2) && dev_finite(x3));
+    } else {
+      for (int e = 0; e < 4 && gcol + e < g.N; ++e) {
+        cp[e] = dev_f32_to_bf16_bits(x[e]);
+        bad |= !dev_finite(x[e]);
+      }
+    }
+  } else {
+    float* cp = static_cast<float*>(g.c) + off;
+    if (whole) {
+      if (g.accumulate) {
+        const float4 old = *reinterpret_cast<const float4*>(cp);
+        x[0] += old.x;
+        x[1] += old.y;
+        x[2] += old.z;
+        x[3] += old.w;
+      }
+      *reinterpret_cast<float4*>(cp) = make_float4(x[0], x[1], x[2], x[3]);
+      bad = !(dev_finite(x[0]) && dev_finite(x[1]) && dev_finite(x[2]) && dev_finite(x[3]));
+    } else {
+      for (int e = 0; e < 4 && gcol + e < g.N; ++e) {
+        float y = g.accumulate ? x[e] + cp[e] : x[e];
+        cp[e] = y;
+        bad |= !dev_finite(y);
+      }
+    }
+  }
+  return bad;
+}
+
+// bf16 kernel with direct-to-LDS loads and a 256 x 256 (variant 0) or
+// 256 x 128 (variant 1) workgroup tile. Needs K % 64 == 0, 16-byte aligned
+// operands, and row counts that are multiples of 8 for k-major operands.
+bool omx_gemm_dma_eligible(const GemmArgs& g, bool a_km, bool b_km);
+void omx_gemm_dma_tile(int variant, int* bm, int* bn);
+int32_t omx_gemm_dma_launch(omx_ctx* ctx, const GemmArgs& g, bool a_km, bool b_km, int variant);

@@ -1,0 +1,227 @@
+// bf16 MFMA GEMM with direct-to-LDS loads (global_load_lds_dwordx4) and a large
+// workgroup tile, for shapes whose output has enough tiles to fill the chip.
+//
+// Same contract as gemm.hip (C[M,N] (+)= A.B, f32 accumulation, every operand
+// layout; reference: ojas-cpu/src/linalg.rs:69-210), different data movement:
+//   * 512 threads (8 waves); tile 256 x 256 (waves 2 x 4, each 128 x 64) or
+//     256 x 128 (waves 4 x 2, each 64 x 64). Twice the tile edge halves the
+//     L2-to-LDS traffic per FLOP, which is what bounds the 128 x 128 kernel.
+//   * operand tiles go from global memory straight into LDS: no staging
+//     registers and no LDS store instructions. A wave-wide load writes 64
+//     consecutive 16-byte slots, so the LDS tile is unpadded and bank conflicts
+//     are avoided by choosing WHICH chunk each lane fetches (an XOR swizzle):
+//       k-contiguous operand, [row][8 chunks]: slot s of row r holds chunk s ^ (r & 7);
+//       k-major operand, [k][ROWS/8 chunks]:   slot s of k row kr holds chunk s ^ 2(kr & 3)
+//     (the latter keeps the four k rows that one ds_read_b64_tr_b16 group
+//     touches on distinct banks).
+//   * two LDS stages: the loads of K step ks+1 are in flight while step ks is
+//     multiplied; one vmcnt(0) + barrier per step.
+// Rows past M (or N) are fetched from a clamped valid address and never stored.
+#include "gemm_args.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+
+namespace {
+
+constexpr int DT = 512;  // threads
+constexpr int DBK = 64;
+
+// Issues this wave's share of one operand tile's loads. ROWS x 64 bf16 = ROWS / 8 KiB,
+// one wave instruction per KiB.
+template <bool KM, int ROWS>
+__device__ __forceinline__ void issue_tile(const unsigned short* __restrict__ p, long ld, int row0, int rows, int k0,
+                                           char* tile, int wave, int lane) {
+  constexpr int NI = ROWS / 8;  // wave instructions per tile
+#pragma unroll
+  for (int i = 0; i < NI / 8; ++i) {
+    const int q = wave + 8 * i;
+    const unsigned short* src;
+    if constexpr (!KM) {
+      const int r = q * 8 + (lane >> 3);
+      const int kc = (lane & 7) ^ (lane >> 3);
+      int gr = row0 + r;
+      gr = gr < rows ? gr : rows - 1;
+      src = p + static_cast<long>(gr) * ld + k0 + kc * 8;
+    } else {
+      constexpr int CPR = ROWS / 8;
+      const int idx = q * 64 + lane;
+      const int kr = idx / CPR, slot = idx % CPR;
+      const int mc = slot ^ ((kr & 3) * 2);
+      int gm = row0 + mc * 8;
+      gm = gm + 8 <= rows ? gm : 0;
+      src = p + static_cast<long>(k0 + kr) * ld + gm;
+    }
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                     (__attribute__((address_space(3))) void*)(tile + q * 1024), 16, 0, 0);
+  }
+}
+
+template <bool KM, int ROWS>
+__device__ __forceinline__ u32x4 frag(const char* tile, int row_base, int kk, int lane) {
+  if constexpr (!KM) {
+    const int l32 = lane & 31, g = lane >> 5;
+    const int r = row_base + l32;
+    const int kc = kk * 2 + g;
+    return *reinterpret_cast<const u32x4*>(tile + r * 128 + ((kc ^ (r & 7)) << 4));
+  } else {
+    const int s = lane & 15, half = (lane >> 4) & 1, g = lane >> 5;
+    const int kr = kk * 16 + g * 8 + (s >> 2);
+    const int col = row_base + half * 16 + (s & 3) * 4;
+    const int slot = (col >> 3) ^ (((s >> 2) & 3) * 2);
+    const char* p = tile + kr * (ROWS * 2) + slot * 16 + (col & 7) * 2;
+    typedef short4v __attribute__((address_space(3))) * lds_ptr;
+    short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
+    short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 4 * ROWS * 2));
+    u32x2 a = __builtin_bit_cast(u32x2, lo), b = __builtin_bit_cast(u32x2, hi);
+    return u32x4{a.x, a.y, b.x, b.y};
+  }
+}
+
+template <bool A_KM, bool B_KM, int WGM, int WGN, int TM, int TN>
+__global__ __launch_bounds__(DT) void gemm_dma_kernel(GemmArgs g) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
+  constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
+  static_assert(WGM * WGN == 8, "eight waves");
+  const unsigned short* __restrict__ A = static_cast<const unsigned short*>(g.a);
+  const unsigned short* __restrict__ B = static_cast<const unsigned short*>(g.b);
+
+  const int total = g.tiles_m * g.tiles_n;
+  const int split = blockIdx.x / total;
+  int id = blockIdx.x - split * total;
+  if (total % 8 == 0) id = (id & 7) * (total >> 3) + (id >> 3);
+  const int band = 4;
+  const int tiles_per_band = band * g.tiles_n;
+  const int band_id = id / tiles_per_band;
+  const int first_m = band_id * band;
+  const int band_rows = min(band, g.tiles_m - first_m);
+  const int in_band = id - band_id * tiles_per_band;
+  const int tile_m = first_m + in_band % band_rows;
+  const int tile_n = in_band / band_rows;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave / WGN, wn = wave % WGN;
+  const int l32 = lane & 31, lg = lane >> 5;
+
+  floatx16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  const int ksteps_all = g.K / DBK;
+  const int ks_begin = split * g.ksteps_per_split;
+  const int ks_end = min(ksteps_all, ks_begin + g.ksteps_per_split);
+  auto issue = [&](int ks, int buf) {
+    char* ta = smem + buf * STAGE;
+    issue_tile<A_KM, BM>(A, g.lda, m0, g.M, ks * DBK, ta, wave, lane);
+    issue_tile<B_KM, BN>(B, g.ldb, n0, g.N, ks * DBK, ta + A_BYTES, wave, lane);
+  };
+
+  issue(ks_begin, 0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+  __syncthreads();
+  for (int ks = ks_begin; ks < ks_end; ++ks) {
+    const int buf = (ks - ks_begin) & 1;
+    if (ks + 1 < ks_end) issue(ks + 1, buf ^ 1);
+    const char* ta = smem + buf * STAGE;
+    const char* tb = ta + A_BYTES;
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      u32x4 af[TM], bf[TN];
+#pragma unroll
+      for (int t = 0; t < TM; ++t) af[t] = frag<A_KM, BM>(ta, (wm * TM + t) * 32, kk, lane);
+#pragma unroll
+      for (int t = 0; t < TN; ++t) bf[t] = frag<B_KM, BN>(tb, (wn * TN + t) * 32, kk, lane);
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn)
+          acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[tm]),
+                                                                __builtin_bit_cast(bf16x8, bf[tn]), acc[tm][tn], 0, 0,
+                                                                0);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // this wave's loads of the next step have landed
+    __syncthreads();                     // ... and everyone's; everyone is done reading `buf`
+  }
+
+  // Epilogue: each wave stages 32 rows of its tile at a time through its own
+  // LDS region and writes whole 4-column pieces.
+  constexpr int CPW = TN * 32 + 4;
+  static_assert(8 * 32 * CPW * 4 <= 2 * STAGE, "staging fits");
+  float* cs = reinterpret_cast<float*>(smem) + wave * (32 * CPW);
+  bool bad = false;
+#pragma unroll
+  for (int tm = 0; tm < TM; ++tm) {
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) cs[(8 * (v >> 2) + 4 * lg + (v & 3)) * CPW + tn * 32 + l32] = acc[tm][tn][v];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    constexpr int PPR = TN * 8;  // 4-column pieces per row
+#pragma unroll
+    for (int c = lane; c < 32 * PPR; c += 64) {
+      const int row = c / PPR, piece = c % PPR;
+      const int grow = m0 + (wm * TM + tm) * 32 + row, gcol = n0 + wn * TN * 32 + piece * 4;
+      if (grow < g.M && gcol < g.N) {
+        const float4 val = *reinterpret_cast<const float4*>(cs + row * CPW + piece * 4);
+        bad |= gemm_store4(g, split, grow, gcol, val.x, val.y, val.z, val.w);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+  if (bad) dev_raise_fault(g.fault, g.tag);
+}
+
+template <bool A_KM, bool B_KM, int WGM, int WGN, int TM, int TN>
+int32_t launch_dma(omx_ctx* ctx, const GemmArgs& g) {
+  constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
+  constexpr int smem = 2 * (BM + BN) * 128;
+  auto kernel = &gemm_dma_kernel<A_KM, B_KM, WGM, WGN, TM, TN>;
+  static bool granted = false;
+  if (!granted) {
+    OMX_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     smem));
+    granted = true;
+  }
+  hipLaunchKernelGGL(kernel, dim3(g.tiles_m * g.tiles_n * g.splits), dim3(DT), smem, ctx->stream, g);
+  OMX_LAUNCH_CHECK(ctx, "gemm_dma_kernel");
+  return OMX_OK;
+}
+
+template <int WGM, int WGN, int TM, int TN>
+int32_t launch_layout(omx_ctx* ctx, const GemmArgs& g, bool a_km, bool b_km) {
+  if (!a_km && !b_km) return launch_dma<false, false, WGM, WGN, TM, TN>(ctx, g);
+  if (!a_km && b_km) return launch_dma<false, true, WGM, WGN, TM, TN>(ctx, g);
+  if (a_km && !b_km) return launch_dma<true, false, WGM, WGN, TM, TN>(ctx, g);
+  return launch_dma<true, true, WGM, WGN, TM, TN>(ctx, g);
+}
+
+}  // namespace
+
+bool omx_gemm_dma_eligible(const GemmArgs& g, bool a_km, bool b_km) {
+  if (g.K % DBK != 0 || !g.a_vec || !g.b_vec) return false;
+  if (a_km && g.M % 8 != 0) return false;
+  if (b_km && g.N % 8 != 0) return false;
+  return true;
+}
+
+void omx_gemm_dma_tile(int variant, int* bm, int* bn) {
+  *bm = 256;
+  *bn = variant == 0 ? 256 : 128;
+}
+
+int32_t omx_gemm_dma_launch(omx_ctx* ctx, const GemmArgs& g, bool a_km, bool b_km, int variant) {
+  if (variant == 0) return launch_layout<2, 4, 4, 2>(ctx, g, a_km, b_km);
+  return launch_layout<4, 2, 2, 2>(ctx, g, a_km, b_km);
+}

@@ -67,6 +67,8 @@ struct omx_ctx {
   uint64_t workspace_bytes[2] = {0, 0};
   int cu_count = 0;
   // Optional per-launch timing of the GEMM kernel (benchmark only).
+  // 0: 128x128 kernel only; 1: choose by shape; 2 / 3: force the 256x256 / 256x128 direct-to-LDS kernel where eligible.
+  int gemm_dma_mode = 1;
   bool profile_gemm = false;
   struct TimedLaunch {
     hipEvent_t start, stop;

@@ -1,0 +1,63 @@
+"""Every GEMM kernel variant against the oracle: the 128x128 kernel and the two
+direct-to-LDS kernels (256x256, 256x128), forced through `omx_set_option`, on
+shapes with ragged M and N (rows past the edge are fetched from a clamped
+address and must never be stored), every operand layout, split-K, bf16 and f32
+outputs and accumulation."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle_api as orc
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def be():
+    from ojas_amd.backend import MiBackend
+
+    backend = MiBackend(0)
+    yield backend
+    backend._lib.omx_set_option(backend._ctx, b"gemm_dma", C.c_int64(1))
+    backend.close()
+
+
+SHAPES = [(256, 64, 256), (300, 128, 520), (64, 192, 96), (513, 256, 257), (1024, 768, 768), (264, 1024, 136)]
+
+
+@pytest.mark.parametrize("mode", [0, 2, 3])
+@pytest.mark.parametrize("rows,kin,nout", SHAPES)
+def test_linear_bf16_under_each_kernel(be, mode, rows, kin, nout):
+    from ojas_amd.backend import BF16, F32
+
+    print(f"gemm mode {mode} {rows}x{kin}x{nout}", flush=True)
+    assert be._lib.omx_set_option(be._ctx, b"gemm_dma", C.c_int64(mode)) == 0
+    r = orc.SplitMix64(5000 + rows + mode)
+    x = orc.round_bf16(r.vec(rows * kin, 0.5)).reshape(rows, kin)
+    w = orc.round_bf16(r.vec(nout * kin, 0.5)).reshape(nout, kin)
+    gy = orc.round_bf16(r.vec(rows * nout, 0.5)).reshape(rows, nout)
+    orc.set_threads(8)
+    oy = orc.linear_forward(x, w)
+    ogx, ogw = orc.linear_backward(x, w, gy)
+    dx, dw, dgy = be.upload(x, BF16), be.upload(w, BF16), be.upload(gy, BF16)
+
+    def close(got, want, tol, what):
+        err = float(np.max(np.abs(np.asarray(got, np.float64) - want)))
+        assert err <= tol * max(1.0, float(np.max(np.abs(want)))), (what, err)
+
+    close(be.download(be.linear_forward(dx, dw)), oy, 1e-5, "fwd f32 out")
+    close(be.download_f32(be.linear_forward(dx, dw, out_dtype=BF16)), oy, 2e-2, "fwd bf16 out")
+    gx, gw = be.linear_backward(dx, dw, dgy, gx_dtype=F32)
+    close(be.download(gx), ogx, 1e-5, "gx")
+    close(be.download(gw), ogw, 1e-5, "gw")
+    # Accumulation into an f32 output continues the stored values.
+    c0 = r.vec(rows * nout, 0.5).reshape(rows, nout)
+    dc = be.upload(c0)
+    be.gemm(dx, (kin, 1), dw, (1, kin), rows, kin, nout, c=dc)
+    close(be.download(dc), oy.astype(np.float64) + c0, 1e-5, "accumulate")
+
+
+def test_unknown_option_is_refused(be):
+    assert be._lib.omx_set_option(be._ctx, b"no_such_knob", C.c_int64(1)) == 11
+    assert be._lib.omx_set_option(be._ctx, b"gemm_dma", C.c_int64(9)) == 3
