@@ -180,15 +180,20 @@ __global__ __launch_bounds__(FT) void flash_fwd_kernel(const unsigned short* __r
   const int block_q0 = qb * 128, block_q1 = min(T - 1, qb * 128 + 127);
   const int kt_first = s.window > 0 ? max(0, block_q0 + 1 - s.window) / 64 : 0;
   const int kt_last = block_q1 / 64;
+  // The next tile's global loads are in flight while the current one is multiplied.
+  u32x4 rk[2], rv[2];
+  tile_load(kp, kt_first * 64, T, rk);
+  tile_load(vp, kt_first * 64, T, rv);
   for (int kt = kt_first; kt <= kt_last; ++kt) {
     const int key0 = kt * 64;
-    u32x4 rk[2], rv[2];
-    tile_load(kp, key0, T, rk);
-    tile_load(vp, key0, T, rv);
     __syncthreads();  // the previous tile's reads are done
     tile_store_rows(k_rows, rk);
     tile_store_transposed(v_tr, rv);
     __syncthreads();
+    if (kt < kt_last) {
+      tile_load(kp, key0 + 64, T, rk);
+      tile_load(vp, key0 + 64, T, rv);
+    }
     const bool active = key0 <= wave_q0 + 31 && (s.window == 0 || key0 + 63 + s.window > wave_q0);
     if (!active) continue;
     floatx16 sc[2] = {zero16(), zero16()};
@@ -277,21 +282,29 @@ __global__ __launch_bounds__(FT) void flash_bwd_dkv_kernel(
   const int qt_first = block_k0 / 64;
   const int qt_last = (s.window > 0 ? min(T - 1, block_k1 + s.window - 1) : T - 1) / 64;
   bool bad = false;
-  for (int r = 0; r < s.rep; ++r) {
+  // One flat loop over (query head of the group, query tile), ascending, so the
+  // next tile's global loads can be in flight while the current one is multiplied.
+  const int nq = qt_last - qt_first + 1;
+  const int steps = s.rep * nq;
+  u32x4 rq[2], rg[2];
+  float row_lse = 0.0f, row_del = 0.0f;
+  auto fetch = [&](int idx) {
+    const int r = idx / nq, q0 = (qt_first + idx % nq) * 64;
     const long q_plane = static_cast<long>(b) * s.heads + static_cast<long>(gidx) * s.rep + r;
-    const unsigned short* qp = q + q_plane * T * FD;
-    const unsigned short* gp = gy + q_plane * T * FD;
-    for (int qt = qt_first; qt <= qt_last; ++qt) {
-      const int q0 = qt * 64;
-      u32x4 rq[2], rg[2];
-      tile_load(qp, q0, T, rq);
-      tile_load(gp, q0, T, rg);
-      float row_lse = 0.0f, row_del = 0.0f;
-      if (threadIdx.x < 64 && q0 + static_cast<int>(threadIdx.x) < T) {
-        row_lse = lse[q_plane * T + q0 + threadIdx.x];
-        row_del = delta[q_plane * T + q0 + threadIdx.x];
-        bad |= !(dev_finite(row_lse) && dev_finite(row_del));
-      }
+    tile_load(q + q_plane * T * FD, q0, T, rq);
+    tile_load(gy + q_plane * T * FD, q0, T, rg);
+    row_lse = 0.0f;
+    row_del = 0.0f;
+    if (threadIdx.x < 64 && q0 + static_cast<int>(threadIdx.x) < T) {
+      row_lse = lse[q_plane * T + q0 + threadIdx.x];
+      row_del = delta[q_plane * T + q0 + threadIdx.x];
+      bad |= !(dev_finite(row_lse) && dev_finite(row_del));
+    }
+  };
+  fetch(0);
+  for (int idx = 0; idx < steps; ++idx) {
+    {
+      const int q0 = (qt_first + idx % nq) * 64;
       __syncthreads();
       tile_store_rows(q_rows, rq);
       tile_store_rows(g_rows, rg);
@@ -302,6 +315,7 @@ __global__ __launch_bounds__(FT) void flash_bwd_dkv_kernel(
         del_s[threadIdx.x] = row_del;
       }
       __syncthreads();
+      if (idx + 1 < steps) fetch(idx + 1);
       const bool active = q0 + 63 >= wave_k0 && (s.window == 0 || q0 < wave_k0 + 31 + s.window);
       if (!active) continue;
 #pragma unroll
@@ -376,16 +390,20 @@ __global__ __launch_bounds__(FT) void flash_bwd_dq_kernel(
   const int block_q0 = qb * 128, block_q1 = min(T - 1, qb * 128 + 127);
   const int kt_first = s.window > 0 ? max(0, block_q0 + 1 - s.window) / 64 : 0;
   const int kt_last = block_q1 / 64;
+  u32x4 rk[2], rv[2];
+  tile_load(kp, kt_first * 64, T, rk);
+  tile_load(vp, kt_first * 64, T, rv);
   for (int kt = kt_first; kt <= kt_last; ++kt) {
     const int key0 = kt * 64;
-    u32x4 rk[2], rv[2];
-    tile_load(kp, key0, T, rk);
-    tile_load(vp, key0, T, rv);
     __syncthreads();
     tile_store_rows(k_rows, rk);
     tile_store_rows(v_rows, rv);
     tile_store_transposed(k_tr, rk);
     __syncthreads();
+    if (kt < kt_last) {
+      tile_load(kp, key0 + 64, T, rk);
+      tile_load(vp, key0 + 64, T, rv);
+    }
     const bool active = key0 <= wave_q0 + 31 && (s.window == 0 || key0 + 63 + s.window > wave_q0);
     if (!active) continue;
 #pragma unroll
