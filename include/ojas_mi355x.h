@@ -221,6 +221,73 @@ int32_t omx_gelu_backward(omx_ctx* ctx, const void* x, const void* gy, void* gx,
 int32_t omx_permute_0213(omx_ctx* ctx, const void* x, void* y, int32_t dtype, uint64_t d0,
                          uint64_t d1, uint64_t d2, uint64_t d3);
 
+/* ---- ops of the nanolab block (graph B) ---- */
+/* BackendFloat::silu_forward / silu_backward (backend.rs:1151-1153; CPU
+ * ojas-cpu/src/pointwise.rs:346-366,515-546): y = x sigmoid(x). */
+int32_t omx_silu_forward(omx_ctx* ctx, const void* x, void* y, int32_t dtype, uint64_t n);
+int32_t omx_silu_backward(omx_ctx* ctx, const void* x, const void* gy, void* gx, int32_t dtype,
+                          uint64_t n);
+/* BackendFloat::mul_forward / mul_backward (backend.rs:1155-1163): out = a b;
+ * ga = gy b, gb = gy a. */
+int32_t omx_mul_forward(omx_ctx* ctx, const void* a, const void* b, void* out, int32_t dtype,
+                        uint64_t n);
+int32_t omx_mul_backward(omx_ctx* ctx, const void* a, const void* b, const void* gy, void* ga,
+                         void* gb, int32_t dtype, uint64_t n);
+/* BackendModule::rope_half_split_forward / _backward (backend.rs:1674-1686; CPU
+ * ojas-cpu/src/norm.rs:271-312). x is [rows, dim] with dim even; cos / sin are
+ * f32. heads > 0: tables are [time, dim] and row r uses table row
+ * (r / heads) % time (x is [.., time, heads, dim]). heads == 0: tables are
+ * shaped like x. The backward takes grad_output in x's place. */
+int32_t omx_rope_half_split_forward(omx_ctx* ctx, const void* x, const void* cos_f32,
+                                    const void* sin_f32, void* y, int32_t dtype, uint64_t rows,
+                                    uint64_t dim, uint64_t time, uint64_t heads);
+int32_t omx_rope_half_split_backward(omx_ctx* ctx, const void* gy, const void* cos_f32,
+                                     const void* sin_f32, void* gx, int32_t dtype, uint64_t rows,
+                                     uint64_t dim, uint64_t time, uint64_t heads);
+/* BackendModule::rms_qk_norm_forward / _backward (backend.rs:1688-1708; CPU
+ * ojas-cpu/src/backend.rs:1011-1040): RMSNorm over the last axis of q and of k,
+ * each with its own weight. Both pairs are validated before either runs. */
+int32_t omx_rms_qk_norm_forward(omx_ctx* ctx, const void* q, const void* k, int32_t x_dtype,
+                                const void* q_weight_f32, const void* k_weight_f32, void* q_out,
+                                void* k_out, int32_t y_dtype, uint64_t q_rows, uint64_t k_rows,
+                                uint64_t dim, float eps);
+int32_t omx_rms_qk_norm_backward(omx_ctx* ctx, const void* q, const void* k, int32_t x_dtype,
+                                 const void* q_weight_f32, const void* k_weight_f32,
+                                 const void* grad_q, const void* grad_k, int32_t gy_dtype, void* gq,
+                                 void* gk, int32_t gx_dtype, void* gq_weight_f32,
+                                 void* gk_weight_f32, uint64_t q_rows, uint64_t k_rows, uint64_t dim,
+                                 float eps);
+/* BackendModule::per_head_sigmoid_gate_forward[_saving] / _backward[_saved]
+ * (backend.rs:1860-1905; CPU ojas-cpu/src/pointwise.rs:1395-1470,1678-1781,
+ * 1853-1894): gates[r, h] = sigmoid(bias[h] + input[r, :] . weight[h, :]),
+ * y[r, h, :] = attn[r, h, :] gates[r, h]. input [rows, d_model] and weight
+ * [heads, d_model] share operand_dtype; bias is f32. `gates_f32` [rows, heads]
+ * may be null: the forward then keeps nothing, and the backward recomputes the
+ * gates instead of reading saved ones. */
+int32_t omx_per_head_sigmoid_gate_forward(omx_ctx* ctx, const void* input, const void* weight,
+                                          int32_t operand_dtype, const void* bias_f32,
+                                          const void* attn, int32_t attn_dtype, void* y,
+                                          int32_t y_dtype, void* gates_f32, uint64_t rows,
+                                          uint64_t d_model, uint64_t heads, uint64_t head_dim);
+int32_t omx_per_head_sigmoid_gate_backward(omx_ctx* ctx, const void* input, const void* weight,
+                                           int32_t operand_dtype, const void* bias_f32,
+                                           const void* attn, int32_t attn_dtype, const void* gy,
+                                           int32_t gy_dtype, const void* gates_f32, void* g_input,
+                                           int32_t g_input_dtype, void* g_weight_f32,
+                                           void* g_bias_f32, void* g_attn, int32_t g_attn_dtype,
+                                           uint64_t rows, uint64_t d_model, uint64_t heads,
+                                           uint64_t head_dim);
+/* BackendModule::value_residual_blend_forward / _backward (backend.rs:1907-1920;
+ * CPU ojas-cpu/src/pointwise.rs:2031-2148): out = (1 - s) v + s v0 with
+ * s = sigmoid(lambda); lambda and grad_lambda are one f32 each on the device. */
+int32_t omx_value_residual_blend_forward(omx_ctx* ctx, const void* value, const void* value0,
+                                         const void* lambda_f32, void* out, int32_t dtype,
+                                         uint64_t n);
+int32_t omx_value_residual_blend_backward(omx_ctx* ctx, const void* value, const void* value0,
+                                          const void* lambda_f32, const void* gy, void* g_value,
+                                          void* g_value0, int32_t dtype, void* g_lambda_f32,
+                                          uint64_t n);
+
 /* ---- BackendInt::argmax_rows / topk_rows (backend.rs:1514-1606) ---- */
 int32_t omx_argmax_rows(omx_ctx* ctx, const void* x_f32, uint64_t rows, uint64_t cols,
                         void* out_u32);

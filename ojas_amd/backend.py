@@ -437,6 +437,164 @@ class MiBackend:
                                                C.c_uint64(d1), C.c_uint64(d2), C.c_uint64(d3)))
         return y
 
+    # ---- ops of the nanolab block (backend.rs:1151-1163,1674-1708,1860-1920) ----
+    def _same(self, op, *tensors):
+        first = tensors[0]
+        for t in tensors[1:]:
+            if t.shape != first.shape:
+                raise OjasError(SHAPE, f"{op}: shapes {first.shape} and {t.shape} differ")
+            if t.dtype != first.dtype:
+                raise OjasError(DTYPE, f"{op}: operands must share a dtype")
+
+    def silu_forward(self, x):
+        y = self.empty(x.shape, x.dtype)
+        self._check(self._lib.omx_silu_forward(self._ctx, self._p(x), self._p(y), C.c_int32(x.dtype),
+                                               C.c_uint64(x.numel)))
+        return y
+
+    def silu_backward(self, x, gy):
+        self._same("silu_backward", x, gy)
+        gx = self.empty(x.shape, x.dtype)
+        self._check(self._lib.omx_silu_backward(self._ctx, self._p(x), self._p(gy), self._p(gx), C.c_int32(x.dtype),
+                                                C.c_uint64(x.numel)))
+        return gx
+
+    def mul_forward(self, a, b):
+        self._same("mul_forward", a, b)
+        out = self.empty(a.shape, a.dtype)
+        self._check(self._lib.omx_mul_forward(self._ctx, self._p(a), self._p(b), self._p(out), C.c_int32(a.dtype),
+                                              C.c_uint64(a.numel)))
+        return out
+
+    def mul_backward(self, a, b, gy):
+        self._same("mul_backward", a, b, gy)
+        ga, gb = self.empty(a.shape, a.dtype), self.empty(a.shape, a.dtype)
+        self._check(self._lib.omx_mul_backward(self._ctx, self._p(a), self._p(b), self._p(gy), self._p(ga),
+                                               self._p(gb), C.c_int32(a.dtype), C.c_uint64(a.numel)))
+        return ga, gb
+
+    def _rope(self, fn, op, x, cos, sin):
+        if cos.shape != sin.shape:
+            raise OjasError(SHAPE, f"{op}: cos shape {cos.shape} != sin shape {sin.shape}")
+        if cos.dtype != F32 or sin.dtype != F32:
+            raise OjasError(DTYPE, f"{op}: cos and sin must be f32")
+        dim = x.shape[-1]
+        if dim % 2:
+            raise OjasError(SHAPE, f"{op}: rope last dim {dim} is odd")
+        rows = x.numel // dim
+        if cos.shape == x.shape:
+            time, heads = 0, 0
+        elif len(x.shape) == 4 and cos.shape == (x.shape[1], dim):
+            time, heads = x.shape[1], x.shape[2]
+        else:
+            raise OjasError(SHAPE, f"{op}: cos/sin shape {cos.shape} does not broadcast onto {x.shape}")
+        y = self.empty(x.shape, x.dtype)
+        self._check(fn(self._ctx, self._p(x), self._p(cos), self._p(sin), self._p(y), C.c_int32(x.dtype),
+                       C.c_uint64(rows), C.c_uint64(dim), C.c_uint64(time), C.c_uint64(heads)))
+        return y
+
+    def rope_half_split_forward(self, x, cos, sin):
+        return self._rope(self._lib.omx_rope_half_split_forward, "rope_half_split_forward", x, cos, sin)
+
+    def rope_half_split_backward(self, grad_output, cos, sin):
+        return self._rope(self._lib.omx_rope_half_split_backward, "rope_half_split_backward", grad_output, cos, sin)
+
+    def rms_qk_norm_forward(self, q, k, q_weight, k_weight, eps: float = 1e-6, out_dtype: Optional[int] = None):
+        dim = q.shape[-1]
+        if k.shape[-1] != dim or q_weight.shape != (dim,) or k_weight.shape != (dim,) or q.dtype != k.dtype:
+            raise OjasError(SHAPE, f"rms_qk_norm_forward: q {q.shape} k {k.shape} weights {q_weight.shape} "
+                                   f"{k_weight.shape}")
+        od = q.dtype if out_dtype is None else out_dtype
+        qn, kn = self.empty(q.shape, od), self.empty(k.shape, od)
+        self._check(self._lib.omx_rms_qk_norm_forward(
+            self._ctx, self._p(q), self._p(k), C.c_int32(q.dtype), self._p(q_weight), self._p(k_weight), self._p(qn),
+            self._p(kn), C.c_int32(od), C.c_uint64(q.numel // dim), C.c_uint64(k.numel // dim), C.c_uint64(dim),
+            C.c_float(eps)))
+        return qn, kn
+
+    def rms_qk_norm_backward(self, q, k, q_weight, k_weight, grad_q, grad_k, eps: float = 1e-6):
+        dim = q.shape[-1]
+        if k.shape[-1] != dim or grad_q.shape != q.shape or grad_k.shape != k.shape or grad_q.dtype != grad_k.dtype:
+            raise OjasError(SHAPE, "rms_qk_norm_backward: gradient shapes do not match q / k")
+        gq, gk = self.empty(q.shape, grad_q.dtype), self.empty(k.shape, grad_q.dtype)
+        gqw, gkw = self.empty((dim,), F32), self.empty((dim,), F32)
+        self._check(self._lib.omx_rms_qk_norm_backward(
+            self._ctx, self._p(q), self._p(k), C.c_int32(q.dtype), self._p(q_weight), self._p(k_weight),
+            self._p(grad_q), self._p(grad_k), C.c_int32(grad_q.dtype), self._p(gq), self._p(gk),
+            C.c_int32(grad_q.dtype), self._p(gqw), self._p(gkw), C.c_uint64(q.numel // dim),
+            C.c_uint64(k.numel // dim), C.c_uint64(dim), C.c_float(eps)))
+        return gq, gk, gqw, gkw
+
+    def _gate_dims(self, op, x, w, b, attn):
+        if len(w.shape) != 2:
+            raise OjasError(SHAPE, f"{op}: gate weight must be [n_head, d_model]")
+        heads, d_model = w.shape
+        if x.shape[-1] != d_model:
+            raise OjasError(SHAPE, f"{op}: gate weight in {d_model} != input dim {x.shape[-1]}")
+        if b.shape != (heads,):
+            raise OjasError(SHAPE, f"{op}: gate bias {b.shape} != [{heads}]")
+        if len(attn.shape) != len(x.shape) + 1 or attn.shape[-2] != heads or attn.shape[:-2] != x.shape[:-1]:
+            raise OjasError(SHAPE, f"{op}: gate attn {attn.shape} does not match input {x.shape}")
+        if x.dtype != w.dtype or b.dtype != F32:
+            raise OjasError(DTYPE, f"{op}: input and weight share a dtype; bias is f32")
+        return x.numel // d_model, d_model, heads, attn.shape[-1]
+
+    def per_head_sigmoid_gate_forward_saving(self, x, w, b, attn, out_dtype: Optional[int] = None, save=True):
+        op = "per_head_sigmoid_gate_forward"
+        rows, d_model, heads, dh = self._gate_dims(op, x, w, b, attn)
+        od = attn.dtype if out_dtype is None else out_dtype
+        y = self.empty(attn.shape, od)
+        gates = self.empty((rows, heads), F32) if save else None
+        self._check(self._lib.omx_per_head_sigmoid_gate_forward(
+            self._ctx, self._p(x), self._p(w), C.c_int32(x.dtype), self._p(b), self._p(attn), C.c_int32(attn.dtype),
+            self._p(y), C.c_int32(od), self._p(gates), C.c_uint64(rows), C.c_uint64(d_model), C.c_uint64(heads),
+            C.c_uint64(dh)))
+        return y, gates
+
+    def per_head_sigmoid_gate_forward(self, x, w, b, attn, out_dtype: Optional[int] = None):
+        return self.per_head_sigmoid_gate_forward_saving(x, w, b, attn, out_dtype, save=False)[0]
+
+    def per_head_sigmoid_gate_backward_saved(self, x, w, b, attn, gy, scales, g_input_dtype: Optional[int] = None):
+        op = "per_head_sigmoid_gate_backward"
+        rows, d_model, heads, dh = self._gate_dims(op, x, w, b, attn)
+        if gy.shape != attn.shape or gy.dtype != attn.dtype:
+            raise OjasError(SHAPE, f"{op}: grad_output {gy.shape} != attn {attn.shape}")
+        if scales is not None and (scales.shape != (rows, heads) or scales.dtype != F32):
+            raise OjasError(SHAPE, f"{op}: gate scale length does not match rows * heads")
+        gxd = x.dtype if g_input_dtype is None else g_input_dtype
+        gx, gw = self.empty(x.shape, gxd), self.empty(w.shape, F32)
+        gb, ga = self.empty((heads,), F32), self.empty(attn.shape, attn.dtype)
+        self._check(self._lib.omx_per_head_sigmoid_gate_backward(
+            self._ctx, self._p(x), self._p(w), C.c_int32(x.dtype), self._p(b), self._p(attn), C.c_int32(attn.dtype),
+            self._p(gy), C.c_int32(gy.dtype), self._p(scales), self._p(gx), C.c_int32(gxd), self._p(gw), self._p(gb),
+            self._p(ga), C.c_int32(attn.dtype), C.c_uint64(rows), C.c_uint64(d_model), C.c_uint64(heads),
+            C.c_uint64(dh)))
+        return gx, gw, gb, ga
+
+    def per_head_sigmoid_gate_backward(self, x, w, b, attn, gy, g_input_dtype: Optional[int] = None):
+        return self.per_head_sigmoid_gate_backward_saved(x, w, b, attn, gy, None, g_input_dtype)
+
+    def value_residual_blend_forward(self, value, value0, lam):
+        self._same("value_residual_blend_forward", value, value0)
+        if lam.numel != 1 or lam.dtype != F32:
+            raise OjasError(SHAPE, "value_residual_blend_forward: lambda must be one f32")
+        out = self.empty(value.shape, value.dtype)
+        self._check(self._lib.omx_value_residual_blend_forward(
+            self._ctx, self._p(value), self._p(value0), self._p(lam), self._p(out), C.c_int32(value.dtype),
+            C.c_uint64(value.numel)))
+        return out
+
+    def value_residual_blend_backward(self, value, value0, lam, gy):
+        self._same("value_residual_blend_backward", value, value0, gy)
+        if lam.numel != 1 or lam.dtype != F32:
+            raise OjasError(SHAPE, "value_residual_blend_backward: lambda must be one f32")
+        gv, gv0 = self.empty(value.shape, value.dtype), self.empty(value.shape, value.dtype)
+        gl = self.empty((1,), F32)
+        self._check(self._lib.omx_value_residual_blend_backward(
+            self._ctx, self._p(value), self._p(value0), self._p(lam), self._p(gy), self._p(gv), self._p(gv0),
+            C.c_int32(value.dtype), self._p(gl), C.c_uint64(value.numel)))
+        return gv, gv0, gl
+
     # ---- integer ops ----
     def argmax_rows(self, x):
         rows, cols = x.shape

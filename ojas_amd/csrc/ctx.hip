@@ -29,6 +29,18 @@ static const char* kFaultNames[F_COUNT] = {
     "gelu_backward",
     "argmax_rows",
     "topk_rows",
+    "silu_forward",
+    "silu_backward",
+    "mul_forward",
+    "mul_backward",
+    "rope_half_split_forward",
+    "rope_half_split_backward",
+    "rms_qk_norm_forward",
+    "rms_qk_norm_backward",
+    "per_head_sigmoid_gate_forward",
+    "per_head_sigmoid_gate_backward",
+    "value_residual_blend_forward",
+    "value_residual_blend_backward",
 };
 
 const char* omx_fault_name(uint32_t op) { return op < F_COUNT ? kFaultNames[op] : "unknown"; }

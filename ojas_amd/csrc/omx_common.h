@@ -39,6 +39,18 @@ enum OmxFaultOp : uint32_t {
   F_GELU_BACKWARD,
   F_ARGMAX,
   F_TOPK,
+  F_SILU_FORWARD,
+  F_SILU_BACKWARD,
+  F_MUL_FORWARD,
+  F_MUL_BACKWARD,
+  F_ROPE_FORWARD,
+  F_ROPE_BACKWARD,
+  F_RMS_QK_FORWARD,
+  F_RMS_QK_BACKWARD,
+  F_GATE_FORWARD,
+  F_GATE_BACKWARD,
+  F_VRES_FORWARD,
+  F_VRES_BACKWARD,
   F_COUNT
 };
 const char* omx_fault_name(uint32_t op);
@@ -91,6 +103,9 @@ inline unsigned long long omx_tag(omx_ctx* ctx, uint32_t op) {
 int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a_rs, uint64_t a_cs, const void* b,
                       uint64_t b_rs, uint64_t b_cs, int32_t operand_dtype, void* c, int32_t c_dtype, uint64_t ldc,
                       uint64_t m, uint64_t k, uint64_t n, int32_t accumulate);
+// out[c] = sum over b < blocks of partial[b * dim + c], added in a fixed order.
+int32_t omx_column_sum(omx_ctx* ctx, const float* partial, float* out, uint64_t blocks, uint64_t dim,
+                       unsigned long long tag);
 // Elementwise conversions on the context's stream (no fault reporting).
 int32_t omx_convert(omx_ctx* ctx, const void* src, int32_t src_dtype, void* dst, int32_t dst_dtype, uint64_t n);
 

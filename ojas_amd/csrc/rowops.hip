@@ -390,7 +390,9 @@ int32_t launch_rms_fwd(omx_ctx* ctx, const void* x, const float* w, void* y, uin
 template <typename TX, typename TG, typename TO>
 int32_t launch_rms_bwd(omx_ctx* ctx, const void* x, const float* w, const void* gy, void* gx, float* gw,
                        uint64_t rows, uint64_t dim, float eps, unsigned long long tag) {
-  const int rows_per_block = 32;
+  // 32 rows per block, more when that would leave over 2048 partial rows to add.
+  int rows_per_block = 32;
+  while ((rows + rows_per_block - 1) / rows_per_block > 2048 && rows_per_block < (1 << 20)) rows_per_block *= 2;
   uint64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
   void* partial = nullptr;
   int32_t rc = omx_workspace(ctx, blocks * dim * sizeof(float), &partial);
@@ -411,27 +413,13 @@ int32_t launch_rms_bwd(omx_ctx* ctx, const void* x, const float* w, const void* 
   }
 #undef RMS_BWD
   OMX_LAUNCH_CHECK(ctx, "rms_bwd_kernel");
-  hipLaunchKernelGGL(column_sum_kernel, dim3(static_cast<unsigned>((dim + 63) / 64)), dim3(256), 0, ctx->stream,
-                     static_cast<const float*>(partial), gw, static_cast<int>(blocks), static_cast<int>(dim),
-                     ctx->fault, tag);
-  OMX_LAUNCH_CHECK(ctx, "column_sum_kernel");
-  return OMX_OK;
+  return omx_column_sum(ctx, static_cast<const float*>(partial), gw, blocks, dim, tag);
 }
 
-}  // namespace
-
-extern "C" {
-
-int32_t omx_rms_norm_forward(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* w, void* y, int32_t y_dtype,
-                             uint64_t rows, uint64_t dim, float eps) {
-  OMX_REQUIRE_CTX(ctx);
-  const char* op = "rms_norm_forward";
-  if (!x || !w || !y) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
-  if (!omx_valid_float_dtype(x_dtype) || !omx_valid_float_dtype(y_dtype))
-    return omx_fail(ctx, OMX_DTYPE, "%s: dtype must be f32 or bf16", op);
-  if (rows == 0 || dim == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
-  if (!(eps == eps) || eps == INFINITY || eps == -INFINITY) return omx_fail(ctx, OMX_NON_FINITE, "%s", op);
-  unsigned long long tag = omx_tag(ctx, F_RMS_FORWARD);
+int32_t rms_forward_impl(omx_ctx* ctx, const char* op, uint32_t fault_op, const void* x, int32_t x_dtype,
+                         const void* w, void* y, int32_t y_dtype, uint64_t rows, uint64_t dim, float eps) {
+  unsigned long long tag = omx_tag(ctx, fault_op);
+  (void)op;
   const float* wf = static_cast<const float*>(w);
   if (x_dtype == OMX_F32 && y_dtype == OMX_F32) return launch_rms_fwd<float, float>(ctx, x, wf, y, rows, dim, eps, tag);
   if (x_dtype == OMX_F32) return launch_rms_fwd<float, unsigned short>(ctx, x, wf, y, rows, dim, eps, tag);
@@ -439,17 +427,10 @@ int32_t omx_rms_norm_forward(omx_ctx* ctx, const void* x, int32_t x_dtype, const
   return launch_rms_fwd<unsigned short, unsigned short>(ctx, x, wf, y, rows, dim, eps, tag);
 }
 
-int32_t omx_rms_norm_backward(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* w, const void* gy,
-                              int32_t gy_dtype, void* gx, int32_t gx_dtype, void* gw, uint64_t rows, uint64_t dim,
-                              float eps) {
-  OMX_REQUIRE_CTX(ctx);
-  const char* op = "rms_norm_backward";
-  if (!x || !w || !gy || !gx || !gw) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
-  if (!omx_valid_float_dtype(x_dtype) || !omx_valid_float_dtype(gy_dtype) || !omx_valid_float_dtype(gx_dtype))
-    return omx_fail(ctx, OMX_DTYPE, "%s: dtype must be f32 or bf16", op);
-  if (rows == 0 || dim == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
-  if (!(eps == eps) || eps == INFINITY || eps == -INFINITY) return omx_fail(ctx, OMX_NON_FINITE, "%s", op);
-  unsigned long long tag = omx_tag(ctx, F_RMS_BACKWARD);
+int32_t rms_backward_impl(omx_ctx* ctx, uint32_t fault_op, const void* x, int32_t x_dtype, const void* w,
+                          const void* gy, int32_t gy_dtype, void* gx, int32_t gx_dtype, void* gw, uint64_t rows,
+                          uint64_t dim, float eps) {
+  unsigned long long tag = omx_tag(ctx, fault_op);
   const float* wf = static_cast<const float*>(w);
   float* gwf = static_cast<float*>(gw);
   typedef unsigned short h16;
@@ -464,6 +445,80 @@ int32_t omx_rms_norm_backward(omx_ctx* ctx, const void* x, int32_t x_dtype, cons
     case 6: return launch_rms_bwd<h16, h16, float>(ctx, x, wf, gy, gx, gwf, rows, dim, eps, tag);
     default: return launch_rms_bwd<h16, h16, h16>(ctx, x, wf, gy, gx, gwf, rows, dim, eps, tag);
   }
+}
+
+bool finite_host(float v) { return v == v && v != INFINITY && v != -INFINITY; }
+
+}  // namespace
+
+int32_t omx_column_sum(omx_ctx* ctx, const float* partial, float* out, uint64_t blocks, uint64_t dim,
+                       unsigned long long tag) {
+  hipLaunchKernelGGL(column_sum_kernel, dim3(static_cast<unsigned>((dim + 63) / 64)), dim3(256), 0, ctx->stream, partial,
+                     out, static_cast<int>(blocks), static_cast<int>(dim), ctx->fault, tag);
+  OMX_LAUNCH_CHECK(ctx, "column_sum_kernel");
+  return OMX_OK;
+}
+
+extern "C" {
+
+int32_t omx_rms_norm_forward(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* w, void* y, int32_t y_dtype,
+                             uint64_t rows, uint64_t dim, float eps) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "rms_norm_forward";
+  if (!x || !w || !y) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  if (!omx_valid_float_dtype(x_dtype) || !omx_valid_float_dtype(y_dtype))
+    return omx_fail(ctx, OMX_DTYPE, "%s: dtype must be f32 or bf16", op);
+  if (rows == 0 || dim == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
+  if (!(eps == eps) || eps == INFINITY || eps == -INFINITY) return omx_fail(ctx, OMX_NON_FINITE, "%s", op);
+  return rms_forward_impl(ctx, op, F_RMS_FORWARD, x, x_dtype, w, y, y_dtype, rows, dim, eps);
+}
+
+int32_t omx_rms_norm_backward(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* w, const void* gy,
+                              int32_t gy_dtype, void* gx, int32_t gx_dtype, void* gw, uint64_t rows, uint64_t dim,
+                              float eps) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "rms_norm_backward";
+  if (!x || !w || !gy || !gx || !gw) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  if (!omx_valid_float_dtype(x_dtype) || !omx_valid_float_dtype(gy_dtype) || !omx_valid_float_dtype(gx_dtype))
+    return omx_fail(ctx, OMX_DTYPE, "%s: dtype must be f32 or bf16", op);
+  if (rows == 0 || dim == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
+  if (!(eps == eps) || eps == INFINITY || eps == -INFINITY) return omx_fail(ctx, OMX_NON_FINITE, "%s", op);
+  return rms_backward_impl(ctx, F_RMS_BACKWARD, x, x_dtype, w, gy, gy_dtype, gx, gx_dtype, gw, rows, dim, eps);
+}
+
+int32_t omx_rms_qk_norm_forward(omx_ctx* ctx, const void* q, const void* k, int32_t x_dtype, const void* q_weight,
+                                const void* k_weight, void* q_out, void* k_out, int32_t y_dtype, uint64_t q_rows,
+                                uint64_t k_rows, uint64_t dim, float eps) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "rms_qk_norm_forward";
+  if (!q || !k || !q_weight || !k_weight || !q_out || !k_out)
+    return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  if (!omx_valid_float_dtype(x_dtype) || !omx_valid_float_dtype(y_dtype))
+    return omx_fail(ctx, OMX_DTYPE, "%s: dtype must be f32 or bf16", op);
+  if (q_rows == 0 || k_rows == 0 || dim == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
+  if (!finite_host(eps)) return omx_fail(ctx, OMX_NON_FINITE, "%s", op);
+  int32_t rc = rms_forward_impl(ctx, op, F_RMS_QK_FORWARD, q, x_dtype, q_weight, q_out, y_dtype, q_rows, dim, eps);
+  if (rc != OMX_OK) return rc;
+  return rms_forward_impl(ctx, op, F_RMS_QK_FORWARD, k, x_dtype, k_weight, k_out, y_dtype, k_rows, dim, eps);
+}
+
+int32_t omx_rms_qk_norm_backward(omx_ctx* ctx, const void* q, const void* k, int32_t x_dtype, const void* q_weight,
+                                 const void* k_weight, const void* grad_q, const void* grad_k, int32_t gy_dtype,
+                                 void* gq, void* gk, int32_t gx_dtype, void* gq_weight, void* gk_weight,
+                                 uint64_t q_rows, uint64_t k_rows, uint64_t dim, float eps) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "rms_qk_norm_backward";
+  if (!q || !k || !q_weight || !k_weight || !grad_q || !grad_k || !gq || !gk || !gq_weight || !gk_weight)
+    return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  if (!omx_valid_float_dtype(x_dtype) || !omx_valid_float_dtype(gy_dtype) || !omx_valid_float_dtype(gx_dtype))
+    return omx_fail(ctx, OMX_DTYPE, "%s: dtype must be f32 or bf16", op);
+  if (q_rows == 0 || k_rows == 0 || dim == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
+  if (!finite_host(eps)) return omx_fail(ctx, OMX_NON_FINITE, "%s", op);
+  int32_t rc = rms_backward_impl(ctx, F_RMS_QK_BACKWARD, q, x_dtype, q_weight, grad_q, gy_dtype, gq, gx_dtype,
+                                 gq_weight, q_rows, dim, eps);
+  if (rc != OMX_OK) return rc;
+  return rms_backward_impl(ctx, F_RMS_QK_BACKWARD, k, x_dtype, k_weight, grad_k, gy_dtype, gk, gx_dtype, gk_weight,
+                           k_rows, dim, eps);
 }
 
 int32_t omx_embedding_forward(omx_ctx* ctx, const void* table, int32_t table_dtype, const void* ids, void* out,

@@ -23,6 +23,9 @@
 //   embedding fwd/bwd         ojas-cuda goldens embed_*.npy; gather is a bit copy
 //   bf16 rounding             integer rule autocast.rs:70-96, value table in the tests
 //   argmax / topk             brute force in the tests
+//   silu, mul, gate, blend    no digest or fixture in the reference holds these; pinned by
+//                             the known answers of ojas-cpu/tests/ops.rs:599-623,667-696,
+//                             the exp_exact pins under sigmoid, and f64 autograd in the tests
 //   gpt step (graph A)        parity unpinned by the reference (no fixture holds this
 //                             graph); pinned by f64 central differences in the tests
 #include "ojas_exact.h"
@@ -1035,6 +1038,115 @@ void orc_gelu_tanh_backward_vec(const float* x, const float* gy, float* gx, size
     for (size_t i = lo; i < hi; ++i) gx[i] = gelu_tanh_backward(x[i], gy[i]);
   });
 }
+// ---- graph-B pointwise ops ----
+// silu: ojas-cpu/src/pointwise.rs:346-366 (forward), :515-546 (backward).
+void orc_silu_forward_vec(const float* x, float* y, size_t n) {
+  parallel_for(n, 4096, [&](size_t lo, size_t hi) {
+    for (size_t i = lo; i < hi; ++i) y[i] = x[i] * orc_sigmoid_exact(x[i]);
+  });
+}
+void orc_silu_backward_vec(const float* x, const float* gy, float* gx, size_t n) {
+  parallel_for(n, 4096, [&](size_t lo, size_t hi) {
+    for (size_t i = lo; i < hi; ++i) {
+      float v = x[i], s = orc_sigmoid_exact(v);
+      gx[i] = gy[i] * s * (1.0f + v * (1.0f - s));
+    }
+  });
+}
+// mul: ojas-cpu/src/pointwise.rs:579-620 (forward), :770-905 (backward).
+int orc_mul_forward(const float* a, const float* b, float* out, size_t n) {
+  for (size_t i = 0; i < n; ++i) out[i] = a[i] * b[i];
+  return all_finite(out, n) ? ORC_OK : ORC_NON_FINITE;
+}
+int orc_mul_backward(const float* a, const float* b, const float* gy, float* ga, float* gb, size_t n) {
+  for (size_t i = 0; i < n; ++i) {
+    ga[i] = gy[i] * b[i];
+    gb[i] = gy[i] * a[i];
+  }
+  return all_finite(ga, n) && all_finite(gb, n) ? ORC_OK : ORC_NON_FINITE;
+}
+
+// Per-head sigmoid gate. gates[r, h] = sigmoid(b[h] + sum_i x[r, i] * w[h, i]),
+// the bias being the first term of the ascending chain
+// (ojas-cpu/src/pointwise.rs:1853-1894); y = attn * gate broadcast over
+// head_dim (:1395-1470).
+int orc_gate_values(const float* x, const float* w, const float* bias, float* gates, size_t rows,
+                    size_t din, size_t heads) {
+  bool ok = true;
+  for (size_t r = 0; r < rows; ++r)
+    for (size_t h = 0; h < heads; ++h) {
+      float z = 0.0f + 1.0f * bias[h];
+      for (size_t i = 0; i < din; ++i) z = z + x[r * din + i] * w[h * din + i];
+      if (!finite32(z)) ok = false;
+      gates[r * heads + h] = orc_sigmoid_exact(z);
+    }
+  return ok ? ORC_OK : ORC_NON_FINITE;
+}
+int orc_gate_forward(const float* x, const float* w, const float* bias, const float* attn, float* y,
+                     size_t rows, size_t din, size_t heads, size_t head_dim) {
+  std::vector<float> gates(rows * heads);
+  int rc = orc_gate_values(x, w, bias, gates.data(), rows, din, heads);
+  if (rc != ORC_OK) return rc;
+  for (size_t r = 0; r < rows; ++r)
+    for (size_t h = 0; h < heads; ++h)
+      for (size_t d = 0; d < head_dim; ++d) {
+        size_t i = (r * heads + h) * head_dim + d;
+        y[i] = attn[i] * gates[r * heads + h];
+      }
+  return all_finite(y, rows * heads * head_dim) ? ORC_OK : ORC_NON_FINITE;
+}
+// ojas-cpu/src/pointwise.rs:1678-1781: grad_attn = gy * g; gz = (gy . attn) g (1 - g)
+// with the dot ascending over head_dim; grad_b adds gz rows in row order;
+// grad_x = gz . W (head ascending); grad_w = gz^T . x (row ascending).
+int orc_gate_backward(const float* x, const float* w, const float* bias, const float* attn,
+                      const float* gy, float* gx, float* gw, float* gb, float* gattn, size_t rows,
+                      size_t din, size_t heads, size_t head_dim) {
+  std::vector<float> gates(rows * heads), gz(rows * heads);
+  int rc = orc_gate_values(x, w, bias, gates.data(), rows, din, heads);
+  if (rc != ORC_OK) return rc;
+  for (size_t r = 0; r < rows; ++r)
+    for (size_t h = 0; h < heads; ++h) {
+      float g = gates[r * heads + h], dot = 0.0f;
+      for (size_t d = 0; d < head_dim; ++d) {
+        size_t i = (r * heads + h) * head_dim + d;
+        gattn[i] = gy[i] * g;
+        dot = dot + gy[i] * attn[i];
+      }
+      gz[r * heads + h] = dot * g * (1.0f - g);
+    }
+  for (size_t h = 0; h < heads; ++h) gb[h] = 0.0f;
+  for (size_t r = 0; r < rows; ++r)
+    for (size_t h = 0; h < heads; ++h) gb[h] += gz[r * heads + h];
+  gemm(gz.data(), heads, 1, w, din, 1, gx, rows, heads, din, false);
+  gemm(gz.data(), 1, heads, x, din, 1, gw, heads, rows, din, false);
+  bool ok = all_finite(gx, rows * din) && all_finite(gw, heads * din) && all_finite(gb, heads) &&
+            all_finite(gattn, rows * heads * head_dim);
+  return ok ? ORC_OK : ORC_NON_FINITE;
+}
+
+// Value-residual blend, ojas-cpu/src/pointwise.rs:2031-2148:
+// out = (1 - s) v + s v0 with s = sigmoid(lambda); grad_lambda is the f32
+// ascending sum of (v0 - v) g times s (1 - s).
+int orc_value_residual_forward(const float* v, const float* v0, float lambda, float* out, size_t n) {
+  float s = orc_sigmoid_exact(lambda);
+  if (!finite32(s)) return ORC_NON_FINITE;
+  for (size_t i = 0; i < n; ++i) out[i] = (1.0f - s) * v[i] + s * v0[i];
+  return all_finite(out, n) ? ORC_OK : ORC_NON_FINITE;
+}
+int orc_value_residual_backward(const float* v, const float* v0, const float* gy, float lambda,
+                                float* gv, float* gv0, float* glambda, size_t n) {
+  float s = orc_sigmoid_exact(lambda);
+  if (!finite32(s)) return ORC_NON_FINITE;
+  float grad_s = 0.0f;
+  for (size_t i = 0; i < n; ++i) {
+    gv[i] = (1.0f - s) * gy[i];
+    gv0[i] = s * gy[i];
+    grad_s += (v0[i] - v[i]) * gy[i];
+  }
+  *glambda = grad_s * s * (1.0f - s);
+  return all_finite(gv, n) && all_finite(gv0, n) && finite32(*glambda) ? ORC_OK : ORC_NON_FINITE;
+}
+
 void orc_permute_0213(const float* x, float* y, size_t d0, size_t d1, size_t d2, size_t d3) {
   for (size_t a = 0; a < d0; ++a)
     for (size_t b = 0; b < d1; ++b)

@@ -140,6 +140,23 @@ void orc_gelu_erf_forward_vec(const float* x, float* y, size_t n);
 void orc_gelu_erf_backward_vec(const float* x, const float* gy, float* gx, size_t n);
 void orc_gelu_tanh_forward_vec(const float* x, float* y, size_t n);
 void orc_gelu_tanh_backward_vec(const float* x, const float* gy, float* gx, size_t n);
+/* ---- graph-B pointwise ops (ojas-cpu/src/pointwise.rs:346-366,515-546,
+ *      579-620,770-905,1395-1470,1678-1781,1853-1894,2031-2148) ---- */
+void orc_silu_forward_vec(const float* x, float* y, size_t n);
+void orc_silu_backward_vec(const float* x, const float* gy, float* gx, size_t n);
+int orc_mul_forward(const float* a, const float* b, float* out, size_t n);
+int orc_mul_backward(const float* a, const float* b, const float* gy, float* ga, float* gb, size_t n);
+/* x [rows, din], w [heads, din], bias [heads], attn / y [rows, heads, head_dim]. */
+int orc_gate_values(const float* x, const float* w, const float* bias, float* gates, size_t rows,
+                    size_t din, size_t heads);
+int orc_gate_forward(const float* x, const float* w, const float* bias, const float* attn, float* y,
+                     size_t rows, size_t din, size_t heads, size_t head_dim);
+int orc_gate_backward(const float* x, const float* w, const float* bias, const float* attn,
+                      const float* gy, float* gx, float* gw, float* gb, float* gattn, size_t rows,
+                      size_t din, size_t heads, size_t head_dim);
+int orc_value_residual_forward(const float* v, const float* v0, float lambda, float* out, size_t n);
+int orc_value_residual_backward(const float* v, const float* v0, const float* gy, float lambda,
+                                float* gv, float* gv0, float* glambda, size_t n);
 /* [d0,d1,d2,d3] -> [d0,d2,d1,d3], bit-preserving (layout.rs:82-118). */
 void orc_permute_0213(const float* x, float* y, size_t d0, size_t d1, size_t d2, size_t d3);
 /* Ties go to the lowest column; NaN or +inf is ORC_NON_FINITE

@@ -454,6 +454,94 @@ def gelu_tanh_backward_vec(x, gy):
     return _vec2(_lib.orc_gelu_tanh_backward_vec, x, gy)
 
 
+def silu_forward(x):
+    return _vec1(_lib.orc_silu_forward_vec, x)
+
+
+def silu_backward(x, gy):
+    return _vec2(_lib.orc_silu_backward_vec, x, gy)
+
+
+def mul_forward(a, b):
+    a, b = _f32(a), _f32(b)
+    out = np.empty_like(a)
+    _check(_lib.orc_mul_forward(_fp(a), _fp(b), _fp(out), _sz(a.size)), "mul_forward")
+    return out
+
+
+def mul_backward(a, b, gy):
+    a, b, gy = _f32(a), _f32(b), _f32(gy)
+    ga, gb = np.empty_like(a), np.empty_like(a)
+    _check(_lib.orc_mul_backward(_fp(a), _fp(b), _fp(gy), _fp(ga), _fp(gb), _sz(a.size)), "mul_backward")
+    return ga, gb
+
+
+def _gate_dims(x, w, attn):
+    din = x.shape[-1]
+    heads, head_dim = attn.shape[-2], attn.shape[-1]
+    assert w.shape == (heads, din) and attn.shape[:-2] == x.shape[:-1]
+    return x.size // din, din, heads, head_dim
+
+
+def gate_values(x, w, bias):
+    x, w, bias = _f32(x), _f32(w), _f32(bias)
+    rows, din, heads = x.size // x.shape[-1], x.shape[-1], w.shape[0]
+    gates = np.empty((rows, heads), np.float32)
+    _check(
+        _lib.orc_gate_values(_fp(x), _fp(w), _fp(bias), _fp(gates), _sz(rows), _sz(din), _sz(heads)),
+        "per_head_sigmoid_gate_forward",
+    )
+    return gates
+
+
+def gate_forward(x, w, bias, attn):
+    x, w, bias, attn = _f32(x), _f32(w), _f32(bias), _f32(attn)
+    rows, din, heads, dh = _gate_dims(x, w, attn)
+    y = np.empty_like(attn)
+    _check(
+        _lib.orc_gate_forward(_fp(x), _fp(w), _fp(bias), _fp(attn), _fp(y), _sz(rows), _sz(din), _sz(heads), _sz(dh)),
+        "per_head_sigmoid_gate_forward",
+    )
+    return y
+
+
+def gate_backward(x, w, bias, attn, gy):
+    x, w, bias, attn, gy = _f32(x), _f32(w), _f32(bias), _f32(attn), _f32(gy)
+    rows, din, heads, dh = _gate_dims(x, w, attn)
+    gx, gw, gb, ga = np.empty_like(x), np.empty_like(w), np.empty_like(bias), np.empty_like(attn)
+    _check(
+        _lib.orc_gate_backward(
+            _fp(x), _fp(w), _fp(bias), _fp(attn), _fp(gy), _fp(gx), _fp(gw), _fp(gb), _fp(ga),
+            _sz(rows), _sz(din), _sz(heads), _sz(dh),
+        ),
+        "per_head_sigmoid_gate_backward",
+    )
+    return gx, gw, gb, ga
+
+
+def value_residual_forward(v, v0, lam):
+    v, v0 = _f32(v), _f32(v0)
+    out = np.empty_like(v)
+    _check(
+        _lib.orc_value_residual_forward(_fp(v), _fp(v0), C.c_float(lam), _fp(out), _sz(v.size)),
+        "value_residual_blend_forward",
+    )
+    return out
+
+
+def value_residual_backward(v, v0, lam, gy):
+    v, v0, gy = _f32(v), _f32(v0), _f32(gy)
+    gv, gv0 = np.empty_like(v), np.empty_like(v)
+    gl = C.c_float()
+    _check(
+        _lib.orc_value_residual_backward(
+            _fp(v), _fp(v0), _fp(gy), C.c_float(lam), _fp(gv), _fp(gv0), C.byref(gl), _sz(v.size)
+        ),
+        "value_residual_blend_backward",
+    )
+    return gv, gv0, np.float32(gl.value)
+
+
 def permute_0213(x):
     x = _f32(x)
     d0, d1, d2, d3 = x.shape

@@ -1,0 +1,247 @@
+"""GPU-vs-oracle parity for the ops only the nanolab block uses (SiLU, product,
+half-split RoPE, q/k RMSNorm, per-head sigmoid gate, value-residual blend),
+through the C ABI.
+
+Template: ojas-wgpu/tests/parity.rs (every op on shapes that break tiles,
+against CPU Exact) and ojas-wgpu/tests/gate_saved.rs (the saved-scale
+backward equals the recomputing one). Tolerances as in the other parity file:
+f32 tier 1e-5 relative to max(1, max|cpu|); bf16 tier 2e-2 with operands
+rounded to bf16 on both sides.
+"""
+import numpy as np
+import pytest
+
+import oracle_api as orc
+
+pytestmark = pytest.mark.gpu
+
+F32_TOL = 1e-5
+BF16_TOL = 2e-2
+
+
+@pytest.fixture(scope="module")
+def be():
+    from ojas_amd.backend import MiBackend
+
+    backend = MiBackend(0)
+    assert backend.device_name().startswith("gfx950")
+    yield backend
+    backend.close()
+
+
+def close(got, want, tol, what=""):
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    assert got.shape == want.shape, (what, got.shape, want.shape)
+    scale = max(1.0, float(np.max(np.abs(want))) if want.size else 1.0)
+    err = float(np.max(np.abs(got - want))) if want.size else 0.0
+    assert np.isfinite(got).all(), f"{what}: non-finite output"
+    assert err <= tol * scale, f"{what}: max err {err:.3e} > {tol:.0e} * {scale:.3e}"
+
+
+def tier(be, bf16):
+    """(upload, tolerance, rounding applied to the oracle's inputs) of a precision tier."""
+    from ojas_amd.backend import BF16
+
+    if bf16:
+        return (lambda a: be.upload(np.asarray(a, np.float32), BF16)), BF16_TOL, orc.round_bf16
+    return (lambda a: be.upload(np.asarray(a, np.float32))), F32_TOL, (lambda a: np.asarray(a, np.float32))
+
+
+SIZES = [1, 3, 255, 1024, 4099, (1 << 16) + 4, 3 * 2048 * 5]
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("n", SIZES)
+def test_silu_and_mul(be, n, bf16):
+    print(f"silu/mul n={n} bf16={bf16}", flush=True)
+    up, tol, rnd = tier(be, bf16)
+    r = orc.SplitMix64(7000 + n)
+    x, b, gy = rnd(r.vec(n, 6.0)), rnd(r.vec(n, 2.0)), rnd(r.vec(n, 1.0))
+    dx, db, dgy = up(x), up(b), up(gy)
+    close(be.download_f32(be.silu_forward(dx)), orc.silu_forward(x), tol, "silu fwd")
+    close(be.download_f32(be.silu_backward(dx, dgy)), orc.silu_backward(x, gy), tol, "silu bwd")
+    close(be.download_f32(be.mul_forward(dx, db)), orc.mul_forward(x, b), tol, "mul fwd")
+    ga, gb = be.mul_backward(dx, db, dgy)
+    wa, wb = orc.mul_backward(x, b, gy)
+    close(be.download_f32(ga), wa, tol, "mul ga")
+    close(be.download_f32(gb), wb, tol, "mul gb")
+    if not bf16:
+        # One rounding per product: the f32 product is bit-exact.
+        assert np.array_equal(be.download(be.mul_forward(dx, db)), orc.mul_forward(x, b))
+
+
+def test_silu_extremes_stay_finite(be):
+    x = np.array([-200.0, -90.0, -20.0, -0.0, 0.0, 20.0, 90.0, 200.0], np.float32)
+    y = be.download(be.silu_forward(be.upload(x)))
+    close(y, orc.silu_forward(x), F32_TOL, "silu extremes")
+    g = be.download(be.silu_backward(be.upload(x), be.upload(np.ones_like(x))))
+    close(g, orc.silu_backward(x, np.ones_like(x)), F32_TOL, "silu grad extremes")
+
+
+ROPE_SHAPES = [(2, 64, 4, 32), (1, 1, 1, 2), (1, 17, 3, 6), (2, 5, 2, 64), (1, 257, 12, 64), (3, 7, 5, 10)]
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("b,t,h,d", ROPE_SHAPES)
+def test_rope_half_split(be, b, t, h, d, bf16):
+    print(f"rope {b}x{t}x{h}x{d} bf16={bf16}", flush=True)
+    up, tol, rnd = tier(be, bf16)
+    r = orc.SplitMix64(500 + t * 3 + d)
+    x = rnd(r.vec(b * t * h * d, 1.0)).reshape(b, t, h, d)
+    cos, sin = r.vec(t * d, 1.0).reshape(t, d), r.vec(t * d, 1.0).reshape(t, d)
+    dx, dc, ds = up(x), be.upload(cos), be.upload(sin)
+    close(be.download_f32(be.rope_half_split_forward(dx, dc, ds)), orc.rope_forward(x, cos, sin), tol, "rope fwd")
+    close(be.download_f32(be.rope_half_split_backward(dx, dc, ds)), orc.rope_backward(x, cos, sin), tol, "rope bwd")
+    # Tables shaped like x (the `Same` layout).
+    cos_full = np.ascontiguousarray(np.broadcast_to(cos[None, :, None, :], x.shape))
+    sin_full = np.ascontiguousarray(np.broadcast_to(sin[None, :, None, :], x.shape))
+    got = be.download_f32(be.rope_half_split_forward(dx, be.upload(cos_full), be.upload(sin_full)))
+    close(got, orc.rope_forward(x, cos, sin), tol, "rope fwd same-layout")
+
+
+def test_rope_golden_inputs_match_the_reference_digest_case(be):
+    # The inputs of ojas-cpu/tests/exact_golden.rs:141-150; with one rounding per product and sum
+    # the device result may differ from the digest's bits only through contraction, which is off.
+    b, t, h, d = 2, 64, 4, 32
+    r = orc.SplitMix64(500)
+    x = r.vec(b * t * h * d, 1.0).reshape(b, t, h, d)
+    cos, sin = r.vec(t * d, 1.0).reshape(t, d), r.vec(t * d, 1.0).reshape(t, d)
+    got = be.download(be.rope_half_split_forward(be.upload(x), be.upload(cos), be.upload(sin)))
+    assert np.array_equal(got, orc.rope_forward(x, cos, sin))
+    got = be.download(be.rope_half_split_backward(be.upload(x), be.upload(cos), be.upload(sin)))
+    assert np.array_equal(got, orc.rope_backward(x, cos, sin))
+
+
+def test_rope_shape_errors(be):
+    from ojas_amd.backend import OjasError
+
+    x = be.upload(np.zeros((1, 4, 2, 6), np.float32))
+    with pytest.raises(OjasError) as e:
+        be.rope_half_split_forward(x, be.upload(np.zeros((3, 6), np.float32)), be.upload(np.zeros((3, 6), np.float32)))
+    assert e.value.variant == "Shape"
+    odd = be.upload(np.zeros((1, 4, 2, 5), np.float32))
+    with pytest.raises(OjasError) as e:
+        be.rope_half_split_forward(odd, be.upload(np.zeros((4, 5), np.float32)), be.upload(np.zeros((4, 5), np.float32)))
+    assert e.value.variant == "Shape"
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("b,t,h,kvh,d", [(2, 17, 4, 2, 64), (1, 5, 3, 3, 24), (1, 300, 12, 12, 64), (1, 9, 2, 1, 128)])
+def test_rms_qk_norm(be, b, t, h, kvh, d, bf16):
+    print(f"rms_qk_norm {b}x{t}x{h}/{kvh}x{d} bf16={bf16}", flush=True)
+    up, tol, rnd = tier(be, bf16)
+    r = orc.SplitMix64(900 + t + d)
+    q = rnd(r.vec(b * t * h * d, 1.0)).reshape(b, t, h, d)
+    k = rnd(r.vec(b * t * kvh * d, 1.0)).reshape(b, t, kvh, d)
+    qw, kw = 1.0 + r.vec(d, 0.1), 1.0 + r.vec(d, 0.1)
+    gq, gk = rnd(r.vec(q.size, 1.0)).reshape(q.shape), rnd(r.vec(k.size, 1.0)).reshape(k.shape)
+    dq, dk, dqw, dkw = up(q), up(k), be.upload(qw), be.upload(kw)
+    qn, kn = be.rms_qk_norm_forward(dq, dk, dqw, dkw, 1e-6)
+    close(be.download_f32(qn), orc.rms_norm_forward(q.reshape(-1, d), qw, 1e-6).reshape(q.shape), tol, "qn")
+    close(be.download_f32(kn), orc.rms_norm_forward(k.reshape(-1, d), kw, 1e-6).reshape(k.shape), tol, "kn")
+    got = be.rms_qk_norm_backward(dq, dk, dqw, dkw, up(gq), up(gk), 1e-6)
+    wq = orc.rms_norm_backward(q.reshape(-1, d), qw, gq.reshape(-1, d), 1e-6)
+    wk = orc.rms_norm_backward(k.reshape(-1, d), kw, gk.reshape(-1, d), 1e-6)
+    close(be.download_f32(got[0]), wq[0].reshape(q.shape), tol, "gq")
+    close(be.download_f32(got[1]), wk[0].reshape(k.shape), tol, "gk")
+    # Weight gradients add rows in another order than the CPU's ascending sum.
+    wtol = max(tol, 2e-5)
+    close(be.download_f32(got[2]), wq[1], wtol, "gq_weight")
+    close(be.download_f32(got[3]), wk[1], wtol, "gk_weight")
+
+
+GATE_SHAPES = [(1, 2, 2, 1), (37, 24, 3, 8), (257, 128, 12, 64), (64, 768, 12, 64), (19, 40, 5, 5), (130, 96, 6, 32)]
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("rows,din,heads,dh", GATE_SHAPES)
+def test_per_head_sigmoid_gate(be, rows, din, heads, dh, bf16):
+    print(f"gate rows={rows} din={din} heads={heads} dh={dh} bf16={bf16}", flush=True)
+    up, tol, rnd = tier(be, bf16)
+    r = orc.SplitMix64(1400 + rows + din)
+    x = rnd(r.vec(rows * din, 1.0)).reshape(rows, din)
+    w = rnd(r.vec(heads * din, 2.0 / np.sqrt(din))).reshape(heads, din)
+    bias = r.vec(heads, 0.5)
+    attn = rnd(r.vec(rows * heads * dh, 1.0)).reshape(rows, heads, dh)
+    gy = rnd(r.vec(rows * heads * dh, 1.0)).reshape(rows, heads, dh)
+    dx, dw, db, da, dgy = up(x), up(w), be.upload(bias), up(attn), up(gy)
+    y, scales = be.per_head_sigmoid_gate_forward_saving(dx, dw, db, da)
+    want = orc.gate_forward(x, w, bias, attn)
+    close(be.download_f32(y), want, tol, "gate fwd")
+    close(be.download(scales), orc.gate_values(x, w, bias), tol, "gate scales")
+    y2 = be.per_head_sigmoid_gate_forward(dx, dw, db, da)
+    assert np.array_equal(be.download(y2), be.download(y)), "saving forward differs from the plain one"
+    wgx, wgw, wgb, wga = orc.gate_backward(x, w, bias, attn, gy)
+    first = None
+    for saved in (None, scales):
+        gx, gw, gb, ga = be.per_head_sigmoid_gate_backward_saved(dx, dw, db, da, dgy, saved)
+        close(be.download_f32(ga), wga, tol, "gate g_attn")
+        # Sums over rows (grad_w, grad_b) and the tiny-K product (grad_x) re-associate.
+        sum_tol = tol if bf16 else 3e-5
+        close(be.download_f32(gx), wgx, sum_tol, "gate g_input")
+        close(be.download_f32(gw), wgw, sum_tol, "gate g_weight")
+        close(be.download_f32(gb), wgb, sum_tol, "gate g_bias")
+        now = [be.download(t) for t in (gx, gw, gb, ga)]
+        if first is None:
+            first = now
+        else:
+            for a, b_ in zip(first, now):
+                assert np.array_equal(a, b_), "saved-scale backward differs from the recomputing one"
+
+
+def test_gate_known_answer_and_nonfinite(be):
+    from ojas_amd.backend import OjasError
+
+    # ojas-cpu/tests/ops.rs:599-614
+    x = be.upload(np.array([[1.0, 2.0]], np.float32))
+    w = be.upload(np.eye(2, dtype=np.float32))
+    b = be.upload(np.zeros(2, np.float32))
+    attn = be.upload(np.ones((1, 2, 1), np.float32))
+    y = be.download(be.per_head_sigmoid_gate_forward(x, w, b, attn)).reshape(-1)
+    assert abs(y[0] - 1.0 / (1.0 + np.exp(-1.0))) < 1e-6 and abs(y[1] - 1.0 / (1.0 + np.exp(-2.0))) < 1e-6
+    bad = be.upload(np.array([[np.nan, 2.0]], np.float32))
+    with pytest.raises(OjasError) as e:
+        be.download(be.per_head_sigmoid_gate_forward(bad, w, b, attn))
+    assert e.value.variant == "NonFinite" and "per_head_sigmoid_gate_forward" in e.value.detail
+    with pytest.raises(OjasError) as e:
+        be.per_head_sigmoid_gate_forward(x, w, be.upload(np.zeros(3, np.float32)), attn)
+    assert e.value.variant == "Shape"
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("n", SIZES)
+def test_value_residual_blend(be, n, bf16):
+    print(f"value_residual n={n} bf16={bf16}", flush=True)
+    up, tol, rnd = tier(be, bf16)
+    r = orc.SplitMix64(2000 + n)
+    v, v0, gy = rnd(r.vec(n, 1.0)), rnd(r.vec(n, 1.0)), rnd(r.vec(n, 1.0))
+    for lam in (0.0, 0.7, -3.0):
+        dl = be.upload(np.array([lam], np.float32))
+        dv, dv0, dgy = up(v), up(v0), up(gy)
+        close(be.download_f32(be.value_residual_blend_forward(dv, dv0, dl)), orc.value_residual_forward(v, v0, lam),
+              tol, "blend fwd")
+        gv, gv0, gl = be.value_residual_blend_backward(dv, dv0, dl, dgy)
+        wv, wv0, wl = orc.value_residual_backward(v, v0, lam, gy)
+        close(be.download_f32(gv), wv, tol, "blend gv")
+        close(be.download_f32(gv0), wv0, tol, "blend gv0")
+        # grad_lambda is a sum of n products; the device adds them as a tree, the CPU as one
+        # chain, so the bound is on the chain's own rounding error (n * eps * sum|terms|).
+        terms = (v0.astype(np.float64) - v) * gy
+        exact = terms.sum() * (1 / (1 + np.exp(-lam))) * (1 - 1 / (1 + np.exp(-lam)))
+        bound = 1e-5 * max(1.0, abs(exact)) + 6e-8 * np.sqrt(n) * np.abs(terms).sum()
+        assert abs(float(be.download(gl)[0]) - exact) <= bound, (lam, float(be.download(gl)[0]), exact, bound)
+        assert abs(float(wl) - exact) <= 1e-5 * max(1.0, abs(exact)) + 6e-8 * n * np.abs(terms).sum()
+
+
+def test_value_residual_known_answer_and_nonfinite_lambda(be):
+    from ojas_amd.backend import OjasError
+
+    # ojas-cpu/tests/ops.rs:616-622
+    out = be.download(be.value_residual_blend_forward(be.upload(np.array([2.0, 2.0], np.float32)),
+                                                      be.upload(np.array([4.0, 6.0], np.float32)),
+                                                      be.upload(np.array([0.0], np.float32))))
+    assert list(out) == [3.0, 4.0]
+    with pytest.raises(OjasError) as e:
+        be.download(be.value_residual_blend_forward(be.upload(np.ones(4, np.float32)), be.upload(np.ones(4, np.float32)),
+                                                    be.upload(np.array([np.nan], np.float32))))
+    assert e.value.variant == "NonFinite"

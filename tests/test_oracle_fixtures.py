@@ -384,3 +384,79 @@ def test_argmax_and_topk_against_brute_force():
         orc.topk_rows(bad, 3)
     with pytest.raises(orc.OracleError):
         orc.argmax_rows(np.where(x == x[0, 0], -np.inf, x).astype(np.float32))
+
+
+# ---- graph-B pointwise ops: the known answers of ojas-cpu/tests/ops.rs:599-623,667-696, and f64
+# autograd for what those leave open (a wrong sign, a swapped operand or a dropped term fails) ----
+def test_silu_and_mul_known_answers_and_derivatives():
+    import torch
+
+    y = orc.silu_forward(np.array([0.0, 1.0, -1.0], np.float32))
+    s1 = 1.0 / (1.0 + math.exp(-1.0))
+    assert abs(y[0]) < 1e-6 and abs(y[1] - s1) < 1e-6 and abs(y[2] + (1.0 - s1)) < 1e-6
+    a, b = np.array([2.0, -3.0], np.float32), np.array([4.0, 0.5], np.float32)
+    assert list(orc.mul_forward(a, b)) == [8.0, -1.5]
+    ga, gb = orc.mul_backward(a, b, np.ones(2, np.float32))
+    assert list(ga) == list(b) and list(gb) == list(a)
+    r = orc.SplitMix64(41)
+    x, gy = r.vec(4000, 6.0), r.vec(4000, 1.0)
+    xt = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+    yt = torch.nn.functional.silu(xt)
+    yt.backward(torch.tensor(gy, dtype=torch.float64))
+    np.testing.assert_allclose(orc.silu_forward(x), yt.detach().numpy(), rtol=3e-7, atol=1e-7)
+    np.testing.assert_allclose(orc.silu_backward(x, gy), xt.grad.numpy(), rtol=1e-6, atol=2e-7)
+    ga, gb = orc.mul_backward(x, gy, x)
+    assert np.array_equal(ga, x * gy) and np.array_equal(gb, x * x)
+
+
+def test_per_head_gate_known_answers_and_autograd():
+    import torch
+
+    y = orc.gate_forward(np.array([[1.0, 2.0]], np.float32), np.eye(2, dtype=np.float32), np.zeros(2, np.float32),
+                         np.ones((1, 2, 1), np.float32))
+    assert abs(y[0, 0, 0] - 1.0 / (1.0 + math.exp(-1.0))) < 1e-6
+    assert abs(y[0, 1, 0] - 1.0 / (1.0 + math.exp(-2.0))) < 1e-6
+    r = orc.SplitMix64(43)
+    rows, din, heads, dh = 37, 24, 3, 8
+    x = r.vec(rows * din, 1.0).reshape(rows, din)
+    w = r.vec(heads * din, 0.5).reshape(heads, din)
+    bias = r.vec(heads, 0.5)
+    attn = r.vec(rows * heads * dh, 1.0).reshape(rows, heads, dh)
+    gy = r.vec(rows * heads * dh, 1.0).reshape(rows, heads, dh)
+    t = lambda a: torch.tensor(a, dtype=torch.float64, requires_grad=True)
+    xt, wt, bt, at = t(x), t(w), t(bias), t(attn)
+    yt = at * torch.sigmoid(xt @ wt.T + bt)[:, :, None]
+    yt.backward(torch.tensor(gy, dtype=torch.float64))
+    np.testing.assert_allclose(orc.gate_forward(x, w, bias, attn), yt.detach().numpy(), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(orc.gate_values(x, w, bias), torch.sigmoid(xt @ wt.T + bt).detach().numpy(), rtol=1e-5)
+    gx, gw, gb, ga = orc.gate_backward(x, w, bias, attn, gy)
+    for got, want in ((gx, xt.grad), (gw, wt.grad), (gb, bt.grad), (ga, at.grad)):
+        want = want.numpy()
+        assert np.abs(got - want).max() <= 2e-5 * max(1.0, np.abs(want).max())
+    # The bias is the first term of each logit's chain: with a zero input the gate is sigmoid(b).
+    zero = orc.gate_values(np.zeros((2, din), np.float32), w, bias)
+    assert np.array_equal(zero[0], np.array([orc.sigmoid_exact(float(v)) for v in bias], np.float32))
+    with pytest.raises(orc.OracleError):
+        orc.gate_forward(np.full((1, din), np.nan, np.float32), w, bias, attn[:1])
+
+
+def test_value_residual_blend_known_answers_and_autograd():
+    import torch
+
+    out = orc.value_residual_forward(np.array([2.0, 2.0], np.float32), np.array([4.0, 6.0], np.float32), 0.0)
+    assert list(out) == [3.0, 4.0]
+    r = orc.SplitMix64(47)
+    n, lam = 5000, 0.7
+    v, v0, gy = r.vec(n, 1.0), r.vec(n, 1.0), r.vec(n, 1.0)
+    t = lambda a: torch.tensor(a, dtype=torch.float64, requires_grad=True)
+    vt, v0t, lt = t(v), t(v0), t(np.float64(np.float32(lam)))
+    s = torch.sigmoid(lt)
+    outt = (1 - s) * vt + s * v0t
+    outt.backward(torch.tensor(gy, dtype=torch.float64))
+    np.testing.assert_allclose(orc.value_residual_forward(v, v0, lam), outt.detach().numpy(), rtol=1e-6, atol=1e-7)
+    gv, gv0, gl = orc.value_residual_backward(v, v0, lam, gy)
+    np.testing.assert_allclose(gv, vt.grad.numpy(), rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(gv0, v0t.grad.numpy(), rtol=1e-6, atol=1e-7)
+    assert abs(gl - lt.grad.item()) < 1e-4 * max(1.0, abs(lt.grad.item()))
+    with pytest.raises(orc.OracleError):
+        orc.value_residual_forward(v, v0, float("nan"))
