@@ -10,7 +10,9 @@
 // tolerance is given):
 //   linear fwd/bwd, gemm      ojas-cpu/tests/exact_golden.rs:206-242 (36 digests)
 //   muon f32                  exact_golden.rs:243-250 (8 digests)
-//   muon bf16                 ojas-oracle/fixtures/tiny/muon_step_bf16.safetensors (tolerance)
+//   muon bf16                 ojas-oracle/fixtures/tiny/muon_step_bf16.safetensors (4 cases, bit for bit)
+//   nanolab graph             ojas-oracle/fixtures/tiny/{init,forward,grads_init}.safetensors at the
+//                             gates of ojas-oracle/src/parity.rs:28-40 (nanolab_exact.cpp)
 //   sdpa fwd/lse/bwd          exact_golden.rs:251-265 (15 digests); window and
 //                             GQA: brute-force softmax in the tests
 //   rms fwd/bwd, rope         exact_golden.rs:266-270; rms_norm_f64.json

@@ -177,6 +177,21 @@ size_t orc_gpt_param_len(const orc_gpt_config* c, size_t index);
 int orc_gpt_loss_and_grads(const orc_gpt_config* c, float* const* params, const uint32_t* ids,
                            const uint32_t* targets, float* loss, float* const* grads);
 
+/* ---- nanolab GPT (the reference's model graph, ojas-model/src/block.rs:218-420) ----
+ * Parameter order as ojas-model/src/names.rs:188-300. window = 0: full causal. */
+typedef struct {
+  uint32_t layers, n_embd, n_head, n_kv_head, head_dim, hidden, vocab, batch, seq, window;
+  float rms_eps;
+  double rope_base;
+} orc_nanolab_config;
+size_t orc_nanolab_param_count(const orc_nanolab_config* c);
+size_t orc_nanolab_param_len(const orc_nanolab_config* c, size_t index);
+/* cos / sin [seq, head_dim] (ojas-model/src/block.rs:31-71). */
+void orc_rope_tables(size_t seq, size_t head_dim, double base, float* cos, float* sin);
+/* logits ([batch*seq, vocab]) and grads may be NULL. */
+int orc_nanolab_loss_and_grads(const orc_nanolab_config* c, float* const* params, const uint32_t* ids,
+                               const uint32_t* targets, float* loss, float* logits, float* const* grads);
+
 #ifdef __cplusplus
 }
 #endif

@@ -10,6 +10,8 @@ Run in the build container (needs /root/reference). Only DATA is taken:
   * 100-step torch AdamW parameters/moments  ojas-model/tests/fixtures/adamw_100/adamw_100.safetensors
   * erf / GELU known-answer tables           ojas-core/src/erf_exact.rs:86-140 (numbers -> JSON)
   * AdamW lerp-branch rows                   ojas-cpu/tests/adamw_lerp_oracle.rs (numbers -> JSON)
+  * torch 2.13 vectors of the tiny nanolab   ojas-oracle/fixtures/tiny/{init,forward,grads_init}.safetensors and
+    model and of stock nanolab's Muon step   muon_step_bf16.safetensors (copied as is)
 No reference source text is kept: numeric literals are parsed into JSON.
 """
 import json
@@ -64,6 +66,9 @@ def copies():
     (OUT / "adamw_100").mkdir(exist_ok=True)
     for f in ("adamw_100.safetensors", "manifest.json"):
         shutil.copyfile(REF / "ojas-model/tests/fixtures/adamw_100" / f, OUT / "adamw_100" / f)
+    (OUT / "tiny").mkdir(exist_ok=True)
+    for f in ("init", "forward", "grads_init", "muon_step_bf16"):
+        shutil.copyfile(REF / "ojas-oracle/fixtures/tiny" / f"{f}.safetensors", OUT / "tiny" / f"{f}.safetensors")
 
 
 if __name__ == "__main__":

@@ -593,3 +593,52 @@ def gpt_loss_and_grads(cfg: GptConfig, params, ids, targets):
     _check(_lib.orc_gpt_loss_and_grads(C.byref(cfg), pp, _up(ids), _up(targets), C.byref(loss), gp),
            "gpt_loss_and_grads")
     return np.float32(loss.value), grads
+
+
+class NanolabConfig(C.Structure):
+    _fields_ = [(n, C.c_uint32) for n in ("layers", "n_embd", "n_head", "n_kv_head", "head_dim", "hidden", "vocab",
+                                          "batch", "seq", "window")] + [("rms_eps", C.c_float),
+                                                                        ("rope_base", C.c_double)]
+
+
+_lib.orc_nanolab_param_count.restype = _sz
+_lib.orc_nanolab_param_len.restype = _sz
+
+# Parameter names in the order of ojas-model/src/names.rs:188-300.
+NANOLAB_BLOCK_PARAMS = ("norm1.weight", "mixer.q_proj.weight", "mixer.k_proj.weight", "mixer.v_proj.weight",
+                        "mixer.o_proj.weight", "mixer.q_norm.weight", "mixer.k_norm.weight", "mixer.gate.weight",
+                        "mixer.gate.bias", "mixer.vr_lambda", "norm2.weight", "ffn.gate.weight", "ffn.up.weight",
+                        "ffn.down.weight")
+
+
+def nanolab_param_names(layers: int):
+    names = ["tok_emb.weight"]
+    for i in range(layers):
+        names += [f"blocks.{i}.{n}" for n in NANOLAB_BLOCK_PARAMS]
+    return names + ["norm_f.weight"]
+
+
+def nanolab_param_lens(cfg: NanolabConfig):
+    n = int(_lib.orc_nanolab_param_count(C.byref(cfg)))
+    return [int(_lib.orc_nanolab_param_len(C.byref(cfg), _sz(i))) for i in range(n)]
+
+
+def rope_tables(seq: int, head_dim: int, base: float = 10000.0):
+    cos, sin = np.empty((seq, head_dim), np.float32), np.empty((seq, head_dim), np.float32)
+    _lib.orc_rope_tables(_sz(seq), _sz(head_dim), C.c_double(base), _fp(cos), _fp(sin))
+    return cos, sin
+
+
+def nanolab_loss_and_grads(cfg: NanolabConfig, params, ids, targets, want_logits=False, want_grads=True):
+    params = [_f32(p).reshape(-1) for p in params]
+    assert [p.size for p in params] == nanolab_param_lens(cfg)
+    ids = np.ascontiguousarray(ids, dtype=np.uint32)
+    targets = np.ascontiguousarray(targets, dtype=np.uint32)
+    grads = [np.zeros_like(p) for p in params]
+    pp = (_f * len(params))(*[_fp(p) for p in params])
+    gp = (_f * len(grads))(*[_fp(g) for g in grads]) if want_grads else None
+    logits = np.empty((cfg.batch * cfg.seq, cfg.vocab), np.float32) if want_logits else None
+    loss = C.c_float()
+    _check(_lib.orc_nanolab_loss_and_grads(C.byref(cfg), pp, _up(ids), _up(targets), C.byref(loss),
+                                           _fp(logits) if want_logits else None, gp), "nanolab_loss_and_grads")
+    return np.float32(loss.value), logits, (grads if want_grads else None)
