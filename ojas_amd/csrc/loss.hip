@@ -61,9 +61,48 @@ __global__ void ce_count_valid_kernel(const unsigned int* __restrict__ targets, 
   if ((threadIdx.x & 63) == 0 && ballot) atomicAdd(valid, static_cast<unsigned int>(__popcll(ballot)));
 }
 
-// One block per row. Folds the tile's columns [col0, col0 + ncols) into the
-// row's running (max, other, picked). `first` starts the state.
+// Loads VEC consecutive logits (one 16-byte access when VEC > 1).
+template <typename T, int VEC>
+__device__ __forceinline__ void ce_load(const T* __restrict__ r, unsigned int c, float (&v)[VEC]) {
+  if constexpr (VEC == 1) {
+    v[0] = dev_load<T>(r, c);
+  } else if constexpr (sizeof(T) == 4) {
+    float4 q = *reinterpret_cast<const float4*>(r + c);
+    v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+  } else {
+    uint4 q = *reinterpret_cast<const uint4*>(r + c);
+    const unsigned int w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      v[2 * j] = __uint_as_float(w[j] << 16);
+      v[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+    }
+  }
+}
+template <typename T, int VEC>
+__device__ __forceinline__ void ce_store(T* __restrict__ g, unsigned int c, const float (&v)[VEC]) {
+  if constexpr (VEC == 1) {
+    dev_store<T>(g, c, v[0]);
+  } else if constexpr (sizeof(T) == 4) {
+    *reinterpret_cast<float4*>(g + c) = make_float4(v[0], v[1], v[2], v[3]);
+  } else {
+    unsigned int w[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      w[j] = static_cast<unsigned int>(dev_f32_to_bf16_bits(v[2 * j])) |
+             (static_cast<unsigned int>(dev_f32_to_bf16_bits(v[2 * j + 1])) << 16);
+    *reinterpret_cast<uint4*>(g + c) = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+}
+// Elements per 16-byte access of T.
 template <typename T>
+constexpr int ce_vec() { return 16 / static_cast<int>(sizeof(T)); }
+
+// One block per row. Folds the tile's columns [col0, col0 + ncols) into the
+// row's running (max, other, picked) in ONE pass over the row: every thread
+// keeps an online (max, sum) pair that is rescaled when its maximum grows,
+// and the pairs are merged once at the end. `first` starts the state.
+template <typename T, int VEC>
 __global__ __launch_bounds__(CE_THREADS) void ce_tile_stats_kernel(const T* __restrict__ tile, size_t ld,
                                                                    size_t row0, unsigned int col0,
                                                                    unsigned int ncols,
@@ -74,29 +113,38 @@ __global__ __launch_bounds__(CE_THREADS) void ce_tile_stats_kernel(const T* __re
   const size_t local = blockIdx.x, row = row0 + local;
   const T* r = tile + local * ld;
   const unsigned int target = targets[row];
-  float mx = -INFINITY;
+  const unsigned int tcol = target - col0;  // wraps to a huge value when the target is left of this tile
+  float mx = -INFINITY, sum = 0.0f;
   bool bad = false;
-  for (unsigned int c = threadIdx.x; c < ncols; c += CE_THREADS) {
-    float v = dev_load<T>(r, c);
-    bad |= !dev_finite(v);
-    mx = fmaxf(mx, v);
+  for (unsigned int c = threadIdx.x * VEC; c < ncols; c += CE_THREADS * VEC) {
+    float v[VEC];
+    ce_load<T, VEC>(r, c, v);
+    float top = v[0];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      bad |= !dev_finite(v[j]);
+      top = fmaxf(top, v[j]);
+    }
+    if (top > mx) {
+      sum *= expf(mx - top);
+      mx = top;
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; ++j)
+      if (c + j != tcol) sum += expf(v[j] - mx);
   }
-  mx = block_max(mx, red);
-  float old_max = first ? -INFINITY : st.max[row];
-  float new_max = fmaxf(old_max, mx);
-  float sum = 0.0f;
-  for (unsigned int c = threadIdx.x; c < ncols; c += CE_THREADS) {
-    if (col0 + c != target) sum += expf(dev_load<T>(r, c) - new_max);
-  }
-  sum = block_sum(sum, red);
+  const float row_max = block_max(mx, red);
+  sum = block_sum(mx == -INFINITY ? 0.0f : sum * expf(mx - row_max), red);
   if (__syncthreads_or(bad)) {
     if (threadIdx.x == 0) dev_raise_fault(fault, tag);
   }
   if (threadIdx.x == 0) {
+    float old_max = first ? -INFINITY : st.max[row];
+    float new_max = fmaxf(old_max, row_max);
     float other = first ? 0.0f : st.other[row] * expf(old_max - new_max);
     st.max[row] = new_max;
-    st.other[row] = other + sum;
-    if (target >= col0 && target < col0 + ncols) st.picked[row] = dev_load<T>(r, target - col0);
+    st.other[row] = other + sum * expf(row_max - new_max);
+    if (target >= col0 && target < col0 + ncols) st.picked[row] = dev_load<T>(r, tcol);
   }
 }
 
@@ -135,7 +183,7 @@ __global__ __launch_bounds__(1024) void ce_mean_kernel(CeState st, const unsigne
 }
 
 // One block per row: tile of logits -> tile of gradients (may be in place).
-template <typename TL, typename TG>
+template <typename TL, typename TG, int VEC>
 __global__ __launch_bounds__(CE_THREADS) void ce_tile_grad_kernel(const TL* __restrict__ tile, TG* __restrict__ grad,
                                                                   size_t ld, size_t ld_grad, size_t row0,
                                                                   unsigned int col0, unsigned int ncols,
@@ -147,34 +195,62 @@ __global__ __launch_bounds__(CE_THREADS) void ce_tile_grad_kernel(const TL* __re
   TG* g = grad + local * ld_grad;
   const unsigned int target = targets[row];
   if (has_ignore && target == ignore) {
-    for (unsigned int c = threadIdx.x; c < ncols; c += CE_THREADS) dev_store<TG>(g, c, 0.0f);
+    float zero[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) zero[j] = 0.0f;
+    for (unsigned int c = threadIdx.x * VEC; c < ncols; c += CE_THREADS * VEC) ce_store<TG, VEC>(g, c, zero);
     return;
   }
+  const unsigned int tcol = target - col0;
   const float m = st.max[row], other = st.other[row], p = st.picked[row];
   const float denom = static_cast<float>(*valid);
   const float sum = other + expf(p - m);
   const bool collapse = (p == m && sum == 1.0f && other > 0.0f);
   const float d = collapse ? 1.0f + other : sum;
   const float target_grad = collapse ? -(other / d) / denom : (expf(p - m) / d) / denom - 1.0f / denom;
-  for (unsigned int c = threadIdx.x; c < ncols; c += CE_THREADS) {
-    float v = (col0 + c == target) ? target_grad : (expf(dev_load<TL>(r, c) - m) / d) / denom;
-    dev_store<TG>(g, c, v);
+  const float scale = (1.0f / d) / denom;
+  for (unsigned int c = threadIdx.x * VEC; c < ncols; c += CE_THREADS * VEC) {
+    float v[VEC], out[VEC];
+    ce_load<TL, VEC>(r, c, v);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) out[j] = (c + j == tcol) ? target_grad : expf(v[j] - m) * scale;
+    ce_store<TG, VEC>(g, c, out);
   }
+}
+
+// Whether rows of `ld` elements starting at `base` (+ col offset) allow 16-byte accesses of T.
+template <typename T>
+bool ce_vector_ok(const void* base, size_t ld, unsigned int ncols) {
+  return (reinterpret_cast<uintptr_t>(base) & 15u) == 0 && (ld * sizeof(T)) % 16 == 0 && ncols % ce_vec<T>() == 0;
 }
 
 template <typename T>
 void launch_stats(omx_ctx* ctx, const void* tile, size_t ld, size_t row0, size_t nrows, unsigned int col0,
                   unsigned int ncols, const unsigned int* targets, CeState st, int first, unsigned long long tag) {
-  hipLaunchKernelGGL((ce_tile_stats_kernel<T>), dim3(static_cast<unsigned>(nrows)), dim3(CE_THREADS), 0, ctx->stream,
-                     static_cast<const T*>(tile), ld, row0, col0, ncols, targets, st, first, ctx->fault, tag);
+  dim3 grid(static_cast<unsigned>(nrows)), block(CE_THREADS);
+  if (ce_vector_ok<T>(tile, ld, ncols))
+    hipLaunchKernelGGL((ce_tile_stats_kernel<T, ce_vec<T>()>), grid, block, 0, ctx->stream,
+                       static_cast<const T*>(tile), ld, row0, col0, ncols, targets, st, first, ctx->fault, tag);
+  else
+    hipLaunchKernelGGL((ce_tile_stats_kernel<T, 1>), grid, block, 0, ctx->stream, static_cast<const T*>(tile), ld,
+                       row0, col0, ncols, targets, st, first, ctx->fault, tag);
 }
 template <typename TL, typename TG>
 void launch_grad(omx_ctx* ctx, const void* tile, void* grad, size_t ld, size_t ld_grad, size_t row0, size_t nrows,
                  unsigned int col0, unsigned int ncols, const unsigned int* targets, int has_ignore,
                  unsigned int ignore, CeState st, const unsigned int* valid) {
-  hipLaunchKernelGGL((ce_tile_grad_kernel<TL, TG>), dim3(static_cast<unsigned>(nrows)), dim3(CE_THREADS), 0,
-                     ctx->stream, static_cast<const TL*>(tile), static_cast<TG*>(grad), ld, ld_grad, row0, col0, ncols,
-                     targets, has_ignore, ignore, st, valid);
+  dim3 grid(static_cast<unsigned>(nrows)), block(CE_THREADS);
+  // 16-byte packs on both sides need logits and gradients of one element size.
+  if constexpr (sizeof(TL) == sizeof(TG)) {
+    if (ce_vector_ok<TL>(tile, ld, ncols) && ce_vector_ok<TG>(grad, ld_grad, ncols)) {
+      hipLaunchKernelGGL((ce_tile_grad_kernel<TL, TG, ce_vec<TL>()>), grid, block, 0, ctx->stream,
+                         static_cast<const TL*>(tile), static_cast<TG*>(grad), ld, ld_grad, row0, col0, ncols, targets,
+                         has_ignore, ignore, st, valid);
+      return;
+    }
+  }
+  hipLaunchKernelGGL((ce_tile_grad_kernel<TL, TG, 1>), grid, block, 0, ctx->stream, static_cast<const TL*>(tile),
+                     static_cast<TG*>(grad), ld, ld_grad, row0, col0, ncols, targets, has_ignore, ignore, st, valid);
 }
 
 // State + valid counter carved out of a workspace block.
