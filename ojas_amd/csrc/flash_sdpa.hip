@@ -37,7 +37,6 @@ constexpr int FPITCH = 144;         // bytes per LDS row: 64 bf16 + 16 pad
 constexpr int FTILE = 64 * FPITCH;  // a 64-row tile
 constexpr int FT = 256;             // threads per block (4 waves of 32 rows)
 constexpr float LOG2E = 1.4426950408889634f;
-constexpr float LN2 = 0.6931471805599453f;
 
 struct FlashShape {
   int batch, heads, kv_heads, time, window, rep;
@@ -152,7 +151,7 @@ __device__ __forceinline__ bool store_transposed_acc(TO* __restrict__ plane, int
 
 // ------------------------------------------------------------------ forward
 template <typename TO>
-__global__ __launch_bounds__(FT) void flash_fwd_kernel(const unsigned short* __restrict__ q,
+__global__ __launch_bounds__(FT, 3) void flash_fwd_kernel(const unsigned short* __restrict__ q,
                                                        const unsigned short* __restrict__ k,
                                                        const unsigned short* __restrict__ v, TO* __restrict__ out,
                                                        float* __restrict__ lse, FlashShape s, OmxFaultWord* fault,
@@ -201,38 +200,46 @@ __global__ __launch_bounds__(FT) void flash_fwd_kernel(const unsigned short* __r
     for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
       for (int kk = 0; kk < 4; ++kk) sc[sub] = mfma(frag_rows(k_rows, sub, kk, l32, lg), qf[kk], sc[sub]);
-    float tmax = -INFINITY;
+    // Only a tile that crosses the diagonal, the sequence end or the window edge needs the mask
+    // (wave-uniform). `m` is the running maximum of the raw scores; the scale joins inside the fma.
+    if (key0 + 63 > wave_q0 || key0 + 63 >= T || s.window > 0) {
 #pragma unroll
-    for (int sub = 0; sub < 2; ++sub)
+      for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
-      for (int vv = 0; vv < 16; ++vv) {
-        const int key = key0 + sub * 32 + acc_row(vv, lg);
-        float val = sc[sub][vv] * scale_log2;
-        const bool masked = key > q_row || key >= T || (s.window > 0 && key + s.window <= q_row);
-        val = masked ? -INFINITY : val;
-        sc[sub][vv] = val;
-        tmax = fmaxf(tmax, val);
-      }
+        for (int vv = 0; vv < 16; ++vv) {
+          const int key = key0 + sub * 32 + acc_row(vv, lg);
+          const bool masked = key > q_row || key >= T || (s.window > 0 && key + s.window <= q_row);
+          sc[sub][vv] = masked ? -INFINITY : sc[sub][vv];
+        }
+    }
+    float tmax = fmaxf(sc[0][0], sc[1][0]);
+#pragma unroll
+    for (int vv = 1; vv < 16; ++vv) tmax = fmaxf(tmax, fmaxf(sc[0][vv], sc[1][vv]));
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
     const float new_m = fmaxf(m, tmax);
     const float m_safe = new_m == -INFINITY ? 0.0f : new_m;
-    const float alpha = __builtin_amdgcn_exp2f(m - m_safe);
+    const float neg_m = -m_safe * scale_log2;
     float psum = 0.0f;
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
       for (int vv = 0; vv < 16; ++vv) {
-        float p = __builtin_amdgcn_exp2f(sc[sub][vv] - m_safe);
+        float p = __builtin_amdgcn_exp2f(fmaf(sc[sub][vv], scale_log2, neg_m));
         sc[sub][vv] = p;
         psum += p;
       }
     psum += __shfl_xor(psum, 32, 64);
-    lsum = lsum * alpha + psum;
+    if (__any(new_m > m)) {
+      // Some row's maximum grew: rescale what is accumulated so far.
+      const float alpha = __builtin_amdgcn_exp2f(fmaf(m, scale_log2, neg_m));
+      lsum *= alpha;
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int vv = 0; vv < 16; ++vv) o[mt][vv] *= alpha;
+    }
+    lsum += psum;
     m = new_m;
-#pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-      for (int vv = 0; vv < 16; ++vv) o[mt][vv] *= alpha;
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
@@ -245,7 +252,7 @@ __global__ __launch_bounds__(FT) void flash_fwd_kernel(const unsigned short* __r
   bool bad = false;
   if (q_row < T) {
     bad |= !(dev_finite(lsum) && lsum > 0.0f);
-    if (lg == 0) lse[plane * T + q_row] = m * LN2 + logf(lsum);
+    if (lg == 0) lse[plane * T + q_row] = m * s.scale + logf(lsum);
   }
   bad |= store_transposed_acc<TO>(out + plane * T * FD, q_row, T, lg, o, 1.0f / lsum);
   if (bad) dev_raise_fault(fault, tag);
@@ -253,7 +260,7 @@ __global__ __launch_bounds__(FT) void flash_fwd_kernel(const unsigned short* __r
 
 // ------------------------------------------------------------------ backward: dK, dV
 template <typename TO>
-__global__ __launch_bounds__(FT) void flash_bwd_dkv_kernel(
+__global__ __launch_bounds__(FT, 2) void flash_bwd_dkv_kernel(
     const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
     const float* __restrict__ lse, const float* __restrict__ delta, const unsigned short* __restrict__ gy,
     TO* __restrict__ gk, TO* __restrict__ gv, FlashShape s, OmxFaultWord* fault, unsigned long long tag) {
@@ -288,8 +295,14 @@ __global__ __launch_bounds__(FT) void flash_bwd_dkv_kernel(
   const int steps = s.rep * nq;
   u32x4 rq[2], rg[2];
   float row_lse = 0.0f, row_del = 0.0f;
-  auto fetch = [&](int idx) {
-    const int r = idx / nq, q0 = (qt_first + idx % nq) * 64;
+  // (head of the group, query tile) of the tile being fetched / being multiplied.
+  int fetch_r = 0, fetch_qt = qt_first, cur_qt = qt_first;
+  auto fetch = [&]() {
+    const int r = fetch_r, q0 = fetch_qt * 64;
+    if (++fetch_qt > qt_last) {
+      fetch_qt = qt_first;
+      ++fetch_r;
+    }
     const long q_plane = static_cast<long>(b) * s.heads + static_cast<long>(gidx) * s.rep + r;
     tile_load(q + q_plane * T * FD, q0, T, rq);
     tile_load(gy + q_plane * T * FD, q0, T, rg);
@@ -301,10 +314,11 @@ __global__ __launch_bounds__(FT) void flash_bwd_dkv_kernel(
       bad |= !(dev_finite(row_lse) && dev_finite(row_del));
     }
   };
-  fetch(0);
+  fetch();
   for (int idx = 0; idx < steps; ++idx) {
     {
-      const int q0 = (qt_first + idx % nq) * 64;
+      const int q0 = cur_qt * 64;
+      if (++cur_qt > qt_last) cur_qt = qt_first;
       __syncthreads();
       tile_store_rows(q_rows, rq);
       tile_store_rows(g_rows, rg);
@@ -315,9 +329,11 @@ __global__ __launch_bounds__(FT) void flash_bwd_dkv_kernel(
         del_s[threadIdx.x] = row_del;
       }
       __syncthreads();
-      if (idx + 1 < steps) fetch(idx + 1);
+      if (idx + 1 < steps) fetch();
       const bool active = q0 + 63 >= wave_k0 && (s.window == 0 || q0 < wave_k0 + 31 + s.window);
       if (!active) continue;
+      // Wave-uniform: a tile whose queries all come after the wave's keys and end inside the sequence has no mask.
+      const bool needs_mask = q0 < wave_k0 + 31 || q0 + 63 >= T || s.window > 0;
 #pragma unroll
       for (int sub = 0; sub < 2; ++sub) {
         floatx16 sc = zero16(), dp = zero16();
@@ -326,16 +342,28 @@ __global__ __launch_bounds__(FT) void flash_bwd_dkv_kernel(
           sc = mfma(frag_rows(q_rows, sub, kk, l32, lg), kf[kk], sc);
           dp = mfma(frag_rows(g_rows, sub, kk, l32, lg), vf[kk], dp);
         }
+        if (needs_mask) {
 #pragma unroll
-        for (int vv = 0; vv < 16; ++vv) {
-          const int qi_local = sub * 32 + acc_row(vv, lg);
-          const int qi = q0 + qi_local;
-          const bool masked =
-              key_row > qi || qi >= T || key_row >= T || (s.window > 0 && key_row + s.window <= qi);
-          float p = masked ? 0.0f : __builtin_amdgcn_exp2f(sc[vv] * scale_log2 - lse_s[qi_local]);
-          float ds = p * (dp[vv] - del_s[qi_local]) * s.scale;
-          sc[vv] = p;
-          dp[vv] = ds;
+          for (int vv = 0; vv < 16; ++vv) {
+            const int qi = q0 + sub * 32 + acc_row(vv, lg);
+            const bool masked =
+                key_row > qi || qi >= T || key_row >= T || (s.window > 0 && key_row + s.window <= qi);
+            sc[vv] = masked ? -INFINITY : sc[vv];
+          }
+        }
+        // P = 2^(s * scale * log2e - lse * log2e); dS / scale = P (dP - delta): the scale joins dK at the end.
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          const float4 l4 = *reinterpret_cast<const float4*>(lse_s + sub * 32 + 8 * q4 + 4 * lg);
+          const float4 d4 = *reinterpret_cast<const float4*>(del_s + sub * 32 + 8 * q4 + 4 * lg);
+          const float lv[4] = {l4.x, l4.y, l4.z, l4.w}, dl[4] = {d4.x, d4.y, d4.z, d4.w};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int vv = 4 * q4 + j;
+            const float p = __builtin_amdgcn_exp2f(fmaf(sc[vv], scale_log2, -lv[j]));
+            dp[vv] = p * (dp[vv] - dl[j]);
+            sc[vv] = p;
+          }
         }
 #pragma unroll
         for (int c = 0; c < 2; ++c) {
@@ -349,14 +377,14 @@ __global__ __launch_bounds__(FT) void flash_bwd_dkv_kernel(
       }
     }
   }
-  bad |= store_transposed_acc<TO>(gk + kv_plane * T * FD, key_row, T, lg, dk, 1.0f);
+  bad |= store_transposed_acc<TO>(gk + kv_plane * T * FD, key_row, T, lg, dk, s.scale);
   bad |= store_transposed_acc<TO>(gv + kv_plane * T * FD, key_row, T, lg, dv, 1.0f);
   if (bad) dev_raise_fault(fault, tag);
 }
 
 // ------------------------------------------------------------------ backward: dQ
 template <typename TO>
-__global__ __launch_bounds__(FT) void flash_bwd_dq_kernel(
+__global__ __launch_bounds__(FT, 3) void flash_bwd_dq_kernel(
     const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
     const float* __restrict__ lse, const float* __restrict__ delta, const unsigned short* __restrict__ gy,
     TO* __restrict__ gq, FlashShape s, OmxFaultWord* fault, unsigned long long tag) {
@@ -384,7 +412,7 @@ __global__ __launch_bounds__(FT) void flash_bwd_dq_kernel(
     row_del = delta[plane * T + q_row];
     bad |= !(dev_finite(row_lse) && dev_finite(row_del));
   }
-  row_lse *= LOG2E;
+  const float neg_lse = -row_lse * LOG2E;
   floatx16 dq[2] = {zero16(), zero16()};
   const float scale_log2 = s.scale * LOG2E;
   const int block_q0 = qb * 128, block_q1 = min(T - 1, qb * 128 + 127);
@@ -406,6 +434,7 @@ __global__ __launch_bounds__(FT) void flash_bwd_dq_kernel(
     }
     const bool active = key0 <= wave_q0 + 31 && (s.window == 0 || key0 + 63 + s.window > wave_q0);
     if (!active) continue;
+    const bool needs_mask = key0 + 63 > wave_q0 || key0 + 63 >= T || s.window > 0;
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub) {
       floatx16 sc = zero16(), dp = zero16();
@@ -414,12 +443,18 @@ __global__ __launch_bounds__(FT) void flash_bwd_dq_kernel(
         sc = mfma(frag_rows(k_rows, sub, kk, l32, lg), qf[kk], sc);
         dp = mfma(frag_rows(v_rows, sub, kk, l32, lg), gf[kk], dp);
       }
+      if (needs_mask) {
+#pragma unroll
+        for (int vv = 0; vv < 16; ++vv) {
+          const int key = key0 + sub * 32 + acc_row(vv, lg);
+          const bool masked = key > q_row || key >= T || q_row >= T || (s.window > 0 && key + s.window <= q_row);
+          sc[vv] = masked ? -INFINITY : sc[vv];
+        }
+      }
 #pragma unroll
       for (int vv = 0; vv < 16; ++vv) {
-        const int key = key0 + sub * 32 + acc_row(vv, lg);
-        const bool masked = key > q_row || key >= T || q_row >= T || (s.window > 0 && key + s.window <= q_row);
-        float p = masked ? 0.0f : __builtin_amdgcn_exp2f(sc[vv] * scale_log2 - row_lse);
-        dp[vv] = p * (dp[vv] - row_del) * s.scale;
+        const float p = __builtin_amdgcn_exp2f(fmaf(sc[vv], scale_log2, neg_lse));
+        dp[vv] = p * (dp[vv] - row_del);  // dS / scale: the scale joins dQ at the end
       }
 #pragma unroll
       for (int c = 0; c < 2; ++c) {
@@ -429,7 +464,7 @@ __global__ __launch_bounds__(FT) void flash_bwd_dq_kernel(
       }
     }
   }
-  bad |= store_transposed_acc<TO>(gq + plane * T * FD, q_row, T, lg, dq, 1.0f);
+  bad |= store_transposed_acc<TO>(gq + plane * T * FD, q_row, T, lg, dq, s.scale);
   if (bad) dev_raise_fault(fault, tag);
 }
 
