@@ -131,6 +131,28 @@ int32_t omx_causal_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, con
                                  uint64_t kv_heads, uint64_t time, uint64_t head_dim,
                                  uint64_t window);
 
+/* ---- causal_attention (ojas-model/src/block.rs:186-199): permute [0,2,1,3],
+ *      causal_sdpa, permute back, done in one pass over time-major tensors.
+ *      q / out / gy / gq are [batch, time, heads, head_dim], k / v / gk / gv
+ *      [batch, time, kv_heads, head_dim]; a token's heads are contiguous and
+ *      token rows are `*_pitch` elements apart (a multiple of 8, at least
+ *      heads * head_dim), so q, k and v may be column blocks of one projection
+ *      output. gq uses q_pitch, gk / gv use kv_pitch. lse is [batch, heads, time]
+ *      f32. bf16 with head_dim 64 only; other shapes return Unsupported and the
+ *      caller composes omx_permute_0213 with omx_causal_sdpa_*. ---- */
+int32_t omx_causal_attention_forward(omx_ctx* ctx, const void* q, uint64_t q_pitch, const void* k,
+                                     const void* v, uint64_t kv_pitch, int32_t operand_dtype,
+                                     void* out, uint64_t out_pitch, int32_t out_dtype, void* lse,
+                                     uint64_t batch, uint64_t time, uint64_t heads,
+                                     uint64_t kv_heads, uint64_t head_dim, uint64_t window);
+int32_t omx_causal_attention_backward(omx_ctx* ctx, const void* q, uint64_t q_pitch, const void* k,
+                                      const void* v, uint64_t kv_pitch, const void* out,
+                                      const void* gy, uint64_t out_pitch, const void* lse,
+                                      int32_t operand_dtype, void* gq, void* gk, void* gv,
+                                      int32_t grad_dtype, uint64_t batch, uint64_t time,
+                                      uint64_t heads, uint64_t kv_heads, uint64_t head_dim,
+                                      uint64_t window);
+
 /* ---- BackendModule::rms_norm_forward / _backward (backend.rs:1658-1672) ---- */
 int32_t omx_rms_norm_forward(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* w_f32,
                              void* y, int32_t y_dtype, uint64_t rows, uint64_t dim, float eps);

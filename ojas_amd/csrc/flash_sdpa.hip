@@ -38,9 +38,14 @@ constexpr int FTILE = 64 * FPITCH;  // a 64-row tile
 constexpr int FT = 256;             // threads per block (4 waves of 32 rows)
 constexpr float LOG2E = 1.4426950408889634f;
 
+// Element strides of one tensor: between rows (time steps), heads and batches.
+struct FlashStrides {
+  long rs, hs, bs;
+};
 struct FlashShape {
   int batch, heads, kv_heads, time, window, rep;
   float scale;
+  FlashStrides q, kv, o;  // q and grad_q; k, v and their gradients; out and grad_out
 };
 
 __device__ __forceinline__ int perm16(int k) { return (k & ~12) | ((k & 4) << 1) | ((k & 8) >> 1); }
@@ -71,13 +76,14 @@ __device__ __forceinline__ floatx16 zero16() {
 // A 64-row x 64-column bf16 tile starting at row `row0` of a [time, 64] plane.
 // Thread t moves rows 2(t>>3) and 2(t>>3)+1, 16-byte chunk t&7; rows at or
 // past `time` read as zeros.
-__device__ __forceinline__ void tile_load(const unsigned short* __restrict__ plane, int row0, int time, u32x4 r[2]) {
+__device__ __forceinline__ void tile_load(const unsigned short* __restrict__ plane, long rs, int row0, int time,
+                                          u32x4 r[2]) {
   const int t = threadIdx.x;
   const int row = row0 + 2 * (t >> 3), kc = t & 7;
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     r[i] = u32x4{0u, 0u, 0u, 0u};
-    if (row + i < time) r[i] = *reinterpret_cast<const u32x4*>(plane + static_cast<long>(row + i) * FD + kc * 8);
+    if (row + i < time) r[i] = *reinterpret_cast<const u32x4*>(plane + static_cast<long>(row + i) * rs + kc * 8);
   }
 }
 // [row][d] form.
@@ -112,12 +118,12 @@ __device__ __forceinline__ u32x4 frag_transposed(const char* lds, int mt, int su
   return *reinterpret_cast<const u32x4*>(lds + (mt * 32 + l32) * FPITCH + (sub * 32 + c * 16 + lg * 8) * 2);
 }
 // B operand held in registers: the lane's own row of a [time, 64] plane.
-__device__ __forceinline__ void row_frags(const unsigned short* __restrict__ plane, int row, int time, int lg,
+__device__ __forceinline__ void row_frags(const unsigned short* __restrict__ plane, long rs, int row, int time, int lg,
                                           u32x4 f[4]) {
 #pragma unroll
   for (int kk = 0; kk < 4; ++kk) {
     f[kk] = u32x4{0u, 0u, 0u, 0u};
-    if (row < time) f[kk] = *reinterpret_cast<const u32x4*>(plane + static_cast<long>(row) * FD + kk * 16 + lg * 8);
+    if (row < time) f[kk] = *reinterpret_cast<const u32x4*>(plane + static_cast<long>(row) * rs + kk * 16 + lg * 8);
   }
 }
 // Row index (within a 32-row sub-tile) that accumulator register v of this lane holds.
@@ -125,7 +131,7 @@ __device__ __forceinline__ int acc_row(int v, int lg) { return 8 * (v >> 2) + 4 
 
 // Stores a transposed accumulator pair (d x rows) as rows of a [time, 64] plane.
 template <typename TO>
-__device__ __forceinline__ bool store_transposed_acc(TO* __restrict__ plane, int row, int time, int lg,
+__device__ __forceinline__ bool store_transposed_acc(TO* __restrict__ plane, long rs, int row, int time, int lg,
                                                      const floatx16 acc[2], float mul) {
   bool bad = false;
   if (row >= time) return false;
@@ -141,9 +147,9 @@ __device__ __forceinline__ bool store_transposed_acc(TO* __restrict__ plane, int
         uint2 w;
         w.x = pack2(x0, x1);
         w.y = pack2(x2, x3);
-        *reinterpret_cast<uint2*>(plane + static_cast<long>(row) * FD + d) = w;
+        *reinterpret_cast<uint2*>(plane + static_cast<long>(row) * rs + d) = w;
       } else {
-        *reinterpret_cast<float4*>(plane + static_cast<long>(row) * FD + d) = make_float4(x0, x1, x2, x3);
+        *reinterpret_cast<float4*>(plane + static_cast<long>(row) * rs + d) = make_float4(x0, x1, x2, x3);
       }
     }
   return bad;
@@ -165,14 +171,14 @@ __global__ __launch_bounds__(FT, 3) void flash_fwd_kernel(const unsigned short* 
   const int qb = gridDim.x - 1 - blockIdx.x;
   const long plane = blockIdx.y;
   const int h = static_cast<int>(plane % s.heads), b = static_cast<int>(plane / s.heads);
-  const long kv_plane = static_cast<long>(b) * s.kv_heads + h / s.rep;
-  const unsigned short* qp = q + plane * T * FD;
-  const unsigned short* kp = k + kv_plane * T * FD;
-  const unsigned short* vp = v + kv_plane * T * FD;
+  const int kvh = h / s.rep;
+  const unsigned short* qp = q + b * s.q.bs + h * s.q.hs;
+  const unsigned short* kp = k + b * s.kv.bs + kvh * s.kv.hs;
+  const unsigned short* vp = v + b * s.kv.bs + kvh * s.kv.hs;
   const int wave_q0 = qb * 128 + wave * 32;
   const int q_row = wave_q0 + l32;
   u32x4 qf[4];
-  row_frags(qp, q_row, T, lg, qf);
+  row_frags(qp, s.q.rs, q_row, T, lg, qf);
   floatx16 o[2] = {zero16(), zero16()};
   float m = -INFINITY, lsum = 0.0f;
   const float scale_log2 = s.scale * LOG2E;
@@ -181,8 +187,8 @@ __global__ __launch_bounds__(FT, 3) void flash_fwd_kernel(const unsigned short* 
   const int kt_last = block_q1 / 64;
   // The next tile's global loads are in flight while the current one is multiplied.
   u32x4 rk[2], rv[2];
-  tile_load(kp, kt_first * 64, T, rk);
-  tile_load(vp, kt_first * 64, T, rv);
+  tile_load(kp, s.kv.rs, kt_first * 64, T, rk);
+  tile_load(vp, s.kv.rs, kt_first * 64, T, rv);
   for (int kt = kt_first; kt <= kt_last; ++kt) {
     const int key0 = kt * 64;
     __syncthreads();  // the previous tile's reads are done
@@ -190,8 +196,8 @@ __global__ __launch_bounds__(FT, 3) void flash_fwd_kernel(const unsigned short* 
     tile_store_transposed(v_tr, rv);
     __syncthreads();
     if (kt < kt_last) {
-      tile_load(kp, key0 + 64, T, rk);
-      tile_load(vp, key0 + 64, T, rv);
+      tile_load(kp, s.kv.rs, key0 + 64, T, rk);
+      tile_load(vp, s.kv.rs, key0 + 64, T, rv);
     }
     const bool active = key0 <= wave_q0 + 31 && (s.window == 0 || key0 + 63 + s.window > wave_q0);
     if (!active) continue;
@@ -254,7 +260,7 @@ __global__ __launch_bounds__(FT, 3) void flash_fwd_kernel(const unsigned short* 
     bad |= !(dev_finite(lsum) && lsum > 0.0f);
     if (lg == 0) lse[plane * T + q_row] = m * s.scale + logf(lsum);
   }
-  bad |= store_transposed_acc<TO>(out + plane * T * FD, q_row, T, lg, o, 1.0f / lsum);
+  bad |= store_transposed_acc<TO>(out + b * s.o.bs + h * s.o.hs, s.o.rs, q_row, T, lg, o, 1.0f / lsum);
   if (bad) dev_raise_fault(fault, tag);
 }
 
@@ -276,13 +282,14 @@ __global__ __launch_bounds__(FT, 2) void flash_bwd_dkv_kernel(
   const int kb = blockIdx.x;  // early key blocks are seen by the most queries: they come first
   const long kv_plane = blockIdx.y;
   const int gidx = static_cast<int>(kv_plane % s.kv_heads), b = static_cast<int>(kv_plane / s.kv_heads);
-  const unsigned short* kp = k + kv_plane * T * FD;
-  const unsigned short* vp = v + kv_plane * T * FD;
+  const long kv_off = b * s.kv.bs + gidx * s.kv.hs;
+  const unsigned short* kp = k + kv_off;
+  const unsigned short* vp = v + kv_off;
   const int wave_k0 = kb * 128 + wave * 32;
   const int key_row = wave_k0 + l32;
   u32x4 kf[4], vf[4];
-  row_frags(kp, key_row, T, lg, kf);
-  row_frags(vp, key_row, T, lg, vf);
+  row_frags(kp, s.kv.rs, key_row, T, lg, kf);
+  row_frags(vp, s.kv.rs, key_row, T, lg, vf);
   floatx16 dk[2] = {zero16(), zero16()}, dv[2] = {zero16(), zero16()};
   const float scale_log2 = s.scale * LOG2E;
   const int block_k0 = kb * 128, block_k1 = min(T - 1, kb * 128 + 127);
@@ -304,8 +311,9 @@ __global__ __launch_bounds__(FT, 2) void flash_bwd_dkv_kernel(
       ++fetch_r;
     }
     const long q_plane = static_cast<long>(b) * s.heads + static_cast<long>(gidx) * s.rep + r;
-    tile_load(q + q_plane * T * FD, q0, T, rq);
-    tile_load(gy + q_plane * T * FD, q0, T, rg);
+    const long head = static_cast<long>(gidx) * s.rep + r;
+    tile_load(q + b * s.q.bs + head * s.q.hs, s.q.rs, q0, T, rq);
+    tile_load(gy + b * s.o.bs + head * s.o.hs, s.o.rs, q0, T, rg);
     row_lse = 0.0f;
     row_del = 0.0f;
     if (threadIdx.x < 64 && q0 + static_cast<int>(threadIdx.x) < T) {
@@ -377,8 +385,8 @@ __global__ __launch_bounds__(FT, 2) void flash_bwd_dkv_kernel(
       }
     }
   }
-  bad |= store_transposed_acc<TO>(gk + kv_plane * T * FD, key_row, T, lg, dk, s.scale);
-  bad |= store_transposed_acc<TO>(gv + kv_plane * T * FD, key_row, T, lg, dv, 1.0f);
+  bad |= store_transposed_acc<TO>(gk + kv_off, s.kv.rs, key_row, T, lg, dk, s.scale);
+  bad |= store_transposed_acc<TO>(gv + kv_off, s.kv.rs, key_row, T, lg, dv, 1.0f);
   if (bad) dev_raise_fault(fault, tag);
 }
 
@@ -397,14 +405,14 @@ __global__ __launch_bounds__(FT, 3) void flash_bwd_dq_kernel(
   const int qb = gridDim.x - 1 - blockIdx.x;
   const long plane = blockIdx.y;
   const int h = static_cast<int>(plane % s.heads), b = static_cast<int>(plane / s.heads);
-  const long kv_plane = static_cast<long>(b) * s.kv_heads + h / s.rep;
-  const unsigned short* kp = k + kv_plane * T * FD;
-  const unsigned short* vp = v + kv_plane * T * FD;
+  const int kvh = h / s.rep;
+  const unsigned short* kp = k + b * s.kv.bs + kvh * s.kv.hs;
+  const unsigned short* vp = v + b * s.kv.bs + kvh * s.kv.hs;
   const int wave_q0 = qb * 128 + wave * 32;
   const int q_row = wave_q0 + l32;
   u32x4 qf[4], gf[4];
-  row_frags(q + plane * T * FD, q_row, T, lg, qf);
-  row_frags(gy + plane * T * FD, q_row, T, lg, gf);
+  row_frags(q + b * s.q.bs + h * s.q.hs, s.q.rs, q_row, T, lg, qf);
+  row_frags(gy + b * s.o.bs + h * s.o.hs, s.o.rs, q_row, T, lg, gf);
   float row_lse = 0.0f, row_del = 0.0f;
   bool bad = false;
   if (q_row < T) {
@@ -419,8 +427,8 @@ __global__ __launch_bounds__(FT, 3) void flash_bwd_dq_kernel(
   const int kt_first = s.window > 0 ? max(0, block_q0 + 1 - s.window) / 64 : 0;
   const int kt_last = block_q1 / 64;
   u32x4 rk[2], rv[2];
-  tile_load(kp, kt_first * 64, T, rk);
-  tile_load(vp, kt_first * 64, T, rv);
+  tile_load(kp, s.kv.rs, kt_first * 64, T, rk);
+  tile_load(vp, s.kv.rs, kt_first * 64, T, rv);
   for (int kt = kt_first; kt <= kt_last; ++kt) {
     const int key0 = kt * 64;
     __syncthreads();
@@ -429,8 +437,8 @@ __global__ __launch_bounds__(FT, 3) void flash_bwd_dq_kernel(
     tile_store_transposed(k_tr, rk);
     __syncthreads();
     if (kt < kt_last) {
-      tile_load(kp, key0 + 64, T, rk);
-      tile_load(vp, key0 + 64, T, rv);
+      tile_load(kp, s.kv.rs, key0 + 64, T, rk);
+      tile_load(vp, s.kv.rs, key0 + 64, T, rv);
     }
     const bool active = key0 <= wave_q0 + 31 && (s.window == 0 || key0 + 63 + s.window > wave_q0);
     if (!active) continue;
@@ -464,24 +472,38 @@ __global__ __launch_bounds__(FT, 3) void flash_bwd_dq_kernel(
       }
     }
   }
-  bad |= store_transposed_acc<TO>(gq + plane * T * FD, q_row, T, lg, dq, s.scale);
+  bad |= store_transposed_acc<TO>(gq + b * s.q.bs + h * s.q.hs, s.q.rs, q_row, T, lg, dq, s.scale);
   if (bad) dev_raise_fault(fault, tag);
 }
 
-// delta[row] = dO[row] . O[row], one wave per row.
+// delta[b, h, t] = dO[b, h, t, :] . O[b, h, t, :], one wave per row.
 __global__ __launch_bounds__(FT) void flash_delta_kernel(const unsigned short* __restrict__ out,
                                                          const unsigned short* __restrict__ gy,
-                                                         float* __restrict__ delta, long rows) {
+                                                         float* __restrict__ delta, long rows, FlashShape s) {
   const int lane = threadIdx.x & 63;
   const long row = static_cast<long>(blockIdx.x) * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
-  float acc = dev_bf16_bits_to_f32(gy[row * FD + lane]) * dev_bf16_bits_to_f32(out[row * FD + lane]);
+  const long t = row % s.time, plane = row / s.time;
+  const long at = (plane / s.heads) * s.o.bs + (plane % s.heads) * s.o.hs + t * s.o.rs + lane;
+  float acc = dev_bf16_bits_to_f32(gy[at]) * dev_bf16_bits_to_f32(out[at]);
   acc = wave_sum(acc);
   if (lane == 0) delta[row] = acc;
 }
 
-FlashShape make_shape(uint64_t batch, uint64_t heads, uint64_t kv_heads, uint64_t time, uint64_t window, float scale) {
+// `strides`: nine element strides (row, head, batch of q; of k / v; of out), or null for
+// contiguous [batch, heads, time, 64] tensors.
+FlashShape make_shape(uint64_t batch, uint64_t heads, uint64_t kv_heads, uint64_t time, uint64_t window, float scale,
+                      const long* strides) {
   FlashShape s;
+  const long T = static_cast<long>(time);
+  s.q = {FD, T * FD, static_cast<long>(heads) * T * FD};
+  s.kv = {FD, T * FD, static_cast<long>(kv_heads) * T * FD};
+  s.o = s.q;
+  if (strides) {
+    s.q = {strides[0], strides[1], strides[2]};
+    s.kv = {strides[3], strides[4], strides[5]};
+    s.o = {strides[6], strides[7], strides[8]};
+  }
   s.batch = static_cast<int>(batch);
   s.heads = static_cast<int>(heads);
   s.kv_heads = static_cast<int>(kv_heads);
@@ -498,9 +520,9 @@ bool omx_flash_sdpa_supports(uint64_t dim, int32_t operand_dtype) { return dim =
 
 int32_t omx_flash_sdpa_forward(omx_ctx* ctx, const void* q, const void* k, const void* v, void* out, int32_t out_dtype,
                                float* lse, uint64_t batch, uint64_t heads, uint64_t kv_heads, uint64_t time,
-                               uint64_t dim, uint64_t window, float scale, unsigned long long tag) {
+                               uint64_t dim, uint64_t window, float scale, unsigned long long tag, const long* strides) {
   if (dim != FD) return omx_fail(ctx, OMX_UNSUPPORTED_HEAD_DIM, "head_dim %llu limit %d", (unsigned long long)dim, FD);
-  FlashShape s = make_shape(batch, heads, kv_heads, time, window, scale);
+  FlashShape s = make_shape(batch, heads, kv_heads, time, window, scale, strides);
   dim3 grid(static_cast<unsigned>((time + 127) / 128), static_cast<unsigned>(batch * heads)), block(FT);
   const unsigned short* qs = static_cast<const unsigned short*>(q);
   const unsigned short* ks = static_cast<const unsigned short*>(k);
@@ -518,9 +540,9 @@ int32_t omx_flash_sdpa_forward(omx_ctx* ctx, const void* q, const void* k, const
 int32_t omx_flash_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, const void* v, const void* out,
                                 const float* lse, const void* gy, void* gq, void* gk, void* gv, int32_t grad_dtype,
                                 uint64_t batch, uint64_t heads, uint64_t kv_heads, uint64_t time, uint64_t dim,
-                                uint64_t window, float scale, unsigned long long tag) {
+                                uint64_t window, float scale, unsigned long long tag, const long* strides) {
   if (dim != FD) return omx_fail(ctx, OMX_UNSUPPORTED_HEAD_DIM, "head_dim %llu limit %d", (unsigned long long)dim, FD);
-  FlashShape s = make_shape(batch, heads, kv_heads, time, window, scale);
+  FlashShape s = make_shape(batch, heads, kv_heads, time, window, scale, strides);
   const long rows = static_cast<long>(batch * heads * time);
   void* ws = nullptr;
   int32_t rc = omx_workspace(ctx, rows * sizeof(float), &ws);
@@ -532,7 +554,7 @@ int32_t omx_flash_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, cons
   const unsigned short* os = static_cast<const unsigned short*>(out);
   const unsigned short* gs = static_cast<const unsigned short*>(gy);
   hipLaunchKernelGGL(flash_delta_kernel, dim3(static_cast<unsigned>((rows + 3) / 4)), dim3(FT), 0, ctx->stream, os, gs,
-                     delta, rows);
+                     delta, rows, s);
   OMX_LAUNCH_CHECK(ctx, "flash_delta_kernel");
   dim3 block(FT);
   dim3 kv_grid(static_cast<unsigned>((time + 127) / 128), static_cast<unsigned>(batch * kv_heads));

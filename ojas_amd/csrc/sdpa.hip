@@ -20,11 +20,12 @@
 
 int32_t omx_flash_sdpa_forward(omx_ctx* ctx, const void* q, const void* k, const void* v, void* out,
                                int32_t out_dtype, float* lse, uint64_t batch, uint64_t heads, uint64_t kv_heads,
-                               uint64_t time, uint64_t dim, uint64_t window, float scale, unsigned long long tag);
+                               uint64_t time, uint64_t dim, uint64_t window, float scale, unsigned long long tag,
+                               const long* strides);
 int32_t omx_flash_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, const void* v, const void* out,
                                 const float* lse, const void* gy, void* gq, void* gk, void* gv, int32_t grad_dtype,
                                 uint64_t batch, uint64_t heads, uint64_t kv_heads, uint64_t time, uint64_t dim,
-                                uint64_t window, float scale, unsigned long long tag);
+                                uint64_t window, float scale, unsigned long long tag, const long* strides);
 bool omx_flash_sdpa_supports(uint64_t dim, int32_t operand_dtype);
 
 namespace {
@@ -334,7 +335,7 @@ int32_t omx_causal_sdpa_forward(omx_ctx* ctx, const void* q, const void* k, cons
   unsigned long long tag = omx_tag(ctx, F_SDPA_FORWARD);
   if (omx_flash_sdpa_supports(head_dim, operand_dtype))
     return omx_flash_sdpa_forward(ctx, q, k, v, out, out_dtype, static_cast<float*>(lse), batch, heads, kv_heads, time,
-                                  head_dim, s.window, s.scale, tag);
+                                  head_dim, s.window, s.scale, tag, nullptr);
   const long rows = static_cast<long>(batch) * heads * time;
   dim3 grid(static_cast<unsigned>((rows + 3) / 4)), block(SD_THREADS);
 #define SDPA_FWD(TI, TO)                                                                                          \
@@ -366,7 +367,7 @@ int32_t omx_causal_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, con
   unsigned long long tag = omx_tag(ctx, F_SDPA_BACKWARD);
   if (omx_flash_sdpa_supports(head_dim, operand_dtype))
     return omx_flash_sdpa_backward(ctx, q, k, v, out, static_cast<const float*>(lse), gy, gq, gk, gv, grad_dtype, batch,
-                                   heads, kv_heads, time, head_dim, s.window, s.scale, tag);
+                                   heads, kv_heads, time, head_dim, s.window, s.scale, tag, nullptr);
   const long rows = static_cast<long>(batch) * heads * time;
   const long kv_rows = static_cast<long>(batch) * kv_heads * time;
   void* ws = nullptr;
@@ -393,6 +394,68 @@ int32_t omx_causal_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, con
 #undef SDPA_BWD
   OMX_LAUNCH_CHECK(ctx, "sdpa backward row kernels");
   return OMX_OK;
+}
+
+// Time-major attention: the permute -> causal_sdpa -> permute of
+// ojas-model/src/block.rs:186-199 (causal_attention) in one pass over [B, T, heads, D] tensors.
+static int32_t check_attention(omx_ctx* ctx, const char* op, int32_t operand_dtype, uint64_t head_dim, uint64_t heads,
+                               uint64_t kv_heads, uint64_t q_pitch, uint64_t kv_pitch, uint64_t out_pitch,
+                               std::initializer_list<const void*> ptrs) {
+  for (const void* p : ptrs) {
+    if (!p) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+    if (reinterpret_cast<uintptr_t>(p) & 15u) return omx_fail(ctx, OMX_SHAPE, "%s: tensor not 16-byte aligned", op);
+  }
+  if (!omx_flash_sdpa_supports(head_dim, operand_dtype))
+    return omx_fail(ctx, OMX_UNSUPPORTED, "%s: only bf16 operands with head_dim 64 (compose permute and causal_sdpa)",
+                    op);
+  if (q_pitch < heads * head_dim || out_pitch < heads * head_dim || kv_pitch < kv_heads * head_dim ||
+      (q_pitch | kv_pitch | out_pitch) % 8 != 0)
+    return omx_fail(ctx, OMX_SHAPE, "%s: row pitch below heads * head_dim or not a multiple of 8", op);
+  return OMX_OK;
+}
+
+int32_t omx_causal_attention_forward(omx_ctx* ctx, const void* q, uint64_t q_pitch, const void* k, const void* v,
+                                     uint64_t kv_pitch, int32_t operand_dtype, void* out, uint64_t out_pitch,
+                                     int32_t out_dtype, void* lse, uint64_t batch, uint64_t time, uint64_t heads,
+                                     uint64_t kv_heads, uint64_t head_dim, uint64_t window) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "causal_attention_forward";
+  if (out_dtype != OMX_BF16) return omx_fail(ctx, OMX_DTYPE, "%s: output must be bf16", op);
+  SdpaShape s;
+  int32_t rc = check_shape(ctx, op, batch, heads, kv_heads, time, head_dim, window, &s);
+  if (rc != OMX_OK) return rc;
+  rc = check_attention(ctx, op, operand_dtype, head_dim, heads, kv_heads, q_pitch, kv_pitch, out_pitch,
+                       {q, k, v, out, lse});
+  if (rc != OMX_OK) return rc;
+  const long D = static_cast<long>(head_dim), T = static_cast<long>(time);
+  const long strides[9] = {static_cast<long>(q_pitch),   D, T * static_cast<long>(q_pitch),
+                           static_cast<long>(kv_pitch),  D, T * static_cast<long>(kv_pitch),
+                           static_cast<long>(out_pitch), D, T * static_cast<long>(out_pitch)};
+  return omx_flash_sdpa_forward(ctx, q, k, v, out, out_dtype, static_cast<float*>(lse), batch, heads, kv_heads, time,
+                                head_dim, s.window, s.scale, omx_tag(ctx, F_SDPA_FORWARD), strides);
+}
+
+int32_t omx_causal_attention_backward(omx_ctx* ctx, const void* q, uint64_t q_pitch, const void* k, const void* v,
+                                      uint64_t kv_pitch, const void* out, const void* gy, uint64_t out_pitch,
+                                      const void* lse, int32_t operand_dtype, void* gq, void* gk, void* gv,
+                                      int32_t grad_dtype, uint64_t batch, uint64_t time, uint64_t heads,
+                                      uint64_t kv_heads, uint64_t head_dim, uint64_t window) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "causal_attention_backward";
+  if (grad_dtype != OMX_BF16) return omx_fail(ctx, OMX_DTYPE, "%s: gradients must be bf16", op);
+  SdpaShape s;
+  int32_t rc = check_shape(ctx, op, batch, heads, kv_heads, time, head_dim, window, &s);
+  if (rc != OMX_OK) return rc;
+  rc = check_attention(ctx, op, operand_dtype, head_dim, heads, kv_heads, q_pitch, kv_pitch, out_pitch,
+                       {q, k, v, out, gy, lse, gq, gk, gv});
+  if (rc != OMX_OK) return rc;
+  const long D = static_cast<long>(head_dim), T = static_cast<long>(time);
+  const long strides[9] = {static_cast<long>(q_pitch),   D, T * static_cast<long>(q_pitch),
+                           static_cast<long>(kv_pitch),  D, T * static_cast<long>(kv_pitch),
+                           static_cast<long>(out_pitch), D, T * static_cast<long>(out_pitch)};
+  return omx_flash_sdpa_backward(ctx, q, k, v, out, static_cast<const float*>(lse), gy, gq, gk, gv, grad_dtype, batch,
+                                 heads, kv_heads, time, head_dim, s.window, s.scale, omx_tag(ctx, F_SDPA_BACKWARD),
+                                 strides);
 }
 
 }  // extern "C"

@@ -61,6 +61,11 @@ struct ogpt {
   void *gu = nullptr, *gg = nullptr;         // [N,mlp] AD
   void *gq = nullptr, *gk = nullptr, *gv = nullptr, *ga = nullptr;  // [N,d] AD
   void* gy16 = nullptr;                      // AD copy of a residual-stream gradient
+  // bf16 tier with head_dim 64: q, k and v are column blocks of one [N, 3d] projection output
+  // (the three weights are adjacent in the arena, so they are one [3d, d] matrix), attention
+  // runs time-major on those blocks, and their gradients are the blocks of `gqkv`.
+  bool fused_qkv = false;
+  void* gqkv = nullptr;                      // [N,3d] AD
   float *gres = nullptr, *gres1 = nullptr, *gt = nullptr, *gh = nullptr;  // [N,d] f32
   float* g_emb = nullptr;                    // [V,d] f32
   void* ghf = nullptr;                       // [N,d] AD
@@ -124,14 +129,19 @@ int32_t forward(ogpt* t) {
     ogpt::Layer& A = t->layers[l];
     float* x_next = (l + 1 < c.layers) ? t->layers[l + 1].x : t->x_final;
     TRY(omx_rms_norm_forward(ctx, A.x, OMX_F32, t->w32(t->li(l, 0)), A.h1, AD, N, d, eps));
-    TRY(omx_linear_forward(ctx, A.h1, AD, t->w(t->li(l, 1)), AD, t->t_a, AD, N, d, d));
-    TRY(omx_permute_0213(ctx, t->t_a, A.q, AD, B, T, H, D));
-    TRY(omx_linear_forward(ctx, A.h1, AD, t->w(t->li(l, 2)), AD, t->t_a, AD, N, d, d));
-    TRY(omx_permute_0213(ctx, t->t_a, A.k, AD, B, T, H, D));
-    TRY(omx_linear_forward(ctx, A.h1, AD, t->w(t->li(l, 3)), AD, t->t_a, AD, N, d, d));
-    TRY(omx_permute_0213(ctx, t->t_a, A.v, AD, B, T, H, D));
-    TRY(omx_causal_sdpa_forward(ctx, A.q, A.k, A.v, AD, A.a, AD, A.lse, B, H, H, T, D, 0));
-    TRY(omx_permute_0213(ctx, A.a, A.ap, AD, B, H, T, D));
+    if (t->fused_qkv) {
+      TRY(omx_linear_forward(ctx, A.h1, AD, t->w(t->li(l, 1)), AD, A.q, AD, N, d, 3 * d));
+      TRY(omx_causal_attention_forward(ctx, A.q, 3 * d, A.k, A.v, 3 * d, AD, A.ap, d, AD, A.lse, B, T, H, H, D, 0));
+    } else {
+      TRY(omx_linear_forward(ctx, A.h1, AD, t->w(t->li(l, 1)), AD, t->t_a, AD, N, d, d));
+      TRY(omx_permute_0213(ctx, t->t_a, A.q, AD, B, T, H, D));
+      TRY(omx_linear_forward(ctx, A.h1, AD, t->w(t->li(l, 2)), AD, t->t_a, AD, N, d, d));
+      TRY(omx_permute_0213(ctx, t->t_a, A.k, AD, B, T, H, D));
+      TRY(omx_linear_forward(ctx, A.h1, AD, t->w(t->li(l, 3)), AD, t->t_a, AD, N, d, d));
+      TRY(omx_permute_0213(ctx, t->t_a, A.v, AD, B, T, H, D));
+      TRY(omx_causal_sdpa_forward(ctx, A.q, A.k, A.v, AD, A.a, AD, A.lse, B, H, H, T, D, 0));
+      TRY(omx_permute_0213(ctx, A.a, A.ap, AD, B, H, T, D));
+    }
     TRY(omx_linear_forward(ctx, A.ap, AD, t->w(t->li(l, 4)), AD, t->t_a, AD, N, d, d));
     TRY(omx_residual_add(ctx, A.x, OMX_F32, t->t_a, AD, A.x1, OMX_F32, N * d));
     TRY(omx_rms_norm_forward(ctx, A.x1, OMX_F32, t->w32(t->li(l, 5)), A.h2, AD, N, d, eps));
@@ -172,6 +182,19 @@ int32_t backward(ogpt* t) {
     // x1 = x + o(attention)
     TRY(to_operand(t, t->gres1, t->gy16, N * d, &gy));
     TRY(omx_linear_backward(ctx, A.ap, t->w(t->li(l, 4)), gy, AD, t->t_a, AD, t->g(t->li(l, 4)), OMX_F32, N, d, d));
+    if (t->fused_qkv) {
+      char* gq = static_cast<char*>(t->gqkv);
+      TRY(omx_causal_attention_backward(ctx, A.q, 3 * d, A.k, A.v, 3 * d, A.ap, t->t_a, d, A.lse, AD, gq,
+                                        gq + d * t->asz, gq + 2 * d * t->asz, AD, B, T, H, H, D, 0));
+      // One product for the three projections: the input gradient is their sum, formed in the
+      // product's f32 accumulators.
+      TRY(omx_linear_backward(ctx, A.h1, t->w(t->li(l, 1)), t->gqkv, AD, t->t_b, AD, t->g(t->li(l, 1)), OMX_F32, N, d,
+                              3 * d));
+      TRY(omx_rms_norm_backward(ctx, A.x, OMX_F32, t->w32(t->li(l, 0)), t->t_b, AD, t->gt, OMX_F32,
+                                t->g(t->li(l, 0)), N, d, eps));
+      TRY(omx_residual_add(ctx, t->gres1, OMX_F32, t->gt, OMX_F32, t->gres, OMX_F32, N * d));
+      continue;
+    }
     TRY(omx_permute_0213(ctx, t->t_a, t->ga, AD, B, T, H, D));
     TRY(omx_causal_sdpa_backward(ctx, A.q, A.k, A.v, A.a, A.lse, t->ga, AD, t->gq, t->gk, t->gv, AD, B, H, H, T, D, 0));
     // h1 feeds q, k, v; their gradients arrive v first, then k, then q.
@@ -226,6 +249,8 @@ int32_t ogpt_create(omx_ctx* ctx, const ogpt_config* config, ogpt** out) {
     push(d * M);
   }
   push(d);
+  // wq, wk, wv sit back to back when d*d needs no padding.
+  t->fused_qkv = c.bf16 && c.head_dim == 64 && (d * d) % kAlign == 0;
   auto fail = [&](int32_t rc) {
     ogpt_destroy(t);
     return rc;
@@ -261,10 +286,17 @@ int32_t ogpt_create(omx_ctx* ctx, const ogpt_config* config, ogpt** out) {
     CREATE_TRY(alloc_t(t, N * d, &A.x));
     CREATE_TRY(alloc_t(t, N * d, &A.x1));
     CREATE_TRY(alloc_act(t, N * d, &A.h1));
-    CREATE_TRY(alloc_act(t, N * d, &A.q));
-    CREATE_TRY(alloc_act(t, N * d, &A.k));
-    CREATE_TRY(alloc_act(t, N * d, &A.v));
-    CREATE_TRY(alloc_act(t, N * d, &A.a));
+    if (t->fused_qkv) {
+      CREATE_TRY(alloc_act(t, 3 * N * d, &A.q));
+      A.k = static_cast<char*>(A.q) + d * t->asz;
+      A.v = static_cast<char*>(A.q) + 2 * d * t->asz;
+      A.a = nullptr;
+    } else {
+      CREATE_TRY(alloc_act(t, N * d, &A.q));
+      CREATE_TRY(alloc_act(t, N * d, &A.k));
+      CREATE_TRY(alloc_act(t, N * d, &A.v));
+      CREATE_TRY(alloc_act(t, N * d, &A.a));
+    }
     CREATE_TRY(alloc_act(t, N * d, &A.ap));
     CREATE_TRY(alloc_act(t, N * d, &A.h2));
     CREATE_TRY(alloc_act(t, N * M, &A.u));
@@ -279,9 +311,13 @@ int32_t ogpt_create(omx_ctx* ctx, const ogpt_config* config, ogpt** out) {
   CREATE_TRY(alloc_act(t, N * d, &t->t_b));
   CREATE_TRY(alloc_act(t, N * M, &t->gu));
   CREATE_TRY(alloc_act(t, N * M, &t->gg));
-  CREATE_TRY(alloc_act(t, N * d, &t->gq));
-  CREATE_TRY(alloc_act(t, N * d, &t->gk));
-  CREATE_TRY(alloc_act(t, N * d, &t->gv));
+  if (t->fused_qkv) {
+    CREATE_TRY(alloc_act(t, 3 * N * d, &t->gqkv));
+  } else {
+    CREATE_TRY(alloc_act(t, N * d, &t->gq));
+    CREATE_TRY(alloc_act(t, N * d, &t->gk));
+    CREATE_TRY(alloc_act(t, N * d, &t->gv));
+  }
   CREATE_TRY(alloc_act(t, N * d, &t->ga));
   CREATE_TRY(alloc_act(t, N * d, &t->gy16));
   CREATE_TRY(alloc_act(t, N * d, &t->ghf));

@@ -233,6 +233,72 @@ def test_value_residual_blend(be, n, bf16):
         assert abs(float(wl) - exact) <= 1e-5 * max(1.0, abs(exact)) + 6e-8 * n * np.abs(terms).sum()
 
 
+@pytest.mark.parametrize("b,t,h,hkv,window", [(2, 64, 4, 4, None), (1, 257, 6, 2, None), (2, 130, 4, 1, 40),
+                                               (1, 1024, 3, 3, None)])
+def test_time_major_attention_equals_permute_sdpa_permute(be, b, t, h, hkv, window):
+    """ojas-model/src/block.rs:186-199: causal_attention = permute, causal_sdpa, permute back. The
+    fused entry point must give the bits of that composition (same kernels, other strides), also
+    when q, k and v are column blocks of one wider buffer, and match the oracle at the bf16 bar."""
+    from ojas_amd.backend import BF16, DeviceTensor
+
+    print(f"time-major attention b={b} t={t} h={h}/{hkv} window={window}", flush=True)
+    d = 64
+    r = orc.SplitMix64(3100 + t + h)
+    rnd = orc.round_bf16
+    q = rnd(r.vec(b * t * h * d, 1.0)).reshape(b, t, h, d)
+    k = rnd(r.vec(b * t * hkv * d, 1.0)).reshape(b, t, hkv, d)
+    v = rnd(r.vec(b * t * hkv * d, 1.0)).reshape(b, t, hkv, d)
+    gy = rnd(r.vec(b * t * h * d, 1.0)).reshape(b, t, h, d)
+    up = lambda a: be.upload(np.ascontiguousarray(a, np.float32), BF16)
+    dq, dk, dv, dgy = up(q), up(k), up(v), up(gy)
+    out, lse = be.causal_attention_forward(dq, dk, dv, window)
+    gq, gk, gv = be.causal_attention_backward(dq, dk, dv, out, lse, dgy, window)
+    # The composition through the trait's [B, H, T, D] op.
+    qh, kh, vh, gyh = (be.permute(x, [0, 2, 1, 3]) for x in (dq, dk, dv, dgy))
+    out_h, lse_h = be.causal_sdpa_forward(qh, kh, vh, window, BF16)
+    gqh, gkh, gvh = be.causal_sdpa_backward(qh, kh, vh, out_h, lse_h, gyh, window, BF16)
+    assert np.array_equal(be.download(out), be.download(be.permute(out_h, [0, 2, 1, 3])))
+    assert np.array_equal(be.download(lse), be.download(lse_h))
+    for got, want in ((gq, gqh), (gk, gkh), (gv, gvh)):
+        assert np.array_equal(be.download(got), be.download(be.permute(want, [0, 2, 1, 3])))
+    # The oracle, at the bf16 bar.
+    tr = lambda a: np.ascontiguousarray(a.transpose(0, 2, 1, 3))
+    w = window or 0
+    o_out, o_lse = orc.causal_sdpa_forward(tr(q), tr(k), tr(v), w)
+    close(be.download_f32(out), tr(o_out), BF16_TOL, "attention out")
+    close(be.download(lse), o_lse, 1e-3, "attention lse")
+    o_gq, o_gk, o_gv = orc.causal_sdpa_backward(tr(q), tr(k), tr(v), o_out, o_lse, tr(gy), w)
+    for got, want, what in ((gq, o_gq, "gq"), (gk, o_gk, "gk"), (gv, o_gv, "gv")):
+        close(be.download_f32(got), tr(want), BF16_TOL, what)
+    # q | k | v as column blocks of one [B*T, (h + 2 hkv) d] buffer, gradients likewise.
+    width = (h + 2 * hkv) * d
+    packed = np.concatenate([q.reshape(b * t, -1), k.reshape(b * t, -1), v.reshape(b * t, -1)], axis=1)
+    dp = up(packed)
+    dgp = be.zeros((b * t, width), BF16)
+    view = lambda base, col, heads: DeviceTensor(be, base.ptr + col * 2, (b, t, heads, d), BF16, owns=False)
+    pq, pk, pv = view(dp, 0, h), view(dp, h * d, hkv), view(dp, (h + hkv) * d, hkv)
+    out2, lse2 = be.causal_attention_forward(pq, pk, pv, window, pitches=(width, width))
+    assert np.array_equal(be.download(out2), be.download(out)) and np.array_equal(be.download(lse2), be.download(lse))
+    be.causal_attention_backward(pq, pk, pv, out2, lse2, dgy, window, pitches=(width, width),
+                                 grads=(view(dgp, 0, h), view(dgp, h * d, hkv), view(dgp, (h + hkv) * d, hkv)))
+    got = be.download(dgp)
+    want = np.concatenate([be.download(x).reshape(b * t, -1) for x in (gq, gk, gv)], axis=1)
+    assert np.array_equal(got, want)
+
+
+def test_time_major_attention_refuses_other_shapes(be):
+    from ojas_amd.backend import BF16, OjasError
+
+    x = be.upload(np.zeros((1, 8, 2, 32), np.float32), BF16)
+    with pytest.raises(OjasError) as e:
+        be.causal_attention_forward(x, x, x)
+    assert e.value.variant == "Unsupported"
+    y = be.upload(np.zeros((1, 8, 2, 64), np.float32))
+    with pytest.raises(OjasError) as e:
+        be.causal_attention_forward(y, y, y)
+    assert e.value.variant == "Unsupported"
+
+
 def test_value_residual_known_answer_and_nonfinite_lambda(be):
     from ojas_amd.backend import OjasError
 
