@@ -160,6 +160,21 @@ int32_t omx_rms_norm_backward(omx_ctx* ctx, const void* x, int32_t x_dtype, cons
                               const void* gy, int32_t gy_dtype, void* gx, int32_t gx_dtype,
                               void* gw_f32, uint64_t rows, uint64_t dim, float eps);
 
+/* Two-op sequences of the block in one pass over HBM, same bits as the separate calls:
+ *   sum = residual_add_forward(x, y); normed = rms_norm_forward(sum, w)
+ *     (ojas-model/src/block.rs:247-249; sum is f32);
+ *   gx = residual_grad + rms_norm_backward(x, w, gy).gx, the gradient fan-in at
+ *     a residual (ojas-autograd/src/tape.rs:2565-2591); gx is f32, gx_bf16
+ *     (may be null) receives the same values rounded to bf16. */
+int32_t omx_residual_add_rms_norm_forward(omx_ctx* ctx, const void* x, int32_t x_dtype,
+                                          const void* y, int32_t y_dtype, const void* w_f32,
+                                          void* sum_f32, void* normed, int32_t normed_dtype,
+                                          uint64_t rows, uint64_t dim, float eps);
+int32_t omx_rms_norm_backward_residual(omx_ctx* ctx, const void* x, int32_t x_dtype,
+                                       const void* w_f32, const void* gy, int32_t gy_dtype,
+                                       const void* residual_grad_f32, void* gx_f32, void* gx_bf16,
+                                       void* gw_f32, uint64_t rows, uint64_t dim, float eps);
+
 /* ---- BackendModule::cross_entropy_mean_forward / _backward
  *      (backend.rs:2451-2466). loss is one f32 on the device. ---- */
 int32_t omx_cross_entropy_mean_forward(omx_ctx* ctx, const void* logits, int32_t logits_dtype,

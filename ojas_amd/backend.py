@@ -343,6 +343,28 @@ class MiBackend:
                                                     C.c_uint64(dim), C.c_float(eps)))
         return gx, gw
 
+    def residual_add_rms_norm_forward(self, x, y, w, eps: float = 1e-6, out_dtype: Optional[int] = None):
+        """`residual_add_forward` then `rms_norm_forward` in one pass: returns (sum f32, normed)."""
+        dim = x.shape[-1]
+        od = y.dtype if out_dtype is None else out_dtype
+        total, normed = self.empty(x.shape, F32), self.empty(x.shape, od)
+        self._check(self._lib.omx_residual_add_rms_norm_forward(
+            self._ctx, self._p(x), C.c_int32(x.dtype), self._p(y), C.c_int32(y.dtype), self._p(w), self._p(total),
+            self._p(normed), C.c_int32(od), C.c_uint64(x.numel // dim), C.c_uint64(dim), C.c_float(eps)))
+        return total, normed
+
+    def rms_norm_backward_residual(self, x, w, gy, residual_grad, eps: float = 1e-6, want_bf16: bool = False):
+        """`rms_norm_backward` whose input gradient is added to `residual_grad` (f32):
+        returns (gx f32, gx bf16 or None, gw)."""
+        dim = x.shape[-1]
+        gx, gw = self.empty(x.shape, F32), self.empty((dim,), F32)
+        gx16 = self.empty(x.shape, BF16) if want_bf16 else None
+        self._check(self._lib.omx_rms_norm_backward_residual(
+            self._ctx, self._p(x), C.c_int32(x.dtype), self._p(w), self._p(gy), C.c_int32(gy.dtype),
+            self._p(residual_grad), self._p(gx), self._p(gx16), self._p(gw), C.c_uint64(x.numel // dim),
+            C.c_uint64(dim), C.c_float(eps)))
+        return gx, gx16, gw
+
     # ---- loss ----
     @staticmethod
     def _ign(ignore_index):

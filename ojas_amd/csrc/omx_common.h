@@ -8,6 +8,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <initializer_list>
 #include <map>
 #include <string>
 #include <vector>
@@ -104,8 +105,19 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
                       uint64_t b_rs, uint64_t b_cs, int32_t operand_dtype, void* c, int32_t c_dtype, uint64_t ldc,
                       uint64_t m, uint64_t k, uint64_t n, int32_t accumulate);
 // out[c] = sum over b < blocks of partial[b * dim + c], added in a fixed order.
+// `scratch` (OMX_COLUMN_SUM_GROUPS * dim floats, may be null) lets a tall `partial` be added in two stages.
+constexpr int OMX_COLUMN_SUM_GROUPS = 32;
 int32_t omx_column_sum(omx_ctx* ctx, const float* partial, float* out, uint64_t blocks, uint64_t dim,
-                       unsigned long long tag);
+                       unsigned long long tag, float* scratch = nullptr);
+// RMSNorm with 16-byte accesses for row widths 256..1024 (rmsvec.hip). `add` (forward) and
+// `add_in` / `gx16` (backward) are optional fused operands.
+bool omx_rms_vec_eligible(uint64_t dim, std::initializer_list<const void*> ptrs);
+int32_t omx_rms_forward_vec(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* add, int32_t add_dtype,
+                            const float* w, float* sum_out, void* y, int32_t y_dtype, uint64_t rows, uint64_t dim,
+                            float eps, unsigned long long tag);
+int32_t omx_rms_backward_vec(omx_ctx* ctx, const void* x, int32_t x_dtype, const float* w, const void* gy,
+                             int32_t gy_dtype, const float* add_in, void* gx, int32_t gx_dtype, void* gx16, float* gw,
+                             uint64_t rows, uint64_t dim, float eps, unsigned long long tag);
 // Elementwise conversions on the context's stream (no fault reporting).
 int32_t omx_convert(omx_ctx* ctx, const void* src, int32_t src_dtype, void* dst, int32_t dst_dtype, uint64_t n);
 
@@ -179,6 +191,31 @@ __device__ __forceinline__ void dev_store<float>(float* p, size_t i, float v) {
 template <>
 __device__ __forceinline__ void dev_store<unsigned short>(unsigned short* p, size_t i, float v) {
   p[i] = dev_f32_to_bf16_bits(v);
+}
+
+// Four consecutive elements starting at element index i (a multiple of 4; the
+// address must be 16-byte aligned for f32 and 8-byte aligned for bf16).
+template <typename T>
+__device__ __forceinline__ void dev_load4(const T* p, size_t i, float (&v)[4]) {
+  if constexpr (sizeof(T) == 4) {
+    const float4 q = *reinterpret_cast<const float4*>(p + i);
+    v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+  } else {
+    const uint2 q = *reinterpret_cast<const uint2*>(p + i);
+    v[0] = __uint_as_float(q.x << 16); v[1] = __uint_as_float(q.x & 0xffff0000u);
+    v[2] = __uint_as_float(q.y << 16); v[3] = __uint_as_float(q.y & 0xffff0000u);
+  }
+}
+template <typename T>
+__device__ __forceinline__ void dev_store4(T* p, size_t i, const float (&v)[4]) {
+  if constexpr (sizeof(T) == 4) {
+    *reinterpret_cast<float4*>(p + i) = make_float4(v[0], v[1], v[2], v[3]);
+  } else {
+    uint2 q;
+    q.x = static_cast<unsigned>(dev_f32_to_bf16_bits(v[0])) | (static_cast<unsigned>(dev_f32_to_bf16_bits(v[1])) << 16);
+    q.y = static_cast<unsigned>(dev_f32_to_bf16_bits(v[2])) | (static_cast<unsigned>(dev_f32_to_bf16_bits(v[3])) << 16);
+    *reinterpret_cast<uint2*>(p + i) = q;
+  }
 }
 
 __device__ __forceinline__ float wave_sum(float v) {

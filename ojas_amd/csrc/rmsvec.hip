@@ -1,0 +1,301 @@
+// RMSNorm for row widths 256..1024 with 16-byte accesses, optionally fused with
+// the residual add in front of it (forward) or behind it (backward).
+//
+// Reference semantics: ojas-cpu/src/norm.rs:24-204 (rms_norm_forward /
+// _backward, trait backend.rs:1658-1672) and ojas-cpu/src/accum.rs:31-106
+// (residual_add_forward). The fused forms are the two-op sequences of
+// ojas-model/src/block.rs:247-249 (x = add(x, o); h = rms_norm(x)) and of the
+// tape's gradient fan-in at a residual (ojas-autograd/src/tape.rs:2565-2591:
+// grad_x = grad_from_add + grad_from_norm), with the same arithmetic per
+// element as the separate kernels, so the results are the same bits.
+//
+// One wave owns a row; lane l owns columns 256 j + 4 l .. + 3 of chunk j, so a
+// wave's loads are contiguous 1 KiB (f32) runs and the row stays in registers
+// between the sum-of-squares pass and the scaling pass.
+#include "omx_common.h"
+
+namespace {
+
+constexpr int RV_THREADS = 256;
+
+template <typename TX, typename TA, typename TY, int NCH>
+__global__ __launch_bounds__(RV_THREADS) void rms_fwd_vec_kernel(const TX* __restrict__ x, const TA* __restrict__ add,
+                                                                 const float* __restrict__ w,
+                                                                 float* __restrict__ sum_out, TY* __restrict__ y,
+                                                                 size_t rows, int dim, float eps, OmxFaultWord* fault,
+                                                                 unsigned long long tag) {
+  const int lane = threadIdx.x & 63;
+  const size_t row = static_cast<size_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const size_t base = row * dim;
+  float xv[NCH][4];
+  float ss = 0.0f;
+  bool bad = false;
+#pragma unroll
+  for (int j = 0; j < NCH; ++j) {
+    const int c = j * 256 + lane * 4;
+    if (c < dim) {
+      dev_load4<TX>(x, base + c, xv[j]);
+      if (add) {
+        float av[4];
+        dev_load4<TA>(add, base + c, av);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          xv[j][e] = xv[j][e] + av[e];
+          bad |= !dev_finite(xv[j][e]);
+        }
+        dev_store4<float>(sum_out, base + c, xv[j]);
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) xv[j][e] = 0.0f;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) ss += xv[j][e] * xv[j][e];
+  }
+  ss = wave_sum(ss);
+  const float denom = ss / static_cast<float>(dim) + eps;
+  const float rstd = 1.0f / sqrtf(denom);
+  bad |= !(dev_finite(denom) && denom > 0.0f && dev_finite(rstd));
+#pragma unroll
+  for (int j = 0; j < NCH; ++j) {
+    const int c = j * 256 + lane * 4;
+    if (c < dim) {
+      float wv[4], out[4];
+      dev_load4<float>(w, c, wv);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        out[e] = xv[j][e] * rstd * wv[e];
+        bad |= !dev_finite(out[e]);
+      }
+      dev_store4<TY>(y, base + c, out);
+    }
+  }
+  if (bad) dev_raise_fault(fault, tag);
+}
+
+// gx = rms_norm_backward(x, w, gy) (+ add_in), optionally also stored as bf16;
+// per-block partial column sums of gy * xhat for the weight gradient.
+template <typename TX, typename TG, typename TO, int NCH>
+__global__ __launch_bounds__(RV_THREADS) void rms_bwd_vec_kernel(
+    const TX* __restrict__ x, const float* __restrict__ w, const TG* __restrict__ gy, const float* __restrict__ add_in,
+    TO* __restrict__ gx, unsigned short* __restrict__ gx16, float* __restrict__ partial, size_t rows, int dim,
+    float eps, int rows_per_block, OmxFaultWord* fault, unsigned long long tag) {
+  extern __shared__ float lds[];  // [4][dim]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const float inv_dim = 1.0f / static_cast<float>(dim);
+  float wv[NCH][4], accw[NCH][4];
+#pragma unroll
+  for (int j = 0; j < NCH; ++j) {
+    const int c = j * 256 + lane * 4;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      wv[j][e] = 0.0f;
+      accw[j][e] = 0.0f;
+    }
+    if (c < dim) dev_load4<float>(w, c, wv[j]);
+  }
+  bool bad = false;
+  const size_t first = static_cast<size_t>(blockIdx.x) * rows_per_block;
+  const size_t last = min(rows, first + rows_per_block);
+  for (size_t row = first + wave; row < last; row += 4) {
+    const size_t base = row * dim;
+    float xv[NCH][4], gv[NCH][4];
+    float ss = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+      const int c = j * 256 + lane * 4;
+      if (c < dim) {
+        dev_load4<TX>(x, base + c, xv[j]);
+        dev_load4<TG>(gy, base + c, gv[j]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          xv[j][e] = 0.0f;
+          gv[j][e] = 0.0f;
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ss += xv[j][e] * xv[j][e];
+    }
+    ss = wave_sum(ss);
+    const float denom = ss * inv_dim + eps;
+    const float rstd = 1.0f / sqrtf(denom);
+    bad |= !(dev_finite(denom) && denom > 0.0f && dev_finite(rstd));
+    float dot = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NCH; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) dot += (gv[j][e] * wv[j][e]) * (xv[j][e] * rstd);
+    dot = wave_sum(dot);
+    const float mean = dot * inv_dim;
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+      const int c = j * 256 + lane * 4;
+      float out[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float xhat = xv[j][e] * rstd;
+        out[e] = (gv[j][e] * wv[j][e] - xhat * mean) * rstd;
+        accw[j][e] += gv[j][e] * xhat;
+      }
+      if (c < dim) {
+        if (add_in) {
+          float av[4];
+          dev_load4<float>(add_in, base + c, av);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) out[e] = av[e] + out[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) bad |= !dev_finite(out[e]);
+        dev_store4<TO>(gx, base + c, out);
+        if (gx16) dev_store4<unsigned short>(gx16, base + c, out);
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < NCH; ++j) {
+    const int c = j * 256 + lane * 4;
+    if (c < dim) dev_store4<float>(lds, static_cast<size_t>(wave) * dim + c, accw[j]);
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < dim; c += RV_THREADS) {
+    float s = ((lds[c] + lds[dim + c]) + lds[2 * dim + c]) + lds[3 * dim + c];
+    partial[static_cast<size_t>(blockIdx.x) * dim + c] = s;
+  }
+  if (bad) dev_raise_fault(fault, tag);
+}
+
+bool aligned16(std::initializer_list<const void*> ptrs) {
+  uintptr_t bits = 0;
+  for (const void* p : ptrs) bits |= reinterpret_cast<uintptr_t>(p);
+  return (bits & 15u) == 0;
+}
+
+}  // namespace
+
+bool omx_rms_vec_eligible(uint64_t dim, std::initializer_list<const void*> ptrs) {
+  return dim % 4 == 0 && dim >= 256 && dim <= 1024 && aligned16(ptrs);
+}
+
+int32_t omx_rms_forward_vec(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* add, int32_t add_dtype,
+                            const float* w, float* sum_out, void* y, int32_t y_dtype, uint64_t rows, uint64_t dim,
+                            float eps, unsigned long long tag) {
+  dim3 grid(static_cast<unsigned>((rows + 3) / 4)), block(RV_THREADS);
+  const int nch = static_cast<int>((dim + 255) / 256);
+  typedef unsigned short h16;
+#define RV_FWD(TX, TA, TY, N)                                                                                   \
+  hipLaunchKernelGGL((rms_fwd_vec_kernel<TX, TA, TY, N>), grid, block, 0, ctx->stream, static_cast<const TX*>(x), \
+                     static_cast<const TA*>(add), w, sum_out, static_cast<TY*>(y), static_cast<size_t>(rows),   \
+                     static_cast<int>(dim), eps, ctx->fault, tag)
+#define RV_FWD_N(TX, TA, TY)      \
+  switch (nch) {                  \
+    case 1: RV_FWD(TX, TA, TY, 1); break; \
+    case 2: RV_FWD(TX, TA, TY, 2); break; \
+    case 3: RV_FWD(TX, TA, TY, 3); break; \
+    default: RV_FWD(TX, TA, TY, 4); break; \
+  }
+  const int key = (x_dtype == OMX_BF16 ? 4 : 0) | (add && add_dtype == OMX_BF16 ? 2 : 0) | (y_dtype == OMX_BF16 ? 1 : 0);
+  switch (key) {
+    case 0: RV_FWD_N(float, float, float) break;
+    case 1: RV_FWD_N(float, float, h16) break;
+    case 2: RV_FWD_N(float, h16, float) break;
+    case 3: RV_FWD_N(float, h16, h16) break;
+    case 4: RV_FWD_N(h16, float, float) break;
+    case 5: RV_FWD_N(h16, float, h16) break;
+    case 6: RV_FWD_N(h16, h16, float) break;
+    default: RV_FWD_N(h16, h16, h16) break;
+  }
+#undef RV_FWD_N
+#undef RV_FWD
+  OMX_LAUNCH_CHECK(ctx, "rms_fwd_vec_kernel");
+  return OMX_OK;
+}
+
+int32_t omx_rms_backward_vec(omx_ctx* ctx, const void* x, int32_t x_dtype, const float* w, const void* gy,
+                             int32_t gy_dtype, const float* add_in, void* gx, int32_t gx_dtype, void* gx16, float* gw,
+                             uint64_t rows, uint64_t dim, float eps, unsigned long long tag) {
+  // Two rows per wave: enough blocks in flight to hide the row's load latency.
+  const int rows_per_block = 8;
+  const uint64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
+  void* ws = nullptr;
+  int32_t rc = omx_workspace(ctx, (blocks + OMX_COLUMN_SUM_GROUPS) * dim * sizeof(float), &ws);
+  if (rc != OMX_OK) return rc;
+  float* partial = static_cast<float*>(ws);
+  float* scratch = partial + blocks * dim;
+  dim3 grid(static_cast<unsigned>(blocks)), block(RV_THREADS);
+  const size_t smem = 4 * dim * sizeof(float);
+  const int nch = static_cast<int>((dim + 255) / 256);
+  typedef unsigned short h16;
+#define RV_BWD(TX, TG, TO, N)                                                                                       \
+  hipLaunchKernelGGL((rms_bwd_vec_kernel<TX, TG, TO, N>), grid, block, smem, ctx->stream, static_cast<const TX*>(x), \
+                     w, static_cast<const TG*>(gy), add_in, static_cast<TO*>(gx), static_cast<h16*>(gx16), partial, \
+                     static_cast<size_t>(rows), static_cast<int>(dim), eps, rows_per_block, ctx->fault, tag)
+#define RV_BWD_N(TX, TG, TO)      \
+  switch (nch) {                  \
+    case 1: RV_BWD(TX, TG, TO, 1); break; \
+    case 2: RV_BWD(TX, TG, TO, 2); break; \
+    case 3: RV_BWD(TX, TG, TO, 3); break; \
+    default: RV_BWD(TX, TG, TO, 4); break; \
+  }
+  const int key = (x_dtype == OMX_BF16 ? 4 : 0) | (gy_dtype == OMX_BF16 ? 2 : 0) | (gx_dtype == OMX_BF16 ? 1 : 0);
+  switch (key) {
+    case 0: RV_BWD_N(float, float, float) break;
+    case 1: RV_BWD_N(float, float, h16) break;
+    case 2: RV_BWD_N(float, h16, float) break;
+    case 3: RV_BWD_N(float, h16, h16) break;
+    case 4: RV_BWD_N(h16, float, float) break;
+    case 5: RV_BWD_N(h16, float, h16) break;
+    case 6: RV_BWD_N(h16, h16, float) break;
+    default: RV_BWD_N(h16, h16, h16) break;
+  }
+#undef RV_BWD_N
+#undef RV_BWD
+  OMX_LAUNCH_CHECK(ctx, "rms_bwd_vec_kernel");
+  return omx_column_sum(ctx, partial, gw, blocks, dim, tag, scratch);
+}
+
+extern "C" {
+
+int32_t omx_residual_add_rms_norm_forward(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* y, int32_t y_dtype,
+                                          const void* w, void* sum_out, void* normed, int32_t normed_dtype,
+                                          uint64_t rows, uint64_t dim, float eps) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "residual_add_rms_norm_forward";
+  if (!x || !y || !w || !sum_out || !normed) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  if (!omx_valid_float_dtype(x_dtype) || !omx_valid_float_dtype(y_dtype) || !omx_valid_float_dtype(normed_dtype))
+    return omx_fail(ctx, OMX_DTYPE, "%s: dtype must be f32 or bf16", op);
+  if (rows == 0 || dim == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
+  if (!(eps == eps) || eps == INFINITY || eps == -INFINITY) return omx_fail(ctx, OMX_NON_FINITE, "%s", op);
+  if (omx_rms_vec_eligible(dim, {x, y, w, sum_out, normed}))
+    return omx_rms_forward_vec(ctx, x, x_dtype, y, y_dtype, static_cast<const float*>(w), static_cast<float*>(sum_out),
+                               normed, normed_dtype, rows, dim, eps, omx_tag(ctx, F_RMS_FORWARD));
+  int32_t rc = omx_residual_add(ctx, x, x_dtype, y, y_dtype, sum_out, OMX_F32, rows * dim);
+  if (rc != OMX_OK) return rc;
+  return omx_rms_norm_forward(ctx, sum_out, OMX_F32, w, normed, normed_dtype, rows, dim, eps);
+}
+
+int32_t omx_rms_norm_backward_residual(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* w, const void* gy,
+                                       int32_t gy_dtype, const void* residual_grad, void* gx, void* gx_bf16, void* gw,
+                                       uint64_t rows, uint64_t dim, float eps) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "rms_norm_backward_residual";
+  if (!x || !w || !gy || !residual_grad || !gx || !gw) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  if (!omx_valid_float_dtype(x_dtype) || !omx_valid_float_dtype(gy_dtype))
+    return omx_fail(ctx, OMX_DTYPE, "%s: dtype must be f32 or bf16", op);
+  if (rows == 0 || dim == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
+  if (!(eps == eps) || eps == INFINITY || eps == -INFINITY) return omx_fail(ctx, OMX_NON_FINITE, "%s", op);
+  if (omx_rms_vec_eligible(dim, {x, w, gy, residual_grad, gx, gx_bf16, gw}))
+    return omx_rms_backward_vec(ctx, x, x_dtype, static_cast<const float*>(w), gy, gy_dtype,
+                                static_cast<const float*>(residual_grad), gx, OMX_F32, gx_bf16,
+                                static_cast<float*>(gw), rows, dim, eps, omx_tag(ctx, F_RMS_BACKWARD));
+  // Other widths: the same three steps as separate kernels (gx is written, then added in place).
+  int32_t rc = omx_rms_norm_backward(ctx, x, x_dtype, w, gy, gy_dtype, gx, OMX_F32, gw, rows, dim, eps);
+  if (rc != OMX_OK) return rc;
+  rc = omx_residual_add(ctx, residual_grad, OMX_F32, gx, OMX_F32, gx, OMX_F32, rows * dim);
+  if (rc != OMX_OK) return rc;
+  if (gx_bf16) return omx_to_bf16(ctx, gx, gx_bf16, rows * dim);
+  return OMX_OK;
+}
+
+}  // extern "C"

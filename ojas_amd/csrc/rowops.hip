@@ -137,6 +137,24 @@ __global__ __launch_bounds__(256) void column_sum_kernel(const float* __restrict
   }
 }
 
+// Stage 1 of a tall column sum: block (x, g) adds rows [g * per_group, (g + 1) * per_group) of its
+// 64 columns, four row groups in parallel, then a fixed four-way sum.
+__global__ __launch_bounds__(256) void column_sum_groups_kernel(const float* __restrict__ partial,
+                                                                float* __restrict__ scratch, int blocks, int dim,
+                                                                int per_group) {
+  __shared__ float red[4][64];
+  const int lane = threadIdx.x & 63, group = threadIdx.x >> 6;
+  const int c = blockIdx.x * 64 + lane;
+  const int first = blockIdx.y * per_group, last = min(blocks, first + per_group);
+  float s = 0.0f;
+  if (c < dim)
+    for (int b = first + group; b < last; b += 4) s += partial[static_cast<size_t>(b) * dim + c];
+  red[group][lane] = s;
+  __syncthreads();
+  if (group == 0 && c < dim)
+    scratch[static_cast<size_t>(blockIdx.y) * dim + c] = ((red[0][lane] + red[1][lane]) + red[2][lane]) + red[3][lane];
+}
+
 // ---------------------------------------------------------------- embedding
 template <typename TT, typename TO>
 __global__ void embedding_fwd_kernel(const TT* __restrict__ table, const unsigned int* __restrict__ ids,
@@ -421,6 +439,8 @@ int32_t rms_forward_impl(omx_ctx* ctx, const char* op, uint32_t fault_op, const 
   unsigned long long tag = omx_tag(ctx, fault_op);
   (void)op;
   const float* wf = static_cast<const float*>(w);
+  if (omx_rms_vec_eligible(dim, {x, w, y}))
+    return omx_rms_forward_vec(ctx, x, x_dtype, nullptr, OMX_F32, wf, nullptr, y, y_dtype, rows, dim, eps, tag);
   if (x_dtype == OMX_F32 && y_dtype == OMX_F32) return launch_rms_fwd<float, float>(ctx, x, wf, y, rows, dim, eps, tag);
   if (x_dtype == OMX_F32) return launch_rms_fwd<float, unsigned short>(ctx, x, wf, y, rows, dim, eps, tag);
   if (y_dtype == OMX_F32) return launch_rms_fwd<unsigned short, float>(ctx, x, wf, y, rows, dim, eps, tag);
@@ -433,6 +453,9 @@ int32_t rms_backward_impl(omx_ctx* ctx, uint32_t fault_op, const void* x, int32_
   unsigned long long tag = omx_tag(ctx, fault_op);
   const float* wf = static_cast<const float*>(w);
   float* gwf = static_cast<float*>(gw);
+  if (omx_rms_vec_eligible(dim, {x, w, gy, gx, gw}))
+    return omx_rms_backward_vec(ctx, x, x_dtype, wf, gy, gy_dtype, nullptr, gx, gx_dtype, nullptr, gwf, rows, dim, eps,
+                                tag);
   typedef unsigned short h16;
   const int key = (x_dtype == OMX_BF16 ? 4 : 0) | (gy_dtype == OMX_BF16 ? 2 : 0) | (gx_dtype == OMX_BF16 ? 1 : 0);
   switch (key) {
@@ -452,9 +475,19 @@ bool finite_host(float v) { return v == v && v != INFINITY && v != -INFINITY; }
 }  // namespace
 
 int32_t omx_column_sum(omx_ctx* ctx, const float* partial, float* out, uint64_t blocks, uint64_t dim,
-                       unsigned long long tag) {
-  hipLaunchKernelGGL(column_sum_kernel, dim3(static_cast<unsigned>((dim + 63) / 64)), dim3(256), 0, ctx->stream, partial,
-                     out, static_cast<int>(blocks), static_cast<int>(dim), ctx->fault, tag);
+                       unsigned long long tag, float* scratch) {
+  const unsigned col_blocks = static_cast<unsigned>((dim + 63) / 64);
+  if (scratch && blocks > 4 * OMX_COLUMN_SUM_GROUPS) {
+    // Stage 1: group g adds its contiguous share of the rows into scratch[g]; stage 2 adds the groups.
+    const int per_group = static_cast<int>((blocks + OMX_COLUMN_SUM_GROUPS - 1) / OMX_COLUMN_SUM_GROUPS);
+    hipLaunchKernelGGL(column_sum_groups_kernel, dim3(col_blocks, OMX_COLUMN_SUM_GROUPS), dim3(256), 0, ctx->stream,
+                       partial, scratch, static_cast<int>(blocks), static_cast<int>(dim), per_group);
+    OMX_LAUNCH_CHECK(ctx, "column_sum_groups_kernel");
+    partial = scratch;
+    blocks = OMX_COLUMN_SUM_GROUPS;
+  }
+  hipLaunchKernelGGL(column_sum_kernel, dim3(col_blocks), dim3(256), 0, ctx->stream, partial, out,
+                     static_cast<int>(blocks), static_cast<int>(dim), ctx->fault, tag);
   OMX_LAUNCH_CHECK(ctx, "column_sum_kernel");
   return OMX_OK;
 }

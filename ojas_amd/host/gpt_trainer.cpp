@@ -123,12 +123,20 @@ int32_t forward(ogpt* t) {
   const float eps = 1e-6f;
   TRY(omx_embedding_forward(ctx, t->w32(0), OMX_F32, t->ids, t->e_tok, OMX_F32, N, c.vocab, d));
   TRY(omx_embedding_forward(ctx, t->w32(1), OMX_F32, t->positions, t->e_pos, OMX_F32, N, T, d));
-  float* x = t->layers.empty() ? t->x_final : t->layers[0].x;
-  TRY(omx_residual_add(ctx, t->e_tok, OMX_F32, t->e_pos, OMX_F32, x, OMX_F32, N * d));
+  // Every residual add is fused with the norm that reads its sum: the sum (f32 residual stream)
+  // and the normed operand leave one kernel.
+  {
+    float* x = t->layers.empty() ? t->x_final : t->layers[0].x;
+    void* h = t->layers.empty() ? t->hf : t->layers[0].h1;
+    const float* nw = t->w32(t->layers.empty() ? t->nf() : t->li(0, 0));
+    TRY(omx_residual_add_rms_norm_forward(ctx, t->e_tok, OMX_F32, t->e_pos, OMX_F32, nw, x, h, AD, N, d, eps));
+  }
   for (uint32_t l = 0; l < c.layers; ++l) {
     ogpt::Layer& A = t->layers[l];
-    float* x_next = (l + 1 < c.layers) ? t->layers[l + 1].x : t->x_final;
-    TRY(omx_rms_norm_forward(ctx, A.x, OMX_F32, t->w32(t->li(l, 0)), A.h1, AD, N, d, eps));
+    const bool last = l + 1 == c.layers;
+    float* x_next = last ? t->x_final : t->layers[l + 1].x;
+    void* h_next = last ? t->hf : t->layers[l + 1].h1;
+    const float* next_norm = t->w32(last ? t->nf() : t->li(l + 1, 0));
     if (t->fused_qkv) {
       TRY(omx_linear_forward(ctx, A.h1, AD, t->w(t->li(l, 1)), AD, A.q, AD, N, d, 3 * d));
       TRY(omx_causal_attention_forward(ctx, A.q, 3 * d, A.k, A.v, 3 * d, AD, A.ap, d, AD, A.lse, B, T, H, H, D, 0));
@@ -143,14 +151,13 @@ int32_t forward(ogpt* t) {
       TRY(omx_permute_0213(ctx, A.a, A.ap, AD, B, H, T, D));
     }
     TRY(omx_linear_forward(ctx, A.ap, AD, t->w(t->li(l, 4)), AD, t->t_a, AD, N, d, d));
-    TRY(omx_residual_add(ctx, A.x, OMX_F32, t->t_a, AD, A.x1, OMX_F32, N * d));
-    TRY(omx_rms_norm_forward(ctx, A.x1, OMX_F32, t->w32(t->li(l, 5)), A.h2, AD, N, d, eps));
+    TRY(omx_residual_add_rms_norm_forward(ctx, A.x, OMX_F32, t->t_a, AD, t->w32(t->li(l, 5)), A.x1, A.h2, AD, N, d,
+                                          eps));
     TRY(omx_linear_forward(ctx, A.h2, AD, t->w(t->li(l, 6)), AD, A.u, AD, N, d, M));
     TRY(omx_gelu_forward(ctx, A.u, A.g, AD, N * M, c.gelu_tanh));
     TRY(omx_linear_forward(ctx, A.g, AD, t->w(t->li(l, 7)), AD, t->t_a, AD, N, M, d));
-    TRY(omx_residual_add(ctx, A.x1, OMX_F32, t->t_a, AD, x_next, OMX_F32, N * d));
+    TRY(omx_residual_add_rms_norm_forward(ctx, A.x1, OMX_F32, t->t_a, AD, next_norm, x_next, h_next, AD, N, d, eps));
   }
-  TRY(omx_rms_norm_forward(ctx, t->x_final, OMX_F32, t->w32(t->nf()), t->hf, AD, N, d, eps));
   return OMX_OK;
 }
 
@@ -167,20 +174,22 @@ int32_t backward(ogpt* t) {
                                     t->loss, t->ghf, AD, t->g(0)));
   TRY(omx_rms_norm_backward(ctx, t->x_final, OMX_F32, t->w32(t->nf()), t->ghf, AD, t->gres, OMX_F32, t->g(t->nf()), N, d,
                             eps));
+  // `gy` is the residual-stream gradient as a GEMM operand: gres itself on the f32 tier, its bf16
+  // copy (written by the kernel that produced gres) on the bf16 tier.
+  const void* gy = nullptr;
+  TRY(to_operand(t, t->gres, t->gy16, N * d, &gy));
+  void* copy16 = AD == OMX_BF16 ? t->gy16 : nullptr;
   for (uint32_t l = c.layers; l-- > 0;) {
     ogpt::Layer& A = t->layers[l];
-    const void* gy = nullptr;
     // x_next = x1 + down(gelu(up(norm2(x1))))
-    TRY(to_operand(t, t->gres, t->gy16, N * d, &gy));
     TRY(omx_linear_backward(ctx, A.g, t->w(t->li(l, 7)), gy, AD, t->gg, AD, t->g(t->li(l, 7)), OMX_F32, N, M, d));
     TRY(omx_gelu_backward(ctx, A.u, t->gg, t->gu, AD, N * M, c.gelu_tanh));
     TRY(omx_linear_backward(ctx, A.h2, t->w(t->li(l, 6)), t->gu, AD, t->t_a, AD, t->g(t->li(l, 6)), OMX_F32, N, d, M));
-    TRY(omx_rms_norm_backward(ctx, A.x1, OMX_F32, t->w32(t->li(l, 5)), t->t_a, AD, t->gt, OMX_F32, t->g(t->li(l, 5)), N,
-                              d, eps));
     // Fan-in at x1: the residual branch arrives first, then the norm branch.
-    TRY(omx_residual_add(ctx, t->gres, OMX_F32, t->gt, OMX_F32, t->gres1, OMX_F32, N * d));
+    TRY(omx_rms_norm_backward_residual(ctx, A.x1, OMX_F32, t->w32(t->li(l, 5)), t->t_a, AD, t->gres, t->gres1, copy16,
+                                       t->g(t->li(l, 5)), N, d, eps));
+    gy = AD == OMX_BF16 ? static_cast<const void*>(t->gy16) : static_cast<const void*>(t->gres1);
     // x1 = x + o(attention)
-    TRY(to_operand(t, t->gres1, t->gy16, N * d, &gy));
     TRY(omx_linear_backward(ctx, A.ap, t->w(t->li(l, 4)), gy, AD, t->t_a, AD, t->g(t->li(l, 4)), OMX_F32, N, d, d));
     if (t->fused_qkv) {
       char* gq = static_cast<char*>(t->gqkv);
@@ -190,9 +199,9 @@ int32_t backward(ogpt* t) {
       // product's f32 accumulators.
       TRY(omx_linear_backward(ctx, A.h1, t->w(t->li(l, 1)), t->gqkv, AD, t->t_b, AD, t->g(t->li(l, 1)), OMX_F32, N, d,
                               3 * d));
-      TRY(omx_rms_norm_backward(ctx, A.x, OMX_F32, t->w32(t->li(l, 0)), t->t_b, AD, t->gt, OMX_F32,
-                                t->g(t->li(l, 0)), N, d, eps));
-      TRY(omx_residual_add(ctx, t->gres1, OMX_F32, t->gt, OMX_F32, t->gres, OMX_F32, N * d));
+      TRY(omx_rms_norm_backward_residual(ctx, A.x, OMX_F32, t->w32(t->li(l, 0)), t->t_b, AD, t->gres1, t->gres, copy16,
+                                         t->g(t->li(l, 0)), N, d, eps));
+      gy = AD == OMX_BF16 ? static_cast<const void*>(t->gy16) : static_cast<const void*>(t->gres);
       continue;
     }
     TRY(omx_permute_0213(ctx, t->t_a, t->ga, AD, B, T, H, D));
@@ -206,9 +215,9 @@ int32_t backward(ogpt* t) {
     TRY(omx_permute_0213(ctx, t->gq, t->t_a, AD, B, H, T, D));
     TRY(omx_linear_backward(ctx, A.h1, t->w(t->li(l, 1)), t->t_a, AD, t->ga, AD, t->g(t->li(l, 1)), OMX_F32, N, d, d));
     TRY(omx_residual_add(ctx, t->gh, OMX_F32, t->ga, AD, t->gh, OMX_F32, N * d));
-    TRY(omx_rms_norm_backward(ctx, A.x, OMX_F32, t->w32(t->li(l, 0)), t->gh, OMX_F32, t->gt, OMX_F32,
-                              t->g(t->li(l, 0)), N, d, eps));
-    TRY(omx_residual_add(ctx, t->gres1, OMX_F32, t->gt, OMX_F32, t->gres, OMX_F32, N * d));
+    TRY(omx_rms_norm_backward_residual(ctx, A.x, OMX_F32, t->w32(t->li(l, 0)), t->gh, OMX_F32, t->gres1, t->gres, copy16,
+                                       t->g(t->li(l, 0)), N, d, eps));
+    gy = AD == OMX_BF16 ? static_cast<const void*>(t->gy16) : static_cast<const void*>(t->gres);
   }
   // x0 = tok[ids] + pos[positions]; the tied table adds the embedding's share to the head's.
   TRY(omx_embedding_backward(ctx, t->positions, t->gres, OMX_F32, t->g(1), N, T, d));

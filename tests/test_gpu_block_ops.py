@@ -286,6 +286,45 @@ def test_time_major_attention_equals_permute_sdpa_permute(be, b, t, h, hkv, wind
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("rows,dim", [(5, 256), (33, 768), (1000, 768), (17, 1024), (9, 260), (40, 96), (12, 2048)])
+def test_fused_residual_rms_norm_equals_the_separate_ops(be, rows, dim, bf16):
+    """block.rs:247-249 (add, then norm) and the tape's fan-in at a residual: the fused entry points
+    must give the bits of the separate calls, and the norm itself must match the oracle."""
+    from ojas_amd.backend import BF16, F32
+
+    print(f"fused add+rms rows={rows} dim={dim} bf16={bf16}", flush=True)
+    up, tol, rnd = tier(be, bf16)
+    r = orc.SplitMix64(5100 + rows + dim)
+    x = r.vec(rows * dim, 1.0).reshape(rows, dim)
+    y = rnd(r.vec(rows * dim, 1.0)).reshape(rows, dim)
+    w = 1.0 + r.vec(dim, 0.1)
+    gy = rnd(r.vec(rows * dim, 1.0)).reshape(rows, dim)
+    res = r.vec(rows * dim, 1.0).reshape(rows, dim)
+    dx, dy, dw, dgy, dres = be.upload(x), up(y), be.upload(w), up(gy), be.upload(res)
+    od = BF16 if bf16 else F32
+    total, normed = be.residual_add_rms_norm_forward(dx, dy, dw, 1e-6, od)
+    total2 = be.residual_add_forward(dx, dy, F32)
+    normed2 = be.rms_norm_forward(total2, dw, 1e-6, od)
+    assert np.array_equal(be.download(total), be.download(total2))
+    assert np.array_equal(be.download(normed), be.download(normed2))
+    want_sum = orc.residual_add(x, y)
+    close(be.download(total), want_sum, F32_TOL, "sum")
+    close(be.download_f32(normed), orc.rms_norm_forward(want_sum, w, 1e-6), tol, "normed")
+    gx, gx16, gw = be.rms_norm_backward_residual(dx, dw, dgy, dres, 1e-6, want_bf16=True)
+    gx_plain, gw_plain = be.rms_norm_backward(dx, dw, dgy, 1e-6)
+    o_gx, o_gw = orc.rms_norm_backward(x, w, gy, 1e-6)
+    close(be.download(gx), res + o_gx, max(tol, 2e-5), "gx + residual")
+    close(be.download_f32(gx16), res + o_gx, BF16_TOL, "gx bf16 copy")
+    assert np.array_equal(be.download(gx16), orc.to_bf16(be.download(gx)))
+    close(be.download(gw), o_gw, max(tol, 3e-5), "gw")
+    assert np.array_equal(be.download(gw), be.download(gw_plain))
+    if not bf16:
+        # f32 gradients: the fused sum is the separate kernels' f32 add of the same two values.
+        sep = be.residual_add_forward(dres, gx_plain, F32)
+        assert np.array_equal(be.download(gx), be.download(sep))
+
+
 def test_time_major_attention_refuses_other_shapes(be):
     from ojas_amd.backend import BF16, OjasError
 
