@@ -55,8 +55,13 @@ __device__ __forceinline__ void issue_tile(const unsigned short* __restrict__ p,
       gm = gm + 8 <= rows ? gm : 0;
       src = p + static_cast<long>(k0 + kr) * ld + gm;
     }
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                     (__attribute__((address_space(3))) void*)(tile + q * 1024), 16, 0, 0);
+    // Written as assembly: the compiler cannot tell that this asynchronous LDS write targets the
+    // stage that is NOT being read, and would otherwise make every LDS read wait for it (vmcnt(0)
+    // right after the issue), which serialises the loads with the products.
+    const unsigned lds_at = static_cast<unsigned>(reinterpret_cast<uintptr_t>(tile + q * 1024));
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src),
+                 "s"(__builtin_amdgcn_readfirstlane(lds_at))
+                 : "memory");
   }
 }
 
