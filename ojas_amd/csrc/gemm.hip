@@ -457,15 +457,14 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
   int dma_variant = -1;
   if (operand_dtype == OMX_BF16 && omx_gemm_dma_eligible(g, a_km, b_km)) {
     const int mode = ctx->gemm_dma_mode;
-    const long t0 = static_cast<long>((g.M + 255) / 256) * ((g.N + 255) / 256);
-    const long t1 = static_cast<long>((g.M + 255) / 256) * ((g.N + 127) / 128);
     if (mode == 1) {
       // Measured on the GPT shapes: small outputs (the d x d weight gradients, the
-      // Newton-Schulz squares) stay on the 128 x 128 kernel; a narrow output with a
-      // long reduction fills the chip better with 256 x 128 tiles; the rest takes 256 x 256.
+      // Newton-Schulz squares) stay on the 128 x 128 kernel; everything else takes 256 x 128
+      // tiles, which leave room for two workgroups per compute unit, so one's output stores and
+      // first loads overlap the other's products (256 x 256 halves the L2 traffic per FLOP but
+      // runs alone on its compute unit and measures slower on every GPT shape).
       if (static_cast<long>(g.M) * g.N <= (1l << 20)) dma_variant = -1;
-      else if (t0 < 256 && g.K >= 2048 && t1 >= 256) dma_variant = 1;
-      else dma_variant = 0;
+      else dma_variant = 1;
     }
     else if (mode == 2) dma_variant = 0;
     else if (mode == 3) dma_variant = 1;

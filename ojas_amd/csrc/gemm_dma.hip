@@ -3,19 +3,20 @@
 //
 // Same contract as gemm.hip (C[M,N] (+)= A.B, f32 accumulation, every operand
 // layout; reference: ojas-cpu/src/linalg.rs:69-210), different data movement:
-//   * 512 threads (8 waves); tile 256 x 256 (waves 2 x 4, each 128 x 64) or
-//     256 x 128 (waves 4 x 2, each 64 x 64). Twice the tile edge halves the
-//     L2-to-LDS traffic per FLOP, which is what bounds the 128 x 128 kernel.
+//   * 512 threads (8 waves); tile 256 x 128 (waves 4 x 2, each 64 x 64; at most 108 VGPRs and
+//     72 KiB of LDS, so two workgroups share a compute unit and one's output stores, first
+//     loads and barrier waits overlap the other's products) or 256 x 256 (waves 2 x 4, each
+//     128 x 64; half the L2-to-LDS traffic per FLOP, one workgroup per compute unit).
 //   * operand tiles go from global memory straight into LDS: no staging
 //     registers and no LDS store instructions. A wave-wide load writes 64
 //     consecutive 16-byte slots, so the LDS tile is unpadded and bank conflicts
 //     are avoided by choosing WHICH chunk each lane fetches (an XOR swizzle):
-//       k-contiguous operand, [row][8 chunks]: slot s of row r holds chunk s ^ (r & 7);
+//       k-contiguous operand, [row][4 chunks]: slot s of row r holds chunk s ^ ((r >> 1) & 3);
 //       k-major operand, [k][ROWS/8 chunks]:   slot s of k row kr holds chunk s ^ 2(kr & 3)
 //     (the latter keeps the four k rows that one ds_read_b64_tr_b16 group
 //     touches on distinct banks).
-//   * two LDS stages: the loads of K step ks+1 are in flight while step ks is
-//     multiplied; one vmcnt(0) + barrier per step.
+//   * three LDS stages of 32 K columns: the loads of K steps ks+1 and ks+2 are in flight while
+//     step ks is multiplied; one counted vmcnt wait + barrier per step.
 // Rows past M (or N) are fetched from a clamped valid address and never stored.
 #include "gemm_args.h"
 
@@ -28,21 +29,23 @@ typedef short short4v __attribute__((ext_vector_type(4)));
 namespace {
 
 constexpr int DT = 512;  // threads
-constexpr int DBK = 64;
+constexpr int DBK = 32;   // K per pipeline step
+constexpr int NST = 3;    // LDS stages: the loads of step s + NST - 1 are issued while step s is multiplied
 
-// Issues this wave's share of one operand tile's loads. ROWS x 64 bf16 = ROWS / 8 KiB,
+// Issues this wave's share of one operand tile's loads. ROWS x 32 bf16 = ROWS / 16 KiB,
 // one wave instruction per KiB.
 template <bool KM, int ROWS>
 __device__ __forceinline__ void issue_tile(const unsigned short* __restrict__ p, long ld, int row0, int rows, int k0,
                                            char* tile, int wave, int lane) {
-  constexpr int NI = ROWS / 8;  // wave instructions per tile
+  constexpr int NI = ROWS / 16;  // wave instructions per tile
 #pragma unroll
   for (int i = 0; i < NI / 8; ++i) {
     const int q = wave + 8 * i;
     const unsigned short* src;
     if constexpr (!KM) {
-      const int r = q * 8 + (lane >> 3);
-      const int kc = (lane & 7) ^ (lane >> 3);
+      // [row][4 chunks of 16 bytes]; slot s of row r holds chunk s ^ ((r >> 1) & 3).
+      const int r = q * 16 + (lane >> 2);
+      const int kc = (lane & 3) ^ ((lane >> 3) & 3);
       int gr = row0 + r;
       gr = gr < rows ? gr : rows - 1;
       src = p + static_cast<long>(gr) * ld + k0 + kc * 8;
@@ -55,7 +58,7 @@ __device__ __forceinline__ void issue_tile(const unsigned short* __restrict__ p,
       gm = gm + 8 <= rows ? gm : 0;
       src = p + static_cast<long>(k0 + kr) * ld + gm;
     }
-    // Written as assembly: the compiler cannot tell that this asynchronous LDS write targets the
+    // Written as assembly: the compiler cannot tell that this asynchronous LDS write targets a
     // stage that is NOT being read, and would otherwise make every LDS read wait for it (vmcnt(0)
     // right after the issue), which serialises the loads with the products.
     const unsigned lds_at = static_cast<unsigned>(reinterpret_cast<uintptr_t>(tile + q * 1024));
@@ -71,7 +74,7 @@ __device__ __forceinline__ u32x4 frag(const char* tile, int row_base, int kk, in
     const int l32 = lane & 31, g = lane >> 5;
     const int r = row_base + l32;
     const int kc = kk * 2 + g;
-    return *reinterpret_cast<const u32x4*>(tile + r * 128 + ((kc ^ (r & 7)) << 4));
+    return *reinterpret_cast<const u32x4*>(tile + r * 64 + ((kc ^ ((r >> 1) & 3)) << 4));
   } else {
     const int s = lane & 15, half = (lane >> 4) & 1, g = lane >> 5;
     const int kr = kk * 16 + g * 8 + (s >> 2);
@@ -87,10 +90,11 @@ __device__ __forceinline__ u32x4 frag(const char* tile, int row_base, int kk, in
 }
 
 template <bool A_KM, bool B_KM, int WGM, int WGN, int TM, int TN>
-__global__ __launch_bounds__(DT) void gemm_dma_kernel(GemmArgs g) {
+__global__ __launch_bounds__(DT, (TM * TN <= 4 ? 4 : 2)) void gemm_dma_kernel(GemmArgs g) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
-  constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
+  constexpr int A_BYTES = BM * 64, B_BYTES = BN * 64, STAGE = A_BYTES + B_BYTES;
+  constexpr int LPS = (BM + BN) / 16 / 8;  // loads per wave per step
   static_assert(WGM * WGN == 8, "eight waves");
   const unsigned short* __restrict__ A = static_cast<const unsigned short*>(g.a);
   const unsigned short* __restrict__ B = static_cast<const unsigned short*>(g.b);
@@ -122,25 +126,32 @@ __global__ __launch_bounds__(DT) void gemm_dma_kernel(GemmArgs g) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  const int ksteps_all = g.K / DBK;
-  const int ks_begin = split * g.ksteps_per_split;
-  const int ks_end = min(ksteps_all, ks_begin + g.ksteps_per_split);
-  auto issue = [&](int ks, int buf) {
-    char* ta = smem + buf * STAGE;
+  // g.ksteps_per_split counts 64-wide K blocks; a pipeline step is half of one.
+  const int ks_begin = 2 * split * g.ksteps_per_split;
+  const int ks_end = min(g.K / DBK, ks_begin + 2 * g.ksteps_per_split);
+  auto issue = [&](int ks) {
+    char* ta = smem + ((ks - ks_begin) % NST) * STAGE;
     issue_tile<A_KM, BM>(A, g.lda, m0, g.M, ks * DBK, ta, wave, lane);
     issue_tile<B_KM, BN>(B, g.ldb, n0, g.N, ks * DBK, ta + A_BYTES, wave, lane);
   };
+  // Waits until at most `groups` of this wave's per-step load groups are still in flight.
+  auto wait_groups = [&](int groups) {
+    if (groups >= 2) __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * LPS));
+    else if (groups == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | LPS);
+    else __builtin_amdgcn_s_waitcnt(0x0F70);
+  };
 
-  issue(ks_begin, 0);
-  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+#pragma unroll
+  for (int i = 0; i < NST - 1; ++i)
+    if (ks_begin + i < ks_end) issue(ks_begin + i);
+  wait_groups(min(NST - 2, ks_end - ks_begin - 1));
   __syncthreads();
   for (int ks = ks_begin; ks < ks_end; ++ks) {
-    const int buf = (ks - ks_begin) & 1;
-    if (ks + 1 < ks_end) issue(ks + 1, buf ^ 1);
-    const char* ta = smem + buf * STAGE;
+    if (ks + NST - 1 < ks_end) issue(ks + NST - 1);
+    const char* ta = smem + ((ks - ks_begin) % NST) * STAGE;
     const char* tb = ta + A_BYTES;
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
+    for (int kk = 0; kk < 2; ++kk) {
       u32x4 af[TM], bf[TN];
 #pragma unroll
       for (int t = 0; t < TM; ++t) af[t] = frag<A_KM, BM>(ta, (wm * TM + t) * 32, kk, lane);
@@ -154,14 +165,16 @@ __global__ __launch_bounds__(DT) void gemm_dma_kernel(GemmArgs g) {
                                                                 __builtin_bit_cast(bf16x8, bf[tn]), acc[tm][tn], 0, 0,
                                                                 0);
     }
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // this wave's loads of the next step have landed
-    __syncthreads();                     // ... and everyone's; everyone is done reading `buf`
+    // Step ks + 1 must have landed (this wave's share, then everyone's); later steps may still be
+    // in flight. The barrier also frees stage ks for the loads of step ks + NST.
+    wait_groups(min(NST - 2, ks_end - ks - 2));
+    __syncthreads();
   }
 
   // Epilogue: each wave stages 32 rows of its tile at a time through its own
   // LDS region and writes whole 4-column pieces.
   constexpr int CPW = TN * 32 + 4;
-  static_assert(8 * 32 * CPW * 4 <= 2 * STAGE, "staging fits");
+  static_assert(8 * 32 * CPW * 4 <= NST * STAGE, "staging fits");
   float* cs = reinterpret_cast<float*>(smem) + wave * (32 * CPW);
   bool bad = false;
 #pragma unroll
@@ -191,7 +204,7 @@ __global__ __launch_bounds__(DT) void gemm_dma_kernel(GemmArgs g) {
 template <bool A_KM, bool B_KM, int WGM, int WGN, int TM, int TN>
 int32_t launch_dma(omx_ctx* ctx, const GemmArgs& g) {
   constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
-  constexpr int smem = 2 * (BM + BN) * 128;
+  constexpr int smem = NST * (BM + BN) * 64;
   auto kernel = &gemm_dma_kernel<A_KM, B_KM, WGM, WGN, TM, TN>;
   static bool granted = false;
   if (!granted) {
@@ -215,7 +228,7 @@ int32_t launch_layout(omx_ctx* ctx, const GemmArgs& g, bool a_km, bool b_km) {
 }  // namespace
 
 bool omx_gemm_dma_eligible(const GemmArgs& g, bool a_km, bool b_km) {
-  if (g.K % DBK != 0 || !g.a_vec || !g.b_vec) return false;
+  if (g.K % 64 != 0 || !g.a_vec || !g.b_vec) return false;
   if (a_km && g.M % 8 != 0) return false;
   if (b_km && g.N % 8 != 0) return false;
   return true;
