@@ -32,55 +32,77 @@ constexpr int DT = 512;  // threads
 constexpr int DBK = 32;   // K per pipeline step
 constexpr int NST = 3;    // LDS stages: the loads of step s + NST - 1 are issued while step s is multiplied
 
-// Issues this wave's share of one operand tile's loads. ROWS x 32 bf16 = ROWS / 16 KiB,
-// one wave instruction per KiB.
+// Per-lane state of one operand's loads: the global address of each of this wave's loads for the
+// current K step (advanced by one step after every issue) and nothing else, so a step costs one
+// 64-bit add per load. ROWS x 32 bf16 = ROWS / 16 KiB per step, one wave instruction per KiB.
 template <bool KM, int ROWS>
-__device__ __forceinline__ void issue_tile(const unsigned short* __restrict__ p, long ld, int row0, int rows, int k0,
-                                           char* tile, int wave, int lane) {
-  constexpr int NI = ROWS / 16;  // wave instructions per tile
-#pragma unroll
-  for (int i = 0; i < NI / 8; ++i) {
-    const int q = wave + 8 * i;
-    const unsigned short* src;
-    if constexpr (!KM) {
-      // [row][4 chunks of 16 bytes]; slot s of row r holds chunk s ^ ((r >> 1) & 3).
-      const int r = q * 16 + (lane >> 2);
-      const int kc = (lane & 3) ^ ((lane >> 3) & 3);
-      int gr = row0 + r;
-      gr = gr < rows ? gr : rows - 1;
-      src = p + static_cast<long>(gr) * ld + k0 + kc * 8;
-    } else {
-      constexpr int CPR = ROWS / 8;
-      const int idx = q * 64 + lane;
-      const int kr = idx / CPR, slot = idx % CPR;
-      const int mc = slot ^ ((kr & 3) * 2);
-      int gm = row0 + mc * 8;
-      gm = gm + 8 <= rows ? gm : 0;
-      src = p + static_cast<long>(k0 + kr) * ld + gm;
-    }
-    // Written as assembly: the compiler cannot tell that this asynchronous LDS write targets a
-    // stage that is NOT being read, and would otherwise make every LDS read wait for it (vmcnt(0)
-    // right after the issue), which serialises the loads with the products.
-    const unsigned lds_at = static_cast<unsigned>(reinterpret_cast<uintptr_t>(tile + q * 1024));
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src),
-                 "s"(__builtin_amdgcn_readfirstlane(lds_at))
-                 : "memory");
-  }
-}
+struct TileLoads {
+  static constexpr int N = ROWS / 16 / 8;  // loads per wave per step
+  const unsigned short* src[N];
+  long step;  // elements between consecutive K steps
 
+  __device__ __forceinline__ void init(const unsigned short* __restrict__ p, long ld, int row0, int rows, int k0,
+                                       int wave, int lane) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int q = wave + 8 * i;
+      if constexpr (!KM) {
+        // [row][4 chunks of 16 bytes]; slot s of row r holds chunk s ^ ((r >> 1) & 3).
+        const int r = q * 16 + (lane >> 2);
+        const int kc = (lane & 3) ^ ((lane >> 3) & 3);
+        int gr = row0 + r;
+        gr = gr < rows ? gr : rows - 1;
+        src[i] = p + static_cast<long>(gr) * ld + k0 + kc * 8;
+      } else {
+        constexpr int CPR = ROWS / 8;
+        const int idx = q * 64 + lane;
+        const int kr = idx / CPR, slot = idx % CPR;
+        const int mc = slot ^ ((kr & 3) * 2);
+        int gm = row0 + mc * 8;
+        gm = gm + 8 <= rows ? gm : 0;
+        src[i] = p + static_cast<long>(k0 + kr) * ld + gm;
+      }
+    }
+    step = KM ? DBK * ld : DBK;
+  }
+  // Starts this step's loads into the operand tile at LDS byte address `tile` and moves on.
+  __device__ __forceinline__ void issue(unsigned tile, int wave) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      // Written as assembly: the compiler cannot tell that this asynchronous LDS write targets a
+      // stage that is NOT being read, and would otherwise make every LDS read wait for it
+      // (vmcnt(0) right after the issue), which serialises the loads with the products.
+      asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src[i]),
+                   "s"(tile + (wave + 8 * i) * 1024)
+                   : "memory");
+      src[i] += step;
+    }
+  }
+};
+
+// Byte offset, inside an operand tile, of this lane's fragment for 32-row block `row_base / 32`
+// and 16-column K slab kk (k-major operands: of its first transposing read; the second is four
+// K rows further).
 template <bool KM, int ROWS>
-__device__ __forceinline__ u32x4 frag(const char* tile, int row_base, int kk, int lane) {
+__device__ __forceinline__ int frag_offset(int row_base, int kk, int lane) {
   if constexpr (!KM) {
     const int l32 = lane & 31, g = lane >> 5;
     const int r = row_base + l32;
     const int kc = kk * 2 + g;
-    return *reinterpret_cast<const u32x4*>(tile + r * 64 + ((kc ^ ((r >> 1) & 3)) << 4));
+    return r * 64 + ((kc ^ ((r >> 1) & 3)) << 4);
   } else {
     const int s = lane & 15, half = (lane >> 4) & 1, g = lane >> 5;
     const int kr = kk * 16 + g * 8 + (s >> 2);
     const int col = row_base + half * 16 + (s & 3) * 4;
     const int slot = (col >> 3) ^ (((s >> 2) & 3) * 2);
-    const char* p = tile + kr * (ROWS * 2) + slot * 16 + (col & 7) * 2;
+    return kr * (ROWS * 2) + slot * 16 + (col & 7) * 2;
+  }
+}
+template <bool KM, int ROWS>
+__device__ __forceinline__ u32x4 frag_at(const char* p) {
+  if constexpr (!KM) {
+    return *reinterpret_cast<const u32x4*>(p);
+  } else {
     typedef short4v __attribute__((address_space(3))) * lds_ptr;
     short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
     short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 4 * ROWS * 2));
@@ -129,11 +151,22 @@ __global__ __launch_bounds__(DT, (TM * TN <= 4 ? 4 : 2)) void gemm_dma_kernel(Ge
   // g.ksteps_per_split counts 64-wide K blocks; a pipeline step is half of one.
   const int ks_begin = 2 * split * g.ksteps_per_split;
   const int ks_end = min(g.K / DBK, ks_begin + 2 * g.ksteps_per_split);
-  auto issue = [&](int ks) {
-    char* ta = smem + ((ks - ks_begin) % NST) * STAGE;
-    issue_tile<A_KM, BM>(A, g.lda, m0, g.M, ks * DBK, ta, wave, lane);
-    issue_tile<B_KM, BN>(B, g.ldb, n0, g.N, ks * DBK, ta + A_BYTES, wave, lane);
-  };
+  // Everything a K step needs is computed here, once per tile: the loads' global addresses and
+  // the fragments' LDS offsets. Inside the loop the stage is a compile-time constant (the loop
+  // body is unrolled over the stages), so a step is loads, LDS reads and MFMAs and little else.
+  TileLoads<A_KM, BM> la;
+  TileLoads<B_KM, BN> lb;
+  la.init(A, g.lda, m0, g.M, ks_begin * DBK, wave, lane);
+  lb.init(B, g.ldb, n0, g.N, ks_begin * DBK, wave, lane);
+  const unsigned lds0 = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(reinterpret_cast<uintptr_t>(smem)));
+  int a_off[TM][2], b_off[TN][2];
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+    for (int t = 0; t < TM; ++t) a_off[t][kk] = frag_offset<A_KM, BM>((wm * TM + t) * 32, kk, lane);
+#pragma unroll
+    for (int t = 0; t < TN; ++t) b_off[t][kk] = A_BYTES + frag_offset<B_KM, BN>((wn * TN + t) * 32, kk, lane);
+  }
   // Waits until at most `groups` of this wave's per-step load groups are still in flight.
   auto wait_groups = [&](int groups) {
     if (groups >= 2) __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * LPS));
@@ -143,32 +176,42 @@ __global__ __launch_bounds__(DT, (TM * TN <= 4 ? 4 : 2)) void gemm_dma_kernel(Ge
 
 #pragma unroll
   for (int i = 0; i < NST - 1; ++i)
-    if (ks_begin + i < ks_end) issue(ks_begin + i);
+    if (ks_begin + i < ks_end) {
+      la.issue(lds0 + i * STAGE, wave);
+      lb.issue(lds0 + i * STAGE + A_BYTES, wave);
+    }
   wait_groups(min(NST - 2, ks_end - ks_begin - 1));
   __syncthreads();
-  for (int ks = ks_begin; ks < ks_end; ++ks) {
-    if (ks + NST - 1 < ks_end) issue(ks + NST - 1);
-    const char* ta = smem + ((ks - ks_begin) % NST) * STAGE;
-    const char* tb = ta + A_BYTES;
+  for (int ks = ks_begin; ks < ks_end;) {
 #pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-      u32x4 af[TM], bf[TN];
+    for (int st = 0; st < NST; ++st) {  // step ks lives in stage st
+      if (ks + NST - 1 < ks_end) {
+        constexpr int kFill[3] = {NST - 1, 0, 1};
+        la.issue(lds0 + kFill[st % 3] * STAGE, wave);
+        lb.issue(lds0 + kFill[st % 3] * STAGE + A_BYTES, wave);
+      }
+      const char* stage = smem + st * STAGE;
 #pragma unroll
-      for (int t = 0; t < TM; ++t) af[t] = frag<A_KM, BM>(ta, (wm * TM + t) * 32, kk, lane);
+      for (int kk = 0; kk < 2; ++kk) {
+        u32x4 af[TM], bf[TN];
 #pragma unroll
-      for (int t = 0; t < TN; ++t) bf[t] = frag<B_KM, BN>(tb, (wn * TN + t) * 32, kk, lane);
+        for (int t = 0; t < TM; ++t) af[t] = frag_at<A_KM, BM>(stage + a_off[t][kk]);
 #pragma unroll
-      for (int tm = 0; tm < TM; ++tm)
+        for (int t = 0; t < TN; ++t) bf[t] = frag_at<B_KM, BN>(stage + b_off[t][kk]);
 #pragma unroll
-        for (int tn = 0; tn < TN; ++tn)
-          acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[tm]),
-                                                                __builtin_bit_cast(bf16x8, bf[tn]), acc[tm][tn], 0, 0,
-                                                                0);
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+          for (int tn = 0; tn < TN; ++tn)
+            acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[tm]),
+                                                                  __builtin_bit_cast(bf16x8, bf[tn]), acc[tm][tn], 0,
+                                                                  0, 0);
+      }
+      // Step ks + 1 must have landed (this wave's share, then everyone's); later steps may still
+      // be in flight. The barrier also frees stage st for the loads of step ks + NST.
+      wait_groups(min(NST - 2, ks_end - ks - 2));
+      __syncthreads();
+      if (++ks >= ks_end) break;
     }
-    // Step ks + 1 must have landed (this wave's share, then everyone's); later steps may still be
-    // in flight. The barrier also frees stage ks for the loads of step ks + NST.
-    wait_groups(min(NST - 2, ks_end - ks - 2));
-    __syncthreads();
   }
 
   // Epilogue: each wave stages 32 rows of its tile at a time through its own
