@@ -131,6 +131,20 @@ int32_t omx_causal_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, con
                                  uint64_t kv_heads, uint64_t time, uint64_t head_dim,
                                  uint64_t window);
 
+/* linear_forward then gelu_{erf,tanh}_forward (backend.rs:1628-1656,1175-1220), the
+ * activation applied while the product is stored: u = x W^T and act = gelu(u),
+ * both bf16 [rows, out_features]; same bits as the two separate calls. The
+ * reverse pair: gu = linear_backward(w, gy).grad_input * gelu'(u), i.e.
+ * gelu_backward(u, gy W) in the product's store pass (gy [rows, out_features],
+ * w [out_features, in_features], u / gu [rows, in_features]). bf16 only. */
+int32_t omx_linear_gelu_forward(omx_ctx* ctx, const void* x, const void* w, int32_t operand_dtype,
+                                void* u, void* act, uint64_t rows, uint64_t in_features,
+                                uint64_t out_features, int32_t tanh_form);
+int32_t omx_linear_backward_input_gelu(omx_ctx* ctx, const void* w, const void* gy,
+                                       int32_t operand_dtype, const void* u, void* gu,
+                                       uint64_t rows, uint64_t in_features, uint64_t out_features,
+                                       int32_t tanh_form);
+
 /* ---- causal_attention (ojas-model/src/block.rs:186-199): permute [0,2,1,3],
  *      causal_sdpa, permute back, done in one pass over time-major tensors.
  *      q / out / gy / gq are [batch, time, heads, head_dim], k / v / gk / gv

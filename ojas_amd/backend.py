@@ -286,6 +286,25 @@ class MiBackend:
                                                        C.c_uint64(window or 0)))
         return gq, gk, gv
 
+    def linear_gelu_forward(self, x, w, tanh_form: bool = False):
+        """`linear_forward` then `gelu_*_forward` in one kernel (bf16): returns (u, gelu(u))."""
+        rows, nout = x.numel // x.shape[-1], w.shape[0]
+        u, act = self.empty(x.shape[:-1] + (nout,), BF16), self.empty(x.shape[:-1] + (nout,), BF16)
+        self._check(self._lib.omx_linear_gelu_forward(
+            self._ctx, self._p(x), self._p(w), C.c_int32(x.dtype), self._p(u), self._p(act), C.c_uint64(rows),
+            C.c_uint64(x.shape[-1]), C.c_uint64(nout), C.c_int32(1 if tanh_form else 0)))
+        return u, act
+
+    def linear_backward_input_gelu(self, w, gy, u, tanh_form: bool = False):
+        """grad_input of `linear_backward(w, gy)` times gelu'(u) in one kernel (bf16)."""
+        nout, nin = w.shape
+        rows = gy.numel // nout
+        gu = self.empty(u.shape, BF16)
+        self._check(self._lib.omx_linear_backward_input_gelu(
+            self._ctx, self._p(w), self._p(gy), C.c_int32(gy.dtype), self._p(u), self._p(gu), C.c_uint64(rows),
+            C.c_uint64(nin), C.c_uint64(nout), C.c_int32(1 if tanh_form else 0)))
+        return gu
+
     def causal_attention_forward(self, q, k, v, window: Optional[int] = None, pitches=None):
         """`causal_attention` (ojas-model/src/block.rs:186-199) over time-major [B, T, heads, D]
         tensors. `pitches` = (q, kv) token-row pitches in elements when q / k / v are column

@@ -70,42 +70,13 @@ __global__ void scale_kernel(float* __restrict__ g, float s, size_t n, OmxFaultW
   if (bad) dev_raise_fault(fault, tag);
 }
 
-// GELU in f32. The erf form is 0.5 x (1 + erf(x / sqrt 2)); the tanh form is
-// x * sigmoid(2 sqrt(2/pi) (x + 0.044715 x^3)), which has no cancellation in
-// the negative tail (ojas-core/src/gelu_tanh.rs:8-15).
-__device__ __forceinline__ float gelu_erf_f(float x) { return 0.5f * x * (1.0f + erff(x * 0.70710678118654752f)); }
-__device__ __forceinline__ float gelu_erf_grad_f(float x) {
-  float cdf = 0.5f * (1.0f + erff(x * 0.70710678118654752f));
-  float pdf = 0.3989422804014327f * __expf(-0.5f * x * x);
-  return cdf + x * pdf;
-}
-__device__ __forceinline__ void sigmoid_pair_f(float u, float* s, float* slope) {
-  float e = __expf(-fabsf(u));
-  float denom = 1.0f + e;
-  *s = u >= 0.0f ? 1.0f / denom : e / denom;
-  *slope = e / (denom * denom);
-}
-__device__ __forceinline__ float gelu_tanh_f(float x) {
-  float u = 2.0f * 0.7978845608028654f * (x + 0.044715f * x * x * x);
-  float s, slope;
-  sigmoid_pair_f(u, &s, &slope);
-  return x * s;
-}
-__device__ __forceinline__ float gelu_tanh_grad_f(float x) {
-  float u = 2.0f * 0.7978845608028654f * (x + 0.044715f * x * x * x);
-  float s, slope;
-  sigmoid_pair_f(u, &s, &slope);
-  float du = 2.0f * 0.7978845608028654f * (1.0f + 3.0f * 0.044715f * x * x);
-  return s + x * slope * du;
-}
-
 template <typename T, bool TANH>
 __global__ void gelu_fwd_kernel(const T* __restrict__ x, T* __restrict__ y, size_t n, OmxFaultWord* fault,
                                 unsigned long long tag) {
   bool bad = false;
   EW_LOOP(i, n) {
     float v = dev_load<T>(x, i);
-    float r = TANH ? gelu_tanh_f(v) : gelu_erf_f(v);
+    float r = TANH ? dev_gelu_tanh(v) : dev_gelu_erf(v);
     bad |= !dev_finite(r);
     dev_store<T>(y, i, r);
   }
@@ -117,7 +88,7 @@ __global__ void gelu_bwd_kernel(const T* __restrict__ x, const T* __restrict__ g
   bool bad = false;
   EW_LOOP(i, n) {
     float v = dev_load<T>(x, i);
-    float r = dev_load<T>(gy, i) * (TANH ? gelu_tanh_grad_f(v) : gelu_erf_grad_f(v));
+    float r = dev_load<T>(gy, i) * (TANH ? dev_gelu_tanh_grad(v) : dev_gelu_erf_grad(v));
     bad |= !dev_finite(r);
     dev_store<T>(gx, i, r);
   }

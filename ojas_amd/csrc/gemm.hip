@@ -343,7 +343,8 @@ __global__ __launch_bounds__(NT) void gemm_kernel(GemmArgs g) {
     const int grow = m0 + row, gcol = n0 + cc;
     if (grow >= g.M || gcol >= g.N) continue;
     const float4 val = *reinterpret_cast<const float4*>(cs + row * CP + cc);
-    bad |= gemm_store4(g, split, grow, gcol, val.x, val.y, val.z, val.w);
+    bad |= g.epi == OMX_EPI_NONE ? gemm_store4(g, split, grow, gcol, val.x, val.y, val.z, val.w)
+                                 : gemm_store4_epi(g, split, grow, gcol, val.x, val.y, val.z, val.w);
   }
   if (bad) dev_raise_fault(g.fault, g.tag);
 }
@@ -406,8 +407,10 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 // Internal entry shared by the linear ops, the fused loss and Muon.
 int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a_rs, uint64_t a_cs, const void* b,
                       uint64_t b_rs, uint64_t b_cs, int32_t operand_dtype, void* c, int32_t c_dtype, uint64_t ldc,
-                      uint64_t m, uint64_t k, uint64_t n, int32_t accumulate) {
+                      uint64_t m, uint64_t k, uint64_t n, int32_t accumulate, const OmxGemmEpilogue* epi) {
   const char* op = omx_fault_name(fault_op);
+  if (epi && epi->mode != OMX_EPI_NONE && c_dtype != OMX_BF16)
+    return omx_fail(ctx, OMX_DTYPE, "%s: a fused activation needs a bf16 output", op);
   if (!a || !b || !c) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
   if (!omx_valid_float_dtype(operand_dtype) || !omx_valid_float_dtype(c_dtype))
     return omx_fail(ctx, OMX_DTYPE, "%s: operands must be f32 or bf16", op);
@@ -482,7 +485,7 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
     const int ksteps = (g.K + bk - 1) / bk;
     const long tiles = static_cast<long>(g.tiles_m) * g.tiles_n;
     int splits = 1;
-    if (tiles < 256 && ksteps >= 32) {
+    if (tiles < 256 && ksteps >= 32 && !(epi && epi->mode != OMX_EPI_NONE)) {
       splits = static_cast<int>((512 + tiles - 1) / tiles);
       if (splits > ksteps / 8) splits = ksteps / 8;
       if (splits < 1) splits = 1;
@@ -497,6 +500,10 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
       g.partial = static_cast<float*>(ws);
     }
   }
+  g.epi = epi ? epi->mode : OMX_EPI_NONE;
+  g.epi_tanh = epi ? epi->tanh_form : 0;
+  g.aux_in = epi ? static_cast<const unsigned short*>(epi->aux_in) : nullptr;
+  g.aux_out = epi ? static_cast<unsigned short*>(epi->aux_out) : nullptr;
   g.fault = ctx->fault;
   g.tag = omx_tag(ctx, fault_op);
   omx_ctx::TimedLaunch timed{};

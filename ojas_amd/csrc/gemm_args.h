@@ -15,6 +15,9 @@ struct GemmArgs {
   int tiles_m, tiles_n;
   int splits, ksteps_per_split;  // split-K: each split writes an f32 partial
   float* partial;                // [splits][M][N] when splits > 1
+  int epi, epi_tanh;             // OMX_EPI_* (bf16 output, no split)
+  const unsigned short* aux_in;
+  unsigned short* aux_out;
   OmxFaultWord* fault;
   unsigned long long tag;
 };
@@ -75,6 +78,60 @@ __device__ __forceinline__ bool gemm_store4(const GemmArgs& g, int split, int gr
     }
   }
   return bad;
+}
+
+// gemm_store4 with the optional activation of OmxGemmEpilogue applied first (bf16 outputs, no
+// split). Kept apart from the plain store so the plain epilogue loops stay small enough to unroll.
+__device__ __forceinline__ bool gemm_store4_epi(const GemmArgs& g, int split, int grow, int gcol, float x0, float x1,
+                                                float x2, float x3) {
+  bool bad = false;
+  const long off = static_cast<long>(grow) * g.ldc + gcol;
+  const bool whole = g.c_vec != 0 && gcol + 4 <= g.N;
+  {
+    if (g.epi == OMX_EPI_GELU_FWD) {
+      // The activation is taken of the value the pre-activation is stored as.
+      const float u0 = dev_round_bf16(x0), u1 = dev_round_bf16(x1), u2 = dev_round_bf16(x2), u3 = dev_round_bf16(x3);
+      const float a0 = g.epi_tanh ? dev_gelu_tanh(u0) : dev_gelu_erf(u0);
+      const float a1 = g.epi_tanh ? dev_gelu_tanh(u1) : dev_gelu_erf(u1);
+      const float a2 = g.epi_tanh ? dev_gelu_tanh(u2) : dev_gelu_erf(u2);
+      const float a3 = g.epi_tanh ? dev_gelu_tanh(u3) : dev_gelu_erf(u3);
+      unsigned short* ap = g.aux_out + off;
+      if (whole) {
+        uint2 w;
+        w.x = static_cast<unsigned int>(dev_f32_to_bf16_bits(a0)) |
+              (static_cast<unsigned int>(dev_f32_to_bf16_bits(a1)) << 16);
+        w.y = static_cast<unsigned int>(dev_f32_to_bf16_bits(a2)) |
+              (static_cast<unsigned int>(dev_f32_to_bf16_bits(a3)) << 16);
+        *reinterpret_cast<uint2*>(ap) = w;
+        bad = !(dev_finite(a0) && dev_finite(a1) && dev_finite(a2) && dev_finite(a3));
+      } else {
+        if (gcol + 0 < g.N) { ap[0] = dev_f32_to_bf16_bits(a0); bad |= !dev_finite(a0); }
+        if (gcol + 1 < g.N) { ap[1] = dev_f32_to_bf16_bits(a1); bad |= !dev_finite(a1); }
+        if (gcol + 2 < g.N) { ap[2] = dev_f32_to_bf16_bits(a2); bad |= !dev_finite(a2); }
+        if (gcol + 3 < g.N) { ap[3] = dev_f32_to_bf16_bits(a3); bad |= !dev_finite(a3); }
+      }
+    } else if (g.epi == OMX_EPI_GELU_BWD) {
+      const unsigned short* ap = g.aux_in + off;
+      float u0 = 0.0f, u1 = 0.0f, u2 = 0.0f, u3 = 0.0f;
+      if (whole) {
+        const uint2 w = *reinterpret_cast<const uint2*>(ap);
+        u0 = __uint_as_float(w.x << 16);
+        u1 = __uint_as_float(w.x & 0xffff0000u);
+        u2 = __uint_as_float(w.y << 16);
+        u3 = __uint_as_float(w.y & 0xffff0000u);
+      } else {
+        if (gcol + 0 < g.N) u0 = dev_bf16_bits_to_f32(ap[0]);
+        if (gcol + 1 < g.N) u1 = dev_bf16_bits_to_f32(ap[1]);
+        if (gcol + 2 < g.N) u2 = dev_bf16_bits_to_f32(ap[2]);
+        if (gcol + 3 < g.N) u3 = dev_bf16_bits_to_f32(ap[3]);
+      }
+      x0 = dev_round_bf16(x0) * (g.epi_tanh ? dev_gelu_tanh_grad(u0) : dev_gelu_erf_grad(u0));
+      x1 = dev_round_bf16(x1) * (g.epi_tanh ? dev_gelu_tanh_grad(u1) : dev_gelu_erf_grad(u1));
+      x2 = dev_round_bf16(x2) * (g.epi_tanh ? dev_gelu_tanh_grad(u2) : dev_gelu_erf_grad(u2));
+      x3 = dev_round_bf16(x3) * (g.epi_tanh ? dev_gelu_tanh_grad(u3) : dev_gelu_erf_grad(u3));
+    }
+  }
+  return gemm_store4(g, split, grow, gcol, x0, x1, x2, x3) || bad;
 }
 
 // bf16 kernel with direct-to-LDS loads and a 256 x 256 (variant 0) or

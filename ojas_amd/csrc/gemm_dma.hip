@@ -229,13 +229,25 @@ __global__ __launch_bounds__(DT, (TM * TN <= 4 ? 4 : 2)) void gemm_dma_kernel(Ge
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     constexpr int PPR = TN * 8;  // 4-column pieces per row
+    if (g.epi == OMX_EPI_NONE) {
 #pragma unroll
-    for (int c = lane; c < 32 * PPR; c += 64) {
-      const int row = c / PPR, piece = c % PPR;
-      const int grow = m0 + (wm * TM + tm) * 32 + row, gcol = n0 + wn * TN * 32 + piece * 4;
-      if (grow < g.M && gcol < g.N) {
-        const float4 val = *reinterpret_cast<const float4*>(cs + row * CPW + piece * 4);
-        bad |= gemm_store4(g, split, grow, gcol, val.x, val.y, val.z, val.w);
+      for (int c = lane; c < 32 * PPR; c += 64) {
+        const int row = c / PPR, piece = c % PPR;
+        const int grow = m0 + (wm * TM + tm) * 32 + row, gcol = n0 + wn * TN * 32 + piece * 4;
+        if (grow < g.M && gcol < g.N) {
+          const float4 val = *reinterpret_cast<const float4*>(cs + row * CPW + piece * 4);
+          bad |= gemm_store4(g, split, grow, gcol, val.x, val.y, val.z, val.w);
+        }
+      }
+    } else {
+#pragma unroll 1
+      for (int c = lane; c < 32 * PPR; c += 64) {
+        const int row = c / PPR, piece = c % PPR;
+        const int grow = m0 + (wm * TM + tm) * 32 + row, gcol = n0 + wn * TN * 32 + piece * 4;
+        if (grow < g.M && gcol < g.N) {
+          const float4 val = *reinterpret_cast<const float4*>(cs + row * CPW + piece * 4);
+          bad |= gemm_store4_epi(g, split, grow, gcol, val.x, val.y, val.z, val.w);
+        }
       }
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");

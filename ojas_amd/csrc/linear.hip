@@ -86,4 +86,33 @@ int32_t omx_linear_backward(omx_ctx* ctx, const void* x, const void* w, const vo
   return OMX_OK;
 }
 
+// linear_forward followed by gelu (ojas-model block: up-projection then activation), the
+// activation applied in the product's store pass: u = x W^T and act = gelu(u), both bf16.
+int32_t omx_linear_gelu_forward(omx_ctx* ctx, const void* x, const void* w, int32_t operand_dtype, void* u, void* act,
+                                uint64_t rows, uint64_t in_features, uint64_t out_features, int32_t tanh_form) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "linear_gelu_forward";
+  if (!x || !w || !u || !act) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  if (operand_dtype != OMX_BF16) return omx_fail(ctx, OMX_UNSUPPORTED, "%s: bf16 operands only", op);
+  if (rows == 0 || in_features == 0 || out_features == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
+  OmxGemmEpilogue epi = {OMX_EPI_GELU_FWD, tanh_form ? 1 : 0, nullptr, act};
+  return omx_gemm_impl(ctx, F_LINEAR_FORWARD, x, in_features, 1, w, 1, in_features, operand_dtype, u, OMX_BF16,
+                       out_features, rows, in_features, out_features, 0, &epi);
+}
+
+// The input gradient of linear_backward followed by gelu_backward: gu = (gy W) * gelu'(u),
+// the derivative applied in the product's store pass. gy [rows, out], w [out, in], u / gu [rows, in].
+int32_t omx_linear_backward_input_gelu(omx_ctx* ctx, const void* w, const void* gy, int32_t operand_dtype,
+                                       const void* u, void* gu, uint64_t rows, uint64_t in_features,
+                                       uint64_t out_features, int32_t tanh_form) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "linear_backward_input_gelu";
+  if (!w || !gy || !u || !gu) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  if (operand_dtype != OMX_BF16) return omx_fail(ctx, OMX_UNSUPPORTED, "%s: bf16 operands only", op);
+  if (rows == 0 || in_features == 0 || out_features == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
+  OmxGemmEpilogue epi = {OMX_EPI_GELU_BWD, tanh_form ? 1 : 0, u, nullptr};
+  return omx_gemm_impl(ctx, F_LINEAR_BACKWARD, gy, out_features, 1, w, in_features, 1, operand_dtype, gu, OMX_BF16,
+                       in_features, rows, out_features, in_features, 0, &epi);
+}
+
 }  // extern "C"

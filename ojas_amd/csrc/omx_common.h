@@ -101,9 +101,19 @@ inline unsigned long long omx_tag(omx_ctx* ctx, uint32_t op) {
 }
 
 // C[m,n] (+)= A.B with element strides; `ldc` is C's row pitch in elements.
+// Optional elementwise work in the GEMM's store pass (bf16 outputs only; `aux` shares C's row pitch):
+//   OMX_EPI_GELU_FWD: C = u (rounded to bf16) and aux_out = gelu(u);
+//   OMX_EPI_GELU_BWD: C = round_bf16(A.B) * gelu'(aux_in).
+enum { OMX_EPI_NONE = 0, OMX_EPI_GELU_FWD = 1, OMX_EPI_GELU_BWD = 2 };
+struct OmxGemmEpilogue {
+  int mode;
+  int tanh_form;
+  const void* aux_in;
+  void* aux_out;
+};
 int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a_rs, uint64_t a_cs, const void* b,
                       uint64_t b_rs, uint64_t b_cs, int32_t operand_dtype, void* c, int32_t c_dtype, uint64_t ldc,
-                      uint64_t m, uint64_t k, uint64_t n, int32_t accumulate);
+                      uint64_t m, uint64_t k, uint64_t n, int32_t accumulate, const OmxGemmEpilogue* epi = nullptr);
 // out[c] = sum over b < blocks of partial[b * dim + c], added in a fixed order.
 // `scratch` (OMX_COLUMN_SUM_GROUPS * dim floats, may be null) lets a tall `partial` be added in two stages.
 constexpr int OMX_COLUMN_SUM_GROUPS = 32;
@@ -227,6 +237,35 @@ __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
   return v;
+}
+
+// GELU in f32. The erf form is 0.5 x (1 + erf(x / sqrt 2)); the tanh form is
+// x * sigmoid(2 sqrt(2/pi) (x + 0.044715 x^3)), which has no cancellation in
+// the negative tail (ojas-core/src/gelu_tanh.rs:8-15).
+__device__ __forceinline__ float dev_gelu_erf(float x) { return 0.5f * x * (1.0f + erff(x * 0.70710678118654752f)); }
+__device__ __forceinline__ float dev_gelu_erf_grad(float x) {
+  float cdf = 0.5f * (1.0f + erff(x * 0.70710678118654752f));
+  float pdf = 0.3989422804014327f * __expf(-0.5f * x * x);
+  return cdf + x * pdf;
+}
+__device__ __forceinline__ void dev_sigmoid_pair(float u, float* s, float* slope) {
+  float e = __expf(-fabsf(u));
+  float denom = 1.0f + e;
+  *s = u >= 0.0f ? 1.0f / denom : e / denom;
+  *slope = e / (denom * denom);
+}
+__device__ __forceinline__ float dev_gelu_tanh(float x) {
+  float u = 2.0f * 0.7978845608028654f * (x + 0.044715f * x * x * x);
+  float s, slope;
+  dev_sigmoid_pair(u, &s, &slope);
+  return x * s;
+}
+__device__ __forceinline__ float dev_gelu_tanh_grad(float x) {
+  float u = 2.0f * 0.7978845608028654f * (x + 0.044715f * x * x * x);
+  float s, slope;
+  dev_sigmoid_pair(u, &s, &slope);
+  float du = 2.0f * 0.7978845608028654f * (1.0f + 3.0f * 0.044715f * x * x);
+  return s + x * slope * du;
 }
 
 inline bool omx_valid_float_dtype(int32_t d) { return d == OMX_F32 || d == OMX_BF16; }

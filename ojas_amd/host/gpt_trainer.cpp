@@ -153,8 +153,13 @@ int32_t forward(ogpt* t) {
     TRY(omx_linear_forward(ctx, A.ap, AD, t->w(t->li(l, 4)), AD, t->t_a, AD, N, d, d));
     TRY(omx_residual_add_rms_norm_forward(ctx, A.x, OMX_F32, t->t_a, AD, t->w32(t->li(l, 5)), A.x1, A.h2, AD, N, d,
                                           eps));
-    TRY(omx_linear_forward(ctx, A.h2, AD, t->w(t->li(l, 6)), AD, A.u, AD, N, d, M));
-    TRY(omx_gelu_forward(ctx, A.u, A.g, AD, N * M, c.gelu_tanh));
+    if (AD == OMX_BF16) {
+      // The activation rides in the up-projection's store pass.
+      TRY(omx_linear_gelu_forward(ctx, A.h2, t->w(t->li(l, 6)), AD, A.u, A.g, N, d, M, c.gelu_tanh));
+    } else {
+      TRY(omx_linear_forward(ctx, A.h2, AD, t->w(t->li(l, 6)), AD, A.u, AD, N, d, M));
+      TRY(omx_gelu_forward(ctx, A.u, A.g, AD, N * M, c.gelu_tanh));
+    }
     TRY(omx_linear_forward(ctx, A.g, AD, t->w(t->li(l, 7)), AD, t->t_a, AD, N, M, d));
     TRY(omx_residual_add_rms_norm_forward(ctx, A.x1, OMX_F32, t->t_a, AD, next_norm, x_next, h_next, AD, N, d, eps));
   }
@@ -182,8 +187,14 @@ int32_t backward(ogpt* t) {
   for (uint32_t l = c.layers; l-- > 0;) {
     ogpt::Layer& A = t->layers[l];
     // x_next = x1 + down(gelu(up(norm2(x1))))
-    TRY(omx_linear_backward(ctx, A.g, t->w(t->li(l, 7)), gy, AD, t->gg, AD, t->g(t->li(l, 7)), OMX_F32, N, M, d));
-    TRY(omx_gelu_backward(ctx, A.u, t->gg, t->gu, AD, N * M, c.gelu_tanh));
+    if (AD == OMX_BF16) {
+      // The activation's derivative rides in the input-gradient product's store pass.
+      TRY(omx_linear_backward(ctx, A.g, nullptr, gy, AD, nullptr, AD, t->g(t->li(l, 7)), OMX_F32, N, M, d));
+      TRY(omx_linear_backward_input_gelu(ctx, t->w(t->li(l, 7)), gy, AD, A.u, t->gu, N, M, d, c.gelu_tanh));
+    } else {
+      TRY(omx_linear_backward(ctx, A.g, t->w(t->li(l, 7)), gy, AD, t->gg, AD, t->g(t->li(l, 7)), OMX_F32, N, M, d));
+      TRY(omx_gelu_backward(ctx, A.u, t->gg, t->gu, AD, N * M, c.gelu_tanh));
+    }
     TRY(omx_linear_backward(ctx, A.h2, t->w(t->li(l, 6)), t->gu, AD, t->t_a, AD, t->g(t->li(l, 6)), OMX_F32, N, d, M));
     // Fan-in at x1: the residual branch arrives first, then the norm branch.
     TRY(omx_rms_norm_backward_residual(ctx, A.x1, OMX_F32, t->w32(t->li(l, 5)), t->t_a, AD, t->gres, t->gres1, copy16,

@@ -325,6 +325,46 @@ def test_fused_residual_rms_norm_equals_the_separate_ops(be, rows, dim, bf16):
         assert np.array_equal(be.download(gx), be.download(sep))
 
 
+@pytest.mark.parametrize("tanh_form", [False, True])
+@pytest.mark.parametrize("rows,nin,nout", [(64, 64, 128), (300, 128, 520), (1024, 768, 3072), (257, 192, 70)])
+def test_linear_with_fused_gelu_equals_the_separate_ops(be, rows, nin, nout, tanh_form):
+    """The activation applied in the product's store pass gives the bits of linear then gelu, in
+    both directions, on tile-aligned and ragged shapes and on both GEMM kernels."""
+    from ojas_amd.backend import BF16
+
+    print(f"linear+gelu rows={rows} in={nin} out={nout} tanh={tanh_form}", flush=True)
+    r = orc.SplitMix64(6100 + rows + nout)
+    x = orc.round_bf16(r.vec(rows * nin, 1.0)).reshape(rows, nin)
+    w = orc.round_bf16(r.vec(nout * nin, 2.0 / np.sqrt(nin))).reshape(nout, nin)
+    gy = orc.round_bf16(r.vec(rows * nout, 1.0)).reshape(rows, nout)
+    dx, dw, dgy = (be.upload(a, BF16) for a in (x, w, gy))
+    fwd = be.gelu_tanh_forward if tanh_form else be.gelu_erf_forward
+    bwd = be.gelu_tanh_backward if tanh_form else be.gelu_erf_backward
+    u, act = be.linear_gelu_forward(dx, dw, tanh_form)
+    u2 = be.linear_forward(dx, dw, BF16)
+    assert np.array_equal(be.download(u), be.download(u2))
+    assert np.array_equal(be.download(act), be.download(fwd(u2)))
+    o_u = orc.linear_forward(x, w)
+    close(be.download_f32(u), o_u, BF16_TOL, "u")
+    o_act = orc.gelu_tanh_forward(o_u) if tanh_form else orc.gelu_erf_forward(o_u)
+    close(be.download_f32(act), o_act, BF16_TOL, "gelu(u)")
+    # Reverse: here the linear maps nout -> nin features... use its transpose roles: the fused
+    # call computes (gy W) * gelu'(pre) with pre [rows, nin].
+    pre = orc.round_bf16(r.vec(rows * nin, 2.0)).reshape(rows, nin)
+    dpre = be.upload(pre, BF16)
+    gu = be.linear_backward_input_gelu(dw, dgy, dpre, tanh_form)
+    gx = be.linear_backward_input(dw, dgy, nin, BF16)
+    if nout < 2048:
+        assert np.array_equal(be.download(gu), be.download(bwd(dpre, gx)))
+    else:
+        # A long reduction over few tiles is split in the plain product (another summation order);
+        # the fused one never splits.
+        close(be.download_f32(gu), be.download_f32(bwd(dpre, gx)), BF16_TOL, "gu vs separate")
+    o_gx, _ = orc.linear_backward(x, w, gy, need_gw=False)
+    o_gu = orc.gelu_tanh_backward_vec(pre, o_gx) if tanh_form else orc.gelu_erf_backward_vec(pre, o_gx)
+    close(be.download_f32(gu), o_gu, BF16_TOL, "gu")
+
+
 def test_time_major_attention_refuses_other_shapes(be):
     from ojas_amd.backend import BF16, OjasError
 
