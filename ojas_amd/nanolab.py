@@ -1,0 +1,176 @@
+"""The nanolab GPT graph over `MiBackend`: forward, loss and every gradient.
+
+Host-side orchestration only, the role of `forward_loss` + `Tape::backward` for the reference's own
+model graph (ojas-model/src/block.rs:218-264 `block_with`, :343-420 `hidden` / tied head;
+ojas-autograd/src/tape.rs:2004-2466 backward rules, :2565-2591 gradient fan-in, later consumer
+first). Every tensor operation is one `MiBackend` method, i.e. one C-ABI call; nothing is computed
+here. Parameters come in the order of ojas-model/src/names.rs:188-300.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+
+from .backend import F32, MiBackend, DeviceTensor
+
+BLOCK_PARAMS = ("norm1.weight", "mixer.q_proj.weight", "mixer.k_proj.weight", "mixer.v_proj.weight",
+                "mixer.o_proj.weight", "mixer.q_norm.weight", "mixer.k_norm.weight", "mixer.gate.weight",
+                "mixer.gate.bias", "mixer.vr_lambda", "norm2.weight", "ffn.gate.weight", "ffn.up.weight",
+                "ffn.down.weight")
+
+
+@dataclass
+class NanolabSpec:
+    """`ojas_model::ModelSpec` (ojas-model/src/spec.rs): the fields the graph reads."""
+    n_layer: int
+    n_embd: int
+    n_head: int
+    n_kv_head: int
+    head_dim: int
+    hidden: int
+    vocab: int
+    rms_eps: float = 1e-6
+    rope_base: float = 10000.0
+    window: Optional[int] = None
+
+    def param_names(self) -> List[str]:
+        names = ["tok_emb.weight"]
+        for i in range(self.n_layer):
+            names += [f"blocks.{i}.{n}" for n in BLOCK_PARAMS]
+        return names + ["norm_f.weight"]
+
+    def param_shapes(self) -> Dict[str, tuple]:
+        d, q, kv = self.n_embd, self.n_head * self.head_dim, self.n_kv_head * self.head_dim
+        per = {"norm1.weight": (d,), "mixer.q_proj.weight": (q, d), "mixer.k_proj.weight": (kv, d),
+               "mixer.v_proj.weight": (kv, d), "mixer.o_proj.weight": (d, q), "mixer.q_norm.weight": (self.head_dim,),
+               "mixer.k_norm.weight": (self.head_dim,), "mixer.gate.weight": (self.n_head, d),
+               "mixer.gate.bias": (self.n_head,), "mixer.vr_lambda": (1,), "norm2.weight": (d,),
+               "ffn.gate.weight": (self.hidden, d), "ffn.up.weight": (self.hidden, d),
+               "ffn.down.weight": (d, self.hidden)}
+        shapes = {"tok_emb.weight": (self.vocab, d), "norm_f.weight": (d,)}
+        for i in range(self.n_layer):
+            for n, shp in per.items():
+                shapes[f"blocks.{i}.{n}"] = shp
+        return shapes
+
+
+def rope_tables(spec: NanolabSpec, seq: int):
+    """`Rope::rows` (ojas-model/src/block.rs:31-71): angles in f64, one rounding to f32, both
+    halves of a row equal. Host arrays; upload them once."""
+    half = spec.head_dim // 2
+    inv = np.array([spec.rope_base ** (-(2 * i) / spec.head_dim) for i in range(half)], np.float64)
+    ang = np.arange(seq, dtype=np.float64)[:, None] * inv[None, :]
+    cos = np.concatenate([np.cos(ang), np.cos(ang)], axis=1).astype(np.float32)
+    sin = np.concatenate([np.sin(ang), np.sin(ang)], axis=1).astype(np.float32)
+    return cos, sin
+
+
+class NanolabGraph:
+    """Runs the graph on one backend. `params` maps names to f32 device tensors."""
+
+    def __init__(self, be: MiBackend, spec: NanolabSpec, params: Dict[str, DeviceTensor]):
+        self.be, self.spec, self.p = be, spec, params
+
+    def _blk(self, i: int, name: str) -> DeviceTensor:
+        return self.p[f"blocks.{i}.{name}"]
+
+    def loss_and_grads(self, ids: DeviceTensor, targets: DeviceTensor, want_logits: bool = False):
+        """Returns (loss [1] f32, logits or None, {name: gradient}). `ids`, `targets` are u32 [B, T]."""
+        be, s = self.be, self.spec
+        B, T = ids.shape
+        N, d, H, KV, D = B * T, s.n_embd, s.n_head, s.n_kv_head, s.head_dim
+        eps, win = s.rms_eps, s.window
+        cos_h, sin_h = rope_tables(s, T)
+        cos, sin = be.upload(cos_h), be.upload(sin_h)
+        swap = [0, 2, 1, 3]
+
+        # ---- forward (block.rs:218-264) ----
+        x = be.embedding_forward(self.p["tok_emb.weight"], ids).reshape(N, d)
+        acts = []
+        v0 = None
+        for i in range(s.n_layer):
+            a = {"x": x}
+            a["h"] = be.rms_norm_forward(x, self._blk(i, "norm1.weight"), eps)
+            a["q_lin"] = be.linear_forward(a["h"], self._blk(i, "mixer.q_proj.weight")).reshape(B, T, H, D)
+            a["k_lin"] = be.linear_forward(a["h"], self._blk(i, "mixer.k_proj.weight")).reshape(B, T, KV, D)
+            a["raw_v"] = be.linear_forward(a["h"], self._blk(i, "mixer.v_proj.weight")).reshape(B, T, KV, D)
+            qn, kn = be.rms_qk_norm_forward(a["q_lin"], a["k_lin"], self._blk(i, "mixer.q_norm.weight"),
+                                            self._blk(i, "mixer.k_norm.weight"), eps)
+            q = be.rope_half_split_forward(qn, cos, sin)
+            k = be.rope_half_split_forward(kn, cos, sin)
+            if v0 is None:
+                v = a["raw_v"]
+                v0 = a["raw_v"]
+            else:
+                v = be.value_residual_blend_forward(a["raw_v"], v0, self._blk(i, "mixer.vr_lambda"))
+            a["qp"], a["kp"], a["vp"] = be.permute(q, swap), be.permute(k, swap), be.permute(v, swap)
+            a["att"], a["lse"] = be.causal_sdpa_forward(a["qp"], a["kp"], a["vp"], win)
+            a["ap"] = be.permute(a["att"], swap)  # [B, T, H, D]
+            a["y"], a["scales"] = be.per_head_sigmoid_gate_forward_saving(
+                a["h"].reshape(B, T, d), self._blk(i, "mixer.gate.weight"), self._blk(i, "mixer.gate.bias"), a["ap"])
+            o = be.linear_forward(a["y"].reshape(N, H * D), self._blk(i, "mixer.o_proj.weight"))
+            a["x1"] = be.residual_add_forward(x, o)
+            a["h2"] = be.rms_norm_forward(a["x1"], self._blk(i, "norm2.weight"), eps)
+            a["g_lin"] = be.linear_forward(a["h2"], self._blk(i, "ffn.gate.weight"))
+            a["g_act"] = be.silu_forward(a["g_lin"])
+            a["up"] = be.linear_forward(a["h2"], self._blk(i, "ffn.up.weight"))
+            a["m"] = be.mul_forward(a["g_act"], a["up"])
+            down = be.linear_forward(a["m"], self._blk(i, "ffn.down.weight"))
+            x = be.residual_add_forward(a["x1"], down)
+            acts.append(a)
+        hf = be.rms_norm_forward(x, self.p["norm_f.weight"], eps)
+        logits = be.linear_forward(hf, self.p["tok_emb.weight"]) if want_logits else None
+        tflat = targets.reshape(N)
+        loss, ghf, g_head = be.linear_cross_entropy_mean(hf, self.p["tok_emb.weight"], tflat)
+
+        # ---- backward: reverse program order; a value's consumers add their gradients later one first ----
+        grads: Dict[str, DeviceTensor] = {}
+        gx, grads["norm_f.weight"] = be.rms_norm_backward(x, self.p["norm_f.weight"], ghf, eps)
+        g_v0 = None  # gradient of block 0's raw v from the later blocks' blends
+        for i in reversed(range(s.n_layer)):
+            a = acts[i]
+            gm, grads[f"blocks.{i}.ffn.down.weight"] = be.linear_backward(a["m"], self._blk(i, "ffn.down.weight"), gx)
+            g_gact, g_up = be.mul_backward(a["g_act"], a["up"], gm)
+            gh2, grads[f"blocks.{i}.ffn.up.weight"] = be.linear_backward(a["h2"], self._blk(i, "ffn.up.weight"), g_up)
+            g_glin = be.silu_backward(a["g_lin"], g_gact)
+            part, grads[f"blocks.{i}.ffn.gate.weight"] = be.linear_backward(a["h2"], self._blk(i, "ffn.gate.weight"),
+                                                                           g_glin)
+            gh2 = be.residual_add_forward(gh2, part)
+            gt, grads[f"blocks.{i}.norm2.weight"] = be.rms_norm_backward(a["x1"], self._blk(i, "norm2.weight"), gh2, eps)
+            gx1 = be.residual_add_forward(gx, gt)
+            gy, grads[f"blocks.{i}.mixer.o_proj.weight"] = be.linear_backward(
+                a["y"].reshape(N, H * D), self._blk(i, "mixer.o_proj.weight"), gx1)
+            gh, grads[f"blocks.{i}.mixer.gate.weight"], grads[f"blocks.{i}.mixer.gate.bias"], gap = \
+                be.per_head_sigmoid_gate_backward_saved(a["h"].reshape(B, T, d), self._blk(i, "mixer.gate.weight"),
+                                                        self._blk(i, "mixer.gate.bias"), a["ap"],
+                                                        gy.reshape(B, T, H, D), a["scales"])
+            gh = gh.reshape(N, d)
+            ga = be.permute(gap, swap)
+            gqp, gkp, gvp = be.causal_sdpa_backward(a["qp"], a["kp"], a["vp"], a["att"], a["lse"], ga, win)
+            gv, gk, gq = be.permute(gvp, swap), be.permute(gkp, swap), be.permute(gqp, swap)
+            if i == 0:
+                g_raw_v = gv if g_v0 is None else be.residual_add_forward(g_v0, gv)
+                grads["blocks.0.mixer.vr_lambda"] = be.zeros((1,), F32)
+            else:
+                g_raw_v, part_v0, grads[f"blocks.{i}.mixer.vr_lambda"] = be.value_residual_blend_backward(
+                    a["raw_v"], acts[0]["raw_v"], self._blk(i, "mixer.vr_lambda"), gv)
+                g_v0 = part_v0 if g_v0 is None else be.residual_add_forward(g_v0, part_v0)
+            gkn = be.rope_half_split_backward(gk, cos, sin)
+            gqn = be.rope_half_split_backward(gq, cos, sin)
+            gq_lin, gk_lin, grads[f"blocks.{i}.mixer.q_norm.weight"], grads[f"blocks.{i}.mixer.k_norm.weight"] = \
+                be.rms_qk_norm_backward(a["q_lin"], a["k_lin"], self._blk(i, "mixer.q_norm.weight"),
+                                        self._blk(i, "mixer.k_norm.weight"), gqn, gkn, eps)
+            for name, g_out in (("v_proj", g_raw_v.reshape(N, KV * D)), ("k_proj", gk_lin.reshape(N, KV * D)),
+                                ("q_proj", gq_lin.reshape(N, H * D))):
+                part, grads[f"blocks.{i}.mixer.{name}.weight"] = be.linear_backward(
+                    a["h"], self._blk(i, f"mixer.{name}.weight"), g_out)
+                gh = be.residual_add_forward(gh, part)
+            gt, grads[f"blocks.{i}.norm1.weight"] = be.rms_norm_backward(a["x"], self._blk(i, "norm1.weight"), gh, eps)
+            gx = be.residual_add_forward(gx1, gt)
+        # The tied table: the head's gradient first, then the embedding's rows.
+        g_emb = be.embedding_backward(ids.reshape(N), gx, s.vocab)
+        grads["tok_emb.weight"] = be.residual_add_forward(g_head, g_emb)
+        return loss, logits, grads

@@ -1,0 +1,130 @@
+"""The nanolab GPT graph on the GPU, op by op through the C ABI (`ojas_amd/nanolab.py`), against the
+reference's torch fixtures at the gates it holds its own device backends to
+(ojas-model/tests/oracle_parity.rs:60-92: GPU_GATES = Gates::EXACT for these quantities; constants
+ojas-oracle/src/parity.rs:28-40), and against the CPU oracle on parameters that keep every gradient
+path live."""
+import json
+from pathlib import Path
+
+import numpy as np
+import pytest
+from safetensors import safe_open
+
+import oracle_api as orc
+
+pytestmark = pytest.mark.gpu
+
+TINY = Path(__file__).parent / "golden" / "tiny"
+FORWARD_LOSS_REL_TOL = 1e-5
+LOGITS_NORMWISE_REL_TOL = 1e-5
+GRAD_NORMWISE_REL_TOL = 1e-4
+
+
+@pytest.fixture(scope="module")
+def be():
+    from ojas_amd.backend import MiBackend
+
+    backend = MiBackend(0)
+    yield backend
+    backend.close()
+
+
+def load(name):
+    with safe_open(str(TINY / f"{name}.safetensors"), "np") as f:
+        meta = {k: json.loads(v) for k, v in (f.metadata() or {}).items()}
+        return {k: f.get_tensor(k) for k in f.keys()}, meta
+
+
+def tiny_spec():
+    from ojas_amd.nanolab import NanolabSpec
+
+    _, meta = load("init")
+    s = meta["ojas.spec"]
+    return NanolabSpec(n_layer=s["n_layer"], n_embd=s["n_embd"], n_head=s["n_head"], n_kv_head=s["n_kv_head"],
+                       head_dim=s["head_dim"], hidden=s["hidden"], vocab=s["vocab"], rms_eps=s["rms_eps"],
+                       rope_base=s["rope_base"])
+
+
+def run(be, spec, host_params, ids, targets, want_logits=False):
+    from ojas_amd.nanolab import NanolabGraph
+
+    shapes = spec.param_shapes()
+    params = {n: be.upload(np.ascontiguousarray(host_params[n], np.float32).reshape(shapes[n]))
+              for n in spec.param_names()}
+    graph = NanolabGraph(be, spec, params)
+    loss, logits, grads = graph.loss_and_grads(be.upload(ids.astype(np.uint32)), be.upload(targets.astype(np.uint32)),
+                                               want_logits)
+    return (float(be.download(loss)[0]), None if logits is None else be.download(logits),
+            {n: be.download(g) for n, g in grads.items()})
+
+
+def test_tiny_fixture_forward_and_gradients(be):
+    print("nanolab tiny fixture on the device", flush=True)
+    spec = tiny_spec()
+    init, _ = load("init")
+    fwd, fmeta = load("forward")
+    want, gmeta = load("grads_init")
+    info = gmeta["ojas.oracle"]
+    loss, logits, grads = run(be, spec, init, fwd["x"], fwd["y"], want_logits=True)
+    want_loss = fmeta["ojas.oracle"]["loss"]
+    assert abs(loss - want_loss) <= FORWARD_LOSS_REL_TOL * abs(want_loss), (loss, want_loss)
+    ref = fwd["logits"].reshape(-1, spec.vocab).astype(np.float64)
+    rel = np.linalg.norm(logits.reshape(ref.shape) - ref) / np.linalg.norm(ref)
+    assert rel <= LOGITS_NORMWISE_REL_TOL, rel
+    seed = np.float32(info["loss_seed"])
+    checked = 0
+    for name in spec.param_names():
+        got = grads[name].reshape(-1)
+        if name in info["no_grad"]:
+            assert not np.any(got), name
+            continue
+        ref = want[name].reshape(-1).astype(np.float64)
+        if name in info["zero_grad"]:
+            assert not np.any(ref) and not np.any(got), f"{name}: torch's gradient is exactly zero"
+            continue
+        rel = np.linalg.norm(got * seed - ref) / np.linalg.norm(ref)
+        assert rel <= GRAD_NORMWISE_REL_TOL, (name, rel)
+        checked += 1
+    assert checked == 6
+
+
+@pytest.mark.parametrize("kv_heads,window", [(4, None), (2, None), (1, 7)])
+def test_every_gradient_against_the_oracle(be, kv_heads, window):
+    """Random parameters (o_proj and ffn.down not zero), grouped heads and a window: loss 1e-5
+    relative, every gradient 1e-4 normwise against CPU Exact, the reference's device gates."""
+    from ojas_amd.nanolab import NanolabSpec
+
+    print(f"nanolab vs oracle kv_heads={kv_heads} window={window}", flush=True)
+    spec = NanolabSpec(n_layer=3, n_embd=64, n_head=4, n_kv_head=kv_heads, head_dim=16, hidden=96, vocab=128,
+                       window=window)
+    B, T = 2, 24
+    r = orc.SplitMix64(4242 + kv_heads)
+    shapes = spec.param_shapes()
+    host = {}
+    for name in spec.param_names():
+        n = int(np.prod(shapes[name]))
+        if "norm" in name:
+            host[name] = 1.0 + r.vec(n, 0.2)
+        elif name.endswith("vr_lambda"):
+            host[name] = r.vec(n, 1.0)
+        elif name.endswith("gate.bias"):
+            host[name] = r.vec(n, 0.5)
+        else:
+            host[name] = r.vec(n, 0.25)
+    ids = np.array([r.below(spec.vocab) for _ in range(B * T)], np.uint32).reshape(B, T)
+    targets = np.array([r.below(spec.vocab) for _ in range(B * T)], np.uint32).reshape(B, T)
+    loss, _, grads = run(be, spec, host, ids, targets)
+    cfg = orc.NanolabConfig(layers=spec.n_layer, n_embd=spec.n_embd, n_head=spec.n_head, n_kv_head=spec.n_kv_head,
+                            head_dim=spec.head_dim, hidden=spec.hidden, vocab=spec.vocab, batch=B, seq=T,
+                            window=window or 0, rms_eps=spec.rms_eps, rope_base=spec.rope_base)
+    names = spec.param_names()
+    assert names == orc.nanolab_param_names(spec.n_layer)
+    o_loss, _, o_grads = orc.nanolab_loss_and_grads(cfg, [host[n] for n in names], ids, targets)
+    assert abs(loss - float(o_loss)) <= FORWARD_LOSS_REL_TOL * abs(float(o_loss)), (loss, o_loss)
+    for name, ref in zip(names, o_grads):
+        got = grads[name].reshape(-1).astype(np.float64)
+        if name == "blocks.0.mixer.vr_lambda":
+            assert not np.any(got) and not np.any(ref)
+            continue
+        rel = np.linalg.norm(got - ref) / max(np.linalg.norm(ref), 1e-30)
+        assert rel <= GRAD_NORMWISE_REL_TOL, (name, rel)
