@@ -28,6 +28,11 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, vendor figure
+# HBM bytes per GEMM op (MFMA kernel + split-K reduce) on the gpt124m workload, averaged over the
+# step's 156 ops: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by what the same
+# counters read for the AdamW pass, whose traffic is known (profiles/gemm_hbm_traffic_gpt124m_bf16.txt).
+# The algorithmic figure (every operand read once, every output written once) is 1.569e8.
+GEMM_HBM_BYTES_PER_LAUNCH_GPT124M = 3.69e8
 
 
 def cpu_baseline(cfg, threads: int):
@@ -119,9 +124,10 @@ def main() -> int:
         "step_tflops": flops / (ms_per_step * 1e-3) / 1e12,
         "pct_bf16_mfma_peak": 100.0 * flops / (ms_per_step * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS,
         "loss_first": losses[0], "loss_last": losses[-1],
-        "roofline": {"bound": "mfma", "kernel": "gemm_kernel (bf16 MFMA, all operand layouts)",
+        "roofline": {"bound": "mfma", "kernel": "gemm_dma_kernel / gemm_kernel (bf16 MFMA GEMM, all operand layouts)",
                      "achieved": achieved, "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / BF16_MFMA_PEAK_TFLOPS, "traffic": None,
+                     "frac": achieved / BF16_MFMA_PEAK_TFLOPS,
+                     "traffic": GEMM_HBM_BYTES_PER_LAUNCH_GPT124M if args.config == "gpt124m" else None,
                      "launches": int(launches.value), "avg_launch_us": gemm_ms.value * 1e3 / max(1, launches.value),
                      "gemm_ms_per_step": gemm_ms.value / args.steps},
     }
