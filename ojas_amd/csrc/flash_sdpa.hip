@@ -48,7 +48,6 @@ struct FlashShape {
   FlashStrides q, kv, o;  // q and grad_q; k, v and their gradients; out and grad_out
 };
 
-__device__ __forceinline__ int perm16(int k) { return (k & ~12) | ((k & 4) << 1) | ((k & 8) >> 1); }
 
 __device__ __forceinline__ unsigned int pack2(float a, float b) {
   floatx2 f = {a, b};
@@ -93,29 +92,26 @@ __device__ __forceinline__ void tile_store_rows(char* lds, const u32x4 r[2]) {
   *reinterpret_cast<u32x4*>(lds + row * FPITCH + kc * 16) = r[0];
   *reinterpret_cast<u32x4*>(lds + (row + 1) * FPITCH + kc * 16) = r[1];
 }
-// [d][row'] form, row' = perm16(row): the two rows a thread holds stay adjacent.
-__device__ __forceinline__ void tile_store_transposed(char* lds, const u32x4 r[2]) {
-  const int t = threadIdx.x;
-  const int row = 2 * (t >> 3), kc = t & 7;
-  const int col_bytes = perm16(row) * 2;
-  const unsigned int a[4] = {r[0].x, r[0].y, r[0].z, r[0].w};
-  const unsigned int b[4] = {r[1].x, r[1].y, r[1].z, r[1].w};
-#pragma unroll
-  for (int w = 0; w < 4; ++w) {
-    // Elements 2w and 2w+1 of both rows.
-    unsigned int lo = (a[w] & 0xffffu) | (b[w] << 16);
-    unsigned int hi = (a[w] >> 16) | (b[w] & 0xffff0000u);
-    *reinterpret_cast<unsigned int*>(lds + (kc * 8 + 2 * w) * FPITCH + col_bytes) = lo;
-    *reinterpret_cast<unsigned int*>(lds + (kc * 8 + 2 * w + 1) * FPITCH + col_bytes) = hi;
-  }
-}
 // A operand from a [row][d] tile: rows sub*32 + lane%32, d-slab kk.
 __device__ __forceinline__ u32x4 frag_rows(const char* lds, int sub, int kk, int l32, int lg) {
   return *reinterpret_cast<const u32x4*>(lds + (sub * 32 + l32) * FPITCH + kk * 32 + lg * 16);
 }
-// A operand from a transposed tile: rows (= d) mt*32 + lane%32, k-slab c of sub-tile sub.
-__device__ __forceinline__ u32x4 frag_transposed(const char* lds, int mt, int sub, int c, int l32, int lg) {
-  return *reinterpret_cast<const u32x4*>(lds + (mt * 32 + l32) * FPITCH + (sub * 32 + c * 16 + lg * 8) * 2);
+// A operand of a product whose K index is the tile's ROW (O^T = V^T P^T, dV^T = dO^T P,
+// dK^T = Q^T dS, dQ^T = K^T dS^T), read straight from the [row][d] tile with the transposing LDS
+// read: a 16-lane group fetches a 4-row x 16-column block (8 bytes per lane) and each lane gets
+// one column's 4 rows. Lane (i = lane % 32, g = lane / 32) ends up with column d = mt*32 + i and
+// rows sub*32 + 16c + {4g..4g+3, 8+4g..8+4g+3}: the order in which an accumulator tile, reused as
+// the B operand, holds its rows.
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ u32x4 frag_tr(const char* lds, int mt, int sub, int c, int lane) {
+  const int s = lane & 15, half = (lane >> 4) & 1, g = lane >> 5;
+  const char* p = lds + (sub * 32 + c * 16 + 4 * g + (s >> 2)) * FPITCH + (mt * 32 + half * 16 + (s & 3) * 4) * 2;
+  typedef short4v __attribute__((address_space(3))) * lds_ptr;
+  const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
+  const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 8 * FPITCH));
+  const u32x2 a = __builtin_bit_cast(u32x2, lo), b = __builtin_bit_cast(u32x2, hi);
+  return u32x4{a.x, a.y, b.x, b.y};
 }
 // B operand held in registers: the lane's own row of a [time, 64] plane.
 __device__ __forceinline__ void row_frags(const unsigned short* __restrict__ plane, long rs, int row, int time, int lg,
@@ -164,7 +160,7 @@ __global__ __launch_bounds__(FT, 3) void flash_fwd_kernel(const unsigned short* 
                                                        unsigned long long tag) {
   __shared__ __attribute__((aligned(16))) char smem[2 * FTILE];
   char* k_rows = smem;
-  char* v_tr = smem + FTILE;
+  char* v_rows = smem + FTILE;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lg = lane >> 5;
   const int T = s.time;
   // Late query blocks see the most keys: schedule them first.
@@ -193,7 +189,7 @@ __global__ __launch_bounds__(FT, 3) void flash_fwd_kernel(const unsigned short* 
     const int key0 = kt * 64;
     __syncthreads();  // the previous tile's reads are done
     tile_store_rows(k_rows, rk);
-    tile_store_transposed(v_tr, rv);
+    tile_store_rows(v_rows, rv);
     __syncthreads();
     if (kt < kt_last) {
       tile_load(kp, s.kv.rs, key0 + 64, T, rk);
@@ -252,7 +248,7 @@ __global__ __launch_bounds__(FT, 3) void flash_fwd_kernel(const unsigned short* 
       for (int c = 0; c < 2; ++c) {
         const u32x4 pb = pack8(sc[sub], c);
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt) o[mt] = mfma(frag_transposed(v_tr, mt, sub, c, l32, lg), pb, o[mt]);
+        for (int mt = 0; mt < 2; ++mt) o[mt] = mfma(frag_tr(v_rows, mt, sub, c, lane), pb, o[mt]);
       }
   }
   bool bad = false;
@@ -270,12 +266,10 @@ __global__ __launch_bounds__(FT, 2) void flash_bwd_dkv_kernel(
     const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
     const float* __restrict__ lse, const float* __restrict__ delta, const unsigned short* __restrict__ gy,
     TO* __restrict__ gk, TO* __restrict__ gv, FlashShape s, OmxFaultWord* fault, unsigned long long tag) {
-  __shared__ __attribute__((aligned(16))) char smem[4 * FTILE + 2 * 64 * 4];
+  __shared__ __attribute__((aligned(16))) char smem[2 * FTILE + 2 * 64 * 4];
   char* q_rows = smem;
   char* g_rows = smem + FTILE;
-  char* q_tr = smem + 2 * FTILE;
-  char* g_tr = smem + 3 * FTILE;
-  float* lse_s = reinterpret_cast<float*>(smem + 4 * FTILE);
+  float* lse_s = reinterpret_cast<float*>(smem + 2 * FTILE);
   float* del_s = lse_s + 64;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lg = lane >> 5;
   const int T = s.time;
@@ -330,8 +324,6 @@ __global__ __launch_bounds__(FT, 2) void flash_bwd_dkv_kernel(
       __syncthreads();
       tile_store_rows(q_rows, rq);
       tile_store_rows(g_rows, rg);
-      tile_store_transposed(q_tr, rq);
-      tile_store_transposed(g_tr, rg);
       if (threadIdx.x < 64) {
         lse_s[threadIdx.x] = row_lse * LOG2E;
         del_s[threadIdx.x] = row_del;
@@ -378,8 +370,8 @@ __global__ __launch_bounds__(FT, 2) void flash_bwd_dkv_kernel(
           const u32x4 pb = pack8(sc, c), dsb = pack8(dp, c);
 #pragma unroll
           for (int mt = 0; mt < 2; ++mt) {
-            dv[mt] = mfma(frag_transposed(g_tr, mt, sub, c, l32, lg), pb, dv[mt]);
-            dk[mt] = mfma(frag_transposed(q_tr, mt, sub, c, l32, lg), dsb, dk[mt]);
+            dv[mt] = mfma(frag_tr(g_rows, mt, sub, c, lane), pb, dv[mt]);
+            dk[mt] = mfma(frag_tr(q_rows, mt, sub, c, lane), dsb, dk[mt]);
           }
         }
       }
@@ -394,12 +386,12 @@ __global__ __launch_bounds__(FT, 2) void flash_bwd_dkv_kernel(
 template <typename TO>
 __global__ __launch_bounds__(FT, 3) void flash_bwd_dq_kernel(
     const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
-    const float* __restrict__ lse, const float* __restrict__ delta, const unsigned short* __restrict__ gy,
-    TO* __restrict__ gq, FlashShape s, OmxFaultWord* fault, unsigned long long tag) {
-  __shared__ __attribute__((aligned(16))) char smem[3 * FTILE];
+    const unsigned short* __restrict__ out, const float* __restrict__ lse, float* __restrict__ delta,
+    const unsigned short* __restrict__ gy, TO* __restrict__ gq, FlashShape s, OmxFaultWord* fault,
+    unsigned long long tag) {
+  __shared__ __attribute__((aligned(16))) char smem[2 * FTILE];
   char* k_rows = smem;
   char* v_rows = smem + FTILE;
-  char* k_tr = smem + 2 * FTILE;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lg = lane >> 5;
   const int T = s.time;
   const int qb = gridDim.x - 1 - blockIdx.x;
@@ -413,11 +405,29 @@ __global__ __launch_bounds__(FT, 3) void flash_bwd_dq_kernel(
   u32x4 qf[4], gf[4];
   row_frags(q + b * s.q.bs + h * s.q.hs, s.q.rs, q_row, T, lg, qf);
   row_frags(gy + b * s.o.bs + h * s.o.hs, s.o.rs, q_row, T, lg, gf);
-  float row_lse = 0.0f, row_del = 0.0f;
+  // delta = dO . O of this lane's row: each half-wave holds half of the row's 64 values. The
+  // dK/dV pass, launched after this one, reads it back from `delta`.
+  float row_del = 0.0f;
+  {
+    u32x4 of[4];
+    row_frags(out + b * s.o.bs + h * s.o.hs, s.o.rs, q_row, T, lg, of);
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      const unsigned int gw[4] = {gf[kk].x, gf[kk].y, gf[kk].z, gf[kk].w};
+      const unsigned int ow[4] = {of[kk].x, of[kk].y, of[kk].z, of[kk].w};
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        row_del += __uint_as_float(gw[w] << 16) * __uint_as_float(ow[w] << 16);
+        row_del += __uint_as_float(gw[w] & 0xffff0000u) * __uint_as_float(ow[w] & 0xffff0000u);
+      }
+    }
+    row_del += __shfl_xor(row_del, 32, 64);
+  }
+  float row_lse = 0.0f;
   bool bad = false;
   if (q_row < T) {
     row_lse = lse[plane * T + q_row];
-    row_del = delta[plane * T + q_row];
+    if (lg == 0) delta[plane * T + q_row] = row_del;
     bad |= !(dev_finite(row_lse) && dev_finite(row_del));
   }
   const float neg_lse = -row_lse * LOG2E;
@@ -434,7 +444,6 @@ __global__ __launch_bounds__(FT, 3) void flash_bwd_dq_kernel(
     __syncthreads();
     tile_store_rows(k_rows, rk);
     tile_store_rows(v_rows, rv);
-    tile_store_transposed(k_tr, rk);
     __syncthreads();
     if (kt < kt_last) {
       tile_load(kp, s.kv.rs, key0 + 64, T, rk);
@@ -468,26 +477,12 @@ __global__ __launch_bounds__(FT, 3) void flash_bwd_dq_kernel(
       for (int c = 0; c < 2; ++c) {
         const u32x4 dsb = pack8(dp, c);
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt) dq[mt] = mfma(frag_transposed(k_tr, mt, sub, c, l32, lg), dsb, dq[mt]);
+        for (int mt = 0; mt < 2; ++mt) dq[mt] = mfma(frag_tr(k_rows, mt, sub, c, lane), dsb, dq[mt]);
       }
     }
   }
   bad |= store_transposed_acc<TO>(gq + b * s.q.bs + h * s.q.hs, s.q.rs, q_row, T, lg, dq, s.scale);
   if (bad) dev_raise_fault(fault, tag);
-}
-
-// delta[b, h, t] = dO[b, h, t, :] . O[b, h, t, :], one wave per row.
-__global__ __launch_bounds__(FT) void flash_delta_kernel(const unsigned short* __restrict__ out,
-                                                         const unsigned short* __restrict__ gy,
-                                                         float* __restrict__ delta, long rows, FlashShape s) {
-  const int lane = threadIdx.x & 63;
-  const long row = static_cast<long>(blockIdx.x) * 4 + (threadIdx.x >> 6);
-  if (row >= rows) return;
-  const long t = row % s.time, plane = row / s.time;
-  const long at = (plane / s.heads) * s.o.bs + (plane % s.heads) * s.o.hs + t * s.o.rs + lane;
-  float acc = dev_bf16_bits_to_f32(gy[at]) * dev_bf16_bits_to_f32(out[at]);
-  acc = wave_sum(acc);
-  if (lane == 0) delta[row] = acc;
 }
 
 // `strides`: nine element strides (row, head, batch of q; of k / v; of out), or null for
@@ -553,22 +548,20 @@ int32_t omx_flash_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, cons
   const unsigned short* vs = static_cast<const unsigned short*>(v);
   const unsigned short* os = static_cast<const unsigned short*>(out);
   const unsigned short* gs = static_cast<const unsigned short*>(gy);
-  hipLaunchKernelGGL(flash_delta_kernel, dim3(static_cast<unsigned>((rows + 3) / 4)), dim3(FT), 0, ctx->stream, os, gs,
-                     delta, rows, s);
-  OMX_LAUNCH_CHECK(ctx, "flash_delta_kernel");
+  // dQ first: it also leaves delta = dO . O per row for the dK/dV pass.
   dim3 block(FT);
   dim3 kv_grid(static_cast<unsigned>((time + 127) / 128), static_cast<unsigned>(batch * kv_heads));
   dim3 q_grid(static_cast<unsigned>((time + 127) / 128), static_cast<unsigned>(batch * heads));
   if (grad_dtype == OMX_BF16) {
+    hipLaunchKernelGGL((flash_bwd_dq_kernel<unsigned short>), q_grid, block, 0, ctx->stream, qs, ks, vs, os, lse, delta,
+                       gs, static_cast<unsigned short*>(gq), s, ctx->fault, tag);
     hipLaunchKernelGGL((flash_bwd_dkv_kernel<unsigned short>), kv_grid, block, 0, ctx->stream, qs, ks, vs, lse, delta,
                        gs, static_cast<unsigned short*>(gk), static_cast<unsigned short*>(gv), s, ctx->fault, tag);
-    hipLaunchKernelGGL((flash_bwd_dq_kernel<unsigned short>), q_grid, block, 0, ctx->stream, qs, ks, vs, lse, delta,
-                       gs, static_cast<unsigned short*>(gq), s, ctx->fault, tag);
   } else {
+    hipLaunchKernelGGL((flash_bwd_dq_kernel<float>), q_grid, block, 0, ctx->stream, qs, ks, vs, os, lse, delta, gs,
+                       static_cast<float*>(gq), s, ctx->fault, tag);
     hipLaunchKernelGGL((flash_bwd_dkv_kernel<float>), kv_grid, block, 0, ctx->stream, qs, ks, vs, lse, delta, gs,
                        static_cast<float*>(gk), static_cast<float*>(gv), s, ctx->fault, tag);
-    hipLaunchKernelGGL((flash_bwd_dq_kernel<float>), q_grid, block, 0, ctx->stream, qs, ks, vs, lse, delta, gs,
-                       static_cast<float*>(gq), s, ctx->fault, tag);
   }
   OMX_LAUNCH_CHECK(ctx, "flash backward kernels");
   return OMX_OK;
