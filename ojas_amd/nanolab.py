@@ -14,7 +14,7 @@ from typing import Dict, List, Optional, Sequence
 
 import numpy as np
 
-from .backend import F32, MiBackend, DeviceTensor
+from .backend import F32, AdamWConfig, MiBackend, MuonNs5Config, DeviceTensor, OjasError, NON_FINITE, OUT_OF_RANGE
 
 BLOCK_PARAMS = ("norm1.weight", "mixer.q_proj.weight", "mixer.k_proj.weight", "mixer.v_proj.weight",
                 "mixer.o_proj.weight", "mixer.q_norm.weight", "mixer.k_norm.weight", "mixer.gate.weight",
@@ -77,8 +77,10 @@ class NanolabGraph:
     def _blk(self, i: int, name: str) -> DeviceTensor:
         return self.p[f"blocks.{i}.{name}"]
 
-    def loss_and_grads(self, ids: DeviceTensor, targets: DeviceTensor, want_logits: bool = False):
-        """Returns (loss [1] f32, logits or None, {name: gradient}). `ids`, `targets` are u32 [B, T]."""
+    def loss_and_grads(self, ids: DeviceTensor, targets: DeviceTensor, want_logits: bool = False,
+                       loss_seed: float = 1.0):
+        """Returns (loss [1] f32, logits or None, {name: gradient}). `ids`, `targets` are u32 [B, T].
+        `loss_seed` is the gradient of the loss the backward starts from (`Tape::backward_seeded`)."""
         be, s = self.be, self.spec
         B, T = ids.shape
         N, d, H, KV, D = B * T, s.n_embd, s.n_head, s.n_kv_head, s.head_dim
@@ -125,6 +127,9 @@ class NanolabGraph:
         logits = be.linear_forward(hf, self.p["tok_emb.weight"]) if want_logits else None
         tflat = targets.reshape(N)
         loss, ghf, g_head = be.linear_cross_entropy_mean(hf, self.p["tok_emb.weight"], tflat)
+        if loss_seed != 1.0:
+            be.scale_grad(ghf, loss_seed)
+            be.scale_grad(g_head, loss_seed)
 
         # ---- backward: reverse program order; a value's consumers add their gradients later one first ----
         grads: Dict[str, DeviceTensor] = {}
@@ -174,3 +179,92 @@ class NanolabGraph:
         g_emb = be.embedding_backward(ids.reshape(N), gx, s.vocab)
         grads["tok_emb.weight"] = be.residual_add_forward(g_head, g_emb)
         return loss, logits, grads
+
+
+# ojas-cpu/src/train.rs:20-62
+MUON_MOMENTUM = 0.99
+MUON_WEIGHT_DECAY = 0.1
+ADAM_HYBRID_WEIGHT_DECAY = 0.0
+FROZEN = ("blocks.0.mixer.vr_lambda",)  # block 0 has no earlier value to blend with: no gradient reaches it
+
+
+@dataclass
+class StepReport:
+    """`ojas_model::StepReport` (ojas-model/src/trainer.rs:280-297)."""
+    loss: float
+    grad_norm: float
+    lr_multiplier: float
+    step: int
+    tokens: int
+
+
+class NanolabTrainer:
+    """`Trainer::run` (ojas-model/src/trainer.rs:754-857) for the f32 tier: micro-batches weighted
+    by their share of the step's valid targets and seeded into the backward (:1089-1119), gradients
+    summed with `accumulate_grad` (:973-978), one `clip_grad_norm`, then per parameter `muon_ns5_step`
+    (matrices other than the embedding) or `adamw_step` (the embedding and the vectors) at the group's
+    peak rate times the schedule multiplier (:858-876, :1004-1028). The multiplier is the caller's:
+    the schedule is host arithmetic outside this path."""
+
+    def __init__(self, be: MiBackend, spec: NanolabSpec, host_params: Dict[str, np.ndarray], adam_lr: float = 6e-4,
+                 matrix_lr: float = 0.025, grad_clip: float = 1.0, ns5_bf16: bool = False):
+        self.be, self.spec = be, spec
+        self.adam_lr, self.matrix_lr, self.grad_clip, self.ns5_bf16 = adam_lr, matrix_lr, grad_clip, ns5_bf16
+        shapes = spec.param_shapes()
+        self.names = spec.param_names()
+        self.params = {n: be.upload(np.ascontiguousarray(host_params[n], np.float32).reshape(shapes[n]))
+                       for n in self.names}
+        self.trainable = [n for n in self.names if n not in FROZEN]
+        self.muon = {n for n in self.trainable if len(shapes[n]) == 2 and n != "tok_emb.weight"}
+        self.state = {n: [be.zeros(shapes[n], F32)] if n in self.muon else [be.zeros(shapes[n], F32),
+                                                                              be.zeros(shapes[n], F32)]
+                      for n in self.trainable}
+        self.graph = NanolabGraph(be, spec, self.params)
+        self.step = 0
+
+    def run(self, batches: Sequence, lr_multiplier: float, ignore_index: Optional[int] = None) -> StepReport:
+        """`batches`: (ids, targets) u32 host arrays [B, T], one per micro-batch."""
+        be = self.be
+        counts = [int(np.count_nonzero(y != ignore_index)) if ignore_index is not None else int(y.size)
+                  for _, y in batches]
+        live = [c for c in counts if c > 0]
+        if not batches:
+            raise OjasError(OUT_OF_RANGE, "Trainer::step: 0 micro-batches")
+        if not live:
+            raise OjasError(NON_FINITE, "Trainer::step: no valid target")
+        uniform = all(c == live[0] for c in live)
+        total = sum(counts)
+        acc, loss_sum = None, None
+        for (ids, targets), count in zip(batches, counts):
+            if count == 0:
+                continue
+            weight = float(np.float32(1.0 / len(live))) if uniform else float(np.float32(count / total))
+            loss, _, grads = self.graph.loss_and_grads(be.upload(np.ascontiguousarray(ids, np.uint32)),
+                                                       be.upload(np.ascontiguousarray(targets, np.uint32)),
+                                                       loss_seed=weight)
+            if acc is None:
+                acc = {n: grads[n] for n in self.trainable}
+            else:
+                for n in self.trainable:
+                    be.accumulate_grad(acc[n], grads[n])
+            if not uniform and weight != 1.0:
+                be.scale_grad(loss, weight)
+            loss_sum = loss if loss_sum is None else be.residual_add_forward(loss_sum, loss)
+        grad_norm = be.clip_grad_norm([acc[n] for n in self.trainable], self.grad_clip)
+        for n in self.trainable:
+            if n in self.muon:
+                cfg = MuonNs5Config(self.matrix_lr * lr_multiplier, MUON_MOMENTUM, MUON_WEIGHT_DECAY, 1,
+                                    int(self.ns5_bf16))
+                be.muon_ns5_step(self.params[n], acc[n], self.state[n][0], cfg)
+            else:
+                cfg = AdamWConfig.nanolab(self.adam_lr * lr_multiplier, ADAM_HYBRID_WEIGHT_DECAY)
+                be.adamw_step(self.params[n], acc[n], self.state[n][0], self.state[n][1], self.step, cfg)
+        value = float(be.download(loss_sum)[0])
+        if not math.isfinite(value):
+            raise OjasError(NON_FINITE, "Trainer::step")
+        self.step += 1
+        return StepReport(loss=value / len(live) if uniform else value, grad_norm=grad_norm,
+                          lr_multiplier=lr_multiplier, step=self.step, tokens=sum(int(x.size) for x, _ in batches))
+
+    def download_params(self) -> Dict[str, np.ndarray]:
+        return {n: self.be.download(t) for n, t in self.params.items()}

@@ -12,6 +12,9 @@ Run in the build container (needs /root/reference). Only DATA is taken:
   * AdamW lerp-branch rows                   ojas-cpu/tests/adamw_lerp_oracle.rs (numbers -> JSON)
   * torch 2.13 vectors of the tiny nanolab   ojas-oracle/fixtures/tiny/{init,forward,grads_init}.safetensors and
     model and of stock nanolab's Muon step   muon_step_bf16.safetensors (copied as is)
+  * the tiny model's 40-step f32-NS5 trace  ojas-oracle/fixtures/tiny/{trace_ns5_f32,grads_step5}.safetensors,
+    (losses, grad norms, step-5 parameters)  its token bin, window starts and LR multipliers: tokens.bin,
+                                             batch_starts.json, lr_schedules.json (copied as is)
 No reference source text is kept: numeric literals are parsed into JSON.
 """
 import json
@@ -67,8 +70,10 @@ def copies():
     for f in ("adamw_100.safetensors", "manifest.json"):
         shutil.copyfile(REF / "ojas-model/tests/fixtures/adamw_100" / f, OUT / "adamw_100" / f)
     (OUT / "tiny").mkdir(exist_ok=True)
-    for f in ("init", "forward", "grads_init", "muon_step_bf16"):
-        shutil.copyfile(REF / "ojas-oracle/fixtures/tiny" / f"{f}.safetensors", OUT / "tiny" / f"{f}.safetensors")
+    for f in ("init.safetensors", "forward.safetensors", "grads_init.safetensors", "muon_step_bf16.safetensors",
+              "trace_ns5_f32.safetensors", "grads_step5.safetensors", "tokens.bin", "batch_starts.json",
+              "lr_schedules.json"):
+        shutil.copyfile(REF / "ojas-oracle/fixtures/tiny" / f, OUT / "tiny" / f)
 
 
 if __name__ == "__main__":

@@ -128,3 +128,26 @@ def test_every_gradient_against_the_oracle(be, kv_heads, window):
             continue
         rel = np.linalg.norm(got - ref) / max(np.linalg.norm(ref), 1e-30)
         assert rel <= GRAD_NORMWISE_REL_TOL, (name, rel)
+
+
+def test_five_trainer_steps_follow_the_torch_trace(be):
+    """`NanolabTrainer.run` on the device, five steps of the reference's torch trace: per-step mean
+    loss within 1e-4 nats, every parameter after step 5 within 1e-4 normwise
+    (ojas-oracle/src/parity.rs:36-41, :468-470)."""
+    import trace_fixture as tf
+    from ojas_amd.nanolab import NanolabTrainer
+
+    print("nanolab five-step trace on the device", flush=True)
+    trace = tf.Trace()
+    spec = tiny_spec()
+    init, _ = load("init")
+    trainer = NanolabTrainer(be, spec, init, adam_lr=trace.cfg["lr"], matrix_lr=trace.cfg["matrix_lr"],
+                             grad_clip=trace.cfg["grad_clip"])
+    losses, norms = [], []
+    for step in range(trace.steps):
+        report = trainer.run([trace.micro(step, m) for m in range(trace.accum)], trace.lr_mult[step])
+        assert report.step == step + 1 and report.tokens == trace.accum * trace.batch * trace.seq
+        losses.append(report.loss)
+        norms.append(report.grad_norm)
+    worst = tf.check_trace(trace, losses, norms, trainer.download_params(), {"blocks.0.mixer.vr_lambda"})
+    print(f"worst parameter distance after step {trace.steps}: {worst:.2e}", flush=True)

@@ -164,3 +164,64 @@ def test_bf16_muon_step_is_stock_nanolab_bit_for_bit():
         want = data[f"c{i}.p_after"].astype(np.float64) - p
         rel32 = np.linalg.norm((p32.astype(np.float64) - p) - want) / np.linalg.norm(want)
         assert rel32 > 1e-2, f"case {i}: the f32 contrast is too close ({rel32:.2e}) to tell"
+
+
+def test_five_trainer_steps_follow_the_torch_trace():
+    """Micro-batch accumulation, the global clip, Muon-NS5 in f32 and AdamW, composed the way
+    `Trainer::run` composes them, against the reference's torch trace: per-step mean loss within
+    1e-4 nats, gradient norm 1e-4 relative, every parameter after step 5 within 1e-4 normwise
+    (ojas-oracle/src/parity.rs:36-41, :468-470). Then the gradients at those parameters against
+    `grads_step5` at the gradient gate."""
+    import trace_fixture as tf
+
+    trace = tf.Trace()
+    init, _ = load("init")
+    cfg = tiny_config(trace.batch, trace.seq)
+    names = orc.nanolab_param_names(cfg.layers)
+    frozen = {"blocks.0.mixer.vr_lambda"}
+    params = {n: np.ascontiguousarray(init[n], np.float32) for n in names}
+    state = {n: [np.zeros_like(params[n]), np.zeros_like(params[n])] for n in names}
+    weight = np.float32(1.0 / trace.accum)
+    losses, norms = [], []
+    for step in range(trace.steps):
+        acc, loss_sum = None, np.float32(0)
+        for micro in range(trace.accum):
+            ids, targets = trace.micro(step, micro)
+            loss, _, grads = orc.nanolab_loss_and_grads(cfg, [params[n].reshape(-1) for n in names], ids, targets)
+            assert abs(float(loss) - trace.micro_loss[step * trace.accum + micro]) <= tf.TRACE_LOSS_ABS_TOL
+            grads = [np.asarray(g, np.float32) * weight for g in grads]
+            acc = grads if acc is None else [a + g for a, g in zip(acc, grads)]
+            loss_sum = np.float32(loss_sum + np.float32(loss))
+        live = [n for n in names if n not in frozen]
+        norm, clipped = orc.clip_grad_norm([acc[names.index(n)] for n in live], trace.cfg["grad_clip"])
+        mult = trace.lr_mult[step]
+        for n, g in zip(live, clipped):
+            shape = params[n].shape
+            if tf.optimizer_of(n, shape) == "muon":
+                p, m = orc.muon_ns5_step(params[n], g.reshape(shape), state[n][0], lr=trace.cfg["matrix_lr"] * mult,
+                                         momentum=tf.MUON_MOMENTUM, weight_decay=tf.MUON_WEIGHT_DECAY, nesterov=True)
+                params[n], state[n][0] = p, m
+            else:
+                p, m, v = orc.adamw_step(params[n].reshape(-1), g.reshape(-1), state[n][0].reshape(-1),
+                                         state[n][1].reshape(-1), step, trace.cfg["lr"] * mult, trace.cfg["beta1"],
+                                         trace.cfg["beta2"], trace.cfg["eps"], tf.ADAM_HYBRID_WEIGHT_DECAY)
+                params[n], state[n] = p.reshape(shape), [m.reshape(shape), v.reshape(shape)]
+        losses.append(float(loss_sum) / trace.accum)
+        norms.append(float(norm))
+    worst = tf.check_trace(trace, losses, norms, params, frozen)
+    print(f"worst parameter distance after step {trace.steps}: {worst:.2e}")
+
+    want, gmeta = load("grads_step5")
+    info = gmeta["ojas.oracle"]
+    ids, targets = trace.micro(0, 0)
+    at = {n: np.ascontiguousarray(trace.params_after[n], np.float32) for n in names}
+    loss, _, grads = orc.nanolab_loss_and_grads(cfg, [at[n].reshape(-1) for n in names], ids, targets)
+    assert abs(float(loss) - info["loss"]) <= FORWARD_LOSS_REL_TOL * abs(info["loss"])
+    seed = np.float32(info["loss_seed"])
+    for n, g in zip(names, grads):
+        if n in info["no_grad"]:
+            continue
+        ref = want[n].reshape(-1).astype(np.float64)
+        assert n not in info["zero_grad"], "after five steps no gradient is exactly zero"
+        rel = np.linalg.norm(np.asarray(g, np.float64) * seed - ref) / np.linalg.norm(ref)
+        assert rel <= GRAD_NORMWISE_REL_TOL, (n, rel)
