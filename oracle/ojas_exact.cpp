@@ -12,7 +12,11 @@
 //   muon f32                  exact_golden.rs:243-250 (8 digests)
 //   muon bf16                 ojas-oracle/fixtures/tiny/muon_step_bf16.safetensors (4 cases, bit for bit)
 //   nanolab graph             ojas-oracle/fixtures/tiny/{init,forward,grads_init}.safetensors at the
-//                             gates of ojas-oracle/src/parity.rs:28-40 (nanolab_exact.cpp)
+//                             gates of ojas-oracle/src/parity.rs:28-40 (nanolab_exact.cpp);
+//                             grads_step5.safetensors at the same gradient gate
+//   trainer step              accumulation + clip + muon f32 + adamw over five steps of
+//                             ojas-oracle/fixtures/tiny/trace_ns5_f32.safetensors (losses 1e-4
+//                             nats, parameters 1e-4 normwise, parity.rs:36-41)
 //   sdpa fwd/lse/bwd          exact_golden.rs:251-265 (15 digests); window and
 //                             GQA: brute-force softmax in the tests
 //   rms fwd/bwd, rope         exact_golden.rs:266-270; rms_norm_f64.json
