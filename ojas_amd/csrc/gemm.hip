@@ -463,14 +463,17 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
     if (mode == 1) {
       // Measured on the GPT shapes: small outputs (the d x d weight gradients, the
       // Newton-Schulz squares) stay on the 128 x 128 kernel; everything else takes 256 x 128
-      // tiles, which leave room for two workgroups per compute unit, so one's output stores and
-      // first loads overlap the other's products (256 x 256 halves the L2 traffic per FLOP but
-      // runs alone on its compute unit and measures slower on every GPT shape).
+      // tiles in 32-column K steps, three stages in 72 KiB, so two workgroups share a compute
+      // unit and one's output stores, first loads and barrier waits overlap the other's
+      // products. The 64-column forms fetch whole cache lines but run alone on their compute
+      // unit; they win only on long reductions with large outputs (8192^3: 1.09 against
+      // 0.95 PFLOP/s for 256 x 256) and lose on every GPT shape.
       if (static_cast<long>(g.M) * g.N <= (1l << 20)) dma_variant = -1;
-      else dma_variant = 1;
+      else dma_variant = 3;
     }
     else if (mode == 2) dma_variant = 0;
-    else if (mode == 3) dma_variant = 1;
+    else if (mode == 3) dma_variant = 3;
+    else if (mode == 4) dma_variant = 1;
   }
   int BM = 128, BN = 128;
   if (dma_variant >= 0) omx_gemm_dma_tile(dma_variant, &BM, &BN);

@@ -3,20 +3,31 @@
 //
 // Same contract as gemm.hip (C[M,N] (+)= A.B, f32 accumulation, every operand
 // layout; reference: ojas-cpu/src/linalg.rs:69-210), different data movement:
-//   * 512 threads (8 waves); tile 256 x 128 (waves 4 x 2, each 64 x 64; at most 108 VGPRs and
-//     72 KiB of LDS, so two workgroups share a compute unit and one's output stores, first
-//     loads and barrier waits overlap the other's products) or 256 x 256 (waves 2 x 4, each
-//     128 x 64; half the L2-to-LDS traffic per FLOP, one workgroup per compute unit).
+//   * 512 threads (8 waves); tile 256 x 128 (waves 4 x 2, each 64 x 64) or 256 x 256 (waves
+//     2 x 4, each 128 x 64; half the L2-to-LDS traffic per FLOP).
+//   * Variant 3, the default: K steps of 32 columns, three stages in 72 KiB and at most 128
+//     VGPRs, so two workgroups share a compute unit and one's output stores, first loads and
+//     barrier waits overlap the other's products. Its weakness: a k-contiguous operand row
+//     contributes half a 128-byte cache line per step, each line is requested twice, far enough
+//     apart that the second request misses L1 again, and the load path then delivers 65 GB/s
+//     per compute unit instead of 107 GB/s (measured with the loads alone).
+//   * Variants 1 (256 x 128, three stages) and 0 (256 x 256, two stages): K steps of 64 columns,
+//     whole cache lines, one workgroup per compute unit. Load latency (about 0.6 us) is then
+//     exposed: with one or two stages in flight the loads alone take as long as the products.
 //   * operand tiles go from global memory straight into LDS: no staging
 //     registers and no LDS store instructions. A wave-wide load writes 64
 //     consecutive 16-byte slots, so the LDS tile is unpadded and bank conflicts
 //     are avoided by choosing WHICH chunk each lane fetches (an XOR swizzle):
-//       k-contiguous operand, [row][4 chunks]: slot s of row r holds chunk s ^ ((r >> 1) & 3);
-//       k-major operand, [k][ROWS/8 chunks]:   slot s of k row kr holds chunk s ^ 2(kr & 3)
-//     (the latter keeps the four k rows that one ds_read_b64_tr_b16 group
-//     touches on distinct banks).
-//   * three LDS stages of 32 K columns: the loads of K steps ks+1 and ks+2 are in flight while
-//     step ks is multiplied; one counted vmcnt wait + barrier per step.
+//       k-contiguous operand, [row][BK/8 chunks]: slot s of row r holds chunk s ^ ((r >> 2) & 3)
+//         for 64-byte rows and s ^ ((r >> 1) & 7) for 128-byte rows;
+//       k-major operand, [k][ROWS/8 chunks]:   slot s of k row kr holds chunk s ^ 4(kr & 3).
+//     LDS has 64 four-byte banks: a 16-byte read serves 16 lanes per clock, i.e. rows r..r+15 of
+//     one chunk column, whose 64-byte rows repeat banks every 4 rows (128-byte rows: every 2),
+//     so the XOR must separate rows r, r+4, r+8, r+12 (r, r+2, ..., r+14); a transposing 8-byte read serves 32 lanes per clock, four k rows of
+//     64 bytes each, which the XOR moves 64 bytes apart. Both measured conflict-free
+//     (4.0 and 1.9 clocks per wave read with 16 waves; 7.1 and 3.0 with a 2-way conflict).
+//   * NST LDS stages: the loads of K steps ks+1 .. ks+NST-1 are in flight while step ks is
+//     multiplied; one counted vmcnt wait + barrier per step.
 // Rows past M (or N) are fetched from a clamped valid address and never stored.
 #include "gemm_args.h"
 
@@ -29,15 +40,13 @@ typedef short short4v __attribute__((ext_vector_type(4)));
 namespace {
 
 constexpr int DT = 512;  // threads
-constexpr int DBK = 32;   // K per pipeline step
-constexpr int NST = 3;    // LDS stages: the loads of step s + NST - 1 are issued while step s is multiplied
 
 // Per-lane state of one operand's loads: the global address of each of this wave's loads for the
 // current K step (advanced by one step after every issue) and nothing else, so a step costs one
-// 64-bit add per load. ROWS x 32 bf16 = ROWS / 16 KiB per step, one wave instruction per KiB.
-template <bool KM, int ROWS>
+// 64-bit add per load. ROWS x BK bf16 per step, one wave instruction per KiB.
+template <bool KM, int ROWS, int BK>
 struct TileLoads {
-  static constexpr int N = ROWS / 16 / 8;  // loads per wave per step
+  static constexpr int N = ROWS * BK * 2 / 1024 / 8;  // loads per wave per step
   const unsigned short* src[N];
   long step;  // elements between consecutive K steps
 
@@ -47,9 +56,10 @@ struct TileLoads {
     for (int i = 0; i < N; ++i) {
       const int q = wave + 8 * i;
       if constexpr (!KM) {
-        // [row][4 chunks of 16 bytes]; slot s of row r holds chunk s ^ ((r >> 1) & 3).
-        const int r = q * 16 + (lane >> 2);
-        const int kc = (lane & 3) ^ ((lane >> 3) & 3);
+        // [row][BK / 8 chunks of 16 bytes], swizzled as frag_offset reads them.
+        constexpr int LPR = BK / 8;  // lanes (chunks) per row
+        const int r = q * (64 / LPR) + lane / LPR;
+        const int kc = (lane % LPR) ^ (BK == 32 ? (r >> 2) & 3 : (r >> 1) & 7);
         int gr = row0 + r;
         gr = gr < rows ? gr : rows - 1;
         src[i] = p + static_cast<long>(gr) * ld + k0 + kc * 8;
@@ -57,13 +67,13 @@ struct TileLoads {
         constexpr int CPR = ROWS / 8;
         const int idx = q * 64 + lane;
         const int kr = idx / CPR, slot = idx % CPR;
-        const int mc = slot ^ ((kr & 3) * 2);
+        const int mc = slot ^ ((kr & 3) * 4);
         int gm = row0 + mc * 8;
         gm = gm + 8 <= rows ? gm : 0;
         src[i] = p + static_cast<long>(k0 + kr) * ld + gm;
       }
     }
-    step = KM ? DBK * ld : DBK;
+    step = KM ? BK * ld : BK;
   }
   // Starts this step's loads into the operand tile at LDS byte address `tile` and moves on.
   __device__ __forceinline__ void issue(unsigned tile, int wave) {
@@ -83,18 +93,18 @@ struct TileLoads {
 // Byte offset, inside an operand tile, of this lane's fragment for 32-row block `row_base / 32`
 // and 16-column K slab kk (k-major operands: of its first transposing read; the second is four
 // K rows further).
-template <bool KM, int ROWS>
+template <bool KM, int ROWS, int BK>
 __device__ __forceinline__ int frag_offset(int row_base, int kk, int lane) {
   if constexpr (!KM) {
     const int l32 = lane & 31, g = lane >> 5;
     const int r = row_base + l32;
     const int kc = kk * 2 + g;
-    return r * 64 + ((kc ^ ((r >> 1) & 3)) << 4);
+    return r * (BK * 2) + ((kc ^ (BK == 32 ? (r >> 2) & 3 : (r >> 1) & 7)) << 4);
   } else {
     const int s = lane & 15, half = (lane >> 4) & 1, g = lane >> 5;
     const int kr = kk * 16 + g * 8 + (s >> 2);
     const int col = row_base + half * 16 + (s & 3) * 4;
-    const int slot = (col >> 3) ^ (((s >> 2) & 3) * 2);
+    const int slot = (col >> 3) ^ (((s >> 2) & 3) * 4);
     return kr * (ROWS * 2) + slot * 16 + (col & 7) * 2;
   }
 }
@@ -111,12 +121,17 @@ __device__ __forceinline__ u32x4 frag_at(const char* p) {
   }
 }
 
-template <bool A_KM, bool B_KM, int WGM, int WGN, int TM, int TN>
-__global__ __launch_bounds__(DT, (TM * TN <= 4 ? 4 : 2)) void gemm_dma_kernel(GemmArgs g) {
+// s_waitcnt operand that waits for vmcnt <= n only (vmcnt is bits 3:0 and 15:14).
+constexpr int vmcnt_only(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
+
+template <bool A_KM, bool B_KM, int WGM, int WGN, int TM, int TN, int DBK, int NST>
+__global__ __launch_bounds__(DT, (NST * (WGM * TM + WGN * TN) * 32 * DBK * 2 <= 80 * 1024 ? 4 : 2)) void gemm_dma_kernel(
+    GemmArgs g) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
-  constexpr int A_BYTES = BM * 64, B_BYTES = BN * 64, STAGE = A_BYTES + B_BYTES;
-  constexpr int LPS = (BM + BN) / 16 / 8;  // loads per wave per step
+  constexpr int A_BYTES = BM * DBK * 2, B_BYTES = BN * DBK * 2, STAGE = A_BYTES + B_BYTES;
+  constexpr int LPS = STAGE / 1024 / 8;  // loads per wave per step
+  constexpr int KK = DBK / 16;           // MFMA K slabs per step
   static_assert(WGM * WGN == 8, "eight waves");
   const unsigned short* __restrict__ A = static_cast<const unsigned short*>(g.a);
   const unsigned short* __restrict__ B = static_cast<const unsigned short*>(g.b);
@@ -148,30 +163,32 @@ __global__ __launch_bounds__(DT, (TM * TN <= 4 ? 4 : 2)) void gemm_dma_kernel(Ge
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  // g.ksteps_per_split counts 64-wide K blocks; a pipeline step is half of one.
-  const int ks_begin = 2 * split * g.ksteps_per_split;
-  const int ks_end = min(g.K / DBK, ks_begin + 2 * g.ksteps_per_split);
+  // g.ksteps_per_split counts 64-wide K blocks.
+  constexpr int SPB = 64 / DBK;  // pipeline steps per block
+  const int ks_begin = SPB * split * g.ksteps_per_split;
+  const int ks_end = min(g.K / DBK, ks_begin + SPB * g.ksteps_per_split);
   // Everything a K step needs is computed here, once per tile: the loads' global addresses and
   // the fragments' LDS offsets. Inside the loop the stage is a compile-time constant (the loop
   // body is unrolled over the stages), so a step is loads, LDS reads and MFMAs and little else.
-  TileLoads<A_KM, BM> la;
-  TileLoads<B_KM, BN> lb;
+  TileLoads<A_KM, BM, DBK> la;
+  TileLoads<B_KM, BN, DBK> lb;
   la.init(A, g.lda, m0, g.M, ks_begin * DBK, wave, lane);
   lb.init(B, g.ldb, n0, g.N, ks_begin * DBK, wave, lane);
   const unsigned lds0 = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(reinterpret_cast<uintptr_t>(smem)));
-  int a_off[TM][2], b_off[TN][2];
+  int a_off[TM][KK], b_off[TN][KK];
 #pragma unroll
-  for (int kk = 0; kk < 2; ++kk) {
+  for (int kk = 0; kk < KK; ++kk) {
 #pragma unroll
-    for (int t = 0; t < TM; ++t) a_off[t][kk] = frag_offset<A_KM, BM>((wm * TM + t) * 32, kk, lane);
+    for (int t = 0; t < TM; ++t) a_off[t][kk] = frag_offset<A_KM, BM, DBK>((wm * TM + t) * 32, kk, lane);
 #pragma unroll
-    for (int t = 0; t < TN; ++t) b_off[t][kk] = A_BYTES + frag_offset<B_KM, BN>((wn * TN + t) * 32, kk, lane);
+    for (int t = 0; t < TN; ++t) b_off[t][kk] = A_BYTES + frag_offset<B_KM, BN, DBK>((wn * TN + t) * 32, kk, lane);
   }
   // Waits until at most `groups` of this wave's per-step load groups are still in flight.
   auto wait_groups = [&](int groups) {
-    if (groups >= 2) __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * LPS));
-    else if (groups == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | LPS);
-    else __builtin_amdgcn_s_waitcnt(0x0F70);
+    static_assert(2 * LPS < 64, "vmcnt is six bits");
+    if (groups >= 2) __builtin_amdgcn_s_waitcnt(vmcnt_only(2 * LPS));
+    else if (groups == 1) __builtin_amdgcn_s_waitcnt(vmcnt_only(LPS));
+    else __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
   };
 
 #pragma unroll
@@ -182,22 +199,46 @@ __global__ __launch_bounds__(DT, (TM * TN <= 4 ? 4 : 2)) void gemm_dma_kernel(Ge
     }
   wait_groups(min(NST - 2, ks_end - ks_begin - 1));
   __syncthreads();
+  // The fragments of the next 16-column slab are read while the current slab is multiplied; the
+  // first slab of the next step is read right after the barrier that publishes its stage, ahead
+  // of the last slab's products, so neither the LDS latency nor the barrier drains the MFMA pipe.
+  u32x4 af[TM], bf[TN];
+  auto read_frags = [&](const char* stage, int kk, u32x4(&a)[TM], u32x4(&b)[TN]) {
+#pragma unroll
+    for (int t = 0; t < TM; ++t) a[t] = frag_at<A_KM, BM>(stage + a_off[t][kk]);
+#pragma unroll
+    for (int t = 0; t < TN; ++t) b[t] = frag_at<B_KM, BN>(stage + b_off[t][kk]);
+  };
+  read_frags(smem, 0, af, bf);
   for (int ks = ks_begin; ks < ks_end;) {
 #pragma unroll
     for (int st = 0; st < NST; ++st) {  // step ks lives in stage st
       if (ks + NST - 1 < ks_end) {
-        constexpr int kFill[3] = {NST - 1, 0, 1};
-        la.issue(lds0 + kFill[st % 3] * STAGE, wave);
-        lb.issue(lds0 + kFill[st % 3] * STAGE + A_BYTES, wave);
+        const int fill = (st + NST - 1) % NST;  // the stage the previous step has released
+        la.issue(lds0 + fill * STAGE, wave);
+        lb.issue(lds0 + fill * STAGE + A_BYTES, wave);
       }
       const char* stage = smem + st * STAGE;
 #pragma unroll
-      for (int kk = 0; kk < 2; ++kk) {
-        u32x4 af[TM], bf[TN];
+      for (int kk = 0; kk < KK; ++kk) {
+        u32x4 an[TM], bn[TN];
 #pragma unroll
-        for (int t = 0; t < TM; ++t) af[t] = frag_at<A_KM, BM>(stage + a_off[t][kk]);
+        for (int t = 0; t < TM; ++t) an[t] = af[t];
 #pragma unroll
-        for (int t = 0; t < TN; ++t) bf[t] = frag_at<B_KM, BN>(stage + b_off[t][kk]);
+        for (int t = 0; t < TN; ++t) bn[t] = bf[t];
+        if (kk + 1 < KK) {
+          read_frags(stage, kk + 1, an, bn);
+        } else {
+          // Step ks + 1 must have landed (this wave's share, then everyone's); later steps may
+          // still be in flight. Every wave has its last fragments of stage st in registers by
+          // now, so the barrier also releases stage st for the loads of step ks + NST.
+          wait_groups(min(NST - 2, ks_end - ks - 2));
+          __syncthreads();
+          if (ks + 1 < ks_end) read_frags(smem + ((st + 1) % NST) * STAGE, 0, an, bn);
+        }
+        // Keeps the reads above the products: the scheduler would otherwise sink them to their
+        // first use to save registers, which puts the LDS latency back in front of every slab.
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
@@ -205,14 +246,16 @@ __global__ __launch_bounds__(DT, (TM * TN <= 4 ? 4 : 2)) void gemm_dma_kernel(Ge
             acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[tm]),
                                                                   __builtin_bit_cast(bf16x8, bf[tn]), acc[tm][tn], 0,
                                                                   0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < TM; ++t) af[t] = an[t];
+#pragma unroll
+        for (int t = 0; t < TN; ++t) bf[t] = bn[t];
       }
-      // Step ks + 1 must have landed (this wave's share, then everyone's); later steps may still
-      // be in flight. The barrier also frees stage st for the loads of step ks + NST.
-      wait_groups(min(NST - 2, ks_end - ks - 2));
-      __syncthreads();
       if (++ks >= ks_end) break;
     }
   }
+  __syncthreads();  // the staging below reuses the stages
 
   // Epilogue: each wave stages 32 rows of its tile at a time through its own
   // LDS region and writes whole 4-column pieces.
@@ -256,11 +299,11 @@ __global__ __launch_bounds__(DT, (TM * TN <= 4 ? 4 : 2)) void gemm_dma_kernel(Ge
   if (bad) dev_raise_fault(g.fault, g.tag);
 }
 
-template <bool A_KM, bool B_KM, int WGM, int WGN, int TM, int TN>
+template <bool A_KM, bool B_KM, int WGM, int WGN, int TM, int TN, int DBK, int NST>
 int32_t launch_dma(omx_ctx* ctx, const GemmArgs& g) {
   constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
-  constexpr int smem = NST * (BM + BN) * 64;
-  auto kernel = &gemm_dma_kernel<A_KM, B_KM, WGM, WGN, TM, TN>;
+  constexpr int smem = NST * (BM + BN) * DBK * 2;
+  auto kernel = &gemm_dma_kernel<A_KM, B_KM, WGM, WGN, TM, TN, DBK, NST>;
   static bool granted = false;
   if (!granted) {
     OMX_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -272,12 +315,12 @@ int32_t launch_dma(omx_ctx* ctx, const GemmArgs& g) {
   return OMX_OK;
 }
 
-template <int WGM, int WGN, int TM, int TN>
+template <int WGM, int WGN, int TM, int TN, int DBK, int NST>
 int32_t launch_layout(omx_ctx* ctx, const GemmArgs& g, bool a_km, bool b_km) {
-  if (!a_km && !b_km) return launch_dma<false, false, WGM, WGN, TM, TN>(ctx, g);
-  if (!a_km && b_km) return launch_dma<false, true, WGM, WGN, TM, TN>(ctx, g);
-  if (a_km && !b_km) return launch_dma<true, false, WGM, WGN, TM, TN>(ctx, g);
-  return launch_dma<true, true, WGM, WGN, TM, TN>(ctx, g);
+  if (!a_km && !b_km) return launch_dma<false, false, WGM, WGN, TM, TN, DBK, NST>(ctx, g);
+  if (!a_km && b_km) return launch_dma<false, true, WGM, WGN, TM, TN, DBK, NST>(ctx, g);
+  if (a_km && !b_km) return launch_dma<true, false, WGM, WGN, TM, TN, DBK, NST>(ctx, g);
+  return launch_dma<true, true, WGM, WGN, TM, TN, DBK, NST>(ctx, g);
 }
 
 }  // namespace
@@ -295,6 +338,7 @@ void omx_gemm_dma_tile(int variant, int* bm, int* bn) {
 }
 
 int32_t omx_gemm_dma_launch(omx_ctx* ctx, const GemmArgs& g, bool a_km, bool b_km, int variant) {
-  if (variant == 0) return launch_layout<2, 4, 4, 2>(ctx, g, a_km, b_km);
-  return launch_layout<4, 2, 2, 2>(ctx, g, a_km, b_km);
+  if (variant == 0) return launch_layout<2, 4, 4, 2, 64, 2>(ctx, g, a_km, b_km);
+  if (variant == 3) return launch_layout<4, 2, 2, 2, 32, 3>(ctx, g, a_km, b_km);
+  return launch_layout<4, 2, 2, 2, 64, 3>(ctx, g, a_km, b_km);
 }
