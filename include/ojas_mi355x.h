@@ -266,6 +266,15 @@ int32_t omx_gelu_forward(omx_ctx* ctx, const void* x, void* y, int32_t dtype, ui
                          int32_t tanh_form);
 int32_t omx_gelu_backward(omx_ctx* ctx, const void* x, const void* gy, void* gx, int32_t dtype,
                           uint64_t n, int32_t tanh_form);
+/* The batch that BatchSampler::next_batch reads (ojas-data/src/sampler.rs:262-275), built on the
+ * device from a token bin resident in HBM: x[b, t] = tokens[starts[b] + t],
+ * y[b, t] = tokens[starts[b] + t + 1], u32 [batch, seq_len]. `tokens` is the bin's little-endian
+ * token words on the device (bytes_per_token 2 or 4, n_tokens of them); `starts` is a HOST array
+ * of `batch` window starts (odata_sampler_next_starts, ojas_data.h). A window that does not lie
+ * inside the bin is OutOfRange and nothing is written. */
+int32_t omx_token_windows(omx_ctx* ctx, const void* tokens, int32_t bytes_per_token,
+                          uint64_t n_tokens, const uint64_t* starts, uint64_t batch,
+                          uint64_t seq_len, void* x, void* y);
 /* BackendFloat::permute with axes [0,2,1,3] (backend.rs:1115-1134; the one
  * permutation the model uses, ojas-model/src/block.rs:25,195-199):
  * [d0,d1,d2,d3] -> [d0,d2,d1,d3]. */

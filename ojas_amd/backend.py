@@ -671,6 +671,18 @@ class MiBackend:
         return gv, gv0, gl
 
     # ---- integer ops ----
+    def token_windows(self, tokens: DeviceTensor, starts, seq_len: int):
+        """(x, y) u32 [batch, seq_len] from a bin resident on the device (`upload` of
+        `TokenBin.read_raw`: U32 words, or u16 words uploaded as BF16-sized storage) and the host
+        array of window starts `BatchSampler.next_starts` returns."""
+        starts = np.ascontiguousarray(starts, np.uint64)
+        batch = int(starts.size)
+        x, y = self.empty((batch, seq_len), U32), self.empty((batch, seq_len), U32)
+        self._check(self._lib.omx_token_windows(self._ctx, self._p(tokens), C.c_int32(_SIZE_OF[tokens.dtype]),
+                                                C.c_uint64(tokens.numel), starts.ctypes.data_as(C.c_void_p),
+                                                C.c_uint64(batch), C.c_uint64(seq_len), self._p(x), self._p(y)))
+        return x, y
+
     def argmax_rows(self, x):
         rows, cols = x.shape
         out = self.empty((rows,), U32)

@@ -110,6 +110,21 @@ __global__ void permute_0213_kernel(const V* __restrict__ x, V* __restrict__ y, 
   }
 }
 
+// x[b, t] = tokens[starts[b] + t], y[b, t] = tokens[starts[b] + t + 1], widened to u32.
+template <typename TOK>
+__global__ void token_windows_kernel(const TOK* __restrict__ tokens, const unsigned long long* __restrict__ starts,
+                                     unsigned int* __restrict__ x, unsigned int* __restrict__ y, size_t batch,
+                                     size_t seq_len) {
+  const size_t n = batch * seq_len;
+  for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+    const size_t b = i / seq_len, t = i - b * seq_len;
+    const TOK* w = tokens + starts[b] + t;
+    x[i] = w[0];
+    y[i] = w[1];
+  }
+}
+
 }  // namespace
 
 int32_t omx_convert(omx_ctx* ctx, const void* src, int32_t src_dtype, void* dst, int32_t dst_dtype, uint64_t n) {
@@ -286,6 +301,42 @@ int32_t omx_permute_0213(omx_ctx* ctx, const void* x, void* y, int32_t dtype, ui
                        d3);
   }
   OMX_LAUNCH_CHECK(ctx, "permute_0213_kernel");
+  return OMX_OK;
+}
+
+int32_t omx_token_windows(omx_ctx* ctx, const void* tokens, int32_t bytes_per_token, uint64_t n_tokens,
+                          const uint64_t* starts, uint64_t batch, uint64_t seq_len, void* x, void* y) {
+  OMX_REQUIRE_CTX(ctx);
+  if (!tokens || !x || !y) return omx_fail(ctx, OMX_PLACEMENT, "token_windows: null device pointer");
+  if (!starts) return omx_fail(ctx, OMX_PLACEMENT, "token_windows: null starts");
+  if (bytes_per_token != 2 && bytes_per_token != 4)
+    return omx_fail(ctx, OMX_DTYPE, "token_windows: tokens are 2 or 4 bytes wide, got %d", bytes_per_token);
+  if (batch == 0 || seq_len == 0) return omx_fail(ctx, OMX_SHAPE, "token_windows: zero-sized axis");
+  if (seq_len >= n_tokens || batch > (1ull << 32) || seq_len > (1ull << 32))
+    return omx_fail(ctx, OMX_OUT_OF_RANGE, "token_windows: a window of %llu + 1 tokens in a bin of %llu",
+                    static_cast<unsigned long long>(seq_len), static_cast<unsigned long long>(n_tokens));
+  for (uint64_t b = 0; b < batch; ++b)
+    if (starts[b] > n_tokens - seq_len - 1)
+      return omx_fail(ctx, OMX_OUT_OF_RANGE, "token_windows: window %llu starts at %llu, past the bin's %llu tokens",
+                      static_cast<unsigned long long>(b), static_cast<unsigned long long>(starts[b]),
+                      static_cast<unsigned long long>(n_tokens));
+  void* ws = nullptr;
+  int32_t rc = omx_workspace(ctx, batch * sizeof(uint64_t), &ws);
+  if (rc != OMX_OK) return rc;
+  // A copy from pageable host memory returns once the source has been staged, so the caller's
+  // array may be reused at once; it is ordered before the kernel on the same stream.
+  OMX_HIP(ctx, hipMemcpyAsync(ws, starts, batch * sizeof(uint64_t), hipMemcpyHostToDevice, ctx->stream));
+  const uint64_t n = batch * seq_len;
+  const unsigned blocks = static_cast<unsigned>(std::min<uint64_t>((n + 255) / 256, 4096));
+  if (bytes_per_token == 2)
+    hipLaunchKernelGGL((token_windows_kernel<unsigned short>), dim3(blocks), dim3(256), 0, ctx->stream,
+                       static_cast<const unsigned short*>(tokens), static_cast<const unsigned long long*>(ws),
+                       static_cast<unsigned int*>(x), static_cast<unsigned int*>(y), batch, seq_len);
+  else
+    hipLaunchKernelGGL((token_windows_kernel<unsigned int>), dim3(blocks), dim3(256), 0, ctx->stream,
+                       static_cast<const unsigned int*>(tokens), static_cast<const unsigned long long*>(ws),
+                       static_cast<unsigned int*>(x), static_cast<unsigned int*>(y), batch, seq_len);
+  OMX_LAUNCH_CHECK(ctx, "token_windows_kernel");
   return OMX_OK;
 }
 

@@ -15,6 +15,7 @@ Run in the build container (needs /root/reference). Only DATA is taken:
   * the tiny model's 40-step f32-NS5 trace  ojas-oracle/fixtures/tiny/{trace_ns5_f32,grads_step5}.safetensors,
     (losses, grad norms, step-5 parameters)  its token bin, window starts and LR multipliers: tokens.bin,
                                              batch_starts.json, lr_schedules.json (copied as is)
+  * pinned window starts of the batch sampler  ojas-data/tests/sampler.rs:231-254 (numbers -> JSON)
 No reference source text is kept: numeric literals are parsed into JSON.
 """
 import json
@@ -59,6 +60,21 @@ def erf_tables():
          "gelu": table("GELU")}, indent=1))
 
 
+def sampler_pins():
+    src = (REF / "ojas-data/tests/sampler.rs").read_text()
+    body = src[src.index("fn permutation_is_pinned"):]
+    body = body[:body.index("];")]
+    cases = []
+    for seed, epoch, starts in re.findall(r"\((0x[0-9A-Fa-f_]+|\d+), (\d+), \[([0-9, ]+)\]\)", body):
+        cases.append({"seed": int(seed.replace("_", ""), 0), "epoch": int(epoch),
+                      "starts": [int(v) for v in starts.split(",")]})
+    assert len(cases) == 6, len(cases)
+    (OUT / "sampler_pins.json").write_text(json.dumps(
+        {"source": "ojas-data/tests/sampler.rs:231-254 (permutation_is_pinned: bin of 1001 tokens, seq_len 10, "
+                   "batch 1, window starts of ordinals 0..8)", "bin_tokens": 1001, "seq_len": 10, "windows": 100,
+         "cases": cases}, indent=1))
+
+
 def copies():
     shutil.copyfile(REF / "ojas-core/src/exp_exact_pins.txt", OUT / "exp_exact_pins.txt")
     shutil.copyfile(REF / "ojas-oracle/fixtures/rms_norm_f64.json", OUT / "rms_norm_f64.json")
@@ -80,5 +96,6 @@ if __name__ == "__main__":
     digests()
     torch_ref()
     erf_tables()
+    sampler_pins()
     copies()
     print("fixtures written to", OUT)
