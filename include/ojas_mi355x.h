@@ -266,6 +266,30 @@ int32_t omx_gelu_forward(omx_ctx* ctx, const void* x, void* y, int32_t dtype, ui
                          int32_t tanh_form);
 int32_t omx_gelu_backward(omx_ctx* ctx, const void* x, const void* gy, void* gx, int32_t dtype,
                           uint64_t n, int32_t tanh_form);
+/* ---- KV-cache attention and cache write (the step after the path: decode) ----
+ * BackendModule::cached_attention_forward (backend.rs:2526-2555; validator
+ * ojas-core/src/shapes.rs:2758-2826; CPU ojas-cpu/src/kv.rs:103-256): q [batch, tq, heads, head_dim]
+ * f32 against caches [batch, capacity, kv_heads, head_dim], time-major rings in which position j
+ * lives in slot j % capacity. Query i sits at position p = kv_len - tq + i and attends to positions
+ * 0..=p, or with a window (0 = none) to p + 1 - window..=p; head h reads KV head
+ * h / (heads / kv_heads). out is f32 [batch, tq, heads, head_dim]. kv_len < tq, or a read the ring
+ * no longer holds, is OutOfRange. Slots that no query reads are never touched; a NaN or infinity in
+ * one that is read raises the deferred NonFinite. cache_dtype OMX_F32 is the trait's contract;
+ * OMX_BF16 caches (half the bytes to read) are this library's addition, widened exactly.
+ * head_dim: a multiple of 4 up to 256, else UnsupportedHeadDim. */
+int32_t omx_cached_attention_forward(omx_ctx* ctx, const void* q, const void* k_cache,
+                                     const void* v_cache, int32_t cache_dtype, void* out,
+                                     uint64_t batch, uint64_t tq, uint64_t heads, uint64_t kv_heads,
+                                     uint64_t head_dim, uint64_t capacity, uint64_t kv_len,
+                                     uint64_t window);
+/* BackendModule::kv_cache_write (backend.rs:2557-2565; validator shapes.rs:2834-2879; CPU
+ * ojas-cpu/src/kv.rs:258-292): src f32 [batch, tn, kv_heads, head_dim] goes to positions
+ * at..at + tn of the ring, position j to slot j % capacity (tn <= capacity). All or nothing: a NaN
+ * or infinity in src leaves the cache unchanged and raises the deferred NonFinite. A bf16 cache
+ * receives the values rounded to nearest even. */
+int32_t omx_kv_cache_write(omx_ctx* ctx, void* cache, int32_t cache_dtype, const void* src,
+                           uint64_t batch, uint64_t capacity, uint64_t kv_heads, uint64_t head_dim,
+                           uint64_t tn, uint64_t at);
 /* The batch that BatchSampler::next_batch reads (ojas-data/src/sampler.rs:262-275), built on the
  * device from a token bin resident in HBM: x[b, t] = tokens[starts[b] + t],
  * y[b, t] = tokens[starts[b] + t + 1], u32 [batch, seq_len]. `tokens` is the bin's little-endian
@@ -359,9 +383,11 @@ int32_t omx_topk_rows(omx_ctx* ctx, const void* x_f32, uint64_t rows, uint64_t c
 int32_t omx_read_scalar_f32(omx_ctx* ctx, const void* src, float* out);
 
 /* Tuning knobs (no counterpart in the reference). "gemm_dma": 0 = 128x128 GEMM
- * kernel only, 1 = choose by shape (default), 2 / 3 = force the 256x256 /
- * 256x128 direct-to-LDS kernel wherever the operands are eligible. Results are
- * within the same tolerances under every setting. */
+ * kernel only, 1 = choose by shape (default), 2 / 3 / 4 = force the 256x256 (64-column
+ * steps) / 256x128 (32-column steps) / 256x128 (64-column steps) direct-to-LDS kernel
+ * wherever the operands are eligible. "kv_attention": 0 = choose by head_dim (default),
+ * 1 = always the LDS-tiled kernel. Results are within the same tolerances under every
+ * setting. */
 int32_t omx_set_option(omx_ctx* ctx, const char* name, int64_t value);
 
 /* Benchmark instrumentation (no counterpart in the reference, whose benches

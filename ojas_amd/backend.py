@@ -191,6 +191,10 @@ class MiBackend:
             return (a.astype(np.uint32) << 16).view(np.float32)
         return a
 
+    def set_option(self, name: str, value: int):
+        """Tuning knobs of the library (`omx_set_option`); no counterpart in the reference."""
+        self._check(self._lib.omx_set_option(self._ctx, name.encode(), C.c_int64(value)))
+
     def sync(self):
         """BackendCore::sync (backend.rs:963-973)."""
         self._check(self._lib.omx_sync(self._ctx))
@@ -671,6 +675,40 @@ class MiBackend:
         return gv, gv0, gl
 
     # ---- integer ops ----
+    # ---- decode: KV cache (backend.rs:2526-2565) ----
+    def cached_attention_forward(self, q, k_cache, v_cache, kv_len: int, window: Optional[int] = None):
+        """q f32 [B,Tq,H,D] against ring caches [B,Tcap,Hkv,D] (f32, or bf16 storage); f32 [B,Tq,H,D]."""
+        if len(q.shape) != 4 or len(k_cache.shape) != 4 or k_cache.shape != v_cache.shape:
+            raise OjasError(SHAPE, "cached_attention_forward: q and the caches are rank 4, k_cache == v_cache")
+        b, tq, h, d = q.shape
+        kb, cap, hkv, kd = k_cache.shape
+        if kb != b or kd != d:
+            raise OjasError(SHAPE, f"cached_attention_forward: q {q.shape} and cache {k_cache.shape} disagree")
+        if window == 0:
+            raise OjasError(SHAPE, "cached_attention_forward: attention window must be at least 1")
+        if q.dtype != F32 or k_cache.dtype != v_cache.dtype:
+            raise OjasError(DTYPE, "cached_attention_forward: q is f32 and the caches share a dtype")
+        out = self.empty(q.shape, F32)
+        self._check(self._lib.omx_cached_attention_forward(
+            self._ctx, self._p(q), self._p(k_cache), self._p(v_cache), C.c_int32(k_cache.dtype), self._p(out),
+            C.c_uint64(b), C.c_uint64(tq), C.c_uint64(h), C.c_uint64(hkv), C.c_uint64(d), C.c_uint64(cap),
+            C.c_uint64(kv_len), C.c_uint64(window or 0)))
+        return out
+
+    def kv_cache_write(self, cache, src, at: int):
+        """In place: src f32 [B,Tn,Hkv,D] to positions at..at+Tn of the ring `cache` [B,Tcap,Hkv,D]."""
+        if len(cache.shape) != 4 or len(src.shape) != 4:
+            raise OjasError(SHAPE, "kv_cache_write: cache and src are rank 4")
+        b, cap, hkv, d = cache.shape
+        sb, tn, sh, sd = src.shape
+        if (sb, sh, sd) != (b, hkv, d):
+            raise OjasError(SHAPE, f"kv_cache_write: src {src.shape} does not fit cache {cache.shape}")
+        if src.dtype != F32:
+            raise OjasError(DTYPE, "kv_cache_write: src is f32")
+        self._check(self._lib.omx_kv_cache_write(self._ctx, self._p(cache), C.c_int32(cache.dtype), self._p(src),
+                                                 C.c_uint64(b), C.c_uint64(cap), C.c_uint64(hkv), C.c_uint64(d),
+                                                 C.c_uint64(tn), C.c_uint64(at)))
+
     def token_windows(self, tokens: DeviceTensor, starts, seq_len: int):
         """(x, y) u32 [batch, seq_len] from a bin resident on the device (`upload` of
         `TokenBin.read_raw`: U32 words, or u16 words uploaded as BF16-sized storage) and the host

@@ -41,6 +41,8 @@ static const char* kFaultNames[F_COUNT] = {
     "per_head_sigmoid_gate_backward",
     "value_residual_blend_forward",
     "value_residual_blend_backward",
+    "cached_attention_forward",
+    "kv_cache_write",
 };
 
 const char* omx_fault_name(uint32_t op) { return op < F_COUNT ? kFaultNames[op] : "unknown"; }

@@ -550,8 +550,13 @@ extern "C" {
 int32_t omx_set_option(omx_ctx* ctx, const char* name, int64_t value) {
   OMX_REQUIRE_CTX(ctx);
   if (name && strcmp(name, "gemm_dma") == 0) {
-    if (value < 0 || value > 3) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: gemm_dma takes 0..3");
+    if (value < 0 || value > 4) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: gemm_dma takes 0..4");
     ctx->gemm_dma_mode = static_cast<int>(value);
+    return OMX_OK;
+  }
+  if (name && strcmp(name, "kv_attention") == 0) {
+    if (value < 0 || value > 1) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: kv_attention takes 0..1");
+    ctx->kv_attention_mode = static_cast<int>(value);
     return OMX_OK;
   }
   return omx_fail(ctx, OMX_UNSUPPORTED, "set_option: unknown option %s", name ? name : "(null)");

@@ -52,6 +52,8 @@ enum OmxFaultOp : uint32_t {
   F_GATE_BACKWARD,
   F_VRES_FORWARD,
   F_VRES_BACKWARD,
+  F_CACHED_ATTENTION,
+  F_KV_CACHE_WRITE,
   F_COUNT
 };
 const char* omx_fault_name(uint32_t op);
@@ -82,6 +84,7 @@ struct omx_ctx {
   // Optional per-launch timing of the GEMM kernel (benchmark only).
   // 0: 128x128 kernel only; 1: choose by shape; 2 / 3: force the 256x256 / 256x128 direct-to-LDS kernel where eligible.
   int gemm_dma_mode = 1;
+  int kv_attention_mode = 0;  // 1: cached attention always takes the LDS-tiled kernel
   bool profile_gemm = false;
   struct TimedLaunch {
     hipEvent_t start, stop;

@@ -29,6 +29,11 @@
 //   embedding fwd/bwd         ojas-cuda goldens embed_*.npy; gather is a bit copy
 //   bf16 rounding             integer rule autocast.rs:70-96, value table in the tests
 //   argmax / topk             brute force in the tests
+//   cached attention, cache   no digest in the reference; with kv_len == Tq it is causal_sdpa_forward
+//   write                     after the layout permute (backend.rs:2526-2542), and for any ring
+//                             rotation its rows are the last Tq rows of causal_sdpa_forward over
+//                             the whole sequence, bit for bit (the digest-pinned routine); f64
+//                             brute-force softmax on top
 //   silu, mul, gate, blend    no digest or fixture in the reference holds these; pinned by
 //                             the known answers of ojas-cpu/tests/ops.rs:599-623,667-696,
 //                             the exp_exact pins under sigmoid, and f64 autograd in the tests
@@ -465,6 +470,87 @@ int orc_causal_sdpa_forward(const float* q, const float* k, const float* v, floa
     }
   });
   return status.load();
+}
+
+// ---- KV-cache attention and cache writes (ojas-cpu/src/kv.rs) ----
+// Caches are time-major rings [B, Tcap, Hkv, D]: position j lives in slot j % Tcap. Query i of Tq
+// sits at position p = kv_len - Tq + i and attends to positions first..=p (first = 0, or
+// p + 1 - window), oldest first, with the per-row arithmetic of causal_sdpa_forward
+// (kv.rs:164-256: score_rows, softmax_range, mix_values). Validation follows
+// cached_attention_dims / kv_cache_write_dims (ojas-core/src/shapes.rs:2758-2879). Only the slots
+// some query reads are checked for NaN / infinity (kv.rs:44-100); other slots may hold anything.
+int orc_cached_attention_forward(const float* q, const float* k_cache, const float* v_cache, float* out,
+                                 size_t batch, size_t tq, size_t heads, size_t kv_heads, size_t dim,
+                                 size_t capacity, size_t kv_len, size_t window) {
+  if (batch == 0 || tq == 0 || heads == 0 || kv_heads == 0 || dim == 0 || capacity == 0) return ORC_SHAPE;
+  if (heads % kv_heads != 0) return ORC_SHAPE;
+  if (kv_len < tq) return ORC_OUT_OF_RANGE;
+  if (window >= kv_len) window = 0;  // a window that covers every position is no window
+  size_t span = kv_len;
+  if (window != 0 && tq + (window - 1) < kv_len) span = tq + (window - 1);
+  if (span > capacity) return ORC_OUT_OF_RANGE;
+  const float scale = 1.0f / std::sqrt(static_cast<float>(static_cast<uint32_t>(dim)));
+  const size_t group = heads / kv_heads, stride = kv_heads * dim;
+  auto first_of = [&](size_t p) { return window == 0 ? size_t{0} : (p + 1 > window ? p + 1 - window : size_t{0}); };
+  // The slots of every position some query reads, both caches.
+  const size_t read_lo = first_of(kv_len - tq);
+  for (size_t b = 0; b < batch; ++b)
+    for (size_t j = read_lo; j < kv_len; ++j) {
+      const size_t at = (b * capacity + j % capacity) * stride;
+      if (!all_finite(k_cache + at, stride) || !all_finite(v_cache + at, stride)) return ORC_NON_FINITE;
+    }
+  if (!all_finite(q, batch * tq * heads * dim)) return ORC_NON_FINITE;
+  std::atomic<int> status{ORC_OK};
+  parallel_for(batch * heads, 1, [&](size_t lo, size_t hi) {
+    std::vector<float> scores(kv_len), probs(kv_len);
+    for (size_t task = lo; task < hi; ++task) {
+      const size_t b = task / heads, h = task % heads;
+      const float* kh = k_cache + (b * capacity * kv_heads + h / group) * dim;
+      const float* vh = v_cache + (b * capacity * kv_heads + h / group) * dim;
+      for (size_t i = 0; i < tq; ++i) {
+        const size_t p = kv_len - tq + i, first = first_of(p), n = p + 1 - first;
+        const float* qr = q + ((b * tq + i) * heads + h) * dim;
+        for (size_t a = 0; a < n; ++a) {
+          const float sc = dot_up(qr, kh + ((first + a) % capacity) * stride, dim) * scale;
+          if (!finite32(sc)) {
+            status = ORC_NON_FINITE;
+            return;
+          }
+          scores[a] = sc;
+        }
+        float max = -std::numeric_limits<float>::infinity();
+        for (size_t a = 0; a < n; ++a) max = (scores[a] > max) ? scores[a] : max;
+        float sum = 0.0f;
+        for (size_t a = 0; a < n; ++a) {
+          probs[a] = exp_exact(scores[a] - max);
+          sum += probs[a];
+        }
+        for (size_t a = 0; a < n; ++a) probs[a] /= sum;
+        if (!(finite32(sum) && sum > 0.0f)) {
+          status = ORC_NON_FINITE;
+          return;
+        }
+        float* o = out + ((b * tq + i) * heads + h) * dim;
+        for (size_t c = 0; c < dim; ++c) o[c] = 0.0f;
+        for (size_t a = 0; a < n; ++a) saxpy_up(o, vh + ((first + a) % capacity) * stride, probs[a], dim);
+      }
+    }
+  });
+  return status.load();
+}
+
+// kv.rs:258-292: all-or-nothing; src [B, Tn, Hkv, D] goes to positions at..at + Tn.
+int orc_kv_cache_write(float* cache, const float* src, size_t batch, size_t capacity, size_t kv_heads, size_t dim,
+                       size_t tn, size_t at) {
+  if (batch == 0 || capacity == 0 || kv_heads == 0 || dim == 0 || tn == 0) return ORC_SHAPE;
+  if (at + tn < at) return ORC_OUT_OF_RANGE;
+  if (tn > capacity) return ORC_OUT_OF_RANGE;
+  const size_t step = kv_heads * dim;
+  if (!all_finite(src, batch * tn * step)) return ORC_NON_FINITE;
+  for (size_t b = 0; b < batch; ++b)
+    for (size_t j = 0; j < tn; ++j)
+      std::memcpy(cache + (b * capacity + (at + j) % capacity) * step, src + (b * tn + j) * step, step * sizeof(float));
+  return ORC_OK;
 }
 
 // ojas-cpu/src/attn.rs:437-597: KV groups are independent; the query heads of

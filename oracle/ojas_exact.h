@@ -89,6 +89,15 @@ int orc_causal_sdpa_backward(const float* q, const float* k, const float* v, con
                              size_t batch, size_t heads, size_t kv_heads, size_t time, size_t dim,
                              size_t window);
 
+/* ---- KV-cache attention (ojas-cpu/src/kv.rs; trait ojas-core/src/backend.rs:2526-2565) ----
+ * q, out: [B,Tq,H,D]; caches: [B,Tcap,Hkv,D] rings (position j in slot j % Tcap).
+ * window = 0 means every earlier position. */
+int orc_cached_attention_forward(const float* q, const float* k_cache, const float* v_cache, float* out,
+                                 size_t batch, size_t tq, size_t heads, size_t kv_heads, size_t dim,
+                                 size_t capacity, size_t kv_len, size_t window);
+int orc_kv_cache_write(float* cache, const float* src, size_t batch, size_t capacity, size_t kv_heads, size_t dim,
+                       size_t tn, size_t at);
+
 /* ---- norms and RoPE (ojas-cpu/src/norm.rs) ---- */
 int orc_rms_norm_forward(const float* x, const float* w, float* y, size_t rows, size_t dim,
                          float eps);

@@ -642,3 +642,26 @@ def nanolab_loss_and_grads(cfg: NanolabConfig, params, ids, targets, want_logits
     _check(_lib.orc_nanolab_loss_and_grads(C.byref(cfg), pp, _up(ids), _up(targets), C.byref(loss),
                                            _fp(logits) if want_logits else None, gp), "nanolab_loss_and_grads")
     return np.float32(loss.value), logits, (grads if want_grads else None)
+
+
+def cached_attention_forward(q, k_cache, v_cache, kv_len: int, window: int = 0):
+    """q [B,Tq,H,D], caches [B,Tcap,Hkv,D] rings; returns [B,Tq,H,D]."""
+    q, k_cache, v_cache = _f32(q), _f32(k_cache), _f32(v_cache)
+    b, tq, h, d = q.shape
+    _, cap, hkv, _ = k_cache.shape
+    out = np.empty_like(q)
+    _check(
+        _lib.orc_cached_attention_forward(_fp(q), _fp(k_cache), _fp(v_cache), _fp(out), _sz(b), _sz(tq), _sz(h),
+                                          _sz(hkv), _sz(d), _sz(cap), _sz(kv_len), _sz(window)),
+        "cached_attention_forward",
+    )
+    return out
+
+
+def kv_cache_write(cache, src, at: int):
+    """Returns the updated copy of `cache` [B,Tcap,Hkv,D] after writing src [B,Tn,Hkv,D] at `at`."""
+    cache, src = _f32(cache).copy(), _f32(src)
+    b, cap, hkv, d = cache.shape
+    _check(_lib.orc_kv_cache_write(_fp(cache), _fp(src), _sz(b), _sz(cap), _sz(hkv), _sz(d), _sz(src.shape[1]), _sz(at)),
+           "kv_cache_write")
+    return cache
