@@ -28,8 +28,9 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, vendor figure
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor figure
 # HBM bytes per GEMM op (MFMA kernel + split-K reduce) on the gpt124m workload, averaged over the
-# step's 156 ops: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by what the same
+# step's GEMM ops (156 when this was measured): rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by what the same
 # counters read for the AdamW pass, whose traffic is known (profiles/gemm_hbm_traffic_gpt124m_bf16.txt).
 # The algorithmic figure (every operand read once, every output written once) is 1.569e8.
 GEMM_HBM_BYTES_PER_LAUNCH_GPT124M = 3.69e8
@@ -62,6 +63,63 @@ def cpu_baseline(cfg, threads: int):
                       f"({dt:.1f} s), scaled per token; C++ restatement of ojas-cpu, not the Rust binary"}
 
 
+def kv_decode(args) -> int:
+    """Secondary workload, the step after the training path: one `cached_attention_forward` call of
+    a decode step (one new token per sequence) over a full KV cache, GPT-124M shape: batch 64,
+    12 heads of 64, 1024 cached positions, f32 caches as the reference's trait prescribes. The op is
+    bound by reading both caches once; `value` is those bytes over the call time."""
+    sys.path.insert(0, str(ROOT / "tests"))
+    from ojas_amd.backend import MiBackend
+
+    b, h, d, t = 64, 12, 64, 1024
+    be = MiBackend(0)
+    r = np.random.default_rng(0)
+    q = be.upload(r.standard_normal((b, 1, h, d)).astype(np.float32))
+    kc = be.upload(r.standard_normal((b, t, h, d)).astype(np.float32))
+    vc = be.upload(r.standard_normal((b, t, h, d)).astype(np.float32))
+    for _ in range(args.warmup):
+        be.cached_attention_forward(q, kc, vc, t)
+    be.sync()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out = be.cached_attention_forward(q, kc, vc, t)
+    be.sync()
+    dt = (time.perf_counter() - t0) / args.steps
+    nbytes = 2 * b * t * h * d * 4
+    gbs = nbytes / dt / 1e9
+    line = {
+        "metric": "KV-cache attention, decode step (GPT-124M shape, batch 64, 1024 cached positions): cache GB/s",
+        "value": gbs, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "cached_attention_forward: q [64,1,12,64], caches [64,1024,12,64] f32, kv_len 1024",
+                   "tokens_per_step": b},
+        "roofline": {"bound": "hbm", "kernel": "cached_attention_group_kernel + cached_attention_merge_kernel",
+                     "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                     "traffic": None, "algorithmic_bytes_per_launch": nbytes},
+    }
+    if not args.no_cpu_baseline:
+        import oracle_api as orc
+
+        sb = 4  # a bounded sample: 4 of the 64 sequences
+        hq, hk, hv = (be.download(x)[:sb] for x in (q, kc, vc))
+        c0 = time.perf_counter()
+        reps = 0
+        while time.perf_counter() - c0 < 5.0:
+            want = orc.cached_attention_forward(hq, hk, hv, t)
+            reps += 1
+        cdt = (time.perf_counter() - c0) / reps
+        got = be.download(out)[:sb]
+        assert np.abs(got - want).max() <= 1e-5 * max(1.0, float(np.abs(want).max()))
+        line["cpu_baseline"] = {"value": 2 * sb * t * h * d * 4 / cdt / 1e9, "unit": "GB/s",
+                                "cores": min(16, os.cpu_count() or 1), "kind": "port",
+                                "sample": f"{sb} of the 64 sequences, {reps} calls in 5 s; C++ restatement of "
+                                          "ojas-cpu/src/kv.rs (per-row Exact kernel), not the Rust binary"}
+    be.close()
+    print(json.dumps(line))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -69,10 +127,14 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--config", default="gpt124m", choices=["gpt124m", "tiny"])
+    ap.add_argument("--workload", default="train_step", choices=["train_step", "kv_decode"],
+                    help="train_step: the headline metric (default); kv_decode: the decode attention op alone")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).", file=sys.stderr)
         return 2
+    if args.workload == "kv_decode":
+        return kv_decode(args)
 
     from ojas_amd.backend import AdamWConfig, MiBackend
     from ojas_amd.trainer import GptTrainer, config_gpt124m_bf16, config_tiny_f32, step_flops, synthetic_batch
