@@ -50,6 +50,12 @@ int32_t ogpt_loss_and_grads(ogpt* t, float* loss);
  * gradients, clip_grad_norm(grad_clip; <= 0 disables clipping but still
  * measures the norm), adamw_step on every parameter, loss readback. */
 int32_t ogpt_step(ogpt* t, const omx_adamw_config* adamw, float grad_clip, float* loss, float* grad_norm);
+/* The same step with the reference trainer's hybrid groups (ojas-model/src/trainer.rs:858-876,
+ * ojas-cpu/src/train.rs:20-62): muon_ns5_step on every 2-D hidden matrix (wq, wk, wv, wo, w1, w2 of
+ * each layer, each its own matrix), adamw_step on the two tables and the norm weights. Muon's
+ * momentum lives where AdamW's first moment would. */
+int32_t ogpt_step_hybrid(ogpt* t, const omx_muon_config* muon, const omx_adamw_config* adamw, float grad_clip,
+                         float* loss, float* grad_norm);
 /* Optimizer steps taken so far. */
 uint64_t ogpt_steps(ogpt* t);
 /* Bytes of device memory the trainer holds. */

@@ -435,4 +435,44 @@ int32_t ogpt_step(ogpt* t, const omx_adamw_config* adamw, float grad_clip, float
   return OMX_OK;
 }
 
+// Trainer::apply with the hybrid groups (ojas-model/src/trainer.rs:858-876, :1004-1028): Muon-NS5
+// on every 2-D hidden matrix, AdamW on the tables and the norm weights.
+int32_t ogpt_step_hybrid(ogpt* t, const omx_muon_config* muon, const omx_adamw_config* adamw, float grad_clip,
+                         float* loss, float* grad_norm) {
+  if (!t || !muon || !adamw) return OMX_BACKEND;
+  TRY(forward(t));
+  TRY(backward(t));
+  void* grads[1] = {t->g32};
+  uint64_t lens[1] = {t->P};
+  float norm = 0.0f;
+  TRY(omx_clip_grad_norm(t->ctx, grads, lens, 1, grad_clip > 0.0f ? grad_clip : INFINITY, &norm));
+  uint16_t* mirror = static_cast<uint16_t*>(t->p16);
+  auto adam = [&](uint64_t first, uint64_t last) -> int32_t {  // slots [first, last] are adjacent in the arena
+    const uint64_t at = t->slots[first].offset, n = t->slots[last].offset + t->slots[last].len - at;
+    return omx_adamw_step(t->ctx, t->p32 + at, t->g32 + at, t->m1 + at, t->m2 + at, n, t->steps, adamw,
+                          mirror ? mirror + at : nullptr);
+  };
+  auto matrix = [&](uint64_t slot, uint64_t rows, uint64_t cols) -> int32_t {
+    const uint64_t at = t->slots[slot].offset;  // the AdamW first-moment arena holds Muon's momentum
+    return omx_muon_ns5_step(t->ctx, t->p32 + at, t->g32 + at, t->m1 + at, rows, cols, muon,
+                             mirror ? mirror + at : nullptr);
+  };
+  const uint64_t d = t->c.d_model, mlp = t->c.mlp;
+  TRY(adam(0, 1));  // token and position tables
+  for (uint64_t l = 0; l < t->c.layers; ++l) {
+    TRY(adam(t->li(l, 0), t->li(l, 0)));
+    for (uint64_t w = 1; w <= 4; ++w) TRY(matrix(t->li(l, w), d, d));
+    TRY(adam(t->li(l, 5), t->li(l, 5)));
+    TRY(matrix(t->li(l, 6), mlp, d));
+    TRY(matrix(t->li(l, 7), d, mlp));
+  }
+  TRY(adam(t->nf(), t->nf()));
+  float l = 0.0f;
+  TRY(omx_read_scalar_f32(t->ctx, t->loss, &l));
+  t->steps += 1;
+  if (loss) *loss = l;
+  if (grad_norm) *grad_norm = norm;
+  return OMX_OK;
+}
+
 }  // extern "C"

@@ -113,6 +113,14 @@ class GptTrainer:
                                                 C.byref(norm)))
         return float(loss.value), float(norm.value)
 
+    def step_hybrid(self, muon, adamw: AdamWConfig, grad_clip: float = 1.0) -> Tuple[float, float]:
+        """One step with Muon-NS5 on the hidden matrices and AdamW on tables and norms
+        (`Trainer::apply`, trainer.rs:1004-1028); `muon` is a `MuonNs5Config`."""
+        loss, norm = C.c_float(), C.c_float()
+        self.backend._check(self._lib.ogpt_step_hybrid(self._h, C.byref(muon), C.byref(adamw), C.c_float(grad_clip),
+                                                       C.byref(loss), C.byref(norm)))
+        return float(loss.value), float(norm.value)
+
     def steps(self) -> int:
         return int(self._lib.ogpt_steps(self._h))
 
