@@ -189,8 +189,13 @@ def main() -> int:
         "vs_baseline": None,
         "dtype": "bf16" if cfg.bf16 else "f32",
         "data": "synthetic",
-        "config": {"workload": "GPT-124M-shape training step (BASELINE configs[2]): L12 d768 H12x64 mlp3072 ctx1024 "
-                               "vocab50304 batch16, bf16 operands, f32 master weights, AdamW lr3e-4 wd0.1, clip 1.0"
+        "config": {"workload": ("GPT-124M-shape training step (BASELINE configs[2]): L12 d768 H12x64 mlp3072 ctx1024 "
+                                "vocab50304 batch16, bf16 operands, f32 master weights, AdamW lr3e-4 wd0.1, clip 1.0"
+                                if args.optimizer == "adamw" else
+                                "GPT-124M-shape training step (BASELINE configs[3]): L12 d768 H12x64 mlp3072 ctx1024 "
+                                "vocab50304 batch16, bf16 operands, f32 master weights, Muon-NS5 (bf16 iteration, lr 0.02, "
+                                "momentum 0.95, wd 0.1, Nesterov) on the 72 hidden matrices, AdamW lr3e-4 on tables and "
+                                "norms, clip 1.0")
                    if args.config == "gpt124m" else "nanolab-GPT tiny f32 step (BASELINE configs[0])",
                    "tokens_per_step": tokens, "params": sum(tr.param_lens())},
         "step_tflops": flops / (ms_per_step * 1e-3) / 1e12,

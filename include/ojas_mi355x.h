@@ -242,6 +242,15 @@ typedef struct {
 int32_t omx_muon_ns5_step(omx_ctx* ctx, void* param_f32, const void* grad_f32, void* momentum_f32,
                           uint64_t rows, uint64_t cols, const omx_muon_config* config,
                           void* param_bf16);
+/* The same step for `count` tensors of one shape in one set of launches (no counterpart in
+ * the reference, whose trainer calls muon_ns5_step once per tensor, trainer.rs:1004-1028): the
+ * arithmetic per tensor is that of omx_muon_ns5_step, the Newton-Schulz products run as strided
+ * batches. The arrays hold `count` device pointers (params_bf16 may be null, or hold nulls).
+ * All or nothing for the whole batch: a non-finite value in any tensor leaves all of them
+ * unchanged. Scratch: count * omx_muon_scratch_bytes(rows, cols), at most 64 tensors at a time. */
+int32_t omx_muon_ns5_step_batched(omx_ctx* ctx, void* const* params_f32, const void* const* grads_f32,
+                                  void* const* momenta_f32, void* const* params_bf16, uint64_t count,
+                                  uint64_t rows, uint64_t cols, const omx_muon_config* config);
 /* Bytes of device scratch omx_muon_ns5_step takes from the budget
  * (BackendCore::optimizer_scratch_bytes, backend.rs:938-961). */
 uint64_t omx_muon_scratch_bytes(uint64_t rows, uint64_t cols);

@@ -458,6 +458,18 @@ class MiBackend:
                                                 C.c_uint64(rows), C.c_uint64(cols), C.byref(config),
                                                 self._p(param_bf16)))
 
+    def muon_ns5_step_batched(self, params, grads, momenta, config: MuonNs5Config, params_bf16=None):
+        """`muon_ns5_step` on several tensors of one shape in one set of launches (in place)."""
+        n = len(params)
+        rows, cols = params[0].shape
+        if any(p.shape != (rows, cols) for p in params) or len(grads) != n or len(momenta) != n:
+            raise OjasError(SHAPE, "muon_ns5_step_batched: tensors of one shape, one gradient and momentum each")
+        table = lambda ts: (C.c_void_p * n)(*[t.ptr for t in ts])
+        mirrors = (C.c_void_p * n)(*[(t.ptr if t is not None else None) for t in params_bf16]) if params_bf16 else None
+        self._check(self._lib.omx_muon_ns5_step_batched(self._ctx, table(params), table(grads), table(momenta), mirrors,
+                                                        C.c_uint64(n), C.c_uint64(rows), C.c_uint64(cols),
+                                                        C.byref(config)))
+
     def clip_grad_norm(self, grads: Sequence[DeviceTensor], max_norm: float) -> float:
         n = len(grads)
         ptrs = (C.c_void_p * max(n, 1))(*[g.ptr for g in grads])

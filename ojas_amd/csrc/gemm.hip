@@ -230,6 +230,7 @@ __global__ __launch_bounds__(NT) void gemm_kernel(GemmArgs g) {
   constexpr int A_BYTES = tile_bytes<T, A_KM, BM>(), B_BYTES = tile_bytes<T, B_KM, BN>();
   constexpr int STAGE = A_BYTES + B_BYTES;
   static_assert(sizeof(T) == 2 || (TM == 2 && TN == 2), "the f32 lane uses 128x128 tiles");
+  gemm_select_batch(g);
   const T* __restrict__ A = static_cast<const T*>(g.a);
   const T* __restrict__ B = static_cast<const T*>(g.b);
 
@@ -378,7 +379,7 @@ int32_t launch_one(omx_ctx* ctx, const GemmArgs& g) {
     granted = true;
   }
   const int total = g.tiles_m * g.tiles_n * g.splits;
-  hipLaunchKernelGGL(kernel, dim3(total), dim3(NT), smem, ctx->stream, g);
+  hipLaunchKernelGGL(kernel, dim3(total, g.batches), dim3(NT), smem, ctx->stream, g);
   OMX_LAUNCH_CHECK(ctx, "gemm_kernel");
   return OMX_OK;
 }
@@ -407,8 +408,11 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 // Internal entry shared by the linear ops, the fused loss and Muon.
 int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a_rs, uint64_t a_cs, const void* b,
                       uint64_t b_rs, uint64_t b_cs, int32_t operand_dtype, void* c, int32_t c_dtype, uint64_t ldc,
-                      uint64_t m, uint64_t k, uint64_t n, int32_t accumulate, const OmxGemmEpilogue* epi) {
+                      uint64_t m, uint64_t k, uint64_t n, int32_t accumulate, const OmxGemmEpilogue* epi,
+                      const OmxGemmBatch* batch) {
   const char* op = omx_fault_name(fault_op);
+  const uint64_t batches = batch ? batch->count : 1;
+  if (batches == 0 || batches > 65535) return omx_fail(ctx, OMX_OUT_OF_RANGE, "%s: 1..65535 products per launch", op);
   if (epi && epi->mode != OMX_EPI_NONE && c_dtype != OMX_BF16)
     return omx_fail(ctx, OMX_DTYPE, "%s: a fused activation needs a bf16 output", op);
   if (!a || !b || !c) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
@@ -454,6 +458,16 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
   g.a_vec = aligned16(a) && (lda % kv == 0);
   g.b_vec = aligned16(b) && (ldb % kv == 0);
   g.c_vec = aligned16(c) && (ldc % 4 == 0);
+  g.batches = static_cast<int>(batches);
+  g.batch_a = g.batch_b = g.batch_c = 0;
+  if (batches > 1) {
+    const uint64_t esz = operand_dtype == OMX_BF16 ? 2 : 4, csz = c_dtype == OMX_BF16 ? 2 : 4;
+    g.batch_a = static_cast<long>(batch->stride_a * esz);
+    g.batch_b = static_cast<long>(batch->stride_b * esz);
+    g.batch_c = static_cast<long>(batch->stride_c * csz);
+    if ((g.batch_a | g.batch_b | g.batch_c) & 15)
+      return omx_fail(ctx, OMX_SHAPE, "%s: batch strides must be multiples of 16 bytes", op);
+  }
   // Kernel choice. bf16 shapes whose output fills the chip with 256 x 256 (or
   // 256 x 128) tiles take the direct-to-LDS kernel; everything else (f32, odd
   // shapes, small outputs that need split-K) takes the 128 x 128 kernel.
@@ -468,7 +482,7 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
       // products. The 64-column forms fetch whole cache lines but run alone on their compute
       // unit; they win only on long reductions with large outputs (8192^3: 1.09 against
       // 0.95 PFLOP/s for 256 x 256) and lose on every GPT shape.
-      if (static_cast<long>(g.M) * g.N <= (1l << 20)) dma_variant = -1;
+      if (static_cast<long>(g.M) * g.N * g.batches <= (1l << 20)) dma_variant = -1;
       else dma_variant = 3;
     }
     else if (mode == 2) dma_variant = 0;
@@ -488,7 +502,7 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
     const int ksteps = (g.K + bk - 1) / bk;
     const long tiles = static_cast<long>(g.tiles_m) * g.tiles_n;
     int splits = 1;
-    if (tiles < 256 && ksteps >= 32 && !(epi && epi->mode != OMX_EPI_NONE)) {
+    if (tiles * g.batches < 256 && g.batches == 1 && ksteps >= 32 && !(epi && epi->mode != OMX_EPI_NONE)) {
       splits = static_cast<int>((512 + tiles - 1) / tiles);
       if (splits > ksteps / 8) splits = ksteps / 8;
       if (splits < 1) splits = 1;
@@ -521,7 +535,7 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
     };
     OMX_HIP(ctx, take(&timed.start));
     OMX_HIP(ctx, take(&timed.stop));
-    timed.flops = 2.0 * static_cast<double>(m) * static_cast<double>(n) * static_cast<double>(k);
+    timed.flops = 2.0 * static_cast<double>(m) * static_cast<double>(n) * static_cast<double>(k) * static_cast<double>(batches);
     OMX_HIP(ctx, hipEventRecord(timed.start, ctx->stream));
   }
   int32_t rc;

@@ -20,7 +20,21 @@ struct GemmArgs {
   unsigned short* aux_out;
   OmxFaultWord* fault;
   unsigned long long tag;
+  // Strided batch: block (x, y) works on product y, whose operands start batch_* BYTES after
+  // product y - 1's. batches == 1 for a single product.
+  int batches;
+  long batch_a, batch_b, batch_c;
 };
+
+// The arguments of the product this block belongs to.
+__device__ __forceinline__ void gemm_select_batch(GemmArgs& g) {
+  if (g.batches > 1) {
+    const long y = blockIdx.y;
+    g.a = static_cast<const char*>(g.a) + y * g.batch_a;
+    g.b = static_cast<const char*>(g.b) + y * g.batch_b;
+    g.c = static_cast<char*>(g.c) + y * g.batch_c;
+  }
+}
 
 // Stores four consecutive columns of one output row (row `grow`, columns
 // gcol..gcol+3, clipped to N): a split-K partial, a bf16 result, or an f32

@@ -133,6 +133,7 @@ __global__ __launch_bounds__(DT, (NST * (WGM * TM + WGN * TN) * 32 * DBK * 2 <= 
   constexpr int LPS = STAGE / 1024 / 8;  // loads per wave per step
   constexpr int KK = DBK / 16;           // MFMA K slabs per step
   static_assert(WGM * WGN == 8, "eight waves");
+  gemm_select_batch(g);
   const unsigned short* __restrict__ A = static_cast<const unsigned short*>(g.a);
   const unsigned short* __restrict__ B = static_cast<const unsigned short*>(g.b);
 
@@ -310,7 +311,7 @@ int32_t launch_dma(omx_ctx* ctx, const GemmArgs& g) {
                                      smem));
     granted = true;
   }
-  hipLaunchKernelGGL(kernel, dim3(g.tiles_m * g.tiles_n * g.splits), dim3(DT), smem, ctx->stream, g);
+  hipLaunchKernelGGL(kernel, dim3(g.tiles_m * g.tiles_n * g.splits, g.batches), dim3(DT), smem, ctx->stream, g);
   OMX_LAUNCH_CHECK(ctx, "gemm_dma_kernel");
   return OMX_OK;
 }

@@ -15,6 +15,7 @@
 //
 // The step is all-or-nothing: a refuse flag raised by any non-finite
 // intermediate keeps the final pass from writing the parameter or the momentum.
+#include <algorithm>
 #include <cmath>
 
 #include "omx_common.h"
@@ -22,7 +23,7 @@
 namespace {
 
 constexpr int MU_THREADS = 256;
-constexpr size_t MU_BLOCK = 1 << 14;  // elements per sum-of-squares partial
+constexpr size_t MU_BLOCK = 1 << 11;  // elements per sum-of-squares partial (8 per thread: a 768 x 768 matrix fills the chip)
 
 struct MuonScalars {
   float mom, alpha, decay, a, b, c;
@@ -35,14 +36,39 @@ inline unsigned mu_grid(uint64_t n) {
   return static_cast<unsigned>(blocks ? blocks : 1);
 }
 
+// One launch serves up to MU_MAX_BATCH matrices of one shape: block (x, y) works on matrix y. The
+// tensors the caller owns come as pointer tables in the kernel arguments; the intermediates of
+// matrix y live `stride` bytes after matrix y - 1's in the workspace, at the offsets of MuonLayout.
+constexpr int MU_MAX_BATCH = 64;
+struct MuonTensors {
+  float* p[MU_MAX_BATCH];
+  const float* g[MU_MAX_BATCH];
+  float* m[MU_MAX_BATCH];
+  unsigned short* p16[MU_MAX_BATCH];  // entries may be null
+};
+struct MuonLayout {
+  uint64_t buf, u, x, xn, a, a2, partial, scalars, total;
+};
+struct MuonWork {
+  char* ws;
+  uint64_t stride;  // bytes between consecutive matrices' blocks
+  MuonLayout L;
+  unsigned int* refuse;  // one flag for the whole launch
+  template <typename T>
+  __device__ __forceinline__ T* at(uint64_t offset) const {
+    return reinterpret_cast<T*>(ws + blockIdx.y * stride + offset);
+  }
+};
+
 // buf, the (possibly bf16-rounded) update u, and per-block f64 sums of u^2.
-__global__ __launch_bounds__(MU_THREADS) void muon_momentum_kernel(const float* __restrict__ g,
-                                                                   const float* __restrict__ m,
-                                                                   float* __restrict__ buf, float* __restrict__ u,
-                                                                   double* __restrict__ partial, size_t n,
-                                                                   MuonScalars s, unsigned int* refuse,
+__global__ __launch_bounds__(MU_THREADS) void muon_momentum_kernel(MuonTensors t, MuonWork w, size_t n, MuonScalars s,
                                                                    OmxFaultWord* fault, unsigned long long tag) {
   __shared__ double red[MU_THREADS];
+  const float* __restrict__ g = t.g[blockIdx.y];
+  const float* __restrict__ m = t.m[blockIdx.y];
+  float* __restrict__ buf = w.at<float>(w.L.buf);
+  float* __restrict__ u = w.at<float>(w.L.u);
+  double* __restrict__ partial = w.at<double>(w.L.partial);
   const size_t begin = static_cast<size_t>(blockIdx.x) * MU_BLOCK, end = min(n, begin + MU_BLOCK);
   double acc = 0.0;
   bool bad = false;
@@ -64,16 +90,16 @@ __global__ __launch_bounds__(MU_THREADS) void muon_momentum_kernel(const float* 
   }
   if (threadIdx.x == 0) partial[blockIdx.x] = red[0];
   if (bad) {
-    atomicOr(refuse, 1u);
+    atomicOr(w.refuse, 1u);
     dev_raise_fault(fault, tag);
   }
 }
 
-__global__ __launch_bounds__(1024) void muon_norm_kernel(const double* __restrict__ partial, size_t count,
-                                                         float* __restrict__ denom_out, int bf16,
-                                                         unsigned int* refuse, OmxFaultWord* fault,
+// One block per matrix (blockIdx.y): the norm and the quotient's denominator.
+__global__ __launch_bounds__(1024) void muon_norm_kernel(MuonWork w, size_t count, int bf16, OmxFaultWord* fault,
                                                          unsigned long long tag) {
   __shared__ double red[1024];
+  const double* __restrict__ partial = w.at<double>(w.L.partial);
   double acc = 0.0;
   for (size_t i = threadIdx.x; i < count; i += 1024) acc += partial[i];
   red[threadIdx.x] = acc;
@@ -86,18 +112,19 @@ __global__ __launch_bounds__(1024) void muon_norm_kernel(const double* __restric
     float norm = static_cast<float>(sqrt(red[0]));
     const float eps = 1e-7f;
     float denom = bf16 ? dev_round_bf16(dev_round_bf16(norm) + eps) : norm + eps;
-    *denom_out = denom;
+    *w.at<float>(w.L.scalars + 16) = denom;
     if (!(dev_finite(denom) && denom != 0.0f)) {
-      atomicOr(refuse, 1u);
+      atomicOr(w.refuse, 1u);
       dev_raise_fault(fault, tag);
     }
   }
 }
 
 template <typename TX>
-__global__ void muon_normalize_kernel(const float* __restrict__ u, const float* __restrict__ denom,
-                                      TX* __restrict__ x, size_t n) {
-  const float d = *denom;
+__global__ void muon_normalize_kernel(MuonWork w, uint64_t x_off, size_t n) {
+  const float* __restrict__ u = w.at<float>(w.L.u);
+  TX* __restrict__ x = w.at<TX>(x_off);
+  const float d = *w.at<float>(w.L.scalars + 16);
   for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
        i += static_cast<size_t>(gridDim.x) * blockDim.x)
     dev_store<TX>(x, i, u[i] / d);  // bf16 storage rounds the quotient
@@ -105,7 +132,9 @@ __global__ void muon_normalize_kernel(const float* __restrict__ u, const float* 
 
 // B = b A + c A2 (in place over A2), with the bf16 roundings of optim.rs:913-921.
 template <typename TX>
-__global__ void muon_combine_b_kernel(const TX* __restrict__ am, TX* __restrict__ a2, size_t n, MuonScalars s) {
+__global__ void muon_combine_b_kernel(MuonWork w, size_t n, MuonScalars s) {
+  const TX* __restrict__ am = w.at<TX>(w.L.a);
+  TX* __restrict__ a2 = w.at<TX>(w.L.a2);
   for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
        i += static_cast<size_t>(gridDim.x) * blockDim.x) {
     float av = dev_load<TX>(am, i), a2v = dev_load<TX>(a2, i);
@@ -118,8 +147,10 @@ __global__ void muon_combine_b_kernel(const TX* __restrict__ am, TX* __restrict_
 
 // X_next = a X + BX (in place over BX), finite-checked (optim.rs:950-962).
 template <typename TX>
-__global__ void muon_combine_x_kernel(const TX* __restrict__ x, TX* __restrict__ bx, size_t n, MuonScalars s,
-                                      unsigned int* refuse, OmxFaultWord* fault, unsigned long long tag) {
+__global__ void muon_combine_x_kernel(MuonWork w, uint64_t x_off, uint64_t bx_off, size_t n, MuonScalars s,
+                                      OmxFaultWord* fault, unsigned long long tag) {
+  const TX* __restrict__ x = w.at<TX>(x_off);
+  TX* __restrict__ bx = w.at<TX>(bx_off);
   bool bad = false;
   for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
        i += static_cast<size_t>(gridDim.x) * blockDim.x) {
@@ -130,15 +161,16 @@ __global__ void muon_combine_x_kernel(const TX* __restrict__ x, TX* __restrict__
     dev_store<TX>(bx, i, r);
   }
   if (bad) {
-    atomicOr(refuse, 1u);
+    atomicOr(w.refuse, 1u);
     dev_raise_fault(fault, tag);
   }
 }
 
 template <typename TX>
-__global__ void muon_check_update_kernel(const float* __restrict__ p, const TX* __restrict__ x, size_t n,
-                                         MuonScalars s, unsigned int* refuse, OmxFaultWord* fault,
-                                         unsigned long long tag) {
+__global__ void muon_check_update_kernel(MuonTensors t, MuonWork w, uint64_t x_off, size_t n, MuonScalars s,
+                                         OmxFaultWord* fault, unsigned long long tag) {
+  const float* __restrict__ p = t.p[blockIdx.y];
+  const TX* __restrict__ x = w.at<TX>(x_off);
   bool bad = false;
   for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
        i += static_cast<size_t>(gridDim.x) * blockDim.x) {
@@ -146,16 +178,19 @@ __global__ void muon_check_update_kernel(const float* __restrict__ p, const TX* 
     bad |= !dev_finite(fmaf(s.alpha, dev_load<TX>(x, i), base));
   }
   if (bad) {
-    atomicOr(refuse, 1u);
+    atomicOr(w.refuse, 1u);
     dev_raise_fault(fault, tag);
   }
 }
 
 template <typename TX>
-__global__ void muon_apply_kernel(float* __restrict__ p, float* __restrict__ m, const float* __restrict__ buf,
-                                  const TX* __restrict__ x, size_t n, MuonScalars s,
-                                  const unsigned int* __restrict__ refuse, unsigned short* __restrict__ p_bf16) {
-  if (*refuse) return;
+__global__ void muon_apply_kernel(MuonTensors t, MuonWork w, uint64_t x_off, size_t n, MuonScalars s) {
+  if (*w.refuse) return;
+  float* __restrict__ p = t.p[blockIdx.y];
+  float* __restrict__ m = t.m[blockIdx.y];
+  unsigned short* __restrict__ p_bf16 = t.p16[blockIdx.y];
+  const float* __restrict__ buf = w.at<float>(w.L.buf);
+  const TX* __restrict__ x = w.at<TX>(x_off);
   for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
        i += static_cast<size_t>(gridDim.x) * blockDim.x) {
     float base = s.decays ? p[i] * s.decay : p[i];
@@ -166,9 +201,6 @@ __global__ void muon_apply_kernel(float* __restrict__ p, float* __restrict__ m, 
   }
 }
 
-struct MuonLayout {
-  uint64_t buf, u, x, xn, a, a2, partial, scalars, total;
-};
 MuonLayout muon_layout(uint64_t rows, uint64_t cols) {
   auto up = [](uint64_t v) { return (v + 255) & ~255ull; };
   const uint64_t len = rows * cols, r = rows < cols ? rows : cols;
@@ -194,77 +226,66 @@ MuonLayout muon_layout(uint64_t rows, uint64_t cols) {
   return L;
 }
 
+// `count` (<= MU_MAX_BATCH) matrices of one shape; ws holds count blocks of L.total bytes.
 template <typename TX>
-int32_t run_muon(omx_ctx* ctx, float* p, const float* g, float* m, uint64_t rows, uint64_t cols, MuonScalars s,
-                 unsigned short* p_bf16, char* ws, const MuonLayout& L, unsigned long long tag) {
+int32_t run_muon(omx_ctx* ctx, const MuonTensors& t, unsigned count, uint64_t rows, uint64_t cols, MuonScalars s,
+                 char* ws, const MuonLayout& L, unsigned long long tag) {
   const uint64_t len = rows * cols;
   const int32_t XD = sizeof(TX) == 2 ? OMX_BF16 : OMX_F32;
-  float* buf = reinterpret_cast<float*>(ws + L.buf);
-  float* u = reinterpret_cast<float*>(ws + L.u);
-  TX* x = reinterpret_cast<TX*>(ws + L.x);
-  TX* xn = reinterpret_cast<TX*>(ws + L.xn);
-  TX* am = reinterpret_cast<TX*>(ws + L.a);
-  TX* a2 = reinterpret_cast<TX*>(ws + L.a2);
-  double* partial = reinterpret_cast<double*>(ws + L.partial);
-  unsigned int* refuse = reinterpret_cast<unsigned int*>(ws + L.scalars);
-  float* denom = reinterpret_cast<float*>(ws + L.scalars + 16);
-  int32_t rc = omx_fill_zero(ctx, refuse, 4);
+  MuonWork w;
+  w.ws = ws;
+  w.stride = L.total;
+  w.L = L;
+  w.refuse = reinterpret_cast<unsigned int*>(ws + L.scalars);
+  int32_t rc = omx_fill_zero(ctx, w.refuse, 4);
   if (rc != OMX_OK) return rc;
+  uint64_t x_off = L.x, xn_off = L.xn;
   const unsigned nb = static_cast<unsigned>((len + MU_BLOCK - 1) / MU_BLOCK);
-  hipLaunchKernelGGL(muon_momentum_kernel, dim3(nb), dim3(MU_THREADS), 0, ctx->stream, g, m, buf, u, partial, len, s,
-                     refuse, ctx->fault, tag);
-  hipLaunchKernelGGL(muon_norm_kernel, dim3(1), dim3(1024), 0, ctx->stream, partial, static_cast<size_t>(nb), denom,
-                     s.bf16, refuse, ctx->fault, tag);
-  hipLaunchKernelGGL((muon_normalize_kernel<TX>), dim3(mu_grid(len)), dim3(MU_THREADS), 0, ctx->stream, u, denom, x,
-                     len);
+  const dim3 block(MU_THREADS), over_len(mu_grid(len), count);
+  hipLaunchKernelGGL(muon_momentum_kernel, dim3(nb, count), block, 0, ctx->stream, t, w, len, s, ctx->fault, tag);
+  hipLaunchKernelGGL(muon_norm_kernel, dim3(1, count), dim3(1024), 0, ctx->stream, w, static_cast<size_t>(nb), s.bf16,
+                     ctx->fault, tag);
+  hipLaunchKernelGGL((muon_normalize_kernel<TX>), over_len, block, 0, ctx->stream, w, x_off, len);
   OMX_LAUNCH_CHECK(ctx, "muon prologue");
   const bool tall = rows > cols;
   const uint64_t r = tall ? cols : rows, c = tall ? rows : cols;
+  const uint64_t es = L.total / sizeof(TX);  // elements between consecutive matrices' buffers
+  const OmxGemmBatch batch{count, es, es, es};
+  const OmxGemmBatch* bp = count > 1 ? &batch : nullptr;
+  TX* am = reinterpret_cast<TX*>(ws + L.a);
+  TX* a2 = reinterpret_cast<TX*>(ws + L.a2);
   for (int it = 0; it < 5; ++it) {
+    TX* x = reinterpret_cast<TX*>(ws + x_off);
+    TX* xn = reinterpret_cast<TX*>(ws + xn_off);
     // A = X' X'^T with X' the short-side-first reading of X.
-    if (!tall) rc = omx_gemm_impl(ctx, F_MUON, x, cols, 1, x, 1, cols, XD, am, XD, r, r, c, r, 0);
-    else rc = omx_gemm_impl(ctx, F_MUON, x, 1, cols, x, cols, 1, XD, am, XD, r, r, c, r, 0);
+    if (!tall) rc = omx_gemm_impl(ctx, F_MUON, x, cols, 1, x, 1, cols, XD, am, XD, r, r, c, r, 0, nullptr, bp);
+    else rc = omx_gemm_impl(ctx, F_MUON, x, 1, cols, x, cols, 1, XD, am, XD, r, r, c, r, 0, nullptr, bp);
     if (rc != OMX_OK) return rc;
-    rc = omx_gemm_impl(ctx, F_MUON, am, r, 1, am, r, 1, XD, a2, XD, r, r, r, r, 0);
+    rc = omx_gemm_impl(ctx, F_MUON, am, r, 1, am, r, 1, XD, a2, XD, r, r, r, r, 0, nullptr, bp);
     if (rc != OMX_OK) return rc;
-    hipLaunchKernelGGL((muon_combine_b_kernel<TX>), dim3(mu_grid(r * r)), dim3(MU_THREADS), 0, ctx->stream, am, a2,
+    hipLaunchKernelGGL((muon_combine_b_kernel<TX>), dim3(mu_grid(r * r), count), block, 0, ctx->stream, w,
                        static_cast<size_t>(r * r), s);
     // BX in X's own physical layout: B X' when wide, X B^T when tall.
-    if (!tall) rc = omx_gemm_impl(ctx, F_MUON, a2, r, 1, x, cols, 1, XD, xn, XD, cols, r, r, c, 0);
-    else rc = omx_gemm_impl(ctx, F_MUON, x, cols, 1, a2, 1, r, XD, xn, XD, cols, rows, cols, cols, 0);
+    if (!tall) rc = omx_gemm_impl(ctx, F_MUON, a2, r, 1, x, cols, 1, XD, xn, XD, cols, r, r, c, 0, nullptr, bp);
+    else rc = omx_gemm_impl(ctx, F_MUON, x, cols, 1, a2, 1, r, XD, xn, XD, cols, rows, cols, cols, 0, nullptr, bp);
     if (rc != OMX_OK) return rc;
-    hipLaunchKernelGGL((muon_combine_x_kernel<TX>), dim3(mu_grid(len)), dim3(MU_THREADS), 0, ctx->stream, x, xn, len,
-                       s, refuse, ctx->fault, tag);
+    hipLaunchKernelGGL((muon_combine_x_kernel<TX>), over_len, block, 0, ctx->stream, w, x_off, xn_off, len, s,
+                       ctx->fault, tag);
     OMX_LAUNCH_CHECK(ctx, "muon newton-schulz step");
-    TX* t = x;
-    x = xn;
-    xn = t;
+    std::swap(x_off, xn_off);
   }
-  hipLaunchKernelGGL((muon_check_update_kernel<TX>), dim3(mu_grid(len)), dim3(MU_THREADS), 0, ctx->stream, p, x, len,
-                     s, refuse, ctx->fault, tag);
-  hipLaunchKernelGGL((muon_apply_kernel<TX>), dim3(mu_grid(len)), dim3(MU_THREADS), 0, ctx->stream, p, m, buf, x, len,
-                     s, refuse, p_bf16);
+  hipLaunchKernelGGL((muon_check_update_kernel<TX>), over_len, block, 0, ctx->stream, t, w, x_off, len, s, ctx->fault,
+                     tag);
+  hipLaunchKernelGGL((muon_apply_kernel<TX>), over_len, block, 0, ctx->stream, t, w, x_off, len, s);
   OMX_LAUNCH_CHECK(ctx, "muon apply");
   return OMX_OK;
 }
 
-}  // namespace
-
-extern "C" {
-
-uint64_t omx_muon_scratch_bytes(uint64_t rows, uint64_t cols) {
-  if (rows == 0 || cols == 0) return 0;
-  return muon_layout(rows, cols).total;
-}
-
-int32_t omx_muon_ns5_step(omx_ctx* ctx, void* param, const void* grad, void* momentum, uint64_t rows, uint64_t cols,
-                          const omx_muon_config* c, void* param_bf16) {
-  OMX_REQUIRE_CTX(ctx);
-  const char* op = "muon_ns5_step";
-  if (!param || !grad || !momentum || !c) return omx_fail(ctx, OMX_PLACEMENT, "%s: null pointer", op);
+// check_muon (ojas-cpu/src/optim.rs:664-681) and the step's scalars.
+int32_t muon_scalars(omx_ctx* ctx, const char* op, const omx_muon_config* c, uint64_t rows, uint64_t cols,
+                     MuonScalars* out) {
   if (rows == 0 || cols == 0) return omx_fail(ctx, OMX_SHAPE, "%s: empty tensor", op);
   if (rows > 0x7fffffffull || cols > 0x7fffffffull) return omx_fail(ctx, OMX_OUT_OF_RANGE, "%s: axis too large", op);
-  // check_muon, ojas-cpu/src/optim.rs:664-681.
   if (!std::isfinite(c->lr) || !std::isfinite(c->momentum) || !std::isfinite(c->weight_decay))
     return omx_fail(ctx, OMX_NON_FINITE, "%s", op);
   if (c->lr < 0.0) return omx_fail(ctx, OMX_OUT_OF_RANGE, "%s: lr %g is negative", op, c->lr);
@@ -282,18 +303,65 @@ int32_t omx_muon_ns5_step(omx_ctx* ctx, void* param, const void* grad, void* mom
   s.nesterov = c->nesterov != 0;
   s.decays = c->weight_decay != 0.0;
   s.bf16 = c->ns5_bf16 != 0;
-  const MuonLayout L = muon_layout(rows, cols);
-  void* ws = nullptr;
-  int32_t rc = omx_workspace(ctx, L.total, &ws);
+  *out = s;
+  return OMX_OK;
+}
+
+int32_t muon_batch(omx_ctx* ctx, const char* op, void* const* params, const void* const* grads, void* const* momenta,
+                   void* const* params_bf16, uint64_t count, uint64_t rows, uint64_t cols, const omx_muon_config* c) {
+  MuonScalars s;
+  int32_t rc = muon_scalars(ctx, op, c, rows, cols, &s);
   if (rc != OMX_OK) return rc;
-  unsigned long long tag = omx_tag(ctx, F_MUON);
-  if (s.bf16)
-    return run_muon<unsigned short>(ctx, static_cast<float*>(param), static_cast<const float*>(grad),
-                                    static_cast<float*>(momentum), rows, cols, s,
-                                    static_cast<unsigned short*>(param_bf16), static_cast<char*>(ws), L, tag);
-  return run_muon<float>(ctx, static_cast<float*>(param), static_cast<const float*>(grad),
-                         static_cast<float*>(momentum), rows, cols, s, static_cast<unsigned short*>(param_bf16),
-                         static_cast<char*>(ws), L, tag);
+  for (uint64_t i = 0; i < count; ++i)
+    if (!params[i] || !grads[i] || !momenta[i]) return omx_fail(ctx, OMX_PLACEMENT, "%s: null pointer", op);
+  const MuonLayout L = muon_layout(rows, cols);
+  for (uint64_t first = 0; first < count; first += MU_MAX_BATCH) {
+    const unsigned n = static_cast<unsigned>(std::min<uint64_t>(MU_MAX_BATCH, count - first));
+    void* ws = nullptr;
+    rc = omx_workspace(ctx, L.total * n, &ws);
+    if (rc != OMX_OK) return rc;
+    MuonTensors t{};
+    for (unsigned i = 0; i < n; ++i) {
+      t.p[i] = static_cast<float*>(params[first + i]);
+      t.g[i] = static_cast<const float*>(grads[first + i]);
+      t.m[i] = static_cast<float*>(momenta[first + i]);
+      t.p16[i] = params_bf16 ? static_cast<unsigned short*>(params_bf16[first + i]) : nullptr;
+    }
+    const unsigned long long tag = omx_tag(ctx, F_MUON);
+    rc = s.bf16 ? run_muon<unsigned short>(ctx, t, n, rows, cols, s, static_cast<char*>(ws), L, tag)
+                : run_muon<float>(ctx, t, n, rows, cols, s, static_cast<char*>(ws), L, tag);
+    if (rc != OMX_OK) return rc;
+  }
+  return OMX_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+uint64_t omx_muon_scratch_bytes(uint64_t rows, uint64_t cols) {
+  if (rows == 0 || cols == 0) return 0;
+  return muon_layout(rows, cols).total;
+}
+
+int32_t omx_muon_ns5_step(omx_ctx* ctx, void* param, const void* grad, void* momentum, uint64_t rows, uint64_t cols,
+                          const omx_muon_config* c, void* param_bf16) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "muon_ns5_step";
+  if (!param || !grad || !momentum || !c) return omx_fail(ctx, OMX_PLACEMENT, "%s: null pointer", op);
+  void* mirrors[1] = {param_bf16};
+  const void* grads[1] = {grad};
+  return muon_batch(ctx, op, &param, grads, &momentum, param_bf16 ? mirrors : nullptr, 1, rows, cols, c);
+}
+
+int32_t omx_muon_ns5_step_batched(omx_ctx* ctx, void* const* params, const void* const* grads, void* const* momenta,
+                                  void* const* params_bf16, uint64_t count, uint64_t rows, uint64_t cols,
+                                  const omx_muon_config* c) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "muon_ns5_step";
+  if (!params || !grads || !momenta || !c) return omx_fail(ctx, OMX_PLACEMENT, "%s: null pointer", op);
+  if (count == 0) return omx_fail(ctx, OMX_SHAPE, "%s: no tensors", op);
+  return muon_batch(ctx, op, params, grads, momenta, params_bf16, count, rows, cols, c);
 }
 
 }  // extern "C"

@@ -114,9 +114,14 @@ struct OmxGemmEpilogue {
   const void* aux_in;
   void* aux_out;
 };
+// `count` products of one shape whose operands lie `stride_*` ELEMENTS apart (16-byte multiples), one launch.
+struct OmxGemmBatch {
+  uint64_t count, stride_a, stride_b, stride_c;
+};
 int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a_rs, uint64_t a_cs, const void* b,
                       uint64_t b_rs, uint64_t b_cs, int32_t operand_dtype, void* c, int32_t c_dtype, uint64_t ldc,
-                      uint64_t m, uint64_t k, uint64_t n, int32_t accumulate, const OmxGemmEpilogue* epi = nullptr);
+                      uint64_t m, uint64_t k, uint64_t n, int32_t accumulate, const OmxGemmEpilogue* epi = nullptr,
+                      const OmxGemmBatch* batch = nullptr);
 // out[c] = sum over b < blocks of partial[b * dim + c], added in a fixed order.
 // `scratch` (OMX_COLUMN_SUM_GROUPS * dim floats, may be null) lets a tall `partial` be added in two stages.
 constexpr int OMX_COLUMN_SUM_GROUPS = 32;

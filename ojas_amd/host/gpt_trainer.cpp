@@ -452,21 +452,33 @@ int32_t ogpt_step_hybrid(ogpt* t, const omx_muon_config* muon, const omx_adamw_c
     return omx_adamw_step(t->ctx, t->p32 + at, t->g32 + at, t->m1 + at, t->m2 + at, n, t->steps, adamw,
                           mirror ? mirror + at : nullptr);
   };
-  auto matrix = [&](uint64_t slot, uint64_t rows, uint64_t cols) -> int32_t {
-    const uint64_t at = t->slots[slot].offset;  // the AdamW first-moment arena holds Muon's momentum
-    return omx_muon_ns5_step(t->ctx, t->p32 + at, t->g32 + at, t->m1 + at, rows, cols, muon,
-                             mirror ? mirror + at : nullptr);
-  };
   const uint64_t d = t->c.d_model, mlp = t->c.mlp;
+  // Matrices of one shape go through Newton-Schulz together: three batched calls per step.
+  struct Group {
+    uint64_t rows, cols;
+    std::vector<void*> p, m, p16;
+    std::vector<const void*> g;
+  };
+  Group groups[3] = {{d, d, {}, {}, {}, {}}, {mlp, d, {}, {}, {}, {}}, {d, mlp, {}, {}, {}, {}}};
+  auto add = [&](Group& grp, uint64_t slot) {
+    const uint64_t at = t->slots[slot].offset;  // the AdamW first-moment arena holds Muon's momentum
+    grp.p.push_back(t->p32 + at);
+    grp.g.push_back(t->g32 + at);
+    grp.m.push_back(t->m1 + at);
+    grp.p16.push_back(mirror ? mirror + at : nullptr);
+  };
   TRY(adam(0, 1));  // token and position tables
   for (uint64_t l = 0; l < t->c.layers; ++l) {
     TRY(adam(t->li(l, 0), t->li(l, 0)));
-    for (uint64_t w = 1; w <= 4; ++w) TRY(matrix(t->li(l, w), d, d));
+    for (uint64_t w = 1; w <= 4; ++w) add(groups[0], t->li(l, w));
     TRY(adam(t->li(l, 5), t->li(l, 5)));
-    TRY(matrix(t->li(l, 6), mlp, d));
-    TRY(matrix(t->li(l, 7), d, mlp));
+    add(groups[1], t->li(l, 6));
+    add(groups[2], t->li(l, 7));
   }
   TRY(adam(t->nf(), t->nf()));
+  for (Group& grp : groups)
+    TRY(omx_muon_ns5_step_batched(t->ctx, grp.p.data(), grp.g.data(), grp.m.data(), mirror ? grp.p16.data() : nullptr,
+                                  grp.p.size(), grp.rows, grp.cols, muon));
   float l = 0.0f;
   TRY(omx_read_scalar_f32(t->ctx, t->loss, &l));
   t->steps += 1;

@@ -81,3 +81,54 @@ def test_muon_is_all_or_nothing_and_refuses_bad_configs(be):
         be.muon_ns5_step(dp, dg, dm, MuonNs5Config(-0.1, 0.9, 0.0, 1, 0))
     assert e.value.code == OUT_OF_RANGE
     assert be._lib.omx_muon_scratch_bytes(768, 3072) >= 4 * 768 * 3072 * 4
+
+
+@pytest.mark.parametrize("rows,cols,count,bf16", [(64, 48, 5, 0), (48, 64, 3, 1), (130, 70, 2, 0), (256, 256, 7, 1),
+                                                  (768, 768, 48, 1), (768, 3072, 12, 1), (3072, 768, 12, 0),
+                                                  (32, 32, 70, 0)])
+def test_batched_step_matches_the_oracle_per_tensor(be, rows, cols, count, bf16):
+    """`omx_muon_ns5_step_batched` holds each tensor to the oracle at the single op's gates (momentum
+    bit for bit; update 2e-3 of its largest element in f32, 5e-2 with the bf16 iteration). 70 tensors
+    go through in two launches of at most 64."""
+    from ojas_amd.backend import BF16, MuonNs5Config
+
+    print(f"muon batched {count} x {rows}x{cols} bf16={bf16}", flush=True)
+    r = np.random.default_rng(rows * 7 + cols + count)
+    ps = [r.standard_normal((rows, cols)).astype(np.float32) * 0.1 for _ in range(count)]
+    gs = [r.standard_normal((rows, cols)).astype(np.float32) * (0.02 + 0.05 * i / count) for i in range(count)]
+    ms = [r.standard_normal((rows, cols)).astype(np.float32) * 0.01 for _ in range(count)]
+    cfg = MuonNs5Config(0.02, 0.95, 0.1, 1, bf16)
+    dp, dg, dm = [be.upload(x) for x in ps], [be.upload(x) for x in gs], [be.upload(x) for x in ms]
+    mirrors = [be.upload(np.zeros((rows, cols), np.float32), BF16) if i % 2 == 0 else None for i in range(count)]
+    be.muon_ns5_step_batched(dp, dg, dm, cfg, mirrors)
+    be.sync()
+    orc.set_threads(8)
+    decay = np.float32(1.0 - 0.02 * 0.1)
+    check = range(count) if rows * cols <= 1 << 17 else (0, count // 2, count - 1)  # the oracle is slow on big ones
+    for i in check:
+        op, om = orc.muon_ns5_step(ps[i], gs[i], ms[i], lr=0.02, momentum=0.95, weight_decay=0.1, nesterov=True,
+                                   bf16=bool(bf16))
+        assert np.array_equal(be.download(dm[i]), om), i
+        got = be.download(dp[i])
+        upd_gpu, upd_cpu = got - ps[i] * decay, op - ps[i] * decay
+        assert np.max(np.abs(upd_gpu - upd_cpu)) <= (5e-2 if bf16 else 2e-3) * np.max(np.abs(upd_cpu)), i
+        if mirrors[i] is not None:
+            assert np.array_equal(be.download(mirrors[i]), orc.to_bf16(got)), i
+
+
+def test_batched_step_refuses_the_whole_batch(be):
+    from ojas_amd.backend import NON_FINITE, MuonNs5Config, OjasError
+
+    print("muon batched refusal", flush=True)
+    r = np.random.default_rng(1)
+    ps = [r.standard_normal((64, 32)).astype(np.float32) for _ in range(4)]
+    gs = [r.standard_normal((64, 32)).astype(np.float32) for _ in range(4)]
+    gs[2][5, 7] = np.nan
+    dp, dg = [be.upload(x) for x in ps], [be.upload(x) for x in gs]
+    dm = [be.zeros((64, 32)) for _ in range(4)]
+    be.muon_ns5_step_batched(dp, dg, dm, MuonNs5Config.nanolab_default())
+    with pytest.raises(OjasError) as e:
+        be.sync()
+    assert e.value.code == NON_FINITE and "muon_ns5_step" in str(e.value)
+    for i in range(4):
+        assert np.array_equal(be.download(dp[i]), ps[i]) and not be.download(dm[i]).any()

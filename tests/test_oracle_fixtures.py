@@ -355,7 +355,7 @@ def test_gemm_chain_is_the_naive_triple_loop_and_fused_ce_is_the_composed_path()
 
 def test_muon_contracts_singular_values_toward_one():
     # numerical_invariants.rs T5: five Newton-Schulz steps push the singular values of the
-    # normalised update into a band around 1.
+    # normalised update into a band about one.
     r = orc.SplitMix64(31)
     for rows, cols, bf16 in ((48, 64, False), (130, 70, False), (64, 48, True)):
         p = np.zeros((rows, cols), np.float32)
