@@ -506,6 +506,11 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
       splits = static_cast<int>((512 + tiles - 1) / tiles);
       if (splits > ksteps / 8) splits = ksteps / 8;
       if (splits < 1) splits = 1;
+      if (dma_variant >= 0) {  // a power of two, so that a split stays on one XCD (see gemm_dma_kernel)
+        int p2 = 1;
+        while (p2 * 2 <= splits + splits / 4) p2 *= 2;  // 7..9 -> 8, 10..12 -> 8, 13..16 -> 16
+        splits = p2;
+      }
     }
     g.ksteps_per_split = (ksteps + splits - 1) / splits;
     g.splits = (ksteps + g.ksteps_per_split - 1) / g.ksteps_per_split;

@@ -137,10 +137,19 @@ __global__ __launch_bounds__(DT, (NST * (WGM * TM + WGN * TN) * 32 * DBK * 2 <= 
   const unsigned short* __restrict__ A = static_cast<const unsigned short*>(g.a);
   const unsigned short* __restrict__ B = static_cast<const unsigned short*>(g.b);
 
+  // Workgroups go to the 8 XCDs round-robin by blockIdx.x, and each XCD has its own L2. Without
+  // split-K an XCD takes a contiguous eighth of the tiles; with it, blockIdx.x % splits is the
+  // split, so (for the power-of-two split counts the host picks) all tiles of one K chunk run on
+  // the same XCD, side by side, and that chunk of both operands is fetched into one L2 once
+  // instead of into all eight.
   const int total = g.tiles_m * g.tiles_n;
-  const int split = blockIdx.x / total;
-  int id = blockIdx.x - split * total;
-  if (total % 8 == 0) id = (id & 7) * (total >> 3) + (id >> 3);
+  int split = 0, id = blockIdx.x;
+  if (g.splits > 1) {
+    split = blockIdx.x % g.splits;
+    id = blockIdx.x / g.splits;
+  } else if (total % 8 == 0) {
+    id = (id & 7) * (total >> 3) + (id >> 3);
+  }
   const int band = 4;
   const int tiles_per_band = band * g.tiles_n;
   const int band_id = id / tiles_per_band;
