@@ -8,9 +8,12 @@ here. Parameters come in the order of ojas-model/src/names.rs:188-300.
 """
 from __future__ import annotations
 
+import json
 import math
 from dataclasses import dataclass
-from typing import Dict, List, Optional, Sequence
+from decimal import Decimal
+from pathlib import Path
+from typing import Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
 
@@ -35,6 +38,7 @@ class NanolabSpec:
     rms_eps: float = 1e-6
     rope_base: float = 10000.0
     window: Optional[int] = None
+    max_seq: int = 0  # only the spec's JSON needs it
 
     def param_names(self) -> List[str]:
         names = ["tok_emb.weight"]
@@ -268,3 +272,179 @@ class NanolabTrainer:
 
     def download_params(self) -> Dict[str, np.ndarray]:
         return {n: self.be.download(t) for n, t in self.params.items()}
+
+
+# ---- the checkpoint directory (ojas-model/src/checkpoint.rs:1-60) ----
+MODEL_FILE, OPTIM_FILE, STATE_FILE = "model.safetensors", "optim.safetensors", "state.ojck"
+STATE_FORMAT = "ojas-train-v1"
+
+
+def rust_f64(x: float) -> str:
+    """An f64 the way Rust's `{:?}` prints it (shortest digits; exponent form below 1e-4 and from
+    1e16 on, without '+' or padding; otherwise at least one fractional digit)."""
+    if x != x or x in (math.inf, -math.inf):
+        raise ValueError("not a finite number")
+    sign, digits, exp = Decimal(repr(float(x))).as_tuple()
+    digits = "".join(map(str, digits)).lstrip("0") or "0"
+    if digits == "0":
+        return "-0.0" if sign else "0.0"
+    stripped = digits.rstrip("0")
+    exp += len(digits) - len(stripped)
+    digits = stripped
+    sci = len(digits) - 1 + exp  # value = d.ddd x 10^sci
+    if sci < -4 or sci >= 16:
+        body = digits[0] + ("." + digits[1:] if len(digits) > 1 else "") + "e" + str(sci)
+    elif exp >= 0:
+        body = digits + "0" * exp + ".0"
+    elif -exp < len(digits):
+        body = digits[:exp] + "." + digits[exp:]
+    else:
+        body = "0." + "0" * (-exp - len(digits)) + digits
+    return ("-" if sign else "") + body
+
+
+def spec_to_json(spec: NanolabSpec) -> str:
+    """`ModelSpec::to_json` (ojas-model/src/spec.rs:246-268): `ojas-spec-v1`, or v2 with a window."""
+    if spec.max_seq <= 0:
+        raise OjasError(OUT_OF_RANGE, "ModelSpec: max_seq is not set")
+    fmt, window = ("ojas-spec-v1", "") if spec.window is None else ("ojas-spec-v2", f',"window":{spec.window}')
+    return (f'{{"format":"{fmt}","arch":"nanolab-gpt","vocab":{spec.vocab},"n_embd":{spec.n_embd},'
+            f'"n_layer":{spec.n_layer},"n_head":{spec.n_head},"n_kv_head":{spec.n_kv_head},"head_dim":{spec.head_dim},'
+            f'"hidden":{spec.hidden},"max_seq":{spec.max_seq},"rope_base":{rust_f64(spec.rope_base)},'
+            f'"rms_eps":{rust_f64(spec.rms_eps)},"tie_embeddings":true,"qk_norm":true,"gated_attention":true,'
+            f'"value_residual":true{window}}}')
+
+
+def spec_from_json(text: str) -> NanolabSpec:
+    """`ModelSpec::from_json` (spec.rs:280-360): the keys of v1 / v2, the four flags true."""
+    d = json.loads(text)
+    want = {"ojas-spec-v1": False, "ojas-spec-v2": True}
+    if d.get("format") not in want or d.get("arch") != "nanolab-gpt":
+        raise OjasError(OUT_OF_RANGE, f"ModelSpec: format {d.get('format')!r} / arch {d.get('arch')!r}")
+    if ("window" in d) != want[d["format"]]:
+        raise OjasError(OUT_OF_RANGE, "ModelSpec: window belongs to ojas-spec-v2 only")
+    for flag in ("tie_embeddings", "qk_norm", "gated_attention", "value_residual"):
+        if d.get(flag) is not True:
+            raise OjasError(OUT_OF_RANGE, f"ModelSpec: {flag} must be true")
+    return NanolabSpec(n_layer=d["n_layer"], n_embd=d["n_embd"], n_head=d["n_head"], n_kv_head=d["n_kv_head"],
+                       head_dim=d["head_dim"], hidden=d["hidden"], vocab=d["vocab"], rms_eps=float(d["rms_eps"]),
+                       rope_base=float(d["rope_base"]), window=d.get("window"), max_seq=d["max_seq"])
+
+
+@dataclass
+class TrainConfig:
+    """`ojas_model::TrainConfig` (ojas-model/src/trainer.rs): the fields its JSON carries."""
+    seq_len: int
+    batch: int
+    accum: int = 1
+    adam_lr: float = 6e-4
+    matrix_lr: float = 0.025
+    grad_clip: float = 1.0
+    data_seed: int = 0
+    schedule: str = "cosine"
+    decay_frac: float = 0.0
+    total_steps: int = 0
+    warmup_steps: int = 0
+    chunk_rows: int = 1024
+    chunk_cols: int = 8192
+    ignore_index: Optional[int] = None
+    on_nonfinite: str = "abort"
+    muon_ns5_bf16: bool = False
+
+    def to_json(self) -> str:
+        """`TrainConfig::to_json` (trainer.rs:179-221): sorted keys, optional ones absent at their defaults."""
+        ns5 = '"muon_ns5":"bf16",' if self.muon_ns5_bf16 else ""
+        return (f'{{"accum":{self.accum},"adam_lr":{rust_f64(self.adam_lr)},"batch":{self.batch},'
+                f'"chunk_cols":{self.chunk_cols},"chunk_rows":{self.chunk_rows},"data_seed":{self.data_seed},'
+                f'"decay_frac":{rust_f64(self.decay_frac)},"grad_clip":{rust_f64(self.grad_clip)},'
+                f'"ignore":{"true" if self.ignore_index is not None else "false"},"ignore_index":{self.ignore_index or 0},'
+                f'"matrix_lr":{rust_f64(self.matrix_lr)},{ns5}"on_nonfinite":{json.dumps(self.on_nonfinite)},'
+                f'"schedule":{json.dumps(self.schedule)},"seq_len":{self.seq_len},"total_steps":{self.total_steps},'
+                f'"warmup_steps":{self.warmup_steps}}}')
+
+
+def save_checkpoint(trainer: NanolabTrainer, directory, cfg: TrainConfig, cursor: Tuple[int, int] = (0, 0),
+                    run: str = "run", tokenizer_hash: bytes = bytes(32), git_sha: bytes = bytes(20)):
+    """`Trainer::save` (ojas-model/src/checkpoint.rs:540-640): `model.safetensors` (F32 weights, table
+    order, metadata ojas.spec / ojas.step / ojas.run), `optim.safetensors` (`muon.<name>`,
+    `adam_m.<name>`, `adam_v.<name>` of every trained parameter, table order) and `state.ojck`
+    (checkpoint v1 with empty tensor sections: step, cursor, the sampler's rng_state, and the config
+    object {"format","run","spec","train"}). One tensor is read back at a time."""
+    from .data import rng_state_encode
+    from .io import CheckpointV1, write_checkpoint, write_safetensors
+
+    directory = Path(directory)
+    directory.mkdir(parents=True, exist_ok=True)
+    be, step = trainer.be, str(trainer.step)
+    spec_json = spec_to_json(trainer.spec)
+    write_safetensors(directory / MODEL_FILE, {n: be.download(trainer.params[n]) for n in trainer.names},
+                      {"ojas.spec": spec_json, "ojas.step": step, "ojas.run": run})
+    moments = {}
+    for n in trainer.trainable:
+        if n in trainer.muon:
+            moments[f"muon.{n}"] = be.download(trainer.state[n][0])
+        else:
+            moments[f"adam_m.{n}"] = be.download(trainer.state[n][0])
+            moments[f"adam_v.{n}"] = be.download(trainer.state[n][1])
+    write_safetensors(directory / OPTIM_FILE, moments, {"ojas.step": step, "ojas.run": run})
+    config = (f'{{"format":{json.dumps(STATE_FORMAT)},"run":{json.dumps(run)},"spec":{spec_json},'
+              f'"train":{cfg.to_json()}}}')
+    write_checkpoint(directory / STATE_FILE,
+                     CheckpointV1(config=config.encode(), tokenizer_hash=tokenizer_hash, git_sha=git_sha,
+                                  step=trainer.step, cursor=cursor, rng_state=rng_state_encode(cfg.data_seed)))
+
+
+def resume_checkpoint(be: MiBackend, directory, cfg: TrainConfig, tokenizer_hash: bytes = bytes(32)):
+    """`Trainer::resume_from` (ojas-model/src/checkpoint.rs:700-900): refuses unless step and run agree
+    across the three files, the saved train config and tokenizer hash equal the caller's, the
+    rng_state is the sampler's v1 layout with the caller's data_seed, and names, dtypes and shapes
+    are exactly the expected ones. Returns (trainer, cursor, run)."""
+    from .data import rng_state_decode
+    from .io import IoError, SafeTensors, read_checkpoint
+
+    directory = Path(directory)
+    state = read_checkpoint(directory / STATE_FILE)
+    if any(state.sections()):
+        raise IoError("state.ojck: tensor sections are not empty")
+    conf = json.loads(state.config)
+    if conf.get("format") != STATE_FORMAT:
+        raise IoError(f"state.ojck: format {conf.get('format')!r}, expected {STATE_FORMAT!r}")
+    if conf.get("train") != json.loads(cfg.to_json()):
+        raise IoError("state.ojck: the saved train config is not the caller's")
+    if state.tokenizer_hash != tokenizer_hash:
+        raise IoError("state.ojck: tokenizer hash differs from the caller's")
+    if rng_state_decode(state.rng_state) != cfg.data_seed:
+        raise IoError("state.ojck: rng_state seed differs from the caller's data_seed")
+    model, optim = SafeTensors(directory / MODEL_FILE), SafeTensors(directory / OPTIM_FILE)
+    run = conf.get("run")
+    for what, meta in ((MODEL_FILE, model.metadata()), (OPTIM_FILE, optim.metadata())):
+        if meta.get("ojas.step") != str(state.step) or meta.get("ojas.run") != run:
+            raise IoError(f"{what}: step / run disagree with state.ojck")
+    spec = spec_from_json(model.metadata().get("ojas.spec", ""))
+    if json.loads(spec_to_json(spec)) != conf.get("spec"):
+        raise IoError("model.safetensors: ojas.spec disagrees with state.ojck")
+    shapes = spec.param_shapes()
+    if model.names() != sorted(spec.param_names(), key=str.encode):
+        raise IoError("model.safetensors: tensor names are not the model's")
+    host = {}
+    for n in spec.param_names():
+        info = model.info(n)
+        if info.dtype != "F32" or info.shape != tuple(shapes[n]):
+            raise IoError(f"model.safetensors: {n} is {info.dtype} {info.shape}, expected F32 {tuple(shapes[n])}")
+        host[n] = model.read(n)
+    trainer = NanolabTrainer(be, spec, host, adam_lr=cfg.adam_lr, matrix_lr=cfg.matrix_lr, grad_clip=cfg.grad_clip,
+                             ns5_bf16=cfg.muon_ns5_bf16)
+    expected = []
+    for n in trainer.trainable:
+        expected += [f"muon.{n}"] if n in trainer.muon else [f"adam_m.{n}", f"adam_v.{n}"]
+    if optim.names() != sorted(expected, key=str.encode):
+        raise IoError("optim.safetensors: tensor names are not the trained parameters' moments")
+    for n in trainer.trainable:
+        keys = [f"muon.{n}"] if n in trainer.muon else [f"adam_m.{n}", f"adam_v.{n}"]
+        for slot, key in enumerate(keys):
+            info = optim.info(key)
+            if info.dtype != "F32" or info.shape != tuple(shapes[n]):
+                raise IoError(f"optim.safetensors: {key} is {info.dtype} {info.shape}")
+            trainer.state[n][slot] = be.upload(optim.read(key))
+    trainer.step = state.step
+    return trainer, state.cursor, run

@@ -151,3 +151,47 @@ def test_five_trainer_steps_follow_the_torch_trace(be):
         norms.append(report.grad_norm)
     worst = tf.check_trace(trace, losses, norms, trainer.download_params(), {"blocks.0.mixer.vr_lambda"})
     print(f"worst parameter distance after step {trace.steps}: {worst:.2e}", flush=True)
+
+
+def test_save_then_resume_continues_bit_for_bit(be, tmp_path):
+    """`Trainer::save` / `resume_from` over the checkpoint directory (ojas-model/src/checkpoint.rs): three
+    steps, a save, a resume into a fresh trainer and two more steps equal five uninterrupted steps bit for
+    bit, as `g9_forty_steps_equal_twenty_saved_dropped_resumed_and_twenty_more`
+    (ojas-model/tests/checkpoint.rs) demands of the CPU. A resume with another seed, config or tokenizer
+    hash is refused."""
+    import trace_fixture as tf
+    from ojas_amd.io import IoError, SafeTensors, read_checkpoint
+    from ojas_amd.nanolab import NanolabTrainer, TrainConfig, resume_checkpoint, save_checkpoint, spec_from_json
+
+    print("nanolab save / resume", flush=True)
+    trace = tf.Trace()
+    init, _ = load("init")
+    spec = spec_from_json(SafeTensors(TINY / "init.safetensors").metadata()["ojas.spec"])
+    cfg = TrainConfig(seq_len=trace.seq, batch=trace.batch, accum=trace.accum, data_seed=1337, total_steps=40,
+                      warmup_steps=4)
+    batches = lambda step: [trace.micro(step, m) for m in range(trace.accum)]
+    whole = NanolabTrainer(be, spec, init)
+    for step in range(5):
+        whole.run(batches(step), trace.lr_mult[step])
+    first = NanolabTrainer(be, spec, init)
+    for step in range(3):
+        first.run(batches(step), trace.lr_mult[step])
+    ckpt = tmp_path / "ckpt"
+    save_checkpoint(first, ckpt, cfg, cursor=(0, 12), run="r1", tokenizer_hash=bytes(range(32)))
+    assert sorted(p.name for p in ckpt.iterdir()) == ["model.safetensors", "optim.safetensors", "state.ojck"]
+    state = read_checkpoint(ckpt / "state.ojck")
+    assert (state.step, state.cursor, len(state.rng_state)) == (3, (0, 12), 16) and not any(state.sections())
+    assert SafeTensors(ckpt / "model.safetensors").metadata()["ojas.step"] == "3"
+    del first
+    resumed, cursor, run = resume_checkpoint(be, ckpt, cfg, tokenizer_hash=bytes(range(32)))
+    assert (resumed.step, cursor, run) == (3, (0, 12), "r1")
+    for step in range(3, 5):
+        resumed.run(batches(step), trace.lr_mult[step])
+    a, b = whole.download_params(), resumed.download_params()
+    for name in spec.param_names():
+        assert np.array_equal(a[name].view(np.uint32), b[name].view(np.uint32)), name
+    for other, what in ((dict(data_seed=7), "train config"), (dict(accum=4), "train config")):
+        with pytest.raises(IoError, match=what):
+            resume_checkpoint(be, ckpt, TrainConfig(**{**cfg.__dict__, **other}), tokenizer_hash=bytes(range(32)))
+    with pytest.raises(IoError, match="tokenizer hash"):
+        resume_checkpoint(be, ckpt, cfg)
