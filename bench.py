@@ -30,10 +30,10 @@ sys.path.insert(0, str(ROOT))
 BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, vendor figure
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor figure
 # HBM bytes per GEMM op (MFMA kernel + split-K reduce) on the gpt124m workload, averaged over the
-# step's GEMM ops (156 when this was measured): rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by what the same
+# step's 150 GEMM ops: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by what the same
 # counters read for the AdamW pass, whose traffic is known (profiles/gemm_hbm_traffic_gpt124m_bf16.txt).
-# The algorithmic figure (every operand read once, every output written once) is 1.569e8.
-GEMM_HBM_BYTES_PER_LAUNCH_GPT124M = 3.69e8
+# The algorithmic figure (every operand read once, every output written once) is 1.550e8.
+GEMM_HBM_BYTES_PER_LAUNCH_GPT124M = 3.15e8
 
 
 def cpu_baseline(cfg, threads: int):
