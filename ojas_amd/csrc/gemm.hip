@@ -488,6 +488,7 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
     else if (mode == 2) dma_variant = 0;
     else if (mode == 3) dma_variant = 3;
     else if (mode == 4) dma_variant = 1;
+    else if (mode == 5) dma_variant = 5;
   }
   int BM = 128, BN = 128;
   if (dma_variant >= 0) omx_gemm_dma_tile(dma_variant, &BM, &BN);
@@ -569,7 +570,7 @@ extern "C" {
 int32_t omx_set_option(omx_ctx* ctx, const char* name, int64_t value) {
   OMX_REQUIRE_CTX(ctx);
   if (name && strcmp(name, "gemm_dma") == 0) {
-    if (value < 0 || value > 4) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: gemm_dma takes 0..4");
+    if (value < 0 || value > 5) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: gemm_dma takes 0..5");
     ctx->gemm_dma_mode = static_cast<int>(value);
     return OMX_OK;
   }

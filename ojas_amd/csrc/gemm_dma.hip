@@ -14,6 +14,11 @@
 //   * Variants 1 (256 x 128, three stages) and 0 (256 x 256, two stages): K steps of 64 columns,
 //     whole cache lines, one workgroup per compute unit. Load latency (about 0.6 us) is then
 //     exposed: with one or two stages in flight the loads alone take as long as the products.
+//   * Variant 5: 256 x 256 with four waves of 128 x 128 (256 accumulator registers per lane, held
+//     in AGPRs), 32-column steps, four stages. Half the LDS reads and two thirds of the loads per
+//     FLOP of the default, but one wave per SIMD: with nothing else to switch to, the products
+//     alone (no loads) run at 0.8x the default's rate, and the whole kernel is slower on every
+//     shape measured. Kept for measurements.
 //   * operand tiles go from global memory straight into LDS: no staging
 //     registers and no LDS store instructions. A wave-wide load writes 64
 //     consecutive 16-byte slots, so the LDS tile is unpadded and bank conflicts
@@ -39,14 +44,13 @@ typedef short short4v __attribute__((ext_vector_type(4)));
 
 namespace {
 
-constexpr int DT = 512;  // threads
 
 // Per-lane state of one operand's loads: the global address of each of this wave's loads for the
 // current K step (advanced by one step after every issue) and nothing else, so a step costs one
 // 64-bit add per load. ROWS x BK bf16 per step, one wave instruction per KiB.
-template <bool KM, int ROWS, int BK>
+template <bool KM, int ROWS, int BK, int NW>  // NW: waves per workgroup
 struct TileLoads {
-  static constexpr int N = ROWS * BK * 2 / 1024 / 8;  // loads per wave per step
+  static constexpr int N = ROWS * BK * 2 / 1024 / NW;  // loads per wave per step
   const unsigned short* src[N];
   long step;  // elements between consecutive K steps
 
@@ -54,7 +58,7 @@ struct TileLoads {
                                        int wave, int lane) {
 #pragma unroll
     for (int i = 0; i < N; ++i) {
-      const int q = wave + 8 * i;
+      const int q = wave + NW * i;
       if constexpr (!KM) {
         // [row][BK / 8 chunks of 16 bytes], swizzled as frag_offset reads them.
         constexpr int LPR = BK / 8;  // lanes (chunks) per row
@@ -83,7 +87,7 @@ struct TileLoads {
       // stage that is NOT being read, and would otherwise make every LDS read wait for it
       // (vmcnt(0) right after the issue), which serialises the loads with the products.
       asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src[i]),
-                   "s"(tile + (wave + 8 * i) * 1024)
+                   "s"(tile + (wave + NW * i) * 1024)
                    : "memory");
       src[i] += step;
     }
@@ -124,15 +128,21 @@ __device__ __forceinline__ u32x4 frag_at(const char* p) {
 // s_waitcnt operand that waits for vmcnt <= n only (vmcnt is bits 3:0 and 15:14).
 constexpr int vmcnt_only(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
 
+// Waves per SIMD the kernel is compiled for: two workgroups per compute unit when its LDS allows,
+// else one.
+constexpr int dma_waves_per_simd(int waves, int lds_bytes) { return (lds_bytes <= 80 * 1024 ? 2 : 1) * waves / 4; }
+
 template <bool A_KM, bool B_KM, int WGM, int WGN, int TM, int TN, int DBK, int NST>
-__global__ __launch_bounds__(DT, (NST * (WGM * TM + WGN * TN) * 32 * DBK * 2 <= 80 * 1024 ? 4 : 2)) void gemm_dma_kernel(
-    GemmArgs g) {
+__global__ __launch_bounds__(WGM* WGN * 64, dma_waves_per_simd(WGM* WGN, NST*(WGM* TM + WGN * TN) * 32 * DBK * 2)) void
+gemm_dma_kernel(GemmArgs g) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
   constexpr int A_BYTES = BM * DBK * 2, B_BYTES = BN * DBK * 2, STAGE = A_BYTES + B_BYTES;
-  constexpr int LPS = STAGE / 1024 / 8;  // loads per wave per step
-  constexpr int KK = DBK / 16;           // MFMA K slabs per step
-  static_assert(WGM * WGN == 8, "eight waves");
+  constexpr int NW = WGM * WGN;           // waves per workgroup
+  constexpr int LPS = STAGE / 1024 / NW;  // loads per wave per step
+  constexpr int KK = DBK / 16;            // MFMA K slabs per step
+  static_assert(NW == 4 || NW == 8, "four or eight waves");
+  static_assert(STAGE % (1024 * NW) == 0, "whole load instructions per wave");
   gemm_select_batch(g);
   const unsigned short* __restrict__ A = static_cast<const unsigned short*>(g.a);
   const unsigned short* __restrict__ B = static_cast<const unsigned short*>(g.b);
@@ -180,8 +190,8 @@ __global__ __launch_bounds__(DT, (NST * (WGM * TM + WGN * TN) * 32 * DBK * 2 <= 
   // Everything a K step needs is computed here, once per tile: the loads' global addresses and
   // the fragments' LDS offsets. Inside the loop the stage is a compile-time constant (the loop
   // body is unrolled over the stages), so a step is loads, LDS reads and MFMAs and little else.
-  TileLoads<A_KM, BM, DBK> la;
-  TileLoads<B_KM, BN, DBK> lb;
+  TileLoads<A_KM, BM, DBK, NW> la;
+  TileLoads<B_KM, BN, DBK, NW> lb;
   la.init(A, g.lda, m0, g.M, ks_begin * DBK, wave, lane);
   lb.init(B, g.ldb, n0, g.N, ks_begin * DBK, wave, lane);
   const unsigned lds0 = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(reinterpret_cast<uintptr_t>(smem)));
@@ -220,49 +230,65 @@ __global__ __launch_bounds__(DT, (NST * (WGM * TM + WGN * TN) * 32 * DBK * 2 <= 
     for (int t = 0; t < TN; ++t) b[t] = frag_at<B_KM, BN>(stage + b_off[t][kk]);
   };
   read_frags(smem, 0, af, bf);
-  for (int ks = ks_begin; ks < ks_end;) {
+  // One K step: the loads of step ks + NST - 1, then the slabs of stage `stage` (fragments one slab
+  // ahead), the wait + barrier before the last slab's products, and the first slab of `next`.
+  auto k_step = [&](int ks, unsigned fill_stage, const char* stage, const char* next) {
+    if (ks + NST - 1 < ks_end) {
+      la.issue(lds0 + fill_stage * STAGE, wave);
+      lb.issue(lds0 + fill_stage * STAGE + A_BYTES, wave);
+    }
 #pragma unroll
-    for (int st = 0; st < NST; ++st) {  // step ks lives in stage st
-      if (ks + NST - 1 < ks_end) {
-        const int fill = (st + NST - 1) % NST;  // the stage the previous step has released
-        la.issue(lds0 + fill * STAGE, wave);
-        lb.issue(lds0 + fill * STAGE + A_BYTES, wave);
+    for (int kk = 0; kk < KK; ++kk) {
+      u32x4 an[TM], bn[TN];
+#pragma unroll
+      for (int t = 0; t < TM; ++t) an[t] = af[t];
+#pragma unroll
+      for (int t = 0; t < TN; ++t) bn[t] = bf[t];
+      if (kk + 1 < KK) {
+        read_frags(stage, kk + 1, an, bn);
+      } else {
+        // Step ks + 1 must have landed (this wave's share, then everyone's); later steps may
+        // still be in flight. Every wave has its last fragments of this stage in registers by
+        // now, so the barrier also releases the stage for the loads of step ks + NST.
+        wait_groups(min(NST - 2, ks_end - ks - 2));
+        __syncthreads();
+        if (ks + 1 < ks_end) read_frags(next, 0, an, bn);
       }
-      const char* stage = smem + st * STAGE;
+      // Keeps the reads above the products: the scheduler would otherwise sink them to their
+      // first use to save registers, which puts the LDS latency back in front of every slab.
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int kk = 0; kk < KK; ++kk) {
-        u32x4 an[TM], bn[TN];
+      for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
-        for (int t = 0; t < TM; ++t) an[t] = af[t];
+        for (int tn = 0; tn < TN; ++tn)
+          acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[tm]),
+                                                                __builtin_bit_cast(bf16x8, bf[tn]), acc[tm][tn], 0, 0,
+                                                                0);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int t = 0; t < TN; ++t) bn[t] = bf[t];
-        if (kk + 1 < KK) {
-          read_frags(stage, kk + 1, an, bn);
-        } else {
-          // Step ks + 1 must have landed (this wave's share, then everyone's); later steps may
-          // still be in flight. Every wave has its last fragments of stage st in registers by
-          // now, so the barrier also releases stage st for the loads of step ks + NST.
-          wait_groups(min(NST - 2, ks_end - ks - 2));
-          __syncthreads();
-          if (ks + 1 < ks_end) read_frags(smem + ((st + 1) % NST) * STAGE, 0, an, bn);
-        }
-        // Keeps the reads above the products: the scheduler would otherwise sink them to their
-        // first use to save registers, which puts the LDS latency back in front of every slab.
-        __builtin_amdgcn_sched_barrier(0);
+      for (int t = 0; t < TM; ++t) af[t] = an[t];
 #pragma unroll
-        for (int tm = 0; tm < TM; ++tm)
+      for (int t = 0; t < TN; ++t) bf[t] = bn[t];
+    }
+  };
+  if constexpr (NW == 8) {
+    // Unrolled over the stages, so every LDS address is the precomputed offset plus a constant.
+    for (int ks = ks_begin; ks < ks_end;) {
 #pragma unroll
-          for (int tn = 0; tn < TN; ++tn)
-            acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[tm]),
-                                                                  __builtin_bit_cast(bf16x8, bf[tn]), acc[tm][tn], 0,
-                                                                  0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int t = 0; t < TM; ++t) af[t] = an[t];
-#pragma unroll
-        for (int t = 0; t < TN; ++t) bf[t] = bn[t];
+      for (int st = 0; st < NST; ++st) {  // step ks lives in stage st
+        k_step(ks, (st + NST - 1) % NST, smem + st * STAGE, smem + ((st + 1) % NST) * STAGE);
+        if (++ks >= ks_end) break;
       }
-      if (++ks >= ks_end) break;
+    }
+  } else {
+    // With 256 accumulator registers per lane the unrolled form runs out of registers; the stage is
+    // a loop variable here, at the price of one address add per fragment read.
+    int st = 0;
+#pragma unroll 1
+    for (int ks = ks_begin; ks < ks_end; ++ks) {
+      const int nx = st + 1 == NST ? 0 : st + 1;
+      k_step(ks, st == 0 ? NST - 1 : st - 1, smem + st * STAGE, smem + nx * STAGE);
+      st = nx;
     }
   }
   __syncthreads();  // the staging below reuses the stages
@@ -270,7 +296,7 @@ __global__ __launch_bounds__(DT, (NST * (WGM * TM + WGN * TN) * 32 * DBK * 2 <= 
   // Epilogue: each wave stages 32 rows of its tile at a time through its own
   // LDS region and writes whole 4-column pieces.
   constexpr int CPW = TN * 32 + 4;
-  static_assert(8 * 32 * CPW * 4 <= NST * STAGE, "staging fits");
+  static_assert(NW * 32 * CPW * 4 <= NST * STAGE, "staging fits");
   float* cs = reinterpret_cast<float*>(smem) + wave * (32 * CPW);
   bool bad = false;
 #pragma unroll
@@ -320,7 +346,7 @@ int32_t launch_dma(omx_ctx* ctx, const GemmArgs& g) {
                                      smem));
     granted = true;
   }
-  hipLaunchKernelGGL(kernel, dim3(g.tiles_m * g.tiles_n * g.splits, g.batches), dim3(DT), smem, ctx->stream, g);
+  hipLaunchKernelGGL(kernel, dim3(g.tiles_m * g.tiles_n * g.splits, g.batches), dim3(WGM * WGN * 64), smem, ctx->stream, g);
   OMX_LAUNCH_CHECK(ctx, "gemm_dma_kernel");
   return OMX_OK;
 }
@@ -344,11 +370,12 @@ bool omx_gemm_dma_eligible(const GemmArgs& g, bool a_km, bool b_km) {
 
 void omx_gemm_dma_tile(int variant, int* bm, int* bn) {
   *bm = 256;
-  *bn = variant == 0 ? 256 : 128;
+  *bn = (variant == 0 || variant == 5) ? 256 : 128;
 }
 
 int32_t omx_gemm_dma_launch(omx_ctx* ctx, const GemmArgs& g, bool a_km, bool b_km, int variant) {
   if (variant == 0) return launch_layout<2, 4, 4, 2, 64, 2>(ctx, g, a_km, b_km);
   if (variant == 3) return launch_layout<4, 2, 2, 2, 32, 3>(ctx, g, a_km, b_km);
+  if (variant == 5) return launch_layout<2, 2, 4, 4, 32, 4>(ctx, g, a_km, b_km);
   return launch_layout<4, 2, 2, 2, 64, 3>(ctx, g, a_km, b_km);
 }
