@@ -303,6 +303,8 @@ class MiBackend:
         """grad_input of `linear_backward(w, gy)` times gelu'(u) in one kernel (bf16)."""
         nout, nin = w.shape
         rows = gy.numel // nout
+        if gy.shape[-1] != nout or u.numel != rows * nin or not (w.dtype == gy.dtype == u.dtype == BF16):
+            raise BackendError(OMX_SHAPE, f"linear_backward_input_gelu: w {w.shape}, gy {gy.shape}, u {u.shape}")
         gu = self.empty(u.shape, BF16)
         self._check(self._lib.omx_linear_backward_input_gelu(
             self._ctx, self._p(w), self._p(gy), C.c_int32(gy.dtype), self._p(u), self._p(gu), C.c_uint64(rows),
