@@ -482,13 +482,23 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
       // products. The 64-column forms fetch whole cache lines but run alone on their compute
       // unit; they win only on long reductions with large outputs (8192^3: 1.09 against
       // 0.95 PFLOP/s for 256 x 256) and lose on every GPT shape.
-      if (static_cast<long>(g.M) * g.N * g.batches <= (1l << 20)) dma_variant = -1;
+      // 128 x 128 tiles with four waves (48 KiB, three workgroups per compute unit) give the
+      // layers' input-gradient products with up to 1024 output columns three tiles per compute
+      // unit instead of one and a half (K = 3072: 94 against 104 us), and are 3 to 20 % ahead on
+      // the layers' weight-gradient products (both operands K-major, K = tokens), d x d included.
+      // The head's products (K or M = vocabulary) are faster on the larger tile.
+      const bool unbatched = g.batches == 1;
+      const long outputs = static_cast<long>(g.M) * g.N;
+      if (unbatched && a_km && b_km && g.K >= 4096 && outputs <= (1l << 22)) dma_variant = 6;
+      else if (outputs * g.batches <= (1l << 20)) dma_variant = -1;
+      else if (unbatched && !a_km && b_km && g.N <= 1024 && g.K <= 4096) dma_variant = 6;
       else dma_variant = 3;
     }
     else if (mode == 2) dma_variant = 0;
     else if (mode == 3) dma_variant = 3;
     else if (mode == 4) dma_variant = 1;
     else if (mode == 5) dma_variant = 5;
+    else if (mode == 6) dma_variant = 6;
   }
   int BM = 128, BN = 128;
   if (dma_variant >= 0) omx_gemm_dma_tile(dma_variant, &BM, &BN);
@@ -570,7 +580,7 @@ extern "C" {
 int32_t omx_set_option(omx_ctx* ctx, const char* name, int64_t value) {
   OMX_REQUIRE_CTX(ctx);
   if (name && strcmp(name, "gemm_dma") == 0) {
-    if (value < 0 || value > 5) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: gemm_dma takes 0..5");
+    if (value < 0 || value > 6) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: gemm_dma takes 0..6");
     ctx->gemm_dma_mode = static_cast<int>(value);
     return OMX_OK;
   }

@@ -128,9 +128,12 @@ __device__ __forceinline__ u32x4 frag_at(const char* p) {
 // s_waitcnt operand that waits for vmcnt <= n only (vmcnt is bits 3:0 and 15:14).
 constexpr int vmcnt_only(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
 
-// Waves per SIMD the kernel is compiled for: two workgroups per compute unit when its LDS allows,
-// else one.
-constexpr int dma_waves_per_simd(int waves, int lds_bytes) { return (lds_bytes <= 80 * 1024 ? 2 : 1) * waves / 4; }
+// Waves per SIMD the kernel is compiled for: as many workgroups per compute unit as its LDS (160
+// KiB) allows, up to four waves per SIMD.
+constexpr int dma_waves_per_simd(int waves, int lds_bytes) {
+  const int by_lds = 160 * 1024 / lds_bytes, by_waves = 16 / waves;
+  return (by_lds < by_waves ? by_lds : by_waves) * waves / 4;
+}
 
 template <bool A_KM, bool B_KM, int WGM, int WGN, int TM, int TN, int DBK, int NST>
 __global__ __launch_bounds__(WGM* WGN * 64, dma_waves_per_simd(WGM* WGN, NST*(WGM* TM + WGN * TN) * 32 * DBK * 2)) void
@@ -271,7 +274,7 @@ gemm_dma_kernel(GemmArgs g) {
       for (int t = 0; t < TN; ++t) bf[t] = bn[t];
     }
   };
-  if constexpr (NW == 8) {
+  if constexpr (TM * TN <= 4) {
     // Unrolled over the stages, so every LDS address is the precomputed offset plus a constant.
     for (int ks = ks_begin; ks < ks_end;) {
 #pragma unroll
@@ -369,7 +372,7 @@ bool omx_gemm_dma_eligible(const GemmArgs& g, bool a_km, bool b_km) {
 }
 
 void omx_gemm_dma_tile(int variant, int* bm, int* bn) {
-  *bm = 256;
+  *bm = variant == 6 ? 128 : 256;
   *bn = (variant == 0 || variant == 5) ? 256 : 128;
 }
 
@@ -377,5 +380,6 @@ int32_t omx_gemm_dma_launch(omx_ctx* ctx, const GemmArgs& g, bool a_km, bool b_k
   if (variant == 0) return launch_layout<2, 4, 4, 2, 64, 2>(ctx, g, a_km, b_km);
   if (variant == 3) return launch_layout<4, 2, 2, 2, 32, 3>(ctx, g, a_km, b_km);
   if (variant == 5) return launch_layout<2, 2, 4, 4, 32, 4>(ctx, g, a_km, b_km);
+  if (variant == 6) return launch_layout<2, 2, 2, 2, 32, 3>(ctx, g, a_km, b_km);
   return launch_layout<4, 2, 2, 2, 64, 3>(ctx, g, a_km, b_km);
 }
