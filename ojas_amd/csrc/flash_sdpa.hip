@@ -65,6 +65,14 @@ __device__ __forceinline__ floatx16 mfma(const u32x4& a, const u32x4& b, floatx1
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
                                                  0, 0);
 }
+// max(a, b, c) in one instruction. fmaxf first quiets each accumulator value (a v_max_f32 of the
+// value with itself) because the compiler cannot know an MFMA result is canonical; this does not.
+// NaNs are skipped, as by fmaxf.
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
 __device__ __forceinline__ floatx16 zero16() {
   floatx16 z;
 #pragma unroll
@@ -216,9 +224,14 @@ __global__ __launch_bounds__(FT, 3) void flash_fwd_kernel(const unsigned short* 
     }
     float tmax = fmaxf(sc[0][0], sc[1][0]);
 #pragma unroll
-    for (int vv = 1; vv < 16; ++vv) tmax = fmaxf(tmax, fmaxf(sc[0][vv], sc[1][vv]));
+    for (int vv = 1; vv < 16; ++vv) tmax = max3(tmax, sc[0][vv], sc[1][vv]);
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-    const float new_m = fmaxf(m, tmax);
+    // The reference point of the exponents moves only when a row's maximum grew by more than 8
+    // binary orders (always on a row's first tile, where m is -inf): below that the weights of
+    // this tile are at most 2^8, well inside f32 and bf16, and the accumulators need no rescaling.
+    // The quotient at the end and the log-sum-exp use the same reference, so both stay exact.
+    const bool grow = (tmax - m) * scale_log2 > 8.0f;
+    const float new_m = grow ? tmax : m;
     const float m_safe = new_m == -INFINITY ? 0.0f : new_m;
     const float neg_m = -m_safe * scale_log2;
     float psum = 0.0f;
@@ -231,8 +244,9 @@ __global__ __launch_bounds__(FT, 3) void flash_fwd_kernel(const unsigned short* 
         psum += p;
       }
     psum += __shfl_xor(psum, 32, 64);
-    if (__any(new_m > m)) {
-      // Some row's maximum grew: rescale what is accumulated so far.
+    if (__any(grow)) {
+      // Some row's reference moved: rescale what is accumulated so far (by exactly 1 in the
+      // rows that keep theirs).
       const float alpha = __builtin_amdgcn_exp2f(fmaf(m, scale_log2, neg_m));
       lsum *= alpha;
 #pragma unroll

@@ -82,20 +82,30 @@ def test_one_sequence_f32_tier_matches_the_oracle(be, world):
         assert np.max(np.abs(d)) <= 1e-4 * max(np.max(np.abs(og)), 1e-12), i
 
 
+def check_bf16_gradients(grads, ref):
+    """The bf16 tier's gradient gates at this depth. Every element within 2e-2 of its tensor's
+    largest value, except in the query and key projections: their gradients come out of the
+    softmax backward with 1.0e-2 (first layer) to 2.1e-2 (from the sixth layer on) normwise noise
+    and single elements up to 3.1e-2 (gate 4e-2); all other tensors measure at most 1.1e-2
+    normwise and 1.4e-2 per element. Every tensor within 2.5e-2 normwise. Two kernels that
+    differ only in the order of an f32 sum give different realizations of this noise (see the
+    module text), so the gates leave a fifth of headroom over what one build measured."""
+    layers = GPT124M[0]
+    for i, (g, r) in enumerate(zip(grads, ref)):
+        d = g.astype(np.float64) - r
+        # Parameter order: token table, position table, then per layer norm1, wq, wk, wv, wo,
+        # norm2, up, down; the final norm last.
+        qk = 2 <= i < 2 + 8 * layers and (i - 2) % 8 in (1, 2)
+        assert np.max(np.abs(d)) <= (4e-2 if qk else 2e-2) * np.max(np.abs(r)), (i, np.max(np.abs(d)), np.max(np.abs(r)))
+        assert np.linalg.norm(d) <= 2.5e-2 * np.linalg.norm(r), (i, np.linalg.norm(d), np.linalg.norm(r))
+
+
 def test_one_sequence_bf16_tier_matches_the_oracle(be, world):
-    """One sequence alone is a harder case than the configuration's batch: twelve layers of bf16
-    rounding with no averaging over sequences. Measured: every tensor within 1.95e-2 normwise,
-    three of the 99 between 2.0e-2 and 2.1e-2 of their largest value at the worst element. The
-    gates here are 2e-2 normwise and 2.5e-2 per element; the configuration's own batch is held
-    to 2e-2 per element in test_full_batch_bf16_tier_within_tolerance_of_the_f32_tier."""
     params, ids, targets, oloss, ograds = world
     tr, loss, grads = gpu_step(be, 1, 1, params, ids[:1], targets[:1])
     tr.close()
     assert abs(loss - oloss) <= 1e-3 * abs(oloss), (loss, oloss)
-    for i, (g, og) in enumerate(zip(grads, ograds)):
-        d = g.astype(np.float64) - og
-        assert np.linalg.norm(d) <= 2e-2 * np.linalg.norm(og), (i, np.linalg.norm(d), np.linalg.norm(og))
-        assert np.max(np.abs(d)) <= 2.5e-2 * np.max(np.abs(og)), (i, np.max(np.abs(d)), np.max(np.abs(og)))
+    check_bf16_gradients(grads, ograds)
 
 
 @pytest.fixture(scope="module")
@@ -134,23 +144,13 @@ def test_full_batch_is_the_mean_of_its_sequences(be, world, full_f32):
 def test_full_batch_bf16_tier_within_tolerance_of_the_f32_tier(be, world, full_f32):
     """configs[2] as benchmarked (bf16 operands, f32 accumulation and master weights) against the
     f32 tier of the same step, which the tests above tie to the oracle within 1e-5. Loss within
-    1e-3 (measured 7e-7). Gradients: every element within 2e-2 of its tensor's largest value,
-    except in the query and key projections, whose gradients pass through the softmax backward
-    of twelve layers and carry 1.9 to 2.0e-2 normwise noise with single elements up to 3.1e-2
-    (gate 4e-2); every tensor within 2.5e-2 normwise (measured at most 2.04e-2)."""
+    1e-3 (measured 3e-6); gradients at the gates of check_bf16_gradients."""
     params, ids, targets, _, _ = world
     loss32, grads32 = full_f32
     tr, loss, grads = gpu_step(be, 16, 1, params, ids, targets)
     tr.close()
     assert abs(loss - loss32) <= 1e-3 * abs(loss32), (loss, loss32)
-    layers = GPT124M[0]
-    for i, (g, g32) in enumerate(zip(grads, grads32)):
-        d = g.astype(np.float64) - g32
-        # Parameter order: token table, position table, then per layer norm1, wq, wk, wv, wo,
-        # norm2, up, down; the final norm last.
-        qk = 2 <= i < 2 + 8 * layers and (i - 2) % 8 in (1, 2)
-        assert np.max(np.abs(d)) <= (4e-2 if qk else 2e-2) * np.max(np.abs(g32)), (i, np.max(np.abs(d)), np.max(np.abs(g32)))
-        assert np.linalg.norm(d) <= 2.5e-2 * np.linalg.norm(g32), (i, np.linalg.norm(d), np.linalg.norm(g32))
+    check_bf16_gradients(grads, grads32)
 
 
 def test_loss_curves_of_the_two_tiers_stay_together(be, world):
