@@ -167,6 +167,28 @@ int32_t omx_causal_attention_backward(omx_ctx* ctx, const void* q, uint64_t q_pi
                                       uint64_t heads, uint64_t kv_heads, uint64_t head_dim,
                                       uint64_t window);
 
+/* The same pair with the output's rounding residual kept for the backward pass:
+ * out_residual = bf16(x - bf16(x)) for every output value x, laid out like out (same pitch).
+ * The backward's row term delta = sum(gy * out) then matches sum_j P dP to 2^-17 instead of 2^-9,
+ * which matters when the value rows (and key rows) share a large common component: the mismatch
+ * times that component lands in gq and gk. The reference's bf16 tier never rounds the saved
+ * output for the same reason ("the backward's dO . O must cancel the softmax row sum",
+ * ojas-core/src/autocast.rs:177-186); with bf16 storage the residual is what keeps it. */
+int32_t omx_causal_attention_forward_saving(omx_ctx* ctx, const void* q, uint64_t q_pitch,
+                                            const void* k, const void* v, uint64_t kv_pitch,
+                                            int32_t operand_dtype, void* out, void* out_residual,
+                                            uint64_t out_pitch, int32_t out_dtype, void* lse,
+                                            uint64_t batch, uint64_t time, uint64_t heads,
+                                            uint64_t kv_heads, uint64_t head_dim, uint64_t window);
+int32_t omx_causal_attention_backward_saved(omx_ctx* ctx, const void* q, uint64_t q_pitch,
+                                            const void* k, const void* v, uint64_t kv_pitch,
+                                            const void* out, const void* out_residual,
+                                            const void* gy, uint64_t out_pitch, const void* lse,
+                                            int32_t operand_dtype, void* gq, void* gk, void* gv,
+                                            int32_t grad_dtype, uint64_t batch, uint64_t time,
+                                            uint64_t heads, uint64_t kv_heads, uint64_t head_dim,
+                                            uint64_t window);
+
 /* ---- BackendModule::rms_norm_forward / _backward (backend.rs:1658-1672) ---- */
 int32_t omx_rms_norm_forward(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* w_f32,
                              void* y, int32_t y_dtype, uint64_t rows, uint64_t dim, float eps);

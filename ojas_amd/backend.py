@@ -311,25 +311,33 @@ class MiBackend:
             C.c_uint64(nin), C.c_uint64(nout), C.c_int32(1 if tanh_form else 0)))
         return gu
 
-    def causal_attention_forward(self, q, k, v, window: Optional[int] = None, pitches=None):
+    def causal_attention_forward(self, q, k, v, window: Optional[int] = None, pitches=None, saving: bool = False):
         """`causal_attention` (ojas-model/src/block.rs:186-199) over time-major [B, T, heads, D]
         tensors. `pitches` = (q, kv) token-row pitches in elements when q / k / v are column
-        blocks of a wider buffer; the output is contiguous."""
+        blocks of a wider buffer; the output is contiguous. `saving=True` also returns the output's
+        rounding residual (what the reference's f32 saved output keeps, autocast.rs:177-186) for
+        `causal_attention_backward(..., residual=)`."""
         b, t, h, d = q.shape
         hkv = k.shape[2]
         qp, kvp = pitches if pitches else (h * d, hkv * d)
         out = self.empty((b, t, h, d), BF16)
         lse = self.empty((b, h, t), F32)
-        self._check(self._lib.omx_causal_attention_forward(
-            self._ctx, self._p(q), C.c_uint64(qp), self._p(k), self._p(v), C.c_uint64(kvp), C.c_int32(q.dtype),
-            self._p(out), C.c_uint64(h * d), C.c_int32(BF16), self._p(lse), C.c_uint64(b), C.c_uint64(t),
-            C.c_uint64(h), C.c_uint64(hkv), C.c_uint64(d), C.c_uint64(window or 0)))
+        tail = (C.c_uint64(h * d), C.c_int32(BF16), self._p(lse), C.c_uint64(b), C.c_uint64(t), C.c_uint64(h),
+                C.c_uint64(hkv), C.c_uint64(d), C.c_uint64(window or 0))
+        head = (self._ctx, self._p(q), C.c_uint64(qp), self._p(k), self._p(v), C.c_uint64(kvp), C.c_int32(q.dtype),
+                self._p(out))
+        if saving:
+            residual = self.empty((b, t, h, d), BF16)
+            self._check(self._lib.omx_causal_attention_forward_saving(*head, self._p(residual), *tail))
+            return out, lse, residual
+        self._check(self._lib.omx_causal_attention_forward(*head, *tail))
         return out, lse
 
     def causal_attention_backward(self, q, k, v, out, lse, gy, window: Optional[int] = None, pitches=None,
-                                  grads=None):
+                                  grads=None, residual=None):
         """Backward of `causal_attention_forward`. `grads` = (gq, gk, gv) tensors to write (they use
-        the operands' pitches); by default contiguous ones are allocated."""
+        the operands' pitches); by default contiguous ones are allocated. `residual`: the third
+        value of the saving forward."""
         b, t, h, d = q.shape
         hkv = k.shape[2]
         qp, kvp = pitches if pitches else (h * d, hkv * d)
@@ -338,11 +346,16 @@ class MiBackend:
                 raise OjasError(SHAPE, "causal_attention_backward: pass `grads` with pitched operands")
             grads = (self.empty(q.shape, BF16), self.empty(k.shape, BF16), self.empty(v.shape, BF16))
         gq, gk, gv = grads
-        self._check(self._lib.omx_causal_attention_backward(
-            self._ctx, self._p(q), C.c_uint64(qp), self._p(k), self._p(v), C.c_uint64(kvp), self._p(out),
-            self._p(gy), C.c_uint64(h * d), self._p(lse), C.c_int32(q.dtype), self._p(gq), self._p(gk), self._p(gv),
-            C.c_int32(BF16), C.c_uint64(b), C.c_uint64(t), C.c_uint64(h), C.c_uint64(hkv), C.c_uint64(d),
-            C.c_uint64(window or 0)))
+        head = (self._ctx, self._p(q), C.c_uint64(qp), self._p(k), self._p(v), C.c_uint64(kvp), self._p(out))
+        tail = (self._p(gy), C.c_uint64(h * d), self._p(lse), C.c_int32(q.dtype), self._p(gq), self._p(gk), self._p(gv),
+                C.c_int32(BF16), C.c_uint64(b), C.c_uint64(t), C.c_uint64(h), C.c_uint64(hkv), C.c_uint64(d),
+                C.c_uint64(window or 0))
+        if residual is not None:
+            if residual.shape != out.shape or residual.dtype != BF16:
+                raise OjasError(SHAPE, "causal_attention_backward: residual must match the output")
+            self._check(self._lib.omx_causal_attention_backward_saved(*head, self._p(residual), *tail))
+        else:
+            self._check(self._lib.omx_causal_attention_backward(*head, *tail))
         return gq, gk, gv
 
     # ---- norms ----

@@ -159,13 +159,39 @@ __device__ __forceinline__ bool store_transposed_acc(TO* __restrict__ plane, lon
   return bad;
 }
 
+// The bf16 store of the output together with what the rounding dropped: residual = x - bf16(x),
+// itself rounded to bf16, so that bf16(x) + residual carries 16 bits of x's mantissa.
+__device__ __forceinline__ bool store_transposed_acc_split(unsigned short* __restrict__ plane,
+                                                           unsigned short* __restrict__ resid, long rs, int row,
+                                                           int time, int lg, const floatx16 acc[2], float mul) {
+  bool bad = false;
+  if (row >= time) return false;
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      const int d = mt * 32 + 8 * q4 + 4 * lg;
+      const float x0 = acc[mt][4 * q4 + 0] * mul, x1 = acc[mt][4 * q4 + 1] * mul, x2 = acc[mt][4 * q4 + 2] * mul,
+                  x3 = acc[mt][4 * q4 + 3] * mul;
+      bad |= !(dev_finite(x0) && dev_finite(x1) && dev_finite(x2) && dev_finite(x3));
+      uint2 w, r;
+      w.x = pack2(x0, x1);
+      w.y = pack2(x2, x3);
+      r.x = pack2(x0 - __uint_as_float(w.x << 16), x1 - __uint_as_float(w.x & 0xffff0000u));
+      r.y = pack2(x2 - __uint_as_float(w.y << 16), x3 - __uint_as_float(w.y & 0xffff0000u));
+      *reinterpret_cast<uint2*>(plane + static_cast<long>(row) * rs + d) = w;
+      *reinterpret_cast<uint2*>(resid + static_cast<long>(row) * rs + d) = r;
+    }
+  return bad;
+}
+
 // ------------------------------------------------------------------ forward
 template <typename TO>
 __global__ __launch_bounds__(FT, 3) void flash_fwd_kernel(const unsigned short* __restrict__ q,
                                                        const unsigned short* __restrict__ k,
                                                        const unsigned short* __restrict__ v, TO* __restrict__ out,
-                                                       float* __restrict__ lse, FlashShape s, OmxFaultWord* fault,
-                                                       unsigned long long tag) {
+                                                       unsigned short* __restrict__ resid, float* __restrict__ lse,
+                                                       FlashShape s, OmxFaultWord* fault, unsigned long long tag) {
   __shared__ __attribute__((aligned(16))) char smem[2 * FTILE];
   char* k_rows = smem;
   char* v_rows = smem + FTILE;
@@ -270,7 +296,13 @@ __global__ __launch_bounds__(FT, 3) void flash_fwd_kernel(const unsigned short* 
     bad |= !(dev_finite(lsum) && lsum > 0.0f);
     if (lg == 0) lse[plane * T + q_row] = m * s.scale + logf(lsum);
   }
-  bad |= store_transposed_acc<TO>(out + b * s.o.bs + h * s.o.hs, s.o.rs, q_row, T, lg, o, 1.0f / lsum);
+  const long o_off = b * s.o.bs + h * s.o.hs;
+  if constexpr (sizeof(TO) == 2) {
+    if (resid) bad |= store_transposed_acc_split(out + o_off, resid + o_off, s.o.rs, q_row, T, lg, o, 1.0f / lsum);
+    else bad |= store_transposed_acc<TO>(out + o_off, s.o.rs, q_row, T, lg, o, 1.0f / lsum);
+  } else {
+    bad |= store_transposed_acc<TO>(out + o_off, s.o.rs, q_row, T, lg, o, 1.0f / lsum);
+  }
   if (bad) dev_raise_fault(fault, tag);
 }
 
@@ -400,9 +432,9 @@ __global__ __launch_bounds__(FT, 2) void flash_bwd_dkv_kernel(
 template <typename TO>
 __global__ __launch_bounds__(FT, 3) void flash_bwd_dq_kernel(
     const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
-    const unsigned short* __restrict__ out, const float* __restrict__ lse, float* __restrict__ delta,
-    const unsigned short* __restrict__ gy, TO* __restrict__ gq, FlashShape s, OmxFaultWord* fault,
-    unsigned long long tag) {
+    const unsigned short* __restrict__ out, const unsigned short* __restrict__ resid, const float* __restrict__ lse,
+    float* __restrict__ delta, const unsigned short* __restrict__ gy, TO* __restrict__ gq, FlashShape s,
+    OmxFaultWord* fault, unsigned long long tag) {
   __shared__ __attribute__((aligned(16))) char smem[2 * FTILE];
   char* k_rows = smem;
   char* v_rows = smem + FTILE;
@@ -420,21 +452,31 @@ __global__ __launch_bounds__(FT, 3) void flash_bwd_dq_kernel(
   row_frags(q + b * s.q.bs + h * s.q.hs, s.q.rs, q_row, T, lg, qf);
   row_frags(gy + b * s.o.bs + h * s.o.hs, s.o.rs, q_row, T, lg, gf);
   // delta = dO . O of this lane's row: each half-wave holds half of the row's 64 values. The
-  // dK/dV pass, launched after this one, reads it back from `delta`.
+  // dK/dV pass, launched after this one, reads it back from `delta`. dS = P (dP - delta) sums to
+  // zero along a row only as far as delta matches sum_j P dP: taken from the bf16 output alone it
+  // is off by 2^-9 of |dO| |O|, which a component shared by all value rows (and by all key rows,
+  // in dQ = dS K) turns into a multiple of the gradient itself. With the saved rounding residual
+  // of the output the mismatch drops to 2^-17.
   float row_del = 0.0f;
   {
-    u32x4 of[4];
-    row_frags(out + b * s.o.bs + h * s.o.hs, s.o.rs, q_row, T, lg, of);
+    auto dot_rows = [&](const unsigned short* plane) {
+      u32x4 of[4];
+      row_frags(plane + b * s.o.bs + h * s.o.hs, s.o.rs, q_row, T, lg, of);
+      float sum = 0.0f;
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      const unsigned int gw[4] = {gf[kk].x, gf[kk].y, gf[kk].z, gf[kk].w};
-      const unsigned int ow[4] = {of[kk].x, of[kk].y, of[kk].z, of[kk].w};
+      for (int kk = 0; kk < 4; ++kk) {
+        const unsigned int gw[4] = {gf[kk].x, gf[kk].y, gf[kk].z, gf[kk].w};
+        const unsigned int ow[4] = {of[kk].x, of[kk].y, of[kk].z, of[kk].w};
 #pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        row_del += __uint_as_float(gw[w] << 16) * __uint_as_float(ow[w] << 16);
-        row_del += __uint_as_float(gw[w] & 0xffff0000u) * __uint_as_float(ow[w] & 0xffff0000u);
+        for (int w = 0; w < 4; ++w) {
+          sum += __uint_as_float(gw[w] << 16) * __uint_as_float(ow[w] << 16);
+          sum += __uint_as_float(gw[w] & 0xffff0000u) * __uint_as_float(ow[w] & 0xffff0000u);
+        }
       }
-    }
+      return sum;
+    };
+    row_del = dot_rows(out);
+    if (resid) row_del += dot_rows(resid);
     row_del += __shfl_xor(row_del, 32, 64);
   }
   float row_lse = 0.0f;
@@ -528,8 +570,9 @@ FlashShape make_shape(uint64_t batch, uint64_t heads, uint64_t kv_heads, uint64_
 bool omx_flash_sdpa_supports(uint64_t dim, int32_t operand_dtype) { return dim == FD && operand_dtype == OMX_BF16; }
 
 int32_t omx_flash_sdpa_forward(omx_ctx* ctx, const void* q, const void* k, const void* v, void* out, int32_t out_dtype,
-                               float* lse, uint64_t batch, uint64_t heads, uint64_t kv_heads, uint64_t time,
-                               uint64_t dim, uint64_t window, float scale, unsigned long long tag, const long* strides) {
+                               void* out_residual, float* lse, uint64_t batch, uint64_t heads, uint64_t kv_heads,
+                               uint64_t time, uint64_t dim, uint64_t window, float scale, unsigned long long tag,
+                               const long* strides) {
   if (dim != FD) return omx_fail(ctx, OMX_UNSUPPORTED_HEAD_DIM, "head_dim %llu limit %d", (unsigned long long)dim, FD);
   FlashShape s = make_shape(batch, heads, kv_heads, time, window, scale, strides);
   dim3 grid(static_cast<unsigned>((time + 127) / 128), static_cast<unsigned>(batch * heads)), block(FT);
@@ -538,16 +581,18 @@ int32_t omx_flash_sdpa_forward(omx_ctx* ctx, const void* q, const void* k, const
   const unsigned short* vs = static_cast<const unsigned short*>(v);
   if (out_dtype == OMX_BF16)
     hipLaunchKernelGGL((flash_fwd_kernel<unsigned short>), grid, block, 0, ctx->stream, qs, ks, vs,
-                       static_cast<unsigned short*>(out), lse, s, ctx->fault, tag);
+                       static_cast<unsigned short*>(out), static_cast<unsigned short*>(out_residual), lse, s,
+                       ctx->fault, tag);
   else
     hipLaunchKernelGGL((flash_fwd_kernel<float>), grid, block, 0, ctx->stream, qs, ks, vs, static_cast<float*>(out),
-                       lse, s, ctx->fault, tag);
+                       static_cast<unsigned short*>(nullptr), lse, s, ctx->fault, tag);
   OMX_LAUNCH_CHECK(ctx, "flash_fwd_kernel");
   return OMX_OK;
 }
 
 int32_t omx_flash_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, const void* v, const void* out,
-                                const float* lse, const void* gy, void* gq, void* gk, void* gv, int32_t grad_dtype,
+                                const void* out_residual, const float* lse, const void* gy, void* gq, void* gk,
+                                void* gv, int32_t grad_dtype,
                                 uint64_t batch, uint64_t heads, uint64_t kv_heads, uint64_t time, uint64_t dim,
                                 uint64_t window, float scale, unsigned long long tag, const long* strides) {
   if (dim != FD) return omx_fail(ctx, OMX_UNSUPPORTED_HEAD_DIM, "head_dim %llu limit %d", (unsigned long long)dim, FD);
@@ -561,18 +606,19 @@ int32_t omx_flash_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, cons
   const unsigned short* ks = static_cast<const unsigned short*>(k);
   const unsigned short* vs = static_cast<const unsigned short*>(v);
   const unsigned short* os = static_cast<const unsigned short*>(out);
+  const unsigned short* rs = static_cast<const unsigned short*>(out_residual);
   const unsigned short* gs = static_cast<const unsigned short*>(gy);
   // dQ first: it also leaves delta = dO . O per row for the dK/dV pass.
   dim3 block(FT);
   dim3 kv_grid(static_cast<unsigned>((time + 127) / 128), static_cast<unsigned>(batch * kv_heads));
   dim3 q_grid(static_cast<unsigned>((time + 127) / 128), static_cast<unsigned>(batch * heads));
   if (grad_dtype == OMX_BF16) {
-    hipLaunchKernelGGL((flash_bwd_dq_kernel<unsigned short>), q_grid, block, 0, ctx->stream, qs, ks, vs, os, lse, delta,
-                       gs, static_cast<unsigned short*>(gq), s, ctx->fault, tag);
+    hipLaunchKernelGGL((flash_bwd_dq_kernel<unsigned short>), q_grid, block, 0, ctx->stream, qs, ks, vs, os, rs, lse,
+                       delta, gs, static_cast<unsigned short*>(gq), s, ctx->fault, tag);
     hipLaunchKernelGGL((flash_bwd_dkv_kernel<unsigned short>), kv_grid, block, 0, ctx->stream, qs, ks, vs, lse, delta,
                        gs, static_cast<unsigned short*>(gk), static_cast<unsigned short*>(gv), s, ctx->fault, tag);
   } else {
-    hipLaunchKernelGGL((flash_bwd_dq_kernel<float>), q_grid, block, 0, ctx->stream, qs, ks, vs, os, lse, delta, gs,
+    hipLaunchKernelGGL((flash_bwd_dq_kernel<float>), q_grid, block, 0, ctx->stream, qs, ks, vs, os, rs, lse, delta, gs,
                        static_cast<float*>(gq), s, ctx->fault, tag);
     hipLaunchKernelGGL((flash_bwd_dkv_kernel<float>), kv_grid, block, 0, ctx->stream, qs, ks, vs, lse, delta, gs,
                        static_cast<float*>(gk), static_cast<float*>(gv), s, ctx->fault, tag);

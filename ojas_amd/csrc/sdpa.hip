@@ -19,11 +19,12 @@
 #include "omx_common.h"
 
 int32_t omx_flash_sdpa_forward(omx_ctx* ctx, const void* q, const void* k, const void* v, void* out,
-                               int32_t out_dtype, float* lse, uint64_t batch, uint64_t heads, uint64_t kv_heads,
-                               uint64_t time, uint64_t dim, uint64_t window, float scale, unsigned long long tag,
-                               const long* strides);
+                               int32_t out_dtype, void* out_residual, float* lse, uint64_t batch, uint64_t heads,
+                               uint64_t kv_heads, uint64_t time, uint64_t dim, uint64_t window, float scale,
+                               unsigned long long tag, const long* strides);
 int32_t omx_flash_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, const void* v, const void* out,
-                                const float* lse, const void* gy, void* gq, void* gk, void* gv, int32_t grad_dtype,
+                                const void* out_residual, const float* lse, const void* gy, void* gq, void* gk,
+                                void* gv, int32_t grad_dtype,
                                 uint64_t batch, uint64_t heads, uint64_t kv_heads, uint64_t time, uint64_t dim,
                                 uint64_t window, float scale, unsigned long long tag, const long* strides);
 bool omx_flash_sdpa_supports(uint64_t dim, int32_t operand_dtype);
@@ -334,8 +335,8 @@ int32_t omx_causal_sdpa_forward(omx_ctx* ctx, const void* q, const void* k, cons
   if (rc != OMX_OK) return rc;
   unsigned long long tag = omx_tag(ctx, F_SDPA_FORWARD);
   if (omx_flash_sdpa_supports(head_dim, operand_dtype))
-    return omx_flash_sdpa_forward(ctx, q, k, v, out, out_dtype, static_cast<float*>(lse), batch, heads, kv_heads, time,
-                                  head_dim, s.window, s.scale, tag, nullptr);
+    return omx_flash_sdpa_forward(ctx, q, k, v, out, out_dtype, nullptr, static_cast<float*>(lse), batch, heads,
+                                  kv_heads, time, head_dim, s.window, s.scale, tag, nullptr);
   const long rows = static_cast<long>(batch) * heads * time;
   dim3 grid(static_cast<unsigned>((rows + 3) / 4)), block(SD_THREADS);
 #define SDPA_FWD(TI, TO)                                                                                          \
@@ -366,8 +367,8 @@ int32_t omx_causal_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, con
   if (rc != OMX_OK) return rc;
   unsigned long long tag = omx_tag(ctx, F_SDPA_BACKWARD);
   if (omx_flash_sdpa_supports(head_dim, operand_dtype))
-    return omx_flash_sdpa_backward(ctx, q, k, v, out, static_cast<const float*>(lse), gy, gq, gk, gv, grad_dtype, batch,
-                                   heads, kv_heads, time, head_dim, s.window, s.scale, tag, nullptr);
+    return omx_flash_sdpa_backward(ctx, q, k, v, out, nullptr, static_cast<const float*>(lse), gy, gq, gk, gv,
+                                   grad_dtype, batch, heads, kv_heads, time, head_dim, s.window, s.scale, tag, nullptr);
   const long rows = static_cast<long>(batch) * heads * time;
   const long kv_rows = static_cast<long>(batch) * kv_heads * time;
   void* ws = nullptr;
@@ -414,12 +415,11 @@ static int32_t check_attention(omx_ctx* ctx, const char* op, int32_t operand_dty
   return OMX_OK;
 }
 
-int32_t omx_causal_attention_forward(omx_ctx* ctx, const void* q, uint64_t q_pitch, const void* k, const void* v,
-                                     uint64_t kv_pitch, int32_t operand_dtype, void* out, uint64_t out_pitch,
-                                     int32_t out_dtype, void* lse, uint64_t batch, uint64_t time, uint64_t heads,
-                                     uint64_t kv_heads, uint64_t head_dim, uint64_t window) {
+static int32_t attention_forward(omx_ctx* ctx, const char* op, const void* q, uint64_t q_pitch, const void* k,
+                                 const void* v, uint64_t kv_pitch, int32_t operand_dtype, void* out,
+                                 void* out_residual, uint64_t out_pitch, int32_t out_dtype, void* lse, uint64_t batch,
+                                 uint64_t time, uint64_t heads, uint64_t kv_heads, uint64_t head_dim, uint64_t window) {
   OMX_REQUIRE_CTX(ctx);
-  const char* op = "causal_attention_forward";
   if (out_dtype != OMX_BF16) return omx_fail(ctx, OMX_DTYPE, "%s: output must be bf16", op);
   SdpaShape s;
   int32_t rc = check_shape(ctx, op, batch, heads, kv_heads, time, head_dim, window, &s);
@@ -427,21 +427,22 @@ int32_t omx_causal_attention_forward(omx_ctx* ctx, const void* q, uint64_t q_pit
   rc = check_attention(ctx, op, operand_dtype, head_dim, heads, kv_heads, q_pitch, kv_pitch, out_pitch,
                        {q, k, v, out, lse});
   if (rc != OMX_OK) return rc;
+  if (reinterpret_cast<uintptr_t>(out_residual) & 15u)
+    return omx_fail(ctx, OMX_SHAPE, "%s: tensor not 16-byte aligned", op);
   const long D = static_cast<long>(head_dim), T = static_cast<long>(time);
   const long strides[9] = {static_cast<long>(q_pitch),   D, T * static_cast<long>(q_pitch),
                            static_cast<long>(kv_pitch),  D, T * static_cast<long>(kv_pitch),
                            static_cast<long>(out_pitch), D, T * static_cast<long>(out_pitch)};
-  return omx_flash_sdpa_forward(ctx, q, k, v, out, out_dtype, static_cast<float*>(lse), batch, heads, kv_heads, time,
-                                head_dim, s.window, s.scale, omx_tag(ctx, F_SDPA_FORWARD), strides);
+  return omx_flash_sdpa_forward(ctx, q, k, v, out, out_dtype, out_residual, static_cast<float*>(lse), batch, heads,
+                                kv_heads, time, head_dim, s.window, s.scale, omx_tag(ctx, F_SDPA_FORWARD), strides);
 }
 
-int32_t omx_causal_attention_backward(omx_ctx* ctx, const void* q, uint64_t q_pitch, const void* k, const void* v,
-                                      uint64_t kv_pitch, const void* out, const void* gy, uint64_t out_pitch,
-                                      const void* lse, int32_t operand_dtype, void* gq, void* gk, void* gv,
-                                      int32_t grad_dtype, uint64_t batch, uint64_t time, uint64_t heads,
-                                      uint64_t kv_heads, uint64_t head_dim, uint64_t window) {
+static int32_t attention_backward(omx_ctx* ctx, const char* op, const void* q, uint64_t q_pitch, const void* k,
+                                  const void* v, uint64_t kv_pitch, const void* out, const void* out_residual,
+                                  const void* gy, uint64_t out_pitch, const void* lse, int32_t operand_dtype, void* gq,
+                                  void* gk, void* gv, int32_t grad_dtype, uint64_t batch, uint64_t time, uint64_t heads,
+                                  uint64_t kv_heads, uint64_t head_dim, uint64_t window) {
   OMX_REQUIRE_CTX(ctx);
-  const char* op = "causal_attention_backward";
   if (grad_dtype != OMX_BF16) return omx_fail(ctx, OMX_DTYPE, "%s: gradients must be bf16", op);
   SdpaShape s;
   int32_t rc = check_shape(ctx, op, batch, heads, kv_heads, time, head_dim, window, &s);
@@ -449,13 +450,55 @@ int32_t omx_causal_attention_backward(omx_ctx* ctx, const void* q, uint64_t q_pi
   rc = check_attention(ctx, op, operand_dtype, head_dim, heads, kv_heads, q_pitch, kv_pitch, out_pitch,
                        {q, k, v, out, gy, lse, gq, gk, gv});
   if (rc != OMX_OK) return rc;
+  if (reinterpret_cast<uintptr_t>(out_residual) & 15u)
+    return omx_fail(ctx, OMX_SHAPE, "%s: tensor not 16-byte aligned", op);
   const long D = static_cast<long>(head_dim), T = static_cast<long>(time);
   const long strides[9] = {static_cast<long>(q_pitch),   D, T * static_cast<long>(q_pitch),
                            static_cast<long>(kv_pitch),  D, T * static_cast<long>(kv_pitch),
                            static_cast<long>(out_pitch), D, T * static_cast<long>(out_pitch)};
-  return omx_flash_sdpa_backward(ctx, q, k, v, out, static_cast<const float*>(lse), gy, gq, gk, gv, grad_dtype, batch,
-                                 heads, kv_heads, time, head_dim, s.window, s.scale, omx_tag(ctx, F_SDPA_BACKWARD),
-                                 strides);
+  return omx_flash_sdpa_backward(ctx, q, k, v, out, out_residual, static_cast<const float*>(lse), gy, gq, gk, gv,
+                                 grad_dtype, batch, heads, kv_heads, time, head_dim, s.window, s.scale,
+                                 omx_tag(ctx, F_SDPA_BACKWARD), strides);
+}
+
+int32_t omx_causal_attention_forward(omx_ctx* ctx, const void* q, uint64_t q_pitch, const void* k, const void* v,
+                                     uint64_t kv_pitch, int32_t operand_dtype, void* out, uint64_t out_pitch,
+                                     int32_t out_dtype, void* lse, uint64_t batch, uint64_t time, uint64_t heads,
+                                     uint64_t kv_heads, uint64_t head_dim, uint64_t window) {
+  return attention_forward(ctx, "causal_attention_forward", q, q_pitch, k, v, kv_pitch, operand_dtype, out, nullptr,
+                           out_pitch, out_dtype, lse, batch, time, heads, kv_heads, head_dim, window);
+}
+
+int32_t omx_causal_attention_backward(omx_ctx* ctx, const void* q, uint64_t q_pitch, const void* k, const void* v,
+                                      uint64_t kv_pitch, const void* out, const void* gy, uint64_t out_pitch,
+                                      const void* lse, int32_t operand_dtype, void* gq, void* gk, void* gv,
+                                      int32_t grad_dtype, uint64_t batch, uint64_t time, uint64_t heads,
+                                      uint64_t kv_heads, uint64_t head_dim, uint64_t window) {
+  return attention_backward(ctx, "causal_attention_backward", q, q_pitch, k, v, kv_pitch, out, nullptr, gy, out_pitch,
+                            lse, operand_dtype, gq, gk, gv, grad_dtype, batch, time, heads, kv_heads, head_dim, window);
+}
+
+int32_t omx_causal_attention_forward_saving(omx_ctx* ctx, const void* q, uint64_t q_pitch, const void* k,
+                                            const void* v, uint64_t kv_pitch, int32_t operand_dtype, void* out,
+                                            void* out_residual, uint64_t out_pitch, int32_t out_dtype, void* lse,
+                                            uint64_t batch, uint64_t time, uint64_t heads, uint64_t kv_heads,
+                                            uint64_t head_dim, uint64_t window) {
+  const char* op = "causal_attention_forward_saving";
+  if (ctx && !out_residual) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  return attention_forward(ctx, op, q, q_pitch, k, v, kv_pitch, operand_dtype, out, out_residual, out_pitch, out_dtype,
+                           lse, batch, time, heads, kv_heads, head_dim, window);
+}
+
+int32_t omx_causal_attention_backward_saved(omx_ctx* ctx, const void* q, uint64_t q_pitch, const void* k,
+                                            const void* v, uint64_t kv_pitch, const void* out,
+                                            const void* out_residual, const void* gy, uint64_t out_pitch,
+                                            const void* lse, int32_t operand_dtype, void* gq, void* gk, void* gv,
+                                            int32_t grad_dtype, uint64_t batch, uint64_t time, uint64_t heads,
+                                            uint64_t kv_heads, uint64_t head_dim, uint64_t window) {
+  const char* op = "causal_attention_backward_saved";
+  if (ctx && !out_residual) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  return attention_backward(ctx, op, q, q_pitch, k, v, kv_pitch, out, out_residual, gy, out_pitch, lse, operand_dtype,
+                            gq, gk, gv, grad_dtype, batch, time, heads, kv_heads, head_dim, window);
 }
 
 }  // extern "C"

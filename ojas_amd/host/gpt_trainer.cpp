@@ -50,6 +50,7 @@ struct ogpt {
   struct Layer {
     float *x, *x1;                          // residual stream (f32)
     void *h1, *q, *k, *v, *a, *ap, *h2, *u, *g;  // AD
+    void* apr = nullptr;  // rounding residual of ap (fused bf16 attention only)
     float* lse;
   };
   std::vector<Layer> layers;
@@ -139,7 +140,10 @@ int32_t forward(ogpt* t) {
     const float* next_norm = t->w32(last ? t->nf() : t->li(l + 1, 0));
     if (t->fused_qkv) {
       TRY(omx_linear_forward(ctx, A.h1, AD, t->w(t->li(l, 1)), AD, A.q, AD, N, d, 3 * d));
-      TRY(omx_causal_attention_forward(ctx, A.q, 3 * d, A.k, A.v, 3 * d, AD, A.ap, d, AD, A.lse, B, T, H, H, D, 0));
+      // The output's rounding residual is kept for the backward's row term, as the reference keeps
+      // its saved output unrounded (ojas-core/src/autocast.rs:177-186).
+      TRY(omx_causal_attention_forward_saving(ctx, A.q, 3 * d, A.k, A.v, 3 * d, AD, A.ap, A.apr, d, AD, A.lse, B, T, H,
+                                              H, D, 0));
     } else {
       TRY(omx_linear_forward(ctx, A.h1, AD, t->w(t->li(l, 1)), AD, t->t_a, AD, N, d, d));
       TRY(omx_permute_0213(ctx, t->t_a, A.q, AD, B, T, H, D));
@@ -204,7 +208,7 @@ int32_t backward(ogpt* t) {
     TRY(omx_linear_backward(ctx, A.ap, t->w(t->li(l, 4)), gy, AD, t->t_a, AD, t->g(t->li(l, 4)), OMX_F32, N, d, d));
     if (t->fused_qkv) {
       char* gq = static_cast<char*>(t->gqkv);
-      TRY(omx_causal_attention_backward(ctx, A.q, 3 * d, A.k, A.v, 3 * d, A.ap, t->t_a, d, A.lse, AD, gq,
+      TRY(omx_causal_attention_backward_saved(ctx, A.q, 3 * d, A.k, A.v, 3 * d, A.ap, A.apr, t->t_a, d, A.lse, AD, gq,
                                         gq + d * t->asz, gq + 2 * d * t->asz, AD, B, T, H, H, D, 0));
       // One product for the three projections: the input gradient is their sum, formed in the
       // product's f32 accumulators.
@@ -311,6 +315,7 @@ int32_t ogpt_create(omx_ctx* ctx, const ogpt_config* config, ogpt** out) {
       A.k = static_cast<char*>(A.q) + d * t->asz;
       A.v = static_cast<char*>(A.q) + 2 * d * t->asz;
       A.a = nullptr;
+      CREATE_TRY(alloc_act(t, N * d, &A.apr));
     } else {
       CREATE_TRY(alloc_act(t, N * d, &A.q));
       CREATE_TRY(alloc_act(t, N * d, &A.k));

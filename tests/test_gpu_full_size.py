@@ -83,21 +83,17 @@ def test_one_sequence_f32_tier_matches_the_oracle(be, world):
 
 
 def check_bf16_gradients(grads, ref):
-    """The bf16 tier's gradient gates at this depth. Every element within 2e-2 of its tensor's
-    largest value, except in the query and key projections: their gradients come out of the
-    softmax backward with 1.0e-2 (first layer) to 2.1e-2 (from the sixth layer on) normwise noise
-    and single elements up to 3.1e-2 (gate 4e-2); all other tensors measure at most 1.1e-2
-    normwise and 1.4e-2 per element. Every tensor within 2.5e-2 normwise. Two kernels that
-    differ only in the order of an f32 sum give different realizations of this noise (see the
-    module text), so the gates leave a fifth of headroom over what one build measured."""
-    layers = GPT124M[0]
+    """The bf16 tier's gradient gate, at this depth as for single ops: every element within 2e-2
+    of its tensor's largest value (measured at most 1.6e-2, in the query and key projections;
+    1.4e-2 elsewhere), and every tensor within 2e-2 normwise (measured 1.4e-2 and 1.1e-2). The
+    query and key projections meet it because the attention backward takes its row term from the
+    output plus its saved rounding residual; from the bf16 output alone they measured up to
+    3.1e-2 per element and 2.1e-2 normwise from the sixth layer on, where the residual stream has
+    grown a component common to all positions."""
     for i, (g, r) in enumerate(zip(grads, ref)):
         d = g.astype(np.float64) - r
-        # Parameter order: token table, position table, then per layer norm1, wq, wk, wv, wo,
-        # norm2, up, down; the final norm last.
-        qk = 2 <= i < 2 + 8 * layers and (i - 2) % 8 in (1, 2)
-        assert np.max(np.abs(d)) <= (4e-2 if qk else 2e-2) * np.max(np.abs(r)), (i, np.max(np.abs(d)), np.max(np.abs(r)))
-        assert np.linalg.norm(d) <= 2.5e-2 * np.linalg.norm(r), (i, np.linalg.norm(d), np.linalg.norm(r))
+        assert np.max(np.abs(d)) <= 2e-2 * np.max(np.abs(r)), (i, np.max(np.abs(d)), np.max(np.abs(r)))
+        assert np.linalg.norm(d) <= 2e-2 * np.linalg.norm(r), (i, np.linalg.norm(d), np.linalg.norm(r))
 
 
 def test_one_sequence_bf16_tier_matches_the_oracle(be, world):
@@ -156,7 +152,7 @@ def test_full_batch_bf16_tier_within_tolerance_of_the_f32_tier(be, world, full_f
 def test_loss_curves_of_the_two_tiers_stay_together(be, world):
     """AdamW (lr 3e-4, betas 0.9/0.95, weight decay 0.1, clip 1.0) on the fixed 16 x 1024 batch: the
     bf16 tier's loss follows the f32 tier's within 1e-2 nats over the first 12 steps (measured at
-    most 4.8e-3 while the loss falls by 2.7 nats), and over 50 steps it keeps falling and ends far
+    most 2.8e-3 while the loss falls by 2.7 nats), and over 50 steps it keeps falling and ends far
     more than the reference's minimum drop of 1 nat below ln V (ojas-oracle/src/parity.rs:58)."""
     from ojas_amd.backend import AdamWConfig
     from ojas_amd.trainer import GptConfig, GptTrainer
