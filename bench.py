@@ -33,7 +33,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor figure
 # step's 150 GEMM ops: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by what the same
 # counters read for the AdamW pass, whose traffic is known (profiles/gemm_hbm_traffic_gpt124m_bf16.txt).
 # The algorithmic figure (every operand read once, every output written once) is 1.550e8.
-GEMM_HBM_BYTES_PER_LAUNCH_GPT124M = 3.15e8
+GEMM_HBM_BYTES_PER_LAUNCH_GPT124M = 2.93e8
 
 
 def cpu_baseline(cfg, threads: int):
