@@ -254,6 +254,22 @@ typedef struct {
 int32_t omx_adamw_step(omx_ctx* ctx, void* param_f32, const void* grad_f32, void* moment1_f32,
                        void* moment2_f32, uint64_t n, uint64_t step, const omx_adamw_config* config,
                        void* param_bf16);
+/* The same update for a caller that owns the tensors between calls (a trainer's arenas). The
+ * reference's all-or-nothing rule (nothing is written when any result is non-finite,
+ * ojas-cpu/src/optim.rs:302-395) costs a checking pass over all four tensors before the writing
+ * one. That pass has nothing to find when every input is below 2^60 in magnitude and the scalars
+ * are moderate (step size <= 2^20, |1 - lr wd| <= 2, eps >= 2^-40): no result can overflow. So:
+ * `unbounded_flag` (device u32, never cleared here) is OR-ed with 1 when a parameter or moment
+ * that stays in memory after the call reaches 2^60 or is not finite: the inputs when the update
+ * is refused or checked, the outputs when it is written. `inputs_bounded` != 0 is the caller's
+ * word that param, both moments (a zero flag since they were last written from outside) and grad
+ * (a finite gradient norm below 2^60) are all below 2^60; the checking pass is then skipped.
+ * Results are bit for bit those of omx_adamw_step. No counterpart in the reference, whose backend
+ * calls are stateless. `omx_set_option("adamw_trust", 0)` makes every call check. */
+int32_t omx_adamw_step_bounded(omx_ctx* ctx, void* param_f32, const void* grad_f32,
+                               void* moment1_f32, void* moment2_f32, uint64_t n, uint64_t step,
+                               const omx_adamw_config* config, void* param_bf16,
+                               int32_t inputs_bounded, void* unbounded_flag);
 /* ojas_core::MuonNs5Config (backend.rs:548-570). */
 typedef struct {
   double lr, momentum, weight_decay;

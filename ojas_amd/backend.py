@@ -467,6 +467,16 @@ class MiBackend:
                                              self._p(moment2), C.c_uint64(param.numel), C.c_uint64(step),
                                              C.byref(config), self._p(param_bf16)))
 
+    def adamw_step_bounded(self, param, grad, moment1, moment2, step: int, config: AdamWConfig, inputs_bounded: bool,
+                           unbounded_flag: DeviceTensor, param_bf16=None):
+        """`adamw_step` for a caller that tracks its tensors between calls: with `inputs_bounded`
+        (every input below 2^60 in magnitude) the checking pass is skipped; `unbounded_flag` (one
+        u32) is OR-ed with 1 when a stored parameter or moment reaches 2^60."""
+        self._check(self._lib.omx_adamw_step_bounded(
+            self._ctx, self._p(param), self._p(grad), self._p(moment1), self._p(moment2), C.c_uint64(param.numel),
+            C.c_uint64(step), C.byref(config), self._p(param_bf16), C.c_int32(1 if inputs_bounded else 0),
+            self._p(unbounded_flag)))
+
     def muon_ns5_step(self, param, grad, momentum, config: MuonNs5Config, param_bf16=None):
         rows, cols = param.shape
         self._check(self._lib.omx_muon_ns5_step(self._ctx, self._p(param), self._p(grad), self._p(momentum),

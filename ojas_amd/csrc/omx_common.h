@@ -85,6 +85,7 @@ struct omx_ctx {
   // 0: 128x128 kernel only; 1: choose by shape; 2 / 3: force the 256x256 / 256x128 direct-to-LDS kernel where eligible.
   int gemm_dma_mode = 1;
   int kv_attention_mode = 0;  // 1: cached attention always takes the LDS-tiled kernel
+  int adamw_trust = 1;        // 0: omx_adamw_step_bounded always runs its checking pass
   bool profile_gemm = false;
   struct TimedLaunch {
     hipEvent_t start, stop;

@@ -38,6 +38,11 @@ struct ogpt {
   int32_t AD = OMX_F32;  // activation / operand dtype
   uint64_t asz = 4;
   uint64_t steps = 0;
+  // omx_adamw_step_bounded's flag word, and which ranges it has covered since they were last
+  // written from outside: nothing, the tables and norms (hybrid steps), or every parameter.
+  void* unbounded = nullptr;
+  enum Tracked { kNone = 0, kHybrid = 1, kFull = 2 };
+  int tracked = kNone;
   uint64_t device_bytes = 0;
   std::vector<void*> owned;
 
@@ -300,6 +305,8 @@ int32_t ogpt_create(omx_ctx* ctx, const ogpt_config* config, ogpt** out) {
   CREATE_TRY(alloc_t(t, N, &t->targets));
   CREATE_TRY(alloc_t(t, N, &t->positions));
   CREATE_TRY(alloc_t(t, 4, &t->loss));
+  CREATE_TRY(alloc(t, 256, &t->unbounded));
+  CREATE_TRY(omx_fill_zero(ctx, t->unbounded, 256));
   {
     std::vector<uint32_t> pos(N);
     for (uint64_t i = 0; i < N; ++i) pos[i] = static_cast<uint32_t>(i % c.ctx);
@@ -370,6 +377,7 @@ uint64_t ogpt_device_bytes(ogpt* t) { return t ? t->device_bytes : 0; }
 int32_t ogpt_set_param(ogpt* t, uint64_t index, const float* host) {
   if (!t || index >= t->slots.size() || !host) return OMX_SHAPE;
   const Slot& s = t->slots[index];
+  t->tracked = ogpt::kNone;
   TRY(omx_upload(t->ctx, t->p32, s.offset * 4, host, s.len * 4));
   if (t->p16) TRY(omx_to_bf16(t->ctx, t->p32 + s.offset, static_cast<uint16_t*>(t->p16) + s.offset, s.len));
   return OMX_OK;
@@ -399,6 +407,7 @@ int32_t ogpt_init(ogpt* t, uint64_t seed) {
   }
   TRY(omx_fill_zero(t->ctx, t->m1, t->P * 4));
   TRY(omx_fill_zero(t->ctx, t->m2, t->P * 4));
+  t->tracked = ogpt::kNone;
   t->steps = 0;
   return omx_sync(t->ctx);
 }
@@ -420,6 +429,21 @@ int32_t ogpt_loss_and_grads(ogpt* t, float* loss) {
   return OMX_OK;
 }
 
+// Whether this step's AdamW inputs are known to be below 2^60 (see omx_adamw_step_bounded): the
+// flag of the previous steps, read at the sync point the gradient norm already made, and the norm
+// itself for the gradients. When they are not known to be, the flag starts afresh with this step.
+static int32_t adamw_inputs_bounded(ogpt* t, int need, float norm, int32_t* bounded) {
+  bool flag_clear = false;
+  if (t->tracked >= need) {
+    uint32_t flag = 1;
+    TRY(omx_download(t->ctx, &flag, t->unbounded, 0, 4));
+    flag_clear = flag == 0;
+  }
+  if (!flag_clear) TRY(omx_fill_zero(t->ctx, t->unbounded, 4));
+  *bounded = flag_clear && std::isfinite(norm) && norm < 0x1p60f;
+  return OMX_OK;
+}
+
 int32_t ogpt_step(ogpt* t, const omx_adamw_config* adamw, float grad_clip, float* loss, float* grad_norm) {
   if (!t || !adamw) return OMX_BACKEND;
   TRY(forward(t));
@@ -430,7 +454,11 @@ int32_t ogpt_step(ogpt* t, const omx_adamw_config* adamw, float grad_clip, float
   float norm = 0.0f;
   TRY(omx_clip_grad_norm(t->ctx, grads, lens, 1, grad_clip > 0.0f ? grad_clip : INFINITY, &norm));
   // One AdamW pass over the arena covers every tensor; the bf16 mirror is refreshed in the same pass.
-  TRY(omx_adamw_step(t->ctx, t->p32, t->g32, t->m1, t->m2, t->P, t->steps, adamw, t->p16));
+  int32_t bounded = 0;
+  TRY(adamw_inputs_bounded(t, ogpt::kFull, norm, &bounded));
+  TRY(omx_adamw_step_bounded(t->ctx, t->p32, t->g32, t->m1, t->m2, t->P, t->steps, adamw, t->p16, bounded,
+                             t->unbounded));
+  t->tracked = ogpt::kFull;
   // Sync point 2: sync + the step's one readback (trainer.rs:1031-1046).
   float l = 0.0f;
   TRY(omx_read_scalar_f32(t->ctx, t->loss, &l));
@@ -452,10 +480,13 @@ int32_t ogpt_step_hybrid(ogpt* t, const omx_muon_config* muon, const omx_adamw_c
   float norm = 0.0f;
   TRY(omx_clip_grad_norm(t->ctx, grads, lens, 1, grad_clip > 0.0f ? grad_clip : INFINITY, &norm));
   uint16_t* mirror = static_cast<uint16_t*>(t->p16);
+  int32_t bounded = 0;
+  TRY(adamw_inputs_bounded(t, ogpt::kHybrid, norm, &bounded));
+  t->tracked = ogpt::kHybrid;  // the matrices and their first-moment slots are Muon's from here on
   auto adam = [&](uint64_t first, uint64_t last) -> int32_t {  // slots [first, last] are adjacent in the arena
     const uint64_t at = t->slots[first].offset, n = t->slots[last].offset + t->slots[last].len - at;
-    return omx_adamw_step(t->ctx, t->p32 + at, t->g32 + at, t->m1 + at, t->m2 + at, n, t->steps, adamw,
-                          mirror ? mirror + at : nullptr);
+    return omx_adamw_step_bounded(t->ctx, t->p32 + at, t->g32 + at, t->m1 + at, t->m2 + at, n, t->steps, adamw,
+                                  mirror ? mirror + at : nullptr, bounded, t->unbounded);
   };
   const uint64_t d = t->c.d_model, mlp = t->c.mlp;
   // Matrices of one shape go through Newton-Schulz together: three batched calls per step.

@@ -107,6 +107,36 @@ def test_optimizer_step_matches_cpu_adamw_on_the_same_gradients(be):
     tr.close()
 
 
+def test_steps_with_the_skipped_adamw_check_equal_steps_with_it(be):
+    """The trainer vouches for its arenas once a step has passed over them (omx_adamw_step_bounded);
+    the parameters after five steps are bit for bit those of a trainer that checks every time,
+    across a parameter written from outside in between (which ends the trainer's word until the
+    next checked step). The flag itself is covered with the op, in test_gpu_parity_ops.py."""
+    from ojas_amd.backend import AdamWConfig
+    from ojas_amd.trainer import GptConfig, GptTrainer, synthetic_batch
+
+    cfg = GptConfig(*SMALL, 1)
+    adam = AdamWConfig.nanolab(3e-3, 0.1)
+    ids, targets = synthetic_batch(cfg, 9)
+    results = []
+    for trust in (1, 0):
+        be.set_option("adamw_trust", trust)
+        tr = GptTrainer(be, cfg)
+        params = make_params(tr.param_lens(), cfg.d_model, 5, 0.05)
+        tr.set_params(params)
+        tr.set_batch(ids, targets)
+        losses = [tr.step(adam, 1.0) for _ in range(3)]
+        planted = tr.params()
+        planted[3][7] = 0.5
+        tr.set_params(planted)
+        losses += [tr.step(adam, 1.0) for _ in range(2)]
+        results.append((losses, tr.params()))
+        tr.close()
+    be.set_option("adamw_trust", 1)
+    assert results[0][0] == results[1][0]
+    assert all(np.array_equal(a, b) for a, b in zip(results[0][1], results[1][1]))
+
+
 @pytest.mark.parametrize("bf16", [0, 1])
 def test_hybrid_step_muon_on_matrices_adamw_on_tables_and_norms(be, bf16):
     """BASELINE configs[3]'s optimizer on a small shape: `ogpt_step_hybrid` against the oracle's

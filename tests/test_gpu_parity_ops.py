@@ -308,6 +308,55 @@ def test_adamw_writes_nothing_when_any_value_is_non_finite(be):
     assert np.array_equal(be.download(dm2), m2)
 
 
+def test_adamw_bounded_form_skips_the_check_only_when_nothing_can_overflow(be):
+    """`omx_adamw_step_bounded`: the bits of `omx_adamw_step` in every case; the flag reports stored
+    values at or above 2^60; a caller's word is not taken when the scalars could overflow."""
+    from ojas_amd.backend import NON_FINITE, U32, AdamWConfig, OjasError
+
+    n = 70_001
+    r = orc.SplitMix64(41)
+    p, g, m1 = r.vec(n, 1.0), r.vec(n, 0.1), r.vec(n, 0.01)
+    m2 = np.abs(r.vec(n, 0.01))
+    cfg = AdamWConfig.nanolab(3e-3, 0.1)
+
+    def run(pp, gg, mm1, mm2, step, config, bounded=None):
+        dp, dg, dm1, dm2 = be.upload(pp), be.upload(gg), be.upload(mm1), be.upload(mm2)
+        flag = be.upload(np.zeros(1, np.uint32))
+        if bounded is None:
+            be.adamw_step(dp, dg, dm1, dm2, step, config)
+        else:
+            be.adamw_step_bounded(dp, dg, dm1, dm2, step, config, bounded, flag)
+        fault = None
+        try:
+            be.sync()
+        except OjasError as e:
+            fault = e
+        return be.download(dp), be.download(dm1), be.download(dm2), int(be.download(flag)[0]), fault
+
+    want = run(p, g, m1, m2, 3, cfg)
+    for bounded in (True, False):
+        got = run(p, g, m1, m2, 3, cfg, bounded)
+        assert all(np.array_equal(a, b) for a, b in zip(got[:3], want[:3])) and got[3] == 0 and got[4] is None
+    # A stored value at 2^61: finite, so the update is written; the flag says the next call must check.
+    big = m1.copy()
+    big[17] = 2.0 ** 61
+    want = run(p, g, big, m2, 3, cfg)
+    got = run(p, g, big, m2, 3, cfg, False)
+    assert all(np.array_equal(a, b) for a, b in zip(got[:3], want[:3])) and got[3] == 1 and got[4] is None
+    # A non-finite gradient (the caller sees a non-finite norm, so it does not vouch): refused, nothing
+    # written, and the flag describes the inputs that stay in memory.
+    bad = g.copy()
+    bad[n - 1] = np.nan
+    got = run(p, bad, m1, m2, 3, cfg, False)
+    assert got[4] is not None and got[4].code == NON_FINITE
+    assert np.array_equal(got[0], p) and np.array_equal(got[1], m1) and np.array_equal(got[2], m2) and got[3] == 0
+    # A step size above 2^20: bounded inputs no longer rule out an overflow, so the caller's word is
+    # not enough and the check runs: 1e30 * m / denom overflows and the update is refused.
+    wild = AdamWConfig.nanolab(1e30, 0.0)
+    got = run(p, np.full(n, 3e10, np.float32), m1, m2, 3, wild, True)
+    assert got[4] is not None and got[4].code == NON_FINITE and np.array_equal(got[0], p)
+
+
 def test_adamw_config_refusals(be):
     from ojas_amd.backend import NON_FINITE, OUT_OF_RANGE, AdamWConfig, OjasError
 
