@@ -108,15 +108,40 @@ __global__ __launch_bounds__(OPT_THREADS) void adamw_apply_kernel(float* __restr
 // block in a fixed order (lane-strided, then a tree), so the norm does not
 // depend on scheduling.
 constexpr size_t NORM_BLOCK = 1 << 16;
+__device__ __forceinline__ double sumsq4(const float4& u) {
+  const double a = u.x, b = u.y, c = u.z, d = u.w;
+  return (a * a + b * b) + (c * c + d * d);
+}
 __global__ __launch_bounds__(OPT_THREADS) void sumsq_partial_kernel(const float* __restrict__ x, size_t n,
                                                                     double* __restrict__ partial) {
   __shared__ double red[OPT_THREADS];
   size_t begin = static_cast<size_t>(blockIdx.x) * NORM_BLOCK;
   size_t end = min(n, begin + NORM_BLOCK);
   double acc = 0.0;
-  for (size_t i = begin + threadIdx.x; i < end; i += OPT_THREADS) {
-    double v = static_cast<double>(x[i]);
-    acc += v * v;
+  if ((reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+    // 16-byte loads, four of them in flight per thread; the tail of the last block one by one.
+    const float4* x4 = reinterpret_cast<const float4*>(x);
+    const size_t q_begin = begin / 4, q_end = end / 4;  // NORM_BLOCK is a multiple of 4
+    double a0 = 0.0, a1 = 0.0, a2 = 0.0, a3 = 0.0;
+    size_t i = q_begin + threadIdx.x;
+    for (; i + 3 * OPT_THREADS < q_end; i += 4 * OPT_THREADS) {
+      const float4 u0 = x4[i], u1 = x4[i + OPT_THREADS], u2 = x4[i + 2 * OPT_THREADS], u3 = x4[i + 3 * OPT_THREADS];
+      a0 += sumsq4(u0);
+      a1 += sumsq4(u1);
+      a2 += sumsq4(u2);
+      a3 += sumsq4(u3);
+    }
+    for (; i < q_end; i += OPT_THREADS) a0 += sumsq4(x4[i]);
+    acc = (a0 + a1) + (a2 + a3);
+    for (size_t j = q_end * 4 + threadIdx.x; j < end; j += OPT_THREADS) {
+      const double v = static_cast<double>(x[j]);
+      acc += v * v;
+    }
+  } else {
+    for (size_t i = begin + threadIdx.x; i < end; i += OPT_THREADS) {
+      double v = static_cast<double>(x[i]);
+      acc += v * v;
+    }
   }
   red[threadIdx.x] = acc;
   __syncthreads();

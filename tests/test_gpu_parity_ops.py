@@ -388,6 +388,13 @@ def test_clip_grad_norm(be):
     be.clip_grad_norm(dg, 1e9)
     for got, want in zip(dg, grads):
         assert np.array_equal(be.download(got), want)
+    # A tensor that does not start on a 16-byte boundary (the kernel's one-by-one path).
+    from ojas_amd.backend import F32, DeviceTensor
+
+    base = be.upload(grads[3])
+    view = DeviceTensor(be, base.ptr + 4, (grads[3].size - 1,), F32, owns=False)
+    want = float(np.sqrt(np.sum(grads[3][1:].astype(np.float64) ** 2)))
+    assert abs(be.clip_grad_norm([view], 1e9) - want) <= 1e-6 * want
 
 
 def test_elementwise_ops(be):
