@@ -584,6 +584,11 @@ int32_t omx_set_option(omx_ctx* ctx, const char* name, int64_t value) {
     ctx->gemm_dma_mode = static_cast<int>(value);
     return OMX_OK;
   }
+  if (name && strcmp(name, "ce_fused") == 0) {
+    if (value < 0 || value > 1) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: ce_fused takes 0..1");
+    ctx->ce_fused = static_cast<int>(value);
+    return OMX_OK;
+  }
   if (name && strcmp(name, "adamw_trust") == 0) {
     if (value < 0 || value > 1) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: adamw_trust takes 0..1");
     ctx->adamw_trust = static_cast<int>(value);

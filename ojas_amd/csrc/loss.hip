@@ -98,10 +98,11 @@ __device__ __forceinline__ void ce_store(T* __restrict__ g, unsigned int c, cons
 template <typename T>
 constexpr int ce_vec() { return 16 / static_cast<int>(sizeof(T)); }
 
-// exp for the running sums of a tile. bf16 logits carry 8 bits of mantissa and the bf16 tier's loss
-// gate is 1e-3, so their exponentials take the hardware exp2 (two instructions; about 1e-6
-// relative with the rounding of the scaled argument) instead of expf's full-precision sequence,
-// which made the pass compute-bound at 2.9 TB/s. f32 logits keep expf.
+// exp for the running sums and the gradients of a tile. bf16 logits carry 8 bits of mantissa, the
+// bf16 tier's loss gate is 1e-3 and its gradients are stored in bf16, so their exponentials take
+// the hardware exp2 (two instructions; about 1e-6 relative with the rounding of the scaled
+// argument) instead of expf's full-precision sequence, which made the passes compute-bound
+// (2.9 TB/s for the statistics, 3.4 for statistics and gradients in one). f32 logits keep expf.
 template <typename T>
 __device__ __forceinline__ float ce_exp(float x) {
   if constexpr (sizeof(T) == 2) return __builtin_amdgcn_exp2f(x * 1.4426950408889634f);
@@ -223,10 +224,141 @@ __global__ __launch_bounds__(CE_THREADS) void ce_tile_grad_kernel(const TL* __re
     float v[VEC], out[VEC];
     ce_load<TL, VEC>(r, c, v);
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) out[j] = (c + j == tcol) ? target_grad : expf(v[j] - m) * scale;
+    for (int j = 0; j < VEC; ++j) out[j] = (c + j == tcol) ? target_grad : ce_exp<TL>(v[j] - m) * scale;
     ce_store<TG, VEC>(g, c, out);
   }
 }
+
+// One block per row, for a tile that holds the row's whole vocabulary: the statistics pass and the
+// gradient pass of the two kernels above over ONE read of the logits, which wait in registers in
+// between (MAXV 16-byte packs per thread), gradients written in place. 1024 threads keep that to
+// 32 registers per thread for 65536 bf16 logits, so eight waves per SIMD overlap one row's loads
+// with another's exponentials. Same formulas as ce_tile_stats_kernel (first tile) followed by
+// ce_tile_grad_kernel; the row sum is formed over 1024 partial sums instead of 256, so it agrees
+// with theirs to rounding, not to the bit.
+constexpr int CE_FUSED_THREADS = 1024;
+__device__ __forceinline__ float fused_block_max(float v, float* red) {
+  v = wave_max(v);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  float r = red[0];
+#pragma unroll
+  for (int i = 1; i < CE_FUSED_THREADS / 64; ++i) r = fmaxf(r, red[i]);
+  return r;
+}
+__device__ __forceinline__ float fused_block_sum(float v, float* red) {
+  v = wave_sum(v);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  float r = red[0];
+#pragma unroll
+  for (int i = 1; i < CE_FUSED_THREADS / 64; ++i) r += red[i];
+  return r;
+}
+template <typename T, int MAXV>
+__global__ __launch_bounds__(CE_FUSED_THREADS, 8) void ce_row_fused_kernel(T* __restrict__ tile, size_t ld, size_t row0,
+                                                                  unsigned int ncols,
+                                                                  const unsigned int* __restrict__ targets,
+                                                                  int has_ignore, unsigned int ignore, CeState st,
+                                                                  const unsigned int* __restrict__ valid,
+                                                                  OmxFaultWord* fault, unsigned long long tag) {
+  constexpr int VEC = ce_vec<T>();
+  __shared__ float red[CE_FUSED_THREADS / 64];
+  __shared__ float picked;
+  const size_t local = blockIdx.x, row = row0 + local;
+  T* r = tile + local * ld;
+  const unsigned int target = targets[row];
+  if (threadIdx.x == 0) picked = target < ncols ? 0.0f : st.picked[row];
+  // Every pack of the row, all loads in flight together. Packs past the end re-read the last one
+  // (unconditional loads; they are masked out below).
+  uint4 q[MAXV];
+  const unsigned int last = ncols - VEC;
+#pragma unroll
+  for (int k = 0; k < MAXV; ++k) {
+    const unsigned int c = (threadIdx.x + k * CE_FUSED_THREADS) * VEC;
+    q[k] = *reinterpret_cast<const uint4*>(r + (c < ncols ? c : last));
+  }
+  auto unpack = [](const uint4& w, float (&v)[VEC]) {
+    const unsigned int u[4] = {w.x, w.y, w.z, w.w};
+    if constexpr (sizeof(T) == 4) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] = __uint_as_float(u[j]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v[2 * j] = __uint_as_float(u[j] << 16);
+        v[2 * j + 1] = __uint_as_float(u[j] & 0xffff0000u);
+      }
+    }
+  };
+  float mx = -INFINITY, sum = 0.0f;
+  bool bad = false;
+  __syncthreads();  // `picked` is initialised before its owner overwrites it
+#pragma unroll
+  for (int k = 0; k < MAXV; ++k) {
+    const unsigned int c = (threadIdx.x + k * CE_FUSED_THREADS) * VEC;
+    if (c < ncols) {
+      float v[VEC];
+      unpack(q[k], v);
+      float top = v[0];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        bad |= !dev_finite(v[j]);
+        top = fmaxf(top, v[j]);
+      }
+      if (top > mx) {
+        sum *= ce_exp<T>(mx - top);
+        mx = top;
+      }
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        if (c + j != target) sum += ce_exp<T>(v[j] - mx);
+        else picked = v[j];
+      }
+    }
+  }
+  const float row_max = fused_block_max(mx, red);
+  sum = fused_block_sum(mx == -INFINITY ? 0.0f : sum * expf(mx - row_max), red);
+  if (__syncthreads_or(bad)) {
+    if (threadIdx.x == 0) dev_raise_fault(fault, tag);
+  }
+  const float m = row_max, other = 0.0f + sum * expf(row_max - row_max), p = picked;
+  if (threadIdx.x == 0) {
+    st.max[row] = m;
+    st.other[row] = other;
+    if (target < ncols) st.picked[row] = p;
+  }
+  if (has_ignore && target == ignore) {
+#pragma unroll
+    for (int k = 0; k < MAXV; ++k) {
+      const unsigned int c = (threadIdx.x + k * CE_FUSED_THREADS) * VEC;
+      if (c < ncols) *reinterpret_cast<uint4*>(r + c) = make_uint4(0u, 0u, 0u, 0u);
+    }
+    return;
+  }
+  const float denom = static_cast<float>(*valid);
+  const float total = other + expf(p - m);
+  const bool collapse = (p == m && total == 1.0f && other > 0.0f);
+  const float d = collapse ? 1.0f + other : total;
+  const float target_grad = collapse ? -(other / d) / denom : (expf(p - m) / d) / denom - 1.0f / denom;
+  const float scale = (1.0f / d) / denom;
+#pragma unroll
+  for (int k = 0; k < MAXV; ++k) {
+    const unsigned int c = (threadIdx.x + k * CE_FUSED_THREADS) * VEC;
+    if (c < ncols) {
+      float v[VEC], out[VEC];
+      unpack(q[k], v);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) out[j] = (c + j == target) ? target_grad : ce_exp<T>(v[j] - m) * scale;
+      ce_store<T, VEC>(r, c, out);
+    }
+  }
+}
+constexpr int CE_FUSED_PACKS = 8;  // per thread: rows of up to 65536 bf16 or 32768 f32 logits
 
 // Whether rows of `ld` elements starting at `base` (+ col offset) allow 16-byte accesses of T.
 template <typename T>
@@ -413,11 +545,28 @@ int32_t omx_linear_cross_entropy_mean(omx_ctx* ctx, const void* x, const void* w
   };
   for (uint64_t r0 = 0; r0 < rows; r0 += R) {
     const uint64_t nr = (rows - r0) < R ? (rows - r0) : R;
+    // The whole vocabulary in one tile, with gradients wanted: one kernel reads the logits once.
+    const bool fuse = ctx->ce_fused && one_tile && want_grads && vocab <= static_cast<uint64_t>(CE_FUSED_THREADS) * CE_FUSED_PACKS * (16 / esz) &&
+                      (operand_dtype == OMX_F32 ? ce_vector_ok<float>(tile, vocab, static_cast<unsigned>(vocab))
+                                                : ce_vector_ok<unsigned short>(tile, vocab, static_cast<unsigned>(vocab)));
     // Pass 1: row statistics over every vocabulary tile.
     for (uint64_t c0 = 0; c0 < vocab; c0 += C) {
       const uint64_t nc = (vocab - c0) < C ? (vocab - c0) : C;
       rc = logits_tile(r0, nr, c0, nc);
       if (rc != OMX_OK) return rc;
+      if (fuse) {
+        dim3 grid(static_cast<unsigned>(nr)), block(CE_FUSED_THREADS);
+        if (operand_dtype == OMX_F32)
+          hipLaunchKernelGGL((ce_row_fused_kernel<float, CE_FUSED_PACKS>), grid, block, 0, ctx->stream,
+                             static_cast<float*>(tile), nc, r0, static_cast<unsigned>(nc), tg, has_ignore,
+                             ignore_index, s.st, s.valid, ctx->fault, tag);
+        else
+          hipLaunchKernelGGL((ce_row_fused_kernel<unsigned short, CE_FUSED_PACKS>), grid, block, 0, ctx->stream,
+                             static_cast<unsigned short*>(tile), nc, r0, static_cast<unsigned>(nc), tg, has_ignore,
+                             ignore_index, s.st, s.valid, ctx->fault, tag);
+        OMX_LAUNCH_CHECK(ctx, "ce_row_fused_kernel");
+        continue;
+      }
       if (operand_dtype == OMX_F32)
         launch_stats<float>(ctx, tile, nc, r0, nr, static_cast<unsigned>(c0), static_cast<unsigned>(nc), tg, s.st,
                             c0 == 0, tag);
@@ -434,7 +583,9 @@ int32_t omx_linear_cross_entropy_mean(omx_ctx* ctx, const void* x, const void* w
         rc = logits_tile(r0, nr, c0, nc);
         if (rc != OMX_OK) return rc;
       }
-      if (operand_dtype == OMX_F32)
+      if (fuse) {
+        // the gradients are already in the tile
+      } else if (operand_dtype == OMX_F32)
         launch_grad<float, float>(ctx, tile, tile, nc, nc, r0, nr, static_cast<unsigned>(c0),
                                   static_cast<unsigned>(nc), tg, has_ignore, ignore_index, s.st, s.valid);
       else

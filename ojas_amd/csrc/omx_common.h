@@ -86,6 +86,7 @@ struct omx_ctx {
   int gemm_dma_mode = 1;
   int kv_attention_mode = 0;  // 1: cached attention always takes the LDS-tiled kernel
   int adamw_trust = 1;        // 0: omx_adamw_step_bounded always runs its checking pass
+  int ce_fused = 1;           // 0: linear-CE always takes the separate statistics and gradient kernels
   bool profile_gemm = false;
   struct TimedLaunch {
     hipEvent_t start, stop;

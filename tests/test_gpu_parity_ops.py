@@ -223,7 +223,8 @@ def test_cross_entropy_collapse_row_and_all_ignored(be):
 
 
 @pytest.mark.parametrize("rows,dim,vocab,chunk", [(10, 16, 300, (1024, 8192)), (70, 48, 1000, (32, 256)),
-                                                  (129, 64, 513, (64, 8192)), (33, 24, 97, (7, 40))])
+                                                  (129, 64, 513, (64, 8192)), (33, 24, 97, (7, 40)),
+                                                  (130, 64, 1024, (64, 8192)), (9, 32, 32768, (1024, 32768))])
 def test_linear_cross_entropy_matches_composed_path(be, rows, dim, vocab, chunk):
     print(f"linear_ce {rows} {dim} {vocab} {chunk}", flush=True)
     r = orc.SplitMix64(800 + rows)
@@ -243,6 +244,45 @@ def test_linear_cross_entropy_matches_composed_path(be, rows, dim, vocab, chunk)
     _, g3, w3 = be.linear_cross_entropy_mean(be.upload(x), be.upload(w), be.upload(targets), 2, chunk, (True, False))
     assert w3 is None
     close(be.download(g3), ogx, F32_TOL, "fused gx alone")
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("rows,dim,vocab,chunk_rows", [(300, 64, 50304, 128), (70, 128, 8192, 1024), (40, 64, 8, 16)])
+def test_linear_cross_entropy_one_read_kernel_agrees_with_the_two_kernels(be, bf16, rows, dim, vocab, chunk_rows):
+    """With the whole vocabulary in one tile the statistics and gradient passes run as one kernel
+    over one read of the logits. Same formulas as the two-kernel path (`ce_fused` 0); only the
+    row sum's partial sums are grouped differently, so the two agree to 2e-6 (f32 rounding of a
+    sum of positive terms) and, with bf16 logit gradients, to 1e-4 (the last bit of the row sum
+    flips the bf16 rounding of a few of them), with ignored rows; both are within their gate of
+    the oracle."""
+    from ojas_amd.backend import BF16
+
+    print(f"linear_ce one-read {rows} {dim} {vocab} bf16={bf16}", flush=True)
+    r = orc.SplitMix64(900 + vocab)
+    x = orc.round_bf16(r.vec(rows * dim, 1.0)).reshape(rows, dim)
+    w = orc.round_bf16(r.vec(vocab * dim, 0.3)).reshape(vocab, dim)
+    targets = np.array([r.below(vocab) for _ in range(rows)], np.uint32)
+    targets[::7] = 3
+    up = (lambda a: be.upload(a, BF16)) if bf16 else be.upload
+    got = {}
+    for fused in (1, 0):
+        be.set_option("ce_fused", fused)
+        loss, gx, gw = be.linear_cross_entropy_mean(up(x), up(w), be.upload(targets), 3, (chunk_rows, vocab))
+        got[fused] = (be.download(loss), be.download(gx), be.download(gw))
+    be.set_option("ce_fused", 1)
+    for a, b in zip(got[1], got[0]):
+        assert np.max(np.abs(a.astype(np.float64) - b)) <= (1e-4 if bf16 else 2e-6) * max(np.max(np.abs(b)), 1e-30)
+    oloss, ogx, ogw = orc.linear_cross_entropy_mean(x, w, targets, 3)
+    tol = BF16_TOL if bf16 else F32_TOL
+    assert abs(float(got[1][0][0]) - float(oloss)) <= (1e-3 if bf16 else F32_TOL) * max(1.0, abs(float(oloss)))
+    f32 = lambda a: be_f32(a)
+    close(f32(got[1][1]), ogx, tol, "one-read gx")
+    close(got[1][2], ogw, tol, "one-read gw")
+
+
+def be_f32(a):
+    """Widens a downloaded bf16 bit array; f32 arrays pass through."""
+    return (a.astype(np.uint32) << 16).view(np.float32) if a.dtype == np.uint16 else a
 
 
 SDPA_SHAPES = [([2, 3, 33, 24], 3, None), ([1, 2, 300, 64], 2, None), ([2, 2, 64, 16], 2, None),
