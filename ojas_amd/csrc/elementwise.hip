@@ -76,7 +76,7 @@ __global__ void gelu_fwd_kernel(const T* __restrict__ x, T* __restrict__ y, size
   bool bad = false;
   EW_LOOP(i, n) {
     float v = dev_load<T>(x, i);
-    float r = TANH ? dev_gelu_tanh(v) : dev_gelu_erf(v);
+    float r = dev_gelu_of<T, TANH>(v);
     bad |= !dev_finite(r);
     dev_store<T>(y, i, r);
   }
@@ -88,7 +88,7 @@ __global__ void gelu_bwd_kernel(const T* __restrict__ x, const T* __restrict__ g
   bool bad = false;
   EW_LOOP(i, n) {
     float v = dev_load<T>(x, i);
-    float r = dev_load<T>(gy, i) * (TANH ? dev_gelu_tanh_grad(v) : dev_gelu_erf_grad(v));
+    float r = dev_load<T>(gy, i) * dev_gelu_grad_of<T, TANH>(v);
     bad |= !dev_finite(r);
     dev_store<T>(gx, i, r);
   }

@@ -105,10 +105,10 @@ __device__ __forceinline__ bool gemm_store4_epi(const GemmArgs& g, int split, in
     if (g.epi == OMX_EPI_GELU_FWD) {
       // The activation is taken of the value the pre-activation is stored as.
       const float u0 = dev_round_bf16(x0), u1 = dev_round_bf16(x1), u2 = dev_round_bf16(x2), u3 = dev_round_bf16(x3);
-      const float a0 = g.epi_tanh ? dev_gelu_tanh(u0) : dev_gelu_erf(u0);
-      const float a1 = g.epi_tanh ? dev_gelu_tanh(u1) : dev_gelu_erf(u1);
-      const float a2 = g.epi_tanh ? dev_gelu_tanh(u2) : dev_gelu_erf(u2);
-      const float a3 = g.epi_tanh ? dev_gelu_tanh(u3) : dev_gelu_erf(u3);
+      const float a0 = g.epi_tanh ? dev_gelu_tanh_fast(u0) : dev_gelu_erf_fast(u0);
+      const float a1 = g.epi_tanh ? dev_gelu_tanh_fast(u1) : dev_gelu_erf_fast(u1);
+      const float a2 = g.epi_tanh ? dev_gelu_tanh_fast(u2) : dev_gelu_erf_fast(u2);
+      const float a3 = g.epi_tanh ? dev_gelu_tanh_fast(u3) : dev_gelu_erf_fast(u3);
       unsigned short* ap = g.aux_out + off;
       if (whole) {
         uint2 w;
@@ -139,13 +139,64 @@ __device__ __forceinline__ bool gemm_store4_epi(const GemmArgs& g, int split, in
         if (gcol + 2 < g.N) u2 = dev_bf16_bits_to_f32(ap[2]);
         if (gcol + 3 < g.N) u3 = dev_bf16_bits_to_f32(ap[3]);
       }
-      x0 = dev_round_bf16(x0) * (g.epi_tanh ? dev_gelu_tanh_grad(u0) : dev_gelu_erf_grad(u0));
-      x1 = dev_round_bf16(x1) * (g.epi_tanh ? dev_gelu_tanh_grad(u1) : dev_gelu_erf_grad(u1));
-      x2 = dev_round_bf16(x2) * (g.epi_tanh ? dev_gelu_tanh_grad(u2) : dev_gelu_erf_grad(u2));
-      x3 = dev_round_bf16(x3) * (g.epi_tanh ? dev_gelu_tanh_grad(u3) : dev_gelu_erf_grad(u3));
+      x0 = dev_round_bf16(x0) * (g.epi_tanh ? dev_gelu_tanh_grad_fast(u0) : dev_gelu_erf_grad_fast(u0));
+      x1 = dev_round_bf16(x1) * (g.epi_tanh ? dev_gelu_tanh_grad_fast(u1) : dev_gelu_erf_grad_fast(u1));
+      x2 = dev_round_bf16(x2) * (g.epi_tanh ? dev_gelu_tanh_grad_fast(u2) : dev_gelu_erf_grad_fast(u2));
+      x3 = dev_round_bf16(x3) * (g.epi_tanh ? dev_gelu_tanh_grad_fast(u3) : dev_gelu_erf_grad_fast(u3));
     }
   }
   return gemm_store4(g, split, grow, gcol, x0, x1, x2, x3) || bad;
+}
+
+// The activation epilogue for a 32-row block of a wave's tile that lies wholly inside the output
+// (16-byte stores allowed): `staged` holds the block's f32 values, `pitch` floats per row,
+// PPR 4-column pieces per row. One straight-line body per piece (the form of the activation is
+// a template argument, the bounds are known), all of the backward's pre-activation loads issued
+// ahead of the arithmetic. Returns true when a stored value is non-finite.
+template <int EPI, bool TANH, int PPR>
+__device__ __forceinline__ bool gemm_epilogue_block(const GemmArgs& g, const float* staged, int pitch, int grow0,
+                                                    int gcol0, int lane) {
+  constexpr int ITERS = 32 * PPR / 64;
+  unsigned short* cbase = static_cast<unsigned short*>(g.c);
+  bool bad = false;
+  long off[ITERS];
+  uint2 aux[ITERS];
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int c = lane + it * 64, row = c / PPR, piece = c % PPR;
+    off[it] = static_cast<long>(grow0 + row) * g.ldc + gcol0 + piece * 4;
+    if constexpr (EPI == OMX_EPI_GELU_BWD) aux[it] = *reinterpret_cast<const uint2*>(g.aux_in + off[it]);
+  }
+  auto pack = [](float a, float b) {
+    return static_cast<unsigned int>(dev_f32_to_bf16_bits(a)) | (static_cast<unsigned int>(dev_f32_to_bf16_bits(b)) << 16);
+  };
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int c = lane + it * 64, row = c / PPR, piece = c % PPR;
+    const float4 val = *reinterpret_cast<const float4*>(staged + row * pitch + piece * 4);
+    float x[4] = {val.x, val.y, val.z, val.w};
+    if constexpr (EPI == OMX_EPI_GELU_FWD) {
+      float a[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float u = dev_round_bf16(x[e]);  // the activation is taken of the value the pre-activation is stored as
+        a[e] = TANH ? dev_gelu_tanh_fast(u) : dev_gelu_erf_fast(u);
+        bad |= !(dev_finite(x[e]) && dev_finite(a[e]));
+      }
+      *reinterpret_cast<uint2*>(cbase + off[it]) = make_uint2(pack(x[0], x[1]), pack(x[2], x[3]));
+      *reinterpret_cast<uint2*>(g.aux_out + off[it]) = make_uint2(pack(a[0], a[1]), pack(a[2], a[3]));
+    } else {
+      const float u[4] = {__uint_as_float(aux[it].x << 16), __uint_as_float(aux[it].x & 0xffff0000u),
+                          __uint_as_float(aux[it].y << 16), __uint_as_float(aux[it].y & 0xffff0000u)};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        x[e] = dev_round_bf16(x[e]) * (TANH ? dev_gelu_tanh_grad_fast(u[e]) : dev_gelu_erf_grad_fast(u[e]));
+        bad |= !dev_finite(x[e]);
+      }
+      *reinterpret_cast<uint2*>(cbase + off[it]) = make_uint2(pack(x[0], x[1]), pack(x[2], x[3]));
+    }
+  }
+  return bad;
 }
 
 // bf16 kernel with direct-to-LDS loads and a 256 x 256 (variant 0) or

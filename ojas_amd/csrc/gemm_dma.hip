@@ -34,6 +34,8 @@
 //   * NST LDS stages: the loads of K steps ks+1 .. ks+NST-1 are in flight while step ks is
 //     multiplied; one counted vmcnt wait + barrier per step.
 // Rows past M (or N) are fetched from a clamped valid address and never stored.
+#include <type_traits>
+
 #include "gemm_args.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -133,6 +135,15 @@ constexpr int vmcnt_only(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
 constexpr int dma_waves_per_simd(int waves, int lds_bytes) {
   const int by_lds = 160 * 1024 / lds_bytes, by_waves = 16 / waves;
   return (by_lds < by_waves ? by_lds : by_waves) * waves / 4;
+}
+
+// f(integral_constant<int, I>) for I = BEGIN .. END - 1.
+template <int BEGIN, int END, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (BEGIN < END) {
+    f(std::integral_constant<int, BEGIN>{});
+    static_for<BEGIN + 1, END>(f);
+  }
 }
 
 template <bool A_KM, bool B_KM, int WGM, int WGN, int TM, int TN, int DBK, int NST>
@@ -302,8 +313,10 @@ gemm_dma_kernel(GemmArgs g) {
   static_assert(NW * 32 * CPW * 4 <= NST * STAGE, "staging fits");
   float* cs = reinterpret_cast<float*>(smem) + wave * (32 * CPW);
   bool bad = false;
-#pragma unroll
-  for (int tm = 0; tm < TM; ++tm) {
+  // The row block is a compile-time index (the body is too long for the unroller to take on its
+  // own, and a run-time index would move the accumulators to scratch memory).
+  static_for<0, TM>([&](auto tm_index) {
+    constexpr int tm = decltype(tm_index)::value;
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
@@ -321,6 +334,17 @@ gemm_dma_kernel(GemmArgs g) {
           bad |= gemm_store4(g, split, grow, gcol, val.x, val.y, val.z, val.w);
         }
       }
+    } else if (DBK == 32 && TM * TN <= 4 &&  // the two forms the dispatcher picks by itself
+               g.c_vec != 0 && m0 + (wm * TM + tm) * 32 + 32 <= g.M && n0 + wn * TN * 32 + TN * 32 <= g.N) {
+      // The block lies inside the output: the branch-free form of the activation epilogue.
+      const int grow0 = m0 + (wm * TM + tm) * 32, gcol0 = n0 + wn * TN * 32;
+      if (g.epi == OMX_EPI_GELU_FWD) {
+        bad |= g.epi_tanh ? gemm_epilogue_block<OMX_EPI_GELU_FWD, true, PPR>(g, cs, CPW, grow0, gcol0, lane)
+                          : gemm_epilogue_block<OMX_EPI_GELU_FWD, false, PPR>(g, cs, CPW, grow0, gcol0, lane);
+      } else {
+        bad |= g.epi_tanh ? gemm_epilogue_block<OMX_EPI_GELU_BWD, true, PPR>(g, cs, CPW, grow0, gcol0, lane)
+                          : gemm_epilogue_block<OMX_EPI_GELU_BWD, false, PPR>(g, cs, CPW, grow0, gcol0, lane);
+      }
     } else {
 #pragma unroll 1
       for (int c = lane; c < 32 * PPR; c += 64) {
@@ -334,7 +358,7 @@ gemm_dma_kernel(GemmArgs g) {
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     __builtin_amdgcn_wave_barrier();
-  }
+  });
   if (bad) dev_raise_fault(g.fault, g.tag);
 }
 
