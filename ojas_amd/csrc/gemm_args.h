@@ -199,6 +199,52 @@ __device__ __forceinline__ bool gemm_epilogue_block(const GemmArgs& g, const flo
   return bad;
 }
 
+// The plain store of a 32-row block that lies wholly inside the output, in the same straight-line
+// form. KIND 0: f32 split-K partial; 1: bf16 result; 2: f32 result; 3: f32 result added to the
+// stored one.
+template <int KIND, int PPR>
+__device__ __forceinline__ bool gemm_store_block(const GemmArgs& g, int split, const float* staged, int pitch,
+                                                 int grow0, int gcol0, int lane) {
+  constexpr int ITERS = 32 * PPR / 64;
+  bool bad = false;
+  const long ld = KIND == 0 ? g.N : g.ldc;
+  float* fbase = KIND == 0 ? g.partial + static_cast<long>(split) * g.M * g.N : static_cast<float*>(g.c);
+  unsigned short* hbase = static_cast<unsigned short*>(g.c);
+  float4 old[ITERS];
+  if constexpr (KIND == 3) {
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int c = lane + it * 64, row = c / PPR, piece = c % PPR;
+      old[it] = *reinterpret_cast<const float4*>(fbase + static_cast<long>(grow0 + row) * ld + gcol0 + piece * 4);
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int c = lane + it * 64, row = c / PPR, piece = c % PPR;
+    const long off = static_cast<long>(grow0 + row) * ld + gcol0 + piece * 4;
+    float4 val = *reinterpret_cast<const float4*>(staged + row * pitch + piece * 4);
+    if constexpr (KIND == 3) {
+      val.x += old[it].x;
+      val.y += old[it].y;
+      val.z += old[it].z;
+      val.w += old[it].w;
+    }
+    if constexpr (KIND == 1) {
+      uint2 w;
+      w.x = static_cast<unsigned int>(dev_f32_to_bf16_bits(val.x)) |
+            (static_cast<unsigned int>(dev_f32_to_bf16_bits(val.y)) << 16);
+      w.y = static_cast<unsigned int>(dev_f32_to_bf16_bits(val.z)) |
+            (static_cast<unsigned int>(dev_f32_to_bf16_bits(val.w)) << 16);
+      *reinterpret_cast<uint2*>(hbase + off) = w;
+    } else {
+      *reinterpret_cast<float4*>(fbase + off) = val;
+    }
+    // Partials are checked by the reduce kernel.
+    if constexpr (KIND != 0) bad |= !(dev_finite(val.x) && dev_finite(val.y) && dev_finite(val.z) && dev_finite(val.w));
+  }
+  return bad;
+}
+
 // bf16 kernel with direct-to-LDS loads and a 256 x 256 (variant 0) or
 // 256 x 128 (variant 1) workgroup tile. Needs K % 64 == 0, 16-byte aligned
 // operands, and row counts that are multiples of 8 for k-major operands.

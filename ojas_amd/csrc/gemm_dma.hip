@@ -324,35 +324,39 @@ gemm_dma_kernel(GemmArgs g) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     constexpr int PPR = TN * 8;  // 4-column pieces per row
-    if (g.epi == OMX_EPI_NONE) {
-#pragma unroll
-      for (int c = lane; c < 32 * PPR; c += 64) {
-        const int row = c / PPR, piece = c % PPR;
-        const int grow = m0 + (wm * TM + tm) * 32 + row, gcol = n0 + wn * TN * 32 + piece * 4;
-        if (grow < g.M && gcol < g.N) {
-          const float4 val = *reinterpret_cast<const float4*>(cs + row * CPW + piece * 4);
-          bad |= gemm_store4(g, split, grow, gcol, val.x, val.y, val.z, val.w);
+    // A block that lies wholly inside the output takes a straight-line store loop (compiled for
+    // the two forms the dispatcher picks by itself); edge blocks and the other forms go piece by piece.
+    constexpr bool kFastStores = DBK == 32 && TM * TN <= 4;
+    const int grow0 = m0 + (wm * TM + tm) * 32, gcol0 = n0 + wn * TN * 32;
+    bool stored = false;
+    if constexpr (kFastStores) {
+      const bool interior = grow0 + 32 <= g.M && gcol0 + TN * 32 <= g.N;
+      if (interior && g.epi == OMX_EPI_NONE && (g.splits > 1 ? (g.N & 3) == 0 : g.c_vec != 0)) {
+        if (g.splits > 1) bad |= gemm_store_block<0, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
+        else if (g.c_bf16) bad |= gemm_store_block<1, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
+        else if (!g.accumulate) bad |= gemm_store_block<2, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
+        else bad |= gemm_store_block<3, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
+        stored = true;
+      } else if (interior && g.epi != OMX_EPI_NONE && g.c_vec != 0) {
+        if (g.epi == OMX_EPI_GELU_FWD) {
+          bad |= g.epi_tanh ? gemm_epilogue_block<OMX_EPI_GELU_FWD, true, PPR>(g, cs, CPW, grow0, gcol0, lane)
+                            : gemm_epilogue_block<OMX_EPI_GELU_FWD, false, PPR>(g, cs, CPW, grow0, gcol0, lane);
+        } else {
+          bad |= g.epi_tanh ? gemm_epilogue_block<OMX_EPI_GELU_BWD, true, PPR>(g, cs, CPW, grow0, gcol0, lane)
+                            : gemm_epilogue_block<OMX_EPI_GELU_BWD, false, PPR>(g, cs, CPW, grow0, gcol0, lane);
         }
+        stored = true;
       }
-    } else if (DBK == 32 && TM * TN <= 4 &&  // the two forms the dispatcher picks by itself
-               g.c_vec != 0 && m0 + (wm * TM + tm) * 32 + 32 <= g.M && n0 + wn * TN * 32 + TN * 32 <= g.N) {
-      // The block lies inside the output: the branch-free form of the activation epilogue.
-      const int grow0 = m0 + (wm * TM + tm) * 32, gcol0 = n0 + wn * TN * 32;
-      if (g.epi == OMX_EPI_GELU_FWD) {
-        bad |= g.epi_tanh ? gemm_epilogue_block<OMX_EPI_GELU_FWD, true, PPR>(g, cs, CPW, grow0, gcol0, lane)
-                          : gemm_epilogue_block<OMX_EPI_GELU_FWD, false, PPR>(g, cs, CPW, grow0, gcol0, lane);
-      } else {
-        bad |= g.epi_tanh ? gemm_epilogue_block<OMX_EPI_GELU_BWD, true, PPR>(g, cs, CPW, grow0, gcol0, lane)
-                          : gemm_epilogue_block<OMX_EPI_GELU_BWD, false, PPR>(g, cs, CPW, grow0, gcol0, lane);
-      }
-    } else {
+    }
+    if (!stored) {
 #pragma unroll 1
       for (int c = lane; c < 32 * PPR; c += 64) {
         const int row = c / PPR, piece = c % PPR;
-        const int grow = m0 + (wm * TM + tm) * 32 + row, gcol = n0 + wn * TN * 32 + piece * 4;
+        const int grow = grow0 + row, gcol = gcol0 + piece * 4;
         if (grow < g.M && gcol < g.N) {
           const float4 val = *reinterpret_cast<const float4*>(cs + row * CPW + piece * 4);
-          bad |= gemm_store4_epi(g, split, grow, gcol, val.x, val.y, val.z, val.w);
+          bad |= g.epi == OMX_EPI_NONE ? gemm_store4(g, split, grow, gcol, val.x, val.y, val.z, val.w)
+                                       : gemm_store4_epi(g, split, grow, gcol, val.x, val.y, val.z, val.w);
         }
       }
     }
