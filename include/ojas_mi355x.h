@@ -439,9 +439,11 @@ int32_t omx_set_option(omx_ctx* ctx, const char* name, int64_t value);
 
 /* Benchmark instrumentation (no counterpart in the reference, whose benches
  * time whole ops from the host, bench/README.md:59): while enabled, every
- * launch of the MFMA GEMM kernel is bracketed by two HIP events on the
- * context's stream. The report waits for the stream, sums the launches'
- * durations and their 2*M*N*K FLOPs, and clears the record. */
+ * GEMM product's kernels carry a pair of HIP events on their dispatches (the
+ * begin timestamp of its first kernel, the end timestamp of its last: the
+ * MFMA kernel, or the split-K reduce after it), on the context's stream. The
+ * report waits for the stream, sums the products' durations and their
+ * 2*M*N*K FLOPs, and clears the record. */
 int32_t omx_profile_gemm(omx_ctx* ctx, int32_t enable);
 int32_t omx_profile_gemm_report(omx_ctx* ctx, uint64_t* launches, double* total_ms,
                                 double* total_flops);

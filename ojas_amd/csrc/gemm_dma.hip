@@ -377,7 +377,8 @@ int32_t launch_dma(omx_ctx* ctx, const GemmArgs& g) {
                                      smem));
     granted = true;
   }
-  hipLaunchKernelGGL(kernel, dim3(g.tiles_m * g.tiles_n * g.splits, g.batches), dim3(WGM * WGN * 64), smem, ctx->stream, g);
+  omx_launch_timed(ctx, kernel, dim3(g.tiles_m * g.tiles_n * g.splits, g.batches), dim3(WGM * WGN * 64), smem,
+                   ctx->timing_start, g.splits > 1 ? nullptr : ctx->timing_stop, g);
   OMX_LAUNCH_CHECK(ctx, "gemm_dma_kernel");
   return OMX_OK;
 }

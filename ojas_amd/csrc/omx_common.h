@@ -2,6 +2,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <hip/hip_bf16.h>
 
 #include <cstdarg>
@@ -88,6 +89,9 @@ struct omx_ctx {
   int adamw_trust = 1;        // 0: omx_adamw_step_bounded always runs its checking pass
   int ce_fused = 1;           // 0: linear-CE always takes the separate statistics and gradient kernels
   bool profile_gemm = false;
+  // The events of the product being launched (null when not timing): the first kernel of the
+  // product takes `timing_start`, its last one `timing_stop`.
+  hipEvent_t timing_start = nullptr, timing_stop = nullptr;
   struct TimedLaunch {
     hipEvent_t start, stop;
     double flops;
@@ -95,6 +99,15 @@ struct omx_ctx {
   std::vector<TimedLaunch> timed;
   std::vector<hipEvent_t> event_pool;
 };
+
+// A kernel launch on the context's stream; with events, the dispatch itself carries them (its own
+// begin and end timestamps, no extra packets in the queue).
+template <typename F, typename... Args>
+inline void omx_launch_timed(omx_ctx* ctx, F kernel, dim3 grid, dim3 block, unsigned smem, hipEvent_t start,
+                             hipEvent_t stop, Args... args) {
+  if (start || stop) hipExtLaunchKernelGGL(kernel, grid, block, smem, ctx->stream, start, stop, 0, args...);
+  else hipLaunchKernelGGL(kernel, grid, block, smem, ctx->stream, args...);
+}
 
 int32_t omx_fail(omx_ctx* ctx, omx_status code, const char* fmt, ...);
 int32_t omx_hip_fail(omx_ctx* ctx, hipError_t err, const char* what);
