@@ -197,8 +197,13 @@ __global__ __launch_bounds__(FT, 3) void flash_fwd_kernel(const unsigned short* 
   char* v_rows = smem + FTILE;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lg = lane >> 5;
   const int T = s.time;
-  // Late query blocks see the most keys: schedule them first.
-  const int qb = gridDim.x - 1 - blockIdx.x;
+  // Query block j sees j / 2 + 1 key tiles (causal): a workgroup takes a late block and then
+  // its mirror image from the front, so every workgroup does the same amount of work and the
+  // grid ends without a tail of half-empty compute units.
+  const int q_blocks = (T + 127) / 128;
+  for (int pass = 0; pass < 2; ++pass) {
+  const int qb = pass == 0 ? q_blocks - 1 - static_cast<int>(blockIdx.x) : static_cast<int>(blockIdx.x);
+  if (pass == 1 && qb >= q_blocks - 1 - static_cast<int>(blockIdx.x)) break;
   const long plane = blockIdx.y;
   const int h = static_cast<int>(plane % s.heads), b = static_cast<int>(plane / s.heads);
   const int kvh = h / s.rep;
@@ -304,6 +309,7 @@ __global__ __launch_bounds__(FT, 3) void flash_fwd_kernel(const unsigned short* 
     bad |= store_transposed_acc<TO>(out + o_off, s.o.rs, q_row, T, lg, o, 1.0f / lsum);
   }
   if (bad) dev_raise_fault(fault, tag);
+  }  // pass
 }
 
 // ------------------------------------------------------------------ backward: dK, dV
@@ -319,7 +325,12 @@ __global__ __launch_bounds__(FT, 2) void flash_bwd_dkv_kernel(
   float* del_s = lse_s + 64;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lg = lane >> 5;
   const int T = s.time;
-  const int kb = blockIdx.x;  // early key blocks are seen by the most queries: they come first
+  // Early key blocks are seen by the most queries: a workgroup takes one of them and then its
+  // mirror image from the back (see the forward kernel).
+  const int k_blocks = (T + 127) / 128;
+  for (int pass = 0; pass < 2; ++pass) {
+  const int kb = pass == 0 ? static_cast<int>(blockIdx.x) : k_blocks - 1 - static_cast<int>(blockIdx.x);
+  if (pass == 1 && kb <= static_cast<int>(blockIdx.x)) break;
   const long kv_plane = blockIdx.y;
   const int gidx = static_cast<int>(kv_plane % s.kv_heads), b = static_cast<int>(kv_plane / s.kv_heads);
   const long kv_off = b * s.kv.bs + gidx * s.kv.hs;
@@ -426,6 +437,7 @@ __global__ __launch_bounds__(FT, 2) void flash_bwd_dkv_kernel(
   bad |= store_transposed_acc<TO>(gk + kv_off, s.kv.rs, key_row, T, lg, dk, s.scale);
   bad |= store_transposed_acc<TO>(gv + kv_off, s.kv.rs, key_row, T, lg, dv, 1.0f);
   if (bad) dev_raise_fault(fault, tag);
+  }  // pass
 }
 
 // ------------------------------------------------------------------ backward: dQ
@@ -440,7 +452,11 @@ __global__ __launch_bounds__(FT, 3) void flash_bwd_dq_kernel(
   char* v_rows = smem + FTILE;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lg = lane >> 5;
   const int T = s.time;
-  const int qb = gridDim.x - 1 - blockIdx.x;
+  // A late query block, then its mirror image from the front (see the forward kernel).
+  const int q_blocks = (T + 127) / 128;
+  for (int pass = 0; pass < 2; ++pass) {
+  const int qb = pass == 0 ? q_blocks - 1 - static_cast<int>(blockIdx.x) : static_cast<int>(blockIdx.x);
+  if (pass == 1 && qb >= q_blocks - 1 - static_cast<int>(blockIdx.x)) break;
   const long plane = blockIdx.y;
   const int h = static_cast<int>(plane % s.heads), b = static_cast<int>(plane / s.heads);
   const int kvh = h / s.rep;
@@ -539,6 +555,7 @@ __global__ __launch_bounds__(FT, 3) void flash_bwd_dq_kernel(
   }
   bad |= store_transposed_acc<TO>(gq + b * s.q.bs + h * s.q.hs, s.q.rs, q_row, T, lg, dq, s.scale);
   if (bad) dev_raise_fault(fault, tag);
+  }  // pass
 }
 
 // `strides`: nine element strides (row, head, batch of q; of k / v; of out), or null for
@@ -575,7 +592,8 @@ int32_t omx_flash_sdpa_forward(omx_ctx* ctx, const void* q, const void* k, const
                                const long* strides) {
   if (dim != FD) return omx_fail(ctx, OMX_UNSUPPORTED_HEAD_DIM, "head_dim %llu limit %d", (unsigned long long)dim, FD);
   FlashShape s = make_shape(batch, heads, kv_heads, time, window, scale, strides);
-  dim3 grid(static_cast<unsigned>((time + 127) / 128), static_cast<unsigned>(batch * heads)), block(FT);
+  // Two 128-row query blocks per workgroup (see the kernel).
+  dim3 grid(static_cast<unsigned>(((time + 127) / 128 + 1) / 2), static_cast<unsigned>(batch * heads)), block(FT);
   const unsigned short* qs = static_cast<const unsigned short*>(q);
   const unsigned short* ks = static_cast<const unsigned short*>(k);
   const unsigned short* vs = static_cast<const unsigned short*>(v);
@@ -610,8 +628,9 @@ int32_t omx_flash_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, cons
   const unsigned short* gs = static_cast<const unsigned short*>(gy);
   // dQ first: it also leaves delta = dO . O per row for the dK/dV pass.
   dim3 block(FT);
-  dim3 kv_grid(static_cast<unsigned>((time + 127) / 128), static_cast<unsigned>(batch * kv_heads));
-  dim3 q_grid(static_cast<unsigned>((time + 127) / 128), static_cast<unsigned>(batch * heads));
+  const unsigned pairs = static_cast<unsigned>(((time + 127) / 128 + 1) / 2);  // two 128-row blocks per workgroup
+  dim3 kv_grid(pairs, static_cast<unsigned>(batch * kv_heads));
+  dim3 q_grid(pairs, static_cast<unsigned>(batch * heads));
   if (grad_dtype == OMX_BF16) {
     hipLaunchKernelGGL((flash_bwd_dq_kernel<unsigned short>), q_grid, block, 0, ctx->stream, qs, ks, vs, os, rs, lse,
                        delta, gs, static_cast<unsigned short*>(gq), s, ctx->fault, tag);
