@@ -182,8 +182,9 @@ int32_t backward(ogpt* t) {
   const int32_t AD = t->AD;
   const float eps = 1e-6f;
   // Tied head: loss, grad of the final norm output, and the head's share of the table gradient.
-  // One row block of the whole vocabulary at a time: no logits are recomputed.
-  const uint64_t chunk_rows = N < 8192 ? N : 8192;
+  // One row block of the whole vocabulary at a time: no logits are recomputed. 16384 rows (the
+  // whole GPT-124M batch, a 1.65 GB bf16 tile) measured 0.1 ms per step ahead of two blocks of 8192.
+  const uint64_t chunk_rows = N < 16384 ? N : 16384;
   TRY(omx_linear_cross_entropy_mean(ctx, t->hf, t->w(0), AD, t->targets, N, d, c.vocab, 0, 0, chunk_rows, c.vocab,
                                     t->loss, t->ghf, AD, t->g(0)));
   TRY(omx_rms_norm_backward(ctx, t->x_final, OMX_F32, t->w32(t->nf()), t->ghf, AD, t->gres, OMX_F32, t->g(t->nf()), N, d,
