@@ -185,6 +185,21 @@ __device__ __forceinline__ bool store_transposed_acc_split(unsigned short* __res
   return bad;
 }
 
+// Workgroup -> (pair of row blocks, plane). Workgroups go to the 8 XCDs round-robin by their
+// linear index and every XCD has its own L2, so the `pairs` workgroups of one plane (one head's
+// K and V, or Q and dO) are given indices that are equal modulo 8: they run on one XCD, side by
+// side, and the plane's tiles are fetched into one L2 instead of into several.
+__device__ __forceinline__ void flash_block_of(int pairs, int planes, int* pair, long* plane) {
+  const int id = blockIdx.x;
+  if ((planes & 7) == 0) {
+    *plane = (id & 7) + 8 * (id / (8 * pairs));
+    *pair = (id >> 3) % pairs;
+  } else {
+    *pair = id % pairs;
+    *plane = id / pairs;
+  }
+}
+
 // ------------------------------------------------------------------ forward
 template <typename TO>
 __global__ __launch_bounds__(FT, 3) void flash_fwd_kernel(const unsigned short* __restrict__ q,
@@ -201,10 +216,12 @@ __global__ __launch_bounds__(FT, 3) void flash_fwd_kernel(const unsigned short* 
   // its mirror image from the front, so every workgroup does the same amount of work and the
   // grid ends without a tail of half-empty compute units.
   const int q_blocks = (T + 127) / 128;
+  int pair;
+  long plane;
+  flash_block_of((q_blocks + 1) / 2, s.batch * s.heads, &pair, &plane);
   for (int pass = 0; pass < 2; ++pass) {
-  const int qb = pass == 0 ? q_blocks - 1 - static_cast<int>(blockIdx.x) : static_cast<int>(blockIdx.x);
-  if (pass == 1 && qb >= q_blocks - 1 - static_cast<int>(blockIdx.x)) break;
-  const long plane = blockIdx.y;
+  const int qb = pass == 0 ? q_blocks - 1 - pair : pair;
+  if (pass == 1 && qb >= q_blocks - 1 - pair) break;
   const int h = static_cast<int>(plane % s.heads), b = static_cast<int>(plane / s.heads);
   const int kvh = h / s.rep;
   const unsigned short* qp = q + b * s.q.bs + h * s.q.hs;
@@ -328,10 +345,12 @@ __global__ __launch_bounds__(FT, 2) void flash_bwd_dkv_kernel(
   // Early key blocks are seen by the most queries: a workgroup takes one of them and then its
   // mirror image from the back (see the forward kernel).
   const int k_blocks = (T + 127) / 128;
+  int pair;
+  long kv_plane;
+  flash_block_of((k_blocks + 1) / 2, s.batch * s.kv_heads, &pair, &kv_plane);
   for (int pass = 0; pass < 2; ++pass) {
-  const int kb = pass == 0 ? static_cast<int>(blockIdx.x) : k_blocks - 1 - static_cast<int>(blockIdx.x);
-  if (pass == 1 && kb <= static_cast<int>(blockIdx.x)) break;
-  const long kv_plane = blockIdx.y;
+  const int kb = pass == 0 ? pair : k_blocks - 1 - pair;
+  if (pass == 1 && kb <= pair) break;
   const int gidx = static_cast<int>(kv_plane % s.kv_heads), b = static_cast<int>(kv_plane / s.kv_heads);
   const long kv_off = b * s.kv.bs + gidx * s.kv.hs;
   const unsigned short* kp = k + kv_off;
@@ -454,10 +473,12 @@ __global__ __launch_bounds__(FT, 3) void flash_bwd_dq_kernel(
   const int T = s.time;
   // A late query block, then its mirror image from the front (see the forward kernel).
   const int q_blocks = (T + 127) / 128;
+  int pair;
+  long plane;
+  flash_block_of((q_blocks + 1) / 2, s.batch * s.heads, &pair, &plane);
   for (int pass = 0; pass < 2; ++pass) {
-  const int qb = pass == 0 ? q_blocks - 1 - static_cast<int>(blockIdx.x) : static_cast<int>(blockIdx.x);
-  if (pass == 1 && qb >= q_blocks - 1 - static_cast<int>(blockIdx.x)) break;
-  const long plane = blockIdx.y;
+  const int qb = pass == 0 ? q_blocks - 1 - pair : pair;
+  if (pass == 1 && qb >= q_blocks - 1 - pair) break;
   const int h = static_cast<int>(plane % s.heads), b = static_cast<int>(plane / s.heads);
   const int kvh = h / s.rep;
   const unsigned short* kp = k + b * s.kv.bs + kvh * s.kv.hs;
@@ -593,7 +614,7 @@ int32_t omx_flash_sdpa_forward(omx_ctx* ctx, const void* q, const void* k, const
   if (dim != FD) return omx_fail(ctx, OMX_UNSUPPORTED_HEAD_DIM, "head_dim %llu limit %d", (unsigned long long)dim, FD);
   FlashShape s = make_shape(batch, heads, kv_heads, time, window, scale, strides);
   // Two 128-row query blocks per workgroup (see the kernel).
-  dim3 grid(static_cast<unsigned>(((time + 127) / 128 + 1) / 2), static_cast<unsigned>(batch * heads)), block(FT);
+  dim3 grid(static_cast<unsigned>(((time + 127) / 128 + 1) / 2 * batch * heads)), block(FT);
   const unsigned short* qs = static_cast<const unsigned short*>(q);
   const unsigned short* ks = static_cast<const unsigned short*>(k);
   const unsigned short* vs = static_cast<const unsigned short*>(v);
@@ -629,8 +650,8 @@ int32_t omx_flash_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, cons
   // dQ first: it also leaves delta = dO . O per row for the dK/dV pass.
   dim3 block(FT);
   const unsigned pairs = static_cast<unsigned>(((time + 127) / 128 + 1) / 2);  // two 128-row blocks per workgroup
-  dim3 kv_grid(pairs, static_cast<unsigned>(batch * kv_heads));
-  dim3 q_grid(pairs, static_cast<unsigned>(batch * heads));
+  dim3 kv_grid(pairs * static_cast<unsigned>(batch * kv_heads));
+  dim3 q_grid(pairs * static_cast<unsigned>(batch * heads));
   if (grad_dtype == OMX_BF16) {
     hipLaunchKernelGGL((flash_bwd_dq_kernel<unsigned short>), q_grid, block, 0, ctx->stream, qs, ks, vs, os, rs, lse,
                        delta, gs, static_cast<unsigned short*>(gq), s, ctx->fault, tag);
