@@ -430,11 +430,14 @@ int32_t omx_topk_rows(omx_ctx* ctx, const void* x_f32, uint64_t rows, uint64_t c
 int32_t omx_read_scalar_f32(omx_ctx* ctx, const void* src, float* out);
 
 /* Tuning knobs (no counterpart in the reference). "gemm_dma": 0 = 128x128 GEMM
- * kernel only, 1 = choose by shape (default), 2 / 3 / 4 / 5 = force the 256x256 (64-column
- * steps) / 256x128 (32-column steps) / 256x128 (64-column steps) / 256x256 four-wave
- * direct-to-LDS kernel wherever the operands are eligible. "kv_attention": 0 = choose by head_dim (default),
- * 1 = always the LDS-tiled kernel. Results are within the same tolerances under every
- * setting. */
+ * kernel only, 1 = choose by shape (default), 2 / 3 / 4 / 5 / 6 / 7 = force the 256x256
+ * (64-column steps) / 256x128 (32-column steps) / 256x128 (64-column steps) / 256x256 four-wave /
+ * 128x128 four-wave / 128x192 six-wave (row-major operands only) direct-to-LDS kernel wherever
+ * the operands are eligible. "kv_attention": 0 = choose by head_dim (default), 1 = always the
+ * LDS-tiled kernel. "ce_fused": 0 = the fused linear-cross-entropy always takes its separate
+ * statistics and gradient kernels (default 1: one kernel when a tile holds the whole
+ * vocabulary). "adamw_trust": 0 = omx_adamw_step_bounded always runs its checking pass
+ * (default 1). Results are within the same tolerances under every setting. */
 int32_t omx_set_option(omx_ctx* ctx, const char* name, int64_t value);
 
 /* Benchmark instrumentation (no counterpart in the reference, whose benches

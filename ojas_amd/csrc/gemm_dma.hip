@@ -52,7 +52,9 @@ namespace {
 // 64-bit add per load. ROWS x BK bf16 per step, one wave instruction per KiB.
 template <bool KM, int ROWS, int BK, int NW>  // NW: waves per workgroup
 struct TileLoads {
-  static constexpr int N = ROWS * BK * 2 / 1024 / NW;  // loads per wave per step
+  static constexpr int TOTAL = ROWS * BK * 2 / 1024;  // loads per step
+  static constexpr int N = (TOTAL + NW - 1) / NW;     // per wave; the last one only in waves < TOTAL % NW
+  static constexpr bool EVEN = TOTAL % NW == 0;
   const unsigned short* src[N];
   long step;  // elements between consecutive K steps
 
@@ -60,7 +62,7 @@ struct TileLoads {
                                        int wave, int lane) {
 #pragma unroll
     for (int i = 0; i < N; ++i) {
-      const int q = wave + NW * i;
+      const int q = EVEN || wave + NW * i < TOTAL ? wave + NW * i : 0;  // an unused slot gets a valid address
       if constexpr (!KM) {
         // [row][BK / 8 chunks of 16 bytes], swizzled as frag_offset reads them.
         constexpr int LPR = BK / 8;  // lanes (chunks) per row
@@ -85,6 +87,7 @@ struct TileLoads {
   __device__ __forceinline__ void issue(unsigned tile, int wave) {
 #pragma unroll
     for (int i = 0; i < N; ++i) {
+      if (!EVEN && wave + NW * i >= TOTAL) break;  // wave-uniform
       // Written as assembly: the compiler cannot tell that this asynchronous LDS write targets a
       // stage that is NOT being read, and would otherwise make every LDS read wait for it
       // (vmcnt(0) right after the issue), which serialises the loads with the products.
@@ -155,8 +158,9 @@ gemm_dma_kernel(GemmArgs g) {
   constexpr int NW = WGM * WGN;           // waves per workgroup
   constexpr int LPS = STAGE / 1024 / NW;  // loads per wave per step
   constexpr int KK = DBK / 16;            // MFMA K slabs per step
-  static_assert(NW == 4 || NW == 8, "four or eight waves");
-  static_assert(STAGE % (1024 * NW) == 0, "whole load instructions per wave");
+  static_assert(NW == 4 || NW == 6 || NW == 8, "four, six or eight waves");
+  // Six waves share 16 + 24 loads unevenly; with two stages every wait is for all of a wave's loads.
+  static_assert(STAGE % (1024 * NW) == 0 || NST == 2, "counted waits need the same number of loads in every wave");
   gemm_select_batch(g);
   const unsigned short* __restrict__ A = static_cast<const unsigned short*>(g.a);
   const unsigned short* __restrict__ B = static_cast<const unsigned short*>(g.b);
@@ -326,7 +330,7 @@ gemm_dma_kernel(GemmArgs g) {
     constexpr int PPR = TN * 8;  // 4-column pieces per row
     // A block that lies wholly inside the output takes a straight-line store loop (compiled for
     // the two forms the dispatcher picks by itself); edge blocks and the other forms go piece by piece.
-    constexpr bool kFastStores = DBK == 32 && TM * TN <= 4;
+    constexpr bool kFastStores = (DBK == 32 && TM * TN <= 4) || NW == 6;
     const int grow0 = m0 + (wm * TM + tm) * 32, gcol0 = n0 + wn * TN * 32;
     bool stored = false;
     if constexpr (kFastStores) {
@@ -401,8 +405,8 @@ bool omx_gemm_dma_eligible(const GemmArgs& g, bool a_km, bool b_km) {
 }
 
 void omx_gemm_dma_tile(int variant, int* bm, int* bn) {
-  *bm = variant == 6 ? 128 : 256;
-  *bn = (variant == 0 || variant == 5) ? 256 : 128;
+  *bm = (variant == 6 || variant == 7) ? 128 : 256;
+  *bn = variant == 7 ? 192 : (variant == 0 || variant == 5) ? 256 : 128;
 }
 
 int32_t omx_gemm_dma_launch(omx_ctx* ctx, const GemmArgs& g, bool a_km, bool b_km, int variant) {
@@ -410,5 +414,10 @@ int32_t omx_gemm_dma_launch(omx_ctx* ctx, const GemmArgs& g, bool a_km, bool b_k
   if (variant == 3) return launch_layout<4, 2, 2, 2, 32, 3>(ctx, g, a_km, b_km);
   if (variant == 5) return launch_layout<2, 2, 4, 4, 32, 4>(ctx, g, a_km, b_km);
   if (variant == 6) return launch_layout<2, 2, 2, 2, 32, 3>(ctx, g, a_km, b_km);
+  // 128 x 192 with six waves and 64-column steps: whole 128-byte lines from both operands, two
+  // stages in 80 KiB, so two workgroups still share a compute unit. Row-major operands only.
+  // Behind the option: with two stages a step's loads have one step of lead, which exposes their
+  // latency (K = 768: 557 against 750 TFLOP/s for the 256 x 128 form; 8192^3: 765 against 898).
+  if (variant == 7 && !a_km && !b_km) return launch_dma<false, false, 2, 3, 2, 2, 64, 2>(ctx, g);
   return launch_layout<4, 2, 2, 2, 64, 3>(ctx, g, a_km, b_km);
 }

@@ -1,6 +1,6 @@
 """Every GEMM kernel variant against the oracle: the 128x128 kernel and the
-direct-to-LDS kernels (256x256, 256x128 and 128x128, 32- and 64-column steps, eight and four
-waves),
+direct-to-LDS kernels (256x256, 256x128, 128x128 and 128x192, 32- and 64-column steps, eight, six
+and four waves),
 forced through `omx_set_option`, on
 shapes with ragged M and N (rows past the edge are fetched from a clamped
 address and must never be stored), every operand layout, split-K, bf16 and f32
@@ -29,7 +29,7 @@ SHAPES = [(256, 64, 256), (300, 128, 520), (64, 192, 96), (513, 256, 257), (1024
           (4160, 136, 264)]  # the last: a weight gradient over 4160 rows, split along K
 
 
-@pytest.mark.parametrize("mode", [0, 1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("mode", [0, 1, 2, 3, 4, 5, 6, 7])
 @pytest.mark.parametrize("rows,kin,nout", SHAPES)
 def test_linear_bf16_under_each_kernel(be, mode, rows, kin, nout):
     from ojas_amd.backend import BF16, F32
