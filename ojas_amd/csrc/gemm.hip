@@ -539,6 +539,8 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
   g.epi_tanh = epi ? epi->tanh_form : 0;
   g.aux_in = epi ? static_cast<const unsigned short*>(epi->aux_in) : nullptr;
   g.aux_out = epi ? static_cast<unsigned short*>(epi->aux_out) : nullptr;
+  // The activation's side tensor is accessed with the output's vector width.
+  if (epi && !((!epi->aux_in || aligned16(epi->aux_in)) && (!epi->aux_out || aligned16(epi->aux_out)))) g.c_vec = 0;
   g.fault = ctx->fault;
   g.tag = omx_tag(ctx, fault_op);
   omx_ctx::TimedLaunch timed{};

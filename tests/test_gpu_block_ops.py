@@ -382,6 +382,35 @@ def test_fused_residual_rms_norm_equals_the_separate_ops(be, rows, dim, bf16):
         assert np.array_equal(be.download(gx), be.download(sep))
 
 
+def test_fused_gelu_side_tensor_off_the_vector_boundary(be):
+    """The activation tensor of the fused forward (and the pre-activation of the fused backward)
+    two bytes off a 16-byte boundary: the store pass must fall back to element accesses and give
+    the same bits."""
+    import ctypes as C
+
+    from ojas_amd.backend import BF16, DeviceTensor
+
+    rows, nin, nout = 512, 128, 256
+    r = orc.SplitMix64(77)
+    x = be.upload(orc.round_bf16(r.vec(rows * nin, 1.0)).reshape(rows, nin), BF16)
+    w = be.upload(orc.round_bf16(r.vec(nout * nin, 0.2)).reshape(nout, nin), BF16)
+    gy = be.upload(orc.round_bf16(r.vec(rows * nout, 1.0)).reshape(rows, nout), BF16)
+    u_ref, act_ref = be.linear_gelu_forward(x, w)
+    u = be.empty((rows, nout), BF16)
+    slab = be.zeros((rows * nout + 8,), BF16)
+    act = DeviceTensor(be, slab.ptr + 2, (rows, nout), BF16, owns=False)
+    be._check(be._lib.omx_linear_gelu_forward(be._ctx, be._p(x), be._p(w), C.c_int32(BF16), be._p(u), be._p(act),
+                                              C.c_uint64(rows), C.c_uint64(nin), C.c_uint64(nout), C.c_int32(0)))
+    assert np.array_equal(be.download(u), be.download(u_ref))
+    assert np.array_equal(be.download(act), be.download(act_ref))
+    # Backward: w maps nin -> nout, the fused call computes (gy W) * gelu'(pre) with pre [rows, nin].
+    pre = orc.round_bf16(r.vec(rows * nin, 2.0)).reshape(rows, nin)
+    want = be.download(be.linear_backward_input_gelu(w, gy, be.upload(pre, BF16)))
+    slab2 = be.upload(np.concatenate([np.zeros(1, np.float32), pre.reshape(-1), np.zeros(7, np.float32)]), BF16)
+    pre_view = DeviceTensor(be, slab2.ptr + 2, (rows, nin), BF16, owns=False)
+    assert np.array_equal(be.download(be.linear_backward_input_gelu(w, gy, pre_view)), want)
+
+
 @pytest.mark.parametrize("tanh_form", [False, True])
 @pytest.mark.parametrize("rows,nin,nout", [(64, 64, 128), (300, 128, 520), (1024, 768, 3072), (257, 192, 70)])
 def test_linear_with_fused_gelu_equals_the_separate_ops(be, rows, nin, nout, tanh_form):
