@@ -539,6 +539,43 @@ FLASH_SHAPES = [([1, 1, 1, 64], 1, None), ([1, 2, 17, 64], 2, None), ([2, 3, 64,
                 ([1, 2, 520, 64], 2, 130)]
 
 
+@pytest.mark.parametrize("per_key", [0.002, 0.05, 0.7])
+def test_causal_sdpa_bf16_scores_that_keep_growing(be, per_key):
+    """Scores that rise steadily along the keys (by `per_key` nats per key: 0.13, 3.2 and 45 nats
+    per 64-key tile). The forward moves the reference point of its exponents only when a row's
+    maximum has grown by more than 8 binary orders, so the first case never moves it after the
+    first tile, the second moves it every other tile and the third on every tile; output and
+    log-sum-exp must not care. The gradients (which do not use the forward's reference point)
+    are checked on the first two; on the third the keys reach 90 in magnitude and the bf16
+    rounding of dS against them is past the bf16 gate whatever the kernel."""
+    from ojas_amd.backend import BF16, F32
+
+    b, h, t, d = 1, 2, 512, 64
+    r = orc.SplitMix64(1234)
+    unit = np.zeros(d, np.float32)
+    unit[:8] = 1.0
+    q = orc.round_bf16(np.broadcast_to(unit * 4.0, (b, h, t, d)) + r.vec(b * h * t * d, 0.05).reshape(b, h, t, d))
+    # q . k / 8 = 4 * 8 * ramp / 8 = 4 * ramp
+    ramp = (np.arange(t, dtype=np.float32) * per_key / 4.0).reshape(1, 1, t, 1)
+    k = orc.round_bf16(np.broadcast_to(unit, (b, h, t, d)) * ramp + r.vec(b * h * t * d, 0.05).reshape(b, h, t, d))
+    v = orc.round_bf16(r.vec(b * h * t * d, 1.0).reshape(b, h, t, d))
+    gy = orc.round_bf16(r.vec(b * h * t * d, 1.0).reshape(b, h, t, d))
+    oy, olse = orc.causal_sdpa_forward(q, k, v, 0)
+    dq, dk, dv, dgy = (be.upload(a, BF16) for a in (q, k, v, gy))
+    y32, lse = be.causal_sdpa_forward(dq, dk, dv, None, out_dtype=F32)
+    close(be.download(y32), oy, 1e-2, "growing scores: out")
+    close(be.download(lse), olse, 1e-5, "growing scores: lse")
+    y16, lse16 = be.causal_sdpa_forward(dq, dk, dv, None, out_dtype=BF16)
+    close(be.download_f32(y16), oy, BF16_TOL, "growing scores: out (bf16 store)")
+    if per_key > 0.1:
+        return
+    ogq, ogk, ogv = orc.causal_sdpa_backward(q, k, v, orc.round_bf16(oy), olse, gy, 0)
+    gq, gk, gv = be.causal_sdpa_backward(dq, dk, dv, y16, lse16, dgy, None, grad_dtype=F32)
+    close(be.download(gq), ogq, BF16_TOL, "growing scores: gq")
+    close(be.download(gk), ogk, BF16_TOL, "growing scores: gk")
+    close(be.download(gv), ogv, BF16_TOL, "growing scores: gv")
+
+
 @pytest.mark.parametrize("shape,hkv,window", FLASH_SHAPES)
 def test_causal_sdpa_bf16_mfma(be, shape, hkv, window):
     """head_dim 64 with bf16 operands takes the MFMA flash kernels. Inputs are
