@@ -40,9 +40,10 @@ struct ogpt {
   uint64_t steps = 0;
   // omx_adamw_step_bounded's flag word, and which ranges it has covered since they were last
   // written from outside: nothing, the tables and norms (hybrid steps), or every parameter.
-  void* unbounded = nullptr;
+  void* unbounded = nullptr;  // the word after the loss, so one readback fetches both
   enum Tracked { kNone = 0, kHybrid = 1, kFull = 2 };
   int tracked = kNone;
+  uint32_t flag_seen = 1;  // the flag as the last step's readback saw it (valid while tracked != kNone)
   uint64_t device_bytes = 0;
   std::vector<void*> owned;
 
@@ -305,9 +306,13 @@ int32_t ogpt_create(omx_ctx* ctx, const ogpt_config* config, ogpt** out) {
   CREATE_TRY(alloc_t(t, N, &t->ids));
   CREATE_TRY(alloc_t(t, N, &t->targets));
   CREATE_TRY(alloc_t(t, N, &t->positions));
-  CREATE_TRY(alloc_t(t, 4, &t->loss));
-  CREATE_TRY(alloc(t, 256, &t->unbounded));
-  CREATE_TRY(omx_fill_zero(ctx, t->unbounded, 256));
+  {
+    void* block = nullptr;
+    CREATE_TRY(alloc(t, 256, &block));
+    CREATE_TRY(omx_fill_zero(ctx, block, 256));
+    t->loss = static_cast<float*>(block);
+    t->unbounded = t->loss + 1;
+  }
   {
     std::vector<uint32_t> pos(N);
     for (uint64_t i = 0; i < N; ++i) pos[i] = static_cast<uint32_t>(i % c.ctx);
@@ -431,17 +436,23 @@ int32_t ogpt_loss_and_grads(ogpt* t, float* loss) {
 }
 
 // Whether this step's AdamW inputs are known to be below 2^60 (see omx_adamw_step_bounded): the
-// flag of the previous steps, read at the sync point the gradient norm already made, and the norm
-// itself for the gradients. When they are not known to be, the flag starts afresh with this step.
+// flag of the previous steps, which came back with the last step's loss, and the gradient norm
+// for the gradients. When they are not known to be, the flag starts afresh with this step.
 static int32_t adamw_inputs_bounded(ogpt* t, int need, float norm, int32_t* bounded) {
-  bool flag_clear = false;
-  if (t->tracked >= need) {
-    uint32_t flag = 1;
-    TRY(omx_download(t->ctx, &flag, t->unbounded, 0, 4));
-    flag_clear = flag == 0;
-  }
+  const bool flag_clear = t->tracked >= need && t->flag_seen == 0;
   if (!flag_clear) TRY(omx_fill_zero(t->ctx, t->unbounded, 4));
   *bounded = flag_clear && std::isfinite(norm) && norm < 0x1p60f;
+  return OMX_OK;
+}
+// The step's one readback at its end (trainer.rs:1031-1046): the loss and, behind it, the flag.
+static int32_t read_loss_and_flag(ogpt* t, float* loss) {
+  struct {
+    float loss;
+    uint32_t flag;
+  } back = {0.0f, 1u};
+  TRY(omx_download(t->ctx, &back, t->loss, 0, sizeof(back)));
+  t->flag_seen = back.flag;
+  *loss = back.loss;
   return OMX_OK;
 }
 
@@ -457,12 +468,13 @@ int32_t ogpt_step(ogpt* t, const omx_adamw_config* adamw, float grad_clip, float
   // One AdamW pass over the arena covers every tensor; the bf16 mirror is refreshed in the same pass.
   int32_t bounded = 0;
   TRY(adamw_inputs_bounded(t, ogpt::kFull, norm, &bounded));
+  t->tracked = ogpt::kNone;  // until the readback below has seen this step through
   TRY(omx_adamw_step_bounded(t->ctx, t->p32, t->g32, t->m1, t->m2, t->P, t->steps, adamw, t->p16, bounded,
                              t->unbounded));
-  t->tracked = ogpt::kFull;
-  // Sync point 2: sync + the step's one readback (trainer.rs:1031-1046).
+  // Sync point 2: sync + the step's one readback.
   float l = 0.0f;
-  TRY(omx_read_scalar_f32(t->ctx, t->loss, &l));
+  TRY(read_loss_and_flag(t, &l));
+  t->tracked = ogpt::kFull;
   t->steps += 1;
   if (loss) *loss = l;
   if (grad_norm) *grad_norm = norm;
@@ -483,7 +495,7 @@ int32_t ogpt_step_hybrid(ogpt* t, const omx_muon_config* muon, const omx_adamw_c
   uint16_t* mirror = static_cast<uint16_t*>(t->p16);
   int32_t bounded = 0;
   TRY(adamw_inputs_bounded(t, ogpt::kHybrid, norm, &bounded));
-  t->tracked = ogpt::kHybrid;  // the matrices and their first-moment slots are Muon's from here on
+  t->tracked = ogpt::kNone;  // until the readback at the end has seen this step through
   auto adam = [&](uint64_t first, uint64_t last) -> int32_t {  // slots [first, last] are adjacent in the arena
     const uint64_t at = t->slots[first].offset, n = t->slots[last].offset + t->slots[last].len - at;
     return omx_adamw_step_bounded(t->ctx, t->p32 + at, t->g32 + at, t->m1 + at, t->m2 + at, n, t->steps, adamw,
@@ -517,7 +529,8 @@ int32_t ogpt_step_hybrid(ogpt* t, const omx_muon_config* muon, const omx_adamw_c
     TRY(omx_muon_ns5_step_batched(t->ctx, grp.p.data(), grp.g.data(), grp.m.data(), mirror ? grp.p16.data() : nullptr,
                                   grp.p.size(), grp.rows, grp.cols, muon));
   float l = 0.0f;
-  TRY(omx_read_scalar_f32(t->ctx, t->loss, &l));
+  TRY(read_loss_and_flag(t, &l));
+  t->tracked = ogpt::kHybrid;  // the matrices and their first-moment slots are Muon's from here on
   t->steps += 1;
   if (loss) *loss = l;
   if (grad_norm) *grad_norm = norm;
