@@ -220,112 +220,112 @@ __global__ __launch_bounds__(FT, 3) void flash_fwd_kernel(const unsigned short* 
   long plane;
   flash_block_of((q_blocks + 1) / 2, s.batch * s.heads, &pair, &plane);
   for (int pass = 0; pass < 2; ++pass) {
-  const int qb = pass == 0 ? q_blocks - 1 - pair : pair;
-  if (pass == 1 && qb >= q_blocks - 1 - pair) break;
-  const int h = static_cast<int>(plane % s.heads), b = static_cast<int>(plane / s.heads);
-  const int kvh = h / s.rep;
-  const unsigned short* qp = q + b * s.q.bs + h * s.q.hs;
-  const unsigned short* kp = k + b * s.kv.bs + kvh * s.kv.hs;
-  const unsigned short* vp = v + b * s.kv.bs + kvh * s.kv.hs;
-  const int wave_q0 = qb * 128 + wave * 32;
-  const int q_row = wave_q0 + l32;
-  u32x4 qf[4];
-  row_frags(qp, s.q.rs, q_row, T, lg, qf);
-  floatx16 o[2] = {zero16(), zero16()};
-  float m = -INFINITY, lsum = 0.0f;
-  const float scale_log2 = s.scale * LOG2E;
-  const int block_q0 = qb * 128, block_q1 = min(T - 1, qb * 128 + 127);
-  const int kt_first = s.window > 0 ? max(0, block_q0 + 1 - s.window) / 64 : 0;
-  const int kt_last = block_q1 / 64;
-  // The next tile's global loads are in flight while the current one is multiplied.
-  u32x4 rk[2], rv[2];
-  tile_load(kp, s.kv.rs, kt_first * 64, T, rk);
-  tile_load(vp, s.kv.rs, kt_first * 64, T, rv);
-  for (int kt = kt_first; kt <= kt_last; ++kt) {
-    const int key0 = kt * 64;
-    __syncthreads();  // the previous tile's reads are done
-    tile_store_rows(k_rows, rk);
-    tile_store_rows(v_rows, rv);
-    __syncthreads();
-    if (kt < kt_last) {
-      tile_load(kp, s.kv.rs, key0 + 64, T, rk);
-      tile_load(vp, s.kv.rs, key0 + 64, T, rv);
-    }
-    const bool active = key0 <= wave_q0 + 31 && (s.window == 0 || key0 + 63 + s.window > wave_q0);
-    if (!active) continue;
-    floatx16 sc[2] = {zero16(), zero16()};
+    const int qb = pass == 0 ? q_blocks - 1 - pair : pair;
+    if (pass == 1 && qb >= q_blocks - 1 - pair) break;
+    const int h = static_cast<int>(plane % s.heads), b = static_cast<int>(plane / s.heads);
+    const int kvh = h / s.rep;
+    const unsigned short* qp = q + b * s.q.bs + h * s.q.hs;
+    const unsigned short* kp = k + b * s.kv.bs + kvh * s.kv.hs;
+    const unsigned short* vp = v + b * s.kv.bs + kvh * s.kv.hs;
+    const int wave_q0 = qb * 128 + wave * 32;
+    const int q_row = wave_q0 + l32;
+    u32x4 qf[4];
+    row_frags(qp, s.q.rs, q_row, T, lg, qf);
+    floatx16 o[2] = {zero16(), zero16()};
+    float m = -INFINITY, lsum = 0.0f;
+    const float scale_log2 = s.scale * LOG2E;
+    const int block_q0 = qb * 128, block_q1 = min(T - 1, qb * 128 + 127);
+    const int kt_first = s.window > 0 ? max(0, block_q0 + 1 - s.window) / 64 : 0;
+    const int kt_last = block_q1 / 64;
+    // The next tile's global loads are in flight while the current one is multiplied.
+    u32x4 rk[2], rv[2];
+    tile_load(kp, s.kv.rs, kt_first * 64, T, rk);
+    tile_load(vp, s.kv.rs, kt_first * 64, T, rv);
+    for (int kt = kt_first; kt <= kt_last; ++kt) {
+      const int key0 = kt * 64;
+      __syncthreads();  // the previous tile's reads are done
+      tile_store_rows(k_rows, rk);
+      tile_store_rows(v_rows, rv);
+      __syncthreads();
+      if (kt < kt_last) {
+        tile_load(kp, s.kv.rs, key0 + 64, T, rk);
+        tile_load(vp, s.kv.rs, key0 + 64, T, rv);
+      }
+      const bool active = key0 <= wave_q0 + 31 && (s.window == 0 || key0 + 63 + s.window > wave_q0);
+      if (!active) continue;
+      floatx16 sc[2] = {zero16(), zero16()};
 #pragma unroll
-    for (int sub = 0; sub < 2; ++sub)
+      for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
-      for (int kk = 0; kk < 4; ++kk) sc[sub] = mfma(frag_rows(k_rows, sub, kk, l32, lg), qf[kk], sc[sub]);
-    // Only a tile that crosses the diagonal, the sequence end or the window edge needs the mask
-    // (wave-uniform). `m` is the running maximum of the raw scores; the scale joins inside the fma.
-    if (key0 + 63 > wave_q0 || key0 + 63 >= T || s.window > 0) {
+        for (int kk = 0; kk < 4; ++kk) sc[sub] = mfma(frag_rows(k_rows, sub, kk, l32, lg), qf[kk], sc[sub]);
+      // Only a tile that crosses the diagonal, the sequence end or the window edge needs the mask
+      // (wave-uniform). `m` is the running maximum of the raw scores; the scale joins inside the fma.
+      if (key0 + 63 > wave_q0 || key0 + 63 >= T || s.window > 0) {
+#pragma unroll
+        for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+          for (int vv = 0; vv < 16; ++vv) {
+            const int key = key0 + sub * 32 + acc_row(vv, lg);
+            const bool masked = key > q_row || key >= T || (s.window > 0 && key + s.window <= q_row);
+            sc[sub][vv] = masked ? -INFINITY : sc[sub][vv];
+          }
+      }
+      float tmax = fmaxf(sc[0][0], sc[1][0]);
+#pragma unroll
+      for (int vv = 1; vv < 16; ++vv) tmax = max3(tmax, sc[0][vv], sc[1][vv]);
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      // The reference point of the exponents moves only when a row's maximum grew by more than 8
+      // binary orders (always on a row's first tile, where m is -inf): below that the weights of
+      // this tile are at most 2^8, well inside f32 and bf16, and the accumulators need no rescaling.
+      // The quotient at the end and the log-sum-exp use the same reference, so both stay exact.
+      const bool grow = (tmax - m) * scale_log2 > 8.0f;
+      const float new_m = grow ? tmax : m;
+      const float m_safe = new_m == -INFINITY ? 0.0f : new_m;
+      const float neg_m = -m_safe * scale_log2;
+      float psum = 0.0f;
 #pragma unroll
       for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
         for (int vv = 0; vv < 16; ++vv) {
-          const int key = key0 + sub * 32 + acc_row(vv, lg);
-          const bool masked = key > q_row || key >= T || (s.window > 0 && key + s.window <= q_row);
-          sc[sub][vv] = masked ? -INFINITY : sc[sub][vv];
+          float p = __builtin_amdgcn_exp2f(fmaf(sc[sub][vv], scale_log2, neg_m));
+          sc[sub][vv] = p;
+          psum += p;
+        }
+      psum += __shfl_xor(psum, 32, 64);
+      if (__any(grow)) {
+        // Some row's reference moved: rescale what is accumulated so far (by exactly 1 in the
+        // rows that keep theirs).
+        const float alpha = __builtin_amdgcn_exp2f(fmaf(m, scale_log2, neg_m));
+        lsum *= alpha;
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+          for (int vv = 0; vv < 16; ++vv) o[mt][vv] *= alpha;
+      }
+      lsum += psum;
+      m = new_m;
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+          const u32x4 pb = pack8(sc[sub], c);
+#pragma unroll
+          for (int mt = 0; mt < 2; ++mt) o[mt] = mfma(frag_tr(v_rows, mt, sub, c, lane), pb, o[mt]);
         }
     }
-    float tmax = fmaxf(sc[0][0], sc[1][0]);
-#pragma unroll
-    for (int vv = 1; vv < 16; ++vv) tmax = max3(tmax, sc[0][vv], sc[1][vv]);
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-    // The reference point of the exponents moves only when a row's maximum grew by more than 8
-    // binary orders (always on a row's first tile, where m is -inf): below that the weights of
-    // this tile are at most 2^8, well inside f32 and bf16, and the accumulators need no rescaling.
-    // The quotient at the end and the log-sum-exp use the same reference, so both stay exact.
-    const bool grow = (tmax - m) * scale_log2 > 8.0f;
-    const float new_m = grow ? tmax : m;
-    const float m_safe = new_m == -INFINITY ? 0.0f : new_m;
-    const float neg_m = -m_safe * scale_log2;
-    float psum = 0.0f;
-#pragma unroll
-    for (int sub = 0; sub < 2; ++sub)
-#pragma unroll
-      for (int vv = 0; vv < 16; ++vv) {
-        float p = __builtin_amdgcn_exp2f(fmaf(sc[sub][vv], scale_log2, neg_m));
-        sc[sub][vv] = p;
-        psum += p;
-      }
-    psum += __shfl_xor(psum, 32, 64);
-    if (__any(grow)) {
-      // Some row's reference moved: rescale what is accumulated so far (by exactly 1 in the
-      // rows that keep theirs).
-      const float alpha = __builtin_amdgcn_exp2f(fmaf(m, scale_log2, neg_m));
-      lsum *= alpha;
-#pragma unroll
-      for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-        for (int vv = 0; vv < 16; ++vv) o[mt][vv] *= alpha;
+    bool bad = false;
+    if (q_row < T) {
+      bad |= !(dev_finite(lsum) && lsum > 0.0f);
+      if (lg == 0) lse[plane * T + q_row] = m * s.scale + logf(lsum);
     }
-    lsum += psum;
-    m = new_m;
-#pragma unroll
-    for (int sub = 0; sub < 2; ++sub)
-#pragma unroll
-      for (int c = 0; c < 2; ++c) {
-        const u32x4 pb = pack8(sc[sub], c);
-#pragma unroll
-        for (int mt = 0; mt < 2; ++mt) o[mt] = mfma(frag_tr(v_rows, mt, sub, c, lane), pb, o[mt]);
-      }
-  }
-  bool bad = false;
-  if (q_row < T) {
-    bad |= !(dev_finite(lsum) && lsum > 0.0f);
-    if (lg == 0) lse[plane * T + q_row] = m * s.scale + logf(lsum);
-  }
-  const long o_off = b * s.o.bs + h * s.o.hs;
-  if constexpr (sizeof(TO) == 2) {
-    if (resid) bad |= store_transposed_acc_split(out + o_off, resid + o_off, s.o.rs, q_row, T, lg, o, 1.0f / lsum);
-    else bad |= store_transposed_acc<TO>(out + o_off, s.o.rs, q_row, T, lg, o, 1.0f / lsum);
-  } else {
-    bad |= store_transposed_acc<TO>(out + o_off, s.o.rs, q_row, T, lg, o, 1.0f / lsum);
-  }
-  if (bad) dev_raise_fault(fault, tag);
+    const long o_off = b * s.o.bs + h * s.o.hs;
+    if constexpr (sizeof(TO) == 2) {
+      if (resid) bad |= store_transposed_acc_split(out + o_off, resid + o_off, s.o.rs, q_row, T, lg, o, 1.0f / lsum);
+      else bad |= store_transposed_acc<TO>(out + o_off, s.o.rs, q_row, T, lg, o, 1.0f / lsum);
+    } else {
+      bad |= store_transposed_acc<TO>(out + o_off, s.o.rs, q_row, T, lg, o, 1.0f / lsum);
+    }
+    if (bad) dev_raise_fault(fault, tag);
   }  // pass
 }
 
@@ -349,113 +349,113 @@ __global__ __launch_bounds__(FT, 2) void flash_bwd_dkv_kernel(
   long kv_plane;
   flash_block_of((k_blocks + 1) / 2, s.batch * s.kv_heads, &pair, &kv_plane);
   for (int pass = 0; pass < 2; ++pass) {
-  const int kb = pass == 0 ? pair : k_blocks - 1 - pair;
-  if (pass == 1 && kb <= pair) break;
-  const int gidx = static_cast<int>(kv_plane % s.kv_heads), b = static_cast<int>(kv_plane / s.kv_heads);
-  const long kv_off = b * s.kv.bs + gidx * s.kv.hs;
-  const unsigned short* kp = k + kv_off;
-  const unsigned short* vp = v + kv_off;
-  const int wave_k0 = kb * 128 + wave * 32;
-  const int key_row = wave_k0 + l32;
-  u32x4 kf[4], vf[4];
-  row_frags(kp, s.kv.rs, key_row, T, lg, kf);
-  row_frags(vp, s.kv.rs, key_row, T, lg, vf);
-  floatx16 dk[2] = {zero16(), zero16()}, dv[2] = {zero16(), zero16()};
-  const float scale_log2 = s.scale * LOG2E;
-  const int block_k0 = kb * 128, block_k1 = min(T - 1, kb * 128 + 127);
-  const int qt_first = block_k0 / 64;
-  const int qt_last = (s.window > 0 ? min(T - 1, block_k1 + s.window - 1) : T - 1) / 64;
-  bool bad = false;
-  // One flat loop over (query head of the group, query tile), ascending, so the
-  // next tile's global loads can be in flight while the current one is multiplied.
-  const int nq = qt_last - qt_first + 1;
-  const int steps = s.rep * nq;
-  u32x4 rq[2], rg[2];
-  float row_lse = 0.0f, row_del = 0.0f;
-  // (head of the group, query tile) of the tile being fetched / being multiplied.
-  int fetch_r = 0, fetch_qt = qt_first, cur_qt = qt_first;
-  auto fetch = [&]() {
-    const int r = fetch_r, q0 = fetch_qt * 64;
-    if (++fetch_qt > qt_last) {
-      fetch_qt = qt_first;
-      ++fetch_r;
-    }
-    const long q_plane = static_cast<long>(b) * s.heads + static_cast<long>(gidx) * s.rep + r;
-    const long head = static_cast<long>(gidx) * s.rep + r;
-    tile_load(q + b * s.q.bs + head * s.q.hs, s.q.rs, q0, T, rq);
-    tile_load(gy + b * s.o.bs + head * s.o.hs, s.o.rs, q0, T, rg);
-    row_lse = 0.0f;
-    row_del = 0.0f;
-    if (threadIdx.x < 64 && q0 + static_cast<int>(threadIdx.x) < T) {
-      row_lse = lse[q_plane * T + q0 + threadIdx.x];
-      row_del = delta[q_plane * T + q0 + threadIdx.x];
-      bad |= !(dev_finite(row_lse) && dev_finite(row_del));
-    }
-  };
-  fetch();
-  for (int idx = 0; idx < steps; ++idx) {
-    {
-      const int q0 = cur_qt * 64;
-      if (++cur_qt > qt_last) cur_qt = qt_first;
-      __syncthreads();
-      tile_store_rows(q_rows, rq);
-      tile_store_rows(g_rows, rg);
-      if (threadIdx.x < 64) {
-        lse_s[threadIdx.x] = row_lse * LOG2E;
-        del_s[threadIdx.x] = row_del;
+    const int kb = pass == 0 ? pair : k_blocks - 1 - pair;
+    if (pass == 1 && kb <= pair) break;
+    const int gidx = static_cast<int>(kv_plane % s.kv_heads), b = static_cast<int>(kv_plane / s.kv_heads);
+    const long kv_off = b * s.kv.bs + gidx * s.kv.hs;
+    const unsigned short* kp = k + kv_off;
+    const unsigned short* vp = v + kv_off;
+    const int wave_k0 = kb * 128 + wave * 32;
+    const int key_row = wave_k0 + l32;
+    u32x4 kf[4], vf[4];
+    row_frags(kp, s.kv.rs, key_row, T, lg, kf);
+    row_frags(vp, s.kv.rs, key_row, T, lg, vf);
+    floatx16 dk[2] = {zero16(), zero16()}, dv[2] = {zero16(), zero16()};
+    const float scale_log2 = s.scale * LOG2E;
+    const int block_k0 = kb * 128, block_k1 = min(T - 1, kb * 128 + 127);
+    const int qt_first = block_k0 / 64;
+    const int qt_last = (s.window > 0 ? min(T - 1, block_k1 + s.window - 1) : T - 1) / 64;
+    bool bad = false;
+    // One flat loop over (query head of the group, query tile), ascending, so the
+    // next tile's global loads can be in flight while the current one is multiplied.
+    const int nq = qt_last - qt_first + 1;
+    const int steps = s.rep * nq;
+    u32x4 rq[2], rg[2];
+    float row_lse = 0.0f, row_del = 0.0f;
+    // (head of the group, query tile) of the tile being fetched / being multiplied.
+    int fetch_r = 0, fetch_qt = qt_first, cur_qt = qt_first;
+    auto fetch = [&]() {
+      const int r = fetch_r, q0 = fetch_qt * 64;
+      if (++fetch_qt > qt_last) {
+        fetch_qt = qt_first;
+        ++fetch_r;
       }
-      __syncthreads();
-      if (idx + 1 < steps) fetch();
-      const bool active = q0 + 63 >= wave_k0 && (s.window == 0 || q0 < wave_k0 + 31 + s.window);
-      if (!active) continue;
-      // Wave-uniform: a tile whose queries all come after the wave's keys and end inside the sequence has no mask.
-      const bool needs_mask = q0 < wave_k0 + 31 || q0 + 63 >= T || s.window > 0;
-#pragma unroll
-      for (int sub = 0; sub < 2; ++sub) {
-        floatx16 sc = zero16(), dp = zero16();
-#pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-          sc = mfma(frag_rows(q_rows, sub, kk, l32, lg), kf[kk], sc);
-          dp = mfma(frag_rows(g_rows, sub, kk, l32, lg), vf[kk], dp);
+      const long q_plane = static_cast<long>(b) * s.heads + static_cast<long>(gidx) * s.rep + r;
+      const long head = static_cast<long>(gidx) * s.rep + r;
+      tile_load(q + b * s.q.bs + head * s.q.hs, s.q.rs, q0, T, rq);
+      tile_load(gy + b * s.o.bs + head * s.o.hs, s.o.rs, q0, T, rg);
+      row_lse = 0.0f;
+      row_del = 0.0f;
+      if (threadIdx.x < 64 && q0 + static_cast<int>(threadIdx.x) < T) {
+        row_lse = lse[q_plane * T + q0 + threadIdx.x];
+        row_del = delta[q_plane * T + q0 + threadIdx.x];
+        bad |= !(dev_finite(row_lse) && dev_finite(row_del));
+      }
+    };
+    fetch();
+    for (int idx = 0; idx < steps; ++idx) {
+      {
+        const int q0 = cur_qt * 64;
+        if (++cur_qt > qt_last) cur_qt = qt_first;
+        __syncthreads();
+        tile_store_rows(q_rows, rq);
+        tile_store_rows(g_rows, rg);
+        if (threadIdx.x < 64) {
+          lse_s[threadIdx.x] = row_lse * LOG2E;
+          del_s[threadIdx.x] = row_del;
         }
-        if (needs_mask) {
+        __syncthreads();
+        if (idx + 1 < steps) fetch();
+        const bool active = q0 + 63 >= wave_k0 && (s.window == 0 || q0 < wave_k0 + 31 + s.window);
+        if (!active) continue;
+        // Wave-uniform: a tile whose queries all come after the wave's keys and end inside the sequence has no mask.
+        const bool needs_mask = q0 < wave_k0 + 31 || q0 + 63 >= T || s.window > 0;
 #pragma unroll
-          for (int vv = 0; vv < 16; ++vv) {
-            const int qi = q0 + sub * 32 + acc_row(vv, lg);
-            const bool masked =
-                key_row > qi || qi >= T || key_row >= T || (s.window > 0 && key_row + s.window <= qi);
-            sc[vv] = masked ? -INFINITY : sc[vv];
+        for (int sub = 0; sub < 2; ++sub) {
+          floatx16 sc = zero16(), dp = zero16();
+#pragma unroll
+          for (int kk = 0; kk < 4; ++kk) {
+            sc = mfma(frag_rows(q_rows, sub, kk, l32, lg), kf[kk], sc);
+            dp = mfma(frag_rows(g_rows, sub, kk, l32, lg), vf[kk], dp);
           }
-        }
-        // P = 2^(s * scale * log2e - lse * log2e); dS / scale = P (dP - delta): the scale joins dK at the end.
+          if (needs_mask) {
 #pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-          const float4 l4 = *reinterpret_cast<const float4*>(lse_s + sub * 32 + 8 * q4 + 4 * lg);
-          const float4 d4 = *reinterpret_cast<const float4*>(del_s + sub * 32 + 8 * q4 + 4 * lg);
-          const float lv[4] = {l4.x, l4.y, l4.z, l4.w}, dl[4] = {d4.x, d4.y, d4.z, d4.w};
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const int vv = 4 * q4 + j;
-            const float p = __builtin_amdgcn_exp2f(fmaf(sc[vv], scale_log2, -lv[j]));
-            dp[vv] = p * (dp[vv] - dl[j]);
-            sc[vv] = p;
+            for (int vv = 0; vv < 16; ++vv) {
+              const int qi = q0 + sub * 32 + acc_row(vv, lg);
+              const bool masked =
+                  key_row > qi || qi >= T || key_row >= T || (s.window > 0 && key_row + s.window <= qi);
+              sc[vv] = masked ? -INFINITY : sc[vv];
+            }
           }
-        }
+          // P = 2^(s * scale * log2e - lse * log2e); dS / scale = P (dP - delta): the scale joins dK at the end.
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
-          const u32x4 pb = pack8(sc, c), dsb = pack8(dp, c);
+          for (int q4 = 0; q4 < 4; ++q4) {
+            const float4 l4 = *reinterpret_cast<const float4*>(lse_s + sub * 32 + 8 * q4 + 4 * lg);
+            const float4 d4 = *reinterpret_cast<const float4*>(del_s + sub * 32 + 8 * q4 + 4 * lg);
+            const float lv[4] = {l4.x, l4.y, l4.z, l4.w}, dl[4] = {d4.x, d4.y, d4.z, d4.w};
 #pragma unroll
-          for (int mt = 0; mt < 2; ++mt) {
-            dv[mt] = mfma(frag_tr(g_rows, mt, sub, c, lane), pb, dv[mt]);
-            dk[mt] = mfma(frag_tr(q_rows, mt, sub, c, lane), dsb, dk[mt]);
+            for (int j = 0; j < 4; ++j) {
+              const int vv = 4 * q4 + j;
+              const float p = __builtin_amdgcn_exp2f(fmaf(sc[vv], scale_log2, -lv[j]));
+              dp[vv] = p * (dp[vv] - dl[j]);
+              sc[vv] = p;
+            }
+          }
+#pragma unroll
+          for (int c = 0; c < 2; ++c) {
+            const u32x4 pb = pack8(sc, c), dsb = pack8(dp, c);
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt) {
+              dv[mt] = mfma(frag_tr(g_rows, mt, sub, c, lane), pb, dv[mt]);
+              dk[mt] = mfma(frag_tr(q_rows, mt, sub, c, lane), dsb, dk[mt]);
+            }
           }
         }
       }
     }
-  }
-  bad |= store_transposed_acc<TO>(gk + kv_off, s.kv.rs, key_row, T, lg, dk, s.scale);
-  bad |= store_transposed_acc<TO>(gv + kv_off, s.kv.rs, key_row, T, lg, dv, 1.0f);
-  if (bad) dev_raise_fault(fault, tag);
+    bad |= store_transposed_acc<TO>(gk + kv_off, s.kv.rs, key_row, T, lg, dk, s.scale);
+    bad |= store_transposed_acc<TO>(gv + kv_off, s.kv.rs, key_row, T, lg, dv, 1.0f);
+    if (bad) dev_raise_fault(fault, tag);
   }  // pass
 }
 
@@ -477,105 +477,105 @@ __global__ __launch_bounds__(FT, 3) void flash_bwd_dq_kernel(
   long plane;
   flash_block_of((q_blocks + 1) / 2, s.batch * s.heads, &pair, &plane);
   for (int pass = 0; pass < 2; ++pass) {
-  const int qb = pass == 0 ? q_blocks - 1 - pair : pair;
-  if (pass == 1 && qb >= q_blocks - 1 - pair) break;
-  const int h = static_cast<int>(plane % s.heads), b = static_cast<int>(plane / s.heads);
-  const int kvh = h / s.rep;
-  const unsigned short* kp = k + b * s.kv.bs + kvh * s.kv.hs;
-  const unsigned short* vp = v + b * s.kv.bs + kvh * s.kv.hs;
-  const int wave_q0 = qb * 128 + wave * 32;
-  const int q_row = wave_q0 + l32;
-  u32x4 qf[4], gf[4];
-  row_frags(q + b * s.q.bs + h * s.q.hs, s.q.rs, q_row, T, lg, qf);
-  row_frags(gy + b * s.o.bs + h * s.o.hs, s.o.rs, q_row, T, lg, gf);
-  // delta = dO . O of this lane's row: each half-wave holds half of the row's 64 values. The
-  // dK/dV pass, launched after this one, reads it back from `delta`. dS = P (dP - delta) sums to
-  // zero along a row only as far as delta matches sum_j P dP: taken from the bf16 output alone it
-  // is off by 2^-9 of |dO| |O|, which a component shared by all value rows (and by all key rows,
-  // in dQ = dS K) turns into a multiple of the gradient itself. With the saved rounding residual
-  // of the output the mismatch drops to 2^-17.
-  float row_del = 0.0f;
-  {
-    auto dot_rows = [&](const unsigned short* plane) {
-      u32x4 of[4];
-      row_frags(plane + b * s.o.bs + h * s.o.hs, s.o.rs, q_row, T, lg, of);
-      float sum = 0.0f;
+    const int qb = pass == 0 ? q_blocks - 1 - pair : pair;
+    if (pass == 1 && qb >= q_blocks - 1 - pair) break;
+    const int h = static_cast<int>(plane % s.heads), b = static_cast<int>(plane / s.heads);
+    const int kvh = h / s.rep;
+    const unsigned short* kp = k + b * s.kv.bs + kvh * s.kv.hs;
+    const unsigned short* vp = v + b * s.kv.bs + kvh * s.kv.hs;
+    const int wave_q0 = qb * 128 + wave * 32;
+    const int q_row = wave_q0 + l32;
+    u32x4 qf[4], gf[4];
+    row_frags(q + b * s.q.bs + h * s.q.hs, s.q.rs, q_row, T, lg, qf);
+    row_frags(gy + b * s.o.bs + h * s.o.hs, s.o.rs, q_row, T, lg, gf);
+    // delta = dO . O of this lane's row: each half-wave holds half of the row's 64 values. The
+    // dK/dV pass, launched after this one, reads it back from `delta`. dS = P (dP - delta) sums to
+    // zero along a row only as far as delta matches sum_j P dP: taken from the bf16 output alone it
+    // is off by 2^-9 of |dO| |O|, which a component shared by all value rows (and by all key rows,
+    // in dQ = dS K) turns into a multiple of the gradient itself. With the saved rounding residual
+    // of the output the mismatch drops to 2^-17.
+    float row_del = 0.0f;
+    {
+      auto dot_rows = [&](const unsigned short* plane) {
+        u32x4 of[4];
+        row_frags(plane + b * s.o.bs + h * s.o.hs, s.o.rs, q_row, T, lg, of);
+        float sum = 0.0f;
 #pragma unroll
-      for (int kk = 0; kk < 4; ++kk) {
-        const unsigned int gw[4] = {gf[kk].x, gf[kk].y, gf[kk].z, gf[kk].w};
-        const unsigned int ow[4] = {of[kk].x, of[kk].y, of[kk].z, of[kk].w};
+        for (int kk = 0; kk < 4; ++kk) {
+          const unsigned int gw[4] = {gf[kk].x, gf[kk].y, gf[kk].z, gf[kk].w};
+          const unsigned int ow[4] = {of[kk].x, of[kk].y, of[kk].z, of[kk].w};
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-          sum += __uint_as_float(gw[w] << 16) * __uint_as_float(ow[w] << 16);
-          sum += __uint_as_float(gw[w] & 0xffff0000u) * __uint_as_float(ow[w] & 0xffff0000u);
+          for (int w = 0; w < 4; ++w) {
+            sum += __uint_as_float(gw[w] << 16) * __uint_as_float(ow[w] << 16);
+            sum += __uint_as_float(gw[w] & 0xffff0000u) * __uint_as_float(ow[w] & 0xffff0000u);
+          }
         }
-      }
-      return sum;
-    };
-    row_del = dot_rows(out);
-    if (resid) row_del += dot_rows(resid);
-    row_del += __shfl_xor(row_del, 32, 64);
-  }
-  float row_lse = 0.0f;
-  bool bad = false;
-  if (q_row < T) {
-    row_lse = lse[plane * T + q_row];
-    if (lg == 0) delta[plane * T + q_row] = row_del;
-    bad |= !(dev_finite(row_lse) && dev_finite(row_del));
-  }
-  const float neg_lse = -row_lse * LOG2E;
-  floatx16 dq[2] = {zero16(), zero16()};
-  const float scale_log2 = s.scale * LOG2E;
-  const int block_q0 = qb * 128, block_q1 = min(T - 1, qb * 128 + 127);
-  const int kt_first = s.window > 0 ? max(0, block_q0 + 1 - s.window) / 64 : 0;
-  const int kt_last = block_q1 / 64;
-  u32x4 rk[2], rv[2];
-  tile_load(kp, s.kv.rs, kt_first * 64, T, rk);
-  tile_load(vp, s.kv.rs, kt_first * 64, T, rv);
-  for (int kt = kt_first; kt <= kt_last; ++kt) {
-    const int key0 = kt * 64;
-    __syncthreads();
-    tile_store_rows(k_rows, rk);
-    tile_store_rows(v_rows, rv);
-    __syncthreads();
-    if (kt < kt_last) {
-      tile_load(kp, s.kv.rs, key0 + 64, T, rk);
-      tile_load(vp, s.kv.rs, key0 + 64, T, rv);
+        return sum;
+      };
+      row_del = dot_rows(out);
+      if (resid) row_del += dot_rows(resid);
+      row_del += __shfl_xor(row_del, 32, 64);
     }
-    const bool active = key0 <= wave_q0 + 31 && (s.window == 0 || key0 + 63 + s.window > wave_q0);
-    if (!active) continue;
-    const bool needs_mask = key0 + 63 > wave_q0 || key0 + 63 >= T || s.window > 0;
-#pragma unroll
-    for (int sub = 0; sub < 2; ++sub) {
-      floatx16 sc = zero16(), dp = zero16();
-#pragma unroll
-      for (int kk = 0; kk < 4; ++kk) {
-        sc = mfma(frag_rows(k_rows, sub, kk, l32, lg), qf[kk], sc);
-        dp = mfma(frag_rows(v_rows, sub, kk, l32, lg), gf[kk], dp);
+    float row_lse = 0.0f;
+    bool bad = false;
+    if (q_row < T) {
+      row_lse = lse[plane * T + q_row];
+      if (lg == 0) delta[plane * T + q_row] = row_del;
+      bad |= !(dev_finite(row_lse) && dev_finite(row_del));
+    }
+    const float neg_lse = -row_lse * LOG2E;
+    floatx16 dq[2] = {zero16(), zero16()};
+    const float scale_log2 = s.scale * LOG2E;
+    const int block_q0 = qb * 128, block_q1 = min(T - 1, qb * 128 + 127);
+    const int kt_first = s.window > 0 ? max(0, block_q0 + 1 - s.window) / 64 : 0;
+    const int kt_last = block_q1 / 64;
+    u32x4 rk[2], rv[2];
+    tile_load(kp, s.kv.rs, kt_first * 64, T, rk);
+    tile_load(vp, s.kv.rs, kt_first * 64, T, rv);
+    for (int kt = kt_first; kt <= kt_last; ++kt) {
+      const int key0 = kt * 64;
+      __syncthreads();
+      tile_store_rows(k_rows, rk);
+      tile_store_rows(v_rows, rv);
+      __syncthreads();
+      if (kt < kt_last) {
+        tile_load(kp, s.kv.rs, key0 + 64, T, rk);
+        tile_load(vp, s.kv.rs, key0 + 64, T, rv);
       }
-      if (needs_mask) {
+      const bool active = key0 <= wave_q0 + 31 && (s.window == 0 || key0 + 63 + s.window > wave_q0);
+      if (!active) continue;
+      const bool needs_mask = key0 + 63 > wave_q0 || key0 + 63 >= T || s.window > 0;
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub) {
+        floatx16 sc = zero16(), dp = zero16();
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+          sc = mfma(frag_rows(k_rows, sub, kk, l32, lg), qf[kk], sc);
+          dp = mfma(frag_rows(v_rows, sub, kk, l32, lg), gf[kk], dp);
+        }
+        if (needs_mask) {
+#pragma unroll
+          for (int vv = 0; vv < 16; ++vv) {
+            const int key = key0 + sub * 32 + acc_row(vv, lg);
+            const bool masked = key > q_row || key >= T || q_row >= T || (s.window > 0 && key + s.window <= q_row);
+            sc[vv] = masked ? -INFINITY : sc[vv];
+          }
+        }
 #pragma unroll
         for (int vv = 0; vv < 16; ++vv) {
-          const int key = key0 + sub * 32 + acc_row(vv, lg);
-          const bool masked = key > q_row || key >= T || q_row >= T || (s.window > 0 && key + s.window <= q_row);
-          sc[vv] = masked ? -INFINITY : sc[vv];
+          const float p = __builtin_amdgcn_exp2f(fmaf(sc[vv], scale_log2, neg_lse));
+          dp[vv] = p * (dp[vv] - row_del);  // dS / scale: the scale joins dQ at the end
+        }
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+          const u32x4 dsb = pack8(dp, c);
+#pragma unroll
+          for (int mt = 0; mt < 2; ++mt) dq[mt] = mfma(frag_tr(k_rows, mt, sub, c, lane), dsb, dq[mt]);
         }
       }
-#pragma unroll
-      for (int vv = 0; vv < 16; ++vv) {
-        const float p = __builtin_amdgcn_exp2f(fmaf(sc[vv], scale_log2, neg_lse));
-        dp[vv] = p * (dp[vv] - row_del);  // dS / scale: the scale joins dQ at the end
-      }
-#pragma unroll
-      for (int c = 0; c < 2; ++c) {
-        const u32x4 dsb = pack8(dp, c);
-#pragma unroll
-        for (int mt = 0; mt < 2; ++mt) dq[mt] = mfma(frag_tr(k_rows, mt, sub, c, lane), dsb, dq[mt]);
-      }
     }
-  }
-  bad |= store_transposed_acc<TO>(gq + b * s.q.bs + h * s.q.hs, s.q.rs, q_row, T, lg, dq, s.scale);
-  if (bad) dev_raise_fault(fault, tag);
+    bad |= store_transposed_acc<TO>(gq + b * s.q.bs + h * s.q.hs, s.q.rs, q_row, T, lg, dq, s.scale);
+    if (bad) dev_raise_fault(fault, tag);
   }  // pass
 }
 
