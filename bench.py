@@ -28,6 +28,7 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, vendor figure
+F32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, vendor figure
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor figure
 # HBM bytes per GEMM op (MFMA kernel + split-K reduce) on the gpt124m workload, averaged over the
 # step's 147 GEMM ops: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by what the same
@@ -59,7 +60,8 @@ def cpu_baseline(cfg, threads: int):
     dt = time.perf_counter() - t0
     tokens = sample.batch * sample.ctx
     return {"value": tokens / dt, "unit": "tokens/s", "cores": threads, "kind": "port",
-            "sample": f"same 124M-shape model, one step on 1x{sample.ctx} tokens in f32 Exact arithmetic "
+            "sample": f"same model (L{sample.layers} d{sample.d_model} vocab{sample.vocab}), one step on "
+                      f"1x{sample.ctx} tokens in f32 Exact arithmetic "
                       f"({dt:.1f} s), scaled per token; C++ restatement of ojas-cpu, not the Rust binary"}
 
 
@@ -180,8 +182,11 @@ def main() -> int:
     value = tokens * args.steps / dt
     flops = step_flops(cfg)
     achieved = gemm_flops.value / (gemm_ms.value * 1e-3) / 1e12 if gemm_ms.value > 0 else 0.0
+    gemm_peak = BF16_MFMA_PEAK_TFLOPS if cfg.bf16 else F32_MFMA_PEAK_TFLOPS
     out = {
-        "metric": "train tokens/s on 1 MI355X (GPT-124M bf16 AdamW step); % bf16 MFMA peak" if args.optimizer == "adamw"
+        "metric": "train tokens/s on 1 MI355X (nanolab-GPT tiny f32 AdamW step, BASELINE configs[0])"
+                  if args.config == "tiny"
+                  else "train tokens/s on 1 MI355X (GPT-124M bf16 AdamW step); % bf16 MFMA peak" if args.optimizer == "adamw"
                   else "train tokens/s on 1 MI355X (GPT-124M bf16 Muon-NS5 + AdamW step, BASELINE configs[3])",
         "value": value,
         "unit": "tokens/s",
@@ -204,11 +209,12 @@ def main() -> int:
                    if args.config == "gpt124m" else "nanolab-GPT tiny f32 step (BASELINE configs[0])",
                    "tokens_per_step": tokens, "params": sum(tr.param_lens())},
         "step_tflops": flops / (ms_per_step * 1e-3) / 1e12,
-        "pct_bf16_mfma_peak": 100.0 * flops / (ms_per_step * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS,
+        "pct_bf16_mfma_peak": 100.0 * flops / (ms_per_step * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS if cfg.bf16 else None,
         "loss_first": losses[0], "loss_last": losses[-1],
-        "roofline": {"bound": "mfma", "kernel": "gemm_dma_kernel / gemm_kernel (bf16 MFMA GEMM, all operand layouts)",
-                     "achieved": achieved, "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / BF16_MFMA_PEAK_TFLOPS,
+        "roofline": {"bound": "mfma",
+                     "kernel": "gemm_dma_kernel / gemm_kernel (bf16 MFMA GEMM, all operand layouts)" if cfg.bf16
+                               else "gemm_kernel<float> (f32 MFMA GEMM, all operand layouts)",
+                     "achieved": achieved, "peak": gemm_peak, "unit": "TFLOP/s", "frac": achieved / gemm_peak,
                      "traffic": GEMM_HBM_BYTES_PER_LAUNCH_GPT124M if args.config == "gpt124m" else None,
                      "launches": int(launches.value), "avg_launch_us": gemm_ms.value * 1e3 / max(1, launches.value),
                      "timed_steps": len(range(0, args.steps, timed_every)),
