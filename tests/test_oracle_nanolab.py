@@ -166,12 +166,14 @@ def test_bf16_muon_step_is_stock_nanolab_bit_for_bit():
         assert rel32 > 1e-2, f"case {i}: the f32 contrast is too close ({rel32:.2e}) to tell"
 
 
-def test_five_trainer_steps_follow_the_torch_trace():
+def test_trainer_steps_follow_the_torch_trace():
     """Micro-batch accumulation, the global clip, Muon-NS5 in f32 and AdamW, composed the way
     `Trainer::run` composes them, against the reference's torch trace: per-step mean loss within
     1e-4 nats, gradient norm 1e-4 relative, every parameter after step 5 within 1e-4 normwise
     (ojas-oracle/src/parity.rs:36-41, :468-470). Then the gradients at those parameters against
-    `grads_step5` at the gradient gate."""
+    `grads_step5` at the gradient gate. The loop goes on to step 40 and the whole loss curve is held to
+    the reference's curve gates (2e-4 nats for the first ten steps, 2e-3 after; it must end a nat
+    below ln V)."""
     import trace_fixture as tf
 
     trace = tf.Trace()
@@ -183,12 +185,15 @@ def test_five_trainer_steps_follow_the_torch_trace():
     state = {n: [np.zeros_like(params[n]), np.zeros_like(params[n])] for n in names}
     weight = np.float32(1.0 / trace.accum)
     losses, norms = [], []
-    for step in range(trace.steps):
+    after_five = None
+    for step in range(len(trace.mean_loss)):
         acc, loss_sum = None, np.float32(0)
         for micro in range(trace.accum):
             ids, targets = trace.micro(step, micro)
             loss, _, grads = orc.nanolab_loss_and_grads(cfg, [params[n].reshape(-1) for n in names], ids, targets)
-            assert abs(float(loss) - trace.micro_loss[step * trace.accum + micro]) <= tf.TRACE_LOSS_ABS_TOL
+            micro_tol = (tf.TRACE_LOSS_ABS_TOL if step < trace.steps else
+                         tf.CURVE_EARLY_ABS_TOL if step < tf.CURVE_EARLY_STEPS else tf.CURVE_LATE_ABS_TOL)
+            assert abs(float(loss) - trace.micro_loss[step * trace.accum + micro]) <= micro_tol, (step, micro)
             grads = [np.asarray(g, np.float32) * weight for g in grads]
             acc = grads if acc is None else [a + g for a, g in zip(acc, grads)]
             loss_sum = np.float32(loss_sum + np.float32(loss))
@@ -208,8 +213,12 @@ def test_five_trainer_steps_follow_the_torch_trace():
                 params[n], state[n] = p.reshape(shape), [m.reshape(shape), v.reshape(shape)]
         losses.append(float(loss_sum) / trace.accum)
         norms.append(float(norm))
-    worst = tf.check_trace(trace, losses, norms, params, frozen)
+        if step + 1 == trace.steps:
+            after_five = {n: params[n].copy() for n in names}
+    worst = tf.check_trace(trace, losses, norms, after_five, frozen)
     print(f"worst parameter distance after step {trace.steps}: {worst:.2e}")
+    # All 40 steps of the curve, at the reference's curve gates (parity.rs:52-58).
+    print(f"worst loss distance over 40 steps: {tf.check_curve(trace, losses, cfg.vocab):.2e}")
 
     want, gmeta = load("grads_step5")
     info = gmeta["ojas.oracle"]

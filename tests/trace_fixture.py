@@ -61,6 +61,32 @@ def optimizer_of(name, shape):
     return "muon" if len(shape) == 2 and name != "tok_emb.weight" else "adamw"
 
 
+# The 40-step curve (framework-design section 10; ojas-oracle/src/parity.rs:52-58): |loss - torch's| per step.
+CURVE_EARLY_ABS_TOL = 2e-4  # steps 1 ..= CURVE_EARLY_STEPS
+CURVE_EARLY_STEPS = 10
+CURVE_LATE_ABS_TOL = 2e-3
+CURVE_MIN_DROP_NATS = 1.0  # the curve must end this far below ln V
+AUTOCAST_GAP_FACTOR = 2.0  # parity.rs:59-74
+
+
+def check_curve(trace, losses, vocab):
+    """The per-step mean losses of all 40 steps against the trace's (`parity.rs:52-58`)."""
+    assert len(losses) == len(trace.mean_loss) == 40
+    worst = 0.0
+    for s, (got, want) in enumerate(zip(losses, trace.mean_loss)):
+        tol = CURVE_EARLY_ABS_TOL if s < CURVE_EARLY_STEPS else CURVE_LATE_ABS_TOL
+        assert abs(got - want) <= tol, (s, got, want)
+        worst = max(worst, abs(got - want))
+    assert losses[-1] <= np.log(vocab) - CURVE_MIN_DROP_NATS, losses[-1]
+    return worst
+
+
+def autocast_gap():
+    """torch's own f32 and autocast-bf16 curves over the same 40 steps (`autocast_gap.json`)."""
+    d = json.loads((TINY / "autocast_gap.json").read_text())
+    return np.array(d["f32_mean_loss"]), np.array(d["bf16_mean_loss"])
+
+
 def check_trace(trace, losses, norms, params, frozen):
     for s in range(trace.steps):
         assert abs(losses[s] - trace.mean_loss[s]) <= TRACE_LOSS_ABS_TOL, (s, losses[s], trace.mean_loss[s])
