@@ -80,6 +80,9 @@ class DeviceTensor:
 
     def __init__(self, backend: "MiBackend", ptr: int, shape: Tuple[int, ...], dtype: int, owns: bool = True):
         self.backend, self.ptr, self.shape, self.dtype, self._owns = backend, ptr, tuple(shape), dtype, owns
+        # The storage compute tag of an f32 tensor (tensor.rs COMPUTE_BF16): True when its values are
+        # known to be bf16-exact, so a second rounding would only clone. Set by `Autocast`.
+        self.compute_bf16 = False
 
     @property
     def numel(self) -> int:
@@ -96,6 +99,7 @@ class DeviceTensor:
             raise OjasError(SHAPE, f"reshape {self.shape} -> {shape}")
         view = DeviceTensor(self.backend, self.ptr, shape, self.dtype, owns=False)
         view._base = self
+        view.compute_bf16 = self.compute_bf16
         return view
 
     def __del__(self):

@@ -10,6 +10,7 @@ from __future__ import annotations
 
 import json
 import math
+from contextlib import nullcontext
 from dataclasses import dataclass
 from decimal import Decimal
 from pathlib import Path
@@ -17,6 +18,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
 
+from .autocast import Autocast
 from .backend import F32, AdamWConfig, MiBackend, MuonNs5Config, DeviceTensor, OjasError, NON_FINITE, OUT_OF_RANGE
 
 BLOCK_PARAMS = ("norm1.weight", "mixer.q_proj.weight", "mixer.k_proj.weight", "mixer.v_proj.weight",
@@ -211,7 +213,13 @@ class NanolabTrainer:
     the schedule is host arithmetic outside this path."""
 
     def __init__(self, be: MiBackend, spec: NanolabSpec, host_params: Dict[str, np.ndarray], adam_lr: float = 6e-4,
-                 matrix_lr: float = 0.025, grad_clip: float = 1.0, ns5_bf16: bool = False):
+                 matrix_lr: float = 0.025, grad_clip: float = 1.0, ns5_bf16: bool = False, autocast: bool = False):
+        # `TrainConfig::precision` (trainer.rs:120-135): bf16 wraps the backend in `Autocast` and the
+        # forward, the backward and the taking of the gradients run inside its region (:935-966);
+        # accumulation, the clip and the optimizers run outside it, on f32 masters.
+        self.autocast = autocast
+        if autocast:
+            be = Autocast(be)
         self.be, self.spec = be, spec
         self.adam_lr, self.matrix_lr, self.grad_clip, self.ns5_bf16 = adam_lr, matrix_lr, grad_clip, ns5_bf16
         shapes = spec.param_shapes()
@@ -243,9 +251,10 @@ class NanolabTrainer:
             if count == 0:
                 continue
             weight = float(np.float32(1.0 / len(live))) if uniform else float(np.float32(count / total))
-            loss, _, grads = self.graph.loss_and_grads(be.upload(np.ascontiguousarray(ids, np.uint32)),
-                                                       be.upload(np.ascontiguousarray(targets, np.uint32)),
-                                                       loss_seed=weight)
+            with (be.region() if self.autocast else nullcontext()):
+                loss, _, grads = self.graph.loss_and_grads(be.upload(np.ascontiguousarray(ids, np.uint32)),
+                                                           be.upload(np.ascontiguousarray(targets, np.uint32)),
+                                                           loss_seed=weight)
             if acc is None:
                 acc = {n: grads[n] for n in self.trainable}
             else:

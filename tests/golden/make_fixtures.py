@@ -15,6 +15,8 @@ Run in the build container (needs /root/reference). Only DATA is taken:
   * the tiny model's 40-step f32-NS5 trace  ojas-oracle/fixtures/tiny/{trace_ns5_f32,grads_step5}.safetensors,
     (losses, grad norms, step-5 parameters)  its token bin, window starts and LR multipliers: tokens.bin,
                                              batch_starts.json, lr_schedules.json (copied as is)
+  * torch's f32 and autocast-bf16 loss curves  ojas-oracle/fixtures/tiny/autocast_gap.json (copied as is)
+    over those 40 steps
   * pinned window starts of the batch sampler  ojas-data/tests/sampler.rs:231-254 (numbers -> JSON)
 No reference source text is kept: numeric literals are parsed into JSON.
 """
@@ -88,7 +90,7 @@ def copies():
     (OUT / "tiny").mkdir(exist_ok=True)
     for f in ("init.safetensors", "forward.safetensors", "grads_init.safetensors", "muon_step_bf16.safetensors",
               "trace_ns5_f32.safetensors", "grads_step5.safetensors", "tokens.bin", "batch_starts.json",
-              "lr_schedules.json"):
+              "lr_schedules.json", "autocast_gap.json"):
         shutil.copyfile(REF / "ojas-oracle/fixtures/tiny" / f, OUT / "tiny" / f)
 
 

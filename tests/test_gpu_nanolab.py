@@ -159,6 +159,35 @@ def test_trainer_steps_follow_the_torch_trace(be):
     print(f"worst loss distance over 40 steps: {tf.check_curve(trace, losses, spec.vocab):.2e}", flush=True)
 
 
+def test_autocast_tier_stays_within_the_reference_gap_of_the_f32_run(be):
+    """`check_autocast_divergence` (ojas-oracle/src/parity.rs:615-690): the same 40 steps under
+    `Autocast` (`ojas_amd/autocast.py`) stay, step by step, within max(2e-3, 2 x torch's own worst
+    f32-to-bf16 gap) of this backend's f32 run, and still end a nat below ln V. torch's bf16 curve is
+    printed beside ours for the record only: two bf16 runs are not comparable step by step."""
+    import trace_fixture as tf
+    from ojas_amd.nanolab import NanolabTrainer
+
+    print("nanolab 40 steps, f32 and autocast", flush=True)
+    trace = tf.Trace()
+    spec = tiny_spec()
+    init, _ = load("init")
+    curves = {}
+    for autocast in (False, True):
+        trainer = NanolabTrainer(be, spec, init, adam_lr=trace.cfg["lr"], matrix_lr=trace.cfg["matrix_lr"],
+                                 grad_clip=trace.cfg["grad_clip"], autocast=autocast)
+        curves[autocast] = np.array([trainer.run([trace.micro(step, m) for m in range(trace.accum)],
+                                                 trace.lr_mult[step]).loss for step in range(40)])
+    torch_f32, torch_bf16 = tf.autocast_gap()
+    bound = max(tf.CURVE_LATE_ABS_TOL, tf.AUTOCAST_GAP_FACTOR * float(np.max(np.abs(torch_bf16 - torch_f32))))
+    gap = np.abs(curves[True] - curves[False])
+    print(f"worst |autocast - f32| {gap.max():.2e} at step {int(gap.argmax()) + 1} (bound {bound:.2e}); "
+          f"torch's own {np.max(np.abs(torch_bf16 - torch_f32)):.2e}; "
+          f"|autocast - torch bf16| {np.max(np.abs(curves[True] - torch_bf16)):.2e}", flush=True)
+    assert np.any(curves[True] != curves[False])  # the tier did round something
+    assert np.all(gap <= bound), (int(gap.argmax()), float(gap.max()))
+    assert curves[True][-1] <= np.log(spec.vocab) - tf.CURVE_MIN_DROP_NATS
+
+
 def test_save_then_resume_continues_bit_for_bit(be, tmp_path):
     """`Trainer::save` / `resume_from` over the checkpoint directory (ojas-model/src/checkpoint.rs): three
     steps, a save, a resume into a fresh trainer and two more steps equal five uninterrupted steps bit for
