@@ -487,12 +487,15 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
       // layers' input-gradient products with up to 1024 output columns three tiles per compute
       // unit instead of one and a half (K = 3072: 94 against 104 us), and are 3 to 20 % ahead on
       // the layers' weight-gradient products (both operands K-major, K = tokens), d x d included.
-      // The head's products (K or M = vocabulary) are faster on the larger tile.
+      // The head's products (K or M = vocabulary) are faster on the larger tile, and its input
+      // gradient (16384 x 768 outputs over K = 50304) on 256 x 256 in whole-line steps: one
+      // workgroup per compute unit, but 2095 steps to amortise that over (1610 against 1824 us).
       const bool unbatched = g.batches == 1;
       const long outputs = static_cast<long>(g.M) * g.N;
       if (unbatched && a_km && b_km && g.K >= 4096 && outputs <= (1l << 22)) dma_variant = 6;
       else if (outputs * g.batches <= (1l << 20)) dma_variant = -1;
       else if (unbatched && !a_km && b_km && g.N <= 1024 && g.K <= 4096) dma_variant = 6;
+      else if (unbatched && !a_km && b_km && g.N <= 1024 && g.K >= 32768 && g.M >= 8192) dma_variant = 0;
       else dma_variant = 3;
     }
     else if (mode == 2) dma_variant = 0;
