@@ -117,6 +117,17 @@ int32_t omx_gemm(omx_ctx* ctx, const void* a, uint64_t a_rs, uint64_t a_cs, cons
                  uint64_t b_rs, uint64_t b_cs, int32_t operand_dtype, void* c, int32_t c_dtype,
                  uint64_t m, uint64_t k, uint64_t n, int32_t accumulate);
 
+/* `count` products of omx_gemm's form in one launch: product i reads its operands stride_a /
+ * stride_b ELEMENTS after product i - 1's and writes stride_c elements after its output (strides
+ * in multiples of 16 bytes; 1..65535 products). No counterpart in the trait, whose linear ops
+ * take one product per call (backend.rs:1628-1656): a caller that keeps the same-shaped layers of
+ * a model at a fixed stride uses it for their weight gradients, whose long reductions with small
+ * outputs fill the chip only together. */
+int32_t omx_gemm_strided_batch(omx_ctx* ctx, const void* a, uint64_t a_rs, uint64_t a_cs, const void* b,
+                               uint64_t b_rs, uint64_t b_cs, int32_t operand_dtype, void* c,
+                               int32_t c_dtype, uint64_t m, uint64_t k, uint64_t n, int32_t accumulate,
+                               uint64_t count, uint64_t stride_a, uint64_t stride_b, uint64_t stride_c);
+
 /* ---- BackendModule::causal_sdpa_forward / _backward (backend.rs:1729-1792).
  *      q,out,gy,gq: [B,H,T,D]; k,v,gk,gv: [B,Hkv,T,D]; lse: [B,H,T] f32.
  *      window = 0: every earlier key. scale = 1/sqrt(D) (backend.rs:159). ---- */

@@ -266,6 +266,21 @@ class MiBackend:
                                        C.c_uint64(k), C.c_uint64(n), C.c_int32(1 if acc else 0)))
         return out
 
+    def gemm_strided_batch(self, a: DeviceTensor, a_strides, b: DeviceTensor, b_strides, m, k, n, count,
+                           batch_strides, out_dtype=F32):
+        """`count` products of `gemm`'s form in one launch; `batch_strides` = element strides between
+        consecutive products' A, B and C. Returns C [count, m, n] when the C stride is m * n."""
+        sa, sb, sc = batch_strides
+        if sc < m * n:
+            raise OjasError(SHAPE, "gemm_strided_batch: outputs overlap")
+        out = self.empty(((count - 1) * sc + m * n,), out_dtype)
+        self._check(self._lib.omx_gemm_strided_batch(
+            self._ctx, self._p(a), C.c_uint64(a_strides[0]), C.c_uint64(a_strides[1]), self._p(b),
+            C.c_uint64(b_strides[0]), C.c_uint64(b_strides[1]), C.c_int32(a.dtype), self._p(out), C.c_int32(out_dtype),
+            C.c_uint64(m), C.c_uint64(k), C.c_uint64(n), C.c_int32(0), C.c_uint64(count), C.c_uint64(sa),
+            C.c_uint64(sb), C.c_uint64(sc)))
+        return out
+
     # ---- attention ----
     def causal_sdpa_forward(self, q, k, v, window: Optional[int] = None, out_dtype: Optional[int] = None):
         b, h, t, d = q.shape

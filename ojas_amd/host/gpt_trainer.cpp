@@ -73,6 +73,14 @@ struct ogpt {
   // runs time-major on those blocks, and their gradients are the blocks of `gqkv`.
   bool fused_qkv = false;
   void* gqkv = nullptr;                      // [N,3d] AD
+  // With the fused projection, the four weight gradients of every layer wait until the backward's
+  // end: each layer's inputs (h1, ap, h2, g) and output gradients (below) sit at a fixed stride in
+  // stacked buffers, the gradient arena holds the layers at a fixed stride too, and four strided-
+  // batch products over the layers replace 4 x layers split-K products.
+  bool deferred_dw = false;
+  void *h1_all = nullptr, *ap_all = nullptr, *h2_all = nullptr, *g_all = nullptr;
+  void *gu_all = nullptr, *gqkv_all = nullptr;  // [layers][N,mlp], [layers][N,3d] AD
+  void *gyd_all = nullptr, *gyo_all = nullptr;  // residual-stream gradient copies feeding down / o: [layers][N,d] AD
   float *gres = nullptr, *gres1 = nullptr, *gt = nullptr, *gh = nullptr;  // [N,d] f32
   float* g_emb = nullptr;                    // [V,d] f32
   void* ghf = nullptr;                       // [N,d] AD
@@ -192,38 +200,50 @@ int32_t backward(ogpt* t) {
                             eps));
   // `gy` is the residual-stream gradient as a GEMM operand: gres itself on the f32 tier, its bf16
   // copy (written by the kernel that produced gres) on the bf16 tier.
+  const bool defer = t->deferred_dw;  // implies the bf16 tier with the fused projection
+  // Layer l's slice of a stacked [layers][per_layer] operand buffer.
+  auto slice = [&](void* all, uint64_t l, uint64_t per_layer) {
+    return static_cast<void*>(static_cast<char*>(all) + l * per_layer * t->asz);
+  };
   const void* gy = nullptr;
-  TRY(to_operand(t, t->gres, t->gy16, N * d, &gy));
+  TRY(to_operand(t, t->gres, defer ? slice(t->gyd_all, c.layers - 1, N * d) : t->gy16, N * d, &gy));
   void* copy16 = AD == OMX_BF16 ? t->gy16 : nullptr;
   for (uint32_t l = c.layers; l-- > 0;) {
     ogpt::Layer& A = t->layers[l];
+    void* gu = defer ? slice(t->gu_all, l, N * M) : t->gu;
+    void* gqkv = defer ? slice(t->gqkv_all, l, 3 * N * d) : t->gqkv;
+    // Where the two norm backwards of this layer leave the bf16 copy of the gradient they produce:
+    // the operand of this layer's o projection, and of the layer below's down projection.
+    void* copy_o = defer ? slice(t->gyo_all, l, N * d) : copy16;
+    void* copy_below = defer && l > 0 ? slice(t->gyd_all, l - 1, N * d) : copy16;
+    // Weight gradients go to the arena now, or wait for the batched products after the loop.
+    auto gw = [&](uint64_t which) { return defer ? nullptr : t->g(t->li(l, which)); };
     // x_next = x1 + down(gelu(up(norm2(x1))))
     if (AD == OMX_BF16) {
       // The activation's derivative rides in the input-gradient product's store pass.
-      TRY(omx_linear_backward(ctx, A.g, nullptr, gy, AD, nullptr, AD, t->g(t->li(l, 7)), OMX_F32, N, M, d));
-      TRY(omx_linear_backward_input_gelu(ctx, t->w(t->li(l, 7)), gy, AD, A.u, t->gu, N, M, d, c.gelu_tanh));
+      if (!defer) TRY(omx_linear_backward(ctx, A.g, nullptr, gy, AD, nullptr, AD, t->g(t->li(l, 7)), OMX_F32, N, M, d));
+      TRY(omx_linear_backward_input_gelu(ctx, t->w(t->li(l, 7)), gy, AD, A.u, gu, N, M, d, c.gelu_tanh));
     } else {
       TRY(omx_linear_backward(ctx, A.g, t->w(t->li(l, 7)), gy, AD, t->gg, AD, t->g(t->li(l, 7)), OMX_F32, N, M, d));
-      TRY(omx_gelu_backward(ctx, A.u, t->gg, t->gu, AD, N * M, c.gelu_tanh));
+      TRY(omx_gelu_backward(ctx, A.u, t->gg, gu, AD, N * M, c.gelu_tanh));
     }
-    TRY(omx_linear_backward(ctx, A.h2, t->w(t->li(l, 6)), t->gu, AD, t->t_a, AD, t->g(t->li(l, 6)), OMX_F32, N, d, M));
+    TRY(omx_linear_backward(ctx, A.h2, t->w(t->li(l, 6)), gu, AD, t->t_a, AD, gw(6), OMX_F32, N, d, M));
     // Fan-in at x1: the residual branch arrives first, then the norm branch.
-    TRY(omx_rms_norm_backward_residual(ctx, A.x1, OMX_F32, t->w32(t->li(l, 5)), t->t_a, AD, t->gres, t->gres1, copy16,
+    TRY(omx_rms_norm_backward_residual(ctx, A.x1, OMX_F32, t->w32(t->li(l, 5)), t->t_a, AD, t->gres, t->gres1, copy_o,
                                        t->g(t->li(l, 5)), N, d, eps));
-    gy = AD == OMX_BF16 ? static_cast<const void*>(t->gy16) : static_cast<const void*>(t->gres1);
+    gy = AD == OMX_BF16 ? static_cast<const void*>(copy_o) : static_cast<const void*>(t->gres1);
     // x1 = x + o(attention)
-    TRY(omx_linear_backward(ctx, A.ap, t->w(t->li(l, 4)), gy, AD, t->t_a, AD, t->g(t->li(l, 4)), OMX_F32, N, d, d));
+    TRY(omx_linear_backward(ctx, A.ap, t->w(t->li(l, 4)), gy, AD, t->t_a, AD, gw(4), OMX_F32, N, d, d));
     if (t->fused_qkv) {
-      char* gq = static_cast<char*>(t->gqkv);
+      char* gq = static_cast<char*>(gqkv);
       TRY(omx_causal_attention_backward_saved(ctx, A.q, 3 * d, A.k, A.v, 3 * d, A.ap, A.apr, t->t_a, d, A.lse, AD, gq,
                                         gq + d * t->asz, gq + 2 * d * t->asz, AD, B, T, H, H, D, 0));
       // One product for the three projections: the input gradient is their sum, formed in the
       // product's f32 accumulators.
-      TRY(omx_linear_backward(ctx, A.h1, t->w(t->li(l, 1)), t->gqkv, AD, t->t_b, AD, t->g(t->li(l, 1)), OMX_F32, N, d,
-                              3 * d));
-      TRY(omx_rms_norm_backward_residual(ctx, A.x, OMX_F32, t->w32(t->li(l, 0)), t->t_b, AD, t->gres1, t->gres, copy16,
-                                         t->g(t->li(l, 0)), N, d, eps));
-      gy = AD == OMX_BF16 ? static_cast<const void*>(t->gy16) : static_cast<const void*>(t->gres);
+      TRY(omx_linear_backward(ctx, A.h1, t->w(t->li(l, 1)), gqkv, AD, t->t_b, AD, gw(1), OMX_F32, N, d, 3 * d));
+      TRY(omx_rms_norm_backward_residual(ctx, A.x, OMX_F32, t->w32(t->li(l, 0)), t->t_b, AD, t->gres1, t->gres,
+                                         copy_below, t->g(t->li(l, 0)), N, d, eps));
+      gy = AD == OMX_BF16 ? static_cast<const void*>(copy_below) : static_cast<const void*>(t->gres);
       continue;
     }
     TRY(omx_permute_0213(ctx, t->t_a, t->ga, AD, B, T, H, D));
@@ -240,6 +260,22 @@ int32_t backward(ogpt* t) {
     TRY(omx_rms_norm_backward_residual(ctx, A.x, OMX_F32, t->w32(t->li(l, 0)), t->gh, OMX_F32, t->gres1, t->gres, copy16,
                                        t->g(t->li(l, 0)), N, d, eps));
     gy = AD == OMX_BF16 ? static_cast<const void*>(t->gy16) : static_cast<const void*>(t->gres);
+  }
+  if (defer) {
+    // gw[l](o, j) = sum_r gy[l][r, o] * x[l][r, j] for every layer l in one launch per weight:
+    // 4 x layers long reductions with small outputs become four products with enough tiles to fill
+    // the chip without splitting K.
+    const uint64_t layers = c.layers, per_layer = t->slots[t->li(1, 0)].offset - t->slots[t->li(0, 0)].offset;
+    struct Deferred {
+      const void *gy, *x;
+      uint64_t which, out, in;
+    } products[4] = {{t->gyd_all, t->g_all, 7, d, M},
+                     {t->gu_all, t->h2_all, 6, M, d},
+                     {t->gyo_all, t->ap_all, 4, d, d},
+                     {t->gqkv_all, t->h1_all, 1, 3 * d, d}};
+    for (const Deferred& p : products)
+      TRY(omx_gemm_strided_batch(ctx, p.gy, 1, p.out, p.x, p.in, 1, AD, t->g(t->li(0, p.which)), OMX_F32, p.out, N, p.in,
+                                 0, layers, N * p.out, N * p.in, per_layer));
   }
   // x0 = tok[ids] + pos[positions]; the tied table adds the embedding's share to the head's.
   TRY(omx_embedding_backward(ctx, t->positions, t->gres, OMX_F32, t->g(1), N, T, d));
@@ -319,10 +355,35 @@ int32_t ogpt_create(omx_ctx* ctx, const ogpt_config* config, ogpt** out) {
     CREATE_TRY(omx_upload(ctx, t->positions, 0, pos.data(), N * 4));
   }
   t->layers.resize(c.layers);
+  t->deferred_dw = t->fused_qkv && c.layers > 1;
+  const uint64_t L = c.layers;
+  if (t->deferred_dw) {
+    CREATE_TRY(alloc_act(t, L * N * d, &t->h1_all));
+    CREATE_TRY(alloc_act(t, L * N * d, &t->ap_all));
+    CREATE_TRY(alloc_act(t, L * N * d, &t->h2_all));
+    CREATE_TRY(alloc_act(t, L * N * M, &t->g_all));
+    CREATE_TRY(alloc_act(t, L * N * M, &t->gu_all));
+    CREATE_TRY(alloc_act(t, L * 3 * N * d, &t->gqkv_all));
+    CREATE_TRY(alloc_act(t, L * N * d, &t->gyd_all));
+    CREATE_TRY(alloc_act(t, L * N * d, &t->gyo_all));
+  }
+  uint64_t layer_index = 0;
   for (auto& A : t->layers) {
+    const uint64_t l = layer_index++;
+    auto slice = [&](void* all, uint64_t per_layer) { return static_cast<void*>(static_cast<char*>(all) + l * per_layer * t->asz); };
     CREATE_TRY(alloc_t(t, N * d, &A.x));
     CREATE_TRY(alloc_t(t, N * d, &A.x1));
-    CREATE_TRY(alloc_act(t, N * d, &A.h1));
+    if (t->deferred_dw) {
+      A.h1 = slice(t->h1_all, N * d);
+      A.ap = slice(t->ap_all, N * d);
+      A.h2 = slice(t->h2_all, N * d);
+      A.g = slice(t->g_all, N * M);
+    } else {
+      CREATE_TRY(alloc_act(t, N * d, &A.h1));
+      CREATE_TRY(alloc_act(t, N * d, &A.ap));
+      CREATE_TRY(alloc_act(t, N * d, &A.h2));
+      CREATE_TRY(alloc_act(t, N * M, &A.g));
+    }
     if (t->fused_qkv) {
       CREATE_TRY(alloc_act(t, 3 * N * d, &A.q));
       A.k = static_cast<char*>(A.q) + d * t->asz;
@@ -335,10 +396,7 @@ int32_t ogpt_create(omx_ctx* ctx, const ogpt_config* config, ogpt** out) {
       CREATE_TRY(alloc_act(t, N * d, &A.v));
       CREATE_TRY(alloc_act(t, N * d, &A.a));
     }
-    CREATE_TRY(alloc_act(t, N * d, &A.ap));
-    CREATE_TRY(alloc_act(t, N * d, &A.h2));
     CREATE_TRY(alloc_act(t, N * M, &A.u));
-    CREATE_TRY(alloc_act(t, N * M, &A.g));
     CREATE_TRY(alloc_t(t, static_cast<uint64_t>(c.batch) * c.heads * c.ctx, &A.lse));
   }
   CREATE_TRY(alloc_t(t, N * d, &t->x_final));
@@ -347,10 +405,10 @@ int32_t ogpt_create(omx_ctx* ctx, const ogpt_config* config, ogpt** out) {
   CREATE_TRY(alloc_t(t, N * d, &t->e_pos));
   CREATE_TRY(alloc_act(t, N * d, &t->t_a));
   CREATE_TRY(alloc_act(t, N * d, &t->t_b));
-  CREATE_TRY(alloc_act(t, N * M, &t->gu));
+  if (!t->deferred_dw) CREATE_TRY(alloc_act(t, N * M, &t->gu));
   CREATE_TRY(alloc_act(t, N * M, &t->gg));
   if (t->fused_qkv) {
-    CREATE_TRY(alloc_act(t, 3 * N * d, &t->gqkv));
+    if (!t->deferred_dw) CREATE_TRY(alloc_act(t, 3 * N * d, &t->gqkv));
   } else {
     CREATE_TRY(alloc_act(t, N * d, &t->gq));
     CREATE_TRY(alloc_act(t, N * d, &t->gk));

@@ -64,3 +64,40 @@ def test_linear_bf16_under_each_kernel(be, mode, rows, kin, nout):
 def test_unknown_option_is_refused(be):
     assert be._lib.omx_set_option(be._ctx, b"no_such_knob", C.c_int64(1)) == 11
     assert be._lib.omx_set_option(be._ctx, b"gemm_dma", C.c_int64(9)) == 3
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2, 3, 6])
+@pytest.mark.parametrize("rows,kin,nout", [(1088, 136, 264), (2048, 768, 256)])
+def test_strided_batch_of_weight_gradients(be, mode, rows, kin, nout):
+    """`omx_gemm_strided_batch` as the step driver uses it: gw[l] = gy[l]^T x[l] for three stacked
+    layers in one launch, outputs at a padded stride; each equals the oracle's `linear_backward`
+    weight gradient."""
+    from ojas_amd.backend import BF16, F32
+
+    print(f"gemm strided batch mode {mode} {rows}x{kin}x{nout}", flush=True)
+    assert be._lib.omx_set_option(be._ctx, b"gemm_dma", C.c_int64(mode)) == 0
+    layers, pad = 3, 64
+    r = orc.SplitMix64(7100 + rows + mode)
+    x = orc.round_bf16(r.vec(layers * rows * kin, 0.5)).reshape(layers, rows, kin)
+    gy = orc.round_bf16(r.vec(layers * rows * nout, 0.5)).reshape(layers, rows, nout)
+    w = np.zeros((nout, kin), np.float32)
+    orc.set_threads(8)
+    stride_c = nout * kin + pad
+    out = be.gemm_strided_batch(be.upload(gy, BF16), (1, nout), be.upload(x, BF16), (kin, 1), nout, rows, kin, layers,
+                                (rows * nout, rows * kin, stride_c))
+    got = be.download(out)
+    for l in range(layers):
+        _, ogw = orc.linear_backward(x[l], w, gy[l])
+        mine = got[l * stride_c:l * stride_c + nout * kin].reshape(nout, kin).astype(np.float64)
+        err = float(np.max(np.abs(mine - ogw)))
+        assert err <= 1e-5 * max(1.0, float(np.max(np.abs(ogw)))), (l, err)
+
+
+def test_strided_batch_refuses_bad_strides(be):
+    from ojas_amd.backend import BF16, OjasError
+
+    a, b = be.zeros((2, 64, 64), BF16), be.zeros((2, 64, 64), BF16)
+    with pytest.raises(OjasError):  # a batch stride that is not a multiple of 16 bytes
+        be.gemm_strided_batch(a, (1, 64), b, (64, 1), 64, 64, 64, 2, (64 * 64 + 2, 64 * 64, 64 * 64))
+    with pytest.raises(OjasError):  # overlapping outputs
+        be.gemm_strided_batch(a, (1, 64), b, (64, 1), 64, 64, 64, 2, (64 * 64, 64 * 64, 64))
