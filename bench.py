@@ -31,10 +31,10 @@ BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, vendor figure
 F32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, vendor figure
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor figure
 # HBM bytes per GEMM op (MFMA kernel + split-K reduce) on the gpt124m workload, averaged over the
-# step's 147 GEMM ops: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by what the same
+# step's 103 GEMM ops (a strided batch of the stacked layers' weight gradients is one op): rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by what the same
 # counters read for the AdamW pass, whose traffic is known (profiles/gemm_hbm_traffic_gpt124m_bf16.txt).
-# The algorithmic figure (every operand read once, every output written once) is 1.582e8.
-GEMM_HBM_BYTES_PER_LAUNCH_GPT124M = 3.13e8
+# The algorithmic figure (every operand read once, every output written once) is 2.258e8.
+GEMM_HBM_BYTES_PER_LAUNCH_GPT124M = 4.68e8
 
 
 def cpu_baseline(cfg, threads: int):
@@ -164,8 +164,8 @@ def main() -> int:
     lib = be._lib
     # The GEMM kernels of every fourth timed step carry HIP events on their dispatches (begin and
     # end timestamps of the kernels themselves). All steps would cost 0.7 ms per step on the
-    # number being measured (the timed launch path is slower: 147 products per step); a quarter
-    # of them is 735 timed products in the default run.
+    # number being measured (the timed launch path is slower: 103 products per step); a quarter
+    # of them is 515 timed products in the default run.
     timed_every = 4
     t0 = time.perf_counter()
     for i in range(args.steps):

@@ -490,9 +490,13 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
       // The head's products (K or M = vocabulary) are faster on the larger tile, and its input
       // gradient (16384 x 768 outputs over K = 50304) on 256 x 256 in whole-line steps: one
       // workgroup per compute unit, but 2095 steps to amortise that over (1610 against 1824 us).
+      // A batch of weight gradients over stacked layers (K = tokens) has tiles enough without
+      // splitting K; its tall form (3072 x 768 outputs, twelve layers) is faster on 256 x 256
+      // (916 against 1121 us), the others on 256 x 128.
       const bool unbatched = g.batches == 1;
       const long outputs = static_cast<long>(g.M) * g.N;
       if (unbatched && a_km && b_km && g.K >= 4096 && outputs <= (1l << 22)) dma_variant = 6;
+      else if (!unbatched && a_km && b_km && g.K >= 4096 && g.M >= 3072 && g.N <= 1024) dma_variant = 0;
       else if (outputs * g.batches <= (1l << 20)) dma_variant = -1;
       else if (unbatched && !a_km && b_km && g.N <= 1024 && g.K <= 4096) dma_variant = 6;
       else if (unbatched && !a_km && b_km && g.N <= 1024 && g.K >= 32768 && g.M >= 8192) dma_variant = 0;
