@@ -34,7 +34,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor figure
 # step's 103 GEMM ops (a strided batch of the stacked layers' weight gradients is one op): rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by what the same
 # counters read for the AdamW pass, whose traffic is known (profiles/gemm_hbm_traffic_gpt124m_bf16.txt).
 # The algorithmic figure (every operand read once, every output written once) is 2.258e8.
-GEMM_HBM_BYTES_PER_LAUNCH_GPT124M = 4.68e8
+GEMM_HBM_BYTES_PER_LAUNCH_GPT124M = 3.82e8
 
 
 def cpu_baseline(cfg, threads: int):

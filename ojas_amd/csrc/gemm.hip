@@ -230,7 +230,7 @@ __global__ __launch_bounds__(NT) void gemm_kernel(GemmArgs g) {
   constexpr int A_BYTES = tile_bytes<T, A_KM, BM>(), B_BYTES = tile_bytes<T, B_KM, BN>();
   constexpr int STAGE = A_BYTES + B_BYTES;
   static_assert(sizeof(T) == 2 || (TM == 2 && TN == 2), "the f32 lane uses 128x128 tiles");
-  gemm_select_batch(g);
+  gemm_select_batch(g, blockIdx.y);
   const T* __restrict__ A = static_cast<const T*>(g.a);
   const T* __restrict__ B = static_cast<const T*>(g.b);
 

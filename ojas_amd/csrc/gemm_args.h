@@ -26,10 +26,10 @@ struct GemmArgs {
   long batch_a, batch_b, batch_c;
 };
 
-// The arguments of the product this block belongs to.
-__device__ __forceinline__ void gemm_select_batch(GemmArgs& g) {
+// The arguments of product `product` of a strided batch.
+__device__ __forceinline__ void gemm_select_batch(GemmArgs& g, int product) {
   if (g.batches > 1) {
-    const long y = blockIdx.y;
+    const long y = product;
     g.a = static_cast<const char*>(g.a) + y * g.batch_a;
     g.b = static_cast<const char*>(g.b) + y * g.batch_b;
     g.c = static_cast<char*>(g.c) + y * g.batch_c;

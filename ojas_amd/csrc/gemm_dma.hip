@@ -161,18 +161,23 @@ gemm_dma_kernel(GemmArgs g) {
   static_assert(NW == 4 || NW == 6 || NW == 8, "four, six or eight waves");
   // Six waves share 16 + 24 loads unevenly; with two stages every wait is for all of a wave's loads.
   static_assert(STAGE % (1024 * NW) == 0 || NST == 2, "counted waits need the same number of loads in every wave");
-  gemm_select_batch(g);
-  const unsigned short* __restrict__ A = static_cast<const unsigned short*>(g.a);
-  const unsigned short* __restrict__ B = static_cast<const unsigned short*>(g.b);
 
   // Workgroups go to the 8 XCDs round-robin by blockIdx.x, and each XCD has its own L2. Without
   // split-K an XCD takes a contiguous eighth of the tiles; with it, blockIdx.x % splits is the
   // split, so (for the power-of-two split counts the host picks) all tiles of one K chunk run on
   // the same XCD, side by side, and that chunk of both operands is fetched into one L2 once
   // instead of into all eight.
+  // In a strided batch (grid.y = products, never split) an XCD takes a contiguous eighth of the
+  // (product, tile) pairs instead of an eighth of every product's tiles, so a product's operands
+  // are fetched into one or two L2s instead of all eight.
   const int total = g.tiles_m * g.tiles_n;
-  int split = 0, id = blockIdx.x;
-  if (g.splits > 1) {
+  int split = 0, id = blockIdx.x, product = blockIdx.y;
+  if (g.batches > 1 && g.splits == 1 && ((total * g.batches) & 7) == 0) {
+    const int linear = blockIdx.y * total + blockIdx.x;
+    const int r = (linear & 7) * ((total * g.batches) >> 3) + (linear >> 3);
+    product = r / total;
+    id = r - product * total;
+  } else if (g.splits > 1) {
     split = blockIdx.x % g.splits;
     id = blockIdx.x / g.splits;
   } else if (total % 8 == 0) {
@@ -187,6 +192,9 @@ gemm_dma_kernel(GemmArgs g) {
   const int tile_m = first_m + in_band % band_rows;
   const int tile_n = in_band / band_rows;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
+  gemm_select_batch(g, product);
+  const unsigned short* __restrict__ A = static_cast<const unsigned short*>(g.a);
+  const unsigned short* __restrict__ B = static_cast<const unsigned short*>(g.b);
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);

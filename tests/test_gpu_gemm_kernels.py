@@ -67,17 +67,18 @@ def test_unknown_option_is_refused(be):
 
 
 @pytest.mark.parametrize("mode", [0, 1, 2, 3, 6])
+@pytest.mark.parametrize("layers", [3, 4])  # 4: a tile count divisible by 8, which takes the XCD-ordered mapping
 @pytest.mark.parametrize("rows,kin,nout", [(1088, 136, 264), (2048, 768, 256)])
-def test_strided_batch_of_weight_gradients(be, mode, rows, kin, nout):
+def test_strided_batch_of_weight_gradients(be, mode, rows, kin, nout, layers):
     """`omx_gemm_strided_batch` as the step driver uses it: gw[l] = gy[l]^T x[l] for three stacked
     layers in one launch, outputs at a padded stride; each equals the oracle's `linear_backward`
     weight gradient."""
     from ojas_amd.backend import BF16, F32
 
-    print(f"gemm strided batch mode {mode} {rows}x{kin}x{nout}", flush=True)
+    print(f"gemm strided batch mode {mode} {rows}x{kin}x{nout} layers {layers}", flush=True)
     assert be._lib.omx_set_option(be._ctx, b"gemm_dma", C.c_int64(mode)) == 0
-    layers, pad = 3, 64
-    r = orc.SplitMix64(7100 + rows + mode)
+    pad = 64
+    r = orc.SplitMix64(7100 + rows + mode + layers)
     x = orc.round_bf16(r.vec(layers * rows * kin, 0.5)).reshape(layers, rows, kin)
     gy = orc.round_bf16(r.vec(layers * rows * nout, 0.5)).reshape(layers, rows, nout)
     w = np.zeros((nout, kin), np.float32)
