@@ -70,7 +70,10 @@ def test_f32_tier_step_matches_cpu_exact(be, shape, std):
     tr.close()
 
 
-@pytest.mark.parametrize("shape,std", [(SMALL, 0.05), (C1, 0.02)])
+ONE_LAYER = (1,) + SMALL[1:]  # weight gradients inside the layer loop; two layers and more batch them at the end
+
+
+@pytest.mark.parametrize("shape,std", [(SMALL, 0.05), (ONE_LAYER, 0.05), (C1, 0.02)])
 def test_bf16_tier_step_within_bf16_tolerance_of_cpu_exact(be, shape, std):
     print(f"gpt bf16 {shape}", flush=True)
     tr, params, (loss, grads), (oloss, ograds) = run_case(be, shape + (1,), 11, std)
