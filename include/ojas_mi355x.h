@@ -135,12 +135,24 @@ int32_t omx_causal_sdpa_forward(omx_ctx* ctx, const void* q, const void* k, cons
                                 int32_t operand_dtype, void* out, int32_t out_dtype, void* lse,
                                 uint64_t batch, uint64_t heads, uint64_t kv_heads, uint64_t time,
                                 uint64_t head_dim, uint64_t window);
+/* out / gy may be stored as f32 or bf16 independently of the operands (the forward writes either;
+ * the reference's tensors here are always f32). With bf16 operands an f32 `out` is read in full:
+ * the row term dO . O sees the unrounded output. */
 int32_t omx_causal_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, const void* v,
                                  const void* out, const void* lse, const void* gy,
-                                 int32_t operand_dtype, void* gq, void* gk, void* gv,
-                                 int32_t grad_dtype, uint64_t batch, uint64_t heads,
-                                 uint64_t kv_heads, uint64_t time, uint64_t head_dim,
+                                 int32_t operand_dtype, int32_t out_dtype, int32_t gy_dtype, void* gq,
+                                 void* gk, void* gv, int32_t grad_dtype, uint64_t batch,
+                                 uint64_t heads, uint64_t kv_heads, uint64_t time, uint64_t head_dim,
                                  uint64_t window);
+/* BackendModule::causal_sdpa_backward_recompute (backend.rs:1781-1792): the backward for a caller
+ * that kept neither output nor lse (Autocast routes a bf16-tagged saved output here,
+ * ojas-core/src/autocast.rs:1200-1233). The forward runs again into the library's scratch with an
+ * f32 output, then the backward reads it; gradient arguments are checked before that forward. */
+int32_t omx_causal_sdpa_backward_recompute(omx_ctx* ctx, const void* q, const void* k, const void* v,
+                                           const void* gy, int32_t operand_dtype, int32_t gy_dtype,
+                                           void* gq, void* gk, void* gv, int32_t grad_dtype,
+                                           uint64_t batch, uint64_t heads, uint64_t kv_heads,
+                                           uint64_t time, uint64_t head_dim, uint64_t window);
 
 /* linear_forward then gelu_{erf,tanh}_forward (backend.rs:1628-1656,1175-1220), the
  * activation applied while the product is stored: u = x W^T and act = gelu(u),

@@ -82,8 +82,15 @@ class Autocast:
         cancel the softmax row sum; the f32 output is recomputed from the same rounded operands."""
         q, k, v, gy = self._prep(q), self._prep(k), self._prep(v), self._prep(gy)
         if out.compute_bf16:
-            out, lse = self.inner.causal_sdpa_forward(q, k, v, window)
-        grads = self.inner.causal_sdpa_backward(q, k, v, out, lse, gy, window, grad_dtype)
+            grads = self.inner.causal_sdpa_backward_recompute(q, k, v, gy, window, grad_dtype)
+        else:
+            grads = self.inner.causal_sdpa_backward(q, k, v, out, lse, gy, window, grad_dtype)
+        return tuple(self._emit(g) for g in grads)
+
+    def causal_sdpa_backward_recompute(self, q, k, v, gy, window=None, grad_dtype=F32):
+        """:1238-1262: the inner backend's own recompute sees the operands the pair above would."""
+        grads = self.inner.causal_sdpa_backward_recompute(self._prep(q), self._prep(k), self._prep(v),
+                                                          self._prep(gy), window, grad_dtype)
         return tuple(self._emit(g) for g in grads)
 
     def per_head_sigmoid_gate_forward_saving(self, x, w, b, attn, *args, **kwargs):

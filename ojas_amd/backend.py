@@ -297,16 +297,37 @@ class MiBackend:
         return out, lse
 
     def causal_sdpa_backward(self, q, k, v, out, lse, gy, window: Optional[int] = None, grad_dtype=F32):
+        """`out` and `gy` are read in their own storage dtypes (f32 or bf16)."""
         b, h, t, d = q.shape
         hkv = k.shape[1]
         if window == 0:
             raise OjasError(SHAPE, "sdpa window must be at least 1")
+        if not (q.dtype == k.dtype == v.dtype):
+            raise OjasError(DTYPE, "causal_sdpa_backward: q, k, v must share a dtype")
+        if out.shape != q.shape or gy.shape != q.shape or lse.dtype != F32:
+            raise OjasError(SHAPE, f"causal_sdpa_backward: out {out.shape} / grad_output {gy.shape} against q {q.shape}")
         gq, gk, gv = self.empty(q.shape, grad_dtype), self.empty(k.shape, grad_dtype), self.empty(v.shape, grad_dtype)
         self._check(self._lib.omx_causal_sdpa_backward(self._ctx, self._p(q), self._p(k), self._p(v), self._p(out),
-                                                       self._p(lse), self._p(gy), C.c_int32(q.dtype), self._p(gq),
+                                                       self._p(lse), self._p(gy), C.c_int32(q.dtype),
+                                                       C.c_int32(out.dtype), C.c_int32(gy.dtype), self._p(gq),
                                                        self._p(gk), self._p(gv), C.c_int32(grad_dtype), C.c_uint64(b),
                                                        C.c_uint64(h), C.c_uint64(hkv), C.c_uint64(t), C.c_uint64(d),
                                                        C.c_uint64(window or 0)))
+        return gq, gk, gv
+
+    def causal_sdpa_backward_recompute(self, q, k, v, gy, window: Optional[int] = None, grad_dtype=F32):
+        """BackendModule::causal_sdpa_backward_recompute (backend.rs:1781-1792), one call."""
+        b, h, t, d = q.shape
+        hkv = k.shape[1]
+        if window == 0:
+            raise OjasError(SHAPE, "sdpa window must be at least 1")
+        if gy.shape != q.shape:
+            raise OjasError(SHAPE, f"causal_sdpa_backward_recompute: grad_output {gy.shape} against q {q.shape}")
+        gq, gk, gv = self.empty(q.shape, grad_dtype), self.empty(k.shape, grad_dtype), self.empty(v.shape, grad_dtype)
+        self._check(self._lib.omx_causal_sdpa_backward_recompute(
+            self._ctx, self._p(q), self._p(k), self._p(v), self._p(gy), C.c_int32(q.dtype), C.c_int32(gy.dtype),
+            self._p(gq), self._p(gk), self._p(gv), C.c_int32(grad_dtype), C.c_uint64(b), C.c_uint64(h),
+            C.c_uint64(hkv), C.c_uint64(t), C.c_uint64(d), C.c_uint64(window or 0)))
         return gq, gk, gv
 
     def linear_gelu_forward(self, x, w, tanh_form: bool = False):

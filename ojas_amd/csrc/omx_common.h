@@ -78,9 +78,10 @@ struct omx_ctx {
   std::string arch;
   // Scratch the library owns (charged to the budget); grown on demand.
   // Slot 0: per-op scratch. Slot 1: split-K partials of the GEMM (which an op
-  // may call while it holds slot 0).
-  void* workspace[2] = {nullptr, nullptr};
-  uint64_t workspace_bytes[2] = {0, 0};
+  // may call while it holds slot 0) and operands converted for an op that holds slot 0.
+  // Slot 2: tensors an op keeps across calls into other ops (a recomputed attention output).
+  void* workspace[3] = {nullptr, nullptr, nullptr};
+  uint64_t workspace_bytes[3] = {0, 0, 0};
   int cu_count = 0;
   // Optional per-launch timing of the GEMM kernel (benchmark only).
   // 0: 128x128 kernel only; 1: choose by shape; 2 / 3: force the 256x256 / 256x128 direct-to-LDS kernel where eligible.

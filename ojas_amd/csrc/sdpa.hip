@@ -16,6 +16,8 @@
 //   * flash kernels (flash_sdpa.hip): bf16 MFMA tiles for head_dim 64 / 128.
 // Neither forms a T x T matrix; no atomics are used, so results do not depend
 // on scheduling.
+#include <algorithm>
+
 #include "omx_common.h"
 
 int32_t omx_flash_sdpa_forward(omx_ctx* ctx, const void* q, const void* k, const void* v, void* out,
@@ -127,16 +129,30 @@ __global__ __launch_bounds__(SD_THREADS) void sdpa_fwd_rows_kernel(const TI* __r
 }
 
 // Dr[row] = dO[row] . O[row] (f32), one wave per row.
-template <typename TI>
-__global__ __launch_bounds__(SD_THREADS) void sdpa_delta_kernel(const TI* __restrict__ out, const TI* __restrict__ gy,
+template <typename TOUT, typename TGY>
+__global__ __launch_bounds__(SD_THREADS) void sdpa_delta_kernel(const TOUT* __restrict__ out,
+                                                                const TGY* __restrict__ gy,
                                                                 float* __restrict__ delta, long rows, int D) {
   const int lane = threadIdx.x & 63;
   const long row = static_cast<long>(blockIdx.x) * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
   float acc = 0.0f;
-  for (int d = lane; d < D; d += 64) acc += dev_load<TI>(gy, row * D + d) * dev_load<TI>(out, row * D + d);
+  for (int d = lane; d < D; d += 64) acc += dev_load<TGY>(gy, row * D + d) * dev_load<TOUT>(out, row * D + d);
   acc = wave_sum(acc);
   if (lane == 0) delta[row] = acc;
+}
+
+// An f32 attention output as the pair the bf16 MFMA backward reads: hi = bf16(x) and
+// residual = bf16(x - hi), so hi + residual carries x to 2^-17.
+__global__ void sdpa_split_output_kernel(const float* __restrict__ x, unsigned short* __restrict__ hi,
+                                         unsigned short* __restrict__ residual, long n) {
+  for (long i = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += static_cast<long>(gridDim.x) * blockDim.x) {
+    const float v = x[i];
+    const unsigned short h = dev_f32_to_bf16_bits(v);
+    hi[i] = h;
+    residual[i] = dev_f32_to_bf16_bits(v - dev_bf16_bits_to_f32(h));
+  }
 }
 
 // dQ: one wave per query row, the forward's structure with dS in place of P.
@@ -353,23 +369,51 @@ int32_t omx_causal_sdpa_forward(omx_ctx* ctx, const void* q, const void* k, cons
 }
 
 int32_t omx_causal_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, const void* v, const void* out,
-                                 const void* lse, const void* gy, int32_t operand_dtype, void* gq, void* gk, void* gv,
-                                 int32_t grad_dtype, uint64_t batch, uint64_t heads, uint64_t kv_heads, uint64_t time,
-                                 uint64_t head_dim, uint64_t window) {
+                                 const void* lse, const void* gy, int32_t operand_dtype, int32_t out_dtype,
+                                 int32_t gy_dtype, void* gq, void* gk, void* gv, int32_t grad_dtype, uint64_t batch,
+                                 uint64_t heads, uint64_t kv_heads, uint64_t time, uint64_t head_dim,
+                                 uint64_t window) {
   OMX_REQUIRE_CTX(ctx);
   const char* op = "causal_sdpa_backward";
   if (!q || !k || !v || !out || !lse || !gy || !gq || !gk || !gv)
     return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
-  if (!omx_valid_float_dtype(operand_dtype) || !omx_valid_float_dtype(grad_dtype))
+  if (!omx_valid_float_dtype(operand_dtype) || !omx_valid_float_dtype(grad_dtype) ||
+      !omx_valid_float_dtype(out_dtype) || !omx_valid_float_dtype(gy_dtype))
     return omx_fail(ctx, OMX_DTYPE, "%s: dtype must be f32 or bf16", op);
   SdpaShape s;
   int32_t rc = check_shape(ctx, op, batch, heads, kv_heads, time, head_dim, window, &s);
   if (rc != OMX_OK) return rc;
   unsigned long long tag = omx_tag(ctx, F_SDPA_BACKWARD);
-  if (omx_flash_sdpa_supports(head_dim, operand_dtype))
-    return omx_flash_sdpa_backward(ctx, q, k, v, out, nullptr, static_cast<const float*>(lse), gy, gq, gk, gv,
-                                   grad_dtype, batch, heads, kv_heads, time, head_dim, s.window, s.scale, tag, nullptr);
   const long rows = static_cast<long>(batch) * heads * time;
+  const uint64_t n = static_cast<uint64_t>(rows) * head_dim;
+  if (omx_flash_sdpa_supports(head_dim, operand_dtype)) {
+    // The MFMA kernels read bf16: an f32 output goes in as bf16 + rounding residual (nothing of it
+    // is lost to the row term dO . O), an f32 grad_output rounded to bf16.
+    const void* out16 = out;
+    const void* residual = nullptr;
+    const void* gy16 = gy;
+    if (out_dtype == OMX_F32 || gy_dtype == OMX_F32) {
+      void* ws = nullptr;
+      rc = omx_workspace(ctx, 3 * n * 2, &ws, 1);
+      if (rc != OMX_OK) return rc;
+      unsigned short* base = static_cast<unsigned short*>(ws);
+      if (out_dtype == OMX_F32) {
+        const unsigned blocks = static_cast<unsigned>(std::min<uint64_t>((n + 255) / 256, 65536));
+        hipLaunchKernelGGL(sdpa_split_output_kernel, dim3(blocks), dim3(256), 0, ctx->stream,
+                           static_cast<const float*>(out), base, base + n, static_cast<long>(n));
+        OMX_LAUNCH_CHECK(ctx, "sdpa_split_output_kernel");
+        out16 = base;
+        residual = base + n;
+      }
+      if (gy_dtype == OMX_F32) {
+        rc = omx_convert(ctx, gy, OMX_F32, base + 2 * n, OMX_BF16, n);
+        if (rc != OMX_OK) return rc;
+        gy16 = base + 2 * n;
+      }
+    }
+    return omx_flash_sdpa_backward(ctx, q, k, v, out16, residual, static_cast<const float*>(lse), gy16, gq, gk, gv,
+                                   grad_dtype, batch, heads, kv_heads, time, head_dim, s.window, s.scale, tag, nullptr);
+  }
   const long kv_rows = static_cast<long>(batch) * kv_heads * time;
   void* ws = nullptr;
   rc = omx_workspace(ctx, rows * sizeof(float), &ws);
@@ -377,10 +421,27 @@ int32_t omx_causal_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, con
   float* delta = static_cast<float*>(ws);
   dim3 grid(static_cast<unsigned>((rows + 3) / 4)), kv_grid(static_cast<unsigned>((kv_rows + 3) / 4)), block(SD_THREADS);
   const float* lsef = static_cast<const float*>(lse);
+  // The row term reads out and grad_output as they are stored; the two passes read grad_output in
+  // the operands' storage type.
+#define SDPA_DELTA(TOUT, TGY)                                                                                 \
+  hipLaunchKernelGGL((sdpa_delta_kernel<TOUT, TGY>), grid, block, 0, ctx->stream, static_cast<const TOUT*>(out), \
+                     static_cast<const TGY*>(gy), delta, rows, s.dim)
+  if (out_dtype == OMX_F32 && gy_dtype == OMX_F32) SDPA_DELTA(float, float);
+  else if (out_dtype == OMX_F32) SDPA_DELTA(float, unsigned short);
+  else if (gy_dtype == OMX_F32) SDPA_DELTA(unsigned short, float);
+  else SDPA_DELTA(unsigned short, unsigned short);
+#undef SDPA_DELTA
+  OMX_LAUNCH_CHECK(ctx, "sdpa_delta_kernel");
+  if (gy_dtype != operand_dtype) {
+    void* conv = nullptr;
+    rc = omx_workspace(ctx, n * omx_dtype_size(operand_dtype), &conv, 1);
+    if (rc != OMX_OK) return rc;
+    rc = omx_convert(ctx, gy, gy_dtype, conv, operand_dtype, n);
+    if (rc != OMX_OK) return rc;
+    gy = conv;
+  }
 #define SDPA_BWD(TI, TO)                                                                                              \
   do {                                                                                                                \
-    hipLaunchKernelGGL((sdpa_delta_kernel<TI>), grid, block, 0, ctx->stream, static_cast<const TI*>(out),             \
-                       static_cast<const TI*>(gy), delta, rows, s.dim);                                               \
     hipLaunchKernelGGL((sdpa_bwd_dq_rows_kernel<TI, TO>), grid, block, 0, ctx->stream, static_cast<const TI*>(q),     \
                        static_cast<const TI*>(k), static_cast<const TI*>(v), lsef, delta, static_cast<const TI*>(gy), \
                        static_cast<TO*>(gq), s, ctx->fault, tag);                                                     \
@@ -395,6 +456,34 @@ int32_t omx_causal_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, con
 #undef SDPA_BWD
   OMX_LAUNCH_CHECK(ctx, "sdpa backward row kernels");
   return OMX_OK;
+}
+
+int32_t omx_causal_sdpa_backward_recompute(omx_ctx* ctx, const void* q, const void* k, const void* v, const void* gy,
+                                           int32_t operand_dtype, int32_t gy_dtype, void* gq, void* gk, void* gv,
+                                           int32_t grad_dtype, uint64_t batch, uint64_t heads, uint64_t kv_heads,
+                                           uint64_t time, uint64_t head_dim, uint64_t window) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "causal_sdpa_backward_recompute";
+  // The gradient's arguments are checked before the forward runs (backend.rs:1781-1792).
+  if (!q || !k || !v || !gy || !gq || !gk || !gv) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  if (!omx_valid_float_dtype(operand_dtype) || !omx_valid_float_dtype(grad_dtype) || !omx_valid_float_dtype(gy_dtype))
+    return omx_fail(ctx, OMX_DTYPE, "%s: dtype must be f32 or bf16", op);
+  SdpaShape s;
+  int32_t rc = check_shape(ctx, op, batch, heads, kv_heads, time, head_dim, window, &s);
+  if (rc != OMX_OK) return rc;
+  // The forward's output stays f32 (the unrounded O the row term needs) in the library's own scratch.
+  const uint64_t rows = batch * heads * time;
+  const uint64_t out_bytes = (rows * head_dim * 4 + 255) & ~255ull;
+  void* ws = nullptr;
+  rc = omx_workspace(ctx, out_bytes + rows * 4, &ws, 2);
+  if (rc != OMX_OK) return rc;
+  void* out = ws;
+  void* lse = static_cast<char*>(ws) + out_bytes;
+  rc = omx_causal_sdpa_forward(ctx, q, k, v, operand_dtype, out, OMX_F32, lse, batch, heads, kv_heads, time, head_dim,
+                               window);
+  if (rc != OMX_OK) return rc;
+  return omx_causal_sdpa_backward(ctx, q, k, v, out, lse, gy, operand_dtype, OMX_F32, gy_dtype, gq, gk, gv, grad_dtype,
+                                  batch, heads, kv_heads, time, head_dim, window);
 }
 
 // Time-major attention: the permute -> causal_sdpa -> permute of

@@ -247,7 +247,7 @@ int32_t backward(ogpt* t) {
       continue;
     }
     TRY(omx_permute_0213(ctx, t->t_a, t->ga, AD, B, T, H, D));
-    TRY(omx_causal_sdpa_backward(ctx, A.q, A.k, A.v, A.a, A.lse, t->ga, AD, t->gq, t->gk, t->gv, AD, B, H, H, T, D, 0));
+    TRY(omx_causal_sdpa_backward(ctx, A.q, A.k, A.v, A.a, A.lse, t->ga, AD, AD, AD, t->gq, t->gk, t->gv, AD, B, H, H, T, D, 0));
     // h1 feeds q, k, v; their gradients arrive v first, then k, then q.
     TRY(omx_permute_0213(ctx, t->gv, t->t_a, AD, B, H, T, D));
     TRY(omx_linear_backward(ctx, A.h1, t->w(t->li(l, 3)), t->t_a, AD, t->t_b, AD, t->g(t->li(l, 3)), OMX_F32, N, d, d));

@@ -609,3 +609,39 @@ def test_causal_sdpa_bf16_mfma(be, shape, hkv, window):
     close(be.download_f32(gq16), ogq, BF16_TOL, "flash gq bf16")
     close(be.download_f32(gk16), ogk, BF16_TOL, "flash gk bf16")
     close(be.download_f32(gv16), ogv, BF16_TOL, "flash gv bf16")
+
+
+@pytest.mark.parametrize("shape,hkv,window", [((1, 2, 200, 64), 2, None), ((2, 4, 129, 64), 2, 50),
+                                              ((1, 2, 70, 24), 1, None)])
+def test_causal_sdpa_backward_reads_out_and_grad_output_in_their_own_dtypes(be, shape, hkv, window):
+    """bf16 operands with the forward's default f32 output, and an f32 grad_output: the backward
+    reads both as stored (head_dim 64: the MFMA kernels, from bf16 + rounding residual; head_dim
+    24: the row kernels). The gradients must equal those of the oracle on the same values; an
+    output read in the wrong storage type is off by orders of magnitude. Then the one-call
+    recompute form (causal_sdpa_backward_recompute), which runs the forward itself."""
+    from ojas_amd.backend import BF16, F32
+
+    print(f"sdpa backward dtypes {shape} hkv {hkv} window {window}", flush=True)
+    b, h, t, d = shape
+    r = orc.SplitMix64(7700 + t)
+    mk = lambda sh: orc.round_bf16(r.vec(int(np.prod(sh)), 1.0)).reshape(sh)
+    q, k, v = mk((b, h, t, d)), mk((b, hkv, t, d)), mk((b, hkv, t, d))
+    gy = r.vec(b * h * t * d, 1.0).reshape(b, h, t, d)  # f32, not bf16-exact
+    oy, olse = orc.causal_sdpa_forward(q, k, v, window or 0)
+    ogq, ogk, ogv = orc.causal_sdpa_backward(q, k, v, oy, olse, gy, window or 0)
+    dq, dk, dv = (be.upload(a, BF16) for a in (q, k, v))
+    dgy = be.upload(gy)
+    y32, lse = be.causal_sdpa_forward(dq, dk, dv, window)  # default out dtype: f32
+    assert y32.dtype == F32
+    for name, grads in (("saved f32 out", be.causal_sdpa_backward(dq, dk, dv, y32, lse, dgy, window)),
+                        ("recompute", be.causal_sdpa_backward_recompute(dq, dk, dv, dgy, window))):
+        for g, og, what in zip(grads, (ogq, ogk, ogv), ("gq", "gk", "gv")):
+            close(be.download(g), og, BF16_TOL, f"{name}: {what}")
+    # All-f32: the recompute form equals forward + backward bit for bit (same kernels, same order).
+    fq, fk, fv = (be.upload(a) for a in (q, k, v))
+    y, l = be.causal_sdpa_forward(fq, fk, fv, window)
+    two = be.causal_sdpa_backward(fq, fk, fv, y, l, dgy, window)
+    one = be.causal_sdpa_backward_recompute(fq, fk, fv, dgy, window)
+    for a, c2, og in zip(one, two, (ogq, ogk, ogv)):
+        assert np.array_equal(be.download(a), be.download(c2))
+        close(be.download(a), og, F32_TOL, "f32 recompute")
