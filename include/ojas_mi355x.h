@@ -239,6 +239,18 @@ int32_t omx_rms_norm_backward_residual(omx_ctx* ctx, const void* x, int32_t x_dt
 int32_t omx_cross_entropy_mean_forward(omx_ctx* ctx, const void* logits, int32_t logits_dtype,
                                        const void* targets_u32, uint64_t rows, uint64_t vocab,
                                        int32_t has_ignore, uint32_t ignore_index, void* loss_f32);
+/* omx_cross_entropy_mean_forward for callers that cannot allocate (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc). No counterpart in the reference. Same
+ * arguments and result; the row state and the valid counter live in a file-scope device array
+ * (786,688 bytes per device, held until the process ends) instead of the context's workspace,
+ * so the call makes no hipMalloc / hipFree and grows nothing. At most 65536 rows: more is
+ * OMX_CAPACITY_EXCEEDED and nothing runs. Every call on a device shares that array: calls that
+ * overlap on one device (two contexts, two streams) race; calls on one context are stream-ordered
+ * and safe. */
+int32_t omx_cross_entropy_mean_forward_static(omx_ctx* ctx, const void* logits, int32_t logits_dtype,
+                                              const void* targets_u32, uint64_t rows, uint64_t vocab,
+                                              int32_t has_ignore, uint32_t ignore_index,
+                                              void* loss_f32);
 int32_t omx_cross_entropy_mean_backward(omx_ctx* ctx, const void* logits, int32_t logits_dtype,
                                         const void* targets_u32, uint64_t rows, uint64_t vocab,
                                         int32_t has_ignore, uint32_t ignore_index, void* grad,

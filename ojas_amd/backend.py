@@ -457,6 +457,16 @@ class MiBackend:
                                                              hi, iv, self._p(loss)))
         return loss
 
+    def cross_entropy_mean_forward_static(self, logits, targets, loss, ignore_index=None):
+        """`cross_entropy_mean_forward` into a caller-allocated `loss`, through the entry point that
+        allocates nothing (row state in a file-scope device array; at most 65536 rows)."""
+        rows, vocab = logits.shape
+        hi, iv = self._ign(ignore_index)
+        self._check(self._lib.omx_cross_entropy_mean_forward_static(
+            self._ctx, self._p(logits), C.c_int32(logits.dtype), self._p(targets), C.c_uint64(rows),
+            C.c_uint64(vocab), hi, iv, self._p(loss)))
+        return loss
+
     def cross_entropy_mean_backward(self, logits, targets, ignore_index=None, grad_dtype=F32):
         rows, vocab = logits.shape
         grad = self.empty(logits.shape, grad_dtype)

@@ -431,7 +431,34 @@ int32_t check_ce_args(omx_ctx* ctx, const char* op, const void* logits, const vo
   return OMX_OK;
 }
 
+// cross_entropy_mean_forward over caller-chosen scratch (ce_scratch_bytes(rows) bytes at `ws`):
+// every word of the scratch that is read is written first (the valid counter by a fill kernel,
+// the row state by the statistics kernel started with `first`), so stale contents do not matter.
+int32_t ce_forward_in(omx_ctx* ctx, const void* logits, int32_t logits_dtype, const void* targets, uint64_t rows,
+                      uint64_t vocab, int32_t has_ignore, uint32_t ignore_index, void* loss, void* ws) {
+  CeScratch s = carve(ws, rows);
+  const unsigned int* tg = static_cast<const unsigned int*>(targets);
+  unsigned long long tag = omx_tag(ctx, F_CE_FORWARD);
+  int32_t rc = count_valid(ctx, tg, rows, vocab, has_ignore, ignore_index, s.valid, tag);
+  if (rc != OMX_OK) return rc;
+  if (logits_dtype == OMX_F32) launch_stats<float>(ctx, logits, vocab, 0, rows, 0, vocab, tg, s.st, 1, tag);
+  else launch_stats<unsigned short>(ctx, logits, vocab, 0, rows, 0, vocab, tg, s.st, 1, tag);
+  OMX_LAUNCH_CHECK(ctx, "ce_tile_stats_kernel");
+  hipLaunchKernelGGL(ce_mean_kernel, dim3(1), dim3(1024), 0, ctx->stream, s.st, tg, rows, has_ignore, ignore_index,
+                     s.valid, static_cast<float*>(loss), ctx->fault, tag);
+  OMX_LAUNCH_CHECK(ctx, "ce_mean_kernel");
+  return OMX_OK;
+}
+
 }  // namespace
+
+// Scratch of omx_cross_entropy_mean_forward_static: row state (max, sum, target logit) and the
+// valid counter for up to CE_STATIC_MAX_ROWS rows, 786,688 bytes held by every device the library
+// runs on until the process ends. All calls on a device share it.
+constexpr uint64_t CE_STATIC_MAX_ROWS = 65536;
+constexpr int CE_STATIC_MAX_DEVICES = 64;
+static __device__ __align__(256) float g_ce_static_scratch[3 * CE_STATIC_MAX_ROWS + 64];
+static void* g_ce_static_ptr[CE_STATIC_MAX_DEVICES] = {};
 
 extern "C" {
 
@@ -446,18 +473,34 @@ int32_t omx_cross_entropy_mean_forward(omx_ctx* ctx, const void* logits, int32_t
   void* ws = nullptr;
   rc = omx_workspace(ctx, ce_scratch_bytes(rows), &ws);
   if (rc != OMX_OK) return rc;
-  CeScratch s = carve(ws, rows);
-  const unsigned int* tg = static_cast<const unsigned int*>(targets);
-  unsigned long long tag = omx_tag(ctx, F_CE_FORWARD);
-  rc = count_valid(ctx, tg, rows, vocab, has_ignore, ignore_index, s.valid, tag);
+  return ce_forward_in(ctx, logits, logits_dtype, targets, rows, vocab, has_ignore, ignore_index, loss, ws);
+}
+
+int32_t omx_cross_entropy_mean_forward_static(omx_ctx* ctx, const void* logits, int32_t logits_dtype,
+                                              const void* targets, uint64_t rows, uint64_t vocab, int32_t has_ignore,
+                                              uint32_t ignore_index, void* loss) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "cross_entropy_mean_forward_static";
+  int32_t rc = check_ce_args(ctx, op, logits, targets, rows, vocab, logits_dtype);
   if (rc != OMX_OK) return rc;
-  if (logits_dtype == OMX_F32) launch_stats<float>(ctx, logits, vocab, 0, rows, 0, vocab, tg, s.st, 1, tag);
-  else launch_stats<unsigned short>(ctx, logits, vocab, 0, rows, 0, vocab, tg, s.st, 1, tag);
-  OMX_LAUNCH_CHECK(ctx, "ce_tile_stats_kernel");
-  hipLaunchKernelGGL(ce_mean_kernel, dim3(1), dim3(1024), 0, ctx->stream, s.st, tg, rows, has_ignore, ignore_index,
-                     s.valid, static_cast<float*>(loss), ctx->fault, tag);
-  OMX_LAUNCH_CHECK(ctx, "ce_mean_kernel");
-  return OMX_OK;
+  if (!loss) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  if (rows > CE_STATIC_MAX_ROWS)
+    return omx_fail(ctx, OMX_CAPACITY_EXCEEDED, "%s: %llu rows, the static scratch holds at most %llu", op,
+                    (unsigned long long)rows, (unsigned long long)CE_STATIC_MAX_ROWS);
+  if (ctx->device < 0 || ctx->device >= CE_STATIC_MAX_DEVICES)
+    return omx_fail(ctx, OMX_UNSUPPORTED, "%s: device ordinal %d is outside 0..%d", op, ctx->device,
+                    CE_STATIC_MAX_DEVICES - 1);
+  // The array's name is a host-side handle; each device holds its own copy at its own address,
+  // looked up once per device with that device current.
+  void*& ws = g_ce_static_ptr[ctx->device];
+  if (!ws) {
+    OMX_HIP(ctx, hipSetDevice(ctx->device));
+    void* p = nullptr;
+    OMX_HIP(ctx, hipGetSymbolAddress(&p, HIP_SYMBOL(g_ce_static_scratch)));
+    if (!p) return omx_fail(ctx, OMX_BACKEND, "%s: the scratch symbol has no device address", op);
+    ws = p;
+  }
+  return ce_forward_in(ctx, logits, logits_dtype, targets, rows, vocab, has_ignore, ignore_index, loss, ws);
 }
 
 int32_t omx_cross_entropy_mean_backward(omx_ctx* ctx, const void* logits, int32_t logits_dtype, const void* targets,

@@ -1,0 +1,51 @@
+"""The entry point that allocates nothing: omx_cross_entropy_mean_forward_static.
+
+It keeps the row state and the valid counter in a file-scope device array instead
+of the context's workspace. Checked through the C ABI against the existing entry
+point (omx_cross_entropy_mean_forward, same kernels: bit-identical loss) and the
+oracle (f32 tier: 1e-5 relative), on two calls in a row, the second with a smaller
+input so it runs over the first call's stale state; then the size limit.
+"""
+import numpy as np
+import pytest
+
+import oracle_api as orc
+
+pytestmark = pytest.mark.gpu
+
+F32_TOL = 1e-5
+
+
+def test_cross_entropy_forward_static_matches_workspace_form():
+    from ojas_amd.backend import BF16, CAPACITY_EXCEEDED, F32, MiBackend, OjasError
+
+    be = MiBackend(0)
+    try:
+        loss_static = be.empty((1,), F32)
+        cases = [(300, 1000, 7, F32), (41, 257, None, F32), (64, 512, 3, BF16)]
+        for call, (rows, vocab, ignore, dtype) in enumerate(cases):
+            print(f"static ce call {call}: {rows}x{vocab} ignore={ignore} dtype={dtype}", flush=True)
+            r = orc.SplitMix64(4100 + rows)
+            logits = r.vec(rows * vocab, 4.0).reshape(rows, vocab)
+            if dtype == BF16:
+                logits = orc.round_bf16(logits)
+            targets = np.array([(ignore or 0) if i % 9 == 2 else r.below(vocab) for i in range(rows)], np.uint32)
+            dl, dt = be.upload(logits, dtype), be.upload(targets)
+            live = be.budget()["live"]
+            got = be.download(be.cross_entropy_mean_forward_static(dl, dt, loss_static, ignore))[0]
+            assert be.budget()["live"] == live, "the static form must not take memory from the budget"
+            ref = be.download(be.cross_entropy_mean_forward(dl, dt, ignore))[0]
+            assert got.tobytes() == ref.tobytes(), (call, got, ref)
+            want = float(orc.cross_entropy_mean_forward(logits, targets, ignore))
+            tol = F32_TOL if dtype == F32 else 1e-3
+            assert abs(float(got) - want) <= tol * max(1.0, abs(want)), (call, got, want)
+        # Beyond the array's size: refused before anything runs.
+        rows = 65537
+        dl = be.upload(np.zeros((rows, 8), np.float32))
+        dt = be.upload(np.zeros(rows, np.uint32))
+        with pytest.raises(OjasError) as e:
+            be.cross_entropy_mean_forward_static(dl, dt, loss_static)
+        assert e.value.code == CAPACITY_EXCEEDED
+        be.sync()
+    finally:
+        be.close()
