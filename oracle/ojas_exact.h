@@ -201,6 +201,26 @@ void orc_rope_tables(size_t seq, size_t head_dim, double base, float* cos, float
 int orc_nanolab_loss_and_grads(const orc_nanolab_config* c, float* const* params, const uint32_t* ids,
                                const uint32_t* targets, float* loss, float* logits, float* const* grads);
 
+/* ---- symmetric int8 weights in groups along the input axis, and the LoRA step over a frozen
+ * decoder (oracle/lora_exact.cpp; ojas-cpu/src/quant_sparse.rs:284-346 applied per group,
+ * ojas-model/src/lora.rs:292-344) ---- */
+int orc_quantize_i8_group(const float* w, int8_t* codes, float* scales, size_t rows, size_t cols, size_t group);
+int orc_dequant_i8_group(const int8_t* codes, const float* scales, float* w, size_t rows, size_t cols, size_t group);
+int orc_linear_i8_group_forward(const float* x, const int8_t* codes, const float* scales, float* y, size_t rows,
+                                size_t kin, size_t nout, size_t group);
+int orc_linear_i8_group_backward_input(const int8_t* codes, const float* scales, const float* gy, float* gx,
+                                       size_t rows, size_t kin, size_t nout, size_t group);
+typedef struct {
+  uint32_t layers, d_model, heads, head_dim, hidden, vocab, batch, seq, rank;
+  float rms_eps, lora_scale;
+  double rope_base;
+} orc_lora_config;
+size_t orc_lora_frozen_count(const orc_lora_config* c);
+size_t orc_lora_adapter_count(const orc_lora_config* c);
+/* frozen: dequantised f32 tensors; grads (one per adapter tensor) may be NULL for the loss alone. */
+int orc_lora_loss_and_grads(const orc_lora_config* c, const float* const* frozen, const float* const* adapters,
+                            const uint32_t* ids, const uint32_t* targets, float* loss, float* const* grads);
+
 #ifdef __cplusplus
 }
 #endif

@@ -665,3 +665,90 @@ def kv_cache_write(cache, src, at: int):
     _check(_lib.orc_kv_cache_write(_fp(cache), _fp(src), _sz(b), _sz(cap), _sz(hkv), _sz(d), _sz(src.shape[1]), _sz(at)),
            "kv_cache_write")
     return cache
+
+
+# ---- symmetric int8 weights in groups, and the LoRA step (oracle/lora_exact.cpp) ----
+_i8 = C.POINTER(C.c_int8)
+
+
+def quantize_i8_group(w, group: int = 32):
+    """w [rows, cols] -> (codes int8 [rows, cols], scales f32 [rows, cols // group])."""
+    w = _f32(w)
+    rows, cols = w.shape
+    codes = np.empty((rows, cols), np.int8)
+    scales = np.empty((rows, cols // group), np.float32)
+    _check(_lib.orc_quantize_i8_group(_fp(w), codes.ctypes.data_as(_i8), _fp(scales), _sz(rows), _sz(cols), _sz(group)),
+           "quantize_i8_group")
+    return codes, scales
+
+
+def dequant_i8_group(codes, scales, group: int = 32):
+    codes = np.ascontiguousarray(codes, dtype=np.int8)
+    scales = _f32(scales)
+    rows, cols = codes.shape
+    w = np.empty((rows, cols), np.float32)
+    _check(_lib.orc_dequant_i8_group(codes.ctypes.data_as(_i8), _fp(scales), _fp(w), _sz(rows), _sz(cols), _sz(group)),
+           "dequant_i8_group")
+    return w
+
+
+def linear_i8_group_forward(x, codes, scales, group: int = 32):
+    x, codes, scales = _f32(x), np.ascontiguousarray(codes, dtype=np.int8), _f32(scales)
+    rows, kin = x.shape
+    nout = codes.shape[0]
+    y = np.empty((rows, nout), np.float32)
+    _check(_lib.orc_linear_i8_group_forward(_fp(x), codes.ctypes.data_as(_i8), _fp(scales), _fp(y), _sz(rows), _sz(kin),
+                                            _sz(nout), _sz(group)), "linear_i8_group_forward")
+    return y
+
+
+def linear_i8_group_backward_input(codes, scales, gy, group: int = 32):
+    gy, codes, scales = _f32(gy), np.ascontiguousarray(codes, dtype=np.int8), _f32(scales)
+    rows, nout = gy.shape
+    kin = codes.shape[1]
+    gx = np.empty((rows, kin), np.float32)
+    _check(_lib.orc_linear_i8_group_backward_input(codes.ctypes.data_as(_i8), _fp(scales), _fp(gy), _fp(gx), _sz(rows),
+                                                   _sz(kin), _sz(nout), _sz(group)), "linear_i8_group_backward_input")
+    return gx
+
+
+class LoraConfig(C.Structure):
+    _fields_ = [(n, C.c_uint32) for n in ("layers", "d_model", "heads", "head_dim", "hidden", "vocab", "batch", "seq",
+                                          "rank")] + [("rms_eps", C.c_float), ("lora_scale", C.c_float),
+                                                      ("rope_base", C.c_double)]
+
+
+_lib.orc_lora_frozen_count.restype = _sz
+_lib.orc_lora_adapter_count.restype = _sz
+
+LORA_FROZEN_PER_LAYER = ("norm1", "wq", "wk", "wv", "wo", "norm2", "wgate", "wup", "wdown")
+LORA_ADAPTERS_PER_LAYER = ("Aq", "Bq", "Ak", "Bk", "Av", "Bv", "Ao", "Bo")
+
+
+def lora_frozen_shapes(cfg: LoraConfig):
+    d, m = cfg.d_model, cfg.hidden
+    per = [(d,), (d, d), (d, d), (d, d), (d, d), (d,), (m, d), (m, d), (d, m)]
+    return [(cfg.vocab, d)] + per * cfg.layers + [(d,)]
+
+
+def lora_adapter_shapes(cfg: LoraConfig):
+    d, r = cfg.d_model, cfg.rank
+    return [(r, d), (d, r)] * 4 * cfg.layers
+
+
+def lora_loss_and_grads(cfg: LoraConfig, frozen, adapters, ids, targets, want_grads=True):
+    """frozen: dequantised f32 tensors in lora_frozen_shapes order; adapters in lora_adapter_shapes order."""
+    frozen = [_f32(p).reshape(-1) for p in frozen]
+    adapters = [_f32(p).reshape(-1) for p in adapters]
+    assert [p.size for p in frozen] == [int(np.prod(s)) for s in lora_frozen_shapes(cfg)]
+    assert [p.size for p in adapters] == [int(np.prod(s)) for s in lora_adapter_shapes(cfg)]
+    ids = np.ascontiguousarray(ids, dtype=np.uint32).reshape(-1)
+    targets = np.ascontiguousarray(targets, dtype=np.uint32).reshape(-1)
+    grads = [np.zeros_like(p) for p in adapters]
+    fp = (_f * len(frozen))(*[_fp(p) for p in frozen])
+    ap = (_f * len(adapters))(*[_fp(p) for p in adapters])
+    gp = (_f * len(grads))(*[_fp(g) for g in grads]) if want_grads else None
+    loss = C.c_float()
+    _check(_lib.orc_lora_loss_and_grads(C.byref(cfg), fp, ap, _up(ids), _up(targets), C.byref(loss), gp),
+           "lora_loss_and_grads")
+    return np.float32(loss.value), (grads if want_grads else None)
