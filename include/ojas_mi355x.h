@@ -128,6 +128,25 @@ int32_t omx_gemm_strided_batch(omx_ctx* ctx, const void* a, uint64_t a_rs, uint6
                                int32_t c_dtype, uint64_t m, uint64_t k, uint64_t n, int32_t accumulate,
                                uint64_t count, uint64_t stride_a, uint64_t stride_b, uint64_t stride_c);
 
+/* A frozen linear layer whose weight is stored as symmetric int8 codes [n_out, k_in] with one f32
+ * scale per `group` consecutive input columns [n_out, k_in / group] (value = code * scale: the
+ * per-channel form of ojas-cpu/src/quant_sparse.rs:284-346 applied to groups; group must be 32).
+ * The codes are widened inside the product, on their way from HBM to the matrix units; no bf16
+ * copy of the weight exists in memory. In the reference a quantised base reaches the graph as
+ * dequantise -> linear_forward (ojas-autograd/src/tape.rs:1514-1518, backend.rs:2586); these two
+ * entry points serve that pair of calls for a frozen base, forward and input gradient (a frozen
+ * weight has no gradient, ojas-model/src/lora.rs:4-8).
+ * x, y, gy, gx, add: bf16. `add` (optional, the output's shape) is added to the product before the
+ * rounding: the place of the adapter's term in lora_linear (lora.rs:332-344).
+ * forward needs k_in % 32 == 0 and n_out % 4 == 0; the input gradient k_in % 32 == 0 and n_out % 32 == 0. */
+int32_t omx_linear_i8_group_forward(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* codes_i8,
+                                    const void* scales_f32, uint64_t group, const void* add, void* y,
+                                    uint64_t rows, uint64_t k_in, uint64_t n_out);
+int32_t omx_linear_i8_group_backward_input(omx_ctx* ctx, const void* codes_i8, const void* scales_f32,
+                                           uint64_t group, const void* gy, int32_t gy_dtype,
+                                           const void* add, void* gx, uint64_t rows, uint64_t k_in,
+                                           uint64_t n_out);
+
 /* ---- BackendModule::causal_sdpa_forward / _backward (backend.rs:1729-1792).
  *      q,out,gy,gq: [B,H,T,D]; k,v,gk,gv: [B,Hkv,T,D]; lse: [B,H,T] f32.
  *      window = 0: every earlier key. scale = 1/sqrt(D) (backend.rs:159). ---- */

@@ -21,8 +21,9 @@ import numpy as np
 LIB_PATH = Path(__file__).resolve().parent / "libojas_mi355x.so"
 
 F32, BF16, U32 = 0, 1, 2
-_NP_OF = {F32: np.float32, BF16: np.uint16, U32: np.uint32}
-_SIZE_OF = {F32: 4, BF16: 2, U32: 4}
+I8 = 3  # int8 weight codes: a host-side tag only (the entry points that take codes take no dtype for them)
+_NP_OF = {F32: np.float32, BF16: np.uint16, U32: np.uint32, I8: np.int8}
+_SIZE_OF = {F32: 4, BF16: 2, U32: 4, I8: 1}
 
 (OK, SHAPE, DTYPE, OUT_OF_RANGE, NON_FINITE, UNSUPPORTED_HEAD_DIM, CAPACITY_EXCEEDED, POISONED, DEVICE_LOST,
  WAIT_TIMEOUT, BACKEND, UNSUPPORTED, PLACEMENT) = range(13)
@@ -169,6 +170,8 @@ class MiBackend:
             src_dtype = U32
         elif host.dtype == np.uint16:
             src_dtype = BF16
+        elif host.dtype == np.int8:
+            src_dtype = I8
         else:
             raise OjasError(DTYPE, f"upload of {host.dtype}")
         t = self.empty(host.shape, src_dtype)
@@ -254,6 +257,30 @@ class MiBackend:
         self._check(self._lib.omx_linear_backward(self._ctx, None, self._p(w), self._p(gy), C.c_int32(w.dtype),
                                                   self._p(gx), C.c_int32(gx_dtype), None, C.c_int32(F32),
                                                   C.c_uint64(rows), C.c_uint64(kin), C.c_uint64(nout)))
+        return gx
+
+    def linear_i8_group_forward(self, x, codes, scales, add=None, group=32):
+        """y = x W^T (+ add) for a frozen weight held as int8 codes [out, in] and f32 group scales
+        [out, in / group] (value = code * scale); bf16 in, bf16 out."""
+        rows, kin, nout = x.numel // x.shape[-1], x.shape[-1], codes.shape[0]
+        if codes.shape != (nout, kin) or scales.shape != (nout, kin // group) or codes.dtype != I8 or scales.dtype != F32:
+            raise OjasError(SHAPE, f"linear_i8_group_forward: input {x.shape} codes {codes.shape} scales {scales.shape}")
+        y = self.empty(x.shape[:-1] + (nout,), BF16)
+        self._check(self._lib.omx_linear_i8_group_forward(
+            self._ctx, self._p(x), C.c_int32(x.dtype), self._p(codes), self._p(scales), C.c_uint64(group), self._p(add),
+            self._p(y), C.c_uint64(rows), C.c_uint64(kin), C.c_uint64(nout)))
+        return y
+
+    def linear_i8_group_backward_input(self, codes, scales, gy, add=None, group=32):
+        """gx = gy W (+ add) for the same weight form; there is no weight gradient (the base is frozen)."""
+        nout, kin = codes.shape
+        rows = gy.numel // gy.shape[-1]
+        if gy.shape[-1] != nout or scales.shape != (nout, kin // group) or codes.dtype != I8 or scales.dtype != F32:
+            raise OjasError(SHAPE, f"linear_i8_group_backward_input: gy {gy.shape} codes {codes.shape}")
+        gx = self.empty(gy.shape[:-1] + (kin,), BF16)
+        self._check(self._lib.omx_linear_i8_group_backward_input(
+            self._ctx, self._p(codes), self._p(scales), C.c_uint64(group), self._p(gy), C.c_int32(gy.dtype),
+            self._p(add), self._p(gx), C.c_uint64(rows), C.c_uint64(kin), C.c_uint64(nout)))
         return gx
 
     def gemm(self, a: DeviceTensor, a_strides, b: DeviceTensor, b_strides, m, k, n, out_dtype=F32, c=None):

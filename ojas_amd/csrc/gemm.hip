@@ -589,6 +589,31 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
   return rc;
 }
 
+int32_t omx_timing_begin(omx_ctx* ctx, double flops, omx_ctx::TimedLaunch* timed) {
+  *timed = omx_ctx::TimedLaunch{};
+  if (!ctx->profile_gemm) return OMX_OK;
+  auto take = [&](hipEvent_t* e) -> hipError_t {
+    if (!ctx->event_pool.empty()) {
+      *e = ctx->event_pool.back();
+      ctx->event_pool.pop_back();
+      return hipSuccess;
+    }
+    return hipEventCreate(e);
+  };
+  OMX_HIP(ctx, take(&timed->start));
+  OMX_HIP(ctx, take(&timed->stop));
+  timed->flops = flops;
+  ctx->timing_start = timed->start;
+  ctx->timing_stop = timed->stop;
+  return OMX_OK;
+}
+
+void omx_timing_end(omx_ctx* ctx, bool launched, const omx_ctx::TimedLaunch& timed) {
+  if (!ctx->profile_gemm) return;
+  ctx->timing_start = ctx->timing_stop = nullptr;
+  if (launched) ctx->timed.push_back(timed);
+}
+
 extern "C" {
 
 int32_t omx_set_option(omx_ctx* ctx, const char* name, int64_t value) {

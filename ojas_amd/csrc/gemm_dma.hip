@@ -34,120 +34,9 @@
 //   * NST LDS stages: the loads of K steps ks+1 .. ks+NST-1 are in flight while step ks is
 //     multiplied; one counted vmcnt wait + barrier per step.
 // Rows past M (or N) are fetched from a clamped valid address and never stored.
-#include <type_traits>
-
-#include "gemm_args.h"
-
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float floatx16 __attribute__((ext_vector_type(16)));
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
-typedef short short4v __attribute__((ext_vector_type(4)));
+#include "gemm_tiles.h"
 
 namespace {
-
-
-// Per-lane state of one operand's loads: the global address of each of this wave's loads for the
-// current K step (advanced by one step after every issue) and nothing else, so a step costs one
-// 64-bit add per load. ROWS x BK bf16 per step, one wave instruction per KiB.
-template <bool KM, int ROWS, int BK, int NW>  // NW: waves per workgroup
-struct TileLoads {
-  static constexpr int TOTAL = ROWS * BK * 2 / 1024;  // loads per step
-  static constexpr int N = (TOTAL + NW - 1) / NW;     // per wave; the last one only in waves < TOTAL % NW
-  static constexpr bool EVEN = TOTAL % NW == 0;
-  const unsigned short* src[N];
-  long step;  // elements between consecutive K steps
-
-  __device__ __forceinline__ void init(const unsigned short* __restrict__ p, long ld, int row0, int rows, int k0,
-                                       int wave, int lane) {
-#pragma unroll
-    for (int i = 0; i < N; ++i) {
-      const int q = EVEN || wave + NW * i < TOTAL ? wave + NW * i : 0;  // an unused slot gets a valid address
-      if constexpr (!KM) {
-        // [row][BK / 8 chunks of 16 bytes], swizzled as frag_offset reads them.
-        constexpr int LPR = BK / 8;  // lanes (chunks) per row
-        const int r = q * (64 / LPR) + lane / LPR;
-        const int kc = (lane % LPR) ^ (BK == 32 ? (r >> 2) & 3 : (r >> 1) & 7);
-        int gr = row0 + r;
-        gr = gr < rows ? gr : rows - 1;
-        src[i] = p + static_cast<long>(gr) * ld + k0 + kc * 8;
-      } else {
-        constexpr int CPR = ROWS / 8;
-        const int idx = q * 64 + lane;
-        const int kr = idx / CPR, slot = idx % CPR;
-        const int mc = slot ^ ((kr & 3) * 4);
-        int gm = row0 + mc * 8;
-        gm = gm + 8 <= rows ? gm : 0;
-        src[i] = p + static_cast<long>(k0 + kr) * ld + gm;
-      }
-    }
-    step = KM ? BK * ld : BK;
-  }
-  // Starts this step's loads into the operand tile at LDS byte address `tile` and moves on.
-  __device__ __forceinline__ void issue(unsigned tile, int wave) {
-#pragma unroll
-    for (int i = 0; i < N; ++i) {
-      if (!EVEN && wave + NW * i >= TOTAL) break;  // wave-uniform
-      // Written as assembly: the compiler cannot tell that this asynchronous LDS write targets a
-      // stage that is NOT being read, and would otherwise make every LDS read wait for it
-      // (vmcnt(0) right after the issue), which serialises the loads with the products.
-      asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src[i]),
-                   "s"(tile + (wave + NW * i) * 1024)
-                   : "memory");
-      src[i] += step;
-    }
-  }
-};
-
-// Byte offset, inside an operand tile, of this lane's fragment for 32-row block `row_base / 32`
-// and 16-column K slab kk (k-major operands: of its first transposing read; the second is four
-// K rows further).
-template <bool KM, int ROWS, int BK>
-__device__ __forceinline__ int frag_offset(int row_base, int kk, int lane) {
-  if constexpr (!KM) {
-    const int l32 = lane & 31, g = lane >> 5;
-    const int r = row_base + l32;
-    const int kc = kk * 2 + g;
-    return r * (BK * 2) + ((kc ^ (BK == 32 ? (r >> 2) & 3 : (r >> 1) & 7)) << 4);
-  } else {
-    const int s = lane & 15, half = (lane >> 4) & 1, g = lane >> 5;
-    const int kr = kk * 16 + g * 8 + (s >> 2);
-    const int col = row_base + half * 16 + (s & 3) * 4;
-    const int slot = (col >> 3) ^ (((s >> 2) & 3) * 4);
-    return kr * (ROWS * 2) + slot * 16 + (col & 7) * 2;
-  }
-}
-template <bool KM, int ROWS>
-__device__ __forceinline__ u32x4 frag_at(const char* p) {
-  if constexpr (!KM) {
-    return *reinterpret_cast<const u32x4*>(p);
-  } else {
-    typedef short4v __attribute__((address_space(3))) * lds_ptr;
-    short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
-    short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 4 * ROWS * 2));
-    u32x2 a = __builtin_bit_cast(u32x2, lo), b = __builtin_bit_cast(u32x2, hi);
-    return u32x4{a.x, a.y, b.x, b.y};
-  }
-}
-
-// s_waitcnt operand that waits for vmcnt <= n only (vmcnt is bits 3:0 and 15:14).
-constexpr int vmcnt_only(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
-
-// Waves per SIMD the kernel is compiled for: as many workgroups per compute unit as its LDS (160
-// KiB) allows, up to four waves per SIMD.
-constexpr int dma_waves_per_simd(int waves, int lds_bytes) {
-  const int by_lds = 160 * 1024 / lds_bytes, by_waves = 16 / waves;
-  return (by_lds < by_waves ? by_lds : by_waves) * waves / 4;
-}
-
-// f(integral_constant<int, I>) for I = BEGIN .. END - 1.
-template <int BEGIN, int END, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-  if constexpr (BEGIN < END) {
-    f(std::integral_constant<int, BEGIN>{});
-    static_for<BEGIN + 1, END>(f);
-  }
-}
 
 template <bool A_KM, bool B_KM, int WGM, int WGN, int TM, int TN, int DBK, int NST>
 __global__ __launch_bounds__(WGM* WGN * 64, dma_waves_per_simd(WGM* WGN, NST*(WGM* TM + WGN * TN) * 32 * DBK * 2)) void

@@ -1,0 +1,410 @@
+// Dequant-fused bf16 MFMA GEMM over a frozen weight stored as symmetric int8 codes in groups of
+// 32 consecutive input columns with one f32 scale per group (value = code * scale; the
+// reference's per-channel form ojas-cpu/src/quant_sparse.rs:284-346 applied per group).
+//
+//   forward        y[n, o]  = sum_k x[n, k]  * W[o, k]   (+ add[n, o])     ojas-model/src/lora.rs:332-344 `base`
+//   input gradient gx[n, k] = sum_o gy[n, o] * W[o, k]   (+ add[n, k])
+// The weight is frozen, so there is no weight gradient.
+//
+// Data movement, per workgroup (512 threads, tile 256 x 128, 32-column K steps):
+//   * the activation operand goes global -> LDS directly, three stages, as in gemm_dma.hip;
+//   * the codes never exist as bf16 in HBM: waves 0..3 each fetch 1 KiB of codes per step
+//     (global -> LDS directly, 16 codes per lane) plus the lane's group scale, three steps ahead;
+//     the wave that fetched them reads its own 16 bytes back, widens them
+//     (fma(byte ^ 0x80, scale, -128 scale) is code * scale rounded once, then round-to-nearest-even
+//     to bf16) and writes them into the swizzled bf16 tile the MFMA fragments are read from.
+//     Fetch and widening stay inside one wave, so the only synchronisation they add is the
+//     step's barrier, which already publishes the activation tile.
+//   * 48 KiB activation stages + 16 KiB of widened weights (two buffers) + 15 KiB of raw codes and
+//     scales = 79 KiB: two workgroups share a compute unit.
+// HBM traffic per product: the activation once per column band, the codes once per row band at
+// ONE byte per weight, the scales at one eighth of that.
+#include "gemm_tiles.h"
+
+typedef __bf16 bf16x2q __attribute__((ext_vector_type(2)));
+typedef float floatx2q __attribute__((ext_vector_type(2)));
+
+namespace {
+
+struct Q8Args {
+  const unsigned short* a;  // [M][K] bf16, K contiguous
+  long lda;
+  const signed char* codes;  // [nout][kin]
+  const float* scales;       // [nout][kin / 32]
+  long kin;
+  unsigned short* c;  // [M][N] bf16
+  long ldc;
+  const unsigned short* add;  // optional [M][N] bf16 with C's pitch, added before the rounding
+  int M, N, K;
+  int tiles_m, tiles_n;
+  OmxFaultWord* fault;
+  unsigned long long tag;
+};
+
+constexpr int QBM = 256, QBN = 128, QBK = 32, QNW = 8;
+constexpr int Q_A_STAGE = QBM * QBK * 2;            // 16 KiB
+constexpr int Q_B16 = QBN * QBK * 2;                // 8 KiB
+constexpr int Q_OFF_B16 = 3 * Q_A_STAGE;            // two widened-weight buffers
+constexpr int Q_OFF_RAW = Q_OFF_B16 + 2 * Q_B16;    // [3 slots][4 waves][1 KiB] codes
+constexpr int Q_OFF_SCL = Q_OFF_RAW + 3 * 4 * 1024; // [3 slots][4 waves][256 B] scales
+constexpr int Q_SMEM = Q_OFF_SCL + 3 * 4 * 256;     // 79 KiB
+
+__device__ __forceinline__ unsigned int q8_pack2(float a, float b) {
+  floatx2q f = {a, b};
+  return __builtin_bit_cast(unsigned int, __builtin_convertvector(f, bf16x2q));
+}
+
+// Waits until at most `newer` of this wave's loads are outstanding (a wave-uniform count).
+__device__ __forceinline__ void q8_wait_newer(int newer) {
+  if (newer >= 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+  else if (newer == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+  else if (newer == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+// B_KM false: forward (the weight tile is [out row][32 k], k contiguous in memory).
+// B_KM true: input gradient (the weight tile is [32 reduction rows = out][128 columns = k]).
+template <bool B_KM>
+__global__ __launch_bounds__(512, 4) void gemm_q8_kernel(Q8Args g) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  constexpr int TM = 2, TN = 2, WGN = 2, KK = QBK / 16;
+  const int total = g.tiles_m * g.tiles_n;
+  int id = blockIdx.x;
+  // An XCD (workgroups go round-robin by index) takes a contiguous eighth of the tiles.
+  if (total % 8 == 0) id = (id & 7) * (total >> 3) + (id >> 3);
+  const int band = 4;
+  const int tiles_per_band = band * g.tiles_n;
+  const int band_id = id / tiles_per_band;
+  const int first_m = band_id * band;
+  const int band_rows = min(band, g.tiles_m - first_m);
+  const int in_band = id - band_id * tiles_per_band;
+  const int tile_m = first_m + in_band % band_rows;
+  const int tile_n = in_band / band_rows;
+  const int m0 = tile_m * QBM, n0 = tile_n * QBN;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave / WGN, wn = wave % WGN;
+  const int l32 = lane & 31, lg = lane >> 5;
+  const bool feeds_b = wave < 4;  // wave-uniform: this wave fetches and widens a quarter of the weight tile
+
+  floatx16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  const int steps = g.K / QBK;
+  TileLoads<false, QBM, QBK, QNW> la;
+  la.init(g.a, g.lda, m0, g.M, 0, wave, lane);
+  const unsigned lds0 = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(reinterpret_cast<uintptr_t>(smem)));
+
+  // This lane's 16 codes of a step, its scale, and where their 16 bf16 go in the widened tile.
+  const signed char* code_src;
+  const float* scale_src;
+  long code_step, scale_step;
+  int w_off0, w_off1;  // byte offsets of the two 16-byte chunks inside a widened buffer
+  const long groups = g.kin / 32;
+  if constexpr (!B_KM) {
+    const int r = wave * 32 + (lane >> 1), h = lane & 1;  // tile row (output feature), half of its 32 codes
+    int gr = n0 + r;
+    gr = gr < g.N ? gr : g.N - 1;
+    code_src = g.codes + static_cast<long>(gr) * g.kin + h * 16;
+    scale_src = g.scales + static_cast<long>(gr) * groups;
+    code_step = QBK;
+    scale_step = 1;
+    const int x = (r >> 2) & 3;
+    w_off0 = r * 64 + (((2 * h) ^ x) << 4);
+    w_off1 = r * 64 + (((2 * h + 1) ^ x) << 4);
+  } else {
+    const int kr = wave * 8 + (lane >> 3), j = lane & 7;  // reduction row of the step, 16-column piece
+    int gc = n0 + j * 16;
+    gc = gc + 16 <= g.N ? gc : 0;
+    code_src = g.codes + static_cast<long>(kr) * g.kin + gc;
+    scale_src = g.scales + static_cast<long>(kr) * groups + gc / 32;
+    code_step = QBK * g.kin;
+    scale_step = QBK * groups;
+    const int x = (kr & 3) * 4;
+    w_off0 = kr * 256 + (((2 * j) ^ x) << 4);
+    w_off1 = kr * 256 + (((2 * j + 1) ^ x) << 4);
+  }
+  const unsigned raw_lds = lds0 + Q_OFF_RAW + wave * 1024;  // + slot * 4096
+  const unsigned scl_lds = lds0 + Q_OFF_SCL + wave * 256;   // + slot * 1024
+  auto issue_raw = [&](int slot) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(code_src),
+                 "s"(raw_lds + slot * 4096)
+                 : "memory");
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(scale_src),
+                 "s"(scl_lds + slot * 1024)
+                 : "memory");
+    code_src += code_step;
+    scale_src += scale_step;
+  };
+  // Reads this lane's own 16 codes and scale back from slot `slot` and writes 16 bf16 into `dst`.
+  auto widen = [&](int slot, char* dst) {
+    const u32x4 cw = *reinterpret_cast<const u32x4*>(smem + Q_OFF_RAW + slot * 4096 + wave * 1024 + lane * 16);
+    const float sc = *reinterpret_cast<const float*>(smem + Q_OFF_SCL + slot * 1024 + wave * 256 + lane * 4);
+    const float nb = -128.0f * sc;
+    const unsigned int w[4] = {cw.x ^ 0x80808080u, cw.y ^ 0x80808080u, cw.z ^ 0x80808080u, cw.w ^ 0x80808080u};
+    unsigned int o[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float f0 = __builtin_fmaf(static_cast<float>(w[i] & 0xffu), sc, nb);
+      const float f1 = __builtin_fmaf(static_cast<float>((w[i] >> 8) & 0xffu), sc, nb);
+      const float f2 = __builtin_fmaf(static_cast<float>((w[i] >> 16) & 0xffu), sc, nb);
+      const float f3 = __builtin_fmaf(static_cast<float>(w[i] >> 24), sc, nb);
+      o[2 * i] = q8_pack2(f0, f1);
+      o[2 * i + 1] = q8_pack2(f2, f3);
+    }
+    *reinterpret_cast<u32x4*>(dst + w_off0) = u32x4{o[0], o[1], o[2], o[3]};
+    *reinterpret_cast<u32x4*>(dst + w_off1) = u32x4{o[4], o[5], o[6], o[7]};
+  };
+
+  int a_off[TM][KK], b_off[TN][KK];
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk) {
+#pragma unroll
+    for (int t = 0; t < TM; ++t) a_off[t][kk] = frag_offset<false, QBM, QBK>((wm * TM + t) * 32, kk, lane);
+#pragma unroll
+    for (int t = 0; t < TN; ++t) b_off[t][kk] = Q_OFF_B16 + frag_offset<B_KM, QBN, QBK>((wn * TN + t) * 32, kk, lane);
+  }
+
+  // Issue order: raw(0), raw(1), raw(2), A(0), A(1); then per step raw(s + 3), A(s + 2). A wave's
+  // loads complete in order, so the wait for A(s + 1) at the end of step s also covers raw(s + 2).
+  const int raw_loads = feeds_b ? 2 : 0;
+  if (feeds_b) {
+#pragma unroll
+    for (int i = 0; i < 3; ++i)
+      if (i < steps) issue_raw(i);
+  }
+  la.issue(lds0, wave);
+  if (steps > 1) la.issue(lds0 + Q_A_STAGE, wave);
+  q8_wait_newer(steps > 1 ? 2 : 0);  // A(0) and every raw slot issued before it
+  if (feeds_b) widen(0, smem + Q_OFF_B16);
+  __syncthreads();
+
+  u32x4 af[TM], bf[TN];
+  auto read_frags = [&](const char* a_stage, const char* b_buf, int kk, u32x4(&a)[TM], u32x4(&b)[TN]) {
+#pragma unroll
+    for (int t = 0; t < TM; ++t) a[t] = frag_at<false, QBM>(a_stage + a_off[t][kk]);
+#pragma unroll
+    for (int t = 0; t < TN; ++t) b[t] = frag_at<B_KM, QBN>(b_buf + b_off[t][kk]);
+  };
+  read_frags(smem, smem, 0, af, bf);
+  // Step ks reads activation stage sa = ks % 3 and widened buffer sb = ks % 2.
+  auto k_step = [&](int ks, int sa, int sb, int raw_slot_next, int raw_slot_fill) {
+    const char* a_stage = smem + sa * Q_A_STAGE;
+    const char* a_next = smem + ((sa + 1) % 3) * Q_A_STAGE;
+    const char* b_buf = smem + sb * Q_B16;
+    char* b_next = smem + (sb ^ 1) * Q_B16;
+    // The weights of step ks + 1 (landed: they were issued before A(ks), which the previous
+    // step's wait covered) are widened into the buffer step ks - 1 read, released by its barrier.
+    if (feeds_b && ks + 1 < steps) widen(raw_slot_next, b_next + Q_OFF_B16);
+    int newer = 0;
+    if (ks + 3 < steps) {
+      if (feeds_b) issue_raw(raw_slot_fill);
+      newer += raw_loads;
+    }
+    if (ks + 2 < steps) {
+      la.issue(lds0 + ((sa + 2) % 3) * Q_A_STAGE, wave);
+      newer += 2;
+    }
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      u32x4 an[TM], bn[TN];
+#pragma unroll
+      for (int t = 0; t < TM; ++t) an[t] = af[t];
+#pragma unroll
+      for (int t = 0; t < TN; ++t) bn[t] = bf[t];
+      if (kk + 1 < KK) {
+        read_frags(a_stage, b_buf, kk + 1, an, bn);
+      } else {
+        q8_wait_newer(newer);  // A(ks + 1) has landed (this wave's share, then everyone's)
+        __syncthreads();
+        if (ks + 1 < steps) read_frags(a_next, b_next, 0, an, bn);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn)
+          acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[tm]),
+                                                                __builtin_bit_cast(bf16x8, bf[tn]), acc[tm][tn], 0, 0,
+                                                                0);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int t = 0; t < TM; ++t) af[t] = an[t];
+#pragma unroll
+      for (int t = 0; t < TN; ++t) bf[t] = bn[t];
+    }
+  };
+  // Unrolled over the six (stage, buffer) combinations so every LDS address is a precomputed
+  // offset plus a constant.
+  for (int ks = 0; ks < steps;) {
+    bool done = false;
+    static_for<0, 6>([&](auto idx) {
+      constexpr int i = decltype(idx)::value;
+      if (done) return;
+      // raw(j) lives in slot j % 3: step ks widens raw(ks + 1) and refills the slot of raw(ks).
+      k_step(ks, i % 3, i % 2, (i + 1) % 3, i % 3);
+      if (++ks >= steps) done = true;
+    });
+  }
+  __syncthreads();  // the staging below reuses the stages
+
+  // Epilogue: each wave stages 32 rows of its tile at a time through its own LDS region and
+  // writes whole 4-column pieces as bf16.
+  constexpr int CPW = TN * 32 + 4;
+  static_assert(QNW * 32 * CPW * 4 <= Q_SMEM, "staging fits");
+  float* cs = reinterpret_cast<float*>(smem) + wave * (32 * CPW);
+  bool bad = false;
+  static_for<0, TM>([&](auto tm_index) {
+    constexpr int tm = decltype(tm_index)::value;
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) cs[(8 * (v >> 2) + 4 * lg + (v & 3)) * CPW + tn * 32 + l32] = acc[tm][tn][v];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    constexpr int PPR = TN * 8;  // 4-column pieces per row
+    constexpr int ITERS = 32 * PPR / 64;
+    const int grow0 = m0 + (wm * TM + tm) * 32, gcol0 = n0 + wn * TN * 32;
+    const bool interior = grow0 + 32 <= g.M && gcol0 + TN * 32 <= g.N;
+    if (interior) {
+      uint2 addv[ITERS];
+      if (g.add) {
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+          const int c = lane + it * 64, row = c / PPR, piece = c % PPR;
+          addv[it] = *reinterpret_cast<const uint2*>(g.add + static_cast<long>(grow0 + row) * g.ldc + gcol0 + piece * 4);
+        }
+      }
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+        const int c = lane + it * 64, row = c / PPR, piece = c % PPR;
+        float4 val = *reinterpret_cast<const float4*>(cs + row * CPW + piece * 4);
+        if (g.add) {
+          val.x += __uint_as_float(addv[it].x << 16);
+          val.y += __uint_as_float(addv[it].x & 0xffff0000u);
+          val.z += __uint_as_float(addv[it].y << 16);
+          val.w += __uint_as_float(addv[it].y & 0xffff0000u);
+        }
+        bad |= !(dev_finite(val.x) && dev_finite(val.y) && dev_finite(val.z) && dev_finite(val.w));
+        *reinterpret_cast<uint2*>(g.c + static_cast<long>(grow0 + row) * g.ldc + gcol0 + piece * 4) =
+            make_uint2(q8_pack2(val.x, val.y), q8_pack2(val.z, val.w));
+      }
+    } else {
+#pragma unroll 1
+      for (int c = lane; c < 32 * PPR; c += 64) {
+        const int row = c / PPR, piece = c % PPR;
+        const int grow = grow0 + row, gcol = gcol0 + piece * 4;
+        if (grow >= g.M) continue;
+        for (int e = 0; e < 4 && gcol + e < g.N; ++e) {
+          const long off = static_cast<long>(grow) * g.ldc + gcol + e;
+          float v = cs[row * CPW + piece * 4 + e];
+          if (g.add) v += dev_bf16_bits_to_f32(g.add[off]);
+          bad |= !dev_finite(v);
+          g.c[off] = dev_f32_to_bf16_bits(v);
+        }
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  });
+  if (bad) dev_raise_fault(g.fault, g.tag);
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+template <bool B_KM>
+int32_t launch_q8(omx_ctx* ctx, const Q8Args& g, double flops) {
+  auto kernel = &gemm_q8_kernel<B_KM>;
+  OMX_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   Q_SMEM));
+  omx_ctx::TimedLaunch timed{};
+  int32_t rc = omx_timing_begin(ctx, flops, &timed);
+  if (rc != OMX_OK) return rc;
+  omx_launch_timed(ctx, kernel, dim3(g.tiles_m * g.tiles_n), dim3(512), Q_SMEM, ctx->timing_start, ctx->timing_stop, g);
+  hipError_t err = hipGetLastError();
+  omx_timing_end(ctx, err == hipSuccess, timed);
+  if (err != hipSuccess) return omx_hip_fail(ctx, err, "gemm_q8_kernel");
+  return OMX_OK;
+}
+
+int32_t check_q8(omx_ctx* ctx, const char* op, const void* act, const void* codes, const void* scales, const void* out,
+                 const void* add, uint64_t rows, uint64_t kin, uint64_t nout, uint64_t group, int32_t dtype) {
+  if (!act || !codes || !scales || !out) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  if (dtype != OMX_BF16) return omx_fail(ctx, OMX_DTYPE, "%s: activations must be bf16", op);
+  if (rows == 0 || kin == 0 || nout == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
+  if (group != 32) return omx_fail(ctx, OMX_UNSUPPORTED, "%s: group size %llu (only 32)", op, (unsigned long long)group);
+  if (kin % 32 != 0) return omx_fail(ctx, OMX_SHAPE, "%s: k_in %llu is not a multiple of the group", op, (unsigned long long)kin);
+  if (rows > 0x7fffffffull || kin > 0x7fffffffull || nout > 0x7fffffffull)
+    return omx_fail(ctx, OMX_OUT_OF_RANGE, "%s: axis does not fit in i32", op);
+  if (!aligned16(act) || !aligned16(codes) || !aligned16(out) || (add && !aligned16(add)) ||
+      (reinterpret_cast<uintptr_t>(scales) & 3u))
+    return omx_fail(ctx, OMX_SHAPE, "%s: operands must be 16-byte aligned", op);
+  return OMX_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t omx_linear_i8_group_forward(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* codes_i8,
+                                    const void* scales_f32, uint64_t group, const void* add, void* y, uint64_t rows,
+                                    uint64_t kin, uint64_t nout) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "linear_i8_group_forward";
+  int32_t rc = check_q8(ctx, op, x, codes_i8, scales_f32, y, add, rows, kin, nout, group, x_dtype);
+  if (rc != OMX_OK) return rc;
+  if (nout % 4 != 0) return omx_fail(ctx, OMX_SHAPE, "%s: n_out %llu is not a multiple of 4", op, (unsigned long long)nout);
+  Q8Args g{};
+  g.a = static_cast<const unsigned short*>(x);
+  g.lda = static_cast<long>(kin);
+  g.codes = static_cast<const signed char*>(codes_i8);
+  g.scales = static_cast<const float*>(scales_f32);
+  g.kin = static_cast<long>(kin);
+  g.c = static_cast<unsigned short*>(y);
+  g.ldc = static_cast<long>(nout);
+  g.add = static_cast<const unsigned short*>(add);
+  g.M = static_cast<int>(rows);
+  g.N = static_cast<int>(nout);
+  g.K = static_cast<int>(kin);
+  g.tiles_m = (g.M + QBM - 1) / QBM;
+  g.tiles_n = (g.N + QBN - 1) / QBN;
+  g.fault = ctx->fault;
+  g.tag = omx_tag(ctx, F_LINEAR_FORWARD);
+  return launch_q8<false>(ctx, g, 2.0 * rows * kin * nout);
+}
+
+int32_t omx_linear_i8_group_backward_input(omx_ctx* ctx, const void* codes_i8, const void* scales_f32, uint64_t group,
+                                           const void* gy, int32_t gy_dtype, const void* add, void* gx, uint64_t rows,
+                                           uint64_t kin, uint64_t nout) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "linear_i8_group_backward_input";
+  int32_t rc = check_q8(ctx, op, gy, codes_i8, scales_f32, gx, add, rows, kin, nout, group, gy_dtype);
+  if (rc != OMX_OK) return rc;
+  if (nout % 32 != 0)
+    return omx_fail(ctx, OMX_SHAPE, "%s: n_out %llu is not a multiple of 32", op, (unsigned long long)nout);
+  Q8Args g{};
+  g.a = static_cast<const unsigned short*>(gy);
+  g.lda = static_cast<long>(nout);
+  g.codes = static_cast<const signed char*>(codes_i8);
+  g.scales = static_cast<const float*>(scales_f32);
+  g.kin = static_cast<long>(kin);
+  g.c = static_cast<unsigned short*>(gx);
+  g.ldc = static_cast<long>(kin);
+  g.add = static_cast<const unsigned short*>(add);
+  g.M = static_cast<int>(rows);
+  g.N = static_cast<int>(kin);
+  g.K = static_cast<int>(nout);
+  g.tiles_m = (g.M + QBM - 1) / QBM;
+  g.tiles_n = (g.N + QBN - 1) / QBN;
+  g.fault = ctx->fault;
+  g.tag = omx_tag(ctx, F_LINEAR_BACKWARD);
+  return launch_q8<true>(ctx, g, 2.0 * rows * kin * nout);
+}
+
+}  // extern "C"

@@ -111,6 +111,11 @@ inline void omx_launch_timed(omx_ctx* ctx, F kernel, dim3 grid, dim3 block, unsi
 }
 
 int32_t omx_fail(omx_ctx* ctx, omx_status code, const char* fmt, ...);
+// Per-product timing for callers outside gemm.hip: takes a pair of events for the product about
+// to be launched (when omx_profile_gemm is on) and files them with its FLOP count afterwards.
+int32_t omx_timing_begin(omx_ctx* ctx, double flops, omx_ctx::TimedLaunch* timed);
+void omx_timing_end(omx_ctx* ctx, bool launched, const omx_ctx::TimedLaunch& timed);
+
 int32_t omx_hip_fail(omx_ctx* ctx, hipError_t err, const char* what);
 // Grows workspace `slot` to at least `bytes` (budget-charged).
 int32_t omx_workspace(omx_ctx* ctx, uint64_t bytes, void** out, int slot = 0);

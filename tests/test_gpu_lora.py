@@ -1,0 +1,108 @@
+"""GPU parity of the LoRA fine-tune path (int8 group weights, head_dim 128 attention, the step)
+against the oracle (oracle/lora_exact.cpp), through the C ABI."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle_api as orc
+
+pytestmark = pytest.mark.gpu
+
+BF16_TOL = 2e-2  # per element, relative to the tensor's largest value (the bf16 tier's gate)
+
+
+@pytest.fixture(scope="module")
+def be():
+    from ojas_amd.backend import MiBackend
+
+    b = MiBackend(0)
+    yield b
+    b.close()
+
+
+def _close(got, want, tol=BF16_TOL):
+    scale = max(float(np.max(np.abs(want))), 1e-12)
+    err = float(np.max(np.abs(got - want)))
+    assert err <= tol * scale, (err / scale, got.shape)
+
+
+# (rows, k_in, n_out): tile-exact, ragged in every direction, one step, many steps.
+Q8_SHAPES = [(256, 64, 128), (300, 96, 100), (77, 32, 36), (512, 2048, 256), (1024, 256, 416), (33, 704, 160)]
+
+
+@pytest.mark.parametrize("rows,kin,nout", Q8_SHAPES)
+@pytest.mark.parametrize("with_add", [False, True])
+def test_linear_i8_group_forward(be, rows, kin, nout, with_add):
+    from ojas_amd.backend import BF16
+
+    print(f"q8 forward rows={rows} kin={kin} nout={nout} add={with_add}", flush=True)
+    rng = np.random.default_rng(rows * 7 + kin)
+    x = orc.round_bf16(rng.normal(0, 1, (rows, kin)).astype(np.float32))
+    codes, scales = orc.quantize_i8_group(rng.normal(0, 0.05, (nout, kin)).astype(np.float32) *
+                                          rng.uniform(0.2, 3.0, (nout, 1)).astype(np.float32), 32)
+    add = orc.round_bf16(rng.normal(0, 0.3, (rows, nout)).astype(np.float32)) if with_add else None
+    want = orc.linear_i8_group_forward(x, codes, scales, 32) + (add if with_add else 0)
+    y = be.linear_i8_group_forward(be.upload(x, BF16), be.upload(codes), be.upload(scales),
+                                   be.upload(add, BF16) if with_add else None)
+    _close(be.download_f32(y), want)
+
+
+@pytest.mark.parametrize("rows,kin,nout", [(256, 128, 64), (300, 96, 160), (77, 32, 32), (512, 256, 2048),
+                                           (1024, 416, 256), (33, 160, 704)])
+@pytest.mark.parametrize("with_add", [False, True])
+def test_linear_i8_group_backward_input(be, rows, kin, nout, with_add):
+    from ojas_amd.backend import BF16
+
+    print(f"q8 input gradient rows={rows} kin={kin} nout={nout} add={with_add}", flush=True)
+    rng = np.random.default_rng(rows * 5 + nout)
+    gy = orc.round_bf16(rng.normal(0, 1, (rows, nout)).astype(np.float32))
+    codes, scales = orc.quantize_i8_group(rng.normal(0, 0.05, (nout, kin)).astype(np.float32) *
+                                          rng.uniform(0.2, 3.0, (nout, 1)).astype(np.float32), 32)
+    add = orc.round_bf16(rng.normal(0, 0.3, (rows, kin)).astype(np.float32)) if with_add else None
+    want = orc.linear_i8_group_backward_input(codes, scales, gy, 32) + (add if with_add else 0)
+    gx = be.linear_i8_group_backward_input(be.upload(codes), be.upload(scales), be.upload(gy, BF16),
+                                           be.upload(add, BF16) if with_add else None)
+    _close(be.download_f32(gx), want)
+
+
+def test_linear_i8_group_scale_per_group_is_exact(be):
+    # One code per group set, powers of two as scales, a one-hot input: the product is exact in
+    # bf16, so a scale taken from the wrong group or row, or a mis-signed code, shows bit for bit.
+    from ojas_amd.backend import BF16
+
+    nout, kin = 160, 128
+    rng = np.random.default_rng(9)
+    codes = rng.integers(-127, 128, (nout, kin)).astype(np.int8)
+    codes[3, 5], codes[7, 64] = -127, 127
+    scales = (2.0 ** rng.integers(-6, 3, (nout, kin // 32))).astype(np.float32)
+    x = np.eye(kin, dtype=np.float32)  # row k picks column k of W
+    y = be.download_f32(be.linear_i8_group_forward(be.upload(x, BF16), be.upload(codes), be.upload(scales)))
+    want = orc.round_bf16(orc.dequant_i8_group(codes, scales, 32)).T
+    assert np.array_equal(y, want)
+    gy = np.eye(nout, dtype=np.float32)
+    gx = be.download_f32(be.linear_i8_group_backward_input(be.upload(codes), be.upload(scales), be.upload(gy, BF16)))
+    assert np.array_equal(gx, want.T)
+
+
+def test_linear_i8_group_refusals(be):
+    from ojas_amd.backend import BF16, DTYPE, SHAPE, UNSUPPORTED, OjasError
+
+    x = be.upload(np.zeros((8, 48), np.float32), BF16)
+    codes = be.upload(np.zeros((32, 48), np.int8))
+    scales = be.upload(np.zeros((32, 1), np.float32))
+    with pytest.raises(OjasError) as e:  # k_in is not a multiple of the group
+        be._check(be._lib.omx_linear_i8_group_forward(be._ctx, be._p(x), C.c_int32(1), be._p(codes), be._p(scales),
+                                                      C.c_uint64(32), None, be._p(x), C.c_uint64(8), C.c_uint64(48),
+                                                      C.c_uint64(32)))
+    assert e.value.code == SHAPE
+    with pytest.raises(OjasError) as e:
+        be._check(be._lib.omx_linear_i8_group_forward(be._ctx, be._p(x), C.c_int32(1), be._p(codes), be._p(scales),
+                                                      C.c_uint64(64), None, be._p(x), C.c_uint64(8), C.c_uint64(64),
+                                                      C.c_uint64(32)))
+    assert e.value.code == UNSUPPORTED
+    with pytest.raises(OjasError) as e:
+        be._check(be._lib.omx_linear_i8_group_forward(be._ctx, be._p(x), C.c_int32(0), be._p(codes), be._p(scales),
+                                                      C.c_uint64(32), None, be._p(x), C.c_uint64(8), C.c_uint64(64),
+                                                      C.c_uint64(32)))
+    assert e.value.code == DTYPE
