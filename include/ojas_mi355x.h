@@ -138,14 +138,27 @@ int32_t omx_gemm_strided_batch(omx_ctx* ctx, const void* a, uint64_t a_rs, uint6
  * weight has no gradient, ojas-model/src/lora.rs:4-8).
  * x, y, gy, gx, add: bf16. `add` (optional, the output's shape) is added to the product before the
  * rounding: the place of the adapter's term in lora_linear (lora.rs:332-344).
- * forward needs k_in % 32 == 0 and n_out % 4 == 0; the input gradient k_in % 32 == 0 and n_out % 32 == 0. */
+ * forward needs k_in % 32 == 0 and n_out % 4 == 0; the input gradient k_in % 32 == 0 and n_out % 32 == 0.
+ * `layout`: OMX_I8_ROW_MAJOR (codes [n_out, k_in], scales [n_out, k_in / 32]) or OMX_I8_BLOCKED, the
+ * form omx_pack_i8_group writes (same bytes, reordered so that both products read whole cache
+ * lines: blocks of 8 rows x 4 groups, [group % 4][row % 8][32 codes] inside a block, the scales
+ * likewise; needs k_in % 128 == 0 and n_out % 8 == 0). */
+enum { OMX_I8_ROW_MAJOR = 0, OMX_I8_BLOCKED = 1 };
 int32_t omx_linear_i8_group_forward(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* codes_i8,
-                                    const void* scales_f32, uint64_t group, const void* add, void* y,
-                                    uint64_t rows, uint64_t k_in, uint64_t n_out);
+                                    const void* scales_f32, uint64_t group, int32_t layout,
+                                    const void* add, void* y, uint64_t rows, uint64_t k_in,
+                                    uint64_t n_out);
 int32_t omx_linear_i8_group_backward_input(omx_ctx* ctx, const void* codes_i8, const void* scales_f32,
-                                           uint64_t group, const void* gy, int32_t gy_dtype,
-                                           const void* add, void* gx, uint64_t rows, uint64_t k_in,
-                                           uint64_t n_out);
+                                           uint64_t group, int32_t layout, const void* gy,
+                                           int32_t gy_dtype, const void* add, void* gx, uint64_t rows,
+                                           uint64_t k_in, uint64_t n_out);
+/* Reorders row-major codes and scales into the blocked layout (unpack = 0), or a blocked pair back
+ * into row-major (unpack = 1: `codes_i8` / `scales_f32` are then the outputs). Out of place. A
+ * load-time step of this library's own; the reference keeps quantised weights as plain tensors
+ * (ojas-core/src/quant.rs:13-22). */
+int32_t omx_pack_i8_group(omx_ctx* ctx, const void* codes_i8, const void* scales_f32, void* blocked_codes,
+                          void* blocked_scales, uint64_t n_out, uint64_t k_in, uint64_t group,
+                          int32_t unpack);
 
 /* ---- BackendModule::causal_sdpa_forward / _backward (backend.rs:1729-1792).
  *      q,out,gy,gq: [B,H,T,D]; k,v,gk,gv: [B,Hkv,T,D]; lse: [B,H,T] f32.

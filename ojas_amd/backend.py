@@ -259,7 +259,23 @@ class MiBackend:
                                                   C.c_uint64(rows), C.c_uint64(kin), C.c_uint64(nout)))
         return gx
 
-    def linear_i8_group_forward(self, x, codes, scales, add=None, group=32):
+    def pack_i8_group(self, codes, scales, group=32):
+        """Row-major codes and scales -> the blocked layout (`omx_pack_i8_group`); same shapes."""
+        nout, kin = codes.shape
+        bc, bs = self.empty(codes.shape, I8), self.empty(scales.shape, F32)
+        self._check(self._lib.omx_pack_i8_group(self._ctx, self._p(codes), self._p(scales), self._p(bc), self._p(bs),
+                                                C.c_uint64(nout), C.c_uint64(kin), C.c_uint64(group), C.c_int32(0)))
+        return bc, bs
+
+    def unpack_i8_group(self, blocked_codes, blocked_scales, group=32):
+        nout, kin = blocked_codes.shape
+        c, s = self.empty(blocked_codes.shape, I8), self.empty(blocked_scales.shape, F32)
+        self._check(self._lib.omx_pack_i8_group(self._ctx, self._p(c), self._p(s), self._p(blocked_codes),
+                                                self._p(blocked_scales), C.c_uint64(nout), C.c_uint64(kin),
+                                                C.c_uint64(group), C.c_int32(1)))
+        return c, s
+
+    def linear_i8_group_forward(self, x, codes, scales, add=None, group=32, blocked=False):
         """y = x W^T (+ add) for a frozen weight held as int8 codes [out, in] and f32 group scales
         [out, in / group] (value = code * scale); bf16 in, bf16 out."""
         rows, kin, nout = x.numel // x.shape[-1], x.shape[-1], codes.shape[0]
@@ -267,11 +283,11 @@ class MiBackend:
             raise OjasError(SHAPE, f"linear_i8_group_forward: input {x.shape} codes {codes.shape} scales {scales.shape}")
         y = self.empty(x.shape[:-1] + (nout,), BF16)
         self._check(self._lib.omx_linear_i8_group_forward(
-            self._ctx, self._p(x), C.c_int32(x.dtype), self._p(codes), self._p(scales), C.c_uint64(group), self._p(add),
-            self._p(y), C.c_uint64(rows), C.c_uint64(kin), C.c_uint64(nout)))
+            self._ctx, self._p(x), C.c_int32(x.dtype), self._p(codes), self._p(scales), C.c_uint64(group),
+            C.c_int32(1 if blocked else 0), self._p(add), self._p(y), C.c_uint64(rows), C.c_uint64(kin), C.c_uint64(nout)))
         return y
 
-    def linear_i8_group_backward_input(self, codes, scales, gy, add=None, group=32):
+    def linear_i8_group_backward_input(self, codes, scales, gy, add=None, group=32, blocked=False):
         """gx = gy W (+ add) for the same weight form; there is no weight gradient (the base is frozen)."""
         nout, kin = codes.shape
         rows = gy.numel // gy.shape[-1]
@@ -279,8 +295,8 @@ class MiBackend:
             raise OjasError(SHAPE, f"linear_i8_group_backward_input: gy {gy.shape} codes {codes.shape}")
         gx = self.empty(gy.shape[:-1] + (kin,), BF16)
         self._check(self._lib.omx_linear_i8_group_backward_input(
-            self._ctx, self._p(codes), self._p(scales), C.c_uint64(group), self._p(gy), C.c_int32(gy.dtype),
-            self._p(add), self._p(gx), C.c_uint64(rows), C.c_uint64(kin), C.c_uint64(nout)))
+            self._ctx, self._p(codes), self._p(scales), C.c_uint64(group), C.c_int32(1 if blocked else 0), self._p(gy),
+            C.c_int32(gy.dtype), self._p(add), self._p(gx), C.c_uint64(rows), C.c_uint64(kin), C.c_uint64(nout)))
         return gx
 
     def gemm(self, a: DeviceTensor, a_strides, b: DeviceTensor, b_strides, m, k, n, out_dtype=F32, c=None):

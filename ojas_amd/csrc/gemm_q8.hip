@@ -37,9 +37,23 @@ struct Q8Args {
   const unsigned short* add;  // optional [M][N] bf16 with C's pitch, added before the rounding
   int M, N, K;
   int tiles_m, tiles_n;
+  int packed;  // the weight is in the blocked layout of omx_pack_i8_group
   OmxFaultWord* fault;
   unsigned long long tag;
 };
+
+// Blocked weight layout (omx_pack_i8_group): the [n_out, k_in] codes are cut into blocks of 8 output
+// rows x 4 groups (128 input columns), stored block after block in row-major block order; inside a
+// block the group index runs slowest: [group % 4][row % 8][32 codes]. A forward step (32 rows, one
+// group) then reads four runs of 256 contiguous bytes instead of 32 pieces of 32 bytes, and an
+// input-gradient step (8 rows, 128 columns per load) reads whole 1 KiB blocks. The scales are
+// blocked the same way, [group % 4][row % 8] floats per block.
+__device__ __forceinline__ long q8_packed_code_offset(long row, long group, long kin) {
+  return ((row >> 3) * (kin >> 7) + (group >> 2)) * 1024 + (group & 3) * 256 + (row & 7) * 32;
+}
+__device__ __forceinline__ long q8_packed_scale_index(long row, long group, long kin) {
+  return ((row >> 3) * (kin >> 7) + (group >> 2)) * 32 + (group & 3) * 8 + (row & 7);
+}
 
 constexpr int QBM = 256, QBN = 128, QBK = 32, QNW = 8;
 constexpr int Q_A_STAGE = QBM * QBK * 2;            // 16 KiB
@@ -111,10 +125,17 @@ __global__ __launch_bounds__(512, 4) void gemm_q8_kernel(Q8Args g) {
     const int r = wave * 32 + (lane >> 1), h = lane & 1;  // tile row (output feature), half of its 32 codes
     int gr = n0 + r;
     gr = gr < g.N ? gr : g.N - 1;
-    code_src = g.codes + static_cast<long>(gr) * g.kin + h * 16;
-    scale_src = g.scales + static_cast<long>(gr) * groups;
-    code_step = QBK;
-    scale_step = 1;
+    if (g.packed) {
+      code_src = g.codes + q8_packed_code_offset(gr, 0, g.kin) + h * 16;
+      scale_src = g.scales + q8_packed_scale_index(gr, 0, g.kin);
+      code_step = 256;
+      scale_step = 8;
+    } else {
+      code_src = g.codes + static_cast<long>(gr) * g.kin + h * 16;
+      scale_src = g.scales + static_cast<long>(gr) * groups;
+      code_step = QBK;
+      scale_step = 1;
+    }
     const int x = (r >> 2) & 3;
     w_off0 = r * 64 + (((2 * h) ^ x) << 4);
     w_off1 = r * 64 + (((2 * h + 1) ^ x) << 4);
@@ -122,8 +143,13 @@ __global__ __launch_bounds__(512, 4) void gemm_q8_kernel(Q8Args g) {
     const int kr = wave * 8 + (lane >> 3), j = lane & 7;  // reduction row of the step, 16-column piece
     int gc = n0 + j * 16;
     gc = gc + 16 <= g.N ? gc : 0;
-    code_src = g.codes + static_cast<long>(kr) * g.kin + gc;
-    scale_src = g.scales + static_cast<long>(kr) * groups + gc / 32;
+    if (g.packed) {
+      code_src = g.codes + q8_packed_code_offset(kr, gc / 32, g.kin) + (j & 1) * 16;
+      scale_src = g.scales + q8_packed_scale_index(kr, gc / 32, g.kin);
+    } else {
+      code_src = g.codes + static_cast<long>(kr) * g.kin + gc;
+      scale_src = g.scales + static_cast<long>(kr) * groups + gc / 32;
+    }
     code_step = QBK * g.kin;
     scale_step = QBK * groups;
     const int x = (kr & 3) * 4;
@@ -316,6 +342,23 @@ __global__ __launch_bounds__(512, 4) void gemm_q8_kernel(Q8Args g) {
   if (bad) dev_raise_fault(g.fault, g.tag);
 }
 
+// One thread per 16 codes: row-major -> blocked (or back).
+__global__ void q8_pack_kernel(const signed char* __restrict__ src, const float* __restrict__ src_scales,
+                               signed char* __restrict__ dst, float* __restrict__ dst_scales, long nout, long kin,
+                               int unpack) {
+  const long pieces = nout * (kin / 16);
+  const long i = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= pieces) return;
+  const long row = i / (kin / 16), p = i % (kin / 16), group = p >> 1;
+  const long rm = row * kin + p * 16, bl = q8_packed_code_offset(row, group, kin) + (p & 1) * 16;
+  const uint4 v = *reinterpret_cast<const uint4*>(src + (unpack ? bl : rm));
+  *reinterpret_cast<uint4*>(dst + (unpack ? rm : bl)) = v;
+  if ((p & 1) == 0) {
+    const long srm = row * (kin / 32) + group, sbl = q8_packed_scale_index(row, group, kin);
+    dst_scales[unpack ? srm : sbl] = src_scales[unpack ? sbl : srm];
+  }
+}
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 template <bool B_KM>
@@ -334,12 +377,17 @@ int32_t launch_q8(omx_ctx* ctx, const Q8Args& g, double flops) {
 }
 
 int32_t check_q8(omx_ctx* ctx, const char* op, const void* act, const void* codes, const void* scales, const void* out,
-                 const void* add, uint64_t rows, uint64_t kin, uint64_t nout, uint64_t group, int32_t dtype) {
+                 const void* add, uint64_t rows, uint64_t kin, uint64_t nout, uint64_t group, int32_t dtype,
+                 int32_t layout) {
   if (!act || !codes || !scales || !out) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
   if (dtype != OMX_BF16) return omx_fail(ctx, OMX_DTYPE, "%s: activations must be bf16", op);
   if (rows == 0 || kin == 0 || nout == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
   if (group != 32) return omx_fail(ctx, OMX_UNSUPPORTED, "%s: group size %llu (only 32)", op, (unsigned long long)group);
   if (kin % 32 != 0) return omx_fail(ctx, OMX_SHAPE, "%s: k_in %llu is not a multiple of the group", op, (unsigned long long)kin);
+  if (layout != OMX_I8_ROW_MAJOR && layout != OMX_I8_BLOCKED)
+    return omx_fail(ctx, OMX_OUT_OF_RANGE, "%s: weight layout %d", op, layout);
+  if (layout == OMX_I8_BLOCKED && (kin % 128 != 0 || nout % 8 != 0))
+    return omx_fail(ctx, OMX_SHAPE, "%s: the blocked layout needs k_in %% 128 == 0 and n_out %% 8 == 0", op);
   if (rows > 0x7fffffffull || kin > 0x7fffffffull || nout > 0x7fffffffull)
     return omx_fail(ctx, OMX_OUT_OF_RANGE, "%s: axis does not fit in i32", op);
   if (!aligned16(act) || !aligned16(codes) || !aligned16(out) || (add && !aligned16(add)) ||
@@ -353,11 +401,11 @@ int32_t check_q8(omx_ctx* ctx, const char* op, const void* act, const void* code
 extern "C" {
 
 int32_t omx_linear_i8_group_forward(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* codes_i8,
-                                    const void* scales_f32, uint64_t group, const void* add, void* y, uint64_t rows,
-                                    uint64_t kin, uint64_t nout) {
+                                    const void* scales_f32, uint64_t group, int32_t layout, const void* add, void* y,
+                                    uint64_t rows, uint64_t kin, uint64_t nout) {
   OMX_REQUIRE_CTX(ctx);
   const char* op = "linear_i8_group_forward";
-  int32_t rc = check_q8(ctx, op, x, codes_i8, scales_f32, y, add, rows, kin, nout, group, x_dtype);
+  int32_t rc = check_q8(ctx, op, x, codes_i8, scales_f32, y, add, rows, kin, nout, group, x_dtype, layout);
   if (rc != OMX_OK) return rc;
   if (nout % 4 != 0) return omx_fail(ctx, OMX_SHAPE, "%s: n_out %llu is not a multiple of 4", op, (unsigned long long)nout);
   Q8Args g{};
@@ -374,17 +422,18 @@ int32_t omx_linear_i8_group_forward(omx_ctx* ctx, const void* x, int32_t x_dtype
   g.K = static_cast<int>(kin);
   g.tiles_m = (g.M + QBM - 1) / QBM;
   g.tiles_n = (g.N + QBN - 1) / QBN;
+  g.packed = layout == OMX_I8_BLOCKED;
   g.fault = ctx->fault;
   g.tag = omx_tag(ctx, F_LINEAR_FORWARD);
   return launch_q8<false>(ctx, g, 2.0 * rows * kin * nout);
 }
 
 int32_t omx_linear_i8_group_backward_input(omx_ctx* ctx, const void* codes_i8, const void* scales_f32, uint64_t group,
-                                           const void* gy, int32_t gy_dtype, const void* add, void* gx, uint64_t rows,
-                                           uint64_t kin, uint64_t nout) {
+                                           int32_t layout, const void* gy, int32_t gy_dtype, const void* add, void* gx,
+                                           uint64_t rows, uint64_t kin, uint64_t nout) {
   OMX_REQUIRE_CTX(ctx);
   const char* op = "linear_i8_group_backward_input";
-  int32_t rc = check_q8(ctx, op, gy, codes_i8, scales_f32, gx, add, rows, kin, nout, group, gy_dtype);
+  int32_t rc = check_q8(ctx, op, gy, codes_i8, scales_f32, gx, add, rows, kin, nout, group, gy_dtype, layout);
   if (rc != OMX_OK) return rc;
   if (nout % 32 != 0)
     return omx_fail(ctx, OMX_SHAPE, "%s: n_out %llu is not a multiple of 32", op, (unsigned long long)nout);
@@ -402,9 +451,34 @@ int32_t omx_linear_i8_group_backward_input(omx_ctx* ctx, const void* codes_i8, c
   g.K = static_cast<int>(nout);
   g.tiles_m = (g.M + QBM - 1) / QBM;
   g.tiles_n = (g.N + QBN - 1) / QBN;
+  g.packed = layout == OMX_I8_BLOCKED;
   g.fault = ctx->fault;
   g.tag = omx_tag(ctx, F_LINEAR_BACKWARD);
   return launch_q8<true>(ctx, g, 2.0 * rows * kin * nout);
+}
+
+int32_t omx_pack_i8_group(omx_ctx* ctx, const void* codes_i8, const void* scales_f32, void* blocked_codes,
+                          void* blocked_scales, uint64_t nout, uint64_t kin, uint64_t group, int32_t unpack) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "pack_i8_group";
+  if (!codes_i8 || !scales_f32 || !blocked_codes || !blocked_scales)
+    return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  if (group != 32) return omx_fail(ctx, OMX_UNSUPPORTED, "%s: group size %llu (only 32)", op, (unsigned long long)group);
+  if (nout == 0 || kin == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
+  if (kin % 128 != 0 || nout % 8 != 0)
+    return omx_fail(ctx, OMX_SHAPE, "%s: the blocked layout needs k_in %% 128 == 0 and n_out %% 8 == 0", op);
+  if (!aligned16(codes_i8) || !aligned16(blocked_codes) || codes_i8 == blocked_codes || scales_f32 == blocked_scales)
+    return omx_fail(ctx, OMX_SHAPE, "%s: codes must be 16-byte aligned and the copy out of place", op);
+  const long pieces = static_cast<long>(nout) * static_cast<long>(kin / 16);
+  // unpack: the first pair is the blocked form and the second receives the row-major one.
+  const signed char* src = static_cast<const signed char*>(unpack ? blocked_codes : codes_i8);
+  const float* src_s = static_cast<const float*>(unpack ? blocked_scales : scales_f32);
+  signed char* dst = static_cast<signed char*>(unpack ? const_cast<void*>(codes_i8) : blocked_codes);
+  float* dst_s = static_cast<float*>(unpack ? const_cast<void*>(scales_f32) : blocked_scales);
+  hipLaunchKernelGGL(q8_pack_kernel, dim3(static_cast<unsigned>((pieces + 255) / 256)), dim3(256), 0, ctx->stream, src,
+                     src_s, dst, dst_s, static_cast<long>(nout), static_cast<long>(kin), unpack);
+  OMX_LAUNCH_CHECK(ctx, "q8_pack_kernel");
+  return OMX_OK;
 }
 
 }  // extern "C"

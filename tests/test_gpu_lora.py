@@ -85,6 +85,42 @@ def test_linear_i8_group_scale_per_group_is_exact(be):
     assert np.array_equal(gx, want.T)
 
 
+@pytest.mark.parametrize("rows,kin,nout", [(300, 128, 104), (512, 2048, 256), (260, 384, 160)])
+def test_blocked_layout_gives_the_same_products(be, rows, kin, nout):
+    from ojas_amd.backend import BF16
+
+    print(f"q8 blocked rows={rows} kin={kin} nout={nout}", flush=True)
+    rng = np.random.default_rng(rows + kin + nout)
+    x = be.upload(rng.normal(0, 1, (rows, kin)).astype(np.float32), BF16)
+    gy = be.upload(rng.normal(0, 1, (rows, nout)).astype(np.float32), BF16)
+    codes_h = rng.integers(-127, 128, (nout, kin)).astype(np.int8)
+    scales_h = rng.uniform(1e-3, 2e-2, (nout, kin // 32)).astype(np.float32)
+    codes, scales = be.upload(codes_h), be.upload(scales_h)
+    bc, bs = be.pack_i8_group(codes, scales)
+    # The blocked form is a permutation of the same bytes, spelled out here from its definition.
+    r, c = np.meshgrid(np.arange(nout), np.arange(kin), indexing="ij")
+    g = c // 32
+    off = ((r // 8) * (kin // 128) + g // 4) * 1024 + (g % 4) * 256 + (r % 8) * 32 + c % 32
+    want = np.empty(nout * kin, np.int8)
+    want[off.reshape(-1)] = codes_h.reshape(-1)
+    assert np.array_equal(be.download(bc).reshape(-1), want)
+    rs, gs = np.meshgrid(np.arange(nout), np.arange(kin // 32), indexing="ij")
+    soff = ((rs // 8) * (kin // 128) + gs // 4) * 32 + (gs % 4) * 8 + rs % 8
+    swant = np.empty(scales_h.size, np.float32)
+    swant[soff.reshape(-1)] = scales_h.reshape(-1)
+    assert np.array_equal(be.download(bs).reshape(-1), swant)
+    uc, us = be.unpack_i8_group(bc, bs)
+    assert np.array_equal(be.download(uc), codes_h) and np.array_equal(be.download(us), scales_h)
+    # Same arithmetic in the same order: bit-identical products.
+    y0 = be.download(be.linear_i8_group_forward(x, codes, scales))
+    y1 = be.download(be.linear_i8_group_forward(x, bc, bs, blocked=True))
+    assert np.array_equal(y0, y1)
+    if nout % 32 == 0:
+        g0 = be.download(be.linear_i8_group_backward_input(codes, scales, gy))
+        g1 = be.download(be.linear_i8_group_backward_input(bc, bs, gy, blocked=True))
+        assert np.array_equal(g0, g1)
+
+
 def test_linear_i8_group_refusals(be):
     from ojas_amd.backend import BF16, DTYPE, SHAPE, UNSUPPORTED, OjasError
 
@@ -93,16 +129,16 @@ def test_linear_i8_group_refusals(be):
     scales = be.upload(np.zeros((32, 1), np.float32))
     with pytest.raises(OjasError) as e:  # k_in is not a multiple of the group
         be._check(be._lib.omx_linear_i8_group_forward(be._ctx, be._p(x), C.c_int32(1), be._p(codes), be._p(scales),
-                                                      C.c_uint64(32), None, be._p(x), C.c_uint64(8), C.c_uint64(48),
+                                                      C.c_uint64(32), C.c_int32(0), None, be._p(x), C.c_uint64(8), C.c_uint64(48),
                                                       C.c_uint64(32)))
     assert e.value.code == SHAPE
     with pytest.raises(OjasError) as e:
         be._check(be._lib.omx_linear_i8_group_forward(be._ctx, be._p(x), C.c_int32(1), be._p(codes), be._p(scales),
-                                                      C.c_uint64(64), None, be._p(x), C.c_uint64(8), C.c_uint64(64),
+                                                      C.c_uint64(64), C.c_int32(0), None, be._p(x), C.c_uint64(8), C.c_uint64(64),
                                                       C.c_uint64(32)))
     assert e.value.code == UNSUPPORTED
     with pytest.raises(OjasError) as e:
         be._check(be._lib.omx_linear_i8_group_forward(be._ctx, be._p(x), C.c_int32(0), be._p(codes), be._p(scales),
-                                                      C.c_uint64(32), None, be._p(x), C.c_uint64(8), C.c_uint64(64),
+                                                      C.c_uint64(32), C.c_int32(0), None, be._p(x), C.c_uint64(8), C.c_uint64(64),
                                                       C.c_uint64(32)))
     assert e.value.code == DTYPE
