@@ -1,4 +1,4 @@
-// bf16 MFMA flash attention for head_dim 64: causal forward, and the backward
+// bf16 MFMA flash attention for head_dim 64 and 128: causal forward, and the backward
 // as two passes (dK/dV per key block, dQ per query block) that recompute the
 // probabilities from the saved log-sum-exp, so no T x T matrix exists and no
 // atomics are needed (the sums of one output never leave one wavefront).
@@ -32,10 +32,10 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 namespace {
 
-constexpr int FD = 64;              // head dim
-constexpr int FPITCH = 144;         // bytes per LDS row: 64 bf16 + 16 pad
-constexpr int FTILE = 64 * FPITCH;  // a 64-row tile
-constexpr int FT = 256;             // threads per block (4 waves of 32 rows)
+// Head dims 64 and 128 (template argument D of everything below).
+constexpr int fpitch(int D) { return D * 2 + 16; }      // bytes per LDS row: D bf16 + 16 pad
+constexpr int ftile(int D) { return 64 * fpitch(D); }   // a 64-row tile
+constexpr int FT = 256;                                 // threads per block (4 waves of 32 rows)
 constexpr float LOG2E = 1.4426950408889634f;
 
 // Element strides of one tensor: between rows (time steps), heads and batches.
@@ -80,29 +80,35 @@ __device__ __forceinline__ floatx16 zero16() {
   return z;
 }
 
-// A 64-row x 64-column bf16 tile starting at row `row0` of a [time, 64] plane.
-// Thread t moves rows 2(t>>3) and 2(t>>3)+1, 16-byte chunk t&7; rows at or
+// A 64-row x D-column bf16 tile starting at row `row0` of a [time, D] plane: D / 32 16-byte
+// chunks per thread. Thread t moves chunk t % (D/8) of rows t / (D/8) + i * (2048 / D); rows at or
 // past `time` read as zeros.
+template <int D>
 __device__ __forceinline__ void tile_load(const unsigned short* __restrict__ plane, long rs, int row0, int time,
-                                          u32x4 r[2]) {
+                                          u32x4 (&r)[D / 32]) {
+  constexpr int CPR = D / 8, RPP = FT / CPR;
   const int t = threadIdx.x;
-  const int row = row0 + 2 * (t >> 3), kc = t & 7;
+  const int row = row0 + t / CPR, kc = t % CPR;
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < D / 32; ++i) {
     r[i] = u32x4{0u, 0u, 0u, 0u};
-    if (row + i < time) r[i] = *reinterpret_cast<const u32x4*>(plane + static_cast<long>(row + i) * rs + kc * 8);
+    if (row + i * RPP < time)
+      r[i] = *reinterpret_cast<const u32x4*>(plane + static_cast<long>(row + i * RPP) * rs + kc * 8);
   }
 }
 // [row][d] form.
-__device__ __forceinline__ void tile_store_rows(char* lds, const u32x4 r[2]) {
+template <int D>
+__device__ __forceinline__ void tile_store_rows(char* lds, const u32x4 (&r)[D / 32]) {
+  constexpr int CPR = D / 8, RPP = FT / CPR;
   const int t = threadIdx.x;
-  const int row = 2 * (t >> 3), kc = t & 7;
-  *reinterpret_cast<u32x4*>(lds + row * FPITCH + kc * 16) = r[0];
-  *reinterpret_cast<u32x4*>(lds + (row + 1) * FPITCH + kc * 16) = r[1];
+  const int row = t / CPR, kc = t % CPR;
+#pragma unroll
+  for (int i = 0; i < D / 32; ++i) *reinterpret_cast<u32x4*>(lds + (row + i * RPP) * fpitch(D) + kc * 16) = r[i];
 }
 // A operand from a [row][d] tile: rows sub*32 + lane%32, d-slab kk.
+template <int D>
 __device__ __forceinline__ u32x4 frag_rows(const char* lds, int sub, int kk, int l32, int lg) {
-  return *reinterpret_cast<const u32x4*>(lds + (sub * 32 + l32) * FPITCH + kk * 32 + lg * 16);
+  return *reinterpret_cast<const u32x4*>(lds + (sub * 32 + l32) * fpitch(D) + kk * 32 + lg * 16);
 }
 // A operand of a product whose K index is the tile's ROW (O^T = V^T P^T, dV^T = dO^T P,
 // dK^T = Q^T dS, dQ^T = K^T dS^T), read straight from the [row][d] tile with the transposing LDS
@@ -112,7 +118,9 @@ __device__ __forceinline__ u32x4 frag_rows(const char* lds, int sub, int kk, int
 // the B operand, holds its rows.
 typedef short short4v __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+template <int D>
 __device__ __forceinline__ u32x4 frag_tr(const char* lds, int mt, int sub, int c, int lane) {
+  constexpr int FPITCH = fpitch(D);
   const int s = lane & 15, half = (lane >> 4) & 1, g = lane >> 5;
   const char* p = lds + (sub * 32 + c * 16 + 4 * g + (s >> 2)) * FPITCH + (mt * 32 + half * 16 + (s & 3) * 4) * 2;
   typedef short4v __attribute__((address_space(3))) * lds_ptr;
@@ -121,11 +129,12 @@ __device__ __forceinline__ u32x4 frag_tr(const char* lds, int mt, int sub, int c
   const u32x2 a = __builtin_bit_cast(u32x2, lo), b = __builtin_bit_cast(u32x2, hi);
   return u32x4{a.x, a.y, b.x, b.y};
 }
-// B operand held in registers: the lane's own row of a [time, 64] plane.
+// B operand held in registers: the lane's own row of a [time, D] plane.
+template <int D>
 __device__ __forceinline__ void row_frags(const unsigned short* __restrict__ plane, long rs, int row, int time, int lg,
-                                          u32x4 f[4]) {
+                                          u32x4 (&f)[D / 16]) {
 #pragma unroll
-  for (int kk = 0; kk < 4; ++kk) {
+  for (int kk = 0; kk < D / 16; ++kk) {
     f[kk] = u32x4{0u, 0u, 0u, 0u};
     if (row < time) f[kk] = *reinterpret_cast<const u32x4*>(plane + static_cast<long>(row) * rs + kk * 16 + lg * 8);
   }
@@ -133,14 +142,14 @@ __device__ __forceinline__ void row_frags(const unsigned short* __restrict__ pla
 // Row index (within a 32-row sub-tile) that accumulator register v of this lane holds.
 __device__ __forceinline__ int acc_row(int v, int lg) { return 8 * (v >> 2) + 4 * lg + (v & 3); }
 
-// Stores a transposed accumulator pair (d x rows) as rows of a [time, 64] plane.
-template <typename TO>
+// Stores transposed accumulators (d x rows) as rows of a [time, D] plane.
+template <int D, typename TO>
 __device__ __forceinline__ bool store_transposed_acc(TO* __restrict__ plane, long rs, int row, int time, int lg,
-                                                     const floatx16 acc[2], float mul) {
+                                                     const floatx16 (&acc)[D / 32], float mul) {
   bool bad = false;
   if (row >= time) return false;
 #pragma unroll
-  for (int mt = 0; mt < 2; ++mt)
+  for (int mt = 0; mt < D / 32; ++mt)
 #pragma unroll
     for (int q4 = 0; q4 < 4; ++q4) {
       const int d = mt * 32 + 8 * q4 + 4 * lg;
@@ -161,13 +170,14 @@ __device__ __forceinline__ bool store_transposed_acc(TO* __restrict__ plane, lon
 
 // The bf16 store of the output together with what the rounding dropped: residual = x - bf16(x),
 // itself rounded to bf16, so that bf16(x) + residual carries 16 bits of x's mantissa.
+template <int D>
 __device__ __forceinline__ bool store_transposed_acc_split(unsigned short* __restrict__ plane,
                                                            unsigned short* __restrict__ resid, long rs, int row,
-                                                           int time, int lg, const floatx16 acc[2], float mul) {
+                                                           int time, int lg, const floatx16 (&acc)[D / 32], float mul) {
   bool bad = false;
   if (row >= time) return false;
 #pragma unroll
-  for (int mt = 0; mt < 2; ++mt)
+  for (int mt = 0; mt < D / 32; ++mt)
 #pragma unroll
     for (int q4 = 0; q4 < 4; ++q4) {
       const int d = mt * 32 + 8 * q4 + 4 * lg;
@@ -201,15 +211,16 @@ __device__ __forceinline__ void flash_block_of(int pairs, int planes, int* pair,
 }
 
 // ------------------------------------------------------------------ forward
-template <typename TO>
-__global__ __launch_bounds__(FT, 3) void flash_fwd_kernel(const unsigned short* __restrict__ q,
+template <int D, typename TO>
+__global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_fwd_kernel(const unsigned short* __restrict__ q,
                                                        const unsigned short* __restrict__ k,
                                                        const unsigned short* __restrict__ v, TO* __restrict__ out,
                                                        unsigned short* __restrict__ resid, float* __restrict__ lse,
                                                        FlashShape s, OmxFaultWord* fault, unsigned long long tag) {
-  __shared__ __attribute__((aligned(16))) char smem[2 * FTILE];
+  constexpr int KK = D / 16, MT = D / 32, NL = D / 32;  // d slabs, d blocks of the output, loads per thread and tile
+  __shared__ __attribute__((aligned(16))) char smem[2 * ftile(D)];
   char* k_rows = smem;
-  char* v_rows = smem + FTILE;
+  char* v_rows = smem + ftile(D);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lg = lane >> 5;
   const int T = s.time;
   // Query block j sees j / 2 + 1 key tiles (causal): a workgroup takes a late block and then
@@ -229,27 +240,29 @@ __global__ __launch_bounds__(FT, 3) void flash_fwd_kernel(const unsigned short* 
     const unsigned short* vp = v + b * s.kv.bs + kvh * s.kv.hs;
     const int wave_q0 = qb * 128 + wave * 32;
     const int q_row = wave_q0 + l32;
-    u32x4 qf[4];
-    row_frags(qp, s.q.rs, q_row, T, lg, qf);
-    floatx16 o[2] = {zero16(), zero16()};
+    u32x4 qf[KK];
+    row_frags<D>(qp, s.q.rs, q_row, T, lg, qf);
+    floatx16 o[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) o[mt] = zero16();
     float m = -INFINITY, lsum = 0.0f;
     const float scale_log2 = s.scale * LOG2E;
     const int block_q0 = qb * 128, block_q1 = min(T - 1, qb * 128 + 127);
     const int kt_first = s.window > 0 ? max(0, block_q0 + 1 - s.window) / 64 : 0;
     const int kt_last = block_q1 / 64;
     // The next tile's global loads are in flight while the current one is multiplied.
-    u32x4 rk[2], rv[2];
-    tile_load(kp, s.kv.rs, kt_first * 64, T, rk);
-    tile_load(vp, s.kv.rs, kt_first * 64, T, rv);
+    u32x4 rk[NL], rv[NL];
+    tile_load<D>(kp, s.kv.rs, kt_first * 64, T, rk);
+    tile_load<D>(vp, s.kv.rs, kt_first * 64, T, rv);
     for (int kt = kt_first; kt <= kt_last; ++kt) {
       const int key0 = kt * 64;
       __syncthreads();  // the previous tile's reads are done
-      tile_store_rows(k_rows, rk);
-      tile_store_rows(v_rows, rv);
+      tile_store_rows<D>(k_rows, rk);
+      tile_store_rows<D>(v_rows, rv);
       __syncthreads();
       if (kt < kt_last) {
-        tile_load(kp, s.kv.rs, key0 + 64, T, rk);
-        tile_load(vp, s.kv.rs, key0 + 64, T, rv);
+        tile_load<D>(kp, s.kv.rs, key0 + 64, T, rk);
+        tile_load<D>(vp, s.kv.rs, key0 + 64, T, rv);
       }
       const bool active = key0 <= wave_q0 + 31 && (s.window == 0 || key0 + 63 + s.window > wave_q0);
       if (!active) continue;
@@ -257,7 +270,7 @@ __global__ __launch_bounds__(FT, 3) void flash_fwd_kernel(const unsigned short* 
 #pragma unroll
       for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) sc[sub] = mfma(frag_rows(k_rows, sub, kk, l32, lg), qf[kk], sc[sub]);
+        for (int kk = 0; kk < KK; ++kk) sc[sub] = mfma(frag_rows<D>(k_rows, sub, kk, l32, lg), qf[kk], sc[sub]);
       // Only a tile that crosses the diagonal, the sequence end or the window edge needs the mask
       // (wave-uniform). `m` is the running maximum of the raw scores; the scale joins inside the fma.
       if (key0 + 63 > wave_q0 || key0 + 63 >= T || s.window > 0) {
@@ -298,7 +311,7 @@ __global__ __launch_bounds__(FT, 3) void flash_fwd_kernel(const unsigned short* 
         const float alpha = __builtin_amdgcn_exp2f(fmaf(m, scale_log2, neg_m));
         lsum *= alpha;
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt)
+        for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
           for (int vv = 0; vv < 16; ++vv) o[mt][vv] *= alpha;
       }
@@ -310,7 +323,7 @@ __global__ __launch_bounds__(FT, 3) void flash_fwd_kernel(const unsigned short* 
         for (int c = 0; c < 2; ++c) {
           const u32x4 pb = pack8(sc[sub], c);
 #pragma unroll
-          for (int mt = 0; mt < 2; ++mt) o[mt] = mfma(frag_tr(v_rows, mt, sub, c, lane), pb, o[mt]);
+          for (int mt = 0; mt < MT; ++mt) o[mt] = mfma(frag_tr<D>(v_rows, mt, sub, c, lane), pb, o[mt]);
         }
     }
     bool bad = false;
@@ -320,155 +333,187 @@ __global__ __launch_bounds__(FT, 3) void flash_fwd_kernel(const unsigned short* 
     }
     const long o_off = b * s.o.bs + h * s.o.hs;
     if constexpr (sizeof(TO) == 2) {
-      if (resid) bad |= store_transposed_acc_split(out + o_off, resid + o_off, s.o.rs, q_row, T, lg, o, 1.0f / lsum);
-      else bad |= store_transposed_acc<TO>(out + o_off, s.o.rs, q_row, T, lg, o, 1.0f / lsum);
+      if (resid) bad |= store_transposed_acc_split<D>(out + o_off, resid + o_off, s.o.rs, q_row, T, lg, o, 1.0f / lsum);
+      else bad |= store_transposed_acc<D, TO>(out + o_off, s.o.rs, q_row, T, lg, o, 1.0f / lsum);
     } else {
-      bad |= store_transposed_acc<TO>(out + o_off, s.o.rs, q_row, T, lg, o, 1.0f / lsum);
+      bad |= store_transposed_acc<D, TO>(out + o_off, s.o.rs, q_row, T, lg, o, 1.0f / lsum);
     }
     if (bad) dev_raise_fault(fault, tag);
   }  // pass
 }
 
 // ------------------------------------------------------------------ backward: dK, dV
-template <typename TO>
+// One key block of one KV head: the loop over the query tiles that see it, accumulating dK
+// (WANT_DK) and / or dV (WANT_DV) for the wave's 32 keys, then their stores. head_dim 64 runs it
+// once for both. At head_dim 128 the two accumulator sets (128 registers), both key / value
+// fragments (64) and the score tiles do not fit the 256 registers of two waves per SIMD, so the
+// block is walked twice, once per gradient; the second walk recomputes the scores.
+template <int D, typename TO, bool WANT_DK, bool WANT_DV>
+__device__ __forceinline__ bool flash_dkv_block(const unsigned short* __restrict__ q,
+                                                const unsigned short* __restrict__ k,
+                                                const unsigned short* __restrict__ v, const float* __restrict__ lse,
+                                                const float* __restrict__ delta, const unsigned short* __restrict__ gy,
+                                                TO* __restrict__ gk, TO* __restrict__ gv, const FlashShape& s, char* smem,
+                                                int kb, int b, int gidx) {
+  constexpr int KK = D / 16, MT = D / 32, NL = D / 32;
+  char* q_rows = smem;
+  char* g_rows = smem + ftile(D);
+  float* lse_s = reinterpret_cast<float*>(smem + 2 * ftile(D));
+  float* del_s = lse_s + 64;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lg = lane >> 5;
+  const int T = s.time;
+  const long kv_off = b * s.kv.bs + gidx * s.kv.hs;
+  const int wave_k0 = kb * 128 + wave * 32;
+  const int key_row = wave_k0 + l32;
+  u32x4 kf[KK], vf[WANT_DK ? KK : 1];
+  row_frags<D>(k + kv_off, s.kv.rs, key_row, T, lg, kf);
+  if constexpr (WANT_DK) row_frags<D>(v + kv_off, s.kv.rs, key_row, T, lg, vf);
+  floatx16 dk[WANT_DK ? MT : 1], dv[WANT_DV ? MT : 1];
+#pragma unroll
+  for (int mt = 0; mt < (WANT_DK ? MT : 1); ++mt) dk[mt] = zero16();
+#pragma unroll
+  for (int mt = 0; mt < (WANT_DV ? MT : 1); ++mt) dv[mt] = zero16();
+  const float scale_log2 = s.scale * LOG2E;
+  const int block_k0 = kb * 128, block_k1 = min(T - 1, kb * 128 + 127);
+  const int qt_first = block_k0 / 64;
+  const int qt_last = (s.window > 0 ? min(T - 1, block_k1 + s.window - 1) : T - 1) / 64;
+  bool bad = false;
+  // One flat loop over (query head of the group, query tile), ascending, so the
+  // next tile's global loads can be in flight while the current one is multiplied.
+  const int nq = qt_last - qt_first + 1;
+  const int steps = s.rep * nq;
+  u32x4 rq[NL], rg[NL];
+  float row_lse = 0.0f, row_del = 0.0f;
+  // (head of the group, query tile) of the tile being fetched / being multiplied.
+  int fetch_r = 0, fetch_qt = qt_first, cur_qt = qt_first;
+  auto fetch = [&]() {
+    const int r = fetch_r, q0 = fetch_qt * 64;
+    if (++fetch_qt > qt_last) {
+      fetch_qt = qt_first;
+      ++fetch_r;
+    }
+    const long q_plane = static_cast<long>(b) * s.heads + static_cast<long>(gidx) * s.rep + r;
+    const long head = static_cast<long>(gidx) * s.rep + r;
+    tile_load<D>(q + b * s.q.bs + head * s.q.hs, s.q.rs, q0, T, rq);
+    tile_load<D>(gy + b * s.o.bs + head * s.o.hs, s.o.rs, q0, T, rg);
+    row_lse = 0.0f;
+    row_del = 0.0f;
+    if (threadIdx.x < 64 && q0 + static_cast<int>(threadIdx.x) < T) {
+      row_lse = lse[q_plane * T + q0 + threadIdx.x];
+      row_del = delta[q_plane * T + q0 + threadIdx.x];
+      bad |= !(dev_finite(row_lse) && dev_finite(row_del));
+    }
+  };
+  fetch();
+  for (int idx = 0; idx < steps; ++idx) {
+    const int q0 = cur_qt * 64;
+    if (++cur_qt > qt_last) cur_qt = qt_first;
+    __syncthreads();
+    tile_store_rows<D>(q_rows, rq);
+    tile_store_rows<D>(g_rows, rg);
+    if (threadIdx.x < 64) {
+      lse_s[threadIdx.x] = row_lse * LOG2E;
+      del_s[threadIdx.x] = row_del;
+    }
+    __syncthreads();
+    if (idx + 1 < steps) fetch();
+    const bool active = q0 + 63 >= wave_k0 && (s.window == 0 || q0 < wave_k0 + 31 + s.window);
+    if (!active) continue;
+    // Wave-uniform: a tile whose queries all come after the wave's keys and end inside the sequence has no mask.
+    const bool needs_mask = q0 < wave_k0 + 31 || q0 + 63 >= T || s.window > 0;
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub) {
+      floatx16 sc = zero16(), dp = zero16();
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) {
+        sc = mfma(frag_rows<D>(q_rows, sub, kk, l32, lg), kf[kk], sc);
+        if constexpr (WANT_DK) dp = mfma(frag_rows<D>(g_rows, sub, kk, l32, lg), vf[kk], dp);
+      }
+      if (needs_mask) {
+#pragma unroll
+        for (int vv = 0; vv < 16; ++vv) {
+          const int qi = q0 + sub * 32 + acc_row(vv, lg);
+          const bool masked = key_row > qi || qi >= T || key_row >= T || (s.window > 0 && key_row + s.window <= qi);
+          sc[vv] = masked ? -INFINITY : sc[vv];
+        }
+      }
+      // P = 2^(s * scale * log2e - lse * log2e); dS / scale = P (dP - delta): the scale joins dK at the end.
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const float4 l4 = *reinterpret_cast<const float4*>(lse_s + sub * 32 + 8 * q4 + 4 * lg);
+        const float lv[4] = {l4.x, l4.y, l4.z, l4.w};
+        float dl[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if constexpr (WANT_DK) {
+          const float4 d4 = *reinterpret_cast<const float4*>(del_s + sub * 32 + 8 * q4 + 4 * lg);
+          dl[0] = d4.x;
+          dl[1] = d4.y;
+          dl[2] = d4.z;
+          dl[3] = d4.w;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int vv = 4 * q4 + j;
+          const float p = __builtin_amdgcn_exp2f(fmaf(sc[vv], scale_log2, -lv[j]));
+          if constexpr (WANT_DK) dp[vv] = p * (dp[vv] - dl[j]);
+          sc[vv] = p;
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        u32x4 pb = u32x4{0u, 0u, 0u, 0u}, dsb = u32x4{0u, 0u, 0u, 0u};
+        if constexpr (WANT_DV) pb = pack8(sc, c);
+        if constexpr (WANT_DK) dsb = pack8(dp, c);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          if constexpr (WANT_DV) dv[mt] = mfma(frag_tr<D>(g_rows, mt, sub, c, lane), pb, dv[mt]);
+          if constexpr (WANT_DK) dk[mt] = mfma(frag_tr<D>(q_rows, mt, sub, c, lane), dsb, dk[mt]);
+        }
+      }
+    }
+  }
+  if constexpr (WANT_DK) bad |= store_transposed_acc<D, TO>(gk + kv_off, s.kv.rs, key_row, T, lg, dk, s.scale);
+  if constexpr (WANT_DV) bad |= store_transposed_acc<D, TO>(gv + kv_off, s.kv.rs, key_row, T, lg, dv, 1.0f);
+  return bad;
+}
+
+template <int D, typename TO>
 __global__ __launch_bounds__(FT, 2) void flash_bwd_dkv_kernel(
     const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
     const float* __restrict__ lse, const float* __restrict__ delta, const unsigned short* __restrict__ gy,
     TO* __restrict__ gk, TO* __restrict__ gv, FlashShape s, OmxFaultWord* fault, unsigned long long tag) {
-  __shared__ __attribute__((aligned(16))) char smem[2 * FTILE + 2 * 64 * 4];
-  char* q_rows = smem;
-  char* g_rows = smem + FTILE;
-  float* lse_s = reinterpret_cast<float*>(smem + 2 * FTILE);
-  float* del_s = lse_s + 64;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lg = lane >> 5;
-  const int T = s.time;
+  __shared__ __attribute__((aligned(16))) char smem[2 * ftile(D) + 2 * 64 * 4];
   // Early key blocks are seen by the most queries: a workgroup takes one of them and then its
   // mirror image from the back (see the forward kernel).
-  const int k_blocks = (T + 127) / 128;
+  const int k_blocks = (s.time + 127) / 128;
   int pair;
   long kv_plane;
   flash_block_of((k_blocks + 1) / 2, s.batch * s.kv_heads, &pair, &kv_plane);
+  const int gidx = static_cast<int>(kv_plane % s.kv_heads), b = static_cast<int>(kv_plane / s.kv_heads);
+  bool bad = false;
   for (int pass = 0; pass < 2; ++pass) {
     const int kb = pass == 0 ? pair : k_blocks - 1 - pair;
     if (pass == 1 && kb <= pair) break;
-    const int gidx = static_cast<int>(kv_plane % s.kv_heads), b = static_cast<int>(kv_plane / s.kv_heads);
-    const long kv_off = b * s.kv.bs + gidx * s.kv.hs;
-    const unsigned short* kp = k + kv_off;
-    const unsigned short* vp = v + kv_off;
-    const int wave_k0 = kb * 128 + wave * 32;
-    const int key_row = wave_k0 + l32;
-    u32x4 kf[4], vf[4];
-    row_frags(kp, s.kv.rs, key_row, T, lg, kf);
-    row_frags(vp, s.kv.rs, key_row, T, lg, vf);
-    floatx16 dk[2] = {zero16(), zero16()}, dv[2] = {zero16(), zero16()};
-    const float scale_log2 = s.scale * LOG2E;
-    const int block_k0 = kb * 128, block_k1 = min(T - 1, kb * 128 + 127);
-    const int qt_first = block_k0 / 64;
-    const int qt_last = (s.window > 0 ? min(T - 1, block_k1 + s.window - 1) : T - 1) / 64;
-    bool bad = false;
-    // One flat loop over (query head of the group, query tile), ascending, so the
-    // next tile's global loads can be in flight while the current one is multiplied.
-    const int nq = qt_last - qt_first + 1;
-    const int steps = s.rep * nq;
-    u32x4 rq[2], rg[2];
-    float row_lse = 0.0f, row_del = 0.0f;
-    // (head of the group, query tile) of the tile being fetched / being multiplied.
-    int fetch_r = 0, fetch_qt = qt_first, cur_qt = qt_first;
-    auto fetch = [&]() {
-      const int r = fetch_r, q0 = fetch_qt * 64;
-      if (++fetch_qt > qt_last) {
-        fetch_qt = qt_first;
-        ++fetch_r;
-      }
-      const long q_plane = static_cast<long>(b) * s.heads + static_cast<long>(gidx) * s.rep + r;
-      const long head = static_cast<long>(gidx) * s.rep + r;
-      tile_load(q + b * s.q.bs + head * s.q.hs, s.q.rs, q0, T, rq);
-      tile_load(gy + b * s.o.bs + head * s.o.hs, s.o.rs, q0, T, rg);
-      row_lse = 0.0f;
-      row_del = 0.0f;
-      if (threadIdx.x < 64 && q0 + static_cast<int>(threadIdx.x) < T) {
-        row_lse = lse[q_plane * T + q0 + threadIdx.x];
-        row_del = delta[q_plane * T + q0 + threadIdx.x];
-        bad |= !(dev_finite(row_lse) && dev_finite(row_del));
-      }
-    };
-    fetch();
-    for (int idx = 0; idx < steps; ++idx) {
-      {
-        const int q0 = cur_qt * 64;
-        if (++cur_qt > qt_last) cur_qt = qt_first;
-        __syncthreads();
-        tile_store_rows(q_rows, rq);
-        tile_store_rows(g_rows, rg);
-        if (threadIdx.x < 64) {
-          lse_s[threadIdx.x] = row_lse * LOG2E;
-          del_s[threadIdx.x] = row_del;
-        }
-        __syncthreads();
-        if (idx + 1 < steps) fetch();
-        const bool active = q0 + 63 >= wave_k0 && (s.window == 0 || q0 < wave_k0 + 31 + s.window);
-        if (!active) continue;
-        // Wave-uniform: a tile whose queries all come after the wave's keys and end inside the sequence has no mask.
-        const bool needs_mask = q0 < wave_k0 + 31 || q0 + 63 >= T || s.window > 0;
-#pragma unroll
-        for (int sub = 0; sub < 2; ++sub) {
-          floatx16 sc = zero16(), dp = zero16();
-#pragma unroll
-          for (int kk = 0; kk < 4; ++kk) {
-            sc = mfma(frag_rows(q_rows, sub, kk, l32, lg), kf[kk], sc);
-            dp = mfma(frag_rows(g_rows, sub, kk, l32, lg), vf[kk], dp);
-          }
-          if (needs_mask) {
-#pragma unroll
-            for (int vv = 0; vv < 16; ++vv) {
-              const int qi = q0 + sub * 32 + acc_row(vv, lg);
-              const bool masked =
-                  key_row > qi || qi >= T || key_row >= T || (s.window > 0 && key_row + s.window <= qi);
-              sc[vv] = masked ? -INFINITY : sc[vv];
-            }
-          }
-          // P = 2^(s * scale * log2e - lse * log2e); dS / scale = P (dP - delta): the scale joins dK at the end.
-#pragma unroll
-          for (int q4 = 0; q4 < 4; ++q4) {
-            const float4 l4 = *reinterpret_cast<const float4*>(lse_s + sub * 32 + 8 * q4 + 4 * lg);
-            const float4 d4 = *reinterpret_cast<const float4*>(del_s + sub * 32 + 8 * q4 + 4 * lg);
-            const float lv[4] = {l4.x, l4.y, l4.z, l4.w}, dl[4] = {d4.x, d4.y, d4.z, d4.w};
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              const int vv = 4 * q4 + j;
-              const float p = __builtin_amdgcn_exp2f(fmaf(sc[vv], scale_log2, -lv[j]));
-              dp[vv] = p * (dp[vv] - dl[j]);
-              sc[vv] = p;
-            }
-          }
-#pragma unroll
-          for (int c = 0; c < 2; ++c) {
-            const u32x4 pb = pack8(sc, c), dsb = pack8(dp, c);
-#pragma unroll
-            for (int mt = 0; mt < 2; ++mt) {
-              dv[mt] = mfma(frag_tr(g_rows, mt, sub, c, lane), pb, dv[mt]);
-              dk[mt] = mfma(frag_tr(q_rows, mt, sub, c, lane), dsb, dk[mt]);
-            }
-          }
-        }
-      }
+    if constexpr (D == 64) {
+      bad |= flash_dkv_block<D, TO, true, true>(q, k, v, lse, delta, gy, gk, gv, s, smem, kb, b, gidx);
+    } else {
+      bad |= flash_dkv_block<D, TO, false, true>(q, k, v, lse, delta, gy, gk, gv, s, smem, kb, b, gidx);
+      bad |= flash_dkv_block<D, TO, true, false>(q, k, v, lse, delta, gy, gk, gv, s, smem, kb, b, gidx);
     }
-    bad |= store_transposed_acc<TO>(gk + kv_off, s.kv.rs, key_row, T, lg, dk, s.scale);
-    bad |= store_transposed_acc<TO>(gv + kv_off, s.kv.rs, key_row, T, lg, dv, 1.0f);
-    if (bad) dev_raise_fault(fault, tag);
-  }  // pass
+  }
+  if (bad) dev_raise_fault(fault, tag);
 }
 
 // ------------------------------------------------------------------ backward: dQ
-template <typename TO>
-__global__ __launch_bounds__(FT, 3) void flash_bwd_dq_kernel(
+template <int D, typename TO>
+__global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_bwd_dq_kernel(
     const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
     const unsigned short* __restrict__ out, const unsigned short* __restrict__ resid, const float* __restrict__ lse,
     float* __restrict__ delta, const unsigned short* __restrict__ gy, TO* __restrict__ gq, FlashShape s,
     OmxFaultWord* fault, unsigned long long tag) {
-  __shared__ __attribute__((aligned(16))) char smem[2 * FTILE];
+  constexpr int KK = D / 16, MT = D / 32, NL = D / 32;
+  __shared__ __attribute__((aligned(16))) char smem[2 * ftile(D)];
   char* k_rows = smem;
-  char* v_rows = smem + FTILE;
+  char* v_rows = smem + ftile(D);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lg = lane >> 5;
   const int T = s.time;
   // A late query block, then its mirror image from the front (see the forward kernel).
@@ -485,10 +530,10 @@ __global__ __launch_bounds__(FT, 3) void flash_bwd_dq_kernel(
     const unsigned short* vp = v + b * s.kv.bs + kvh * s.kv.hs;
     const int wave_q0 = qb * 128 + wave * 32;
     const int q_row = wave_q0 + l32;
-    u32x4 qf[4], gf[4];
-    row_frags(q + b * s.q.bs + h * s.q.hs, s.q.rs, q_row, T, lg, qf);
-    row_frags(gy + b * s.o.bs + h * s.o.hs, s.o.rs, q_row, T, lg, gf);
-    // delta = dO . O of this lane's row: each half-wave holds half of the row's 64 values. The
+    u32x4 qf[KK], gf[KK];
+    row_frags<D>(q + b * s.q.bs + h * s.q.hs, s.q.rs, q_row, T, lg, qf);
+    row_frags<D>(gy + b * s.o.bs + h * s.o.hs, s.o.rs, q_row, T, lg, gf);
+    // delta = dO . O of this lane's row: each half-wave holds half of the row's values. The
     // dK/dV pass, launched after this one, reads it back from `delta`. dS = P (dP - delta) sums to
     // zero along a row only as far as delta matches sum_j P dP: taken from the bf16 output alone it
     // is off by 2^-9 of |dO| |O|, which a component shared by all value rows (and by all key rows,
@@ -497,11 +542,11 @@ __global__ __launch_bounds__(FT, 3) void flash_bwd_dq_kernel(
     float row_del = 0.0f;
     {
       auto dot_rows = [&](const unsigned short* plane) {
-        u32x4 of[4];
-        row_frags(plane + b * s.o.bs + h * s.o.hs, s.o.rs, q_row, T, lg, of);
+        u32x4 of[KK];
+        row_frags<D>(plane + b * s.o.bs + h * s.o.hs, s.o.rs, q_row, T, lg, of);
         float sum = 0.0f;
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
+        for (int kk = 0; kk < KK; ++kk) {
           const unsigned int gw[4] = {gf[kk].x, gf[kk].y, gf[kk].z, gf[kk].w};
           const unsigned int ow[4] = {of[kk].x, of[kk].y, of[kk].z, of[kk].w};
 #pragma unroll
@@ -524,23 +569,25 @@ __global__ __launch_bounds__(FT, 3) void flash_bwd_dq_kernel(
       bad |= !(dev_finite(row_lse) && dev_finite(row_del));
     }
     const float neg_lse = -row_lse * LOG2E;
-    floatx16 dq[2] = {zero16(), zero16()};
+    floatx16 dq[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) dq[mt] = zero16();
     const float scale_log2 = s.scale * LOG2E;
     const int block_q0 = qb * 128, block_q1 = min(T - 1, qb * 128 + 127);
     const int kt_first = s.window > 0 ? max(0, block_q0 + 1 - s.window) / 64 : 0;
     const int kt_last = block_q1 / 64;
-    u32x4 rk[2], rv[2];
-    tile_load(kp, s.kv.rs, kt_first * 64, T, rk);
-    tile_load(vp, s.kv.rs, kt_first * 64, T, rv);
+    u32x4 rk[NL], rv[NL];
+    tile_load<D>(kp, s.kv.rs, kt_first * 64, T, rk);
+    tile_load<D>(vp, s.kv.rs, kt_first * 64, T, rv);
     for (int kt = kt_first; kt <= kt_last; ++kt) {
       const int key0 = kt * 64;
       __syncthreads();
-      tile_store_rows(k_rows, rk);
-      tile_store_rows(v_rows, rv);
+      tile_store_rows<D>(k_rows, rk);
+      tile_store_rows<D>(v_rows, rv);
       __syncthreads();
       if (kt < kt_last) {
-        tile_load(kp, s.kv.rs, key0 + 64, T, rk);
-        tile_load(vp, s.kv.rs, key0 + 64, T, rv);
+        tile_load<D>(kp, s.kv.rs, key0 + 64, T, rk);
+        tile_load<D>(vp, s.kv.rs, key0 + 64, T, rv);
       }
       const bool active = key0 <= wave_q0 + 31 && (s.window == 0 || key0 + 63 + s.window > wave_q0);
       if (!active) continue;
@@ -549,9 +596,9 @@ __global__ __launch_bounds__(FT, 3) void flash_bwd_dq_kernel(
       for (int sub = 0; sub < 2; ++sub) {
         floatx16 sc = zero16(), dp = zero16();
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-          sc = mfma(frag_rows(k_rows, sub, kk, l32, lg), qf[kk], sc);
-          dp = mfma(frag_rows(v_rows, sub, kk, l32, lg), gf[kk], dp);
+        for (int kk = 0; kk < KK; ++kk) {
+          sc = mfma(frag_rows<D>(k_rows, sub, kk, l32, lg), qf[kk], sc);
+          dp = mfma(frag_rows<D>(v_rows, sub, kk, l32, lg), gf[kk], dp);
         }
         if (needs_mask) {
 #pragma unroll
@@ -570,21 +617,21 @@ __global__ __launch_bounds__(FT, 3) void flash_bwd_dq_kernel(
         for (int c = 0; c < 2; ++c) {
           const u32x4 dsb = pack8(dp, c);
 #pragma unroll
-          for (int mt = 0; mt < 2; ++mt) dq[mt] = mfma(frag_tr(k_rows, mt, sub, c, lane), dsb, dq[mt]);
+          for (int mt = 0; mt < MT; ++mt) dq[mt] = mfma(frag_tr<D>(k_rows, mt, sub, c, lane), dsb, dq[mt]);
         }
       }
     }
-    bad |= store_transposed_acc<TO>(gq + b * s.q.bs + h * s.q.hs, s.q.rs, q_row, T, lg, dq, s.scale);
+    bad |= store_transposed_acc<D, TO>(gq + b * s.q.bs + h * s.q.hs, s.q.rs, q_row, T, lg, dq, s.scale);
     if (bad) dev_raise_fault(fault, tag);
   }  // pass
 }
 
 // `strides`: nine element strides (row, head, batch of q; of k / v; of out), or null for
-// contiguous [batch, heads, time, 64] tensors.
-FlashShape make_shape(uint64_t batch, uint64_t heads, uint64_t kv_heads, uint64_t time, uint64_t window, float scale,
-                      const long* strides) {
+// contiguous [batch, heads, time, dim] tensors.
+FlashShape make_shape(uint64_t batch, uint64_t heads, uint64_t kv_heads, uint64_t time, uint64_t dim, uint64_t window,
+                      float scale, const long* strides) {
   FlashShape s;
-  const long T = static_cast<long>(time);
+  const long T = static_cast<long>(time), FD = static_cast<long>(dim);
   s.q = {FD, T * FD, static_cast<long>(heads) * T * FD};
   s.kv = {FD, T * FD, static_cast<long>(kv_heads) * T * FD};
   s.o = s.q;
@@ -603,28 +650,62 @@ FlashShape make_shape(uint64_t batch, uint64_t heads, uint64_t kv_heads, uint64_
   return s;
 }
 
+template <int D>
+void launch_forward(omx_ctx* ctx, const unsigned short* q, const unsigned short* k, const unsigned short* v, void* out,
+                    int32_t out_dtype, void* out_residual, float* lse, const FlashShape& s, unsigned long long tag) {
+  // Two 128-row query blocks per workgroup (see the kernel).
+  dim3 grid(static_cast<unsigned>((s.time + 127) / 128 + 1) / 2 * s.batch * s.heads), block(FT);
+  if (out_dtype == OMX_BF16)
+    hipLaunchKernelGGL((flash_fwd_kernel<D, unsigned short>), grid, block, 0, ctx->stream, q, k, v,
+                       static_cast<unsigned short*>(out), static_cast<unsigned short*>(out_residual), lse, s,
+                       ctx->fault, tag);
+  else
+    hipLaunchKernelGGL((flash_fwd_kernel<D, float>), grid, block, 0, ctx->stream, q, k, v, static_cast<float*>(out),
+                       static_cast<unsigned short*>(nullptr), lse, s, ctx->fault, tag);
+}
+
+template <int D>
+void launch_backward(omx_ctx* ctx, const unsigned short* q, const unsigned short* k, const unsigned short* v,
+                     const unsigned short* out, const unsigned short* resid, const float* lse, float* delta,
+                     const unsigned short* gy, void* gq, void* gk, void* gv, int32_t grad_dtype, const FlashShape& s,
+                     unsigned long long tag) {
+  // dQ first: it also leaves delta = dO . O per row for the dK/dV pass.
+  dim3 block(FT);
+  const unsigned pairs = static_cast<unsigned>((s.time + 127) / 128 + 1) / 2;  // two 128-row blocks per workgroup
+  dim3 kv_grid(pairs * static_cast<unsigned>(s.batch * s.kv_heads));
+  dim3 q_grid(pairs * static_cast<unsigned>(s.batch * s.heads));
+  if (grad_dtype == OMX_BF16) {
+    hipLaunchKernelGGL((flash_bwd_dq_kernel<D, unsigned short>), q_grid, block, 0, ctx->stream, q, k, v, out, resid,
+                       lse, delta, gy, static_cast<unsigned short*>(gq), s, ctx->fault, tag);
+    hipLaunchKernelGGL((flash_bwd_dkv_kernel<D, unsigned short>), kv_grid, block, 0, ctx->stream, q, k, v, lse, delta,
+                       gy, static_cast<unsigned short*>(gk), static_cast<unsigned short*>(gv), s, ctx->fault, tag);
+  } else {
+    hipLaunchKernelGGL((flash_bwd_dq_kernel<D, float>), q_grid, block, 0, ctx->stream, q, k, v, out, resid, lse, delta,
+                       gy, static_cast<float*>(gq), s, ctx->fault, tag);
+    hipLaunchKernelGGL((flash_bwd_dkv_kernel<D, float>), kv_grid, block, 0, ctx->stream, q, k, v, lse, delta, gy,
+                       static_cast<float*>(gk), static_cast<float*>(gv), s, ctx->fault, tag);
+  }
+}
+
 }  // namespace
 
-bool omx_flash_sdpa_supports(uint64_t dim, int32_t operand_dtype) { return dim == FD && operand_dtype == OMX_BF16; }
+bool omx_flash_sdpa_supports(uint64_t dim, int32_t operand_dtype) {
+  return (dim == 64 || dim == 128) && operand_dtype == OMX_BF16;
+}
 
 int32_t omx_flash_sdpa_forward(omx_ctx* ctx, const void* q, const void* k, const void* v, void* out, int32_t out_dtype,
                                void* out_residual, float* lse, uint64_t batch, uint64_t heads, uint64_t kv_heads,
                                uint64_t time, uint64_t dim, uint64_t window, float scale, unsigned long long tag,
                                const long* strides) {
-  if (dim != FD) return omx_fail(ctx, OMX_UNSUPPORTED_HEAD_DIM, "head_dim %llu limit %d", (unsigned long long)dim, FD);
-  FlashShape s = make_shape(batch, heads, kv_heads, time, window, scale, strides);
-  // Two 128-row query blocks per workgroup (see the kernel).
-  dim3 grid(static_cast<unsigned>(((time + 127) / 128 + 1) / 2 * batch * heads)), block(FT);
+  if (dim != 64 && dim != 128)
+    return omx_fail(ctx, OMX_UNSUPPORTED_HEAD_DIM, "head_dim %llu: the MFMA kernels take 64 and 128",
+                    (unsigned long long)dim);
+  FlashShape s = make_shape(batch, heads, kv_heads, time, dim, window, scale, strides);
   const unsigned short* qs = static_cast<const unsigned short*>(q);
   const unsigned short* ks = static_cast<const unsigned short*>(k);
   const unsigned short* vs = static_cast<const unsigned short*>(v);
-  if (out_dtype == OMX_BF16)
-    hipLaunchKernelGGL((flash_fwd_kernel<unsigned short>), grid, block, 0, ctx->stream, qs, ks, vs,
-                       static_cast<unsigned short*>(out), static_cast<unsigned short*>(out_residual), lse, s,
-                       ctx->fault, tag);
-  else
-    hipLaunchKernelGGL((flash_fwd_kernel<float>), grid, block, 0, ctx->stream, qs, ks, vs, static_cast<float*>(out),
-                       static_cast<unsigned short*>(nullptr), lse, s, ctx->fault, tag);
+  if (dim == 64) launch_forward<64>(ctx, qs, ks, vs, out, out_dtype, out_residual, lse, s, tag);
+  else launch_forward<128>(ctx, qs, ks, vs, out, out_dtype, out_residual, lse, s, tag);
   OMX_LAUNCH_CHECK(ctx, "flash_fwd_kernel");
   return OMX_OK;
 }
@@ -634,8 +715,10 @@ int32_t omx_flash_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, cons
                                 void* gv, int32_t grad_dtype,
                                 uint64_t batch, uint64_t heads, uint64_t kv_heads, uint64_t time, uint64_t dim,
                                 uint64_t window, float scale, unsigned long long tag, const long* strides) {
-  if (dim != FD) return omx_fail(ctx, OMX_UNSUPPORTED_HEAD_DIM, "head_dim %llu limit %d", (unsigned long long)dim, FD);
-  FlashShape s = make_shape(batch, heads, kv_heads, time, window, scale, strides);
+  if (dim != 64 && dim != 128)
+    return omx_fail(ctx, OMX_UNSUPPORTED_HEAD_DIM, "head_dim %llu: the MFMA kernels take 64 and 128",
+                    (unsigned long long)dim);
+  FlashShape s = make_shape(batch, heads, kv_heads, time, dim, window, scale, strides);
   const long rows = static_cast<long>(batch * heads * time);
   void* ws = nullptr;
   int32_t rc = omx_workspace(ctx, rows * sizeof(float), &ws);
@@ -647,22 +730,8 @@ int32_t omx_flash_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, cons
   const unsigned short* os = static_cast<const unsigned short*>(out);
   const unsigned short* rs = static_cast<const unsigned short*>(out_residual);
   const unsigned short* gs = static_cast<const unsigned short*>(gy);
-  // dQ first: it also leaves delta = dO . O per row for the dK/dV pass.
-  dim3 block(FT);
-  const unsigned pairs = static_cast<unsigned>(((time + 127) / 128 + 1) / 2);  // two 128-row blocks per workgroup
-  dim3 kv_grid(pairs * static_cast<unsigned>(batch * kv_heads));
-  dim3 q_grid(pairs * static_cast<unsigned>(batch * heads));
-  if (grad_dtype == OMX_BF16) {
-    hipLaunchKernelGGL((flash_bwd_dq_kernel<unsigned short>), q_grid, block, 0, ctx->stream, qs, ks, vs, os, rs, lse,
-                       delta, gs, static_cast<unsigned short*>(gq), s, ctx->fault, tag);
-    hipLaunchKernelGGL((flash_bwd_dkv_kernel<unsigned short>), kv_grid, block, 0, ctx->stream, qs, ks, vs, lse, delta,
-                       gs, static_cast<unsigned short*>(gk), static_cast<unsigned short*>(gv), s, ctx->fault, tag);
-  } else {
-    hipLaunchKernelGGL((flash_bwd_dq_kernel<float>), q_grid, block, 0, ctx->stream, qs, ks, vs, os, rs, lse, delta, gs,
-                       static_cast<float*>(gq), s, ctx->fault, tag);
-    hipLaunchKernelGGL((flash_bwd_dkv_kernel<float>), kv_grid, block, 0, ctx->stream, qs, ks, vs, lse, delta, gs,
-                       static_cast<float*>(gk), static_cast<float*>(gv), s, ctx->fault, tag);
-  }
+  if (dim == 64) launch_backward<64>(ctx, qs, ks, vs, os, rs, lse, delta, gs, gq, gk, gv, grad_dtype, s, tag);
+  else launch_backward<128>(ctx, qs, ks, vs, os, rs, lse, delta, gs, gq, gk, gv, grad_dtype, s, tag);
   OMX_LAUNCH_CHECK(ctx, "flash backward kernels");
   return OMX_OK;
 }

@@ -536,7 +536,11 @@ def test_budget_refuses_rather_than_clamps_and_unsupported_ops_name_themselves(b
 FLASH_SHAPES = [([1, 1, 1, 64], 1, None), ([1, 2, 17, 64], 2, None), ([2, 3, 64, 64], 3, None),
                 ([1, 2, 128, 64], 2, None), ([1, 2, 129, 64], 1, None), ([1, 4, 300, 64], 2, None),
                 ([2, 2, 257, 64], 2, 40), ([1, 2, 200, 64], 2, 1), ([1, 1, 1024, 64], 1, None),
-                ([1, 2, 520, 64], 2, 130)]
+                ([1, 2, 520, 64], 2, 130),
+                # head_dim 128 (the dK / dV pass walks a key block once per gradient)
+                ([1, 1, 1, 128], 1, None), ([1, 2, 33, 128], 2, None), ([2, 2, 128, 128], 2, None),
+                ([1, 4, 300, 128], 2, None), ([1, 2, 257, 128], 1, 40), ([1, 1, 1024, 128], 1, None),
+                ([1, 2, 520, 128], 2, 130)]
 
 
 @pytest.mark.parametrize("per_key", [0.002, 0.05, 0.7])
@@ -578,7 +582,7 @@ def test_causal_sdpa_bf16_scores_that_keep_growing(be, per_key):
 
 @pytest.mark.parametrize("shape,hkv,window", FLASH_SHAPES)
 def test_causal_sdpa_bf16_mfma(be, shape, hkv, window):
-    """head_dim 64 with bf16 operands takes the MFMA flash kernels. Inputs are
+    """head_dim 64 or 128 with bf16 operands takes the MFMA flash kernels. Inputs are
     bf16-exact on both sides; the GPU additionally rounds P and dS to bf16 for
     the second product, so the gate is the bf16 one (2e-2 of the largest value)."""
     from ojas_amd.backend import BF16, F32
