@@ -117,6 +117,12 @@ int32_t omx_gemm(omx_ctx* ctx, const void* a, uint64_t a_rs, uint64_t a_cs, cons
                  uint64_t b_rs, uint64_t b_cs, int32_t operand_dtype, void* c, int32_t c_dtype,
                  uint64_t m, uint64_t k, uint64_t n, int32_t accumulate);
 
+/* omx_gemm whose output rows are `ldc` elements apart (ldc >= n), so the product can be a column
+ * block of a wider tensor. No counterpart in the trait. */
+int32_t omx_gemm_pitched(omx_ctx* ctx, const void* a, uint64_t a_rs, uint64_t a_cs, const void* b,
+                         uint64_t b_rs, uint64_t b_cs, int32_t operand_dtype, void* c, int32_t c_dtype,
+                         uint64_t ldc, uint64_t m, uint64_t k, uint64_t n, int32_t accumulate);
+
 /* `count` products of omx_gemm's form in one launch: product i reads its operands stride_a /
  * stride_b ELEMENTS after product i - 1's and writes stride_c elements after its output (strides
  * in multiples of 16 bytes; 1..65535 products). No counterpart in the trait, whose linear ops
@@ -142,15 +148,28 @@ int32_t omx_gemm_strided_batch(omx_ctx* ctx, const void* a, uint64_t a_rs, uint6
  * `layout`: OMX_I8_ROW_MAJOR (codes [n_out, k_in], scales [n_out, k_in / 32]) or OMX_I8_BLOCKED, the
  * form omx_pack_i8_group writes (same bytes, reordered so that both products read whole cache
  * lines: blocks of 8 rows x 4 groups, [group % 4][row % 8][32 codes] inside a block, the scales
- * likewise; needs k_in % 128 == 0 and n_out % 8 == 0). */
+ * likewise; needs k_in % 128 == 0 and n_out % 8 == 0).
+ * `low_rank` (optional): the adapter's second product, formed in the same accumulators instead of
+ * as a tensor of its own (lora_up + add of lora.rs:326-344): out[n, c] += sum_p h[n][off + p] *
+ * w[c][p] for p < rank, with h bf16 [rows, h_pitch] (h_pitch elements between rows) and w bf16
+ * [output columns, rank]; rank is a multiple of 16. block_cols > 0: column c reads h at
+ * off = (c / block_cols) * rank, so one h [rows, 3 rank] serves a fused q / k / v projection
+ * whose three up matrices are stacked in w (block_cols = d; a multiple of 128). For the forward,
+ * h = x A^T and w = scale * B; for the input gradient, h = gy (scale * B) and w = A^T. */
 enum { OMX_I8_ROW_MAJOR = 0, OMX_I8_BLOCKED = 1 };
+typedef struct {
+  const void* h;
+  const void* w;
+  uint64_t h_pitch, rank, block_cols;
+} omx_low_rank;
 int32_t omx_linear_i8_group_forward(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* codes_i8,
                                     const void* scales_f32, uint64_t group, int32_t layout,
-                                    const void* add, void* y, uint64_t rows, uint64_t k_in,
-                                    uint64_t n_out);
+                                    const void* add, const omx_low_rank* low_rank, void* y,
+                                    uint64_t rows, uint64_t k_in, uint64_t n_out);
 int32_t omx_linear_i8_group_backward_input(omx_ctx* ctx, const void* codes_i8, const void* scales_f32,
                                            uint64_t group, int32_t layout, const void* gy,
-                                           int32_t gy_dtype, const void* add, void* gx, uint64_t rows,
+                                           int32_t gy_dtype, const void* add,
+                                           const omx_low_rank* low_rank, void* gx, uint64_t rows,
                                            uint64_t k_in, uint64_t n_out);
 /* Reorders row-major codes and scales into the blocked layout (unpack = 0), or a blocked pair back
  * into row-major (unpack = 1: `codes_i8` / `scales_f32` are then the outputs). Out of place. A
@@ -442,6 +461,22 @@ int32_t omx_rope_half_split_forward(omx_ctx* ctx, const void* x, const void* cos
 int32_t omx_rope_half_split_backward(omx_ctx* ctx, const void* gy, const void* cos_f32,
                                      const void* sin_f32, void* gx, int32_t dtype, uint64_t rows,
                                      uint64_t dim, uint64_t time, uint64_t heads);
+/* rope_half_split_forward / _backward (backend.rs:1674-1686) applied IN PLACE to the first
+ * heads * dim columns of every row of a bf16 [tokens, pitch] tensor: the q and k column blocks
+ * of a fused q | k | v projection output (heads = query heads + key heads), which the attention
+ * entry points above then read where they lie. cos / sin are f32 [time, dim]; row r uses table
+ * row r % time. backward != 0 rotates by the opposite angle (the op's gradient). dim % 16 == 0. */
+int32_t omx_rope_half_split_inplace(omx_ctx* ctx, void* x, int32_t dtype, uint64_t pitch,
+                                    const void* cos_f32, const void* sin_f32, uint64_t tokens,
+                                    uint64_t time, uint64_t heads, uint64_t dim, int32_t backward);
+/* silu_forward then mul_forward (backend.rs:1151-1163; ojas-model/src/block.rs:248-262) on a fused
+ * gate | up projection output: gate_up is bf16 [rows, 2 hidden] with the gate columns first,
+ * out[r, c] = silu(gate[r, c]) * up[r, c]. The backward writes the gradient of gate_up in the
+ * same layout from gy [rows, hidden] (mul_backward then silu_backward). bf16, hidden % 8 == 0. */
+int32_t omx_swiglu_forward(omx_ctx* ctx, const void* gate_up, void* out, int32_t dtype, uint64_t rows,
+                           uint64_t hidden);
+int32_t omx_swiglu_backward(omx_ctx* ctx, const void* gate_up, const void* gy, void* g_gate_up,
+                            int32_t dtype, uint64_t rows, uint64_t hidden);
 /* BackendModule::rms_qk_norm_forward / _backward (backend.rs:1688-1708; CPU
  * ojas-cpu/src/backend.rs:1011-1040): RMSNorm over the last axis of q and of k,
  * each with its own weight. Both pairs are validated before either runs. */

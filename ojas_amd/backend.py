@@ -62,6 +62,12 @@ class MuonNs5Config(C.Structure):
         return cls(0.025, 0.99, 0.1, 1, 0)
 
 
+class LowRank(C.Structure):
+    """omx_low_rank: the adapter's second product, added in a quantised product's accumulators."""
+    _fields_ = [("h", C.c_void_p), ("w", C.c_void_p), ("h_pitch", C.c_uint64), ("rank", C.c_uint64),
+                ("block_cols", C.c_uint64)]
+
+
 def load_library() -> C.CDLL:
     if not LIB_PATH.exists():
         raise OjasError(BACKEND, f"{LIB_PATH} is not built; run __graft_entry__.build()")
@@ -259,6 +265,27 @@ class MiBackend:
                                                   C.c_uint64(rows), C.c_uint64(kin), C.c_uint64(nout)))
         return gx
 
+    def rope_half_split_inplace(self, x, cos, sin, tokens, time, heads, dim, backward=False):
+        """The rotary embedding applied in place to the first heads * dim columns of bf16 x [tokens, pitch]."""
+        self._check(self._lib.omx_rope_half_split_inplace(
+            self._ctx, self._p(x), C.c_int32(x.dtype), C.c_uint64(x.shape[-1]), self._p(cos), self._p(sin),
+            C.c_uint64(tokens), C.c_uint64(time), C.c_uint64(heads), C.c_uint64(dim), C.c_int32(1 if backward else 0)))
+        return x
+
+    def swiglu_forward(self, gate_up):
+        rows, two_h = gate_up.shape
+        out = self.empty((rows, two_h // 2), gate_up.dtype)
+        self._check(self._lib.omx_swiglu_forward(self._ctx, self._p(gate_up), self._p(out), C.c_int32(gate_up.dtype),
+                                                 C.c_uint64(rows), C.c_uint64(two_h // 2)))
+        return out
+
+    def swiglu_backward(self, gate_up, gy):
+        rows, two_h = gate_up.shape
+        g = self.empty(gate_up.shape, gate_up.dtype)
+        self._check(self._lib.omx_swiglu_backward(self._ctx, self._p(gate_up), self._p(gy), self._p(g),
+                                                  C.c_int32(gate_up.dtype), C.c_uint64(rows), C.c_uint64(two_h // 2)))
+        return g
+
     def pack_i8_group(self, codes, scales, group=32):
         """Row-major codes and scales -> the blocked layout (`omx_pack_i8_group`); same shapes."""
         nout, kin = codes.shape
@@ -275,7 +302,15 @@ class MiBackend:
                                                 C.c_uint64(group), C.c_int32(1)))
         return c, s
 
-    def linear_i8_group_forward(self, x, codes, scales, add=None, group=32, blocked=False):
+    @staticmethod
+    def _low_rank(low_rank):
+        """(h [rows, pitch] bf16, w [cols, rank] bf16, block_cols) -> a pointer to omx_low_rank, or None."""
+        if low_rank is None:
+            return None
+        h, w, block_cols = low_rank
+        return C.byref(LowRank(h.ptr, w.ptr, h.shape[-1], w.shape[-1], block_cols))
+
+    def linear_i8_group_forward(self, x, codes, scales, add=None, group=32, blocked=False, low_rank=None):
         """y = x W^T (+ add) for a frozen weight held as int8 codes [out, in] and f32 group scales
         [out, in / group] (value = code * scale); bf16 in, bf16 out."""
         rows, kin, nout = x.numel // x.shape[-1], x.shape[-1], codes.shape[0]
@@ -284,10 +319,10 @@ class MiBackend:
         y = self.empty(x.shape[:-1] + (nout,), BF16)
         self._check(self._lib.omx_linear_i8_group_forward(
             self._ctx, self._p(x), C.c_int32(x.dtype), self._p(codes), self._p(scales), C.c_uint64(group),
-            C.c_int32(1 if blocked else 0), self._p(add), self._p(y), C.c_uint64(rows), C.c_uint64(kin), C.c_uint64(nout)))
+            C.c_int32(1 if blocked else 0), self._p(add), self._low_rank(low_rank), self._p(y), C.c_uint64(rows), C.c_uint64(kin), C.c_uint64(nout)))
         return y
 
-    def linear_i8_group_backward_input(self, codes, scales, gy, add=None, group=32, blocked=False):
+    def linear_i8_group_backward_input(self, codes, scales, gy, add=None, group=32, blocked=False, low_rank=None):
         """gx = gy W (+ add) for the same weight form; there is no weight gradient (the base is frozen)."""
         nout, kin = codes.shape
         rows = gy.numel // gy.shape[-1]
@@ -296,7 +331,7 @@ class MiBackend:
         gx = self.empty(gy.shape[:-1] + (kin,), BF16)
         self._check(self._lib.omx_linear_i8_group_backward_input(
             self._ctx, self._p(codes), self._p(scales), C.c_uint64(group), C.c_int32(1 if blocked else 0), self._p(gy),
-            C.c_int32(gy.dtype), self._p(add), self._p(gx), C.c_uint64(rows), C.c_uint64(kin), C.c_uint64(nout)))
+            C.c_int32(gy.dtype), self._p(add), self._low_rank(low_rank), self._p(gx), C.c_uint64(rows), C.c_uint64(kin), C.c_uint64(nout)))
         return gx
 
     def gemm(self, a: DeviceTensor, a_strides, b: DeviceTensor, b_strides, m, k, n, out_dtype=F32, c=None):

@@ -673,6 +673,15 @@ int32_t omx_gemm(omx_ctx* ctx, const void* a, uint64_t a_rs, uint64_t a_cs, cons
   return omx_gemm_impl(ctx, F_GEMM, a, a_rs, a_cs, b, b_rs, b_cs, operand_dtype, c, c_dtype, n, m, k, n, accumulate);
 }
 
+int32_t omx_gemm_pitched(omx_ctx* ctx, const void* a, uint64_t a_rs, uint64_t a_cs, const void* b, uint64_t b_rs,
+                         uint64_t b_cs, int32_t operand_dtype, void* c, int32_t c_dtype, uint64_t ldc, uint64_t m,
+                         uint64_t k, uint64_t n, int32_t accumulate) {
+  OMX_REQUIRE_CTX(ctx);
+  if (ldc < n) return omx_fail(ctx, OMX_SHAPE, "gemm: output pitch %llu is below its %llu columns", (unsigned long long)ldc,
+                               (unsigned long long)n);
+  return omx_gemm_impl(ctx, F_GEMM, a, a_rs, a_cs, b, b_rs, b_cs, operand_dtype, c, c_dtype, ldc, m, k, n, accumulate);
+}
+
 int32_t omx_gemm_strided_batch(omx_ctx* ctx, const void* a, uint64_t a_rs, uint64_t a_cs, const void* b,
                                uint64_t b_rs, uint64_t b_cs, int32_t operand_dtype, void* c, int32_t c_dtype,
                                uint64_t m, uint64_t k, uint64_t n, int32_t accumulate, uint64_t count,

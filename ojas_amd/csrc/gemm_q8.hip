@@ -38,6 +38,12 @@ struct Q8Args {
   int M, N, K;
   int tiles_m, tiles_n;
   int packed;  // the weight is in the blocked layout of omx_pack_i8_group
+  // Optional low-rank term added in the accumulators: C[m, n] += sum_p lr_h[m][off + p] * lr_w[n][p],
+  // p < lr_rank (a multiple of 16), off = (n / lr_block_cols) * lr_rank when lr_block_cols > 0.
+  const unsigned short* lr_h;  // [M][lr_pitch] bf16
+  const unsigned short* lr_w;  // [N][lr_rank] bf16
+  long lr_pitch;
+  int lr_rank, lr_block_cols;
   OmxFaultWord* fault;
   unsigned long long tag;
 };
@@ -278,6 +284,33 @@ __global__ __launch_bounds__(512, 4) void gemm_q8_kernel(Q8Args g) {
       if (++ks >= steps) done = true;
     });
   }
+  // The low-rank term: lr_rank / 16 more MFMA slabs whose fragments come straight from global
+  // memory (16 bytes per lane and fragment; every load of the main loop has landed by now).
+  if (g.lr_rank > 0) {
+    const int h_off = g.lr_block_cols > 0 ? (n0 / g.lr_block_cols) * g.lr_rank : 0;
+    for (int p = 0; p < g.lr_rank; p += 16) {
+      u32x4 ta[TM], tb[TN];
+#pragma unroll
+      for (int t = 0; t < TM; ++t) {
+        int row = m0 + (wm * TM + t) * 32 + l32;
+        row = row < g.M ? row : g.M - 1;
+        ta[t] = *reinterpret_cast<const u32x4*>(g.lr_h + static_cast<long>(row) * g.lr_pitch + h_off + p + lg * 8);
+      }
+#pragma unroll
+      for (int t = 0; t < TN; ++t) {
+        int col = n0 + (wn * TN + t) * 32 + l32;
+        col = col < g.N ? col : g.N - 1;
+        tb[t] = *reinterpret_cast<const u32x4*>(g.lr_w + static_cast<long>(col) * g.lr_rank + p + lg * 8);
+      }
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn)
+          acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ta[tm]),
+                                                                __builtin_bit_cast(bf16x8, tb[tn]), acc[tm][tn], 0, 0,
+                                                                0);
+    }
+  }
   __syncthreads();  // the staging below reuses the stages
 
   // Epilogue: each wave stages 32 rows of its tile at a time through its own LDS region and
@@ -396,13 +429,40 @@ int32_t check_q8(omx_ctx* ctx, const char* op, const void* act, const void* code
   return OMX_OK;
 }
 
+// Validates and installs the optional low-rank term of an entry point (`cols`: the product's output columns).
+int32_t set_low_rank(omx_ctx* ctx, const char* op, Q8Args* g, const omx_low_rank* lr, uint64_t cols) {
+  g->lr_h = nullptr;
+  g->lr_w = nullptr;
+  g->lr_pitch = 0;
+  g->lr_rank = 0;
+  g->lr_block_cols = 0;
+  if (!lr || lr->rank == 0) return OMX_OK;
+  if (!lr->h || !lr->w) return omx_fail(ctx, OMX_PLACEMENT, "%s: low-rank term with a null pointer", op);
+  if (lr->rank % 16 != 0 || lr->rank > 1024)
+    return omx_fail(ctx, OMX_SHAPE, "%s: low-rank width %llu is not a multiple of 16 up to 1024", op,
+                    (unsigned long long)lr->rank);
+  if (lr->block_cols != 0 && (lr->block_cols % QBN != 0 || cols % lr->block_cols != 0))
+    return omx_fail(ctx, OMX_SHAPE, "%s: low-rank column blocks of %llu do not tile %llu columns in steps of %d", op,
+                    (unsigned long long)lr->block_cols, (unsigned long long)cols, QBN);
+  const uint64_t blocks = lr->block_cols ? cols / lr->block_cols : 1;
+  if (lr->h_pitch % 8 != 0 || lr->h_pitch < blocks * lr->rank || !aligned16(lr->h) || !aligned16(lr->w))
+    return omx_fail(ctx, OMX_SHAPE, "%s: low-rank operands must be 16-byte aligned with a pitch that holds them", op);
+  g->lr_h = static_cast<const unsigned short*>(lr->h);
+  g->lr_w = static_cast<const unsigned short*>(lr->w);
+  g->lr_pitch = static_cast<long>(lr->h_pitch);
+  g->lr_rank = static_cast<int>(lr->rank);
+  g->lr_block_cols = static_cast<int>(lr->block_cols);
+  return OMX_OK;
+}
+
 }  // namespace
 
 extern "C" {
 
 int32_t omx_linear_i8_group_forward(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* codes_i8,
-                                    const void* scales_f32, uint64_t group, int32_t layout, const void* add, void* y,
-                                    uint64_t rows, uint64_t kin, uint64_t nout) {
+                                    const void* scales_f32, uint64_t group, int32_t layout, const void* add,
+                                    const omx_low_rank* low_rank, void* y, uint64_t rows, uint64_t kin,
+                                    uint64_t nout) {
   OMX_REQUIRE_CTX(ctx);
   const char* op = "linear_i8_group_forward";
   int32_t rc = check_q8(ctx, op, x, codes_i8, scales_f32, y, add, rows, kin, nout, group, x_dtype, layout);
@@ -424,13 +484,16 @@ int32_t omx_linear_i8_group_forward(omx_ctx* ctx, const void* x, int32_t x_dtype
   g.tiles_n = (g.N + QBN - 1) / QBN;
   g.packed = layout == OMX_I8_BLOCKED;
   g.fault = ctx->fault;
+  rc = set_low_rank(ctx, op, &g, low_rank, nout);
+  if (rc != OMX_OK) return rc;
   g.tag = omx_tag(ctx, F_LINEAR_FORWARD);
   return launch_q8<false>(ctx, g, 2.0 * rows * kin * nout);
 }
 
 int32_t omx_linear_i8_group_backward_input(omx_ctx* ctx, const void* codes_i8, const void* scales_f32, uint64_t group,
-                                           int32_t layout, const void* gy, int32_t gy_dtype, const void* add, void* gx,
-                                           uint64_t rows, uint64_t kin, uint64_t nout) {
+                                           int32_t layout, const void* gy, int32_t gy_dtype, const void* add,
+                                           const omx_low_rank* low_rank, void* gx, uint64_t rows, uint64_t kin,
+                                           uint64_t nout) {
   OMX_REQUIRE_CTX(ctx);
   const char* op = "linear_i8_group_backward_input";
   int32_t rc = check_q8(ctx, op, gy, codes_i8, scales_f32, gx, add, rows, kin, nout, group, gy_dtype, layout);
@@ -453,6 +516,8 @@ int32_t omx_linear_i8_group_backward_input(omx_ctx* ctx, const void* codes_i8, c
   g.tiles_n = (g.N + QBN - 1) / QBN;
   g.packed = layout == OMX_I8_BLOCKED;
   g.fault = ctx->fault;
+  rc = set_low_rank(ctx, op, &g, low_rank, kin);
+  if (rc != OMX_OK) return rc;
   g.tag = omx_tag(ctx, F_LINEAR_BACKWARD);
   return launch_q8<true>(ctx, g, 2.0 * rows * kin * nout);
 }

@@ -121,6 +121,70 @@ def test_blocked_layout_gives_the_same_products(be, rows, kin, nout):
         assert np.array_equal(g0, g1)
 
 
+@pytest.mark.parametrize("rows,kin,nout,rank,blocks", [(300, 128, 256, 16, 1), (520, 256, 384, 16, 3),
+                                                         (256, 64, 128, 48, 1)])
+def test_low_rank_term_rides_in_the_accumulators(be, rows, kin, nout, rank, blocks):
+    from ojas_amd.backend import BF16
+
+    print(f"q8 low-rank rows={rows} kin={kin} nout={nout} rank={rank} blocks={blocks}", flush=True)
+    rng = np.random.default_rng(rows + rank)
+    bf = lambda a: orc.round_bf16(a.astype(np.float32))
+    x = bf(rng.normal(0, 1, (rows, kin)))
+    codes, scales = orc.quantize_i8_group(rng.normal(0, 0.05, (nout, kin)).astype(np.float32), 32)
+    h = bf(rng.normal(0, 1, (rows, blocks * rank)))
+    w = bf(rng.normal(0, 0.3, (nout, rank)))
+    block_cols = nout // blocks
+    want = orc.linear_i8_group_forward(x, codes, scales, 32)
+    for j in range(blocks):
+        cols = slice(j * block_cols, (j + 1) * block_cols)
+        want[:, cols] += h[:, j * rank:(j + 1) * rank].astype(np.float64) @ w[cols].astype(np.float64).T
+    y = be.linear_i8_group_forward(be.upload(x, BF16), be.upload(codes), be.upload(scales),
+                                   low_rank=(be.upload(h, BF16), be.upload(w, BF16), block_cols if blocks > 1 else 0))
+    _close(be.download_f32(y), want)
+    # Input gradient: gx = gy W + gh A with A^T [kin, rank] as the term's second operand.
+    gy = bf(rng.normal(0, 1, (rows, nout)))
+    gh = bf(rng.normal(0, 1, (rows, rank)))
+    at = bf(rng.normal(0, 0.3, (kin, rank)))
+    if nout % 32 == 0:
+        want = orc.linear_i8_group_backward_input(codes, scales, gy, 32) + gh.astype(np.float64) @ at.astype(np.float64).T
+        gx = be.linear_i8_group_backward_input(be.upload(codes), be.upload(scales), be.upload(gy, BF16),
+                                               low_rank=(be.upload(gh, BF16), be.upload(at, BF16), 0))
+        _close(be.download_f32(gx), want)
+
+
+def test_rope_in_place_and_swiglu(be):
+    from ojas_amd.backend import BF16
+
+    tokens, time, heads, dim, pitch = 48, 12, 6, 32, 6 * 32 + 64  # 4 query + 2 key heads, then 64 value columns
+    rng = np.random.default_rng(21)
+    x = orc.round_bf16(rng.normal(0, 1, (tokens, pitch)).astype(np.float32))
+    cos, sin = orc.rope_tables(time, dim)
+    rot = orc.rope_forward(np.ascontiguousarray(x[:, :heads * dim]).reshape(tokens // time, time, heads, dim), cos, sin)
+    dx = be.upload(x, BF16)
+    be.rope_half_split_inplace(dx, be.upload(cos), be.upload(sin), tokens, time, heads, dim)
+    got = be.download_f32(dx)
+    _close(got[:, :heads * dim], rot.reshape(tokens, heads * dim), 1e-2)
+    assert np.array_equal(got[:, heads * dim:], x[:, heads * dim:])  # the value block is untouched
+    # The backward is the inverse rotation: forward then backward returns the input (to bf16 rounding).
+    be.rope_half_split_inplace(dx, be.upload(cos), be.upload(sin), tokens, time, heads, dim, backward=True)
+    back = orc.rope_backward(rot, cos, sin).reshape(tokens, heads * dim)
+    _close(be.download_f32(dx)[:, :heads * dim], back, 2e-2)
+    # SwiGLU on a fused gate | up tensor.
+    rows, hidden = 37, 72
+    gu = orc.round_bf16(rng.normal(0, 1.5, (rows, 2 * hidden)).astype(np.float32))
+    gm = orc.round_bf16(rng.normal(0, 1, (rows, hidden)).astype(np.float32))
+    gate, up = np.ascontiguousarray(gu[:, :hidden]), np.ascontiguousarray(gu[:, hidden:])
+    act = orc.silu_forward(gate)
+    want = orc.mul_forward(act, up)
+    dgu = be.upload(gu, BF16)
+    _close(be.download_f32(be.swiglu_forward(dgu)), want)
+    g_act, g_up = orc.mul_backward(act, up, gm)
+    g_gate = orc.silu_backward(gate, g_act)
+    got = be.download_f32(be.swiglu_backward(dgu, be.upload(gm, BF16)))
+    _close(got[:, :hidden], g_gate)
+    _close(got[:, hidden:], g_up)
+
+
 def test_linear_i8_group_refusals(be):
     from ojas_amd.backend import BF16, DTYPE, SHAPE, UNSUPPORTED, OjasError
 
@@ -129,16 +193,16 @@ def test_linear_i8_group_refusals(be):
     scales = be.upload(np.zeros((32, 1), np.float32))
     with pytest.raises(OjasError) as e:  # k_in is not a multiple of the group
         be._check(be._lib.omx_linear_i8_group_forward(be._ctx, be._p(x), C.c_int32(1), be._p(codes), be._p(scales),
-                                                      C.c_uint64(32), C.c_int32(0), None, be._p(x), C.c_uint64(8), C.c_uint64(48),
+                                                      C.c_uint64(32), C.c_int32(0), None, None, be._p(x), C.c_uint64(8), C.c_uint64(48),
                                                       C.c_uint64(32)))
     assert e.value.code == SHAPE
     with pytest.raises(OjasError) as e:
         be._check(be._lib.omx_linear_i8_group_forward(be._ctx, be._p(x), C.c_int32(1), be._p(codes), be._p(scales),
-                                                      C.c_uint64(64), C.c_int32(0), None, be._p(x), C.c_uint64(8), C.c_uint64(64),
+                                                      C.c_uint64(64), C.c_int32(0), None, None, be._p(x), C.c_uint64(8), C.c_uint64(64),
                                                       C.c_uint64(32)))
     assert e.value.code == UNSUPPORTED
     with pytest.raises(OjasError) as e:
         be._check(be._lib.omx_linear_i8_group_forward(be._ctx, be._p(x), C.c_int32(0), be._p(codes), be._p(scales),
-                                                      C.c_uint64(32), C.c_int32(0), None, be._p(x), C.c_uint64(8), C.c_uint64(64),
+                                                      C.c_uint64(32), C.c_int32(0), None, None, be._p(x), C.c_uint64(8), C.c_uint64(64),
                                                       C.c_uint64(32)))
     assert e.value.code == DTYPE
