@@ -151,8 +151,9 @@ int32_t omx_gemm_strided_batch(omx_ctx* ctx, const void* a, uint64_t a_rs, uint6
  * likewise; needs k_in % 128 == 0 and n_out % 8 == 0).
  * `low_rank` (optional): the adapter's second product, formed in the same accumulators instead of
  * as a tensor of its own (lora_up + add of lora.rs:326-344): out[n, c] += sum_p h[n][off + p] *
- * w[c][p] for p < rank, with h bf16 [rows, h_pitch] (h_pitch elements between rows) and w bf16
- * [output columns, rank]; rank is a multiple of 16. block_cols > 0: column c reads h at
+ * w[c][p] for p < rank, with h bf16 [rows, h_pitch] and w bf16 [output columns, w_pitch] (pitches:
+ * elements between rows, multiples of 8, so either may be a column block of a wider tensor); rank
+ * is a multiple of 16. block_cols > 0: column c reads h at
  * off = (c / block_cols) * rank, so one h [rows, 3 rank] serves a fused q / k / v projection
  * whose three up matrices are stacked in w (block_cols = d; a multiple of 128). For the forward,
  * h = x A^T and w = scale * B; for the input gradient, h = gy (scale * B) and w = A^T. */
@@ -160,7 +161,7 @@ enum { OMX_I8_ROW_MAJOR = 0, OMX_I8_BLOCKED = 1 };
 typedef struct {
   const void* h;
   const void* w;
-  uint64_t h_pitch, rank, block_cols;
+  uint64_t h_pitch, w_pitch, rank, block_cols;
 } omx_low_rank;
 int32_t omx_linear_i8_group_forward(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* codes_i8,
                                     const void* scales_f32, uint64_t group, int32_t layout,
@@ -477,6 +478,13 @@ int32_t omx_swiglu_forward(omx_ctx* ctx, const void* gate_up, void* out, int32_t
                            uint64_t hidden);
 int32_t omx_swiglu_backward(omx_ctx* ctx, const void* gate_up, const void* gy, void* g_gate_up,
                             int32_t dtype, uint64_t rows, uint64_t hidden);
+/* Synthetic weights made on the device (no counterpart in the reference, whose init runs on the
+ * host, ojas-model/src/init.rs:67-114): element i is N(0, std) from a counter-based generator of
+ * (seed, i). omx_init_normal_i8_group draws row-major [n_out, k_in] values and stores them
+ * quantised, codes and one scale per group of 32 (the rule of quant_sparse.rs:306-326 per group). */
+int32_t omx_init_normal(omx_ctx* ctx, void* dst, int32_t dtype, uint64_t n, uint64_t seed, float std);
+int32_t omx_init_normal_i8_group(omx_ctx* ctx, void* codes_i8, void* scales_f32, uint64_t n_out,
+                                 uint64_t k_in, uint64_t group, uint64_t seed, float std);
 /* BackendModule::rms_qk_norm_forward / _backward (backend.rs:1688-1708; CPU
  * ojas-cpu/src/backend.rs:1011-1040): RMSNorm over the last axis of q and of k,
  * each with its own weight. Both pairs are validated before either runs. */

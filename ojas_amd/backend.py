@@ -64,8 +64,8 @@ class MuonNs5Config(C.Structure):
 
 class LowRank(C.Structure):
     """omx_low_rank: the adapter's second product, added in a quantised product's accumulators."""
-    _fields_ = [("h", C.c_void_p), ("w", C.c_void_p), ("h_pitch", C.c_uint64), ("rank", C.c_uint64),
-                ("block_cols", C.c_uint64)]
+    _fields_ = [("h", C.c_void_p), ("w", C.c_void_p), ("h_pitch", C.c_uint64), ("w_pitch", C.c_uint64),
+                ("rank", C.c_uint64), ("block_cols", C.c_uint64)]
 
 
 def load_library() -> C.CDLL:
@@ -308,7 +308,7 @@ class MiBackend:
         if low_rank is None:
             return None
         h, w, block_cols = low_rank
-        return C.byref(LowRank(h.ptr, w.ptr, h.shape[-1], w.shape[-1], block_cols))
+        return C.byref(LowRank(h.ptr, w.ptr, h.shape[-1], w.shape[-1], w.shape[-1], block_cols))
 
     def linear_i8_group_forward(self, x, codes, scales, add=None, group=32, blocked=False, low_rank=None):
         """y = x W^T (+ add) for a frozen weight held as int8 codes [out, in] and f32 group scales

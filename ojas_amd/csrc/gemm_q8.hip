@@ -41,8 +41,8 @@ struct Q8Args {
   // Optional low-rank term added in the accumulators: C[m, n] += sum_p lr_h[m][off + p] * lr_w[n][p],
   // p < lr_rank (a multiple of 16), off = (n / lr_block_cols) * lr_rank when lr_block_cols > 0.
   const unsigned short* lr_h;  // [M][lr_pitch] bf16
-  const unsigned short* lr_w;  // [N][lr_rank] bf16
-  long lr_pitch;
+  const unsigned short* lr_w;  // [N][lr_w_pitch] bf16
+  long lr_pitch, lr_w_pitch;
   int lr_rank, lr_block_cols;
   OmxFaultWord* fault;
   unsigned long long tag;
@@ -300,7 +300,7 @@ __global__ __launch_bounds__(512, 4) void gemm_q8_kernel(Q8Args g) {
       for (int t = 0; t < TN; ++t) {
         int col = n0 + (wn * TN + t) * 32 + l32;
         col = col < g.N ? col : g.N - 1;
-        tb[t] = *reinterpret_cast<const u32x4*>(g.lr_w + static_cast<long>(col) * g.lr_rank + p + lg * 8);
+        tb[t] = *reinterpret_cast<const u32x4*>(g.lr_w + static_cast<long>(col) * g.lr_w_pitch + p + lg * 8);
       }
 #pragma unroll
       for (int tm = 0; tm < TM; ++tm)
@@ -434,6 +434,7 @@ int32_t set_low_rank(omx_ctx* ctx, const char* op, Q8Args* g, const omx_low_rank
   g->lr_h = nullptr;
   g->lr_w = nullptr;
   g->lr_pitch = 0;
+  g->lr_w_pitch = 0;
   g->lr_rank = 0;
   g->lr_block_cols = 0;
   if (!lr || lr->rank == 0) return OMX_OK;
@@ -445,11 +446,13 @@ int32_t set_low_rank(omx_ctx* ctx, const char* op, Q8Args* g, const omx_low_rank
     return omx_fail(ctx, OMX_SHAPE, "%s: low-rank column blocks of %llu do not tile %llu columns in steps of %d", op,
                     (unsigned long long)lr->block_cols, (unsigned long long)cols, QBN);
   const uint64_t blocks = lr->block_cols ? cols / lr->block_cols : 1;
-  if (lr->h_pitch % 8 != 0 || lr->h_pitch < blocks * lr->rank || !aligned16(lr->h) || !aligned16(lr->w))
+  if (lr->h_pitch % 8 != 0 || lr->h_pitch < blocks * lr->rank || lr->w_pitch % 8 != 0 || lr->w_pitch < lr->rank ||
+      !aligned16(lr->h) || !aligned16(lr->w))
     return omx_fail(ctx, OMX_SHAPE, "%s: low-rank operands must be 16-byte aligned with a pitch that holds them", op);
   g->lr_h = static_cast<const unsigned short*>(lr->h);
   g->lr_w = static_cast<const unsigned short*>(lr->w);
   g->lr_pitch = static_cast<long>(lr->h_pitch);
+  g->lr_w_pitch = static_cast<long>(lr->w_pitch);
   g->lr_rank = static_cast<int>(lr->rank);
   g->lr_block_cols = static_cast<int>(lr->block_cols);
   return OMX_OK;

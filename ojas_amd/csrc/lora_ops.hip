@@ -111,6 +111,69 @@ __global__ void swiglu_bwd_kernel(const unsigned short* __restrict__ gate_up, co
   if (bad) dev_raise_fault(fault, tag);
 }
 
+// Counter-based generator for synthetic weights: SplitMix64's output function of (seed, counter),
+// two 24-bit uniforms, Box-Muller. Element i of a tensor is a function of (seed, i) alone.
+__device__ __forceinline__ unsigned long long mix64(unsigned long long z) {
+  z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+  z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+  return z ^ (z >> 31);
+}
+__device__ __forceinline__ void normal_pair(unsigned long long seed, unsigned long long pair, float* a, float* b) {
+  const unsigned long long bits = mix64(seed + 0x9e3779b97f4a7c15ull * (pair + 1));
+  const float u1 = (static_cast<float>(bits & 0xffffffu) + 1.0f) * (1.0f / 16777216.0f);  // (0, 1]
+  const float u2 = static_cast<float>((bits >> 24) & 0xffffffu) * (1.0f / 16777216.0f);
+  const float rad = sqrtf(-2.0f * __logf(u1));
+  float sn, cs;
+  __sincosf(6.28318530717958647692f * u2, &sn, &cs);
+  *a = rad * cs;
+  *b = rad * sn;
+}
+
+template <typename T>
+__global__ void init_normal_kernel(T* __restrict__ dst, long n, unsigned long long seed, float std) {
+  const long pair = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (2 * pair >= n) return;
+  float a, b;
+  normal_pair(seed, static_cast<unsigned long long>(pair), &a, &b);
+  dev_store<T>(dst, 2 * pair, a * std);
+  if (2 * pair + 1 < n) dev_store<T>(dst, 2 * pair + 1, b * std);
+}
+
+// One thread per group of 32: draws the group's values, then quantises them with the rule of
+// ojas-cpu/src/quant_sparse.rs:306-326 applied to the group (scale = abs_max / 127, or 1 for zeros;
+// code = round half away from zero of v * 127 / abs_max, clamped to +-127).
+__global__ void init_normal_i8_group_kernel(signed char* __restrict__ codes, float* __restrict__ scales, long groups,
+                                            unsigned long long seed, float std) {
+  const long gi = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (gi >= groups) return;
+  float v[32];
+  float abs_max = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    normal_pair(seed, static_cast<unsigned long long>(gi) * 16 + i, &v[2 * i], &v[2 * i + 1]);
+    v[2 * i] *= std;
+    v[2 * i + 1] *= std;
+    abs_max = fmaxf(abs_max, fmaxf(fabsf(v[2 * i]), fabsf(v[2 * i + 1])));
+  }
+  scales[gi] = abs_max > 0.0f ? abs_max / 127.0f : 1.0f;
+  const float inv = abs_max > 0.0f ? 127.0f / abs_max : 0.0f;
+  unsigned int words[8];
+#pragma unroll
+  for (int w = 0; w < 8; ++w) {
+    unsigned int word = 0;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      float q = roundf(v[4 * w + b] * inv);
+      q = fminf(fmaxf(q, -127.0f), 127.0f);
+      word |= (static_cast<unsigned int>(static_cast<int>(q)) & 0xffu) << (8 * b);
+    }
+    words[w] = word;
+  }
+  uint4* out = reinterpret_cast<uint4*>(codes + gi * 32);
+  out[0] = make_uint4(words[0], words[1], words[2], words[3]);
+  out[1] = make_uint4(words[4], words[5], words[6], words[7]);
+}
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 }  // namespace
@@ -138,6 +201,39 @@ int32_t omx_rope_half_split_inplace(omx_ctx* ctx, void* x, int32_t dtype, uint64
                      static_cast<int>(heads), static_cast<int>(dim), backward ? -1.0f : 1.0f, ctx->fault,
                      omx_tag(ctx, backward ? F_ROPE_BACKWARD : F_ROPE_FORWARD));
   OMX_LAUNCH_CHECK(ctx, "rope_pitched_kernel");
+  return OMX_OK;
+}
+
+int32_t omx_init_normal(omx_ctx* ctx, void* dst, int32_t dtype, uint64_t n, uint64_t seed, float std) {
+  OMX_REQUIRE_CTX(ctx);
+  if (!dst) return omx_fail(ctx, OMX_PLACEMENT, "init_normal: null device pointer");
+  if (!omx_valid_float_dtype(dtype)) return omx_fail(ctx, OMX_DTYPE, "init_normal: dtype must be f32 or bf16");
+  if (n == 0) return OMX_OK;
+  const long pairs = static_cast<long>((n + 1) / 2);
+  dim3 grid(static_cast<unsigned>((pairs + 255) / 256)), block(256);
+  if (dtype == OMX_F32)
+    hipLaunchKernelGGL(init_normal_kernel<float>, grid, block, 0, ctx->stream, static_cast<float*>(dst),
+                       static_cast<long>(n), static_cast<unsigned long long>(seed), std);
+  else
+    hipLaunchKernelGGL(init_normal_kernel<unsigned short>, grid, block, 0, ctx->stream,
+                       static_cast<unsigned short*>(dst), static_cast<long>(n), static_cast<unsigned long long>(seed), std);
+  OMX_LAUNCH_CHECK(ctx, "init_normal_kernel");
+  return OMX_OK;
+}
+
+int32_t omx_init_normal_i8_group(omx_ctx* ctx, void* codes_i8, void* scales_f32, uint64_t nout, uint64_t kin,
+                                 uint64_t group, uint64_t seed, float std) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "init_normal_i8_group";
+  if (!codes_i8 || !scales_f32) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  if (group != 32) return omx_fail(ctx, OMX_UNSUPPORTED, "%s: group size %llu (only 32)", op, (unsigned long long)group);
+  if (nout == 0 || kin == 0 || kin % 32 != 0) return omx_fail(ctx, OMX_SHAPE, "%s: k_in must be a positive multiple of 32", op);
+  if (!aligned16(codes_i8)) return omx_fail(ctx, OMX_SHAPE, "%s: codes must be 16-byte aligned", op);
+  const long groups = static_cast<long>(nout * (kin / 32));
+  hipLaunchKernelGGL(init_normal_i8_group_kernel, dim3(static_cast<unsigned>((groups + 255) / 256)), dim3(256), 0,
+                     ctx->stream, static_cast<signed char*>(codes_i8), static_cast<float*>(scales_f32), groups,
+                     static_cast<unsigned long long>(seed), std);
+  OMX_LAUNCH_CHECK(ctx, "init_normal_i8_group_kernel");
   return OMX_OK;
 }
 

@@ -148,7 +148,7 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
 constexpr int OMX_COLUMN_SUM_GROUPS = 32;
 int32_t omx_column_sum(omx_ctx* ctx, const float* partial, float* out, uint64_t blocks, uint64_t dim,
                        unsigned long long tag, float* scratch = nullptr);
-// RMSNorm with 16-byte accesses for row widths 256..1024 (rmsvec.hip). `add` (forward) and
+// RMSNorm with 16-byte accesses for row widths 256..2048 (rmsvec.hip). `add` (forward) and
 // `add_in` / `gx16` (backward) are optional fused operands.
 bool omx_rms_vec_eligible(uint64_t dim, std::initializer_list<const void*> ptrs);
 int32_t omx_rms_forward_vec(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* add, int32_t add_dtype,

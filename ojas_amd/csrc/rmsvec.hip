@@ -1,4 +1,4 @@
-// RMSNorm for row widths 256..1024 with 16-byte accesses, optionally fused with
+// RMSNorm for row widths 256..2048 with 16-byte accesses, optionally fused with
 // the residual add in front of it (forward) or behind it (backward).
 //
 // Reference semantics: ojas-cpu/src/norm.rs:24-204 (rms_norm_forward /
@@ -175,7 +175,7 @@ bool aligned16(std::initializer_list<const void*> ptrs) {
 }  // namespace
 
 bool omx_rms_vec_eligible(uint64_t dim, std::initializer_list<const void*> ptrs) {
-  return dim % 4 == 0 && dim >= 256 && dim <= 1024 && aligned16(ptrs);
+  return dim % 4 == 0 && dim >= 256 && dim <= 2048 && aligned16(ptrs);
 }
 
 int32_t omx_rms_forward_vec(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* add, int32_t add_dtype,
@@ -193,7 +193,11 @@ int32_t omx_rms_forward_vec(omx_ctx* ctx, const void* x, int32_t x_dtype, const 
     case 1: RV_FWD(TX, TA, TY, 1); break; \
     case 2: RV_FWD(TX, TA, TY, 2); break; \
     case 3: RV_FWD(TX, TA, TY, 3); break; \
-    default: RV_FWD(TX, TA, TY, 4); break; \
+    case 4: RV_FWD(TX, TA, TY, 4); break; \
+    case 5: RV_FWD(TX, TA, TY, 5); break; \
+    case 6: RV_FWD(TX, TA, TY, 6); break; \
+    case 7: RV_FWD(TX, TA, TY, 7); break; \
+    default: RV_FWD(TX, TA, TY, 8); break; \
   }
   const int key = (x_dtype == OMX_BF16 ? 4 : 0) | (add && add_dtype == OMX_BF16 ? 2 : 0) | (y_dtype == OMX_BF16 ? 1 : 0);
   switch (key) {
@@ -236,7 +240,11 @@ int32_t omx_rms_backward_vec(omx_ctx* ctx, const void* x, int32_t x_dtype, const
     case 1: RV_BWD(TX, TG, TO, 1); break; \
     case 2: RV_BWD(TX, TG, TO, 2); break; \
     case 3: RV_BWD(TX, TG, TO, 3); break; \
-    default: RV_BWD(TX, TG, TO, 4); break; \
+    case 4: RV_BWD(TX, TG, TO, 4); break; \
+    case 5: RV_BWD(TX, TG, TO, 5); break; \
+    case 6: RV_BWD(TX, TG, TO, 6); break; \
+    case 7: RV_BWD(TX, TG, TO, 7); break; \
+    default: RV_BWD(TX, TG, TO, 8); break; \
   }
   const int key = (x_dtype == OMX_BF16 ? 4 : 0) | (gy_dtype == OMX_BF16 ? 2 : 0) | (gx_dtype == OMX_BF16 ? 1 : 0);
   switch (key) {

@@ -206,3 +206,91 @@ def test_linear_i8_group_refusals(be):
                                                       C.c_uint64(32), C.c_int32(0), None, None, be._p(x), C.c_uint64(8), C.c_uint64(64),
                                                       C.c_uint64(32)))
     assert e.value.code == DTYPE
+
+
+# ---- the step: reduced shapes against the oracle ----
+def _load_case(tr, cfg, frozen, quant):
+    """Hands a seeded case (test_oracle_lora.make_lora_case) to the device trainer."""
+    tr.set_embedding(frozen[0])
+    for l in range(cfg.layers):
+        base = 1 + 9 * l
+        tr.set_norm(l, 0, frozen[base + 0])
+        tr.set_norm(l, 1, frozen[base + 5])
+        for which, idx in enumerate((1, 2, 3, 4, 6, 7, 8)):
+            codes, scales = quant[base + idx]
+            tr.set_matrix(l, which, codes, scales)
+    tr.set_norm(cfg.layers, 0, frozen[-1])
+
+
+# (layers, d, heads, head_dim, hidden, vocab, batch, seq, rank, scale)
+LORA_STEP_SHAPES = [(2, 128, 2, 64, 256, 96, 2, 48, 16, 2.0), (1, 256, 2, 128, 384, 200, 1, 130, 16, 1.0),
+                    (2, 128, 1, 128, 128, 64, 2, 64, 32, 0.5)]
+
+
+@pytest.mark.parametrize("shape", LORA_STEP_SHAPES)
+def test_lora_step_matches_the_oracle(be, shape):
+    from test_oracle_lora import make_lora_case
+
+    from ojas_amd.backend import AdamWConfig
+    from ojas_amd.lora import LoraConfig, LoraTrainer
+
+    print(f"lora step {shape}", flush=True)
+    cfg = LoraConfig(*shape[:9], 1e-6, shape[9], 10000.0)
+    ocfg = orc.LoraConfig(*shape[:9], 1e-6, shape[9], 10000.0)
+    frozen, quant, adapters, ids, targets = make_lora_case(ocfg, 31 + shape[1])
+    adapters = [orc.round_bf16(a) for a in adapters]  # bf16-exact operands on both sides
+    tr = LoraTrainer(be, cfg)
+    try:
+        _load_case(tr, cfg, frozen, quant)
+        tr.set_adapters(adapters)
+        tr.set_batch(ids, targets)
+        loss = tr.loss_and_grads()
+        grads = tr.grads()
+        oloss, ograds = orc.lora_loss_and_grads(ocfg, frozen, adapters, ids, targets)
+        assert abs(loss - float(oloss)) <= 1e-3 * abs(float(oloss)), (loss, oloss)  # the bf16 tier's loss gate
+        for i, (g, og) in enumerate(zip(grads, ograds)):
+            scale = float(np.max(np.abs(og)))
+            assert scale > 0, i
+            err = float(np.max(np.abs(g - og)))
+            assert err <= BF16_TOL * scale, (i, err / scale)
+            assert np.linalg.norm(g - og) <= BF16_TOL * np.linalg.norm(og), i
+        # One AdamW step moves every adapter element against its gradient's sign by about lr, and
+        # nothing else: the update of an element with a solid gradient is lr to within 1 %.
+        lr = 1e-3
+        step_loss, norm = tr.step(AdamWConfig(lr, 0.9, 0.95, 1e-8, 0.0), 0.0)
+        assert abs(step_loss - loss) <= 1e-6 * abs(loss)
+        want_norm = float(np.sqrt(sum(float(np.sum(g.astype(np.float64) ** 2)) for g in grads)))
+        assert abs(norm - want_norm) <= 1e-4 * want_norm
+        after = tr.adapters()
+        for a0, a1, g in zip(adapters, after, grads):
+            solid = np.abs(g) > 1e-3 * np.max(np.abs(g))
+            move = (a1 - a0.reshape(-1))[solid]
+            assert np.all(np.abs(move + lr * np.sign(g[solid])) <= 1e-2 * lr + 4e-8 * np.abs(a0.reshape(-1)[solid]))
+        assert tr.steps() == 1
+    finally:
+        tr.close()
+
+
+def test_lora_adapter_starts_as_the_identity(be):
+    # B = 0 (lora.rs:9-12): the loss is the base model's whatever A holds, dA is exactly zero and dB is not.
+    from test_oracle_lora import make_lora_case
+
+    from ojas_amd.lora import LoraConfig, LoraTrainer
+
+    shape = (2, 128, 2, 64, 256, 96, 2, 48, 16)
+    cfg = LoraConfig(*shape, 1e-6, 2.0, 10000.0)
+    ocfg = orc.LoraConfig(*shape, 1e-6, 2.0, 10000.0)
+    frozen, quant, adapters, ids, targets = make_lora_case(ocfg, 5)
+    zero_b = [orc.round_bf16(a) if i % 2 == 0 else np.zeros_like(a) for i, a in enumerate(adapters)]
+    tr = LoraTrainer(be, cfg)
+    try:
+        _load_case(tr, cfg, frozen, quant)
+        tr.set_batch(ids, targets)
+        tr.set_adapters(zero_b)
+        loss0 = tr.loss_and_grads()
+        grads = tr.grads()
+        assert all(not np.any(g) for g in grads[0::2]) and all(np.any(g) for g in grads[1::2])
+        tr.set_adapters([2 * a if i % 2 == 0 else a for i, a in enumerate(zero_b)])
+        assert tr.loss_and_grads() == loss0
+    finally:
+        tr.close()
