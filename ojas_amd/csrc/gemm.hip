@@ -508,6 +508,7 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
     else if (mode == 5) dma_variant = 5;
     else if (mode == 6) dma_variant = 6;
     else if (mode == 7) dma_variant = (!a_km && !b_km) ? 7 : 3;
+    else if (mode == 8) dma_variant = 8;
   }
   int BM = 128, BN = 128;
   if (dma_variant >= 0) omx_gemm_dma_tile(dma_variant, &BM, &BN);
@@ -618,8 +619,17 @@ extern "C" {
 
 int32_t omx_set_option(omx_ctx* ctx, const char* name, int64_t value) {
   OMX_REQUIRE_CTX(ctx);
+  if (name && strcmp(name, "gemm_persistent_min_steps") == 0) {
+    if (value < 2) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: gemm_persistent_min_steps is at least 2");
+    ctx->gemm_persistent_min_steps = static_cast<int>(value);
+    return OMX_OK;
+  }
+  if (name && strcmp(name, "gemm_persistent") == 0) {
+    ctx->gemm_persistent = static_cast<int>(value) & 15;
+    return OMX_OK;
+  }
   if (name && strcmp(name, "gemm_dma") == 0) {
-    if (value < 0 || value > 7) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: gemm_dma takes 0..7");
+    if (value < 0 || value > 8) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: gemm_dma takes 0..8");
     ctx->gemm_dma_mode = static_cast<int>(value);
     return OMX_OK;
   }

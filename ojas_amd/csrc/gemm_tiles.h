@@ -67,6 +67,81 @@ struct TileLoads {
   }
 };
 
+// The same loads with one scalar base address per operand and a 32-bit byte offset per lane and
+// load, taken from the tile's first element: the offsets do not depend on the tile, so a
+// workgroup that walks several tiles only moves the scalar base (no per-lane address is ever
+// recomputed), and a K step advances one scalar instead of every lane's pointer. The per-lane
+// offsets are parked in LDS (`park`: N x threads words) and fetched back at each issue, which
+// keeps them out of the registers the accumulators and fragments need. For tiles that lie
+// wholly inside the operand (no row is clamped).
+template <bool KM, int ROWS, int BK, int NW>
+struct TileLoadsScalarBase {
+  static constexpr int TOTAL = ROWS * BK * 2 / 1024;
+  static constexpr int N = TOTAL / NW;
+  static_assert(TOTAL % NW == 0, "the same number of loads in every wave");
+  static constexpr int PARK_BYTES = N * NW * 64 * 4;
+  const char* base;  // wave-uniform: the tile's first element + the current K step's byte offset
+  long step;         // bytes between consecutive K steps
+
+  __device__ __forceinline__ void init_lanes(unsigned* park, long ld, int wave, int lane) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int q = wave + NW * i;
+      unsigned off;
+      if constexpr (!KM) {
+        constexpr int LPR = BK / 8;
+        const int r = q * (64 / LPR) + lane / LPR;
+        const int kc = (lane % LPR) ^ (BK == 32 ? (r >> 2) & 3 : (r >> 1) & 7);
+        off = static_cast<unsigned>(r) * static_cast<unsigned>(ld * 2) + kc * 16;
+      } else {
+        constexpr int CPR = ROWS / 8;
+        const int idx = q * 64 + lane;
+        const int kr = idx / CPR, slot = idx % CPR;
+        const int mc = slot ^ ((kr & 3) * 4);
+        off = static_cast<unsigned>(kr) * static_cast<unsigned>(ld * 2) + mc * 16;
+      }
+      park[i * NW * 64 + threadIdx.x] = off;
+    }
+    step = (KM ? BK * ld : BK) * 2;
+  }
+  // Tile rows row0.. of the operand at `origin`, from K step 0.
+  __device__ __forceinline__ void aim(const void* origin, long ld, int row0) {
+    base = static_cast<const char*>(origin) + (KM ? static_cast<long>(row0) : static_cast<long>(row0) * ld) * 2;
+  }
+  // `lds_wave`: the LDS address of this wave's first KiB of the stage area; TILE: the byte offset
+  // of the operand's tile in it. M0 is formed from the one scalar and an immediate.
+  // The parked offsets of this lane, fetched with one wait for all of them.
+  __device__ __forceinline__ void fetch(const unsigned* park, unsigned (&off)[N]) const {
+    // (the index is formed here for the same reason as in xor_here)
+    unsigned slot;
+    asm volatile("v_lshlrev_b32 %0, 2, %1" : "=v"(slot) : "v"(threadIdx.x));
+#pragma unroll
+    for (int i = 0; i < N; ++i)
+      off[i] = *reinterpret_cast<const unsigned*>(reinterpret_cast<const char*>(park) + i * NW * 64 * 4 + slot);
+  }
+  template <int TILE>
+  __device__ __forceinline__ void issue(const unsigned (&off)[N], unsigned lds_wave) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off[i]), "s"(base),
+                   "s"(lds_wave), "n"(TILE + NW * i * 1024)
+                   : "memory", "scc");
+    }
+    base += step;
+  }
+  // The same with the stage's byte offset in a scalar register.
+  template <int TILE>
+  __device__ __forceinline__ void issue_at(const unsigned (&off)[N], unsigned lds_wave, unsigned stage_bytes) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      asm volatile("s_add_u32 m0, %2, %3\n\ts_add_u32 m0, m0, %4\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off[i]),
+                   "s"(base), "s"(lds_wave), "s"(stage_bytes), "n"(TILE + NW * i * 1024)
+                   : "memory", "scc");
+    }
+    base += step;
+  }
+};
+
 // Byte offset, inside an operand tile, of this lane's fragment for 32-row block `row_base / 32`
 // and 16-column K slab kk (k-major operands: of its first transposing read; the second is four
 // K rows further).
@@ -84,6 +159,25 @@ __device__ __forceinline__ int frag_offset(int row_base, int kk, int lane) {
     const int slot = (col >> 3) ^ (((s >> 2) & 3) * 4);
     return kr * (ROWS * 2) + slot * 16 + (col & 7) * 2;
   }
+}
+// frag_offset(row_base + 32 t, kk, lane) from `first` = frag_offset(row_base, 0, lane), for a
+// row_base that is a multiple of 64. k-contiguous tiles: a 32-row block further is 32 rows of
+// bytes further (the swizzle repeats every 8 or 16 rows), and slab kk flips the chunk index's bits
+// 1.., i.e. bits 5.. of the offset. k-major tiles: slab kk is 16 K rows further, and a 32-column
+// block further flips bit 2 of the chunk slot (bit 6 of the offset).
+// x ^ bits, computed where it is used: the assembly statement keeps the compiler from hoisting
+// the result out of the K loop into a register of its own (the accumulators need them all).
+template <int BITS>
+__device__ __forceinline__ int xor_here(int x) {
+  if constexpr (BITS == 0) return x;
+  int r;
+  asm volatile("v_xor_b32 %0, %1, %2" : "=v"(r) : "n"(BITS), "v"(x));
+  return r;
+}
+template <bool KM, int ROWS, int BK, int T, int KKI>
+__device__ __forceinline__ int frag_from_first(int first) {
+  if constexpr (!KM) return xor_here<(KKI << 5)>(first) + T * 32 * BK * 2;
+  else return xor_here<(T << 6)>(first) + KKI * 16 * ROWS * 2;
 }
 template <bool KM, int ROWS>
 __device__ __forceinline__ u32x4 frag_at(const char* p) {
