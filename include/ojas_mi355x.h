@@ -539,11 +539,13 @@ int32_t omx_topk_rows(omx_ctx* ctx, const void* x_f32, uint64_t rows, uint64_t c
  * ojas-model/src/trainer.rs:1031-1046). */
 int32_t omx_read_scalar_f32(omx_ctx* ctx, const void* src, float* out);
 
-/* Tuning knobs (no counterpart in the reference). "gemm_dma": 0 = 128x128 GEMM
- * kernel only, 1 = choose by shape (default), 2 / 3 / 4 / 5 / 6 / 7 = force the 256x256
- * (64-column steps) / 256x128 (32-column steps) / 256x128 (64-column steps) / 256x256 four-wave /
- * 128x128 four-wave / 128x192 six-wave (row-major operands only) direct-to-LDS kernel wherever
- * the operands are eligible. "kv_attention": 0 = choose by head_dim (default), 1 = always the
+/* Tuning knobs (no counterpart in the reference). "gemm_dma": 0 = register-staged 128x128 GEMM
+ * kernel only, 1 = choose by shape (default), 2 / 3 / 4 = force the 256x256 (64-column steps) /
+ * 256x128 (32-column steps) / 128x128 four-wave direct-to-LDS kernel wherever the operands are
+ * eligible. "gemm_persistent": bit mask over operand layouts (bit 2 * A k-major + B k-major) that
+ * take the persistent form of the direct-to-LDS kernel (default 15), and
+ * "gemm_persistent_min_steps": only for reductions of at least this many 32-column steps
+ * (default 64). "kv_attention": 0 = choose by head_dim (default), 1 = always the
  * LDS-tiled kernel. "ce_fused": 0 = the fused linear-cross-entropy always takes its separate
  * statistics and gradient kernels (default 1: one kernel when a tile holds the whole
  * vocabulary). "adamw_trust": 0 = omx_adamw_step_bounded always runs its checking pass

@@ -123,6 +123,7 @@ void omx_close(omx_ctx* ctx) {
   (void)hipSetDevice(ctx->device);
   (void)hipStreamSynchronize(ctx->stream);
   for (auto& kv : ctx->allocations) (void)hipFree(kv.first);
+  for (auto& kv : ctx->pool) (void)hipFree(kv.second);
   if (ctx->fault) (void)hipFree(ctx->fault);
   if (ctx->fault_host) (void)hipHostFree(ctx->fault_host);
   if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
@@ -149,6 +150,19 @@ size_t omx_device_name(omx_ctx* ctx, char* buf, size_t cap) {
   return ctx->arch.size();
 }
 
+}  // extern "C"
+
+// Returns every parked block to the device (waits for the stream first).
+void omx_release_pool(omx_ctx* ctx) {
+  if (ctx->pool.empty()) return;
+  (void)hipStreamSynchronize(ctx->stream);
+  for (auto& kv : ctx->pool) (void)hipFree(kv.second);
+  ctx->pool.clear();
+  ctx->pooled_bytes = 0;
+}
+
+extern "C" {
+
 int32_t omx_alloc(omx_ctx* ctx, uint64_t bytes, void** out) {
   OMX_REQUIRE_CTX(ctx);
   if (!out) return omx_fail(ctx, OMX_BACKEND, "omx_alloc: null out");
@@ -159,8 +173,23 @@ int32_t omx_alloc(omx_ctx* ctx, uint64_t bytes, void** out) {
     return omx_fail(ctx, OMX_CAPACITY_EXCEEDED, "requested %llu cap %llu live %llu", (unsigned long long)bytes,
                     (unsigned long long)ctx->budget_limit, (unsigned long long)ctx->budget_live);
   void* p = nullptr;
-  hipError_t err = hipMalloc(&p, bytes);
-  if (err != hipSuccess) return omx_hip_fail(ctx, err, "hipMalloc");
+  auto pooled = ctx->pool.find(bytes);
+  if (pooled != ctx->pool.end()) {
+    // A block of this size freed earlier: every use of it is on this context's stream, so work
+    // launched from here on is ordered after whatever still reads it.
+    p = pooled->second;
+    ctx->pool.erase(pooled);
+    ctx->pooled_bytes -= bytes;
+  } else {
+    hipError_t err = hipMalloc(&p, bytes);
+    if (err != hipSuccess && !ctx->pool.empty()) {
+      // Out of device memory with blocks parked in the pool: give them back and try once more.
+      (void)hipGetLastError();
+      omx_release_pool(ctx);
+      err = hipMalloc(&p, bytes);
+    }
+    if (err != hipSuccess) return omx_hip_fail(ctx, err, "hipMalloc");
+  }
   ctx->allocations[p] = bytes;
   ctx->budget_live += bytes;
   if (ctx->budget_live > ctx->budget_peak) ctx->budget_peak = ctx->budget_live;
@@ -173,11 +202,22 @@ int32_t omx_free(omx_ctx* ctx, void* ptr) {
   if (!ptr) return OMX_OK;
   auto it = ctx->allocations.find(ptr);
   if (it == ctx->allocations.end()) return omx_fail(ctx, OMX_PLACEMENT, "omx_free: pointer not from this context");
-  // Work that still reads the buffer is on the context's stream.
+  const uint64_t bytes = it->second;
+  ctx->budget_live -= bytes;
+  ctx->allocations.erase(it);
+  // Freeing for real would wait for the stream (work that still reads the buffer is on it) and for
+  // the whole device (hipFree). Blocks of moderate size are parked instead and handed out again by
+  // omx_alloc to a request of the same size; reuse is safe without a wait because the next user's
+  // work goes onto the same stream. The pool is not charged to the budget: the budget counts what
+  // callers hold.
+  constexpr uint64_t kMaxBlock = 256ull << 20, kMaxPool = 4ull << 30;
+  if (bytes <= kMaxBlock && ctx->pooled_bytes + bytes <= kMaxPool) {
+    ctx->pool.emplace(bytes, ptr);
+    ctx->pooled_bytes += bytes;
+    return OMX_OK;
+  }
   OMX_HIP(ctx, hipStreamSynchronize(ctx->stream));
   OMX_HIP(ctx, hipFree(ptr));
-  ctx->budget_live -= it->second;
-  ctx->allocations.erase(it);
   return OMX_OK;
 }
 

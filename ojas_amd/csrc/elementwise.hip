@@ -323,9 +323,10 @@ int32_t omx_token_windows(omx_ctx* ctx, const void* tokens, int32_t bytes_per_to
   void* ws = nullptr;
   int32_t rc = omx_workspace(ctx, batch * sizeof(uint64_t), &ws);
   if (rc != OMX_OK) return rc;
-  // A copy from pageable host memory returns once the source has been staged, so the caller's
-  // array may be reused at once; it is ordered before the kernel on the same stream.
+  // The caller may reuse or free `starts` as soon as this returns, and an asynchronous copy from
+  // pageable memory is not guaranteed to have read its source by then: wait for it, as omx_upload does.
   OMX_HIP(ctx, hipMemcpyAsync(ws, starts, batch * sizeof(uint64_t), hipMemcpyHostToDevice, ctx->stream));
+  OMX_HIP(ctx, hipStreamSynchronize(ctx->stream));
   const uint64_t n = batch * seq_len;
   const unsigned blocks = static_cast<unsigned>(std::min<uint64_t>((n + 255) / 256, 4096));
   if (bytes_per_token == 2)

@@ -371,13 +371,9 @@ int32_t launch_one(omx_ctx* ctx, const GemmArgs& g) {
   constexpr int BM = 64 * TM, BN = 64 * TN;
   constexpr int smem = 2 * (tile_bytes<T, A_KM, BM>() + tile_bytes<T, B_KM, BN>());
   auto kernel = &gemm_kernel<T, A_KM, B_KM, TM, TN>;
-  // More than 64 KiB of dynamic LDS has to be granted per kernel, once.
-  static bool granted = false;
-  if (!granted) {
-    OMX_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     smem));
-    granted = true;
-  }
+  // More than 64 KiB of dynamic LDS has to be granted per kernel (and per device: asked every time).
+  OMX_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   smem));
   const int total = g.tiles_m * g.tiles_n * g.splits;
   omx_launch_timed(ctx, kernel, dim3(total, g.batches), dim3(NT), smem, ctx->timing_start,
                    g.splits > 1 ? nullptr : ctx->timing_stop, g);
@@ -504,11 +500,7 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
     }
     else if (mode == 2) dma_variant = 0;
     else if (mode == 3) dma_variant = 3;
-    else if (mode == 4) dma_variant = 1;
-    else if (mode == 5) dma_variant = 5;
-    else if (mode == 6) dma_variant = 6;
-    else if (mode == 7) dma_variant = (!a_km && !b_km) ? 7 : 3;
-    else if (mode == 8) dma_variant = 8;
+    else if (mode == 4) dma_variant = 6;
   }
   int BM = 128, BN = 128;
   if (dma_variant >= 0) omx_gemm_dma_tile(dma_variant, &BM, &BN);
@@ -629,7 +621,7 @@ int32_t omx_set_option(omx_ctx* ctx, const char* name, int64_t value) {
     return OMX_OK;
   }
   if (name && strcmp(name, "gemm_dma") == 0) {
-    if (value < 0 || value > 8) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: gemm_dma takes 0..8");
+    if (value < 0 || value > 4) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: gemm_dma takes 0..4");
     ctx->gemm_dma_mode = static_cast<int>(value);
     return OMX_OK;
   }

@@ -11,14 +11,9 @@
 //     contributes half a 128-byte cache line per step, each line is requested twice, far enough
 //     apart that the second request misses L1 again, and the load path then delivers 65 GB/s
 //     per compute unit instead of 107 GB/s (measured with the loads alone).
-//   * Variants 1 (256 x 128, three stages) and 0 (256 x 256, two stages): K steps of 64 columns,
-//     whole cache lines, one workgroup per compute unit. Load latency (about 0.6 us) is then
-//     exposed: with one or two stages in flight the loads alone take as long as the products.
-//   * Variant 5: 256 x 256 with four waves of 128 x 128 (256 accumulator registers per lane, held
-//     in AGPRs), 32-column steps, four stages. Half the LDS reads and two thirds of the loads per
-//     FLOP of the default, but one wave per SIMD: with nothing else to switch to, the products
-//     alone (no loads) run at 0.8x the default's rate, and the whole kernel is slower on every
-//     shape measured. Kept for measurements.
+//   * Variant 0 (256 x 256, two stages): K steps of 64 columns, whole cache lines, one workgroup per
+//     compute unit. Load latency (about 0.6 us) is then exposed; it wins on long reductions with
+//     large outputs only.
 //   * operand tiles go from global memory straight into LDS: no staging
 //     registers and no LDS store instructions. A wave-wide load writes 64
 //     consecutive 16-byte slots, so the LDS tile is unpadded and bank conflicts
@@ -47,7 +42,7 @@ gemm_dma_kernel(GemmArgs g) {
   constexpr int NW = WGM * WGN;           // waves per workgroup
   constexpr int LPS = STAGE / 1024 / NW;  // loads per wave per step
   constexpr int KK = DBK / 16;            // MFMA K slabs per step
-  static_assert(NW == 4 || NW == 6 || NW == 8, "four, six or eight waves");
+  static_assert(NW == 4 || NW == 8, "four or eight waves");
   // Six waves share 16 + 24 loads unevenly; with two stages every wait is for all of a wave's loads.
   static_assert(STAGE % (1024 * NW) == 0 || NST == 2, "counted waits need the same number of loads in every wave");
 
@@ -642,20 +637,15 @@ bool omx_gemm_dma_eligible(const GemmArgs& g, bool a_km, bool b_km) {
 }
 
 void omx_gemm_dma_tile(int variant, int* bm, int* bn) {
-  *bm = (variant == 6 || variant == 7) ? 128 : 256;
-  *bn = variant == 7 ? 192 : (variant == 0 || variant == 5 || variant == 8) ? 256 : 128;
+  *bm = variant == 6 ? 128 : 256;
+  *bn = variant == 0 ? 256 : 128;
 }
 
+// The three tilings the dispatcher chooses among: 0: 256 x 256 in 64-column steps (whole cache
+// lines, two stages, one workgroup per compute unit); 3: 256 x 128 in 32-column steps (three
+// stages, two workgroups per compute unit); 6: 128 x 128 with four waves (three per compute unit).
 int32_t omx_gemm_dma_launch(omx_ctx* ctx, const GemmArgs& g, bool a_km, bool b_km, int variant) {
   if (variant == 0) return launch_layout<2, 4, 4, 2, 64, 2>(ctx, g, a_km, b_km);
-  if (variant == 3) return launch_layout<4, 2, 2, 2, 32, 3>(ctx, g, a_km, b_km);
-  if (variant == 5) return launch_layout<2, 2, 4, 4, 32, 4>(ctx, g, a_km, b_km);
-  if (variant == 8) return launch_layout<2, 4, 4, 2, 32, 4>(ctx, g, a_km, b_km);
   if (variant == 6) return launch_layout<2, 2, 2, 2, 32, 3>(ctx, g, a_km, b_km);
-  // 128 x 192 with six waves and 64-column steps: whole 128-byte lines from both operands, two
-  // stages in 80 KiB, so two workgroups still share a compute unit. Row-major operands only.
-  // Behind the option: with two stages a step's loads have one step of lead, which exposes their
-  // latency (K = 768: 557 against 750 TFLOP/s for the 256 x 128 form; 8192^3: 765 against 898).
-  if (variant == 7 && !a_km && !b_km) return launch_dma<false, false, 2, 3, 2, 2, 64, 2>(ctx, g);
-  return launch_layout<4, 2, 2, 2, 64, 3>(ctx, g, a_km, b_km);
+  return launch_layout<4, 2, 2, 2, 32, 3>(ctx, g, a_km, b_km);
 }

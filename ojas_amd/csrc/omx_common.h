@@ -71,6 +71,9 @@ struct omx_ctx {
   hipStream_t stream = nullptr;
   uint64_t budget_limit = 0, budget_live = 0, budget_peak = 0;
   std::map<void*, uint64_t> allocations;
+  // Freed blocks kept for reuse by size (see omx_free); not charged to the budget.
+  std::multimap<uint64_t, void*> pool;
+  uint64_t pooled_bytes = 0;
   OmxFaultWord* fault = nullptr;  // device
   OmxFaultWord* fault_host = nullptr;  // pinned
   uint64_t sequence = 0;
@@ -114,6 +117,7 @@ inline void omx_launch_timed(omx_ctx* ctx, F kernel, dim3 grid, dim3 block, unsi
 }
 
 int32_t omx_fail(omx_ctx* ctx, omx_status code, const char* fmt, ...);
+void omx_release_pool(omx_ctx* ctx);
 // Per-product timing for callers outside gemm.hip: takes a pair of events for the product about
 // to be launched (when omx_profile_gemm is on) and files them with its FLOP count afterwards.
 int32_t omx_timing_begin(omx_ctx* ctx, double flops, omx_ctx::TimedLaunch* timed);

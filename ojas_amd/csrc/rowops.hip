@@ -237,13 +237,99 @@ __global__ void fill_positions_kernel(const unsigned int* __restrict__ ids, unsi
   positions[slot] = static_cast<unsigned int>(n);
 }
 
-// One wave per table row: zero it, or add its tokens' gradient rows in
-// ascending token order (the order of the CPU scatter, pointwise.rs:196-207),
-// so the f32 sums carry the same bits. The unordered segment is walked by
-// repeated minimum selection.
+// fill_positions_kernel leaves a row's token positions in arrival order. The sums below must run
+// in ascending token order (the order of the CPU scatter, pointwise.rs:196-207) to carry the same
+// bits, so every row's segment is sorted first, out of place:
+//   * up to 64 positions: one wave, a bitonic network over lane shuffles;
+//   * longer segments (one id filling a large share of the batch) are queued and sorted by
+//     sort_long_segments_kernel below.
+__global__ __launch_bounds__(ROW_THREADS) void sort_short_segments_kernel(const unsigned int* __restrict__ offsets,
+                                                                          const unsigned int* __restrict__ positions,
+                                                                          unsigned int* __restrict__ sorted,
+                                                                          unsigned int* __restrict__ long_count,
+                                                                          unsigned int* __restrict__ long_rows,
+                                                                          size_t vocab) {
+  const int lane = threadIdx.x & 63;
+  const size_t v = static_cast<size_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (v >= vocab) return;
+  const unsigned int begin = offsets[v], end = offsets[v + 1], len = end - begin;
+  if (len == 0) return;
+  if (len > 64) {
+    if (lane == 0) long_rows[atomicAdd(long_count, 1u)] = static_cast<unsigned int>(v);
+    return;
+  }
+  unsigned int p = static_cast<unsigned int>(lane) < len ? positions[begin + lane] : 0xffffffffu;
+#pragma unroll
+  for (int k = 2; k <= 64; k <<= 1)
+#pragma unroll
+    for (int j = k >> 1; j > 0; j >>= 1) {
+      const unsigned int other = __shfl_xor(p, j, 64);
+      const bool ascending = (lane & k) == 0;
+      const bool keep_min = ((lane & j) == 0) == ascending;
+      p = keep_min ? min(p, other) : max(p, other);
+    }
+  if (static_cast<unsigned int>(lane) < len) sorted[begin + lane] = p;
+}
+
+// One 1024-thread block per queued row. Positions are distinct token indices, so a bitmap orders
+// them: for each window of 32768 tokens the block marks the row's positions that fall into it
+// (one word per thread), then writes the set bits out in order at a running offset. Linear in
+// the segment's length per window, whatever the length.
+__global__ __launch_bounds__(1024) void sort_long_segments_kernel(const unsigned int* __restrict__ offsets,
+                                                                   const unsigned int* __restrict__ positions,
+                                                                   unsigned int* __restrict__ sorted,
+                                                                   const unsigned int* __restrict__ long_count,
+                                                                   const unsigned int* __restrict__ long_rows,
+                                                                   size_t tokens) {
+  __shared__ unsigned int bitmap[1024];
+  __shared__ unsigned int wave_tot[16];
+  __shared__ unsigned int written;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const unsigned int rows = *long_count;
+  for (unsigned int q = blockIdx.x; q < rows; q += gridDim.x) {
+    const unsigned int v = long_rows[q];
+    const unsigned int begin = offsets[v], end = offsets[v + 1];
+    if (threadIdx.x == 0) written = 0;
+    for (size_t base = 0; base < tokens; base += 32768) {
+      bitmap[threadIdx.x] = 0;
+      __syncthreads();
+      if (written == end - begin) break;  // uniform: read after the barrier, written before the previous one
+      for (unsigned int s = begin + threadIdx.x; s < end; s += 1024) {
+        const size_t rel = static_cast<size_t>(positions[s]) - base;  // wraps far above the window when below it
+        if (rel < 32768) atomicOr(&bitmap[rel >> 5], 1u << (rel & 31));
+      }
+      __syncthreads();
+      unsigned int w = bitmap[threadIdx.x];
+      const unsigned int c = __popc(w);
+      unsigned int incl = c;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const unsigned int t = __shfl_up(incl, off, 64);
+        if (lane >= off) incl += t;
+      }
+      if (lane == 63) wave_tot[wave] = incl;
+      __syncthreads();
+      unsigned int before = written;
+      for (int wv = 0; wv < wave; ++wv) before += wave_tot[wv];
+      unsigned int at = begin + before + incl - c;
+      while (w) {
+        const int bit = __ffs(w) - 1;
+        sorted[at++] = static_cast<unsigned int>(base) + threadIdx.x * 32 + bit;
+        w &= w - 1;
+      }
+      __syncthreads();
+      if (threadIdx.x == 1023) written = before + incl;
+      __syncthreads();
+    }
+    __syncthreads();
+  }
+}
+
+// One wave per table row: zero it, or add its tokens' gradient rows in ascending token order
+// (`sorted`: the row's positions, ascending), so the f32 sums carry the CPU scatter's bits.
 template <typename TG>
 __global__ __launch_bounds__(ROW_THREADS) void embedding_bwd_kernel(const unsigned int* __restrict__ offsets,
-                                                                    const unsigned int* __restrict__ positions,
+                                                                    const unsigned int* __restrict__ sorted,
                                                                     const TG* __restrict__ grad,
                                                                     float* __restrict__ table_grad, size_t vocab,
                                                                     int dim, OmxFaultWord* fault,
@@ -262,17 +348,8 @@ __global__ __launch_bounds__(ROW_THREADS) void embedding_bwd_kernel(const unsign
     float acc[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
-    long last = -1;
-    for (unsigned int step = begin; step < end; ++step) {
-      unsigned int best = 0xffffffffu;
-      for (unsigned int s = begin + lane; s < end; s += 64) {
-        unsigned int p = positions[s];
-        if (static_cast<long>(p) > last && p < best) best = p;
-      }
-#pragma unroll
-      for (int off = 32; off > 0; off >>= 1) best = min(best, static_cast<unsigned int>(__shfl_xor(best, off, 64)));
-      last = best;
-      const TG* src = grad + static_cast<size_t>(best) * dim;
+    for (unsigned int s = begin; s < end; ++s) {
+      const TG* src = grad + static_cast<size_t>(sorted[s]) * dim;
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         int c = c0 + j * 64 + lane;
@@ -587,8 +664,9 @@ int32_t omx_embedding_backward(omx_ctx* ctx, const void* ids, const void* grad, 
   if (tokens == 0 || vocab == 0 || dim == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
   if (tokens > 0xfffffffeull || vocab > 0xfffffffeull || dim > 0x7fffffffull)
     return omx_fail(ctx, OMX_OUT_OF_RANGE, "%s: axis does not fit in u32", op);
-  // Workspace: counts[V], offsets[V+1], cursor[V], positions[N].
-  uint64_t words = vocab + (vocab + 1) + vocab + tokens;
+  // Workspace: counts[V], offsets[V+1], cursor[V], positions[N], sorted[N], the count of rows with
+  // more than 64 tokens (one word, padded to four) and their list (at most N / 65 of them).
+  uint64_t words = vocab + (vocab + 1) + vocab + tokens + tokens + 4 + (tokens / 64 + 1);
   void* ws = nullptr;
   int32_t rc = omx_workspace(ctx, words * 4, &ws);
   if (rc != OMX_OK) return rc;
@@ -596,8 +674,13 @@ int32_t omx_embedding_backward(omx_ctx* ctx, const void* ids, const void* grad, 
   unsigned int* offsets = counts + vocab;
   unsigned int* cursor = offsets + vocab + 1;
   unsigned int* positions = cursor + vocab;
+  unsigned int* sorted = positions + tokens;
+  unsigned int* long_count = sorted + tokens;
+  unsigned int* long_rows = long_count + 4;
   unsigned long long tag = omx_tag(ctx, F_EMBEDDING_BACKWARD);
   rc = omx_fill_zero(ctx, counts, vocab * 4);
+  if (rc != OMX_OK) return rc;
+  rc = omx_fill_zero(ctx, long_count, 16);
   if (rc != OMX_OK) return rc;
   const unsigned int* idp = static_cast<const unsigned int*>(ids);
   dim3 tgrid(static_cast<unsigned>((tokens + 255) / 256));
@@ -608,13 +691,19 @@ int32_t omx_embedding_backward(omx_ctx* ctx, const void* ids, const void* grad, 
   hipLaunchKernelGGL(fill_positions_kernel, tgrid, dim3(256), 0, ctx->stream, idp, cursor, positions, tokens, vocab);
   OMX_LAUNCH_CHECK(ctx, "fill_positions_kernel");
   dim3 vgrid(static_cast<unsigned>((vocab + 3) / 4));
+  hipLaunchKernelGGL(sort_short_segments_kernel, vgrid, dim3(ROW_THREADS), 0, ctx->stream, offsets, positions, sorted,
+                     long_count, long_rows, vocab);
+  OMX_LAUNCH_CHECK(ctx, "sort_short_segments_kernel");
+  hipLaunchKernelGGL(sort_long_segments_kernel, dim3(256), dim3(1024), 0, ctx->stream, offsets, positions, sorted,
+                     long_count, long_rows, tokens);
+  OMX_LAUNCH_CHECK(ctx, "sort_long_segments_kernel");
   if (grad_dtype == OMX_F32)
-    hipLaunchKernelGGL((embedding_bwd_kernel<float>), vgrid, dim3(ROW_THREADS), 0, ctx->stream, offsets, positions,
+    hipLaunchKernelGGL((embedding_bwd_kernel<float>), vgrid, dim3(ROW_THREADS), 0, ctx->stream, offsets, sorted,
                        static_cast<const float*>(grad), static_cast<float*>(table_grad), vocab, static_cast<int>(dim),
                        ctx->fault, tag);
   else
     hipLaunchKernelGGL((embedding_bwd_kernel<unsigned short>), vgrid, dim3(ROW_THREADS), 0, ctx->stream, offsets,
-                       positions, static_cast<const unsigned short*>(grad), static_cast<float*>(table_grad), vocab,
+                       sorted, static_cast<const unsigned short*>(grad), static_cast<float*>(table_grad), vocab,
                        static_cast<int>(dim), ctx->fault, tag);
   OMX_LAUNCH_CHECK(ctx, "embedding_bwd_kernel");
   return OMX_OK;

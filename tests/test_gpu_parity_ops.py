@@ -164,6 +164,20 @@ def test_embedding_heavy_collisions_and_bf16_table(be):
     assert np.array_equal(out.view(np.uint32), orc.embedding_forward(table, ids).view(np.uint32))
 
 
+@pytest.mark.parametrize("tokens,vocab,dim", [(16384, 50, 48), (70000, 7, 8), (65, 1, 16)])
+def test_embedding_backward_with_one_id_filling_the_batch(be, tokens, vocab, dim):
+    """Rows with more than 64 tokens take the bitmap sort (windows of 32768 tokens: the second case
+    crosses two window edges); one id that takes most of the batch must cost no more than its share
+    and keep the ascending-token order of the sums bit for bit."""
+    print(f"embedding long segments {tokens} {vocab} {dim}", flush=True)
+    r = orc.SplitMix64(77 + tokens)
+    ids = np.array([r.below(vocab) for _ in range(tokens)], dtype=np.uint32)
+    ids[np.arange(tokens) % 3 != 0] = 0  # two thirds of the batch are id 0
+    grad = r.vec(tokens * dim, 1.0).reshape(tokens, dim)
+    tg = be.download(be.embedding_backward(be.upload(ids), be.upload(grad), vocab))
+    assert np.array_equal(tg.view(np.uint32), orc.embedding_backward(ids, grad, vocab).view(np.uint32))
+
+
 def test_embedding_out_of_range_id_is_reported_at_sync(be):
     from ojas_amd.backend import OUT_OF_RANGE, OjasError
 
