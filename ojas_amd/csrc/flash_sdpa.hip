@@ -61,6 +61,12 @@ __device__ __forceinline__ u32x4 pack8(const floatx16& acc, int c) {
   r.w = pack2(acc[8 * c + 6], acc[8 * c + 7]);
   return r;
 }
+// acc + both bf16 halves of w (v_dot2c_f32_bf16 against a pair of ones).
+__device__ __forceinline__ float sum_pairs(unsigned int w, float acc) {
+  typedef __bf16 bf16_pair __attribute__((ext_vector_type(2)));
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16_pair, w), __builtin_bit_cast(bf16_pair, 0x3F803F80u),
+                                         acc, false);
+}
 __device__ __forceinline__ floatx16 mfma(const u32x4& a, const u32x4& b, floatx16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
                                                  0, 0);
@@ -245,7 +251,13 @@ __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_fwd_kernel(const un
     floatx16 o[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) o[mt] = zero16();
-    float m = -INFINITY, lsum = 0.0f;
+    // `lsum` sums the weights as computed (the log-sum-exp, from which the backward pass rebuilds
+    // them); `wsum` sums the bf16 copies the matrix units multiply into V (this lane's half of
+    // the keys), and the output is divided by that: the output is then an exact weighted mean of
+    // value rows, so a component shared by all of them passes through unchanged, and
+    // dO . out cancels it against dP = dO . V in the backward pass. Divided by lsum it would
+    // come through scaled by (sum of rounded weights) / (sum of weights).
+    float m = -INFINITY, lsum = 0.0f, wsum = 0.0f;
     const float scale_log2 = s.scale * LOG2E;
     const int block_q0 = qb * 128, block_q1 = min(T - 1, qb * 128 + 127);
     const int kt_first = s.window > 0 ? max(0, block_q0 + 1 - s.window) / 64 : 0;
@@ -310,6 +322,7 @@ __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_fwd_kernel(const un
         // rows that keep theirs).
         const float alpha = __builtin_amdgcn_exp2f(fmaf(m, scale_log2, neg_m));
         lsum *= alpha;
+        wsum *= alpha;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -322,21 +335,23 @@ __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_fwd_kernel(const un
 #pragma unroll
         for (int c = 0; c < 2; ++c) {
           const u32x4 pb = pack8(sc[sub], c);
+          wsum = sum_pairs(pb.x, sum_pairs(pb.y, sum_pairs(pb.z, sum_pairs(pb.w, wsum))));
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) o[mt] = mfma(frag_tr<D>(v_rows, mt, sub, c, lane), pb, o[mt]);
         }
     }
+    wsum += __shfl_xor(wsum, 32, 64);
     bool bad = false;
     if (q_row < T) {
-      bad |= !(dev_finite(lsum) && lsum > 0.0f);
+      bad |= !(dev_finite(lsum) && lsum > 0.0f && wsum > 0.0f);
       if (lg == 0) lse[plane * T + q_row] = m * s.scale + logf(lsum);
     }
     const long o_off = b * s.o.bs + h * s.o.hs;
     if constexpr (sizeof(TO) == 2) {
-      if (resid) bad |= store_transposed_acc_split<D>(out + o_off, resid + o_off, s.o.rs, q_row, T, lg, o, 1.0f / lsum);
-      else bad |= store_transposed_acc<D, TO>(out + o_off, s.o.rs, q_row, T, lg, o, 1.0f / lsum);
+      if (resid) bad |= store_transposed_acc_split<D>(out + o_off, resid + o_off, s.o.rs, q_row, T, lg, o, 1.0f / wsum);
+      else bad |= store_transposed_acc<D, TO>(out + o_off, s.o.rs, q_row, T, lg, o, 1.0f / wsum);
     } else {
-      bad |= store_transposed_acc<D, TO>(out + o_off, s.o.rs, q_row, T, lg, o, 1.0f / lsum);
+      bad |= store_transposed_acc<D, TO>(out + o_off, s.o.rs, q_row, T, lg, o, 1.0f / wsum);
     }
     if (bad) dev_raise_fault(fault, tag);
   }  // pass
@@ -503,13 +518,44 @@ __global__ __launch_bounds__(FT, 2) void flash_bwd_dkv_kernel(
   if (bad) dev_raise_fault(fault, tag);
 }
 
+// ------------------------------------------------------------------ backward: the mean key row
+// key_mean[b, kv head, :] = the mean over time of that head's key rows, in f32. One workgroup per
+// (batch, kv head); a lane reads 8 values of a row, 256 / (D / 8) rows go round at once.
+template <int D>
+__global__ __launch_bounds__(256) void flash_key_mean_kernel(const unsigned short* __restrict__ k,
+                                                             float* __restrict__ key_mean, FlashShape s) {
+  constexpr int LPR = D / 8, ROWS = 256 / LPR;
+  __shared__ float part[ROWS][D];
+  const int b = blockIdx.x / s.kv_heads, h = blockIdx.x % s.kv_heads;
+  const unsigned short* kp = k + b * s.kv.bs + h * s.kv.hs;
+  const int col = (threadIdx.x % LPR) * 8, first = threadIdx.x / LPR;
+  float sum[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int row = first; row < s.time; row += ROWS) {
+    const u32x4 w = *reinterpret_cast<const u32x4*>(kp + static_cast<long>(row) * s.kv.rs + col);
+    const unsigned int ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      sum[2 * i] += __uint_as_float(ww[i] << 16);
+      sum[2 * i + 1] += __uint_as_float(ww[i] & 0xffff0000u);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) part[first][col + i] = sum[i];
+  __syncthreads();
+  if (threadIdx.x < D) {
+    float total = 0.0f;
+    for (int r = 0; r < ROWS; ++r) total += part[r][threadIdx.x];
+    key_mean[static_cast<long>(blockIdx.x) * D + threadIdx.x] = total / static_cast<float>(s.time);
+  }
+}
+
 // ------------------------------------------------------------------ backward: dQ
 template <int D, typename TO>
 __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_bwd_dq_kernel(
     const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
     const unsigned short* __restrict__ out, const unsigned short* __restrict__ resid, const float* __restrict__ lse,
-    float* __restrict__ delta, const unsigned short* __restrict__ gy, TO* __restrict__ gq, FlashShape s,
-    OmxFaultWord* fault, unsigned long long tag) {
+    float* __restrict__ delta, const float* __restrict__ key_mean, const unsigned short* __restrict__ gy,
+    TO* __restrict__ gq, FlashShape s, OmxFaultWord* fault, unsigned long long tag) {
   constexpr int KK = D / 16, MT = D / 32, NL = D / 32;
   __shared__ __attribute__((aligned(16))) char smem[2 * ftile(D)];
   char* k_rows = smem;
@@ -572,6 +618,12 @@ __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_bwd_dq_kernel(
     floatx16 dq[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) dq[mt] = zero16();
+    // A row of dS sums to zero, so dQ = dS K does not see a vector added to every key row. The
+    // bf16 copy of dS that the matrix units read sums to its rounding error instead, and that
+    // error times a component shared by all key rows (a residual stream grows one) lands in dQ at
+    // 2^-9 of the component, however small the part of K that varies. `ds_sum` collects this
+    // lane's share of the row sum of the rounded dS; the end takes (row sum) x (mean key) off.
+    float ds_sum = 0.0f;
     const float scale_log2 = s.scale * LOG2E;
     const int block_q0 = qb * 128, block_q1 = min(T - 1, qb * 128 + 127);
     const int kt_first = s.window > 0 ? max(0, block_q0 + 1 - s.window) / 64 : 0;
@@ -618,8 +670,23 @@ __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_bwd_dq_kernel(
           const u32x4 dsb = pack8(dp, c);
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) dq[mt] = mfma(frag_tr<D>(k_rows, mt, sub, c, lane), dsb, dq[mt]);
+          ds_sum = sum_pairs(dsb.x, sum_pairs(dsb.y, sum_pairs(dsb.z, sum_pairs(dsb.w, ds_sum))));
         }
       }
+    }
+    {
+      const float* mean = key_mean + (static_cast<long>(b) * s.kv_heads + kvh) * D;
+      const float row_sum = ds_sum + __shfl_xor(ds_sum, 32, 64);  // the two half-waves hold half the keys each
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          const float4 m = *reinterpret_cast<const float4*>(mean + mt * 32 + 8 * q4 + 4 * lg);
+          dq[mt][4 * q4 + 0] = fmaf(-row_sum, m.x, dq[mt][4 * q4 + 0]);
+          dq[mt][4 * q4 + 1] = fmaf(-row_sum, m.y, dq[mt][4 * q4 + 1]);
+          dq[mt][4 * q4 + 2] = fmaf(-row_sum, m.z, dq[mt][4 * q4 + 2]);
+          dq[mt][4 * q4 + 3] = fmaf(-row_sum, m.w, dq[mt][4 * q4 + 3]);
+        }
     }
     bad |= store_transposed_acc<D, TO>(gq + b * s.q.bs + h * s.q.hs, s.q.rs, q_row, T, lg, dq, s.scale);
     if (bad) dev_raise_fault(fault, tag);
@@ -667,8 +734,10 @@ void launch_forward(omx_ctx* ctx, const unsigned short* q, const unsigned short*
 template <int D>
 void launch_backward(omx_ctx* ctx, const unsigned short* q, const unsigned short* k, const unsigned short* v,
                      const unsigned short* out, const unsigned short* resid, const float* lse, float* delta,
-                     const unsigned short* gy, void* gq, void* gk, void* gv, int32_t grad_dtype, const FlashShape& s,
-                     unsigned long long tag) {
+                     float* key_mean, const unsigned short* gy, void* gq, void* gk, void* gv, int32_t grad_dtype,
+                     const FlashShape& s, unsigned long long tag) {
+  hipLaunchKernelGGL((flash_key_mean_kernel<D>), dim3(static_cast<unsigned>(s.batch * s.kv_heads)), dim3(256), 0,
+                     ctx->stream, k, key_mean, s);
   // dQ first: it also leaves delta = dO . O per row for the dK/dV pass.
   dim3 block(FT);
   const unsigned pairs = static_cast<unsigned>((s.time + 127) / 128 + 1) / 2;  // two 128-row blocks per workgroup
@@ -676,12 +745,12 @@ void launch_backward(omx_ctx* ctx, const unsigned short* q, const unsigned short
   dim3 q_grid(pairs * static_cast<unsigned>(s.batch * s.heads));
   if (grad_dtype == OMX_BF16) {
     hipLaunchKernelGGL((flash_bwd_dq_kernel<D, unsigned short>), q_grid, block, 0, ctx->stream, q, k, v, out, resid,
-                       lse, delta, gy, static_cast<unsigned short*>(gq), s, ctx->fault, tag);
+                       lse, delta, key_mean, gy, static_cast<unsigned short*>(gq), s, ctx->fault, tag);
     hipLaunchKernelGGL((flash_bwd_dkv_kernel<D, unsigned short>), kv_grid, block, 0, ctx->stream, q, k, v, lse, delta,
                        gy, static_cast<unsigned short*>(gk), static_cast<unsigned short*>(gv), s, ctx->fault, tag);
   } else {
     hipLaunchKernelGGL((flash_bwd_dq_kernel<D, float>), q_grid, block, 0, ctx->stream, q, k, v, out, resid, lse, delta,
-                       gy, static_cast<float*>(gq), s, ctx->fault, tag);
+                       key_mean, gy, static_cast<float*>(gq), s, ctx->fault, tag);
     hipLaunchKernelGGL((flash_bwd_dkv_kernel<D, float>), kv_grid, block, 0, ctx->stream, q, k, v, lse, delta, gy,
                        static_cast<float*>(gk), static_cast<float*>(gv), s, ctx->fault, tag);
   }
@@ -721,17 +790,19 @@ int32_t omx_flash_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, cons
   FlashShape s = make_shape(batch, heads, kv_heads, time, dim, window, scale, strides);
   const long rows = static_cast<long>(batch * heads * time);
   void* ws = nullptr;
-  int32_t rc = omx_workspace(ctx, rows * sizeof(float), &ws);
+  const long rows4 = (rows + 3) & ~3L;  // the mean key rows are read four values at a time
+  int32_t rc = omx_workspace(ctx, (rows4 + static_cast<long>(batch * kv_heads * dim)) * sizeof(float), &ws);
   if (rc != OMX_OK) return rc;
   float* delta = static_cast<float*>(ws);
+  float* key_mean = delta + rows4;
   const unsigned short* qs = static_cast<const unsigned short*>(q);
   const unsigned short* ks = static_cast<const unsigned short*>(k);
   const unsigned short* vs = static_cast<const unsigned short*>(v);
   const unsigned short* os = static_cast<const unsigned short*>(out);
   const unsigned short* rs = static_cast<const unsigned short*>(out_residual);
   const unsigned short* gs = static_cast<const unsigned short*>(gy);
-  if (dim == 64) launch_backward<64>(ctx, qs, ks, vs, os, rs, lse, delta, gs, gq, gk, gv, grad_dtype, s, tag);
-  else launch_backward<128>(ctx, qs, ks, vs, os, rs, lse, delta, gs, gq, gk, gv, grad_dtype, s, tag);
+  if (dim == 64) launch_backward<64>(ctx, qs, ks, vs, os, rs, lse, delta, key_mean, gs, gq, gk, gv, grad_dtype, s, tag);
+  else launch_backward<128>(ctx, qs, ks, vs, os, rs, lse, delta, key_mean, gs, gq, gk, gv, grad_dtype, s, tag);
   OMX_LAUNCH_CHECK(ctx, "flash backward kernels");
   return OMX_OK;
 }

@@ -335,12 +335,13 @@ def test_attention_saved_residual_keeps_the_row_term_exact(be, b, t, h, hkv, win
         print("   common", common, "normwise error plain / saved: gq %.2e / %.2e, gk %.2e / %.2e"
               % (errs[0] + errs[1]), flush=True)
         for plain_e, saved_e in errs:
-            assert saved_e <= (3e-2 if common else 5e-3) and saved_e <= 1.05 * plain_e
+            assert saved_e <= 4e-3 and saved_e <= 1.05 * plain_e
         if common:
-            # Measured at a common component of 2 (3.6 sigma): gq 1.6e-1 -> 2.3e-2, gk 6.3e-3 ->
-            # 3.0e-3. What is left in gq is the bf16 rounding of P (forward) and of dS (backward)
-            # against the same common key.
-            assert errs[0][1] <= errs[0][0] / 5
+            # Measured at a common component of 2 (3.6 sigma): gq 5.5e-3 -> 2.3e-3, gk 5.9e-3 ->
+            # 2.3e-3, the level of the case without one. (The gap was 1.6e-1 -> 2.3e-2 while the
+            # forward divided by the unrounded sum of its weights and the dQ pass left the rounding
+            # of dS against the common key in.)
+            assert errs[0][1] <= errs[0][0] / 2 and errs[1][1] <= errs[1][0] / 2
 
 
 @pytest.mark.parametrize("bf16", [False, True])
