@@ -10,9 +10,14 @@ tokens that are resident in HBM before the clock starts.
 Prints one JSON line. `roofline` covers the dominant kernel, the bf16 MFMA GEMM:
 algorithmic 2*M*N*K FLOPs of its launches divided by their summed duration,
 measured with HIP events on the library's own stream during the timed steps.
-`cpu_baseline` times the CPU oracle (a C++ restatement of the reference's CPU
-Exact arithmetic; the Rust reference cannot be built without cargo) on the
-host cores, on a bounded sample of the same workload.
+`roofline_per_kernel` gives the same for the other kernel classes of the step
+(flash attention forward and backward against the MFMA peak; cross-entropy,
+AdamW, RMSNorm forward and backward and the embedding backward against HBM
+bandwidth), each from the dispatch timestamps of its own launches in the same
+timed steps. `cpu_baseline` times the CPU oracle (a C++ restatement of the
+reference's CPU Exact arithmetic; the Rust reference cannot be built without
+cargo) on the host cores, on a bounded sample of the same workload, with all
+cores and with one thread, three repeats each.
 """
 import argparse
 import ctypes as C
@@ -37,32 +42,129 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor figure
 GEMM_HBM_BYTES_PER_LAUNCH_GPT124M = 3.82e8
 
 
+# Kernel classes of omx_profile_kernels beyond the GEMM products: (bit, key, kernels, roofline).
+KERNEL_CLASSES = [
+    (1, "flash_attention_forward", "flash_fwd_kernel", "mfma"),
+    (2, "flash_attention_backward", "flash_key_mean_kernel + flash_bwd_dq_kernel + flash_bwd_dkv_kernel", "mfma"),
+    (3, "cross_entropy", "ce_row_fused_kernel", "hbm"),
+    (4, "adamw", "adamw_apply_kernel (after adamw_check_kernel when it runs)", "hbm"),
+    (5, "rms_norm_forward", "rms_fwd_vec_kernel", "hbm"),
+    (6, "rms_norm_backward", "rms_bwd_vec_kernel + column_sum kernels", "hbm"),
+    (7, "embedding_backward", "count / scan / fill / sort kernels + embedding_bwd_kernel", "hbm"),
+]
+ALL_CLASSES_MASK = 0xFF
+
+
+def kernel_rooflines(lib, ctx, timed_steps: int):
+    """Reads the per-class records of omx_profile_kernels: achieved = the launches' algorithmic FLOPs
+    (matrix-unit classes, causal-counted for attention) or bytes (every operand read once, every
+    result written once) over their summed dispatch durations."""
+    out = {}
+    for bit, key, kernels, bound in KERNEL_CLASSES:
+        launches, ms, work = C.c_uint64(), C.c_double(), C.c_double()
+        lib.omx_profile_kernels_report(ctx, C.c_int32(bit), C.byref(launches), C.byref(ms), C.byref(work))
+        if launches.value == 0:
+            continue
+        peak = BF16_MFMA_PEAK_TFLOPS if bound == "mfma" else HBM_PEAK_GBS
+        achieved = work.value / (ms.value * 1e-3) / (1e12 if bound == "mfma" else 1e9)
+        out[key] = {"bound": bound, "kernel": kernels, "achieved": achieved, "peak": peak,
+                    "unit": "TFLOP/s" if bound == "mfma" else "GB/s", "frac": achieved / peak, "traffic": None,
+                    "launches": int(launches.value), "avg_launch_us": ms.value * 1e3 / launches.value,
+                    "ms_per_step": ms.value / max(1, timed_steps)}
+    return out
+
+
+def cpu_model() -> str:
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def repeat_timed(fn, repeats: int = 3):
+    """fn() -> seconds of the part it times itself; returns the sorted list of `repeats` runs."""
+    return sorted(fn() for _ in range(repeats))
+
+
 def cpu_baseline(cfg, threads: int):
-    """Times the oracle on a bounded sample: the same model on one 1 x 1024 token
-    sequence (forward + backward + clip + AdamW), reported per token."""
+    """Times the oracle on a bounded sample of the same model and scales it to the step.
+
+    Sequences share nothing but the weights and blocks cost the same, so the step's time is
+    tokens x (rest + layers x block) / sample tokens + the optimizer pass, with `block` and `rest`
+    from the model at one and at two blocks on one short sequence, and the optimizer (clip +
+    AdamW) timed on one block's parameters and scaled by the parameter count. A configuration small
+    enough (the tiny one) is timed whole instead. All cores and one thread, three repeats each;
+    `value` is the median of the all-cores runs."""
     sys.path.insert(0, str(ROOT / "tests"))
     import oracle_api as orc
     from ojas_amd.trainer import GptConfig, synthetic_batch
 
-    sample = GptConfig(cfg.layers, cfg.d_model, cfg.heads, cfg.head_dim, cfg.mlp, min(cfg.ctx, 1024), cfg.vocab, 1, cfg.gelu_tanh, 0)
-    ocfg = orc.GptConfig(sample.layers, sample.d_model, sample.heads, sample.head_dim, sample.mlp, sample.ctx,
-                         sample.vocab, sample.batch, sample.gelu_tanh)
-    orc.set_threads(threads)
+    tokens = cfg.batch * cfg.ctx
+    whole = tokens * cfg.layers * cfg.d_model * cfg.d_model < 3e9  # the tiny configuration: 0.5e9
     rng = np.random.default_rng(0)
-    params = [np.ones(n, np.float32) if n == sample.d_model else rng.normal(0, 0.02, n).astype(np.float32)
-              for n in orc.gpt_param_lens(ocfg)]
-    ids, targets = synthetic_batch(sample, 1)
-    t0 = time.perf_counter()
-    _, grads = orc.gpt_loss_and_grads(ocfg, params, ids.reshape(-1), targets.reshape(-1))
-    _, grads = orc.clip_grad_norm(grads, 1.0)
-    for p, g in zip(params, grads):
-        orc.adamw_step(p, g, np.zeros_like(p), np.zeros_like(p), 0, 3e-4, 0.9, 0.95, 1e-8, 0.1, exact=True)
-    dt = time.perf_counter() - t0
-    tokens = sample.batch * sample.ctx
-    return {"value": tokens / dt, "unit": "tokens/s", "cores": threads, "kind": "port",
-            "sample": f"same model (L{sample.layers} d{sample.d_model} vocab{sample.vocab}), one step on "
-                      f"1x{sample.ctx} tokens in f32 Exact arithmetic "
-                      f"({dt:.1f} s), scaled per token; C++ restatement of ojas-cpu, not the Rust binary"}
+
+    def model(layers, batch, ctx):
+        sample = GptConfig(layers, cfg.d_model, cfg.heads, cfg.head_dim, cfg.mlp, ctx, cfg.vocab, batch, cfg.gelu_tanh, 0)
+        ocfg = orc.GptConfig(layers, cfg.d_model, cfg.heads, cfg.head_dim, cfg.mlp, ctx, cfg.vocab, batch, cfg.gelu_tanh)
+        params = [np.ones(n, np.float32) if n == cfg.d_model else rng.normal(0, 0.02, n).astype(np.float32)
+                  for n in orc.gpt_param_lens(ocfg)]
+        ids, targets = synthetic_batch(sample, 1)
+        return ocfg, params, ids.reshape(-1), targets.reshape(-1)
+
+    def optimizer_seconds(params, grads):
+        moments = [(np.zeros_like(p), np.zeros_like(p)) for p in params]
+        t0 = time.perf_counter()
+        _, clipped = orc.clip_grad_norm(grads, 1.0)
+        for p, g, (m, v) in zip(params, clipped, moments):
+            orc.adamw_step(p, g, m, v, 0, 3e-4, 0.9, 0.95, 1e-8, 0.1, exact=True)
+        return time.perf_counter() - t0
+
+    def measure(n_threads, sample_ctx):
+        orc.set_threads(n_threads)
+        if whole:
+            ocfg, params, ids, targets = model(cfg.layers, cfg.batch, cfg.ctx)
+
+            def once():
+                t0 = time.perf_counter()
+                _, grads = orc.gpt_loss_and_grads(ocfg, params, ids, targets)
+                return time.perf_counter() - t0 + optimizer_seconds(params, grads)
+
+            runs = repeat_timed(once)
+            return runs, f"the whole step ({cfg.batch}x{cfg.ctx} tokens)"
+        one, two = model(1, 1, sample_ctx), model(2, 1, sample_ctx)
+        n_params = sum(orc.gpt_param_lens(orc.GptConfig(cfg.layers, cfg.d_model, cfg.heads, cfg.head_dim, cfg.mlp,
+                                                        cfg.ctx, cfg.vocab, cfg.batch, cfg.gelu_tanh)))
+        block_params = [p for p in one[1][2:-1]]  # the block's eight tensors
+
+        def once():
+            t = []
+            for ocfg, params, ids, targets in (one, two):
+                t0 = time.perf_counter()
+                orc.gpt_loss_and_grads(ocfg, params, ids, targets)
+                t.append(time.perf_counter() - t0)
+            block = max(t[1] - t[0], 1e-9)
+            rest = max(t[0] - block, 0.0)
+            opt = optimizer_seconds(block_params, [np.full_like(p, 1e-3) for p in block_params])
+            opt *= n_params / sum(p.size for p in block_params)
+            return tokens * (rest + cfg.layers * block) / sample_ctx + opt
+
+        runs = repeat_timed(once)
+        return runs, (f"one and two blocks on 1x{sample_ctx} tokens (block and rest), clip + AdamW on one block's "
+                      f"parameters, scaled to {cfg.layers} blocks, {tokens} tokens and {n_params} parameters")
+
+    all_runs, how = measure(threads, 256)
+    one_runs, how_one = measure(1, 64)
+    note = ("" if whole else " Attention grows with the sequence: at these sample lengths it is a smaller share than at "
+            f"{cfg.ctx}, so the estimate favours the CPU by up to its 8 % of the step's work.")
+    return {"value": tokens / all_runs[1], "unit": "tokens/s", "cores": threads, "kind": "port",
+            "cpu_model": cpu_model(), "repeats": 3, "step_seconds_min": all_runs[0], "step_seconds_median": all_runs[1],
+            "single_thread": {"value": tokens / one_runs[1], "cores": 1, "step_seconds_min": one_runs[0],
+                              "step_seconds_median": one_runs[1], "sample": how_one},
+            "sample": f"same model (L{cfg.layers} d{cfg.d_model} vocab{cfg.vocab}) in f32 Exact arithmetic: {how}."
+                      f"{note} C++ restatement of ojas-cpu, not the Rust binary"}
 
 
 def kv_decode(args) -> int:
@@ -123,17 +225,18 @@ def kv_decode(args) -> int:
 
 
 def lora_cpu_baseline(cfg, threads: int):
-    """Times the oracle's LoRA step on a bounded sample of the same model: full width, 256 tokens of
-    one sequence, once with one block and once with two; the difference is a block's time, the rest
-    the table, final norm and head, and the model's 16 blocks are extrapolated from the two."""
+    """Times the oracle's LoRA step on a bounded sample of the same model at full width: one short
+    sequence, once with one block and once with two; the difference is a block's time, the rest the
+    table, final norm and head; the step is tokens x (rest + layers x block) / sample tokens plus
+    clip + AdamW on the adapters (timed on the two-block model's, scaled by their count). All cores
+    and one thread, three repeats each; `value` is the median of the all-cores runs."""
     sys.path.insert(0, str(ROOT / "tests"))
     import oracle_api as orc
 
-    orc.set_threads(threads)
-    seq = 256
+    tokens = cfg.batch * cfg.seq
     rng = np.random.default_rng(0)
-    times = []
-    for layers in (1, 2):
+
+    def model(layers, seq):
         ocfg = orc.LoraConfig(layers, cfg.d_model, cfg.heads, cfg.head_dim, cfg.hidden, cfg.vocab, 1, seq, cfg.rank,
                               cfg.rms_eps, cfg.lora_scale, cfg.rope_base)
         frozen = []
@@ -142,26 +245,49 @@ def lora_cpu_baseline(cfg, threads: int):
                 frozen.append(np.ones(shape, np.float32))
             elif shape[0] == cfg.vocab:
                 frozen.append(rng.normal(0, 0.02, shape).astype(np.float32))
-            else:
-                codes, scales = orc.quantize_i8_group(rng.normal(0, 0.02, shape).astype(np.float32), 32)
+            else:  # codes and scales drawn directly: the values a quantised N(0, 0.02) matrix dequantises to
+                codes = rng.integers(-127, 128, shape).astype(np.int8)
+                scales = np.full((shape[0], shape[1] // 32), 0.05 / 127, np.float32)
                 frozen.append(orc.dequant_i8_group(codes, scales, 32))
         adapters = [rng.normal(0, 0.02, sh).astype(np.float32) for sh in orc.lora_adapter_shapes(ocfg)]
         ids = rng.integers(0, cfg.vocab, seq).astype(np.uint32)
         targets = rng.integers(0, cfg.vocab, seq).astype(np.uint32)
-        t0 = time.perf_counter()
-        _, grads = orc.lora_loss_and_grads(ocfg, frozen, adapters, ids, targets)
-        _, grads = orc.clip_grad_norm(grads, 1.0)
-        for p, g in zip(adapters, grads):
-            p = p.reshape(-1)
-            orc.adamw_step(p, g, np.zeros_like(p), np.zeros_like(p), 0, 1e-4, 0.9, 0.95, 1e-8, 0.0, exact=True)
-        times.append(time.perf_counter() - t0)
-    per_block = max(times[1] - times[0], 1e-9)
-    rest = max(times[0] - per_block, 0.0)
-    full = rest + cfg.layers * per_block
-    return {"value": seq / full, "unit": "tokens/s", "cores": threads, "kind": "port",
-            "sample": f"same model at full width, 1x{seq} tokens, f32 Exact arithmetic on dequantised weights: "
-                      f"1 block {times[0]:.1f} s, 2 blocks {times[1]:.1f} s, extrapolated to {cfg.layers} blocks "
-                      f"({full:.1f} s); C++ restatement of ojas-cpu, not the Rust binary"}
+        return ocfg, frozen, adapters, ids, targets
+
+    def measure(n_threads, seq):
+        orc.set_threads(n_threads)
+        one, two = model(1, seq), model(2, seq)
+
+        def once():
+            t = []
+            for ocfg, frozen, adapters, ids, targets in (one, two):
+                t0 = time.perf_counter()
+                _, grads = orc.lora_loss_and_grads(ocfg, frozen, adapters, ids, targets)
+                t.append(time.perf_counter() - t0)
+            flat = [a.reshape(-1).copy() for a in two[2]]
+            moments = [(np.zeros_like(p), np.zeros_like(p)) for p in flat]
+            t0 = time.perf_counter()
+            _, clipped = orc.clip_grad_norm(grads, 1.0)
+            for p, g, (m, v) in zip(flat, clipped, moments):
+                orc.adamw_step(p, g, m, v, 0, 1e-4, 0.9, 0.95, 1e-8, 0.0, exact=True)
+            opt = (time.perf_counter() - t0) * cfg.layers / 2
+            block = max(t[1] - t[0], 1e-9)
+            rest = max(t[0] - block, 0.0)
+            return tokens * (rest + cfg.layers * block) / seq + opt
+
+        return repeat_timed(once)
+
+    all_runs = measure(threads, 128)
+    one_runs = measure(1, 32)
+    return {"value": tokens / all_runs[1], "unit": "tokens/s", "cores": threads, "kind": "port",
+            "cpu_model": cpu_model(), "repeats": 3, "step_seconds_min": all_runs[0], "step_seconds_median": all_runs[1],
+            "single_thread": {"value": tokens / one_runs[1], "cores": 1, "step_seconds_min": one_runs[0],
+                              "step_seconds_median": one_runs[1], "sample": "as below on 1x32 tokens"},
+            "sample": f"same model at full width in f32 Exact arithmetic on dequantised weights: one and two blocks on "
+                      f"1x128 tokens (block and rest), clip + AdamW on two blocks' adapters, scaled to {cfg.layers} "
+                      f"blocks and {tokens} tokens. Attention grows with the sequence: at this sample length it is a "
+                      f"smaller share than at {cfg.seq}, so the estimate favours the CPU by up to its 9 % of the step's "
+                      f"work. C++ restatement of ojas-cpu, not the Rust binary"}
 
 
 def lora_step(args) -> int:
@@ -185,7 +311,7 @@ def lora_step(args) -> int:
     step_ms = []
     t0 = time.perf_counter()
     for i in range(args.steps):
-        lib.omx_profile_gemm(be._ctx, C.c_int32(1 if i % timed_every == 0 else 0))
+        lib.omx_profile_kernels(be._ctx, C.c_uint32(ALL_CLASSES_MASK if i % timed_every == 0 else 0))
         s0 = time.perf_counter()
         losses.append(tr.step(adamw, 1.0)[0])  # ends with the loss readback: the step is complete
         step_ms.append((time.perf_counter() - s0) * 1e3)
@@ -193,7 +319,8 @@ def lora_step(args) -> int:
     dt = time.perf_counter() - t0
     launches, gemm_ms, gemm_flops = C.c_uint64(), C.c_double(), C.c_double()
     lib.omx_profile_gemm_report(be._ctx, C.byref(launches), C.byref(gemm_ms), C.byref(gemm_flops))
-    lib.omx_profile_gemm(be._ctx, C.c_int32(0))
+    per_kernel = kernel_rooflines(lib, be._ctx, len(range(0, args.steps, timed_every)))
+    lib.omx_profile_kernels(be._ctx, C.c_uint32(0))
     tokens = cfg.batch * cfg.seq
     ms_per_step = dt / args.steps * 1e3
     flops = step_flops(cfg)
@@ -220,6 +347,7 @@ def lora_step(args) -> int:
                      "frac": achieved / BF16_MFMA_PEAK_TFLOPS, "traffic": None, "launches": int(launches.value),
                      "avg_launch_us": gemm_ms.value * 1e3 / max(1, launches.value), "timed_steps": timed_steps,
                      "gemm_ms_per_step": gemm_ms.value / max(1, timed_steps)},
+        "roofline_per_kernel": per_kernel,
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = lora_cpu_baseline(cfg, min(16, os.cpu_count() or 1))
@@ -271,20 +399,25 @@ def main() -> int:
         losses.append(one_step())
     be.sync()
     lib = be._lib
-    # The GEMM kernels of every fourth timed step carry HIP events on their dispatches (begin and
-    # end timestamps of the kernels themselves). All steps would cost 0.7 ms per step on the
-    # number being measured (the timed launch path is slower: 103 products per step); a quarter
-    # of them is 515 timed products in the default run.
+    # The kernels of every fourth timed step carry HIP events on their dispatches (begin and end
+    # timestamps of the kernels themselves): the GEMM products and the classes of KERNEL_CLASSES.
+    # All steps would cost about a millisecond per step on the number being measured (the timed
+    # launch path is slower: 103 products and some 80 other launches per step); a quarter of them
+    # is 515 timed products in the default run.
     timed_every = 4
+    step_ms = []
     t0 = time.perf_counter()
     for i in range(args.steps):
-        lib.omx_profile_gemm(be._ctx, C.c_int32(1 if i % timed_every == 0 else 0))
-        losses.append(one_step())
+        lib.omx_profile_kernels(be._ctx, C.c_uint32(ALL_CLASSES_MASK if i % timed_every == 0 else 0))
+        s0 = time.perf_counter()
+        losses.append(one_step())  # ends with the loss readback: the step is complete
+        step_ms.append((time.perf_counter() - s0) * 1e3)
     be.sync()
     dt = time.perf_counter() - t0
     launches, gemm_ms, gemm_flops = C.c_uint64(), C.c_double(), C.c_double()
     lib.omx_profile_gemm_report(be._ctx, C.byref(launches), C.byref(gemm_ms), C.byref(gemm_flops))
-    lib.omx_profile_gemm(be._ctx, C.c_int32(0))
+    per_kernel = kernel_rooflines(lib, be._ctx, len(range(0, args.steps, timed_every)))
+    lib.omx_profile_kernels(be._ctx, C.c_uint32(0))
 
     tokens = cfg.batch * cfg.ctx
     ms_per_step = dt / args.steps * 1e3
@@ -303,6 +436,8 @@ def main() -> int:
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": ms_per_step,
+        "ms_per_step_min": float(np.min(step_ms)),
+        "ms_per_step_median": float(np.median(step_ms)),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -324,10 +459,13 @@ def main() -> int:
                      "kernel": "gemm_dma_kernel / gemm_kernel (bf16 MFMA GEMM, all operand layouts)" if cfg.bf16
                                else "gemm_kernel<float> (f32 MFMA GEMM, all operand layouts)",
                      "achieved": achieved, "peak": gemm_peak, "unit": "TFLOP/s", "frac": achieved / gemm_peak,
-                     "traffic": GEMM_HBM_BYTES_PER_LAUNCH_GPT124M if args.config == "gpt124m" else None,
+                     # measured on the AdamW step of this configuration only
+                     "traffic": GEMM_HBM_BYTES_PER_LAUNCH_GPT124M
+                     if args.config == "gpt124m" and args.optimizer == "adamw" else None,
                      "launches": int(launches.value), "avg_launch_us": gemm_ms.value * 1e3 / max(1, launches.value),
                      "timed_steps": len(range(0, args.steps, timed_every)),
                      "gemm_ms_per_step": gemm_ms.value / max(1, len(range(0, args.steps, timed_every)))},
+        "roofline_per_kernel": per_kernel,
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, min(16, os.cpu_count() or 1))

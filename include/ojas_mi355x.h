@@ -562,6 +562,21 @@ int32_t omx_set_option(omx_ctx* ctx, const char* name, int64_t value);
 int32_t omx_profile_gemm(omx_ctx* ctx, int32_t enable);
 int32_t omx_profile_gemm_report(omx_ctx* ctx, uint64_t* launches, double* total_ms,
                                 double* total_flops);
+/* The same for the other kernel classes of the step (same standing: benchmark
+ * instrumentation with no counterpart in the reference). `class_mask` has one
+ * bit per class: 0 the GEMM products (as omx_profile_gemm), 1 flash attention
+ * forward, 2 flash attention backward (mean key row, dQ, dK / dV kernels as one
+ * launch), 3 the fused cross-entropy row kernel, 4 AdamW (checking pass, when
+ * it runs, and update), 5 RMSNorm forward and 6 backward (with the weight
+ * gradient's column sum) for row widths 256..2048, 7 embedding backward (count,
+ * scan, fill, sort and accumulate kernels as one launch). A launch's work is
+ * its algorithmic FLOPs (classes 0..2: 2 B H T^2 D forward and 5 B H T^2 D
+ * backward, causal-counted) or its algorithmic bytes (classes 3..7: every
+ * operand read once and every result written once). The report sums one class
+ * and clears its record. */
+int32_t omx_profile_kernels(omx_ctx* ctx, uint32_t class_mask);
+int32_t omx_profile_kernels_report(omx_ctx* ctx, int32_t kernel_class, uint64_t* launches,
+                                   double* total_ms, double* total_work);
 
 /* Every Backend method outside the GPT op set answers through this: sets the
  * error text to the op's name and returns OMX_UNSUPPORTED

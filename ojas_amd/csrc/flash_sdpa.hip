@@ -722,13 +722,15 @@ void launch_forward(omx_ctx* ctx, const unsigned short* q, const unsigned short*
                     int32_t out_dtype, void* out_residual, float* lse, const FlashShape& s, unsigned long long tag) {
   // Two 128-row query blocks per workgroup (see the kernel).
   dim3 grid(static_cast<unsigned>((s.time + 127) / 128 + 1) / 2 * s.batch * s.heads), block(FT);
+  // Causal-counted work: half of the 4 B H T^2 D of the two full products.
+  OmxKernelTimer timer(ctx, OMX_K_FLASH_FWD, 2.0 * s.batch * s.heads * static_cast<double>(s.time) * s.time * D);
   if (out_dtype == OMX_BF16)
-    hipLaunchKernelGGL((flash_fwd_kernel<D, unsigned short>), grid, block, 0, ctx->stream, q, k, v,
-                       static_cast<unsigned short*>(out), static_cast<unsigned short*>(out_residual), lse, s,
-                       ctx->fault, tag);
+    omx_launch_timed(ctx, flash_fwd_kernel<D, unsigned short>, grid, block, 0, timer.start(), timer.stop(), q, k, v,
+                     static_cast<unsigned short*>(out), static_cast<unsigned short*>(out_residual), lse, s, ctx->fault,
+                     tag);
   else
-    hipLaunchKernelGGL((flash_fwd_kernel<D, float>), grid, block, 0, ctx->stream, q, k, v, static_cast<float*>(out),
-                       static_cast<unsigned short*>(nullptr), lse, s, ctx->fault, tag);
+    omx_launch_timed(ctx, flash_fwd_kernel<D, float>, grid, block, 0, timer.start(), timer.stop(), q, k, v,
+                     static_cast<float*>(out), static_cast<unsigned short*>(nullptr), lse, s, ctx->fault, tag);
 }
 
 template <int D>
@@ -736,8 +738,10 @@ void launch_backward(omx_ctx* ctx, const unsigned short* q, const unsigned short
                      const unsigned short* out, const unsigned short* resid, const float* lse, float* delta,
                      float* key_mean, const unsigned short* gy, void* gq, void* gk, void* gv, int32_t grad_dtype,
                      const FlashShape& s, unsigned long long tag) {
-  hipLaunchKernelGGL((flash_key_mean_kernel<D>), dim3(static_cast<unsigned>(s.batch * s.kv_heads)), dim3(256), 0,
-                     ctx->stream, k, key_mean, s);
+  // Five causal-counted products (S and dP twice each way, dV, dQ, dK) of B H T^2 D each.
+  OmxKernelTimer timer(ctx, OMX_K_FLASH_BWD, 5.0 * s.batch * s.heads * static_cast<double>(s.time) * s.time * D);
+  omx_launch_timed(ctx, flash_key_mean_kernel<D>, dim3(static_cast<unsigned>(s.batch * s.kv_heads)), dim3(256), 0,
+                   timer.start(), nullptr, k, key_mean, s);
   // dQ first: it also leaves delta = dO . O per row for the dK/dV pass.
   dim3 block(FT);
   const unsigned pairs = static_cast<unsigned>((s.time + 127) / 128 + 1) / 2;  // two 128-row blocks per workgroup
@@ -746,13 +750,14 @@ void launch_backward(omx_ctx* ctx, const unsigned short* q, const unsigned short
   if (grad_dtype == OMX_BF16) {
     hipLaunchKernelGGL((flash_bwd_dq_kernel<D, unsigned short>), q_grid, block, 0, ctx->stream, q, k, v, out, resid,
                        lse, delta, key_mean, gy, static_cast<unsigned short*>(gq), s, ctx->fault, tag);
-    hipLaunchKernelGGL((flash_bwd_dkv_kernel<D, unsigned short>), kv_grid, block, 0, ctx->stream, q, k, v, lse, delta,
-                       gy, static_cast<unsigned short*>(gk), static_cast<unsigned short*>(gv), s, ctx->fault, tag);
+    omx_launch_timed(ctx, flash_bwd_dkv_kernel<D, unsigned short>, kv_grid, block, 0, nullptr, timer.stop(), q, k, v,
+                     lse, delta, gy, static_cast<unsigned short*>(gk), static_cast<unsigned short*>(gv), s, ctx->fault,
+                     tag);
   } else {
     hipLaunchKernelGGL((flash_bwd_dq_kernel<D, float>), q_grid, block, 0, ctx->stream, q, k, v, out, resid, lse, delta,
                        key_mean, gy, static_cast<float*>(gq), s, ctx->fault, tag);
-    hipLaunchKernelGGL((flash_bwd_dkv_kernel<D, float>), kv_grid, block, 0, ctx->stream, q, k, v, lse, delta, gy,
-                       static_cast<float*>(gk), static_cast<float*>(gv), s, ctx->fault, tag);
+    omx_launch_timed(ctx, flash_bwd_dkv_kernel<D, float>, kv_grid, block, 0, nullptr, timer.stop(), q, k, v, lse, delta,
+                     gy, static_cast<float*>(gk), static_cast<float*>(gv), s, ctx->fault, tag);
   }
 }
 

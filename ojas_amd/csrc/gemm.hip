@@ -607,6 +607,28 @@ void omx_timing_end(omx_ctx* ctx, bool launched, const omx_ctx::TimedLaunch& tim
   if (launched) ctx->timed.push_back(timed);
 }
 
+OmxKernelTimer::OmxKernelTimer(omx_ctx* c, int cls, double work) : ctx(c) {
+  if (!(ctx->profile_classes >> cls & 1u)) return;
+  hipEvent_t* both[2] = {&t.start, &t.stop};
+  for (hipEvent_t* e : both) {
+    if (!ctx->event_pool.empty()) {
+      *e = ctx->event_pool.back();
+      ctx->event_pool.pop_back();
+    } else if (hipEventCreate(e) != hipSuccess) {
+      (void)hipGetLastError();
+      if (e == &t.stop) ctx->event_pool.push_back(t.start);
+      return;  // this launch goes untimed
+    }
+  }
+  t.flops = work;
+  t.cls = cls;
+  on = true;
+}
+
+OmxKernelTimer::~OmxKernelTimer() {
+  if (on) ctx->timed.push_back(t);
+}
+
 extern "C" {
 
 int32_t omx_set_option(omx_ctx* ctx, const char* name, int64_t value) {
@@ -649,23 +671,43 @@ int32_t omx_profile_gemm(omx_ctx* ctx, int32_t enable) {
   return OMX_OK;
 }
 
-int32_t omx_profile_gemm_report(omx_ctx* ctx, uint64_t* launches, double* total_ms, double* total_flops) {
+int32_t omx_profile_kernels(omx_ctx* ctx, uint32_t class_mask) {
   OMX_REQUIRE_CTX(ctx);
+  if (class_mask >> OMX_K_CLASSES) return omx_fail(ctx, OMX_OUT_OF_RANGE, "profile_kernels: classes 0..%d", OMX_K_CLASSES - 1);
+  ctx->profile_gemm = (class_mask & 1u) != 0;
+  ctx->profile_classes = class_mask & ~1u;
+  return OMX_OK;
+}
+
+int32_t omx_profile_kernels_report(omx_ctx* ctx, int32_t cls, uint64_t* launches, double* total_ms, double* total_work) {
+  OMX_REQUIRE_CTX(ctx);
+  if (cls < 0 || cls >= OMX_K_CLASSES) return omx_fail(ctx, OMX_OUT_OF_RANGE, "profile_kernels_report: class %d", cls);
   OMX_HIP(ctx, hipStreamSynchronize(ctx->stream));
-  double ms = 0.0, flops = 0.0;
+  double ms = 0.0, work = 0.0;
+  uint64_t count = 0;
+  std::vector<omx_ctx::TimedLaunch> rest;
   for (auto& t : ctx->timed) {
+    if (t.cls != cls) {
+      rest.push_back(t);
+      continue;
+    }
     float one = 0.0f;
     OMX_HIP(ctx, hipEventElapsedTime(&one, t.start, t.stop));
     ms += one;
-    flops += t.flops;
+    work += t.flops;
+    ++count;
     ctx->event_pool.push_back(t.start);
     ctx->event_pool.push_back(t.stop);
   }
-  if (launches) *launches = ctx->timed.size();
+  ctx->timed.swap(rest);
+  if (launches) *launches = count;
   if (total_ms) *total_ms = ms;
-  if (total_flops) *total_flops = flops;
-  ctx->timed.clear();
+  if (total_work) *total_work = work;
   return OMX_OK;
+}
+
+int32_t omx_profile_gemm_report(omx_ctx* ctx, uint64_t* launches, double* total_ms, double* total_flops) {
+  return omx_profile_kernels_report(ctx, OMX_K_GEMM, launches, total_ms, total_flops);
 }
 
 int32_t omx_gemm(omx_ctx* ctx, const void* a, uint64_t a_rs, uint64_t a_cs, const void* b, uint64_t b_rs,

@@ -599,14 +599,16 @@ int32_t omx_linear_cross_entropy_mean(omx_ctx* ctx, const void* x, const void* w
       if (rc != OMX_OK) return rc;
       if (fuse) {
         dim3 grid(static_cast<unsigned>(nr)), block(CE_FUSED_THREADS);
+        // One read of the logits tile and one write of the gradient over it.
+        OmxKernelTimer timer(ctx, OMX_K_CE, 2.0 * static_cast<double>(nr) * static_cast<double>(nc) * esz);
         if (operand_dtype == OMX_F32)
-          hipLaunchKernelGGL((ce_row_fused_kernel<float, CE_FUSED_PACKS>), grid, block, 0, ctx->stream,
-                             static_cast<float*>(tile), nc, r0, static_cast<unsigned>(nc), tg, has_ignore,
-                             ignore_index, s.st, s.valid, ctx->fault, tag);
+          omx_launch_timed(ctx, ce_row_fused_kernel<float, CE_FUSED_PACKS>, grid, block, 0, timer.start(), timer.stop(),
+                           static_cast<float*>(tile), nc, r0, static_cast<unsigned>(nc), tg, has_ignore, ignore_index,
+                           s.st, s.valid, ctx->fault, tag);
         else
-          hipLaunchKernelGGL((ce_row_fused_kernel<unsigned short, CE_FUSED_PACKS>), grid, block, 0, ctx->stream,
-                             static_cast<unsigned short*>(tile), nc, r0, static_cast<unsigned>(nc), tg, has_ignore,
-                             ignore_index, s.st, s.valid, ctx->fault, tag);
+          omx_launch_timed(ctx, ce_row_fused_kernel<unsigned short, CE_FUSED_PACKS>, grid, block, 0, timer.start(),
+                           timer.stop(), static_cast<unsigned short*>(tile), nc, r0, static_cast<unsigned>(nc), tg,
+                           has_ignore, ignore_index, s.st, s.valid, ctx->fault, tag);
         OMX_LAUNCH_CHECK(ctx, "ce_row_fused_kernel");
         continue;
       }

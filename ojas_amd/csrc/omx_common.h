@@ -96,12 +96,14 @@ struct omx_ctx {
   int adamw_trust = 1;        // 0: omx_adamw_step_bounded always runs its checking pass
   int ce_fused = 1;           // 0: linear-CE always takes the separate statistics and gradient kernels
   bool profile_gemm = false;
+  uint32_t profile_classes = 0;  // bit per OmxKernelClass other than the products (omx_profile_kernels)
   // The events of the product being launched (null when not timing): the first kernel of the
   // product takes `timing_start`, its last one `timing_stop`.
   hipEvent_t timing_start = nullptr, timing_stop = nullptr;
   struct TimedLaunch {
     hipEvent_t start, stop;
-    double flops;
+    double flops;  // the launch's algorithmic work: FLOPs for the matrix-unit classes, bytes for the others
+    int cls = 0;
   };
   std::vector<TimedLaunch> timed;
   std::vector<hipEvent_t> event_pool;
@@ -122,6 +124,27 @@ void omx_release_pool(omx_ctx* ctx);
 // to be launched (when omx_profile_gemm is on) and files them with its FLOP count afterwards.
 int32_t omx_timing_begin(omx_ctx* ctx, double flops, omx_ctx::TimedLaunch* timed);
 void omx_timing_end(omx_ctx* ctx, bool launched, const omx_ctx::TimedLaunch& timed);
+
+// Kernel classes that can be timed per launch (benchmark only); the values are those of
+// omx_profile_kernels in the public header.
+enum OmxKernelClass {
+  OMX_K_GEMM = 0, OMX_K_FLASH_FWD = 1, OMX_K_FLASH_BWD = 2, OMX_K_CE = 3, OMX_K_ADAMW = 4, OMX_K_RMS_FWD = 5,
+  OMX_K_RMS_BWD = 6, OMX_K_EMBED_BWD = 7, OMX_K_CLASSES = 8
+};
+// Events for one launch (or one run of launches) of a timed class: the first kernel is launched
+// with start(), the last with stop() (both null while the class is off, which makes
+// omx_launch_timed an ordinary launch); the destructor files the pair with `work`.
+struct OmxKernelTimer {
+  omx_ctx* ctx;
+  omx_ctx::TimedLaunch t{};
+  bool on = false;
+  OmxKernelTimer(omx_ctx* ctx, int cls, double work);
+  ~OmxKernelTimer();
+  OmxKernelTimer(const OmxKernelTimer&) = delete;
+  OmxKernelTimer& operator=(const OmxKernelTimer&) = delete;
+  hipEvent_t start() const { return on ? t.start : nullptr; }
+  hipEvent_t stop() const { return on ? t.stop : nullptr; }
+};
 
 int32_t omx_hip_fail(omx_ctx* ctx, hipError_t err, const char* what);
 // Grows workspace `slot` to at least `bytes` (budget-charged).
@@ -154,7 +177,7 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
 // `scratch` (OMX_COLUMN_SUM_GROUPS * dim floats, may be null) lets a tall `partial` be added in two stages.
 constexpr int OMX_COLUMN_SUM_GROUPS = 32;
 int32_t omx_column_sum(omx_ctx* ctx, const float* partial, float* out, uint64_t blocks, uint64_t dim,
-                       unsigned long long tag, float* scratch = nullptr);
+                       unsigned long long tag, float* scratch = nullptr, hipEvent_t stop = nullptr);
 // RMSNorm with 16-byte accesses for row widths 256..2048 (rmsvec.hip). `add` (forward) and
 // `add_in` / `gx16` (backward) are optional fused operands.
 bool omx_rms_vec_eligible(uint64_t dim, std::initializer_list<const void*> ptrs);

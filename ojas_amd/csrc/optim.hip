@@ -225,6 +225,9 @@ static int32_t adamw_impl(omx_ctx* ctx, const char* op, void* param, const void*
   const bool skip_check = inputs_bounded && moderate;
   dim3 grid(grid_for(n, ctx->cu_count)), block(OPT_THREADS);
   unsigned int* refuse = nullptr;
+  // Parameter, gradient and both moments read, parameter and moments written: 28 bytes per
+  // element, and 2 more with the bf16 copy of the parameter.
+  OmxKernelTimer timer(ctx, OMX_K_ADAMW, (param_bf16 ? 30.0 : 28.0) * static_cast<double>(n));
   if (!skip_check) {
     void* ws = nullptr;
     int32_t rc = omx_workspace(ctx, 256, &ws);
@@ -232,14 +235,14 @@ static int32_t adamw_impl(omx_ctx* ctx, const char* op, void* param, const void*
     refuse = static_cast<unsigned int*>(ws);
     rc = omx_fill_zero(ctx, refuse, 4);
     if (rc != OMX_OK) return rc;
-    hipLaunchKernelGGL(adamw_check_kernel, grid, block, 0, ctx->stream, static_cast<const float*>(param),
-                       static_cast<const float*>(grad), static_cast<const float*>(moment1),
-                       static_cast<const float*>(moment2), n, a, refuse, unbounded, ctx->fault, omx_tag(ctx, F_ADAMW));
+    omx_launch_timed(ctx, adamw_check_kernel, grid, block, 0, timer.start(), nullptr, static_cast<const float*>(param),
+                     static_cast<const float*>(grad), static_cast<const float*>(moment1),
+                     static_cast<const float*>(moment2), n, a, refuse, unbounded, ctx->fault, omx_tag(ctx, F_ADAMW));
     OMX_LAUNCH_CHECK(ctx, "adamw_check_kernel");
   }
-  hipLaunchKernelGGL(adamw_apply_kernel, grid, block, 0, ctx->stream, static_cast<float*>(param),
-                     static_cast<const float*>(grad), static_cast<float*>(moment1), static_cast<float*>(moment2), n, a,
-                     refuse, unbounded, static_cast<unsigned short*>(param_bf16));
+  omx_launch_timed(ctx, adamw_apply_kernel, grid, block, 0, skip_check ? timer.start() : nullptr, timer.stop(),
+                   static_cast<float*>(param), static_cast<const float*>(grad), static_cast<float*>(moment1),
+                   static_cast<float*>(moment2), n, a, refuse, unbounded, static_cast<unsigned short*>(param_bf16));
   OMX_LAUNCH_CHECK(ctx, "adamw_apply_kernel");
   return OMX_OK;
 }

@@ -184,10 +184,14 @@ int32_t omx_rms_forward_vec(omx_ctx* ctx, const void* x, int32_t x_dtype, const 
   dim3 grid(static_cast<unsigned>((rows + 3) / 4)), block(RV_THREADS);
   const int nch = static_cast<int>((dim + 255) / 256);
   typedef unsigned short h16;
-#define RV_FWD(TX, TA, TY, N)                                                                                   \
-  hipLaunchKernelGGL((rms_fwd_vec_kernel<TX, TA, TY, N>), grid, block, 0, ctx->stream, static_cast<const TX*>(x), \
-                     static_cast<const TA*>(add), w, sum_out, static_cast<TY*>(y), static_cast<size_t>(rows),   \
-                     static_cast<int>(dim), eps, ctx->fault, tag)
+  // Bytes: the row read (and the row added to it), the sum written when there is one, the normed row written.
+  const auto width = [](int32_t dtype) { return dtype == OMX_BF16 ? 2.0 : 4.0; };
+  OmxKernelTimer timer(ctx, OMX_K_RMS_FWD, static_cast<double>(rows) * static_cast<double>(dim) *
+                                               (width(x_dtype) + (add ? width(add_dtype) + 4.0 : 0.0) + width(y_dtype)));
+#define RV_FWD(TX, TA, TY, N)                                                                                      \
+  omx_launch_timed(ctx, rms_fwd_vec_kernel<TX, TA, TY, N>, grid, block, 0, timer.start(), timer.stop(),            \
+                   static_cast<const TX*>(x), static_cast<const TA*>(add), w, sum_out, static_cast<TY*>(y),        \
+                   static_cast<size_t>(rows), static_cast<int>(dim), eps, ctx->fault, tag)
 #define RV_FWD_N(TX, TA, TY)      \
   switch (nch) {                  \
     case 1: RV_FWD(TX, TA, TY, 1); break; \
@@ -231,10 +235,17 @@ int32_t omx_rms_backward_vec(omx_ctx* ctx, const void* x, int32_t x_dtype, const
   const size_t smem = 4 * dim * sizeof(float);
   const int nch = static_cast<int>((dim + 255) / 256);
   typedef unsigned short h16;
-#define RV_BWD(TX, TG, TO, N)                                                                                       \
-  hipLaunchKernelGGL((rms_bwd_vec_kernel<TX, TG, TO, N>), grid, block, smem, ctx->stream, static_cast<const TX*>(x), \
-                     w, static_cast<const TG*>(gy), add_in, static_cast<TO*>(gx), static_cast<h16*>(gx16), partial, \
-                     static_cast<size_t>(rows), static_cast<int>(dim), eps, rows_per_block, ctx->fault, tag)
+  // Bytes: the row and its gradient read (and the gradient added in), the input gradient written
+  // (and its bf16 copy); the weight gradient's partial sums are the kernels' own traffic.
+  const auto width = [](int32_t dtype) { return dtype == OMX_BF16 ? 2.0 : 4.0; };
+  OmxKernelTimer timer(ctx, OMX_K_RMS_BWD,
+                       static_cast<double>(rows) * static_cast<double>(dim) *
+                           (width(x_dtype) + width(gy_dtype) + (add_in ? 4.0 : 0.0) + width(gx_dtype) + (gx16 ? 2.0 : 0.0)));
+#define RV_BWD(TX, TG, TO, N)                                                                                        \
+  omx_launch_timed(ctx, rms_bwd_vec_kernel<TX, TG, TO, N>, grid, block, smem, timer.start(), nullptr,                \
+                   static_cast<const TX*>(x), w, static_cast<const TG*>(gy), add_in, static_cast<TO*>(gx),           \
+                   static_cast<h16*>(gx16), partial, static_cast<size_t>(rows), static_cast<int>(dim), eps,          \
+                   rows_per_block, ctx->fault, tag)
 #define RV_BWD_N(TX, TG, TO)      \
   switch (nch) {                  \
     case 1: RV_BWD(TX, TG, TO, 1); break; \
@@ -260,7 +271,7 @@ int32_t omx_rms_backward_vec(omx_ctx* ctx, const void* x, int32_t x_dtype, const
 #undef RV_BWD_N
 #undef RV_BWD
   OMX_LAUNCH_CHECK(ctx, "rms_bwd_vec_kernel");
-  return omx_column_sum(ctx, partial, gw, blocks, dim, tag, scratch);
+  return omx_column_sum(ctx, partial, gw, blocks, dim, tag, scratch, timer.stop());
 }
 
 extern "C" {

@@ -552,7 +552,7 @@ bool finite_host(float v) { return v == v && v != INFINITY && v != -INFINITY; }
 }  // namespace
 
 int32_t omx_column_sum(omx_ctx* ctx, const float* partial, float* out, uint64_t blocks, uint64_t dim,
-                       unsigned long long tag, float* scratch) {
+                       unsigned long long tag, float* scratch, hipEvent_t stop) {
   const unsigned col_blocks = static_cast<unsigned>((dim + 63) / 64);
   if (scratch && blocks > 4 * OMX_COLUMN_SUM_GROUPS) {
     // Stage 1: group g adds its contiguous share of the rows into scratch[g]; stage 2 adds the groups.
@@ -563,8 +563,8 @@ int32_t omx_column_sum(omx_ctx* ctx, const float* partial, float* out, uint64_t 
     partial = scratch;
     blocks = OMX_COLUMN_SUM_GROUPS;
   }
-  hipLaunchKernelGGL(column_sum_kernel, dim3(col_blocks), dim3(256), 0, ctx->stream, partial, out,
-                     static_cast<int>(blocks), static_cast<int>(dim), ctx->fault, tag);
+  omx_launch_timed(ctx, column_sum_kernel, dim3(col_blocks), dim3(256), 0, nullptr, stop, partial, out,
+                   static_cast<int>(blocks), static_cast<int>(dim), ctx->fault, tag);
   OMX_LAUNCH_CHECK(ctx, "column_sum_kernel");
   return OMX_OK;
 }
@@ -684,7 +684,12 @@ int32_t omx_embedding_backward(omx_ctx* ctx, const void* ids, const void* grad, 
   if (rc != OMX_OK) return rc;
   const unsigned int* idp = static_cast<const unsigned int*>(ids);
   dim3 tgrid(static_cast<unsigned>((tokens + 255) / 256));
-  hipLaunchKernelGGL(count_ids_kernel, tgrid, dim3(256), 0, ctx->stream, idp, counts, tokens, vocab, ctx->fault, tag);
+  // Bytes: every gradient row read once, every table row written once (rows no token names get zeros).
+  OmxKernelTimer timer(ctx, OMX_K_EMBED_BWD,
+                       static_cast<double>(dim) * (static_cast<double>(tokens) * (grad_dtype == OMX_BF16 ? 2.0 : 4.0) +
+                                                   static_cast<double>(vocab) * 4.0));
+  omx_launch_timed(ctx, count_ids_kernel, tgrid, dim3(256), 0, timer.start(), nullptr, idp, counts, tokens, vocab,
+                   ctx->fault, tag);
   OMX_LAUNCH_CHECK(ctx, "count_ids_kernel");
   hipLaunchKernelGGL(scan_counts_kernel, dim3(1), dim3(1024), 0, ctx->stream, counts, offsets, cursor, vocab);
   OMX_LAUNCH_CHECK(ctx, "scan_counts_kernel");
@@ -698,13 +703,13 @@ int32_t omx_embedding_backward(omx_ctx* ctx, const void* ids, const void* grad, 
                      long_count, long_rows, tokens);
   OMX_LAUNCH_CHECK(ctx, "sort_long_segments_kernel");
   if (grad_dtype == OMX_F32)
-    hipLaunchKernelGGL((embedding_bwd_kernel<float>), vgrid, dim3(ROW_THREADS), 0, ctx->stream, offsets, sorted,
-                       static_cast<const float*>(grad), static_cast<float*>(table_grad), vocab, static_cast<int>(dim),
-                       ctx->fault, tag);
+    omx_launch_timed(ctx, embedding_bwd_kernel<float>, vgrid, dim3(ROW_THREADS), 0, nullptr, timer.stop(), offsets,
+                     sorted, static_cast<const float*>(grad), static_cast<float*>(table_grad), vocab,
+                     static_cast<int>(dim), ctx->fault, tag);
   else
-    hipLaunchKernelGGL((embedding_bwd_kernel<unsigned short>), vgrid, dim3(ROW_THREADS), 0, ctx->stream, offsets,
-                       sorted, static_cast<const unsigned short*>(grad), static_cast<float*>(table_grad), vocab,
-                       static_cast<int>(dim), ctx->fault, tag);
+    omx_launch_timed(ctx, embedding_bwd_kernel<unsigned short>, vgrid, dim3(ROW_THREADS), 0, nullptr, timer.stop(),
+                     offsets, sorted, static_cast<const unsigned short*>(grad), static_cast<float*>(table_grad), vocab,
+                     static_cast<int>(dim), ctx->fault, tag);
   OMX_LAUNCH_CHECK(ctx, "embedding_bwd_kernel");
   return OMX_OK;
 }
