@@ -357,13 +357,149 @@ def lora_step(args) -> int:
     return 0
 
 
+def nanolab_cpu_baseline(spec, batch, seq, threads: int):
+    """The oracle's nanolab step on a bounded sample: one and two blocks on one short sequence give a
+    block's time and the rest (table, final norm, head); clip + Muon-NS5 (f32 iteration) on one
+    block's matrices and AdamW on its vectors and on the table give the optimizer's. Scaled to the
+    model's blocks and the step's tokens. All cores and one thread, three repeats each."""
+    sys.path.insert(0, str(ROOT / "tests"))
+    import oracle_api as orc
+    from ojas_amd.nanolab import NanolabSpec
+
+    tokens = batch * seq
+    rng = np.random.default_rng(0)
+
+    def model(layers, sample_seq):
+        sp = NanolabSpec(**{**spec.__dict__, "n_layer": layers})
+        cfg = orc.NanolabConfig(layers=layers, n_embd=sp.n_embd, n_head=sp.n_head, n_kv_head=sp.n_kv_head,
+                                head_dim=sp.head_dim, hidden=sp.hidden, vocab=sp.vocab, batch=1, seq=sample_seq, window=0,
+                                rms_eps=sp.rms_eps, rope_base=sp.rope_base)
+        shapes = sp.param_shapes()
+        params = [np.ones(shapes[n], np.float32).reshape(-1) if len(shapes[n]) == 1
+                  else rng.normal(0, 0.02, shapes[n]).astype(np.float32).reshape(-1) for n in sp.param_names()]
+        ids = rng.integers(0, sp.vocab, (1, sample_seq)).astype(np.uint32)
+        return sp, cfg, params, ids
+
+    def measure(n_threads, sample_seq):
+        orc.set_threads(n_threads)
+        one, two = model(1, sample_seq), model(2, sample_seq)
+        shapes = one[0].param_shapes()
+        names = one[0].param_names()
+
+        def once():
+            t = []
+            for sp, cfg, params, ids in (one, two):
+                t0 = time.perf_counter()
+                _, _, grads = orc.nanolab_loss_and_grads(cfg, params, ids, ids)
+                t.append(time.perf_counter() - t0)
+            block = max(t[1] - t[0], 1e-9)
+            rest = max(t[0] - block, 0.0)
+            # optimizer on the one-block model: the table and final norm once, the block's tensors per block
+            t_table, t_block = 0.0, 0.0
+            for n, p in zip(names, one[2]):
+                g = np.full_like(p, 1e-3)
+                t0 = time.perf_counter()
+                if len(shapes[n]) == 2 and n != "tok_emb.weight":
+                    orc.muon_ns5_step(p.reshape(shapes[n]).copy(), g.reshape(shapes[n]), np.zeros(shapes[n], np.float32),
+                                      lr=0.025, momentum=0.99, weight_decay=0.1, nesterov=True, bf16=False)
+                else:
+                    orc.adamw_step(p.copy(), g, np.zeros_like(p), np.zeros_like(p), 0, 6e-4, 0.9, 0.95, 1e-8, 0.0, exact=True)
+                dt = time.perf_counter() - t0
+                if n.startswith("blocks."):
+                    t_block += dt
+                else:
+                    t_table += dt
+            return tokens * (rest + spec.n_layer * block) / sample_seq + t_table + spec.n_layer * t_block
+
+        return repeat_timed(once)
+
+    all_runs = measure(threads, 128)
+    one_runs = measure(1, 32)
+    return {"value": tokens / all_runs[1], "unit": "tokens/s", "cores": threads, "kind": "port",
+            "cpu_model": cpu_model(), "repeats": 3, "step_seconds_min": all_runs[0], "step_seconds_median": all_runs[1],
+            "single_thread": {"value": tokens / one_runs[1], "cores": 1, "step_seconds_min": one_runs[0],
+                              "step_seconds_median": one_runs[1], "sample": "as below on 1x32 tokens"},
+            "sample": f"same model in f32 Exact arithmetic: one and two blocks on 1x128 tokens (block and rest), Muon-NS5 "
+                      f"and AdamW on one block's parameters and the table, scaled to {spec.n_layer} blocks and {tokens} "
+                      f"tokens. Attention grows with the sequence: at this sample length it is a smaller share than at "
+                      f"{seq}, so the estimate favours the CPU by up to its 8 % of the step's work. C++ restatement of "
+                      f"ojas-cpu, not the Rust binary"}
+
+
+def nanolab_step(args) -> int:
+    """The reference's own model at its 124M size (ModelSpec::nanolab_124m, ojas-model/src/spec.rs:74-91):
+    one Trainer::run step (Muon-NS5 on the matrices, AdamW on the table and the vectors) of one
+    16 x 1024 micro-batch through the C++ step driver, bf16 storage."""
+    from ojas_amd.backend import MiBackend
+    from ojas_amd.nanolab import NativeNanolabTrainer, nanolab_step_flops, spec_nanolab_124m
+
+    spec = spec_nanolab_124m()
+    batch, seq = 16, 1024
+    be = MiBackend(0)
+    tr = NativeNanolabTrainer(be, spec, batch, seq, bf16=True, ns5_bf16=True)
+    tr.init(1234)
+    rng = np.random.default_rng(42)
+    window = rng.integers(0, spec.vocab, (batch, seq + 1)).astype(np.uint32)
+    tr._micro(window[:, :-1], window[:, 1:], 1.0, 1.0, True)  # uploads the batch; it stays resident
+    losses = [tr.run_resident(1.0).loss for _ in range(args.warmup)]
+    be.sync()
+    lib = be._lib
+    timed_every = 4
+    step_ms = []
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        lib.omx_profile_kernels(be._ctx, C.c_uint32(ALL_CLASSES_MASK if i % timed_every == 0 else 0))
+        s0 = time.perf_counter()
+        losses.append(tr.run_resident(1.0).loss)  # ends with the loss readback: the step is complete
+        step_ms.append((time.perf_counter() - s0) * 1e3)
+    be.sync()
+    dt = time.perf_counter() - t0
+    timed_steps = len(range(0, args.steps, timed_every))
+    launches, gemm_ms, gemm_flops = C.c_uint64(), C.c_double(), C.c_double()
+    lib.omx_profile_gemm_report(be._ctx, C.byref(launches), C.byref(gemm_ms), C.byref(gemm_flops))
+    per_kernel = kernel_rooflines(lib, be._ctx, timed_steps)
+    lib.omx_profile_kernels(be._ctx, C.c_uint32(0))
+    tokens = batch * seq
+    ms_per_step = dt / args.steps * 1e3
+    flops = nanolab_step_flops(spec, batch, seq)
+    achieved = gemm_flops.value / (gemm_ms.value * 1e-3) / 1e12 if gemm_ms.value > 0 else 0.0
+    out = {
+        "metric": "train tokens/s on 1 MI355X (nanolab-124M bf16 step: Muon-NS5 + AdamW, the reference's own model)",
+        "value": tokens * args.steps / dt, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "ms_per_step_min": float(np.min(step_ms)),
+        "ms_per_step_median": float(np.median(step_ms)), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "nanolab-124M training step (ModelSpec::nanolab_124m): L12 d768 H12x64 (12 KV heads) SwiGLU "
+                               "2048 vocab 50304 ctx 1024 batch 16, QK-norm, RoPE 1e4, per-head sigmoid gate, value "
+                               "residual, tied head; bf16 activations and operand copies, f32 master weights; Muon-NS5 "
+                               "(bf16 iteration, lr 0.025, momentum 0.99, wd 0.1) on the matrices, AdamW lr 6e-4 on the "
+                               "table and the vectors, clip 1.0; one micro-batch per step",
+                   "tokens_per_step": tokens, "params": int(sum(tr.lens))},
+        "step_tflops": flops / (ms_per_step * 1e-3) / 1e12,
+        "pct_bf16_mfma_peak": 100.0 * flops / (ms_per_step * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS,
+        "loss_first": losses[0], "loss_last": losses[-1],
+        "roofline": {"bound": "mfma", "kernel": "gemm_dma_kernel / gemm_kernel (bf16 MFMA GEMM, all operand layouts)",
+                     "achieved": achieved, "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / BF16_MFMA_PEAK_TFLOPS, "traffic": None, "launches": int(launches.value),
+                     "avg_launch_us": gemm_ms.value * 1e3 / max(1, launches.value), "timed_steps": timed_steps,
+                     "gemm_ms_per_step": gemm_ms.value / max(1, timed_steps)},
+        "roofline_per_kernel": per_kernel,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = nanolab_cpu_baseline(spec, batch, seq, min(16, os.cpu_count() or 1))
+    tr.close()
+    be.close()
+    print(json.dumps(out))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--config", default="gpt124m", choices=["gpt124m", "tiny", "lora1b"])
+    ap.add_argument("--config", default="gpt124m", choices=["gpt124m", "tiny", "lora1b", "nanolab124m"])
     ap.add_argument("--optimizer", default="adamw", choices=["adamw", "muon"],
                     help="adamw: BASELINE configs[2], the headline (default); muon: configs[3], Muon-NS5 (bf16 "
                          "iteration, lr 0.02, momentum 0.95) on the hidden matrices and AdamW on tables and norms")
@@ -377,6 +513,8 @@ def main() -> int:
         return kv_decode(args)
     if args.config == "lora1b":
         return lora_step(args)
+    if args.config == "nanolab124m":
+        return nanolab_step(args)
 
     from ojas_amd.backend import AdamWConfig, MiBackend, MuonNs5Config
     from ojas_amd.trainer import GptTrainer, config_gpt124m_bf16, config_tiny_f32, step_flops, synthetic_batch

@@ -519,8 +519,10 @@ __global__ __launch_bounds__(FT, 2) void flash_bwd_dkv_kernel(
 }
 
 // ------------------------------------------------------------------ backward: the mean key row
-// key_mean[b, kv head, :] = the mean over time of that head's key rows, in f32. One workgroup per
-// (batch, kv head); a lane reads 8 values of a row, 256 / (D / 8) rows go round at once.
+// key_mean[b, kv head, :] = the mean of up to 64 of that head's key rows, evenly spaced in time, in
+// f32. The dQ pass needs a vector close to what the key rows share, not the exact mean (what it
+// does with it is exact for any vector), so a sample is enough. One workgroup per (batch, kv head);
+// a lane reads 8 values of a row, 256 / (D / 8) rows go round at once.
 template <int D>
 __global__ __launch_bounds__(256) void flash_key_mean_kernel(const unsigned short* __restrict__ k,
                                                              float* __restrict__ key_mean, FlashShape s) {
@@ -529,14 +531,16 @@ __global__ __launch_bounds__(256) void flash_key_mean_kernel(const unsigned shor
   const int b = blockIdx.x / s.kv_heads, h = blockIdx.x % s.kv_heads;
   const unsigned short* kp = k + b * s.kv.bs + h * s.kv.hs;
   const int col = (threadIdx.x % LPR) * 8, first = threadIdx.x / LPR;
+  const int samples = min(s.time, 64);
   float sum[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  for (int row = first; row < s.time; row += ROWS) {
-    const u32x4 w = *reinterpret_cast<const u32x4*>(kp + static_cast<long>(row) * s.kv.rs + col);
+  for (int i = first; i < samples; i += ROWS) {
+    const long row = static_cast<long>(i) * s.time / samples;
+    const u32x4 w = *reinterpret_cast<const u32x4*>(kp + row * s.kv.rs + col);
     const unsigned int ww[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      sum[2 * i] += __uint_as_float(ww[i] << 16);
-      sum[2 * i + 1] += __uint_as_float(ww[i] & 0xffff0000u);
+    for (int j = 0; j < 4; ++j) {
+      sum[2 * j] += __uint_as_float(ww[j] << 16);
+      sum[2 * j + 1] += __uint_as_float(ww[j] & 0xffff0000u);
     }
   }
 #pragma unroll
@@ -545,7 +549,7 @@ __global__ __launch_bounds__(256) void flash_key_mean_kernel(const unsigned shor
   if (threadIdx.x < D) {
     float total = 0.0f;
     for (int r = 0; r < ROWS; ++r) total += part[r][threadIdx.x];
-    key_mean[static_cast<long>(blockIdx.x) * D + threadIdx.x] = total / static_cast<float>(s.time);
+    key_mean[static_cast<long>(blockIdx.x) * D + threadIdx.x] = total / static_cast<float>(samples);
   }
 }
 

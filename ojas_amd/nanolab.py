@@ -8,6 +8,7 @@ here. Parameters come in the order of ojas-model/src/names.rs:188-300.
 """
 from __future__ import annotations
 
+import ctypes as C
 import json
 import math
 from contextlib import nullcontext
@@ -281,6 +282,146 @@ class NanolabTrainer:
 
     def download_params(self) -> Dict[str, np.ndarray]:
         return {n: self.be.download(t) for n, t in self.params.items()}
+
+
+class OnanoConfig(C.Structure):
+    """onano_config of include/ojas_nanolab.h."""
+    _fields_ = [(n, C.c_uint32) for n in ("layers", "n_embd", "heads", "kv_heads", "head_dim", "hidden", "vocab", "batch",
+                                          "seq", "window", "bf16")] + [("rms_eps", C.c_float), ("rope_base", C.c_double)]
+
+
+NATIVE_LIB_PATH = Path(__file__).resolve().parent / "libojas_nanolab.so"
+
+
+class NativeNanolabTrainer:
+    """`Trainer::run` (ojas-model/src/trainer.rs:754-857) through the C++ step driver of
+    include/ojas_nanolab.h: the same step as `NanolabTrainer`, with the graph's ~60 calls per block
+    made from C++ over buffers allocated once, and bf16 storage of activations and operand copies
+    when `bf16` is set. The schedule multiplier is the caller's."""
+
+    def __init__(self, be: MiBackend, spec: NanolabSpec, batch: int, seq: int, host_params=None, adam_lr: float = 6e-4,
+                 matrix_lr: float = 0.025, grad_clip: float = 1.0, ns5_bf16: bool = False, bf16: bool = False):
+        if not NATIVE_LIB_PATH.exists():
+            raise OjasError(10, f"{NATIVE_LIB_PATH} is not built; run __graft_entry__.build()")
+        self._lib = C.CDLL(str(NATIVE_LIB_PATH))
+        for name in ("onano_param_count", "onano_param_len", "onano_steps", "onano_device_bytes"):
+            getattr(self._lib, name).restype = C.c_uint64
+        self.be, self.spec, self.batch, self.seq = be, spec, batch, seq
+        self.adam_lr, self.matrix_lr, self.grad_clip, self.ns5_bf16 = adam_lr, matrix_lr, grad_clip, ns5_bf16
+        self.names = spec.param_names()
+        cfg = OnanoConfig(spec.n_layer, spec.n_embd, spec.n_head, spec.n_kv_head, spec.head_dim, spec.hidden, spec.vocab,
+                          batch, seq, spec.window or 0, int(bf16), spec.rms_eps, spec.rope_base)
+        h = C.c_void_p()
+        rc = self._lib.onano_create(be._ctx, C.byref(cfg), C.byref(h))
+        self._h = h if rc == 0 else None
+        be._check(rc)
+        shapes = spec.param_shapes()
+        lens = [int(self._lib.onano_param_len(self._h, C.c_uint64(i))) for i in range(len(self.names))]
+        assert int(self._lib.onano_param_count(self._h)) == len(self.names)
+        assert lens == [int(np.prod(shapes[n])) for n in self.names]
+        self.lens = lens
+        if host_params is not None:
+            self.set_params(host_params)
+
+    def close(self):
+        if self._h:
+            self._lib.onano_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        self.close()
+
+    @property
+    def step(self) -> int:
+        return int(self._lib.onano_steps(self._h))
+
+    def init(self, seed: int):
+        self.be._check(self._lib.onano_init(self._h, C.c_uint64(seed)))
+
+    def set_params(self, host_params: Dict[str, np.ndarray]):
+        for i, n in enumerate(self.names):
+            a = np.ascontiguousarray(host_params[n], np.float32).reshape(-1)
+            self.be._check(self._lib.onano_set_param(self._h, C.c_uint64(i), a.ctypes.data_as(C.c_void_p)))
+
+    def _get(self, fn, *extra) -> Dict[str, np.ndarray]:
+        out = {}
+        for i, (n, length) in enumerate(zip(self.names, self.lens)):
+            a = np.empty(length, np.float32)
+            self.be._check(fn(self._h, C.c_uint64(i), *extra, a.ctypes.data_as(C.c_void_p)))
+            out[n] = a
+        return out
+
+    def download_params(self) -> Dict[str, np.ndarray]:
+        shapes = self.spec.param_shapes()
+        return {n: a.reshape(shapes[n]) for n, a in self._get(self._lib.onano_get_param).items()}
+
+    def grads(self) -> Dict[str, np.ndarray]:
+        return self._get(self._lib.onano_get_grad)
+
+    def state(self, slot: int) -> Dict[str, np.ndarray]:
+        return self._get(self._lib.onano_get_state, C.c_uint32(slot))
+
+    def loss_and_grads(self, ids, targets, loss_seed: float = 1.0):
+        """One micro-batch on its own: (loss, {name: gradient})."""
+        self._micro(ids, targets, loss_seed, 1.0, True)
+        loss = C.c_float()
+        self.be._check(self._lib.onano_loss(self._h, C.byref(loss)))
+        return float(loss.value), self.grads()
+
+    def _micro(self, ids, targets, seed, scale, first):
+        ids = np.ascontiguousarray(ids, np.uint32).reshape(-1)
+        targets = np.ascontiguousarray(targets, np.uint32).reshape(-1)
+        if ids.size != self.batch * self.seq or targets.size != ids.size:
+            raise OjasError(1, f"micro-batch: expected {self.batch} x {self.seq} ids and targets")
+        self.be._check(self._lib.onano_micro_batch(self._h, ids.ctypes.data_as(C.c_void_p),
+                                                   targets.ctypes.data_as(C.c_void_p), C.c_float(seed), C.c_float(scale),
+                                                   C.c_int32(1 if first else 0)))
+
+    def run(self, batches: Sequence, lr_multiplier: float) -> StepReport:
+        """`batches`: (ids, targets) u32 host arrays [batch, seq], one per micro-batch; every target counts."""
+        if not batches:
+            raise OjasError(OUT_OF_RANGE, "Trainer::step: 0 micro-batches")
+        weight = float(np.float32(1.0 / len(batches)))  # equal counts: the uniform weights of trainer.rs:1089-1119
+        for k, (ids, targets) in enumerate(batches):
+            self._micro(ids, targets, weight, 1.0, k == 0)
+        return self.apply(lr_multiplier, len(batches))
+
+    def run_resident(self, lr_multiplier: float) -> StepReport:
+        """One step of one micro-batch on the ids and targets uploaded last."""
+        self.be._check(self._lib.onano_micro_batch_resident(self._h, C.c_float(1.0), C.c_float(1.0), C.c_int32(1)))
+        return self.apply(lr_multiplier, 1)
+
+    def apply(self, lr_multiplier: float, micro_batches: int) -> StepReport:
+        muon = MuonNs5Config(self.matrix_lr * lr_multiplier, MUON_MOMENTUM, MUON_WEIGHT_DECAY, 1, int(self.ns5_bf16))
+        adamw = AdamWConfig.nanolab(self.adam_lr * lr_multiplier, ADAM_HYBRID_WEIGHT_DECAY)
+        loss, norm = C.c_float(), C.c_float()
+        self.be._check(self._lib.onano_apply(self._h, C.byref(muon), C.byref(adamw), C.c_float(self.grad_clip),
+                                             C.byref(loss), C.byref(norm)))
+        value = float(loss.value)
+        if not math.isfinite(value):
+            raise OjasError(NON_FINITE, "Trainer::step")
+        return StepReport(loss=value / micro_batches, grad_norm=float(norm.value), lr_multiplier=lr_multiplier,
+                          step=self.step, tokens=micro_batches * self.batch * self.seq)
+
+    def device_bytes(self) -> int:
+        return int(self._lib.onano_device_bytes(self._h))
+
+
+def nanolab_step_flops(spec: NanolabSpec, batch: int, seq: int) -> float:
+    """Algorithmic FLOPs of one step: 6 N P over the weights that take part in products (the
+    projections, the gate, the SwiGLU matrices and the tied head) and causal attention at half the
+    square (forward 2, backward 5 products)."""
+    d, q, kv = spec.n_embd, spec.n_head * spec.head_dim, spec.n_kv_head * spec.head_dim
+    per_block = d * q + 2 * d * kv + q * d + spec.n_head * d + 3 * d * spec.hidden
+    n = batch * seq
+    attention = 7.0 * batch * spec.n_head * seq * seq * spec.head_dim * spec.n_layer
+    return 6.0 * n * (spec.n_layer * per_block + spec.vocab * d) + attention
+
+
+def spec_nanolab_124m() -> NanolabSpec:
+    """`ModelSpec::nanolab_124m` (ojas-model/src/spec.rs:74-91)."""
+    return NanolabSpec(n_layer=12, n_embd=768, n_head=12, n_kv_head=12, head_dim=64, hidden=2048, vocab=50304,
+                       rms_eps=1e-6, rope_base=10000.0, window=None, max_seq=1024)
 
 
 # ---- the checkpoint directory (ojas-model/src/checkpoint.rs:1-60) ----

@@ -9,12 +9,14 @@ import pytest
 
 ROOT = Path(__file__).resolve().parent.parent
 HEADERS = {"ojas_mi355x.h": ROOT / "ojas_amd" / "libojas_mi355x.so", "ojas_gpt.h": ROOT / "ojas_amd" / "libojas_gpt.so",
-           "ojas_data.h": ROOT / "ojas_amd" / "libojas_data.so", "ojas_io.h": ROOT / "ojas_amd" / "libojas_io.so"}
+           "ojas_data.h": ROOT / "ojas_amd" / "libojas_data.so", "ojas_io.h": ROOT / "ojas_amd" / "libojas_io.so",
+           "ojas_lora.h": ROOT / "ojas_amd" / "libojas_lora.so",
+           "ojas_nanolab.h": ROOT / "ojas_amd" / "libojas_nanolab.so"}
 
 
 def declared(header: Path):
     text = re.sub(r"/\*.*?\*/", "", header.read_text(), flags=re.S)
-    return sorted(set(re.findall(r"\b((?:omx|ogpt|odata|oio)_\w+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b((?:omx|ogpt|odata|oio|olora|onano)_\w+)\s*\(", text)))
 
 
 @pytest.mark.parametrize("header", sorted(HEADERS))
