@@ -490,8 +490,10 @@ int32_t launch_rms_bwd(omx_ctx* ctx, const void* x, const float* w, const void* 
   while ((rows + rows_per_block - 1) / rows_per_block > 2048 && rows_per_block < (1 << 20)) rows_per_block *= 2;
   uint64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
   void* partial = nullptr;
-  int32_t rc = omx_workspace(ctx, blocks * dim * sizeof(float), &partial);
+  int32_t rc = omx_workspace(ctx, (blocks + OMX_COLUMN_SUM_GROUPS) * dim * sizeof(float), &partial);
   if (rc != OMX_OK) return rc;
+  // A narrow row leaves the column sum one or two workgroups: it then adds its rows in two stages.
+  float* stage = static_cast<float*>(partial) + blocks * dim;
   dim3 grid(static_cast<unsigned>(blocks)), block(ROW_THREADS);
   size_t smem = 4 * dim * sizeof(float);
   int per = per_for_dim(dim);
@@ -508,7 +510,7 @@ int32_t launch_rms_bwd(omx_ctx* ctx, const void* x, const float* w, const void* 
   }
 #undef RMS_BWD
   OMX_LAUNCH_CHECK(ctx, "rms_bwd_kernel");
-  return omx_column_sum(ctx, static_cast<const float*>(partial), gw, blocks, dim, tag);
+  return omx_column_sum(ctx, static_cast<const float*>(partial), gw, blocks, dim, tag, stage);
 }
 
 int32_t rms_forward_impl(omx_ctx* ctx, const char* op, uint32_t fault_op, const void* x, int32_t x_dtype,
