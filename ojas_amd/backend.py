@@ -18,6 +18,8 @@ from typing import Optional, Sequence, Tuple
 
 import numpy as np
 
+from . import shapes
+
 LIB_PATH = Path(__file__).resolve().parent / "libojas_mi355x.so"
 
 F32, BF16, U32 = 0, 1, 2
@@ -909,3 +911,103 @@ class MiBackend:
             raise OjasError(UNSUPPORTED, name)
 
         return refuse
+
+
+# ---- shape first (docs/shape-contract.md): every op runs its validator before placement, values,
+# budget or launches. The table gives, per method, the validator call on the method's own
+# arguments and how many leading arguments are tensor operands (checked for placement next).
+class _Meta:
+    """Shape and dtype of an operand the method does not take as a tensor (a table given by its
+    vocabulary size)."""
+
+    def __init__(self, shape, dtype):
+        self.shape, self.dtype = tuple(shape), dtype
+
+
+def _elementwise(op, n):
+    return (lambda *a, **_k: shapes.elementwise_dims(op, *a[:n])), n
+
+
+_VALIDATED = {
+    "linear_forward": (lambda x, w, *_a, **_k: shapes.linear_forward_dims(x, w), 2),
+    "linear_backward": (lambda x, w, gy, *_a, **_k: shapes.linear_backward_dims(x, w, gy), 3),
+    "causal_sdpa_forward": (lambda q, k, v, window=None, *_a, **_k: shapes.causal_sdpa_forward_dims(q, k, v, window), 3),
+    "causal_sdpa_backward": (lambda q, k, v, out, lse, gy, window=None, *_a, **_k:
+                             shapes.causal_sdpa_backward_dims(q, k, v, out, lse, gy, window), 6),
+    "rms_norm_forward": (lambda x, w, eps=1e-6, *_a, **_k: shapes.rms_norm_forward_dims(x, w, eps), 2),
+    "rms_norm_backward": (lambda x, w, gy, eps=1e-6, *_a, **_k: shapes.rms_norm_backward_dims(x, w, gy, eps), 3),
+    "rms_qk_norm_forward": (lambda q, k, qw, kw, eps=1e-6, *_a, **_k: shapes.rms_qk_norm_forward_dims(q, k, qw, kw, eps), 4),
+    "rms_qk_norm_backward": (lambda q, k, qw, kw, gq, gk, eps=1e-6, *_a, **_k:
+                             shapes.rms_qk_norm_backward_dims(q, k, qw, kw, gq, gk, eps), 6),
+    "rope_half_split_forward": (lambda x, c, s: shapes.rope_half_split_forward_dims(x, c, s), 3),
+    "rope_half_split_backward": (lambda g, c, s: shapes.rope_half_split_backward_dims(g, c, s), 3),
+    "cross_entropy_mean_forward": (lambda l, t, *_a, **_k: shapes.cross_entropy_mean_forward_dims(l, t), 2),
+    "cross_entropy_mean_backward": (lambda l, t, *_a, **_k: shapes.cross_entropy_mean_backward_dims(l, t), 2),
+    "linear_cross_entropy_mean": (lambda x, w, t, ignore_index=None, chunk=(1024, 8192), *_a, **_k:
+                                  shapes.linear_ce_dims(x, w, t, chunk), 3),
+    "embedding_forward": (lambda table, ids, *_a, **_k: shapes.embedding_forward_dims(table, ids), 2),
+    # The table itself is not an argument here: its vocabulary size stands in for it.
+    "embedding_backward": (lambda ids, grad, vocab: shapes.embedding_backward_dims(
+        _Meta((vocab, grad.shape[-1] if len(grad.shape) else 0), F32), ids, grad), 2),
+    "adamw_step": (lambda p, g, m1, m2, *_a, **_k: shapes.adamw_step_dims(p, g, m1, m2), 4),
+    "muon_ns5_step": (lambda p, g, m, *_a, **_k: shapes.muon_ns5_step_dims(p, g, m), 3),
+    "residual_add_forward": _elementwise("residual_add_forward", 2),
+    "accumulate_grad": _elementwise("accumulate_grad", 2),
+    "scale_grad": (lambda g, *_a, **_k: shapes.scale_grad_dims(g), 1),
+    "gelu_erf_forward": _elementwise("gelu_erf_forward", 1),
+    "gelu_erf_backward": _elementwise("gelu_erf_backward", 2),
+    "gelu_tanh_forward": _elementwise("gelu_tanh_forward", 1),
+    "gelu_tanh_backward": _elementwise("gelu_tanh_backward", 2),
+    "silu_forward": _elementwise("silu_forward", 1),
+    "silu_backward": _elementwise("silu_backward", 2),
+    "mul_forward": _elementwise("mul_forward", 2),
+    "mul_backward": _elementwise("mul_backward", 3),
+    "permute": (lambda x, axes: shapes.permute_dims(x, axes), 1),
+    "per_head_sigmoid_gate_forward": (lambda x, w, b, a, *_a, **_k: shapes.per_head_sigmoid_gate_forward_dims(x, w, b, a), 4),
+    "per_head_sigmoid_gate_forward_saving": (lambda x, w, b, a, *_a, **_k:
+                                             shapes.per_head_sigmoid_gate_forward_dims(x, w, b, a), 4),
+    "per_head_sigmoid_gate_backward": (lambda x, w, b, a, gy, *_a, **_k:
+                                       shapes.per_head_sigmoid_gate_backward_dims(x, w, b, a, gy), 5),
+    "per_head_sigmoid_gate_backward_saved": (lambda x, w, b, a, gy, *_a, **_k:
+                                             shapes.per_head_sigmoid_gate_backward_dims(x, w, b, a, gy), 5),
+    "value_residual_blend_forward": (lambda v, v0, lam: shapes.value_residual_blend_forward_dims(v, v0, lam), 3),
+    "value_residual_blend_backward": (lambda v, v0, lam, gy: shapes.value_residual_blend_backward_dims(v, v0, lam, gy), 4),
+    "cached_attention_forward": (lambda q, kc, vc, kv_len, window=None: shapes.cached_attention_dims(q, kc, vc, kv_len, window), 3),
+    "kv_cache_write": (lambda cache, src, at: shapes.kv_cache_write_dims(cache, src, at), 2),
+    "argmax_rows": (lambda x: shapes.argmax_rows_dims(x), 1),
+    "topk_rows": (lambda x, k: shapes.topk_rows_dims(x, k), 1),
+}
+
+
+def _shape_first(name, method, validator, operands):
+    def checked(self, *args, **kwargs):
+        try:
+            validator(*args, **kwargs)
+        except shapes.ShapeError as e:
+            raise OjasError(e.code, f"{e.op}: {e.detail}") from None
+        for t in args[:operands]:
+            if t is not None and not isinstance(t, DeviceTensor):
+                raise OjasError(PLACEMENT, f"{name}: operand is in host memory")
+        return method(self, *args, **kwargs)
+
+    checked.__name__, checked.__doc__ = name, method.__doc__
+    return checked
+
+
+def _clip_shape_first(method):
+    def checked(self, grads, max_norm):
+        try:
+            shapes.clip_grad_norm_dims(list(grads))
+        except shapes.ShapeError as e:
+            raise OjasError(e.code, f"{e.op}: {e.detail}") from None
+        if any(not isinstance(g, DeviceTensor) for g in grads):
+            raise OjasError(PLACEMENT, "clip_grad_norm: operand is in host memory")
+        return method(self, grads, max_norm)
+
+    checked.__name__, checked.__doc__ = "clip_grad_norm", method.__doc__
+    return checked
+
+
+for _name, (_validator, _operands) in _VALIDATED.items():
+    setattr(MiBackend, _name, _shape_first(_name, getattr(MiBackend, _name), _validator, _operands))
+MiBackend.clip_grad_norm = _clip_shape_first(MiBackend.clip_grad_norm)
