@@ -227,7 +227,7 @@ int32_t omx_linear_backward_input_gelu(omx_ctx* ctx, const void* w, const void* 
  *      token rows are `*_pitch` elements apart (a multiple of 8, at least
  *      heads * head_dim), so q, k and v may be column blocks of one projection
  *      output. gq uses q_pitch, gk / gv use kv_pitch. lse is [batch, heads, time]
- *      f32. bf16 with head_dim 64 only; other shapes return Unsupported and the
+ *      f32. bf16 with head_dim 64 or 128; other shapes return Unsupported and the
  *      caller composes omx_permute_0213 with omx_causal_sdpa_*. ---- */
 int32_t omx_causal_attention_forward(omx_ctx* ctx, const void* q, uint64_t q_pitch, const void* k,
                                      const void* v, uint64_t kv_pitch, int32_t operand_dtype,
