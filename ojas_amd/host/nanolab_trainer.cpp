@@ -74,6 +74,14 @@ struct onano {
   void *gqp = nullptr, *gkp = nullptr, *gvp = nullptr, *gap_p = nullptr;  // permuted gradients (row kernels)
   void *gy16 = nullptr, *ghf = nullptr;
   float *gres = nullptr, *gres1 = nullptr, *gh = nullptr, *g_emb = nullptr;
+  // bf16 tier with more than one block: the seven weight gradients of every block wait until the
+  // backward's end. Each block's product inputs (h, y, h2, m) and output gradients sit at a fixed
+  // stride in stacked buffers, the gradient arena holds the blocks at a fixed stride too, and seven
+  // strided-batch products over the blocks replace 7 x layers split-K products: long reductions
+  // (the step's tokens) with small outputs fill the chip only together.
+  bool deferred_dw = false;
+  void *h_all = nullptr, *y_all = nullptr, *h2_all = nullptr, *m_all = nullptr;
+  void *gyd_all = nullptr, *ggu_all = nullptr, *gyo_all = nullptr, *gq_all = nullptr, *gk_all = nullptr, *gv_all = nullptr;
 
   const void* w(uint64_t i) const {
     return AD == OMX_BF16 ? static_cast<const void*>(static_cast<const uint16_t*>(p16) + slots[i].offset)
@@ -208,21 +216,35 @@ int32_t backward(onano* t, float loss_seed) {
   }
   TRY(omx_rms_norm_backward(ctx, t->x_final, OMX_F32, t->w32(t->nf()), t->ghf, AD, t->gres, OMX_F32, t->g(t->nf()), N, d,
                             eps));
+  const bool defer = t->deferred_dw;  // implies the bf16 tier
+  auto slice = [&](void* all, uint64_t l, uint64_t per_layer) {
+    return static_cast<void*>(static_cast<char*>(all) + l * per_layer * t->asz);
+  };
   const void* gy = nullptr;
-  TRY(to_operand(t, t->gres, t->gy16, N * d, &gy));
+  TRY(to_operand(t, t->gres, defer ? slice(t->gyd_all, c.layers - 1, N * d) : t->gy16, N * d, &gy));
   void* copy16 = AD == OMX_BF16 ? t->gy16 : nullptr;
   bool have_g_v0 = false;
   for (uint32_t l = c.layers; l-- > 0;) {
     onano::Layer& A = t->layers[l];
+    // Where this block's output gradients go: scratch, or the block's slice of the stacked buffers.
+    void* ggu = defer ? slice(t->ggu_all, l, 2 * N * Hd) : t->ggu;
+    void* gq_lin = defer ? slice(t->gq_all, l, N * qd) : t->gq;
+    void* gk_lin = defer ? slice(t->gk_all, l, N * kd) : t->gk;
+    void* g_raw_v_out = defer ? slice(t->gv_all, l, N * kd) : t->g_raw_v;
+    // Where the two norm backwards of this block leave the bf16 copy of the gradient they produce:
+    // the operand of this block's o projection, and of the block below's down projection.
+    void* copy_o = defer ? slice(t->gyo_all, l, N * d) : copy16;
+    void* copy_below = defer && l > 0 ? slice(t->gyd_all, l - 1, N * d) : copy16;
+    // Weight gradients go to the arena now, or wait for the batched products after the loop.
+    auto gw = [&](uint64_t which) { return defer ? nullptr : t->g(t->li(l, which)); };
     // x_next = x1 + down(silu(gate(h2)) * up(h2))
-    TRY(omx_linear_backward(ctx, A.m, t->w(t->li(l, FFN_DOWN)), gy, AD, t->gm, AD, t->g(t->li(l, FFN_DOWN)), OMX_F32, N, Hd,
-                            d));
+    TRY(omx_linear_backward(ctx, A.m, t->w(t->li(l, FFN_DOWN)), gy, AD, t->gm, AD, gw(FFN_DOWN), OMX_F32, N, Hd, d));
     if (t->fused_mlp) {
-      TRY(omx_swiglu_backward(ctx, A.gu, t->gm, t->ggu, AD, N, Hd));
+      TRY(omx_swiglu_backward(ctx, A.gu, t->gm, ggu, AD, N, Hd));
       // One product for both projections: their input gradients add in its f32 accumulators.
-      TRY(omx_linear_backward(ctx, A.h2, t->w(t->li(l, FFN_GATE)), t->ggu, AD, t->t_a, AD, t->g(t->li(l, FFN_GATE)), OMX_F32,
-                              N, d, 2 * Hd));
-      TRY(omx_rms_norm_backward_residual(ctx, A.x1, OMX_F32, t->w32(t->li(l, NORM2)), t->t_a, AD, t->gres, t->gres1, copy16,
+      TRY(omx_linear_backward(ctx, A.h2, t->w(t->li(l, FFN_GATE)), ggu, AD, t->t_a, AD, gw(FFN_GATE), OMX_F32, N, d,
+                              2 * Hd));
+      TRY(omx_rms_norm_backward_residual(ctx, A.x1, OMX_F32, t->w32(t->li(l, NORM2)), t->t_a, AD, t->gres, t->gres1, copy_o,
                                          t->g(t->li(l, NORM2)), N, d, eps));
     } else {
       TRY(omx_mul_backward(ctx, A.g_act, A.up, t->gm, t->g_gact, t->g_up, AD, N * Hd));
@@ -236,9 +258,9 @@ int32_t backward(onano* t, float loss_seed) {
       TRY(omx_rms_norm_backward_residual(ctx, A.x1, OMX_F32, t->w32(t->li(l, NORM2)), t->gh, OMX_F32, t->gres, t->gres1,
                                          copy16, t->g(t->li(l, NORM2)), N, d, eps));
     }
-    gy = AD == OMX_BF16 ? static_cast<const void*>(copy16) : static_cast<const void*>(t->gres1);
+    gy = AD == OMX_BF16 ? static_cast<const void*>(t->fused_mlp ? copy_o : copy16) : static_cast<const void*>(t->gres1);
     // x1 = x + o(gate(h) * attention)
-    TRY(omx_linear_backward(ctx, A.y, t->w(t->li(l, WO)), gy, AD, t->gyy, AD, t->g(t->li(l, WO)), OMX_F32, N, qd, d));
+    TRY(omx_linear_backward(ctx, A.y, t->w(t->li(l, WO)), gy, AD, t->gyy, AD, gw(WO), OMX_F32, N, qd, d));
     TRY(omx_per_head_sigmoid_gate_backward(ctx, A.h, t->w(t->li(l, GATE_W)), AD, t->w32(t->li(l, GATE_B)), A.ap, AD, t->gyy,
                                            AD, A.gates, t->gh, OMX_F32, t->g(t->li(l, GATE_W)), t->g(t->li(l, GATE_B)),
                                            t->gap, AD, N, d, H, D));
@@ -257,35 +279,47 @@ int32_t backward(onano* t, float loss_seed) {
     const void* g_raw_v = t->gv;
     if (l == 0) {
       if (have_g_v0) {
-        TRY(omx_residual_add(ctx, t->g_v0, AD, t->gv, AD, t->g_raw_v, AD, N * kd));
-        g_raw_v = t->g_raw_v;
+        TRY(omx_residual_add(ctx, t->g_v0, AD, t->gv, AD, g_raw_v_out, AD, N * kd));
+        g_raw_v = g_raw_v_out;
       }
       TRY(omx_fill_zero(ctx, t->g(t->li(0, LAMBDA)), 4));
     } else {
       void* to_v0 = have_g_v0 ? t->part_v0 : t->g_v0;
-      TRY(omx_value_residual_blend_backward(ctx, A.raw_v, t->layers[0].raw_v, t->w32(t->li(l, LAMBDA)), t->gv, t->g_raw_v,
+      TRY(omx_value_residual_blend_backward(ctx, A.raw_v, t->layers[0].raw_v, t->w32(t->li(l, LAMBDA)), t->gv, g_raw_v_out,
                                             to_v0, AD, t->g(t->li(l, LAMBDA)), N * kd));
       if (have_g_v0) TRY(omx_residual_add(ctx, t->g_v0, AD, t->part_v0, AD, t->g_v0, AD, N * kd));
       have_g_v0 = true;
-      g_raw_v = t->g_raw_v;
+      g_raw_v = g_raw_v_out;
     }
     TRY(omx_rope_half_split_backward(ctx, t->gk, t->cos_t, t->sin_t, t->t_k, AD, N * KV, D, T, KV));
     TRY(omx_rope_half_split_backward(ctx, t->gq, t->cos_t, t->sin_t, t->t_q, AD, N * H, D, T, H));
     TRY(omx_rms_qk_norm_backward(ctx, A.q_lin, A.k_lin, AD, t->w32(t->li(l, QNORM)), t->w32(t->li(l, KNORM)), t->t_q, t->t_k,
-                                 AD, t->gq, t->gk, AD, t->g(t->li(l, QNORM)), t->g(t->li(l, KNORM)), N * H, N * KV, D, eps));
+                                 AD, gq_lin, gk_lin, AD, t->g(t->li(l, QNORM)), t->g(t->li(l, KNORM)), N * H, N * KV, D, eps));
     // h feeds the gate, v, k and q; their gradients arrive in that order (the later consumer first).
     struct Proj {
       uint64_t which, out;
       const void* gy;
-    } projections[3] = {{WV, kd, g_raw_v}, {WK, kd, t->gk}, {WQ, qd, t->gq}};
+    } projections[3] = {{WV, kd, g_raw_v}, {WK, kd, gk_lin}, {WQ, qd, gq_lin}};
     for (const Proj& p : projections) {
-      TRY(omx_linear_backward(ctx, A.h, t->w(t->li(l, p.which)), p.gy, AD, t->t_a, AD, t->g(t->li(l, p.which)), OMX_F32, N,
-                              d, p.out));
+      TRY(omx_linear_backward(ctx, A.h, t->w(t->li(l, p.which)), p.gy, AD, t->t_a, AD, gw(p.which), OMX_F32, N, d, p.out));
       TRY(omx_residual_add(ctx, t->gh, OMX_F32, t->t_a, AD, t->gh, OMX_F32, N * d));
     }
-    TRY(omx_rms_norm_backward_residual(ctx, A.x, OMX_F32, t->w32(t->li(l, NORM1)), t->gh, OMX_F32, t->gres1, t->gres, copy16,
-                                       t->g(t->li(l, NORM1)), N, d, eps));
-    gy = AD == OMX_BF16 ? static_cast<const void*>(copy16) : static_cast<const void*>(t->gres);
+    TRY(omx_rms_norm_backward_residual(ctx, A.x, OMX_F32, t->w32(t->li(l, NORM1)), t->gh, OMX_F32, t->gres1, t->gres,
+                                       copy_below, t->g(t->li(l, NORM1)), N, d, eps));
+    gy = AD == OMX_BF16 ? static_cast<const void*>(copy_below) : static_cast<const void*>(t->gres);
+  }
+  if (defer) {
+    // gw[l](o, j) = sum_r gy[l][r, o] * x[l][r, j] for every block l, one launch per weight.
+    const uint64_t layers = c.layers, per_layer = t->slots[t->li(1, NORM1)].offset - t->slots[t->li(0, NORM1)].offset;
+    struct Deferred {
+      const void *gy, *x;
+      uint64_t which, out, in;
+    } products[6] = {{t->gyd_all, t->m_all, FFN_DOWN, d, Hd}, {t->ggu_all, t->h2_all, FFN_GATE, 2 * Hd, d},
+                     {t->gyo_all, t->y_all, WO, d, qd},       {t->gv_all, t->h_all, WV, kd, d},
+                     {t->gk_all, t->h_all, WK, kd, d},        {t->gq_all, t->h_all, WQ, qd, d}};
+    for (const Deferred& p : products)
+      TRY(omx_gemm_strided_batch(ctx, p.gy, 1, p.out, p.x, p.in, 1, AD, t->g(t->li(0, p.which)), OMX_F32, p.out, N, p.in, 0,
+                                 layers, N * p.out, N * p.in, per_layer));
   }
   // The tied table: the head's gradient first, then the embedding's rows.
   TRY(omx_embedding_backward(ctx, t->ids, t->gres, OMX_F32, t->g_emb, N, c.vocab, d));
@@ -328,6 +362,7 @@ int32_t onano_create(omx_ctx* ctx, const onano_config* config, onano** out) {
   t->N = static_cast<uint64_t>(c.batch) * c.seq;
   t->flash = c.bf16 && (c.head_dim == 64 || c.head_dim == 128);
   t->fused_mlp = c.bf16 && c.hidden % 8 == 0;
+  t->deferred_dw = t->fused_mlp && c.layers > 1;
   const uint64_t N = t->N, d = c.n_embd, H = c.heads, KV = c.kv_heads, D = c.head_dim, Hd = c.hidden;
   const uint64_t qd = H * D, kd = KV * D;
   uint64_t at = 0;
@@ -400,13 +435,38 @@ int32_t onano_create(omx_ctx* ctx, const onano_config* config, onano** out) {
     CREATE_TRY(omx_upload(ctx, t->sin_t, 0, sn.data(), sn.size() * 4));
   }
   t->layers.resize(c.layers);
+  const uint64_t L = c.layers;
+  if (t->deferred_dw) {
+    CREATE_TRY(alloc_act(t, L * N * d, &t->h_all));
+    CREATE_TRY(alloc_act(t, L * N * qd, &t->y_all));
+    CREATE_TRY(alloc_act(t, L * N * d, &t->h2_all));
+    CREATE_TRY(alloc_act(t, L * N * Hd, &t->m_all));
+    CREATE_TRY(alloc_act(t, L * N * d, &t->gyd_all));
+    CREATE_TRY(alloc_act(t, L * 2 * N * Hd, &t->ggu_all));
+    CREATE_TRY(alloc_act(t, L * N * d, &t->gyo_all));
+    CREATE_TRY(alloc_act(t, L * N * qd, &t->gq_all));
+    CREATE_TRY(alloc_act(t, L * N * kd, &t->gk_all));
+    CREATE_TRY(alloc_act(t, L * N * kd, &t->gv_all));
+  }
   uint32_t index = 0;
   for (auto& A : t->layers) {
+    const uint64_t l = index;
     const bool first = index++ == 0;
     std::memset(&A, 0, sizeof(A));
+    auto stacked = [&](void* all, uint64_t per_layer) { return static_cast<void*>(static_cast<char*>(all) + l * per_layer * t->asz); };
     CREATE_TRY(alloc_t(t, N * d, &A.x));
     CREATE_TRY(alloc_t(t, N * d, &A.x1));
-    CREATE_TRY(alloc_act(t, N * d, &A.h));
+    if (t->deferred_dw) {
+      A.h = stacked(t->h_all, N * d);
+      A.y = stacked(t->y_all, N * qd);
+      A.h2 = stacked(t->h2_all, N * d);
+      A.m = stacked(t->m_all, N * Hd);
+    } else {
+      CREATE_TRY(alloc_act(t, N * d, &A.h));
+      CREATE_TRY(alloc_act(t, N * qd, &A.y));
+      CREATE_TRY(alloc_act(t, N * d, &A.h2));
+      CREATE_TRY(alloc_act(t, N * Hd, &A.m));
+    }
     CREATE_TRY(alloc_act(t, N * qd, &A.q_lin));
     CREATE_TRY(alloc_act(t, N * kd, &A.k_lin));
     CREATE_TRY(alloc_act(t, N * qd, &A.q));
@@ -415,9 +475,6 @@ int32_t onano_create(omx_ctx* ctx, const onano_config* config, onano** out) {
     if (first) A.v = A.raw_v;
     else CREATE_TRY(alloc_act(t, N * kd, &A.v));
     CREATE_TRY(alloc_act(t, N * qd, &A.ap));
-    CREATE_TRY(alloc_act(t, N * qd, &A.y));
-    CREATE_TRY(alloc_act(t, N * d, &A.h2));
-    CREATE_TRY(alloc_act(t, N * Hd, &A.m));
     if (t->fused_mlp) {
       CREATE_TRY(alloc_act(t, 2 * N * Hd, &A.gu));
     } else {
@@ -443,7 +500,7 @@ int32_t onano_create(omx_ctx* ctx, const onano_config* config, onano** out) {
   CREATE_TRY(alloc_act(t, N * (d > qd ? d : qd), &t->t_a));
   CREATE_TRY(alloc_act(t, N * Hd, &t->gm));
   if (t->fused_mlp) {
-    CREATE_TRY(alloc_act(t, 2 * N * Hd, &t->ggu));
+    if (!t->deferred_dw) CREATE_TRY(alloc_act(t, 2 * N * Hd, &t->ggu));
   } else {
     CREATE_TRY(alloc_act(t, N * Hd, &t->g_gact));
     CREATE_TRY(alloc_act(t, N * Hd, &t->g_up));
