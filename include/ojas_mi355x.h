@@ -529,6 +529,31 @@ int32_t omx_value_residual_blend_backward(omx_ctx* ctx, const void* value, const
                                           void* g_value0, int32_t dtype, void* g_lambda_f32,
                                           uint64_t n);
 
+/* rms_qk_norm_forward, rope_half_split_forward and value_residual_blend_forward (backend.rs:1674-1699,
+ * 1907-1920; the sequence of ojas-model/src/block.rs:225-240) in one pass over a fused q | k | v
+ * projection output: bf16 [tokens, pitch] whose token rows hold the query heads, then the key heads,
+ * then the value heads. q and k heads are normed (weights f32 [head_dim]) and rotated (cos / sin f32
+ * [time, head_dim], row r uses table row r % time); the normed row is not rounded to bf16 in
+ * between, where the separate calls round. The value heads are blended with those of `value0`
+ * (block 0's projection output: same layout and pitch; lambda f32 [1]), or copied when value0 is
+ * NULL. head_dim 64 or 128. The backward takes the gradient of the prepared tensor in the same
+ * layout and writes that of the projection output; what the blend sends to block 0's value is
+ * written to (value0_grad_first != 0) or added to value0_grad_f32 [tokens, kv_heads * head_dim];
+ * add_value_grad_f32 (same shape; the block without a blend) is added to the value's gradient.
+ * No counterpart in the trait: a fusion of three of its calls. */
+int32_t omx_qkv_prepare_forward(omx_ctx* ctx, const void* qkv_lin, void* qkv_out, uint64_t pitch,
+                                const void* q_weight_f32, const void* k_weight_f32, const void* cos_f32,
+                                const void* sin_f32, const void* value0, const void* lambda_f32,
+                                uint64_t tokens, uint64_t time, uint64_t heads, uint64_t kv_heads,
+                                uint64_t head_dim, float eps);
+int32_t omx_qkv_prepare_backward(omx_ctx* ctx, const void* qkv_lin, const void* g_qkv, void* g_qkv_lin,
+                                 uint64_t pitch, const void* q_weight_f32, const void* k_weight_f32,
+                                 const void* cos_f32, const void* sin_f32, const void* value0,
+                                 const void* lambda_f32, void* value0_grad_f32, int32_t value0_grad_first,
+                                 const void* add_value_grad_f32, void* g_q_weight_f32, void* g_k_weight_f32,
+                                 void* g_lambda_f32, uint64_t tokens, uint64_t time, uint64_t heads,
+                                 uint64_t kv_heads, uint64_t head_dim, float eps);
+
 /* ---- BackendInt::argmax_rows / topk_rows (backend.rs:1514-1606) ---- */
 int32_t omx_argmax_rows(omx_ctx* ctx, const void* x_f32, uint64_t rows, uint64_t cols,
                         void* out_u32);

@@ -820,6 +820,33 @@ class MiBackend:
     def per_head_sigmoid_gate_backward(self, x, w, b, attn, gy, g_input_dtype: Optional[int] = None):
         return self.per_head_sigmoid_gate_backward_saved(x, w, b, attn, gy, None, g_input_dtype)
 
+    def qkv_prepare_forward(self, qkv_lin, q_weight, k_weight, cos, sin, heads, kv_heads, head_dim, value0=None, lam=None,
+                            eps: float = 1e-6):
+        """QK-norm, RoPE and the value blend over a fused q | k | v projection output (`omx_qkv_prepare_forward`):
+        bf16 [batch, time, (heads + 2 kv_heads) head_dim]."""
+        b, t, pitch = qkv_lin.shape
+        out = self.empty(qkv_lin.shape, BF16)
+        self._check(self._lib.omx_qkv_prepare_forward(
+            self._ctx, self._p(qkv_lin), self._p(out), C.c_uint64(pitch), self._p(q_weight), self._p(k_weight),
+            self._p(cos), self._p(sin), self._p(value0), self._p(lam), C.c_uint64(b * t), C.c_uint64(t), C.c_uint64(heads),
+            C.c_uint64(kv_heads), C.c_uint64(head_dim), C.c_float(eps)))
+        return out
+
+    def qkv_prepare_backward(self, qkv_lin, g_qkv, q_weight, k_weight, cos, sin, heads, kv_heads, head_dim, value0=None,
+                             lam=None, value0_grad=None, value0_grad_first=True, add_value_grad=None, eps: float = 1e-6):
+        """Returns (g_qkv_lin, g_q_weight, g_k_weight, g_lambda or None); `value0_grad` (f32
+        [batch, time, kv_heads head_dim]) is written or added to in place."""
+        b, t, pitch = qkv_lin.shape
+        g_lin = self.empty(qkv_lin.shape, BF16)
+        gqw, gkw = self.empty((head_dim,), F32), self.empty((head_dim,), F32)
+        g_lam = self.empty((1,), F32) if value0 is not None else None
+        self._check(self._lib.omx_qkv_prepare_backward(
+            self._ctx, self._p(qkv_lin), self._p(g_qkv), self._p(g_lin), C.c_uint64(pitch), self._p(q_weight),
+            self._p(k_weight), self._p(cos), self._p(sin), self._p(value0), self._p(lam), self._p(value0_grad),
+            C.c_int32(1 if value0_grad_first else 0), self._p(add_value_grad), self._p(gqw), self._p(gkw), self._p(g_lam),
+            C.c_uint64(b * t), C.c_uint64(t), C.c_uint64(heads), C.c_uint64(kv_heads), C.c_uint64(head_dim), C.c_float(eps)))
+        return g_lin, gqw, gkw, g_lam
+
     def value_residual_blend_forward(self, value, value0, lam):
         self._same("value_residual_blend_forward", value, value0)
         if lam.numel != 1 or lam.dtype != F32:

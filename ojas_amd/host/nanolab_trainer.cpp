@@ -45,6 +45,10 @@ struct onano {
   uint64_t asz = 4;
   bool flash = false;      // time-major MFMA attention (bf16, head_dim 64 or 128)
   bool fused_mlp = false;  // one gate | up product and the fused SwiGLU (bf16)
+  // With MFMA attention the q, k and v projections are one product (their weights are adjacent in
+  // the arena: one [(heads + 2 kv_heads) head_dim, n_embd] matrix), QK-norm, RoPE and the value blend
+  // are one pass over its output, and attention reads q, k and v where that pass left them.
+  bool fused_qkv = false;
   uint64_t steps = 0;
   uint64_t device_bytes = 0;
   std::vector<void*> owned;
@@ -60,6 +64,7 @@ struct onano {
     float *x, *x1;  // residual stream entering the block and after attention (f32)
     void *h, *q_lin, *k_lin, *q, *k, *raw_v, *v, *ap, *apr, *y, *h2, *gu, *g_lin, *up, *g_act, *m;
     void *qp, *kp, *vp, *att;  // [B, heads, T, D] copies for the row kernels (no MFMA attention)
+    void *qkv_lin, *qkv;       // fused projection output and what attention reads: [N, (heads + 2 kv_heads) D]
     float *lse, *gates;
   };
   std::vector<Layer> layers;
@@ -71,6 +76,8 @@ struct onano {
   void *gm = nullptr, *ggu = nullptr, *g_gact = nullptr, *g_up = nullptr;  // MLP gradients AD
   void *gyy = nullptr, *gap = nullptr, *gq = nullptr, *gk = nullptr, *gv = nullptr, *g_raw_v = nullptr, *part_v0 = nullptr;
   void *g_v0 = nullptr;                  // [N, KV D] AD: what the later blocks' blends send to block 0's v
+  void *g_qkv = nullptr, *g_qkv_lin = nullptr, *gqkv_all = nullptr;  // fused projection: gradients [N, P3] AD
+  float* v0_acc = nullptr;               // the same as g_v0 in f32 (fused projection)
   void *gqp = nullptr, *gkp = nullptr, *gvp = nullptr, *gap_p = nullptr;  // permuted gradients (row kernels)
   void *gy16 = nullptr, *ghf = nullptr;
   float *gres = nullptr, *gres1 = nullptr, *gh = nullptr, *g_emb = nullptr;
@@ -150,6 +157,17 @@ int32_t forward(onano* t) {
     float* x_next = last ? t->x_final : t->layers[l + 1].x;
     void* h_next = last ? t->hf : t->layers[l + 1].h;
     const float* next_norm = t->w32(last ? t->nf() : t->li(l + 1, NORM1));
+    if (t->fused_qkv) {
+      const uint64_t P3 = qd + 2 * kd;
+      char* prepared = static_cast<char*>(A.qkv);
+      TRY(omx_linear_forward(ctx, A.h, AD, t->w(t->li(l, WQ)), AD, A.qkv_lin, AD, N, d, P3));
+      // Block 0 has no earlier value to blend with (block.rs:232-238).
+      TRY(omx_qkv_prepare_forward(ctx, A.qkv_lin, A.qkv, P3, t->w32(t->li(l, QNORM)), t->w32(t->li(l, KNORM)), t->cos_t,
+                                  t->sin_t, l > 0 ? t->layers[0].qkv_lin : nullptr,
+                                  l > 0 ? t->w32(t->li(l, LAMBDA)) : nullptr, N, T, H, KV, D, eps));
+      TRY(omx_causal_attention_forward_saving(ctx, prepared, P3, prepared + qd * 2, prepared + (qd + kd) * 2, P3, AD, A.ap,
+                                              A.apr, qd, AD, A.lse, B, T, H, KV, D, W));
+    } else {
     TRY(omx_linear_forward(ctx, A.h, AD, t->w(t->li(l, WQ)), AD, A.q_lin, AD, N, d, qd));
     TRY(omx_linear_forward(ctx, A.h, AD, t->w(t->li(l, WK)), AD, A.k_lin, AD, N, d, kd));
     TRY(omx_linear_forward(ctx, A.h, AD, t->w(t->li(l, WV)), AD, A.raw_v, AD, N, d, kd));
@@ -171,6 +189,7 @@ int32_t forward(onano* t) {
       TRY(omx_permute_0213(ctx, A.v, A.vp, AD, B, T, KV, D));
       TRY(omx_causal_sdpa_forward(ctx, A.qp, A.kp, A.vp, AD, A.att, AD, A.lse, B, H, KV, T, D, W));
       TRY(omx_permute_0213(ctx, A.att, A.ap, AD, B, H, T, D));
+    }
     }
     TRY(omx_per_head_sigmoid_gate_forward(ctx, A.h, t->w(t->li(l, GATE_W)), AD, t->w32(t->li(l, GATE_B)), A.ap, AD, A.y,
                                           AD, A.gates, N, d, H, D));
@@ -264,6 +283,31 @@ int32_t backward(onano* t, float loss_seed) {
     TRY(omx_per_head_sigmoid_gate_backward(ctx, A.h, t->w(t->li(l, GATE_W)), AD, t->w32(t->li(l, GATE_B)), A.ap, AD, t->gyy,
                                            AD, A.gates, t->gh, OMX_F32, t->g(t->li(l, GATE_W)), t->g(t->li(l, GATE_B)),
                                            t->gap, AD, N, d, H, D));
+    if (t->fused_qkv) {
+      const uint64_t P3 = qd + 2 * kd;
+      char* prepared = static_cast<char*>(A.qkv);
+      char* gp = static_cast<char*>(t->g_qkv);
+      void* g_lin = defer ? slice(t->gqkv_all, l, N * P3) : t->g_qkv_lin;
+      TRY(omx_causal_attention_backward_saved(ctx, prepared, P3, prepared + qd * 2, prepared + (qd + kd) * 2, P3, A.ap, A.apr,
+                                              t->gap, qd, A.lse, AD, gp, gp + qd * 2, gp + (qd + kd) * 2, AD, B, T, H, KV, D,
+                                              W));
+      // Block 0's value also feeds every later block's blend: their shares collect in v0_acc (the
+      // last block writes it, the others add) and join block 0's own gradient here.
+      const bool blends = l > 0, last = l + 1 == c.layers;
+      TRY(omx_qkv_prepare_backward(ctx, A.qkv_lin, t->g_qkv, g_lin, P3, t->w32(t->li(l, QNORM)), t->w32(t->li(l, KNORM)),
+                                   t->cos_t, t->sin_t, blends ? t->layers[0].qkv_lin : nullptr,
+                                   blends ? t->w32(t->li(l, LAMBDA)) : nullptr, blends ? t->v0_acc : nullptr, last ? 1 : 0,
+                                   !blends && c.layers > 1 ? t->v0_acc : nullptr, t->g(t->li(l, QNORM)),
+                                   t->g(t->li(l, KNORM)), blends ? t->g(t->li(l, LAMBDA)) : nullptr, N, T, H, KV, D, eps));
+      if (!blends) TRY(omx_fill_zero(ctx, t->g(t->li(0, LAMBDA)), 4));
+      // One product for the three projections: their input gradients add in its f32 accumulators.
+      TRY(omx_linear_backward(ctx, A.h, t->w(t->li(l, WQ)), g_lin, AD, t->t_a, AD, gw(WQ), OMX_F32, N, d, P3));
+      TRY(omx_residual_add(ctx, t->gh, OMX_F32, t->t_a, AD, t->gh, OMX_F32, N * d));
+      TRY(omx_rms_norm_backward_residual(ctx, A.x, OMX_F32, t->w32(t->li(l, NORM1)), t->gh, OMX_F32, t->gres1, t->gres,
+                                         copy_below, t->g(t->li(l, NORM1)), N, d, eps));
+      gy = static_cast<const void*>(copy_below);
+      continue;
+    }
     if (t->flash) {
       TRY(omx_causal_attention_backward_saved(ctx, A.q, qd, A.k, A.v, kd, A.ap, A.apr, t->gap, qd, A.lse, AD, t->gq, t->gk,
                                               t->gv, AD, B, T, H, KV, D, W));
@@ -317,9 +361,13 @@ int32_t backward(onano* t, float loss_seed) {
     } products[6] = {{t->gyd_all, t->m_all, FFN_DOWN, d, Hd}, {t->ggu_all, t->h2_all, FFN_GATE, 2 * Hd, d},
                      {t->gyo_all, t->y_all, WO, d, qd},       {t->gv_all, t->h_all, WV, kd, d},
                      {t->gk_all, t->h_all, WK, kd, d},        {t->gq_all, t->h_all, WQ, qd, d}};
-    for (const Deferred& p : products)
+    if (t->fused_qkv) products[3] = {t->gqkv_all, t->h_all, WQ, qd + 2 * kd, d};
+    const int count = t->fused_qkv ? 4 : 6;
+    for (int i = 0; i < count; ++i) {
+      const Deferred& p = products[i];
       TRY(omx_gemm_strided_batch(ctx, p.gy, 1, p.out, p.x, p.in, 1, AD, t->g(t->li(0, p.which)), OMX_F32, p.out, N, p.in, 0,
                                  layers, N * p.out, N * p.in, per_layer));
+    }
   }
   // The tied table: the head's gradient first, then the embedding's rows.
   TRY(omx_embedding_backward(ctx, t->ids, t->gres, OMX_F32, t->g_emb, N, c.vocab, d));
@@ -363,6 +411,9 @@ int32_t onano_create(omx_ctx* ctx, const onano_config* config, onano** out) {
   t->flash = c.bf16 && (c.head_dim == 64 || c.head_dim == 128);
   t->fused_mlp = c.bf16 && c.hidden % 8 == 0;
   t->deferred_dw = t->fused_mlp && c.layers > 1;
+  // The three projections are one matrix only if nothing pads the arena between them.
+  t->fused_qkv = t->flash && (static_cast<uint64_t>(c.heads) * c.head_dim * c.n_embd) % kAlign == 0 &&
+                 (static_cast<uint64_t>(c.kv_heads) * c.head_dim * c.n_embd) % kAlign == 0;
   const uint64_t N = t->N, d = c.n_embd, H = c.heads, KV = c.kv_heads, D = c.head_dim, Hd = c.hidden;
   const uint64_t qd = H * D, kd = KV * D;
   uint64_t at = 0;
@@ -444,9 +495,13 @@ int32_t onano_create(omx_ctx* ctx, const onano_config* config, onano** out) {
     CREATE_TRY(alloc_act(t, L * N * d, &t->gyd_all));
     CREATE_TRY(alloc_act(t, L * 2 * N * Hd, &t->ggu_all));
     CREATE_TRY(alloc_act(t, L * N * d, &t->gyo_all));
-    CREATE_TRY(alloc_act(t, L * N * qd, &t->gq_all));
-    CREATE_TRY(alloc_act(t, L * N * kd, &t->gk_all));
-    CREATE_TRY(alloc_act(t, L * N * kd, &t->gv_all));
+    if (t->fused_qkv) {
+      CREATE_TRY(alloc_act(t, L * N * (qd + 2 * kd), &t->gqkv_all));
+    } else {
+      CREATE_TRY(alloc_act(t, L * N * qd, &t->gq_all));
+      CREATE_TRY(alloc_act(t, L * N * kd, &t->gk_all));
+      CREATE_TRY(alloc_act(t, L * N * kd, &t->gv_all));
+    }
   }
   uint32_t index = 0;
   for (auto& A : t->layers) {
@@ -467,13 +522,18 @@ int32_t onano_create(omx_ctx* ctx, const onano_config* config, onano** out) {
       CREATE_TRY(alloc_act(t, N * d, &A.h2));
       CREATE_TRY(alloc_act(t, N * Hd, &A.m));
     }
-    CREATE_TRY(alloc_act(t, N * qd, &A.q_lin));
-    CREATE_TRY(alloc_act(t, N * kd, &A.k_lin));
-    CREATE_TRY(alloc_act(t, N * qd, &A.q));
-    CREATE_TRY(alloc_act(t, N * kd, &A.k));
-    CREATE_TRY(alloc_act(t, N * kd, &A.raw_v));
-    if (first) A.v = A.raw_v;
-    else CREATE_TRY(alloc_act(t, N * kd, &A.v));
+    if (t->fused_qkv) {
+      CREATE_TRY(alloc_act(t, N * (qd + 2 * kd), &A.qkv_lin));
+      CREATE_TRY(alloc_act(t, N * (qd + 2 * kd), &A.qkv));
+    } else {
+      CREATE_TRY(alloc_act(t, N * qd, &A.q_lin));
+      CREATE_TRY(alloc_act(t, N * kd, &A.k_lin));
+      CREATE_TRY(alloc_act(t, N * qd, &A.q));
+      CREATE_TRY(alloc_act(t, N * kd, &A.k));
+      CREATE_TRY(alloc_act(t, N * kd, &A.raw_v));
+      if (first) A.v = A.raw_v;
+      else CREATE_TRY(alloc_act(t, N * kd, &A.v));
+    }
     CREATE_TRY(alloc_act(t, N * qd, &A.ap));
     if (t->fused_mlp) {
       CREATE_TRY(alloc_act(t, 2 * N * Hd, &A.gu));
@@ -504,6 +564,11 @@ int32_t onano_create(omx_ctx* ctx, const onano_config* config, onano** out) {
   } else {
     CREATE_TRY(alloc_act(t, N * Hd, &t->g_gact));
     CREATE_TRY(alloc_act(t, N * Hd, &t->g_up));
+  }
+  if (t->fused_qkv) {
+    CREATE_TRY(alloc_act(t, N * (qd + 2 * kd), &t->g_qkv));
+    if (!t->deferred_dw) CREATE_TRY(alloc_act(t, N * (qd + 2 * kd), &t->g_qkv_lin));
+    CREATE_TRY(alloc_t(t, N * kd, &t->v0_acc));
   }
   CREATE_TRY(alloc_act(t, N * qd, &t->gyy));
   CREATE_TRY(alloc_act(t, N * qd, &t->gap));

@@ -477,3 +477,72 @@ def test_value_residual_known_answer_and_nonfinite_lambda(be):
         be.download(be.value_residual_blend_forward(be.upload(np.ones(4, np.float32)), be.upload(np.ones(4, np.float32)),
                                                     be.upload(np.array([np.nan], np.float32))))
     assert e.value.variant == "NonFinite"
+
+
+@pytest.mark.parametrize("heads,kv_heads,dim,blend", [(4, 2, 64, True), (2, 2, 128, True), (3, 1, 64, False), (2, 1, 128, False)])
+def test_qkv_prepare_equals_norm_then_rope_then_blend(be, heads, kv_heads, dim, blend):
+    """`omx_qkv_prepare_forward / _backward` over a fused q | k | v projection output against the
+    oracle's separate ops in sequence (rms_norm per head, half-split RoPE, value-residual blend):
+    forward and every gradient within the bf16 gate of the largest value. Without a blend the value
+    block is copied and `add_value_grad` joins its gradient (block 0 of the model, which every later
+    block's blend feeds)."""
+    from ojas_amd.backend import BF16
+
+    print(f"qkv prepare heads={heads}/{kv_heads} dim={dim} blend={blend}", flush=True)
+    b, t = 2, 37
+    slots = heads + 2 * kv_heads
+    r = orc.SplitMix64(500 + dim + heads)
+    rnd = orc.round_bf16
+    lin = rnd(r.vec(b * t * slots * dim, 1.0)).reshape(b, t, slots * dim)
+    lin0 = rnd(r.vec(b * t * slots * dim, 1.0)).reshape(b, t, slots * dim)
+    g = rnd(r.vec(b * t * slots * dim, 1.0)).reshape(b, t, slots * dim)
+    qw, kw = 1.0 + r.vec(dim, 0.2), 1.0 + r.vec(dim, 0.2)
+    lam = np.array([0.3], np.float32)
+    add_v = r.vec(b * t * kv_heads * dim, 1.0).reshape(b, t, kv_heads * dim)
+    cos, sin = orc.rope_tables(t, dim)
+    qd, kd = heads * dim, kv_heads * dim
+    split = lambda a: (a[..., :qd].reshape(b, t, heads, dim), a[..., qd:qd + kd].reshape(b, t, kv_heads, dim),
+                       a[..., qd + kd:].reshape(b, t, kv_heads, dim))
+    q, k, v = split(lin)
+    _, _, v0 = split(lin0)
+    gq, gk, gv = split(g)
+    # the oracle's sequence
+    qn, kn = orc.rms_norm_forward(q, qw), orc.rms_norm_forward(k, kw)
+    want_q, want_k = orc.rope_forward(qn, cos, sin), orc.rope_forward(kn, cos, sin)
+    want_v = orc.value_residual_forward(v, v0, float(lam[0])) if blend else v
+    gqn, gkn = orc.rope_backward(gq, cos, sin), orc.rope_backward(gk, cos, sin)
+    want_gq, want_gqw = orc.rms_norm_backward(q, qw, gqn)
+    want_gk, want_gkw = orc.rms_norm_backward(k, kw, gkn)
+    if blend:
+        want_gv, want_gv0, want_gl = orc.value_residual_backward(v, v0, float(lam[0]), gv)
+    else:
+        want_gv = gv + add_v.reshape(gv.shape)
+    # the device, one call each way
+    d_lin, d_lin0, d_g = (be.upload(a, BF16) for a in (lin, lin0, g))
+    d_qw, d_kw, d_cos, d_sin, d_lam = (be.upload(a) for a in (qw, kw, cos, sin, lam))
+    out = be.qkv_prepare_forward(d_lin, d_qw, d_kw, d_cos, d_sin, heads, kv_heads, dim, d_lin0 if blend else None,
+                                 d_lam if blend else None)
+    got_q, got_k, got_v = split(be.download_f32(out))
+    close(got_q, want_q, BF16_TOL, "prepared q")
+    close(got_k, want_k, BF16_TOL, "prepared k")
+    close(got_v, want_v, BF16_TOL, "prepared v")
+    if blend:
+        before = r.vec(b * t * kd, 1.0).reshape(b, t, kd)
+        acc = be.upload(before)
+        g_lin, gqw, gkw, g_lam = be.qkv_prepare_backward(d_lin, d_g, d_qw, d_kw, d_cos, d_sin, heads, kv_heads, dim, d_lin0,
+                                                         d_lam, value0_grad=acc, value0_grad_first=False)
+        close(be.download(acc), before + want_gv0.reshape(before.shape), BF16_TOL, "value0 gradient, added")
+        be.qkv_prepare_backward(d_lin, d_g, d_qw, d_kw, d_cos, d_sin, heads, kv_heads, dim, d_lin0, d_lam, value0_grad=acc,
+                                value0_grad_first=True)
+        close(be.download(acc), want_gv0.reshape(before.shape), BF16_TOL, "value0 gradient, written")
+        assert abs(float(be.download(g_lam)[0]) - float(want_gl)) <= BF16_TOL * max(1.0, abs(float(want_gl)))
+    else:
+        g_lin, gqw, gkw, g_lam = be.qkv_prepare_backward(d_lin, d_g, d_qw, d_kw, d_cos, d_sin, heads, kv_heads, dim,
+                                                         add_value_grad=be.upload(add_v))
+        assert g_lam is None
+    got_gq, got_gk, got_gv = split(be.download_f32(g_lin))
+    close(got_gq, want_gq, BF16_TOL, "gq")
+    close(got_gk, want_gk, BF16_TOL, "gk")
+    close(got_gv, want_gv, BF16_TOL, "gv")
+    close(be.download(gqw), want_gqw, BF16_TOL, "q norm weight gradient")
+    close(be.download(gkw), want_gkw, BF16_TOL, "k norm weight gradient")
