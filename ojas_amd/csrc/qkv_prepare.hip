@@ -338,11 +338,12 @@ int32_t omx_qkv_prepare_backward(omx_ctx* ctx, const void* qkv_lin, const void* 
   if (blocks > 1024) blocks = 1024;
   void* ws = nullptr;
   const uint64_t partial_w_floats = static_cast<uint64_t>(blocks) * 2 * head_dim;
-  rc = omx_workspace(ctx, (partial_w_floats + 2 * head_dim + blocks + 64) * sizeof(float), &ws);
+  rc = omx_workspace(ctx, (partial_w_floats + (1 + OMX_COLUMN_SUM_GROUPS) * 2 * head_dim + blocks + 64) * sizeof(float), &ws);
   if (rc != OMX_OK) return rc;
   float* partial_w = static_cast<float*>(ws);
   float* summed = partial_w + partial_w_floats;  // [2][D]
-  float* partial_lambda = summed + 2 * head_dim;
+  float* stage = summed + 2 * head_dim;          // the column sum's first stage
+  float* partial_lambda = stage + OMX_COLUMN_SUM_GROUPS * 2 * head_dim;
   const unsigned long long tag = omx_tag(ctx, F_RMS_BACKWARD);
 #define QP_BWD(D_)                                                                                                     \
   hipLaunchKernelGGL((qkv_prepare_bwd_kernel<D_>), dim3(blocks), dim3(QP_THREADS), 0, ctx->stream,                     \
@@ -357,7 +358,7 @@ int32_t omx_qkv_prepare_backward(omx_ctx* ctx, const void* qkv_lin, const void* 
 #undef QP_BWD
   OMX_LAUNCH_CHECK(ctx, "qkv_prepare_bwd_kernel");
   // partial_w is [blocks][2 D]: one column sum gives both weights' gradients side by side.
-  rc = omx_column_sum(ctx, partial_w, summed, blocks, 2 * head_dim, tag);
+  rc = omx_column_sum(ctx, partial_w, summed, blocks, 2 * head_dim, tag, stage);
   if (rc != OMX_OK) return rc;
   rc = omx_copy(ctx, g_q_weight, summed, head_dim * sizeof(float));
   if (rc != OMX_OK) return rc;

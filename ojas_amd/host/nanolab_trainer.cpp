@@ -40,6 +40,7 @@ struct onano {
   omx_ctx* ctx = nullptr;
   onano_config c{};
   uint64_t N = 0, P = 0;
+  uint64_t adam_end = 0;  // the arena's first adam_end elements are AdamW's (table and vectors)
   std::vector<Slot> slots;
   int32_t AD = OMX_F32;
   uint64_t asz = 4;
@@ -354,7 +355,7 @@ int32_t backward(onano* t, float loss_seed) {
   }
   if (defer) {
     // gw[l](o, j) = sum_r gy[l][r, o] * x[l][r, j] for every block l, one launch per weight.
-    const uint64_t layers = c.layers, per_layer = t->slots[t->li(1, NORM1)].offset - t->slots[t->li(0, NORM1)].offset;
+    const uint64_t layers = c.layers, per_layer = t->slots[t->li(1, WQ)].offset - t->slots[t->li(0, WQ)].offset;
     struct Deferred {
       const void *gy, *x;
       uint64_t which, out, in;
@@ -416,30 +417,36 @@ int32_t onano_create(omx_ctx* ctx, const onano_config* config, onano** out) {
                  (static_cast<uint64_t>(c.kv_heads) * c.head_dim * c.n_embd) % kAlign == 0;
   const uint64_t N = t->N, d = c.n_embd, H = c.heads, KV = c.kv_heads, D = c.head_dim, Hd = c.hidden;
   const uint64_t qd = H * D, kd = KV * D;
+  // Arena order (the parameter indices keep the order of names.rs): the table, then every vector of
+  // every block and the final norm side by side (one AdamW pass covers them), block 0's vr_lambda
+  // last among them (no gradient reaches it and no optimizer touches it), then the matrices block
+  // by block at a fixed stride.
+  struct Shape {
+    uint64_t rows, cols;
+  };
+  std::vector<Shape> shapes;
+  shapes.push_back({c.vocab, d});
+  for (uint32_t l = 0; l < c.layers; ++l) {
+    const Shape block[kPerBlock] = {{d, 0}, {qd, d}, {kd, d}, {kd, d}, {d, qd}, {D, 0}, {D, 0}, {H, d}, {H, 0}, {1, 0},
+                                    {d, 0}, {Hd, d}, {Hd, d}, {d, Hd}};
+    shapes.insert(shapes.end(), block, block + kPerBlock);
+  }
+  shapes.push_back({d, 0});
+  t->slots.resize(shapes.size());
   uint64_t at = 0;
-  auto add = [&](uint64_t rows, uint64_t cols) {
-    const uint64_t len = cols ? rows * cols : rows;
-    t->slots.push_back({at, len, rows, cols});
+  auto place = [&](uint64_t i) {
+    const uint64_t len = shapes[i].cols ? shapes[i].rows * shapes[i].cols : shapes[i].rows;
+    t->slots[i] = {at, len, shapes[i].rows, shapes[i].cols};
     at += (len + kAlign - 1) / kAlign * kAlign;
   };
-  add(c.vocab, d);
-  for (uint32_t l = 0; l < c.layers; ++l) {
-    add(d, 0);
-    add(qd, d);
-    add(kd, d);
-    add(kd, d);
-    add(d, qd);
-    add(D, 0);
-    add(D, 0);
-    add(H, d);
-    add(H, 0);
-    add(1, 0);
-    add(d, 0);
-    add(Hd, d);
-    add(Hd, d);
-    add(d, Hd);
-  }
-  add(d, 0);
+  const uint64_t frozen = 1 + LAMBDA;
+  place(0);
+  for (uint64_t i = 1; i < shapes.size(); ++i)
+    if (shapes[i].cols == 0 && i != frozen) place(i);
+  t->adam_end = at;
+  place(frozen);
+  for (uint64_t i = 1; i < shapes.size(); ++i)
+    if (shapes[i].cols != 0) place(i);
   t->P = at;
 #define CREATE_TRY(expr)           \
   do {                             \
@@ -692,20 +699,9 @@ int32_t onano_apply(onano* t, const omx_muon_config* muon, const omx_adamw_confi
   // padding and block 0's vr_lambda hold zeros and add nothing to it.
   TRY(omx_clip_grad_norm(t->ctx, grads, lens, 1, grad_clip > 0.0f ? grad_clip : INFINITY, &norm));
   uint16_t* mirror = static_cast<uint16_t*>(t->p16);
-  // AdamW: runs of adjacent parameters share a pass.
+  // AdamW: the table and every vector sit side by side at the arena's start.
+  TRY(omx_adamw_step(t->ctx, t->p32, t->acc, t->m1, t->m2, t->adam_end, t->steps, adamw, mirror));
   const uint64_t count = t->slots.size();
-  for (uint64_t i = 0; i < count;) {
-    if (t->is_muon(i) || t->is_frozen(i)) {
-      ++i;
-      continue;
-    }
-    uint64_t j = i;
-    while (j + 1 < count && !t->is_muon(j + 1) && !t->is_frozen(j + 1)) ++j;
-    const uint64_t at = t->slots[i].offset, n = t->slots[j].offset + t->slots[j].len - at;
-    TRY(omx_adamw_step(t->ctx, t->p32 + at, t->acc + at, t->m1 + at, t->m2 + at, n, t->steps, adamw,
-                       mirror ? mirror + at : nullptr));
-    i = j + 1;
-  }
   // Muon: matrices of one shape go through Newton-Schulz together.
   struct Group {
     std::vector<void*> p, m, p16;
