@@ -224,9 +224,9 @@ __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_fwd_kernel(const un
                                                        unsigned short* __restrict__ resid, float* __restrict__ lse,
                                                        FlashShape s, OmxFaultWord* fault, unsigned long long tag) {
   constexpr int KK = D / 16, MT = D / 32, NL = D / 32;  // d slabs, d blocks of the output, loads per thread and tile
-  __shared__ __attribute__((aligned(16))) char smem[2 * ftile(D)];
-  char* k_rows = smem;
-  char* v_rows = smem + ftile(D);
+  // Two key / value tile pairs: the next tile is stored while this one is multiplied, so a tile
+  // costs one barrier.
+  __shared__ __attribute__((aligned(16))) char smem[4 * ftile(D)];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lg = lane >> 5;
   const int T = s.time;
   // Query block j sees j / 2 + 1 key tiles (causal): a workgroup takes a late block and then
@@ -266,15 +266,27 @@ __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_fwd_kernel(const un
     u32x4 rk[NL], rv[NL];
     tile_load<D>(kp, s.kv.rs, kt_first * 64, T, rk);
     tile_load<D>(vp, s.kv.rs, kt_first * 64, T, rv);
+    __syncthreads();  // the previous pass's reads of the first pair are done
+    tile_store_rows<D>(smem, rk);
+    tile_store_rows<D>(smem + ftile(D), rv);
+    if (kt_first < kt_last) {
+      tile_load<D>(kp, s.kv.rs, kt_first * 64 + 64, T, rk);
+      tile_load<D>(vp, s.kv.rs, kt_first * 64 + 64, T, rv);
+    }
     for (int kt = kt_first; kt <= kt_last; ++kt) {
       const int key0 = kt * 64;
-      __syncthreads();  // the previous tile's reads are done
-      tile_store_rows<D>(k_rows, rk);
-      tile_store_rows<D>(v_rows, rv);
-      __syncthreads();
+      const int cur = (kt - kt_first) & 1;
+      char* k_rows = smem + cur * 2 * ftile(D);
+      char* v_rows = k_rows + ftile(D);
+      __syncthreads();  // this pair is complete, and every wave is done with the other one
       if (kt < kt_last) {
-        tile_load<D>(kp, s.kv.rs, key0 + 64, T, rk);
-        tile_load<D>(vp, s.kv.rs, key0 + 64, T, rv);
+        char* next = smem + (cur ^ 1) * 2 * ftile(D);
+        tile_store_rows<D>(next, rk);
+        tile_store_rows<D>(next + ftile(D), rv);
+        if (kt + 1 < kt_last) {
+          tile_load<D>(kp, s.kv.rs, key0 + 128, T, rk);
+          tile_load<D>(vp, s.kv.rs, key0 + 128, T, rv);
+        }
       }
       const bool active = key0 <= wave_q0 + 31 && (s.window == 0 || key0 + 63 + s.window > wave_q0);
       if (!active) continue;
@@ -371,10 +383,7 @@ __device__ __forceinline__ bool flash_dkv_block(const unsigned short* __restrict
                                                 TO* __restrict__ gk, TO* __restrict__ gv, const FlashShape& s, char* smem,
                                                 int kb, int b, int gidx) {
   constexpr int KK = D / 16, MT = D / 32, NL = D / 32;
-  char* q_rows = smem;
-  char* g_rows = smem + ftile(D);
-  float* lse_s = reinterpret_cast<float*>(smem + 2 * ftile(D));
-  float* del_s = lse_s + 64;
+  constexpr int SET = 2 * ftile(D) + 2 * 64 * 4;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lg = lane >> 5;
   const int T = s.time;
   const long kv_off = b * s.kv.bs + gidx * s.kv.hs;
@@ -419,19 +428,31 @@ __device__ __forceinline__ bool flash_dkv_block(const unsigned short* __restrict
       bad |= !(dev_finite(row_lse) && dev_finite(row_del));
     }
   };
+  auto store_set = [&](char* set) {
+    tile_store_rows<D>(set, rq);
+    tile_store_rows<D>(set + ftile(D), rg);
+    if (threadIdx.x < 64) {
+      float* stats = reinterpret_cast<float*>(set + 2 * ftile(D));
+      stats[threadIdx.x] = row_lse * LOG2E;
+      stats[64 + threadIdx.x] = row_del;
+    }
+  };
   fetch();
+  __syncthreads();  // an earlier walk's reads of the first set are done
+  store_set(smem);
+  if (steps > 1) fetch();
   for (int idx = 0; idx < steps; ++idx) {
     const int q0 = cur_qt * 64;
     if (++cur_qt > qt_last) cur_qt = qt_first;
-    __syncthreads();
-    tile_store_rows<D>(q_rows, rq);
-    tile_store_rows<D>(g_rows, rg);
-    if (threadIdx.x < 64) {
-      lse_s[threadIdx.x] = row_lse * LOG2E;
-      del_s[threadIdx.x] = row_del;
+    char* q_rows = smem + (idx & 1) * SET;
+    char* g_rows = q_rows + ftile(D);
+    const float* lse_s = reinterpret_cast<const float*>(q_rows + 2 * ftile(D));
+    const float* del_s = lse_s + 64;
+    __syncthreads();  // this set is complete, and every wave is done with the other one
+    if (idx + 1 < steps) {
+      store_set(smem + ((idx & 1) ^ 1) * SET);
+      if (idx + 2 < steps) fetch();
     }
-    __syncthreads();
-    if (idx + 1 < steps) fetch();
     const bool active = q0 + 63 >= wave_k0 && (s.window == 0 || q0 < wave_k0 + 31 + s.window);
     if (!active) continue;
     // Wave-uniform: a tile whose queries all come after the wave's keys and end inside the sequence has no mask.
@@ -496,7 +517,9 @@ __global__ __launch_bounds__(FT, 2) void flash_bwd_dkv_kernel(
     const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
     const float* __restrict__ lse, const float* __restrict__ delta, const unsigned short* __restrict__ gy,
     TO* __restrict__ gk, TO* __restrict__ gv, FlashShape s, OmxFaultWord* fault, unsigned long long tag) {
-  __shared__ __attribute__((aligned(16))) char smem[2 * ftile(D) + 2 * 64 * 4];
+  // Two sets of (query tile, gradient tile, 64 log-sum-exp values, 64 row terms): the next set is
+  // stored while this one is multiplied, so a tile costs one barrier.
+  __shared__ __attribute__((aligned(16))) char smem[2 * (2 * ftile(D) + 2 * 64 * 4)];
   // Early key blocks are seen by the most queries: a workgroup takes one of them and then its
   // mirror image from the back (see the forward kernel).
   const int k_blocks = (s.time + 127) / 128;
@@ -561,9 +584,8 @@ __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_bwd_dq_kernel(
     float* __restrict__ delta, const float* __restrict__ key_mean, const unsigned short* __restrict__ gy,
     TO* __restrict__ gq, FlashShape s, OmxFaultWord* fault, unsigned long long tag) {
   constexpr int KK = D / 16, MT = D / 32, NL = D / 32;
-  __shared__ __attribute__((aligned(16))) char smem[2 * ftile(D)];
-  char* k_rows = smem;
-  char* v_rows = smem + ftile(D);
+  // Two key / value tile pairs, as in the forward: one barrier per tile.
+  __shared__ __attribute__((aligned(16))) char smem[4 * ftile(D)];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lg = lane >> 5;
   const int T = s.time;
   // A late query block, then its mirror image from the front (see the forward kernel).
@@ -635,15 +657,27 @@ __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_bwd_dq_kernel(
     u32x4 rk[NL], rv[NL];
     tile_load<D>(kp, s.kv.rs, kt_first * 64, T, rk);
     tile_load<D>(vp, s.kv.rs, kt_first * 64, T, rv);
+    __syncthreads();  // the previous pass's reads of the first pair are done
+    tile_store_rows<D>(smem, rk);
+    tile_store_rows<D>(smem + ftile(D), rv);
+    if (kt_first < kt_last) {
+      tile_load<D>(kp, s.kv.rs, kt_first * 64 + 64, T, rk);
+      tile_load<D>(vp, s.kv.rs, kt_first * 64 + 64, T, rv);
+    }
     for (int kt = kt_first; kt <= kt_last; ++kt) {
       const int key0 = kt * 64;
-      __syncthreads();
-      tile_store_rows<D>(k_rows, rk);
-      tile_store_rows<D>(v_rows, rv);
-      __syncthreads();
+      const int cur = (kt - kt_first) & 1;
+      char* k_rows = smem + cur * 2 * ftile(D);
+      char* v_rows = k_rows + ftile(D);
+      __syncthreads();  // this pair is complete, and every wave is done with the other one
       if (kt < kt_last) {
-        tile_load<D>(kp, s.kv.rs, key0 + 64, T, rk);
-        tile_load<D>(vp, s.kv.rs, key0 + 64, T, rv);
+        char* next = smem + (cur ^ 1) * 2 * ftile(D);
+        tile_store_rows<D>(next, rk);
+        tile_store_rows<D>(next + ftile(D), rv);
+        if (kt + 1 < kt_last) {
+          tile_load<D>(kp, s.kv.rs, key0 + 128, T, rk);
+          tile_load<D>(vp, s.kv.rs, key0 + 128, T, rv);
+        }
       }
       const bool active = key0 <= wave_q0 + 31 && (s.window == 0 || key0 + 63 + s.window > wave_q0);
       if (!active) continue;
