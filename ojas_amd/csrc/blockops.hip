@@ -580,17 +580,18 @@ int32_t omx_per_head_sigmoid_gate_backward(omx_ctx* ctx, const void* input, cons
   if (attn_dtype != gy_dtype)
     return omx_fail(ctx, OMX_DTYPE, "%s: attn and grad_output must share a dtype", op);
 
-  // Workspace: [gates f32][gz in the operand dtype][per-block bias partials].
+  // Workspace: [gates f32][gz in the operand dtype][per-block bias partials][two-stage sum scratch].
   const int block_rows = 16;
   const uint64_t blocks = (rows + block_rows - 1) / block_rows;
   const uint64_t items = rows * heads;
   const uint64_t gates_bytes = round_up(items * sizeof(float), 256);
   const uint64_t gz_bytes = round_up(items * omx_dtype_size(operand_dtype), 256);
-  const uint64_t partial_bytes = blocks * heads * sizeof(float);
+  const uint64_t partial_bytes = round_up(blocks * heads * sizeof(float), 256);
+  const uint64_t stage_bytes = OMX_COLUMN_SUM_GROUPS * heads * sizeof(float);
   const size_t lds_bytes = static_cast<size_t>(block_rows) * heads * sizeof(float);
   if (lds_bytes > 64 * 1024) return omx_fail(ctx, OMX_UNSUPPORTED, "%s: %llu heads above 1024", op, (unsigned long long)heads);
   void* ws = nullptr;
-  rc = omx_workspace(ctx, gates_bytes + gz_bytes + partial_bytes, &ws);
+  rc = omx_workspace(ctx, gates_bytes + gz_bytes + partial_bytes + stage_bytes, &ws);
   if (rc != OMX_OK) return rc;
   char* base = static_cast<char*>(ws);
   const float* gates = static_cast<const float*>(gates_saved);
@@ -602,6 +603,7 @@ int32_t omx_per_head_sigmoid_gate_backward(omx_ctx* ctx, const void* input, cons
   }
   void* gz = base + gates_bytes;
   float* partial = reinterpret_cast<float*>(base + gates_bytes + gz_bytes);
+  float* stage = reinterpret_cast<float*>(base + gates_bytes + gz_bytes + partial_bytes);
 
   const bool vec = head_dim % 4 == 0 && packs_of_four(4, omx_dtype_size(attn_dtype), {attn, gy}) &&
                    packs_of_four(4, omx_dtype_size(g_attn_dtype), {g_attn});
@@ -637,7 +639,7 @@ int32_t omx_per_head_sigmoid_gate_backward(omx_ctx* ctx, const void* input, cons
 #undef GATE_BWD_V
 #undef GATE_BWD
   OMX_LAUNCH_CHECK(ctx, "gate_bwd_kernel");
-  rc = omx_column_sum(ctx, partial, static_cast<float*>(g_bias), blocks, heads, tag);
+  rc = omx_column_sum(ctx, partial, static_cast<float*>(g_bias), blocks, heads, tag, stage);
   if (rc != OMX_OK) return rc;
   // grad_input[r, i] = sum_h gz[r, h] weight[h, i]
   rc = omx_gemm_impl(ctx, F_GATE_BACKWARD, gz, heads, 1, weight, d_model, 1, operand_dtype, g_input, g_input_dtype,

@@ -16,6 +16,10 @@ configs[4]: (1) the model at full width (d 2048, 16 heads of 128, SwiGLU 8192, v
 products equal the bf16 products of the dequantised weights; (3) the adapter starts as the identity
 (B = 0: the loss does not depend on A and dA is exactly zero); (4) the gradient predicts the change
 of the loss along itself; (5) AdamW on the adapters lowers the loss on a fixed batch.
+
+The nanolab graph at the 124M size: the bf16 tier against the f32 tier (which the oracle pins at
+small sizes, tests/test_gpu_nanolab_native.py), the same derivative check, micro-batch accumulation
+and the hybrid step.
 """
 import numpy as np
 import pytest
@@ -262,5 +266,98 @@ def test_lora_step_at_full_size(be):
         adamw = AdamWConfig(1e-3, 0.9, 0.95, 1e-8, 0.0)
         curve = [tr.step(adamw, 1.0)[0] for _ in range(6)]
         assert curve[0] == base and curve[-1] < curve[0] - 1e-3 and tr.steps() == 6, curve
+    finally:
+        tr.close()
+
+
+# ------------------------------------------------------------------ the nanolab graph at the 124M size
+def test_nanolab_124m_step_at_full_size(be):
+    """The native nanolab driver at `ModelSpec::nanolab_124m` (ojas-model/src/spec.rs:74-91), 16 x 1024
+    tokens, bf16 tier: the paths only this size takes (MFMA attention on the fused q | k | v output,
+    the weight gradients as strided batches after the backward, one AdamW pass over the table and
+    the vectors). The f32 tier, which the oracle pins at small sizes, gives the same gradients at
+    4 x 1024 tokens; the gradient predicts the change of the loss along itself; two half-weighted
+    micro-batches add up to the whole one; six hybrid steps on one batch lower the loss."""
+    from ojas_amd.nanolab import NativeNanolabTrainer, spec_nanolab_124m
+
+    spec = spec_nanolab_124m()
+    rng = np.random.default_rng(31)
+    print("nanolab 124M: tiers at 4 x 1024", flush=True)
+    small = rng.integers(0, spec.vocab, (4, 1025)).astype(np.uint32)
+    tier = {}
+    params = None
+    for bf16 in (True, False):
+        tr = NativeNanolabTrainer(be, spec, 4, 1024, bf16=bf16)
+        try:
+            if params is None:
+                tr.init(17)
+                params = tr.download_params()
+                # a gate that is not flat and value residuals that are not at their start
+                for name in params:
+                    if name.endswith("vr_lambda"):
+                        params[name] = rng.uniform(0.2, 0.8, params[name].shape).astype(np.float32)
+                    if name.endswith("gate.bias"):
+                        params[name] = rng.normal(0, 0.5, params[name].shape).astype(np.float32)
+            tr.set_params(params)
+            tier[bf16] = tr.loss_and_grads(small[:, :-1], small[:, 1:])
+        finally:
+            tr.close()
+    (loss16, g16), (loss32, g32) = tier[True], tier[False]
+    print(f"loss bf16 {loss16:.5f} f32 {loss32:.5f}", flush=True)
+    assert abs(loss32 - np.log(spec.vocab)) < 1.0 and abs(loss16 - loss32) <= 1e-3 * abs(loss32)
+    table = []
+    for name, want in g32.items():
+        if name == "blocks.0.mixer.vr_lambda":
+            assert not np.any(want) and not np.any(g16[name])  # block 0 blends with itself: no gradient
+            continue
+        scale = float(np.linalg.norm(want.astype(np.float64)))
+        assert scale > 0, name
+        diff = g16[name].astype(np.float64) - want
+        table.append((float(np.linalg.norm(diff)) / scale, float(np.max(np.abs(diff)) / np.max(np.abs(want))), name,
+                      want.size))
+    table.sort(reverse=True)
+    for row in table[:6]:
+        print("tier distance (normwise, worst element / largest, name, size)", row, flush=True)
+    # Every bf16 rounding of a block (ten stored activations each way) adds its share in quadrature:
+    # measured at this width the distance of every matrix gradient, first block or last, is about
+    # 0.9e-2 x sqrt(blocks) (1 block 0.7-1.1e-2, 2: 1.1-2.0, 4: 1.7-2.8, 8: 2.4-4.0, 12: 2.8-4.9,
+    # the q and k projections at the top of each range: their path runs through the softmax at
+    # scores of order one, which QK-norm gives from the first step). At 12 blocks: matrices at most
+    # 4.9e-2 normwise, the 64-element QK-norm weights 5.7e-2, one lambda of one element 1.3e-1.
+    for normwise, _, name, size in table:
+        assert normwise <= (6e-2 if size >= spec.n_embd * spec.n_head else 1.6e-1 if size == 1 else 8e-2), (name, normwise)
+    print("nanolab 124M: 16 x 1024", flush=True)
+    window = rng.integers(0, spec.vocab, (16, 1025)).astype(np.uint32)
+    ids, targets = window[:, :-1], window[:, 1:]
+    tr = NativeNanolabTrainer(be, spec, 16, 1024, bf16=True, adam_lr=1e-3, matrix_lr=0.02)
+    try:
+        tr.set_params(params)
+        base, grads = tr.loss_and_grads(ids, targets)
+        # two micro-batches at half weight add up to the whole one
+        tr._micro(ids, targets, 0.5, 0.5, True)
+        tr._micro(ids, targets, 0.5, 0.5, False)
+        twice = tr.grads()
+        for name, g in grads.items():
+            scale = float(np.max(np.abs(g)))
+            assert float(np.max(np.abs(twice[name] - g))) <= 1e-6 * scale, name
+        # along the gradient
+        sq = sum(float(np.sum(g.astype(np.float64) ** 2)) for g in grads.values())
+        eps = 0.02 / sq
+        losses = []
+        for sign in (1.0, -1.0):
+            tr.set_params({n: params[n] + np.float32(sign * eps) * grads[n].reshape(params[n].shape) for n in params})
+            losses.append(tr.loss_and_grads(ids, targets)[0])
+        measured = losses[0] - losses[1]
+        print(f"loss {base:.5f}; along the gradient: measured {measured:.5f}, predicted {2 * eps * sq:.5f}", flush=True)
+        assert losses[1] < base < losses[0]
+        assert abs(measured - 2 * eps * sq) <= 0.1 * 2 * eps * sq, (measured, 2 * eps * sq)
+        # the hybrid step
+        tr.set_params(params)
+        curve = [tr.run([(ids, targets)], 1.0).loss for _ in range(6)]
+        print("curve", curve, flush=True)
+        assert abs(curve[0] - base) <= 1e-6 * base and curve[-1] < curve[0] - 0.1 and tr.step == 6, curve
+        after = tr.download_params()
+        assert np.array_equal(after["blocks.0.mixer.vr_lambda"], params["blocks.0.mixer.vr_lambda"])
+        assert all(np.all(np.isfinite(a)) for a in after.values())
     finally:
         tr.close()
