@@ -237,6 +237,17 @@ __global__ __launch_bounds__(CE_THREADS) void ce_tile_grad_kernel(const TL* __re
 // ce_tile_grad_kernel; the row sum is formed over 1024 partial sums instead of 256, so it agrees
 // with theirs to rounding, not to the bit.
 constexpr int CE_FUSED_THREADS = 1024;
+// max / min of three in one instruction (NaNs are skipped, as by fmaxf / fminf).
+__device__ __forceinline__ float ce_max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+__device__ __forceinline__ float ce_min3(float a, float b, float c) {
+  float r;
+  asm("v_min3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
 __device__ __forceinline__ float fused_block_max(float v, float* red) {
   v = wave_max(v);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -298,26 +309,61 @@ __global__ __launch_bounds__(CE_FUSED_THREADS, 8) void ce_row_fused_kernel(T* __
   float mx = -INFINITY, sum = 0.0f;
   bool bad = false;
   __syncthreads();  // `picked` is initialised before its owner overwrites it
+  if constexpr (sizeof(T) == 2) {
+    // bf16 logits: a pack's largest and smallest value through three-input max / min, the
+    // exponent as one fma (v log2e - max log2e) into the hardware exp2, and the comparison with
+    // the target column only in the one pack that holds it. A NaN or an infinity among the logits
+    // shows in the smallest / largest value, in the sum or in the picked logit.
+    constexpr float LOG2E = 1.4426950408889634f;
+    float mn = INFINITY, mine = 0.0f;
 #pragma unroll
-  for (int k = 0; k < MAXV; ++k) {
-    const unsigned int c = (threadIdx.x + k * CE_FUSED_THREADS) * VEC;
-    if (c < ncols) {
-      float v[VEC];
-      unpack(q[k], v);
-      float top = v[0];
+    for (int k = 0; k < MAXV; ++k) {
+      const unsigned int c = (threadIdx.x + k * CE_FUSED_THREADS) * VEC;
+      if (c < ncols) {
+        float v[VEC];
+        unpack(q[k], v);
+        const float top = fmaxf(ce_max3(ce_max3(ce_max3(v[0], v[1], v[2]), v[3], v[4]), v[5], v[6]), v[7]);
+        mn = fminf(ce_min3(ce_min3(ce_min3(mn, v[0], v[1]), v[2], v[3]), v[4], v[5]), fminf(v[6], v[7]));
+        if (top > mx) {
+          sum *= __builtin_amdgcn_exp2f((mx - top) * LOG2E);
+          mx = top;
+        }
+        const float shift = -mx * LOG2E;
+        if (target - c >= static_cast<unsigned int>(VEC)) {
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        bad |= !dev_finite(v[j]);
-        top = fmaxf(top, v[j]);
+          for (int j = 0; j < VEC; ++j) sum += __builtin_amdgcn_exp2f(fmaf(v[j], LOG2E, shift));
+        } else {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) {
+            if (c + j != target) sum += __builtin_amdgcn_exp2f(fmaf(v[j], LOG2E, shift));
+            else picked = mine = v[j];
+          }
+        }
       }
-      if (top > mx) {
-        sum *= ce_exp<T>(mx - top);
-        mx = top;
-      }
+    }
+    bad = !(mn > -INFINITY && mx < INFINITY && sum == sum && dev_finite(mine));
+  } else {
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        if (c + j != target) sum += ce_exp<T>(v[j] - mx);
-        else picked = v[j];
+    for (int k = 0; k < MAXV; ++k) {
+      const unsigned int c = (threadIdx.x + k * CE_FUSED_THREADS) * VEC;
+      if (c < ncols) {
+        float v[VEC];
+        unpack(q[k], v);
+        float top = v[0];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          bad |= !dev_finite(v[j]);
+          top = fmaxf(top, v[j]);
+        }
+        if (top > mx) {
+          sum *= ce_exp<T>(mx - top);
+          mx = top;
+        }
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          if (c + j != target) sum += ce_exp<T>(v[j] - mx);
+          else picked = v[j];
+        }
       }
     }
   }
@@ -352,9 +398,31 @@ __global__ __launch_bounds__(CE_FUSED_THREADS, 8) void ce_row_fused_kernel(T* __
     if (c < ncols) {
       float v[VEC], out[VEC];
       unpack(q[k], v);
+      if constexpr (sizeof(T) == 2) {
+        constexpr float LOG2E = 1.4426950408889634f;
+        const float shift = -m * LOG2E;
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) out[j] = (c + j == target) ? target_grad : ce_exp<T>(v[j] - m) * scale;
-      ce_store<T, VEC>(r, c, out);
+        for (int j = 0; j < VEC; ++j) out[j] = __builtin_amdgcn_exp2f(fmaf(v[j], LOG2E, shift)) * scale;
+        if (target - c < static_cast<unsigned int>(VEC)) {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j)
+            if (c + j == target) out[j] = target_grad;
+        }
+        // Finite values (a non-finite logit has raised the fault): the conversion instruction
+        // rounds to nearest even as dev_f32_to_bf16_bits does.
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        typedef float floatx2 __attribute__((ext_vector_type(2)));
+        uint4 w;
+        w.x = __builtin_bit_cast(unsigned int, __builtin_convertvector(floatx2{out[0], out[1]}, bf16x2));
+        w.y = __builtin_bit_cast(unsigned int, __builtin_convertvector(floatx2{out[2], out[3]}, bf16x2));
+        w.z = __builtin_bit_cast(unsigned int, __builtin_convertvector(floatx2{out[4], out[5]}, bf16x2));
+        w.w = __builtin_bit_cast(unsigned int, __builtin_convertvector(floatx2{out[6], out[7]}, bf16x2));
+        *reinterpret_cast<uint4*>(r + c) = w;
+      } else {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) out[j] = (c + j == target) ? target_grad : ce_exp<T>(v[j] - m) * scale;
+        ce_store<T, VEC>(r, c, out);
+      }
     }
   }
 }
@@ -601,14 +669,24 @@ int32_t omx_linear_cross_entropy_mean(omx_ctx* ctx, const void* x, const void* w
         dim3 grid(static_cast<unsigned>(nr)), block(CE_FUSED_THREADS);
         // One read of the logits tile and one write of the gradient over it.
         OmxKernelTimer timer(ctx, OMX_K_CE, 2.0 * static_cast<double>(nr) * static_cast<double>(nc) * esz);
-        if (operand_dtype == OMX_F32)
-          omx_launch_timed(ctx, ce_row_fused_kernel<float, CE_FUSED_PACKS>, grid, block, 0, timer.start(), timer.stop(),
-                           static_cast<float*>(tile), nc, r0, static_cast<unsigned>(nc), tg, has_ignore, ignore_index,
-                           s.st, s.valid, ctx->fault, tag);
-        else
-          omx_launch_timed(ctx, ce_row_fused_kernel<unsigned short, CE_FUSED_PACKS>, grid, block, 0, timer.start(),
-                           timer.stop(), static_cast<unsigned short*>(tile), nc, r0, static_cast<unsigned>(nc), tg,
-                           has_ignore, ignore_index, s.st, s.valid, ctx->fault, tag);
+        // As many 16-byte packs per thread as the row needs (fewer registers for shorter rows).
+        const uint64_t packs = (nc * esz / 16 + CE_FUSED_THREADS - 1) / CE_FUSED_THREADS;
+#define CE_FUSED(T_, P_)                                                                                          \
+  omx_launch_timed(ctx, ce_row_fused_kernel<T_, P_>, grid, block, 0, timer.start(), timer.stop(),                 \
+                   static_cast<T_*>(tile), nc, r0, static_cast<unsigned>(nc), tg, has_ignore, ignore_index, s.st, \
+                   s.valid, ctx->fault, tag)
+#define CE_FUSED_P(T_)                              \
+  do {                                              \
+    if (packs <= 2) CE_FUSED(T_, 2);                \
+    else if (packs <= 4) CE_FUSED(T_, 4);           \
+    else if (packs <= 6) CE_FUSED(T_, 6);           \
+    else if (packs <= 7) CE_FUSED(T_, 7);           \
+    else CE_FUSED(T_, CE_FUSED_PACKS);              \
+  } while (0)
+        if (operand_dtype == OMX_F32) CE_FUSED_P(float);
+        else CE_FUSED_P(unsigned short);
+#undef CE_FUSED_P
+#undef CE_FUSED
         OMX_LAUNCH_CHECK(ctx, "ce_row_fused_kernel");
         continue;
       }

@@ -176,6 +176,8 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
 // out[c] = sum over b < blocks of partial[b * dim + c], added in a fixed order.
 // `scratch` (OMX_COLUMN_SUM_GROUPS * dim floats, may be null) lets a tall `partial` be added in two stages.
 constexpr int OMX_COLUMN_SUM_GROUPS = 32;
+// Up to this many rows a tall sum is one launch of 1024-thread workgroups.
+constexpr int OMX_COLUMN_SUM_WIDE_ROWS = 1024;
 int32_t omx_column_sum(omx_ctx* ctx, const float* partial, float* out, uint64_t blocks, uint64_t dim,
                        unsigned long long tag, float* scratch = nullptr, hipEvent_t stop = nullptr);
 // RMSNorm with 16-byte accesses for row widths 256..2048 (rmsvec.hip). `add` (forward) and

@@ -74,49 +74,121 @@ __global__ __launch_bounds__(RV_THREADS) void rms_fwd_vec_kernel(const TX* __res
   if (bad) dev_raise_fault(fault, tag);
 }
 
+// Four elements as they sit in memory: the row waits in registers in this form between the passes
+// (a bf16 operand at half the registers of its f32 values).
+template <typename T>
+struct Raw4 {
+  float4 q;
+  __device__ __forceinline__ void load(const T* p) { q = *reinterpret_cast<const float4*>(p); }
+  __device__ __forceinline__ void clear() { q = make_float4(0.0f, 0.0f, 0.0f, 0.0f); }
+  __device__ __forceinline__ void get(float (&v)[4]) const { v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w; }
+};
+template <>
+struct Raw4<unsigned short> {
+  uint2 q;
+  __device__ __forceinline__ void load(const unsigned short* p) { q = *reinterpret_cast<const uint2*>(p); }
+  __device__ __forceinline__ void clear() { q = make_uint2(0u, 0u); }
+  __device__ __forceinline__ void get(float (&v)[4]) const {
+    v[0] = __uint_as_float(q.x << 16); v[1] = __uint_as_float(q.x & 0xffff0000u);
+    v[2] = __uint_as_float(q.y << 16); v[3] = __uint_as_float(q.y & 0xffff0000u);
+  }
+};
+
+// Stores four values; a bf16 destination is rounded by the conversion instruction (round to nearest
+// even, as dev_f32_to_bf16_bits; the two differ in a NaN's payload only, and a kernel that stores
+// through this raises the fault for any non-finite value it writes).
+template <typename T>
+__device__ __forceinline__ void store4_rounded(T* p, const float (&v)[4]) {
+  if constexpr (sizeof(T) == 4) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  } else {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    typedef float floatx2 __attribute__((ext_vector_type(2)));
+    uint2 q;
+    q.x = __builtin_bit_cast(unsigned int, __builtin_convertvector(floatx2{v[0], v[1]}, bf16x2));
+    q.y = __builtin_bit_cast(unsigned int, __builtin_convertvector(floatx2{v[2], v[3]}, bf16x2));
+    *reinterpret_cast<uint2*>(p) = q;
+  }
+}
+
 // gx = rms_norm_backward(x, w, gy) (+ add_in), optionally also stored as bf16;
 // per-block partial column sums of gy * xhat for the weight gradient.
-template <typename TX, typename TG, typename TO, int NCH>
+// Row bases are wave-uniform (scalar registers) and lane offsets 32 bits wide; all of a row's loads
+// (the gradient to add included) are issued before the first reduction. FULL: dim == 256 NCH, no
+// column guards. WIDE (rows above 1024 columns): the weight row is read again in each pass instead
+// of waiting in registers and the lane's column sums wait in LDS, so that enough waves fit a SIMD
+// to keep the loads in flight.
+template <typename TX, typename TG, typename TO, int NCH, bool WIDE, bool FULL>
 __global__ __launch_bounds__(RV_THREADS) void rms_bwd_vec_kernel(
     const TX* __restrict__ x, const float* __restrict__ w, const TG* __restrict__ gy, const float* __restrict__ add_in,
     TO* __restrict__ gx, unsigned short* __restrict__ gx16, float* __restrict__ partial, size_t rows, int dim,
     float eps, int rows_per_block, OmxFaultWord* fault, unsigned long long tag) {
   extern __shared__ float lds[];  // [4][dim]
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const unsigned lane = threadIdx.x & 63;
+  const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const unsigned udim = FULL ? NCH * 256u : static_cast<unsigned>(dim);
   const float inv_dim = 1.0f / static_cast<float>(dim);
-  float wv[NCH][4], accw[NCH][4];
+  constexpr int NW = WIDE ? 1 : NCH;
+  float wv[NW][4], accw[NW][4];
+  float* mine = lds + static_cast<size_t>(wave) * udim;
 #pragma unroll
   for (int j = 0; j < NCH; ++j) {
-    const int c = j * 256 + lane * 4;
+    const unsigned c = j * 256 + lane * 4;
+    if constexpr (WIDE) {
+      if (FULL || c < udim) *reinterpret_cast<float4*>(mine + c) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    } else {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      wv[j][e] = 0.0f;
-      accw[j][e] = 0.0f;
+      for (int e = 0; e < 4; ++e) {
+        wv[j][e] = 0.0f;
+        accw[j][e] = 0.0f;
+      }
+      if (FULL || c < udim) dev_load4<float>(w, c, wv[j]);
     }
-    if (c < dim) dev_load4<float>(w, c, wv[j]);
   }
   bool bad = false;
   const size_t first = static_cast<size_t>(blockIdx.x) * rows_per_block;
   const size_t last = min(rows, first + rows_per_block);
   for (size_t row = first + wave; row < last; row += 4) {
-    const size_t base = row * dim;
-    float xv[NCH][4], gv[NCH][4];
+    const size_t base = row * udim;
+    const TX* xr = x + base;
+    const TG* gr = gy + base;
+    // The weight row's address passes through an opaque scalar so its loads stay inside the loop.
+    size_t wofs = 0;
+    if constexpr (WIDE) asm volatile("" : "+s"(wofs));
+    const float* wr = w + wofs;
+    Raw4<TX> xq[NCH];
+    Raw4<TG> gq[NCH];
+    Raw4<float> aq[NCH];
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+      const unsigned c = j * 256 + lane * 4;
+      if (FULL || c < udim) {
+        xq[j].load(xr + c);
+        gq[j].load(gr + c);
+      } else {
+        xq[j].clear();
+        gq[j].clear();
+      }
+    }
+    if (add_in) {
+      const float* ar = add_in + base;
+#pragma unroll
+      for (int j = 0; j < NCH; ++j) {
+        const unsigned c = j * 256 + lane * 4;
+        if (FULL || c < udim) aq[j].load(ar + c);
+        else aq[j].clear();
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < NCH; ++j) aq[j].clear();
+    }
     float ss = 0.0f;
 #pragma unroll
     for (int j = 0; j < NCH; ++j) {
-      const int c = j * 256 + lane * 4;
-      if (c < dim) {
-        dev_load4<TX>(x, base + c, xv[j]);
-        dev_load4<TG>(gy, base + c, gv[j]);
-      } else {
+      float xv[4];
+      xq[j].get(xv);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          xv[j][e] = 0.0f;
-          gv[j][e] = 0.0f;
-        }
-      }
-#pragma unroll
-      for (int e = 0; e < 4; ++e) ss += xv[j][e] * xv[j][e];
+      for (int e = 0; e < 4; ++e) ss += xv[e] * xv[e];
     }
     ss = wave_sum(ss);
     const float denom = ss * inv_dim + eps;
@@ -124,44 +196,70 @@ __global__ __launch_bounds__(RV_THREADS) void rms_bwd_vec_kernel(
     bad |= !(dev_finite(denom) && denom > 0.0f && dev_finite(rstd));
     float dot = 0.0f;
 #pragma unroll
-    for (int j = 0; j < NCH; ++j)
+    for (int j = 0; j < NCH; ++j) {
+      const unsigned c = j * 256 + lane * 4;
+      float xv[4], gv[4], ww[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+      xq[j].get(xv);
+      gq[j].get(gv);
+      if constexpr (WIDE) {
+        if (FULL || c < udim) dev_load4<float>(wr, c, ww);
+      }
 #pragma unroll
-      for (int e = 0; e < 4; ++e) dot += (gv[j][e] * wv[j][e]) * (xv[j][e] * rstd);
+      for (int e = 0; e < 4; ++e) dot += (gv[e] * (WIDE ? ww[e] : wv[WIDE ? 0 : j][e])) * (xv[e] * rstd);
+    }
     dot = wave_sum(dot);
     const float mean = dot * inv_dim;
+    TO* outr = gx + base;
+    unsigned short* out16r = gx16 + (gx16 ? base : 0);
 #pragma unroll
     for (int j = 0; j < NCH; ++j) {
-      const int c = j * 256 + lane * 4;
-      float out[4];
+      const unsigned c = j * 256 + lane * 4;
+      float xv[4], gv[4], ww[4] = {0.0f, 0.0f, 0.0f, 0.0f}, out[4], aw[4];
+      xq[j].get(xv);
+      gq[j].get(gv);
+      if constexpr (WIDE) {
+        if (FULL || c < udim) dev_load4<float>(wr, c, ww);
+      }
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const float xhat = xv[j][e] * rstd;
-        out[e] = (gv[j][e] * wv[j][e] - xhat * mean) * rstd;
-        accw[j][e] += gv[j][e] * xhat;
+        const float xhat = xv[e] * rstd;
+        out[e] = (gv[e] * (WIDE ? ww[e] : wv[WIDE ? 0 : j][e]) - xhat * mean) * rstd;
+        aw[e] = gv[e] * xhat;
       }
-      if (c < dim) {
-        if (add_in) {
-          float av[4];
-          dev_load4<float>(add_in, base + c, av);
+      if constexpr (!WIDE) {
 #pragma unroll
-          for (int e = 0; e < 4; ++e) out[e] = av[e] + out[e];
+        for (int e = 0; e < 4; ++e) accw[j][e] += aw[e];
+      }
+      if (add_in) {
+        float av[4];
+        aq[j].get(av);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) out[e] = av[e] + out[e];
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) bad |= !dev_finite(out[e]);
+      if (FULL || c < udim) {
+        if constexpr (WIDE) {
+          float4 a = *reinterpret_cast<const float4*>(mine + c);
+          a.x += aw[0]; a.y += aw[1]; a.z += aw[2]; a.w += aw[3];
+          *reinterpret_cast<float4*>(mine + c) = a;
         }
-#pragma unroll
-        for (int e = 0; e < 4; ++e) bad |= !dev_finite(out[e]);
-        dev_store4<TO>(gx, base + c, out);
-        if (gx16) dev_store4<unsigned short>(gx16, base + c, out);
+        store4_rounded<TO>(outr + c, out);
+        if (gx16) store4_rounded<unsigned short>(out16r + c, out);
       }
     }
   }
+  if constexpr (!WIDE) {
 #pragma unroll
-  for (int j = 0; j < NCH; ++j) {
-    const int c = j * 256 + lane * 4;
-    if (c < dim) dev_store4<float>(lds, static_cast<size_t>(wave) * dim + c, accw[j]);
+    for (int j = 0; j < NCH; ++j) {
+      const unsigned c = j * 256 + lane * 4;
+      if (FULL || c < udim) dev_store4<float>(mine, c, accw[j]);
+    }
   }
   __syncthreads();
-  for (int c = threadIdx.x; c < dim; c += RV_THREADS) {
-    float s = ((lds[c] + lds[dim + c]) + lds[2 * dim + c]) + lds[3 * dim + c];
-    partial[static_cast<size_t>(blockIdx.x) * dim + c] = s;
+  for (unsigned c = threadIdx.x; c < udim; c += RV_THREADS) {
+    float s = ((lds[c] + lds[udim + c]) + lds[2 * udim + c]) + lds[3 * udim + c];
+    partial[static_cast<size_t>(blockIdx.x) * udim + c] = s;
   }
   if (bad) dev_raise_fault(fault, tag);
 }
@@ -223,8 +321,10 @@ int32_t omx_rms_forward_vec(omx_ctx* ctx, const void* x, int32_t x_dtype, const 
 int32_t omx_rms_backward_vec(omx_ctx* ctx, const void* x, int32_t x_dtype, const float* w, const void* gy,
                              int32_t gy_dtype, const float* add_in, void* gx, int32_t gx_dtype, void* gx16, float* gw,
                              uint64_t rows, uint64_t dim, float eps, unsigned long long tag) {
-  // Two rows per wave: enough blocks in flight to hide the row's load latency.
-  const int rows_per_block = 8;
+  // The kernel's time does not depend on the rows a block takes between 2 and 16 per wave (the
+  // loads of a row are all in flight at once); fewer blocks leave fewer partial rows to add.
+  int rows_per_block = 8;
+  while (rows_per_block < (dim > 1024 ? 16 : 32) && rows / rows_per_block > 512) rows_per_block *= 2;
   const uint64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
   void* ws = nullptr;
   int32_t rc = omx_workspace(ctx, (blocks + OMX_COLUMN_SUM_GROUPS) * dim * sizeof(float), &ws);
@@ -234,6 +334,7 @@ int32_t omx_rms_backward_vec(omx_ctx* ctx, const void* x, int32_t x_dtype, const
   dim3 grid(static_cast<unsigned>(blocks)), block(RV_THREADS);
   const size_t smem = 4 * dim * sizeof(float);
   const int nch = static_cast<int>((dim + 255) / 256);
+  const bool full = dim == static_cast<uint64_t>(nch) * 256;
   typedef unsigned short h16;
   // Bytes: the row and its gradient read (and the gradient added in), the input gradient written
   // (and its bf16 copy); the weight gradient's partial sums are the kernels' own traffic.
@@ -242,10 +343,18 @@ int32_t omx_rms_backward_vec(omx_ctx* ctx, const void* x, int32_t x_dtype, const
                        static_cast<double>(rows) * static_cast<double>(dim) *
                            (width(x_dtype) + width(gy_dtype) + (add_in ? 4.0 : 0.0) + width(gx_dtype) + (gx16 ? 2.0 : 0.0)));
 #define RV_BWD(TX, TG, TO, N)                                                                                        \
-  omx_launch_timed(ctx, rms_bwd_vec_kernel<TX, TG, TO, N>, grid, block, smem, timer.start(), nullptr,                \
-                   static_cast<const TX*>(x), w, static_cast<const TG*>(gy), add_in, static_cast<TO*>(gx),           \
-                   static_cast<h16*>(gx16), partial, static_cast<size_t>(rows), static_cast<int>(dim), eps,          \
-                   rows_per_block, ctx->fault, tag)
+  do {                                                                                                               \
+    if (full)                                                                                                        \
+      omx_launch_timed(ctx, rms_bwd_vec_kernel<TX, TG, TO, N, (N > 4), true>, grid, block, smem, timer.start(),      \
+                       nullptr, static_cast<const TX*>(x), w, static_cast<const TG*>(gy), add_in,                    \
+                       static_cast<TO*>(gx), static_cast<h16*>(gx16), partial, static_cast<size_t>(rows),            \
+                       static_cast<int>(dim), eps, rows_per_block, ctx->fault, tag);                                 \
+    else                                                                                                             \
+      omx_launch_timed(ctx, rms_bwd_vec_kernel<TX, TG, TO, N, (N > 4), false>, grid, block, smem, timer.start(),     \
+                       nullptr, static_cast<const TX*>(x), w, static_cast<const TG*>(gy), add_in,                    \
+                       static_cast<TO*>(gx), static_cast<h16*>(gx16), partial, static_cast<size_t>(rows),            \
+                       static_cast<int>(dim), eps, rows_per_block, ctx->fault, tag);                                 \
+  } while (0)
 #define RV_BWD_N(TX, TG, TO)      \
   switch (nch) {                  \
     case 1: RV_BWD(TX, TG, TO, 1); break; \

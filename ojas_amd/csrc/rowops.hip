@@ -137,6 +137,37 @@ __global__ __launch_bounds__(256) void column_sum_kernel(const float* __restrict
   }
 }
 
+// The same for a few hundred rows in one launch: 16 row groups of 64 columns (1024 threads), four
+// loads in flight per thread, the groups added in a fixed order.
+__global__ __launch_bounds__(1024) void column_sum_wide_kernel(const float* __restrict__ partial,
+                                                               float* __restrict__ out, int blocks, int dim,
+                                                               OmxFaultWord* fault, unsigned long long tag) {
+  __shared__ float red[16][64];
+  const int lane = threadIdx.x & 63, group = threadIdx.x >> 6;
+  const int c = blockIdx.x * 64 + lane;
+  float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+  if (c < dim) {
+    const float* col = partial + c;
+    int b = group;
+    for (; b + 48 < blocks; b += 64) {
+      s0 += col[static_cast<size_t>(b) * dim];
+      s1 += col[static_cast<size_t>(b + 16) * dim];
+      s2 += col[static_cast<size_t>(b + 32) * dim];
+      s3 += col[static_cast<size_t>(b + 48) * dim];
+    }
+    for (; b < blocks; b += 16) s0 += col[static_cast<size_t>(b) * dim];
+  }
+  red[group][lane] = (s0 + s1) + (s2 + s3);
+  __syncthreads();
+  if (group == 0 && c < dim) {
+    float total = 0.0f;
+#pragma unroll
+    for (int g = 0; g < 16; ++g) total += red[g][lane];
+    out[c] = total;
+    if (!dev_finite(total)) dev_raise_fault(fault, tag);
+  }
+}
+
 // Stage 1 of a tall column sum: block (x, g) adds rows [g * per_group, (g + 1) * per_group) of its
 // 64 columns, four row groups in parallel, then a fixed four-way sum.
 __global__ __launch_bounds__(256) void column_sum_groups_kernel(const float* __restrict__ partial,
@@ -556,6 +587,12 @@ bool finite_host(float v) { return v == v && v != INFINITY && v != -INFINITY; }
 int32_t omx_column_sum(omx_ctx* ctx, const float* partial, float* out, uint64_t blocks, uint64_t dim,
                        unsigned long long tag, float* scratch, hipEvent_t stop) {
   const unsigned col_blocks = static_cast<unsigned>((dim + 63) / 64);
+  if (blocks > 4 * OMX_COLUMN_SUM_GROUPS && blocks <= OMX_COLUMN_SUM_WIDE_ROWS) {
+    omx_launch_timed(ctx, column_sum_wide_kernel, dim3(col_blocks), dim3(1024), 0, nullptr, stop, partial, out,
+                     static_cast<int>(blocks), static_cast<int>(dim), ctx->fault, tag);
+    OMX_LAUNCH_CHECK(ctx, "column_sum_wide_kernel");
+    return OMX_OK;
+  }
   if (scratch && blocks > 4 * OMX_COLUMN_SUM_GROUPS) {
     // Stage 1: group g adds its contiguous share of the rows into scratch[g]; stage 2 adds the groups.
     const int per_group = static_cast<int>((blocks + OMX_COLUMN_SUM_GROUPS - 1) / OMX_COLUMN_SUM_GROUPS);

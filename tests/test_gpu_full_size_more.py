@@ -323,9 +323,17 @@ def test_nanolab_124m_step_at_full_size(be):
     # 0.9e-2 x sqrt(blocks) (1 block 0.7-1.1e-2, 2: 1.1-2.0, 4: 1.7-2.8, 8: 2.4-4.0, 12: 2.8-4.9,
     # the q and k projections at the top of each range: their path runs through the softmax at
     # scores of order one, which QK-norm gives from the first step). At 12 blocks: matrices at most
-    # 4.9e-2 normwise, the 64-element QK-norm weights 5.7e-2, one lambda of one element 1.3e-1.
+    # 4.9e-2 normwise, the 64-element QK-norm weights 5.7e-2. A lambda's gradient is one number, a
+    # sum over every value element with both signs; one of them alone reads 6e-2 to 1.8e-1 from run
+    # to run of the kernels' summation orders, so the eleven are held as one vector.
     for normwise, _, name, size in table:
-        assert normwise <= (6e-2 if size >= spec.n_embd * spec.n_head else 1.6e-1 if size == 1 else 8e-2), (name, normwise)
+        if size > 1:
+            assert normwise <= (6e-2 if size >= spec.n_embd * spec.n_head else 8e-2), (name, normwise)
+    lam = [n for n in g32 if n.endswith("vr_lambda") and n != "blocks.0.mixer.vr_lambda"]
+    want = np.array([g32[n][0] for n in lam], np.float64)
+    got = np.array([g16[n][0] for n in lam], np.float64)
+    print("lambda gradients: distance", float(np.linalg.norm(got - want) / np.linalg.norm(want)), flush=True)
+    assert np.linalg.norm(got - want) <= 8e-2 * np.linalg.norm(want), (got, want)
     print("nanolab 124M: 16 x 1024", flush=True)
     window = rng.integers(0, spec.vocab, (16, 1025)).astype(np.uint32)
     ids, targets = window[:, :-1], window[:, 1:]

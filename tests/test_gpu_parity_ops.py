@@ -294,6 +294,31 @@ def test_linear_cross_entropy_one_read_kernel_agrees_with_the_two_kernels(be, bf
     close(got[1][2], ogw, tol, "one-read gw")
 
 
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("poison", ["nan", "+inf", "-inf"])
+@pytest.mark.parametrize("as_target", [False, True])
+def test_linear_cross_entropy_one_read_kernel_reports_a_non_finite_logit(be, bf16, poison, as_target):
+    """One vocabulary column of NaN, +inf or -inf logits (a poisoned weight row), either never the
+    target (it enters the row sums) or every row's target (it is only ever the picked logit): the
+    one-read kernel raises NonFinite either way, reported at the next sync."""
+    from ojas_amd.backend import BF16, NON_FINITE, OjasError
+
+    print(f"linear_ce one-read non-finite bf16={bf16} {poison} target={as_target}", flush=True)
+    rows, dim, vocab, col = 24, 64, 520, 77
+    r = orc.SplitMix64(77)
+    x = orc.round_bf16(np.abs(r.vec(rows * dim, 1.0)) + 0.5).reshape(rows, dim)
+    w = orc.round_bf16(r.vec(vocab * dim, 0.3)).reshape(vocab, dim)
+    w[col] = {"nan": np.nan, "+inf": 3e38, "-inf": -3e38}[poison]
+    targets = np.full(rows, col if as_target else 5, np.uint32)
+    up = (lambda a: be.upload(a, BF16)) if bf16 else be.upload
+    be.sync()
+    be.linear_cross_entropy_mean(up(x), up(orc.round_bf16(w)), be.upload(targets), None, (rows, vocab))
+    with pytest.raises(OjasError) as e:
+        be.sync()
+    assert e.value.code == NON_FINITE and "linear_cross_entropy" in e.value.detail, e.value.detail
+    be.sync()
+
+
 def be_f32(a):
     """Widens a downloaded bf16 bit array; f32 arrays pass through."""
     return (a.astype(np.uint32) << 16).view(np.float32) if a.dtype == np.uint16 else a
