@@ -59,6 +59,12 @@ struct onano {
   void* p16 = nullptr;
   uint32_t *ids = nullptr, *targets = nullptr;
   float *loss = nullptr, *loss_acc = nullptr;
+  // omx_adamw_step_bounded's flag word (the word after the accumulated loss, so one readback
+  // fetches both), whether it has covered AdamW's range since that was last written from outside,
+  // and the flag as the last step's readback saw it.
+  void* unbounded = nullptr;
+  bool tracked = false;
+  uint32_t flag_seen = 1;
   float *cos_t = nullptr, *sin_t = nullptr;
 
   struct Layer {
@@ -474,6 +480,7 @@ int32_t onano_create(omx_ctx* ctx, const onano_config* config, onano** out) {
     CREATE_TRY(omx_fill_zero(ctx, block, 256));
     t->loss = static_cast<float*>(block);
     t->loss_acc = t->loss + 16;
+    t->unbounded = t->loss_acc + 1;
   }
   {
     // Rope::rows (ojas-model/src/block.rs:31-71): angles in f64, one rounding to f32, both halves
@@ -622,6 +629,7 @@ int32_t onano_set_steps(onano* t, uint64_t steps) {
 int32_t onano_set_param(onano* t, uint64_t index, const float* host) {
   if (!t || index >= t->slots.size() || !host) return OMX_SHAPE;
   const Slot& s = t->slots[index];
+  t->tracked = false;
   TRY(omx_upload(t->ctx, t->p32, s.offset * 4, host, s.len * 4));
   if (t->p16) TRY(omx_to_bf16(t->ctx, t->p32 + s.offset, static_cast<uint16_t*>(t->p16) + s.offset, s.len));
   return OMX_OK;
@@ -644,6 +652,7 @@ int32_t onano_get_state(onano* t, uint64_t index, uint32_t slot, float* host) {
 int32_t onano_set_state(onano* t, uint64_t index, uint32_t slot, const float* host) {
   if (!t || index >= t->slots.size() || !host || slot > 1) return OMX_SHAPE;
   const Slot& s = t->slots[index];
+  t->tracked = false;
   return omx_upload(t->ctx, slot == 0 ? t->m1 : t->m2, s.offset * 4, host, s.len * 4);
 }
 
@@ -667,6 +676,7 @@ int32_t onano_init(onano* t, uint64_t seed) {
   TRY(omx_fill_zero(t->ctx, t->m1, t->P * 4));
   TRY(omx_fill_zero(t->ctx, t->m2, t->P * 4));
   t->steps = 0;
+  t->tracked = false;
   return omx_sync(t->ctx);
 }
 
@@ -699,8 +709,16 @@ int32_t onano_apply(onano* t, const omx_muon_config* muon, const omx_adamw_confi
   // padding and block 0's vr_lambda hold zeros and add nothing to it.
   TRY(omx_clip_grad_norm(t->ctx, grads, lens, 1, grad_clip > 0.0f ? grad_clip : INFINITY, &norm));
   uint16_t* mirror = static_cast<uint16_t*>(t->p16);
-  // AdamW: the table and every vector sit side by side at the arena's start.
-  TRY(omx_adamw_step(t->ctx, t->p32, t->acc, t->m1, t->m2, t->adam_end, t->steps, adamw, mirror));
+  // AdamW: the table and every vector sit side by side at the arena's start. Its checking pass is
+  // skipped when nothing in its range can overflow: the flag of the previous steps, which came back
+  // with the last step's loss, vouches for the parameters and moments, the gradient norm for the
+  // gradients. When they are not known to be bounded the flag starts afresh with this step.
+  const bool flag_clear = t->tracked && t->flag_seen == 0;
+  if (!flag_clear) TRY(omx_fill_zero(t->ctx, t->unbounded, 4));
+  const int32_t bounded = flag_clear && std::isfinite(norm) && norm < 0x1p60f;
+  t->tracked = false;  // until the readback below has seen this step through
+  TRY(omx_adamw_step_bounded(t->ctx, t->p32, t->acc, t->m1, t->m2, t->adam_end, t->steps, adamw, mirror, bounded,
+                             t->unbounded));
   const uint64_t count = t->slots.size();
   // Muon: matrices of one shape go through Newton-Schulz together.
   struct Group {
@@ -723,8 +741,14 @@ int32_t onano_apply(onano* t, const omx_muon_config* muon, const omx_adamw_confi
                                   grp.p.size(), kv.first.first, kv.first.second, muon));
   }
   // Sync point 2: the step's one readback (trainer.rs:1031-1046).
-  float l = 0.0f;
-  TRY(omx_read_scalar_f32(t->ctx, t->loss_acc, &l));
+  struct {
+    float loss;
+    uint32_t flag;
+  } back = {0.0f, 1u};
+  TRY(omx_download(t->ctx, &back, t->loss_acc, 0, sizeof(back)));
+  t->flag_seen = back.flag;
+  t->tracked = true;
+  const float l = back.loss;
   t->steps += 1;
   if (loss) *loss = l;
   if (grad_norm) *grad_norm = norm;
