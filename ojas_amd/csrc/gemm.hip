@@ -539,6 +539,8 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
   g.epi_tanh = epi ? epi->tanh_form : 0;
   g.aux_in = epi ? static_cast<const unsigned short*>(epi->aux_in) : nullptr;
   g.aux_out = epi ? static_cast<unsigned short*>(epi->aux_out) : nullptr;
+  g.epi_s1 = epi ? epi->s1 : 0.0f;
+  g.epi_s2 = epi ? epi->s2 : 0.0f;
   // The activation's side tensor is accessed with the output's vector width.
   if (epi && !((!epi->aux_in || aligned16(epi->aux_in)) && (!epi->aux_out || aligned16(epi->aux_out)))) g.c_vec = 0;
   g.fault = ctx->fault;
@@ -650,6 +652,11 @@ int32_t omx_set_option(omx_ctx* ctx, const char* name, int64_t value) {
   if (name && strcmp(name, "ce_fused") == 0) {
     if (value < 0 || value > 1) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: ce_fused takes 0..1");
     ctx->ce_fused = static_cast<int>(value);
+    return OMX_OK;
+  }
+  if (name && strcmp(name, "muon_fused_sums") == 0) {
+    if (value < 0 || value > 1) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: muon_fused_sums takes 0..1");
+    ctx->muon_fused_sums = static_cast<int>(value);
     return OMX_OK;
   }
   if (name && strcmp(name, "adamw_trust") == 0) {

@@ -18,6 +18,7 @@ struct GemmArgs {
   int epi, epi_tanh;             // OMX_EPI_* (bf16 output, no split)
   const unsigned short* aux_in;
   unsigned short* aux_out;
+  float epi_s1, epi_s2;  // OMX_EPI_AXPBY
   OmxFaultWord* fault;
   unsigned long long tag;
   // Strided batch: block (x, y) works on product y, whose operands start batch_* BYTES after
@@ -34,6 +35,9 @@ __device__ __forceinline__ void gemm_select_batch(GemmArgs& g, int product) {
     g.a = static_cast<const char*>(g.a) + y * g.batch_a;
     g.b = static_cast<const char*>(g.b) + y * g.batch_b;
     g.c = static_cast<char*>(g.c) + y * g.batch_c;
+    // aux tensors are bf16 like the output they accompany: the same byte stride.
+    if (g.aux_in) g.aux_in = reinterpret_cast<const unsigned short*>(reinterpret_cast<const char*>(g.aux_in) + y * g.batch_c);
+    if (g.aux_out) g.aux_out = reinterpret_cast<unsigned short*>(reinterpret_cast<char*>(g.aux_out) + y * g.batch_c);
   }
 }
 
@@ -97,6 +101,11 @@ __device__ __forceinline__ bool gemm_store4(const GemmArgs& g, int split, int gr
 
 // gemm_store4 with the optional activation of OmxGemmEpilogue applied first (bf16 outputs, no
 // split). Kept apart from the plain store so the plain epilogue loops stay small enough to unroll.
+// OMX_EPI_AXPBY on one element: `aux` as stored, `acc` the product's f32 accumulator.
+__device__ __forceinline__ float gemm_axpby(const GemmArgs& g, float aux, float acc) {
+  return dev_round_bf16(g.epi_s1 * aux) + dev_round_bf16(g.epi_s2 * dev_round_bf16(acc));
+}
+
 __device__ __forceinline__ bool gemm_store4_epi(const GemmArgs& g, int split, int grow, int gcol, float x0, float x1,
                                                 float x2, float x3) {
   bool bad = false;
@@ -125,7 +134,7 @@ __device__ __forceinline__ bool gemm_store4_epi(const GemmArgs& g, int split, in
         if (gcol + 2 < g.N) { ap[2] = dev_f32_to_bf16_bits(a2); bad |= !dev_finite(a2); }
         if (gcol + 3 < g.N) { ap[3] = dev_f32_to_bf16_bits(a3); bad |= !dev_finite(a3); }
       }
-    } else if (g.epi == OMX_EPI_GELU_BWD) {
+    } else if (g.epi == OMX_EPI_GELU_BWD || g.epi == OMX_EPI_AXPBY) {
       const unsigned short* ap = g.aux_in + off;
       float u0 = 0.0f, u1 = 0.0f, u2 = 0.0f, u3 = 0.0f;
       if (whole) {
@@ -140,10 +149,17 @@ __device__ __forceinline__ bool gemm_store4_epi(const GemmArgs& g, int split, in
         if (gcol + 2 < g.N) u2 = dev_bf16_bits_to_f32(ap[2]);
         if (gcol + 3 < g.N) u3 = dev_bf16_bits_to_f32(ap[3]);
       }
-      x0 = dev_round_bf16(x0) * (g.epi_tanh ? dev_gelu_tanh_grad_fast(u0) : dev_gelu_erf_grad_fast(u0));
-      x1 = dev_round_bf16(x1) * (g.epi_tanh ? dev_gelu_tanh_grad_fast(u1) : dev_gelu_erf_grad_fast(u1));
-      x2 = dev_round_bf16(x2) * (g.epi_tanh ? dev_gelu_tanh_grad_fast(u2) : dev_gelu_erf_grad_fast(u2));
-      x3 = dev_round_bf16(x3) * (g.epi_tanh ? dev_gelu_tanh_grad_fast(u3) : dev_gelu_erf_grad_fast(u3));
+      if (g.epi == OMX_EPI_AXPBY) {
+        x0 = gemm_axpby(g, u0, x0);
+        x1 = gemm_axpby(g, u1, x1);
+        x2 = gemm_axpby(g, u2, x2);
+        x3 = gemm_axpby(g, u3, x3);
+      } else {
+        x0 = dev_round_bf16(x0) * (g.epi_tanh ? dev_gelu_tanh_grad_fast(u0) : dev_gelu_erf_grad_fast(u0));
+        x1 = dev_round_bf16(x1) * (g.epi_tanh ? dev_gelu_tanh_grad_fast(u1) : dev_gelu_erf_grad_fast(u1));
+        x2 = dev_round_bf16(x2) * (g.epi_tanh ? dev_gelu_tanh_grad_fast(u2) : dev_gelu_erf_grad_fast(u2));
+        x3 = dev_round_bf16(x3) * (g.epi_tanh ? dev_gelu_tanh_grad_fast(u3) : dev_gelu_erf_grad_fast(u3));
+      }
     }
   }
   return gemm_store4(g, split, grow, gcol, x0, x1, x2, x3) || bad;
@@ -166,7 +182,7 @@ __device__ __forceinline__ bool gemm_epilogue_block(const GemmArgs& g, const flo
   for (int it = 0; it < ITERS; ++it) {
     const int c = lane + it * 64, row = c / PPR, piece = c % PPR;
     off[it] = static_cast<long>(grow0 + row) * g.ldc + gcol0 + piece * 4;
-    if constexpr (EPI == OMX_EPI_GELU_BWD) aux[it] = *reinterpret_cast<const uint2*>(g.aux_in + off[it]);
+    if constexpr (EPI != OMX_EPI_GELU_FWD) aux[it] = *reinterpret_cast<const uint2*>(g.aux_in + off[it]);
   }
   auto pack = [](float a, float b) {
     return static_cast<unsigned int>(dev_f32_to_bf16_bits(a)) | (static_cast<unsigned int>(dev_f32_to_bf16_bits(b)) << 16);
@@ -191,7 +207,8 @@ __device__ __forceinline__ bool gemm_epilogue_block(const GemmArgs& g, const flo
                           __uint_as_float(aux[it].y << 16), __uint_as_float(aux[it].y & 0xffff0000u)};
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        x[e] = dev_round_bf16(x[e]) * (TANH ? dev_gelu_tanh_grad_fast(u[e]) : dev_gelu_erf_grad_fast(u[e]));
+        if constexpr (EPI == OMX_EPI_AXPBY) x[e] = gemm_axpby(g, u[e], x[e]);
+        else x[e] = dev_round_bf16(x[e]) * (TANH ? dev_gelu_tanh_grad_fast(u[e]) : dev_gelu_erf_grad_fast(u[e]));
         bad |= !dev_finite(x[e]);
       }
       *reinterpret_cast<uint2*>(cbase + off[it]) = make_uint2(pack(x[0], x[1]), pack(x[2], x[3]));

@@ -237,6 +237,8 @@ gemm_dma_kernel(GemmArgs g) {
         if (g.epi == OMX_EPI_GELU_FWD) {
           bad |= g.epi_tanh ? gemm_epilogue_block<OMX_EPI_GELU_FWD, true, PPR>(g, cs, CPW, grow0, gcol0, lane)
                             : gemm_epilogue_block<OMX_EPI_GELU_FWD, false, PPR>(g, cs, CPW, grow0, gcol0, lane);
+        } else if (g.epi == OMX_EPI_AXPBY) {
+          bad |= gemm_epilogue_block<OMX_EPI_AXPBY, false, PPR>(g, cs, CPW, grow0, gcol0, lane);
         } else {
           bad |= g.epi_tanh ? gemm_epilogue_block<OMX_EPI_GELU_BWD, true, PPR>(g, cs, CPW, grow0, gcol0, lane)
                             : gemm_epilogue_block<OMX_EPI_GELU_BWD, false, PPR>(g, cs, CPW, grow0, gcol0, lane);
@@ -348,6 +350,10 @@ __device__ __forceinline__ bool store_block_direct(const GemmArgs& g, char* cbas
         const float u0 = __uint_as_float(w << 16), u1 = __uint_as_float(w & 0xffff0000u);
         x0 = dev_round_bf16(x0) * (g.epi_tanh ? dev_gelu_tanh_grad_fast(u0) : dev_gelu_erf_grad_fast(u0));
         x1 = dev_round_bf16(x1) * (g.epi_tanh ? dev_gelu_tanh_grad_fast(u1) : dev_gelu_erf_grad_fast(u1));
+      } else if constexpr (EPI == OMX_EPI_AXPBY) {
+        const unsigned int w = *reinterpret_cast<const unsigned int*>(aux_in + off);
+        x0 = gemm_axpby(g, __uint_as_float(w << 16), x0);
+        x1 = gemm_axpby(g, __uint_as_float(w & 0xffff0000u), x1);
       }
       bad |= !(dev_finite(x0) && dev_finite(x1));
       *reinterpret_cast<unsigned int*>(c16 + off) = pack_bf16_pair(x0, x1);
@@ -567,12 +573,17 @@ gemm_dma_persistent_kernel(GemmArgs g) {
     int m0, n0;
     store_at.coords(band_rows, BM, BN, &m0, &n0);
     char* cbase = static_cast<char*>(g.c) + store_at.product * g.batch_c;
+    // aux tensors are bf16 like the output they accompany: the same byte stride between products.
+    const unsigned short* aux_in = g.aux_in;
+    unsigned short* aux_out = g.aux_out;
+    if (aux_in) aux_in = reinterpret_cast<const unsigned short*>(reinterpret_cast<const char*>(aux_in) + store_at.product * g.batch_c);
+    if (aux_out) aux_out = reinterpret_cast<unsigned short*>(reinterpret_cast<char*>(aux_out) + store_at.product * g.batch_c);
     bool bad = false;
     static_for<0, TM>([&](auto tm_index) {
       constexpr int tm = decltype(tm_index)::value;
 #pragma unroll
       for (int tn = 0; tn < TN; ++tn)
-        bad |= store_block_direct<EPI>(g, cbase, g.aux_in, g.aux_out, acc[tm][tn], m0 + (wm * TM + tm) * 32,
+        bad |= store_block_direct<EPI>(g, cbase, aux_in, aux_out, acc[tm][tn], m0 + (wm * TM + tm) * 32,
                                        n0 + (wn * TN + tn) * 32, threadIdx.x & 31, (threadIdx.x >> 5) & 1);
     });
     if (bad) dev_raise_fault(g.fault, g.tag);
@@ -596,6 +607,7 @@ int32_t launch_dma(omx_ctx* ctx, const GemmArgs& g) {
       gp.band_rows = g.tiles_m % 4 == 0 ? 4 : g.tiles_m % 3 == 0 ? 3 : g.tiles_m % 2 == 0 ? 2 : 1;
       auto pk = g.epi == OMX_EPI_GELU_FWD   ? &gemm_dma_persistent_kernel<A_KM, B_KM, WGM, WGN, TM, TN, DBK, NST, OMX_EPI_GELU_FWD>
                 : g.epi == OMX_EPI_GELU_BWD ? &gemm_dma_persistent_kernel<A_KM, B_KM, WGM, WGN, TM, TN, DBK, NST, OMX_EPI_GELU_BWD>
+                : g.epi == OMX_EPI_AXPBY    ? &gemm_dma_persistent_kernel<A_KM, B_KM, WGM, WGN, TM, TN, DBK, NST, OMX_EPI_AXPBY>
                                             : &gemm_dma_persistent_kernel<A_KM, B_KM, WGM, WGN, TM, TN, DBK, NST, OMX_EPI_NONE>;
       // The stages, then the parked load offsets: one word per thread and load.
       constexpr int psmem = smem + (BM + BN) * DBK * 2 / 1024 * 64 * 4;

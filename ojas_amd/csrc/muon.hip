@@ -254,6 +254,11 @@ int32_t run_muon(omx_ctx* ctx, const MuonTensors& t, unsigned count, uint64_t ro
   const OmxGemmBatch* bp = count > 1 ? &batch : nullptr;
   TX* am = reinterpret_cast<TX*>(ws + L.a);
   TX* a2 = reinterpret_cast<TX*>(ws + L.a2);
+  // bf16 tier: the two-term sums after the second and third product ride in those products' store
+  // passes (the same roundings in the same order as the combine kernels below; a non-finite value
+  // raises the fault there and reaches the final check through the remaining products). Strided
+  // batches only: a single product may split its reduction, which a store-pass sum cannot follow.
+  const bool fused = sizeof(TX) == 2 && s.bf16 && ctx->muon_fused_sums && count > 1;
   for (int it = 0; it < 5; ++it) {
     TX* x = reinterpret_cast<TX*>(ws + x_off);
     TX* xn = reinterpret_cast<TX*>(ws + xn_off);
@@ -261,16 +266,22 @@ int32_t run_muon(omx_ctx* ctx, const MuonTensors& t, unsigned count, uint64_t ro
     if (!tall) rc = omx_gemm_impl(ctx, F_MUON, x, cols, 1, x, 1, cols, XD, am, XD, r, r, c, r, 0, nullptr, bp);
     else rc = omx_gemm_impl(ctx, F_MUON, x, 1, cols, x, cols, 1, XD, am, XD, r, r, c, r, 0, nullptr, bp);
     if (rc != OMX_OK) return rc;
-    rc = omx_gemm_impl(ctx, F_MUON, am, r, 1, am, r, 1, XD, a2, XD, r, r, r, r, 0, nullptr, bp);
+    // B = b A + c A^2
+    const OmxGemmEpilogue sum_b{OMX_EPI_AXPBY, 0, am, nullptr, s.b, s.c};
+    rc = omx_gemm_impl(ctx, F_MUON, am, r, 1, am, r, 1, XD, a2, XD, r, r, r, r, 0, fused ? &sum_b : nullptr, bp);
     if (rc != OMX_OK) return rc;
-    hipLaunchKernelGGL((muon_combine_b_kernel<TX>), dim3(mu_grid(r * r), count), block, 0, ctx->stream, w,
-                       static_cast<size_t>(r * r), s);
-    // BX in X's own physical layout: B X' when wide, X B^T when tall.
-    if (!tall) rc = omx_gemm_impl(ctx, F_MUON, a2, r, 1, x, cols, 1, XD, xn, XD, cols, r, r, c, 0, nullptr, bp);
-    else rc = omx_gemm_impl(ctx, F_MUON, x, cols, 1, a2, 1, r, XD, xn, XD, cols, rows, cols, cols, 0, nullptr, bp);
+    if (!fused)
+      hipLaunchKernelGGL((muon_combine_b_kernel<TX>), dim3(mu_grid(r * r), count), block, 0, ctx->stream, w,
+                         static_cast<size_t>(r * r), s);
+    // X_next = a X + B X, with BX in X's own physical layout: B X' when wide, X B^T when tall.
+    const OmxGemmEpilogue sum_x{OMX_EPI_AXPBY, 0, x, nullptr, s.a, 1.0f};
+    const OmxGemmEpilogue* ex = fused ? &sum_x : nullptr;
+    if (!tall) rc = omx_gemm_impl(ctx, F_MUON, a2, r, 1, x, cols, 1, XD, xn, XD, cols, r, r, c, 0, ex, bp);
+    else rc = omx_gemm_impl(ctx, F_MUON, x, cols, 1, a2, 1, r, XD, xn, XD, cols, rows, cols, cols, 0, ex, bp);
     if (rc != OMX_OK) return rc;
-    hipLaunchKernelGGL((muon_combine_x_kernel<TX>), over_len, block, 0, ctx->stream, w, x_off, xn_off, len, s,
-                       ctx->fault, tag);
+    if (!fused)
+      hipLaunchKernelGGL((muon_combine_x_kernel<TX>), over_len, block, 0, ctx->stream, w, x_off, xn_off, len, s,
+                         ctx->fault, tag);
     OMX_LAUNCH_CHECK(ctx, "muon newton-schulz step");
     std::swap(x_off, xn_off);
   }

@@ -95,6 +95,7 @@ struct omx_ctx {
   int kv_attention_mode = 0;  // 1: cached attention always takes the LDS-tiled kernel
   int adamw_trust = 1;        // 0: omx_adamw_step_bounded always runs its checking pass
   int ce_fused = 1;           // 0: linear-CE always takes the separate statistics and gradient kernels
+  int muon_fused_sums = 1;    // 0: Newton-Schulz forms b A + c A^2 and a X + B X in kernels of their own (bf16 tier)
   bool profile_gemm = false;
   uint32_t profile_classes = 0;  // bit per OmxKernelClass other than the products (omx_profile_kernels)
   // The events of the product being launched (null when not timing): the first kernel of the
@@ -157,13 +158,17 @@ inline unsigned long long omx_tag(omx_ctx* ctx, uint32_t op) {
 // C[m,n] (+)= A.B with element strides; `ldc` is C's row pitch in elements.
 // Optional elementwise work in the GEMM's store pass (bf16 outputs only; `aux` shares C's row pitch):
 //   OMX_EPI_GELU_FWD: C = u (rounded to bf16) and aux_out = gelu(u);
-//   OMX_EPI_GELU_BWD: C = round_bf16(A.B) * gelu'(aux_in).
-enum { OMX_EPI_NONE = 0, OMX_EPI_GELU_FWD = 1, OMX_EPI_GELU_BWD = 2 };
+//   OMX_EPI_GELU_BWD: C = round_bf16(A.B) * gelu'(aux_in);
+//   OMX_EPI_AXPBY: C = round_bf16(s1 aux_in) + round_bf16(s2 round_bf16(A.B)): the product stored as
+//     bf16, then the two-term sum a separate pass over it would form, in one store.
+// aux tensors have C's layout (pitch, and batch stride in a strided batch).
+enum { OMX_EPI_NONE = 0, OMX_EPI_GELU_FWD = 1, OMX_EPI_GELU_BWD = 2, OMX_EPI_AXPBY = 3 };
 struct OmxGemmEpilogue {
   int mode;
   int tanh_form;
   const void* aux_in;
   void* aux_out;
+  float s1 = 0.0f, s2 = 0.0f;  // OMX_EPI_AXPBY
 };
 // `count` products of one shape whose operands lie `stride_*` ELEMENTS apart (16-byte multiples), one launch.
 struct OmxGemmBatch {

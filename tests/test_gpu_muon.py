@@ -132,3 +132,44 @@ def test_batched_step_refuses_the_whole_batch(be):
     assert e.value.code == NON_FINITE and "muon_ns5_step" in str(e.value)
     for i in range(4):
         assert np.array_equal(be.download(dp[i]), ps[i]) and not be.download(dm[i]).any()
+
+
+@pytest.mark.parametrize("rows,cols,count", [(64, 48, 2), (130, 70, 3), (768, 768, 6), (768, 3072, 2), (3072, 768, 2),
+                                             (2048, 2048, 2), (2048, 2048, 1)])
+def test_bf16_iteration_sums_in_the_store_pass_carry_the_separate_kernels_bits(be, rows, cols, count):
+    """The bf16 iteration forms b A + c A^2 and a X + B X in the store passes of the products that
+    feed them (`muon_fused_sums`, the default, for calls on more than one tensor): same roundings in
+    the same order as the separate kernels, so parameters, momenta and bf16 copies are the same bits; and a NaN gradient leaves
+    every tensor of the call untouched under either setting."""
+    from ojas_amd.backend import BF16, NON_FINITE, MuonNs5Config, OjasError
+
+    print(f"muon fused sums {count} x {rows}x{cols}", flush=True)
+    r = np.random.default_rng(rows + 3 * cols + count)
+    ps = [r.standard_normal((rows, cols)).astype(np.float32) * 0.1 for _ in range(count)]
+    gs = [r.standard_normal((rows, cols)).astype(np.float32) * 0.03 for _ in range(count)]
+    ms = [r.standard_normal((rows, cols)).astype(np.float32) * 0.01 for _ in range(count)]
+    cfg = MuonNs5Config(0.02, 0.95, 0.1, 1, 1)
+    got = {}
+    try:
+        for fused in (1, 0):
+            be.set_option("muon_fused_sums", fused)
+            dp, dg, dm = [be.upload(x) for x in ps], [be.upload(x) for x in gs], [be.upload(x) for x in ms]
+            mirrors = [be.upload(np.zeros((rows, cols), np.float32), BF16) for _ in range(count)]
+            be.muon_ns5_step_batched(dp, dg, dm, cfg, mirrors)
+            be.sync()
+            got[fused] = [be.download(t) for t in dp + dm + mirrors]
+            # all or nothing
+            bad = [g.copy() for g in gs]
+            bad[-1][rows // 2, cols // 3] = np.nan
+            dp, dg, dm = [be.upload(x) for x in ps], [be.upload(x) for x in bad], [be.upload(x) for x in ms]
+            be.muon_ns5_step_batched(dp, dg, dm, cfg, None)
+            with pytest.raises(OjasError) as e:
+                be.sync()
+            assert e.value.code == NON_FINITE and "muon" in e.value.detail
+            for t, want in zip(dp + dm, ps + ms):
+                assert np.array_equal(be.download(t), want)
+    finally:
+        be.set_option("muon_fused_sums", 1)
+    for a, b in zip(got[1], got[0]):
+        assert np.array_equal(a, b)
+    assert any(np.any(a != p) for a, p in zip(got[1][:count], ps))
