@@ -576,7 +576,9 @@ int32_t omx_read_scalar_f32(omx_ctx* ctx, const void* src, float* out);
  * vocabulary). "adamw_trust": 0 = omx_adamw_step_bounded always runs its checking pass
  * (default 1). "muon_fused_sums": 0 = the bf16 Newton-Schulz iteration forms b A + c A^2 and
  * a X + B X in kernels of their own instead of in the products' store passes (default 1; the
- * same bits either way). Results are within the same tolerances under every setting. */
+ * same bits either way). "sdpa_tiled": 0 = f32 attention always takes the one-wave-per-row
+ * kernels (default 1: LDS-tiled kernels at head_dim 16 / 32 / 64 / 128 with 16-byte aligned
+ * f32 tensors). Results are within the same tolerances under every setting. */
 int32_t omx_set_option(omx_ctx* ctx, const char* name, int64_t value);
 
 /* Benchmark instrumentation (no counterpart in the reference, whose benches

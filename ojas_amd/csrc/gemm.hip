@@ -654,6 +654,11 @@ int32_t omx_set_option(omx_ctx* ctx, const char* name, int64_t value) {
     ctx->ce_fused = static_cast<int>(value);
     return OMX_OK;
   }
+  if (name && strcmp(name, "sdpa_tiled") == 0) {
+    if (value < 0 || value > 1) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: sdpa_tiled takes 0..1");
+    ctx->sdpa_tiled = static_cast<int>(value);
+    return OMX_OK;
+  }
   if (name && strcmp(name, "muon_fused_sums") == 0) {
     if (value < 0 || value > 1) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: muon_fused_sums takes 0..1");
     ctx->muon_fused_sums = static_cast<int>(value);

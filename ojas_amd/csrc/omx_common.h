@@ -95,6 +95,7 @@ struct omx_ctx {
   int kv_attention_mode = 0;  // 1: cached attention always takes the LDS-tiled kernel
   int adamw_trust = 1;        // 0: omx_adamw_step_bounded always runs its checking pass
   int ce_fused = 1;           // 0: linear-CE always takes the separate statistics and gradient kernels
+  int sdpa_tiled = 1;         // 0: f32 attention always takes the one-wave-per-row kernels
   int muon_fused_sums = 1;    // 0: Newton-Schulz forms b A + c A^2 and a X + B X in kernels of their own (bf16 tier)
   bool profile_gemm = false;
   uint32_t profile_classes = 0;  // bit per OmxKernelClass other than the products (omx_profile_kernels)

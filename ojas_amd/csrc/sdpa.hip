@@ -312,6 +312,395 @@ __global__ __launch_bounds__(SD_THREADS) void sdpa_bwd_dkv_rows_kernel(
   if (bad) dev_raise_fault(fault, tag);
 }
 
+// ---------------------------------------------------------------- tiled f32 kernels
+// The f32 tier at head dims 16 / 32 / 64 / 128: 64 query rows x 64 key rows per step, tiles staged
+// in LDS (row pitch D + 4 floats, so that 16-byte reads of 16 consecutive rows fall in distinct
+// banks), 256 threads as a 16 x 16 grid. Thread (ty, tx) owns the scores of query rows ty + 16 i
+// and key rows tx + 16 c, and of the row-by-D results the rows ty + 16 i at columns
+// VW tx + 16 VW cc. Same formulas as the row kernels above; sums run in tile order.
+constexpr int ST_THREADS = 256;
+constexpr int ST_WP = 68;  // pitch of the 64 x 64 weight tile
+
+template <int D>
+struct StCols {
+  static constexpr int DC = D / 16;            // result columns per thread
+  static constexpr int VW = DC >= 4 ? 4 : DC;  // in chunks of this many
+  static constexpr int NCH = DC / VW;
+};
+
+// 64 rows of D floats starting at row r0 of a [rows, D] plane; rows past `rows` read as zeros.
+template <int D>
+__device__ __forceinline__ void st_load_tile(float* __restrict__ lds, const float* __restrict__ g, int r0, int rows) {
+  constexpr int V4 = D / 4, P = D + 4;
+  for (int idx = threadIdx.x; idx < 64 * V4; idx += ST_THREADS) {
+    const int r = idx / V4, c4 = idx - r * V4;
+    float4 val = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (r0 + r < rows) val = *reinterpret_cast<const float4*>(g + static_cast<long>(r0 + r) * D + 4 * c4);
+    *reinterpret_cast<float4*>(lds + r * P + 4 * c4) = val;
+  }
+}
+
+// s[i][c] = A[ty + 16 i] . B[tx + 16 c] over D.
+template <int D>
+__device__ __forceinline__ void st_dot(const float* __restrict__ A, const float* __restrict__ B, int ty, int tx,
+                                       float (&s)[4][4]) {
+  constexpr int P = D + 4;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int c = 0; c < 4; ++c) s[i][c] = 0.0f;
+#pragma unroll 4
+  for (int d = 0; d < D; d += 4) {
+    float4 a[4], b[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) a[i] = *reinterpret_cast<const float4*>(A + (ty + 16 * i) * P + d);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) b[c] = *reinterpret_cast<const float4*>(B + (tx + 16 * c) * P + d);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        float acc = s[i][c];
+        acc = fmaf(a[i].x, b[c].x, acc);
+        acc = fmaf(a[i].y, b[c].y, acc);
+        acc = fmaf(a[i].z, b[c].z, acc);
+        acc = fmaf(a[i].w, b[c].w, acc);
+        s[i][c] = acc;
+      }
+  }
+}
+
+// acc[i][..] += sum over k of W[ty + 16 i][k] M[k][columns of this thread]; W is a 64 x 64 tile of
+// pitch ST_WP, M a 64 x D tile.
+template <int D>
+__device__ __forceinline__ void st_accumulate(const float* __restrict__ W, const float* __restrict__ M, int ty, int tx,
+                                              float (&acc)[4][StCols<D>::DC]) {
+  constexpr int P = D + 4, VW = StCols<D>::VW, NCH = StCols<D>::NCH;
+#pragma unroll 2
+  for (int k = 0; k < 64; k += 4) {
+    float4 w4[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w4[i] = *reinterpret_cast<const float4*>(W + (ty + 16 * i) * ST_WP + k);
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      float m[NCH * VW];
+#pragma unroll
+      for (int cc = 0; cc < NCH; ++cc) {
+        const float* src = M + (k + kk) * P + VW * tx + 16 * VW * cc;
+        if constexpr (VW == 4) {
+          const float4 v = *reinterpret_cast<const float4*>(src);
+          m[4 * cc] = v.x; m[4 * cc + 1] = v.y; m[4 * cc + 2] = v.z; m[4 * cc + 3] = v.w;
+        } else if constexpr (VW == 2) {
+          const float2 v = *reinterpret_cast<const float2*>(src);
+          m[0] = v.x; m[1] = v.y;
+        } else {
+          m[0] = src[0];
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float wv = kk == 0 ? w4[i].x : kk == 1 ? w4[i].y : kk == 2 ? w4[i].z : w4[i].w;
+#pragma unroll
+        for (int e = 0; e < NCH * VW; ++e) acc[i][e] = fmaf(wv, m[e], acc[i][e]);
+      }
+    }
+  }
+}
+
+// Stores the thread's columns of row `row` of a [rows, D] plane; returns whether a value was non-finite.
+template <int D>
+__device__ __forceinline__ bool st_store_row(float* __restrict__ g, long row, int tx, const float (&v)[StCols<D>::DC],
+                                             float scale) {
+  constexpr int VW = StCols<D>::VW, NCH = StCols<D>::NCH;
+  bool bad = false;
+#pragma unroll
+  for (int cc = 0; cc < NCH; ++cc) {
+    float* dst = g + row * D + VW * tx + 16 * VW * cc;
+#pragma unroll
+    for (int e = 0; e < VW; ++e) {
+      const float o = v[VW * cc + e] * scale;
+      bad |= !dev_finite(o);
+      dst[e] = o;
+    }
+  }
+  return bad;
+}
+
+// The largest / the sum of a value over the 16 threads that share a query row.
+__device__ __forceinline__ float st_row_max(float v) {
+#pragma unroll
+  for (int off = 8; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+__device__ __forceinline__ float st_row_sum(float v) {
+#pragma unroll
+  for (int off = 8; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+// Forward: one workgroup per 64 query rows of a head.
+template <int D>
+__global__ __launch_bounds__(ST_THREADS) void sdpa_tiled_fwd_kernel(const float* __restrict__ q,
+                                                                    const float* __restrict__ k,
+                                                                    const float* __restrict__ v,
+                                                                    float* __restrict__ out, float* __restrict__ lse,
+                                                                    SdpaShape s, OmxFaultWord* fault,
+                                                                    unsigned long long tag) {
+  constexpr int P = D + 4, DC = StCols<D>::DC;
+  __shared__ __align__(16) float Qs[64 * P];
+  __shared__ __align__(16) float Ks[64 * P];
+  __shared__ __align__(16) float Vs[64 * P];
+  __shared__ __align__(16) float Ws[64 * ST_WP];
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  const int plane = blockIdx.y, h = plane % s.heads, b = plane / s.heads;
+  const long kv_plane = static_cast<long>(b) * s.kv_heads + h / s.rep;
+  const float* qh = q + static_cast<long>(plane) * s.time * D;
+  const float* kh = k + kv_plane * s.time * D;
+  const float* vh = v + kv_plane * s.time * D;
+  const int t0 = blockIdx.x * 64;
+  st_load_tile<D>(Qs, qh, t0, s.time);
+  float o[4][DC], mx[4], sum[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    mx[i] = -INFINITY;
+    sum[i] = 0.0f;
+#pragma unroll
+    for (int e = 0; e < DC; ++e) o[i][e] = 0.0f;
+  }
+  bool bad = false;
+  const int t_last = min(s.time, t0 + 64) - 1;
+  const int kb_first = first_key(s, t0) / 64, kb_last = t_last / 64;
+  for (int kb = kb_first; kb <= kb_last; ++kb) {
+    __syncthreads();  // the previous step's reads of Ks, Vs and Ws are done
+    st_load_tile<D>(Ks, kh, kb * 64, s.time);
+    st_load_tile<D>(Vs, vh, kb * 64, s.time);
+    __syncthreads();
+    float sc[4][4];
+    st_dot<D>(Qs, Ks, ty, tx, sc);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int t = t0 + ty + 16 * i, lo = first_key(s, t);
+      float top = -INFINITY;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int j = kb * 64 + tx + 16 * c;
+        const bool seen = t < s.time && j <= t && j >= lo;
+        const float val = sc[i][c] * s.scale;
+        bad |= seen && !dev_finite(val);
+        sc[i][c] = seen ? val : -INFINITY;
+        top = fmaxf(top, sc[i][c]);
+      }
+      top = st_row_max(top);
+      const float new_max = fmaxf(mx[i], top);
+      // A row that has seen no key yet keeps its empty state.
+      const float rescale = new_max == -INFINITY ? 1.0f : expf(mx[i] - new_max);
+      float part = 0.0f;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const float p = sc[i][c] == -INFINITY ? 0.0f : expf(sc[i][c] - new_max);
+        part += p;
+        Ws[(ty + 16 * i) * ST_WP + tx + 16 * c] = p;
+      }
+      part = st_row_sum(part);
+      sum[i] = sum[i] * rescale + part;
+      mx[i] = new_max;
+#pragma unroll
+      for (int e = 0; e < DC; ++e) o[i][e] *= rescale;
+    }
+    __syncthreads();
+    st_accumulate<D>(Ws, Vs, ty, tx, o);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int t = t0 + ty + 16 * i;
+    if (t < s.time) {
+      bad |= !(dev_finite(sum[i]) && sum[i] > 0.0f);
+      const long row = static_cast<long>(plane) * s.time + t;
+      bad |= st_store_row<D>(out, row, tx, o[i], 1.0f / sum[i]);
+      if (tx == 0) lse[row] = mx[i] + logf(sum[i]);
+    }
+  }
+  if (bad) dev_raise_fault(fault, tag);
+}
+
+// The weights of one 64 x 64 step of the backward: p = e^(S - lse) and dS = scale p (dP - Dr) for
+// the thread's 4 x 4 scores; `bad` gathers non-finite scores and probabilities.
+struct StRows {
+  float lse[4], dr[4];
+};
+__device__ __forceinline__ void st_backward_weights(const SdpaShape& s, int t0, int j0, int ty, int tx,
+                                                    const StRows& rows, const float (&sc)[4][4],
+                                                    const float (&dp)[4][4], float (&p)[4][4], float (&ds)[4][4],
+                                                    bool& bad) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int t = t0 + ty + 16 * i, lo = first_key(s, t);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int j = j0 + tx + 16 * c;
+      const bool seen = t < s.time && j <= t && j >= lo;
+      const float val = sc[i][c] * s.scale;
+      const float pr = seen ? expf(val - rows.lse[i]) : 0.0f;
+      bad |= seen && !(dev_finite(val) && dev_finite(pr));
+      p[i][c] = pr;
+      ds[i][c] = seen ? s.scale * (pr * (dp[i][c] - rows.dr[i])) : 0.0f;
+    }
+  }
+}
+
+// dQ: one workgroup per 64 query rows of a head.
+template <int D>
+__global__ __launch_bounds__(ST_THREADS) void sdpa_tiled_dq_kernel(const float* __restrict__ q,
+                                                                   const float* __restrict__ k,
+                                                                   const float* __restrict__ v,
+                                                                   const float* __restrict__ lse,
+                                                                   const float* __restrict__ delta,
+                                                                   const float* __restrict__ gy,
+                                                                   float* __restrict__ gq, SdpaShape s,
+                                                                   OmxFaultWord* fault, unsigned long long tag) {
+  constexpr int P = D + 4, DC = StCols<D>::DC;
+  __shared__ __align__(16) float Qs[64 * P];
+  __shared__ __align__(16) float Gs[64 * P];
+  __shared__ __align__(16) float Ks[64 * P];
+  __shared__ __align__(16) float Vs[64 * P];
+  __shared__ __align__(16) float Ws[64 * ST_WP];
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  const int plane = blockIdx.y, h = plane % s.heads, b = plane / s.heads;
+  const long kv_plane = static_cast<long>(b) * s.kv_heads + h / s.rep;
+  const long row0 = static_cast<long>(plane) * s.time;
+  const float* kh = k + kv_plane * s.time * D;
+  const float* vh = v + kv_plane * s.time * D;
+  const int t0 = blockIdx.x * 64;
+  st_load_tile<D>(Qs, q + row0 * D, t0, s.time);
+  st_load_tile<D>(Gs, gy + row0 * D, t0, s.time);
+  bool bad = false;
+  StRows rows;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int t = t0 + ty + 16 * i;
+    rows.lse[i] = t < s.time ? lse[row0 + t] : 0.0f;
+    rows.dr[i] = t < s.time ? delta[row0 + t] : 0.0f;
+    bad |= !(dev_finite(rows.lse[i]) && dev_finite(rows.dr[i]));
+  }
+  float acc[4][DC];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int e = 0; e < DC; ++e) acc[i][e] = 0.0f;
+  const int t_last = min(s.time, t0 + 64) - 1;
+  const int kb_first = first_key(s, t0) / 64, kb_last = t_last / 64;
+  for (int kb = kb_first; kb <= kb_last; ++kb) {
+    __syncthreads();
+    st_load_tile<D>(Ks, kh, kb * 64, s.time);
+    st_load_tile<D>(Vs, vh, kb * 64, s.time);
+    __syncthreads();
+    float sc[4][4], dp[4][4], p[4][4], ds[4][4];
+    st_dot<D>(Qs, Ks, ty, tx, sc);
+    st_dot<D>(Gs, Vs, ty, tx, dp);
+    st_backward_weights(s, t0, kb * 64, ty, tx, rows, sc, dp, p, ds, bad);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) Ws[(ty + 16 * i) * ST_WP + tx + 16 * c] = ds[i][c];
+    __syncthreads();
+    st_accumulate<D>(Ws, Ks, ty, tx, acc);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int t = t0 + ty + 16 * i;
+    if (t < s.time) bad |= st_store_row<D>(gq, row0 + t, tx, acc[i], 1.0f);
+  }
+  if (bad) dev_raise_fault(fault, tag);
+}
+
+// dK, dV: one workgroup per 64 key rows of a KV head; the query heads of the group in ascending
+// order and, within a head, query blocks in ascending order.
+template <int D>
+__global__ __launch_bounds__(ST_THREADS) void sdpa_tiled_dkv_kernel(const float* __restrict__ q,
+                                                                    const float* __restrict__ k,
+                                                                    const float* __restrict__ v,
+                                                                    const float* __restrict__ lse,
+                                                                    const float* __restrict__ delta,
+                                                                    const float* __restrict__ gy,
+                                                                    float* __restrict__ gk, float* __restrict__ gv,
+                                                                    SdpaShape s, OmxFaultWord* fault,
+                                                                    unsigned long long tag) {
+  constexpr int P = D + 4, DC = StCols<D>::DC;
+  __shared__ __align__(16) float Qs[64 * P];
+  __shared__ __align__(16) float Gs[64 * P];
+  __shared__ __align__(16) float Ks[64 * P];
+  __shared__ __align__(16) float Vs[64 * P];
+  __shared__ __align__(16) float Wt[64 * ST_WP];  // [key][query]
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  const int kv_plane = blockIdx.y, g = kv_plane % s.kv_heads, b = kv_plane / s.kv_heads;
+  const long kv_row0 = static_cast<long>(kv_plane) * s.time;
+  const int j0 = blockIdx.x * 64;
+  st_load_tile<D>(Ks, k + kv_row0 * D, j0, s.time);
+  st_load_tile<D>(Vs, v + kv_row0 * D, j0, s.time);
+  float acck[4][DC], accv[4][DC];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int e = 0; e < DC; ++e) acck[i][e] = accv[i][e] = 0.0f;
+  bool bad = false;
+  const int j_last = min(s.time, j0 + 64) - 1;
+  const int qb_last = last_query(s, j_last) / 64;
+  for (int r = 0; r < s.rep; ++r) {
+    const long row0 = (static_cast<long>(b) * s.heads + static_cast<long>(g) * s.rep + r) * s.time;
+    for (int qb = blockIdx.x; qb <= qb_last; ++qb) {
+      const int t0 = qb * 64;
+      __syncthreads();  // the previous step's reads of Qs, Gs and Wt are done
+      st_load_tile<D>(Qs, q + row0 * D, t0, s.time);
+      st_load_tile<D>(Gs, gy + row0 * D, t0, s.time);
+      StRows rows;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int t = t0 + ty + 16 * i;
+        rows.lse[i] = t < s.time ? lse[row0 + t] : 0.0f;
+        rows.dr[i] = t < s.time ? delta[row0 + t] : 0.0f;
+      }
+      __syncthreads();
+      float sc[4][4], dp[4][4], p[4][4], ds[4][4];
+      st_dot<D>(Qs, Ks, ty, tx, sc);
+      st_dot<D>(Gs, Vs, ty, tx, dp);
+      st_backward_weights(s, t0, j0, ty, tx, rows, sc, dp, p, ds, bad);
+      // dV += P^T dO
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) Wt[(tx + 16 * c) * ST_WP + ty + 16 * i] = p[i][c];
+      __syncthreads();
+      st_accumulate<D>(Wt, Gs, ty, tx, accv);
+      __syncthreads();
+      // dK += dS^T Q
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) Wt[(tx + 16 * c) * ST_WP + ty + 16 * i] = ds[i][c];
+      __syncthreads();
+      st_accumulate<D>(Wt, Qs, ty, tx, acck);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int j = j0 + ty + 16 * i;
+    if (j < s.time) {
+      bad |= st_store_row<D>(gk, kv_row0 + j, tx, acck[i], 1.0f);
+      bad |= st_store_row<D>(gv, kv_row0 + j, tx, accv[i], 1.0f);
+    }
+  }
+  if (bad) dev_raise_fault(fault, tag);
+}
+
+bool sdpa_tiled_supports(uint64_t dim, std::initializer_list<int32_t> dtypes, std::initializer_list<const void*> ptrs) {
+  if (dim != 16 && dim != 32 && dim != 64 && dim != 128) return false;
+  for (int32_t d : dtypes)
+    if (d != OMX_F32) return false;
+  for (const void* p : ptrs)
+    if (reinterpret_cast<uintptr_t>(p) & 15u) return false;
+  return true;
+}
+
 int32_t check_shape(omx_ctx* ctx, const char* op, uint64_t batch, uint64_t heads, uint64_t kv_heads, uint64_t time,
                     uint64_t dim, uint64_t window, SdpaShape* s) {
   if (batch == 0 || heads == 0 || kv_heads == 0 || time == 0 || dim == 0)
@@ -353,6 +742,20 @@ int32_t omx_causal_sdpa_forward(omx_ctx* ctx, const void* q, const void* k, cons
   if (omx_flash_sdpa_supports(head_dim, operand_dtype))
     return omx_flash_sdpa_forward(ctx, q, k, v, out, out_dtype, nullptr, static_cast<float*>(lse), batch, heads,
                                   kv_heads, time, head_dim, s.window, s.scale, tag, nullptr);
+  if (ctx->sdpa_tiled && sdpa_tiled_supports(head_dim, {operand_dtype, out_dtype}, {q, k, v, out})) {
+    dim3 tgrid(static_cast<unsigned>((time + 63) / 64), static_cast<unsigned>(batch * heads));
+#define SDPA_TILED_FWD(D_)                                                                                      \
+  hipLaunchKernelGGL((sdpa_tiled_fwd_kernel<D_>), tgrid, dim3(ST_THREADS), 0, ctx->stream,                      \
+                     static_cast<const float*>(q), static_cast<const float*>(k), static_cast<const float*>(v),  \
+                     static_cast<float*>(out), static_cast<float*>(lse), s, ctx->fault, tag)
+    if (head_dim == 16) SDPA_TILED_FWD(16);
+    else if (head_dim == 32) SDPA_TILED_FWD(32);
+    else if (head_dim == 64) SDPA_TILED_FWD(64);
+    else SDPA_TILED_FWD(128);
+#undef SDPA_TILED_FWD
+    OMX_LAUNCH_CHECK(ctx, "sdpa_tiled_fwd_kernel");
+    return OMX_OK;
+  }
   const long rows = static_cast<long>(batch) * heads * time;
   dim3 grid(static_cast<unsigned>((rows + 3) / 4)), block(SD_THREADS);
 #define SDPA_FWD(TI, TO)                                                                                          \
@@ -439,6 +842,27 @@ int32_t omx_causal_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, con
     rc = omx_convert(ctx, gy, gy_dtype, conv, operand_dtype, n);
     if (rc != OMX_OK) return rc;
     gy = conv;
+  }
+  if (ctx->sdpa_tiled && sdpa_tiled_supports(head_dim, {operand_dtype, grad_dtype}, {q, k, v, gy, gq, gk, gv})) {
+    dim3 qgrid(static_cast<unsigned>((time + 63) / 64), static_cast<unsigned>(batch * heads));
+    dim3 kgrid(static_cast<unsigned>((time + 63) / 64), static_cast<unsigned>(batch * kv_heads));
+#define SDPA_TILED_BWD(D_)                                                                                          \
+  do {                                                                                                              \
+    hipLaunchKernelGGL((sdpa_tiled_dq_kernel<D_>), qgrid, dim3(ST_THREADS), 0, ctx->stream,                         \
+                       static_cast<const float*>(q), static_cast<const float*>(k), static_cast<const float*>(v),    \
+                       lsef, delta, static_cast<const float*>(gy), static_cast<float*>(gq), s, ctx->fault, tag);    \
+    hipLaunchKernelGGL((sdpa_tiled_dkv_kernel<D_>), kgrid, dim3(ST_THREADS), 0, ctx->stream,                        \
+                       static_cast<const float*>(q), static_cast<const float*>(k), static_cast<const float*>(v),    \
+                       lsef, delta, static_cast<const float*>(gy), static_cast<float*>(gk), static_cast<float*>(gv), \
+                       s, ctx->fault, tag);                                                                         \
+  } while (0)
+    if (head_dim == 16) SDPA_TILED_BWD(16);
+    else if (head_dim == 32) SDPA_TILED_BWD(32);
+    else if (head_dim == 64) SDPA_TILED_BWD(64);
+    else SDPA_TILED_BWD(128);
+#undef SDPA_TILED_BWD
+    OMX_LAUNCH_CHECK(ctx, "sdpa tiled backward kernels");
+    return OMX_OK;
   }
 #define SDPA_BWD(TI, TO)                                                                                              \
   do {                                                                                                                \

@@ -350,6 +350,40 @@ def test_causal_sdpa_f32(be, shape, hkv, window):
     close(be.download(gv), ogv, F32_TOL, "sdpa gv")
 
 
+@pytest.mark.parametrize("shape,hkv,window", [([1, 4, 333, 64], 2, 100), ([2, 2, 200, 128], 2, None),
+                                              ([1, 6, 129, 32], 3, 64), ([3, 2, 64, 16], 1, 5),
+                                              ([1, 2, 1024, 64], 2, None)])
+def test_causal_sdpa_f32_tiled_kernels_agree_with_the_row_kernels(be, shape, hkv, window):
+    """The f32 tier's LDS-tiled attention kernels (head_dim 16 / 32 / 64 / 128) against the
+    one-wave-per-row kernels (`sdpa_tiled` 0) and the oracle: several 64-row blocks, windows that
+    start inside an earlier block, grouped heads, a ragged last block."""
+    print(f"sdpa f32 tiled {shape} hkv {hkv} window {window}", flush=True)
+    b, h, t, d = shape
+    r = orc.SplitMix64(500 + t + d)
+    q = r.vec(b * h * t * d, 0.5).reshape(b, h, t, d)
+    k = r.vec(b * hkv * t * d, 0.5).reshape(b, hkv, t, d)
+    v = r.vec(b * hkv * t * d, 0.5).reshape(b, hkv, t, d)
+    gy = r.vec(b * h * t * d, 0.5).reshape(b, h, t, d)
+    dq, dk, dv, dgy = be.upload(q), be.upload(k), be.upload(v), be.upload(gy)
+    got = {}
+    try:
+        for tiled in (1, 0):
+            be.set_option("sdpa_tiled", tiled)
+            y, lse = be.causal_sdpa_forward(dq, dk, dv, window)
+            gq, gk, gv = be.causal_sdpa_backward(dq, dk, dv, y, lse, dgy, window)
+            got[tiled] = [be.download(x) for x in (y, lse, gq, gk, gv)]
+    finally:
+        be.set_option("sdpa_tiled", 1)
+    for name, a, c in zip(("out", "lse", "gq", "gk", "gv"), got[1], got[0]):
+        close(a, c, F32_TOL, "tiled against rows: " + name)
+    if t <= 400:
+        orc.set_threads(8)
+        oy, olse = orc.causal_sdpa_forward(q, k, v, window or 0)
+        ogq, ogk, ogv = orc.causal_sdpa_backward(q, k, v, oy, olse, gy, window or 0)
+        for name, a, c in zip(("out", "lse", "gq", "gk", "gv"), got[1], (oy, olse, ogq, ogk, ogv)):
+            close(a, c, F32_TOL, "tiled against the oracle: " + name)
+
+
 def test_adamw_matches_fast_f32_contract_bitwise_and_exact_within_1e6(be):
     from ojas_amd.backend import AdamWConfig
 
