@@ -515,9 +515,11 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
     const int ksteps = (g.K + bk - 1) / bk;
     const long tiles = static_cast<long>(g.tiles_m) * g.tiles_n;
     int splits = 1;
-    if (tiles * g.batches < 256 && g.batches == 1 && ksteps >= 32 && !(epi && epi->mode != OMX_EPI_NONE)) {
+    // An f32 step is 64 MFMAs per wave (1.7 us): two of them already pay for a split.
+    const int min_steps = operand_dtype == OMX_BF16 ? 8 : 2;
+    if (tiles * g.batches < 256 && g.batches == 1 && ksteps >= 4 * min_steps && !(epi && epi->mode != OMX_EPI_NONE)) {
       splits = static_cast<int>((512 + tiles - 1) / tiles);
-      if (splits > ksteps / 8) splits = ksteps / 8;
+      if (splits > ksteps / min_steps) splits = ksteps / min_steps;
       if (splits < 1) splits = 1;
       if (dma_variant >= 0) {  // a power of two, so that a split stays on one XCD (see gemm_dma_kernel)
         int p2 = 1;
