@@ -35,11 +35,13 @@ sys.path.insert(0, str(ROOT))
 BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, vendor figure
 F32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, vendor figure
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor figure
-# HBM bytes per GEMM op (MFMA kernel + split-K reduce) on the gpt124m workload, averaged over the
-# step's 103 GEMM ops (a strided batch of the stacked layers' weight gradients is one op): rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by what the same
-# counters read for the AdamW pass, whose traffic is known (profiles/gemm_hbm_traffic_gpt124m_bf16.txt).
-# The algorithmic figure (every operand read once, every output written once) is 2.258e8.
-GEMM_HBM_BYTES_PER_LAUNCH_GPT124M = 3.82e8
+# HBM bytes per GEMM op (MFMA kernel + split-K reduce), averaged over a step's GEMM ops (a strided
+# batch of the stacked layers' weight gradients is one op): rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per
+# dispatch, scaled by what the same counters read for the AdamW pass, whose traffic is known
+# (profiles/gemm_hbm_traffic_all_workloads.txt holds the runs and the tables for each workload).
+# The algorithmic figure of the gpt124m step (every operand read once, every output written once)
+# is 2.258e8 per op.
+GEMM_HBM_BYTES_PER_LAUNCH = {"gpt124m": 3.93e8, "gpt124m-muon": 3.13e8, "lora1b": 2.38e8, "nanolab124m": 2.28e8}
 
 
 # Kernel classes of omx_profile_kernels beyond the GEMM products: (bit, key, kernels, roofline).
@@ -344,7 +346,8 @@ def lora_step(args) -> int:
                      "kernel": "gemm_q8_kernel (int8-g32 dequant-fused bf16 MFMA product) with the adapters' and the "
                                "head's bf16 products",
                      "achieved": achieved, "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / BF16_MFMA_PEAK_TFLOPS, "traffic": None, "launches": int(launches.value),
+                     "frac": achieved / BF16_MFMA_PEAK_TFLOPS, "traffic": GEMM_HBM_BYTES_PER_LAUNCH["lora1b"],
+                     "launches": int(launches.value),
                      "avg_launch_us": gemm_ms.value * 1e3 / max(1, launches.value), "timed_steps": timed_steps,
                      "gemm_ms_per_step": gemm_ms.value / max(1, timed_steps)},
         "roofline_per_kernel": per_kernel,
@@ -480,7 +483,8 @@ def nanolab_step(args) -> int:
         "loss_first": losses[0], "loss_last": losses[-1],
         "roofline": {"bound": "mfma", "kernel": "gemm_dma_kernel / gemm_kernel (bf16 MFMA GEMM, all operand layouts)",
                      "achieved": achieved, "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / BF16_MFMA_PEAK_TFLOPS, "traffic": None, "launches": int(launches.value),
+                     "frac": achieved / BF16_MFMA_PEAK_TFLOPS, "traffic": GEMM_HBM_BYTES_PER_LAUNCH["nanolab124m"],
+                     "launches": int(launches.value),
                      "avg_launch_us": gemm_ms.value * 1e3 / max(1, launches.value), "timed_steps": timed_steps,
                      "gemm_ms_per_step": gemm_ms.value / max(1, timed_steps)},
         "roofline_per_kernel": per_kernel,
@@ -597,9 +601,8 @@ def main() -> int:
                      "kernel": "gemm_dma_kernel / gemm_kernel (bf16 MFMA GEMM, all operand layouts)" if cfg.bf16
                                else "gemm_kernel<float> (f32 MFMA GEMM, all operand layouts)",
                      "achieved": achieved, "peak": gemm_peak, "unit": "TFLOP/s", "frac": achieved / gemm_peak,
-                     # measured on the AdamW step of this configuration only
-                     "traffic": GEMM_HBM_BYTES_PER_LAUNCH_GPT124M
-                     if args.config == "gpt124m" and args.optimizer == "adamw" else None,
+                     "traffic": GEMM_HBM_BYTES_PER_LAUNCH.get(
+                         "gpt124m" if args.optimizer == "adamw" else "gpt124m-muon") if args.config == "gpt124m" else None,
                      "launches": int(launches.value), "avg_launch_us": gemm_ms.value * 1e3 / max(1, launches.value),
                      "timed_steps": len(range(0, args.steps, timed_every)),
                      "gemm_ms_per_step": gemm_ms.value / max(1, len(range(0, args.steps, timed_every)))},
