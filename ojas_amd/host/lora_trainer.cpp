@@ -60,6 +60,12 @@ struct olora {
   };
   std::vector<Layer> layers;
   void *stage_codes = nullptr, *stage_scales = nullptr;  // row-major staging of one sub-matrix
+  // The operands of the adapters' weight gradients, every layer's at a fixed stride (bf16): the
+  // layers' h1, ha and ap point into the first three; gy_o, gqkv_all and gh_all keep each layer's
+  // output gradients of the o site and of q | k | v and their gh = gy B until the end of the
+  // backward, where six strided-batch products over the layers form every dA and dB (a reduction
+  // over the tokens with an output of rank x d fills the chip only with the layers side by side).
+  void *h1_all = nullptr, *ha_all = nullptr, *ap_all = nullptr, *gy_o = nullptr, *gqkv_all = nullptr, *gh_all = nullptr;
 
   // Adapters.
   float *p32 = nullptr, *g32 = nullptr, *m1 = nullptr, *m2 = nullptr, *tmp_b = nullptr;
@@ -71,7 +77,7 @@ struct olora {
   // Scratch.
   float *x_final = nullptr, *gres = nullptr, *gres1 = nullptr;
   void *hf = nullptr, *h2 = nullptr, *m = nullptr, *t_a = nullptr, *t_b = nullptr, *gy16 = nullptr, *gm = nullptr,
-       *ggu = nullptr, *gh = nullptr, *ga = nullptr, *gqkv = nullptr, *ghf = nullptr;
+       *ggu = nullptr, *ga = nullptr, *ghf = nullptr;
 
   // Arena offsets (elements). which: 0 q, 1 k, 2 v, 3 o.
   uint64_t a_off(uint64_t l, uint64_t which) const { return (l * 4 + which) * rd; }
@@ -188,39 +194,49 @@ int32_t backward(olora* t) {
   TRY(omx_to_bf16(ctx, t->gres, t->gy16, N * d));
   for (uint32_t l = c.layers; l-- > 0;) {
     olora::Layer& A = t->layers[l];
-    auto ga_ = [&](uint64_t which) { return t->g32 + t->a_off(l, which); };
-    auto gb_ = [&](uint64_t which) { return t->g32 + t->b_off(l, which); };
     // x_next = x1 + down(silu(gate) * up)
     TRY(q8_backward(t, A.dn, t->gy16, nullptr, t->gm));
     TRY(omx_swiglu_backward(ctx, A.gu_out, t->gm, t->ggu, OMX_BF16, N, Hd));
     TRY(q8_backward(t, A.gu, t->ggu, nullptr, t->t_a));
-    // Fan-in at x1: the residual branch first, then the norm branch.
-    TRY(omx_rms_norm_backward_residual(ctx, A.x1, OMX_F32, t->norm(l, 1), t->t_a, OMX_BF16, t->gres, t->gres1, t->gy16,
+    // Fan-in at x1: the residual branch first, then the norm branch. The bf16 copy is this layer's
+    // own: the o site's weight gradients read it after the loop.
+    uint16_t* gy_mid = off16(t->gy_o, l * N * d);
+    uint16_t* gqkv = off16(t->gqkv_all, l * N * 3 * d);
+    uint16_t* gh = off16(t->gh_all, l * N * 4 * r);
+    TRY(omx_rms_norm_backward_residual(ctx, A.x1, OMX_F32, t->norm(l, 1), t->t_a, OMX_BF16, t->gres, t->gres1, gy_mid,
                                        t->dummy_gw, N, d, eps));
     // x1 = x + lora_linear(ap; Wo, Ao, Bo). With gy the gradient of the site's output:
     //   gh = gy B_eff [N, r];  dB_eff = gy^T h;  dA = gh^T x;  gx = gy W + gh A.
-    TRY(omx_gemm_pitched(ctx, t->gy16, d, 1, t->b16(l, 3), r, 1, OMX_BF16, off16(t->gh, 3 * r), OMX_BF16, 4 * r, N, d, r, 0));
-    TRY(omx_gemm(ctx, t->gy16, 1, d, off16(A.ha, 3 * r), 4 * r, 1, OMX_BF16, gb_(3), OMX_F32, d, N, r, 0));
-    TRY(omx_gemm(ctx, off16(t->gh, 3 * r), 1, 4 * r, A.ap, d, 1, OMX_BF16, ga_(3), OMX_F32, r, N, d, 0));
-    omx_low_rank lr_o{off16(t->gh, 3 * r), t->at(l) + 3 * r, 4 * r, 4 * r, r, 0};
-    TRY(q8_backward(t, A.o, t->gy16, &lr_o, t->ga));
-    char* gq = static_cast<char*>(t->gqkv);
+    TRY(omx_gemm_pitched(ctx, gy_mid, d, 1, t->b16(l, 3), r, 1, OMX_BF16, off16(gh, 3 * r), OMX_BF16, 4 * r, N, d, r, 0));
+    omx_low_rank lr_o{off16(gh, 3 * r), t->at(l) + 3 * r, 4 * r, 4 * r, r, 0};
+    TRY(q8_backward(t, A.o, gy_mid, &lr_o, t->ga));
+    char* gq = reinterpret_cast<char*>(gqkv);
     TRY(omx_causal_attention_backward_saved(ctx, A.qkv_out, 3 * d, off16(A.qkv_out, d), off16(A.qkv_out, 2 * d), 3 * d,
                                             A.ap, A.apr, t->ga, d, A.lse, OMX_BF16, gq, gq + d * 2, gq + 2 * d * 2,
                                             OMX_BF16, B, T, H, H, D, 0));
-    TRY(omx_rope_half_split_inplace(ctx, t->gqkv, OMX_BF16, 3 * d, t->cos_t, t->sin_t, N, T, 2 * H, D, 1));
-    for (uint64_t j = 0; j < 3; ++j) {
-      TRY(omx_gemm_pitched(ctx, off16(t->gqkv, j * d), 3 * d, 1, t->b16(l, j), r, 1, OMX_BF16, off16(t->gh, j * r),
-                           OMX_BF16, 4 * r, N, d, r, 0));
-      TRY(omx_gemm(ctx, off16(t->gqkv, j * d), 1, 3 * d, off16(A.ha, j * r), 4 * r, 1, OMX_BF16, gb_(j), OMX_F32, d, N, r,
-                   0));
-    }
-    // [Aq; Ak; Av] are adjacent: one product for the three down-projections' gradients.
-    TRY(omx_gemm(ctx, t->gh, 1, 4 * r, A.h1, d, 1, OMX_BF16, ga_(0), OMX_F32, 3 * r, N, d, 0));
-    omx_low_rank lr_qkv{t->gh, t->at(l), 4 * r, 4 * r, 3 * r, 0};
-    TRY(q8_backward(t, A.qkv, t->gqkv, &lr_qkv, t->t_b));
+    TRY(omx_rope_half_split_inplace(ctx, gqkv, OMX_BF16, 3 * d, t->cos_t, t->sin_t, N, T, 2 * H, D, 1));
+    for (uint64_t j = 0; j < 3; ++j)
+      TRY(omx_gemm_pitched(ctx, off16(gqkv, j * d), 3 * d, 1, t->b16(l, j), r, 1, OMX_BF16, off16(gh, j * r), OMX_BF16,
+                           4 * r, N, d, r, 0));
+    omx_low_rank lr_qkv{gh, t->at(l), 4 * r, 4 * r, 3 * r, 0};
+    TRY(q8_backward(t, A.qkv, gqkv, &lr_qkv, t->t_b));
     TRY(omx_rms_norm_backward_residual(ctx, A.x, OMX_F32, t->norm(l, 0), t->t_b, OMX_BF16, t->gres1, t->gres, t->gy16,
                                        t->dummy_gw, N, d, eps));
+  }
+  // The adapters' weight gradients, every layer's in one launch per site: dB_eff = gy^T h for q, k,
+  // v and o; dA = gh^T x for [Aq; Ak; Av] (adjacent in the arena: one product) and for Ao.
+  {
+    const uint64_t L = c.layers, rd = t->rd;
+    const uint64_t s_d = N * d, s_3d = N * 3 * d, s_4r = N * 4 * r, s_c = 4 * rd;
+    for (uint64_t j = 0; j < 3; ++j)
+      TRY(omx_gemm_strided_batch(ctx, off16(t->gqkv_all, j * d), 1, 3 * d, off16(t->ha_all, j * r), 4 * r, 1, OMX_BF16,
+                                 t->g32 + t->b_off(0, j), OMX_F32, d, N, r, 0, L, s_3d, s_4r, s_c));
+    TRY(omx_gemm_strided_batch(ctx, t->gy_o, 1, d, off16(t->ha_all, 3 * r), 4 * r, 1, OMX_BF16, t->g32 + t->b_off(0, 3),
+                               OMX_F32, d, N, r, 0, L, s_d, s_4r, s_c));
+    TRY(omx_gemm_strided_batch(ctx, t->gh_all, 1, 4 * r, t->h1_all, d, 1, OMX_BF16, t->g32 + t->a_off(0, 0), OMX_F32,
+                               3 * r, N, d, 0, L, s_4r, s_d, s_c));
+    TRY(omx_gemm_strided_batch(ctx, off16(t->gh_all, 3 * r), 1, 4 * r, t->ap_all, d, 1, OMX_BF16,
+                               t->g32 + t->a_off(0, 3), OMX_F32, r, N, d, 0, L, s_4r, s_d, s_c));
   }
   // B reaches the graph as scale * B (lora.rs:309-323): its gradient carries the factor.
   if (c.lora_scale != 1.0f) {
@@ -300,6 +316,13 @@ int32_t olora_create(omx_ctx* ctx, const olora_config* config, olora** out) {
   CREATE_TRY(alloc(t, stage_elems, &t->stage_codes));
   CREATE_TRY(alloc(t, stage_elems / 32 * 4, &t->stage_scales));
   t->layers.resize(L);
+  CREATE_TRY(alloc16(t, L * N * d, &t->h1_all));
+  CREATE_TRY(alloc16(t, L * N * 4 * r, &t->ha_all));
+  CREATE_TRY(alloc16(t, L * N * d, &t->ap_all));
+  CREATE_TRY(alloc16(t, L * N * d, &t->gy_o));
+  CREATE_TRY(alloc16(t, L * N * 3 * d, &t->gqkv_all));
+  CREATE_TRY(alloc16(t, L * N * 4 * r, &t->gh_all));
+  uint64_t layer_index = 0;
   for (auto& A : t->layers) {
     CREATE_TRY(alloc_qmat(t, &A.qkv, 3 * d, d));
     CREATE_TRY(alloc_qmat(t, &A.o, d, d));
@@ -307,10 +330,11 @@ int32_t olora_create(omx_ctx* ctx, const olora_config* config, olora** out) {
     CREATE_TRY(alloc_qmat(t, &A.dn, d, h));
     CREATE_TRY(alloc_t(t, N * d, &A.x));
     CREATE_TRY(alloc_t(t, N * d, &A.x1));
-    CREATE_TRY(alloc16(t, N * d, &A.h1));
-    CREATE_TRY(alloc16(t, N * 4 * r, &A.ha));
+    A.h1 = off16(t->h1_all, layer_index * N * d);
+    A.ha = off16(t->ha_all, layer_index * N * 4 * r);
+    A.ap = off16(t->ap_all, layer_index * N * d);
+    ++layer_index;
     CREATE_TRY(alloc16(t, N * 3 * d, &A.qkv_out));
-    CREATE_TRY(alloc16(t, N * d, &A.ap));
     CREATE_TRY(alloc16(t, N * d, &A.apr));
     CREATE_TRY(alloc16(t, N * 2 * h, &A.gu_out));
     CREATE_TRY(alloc_t(t, static_cast<uint64_t>(c.batch) * c.heads * c.seq, &A.lse));
@@ -357,9 +381,7 @@ int32_t olora_create(omx_ctx* ctx, const olora_config* config, olora** out) {
   CREATE_TRY(alloc16(t, N * d, &t->gy16));
   CREATE_TRY(alloc16(t, N * h, &t->gm));
   CREATE_TRY(alloc16(t, N * 2 * h, &t->ggu));
-  CREATE_TRY(alloc16(t, N * 4 * r, &t->gh));
   CREATE_TRY(alloc16(t, N * d, &t->ga));
-  CREATE_TRY(alloc16(t, N * 3 * d, &t->gqkv));
   CREATE_TRY(alloc16(t, N * d, &t->ghf));
   CREATE_TRY(refresh_operands(t));
 #undef CREATE_TRY
