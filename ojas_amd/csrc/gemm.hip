@@ -351,6 +351,7 @@ __global__ __launch_bounds__(NT) void gemm_kernel(GemmArgs g) {
 }
 
 __global__ void splitk_reduce_kernel(GemmArgs g) {
+  gemm_select_batch(g, blockIdx.y);
   const long total = static_cast<long>(g.M) * g.N;
   bool bad = false;
   for (long i = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x; i < total;
@@ -392,7 +393,7 @@ int32_t launch(omx_ctx* ctx, const GemmArgs& g, bool a_km, bool b_km) {
   if (g.splits > 1) {
     long elems = static_cast<long>(g.M) * g.N;
     unsigned blocks = static_cast<unsigned>(std::min<long>((elems + 255) / 256, 4096));
-    omx_launch_timed(ctx, splitk_reduce_kernel, dim3(blocks), dim3(256), 0, nullptr, ctx->timing_stop, g);
+    omx_launch_timed(ctx, splitk_reduce_kernel, dim3(blocks, g.batches), dim3(256), 0, nullptr, ctx->timing_stop, g);
     OMX_LAUNCH_CHECK(ctx, "splitk_reduce_kernel");
   }
   return OMX_OK;
@@ -517,8 +518,12 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
     int splits = 1;
     // An f32 step is 64 MFMAs per wave (1.7 us): two of them already pay for a split.
     const int min_steps = operand_dtype == OMX_BF16 ? 8 : 2;
-    if (tiles * g.batches < 256 && g.batches == 1 && ksteps >= 4 * min_steps && !(epi && epi->mode != OMX_EPI_NONE)) {
-      splits = static_cast<int>((512 + tiles - 1) / tiles);
+    // A strided batch splits only on the register-staged kernel (thin outputs over a long
+    // reduction: 16 products of 16 tiles each leave three quarters of the chip's wave slots empty).
+    const long all_tiles = tiles * g.batches;
+    const bool may_split = g.batches == 1 ? tiles < 256 : (dma_variant < 0 && all_tiles < 512);
+    if (may_split && ksteps >= 4 * min_steps && !(epi && epi->mode != OMX_EPI_NONE)) {
+      splits = static_cast<int>(((g.batches == 1 ? 512 : 1024) + all_tiles - 1) / all_tiles);
       if (splits > ksteps / min_steps) splits = ksteps / min_steps;
       if (splits < 1) splits = 1;
       if (dma_variant >= 0) {  // a power of two, so that a split stays on one XCD (see gemm_dma_kernel)
@@ -532,7 +537,7 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
     g.partial = nullptr;
     if (g.splits > 1) {
       void* ws = nullptr;
-      int32_t wrc = omx_workspace(ctx, static_cast<uint64_t>(g.splits) * m * n * sizeof(float), &ws, 1);
+      int32_t wrc = omx_workspace(ctx, static_cast<uint64_t>(g.splits) * batches * m * n * sizeof(float), &ws, 1);
       if (wrc != OMX_OK) return wrc;
       g.partial = static_cast<float*>(ws);
     }
@@ -571,7 +576,7 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
     if (rc == OMX_OK && g.splits > 1) {
       long elems = static_cast<long>(g.M) * g.N;
       unsigned blocks = static_cast<unsigned>(std::min<long>((elems + 255) / 256, 4096));
-      omx_launch_timed(ctx, splitk_reduce_kernel, dim3(blocks), dim3(256), 0, nullptr, ctx->timing_stop, g);
+      omx_launch_timed(ctx, splitk_reduce_kernel, dim3(blocks, g.batches), dim3(256), 0, nullptr, ctx->timing_stop, g);
       OMX_LAUNCH_CHECK(ctx, "splitk_reduce_kernel");
     }
   } else if (operand_dtype != OMX_BF16) {

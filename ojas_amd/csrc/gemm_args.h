@@ -35,6 +35,8 @@ __device__ __forceinline__ void gemm_select_batch(GemmArgs& g, int product) {
     g.a = static_cast<const char*>(g.a) + y * g.batch_a;
     g.b = static_cast<const char*>(g.b) + y * g.batch_b;
     g.c = static_cast<char*>(g.c) + y * g.batch_c;
+    // A split product of a batch keeps its partial sums behind the earlier products'.
+    if (g.splits > 1) g.partial += y * g.splits * static_cast<long>(g.M) * g.N;
     // aux tensors are bf16 like the output they accompany: the same byte stride.
     if (g.aux_in) g.aux_in = reinterpret_cast<const unsigned short*>(reinterpret_cast<const char*>(g.aux_in) + y * g.batch_c);
     if (g.aux_out) g.aux_out = reinterpret_cast<unsigned short*>(reinterpret_cast<char*>(g.aux_out) + y * g.batch_c);

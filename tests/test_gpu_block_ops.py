@@ -345,10 +345,14 @@ def test_attention_saved_residual_keeps_the_row_term_exact(be, b, t, h, hkv, win
 
 
 @pytest.mark.parametrize("bf16", [False, True])
-@pytest.mark.parametrize("rows,dim", [(5, 256), (33, 768), (1000, 768), (17, 1024), (9, 260), (40, 96), (12, 2048)])
+@pytest.mark.parametrize("rows,dim", [(5, 256), (33, 768), (1000, 768), (17, 1024), (9, 260), (40, 96), (12, 2048),
+                                      (33, 1284), (70, 2044), (9000, 768), (40000, 512), (5000, 2048)])
 def test_fused_residual_rms_norm_equals_the_separate_ops(be, rows, dim, bf16):
     """block.rs:247-249 (add, then norm) and the tape's fan-in at a residual: the fused entry points
-    must give the bits of the separate calls, and the norm itself must match the oracle."""
+    must give the bits of the separate calls, and the norm itself must match the oracle. The
+    shapes take every form of the backward: whole and ragged 256-column chunks, the wide-row form
+    above 1024 columns, and partial sums for the weight gradient added by one small workgroup, by
+    one launch of 1024-thread workgroups, or in two stages (above 1024 partial rows)."""
     from ojas_amd.backend import BF16, F32
 
     print(f"fused add+rms rows={rows} dim={dim} bf16={bf16}", flush=True)

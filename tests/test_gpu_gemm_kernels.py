@@ -94,6 +94,31 @@ def test_strided_batch_of_weight_gradients(be, mode, rows, kin, nout, layers):
         assert err <= 1e-5 * max(1.0, float(np.max(np.abs(ogw)))), (l, err)
 
 
+@pytest.mark.parametrize("rows,kin,nout,layers", [(4096, 16, 512, 6), (4096, 384, 48, 5), (2048, 8, 256, 16)])
+def test_strided_batch_of_thin_weight_gradients_splits_the_reduction(be, rows, kin, nout, layers):
+    """A batch of thin outputs over a long reduction (an adapter's rank x d gradients over the
+    tokens of every layer): too few tiles to fill the chip, so each product's reduction is split
+    and the partial sums of every product are added by one reduce launch. Outputs at a padded
+    stride, untouched between them."""
+    from ojas_amd.backend import BF16
+
+    print(f"gemm strided batch thin {rows}x{kin}x{nout} layers {layers}", flush=True)
+    be.set_option("gemm_dma", 1)
+    pad = 32
+    r = orc.SplitMix64(7300 + rows + kin + layers)
+    x = orc.round_bf16(r.vec(layers * rows * kin, 0.5)).reshape(layers, rows, kin)
+    gy = orc.round_bf16(r.vec(layers * rows * nout, 0.5)).reshape(layers, rows, nout)
+    stride_c = nout * kin + pad
+    out = be.gemm_strided_batch(be.upload(gy, BF16), (1, nout), be.upload(x, BF16), (kin, 1), nout, rows, kin, layers,
+                                (rows * nout, rows * kin, stride_c))
+    got = be.download(out)
+    for l in range(layers):
+        want = gy[l].astype(np.float64).T @ x[l].astype(np.float64)
+        mine = got[l * stride_c:l * stride_c + nout * kin].reshape(nout, kin).astype(np.float64)
+        err = float(np.max(np.abs(mine - want)))
+        assert err <= 1e-5 * max(1.0, float(np.max(np.abs(want)))), (l, err)
+
+
 def test_strided_batch_refuses_bad_strides(be):
     from ojas_amd.backend import BF16, OjasError
 
