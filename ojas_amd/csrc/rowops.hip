@@ -358,7 +358,8 @@ __global__ __launch_bounds__(1024) void sort_long_segments_kernel(const unsigned
 
 // One wave per table row: zero it, or add its tokens' gradient rows in ascending token order
 // (`sorted`: the row's positions, ascending), so the f32 sums carry the CPU scatter's bits.
-template <typename TG>
+// V = 4: a lane owns four consecutive columns (16-byte accesses; dim a multiple of 4, aligned rows).
+template <typename TG, int V>
 __global__ __launch_bounds__(ROW_THREADS) void embedding_bwd_kernel(const unsigned int* __restrict__ offsets,
                                                                     const unsigned int* __restrict__ sorted,
                                                                     const TG* __restrict__ grad,
@@ -371,28 +372,46 @@ __global__ __launch_bounds__(ROW_THREADS) void embedding_bwd_kernel(const unsign
   const unsigned int begin = offsets[v], end = offsets[v + 1];
   float* dst = table_grad + v * dim;
   if (begin == end) {
-    for (int c = lane; c < dim; c += 64) dst[c] = 0.0f;
+    if constexpr (V == 4) {
+      for (int c = lane * 4; c < dim; c += 256) *reinterpret_cast<float4*>(dst + c) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    } else {
+      for (int c = lane; c < dim; c += 64) dst[c] = 0.0f;
+    }
     return;
   }
   bool bad = false;
+  constexpr int CHUNKS = 8 / V;  // 8 columns per lane and pass
   for (int c0 = 0; c0 < dim; c0 += 64 * 8) {
-    float acc[8];
+    float acc[CHUNKS][V];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
+    for (int j = 0; j < CHUNKS; ++j)
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc[j][e] = 0.0f;
     for (unsigned int s = begin; s < end; ++s) {
       const TG* src = grad + static_cast<size_t>(sorted[s]) * dim;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        int c = c0 + j * 64 + lane;
-        if (c < dim) acc[j] = acc[j] + dev_load<TG>(src, c);
+      for (int j = 0; j < CHUNKS; ++j) {
+        const int c = c0 + (j * 64 + lane) * V;
+        if (c < dim) {
+          if constexpr (V == 4) {
+            float g[4];
+            dev_load4<TG>(src, c, g);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[j][e] = acc[j][e] + g[e];
+          } else {
+            acc[j][0] = acc[j][0] + dev_load<TG>(src, c);
+          }
+        }
       }
     }
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      int c = c0 + j * 64 + lane;
+    for (int j = 0; j < CHUNKS; ++j) {
+      const int c = c0 + (j * 64 + lane) * V;
       if (c < dim) {
-        bad |= !dev_finite(acc[j]);
-        dst[c] = acc[j];
+#pragma unroll
+        for (int e = 0; e < V; ++e) bad |= !dev_finite(acc[j][e]);
+        if constexpr (V == 4) *reinterpret_cast<float4*>(dst + c) = make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
+        else dst[c] = acc[j][0];
       }
     }
   }
@@ -741,14 +760,20 @@ int32_t omx_embedding_backward(omx_ctx* ctx, const void* ids, const void* grad, 
   hipLaunchKernelGGL(sort_long_segments_kernel, dim3(256), dim3(1024), 0, ctx->stream, offsets, positions, sorted,
                      long_count, long_rows, tokens);
   OMX_LAUNCH_CHECK(ctx, "sort_long_segments_kernel");
-  if (grad_dtype == OMX_F32)
-    omx_launch_timed(ctx, embedding_bwd_kernel<float>, vgrid, dim3(ROW_THREADS), 0, nullptr, timer.stop(), offsets,
-                     sorted, static_cast<const float*>(grad), static_cast<float*>(table_grad), vocab,
-                     static_cast<int>(dim), ctx->fault, tag);
-  else
-    omx_launch_timed(ctx, embedding_bwd_kernel<unsigned short>, vgrid, dim3(ROW_THREADS), 0, nullptr, timer.stop(),
-                     offsets, sorted, static_cast<const unsigned short*>(grad), static_cast<float*>(table_grad), vocab,
-                     static_cast<int>(dim), ctx->fault, tag);
+  const bool vec4 = dim % 4 == 0 && (reinterpret_cast<uintptr_t>(grad) & 15u) == 0 &&
+                    (reinterpret_cast<uintptr_t>(table_grad) & 15u) == 0 && (grad_dtype == OMX_F32 || dim % 8 == 0);
+#define EMB_BWD(TG_, V_)                                                                                           \
+  omx_launch_timed(ctx, embedding_bwd_kernel<TG_, V_>, vgrid, dim3(ROW_THREADS), 0, nullptr, timer.stop(), offsets, \
+                   sorted, static_cast<const TG_*>(grad), static_cast<float*>(table_grad), vocab,                  \
+                   static_cast<int>(dim), ctx->fault, tag)
+  if (grad_dtype == OMX_F32) {
+    if (vec4) EMB_BWD(float, 4);
+    else EMB_BWD(float, 1);
+  } else {
+    if (vec4) EMB_BWD(unsigned short, 4);
+    else EMB_BWD(unsigned short, 1);
+  }
+#undef EMB_BWD
   OMX_LAUNCH_CHECK(ctx, "embedding_bwd_kernel");
   return OMX_OK;
 }
