@@ -41,8 +41,8 @@ __device__ __forceinline__ void store_pack(T* __restrict__ p, size_t pack, const
     reinterpret_cast<float4*>(p)[pack] = make_float4(v[0], v[1], v[2], v[3]);
   } else {
     uint2 q;
-    q.x = static_cast<unsigned>(dev_f32_to_bf16_bits(v[0])) | (static_cast<unsigned>(dev_f32_to_bf16_bits(v[1])) << 16);
-    q.y = static_cast<unsigned>(dev_f32_to_bf16_bits(v[2])) | (static_cast<unsigned>(dev_f32_to_bf16_bits(v[3])) << 16);
+    q.x = dev_pack_bf16_pair(v[0], v[1]);
+    q.y = dev_pack_bf16_pair(v[2], v[3]);
     reinterpret_cast<uint2*>(p)[pack] = q;
   }
 }

@@ -66,10 +66,8 @@ __device__ __forceinline__ bool gemm_store4(const GemmArgs& g, int split, int gr
     unsigned short* cp = static_cast<unsigned short*>(g.c) + off;
     if (whole) {
       uint2 w;
-      w.x = static_cast<unsigned int>(dev_f32_to_bf16_bits(x0)) |
-            (static_cast<unsigned int>(dev_f32_to_bf16_bits(x1)) << 16);
-      w.y = static_cast<unsigned int>(dev_f32_to_bf16_bits(x2)) |
-            (static_cast<unsigned int>(dev_f32_to_bf16_bits(x3)) << 16);
+      w.x = dev_pack_bf16_pair(x0, x1);
+      w.y = dev_pack_bf16_pair(x2, x3);
       *reinterpret_cast<uint2*>(cp) = w;
       bad = !(dev_finite(x0) && dev_finite(x1) && dev_finite(x2) && dev_finite(x3));
     } else {
@@ -124,10 +122,8 @@ __device__ __forceinline__ bool gemm_store4_epi(const GemmArgs& g, int split, in
       unsigned short* ap = g.aux_out + off;
       if (whole) {
         uint2 w;
-        w.x = static_cast<unsigned int>(dev_f32_to_bf16_bits(a0)) |
-              (static_cast<unsigned int>(dev_f32_to_bf16_bits(a1)) << 16);
-        w.y = static_cast<unsigned int>(dev_f32_to_bf16_bits(a2)) |
-              (static_cast<unsigned int>(dev_f32_to_bf16_bits(a3)) << 16);
+        w.x = dev_pack_bf16_pair(a0, a1);
+        w.y = dev_pack_bf16_pair(a2, a3);
         *reinterpret_cast<uint2*>(ap) = w;
         bad = !(dev_finite(a0) && dev_finite(a1) && dev_finite(a2) && dev_finite(a3));
       } else {
@@ -187,7 +183,7 @@ __device__ __forceinline__ bool gemm_epilogue_block(const GemmArgs& g, const flo
     if constexpr (EPI != OMX_EPI_GELU_FWD) aux[it] = *reinterpret_cast<const uint2*>(g.aux_in + off[it]);
   }
   auto pack = [](float a, float b) {
-    return static_cast<unsigned int>(dev_f32_to_bf16_bits(a)) | (static_cast<unsigned int>(dev_f32_to_bf16_bits(b)) << 16);
+    return dev_pack_bf16_pair(a, b);
   };
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
@@ -251,10 +247,8 @@ __device__ __forceinline__ bool gemm_store_block(const GemmArgs& g, int split, c
     }
     if constexpr (KIND == 1) {
       uint2 w;
-      w.x = static_cast<unsigned int>(dev_f32_to_bf16_bits(val.x)) |
-            (static_cast<unsigned int>(dev_f32_to_bf16_bits(val.y)) << 16);
-      w.y = static_cast<unsigned int>(dev_f32_to_bf16_bits(val.z)) |
-            (static_cast<unsigned int>(dev_f32_to_bf16_bits(val.w)) << 16);
+      w.x = dev_pack_bf16_pair(val.x, val.y);
+      w.y = dev_pack_bf16_pair(val.z, val.w);
       *reinterpret_cast<uint2*>(hbase + off) = w;
     } else {
       *reinterpret_cast<float4*>(fbase + off) = val;

@@ -311,7 +311,7 @@ struct TileCursor {
 };
 
 __device__ __forceinline__ unsigned int pack_bf16_pair(float a, float b) {
-  return static_cast<unsigned int>(dev_f32_to_bf16_bits(a)) | (static_cast<unsigned int>(dev_f32_to_bf16_bits(b)) << 16);
+  return dev_pack_bf16_pair(a, b);
 }
 // The value lane ^ 1 holds in `x`.
 __device__ __forceinline__ float from_neighbour(float x) {

@@ -22,8 +22,7 @@ __device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
   unsigned int u[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
-    u[i] = static_cast<unsigned int>(dev_f32_to_bf16_bits(f[2 * i])) |
-           (static_cast<unsigned int>(dev_f32_to_bf16_bits(f[2 * i + 1])) << 16);
+    u[i] = dev_pack_bf16_pair(f[2 * i], f[2 * i + 1]);
   return make_uint4(u[0], u[1], u[2], u[3]);
 }
 

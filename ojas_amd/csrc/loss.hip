@@ -89,8 +89,7 @@ __device__ __forceinline__ void ce_store(T* __restrict__ g, unsigned int c, cons
     unsigned int w[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
-      w[j] = static_cast<unsigned int>(dev_f32_to_bf16_bits(v[2 * j])) |
-             (static_cast<unsigned int>(dev_f32_to_bf16_bits(v[2 * j + 1])) << 16);
+      w[j] = dev_pack_bf16_pair(v[2 * j], v[2 * j + 1]);
     *reinterpret_cast<uint4*>(g + c) = make_uint4(w[0], w[1], w[2], w[3]);
   }
 }
@@ -408,15 +407,11 @@ __global__ __launch_bounds__(CE_FUSED_THREADS, 8) void ce_row_fused_kernel(T* __
           for (int j = 0; j < VEC; ++j)
             if (c + j == target) out[j] = target_grad;
         }
-        // Finite values (a non-finite logit has raised the fault): the conversion instruction
-        // rounds to nearest even as dev_f32_to_bf16_bits does.
-        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-        typedef float floatx2 __attribute__((ext_vector_type(2)));
         uint4 w;
-        w.x = __builtin_bit_cast(unsigned int, __builtin_convertvector(floatx2{out[0], out[1]}, bf16x2));
-        w.y = __builtin_bit_cast(unsigned int, __builtin_convertvector(floatx2{out[2], out[3]}, bf16x2));
-        w.z = __builtin_bit_cast(unsigned int, __builtin_convertvector(floatx2{out[4], out[5]}, bf16x2));
-        w.w = __builtin_bit_cast(unsigned int, __builtin_convertvector(floatx2{out[6], out[7]}, bf16x2));
+        w.x = dev_pack_bf16_pair(out[0], out[1]);
+        w.y = dev_pack_bf16_pair(out[2], out[3]);
+        w.z = dev_pack_bf16_pair(out[4], out[5]);
+        w.w = dev_pack_bf16_pair(out[6], out[7]);
         *reinterpret_cast<uint4*>(r + c) = w;
       } else {
 #pragma unroll

@@ -137,8 +137,8 @@ __global__ __launch_bounds__(OPT_THREADS) void adamw_apply_vec_kernel(float* __r
     v4[i] = make_float4(nv[0], nv[1], nv[2], nv[3]);
     if (p_bf16) {
       uint2 q;
-      q.x = static_cast<unsigned>(dev_f32_to_bf16_bits(np[0])) | (static_cast<unsigned>(dev_f32_to_bf16_bits(np[1])) << 16);
-      q.y = static_cast<unsigned>(dev_f32_to_bf16_bits(np[2])) | (static_cast<unsigned>(dev_f32_to_bf16_bits(np[3])) << 16);
+      q.x = dev_pack_bf16_pair(np[0], np[1]);
+      q.y = dev_pack_bf16_pair(np[2], np[3]);
       reinterpret_cast<uint2*>(p_bf16)[i] = q;
     }
   }

@@ -33,7 +33,7 @@ __device__ __forceinline__ uint4 pack8(const float (&v)[8]) {
   unsigned int w[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
-    w[i] = static_cast<unsigned>(dev_f32_to_bf16_bits(v[2 * i])) | (static_cast<unsigned>(dev_f32_to_bf16_bits(v[2 * i + 1])) << 16);
+    w[i] = dev_pack_bf16_pair(v[2 * i], v[2 * i + 1]);
   return make_uint4(w[0], w[1], w[2], w[3]);
 }
 __device__ __forceinline__ void load8f(const float* __restrict__ p, float (&v)[8]) {

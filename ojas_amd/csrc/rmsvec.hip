@@ -94,23 +94,6 @@ struct Raw4<unsigned short> {
   }
 };
 
-// Stores four values; a bf16 destination is rounded by the conversion instruction (round to nearest
-// even, as dev_f32_to_bf16_bits; the two differ in a NaN's payload only, and a kernel that stores
-// through this raises the fault for any non-finite value it writes).
-template <typename T>
-__device__ __forceinline__ void store4_rounded(T* p, const float (&v)[4]) {
-  if constexpr (sizeof(T) == 4) {
-    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
-  } else {
-    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-    typedef float floatx2 __attribute__((ext_vector_type(2)));
-    uint2 q;
-    q.x = __builtin_bit_cast(unsigned int, __builtin_convertvector(floatx2{v[0], v[1]}, bf16x2));
-    q.y = __builtin_bit_cast(unsigned int, __builtin_convertvector(floatx2{v[2], v[3]}, bf16x2));
-    *reinterpret_cast<uint2*>(p) = q;
-  }
-}
-
 // gx = rms_norm_backward(x, w, gy) (+ add_in), optionally also stored as bf16;
 // per-block partial column sums of gy * xhat for the weight gradient.
 // Row bases are wave-uniform (scalar registers) and lane offsets 32 bits wide; all of a row's loads
@@ -244,8 +227,8 @@ __global__ __launch_bounds__(RV_THREADS) void rms_bwd_vec_kernel(
           a.x += aw[0]; a.y += aw[1]; a.z += aw[2]; a.w += aw[3];
           *reinterpret_cast<float4*>(mine + c) = a;
         }
-        store4_rounded<TO>(outr + c, out);
-        if (gx16) store4_rounded<unsigned short>(out16r + c, out);
+        dev_store4<TO>(outr, c, out);
+        if (gx16) dev_store4<unsigned short>(out16r, c, out);
       }
     }
   }

@@ -549,6 +549,34 @@ def test_casts_and_permute_are_bit_exact(be):
         assert np.array_equal(gb, orc.to_bf16(a).transpose(0, 2, 1, 3))
 
 
+def test_bf16_rounding_carries_the_integer_rule_over_every_exponent_and_low_half(be):
+    """The device rounds f32 to bf16 with its conversion instruction; the reference's rule is integer
+    arithmetic on the bits (ojas-core/src/autocast.rs:70-96: round to nearest even on the dropped 16
+    bits, a NaN keeps sign and payload and gains the quiet bit). Every combination of exponent
+    (256, zero / denormals and infinity / NaN included), the kept mantissa's low bit and a full or
+    an empty kept mantissa (ties to even, the carry into the exponent and into infinity), sign and
+    all 65536 values of the dropped half: 134 M patterns, each equal to the rule written in numpy."""
+    low = np.arange(1 << 16, dtype=np.uint32)
+    for sign in (0, 1):
+        for high in (0x00, 0x01, 0x7E, 0x7F):  # kept mantissa bits 22..16
+            exps = np.arange(256, dtype=np.uint32)
+            bits = ((sign << 31) | (exps[:, None] << 23) | (high << 16) | low[None, :]).astype(np.uint32).reshape(-1)
+            x = bits.view(np.float32)
+            nan = (bits & 0x7FFFFFFF) > 0x7F800000
+            wide = bits.astype(np.uint64)
+            rule = np.where(nan, (wide >> 16) | 0x40, (wide + 0x7FFF + ((wide >> 16) & 1)) >> 16).astype(np.uint16)
+            got = be.download(be.to_bf16(be.upload(x)))
+            assert np.array_equal(got, rule), (sign, high, int(np.flatnonzero(got != rule)[0]))
+            rounded = be.download(be.cast_bf16(be.upload(x))).view(np.uint32)
+            assert np.array_equal(rounded, rule.astype(np.uint32) << 16)
+    # and the oracle's own cast is that rule
+    x = (np.arange(1 << 20, dtype=np.uint32) * np.uint32(4099)).view(np.float32)
+    bits = x.view(np.uint32)
+    nan = (bits & 0x7FFFFFFF) > 0x7F800000
+    rule = np.where(nan, (bits >> 16) | 0x40, (bits.astype(np.uint64) + 0x7FFF + ((bits >> 16) & 1)) >> 16).astype(np.uint16)
+    assert np.array_equal(orc.to_bf16(x), rule)
+
+
 def test_argmax_and_topk_are_bit_exact(be):
     from ojas_amd.backend import NON_FINITE, OjasError
 
