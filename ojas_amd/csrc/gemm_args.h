@@ -191,14 +191,18 @@ __device__ __forceinline__ bool gemm_epilogue_block(const GemmArgs& g, const flo
     const float4 val = *reinterpret_cast<const float4*>(staged + row * pitch + piece * 4);
     float x[4] = {val.x, val.y, val.z, val.w};
     if constexpr (EPI == OMX_EPI_GELU_FWD) {
+      // The activation is taken of the value the pre-activation is stored as: one conversion per
+      // pair gives both the stored word and, widened again, the activation's argument.
+      const unsigned int w01 = pack(x[0], x[1]), w23 = pack(x[2], x[3]);
+      const float u[4] = {__uint_as_float(w01 << 16), __uint_as_float(w01 & 0xffff0000u), __uint_as_float(w23 << 16),
+                          __uint_as_float(w23 & 0xffff0000u)};
       float a[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const float u = dev_round_bf16(x[e]);  // the activation is taken of the value the pre-activation is stored as
-        a[e] = TANH ? dev_gelu_tanh_fast(u) : dev_gelu_erf_fast(u);
+        a[e] = TANH ? dev_gelu_tanh_fast(u[e]) : dev_gelu_erf_fast(u[e]);
         bad |= !(dev_finite(x[e]) && dev_finite(a[e]));
       }
-      *reinterpret_cast<uint2*>(cbase + off[it]) = make_uint2(pack(x[0], x[1]), pack(x[2], x[3]));
+      *reinterpret_cast<uint2*>(cbase + off[it]) = make_uint2(w01, w23);
       *reinterpret_cast<uint2*>(g.aux_out + off[it]) = make_uint2(pack(a[0], a[1]), pack(a[2], a[3]));
     } else {
       const float u[4] = {__uint_as_float(aux[it].x << 16), __uint_as_float(aux[it].x & 0xffff0000u),

@@ -33,7 +33,11 @@
 
 namespace {
 
-template <bool A_KM, bool B_KM, int WGM, int WGN, int TM, int TN, int DBK, int NST>
+// EPI: the store pass this instantiation is compiled for (OMX_EPI_*), or OMX_EPI_ANY for the one
+// that chooses at run time. A kernel of its own per store pass keeps each one's code (a few KiB of
+// straight-line stores) and registers out of the others.
+constexpr int OMX_EPI_ANY = -1;
+template <bool A_KM, bool B_KM, int WGM, int WGN, int TM, int TN, int DBK, int NST, int EPI = OMX_EPI_ANY>
 __global__ __launch_bounds__(WGM* WGN * 64, dma_waves_per_simd(WGM* WGN, NST*(WGM* TM + WGN * TN) * 32 * DBK * 2)) void
 gemm_dma_kernel(GemmArgs g) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -227,23 +231,39 @@ gemm_dma_kernel(GemmArgs g) {
     bool stored = false;
     if constexpr (kFastStores) {
       const bool interior = grow0 + 32 <= g.M && gcol0 + TN * 32 <= g.N;
-      if (interior && g.epi == OMX_EPI_NONE && (g.splits > 1 ? (g.N & 3) == 0 : g.c_vec != 0)) {
-        if (g.splits > 1) bad |= gemm_store_block<0, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
-        else if (g.c_bf16) bad |= gemm_store_block<1, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
-        else if (!g.accumulate) bad |= gemm_store_block<2, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
-        else bad |= gemm_store_block<3, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
-        stored = true;
-      } else if (interior && g.epi != OMX_EPI_NONE && g.c_vec != 0) {
-        if (g.epi == OMX_EPI_GELU_FWD) {
-          bad |= g.epi_tanh ? gemm_epilogue_block<OMX_EPI_GELU_FWD, true, PPR>(g, cs, CPW, grow0, gcol0, lane)
-                            : gemm_epilogue_block<OMX_EPI_GELU_FWD, false, PPR>(g, cs, CPW, grow0, gcol0, lane);
-        } else if (g.epi == OMX_EPI_AXPBY) {
-          bad |= gemm_epilogue_block<OMX_EPI_AXPBY, false, PPR>(g, cs, CPW, grow0, gcol0, lane);
-        } else {
-          bad |= g.epi_tanh ? gemm_epilogue_block<OMX_EPI_GELU_BWD, true, PPR>(g, cs, CPW, grow0, gcol0, lane)
-                            : gemm_epilogue_block<OMX_EPI_GELU_BWD, false, PPR>(g, cs, CPW, grow0, gcol0, lane);
+      if constexpr (EPI == OMX_EPI_ANY || EPI == OMX_EPI_NONE) {
+        if (interior && g.epi == OMX_EPI_NONE && (g.splits > 1 ? (g.N & 3) == 0 : g.c_vec != 0)) {
+          if (g.splits > 1) bad |= gemm_store_block<0, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
+          else if (g.c_bf16) bad |= gemm_store_block<1, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
+          else if (!g.accumulate) bad |= gemm_store_block<2, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
+          else bad |= gemm_store_block<3, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
+          stored = true;
         }
-        stored = true;
+      }
+      if constexpr (EPI == OMX_EPI_ANY) {
+        if (!stored && interior && g.epi != OMX_EPI_NONE && g.c_vec != 0) {
+          if (g.epi == OMX_EPI_GELU_FWD) {
+            bad |= g.epi_tanh ? gemm_epilogue_block<OMX_EPI_GELU_FWD, true, PPR>(g, cs, CPW, grow0, gcol0, lane)
+                              : gemm_epilogue_block<OMX_EPI_GELU_FWD, false, PPR>(g, cs, CPW, grow0, gcol0, lane);
+          } else if (g.epi == OMX_EPI_AXPBY) {
+            bad |= gemm_epilogue_block<OMX_EPI_AXPBY, false, PPR>(g, cs, CPW, grow0, gcol0, lane);
+          } else {
+            bad |= g.epi_tanh ? gemm_epilogue_block<OMX_EPI_GELU_BWD, true, PPR>(g, cs, CPW, grow0, gcol0, lane)
+                              : gemm_epilogue_block<OMX_EPI_GELU_BWD, false, PPR>(g, cs, CPW, grow0, gcol0, lane);
+          }
+          stored = true;
+        }
+      } else if constexpr (EPI == OMX_EPI_AXPBY) {
+        if (interior && g.c_vec != 0) {
+          bad |= gemm_epilogue_block<OMX_EPI_AXPBY, false, PPR>(g, cs, CPW, grow0, gcol0, lane);
+          stored = true;
+        }
+      } else if constexpr (EPI != OMX_EPI_NONE) {
+        if (interior && g.c_vec != 0) {
+          bad |= g.epi_tanh ? gemm_epilogue_block<EPI, true, PPR>(g, cs, CPW, grow0, gcol0, lane)
+                            : gemm_epilogue_block<EPI, false, PPR>(g, cs, CPW, grow0, gcol0, lane);
+          stored = true;
+        }
       }
     }
     if (!stored) {
@@ -623,6 +643,13 @@ int32_t launch_dma(omx_ctx* ctx, const GemmArgs& g) {
     }
   }
   auto kernel = &gemm_dma_kernel<A_KM, B_KM, WGM, WGN, TM, TN, DBK, NST>;
+  // The two tiles the dispatcher picks by itself have a kernel per store pass.
+  if constexpr (DBK == 32 && TM * TN <= 4 && NST == 3) {
+    kernel = g.epi == OMX_EPI_GELU_FWD   ? &gemm_dma_kernel<A_KM, B_KM, WGM, WGN, TM, TN, DBK, NST, OMX_EPI_GELU_FWD>
+             : g.epi == OMX_EPI_GELU_BWD ? &gemm_dma_kernel<A_KM, B_KM, WGM, WGN, TM, TN, DBK, NST, OMX_EPI_GELU_BWD>
+             : g.epi == OMX_EPI_AXPBY    ? &gemm_dma_kernel<A_KM, B_KM, WGM, WGN, TM, TN, DBK, NST, OMX_EPI_AXPBY>
+                                         : &gemm_dma_kernel<A_KM, B_KM, WGM, WGN, TM, TN, DBK, NST, OMX_EPI_NONE>;
+  }
   OMX_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    smem));
   omx_launch_timed(ctx, kernel, dim3(g.tiles_m * g.tiles_n * g.splits, g.batches), dim3(WGM * WGN * 64), smem,
