@@ -518,6 +518,18 @@ int32_t omx_per_head_sigmoid_gate_backward(omx_ctx* ctx, const void* input, cons
                                            void* g_bias_f32, void* g_attn, int32_t g_attn_dtype,
                                            uint64_t rows, uint64_t d_model, uint64_t heads,
                                            uint64_t head_dim);
+/* per_head_sigmoid_gate_backward (backend.rs:1883-1905) without its weight gradient: `gz`
+ * [rows, heads] in operand_dtype receives the gradient of the gate's pre-activation, from which
+ * the caller forms grad_weight[h, i] = sum_r gz[r, h] input[r, i] itself. For a caller that
+ * keeps the layers of a model at a fixed stride and adds up every layer's weight gradient in
+ * one omx_gemm_strided_batch at the end of its backward (a 12 x d output over all tokens fills
+ * the chip only with the layers side by side). Every other result is the bits of
+ * omx_per_head_sigmoid_gate_backward. */
+int32_t omx_per_head_sigmoid_gate_backward_deferred(
+    omx_ctx* ctx, const void* input, const void* weight, int32_t operand_dtype, const void* bias_f32,
+    const void* attn, int32_t attn_dtype, const void* gy, int32_t gy_dtype, const void* gates_f32,
+    void* g_input, int32_t g_input_dtype, void* gz, void* g_bias_f32, void* g_attn,
+    int32_t g_attn_dtype, uint64_t rows, uint64_t d_model, uint64_t heads, uint64_t head_dim);
 /* BackendModule::value_residual_blend_forward / _backward (backend.rs:1907-1920;
  * CPU ojas-cpu/src/pointwise.rs:2031-2148): out = (1 - s) v + s v0 with
  * s = sigmoid(lambda); lambda and grad_lambda are one f32 each on the device. */

@@ -820,6 +820,26 @@ class MiBackend:
     def per_head_sigmoid_gate_backward(self, x, w, b, attn, gy, g_input_dtype: Optional[int] = None):
         return self.per_head_sigmoid_gate_backward_saved(x, w, b, attn, gy, None, g_input_dtype)
 
+    def per_head_sigmoid_gate_backward_deferred(self, x, w, b, attn, gy, scales, g_input_dtype: Optional[int] = None):
+        """`per_head_sigmoid_gate_backward_saved` without the weight gradient: returns (grad_input, gz
+        [rows, heads] in the operands' dtype, grad_bias, grad_attn); grad_weight = gz^T input is the
+        caller's (`omx_per_head_sigmoid_gate_backward_deferred`)."""
+        op = "per_head_sigmoid_gate_backward"
+        rows, d_model, heads, dh = self._gate_dims(op, x, w, b, attn)
+        if gy.shape != attn.shape or gy.dtype != attn.dtype:
+            raise OjasError(SHAPE, f"{op}: grad_output {gy.shape} != attn {attn.shape}")
+        if scales is not None and (scales.shape != (rows, heads) or scales.dtype != F32):
+            raise OjasError(SHAPE, f"{op}: gate scale length does not match rows * heads")
+        gxd = x.dtype if g_input_dtype is None else g_input_dtype
+        gx, gz = self.empty(x.shape, gxd), self.empty((rows, heads), x.dtype)
+        gb, ga = self.empty((heads,), F32), self.empty(attn.shape, attn.dtype)
+        self._check(self._lib.omx_per_head_sigmoid_gate_backward_deferred(
+            self._ctx, self._p(x), self._p(w), C.c_int32(x.dtype), self._p(b), self._p(attn), C.c_int32(attn.dtype),
+            self._p(gy), C.c_int32(gy.dtype), self._p(scales), self._p(gx), C.c_int32(gxd), self._p(gz), self._p(gb),
+            self._p(ga), C.c_int32(attn.dtype), C.c_uint64(rows), C.c_uint64(d_model), C.c_uint64(heads),
+            C.c_uint64(dh)))
+        return gx, gz, gb, ga
+
     def qkv_prepare_forward(self, qkv_lin, q_weight, k_weight, cos, sin, heads, kv_heads, head_dim, value0=None, lam=None,
                             eps: float = 1e-6):
         """QK-norm, RoPE and the value blend over a fused q | k | v projection output (`omx_qkv_prepare_forward`):
@@ -997,6 +1017,8 @@ _VALIDATED = {
                                        shapes.per_head_sigmoid_gate_backward_dims(x, w, b, a, gy), 5),
     "per_head_sigmoid_gate_backward_saved": (lambda x, w, b, a, gy, *_a, **_k:
                                              shapes.per_head_sigmoid_gate_backward_dims(x, w, b, a, gy), 5),
+    "per_head_sigmoid_gate_backward_deferred": (lambda x, w, b, a, gy, *_a, **_k:
+                                                shapes.per_head_sigmoid_gate_backward_dims(x, w, b, a, gy), 5),
     "value_residual_blend_forward": (lambda v, v0, lam: shapes.value_residual_blend_forward_dims(v, v0, lam), 3),
     "value_residual_blend_backward": (lambda v, v0, lam, gy: shapes.value_residual_blend_backward_dims(v, v0, lam, gy), 4),
     "cached_attention_forward": (lambda q, kc, vc, kv_len, window=None: shapes.cached_attention_dims(q, kc, vc, kv_len, window), 3),

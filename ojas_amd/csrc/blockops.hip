@@ -564,15 +564,16 @@ int32_t omx_per_head_sigmoid_gate_forward(omx_ctx* ctx, const void* input, const
   return OMX_OK;
 }
 
-int32_t omx_per_head_sigmoid_gate_backward(omx_ctx* ctx, const void* input, const void* weight, int32_t operand_dtype,
-                                           const void* bias, const void* attn, int32_t attn_dtype, const void* gy,
-                                           int32_t gy_dtype, const void* gates_saved, void* g_input,
-                                           int32_t g_input_dtype, void* g_weight, void* g_bias, void* g_attn,
-                                           int32_t g_attn_dtype, uint64_t rows, uint64_t d_model, uint64_t heads,
-                                           uint64_t head_dim) {
+// The backward of the gate. `g_weight` may be null (the weight gradient is then left to the caller)
+// and `gz_out` may be null (gz then lives in the workspace only).
+static int32_t gate_backward_impl(omx_ctx* ctx, const char* op, const void* input, const void* weight,
+                                  int32_t operand_dtype, const void* bias, const void* attn, int32_t attn_dtype,
+                                  const void* gy, int32_t gy_dtype, const void* gates_saved, void* g_input,
+                                  int32_t g_input_dtype, void* g_weight, void* gz_out, void* g_bias, void* g_attn,
+                                  int32_t g_attn_dtype, uint64_t rows, uint64_t d_model, uint64_t heads,
+                                  uint64_t head_dim) {
   OMX_REQUIRE_CTX(ctx);
-  const char* op = "per_head_sigmoid_gate_backward";
-  if (!input || !weight || !bias || !attn || !gy || !g_input || !g_weight || !g_bias || !g_attn)
+  if (!input || !weight || !bias || !attn || !gy || !g_input || !g_bias || !g_attn || (!g_weight && !gz_out))
     return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
   int32_t rc = check_gate(ctx, op, operand_dtype, {attn_dtype, gy_dtype, g_input_dtype, g_attn_dtype}, rows, d_model,
                           heads, head_dim);
@@ -601,7 +602,7 @@ int32_t omx_per_head_sigmoid_gate_backward(omx_ctx* ctx, const void* input, cons
     if (rc != OMX_OK) return rc;
     gates = fresh;
   }
-  void* gz = base + gates_bytes;
+  void* gz = gz_out ? gz_out : static_cast<void*>(base + gates_bytes);
   float* partial = reinterpret_cast<float*>(base + gates_bytes + gz_bytes);
   float* stage = reinterpret_cast<float*>(base + gates_bytes + gz_bytes + partial_bytes);
 
@@ -646,8 +647,35 @@ int32_t omx_per_head_sigmoid_gate_backward(omx_ctx* ctx, const void* input, cons
                      d_model, rows, heads, d_model, 0);
   if (rc != OMX_OK) return rc;
   // grad_weight[h, i] = sum_r gz[r, h] input[r, i]
+  if (!g_weight) return OMX_OK;
   return omx_gemm_impl(ctx, F_GATE_BACKWARD, gz, 1, heads, input, d_model, 1, operand_dtype, g_weight, OMX_F32, d_model,
                        heads, rows, d_model, 0);
+}
+
+int32_t omx_per_head_sigmoid_gate_backward(omx_ctx* ctx, const void* input, const void* weight, int32_t operand_dtype,
+                                           const void* bias, const void* attn, int32_t attn_dtype, const void* gy,
+                                           int32_t gy_dtype, const void* gates_saved, void* g_input,
+                                           int32_t g_input_dtype, void* g_weight, void* g_bias, void* g_attn,
+                                           int32_t g_attn_dtype, uint64_t rows, uint64_t d_model, uint64_t heads,
+                                           uint64_t head_dim) {
+  if (ctx && !g_weight) return omx_fail(ctx, OMX_PLACEMENT, "per_head_sigmoid_gate_backward: null device pointer");
+  return gate_backward_impl(ctx, "per_head_sigmoid_gate_backward", input, weight, operand_dtype, bias, attn, attn_dtype,
+                            gy, gy_dtype, gates_saved, g_input, g_input_dtype, g_weight, nullptr, g_bias, g_attn,
+                            g_attn_dtype, rows, d_model, heads, head_dim);
+}
+
+int32_t omx_per_head_sigmoid_gate_backward_deferred(omx_ctx* ctx, const void* input, const void* weight,
+                                                    int32_t operand_dtype, const void* bias, const void* attn,
+                                                    int32_t attn_dtype, const void* gy, int32_t gy_dtype,
+                                                    const void* gates_saved, void* g_input, int32_t g_input_dtype,
+                                                    void* gz_out, void* g_bias, void* g_attn, int32_t g_attn_dtype,
+                                                    uint64_t rows, uint64_t d_model, uint64_t heads,
+                                                    uint64_t head_dim) {
+  if (ctx && !gz_out)
+    return omx_fail(ctx, OMX_PLACEMENT, "per_head_sigmoid_gate_backward_deferred: null device pointer");
+  return gate_backward_impl(ctx, "per_head_sigmoid_gate_backward_deferred", input, weight, operand_dtype, bias, attn,
+                            attn_dtype, gy, gy_dtype, gates_saved, g_input, g_input_dtype, nullptr, gz_out, g_bias,
+                            g_attn, g_attn_dtype, rows, d_model, heads, head_dim);
 }
 
 int32_t omx_value_residual_blend_forward(omx_ctx* ctx, const void* value, const void* value0, const void* lambda,

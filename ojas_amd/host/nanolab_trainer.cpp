@@ -84,6 +84,7 @@ struct onano {
   void *gyy = nullptr, *gap = nullptr, *gq = nullptr, *gk = nullptr, *gv = nullptr, *g_raw_v = nullptr, *part_v0 = nullptr;
   void *g_v0 = nullptr;                  // [N, KV D] AD: what the later blocks' blends send to block 0's v
   void *g_qkv = nullptr, *g_qkv_lin = nullptr, *gqkv_all = nullptr;  // fused projection: gradients [N, P3] AD
+  void* gz_all = nullptr;  // the gates' pre-activation gradients [layers][N, heads] AD (deferred weight gradients)
   float* v0_acc = nullptr;               // the same as g_v0 in f32 (fused projection)
   void *gqp = nullptr, *gkp = nullptr, *gvp = nullptr, *gap_p = nullptr;  // permuted gradients (row kernels)
   void *gy16 = nullptr, *ghf = nullptr;
@@ -287,9 +288,14 @@ int32_t backward(onano* t, float loss_seed) {
     gy = AD == OMX_BF16 ? static_cast<const void*>(t->fused_mlp ? copy_o : copy16) : static_cast<const void*>(t->gres1);
     // x1 = x + o(gate(h) * attention)
     TRY(omx_linear_backward(ctx, A.y, t->w(t->li(l, WO)), gy, AD, t->gyy, AD, gw(WO), OMX_F32, N, qd, d));
-    TRY(omx_per_head_sigmoid_gate_backward(ctx, A.h, t->w(t->li(l, GATE_W)), AD, t->w32(t->li(l, GATE_B)), A.ap, AD, t->gyy,
-                                           AD, A.gates, t->gh, OMX_F32, t->g(t->li(l, GATE_W)), t->g(t->li(l, GATE_B)),
-                                           t->gap, AD, N, d, H, D));
+    if (defer && t->gz_all)  // the gate's weight gradient waits for the batched product below
+      TRY(omx_per_head_sigmoid_gate_backward_deferred(ctx, A.h, t->w(t->li(l, GATE_W)), AD, t->w32(t->li(l, GATE_B)), A.ap,
+                                                      AD, t->gyy, AD, A.gates, t->gh, OMX_F32, slice(t->gz_all, l, N * H),
+                                                      t->g(t->li(l, GATE_B)), t->gap, AD, N, d, H, D));
+    else
+      TRY(omx_per_head_sigmoid_gate_backward(ctx, A.h, t->w(t->li(l, GATE_W)), AD, t->w32(t->li(l, GATE_B)), A.ap, AD,
+                                             t->gyy, AD, A.gates, t->gh, OMX_F32, t->g(t->li(l, GATE_W)),
+                                             t->g(t->li(l, GATE_B)), t->gap, AD, N, d, H, D));
     if (t->fused_qkv) {
       const uint64_t P3 = qd + 2 * kd;
       char* prepared = static_cast<char*>(A.qkv);
@@ -375,6 +381,10 @@ int32_t backward(onano* t, float loss_seed) {
       TRY(omx_gemm_strided_batch(ctx, p.gy, 1, p.out, p.x, p.in, 1, AD, t->g(t->li(0, p.which)), OMX_F32, p.out, N, p.in, 0,
                                  layers, N * p.out, N * p.in, per_layer));
     }
+    // The gates' weight gradients: heads x d each over all tokens, every block in one launch.
+    if (t->gz_all)
+      TRY(omx_gemm_strided_batch(ctx, t->gz_all, 1, H, t->h_all, d, 1, AD, t->g(t->li(0, GATE_W)), OMX_F32, H, N, d, 0, layers,
+                               N * H, N * d, per_layer));
   }
   // The tied table: the head's gradient first, then the embedding's rows.
   TRY(omx_embedding_backward(ctx, t->ids, t->gres, OMX_F32, t->g_emb, N, c.vocab, d));
@@ -509,6 +519,8 @@ int32_t onano_create(omx_ctx* ctx, const onano_config* config, onano** out) {
     CREATE_TRY(alloc_act(t, L * N * d, &t->gyd_all));
     CREATE_TRY(alloc_act(t, L * 2 * N * Hd, &t->ggu_all));
     CREATE_TRY(alloc_act(t, L * N * d, &t->gyo_all));
+    // (a strided batch wants its products 16 bytes apart at least)
+    if ((N * c.heads * t->asz) % 16 == 0) CREATE_TRY(alloc_act(t, L * N * c.heads, &t->gz_all));
     if (t->fused_qkv) {
       CREATE_TRY(alloc_act(t, L * N * (qd + 2 * kd), &t->gqkv_all));
     } else {

@@ -345,6 +345,34 @@ def test_attention_saved_residual_keeps_the_row_term_exact(be, b, t, h, hkv, win
 
 
 @pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("rows,d_model,heads,head_dim", [(64, 96, 3, 8), (300, 256, 12, 64), (1024, 768, 12, 64)])
+def test_gate_backward_without_its_weight_gradient(be, rows, d_model, heads, head_dim, bf16):
+    """`per_head_sigmoid_gate_backward_deferred` gives the bits of `per_head_sigmoid_gate_backward`
+    for the input, bias and attention gradients, and a `gz` whose product with the input is that
+    op's weight gradient (to the tolerance of a sum taken in another order)."""
+    from ojas_amd.backend import BF16, F32
+
+    print(f"gate deferred rows={rows} d={d_model} heads={heads} dim={head_dim} bf16={bf16}", flush=True)
+    up, tol, rnd = tier(be, bf16)
+    r = orc.SplitMix64(9100 + rows + heads)
+    x = rnd(r.vec(rows * d_model, 1.0)).reshape(1, rows, d_model)
+    w = rnd(r.vec(heads * d_model, 0.2)).reshape(heads, d_model)
+    b = r.vec(heads, 0.5)
+    attn = rnd(r.vec(rows * heads * head_dim, 1.0)).reshape(1, rows, heads, head_dim)
+    gy = rnd(r.vec(rows * heads * head_dim, 1.0)).reshape(1, rows, heads, head_dim)
+    dx, dw, db, da, dgy = up(x), up(w), be.upload(b), up(attn), up(gy)
+    _, scales = be.per_head_sigmoid_gate_forward_saving(dx, dw, db, da)
+    gx, gw, gb, ga = be.per_head_sigmoid_gate_backward_saved(dx, dw, db, da, dgy, scales, F32)
+    gx2, gz, gb2, ga2 = be.per_head_sigmoid_gate_backward_deferred(dx, dw, db, da, dgy, scales, F32)
+    assert np.array_equal(be.download(gx), be.download(gx2))
+    assert np.array_equal(be.download(gb), be.download(gb2))
+    assert np.array_equal(be.download(ga), be.download(ga2))
+    z = be.download_f32(gz).astype(np.float64).reshape(rows, heads)
+    want = z.T @ be.download_f32(dx).astype(np.float64).reshape(rows, d_model)
+    close(be.download(gw), want, max(tol, 1e-5), "gz^T input against the op's weight gradient")
+
+
+@pytest.mark.parametrize("bf16", [False, True])
 @pytest.mark.parametrize("rows,dim", [(5, 256), (33, 768), (1000, 768), (17, 1024), (9, 260), (40, 96), (12, 2048),
                                       (33, 1284), (70, 2044), (9000, 768), (40000, 512), (5000, 2048)])
 def test_fused_residual_rms_norm_equals_the_separate_ops(be, rows, dim, bf16):
