@@ -39,6 +39,12 @@ uint64_t ogpt_param_len(ogpt* t, uint64_t index);
 int32_t ogpt_set_param(ogpt* t, uint64_t index, const float* host);
 int32_t ogpt_get_param(ogpt* t, uint64_t index, float* host);
 int32_t ogpt_get_grad(ogpt* t, uint64_t index, float* host);
+/* Optimizer state, for a run that resumes (TrainState, ojas-model/src/trainer.rs:300-330): slot 0 is
+ * AdamW's first moment or, under ogpt_step_hybrid, a matrix's Muon momentum; slot 1 AdamW's second
+ * moment; ogpt_set_steps sets the count that AdamW's bias correction starts from. */
+int32_t ogpt_get_state(ogpt* t, uint64_t index, uint32_t slot, float* host);
+int32_t ogpt_set_state(ogpt* t, uint64_t index, uint32_t slot, const float* host);
+int32_t ogpt_set_steps(ogpt* t, uint64_t steps);
 /* N(0, 0.02) matrices and tables from a seeded generator, norm weights 1, moments 0. */
 int32_t ogpt_init(ogpt* t, uint64_t seed);
 

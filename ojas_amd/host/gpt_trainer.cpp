@@ -457,6 +457,23 @@ int32_t ogpt_get_grad(ogpt* t, uint64_t index, float* host) {
   return omx_download(t->ctx, host, t->g32, s.offset * 4, s.len * 4);
 }
 
+int32_t ogpt_get_state(ogpt* t, uint64_t index, uint32_t slot, float* host) {
+  if (!t || index >= t->slots.size() || !host || slot > 1) return OMX_SHAPE;
+  const Slot& s = t->slots[index];
+  return omx_download(t->ctx, host, slot == 0 ? t->m1 : t->m2, s.offset * 4, s.len * 4);
+}
+int32_t ogpt_set_state(ogpt* t, uint64_t index, uint32_t slot, const float* host) {
+  if (!t || index >= t->slots.size() || !host || slot > 1) return OMX_SHAPE;
+  const Slot& s = t->slots[index];
+  t->tracked = ogpt::kNone;  // the next AdamW pass checks its operands again
+  return omx_upload(t->ctx, slot == 0 ? t->m1 : t->m2, s.offset * 4, host, s.len * 4);
+}
+int32_t ogpt_set_steps(ogpt* t, uint64_t steps) {
+  if (!t) return OMX_BACKEND;
+  t->steps = steps;
+  return OMX_OK;
+}
+
 int32_t ogpt_init(ogpt* t, uint64_t seed) {
   if (!t) return OMX_BACKEND;
   std::mt19937_64 rng(seed);

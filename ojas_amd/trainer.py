@@ -89,6 +89,20 @@ class GptTrainer:
     def grads(self) -> List[np.ndarray]:
         return self._get(self._lib.ogpt_get_grad)
 
+    def state(self, slot: int) -> List[np.ndarray]:
+        """Every parameter's optimizer state: slot 0 the first moment (Muon's momentum for a matrix
+        under `step_hybrid`), slot 1 AdamW's second moment."""
+        return self._get(lambda h, i, a: self._lib.ogpt_get_state(h, i, C.c_uint32(slot), a))
+
+    def set_state(self, slot: int, arrays):
+        for i, a in enumerate(arrays):
+            a = np.ascontiguousarray(a, np.float32).reshape(-1)
+            self.backend._check(self._lib.ogpt_set_state(self._h, C.c_uint64(i), C.c_uint32(slot),
+                                                         a.ctypes.data_as(C.c_void_p)))
+
+    def set_steps(self, steps: int):
+        self.backend._check(self._lib.ogpt_set_steps(self._h, C.c_uint64(steps)))
+
     def init(self, seed: int):
         self.backend._check(self._lib.ogpt_init(self._h, C.c_uint64(seed)))
 

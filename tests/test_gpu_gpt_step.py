@@ -140,6 +140,44 @@ def test_steps_with_the_skipped_adamw_check_equal_steps_with_it(be):
     assert all(np.array_equal(a, b) for a, b in zip(results[0][1], results[1][1]))
 
 
+@pytest.mark.parametrize("hybrid", [False, True])
+def test_a_trainer_resumed_from_exported_state_takes_the_same_steps(be, hybrid):
+    """Parameters, both state slots and the step count carried into a fresh trainer
+    (`ogpt_get_state` / `ogpt_set_state` / `ogpt_set_steps`) give, bit for bit, the steps the first
+    trainer goes on to take."""
+    from ojas_amd.backend import AdamWConfig, MuonNs5Config
+    from ojas_amd.trainer import GptConfig, GptTrainer, synthetic_batch
+
+    cfg = GptConfig(*SMALL, 1)
+    adam = AdamWConfig.nanolab(3e-3, 0.1)
+    muon = MuonNs5Config(0.02, 0.95, 0.1, 1, 1)
+    ids, targets = synthetic_batch(cfg, 21)
+
+    def step(tr):
+        return tr.step_hybrid(muon, adam, 1.0) if hybrid else tr.step(adam, 1.0)
+
+    first = GptTrainer(be, cfg)
+    first.set_params(make_params(first.param_lens(), cfg.d_model, 6, 0.05))
+    first.set_batch(ids, targets)
+    for _ in range(3):
+        step(first)
+    params, m1, m2, steps = first.params(), first.state(0), first.state(1), first.steps()
+    assert steps == 3 and any(np.any(m != 0) for m in m1)
+    second = GptTrainer(be, cfg)
+    second.set_params(params)
+    second.set_state(0, m1)
+    second.set_state(1, m2)
+    second.set_steps(steps)
+    second.set_batch(ids, targets)
+    for _ in range(2):
+        assert step(first) == step(second)
+    assert second.steps() == 5
+    assert all(np.array_equal(a, b) for a, b in zip(first.params(), second.params()))
+    assert all(np.array_equal(a, b) for a, b in zip(first.state(1), second.state(1)))
+    first.close()
+    second.close()
+
+
 def hybrid_expectation(params, grads, d, mlp, bf16, lr_adamw):
     """The oracle's hybrid update of every parameter from `grads` (already clipped): Muon-NS5 on the
     six hidden matrices of a layer, AdamW on tables and norms. Returns [(kind, want)]."""
