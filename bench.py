@@ -226,6 +226,51 @@ def kv_decode(args) -> int:
     return 0
 
 
+def attention(args) -> int:
+    """Secondary workload: the training step's attention alone, forward + backward of one block's
+    causal attention at the headline shape (batch 16, 12 heads, 1024 tokens, head_dim 64, bf16)
+    through `causal_sdpa_forward` / `causal_sdpa_backward`. `value` is causal-counted TFLOP/s over
+    both passes (forward 2 B H T^2 D, backward 5 B H T^2 D)."""
+    from ojas_amd.backend import BF16, MiBackend
+
+    b, h, t, d = 16, 12, 1024, 64
+    be = MiBackend(0)
+    r = np.random.default_rng(0)
+    q, k, v, gy = (be.upload(r.standard_normal((b, h, t, d)).astype(np.float32), BF16) for _ in range(4))
+    out, lse = be.causal_sdpa_forward(q, k, v, None, BF16)
+    times = {}
+    for name, fn in (("forward", lambda: be.causal_sdpa_forward(q, k, v, None, BF16)),
+                     ("backward", lambda: be.causal_sdpa_backward(q, k, v, out, lse, gy, None, BF16))):
+        for _ in range(args.warmup):
+            fn()
+        be.sync()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fn()
+        be.sync()
+        times[name] = (time.perf_counter() - t0) / args.steps
+    unit = 2.0 * b * h * t * t * d
+    flops = {"forward": unit, "backward": 2.5 * unit}
+    total = sum(times.values())
+    line = {
+        "metric": "causal attention forward + backward (B16 H12 T1024 D64 bf16): causal-counted TFLOP/s",
+        "value": sum(flops.values()) / total / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": total * 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "causal_sdpa_forward + causal_sdpa_backward: q, k, v [16,12,1024,64] bf16",
+                   "tokens_per_step": b * t},
+        "roofline": {"bound": "mfma", "kernel": "flash_fwd_kernel; flash_key_mean_kernel + flash_bwd_dq_kernel + "
+                                                "flash_bwd_dkv_kernel",
+                     "achieved": sum(flops.values()) / total / 1e12, "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": sum(flops.values()) / total / 1e12 / BF16_MFMA_PEAK_TFLOPS, "traffic": None},
+        "us": {name: dt * 1e6 for name, dt in times.items()},
+        "tflops": {name: flops[name] / dt / 1e12 for name, dt in times.items()},
+    }
+    be.close()
+    print(json.dumps(line))
+    return 0
+
+
 def lora_cpu_baseline(cfg, threads: int):
     """Times the oracle's LoRA step on a bounded sample of the same model at full width: one short
     sequence, once with one block and once with two; the difference is a block's time, the rest the
@@ -507,14 +552,17 @@ def main() -> int:
     ap.add_argument("--optimizer", default="adamw", choices=["adamw", "muon"],
                     help="adamw: BASELINE configs[2], the headline (default); muon: configs[3], Muon-NS5 (bf16 "
                          "iteration, lr 0.02, momentum 0.95) on the hidden matrices and AdamW on tables and norms")
-    ap.add_argument("--workload", default="train_step", choices=["train_step", "kv_decode"],
-                    help="train_step: the headline metric (default); kv_decode: the decode attention op alone")
+    ap.add_argument("--workload", default="train_step", choices=["train_step", "kv_decode", "attention"],
+                    help="train_step: the headline metric (default); kv_decode: the decode attention op alone; "
+                         "attention: the step's causal attention alone, forward + backward")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).", file=sys.stderr)
         return 2
     if args.workload == "kv_decode":
         return kv_decode(args)
+    if args.workload == "attention":
+        return attention(args)
     if args.config == "lora1b":
         return lora_step(args)
     if args.config == "nanolab124m":
