@@ -297,7 +297,16 @@ __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_fwd_kernel(const un
         for (int kk = 0; kk < KK; ++kk) sc[sub] = mfma(frag_rows<D>(k_rows, sub, kk, l32, lg), qf[kk], sc[sub]);
       // Only a tile that crosses the diagonal, the sequence end or the window edge needs the mask
       // (wave-uniform). `m` is the running maximum of the raw scores; the scale joins inside the fma.
-      if (key0 + 63 > wave_q0 || key0 + 63 >= T || s.window > 0) {
+      if (s.window == 0 && key0 + 63 < T) {
+        // The diagonal alone: key > q_row is one compare of a constant with the lane's offset.
+        if (key0 + 63 > wave_q0) {
+          const int rel = q_row - key0 - 4 * lg;
+#pragma unroll
+          for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+            for (int vv = 0; vv < 16; ++vv) sc[sub][vv] = sub * 32 + acc_row(vv, 0) > rel ? -INFINITY : sc[sub][vv];
+        }
+      } else if (key0 + 63 > wave_q0 || key0 + 63 >= T || s.window > 0) {
 #pragma unroll
         for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
@@ -457,6 +466,8 @@ __device__ __forceinline__ bool flash_dkv_block(const unsigned short* __restrict
     if (!active) continue;
     // Wave-uniform: a tile whose queries all come after the wave's keys and end inside the sequence has no mask.
     const bool needs_mask = q0 < wave_k0 + 31 || q0 + 63 >= T || s.window > 0;
+    // Wave-uniform: the tile and the wave's keys end inside the sequence and only the diagonal cuts it.
+    const bool diagonal_only = needs_mask && s.window == 0 && q0 + 63 < T && wave_k0 + 31 < T;
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub) {
       floatx16 sc = zero16(), dp = zero16();
@@ -465,7 +476,11 @@ __device__ __forceinline__ bool flash_dkv_block(const unsigned short* __restrict
         sc = mfma(frag_rows<D>(q_rows, sub, kk, l32, lg), kf[kk], sc);
         if constexpr (WANT_DK) dp = mfma(frag_rows<D>(g_rows, sub, kk, l32, lg), vf[kk], dp);
       }
-      if (needs_mask) {
+      if (diagonal_only) {
+        const int rel = key_row - q0 - 4 * lg;  // key_row > query: a constant against the lane's offset
+#pragma unroll
+        for (int vv = 0; vv < 16; ++vv) sc[vv] = sub * 32 + acc_row(vv, 0) < rel ? -INFINITY : sc[vv];
+      } else if (needs_mask) {
 #pragma unroll
         for (int vv = 0; vv < 16; ++vv) {
           const int qi = q0 + sub * 32 + acc_row(vv, lg);
@@ -682,6 +697,8 @@ __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_bwd_dq_kernel(
       const bool active = key0 <= wave_q0 + 31 && (s.window == 0 || key0 + 63 + s.window > wave_q0);
       if (!active) continue;
       const bool needs_mask = key0 + 63 > wave_q0 || key0 + 63 >= T || s.window > 0;
+      // Wave-uniform: the tile and the wave's rows end inside the sequence and only the diagonal cuts it.
+      const bool diagonal_only = needs_mask && s.window == 0 && key0 + 63 < T && wave_q0 + 31 < T;
 #pragma unroll
       for (int sub = 0; sub < 2; ++sub) {
         floatx16 sc = zero16(), dp = zero16();
@@ -690,7 +707,11 @@ __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_bwd_dq_kernel(
           sc = mfma(frag_rows<D>(k_rows, sub, kk, l32, lg), qf[kk], sc);
           dp = mfma(frag_rows<D>(v_rows, sub, kk, l32, lg), gf[kk], dp);
         }
-        if (needs_mask) {
+        if (diagonal_only) {
+          const int rel = q_row - key0 - 4 * lg;  // key > q_row: a constant against the lane's offset
+#pragma unroll
+          for (int vv = 0; vv < 16; ++vv) sc[vv] = sub * 32 + acc_row(vv, 0) > rel ? -INFINITY : sc[vv];
+        } else if (needs_mask) {
 #pragma unroll
           for (int vv = 0; vv < 16; ++vv) {
             const int key = key0 + sub * 32 + acc_row(vv, lg);
