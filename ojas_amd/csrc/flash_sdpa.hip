@@ -67,6 +67,12 @@ __device__ __forceinline__ float sum_pairs(unsigned int w, float acc) {
   return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16_pair, w), __builtin_bit_cast(bf16_pair, 0x3F803F80u),
                                          acc, false);
 }
+// acc + the products of the two bf16 halves of a and b (v_dot2c_f32_bf16; a product of two bf16
+// values is exact in f32).
+__device__ __forceinline__ float dot_pairs(unsigned int a, unsigned int b, float acc) {
+  typedef __bf16 bf16_pair __attribute__((ext_vector_type(2)));
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16_pair, a), __builtin_bit_cast(bf16_pair, b), acc, false);
+}
 __device__ __forceinline__ floatx16 mfma(const u32x4& a, const u32x4& b, floatx16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
                                                  0, 0);
@@ -637,10 +643,7 @@ __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_bwd_dq_kernel(
           const unsigned int gw[4] = {gf[kk].x, gf[kk].y, gf[kk].z, gf[kk].w};
           const unsigned int ow[4] = {of[kk].x, of[kk].y, of[kk].z, of[kk].w};
 #pragma unroll
-          for (int w = 0; w < 4; ++w) {
-            sum += __uint_as_float(gw[w] << 16) * __uint_as_float(ow[w] << 16);
-            sum += __uint_as_float(gw[w] & 0xffff0000u) * __uint_as_float(ow[w] & 0xffff0000u);
-          }
+          for (int w = 0; w < 4; ++w) sum = dot_pairs(gw[w], ow[w], sum);
         }
         return sum;
       };
