@@ -326,6 +326,14 @@ int32_t omx_embedding_forward(omx_ctx* ctx, const void* table, int32_t table_dty
 int32_t omx_embedding_backward(omx_ctx* ctx, const void* ids_u32, const void* grad,
                                int32_t grad_dtype, void* table_grad_f32, uint64_t tokens,
                                uint64_t vocab, uint64_t dim);
+/* embedding_backward followed by accumulate_grad onto `table_grad_f32` (backend.rs:1620-1626, then
+ * the tape's sum of the gradients of a value used twice, as a tied table is,
+ * ojas-autograd/src/tape.rs:2551-2585) in one pass:
+ * each named row's sum is formed as above, then added to what the row holds; rows no token names
+ * are neither read nor written. The bits are those of the two ops in sequence. */
+int32_t omx_embedding_backward_accumulate(omx_ctx* ctx, const void* ids_u32, const void* grad,
+                                          int32_t grad_dtype, void* table_grad_f32,
+                                          uint64_t tokens, uint64_t vocab, uint64_t dim);
 
 /* ---- optimizers ---- */
 /* ojas_core::AdamWConfig (backend.rs:494-517). */

@@ -106,6 +106,7 @@ extern "C" {
     pub fn omx_linear_cross_entropy_mean(ctx: *mut OmxCtx, x: *const c_void, w: *const c_void, operand_dtype: i32, targets_u32: *const c_void, rows: u64, dim: u64, vocab: u64, has_ignore: i32, ignore_index: u32, chunk_rows: u64, chunk_cols: u64, loss_f32: *mut c_void, gx: *mut c_void, gx_dtype: i32, gw_f32: *mut c_void) -> i32;
     pub fn omx_embedding_forward(ctx: *mut OmxCtx, table: *const c_void, table_dtype: i32, ids_u32: *const c_void, out: *mut c_void, out_dtype: i32, tokens: u64, vocab: u64, dim: u64) -> i32;
     pub fn omx_embedding_backward(ctx: *mut OmxCtx, ids_u32: *const c_void, grad: *const c_void, grad_dtype: i32, table_grad_f32: *mut c_void, tokens: u64, vocab: u64, dim: u64) -> i32;
+    pub fn omx_embedding_backward_accumulate(ctx: *mut OmxCtx, ids_u32: *const c_void, grad: *const c_void, grad_dtype: i32, table_grad_f32: *mut c_void, tokens: u64, vocab: u64, dim: u64) -> i32;
     pub fn omx_adamw_step(ctx: *mut OmxCtx, param_f32: *mut c_void, grad_f32: *const c_void, moment1_f32: *mut c_void, moment2_f32: *mut c_void, n: u64, step: u64, config: *const OmxAdamwConfig, param_bf16: *mut c_void) -> i32;
     pub fn omx_adamw_step_bounded(ctx: *mut OmxCtx, param_f32: *mut c_void, grad_f32: *const c_void, moment1_f32: *mut c_void, moment2_f32: *mut c_void, n: u64, step: u64, config: *const OmxAdamwConfig, param_bf16: *mut c_void, inputs_bounded: i32, unbounded_flag: *mut c_void) -> i32;
     pub fn omx_muon_ns5_step(ctx: *mut OmxCtx, param_f32: *mut c_void, grad_f32: *const c_void, momentum_f32: *mut c_void, rows: u64, cols: u64, config: *const OmxMuonConfig, param_bf16: *mut c_void) -> i32;

@@ -591,6 +591,16 @@ class MiBackend:
                                                      C.c_uint64(dim)))
         return out
 
+    def embedding_backward_accumulate(self, ids, grad, table_grad):
+        """`embedding_backward` then `accumulate_grad` onto `table_grad` (f32 [vocab, dim]) in one
+        pass over the rows the ids name (`omx_embedding_backward_accumulate`)."""
+        vocab, dim = table_grad.shape
+        if table_grad.dtype != F32 or grad.shape[-1] != dim:
+            raise OjasError(SHAPE, f"embedding_backward_accumulate: grad {grad.shape} against table_grad {table_grad.shape}")
+        self._check(self._lib.omx_embedding_backward_accumulate(
+            self._ctx, self._p(ids), self._p(grad), C.c_int32(grad.dtype), self._p(table_grad), C.c_uint64(ids.numel),
+            C.c_uint64(vocab), C.c_uint64(dim)))
+
     # ---- optimizers (in place) ----
     def adamw_step(self, param, grad, moment1, moment2, step: int, config: AdamWConfig, param_bf16=None):
         self._check(self._lib.omx_adamw_step(self._ctx, self._p(param), self._p(grad), self._p(moment1),

@@ -359,7 +359,9 @@ __global__ __launch_bounds__(1024) void sort_long_segments_kernel(const unsigned
 // One wave per table row: zero it, or add its tokens' gradient rows in ascending token order
 // (`sorted`: the row's positions, ascending), so the f32 sums carry the CPU scatter's bits.
 // V = 4: a lane owns four consecutive columns (16-byte accesses; dim a multiple of 4, aligned rows).
-template <typename TG, int V>
+// ADD: the row's sum, complete, is added to what `table_grad` holds (the bits of the scatter
+// followed by accumulate_grad), and rows no token names are left alone.
+template <typename TG, int V, bool ADD>
 __global__ __launch_bounds__(ROW_THREADS) void embedding_bwd_kernel(const unsigned int* __restrict__ offsets,
                                                                     const unsigned int* __restrict__ sorted,
                                                                     const TG* __restrict__ grad,
@@ -372,6 +374,7 @@ __global__ __launch_bounds__(ROW_THREADS) void embedding_bwd_kernel(const unsign
   const unsigned int begin = offsets[v], end = offsets[v + 1];
   float* dst = table_grad + v * dim;
   if (begin == end) {
+    if constexpr (ADD) return;
     if constexpr (V == 4) {
       for (int c = lane * 4; c < dim; c += 256) *reinterpret_cast<float4*>(dst + c) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     } else {
@@ -410,6 +413,17 @@ __global__ __launch_bounds__(ROW_THREADS) void embedding_bwd_kernel(const unsign
       if (c < dim) {
 #pragma unroll
         for (int e = 0; e < V; ++e) bad |= !dev_finite(acc[j][e]);
+        if constexpr (ADD) {
+          if constexpr (V == 4) {
+            const float4 old = *reinterpret_cast<const float4*>(dst + c);
+            acc[j][0] = old.x + acc[j][0];
+            acc[j][1] = old.y + acc[j][1];
+            acc[j][2] = old.z + acc[j][2];
+            acc[j][3] = old.w + acc[j][3];
+          } else {
+            acc[j][0] = dst[c] + acc[j][0];
+          }
+        }
         if constexpr (V == 4) *reinterpret_cast<float4*>(dst + c) = make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
         else dst[c] = acc[j][0];
       }
@@ -713,10 +727,10 @@ int32_t omx_embedding_forward(omx_ctx* ctx, const void* table, int32_t table_dty
   return OMX_OK;
 }
 
-int32_t omx_embedding_backward(omx_ctx* ctx, const void* ids, const void* grad, int32_t grad_dtype, void* table_grad,
-                               uint64_t tokens, uint64_t vocab, uint64_t dim) {
+static int32_t embedding_backward_impl(omx_ctx* ctx, const void* ids, const void* grad, int32_t grad_dtype,
+                                       void* table_grad, uint64_t tokens, uint64_t vocab, uint64_t dim, bool add) {
   OMX_REQUIRE_CTX(ctx);
-  const char* op = "embedding_backward";
+  const char* op = add ? "embedding_backward_accumulate" : "embedding_backward";
   if (!ids || !grad || !table_grad) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
   if (!omx_valid_float_dtype(grad_dtype)) return omx_fail(ctx, OMX_DTYPE, "%s: dtype must be f32 or bf16", op);
   if (tokens == 0 || vocab == 0 || dim == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
@@ -742,10 +756,12 @@ int32_t omx_embedding_backward(omx_ctx* ctx, const void* ids, const void* grad, 
   if (rc != OMX_OK) return rc;
   const unsigned int* idp = static_cast<const unsigned int*>(ids);
   dim3 tgrid(static_cast<unsigned>((tokens + 255) / 256));
-  // Bytes: every gradient row read once, every table row written once (rows no token names get zeros).
+  // Bytes: every gradient row read once, every table row written once (rows no token names get
+  // zeros); the adding form reads and writes at most one table row per token.
+  const double table_rows = add ? 2.0 * static_cast<double>(tokens < vocab ? tokens : vocab) : static_cast<double>(vocab);
   OmxKernelTimer timer(ctx, OMX_K_EMBED_BWD,
                        static_cast<double>(dim) * (static_cast<double>(tokens) * (grad_dtype == OMX_BF16 ? 2.0 : 4.0) +
-                                                   static_cast<double>(vocab) * 4.0));
+                                                   table_rows * 4.0));
   omx_launch_timed(ctx, count_ids_kernel, tgrid, dim3(256), 0, timer.start(), nullptr, idp, counts, tokens, vocab,
                    ctx->fault, tag);
   OMX_LAUNCH_CHECK(ctx, "count_ids_kernel");
@@ -762,10 +778,17 @@ int32_t omx_embedding_backward(omx_ctx* ctx, const void* ids, const void* grad, 
   OMX_LAUNCH_CHECK(ctx, "sort_long_segments_kernel");
   const bool vec4 = dim % 4 == 0 && (reinterpret_cast<uintptr_t>(grad) & 15u) == 0 &&
                     (reinterpret_cast<uintptr_t>(table_grad) & 15u) == 0 && (grad_dtype == OMX_F32 || dim % 8 == 0);
-#define EMB_BWD(TG_, V_)                                                                                           \
-  omx_launch_timed(ctx, embedding_bwd_kernel<TG_, V_>, vgrid, dim3(ROW_THREADS), 0, nullptr, timer.stop(), offsets, \
-                   sorted, static_cast<const TG_*>(grad), static_cast<float*>(table_grad), vocab,                  \
-                   static_cast<int>(dim), ctx->fault, tag)
+#define EMB_BWD(TG_, V_)                                                                                         \
+  do {                                                                                                          \
+    if (add)                                                                                                    \
+      omx_launch_timed(ctx, embedding_bwd_kernel<TG_, V_, true>, vgrid, dim3(ROW_THREADS), 0, nullptr,          \
+                       timer.stop(), offsets, sorted, static_cast<const TG_*>(grad),                            \
+                       static_cast<float*>(table_grad), vocab, static_cast<int>(dim), ctx->fault, tag);         \
+    else                                                                                                        \
+      omx_launch_timed(ctx, embedding_bwd_kernel<TG_, V_, false>, vgrid, dim3(ROW_THREADS), 0, nullptr,         \
+                       timer.stop(), offsets, sorted, static_cast<const TG_*>(grad),                            \
+                       static_cast<float*>(table_grad), vocab, static_cast<int>(dim), ctx->fault, tag);         \
+  } while (0)
   if (grad_dtype == OMX_F32) {
     if (vec4) EMB_BWD(float, 4);
     else EMB_BWD(float, 1);
@@ -776,6 +799,16 @@ int32_t omx_embedding_backward(omx_ctx* ctx, const void* ids, const void* grad, 
 #undef EMB_BWD
   OMX_LAUNCH_CHECK(ctx, "embedding_bwd_kernel");
   return OMX_OK;
+}
+
+int32_t omx_embedding_backward(omx_ctx* ctx, const void* ids, const void* grad, int32_t grad_dtype, void* table_grad,
+                               uint64_t tokens, uint64_t vocab, uint64_t dim) {
+  return embedding_backward_impl(ctx, ids, grad, grad_dtype, table_grad, tokens, vocab, dim, false);
+}
+
+int32_t omx_embedding_backward_accumulate(omx_ctx* ctx, const void* ids, const void* grad, int32_t grad_dtype,
+                                          void* table_grad, uint64_t tokens, uint64_t vocab, uint64_t dim) {
+  return embedding_backward_impl(ctx, ids, grad, grad_dtype, table_grad, tokens, vocab, dim, true);
 }
 
 int32_t omx_argmax_rows(omx_ctx* ctx, const void* x, uint64_t rows, uint64_t cols, void* out) {

@@ -82,7 +82,6 @@ struct ogpt {
   void *gu_all = nullptr, *gqkv_all = nullptr;  // [layers][N,mlp], [layers][N,3d] AD
   void *gyd_all = nullptr, *gyo_all = nullptr;  // residual-stream gradient copies feeding down / o: [layers][N,d] AD
   float *gres = nullptr, *gres1 = nullptr, *gt = nullptr, *gh = nullptr;  // [N,d] f32
-  float* g_emb = nullptr;                    // [V,d] f32
   void* ghf = nullptr;                       // [N,d] AD
 
   // Parameter views.
@@ -279,8 +278,8 @@ int32_t backward(ogpt* t) {
   }
   // x0 = tok[ids] + pos[positions]; the tied table adds the embedding's share to the head's.
   TRY(omx_embedding_backward(ctx, t->positions, t->gres, OMX_F32, t->g(1), N, T, d));
-  TRY(omx_embedding_backward(ctx, t->ids, t->gres, OMX_F32, t->g_emb, N, c.vocab, d));
-  TRY(omx_accumulate_grad(ctx, t->g(0), t->g_emb, static_cast<uint64_t>(c.vocab) * d));
+  // The tied table: the gather's gradient joins the head's where it lies, row by named row.
+  TRY(omx_embedding_backward_accumulate(ctx, t->ids, t->gres, OMX_F32, t->g(0), N, c.vocab, d));
   return OMX_OK;
 }
 
@@ -421,7 +420,6 @@ int32_t ogpt_create(omx_ctx* ctx, const ogpt_config* config, ogpt** out) {
   CREATE_TRY(alloc_t(t, N * d, &t->gres1));
   CREATE_TRY(alloc_t(t, N * d, &t->gt));
   CREATE_TRY(alloc_t(t, N * d, &t->gh));
-  CREATE_TRY(alloc_t(t, static_cast<uint64_t>(c.vocab) * d, &t->g_emb));
 #undef CREATE_TRY
   *out = t;
   return OMX_OK;

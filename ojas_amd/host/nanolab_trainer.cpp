@@ -88,7 +88,7 @@ struct onano {
   float* v0_acc = nullptr;               // the same as g_v0 in f32 (fused projection)
   void *gqp = nullptr, *gkp = nullptr, *gvp = nullptr, *gap_p = nullptr;  // permuted gradients (row kernels)
   void *gy16 = nullptr, *ghf = nullptr;
-  float *gres = nullptr, *gres1 = nullptr, *gh = nullptr, *g_emb = nullptr;
+  float *gres = nullptr, *gres1 = nullptr, *gh = nullptr;
   // bf16 tier with more than one block: the seven weight gradients of every block wait until the
   // backward's end. Each block's product inputs (h, y, h2, m) and output gradients sit at a fixed
   // stride in stacked buffers, the gradient arena holds the blocks at a fixed stride too, and seven
@@ -387,8 +387,8 @@ int32_t backward(onano* t, float loss_seed) {
                                N * H, N * d, per_layer));
   }
   // The tied table: the head's gradient first, then the embedding's rows.
-  TRY(omx_embedding_backward(ctx, t->ids, t->gres, OMX_F32, t->g_emb, N, c.vocab, d));
-  TRY(omx_accumulate_grad(ctx, t->g(0), t->g_emb, static_cast<uint64_t>(c.vocab) * d));
+  // The tied table: the gather's gradient joins the head's where it lies, row by named row.
+  TRY(omx_embedding_backward_accumulate(ctx, t->ids, t->gres, OMX_F32, t->g(0), N, c.vocab, d));
   return OMX_OK;
 }
 
@@ -615,7 +615,6 @@ int32_t onano_create(omx_ctx* ctx, const onano_config* config, onano** out) {
   CREATE_TRY(alloc_t(t, N * d, &t->gres));
   CREATE_TRY(alloc_t(t, N * d, &t->gres1));
   CREATE_TRY(alloc_t(t, N * d, &t->gh));
-  CREATE_TRY(alloc_t(t, static_cast<uint64_t>(c.vocab) * d, &t->g_emb));
 #undef CREATE_TRY
   *out = t;
   return OMX_OK;

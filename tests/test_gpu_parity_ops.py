@@ -178,6 +178,37 @@ def test_embedding_backward_with_one_id_filling_the_batch(be, tokens, vocab, dim
     assert np.array_equal(tg.view(np.uint32), orc.embedding_backward(ids, grad, vocab).view(np.uint32))
 
 
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("tokens,vocab,dim", [(12, 10, 8), (257, 500, 64), (1000, 37, 65), (4096, 50304, 768)])
+def test_embedding_backward_accumulate_is_the_scatter_then_the_sum(be, tokens, vocab, dim, bf16):
+    """`embedding_backward_accumulate` leaves in the table gradient the bits of `embedding_backward`
+    into a fresh buffer followed by `accumulate_grad`: the oracle's scatter, then one f32 add per
+    element, and rows that no id names keep their bits (a -0.0 planted there stays -0.0)."""
+    from ojas_amd.backend import BF16
+
+    print(f"embedding accumulate {tokens} {vocab} {dim} bf16={bf16}", flush=True)
+    r = orc.SplitMix64(4242 + tokens)
+    ids = np.array([r.below(vocab) for _ in range(tokens)], dtype=np.uint32)
+    grad = r.vec(tokens * dim, 1.0).reshape(tokens, dim)
+    if bf16:
+        grad = orc.round_bf16(grad)
+    base = r.vec(vocab * dim, 1.0).reshape(vocab, dim)
+    unnamed = np.setdiff1d(np.arange(vocab), ids)
+    if unnamed.size:
+        base[unnamed[0], 0] = -0.0
+    acc = be.upload(base)
+    be.embedding_backward_accumulate(be.upload(ids), be.upload(grad, BF16) if bf16 else be.upload(grad), acc)
+    want = base + orc.embedding_backward(ids, grad, vocab)
+    if unnamed.size:
+        want[unnamed] = base[unnamed]
+    assert np.array_equal(be.download(acc).view(np.uint32), want.view(np.uint32))
+    # ... and the two ops in sequence on the device give the same.
+    two = be.upload(base)
+    be.accumulate_grad(two, be.embedding_backward(be.upload(ids), be.upload(grad, BF16) if bf16 else be.upload(grad), vocab))
+    named = np.unique(ids)
+    assert np.array_equal(be.download(two)[named].view(np.uint32), want[named].view(np.uint32))
+
+
 def test_embedding_out_of_range_id_is_reported_at_sync(be):
     from ojas_amd.backend import OUT_OF_RANGE, OjasError
 
