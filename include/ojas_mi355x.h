@@ -133,6 +133,15 @@ int32_t omx_gemm_strided_batch(omx_ctx* ctx, const void* a, uint64_t a_rs, uint6
                                uint64_t b_rs, uint64_t b_cs, int32_t operand_dtype, void* c,
                                int32_t c_dtype, uint64_t m, uint64_t k, uint64_t n, int32_t accumulate,
                                uint64_t count, uint64_t stride_a, uint64_t stride_b, uint64_t stride_c);
+/* omx_gemm_strided_batch with omx_gemm_pitched's output pitch: product i writes the n columns that
+ * start stride_c elements after product i - 1's, in rows `ldc` elements apart, so the products can
+ * be adjacent column blocks of one tensor (stride_c = n). No counterpart in the trait. */
+int32_t omx_gemm_pitched_strided_batch(omx_ctx* ctx, const void* a, uint64_t a_rs, uint64_t a_cs,
+                                       const void* b, uint64_t b_rs, uint64_t b_cs,
+                                       int32_t operand_dtype, void* c, int32_t c_dtype,
+                                       uint64_t ldc, uint64_t m, uint64_t k, uint64_t n,
+                                       int32_t accumulate, uint64_t count, uint64_t stride_a,
+                                       uint64_t stride_b, uint64_t stride_c);
 
 /* A frozen linear layer whose weight is stored as symmetric int8 codes [n_out, k_in] with one f32
  * scale per `group` consecutive input columns [n_out, k_in / group] (value = code * scale: the

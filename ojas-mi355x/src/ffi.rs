@@ -84,6 +84,7 @@ extern "C" {
     pub fn omx_gemm(ctx: *mut OmxCtx, a: *const c_void, a_rs: u64, a_cs: u64, b: *const c_void, b_rs: u64, b_cs: u64, operand_dtype: i32, c: *mut c_void, c_dtype: i32, m: u64, k: u64, n: u64, accumulate: i32) -> i32;
     pub fn omx_gemm_pitched(ctx: *mut OmxCtx, a: *const c_void, a_rs: u64, a_cs: u64, b: *const c_void, b_rs: u64, b_cs: u64, operand_dtype: i32, c: *mut c_void, c_dtype: i32, ldc: u64, m: u64, k: u64, n: u64, accumulate: i32) -> i32;
     pub fn omx_gemm_strided_batch(ctx: *mut OmxCtx, a: *const c_void, a_rs: u64, a_cs: u64, b: *const c_void, b_rs: u64, b_cs: u64, operand_dtype: i32, c: *mut c_void, c_dtype: i32, m: u64, k: u64, n: u64, accumulate: i32, count: u64, stride_a: u64, stride_b: u64, stride_c: u64) -> i32;
+    pub fn omx_gemm_pitched_strided_batch(ctx: *mut OmxCtx, a: *const c_void, a_rs: u64, a_cs: u64, b: *const c_void, b_rs: u64, b_cs: u64, operand_dtype: i32, c: *mut c_void, c_dtype: i32, ldc: u64, m: u64, k: u64, n: u64, accumulate: i32, count: u64, stride_a: u64, stride_b: u64, stride_c: u64) -> i32;
     pub fn omx_linear_i8_group_forward(ctx: *mut OmxCtx, x: *const c_void, x_dtype: i32, codes_i8: *const c_void, scales_f32: *const c_void, group: u64, layout: i32, add: *const c_void, low_rank: *const OmxLowRank, y: *mut c_void, rows: u64, k_in: u64, n_out: u64) -> i32;
     pub fn omx_linear_i8_group_backward_input(ctx: *mut OmxCtx, codes_i8: *const c_void, scales_f32: *const c_void, group: u64, layout: i32, gy: *const c_void, gy_dtype: i32, add: *const c_void, low_rank: *const OmxLowRank, gx: *mut c_void, rows: u64, k_in: u64, n_out: u64) -> i32;
     pub fn omx_pack_i8_group(ctx: *mut OmxCtx, codes_i8: *const c_void, scales_f32: *const c_void, blocked_codes: *mut c_void, blocked_scales: *mut c_void, n_out: u64, k_in: u64, group: u64, unpack: i32) -> i32;

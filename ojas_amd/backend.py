@@ -361,6 +361,17 @@ class MiBackend:
             C.c_uint64(sb), C.c_uint64(sc)))
         return out
 
+    def gemm_pitched_strided_batch(self, a: DeviceTensor, a_strides, b: DeviceTensor, b_strides, c: DeviceTensor, ldc,
+                                   m, k, n, count, batch_strides):
+        """`gemm_strided_batch` into column blocks of `c`, whose rows are `ldc` elements apart
+        (`omx_gemm_pitched_strided_batch`); writes `c` in place."""
+        sa, sb, sc = batch_strides
+        self._check(self._lib.omx_gemm_pitched_strided_batch(
+            self._ctx, self._p(a), C.c_uint64(a_strides[0]), C.c_uint64(a_strides[1]), self._p(b),
+            C.c_uint64(b_strides[0]), C.c_uint64(b_strides[1]), C.c_int32(a.dtype), self._p(c), C.c_int32(c.dtype),
+            C.c_uint64(ldc), C.c_uint64(m), C.c_uint64(k), C.c_uint64(n), C.c_int32(0), C.c_uint64(count),
+            C.c_uint64(sa), C.c_uint64(sb), C.c_uint64(sc)))
+
     # ---- attention ----
     def causal_sdpa_forward(self, q, k, v, window: Optional[int] = None, out_dtype: Optional[int] = None):
         b, h, t, d = q.shape

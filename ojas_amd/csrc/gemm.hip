@@ -755,4 +755,16 @@ int32_t omx_gemm_strided_batch(omx_ctx* ctx, const void* a, uint64_t a_rs, uint6
                        nullptr, &batch);
 }
 
+int32_t omx_gemm_pitched_strided_batch(omx_ctx* ctx, const void* a, uint64_t a_rs, uint64_t a_cs, const void* b,
+                                       uint64_t b_rs, uint64_t b_cs, int32_t operand_dtype, void* c, int32_t c_dtype,
+                                       uint64_t ldc, uint64_t m, uint64_t k, uint64_t n, int32_t accumulate,
+                                       uint64_t count, uint64_t stride_a, uint64_t stride_b, uint64_t stride_c) {
+  OMX_REQUIRE_CTX(ctx);
+  if (ldc < n) return omx_fail(ctx, OMX_SHAPE, "gemm: output pitch %llu is below its %llu columns", (unsigned long long)ldc,
+                               (unsigned long long)n);
+  const OmxGemmBatch batch{count, stride_a, stride_b, stride_c};
+  return omx_gemm_impl(ctx, F_GEMM, a, a_rs, a_cs, b, b_rs, b_cs, operand_dtype, c, c_dtype, ldc, m, k, n, accumulate,
+                       nullptr, &batch);
+}
+
 }  // extern "C"

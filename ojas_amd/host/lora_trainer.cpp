@@ -17,6 +17,7 @@
 //    pass and one AdamW pass cover every adapter.
 //  * The second adapter product never exists as a tensor: it is added in the accumulators of the
 //    quantised product (omx_low_rank), forward and backward.
+#include <cstdlib>
 #include <cmath>
 #include <cstdint>
 #include <cstring>
@@ -215,9 +216,10 @@ int32_t backward(olora* t) {
                                             A.ap, A.apr, t->ga, d, A.lse, OMX_BF16, gq, gq + d * 2, gq + 2 * d * 2,
                                             OMX_BF16, B, T, H, H, D, 0));
     TRY(omx_rope_half_split_inplace(ctx, gqkv, OMX_BF16, 3 * d, t->cos_t, t->sin_t, N, T, 2 * H, D, 1));
-    for (uint64_t j = 0; j < 3; ++j)
-      TRY(omx_gemm_pitched(ctx, off16(gqkv, j * d), 3 * d, 1, t->b16(l, j), r, 1, OMX_BF16, off16(gh, j * r), OMX_BF16,
-                           4 * r, N, d, r, 0));
+    // gh for q, k and v in one launch: column blocks of gqkv against B_q, B_k, B_v (adjacent in the
+    // arena) into adjacent column blocks of gh.
+    TRY(omx_gemm_pitched_strided_batch(ctx, gqkv, 3 * d, 1, t->b16(l, 0), r, 1, OMX_BF16, gh, OMX_BF16, 4 * r, N, d, r, 0,
+                                       3, d, t->b_off(0, 1) - t->b_off(0, 0), r));
     omx_low_rank lr_qkv{gh, t->at(l), 4 * r, 4 * r, 3 * r, 0};
     TRY(q8_backward(t, A.qkv, gqkv, &lr_qkv, t->t_b));
     TRY(omx_rms_norm_backward_residual(ctx, A.x, OMX_F32, t->norm(l, 0), t->t_b, OMX_BF16, t->gres1, t->gres, t->gy16,

@@ -119,6 +119,40 @@ def test_strided_batch_of_thin_weight_gradients_splits_the_reduction(be, rows, k
         assert err <= 1e-5 * max(1.0, float(np.max(np.abs(want)))), (l, err)
 
 
+@pytest.mark.parametrize("rows,d,r", [(2048, 256, 16), (8192, 2048, 16), (300, 128, 8)])
+def test_pitched_strided_batch_writes_adjacent_column_blocks(be, rows, d, r):
+    """Three thin products in one launch (an adapter's gh = gy B for the q, k and v sites): operand i
+    is column block i of a [rows, 3 d] tensor, its B the i-th of three adjacent [d, r] matrices, its
+    output column block i of a [rows, 4 r] tensor whose fourth block keeps what it held. The bits
+    are those of three `gemm_pitched` calls."""
+    import ctypes as C
+
+    from ojas_amd.backend import BF16
+
+    print(f"gemm pitched strided batch {rows} {d} {r}", flush=True)
+    be.set_option("gemm_dma", 1)
+    rng = orc.SplitMix64(8800 + rows + d)
+    gy = orc.round_bf16(rng.vec(rows * 3 * d, 0.5)).reshape(rows, 3 * d)
+    bm = orc.round_bf16(rng.vec(3 * d * r, 0.5)).reshape(3, d, r)
+    held = orc.round_bf16(rng.vec(rows * 4 * r, 1.0)).reshape(rows, 4 * r)
+    dgy, dbm = be.upload(gy, BF16), be.upload(bm, BF16)
+    out = be.upload(held, BF16)
+    be.gemm_pitched_strided_batch(dgy, (3 * d, 1), dbm, (r, 1), out, 4 * r, rows, d, r, 3, (d, d * r, r))
+    got = be.download_f32(out).reshape(rows, 4 * r)
+    assert np.array_equal(got[:, 3 * r:], held[:, 3 * r:])
+    for j in range(3):
+        want = gy[:, j * d:(j + 1) * d].astype(np.float64) @ bm[j].astype(np.float64)
+        err = float(np.max(np.abs(got[:, j * r:(j + 1) * r] - want)))
+        assert err <= 2e-2 * max(1.0, float(np.max(np.abs(want)))), (j, err)
+    one = be.upload(held, BF16)
+    for j in range(3):
+        assert be._lib.omx_gemm_pitched(
+            be._ctx, C.c_void_p(dgy.ptr + j * d * 2), C.c_uint64(3 * d), C.c_uint64(1), C.c_void_p(dbm.ptr + j * d * r * 2),
+            C.c_uint64(r), C.c_uint64(1), C.c_int32(BF16), C.c_void_p(one.ptr + j * r * 2), C.c_int32(BF16),
+            C.c_uint64(4 * r), C.c_uint64(rows), C.c_uint64(d), C.c_uint64(r), C.c_int32(0)) == 0
+    assert np.array_equal(be.download(one), be.download(out))
+
+
 def test_strided_batch_refuses_bad_strides(be):
     from ojas_amd.backend import BF16, OjasError
 
