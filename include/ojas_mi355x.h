@@ -541,12 +541,22 @@ int32_t omx_per_head_sigmoid_gate_backward(omx_ctx* ctx, const void* input, cons
  * keeps the layers of a model at a fixed stride and adds up every layer's weight gradient in
  * one omx_gemm_strided_batch at the end of its backward (a 12 x d output over all tokens fills
  * the chip only with the layers side by side). Every other result is the bits of
- * omx_per_head_sigmoid_gate_backward. */
+ * omx_per_head_sigmoid_gate_backward. `g_input` may be null: the caller then takes the input
+ * gradient from gz too (omx_per_head_sigmoid_gate_input_grad_add). */
 int32_t omx_per_head_sigmoid_gate_backward_deferred(
     omx_ctx* ctx, const void* input, const void* weight, int32_t operand_dtype, const void* bias_f32,
     const void* attn, int32_t attn_dtype, const void* gy, int32_t gy_dtype, const void* gates_f32,
     void* g_input, int32_t g_input_dtype, void* gz, void* g_bias_f32, void* g_attn,
     int32_t g_attn_dtype, uint64_t rows, uint64_t d_model, uint64_t heads, uint64_t head_dim);
+/* out_f32[r, i] = add_in[r, i] + sum_h gz[r, h] weight[h, i]: the grad_input of
+ * per_head_sigmoid_gate_backward (backend.rs:1883-1905) from the gz that the deferred form hands
+ * back, added to another gradient of the same input (residual_add_forward, backend.rs:1165-1173)
+ * in one pass, for a caller that passed a null g_input to the deferred form. `out` may not be
+ * `add_in`. */
+int32_t omx_per_head_sigmoid_gate_input_grad_add(omx_ctx* ctx, const void* gz, const void* weight,
+                                                 int32_t operand_dtype, const void* add_in,
+                                                 int32_t add_dtype, void* out_f32, uint64_t rows,
+                                                 uint64_t d_model, uint64_t heads);
 /* BackendModule::value_residual_blend_forward / _backward (backend.rs:1907-1920;
  * CPU ojas-cpu/src/pointwise.rs:2031-2148): out = (1 - s) v + s v0 with
  * s = sigmoid(lambda); lambda and grad_lambda are one f32 each on the device. */

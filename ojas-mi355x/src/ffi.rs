@@ -139,6 +139,7 @@ extern "C" {
     pub fn omx_per_head_sigmoid_gate_forward(ctx: *mut OmxCtx, input: *const c_void, weight: *const c_void, operand_dtype: i32, bias_f32: *const c_void, attn: *const c_void, attn_dtype: i32, y: *mut c_void, y_dtype: i32, gates_f32: *mut c_void, rows: u64, d_model: u64, heads: u64, head_dim: u64) -> i32;
     pub fn omx_per_head_sigmoid_gate_backward(ctx: *mut OmxCtx, input: *const c_void, weight: *const c_void, operand_dtype: i32, bias_f32: *const c_void, attn: *const c_void, attn_dtype: i32, gy: *const c_void, gy_dtype: i32, gates_f32: *const c_void, g_input: *mut c_void, g_input_dtype: i32, g_weight_f32: *mut c_void, g_bias_f32: *mut c_void, g_attn: *mut c_void, g_attn_dtype: i32, rows: u64, d_model: u64, heads: u64, head_dim: u64) -> i32;
     pub fn omx_per_head_sigmoid_gate_backward_deferred(ctx: *mut OmxCtx, input: *const c_void, weight: *const c_void, operand_dtype: i32, bias_f32: *const c_void, attn: *const c_void, attn_dtype: i32, gy: *const c_void, gy_dtype: i32, gates_f32: *const c_void, g_input: *mut c_void, g_input_dtype: i32, gz: *mut c_void, g_bias_f32: *mut c_void, g_attn: *mut c_void, g_attn_dtype: i32, rows: u64, d_model: u64, heads: u64, head_dim: u64) -> i32;
+    pub fn omx_per_head_sigmoid_gate_input_grad_add(ctx: *mut OmxCtx, gz: *const c_void, weight: *const c_void, operand_dtype: i32, add_in: *const c_void, add_dtype: i32, out_f32: *mut c_void, rows: u64, d_model: u64, heads: u64) -> i32;
     pub fn omx_value_residual_blend_forward(ctx: *mut OmxCtx, value: *const c_void, value0: *const c_void, lambda_f32: *const c_void, out: *mut c_void, dtype: i32, n: u64) -> i32;
     pub fn omx_value_residual_blend_backward(ctx: *mut OmxCtx, value: *const c_void, value0: *const c_void, lambda_f32: *const c_void, gy: *const c_void, g_value: *mut c_void, g_value0: *mut c_void, dtype: i32, g_lambda_f32: *mut c_void, n: u64) -> i32;
     pub fn omx_qkv_prepare_forward(ctx: *mut OmxCtx, qkv_lin: *const c_void, qkv_out: *mut c_void, pitch: u64, q_weight_f32: *const c_void, k_weight_f32: *const c_void, cos_f32: *const c_void, sin_f32: *const c_void, value0: *const c_void, lambda_f32: *const c_void, tokens: u64, time: u64, heads: u64, kv_heads: u64, head_dim: u64, eps: f32) -> i32;

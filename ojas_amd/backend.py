@@ -841,10 +841,26 @@ class MiBackend:
     def per_head_sigmoid_gate_backward(self, x, w, b, attn, gy, g_input_dtype: Optional[int] = None):
         return self.per_head_sigmoid_gate_backward_saved(x, w, b, attn, gy, None, g_input_dtype)
 
-    def per_head_sigmoid_gate_backward_deferred(self, x, w, b, attn, gy, scales, g_input_dtype: Optional[int] = None):
+    def per_head_sigmoid_gate_input_grad_add(self, gz, w, add_in):
+        """add_in + gz w as f32 [rows, d_model]: the gate's input gradient from `gz`, joined to another
+        gradient of the same input (`omx_per_head_sigmoid_gate_input_grad_add`)."""
+        rows, heads = gz.shape
+        d_model = w.shape[1]
+        if w.shape[0] != heads or add_in.numel != rows * d_model or gz.dtype != w.dtype:
+            raise OjasError(SHAPE, f"per_head_sigmoid_gate_input_grad_add: gz {gz.shape}, weight {w.shape}, "
+                                   f"add_in {add_in.shape}")
+        out = self.empty(add_in.shape, F32)
+        self._check(self._lib.omx_per_head_sigmoid_gate_input_grad_add(
+            self._ctx, self._p(gz), self._p(w), C.c_int32(w.dtype), self._p(add_in), C.c_int32(add_in.dtype),
+            self._p(out), C.c_uint64(rows), C.c_uint64(d_model), C.c_uint64(heads)))
+        return out
+
+    def per_head_sigmoid_gate_backward_deferred(self, x, w, b, attn, gy, scales, g_input_dtype: Optional[int] = None,
+                                                want_input_grad: bool = True):
         """`per_head_sigmoid_gate_backward_saved` without the weight gradient: returns (grad_input, gz
         [rows, heads] in the operands' dtype, grad_bias, grad_attn); grad_weight = gz^T input is the
-        caller's (`omx_per_head_sigmoid_gate_backward_deferred`)."""
+        caller's (`omx_per_head_sigmoid_gate_backward_deferred`). `want_input_grad=False` leaves the
+        input gradient to the caller as well (None comes back in its place)."""
         op = "per_head_sigmoid_gate_backward"
         rows, d_model, heads, dh = self._gate_dims(op, x, w, b, attn)
         if gy.shape != attn.shape or gy.dtype != attn.dtype:
@@ -852,7 +868,8 @@ class MiBackend:
         if scales is not None and (scales.shape != (rows, heads) or scales.dtype != F32):
             raise OjasError(SHAPE, f"{op}: gate scale length does not match rows * heads")
         gxd = x.dtype if g_input_dtype is None else g_input_dtype
-        gx, gz = self.empty(x.shape, gxd), self.empty((rows, heads), x.dtype)
+        gx = self.empty(x.shape, gxd) if want_input_grad else None
+        gz = self.empty((rows, heads), x.dtype)
         gb, ga = self.empty((heads,), F32), self.empty(attn.shape, attn.dtype)
         self._check(self._lib.omx_per_head_sigmoid_gate_backward_deferred(
             self._ctx, self._p(x), self._p(w), C.c_int32(x.dtype), self._p(b), self._p(attn), C.c_int32(attn.dtype),

@@ -444,6 +444,49 @@ int32_t compute_gates(omx_ctx* ctx, uint32_t fault_op, const void* input, const 
   return OMX_OK;
 }
 
+// out[r, c] = add[r, c] + sum_h gz[r, h] w[h, c]: the gate's input gradient (a product with a reduction
+// of `heads` terms) joined to another gradient of the same input. A thread owns four columns and
+// keeps their `heads` weights in registers; a wave reads a row's gz once (lane h holds head h) and
+// hands the values round through readlane. bf16 x bf16 products are exact in f32; the sum runs
+// h = 0, 1, ... in f32.
+constexpr int GATE_JOIN_HEADS = 16;
+template <typename TA>
+__global__ __launch_bounds__(256) void gate_input_grad_add_kernel(const unsigned short* __restrict__ gz,
+                                                                  const unsigned short* __restrict__ w,
+                                                                  const TA* __restrict__ add, float* __restrict__ out,
+                                                                  size_t rows, int d, int heads, int rows_per_block,
+                                                                  OmxFaultWord* fault, unsigned long long tag) {
+  const int c = static_cast<int>(threadIdx.x) * 4, lane = threadIdx.x & 63;
+  const bool live = c < d;
+  float wr[GATE_JOIN_HEADS][4];
+#pragma unroll
+  for (int h = 0; h < GATE_JOIN_HEADS; ++h) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) wr[h][e] = 0.0f;
+    if (live && h < heads) dev_load4<unsigned short>(w + static_cast<size_t>(h) * d, c, wr[h]);
+  }
+  const size_t r0 = static_cast<size_t>(blockIdx.x) * rows_per_block;
+  const size_t r1 = r0 + rows_per_block < rows ? r0 + rows_per_block : rows;
+  bool bad = false;
+  for (size_t r = r0; r < r1; ++r) {
+    const float zv = lane < heads ? dev_load<unsigned short>(gz + r * heads, lane) : 0.0f;
+    float a[4] = {0.0f, 0.0f, 0.0f, 0.0f}, acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (live) dev_load4<TA>(add + r * d, c, a);
+#pragma unroll
+    for (int h = 0; h < GATE_JOIN_HEADS; ++h) {
+      const float z = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(zv), h));
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[e] = fmaf(z, wr[h][e], acc[e]);
+    }
+    if (live) {
+      float4 o = make_float4(a[0] + acc[0], a[1] + acc[1], a[2] + acc[2], a[3] + acc[3]);
+      bad |= !(dev_finite(o.x) && dev_finite(o.y) && dev_finite(o.z) && dev_finite(o.w));
+      *reinterpret_cast<float4*>(out + r * d + c) = o;
+    }
+  }
+  if (bad) dev_raise_fault(fault, tag);
+}
+
 }  // namespace
 
 extern "C" {
@@ -573,7 +616,8 @@ static int32_t gate_backward_impl(omx_ctx* ctx, const char* op, const void* inpu
                                   int32_t g_attn_dtype, uint64_t rows, uint64_t d_model, uint64_t heads,
                                   uint64_t head_dim) {
   OMX_REQUIRE_CTX(ctx);
-  if (!input || !weight || !bias || !attn || !gy || !g_input || !g_bias || !g_attn || (!g_weight && !gz_out))
+  // The deferred form may leave the input gradient to the caller as well (it has gz for it).
+  if (!input || !weight || !bias || !attn || !gy || (!g_input && !gz_out) || !g_bias || !g_attn || (!g_weight && !gz_out))
     return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
   int32_t rc = check_gate(ctx, op, operand_dtype, {attn_dtype, gy_dtype, g_input_dtype, g_attn_dtype}, rows, d_model,
                           heads, head_dim);
@@ -643,9 +687,11 @@ static int32_t gate_backward_impl(omx_ctx* ctx, const char* op, const void* inpu
   rc = omx_column_sum(ctx, partial, static_cast<float*>(g_bias), blocks, heads, tag, stage);
   if (rc != OMX_OK) return rc;
   // grad_input[r, i] = sum_h gz[r, h] weight[h, i]
-  rc = omx_gemm_impl(ctx, F_GATE_BACKWARD, gz, heads, 1, weight, d_model, 1, operand_dtype, g_input, g_input_dtype,
-                     d_model, rows, heads, d_model, 0);
-  if (rc != OMX_OK) return rc;
+  if (g_input) {
+    rc = omx_gemm_impl(ctx, F_GATE_BACKWARD, gz, heads, 1, weight, d_model, 1, operand_dtype, g_input, g_input_dtype,
+                       d_model, rows, heads, d_model, 0);
+    if (rc != OMX_OK) return rc;
+  }
   // grad_weight[h, i] = sum_r gz[r, h] input[r, i]
   if (!g_weight) return OMX_OK;
   return omx_gemm_impl(ctx, F_GATE_BACKWARD, gz, 1, heads, input, d_model, 1, operand_dtype, g_weight, OMX_F32, d_model,
@@ -676,6 +722,41 @@ int32_t omx_per_head_sigmoid_gate_backward_deferred(omx_ctx* ctx, const void* in
   return gate_backward_impl(ctx, "per_head_sigmoid_gate_backward_deferred", input, weight, operand_dtype, bias, attn,
                             attn_dtype, gy, gy_dtype, gates_saved, g_input, g_input_dtype, nullptr, gz_out, g_bias,
                             g_attn, g_attn_dtype, rows, d_model, heads, head_dim);
+}
+
+int32_t omx_per_head_sigmoid_gate_input_grad_add(omx_ctx* ctx, const void* gz, const void* weight, int32_t operand_dtype,
+                                                 const void* add_in, int32_t add_dtype, void* out, uint64_t rows,
+                                                 uint64_t d_model, uint64_t heads) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "per_head_sigmoid_gate_input_grad_add";
+  if (!gz || !weight || !add_in || !out) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  if (!omx_valid_float_dtype(operand_dtype) || !omx_valid_float_dtype(add_dtype))
+    return omx_fail(ctx, OMX_DTYPE, "%s: dtype must be f32 or bf16", op);
+  if (rows == 0 || d_model == 0 || heads == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
+  if (out == add_in) return omx_fail(ctx, OMX_SHAPE, "%s: the output may not be the gradient it is added to", op);
+  const bool aligned = ((reinterpret_cast<uintptr_t>(weight) | reinterpret_cast<uintptr_t>(add_in)) & 7u) == 0 &&
+                       (reinterpret_cast<uintptr_t>(out) & 15u) == 0 &&
+                       (add_dtype == OMX_BF16 || (reinterpret_cast<uintptr_t>(add_in) & 15u) == 0);
+  if (operand_dtype == OMX_BF16 && d_model % 4 == 0 && d_model <= 1024 && heads <= GATE_JOIN_HEADS && aligned) {
+    const int rows_per_block = 8;
+    const unsigned long long tag = omx_tag(ctx, F_GATE_BACKWARD);
+    dim3 grid(static_cast<unsigned>((rows + rows_per_block - 1) / rows_per_block));
+#define GATE_JOIN(TA_)                                                                                        \
+  hipLaunchKernelGGL(gate_input_grad_add_kernel<TA_>, grid, dim3(256), 0, ctx->stream,                        \
+                     static_cast<const unsigned short*>(gz), static_cast<const unsigned short*>(weight),      \
+                     static_cast<const TA_*>(add_in), static_cast<float*>(out), rows, static_cast<int>(d_model), \
+                     static_cast<int>(heads), rows_per_block, ctx->fault, tag)
+    if (add_dtype == OMX_BF16) GATE_JOIN(unsigned short);
+    else GATE_JOIN(float);
+#undef GATE_JOIN
+    OMX_LAUNCH_CHECK(ctx, "gate_input_grad_add_kernel");
+    return OMX_OK;
+  }
+  // Any other shape: the product, then the sum.
+  int32_t rc = omx_gemm_impl(ctx, F_GATE_BACKWARD, gz, heads, 1, weight, d_model, 1, operand_dtype, out, OMX_F32, d_model,
+                             rows, heads, d_model, 0);
+  if (rc != OMX_OK) return rc;
+  return omx_residual_add(ctx, out, OMX_F32, add_in, add_dtype, out, OMX_F32, rows * d_model);
 }
 
 int32_t omx_value_residual_blend_forward(omx_ctx* ctx, const void* value, const void* value0, const void* lambda,

@@ -12,6 +12,7 @@
 // Newton-Schulz call); the bf16 tier keeps a bf16 mirror of the parameters that the optimizers
 // refresh. The gate and up projections are adjacent in the arena, so on the bf16 tier they are one
 // [2 hidden, n_embd] matrix whose product feeds the fused SwiGLU.
+#include <cstdlib>
 #include <cmath>
 #include <cstdint>
 #include <cstring>
@@ -290,7 +291,8 @@ int32_t backward(onano* t, float loss_seed) {
     TRY(omx_linear_backward(ctx, A.y, t->w(t->li(l, WO)), gy, AD, t->gyy, AD, gw(WO), OMX_F32, N, qd, d));
     if (defer && t->gz_all)  // the gate's weight gradient waits for the batched product below
       TRY(omx_per_head_sigmoid_gate_backward_deferred(ctx, A.h, t->w(t->li(l, GATE_W)), AD, t->w32(t->li(l, GATE_B)), A.ap,
-                                                      AD, t->gyy, AD, A.gates, t->gh, OMX_F32, slice(t->gz_all, l, N * H),
+                                                      AD, t->gyy, AD, A.gates, t->fused_qkv ? nullptr : t->gh, OMX_F32,
+                                                      slice(t->gz_all, l, N * H),
                                                       t->g(t->li(l, GATE_B)), t->gap, AD, N, d, H, D));
     else
       TRY(omx_per_head_sigmoid_gate_backward(ctx, A.h, t->w(t->li(l, GATE_W)), AD, t->w32(t->li(l, GATE_B)), A.ap, AD,
@@ -315,7 +317,11 @@ int32_t backward(onano* t, float loss_seed) {
       if (!blends) TRY(omx_fill_zero(ctx, t->g(t->li(0, LAMBDA)), 4));
       // One product for the three projections: their input gradients add in its f32 accumulators.
       TRY(omx_linear_backward(ctx, A.h, t->w(t->li(l, WQ)), g_lin, AD, t->t_a, AD, gw(WQ), OMX_F32, N, d, P3));
-      TRY(omx_residual_add(ctx, t->gh, OMX_F32, t->t_a, AD, t->gh, OMX_F32, N * d));
+      if (defer && t->gz_all)  // the gate's input gradient, left out above, joins here in one pass
+        TRY(omx_per_head_sigmoid_gate_input_grad_add(ctx, slice(t->gz_all, l, N * H), t->w(t->li(l, GATE_W)), AD, t->t_a,
+                                                     AD, t->gh, N, d, H));
+      else
+        TRY(omx_residual_add(ctx, t->gh, OMX_F32, t->t_a, AD, t->gh, OMX_F32, N * d));
       TRY(omx_rms_norm_backward_residual(ctx, A.x, OMX_F32, t->w32(t->li(l, NORM1)), t->gh, OMX_F32, t->gres1, t->gres,
                                          copy_below, t->g(t->li(l, NORM1)), N, d, eps));
       gy = static_cast<const void*>(copy_below);

@@ -370,6 +370,17 @@ def test_gate_backward_without_its_weight_gradient(be, rows, d_model, heads, hea
     z = be.download_f32(gz).astype(np.float64).reshape(rows, heads)
     want = z.T @ be.download_f32(dx).astype(np.float64).reshape(rows, d_model)
     close(be.download(gw), want, max(tol, 1e-5), "gz^T input against the op's weight gradient")
+    # The input gradient left to the caller too: gz w joined to another gradient of the input.
+    none, gz3, gb3, ga3 = be.per_head_sigmoid_gate_backward_deferred(dx, dw, db, da, dgy, scales, F32,
+                                                                    want_input_grad=False)
+    assert none is None and np.array_equal(be.download(gz3), be.download(gz))
+    assert np.array_equal(be.download(gb3), be.download(gb)) and np.array_equal(be.download(ga3), be.download(ga))
+    other = rnd(r.vec(rows * d_model, 1.0)).reshape(1, rows, d_model)
+    joined = be.download(be.per_head_sigmoid_gate_input_grad_add(gz, dw, up(other)))
+    want_in = z @ be.download_f32(dw).astype(np.float64) + other.astype(np.float64).reshape(rows, d_model)
+    close(joined.reshape(rows, d_model), want_in, 1e-5, "add_in + gz w")
+    close(joined.reshape(rows, d_model), be.download(gx).astype(np.float64).reshape(rows, d_model) +
+          other.astype(np.float64).reshape(rows, d_model), max(tol, 1e-5), "against the op's input gradient + add_in")
 
 
 @pytest.mark.parametrize("bf16", [False, True])
