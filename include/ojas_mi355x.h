@@ -609,7 +609,9 @@ int32_t omx_read_scalar_f32(omx_ctx* ctx, const void* src, float* out);
  * eligible. "gemm_persistent": bit mask over operand layouts (bit 2 * A k-major + B k-major) that
  * take the persistent form of the direct-to-LDS kernel (default 15), and
  * "gemm_persistent_min_steps": only for reductions of at least this many 32-column steps
- * (default 64). "kv_attention": 0 = choose by head_dim (default), 1 = always the
+ * (default 64). "gemm_thin": 0 = bf16 products with at most 64 output columns over 1024 rows or
+ * more go through the tiled kernels and their split-K reduce instead of the one-pass kernel for
+ * thin outputs (default 1). "kv_attention": 0 = choose by head_dim (default), 1 = always the
  * LDS-tiled kernel. "ce_fused": 0 = the fused linear-cross-entropy always takes its separate
  * statistics and gradient kernels (default 1: one kernel when a tile holds the whole
  * vocabulary). "adamw_trust": 0 = omx_adamw_step_bounded always runs its checking pass

@@ -469,8 +469,12 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
   // Kernel choice. bf16 shapes whose output fills the chip with 256 x 256 (or
   // 256 x 128) tiles take the direct-to-LDS kernel; everything else (f32, odd
   // shapes, small outputs that need split-K) takes the 128 x 128 kernel.
+  // A thin output over many rows (an adapter's rank, a gate's heads) is bound by reading A once: its
+  // own kernel, which neither tiles the output nor splits K across launches.
+  const bool thin = operand_dtype == OMX_BF16 && ctx->gemm_thin && !(epi && epi->mode != OMX_EPI_NONE) &&
+                    omx_gemm_thin_eligible(g, a_km, b_km);
   int dma_variant = -1;
-  if (operand_dtype == OMX_BF16 && omx_gemm_dma_eligible(g, a_km, b_km)) {
+  if (!thin && operand_dtype == OMX_BF16 && omx_gemm_dma_eligible(g, a_km, b_km)) {
     const int mode = ctx->gemm_dma_mode;
     if (mode == 1) {
       // Measured on the GPT shapes: small outputs (the d x d weight gradients, the
@@ -521,7 +525,7 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
     // A strided batch splits only on the register-staged kernel (thin outputs over a long
     // reduction: 16 products of 16 tiles each leave three quarters of the chip's wave slots empty).
     const long all_tiles = tiles * g.batches;
-    const bool may_split = g.batches == 1 ? tiles < 256 : (dma_variant < 0 && all_tiles < 512);
+    const bool may_split = !thin && (g.batches == 1 ? tiles < 256 : (dma_variant < 0 && all_tiles < 512));
     if (may_split && ksteps >= 4 * min_steps && !(epi && epi->mode != OMX_EPI_NONE)) {
       splits = static_cast<int>(((g.batches == 1 ? 512 : 1024) + all_tiles - 1) / all_tiles);
       if (splits > ksteps / min_steps) splits = ksteps / min_steps;
@@ -571,7 +575,9 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
     ctx->timing_stop = timed.stop;
   }
   int32_t rc;
-  if (dma_variant >= 0) {
+  if (thin) {
+    rc = omx_gemm_thin_launch(ctx, g, b_km);
+  } else if (dma_variant >= 0) {
     rc = omx_gemm_dma_launch(ctx, g, a_km, b_km, dma_variant);
     if (rc == OMX_OK && g.splits > 1) {
       long elems = static_cast<long>(g.M) * g.N;
@@ -645,6 +651,10 @@ int32_t omx_set_option(omx_ctx* ctx, const char* name, int64_t value) {
   if (name && strcmp(name, "gemm_persistent_min_steps") == 0) {
     if (value < 2) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: gemm_persistent_min_steps is at least 2");
     ctx->gemm_persistent_min_steps = static_cast<int>(value);
+    return OMX_OK;
+  }
+  if (name && strcmp(name, "gemm_thin") == 0) {
+    ctx->gemm_thin = value != 0;
     return OMX_OK;
   }
   if (name && strcmp(name, "gemm_persistent") == 0) {

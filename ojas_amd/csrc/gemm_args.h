@@ -269,3 +269,8 @@ __device__ __forceinline__ bool gemm_store_block(const GemmArgs& g, int split, c
 bool omx_gemm_dma_eligible(const GemmArgs& g, bool a_km, bool b_km);
 void omx_gemm_dma_tile(int variant, int* bm, int* bn);
 int32_t omx_gemm_dma_launch(omx_ctx* ctx, const GemmArgs& g, bool a_km, bool b_km, int variant);
+
+// bf16 kernel for outputs of at most 64 columns over at least 1024 rows of a k-contiguous A
+// (K a multiple of 128, no accumulation): one pass over A, no split-K reduce.
+bool omx_gemm_thin_eligible(const GemmArgs& g, bool a_km, bool b_km);
+int32_t omx_gemm_thin_launch(omx_ctx* ctx, const GemmArgs& g, bool b_km);

@@ -153,6 +153,48 @@ def test_pitched_strided_batch_writes_adjacent_column_blocks(be, rows, d, r):
     assert np.array_equal(be.download(one), be.download(out))
 
 
+@pytest.mark.parametrize("rows,k,n,b_km,f32_out", [
+    (8192, 2048, 16, False, False), (8192, 2048, 48, False, False), (8192, 2048, 16, True, False),
+    (16384, 768, 12, False, True), (1030, 128, 64, True, False), (4096, 384, 5, False, False), (2048, 256, 33, True, True)])
+def test_thin_outputs_take_one_pass_over_a(be, rows, k, n, b_km, f32_out):
+    """Outputs of at most 64 columns over many rows (an adapter's h = x A^T and gh = gy B, a gate's
+    logits) take `gemm_thin_kernel`; held to the f64 product at the bf16-storage tolerance (1e-5 for an
+    f32 output: bf16 products are exact and both sums are f32) and to the tiled kernels' result, with
+    ragged rows and column counts that are not multiples of 16 or 4, into a pitched output whose
+    other columns keep their values."""
+    import ctypes as C
+
+    from ojas_amd.backend import BF16, F32
+
+    print(f"gemm thin {rows}x{k}x{n} b_km={b_km} f32_out={f32_out}", flush=True)
+    be.set_option("gemm_dma", 1)
+    rng = orc.SplitMix64(9900 + rows + k + n)
+    a = orc.round_bf16(rng.vec(rows * k, 0.5)).reshape(rows, k)
+    b = orc.round_bf16(rng.vec(k * n, 0.5)).reshape(k, n)  # B[k, n]
+    ldc = n + 8
+    held = orc.round_bf16(rng.vec(rows * ldc, 1.0)).reshape(rows, ldc)
+    da = be.upload(a, BF16)
+    db = be.upload(b if b_km else np.ascontiguousarray(b.T), BF16)
+    b_rs, b_cs = (n, 1) if b_km else (1, k)
+    od = F32 if f32_out else BF16
+    outs = []
+    for thin in (1, 0):
+        be.set_option("gemm_thin", thin)
+        out = be.upload(held, od)
+        assert be._lib.omx_gemm_pitched(
+            be._ctx, C.c_void_p(da.ptr), C.c_uint64(k), C.c_uint64(1), C.c_void_p(db.ptr), C.c_uint64(b_rs),
+            C.c_uint64(b_cs), C.c_int32(BF16), C.c_void_p(out.ptr), C.c_int32(od), C.c_uint64(ldc), C.c_uint64(rows),
+            C.c_uint64(k), C.c_uint64(n), C.c_int32(0)) == 0
+        outs.append(be.download_f32(out).reshape(rows, ldc))
+    be.set_option("gemm_thin", 1)
+    want = a.astype(np.float64) @ b.astype(np.float64)
+    scale = max(1.0, float(np.max(np.abs(want))))
+    for got in outs:
+        assert np.array_equal(got[:, n:], held[:, n:])
+        assert float(np.max(np.abs(got[:, :n] - want))) <= (1e-5 if f32_out else 2e-2) * scale
+    assert float(np.max(np.abs(outs[0][:, :n] - outs[1][:, :n]))) <= (2e-6 if f32_out else 8e-3) * scale
+
+
 def test_strided_batch_refuses_bad_strides(be):
     from ojas_amd.backend import BF16, OjasError
 
