@@ -446,42 +446,74 @@ int32_t compute_gates(omx_ctx* ctx, uint32_t fault_op, const void* input, const 
 
 // out[r, c] = add[r, c] + sum_h gz[r, h] w[h, c]: the gate's input gradient (a product with a reduction
 // of `heads` terms) joined to another gradient of the same input. A thread owns four columns and
-// keeps their `heads` weights in registers; a wave reads a row's gz once (lane h holds head h) and
-// hands the values round through readlane. bf16 x bf16 products are exact in f32; the sum runs
-// h = 0, 1, ... in f32.
+// keeps their weights in registers as bf16 pairs of consecutive heads; a wave reads a row's gz once
+// (lane p holds heads 2p and 2p + 1, packed) and hands the pairs round through readlane, so a
+// column takes heads / 2 v_dot2c_f32_bf16 (bf16 x bf16 products are exact in f32; the sum runs
+// pair by pair in f32). The block is d / 4 threads rounded up to whole waves.
 constexpr int GATE_JOIN_HEADS = 16;
+__device__ __forceinline__ float gate_join_dot(unsigned int a, unsigned int b, float acc) {
+  typedef __bf16 bf16_pair __attribute__((ext_vector_type(2)));
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16_pair, a), __builtin_bit_cast(bf16_pair, b), acc, false);
+}
 template <typename TA>
 __global__ __launch_bounds__(256) void gate_input_grad_add_kernel(const unsigned short* __restrict__ gz,
                                                                   const unsigned short* __restrict__ w,
                                                                   const TA* __restrict__ add, float* __restrict__ out,
                                                                   size_t rows, int d, int heads, int rows_per_block,
                                                                   OmxFaultWord* fault, unsigned long long tag) {
+  constexpr int PAIRS = GATE_JOIN_HEADS / 2;
   const int c = static_cast<int>(threadIdx.x) * 4, lane = threadIdx.x & 63;
   const bool live = c < d;
-  float wr[GATE_JOIN_HEADS][4];
+  const int pairs = (heads + 1) / 2;
+  unsigned int wp[PAIRS][4];  // (w[2p][c + e], w[2p + 1][c + e]) as a bf16 pair
 #pragma unroll
-  for (int h = 0; h < GATE_JOIN_HEADS; ++h) {
+  for (int p = 0; p < PAIRS; ++p) {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) wr[h][e] = 0.0f;
-    if (live && h < heads) dev_load4<unsigned short>(w + static_cast<size_t>(h) * d, c, wr[h]);
+    for (int e = 0; e < 4; ++e) wp[p][e] = 0u;
+    if (live && p < pairs) {
+      const uint2 lo = *reinterpret_cast<const uint2*>(w + static_cast<size_t>(2 * p) * d + c);
+      uint2 hi = make_uint2(0u, 0u);
+      if (2 * p + 1 < heads) hi = *reinterpret_cast<const uint2*>(w + static_cast<size_t>(2 * p + 1) * d + c);
+      wp[p][0] = (lo.x & 0xffffu) | (hi.x << 16);
+      wp[p][1] = (lo.x >> 16) | (hi.x & 0xffff0000u);
+      wp[p][2] = (lo.y & 0xffffu) | (hi.y << 16);
+      wp[p][3] = (lo.y >> 16) | (hi.y & 0xffff0000u);
+    }
   }
   const size_t r0 = static_cast<size_t>(blockIdx.x) * rows_per_block;
   const size_t r1 = r0 + rows_per_block < rows ? r0 + rows_per_block : rows;
   bool bad = false;
-  for (size_t r = r0; r < r1; ++r) {
-    const float zv = lane < heads ? dev_load<unsigned short>(gz + r * heads, lane) : 0.0f;
-    float a[4] = {0.0f, 0.0f, 0.0f, 0.0f}, acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (live) dev_load4<TA>(add + r * d, c, a);
+  constexpr int G = 4;  // rows whose loads are in flight together
+  for (size_t rg = r0; rg < r1; rg += G) {
+    unsigned int zv[G];
+    float a[G][4];
 #pragma unroll
-    for (int h = 0; h < GATE_JOIN_HEADS; ++h) {
-      const float z = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(zv), h));
+    for (int i = 0; i < G; ++i) {
+      const size_t r = rg + i < r1 ? rg + i : r1 - 1;
+      const unsigned short* zr = gz + r * heads;
+      zv[i] = 0u;
+      if (2 * lane < heads) zv[i] = zr[2 * lane];
+      if (2 * lane + 1 < heads) zv[i] |= static_cast<unsigned int>(zr[2 * lane + 1]) << 16;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) acc[e] = fmaf(z, wr[h][e], acc[e]);
+      for (int e = 0; e < 4; ++e) a[i][e] = 0.0f;
+      if (live) dev_load4<TA>(add + r * d, c, a[i]);
     }
-    if (live) {
-      float4 o = make_float4(a[0] + acc[0], a[1] + acc[1], a[2] + acc[2], a[3] + acc[3]);
-      bad |= !(dev_finite(o.x) && dev_finite(o.y) && dev_finite(o.z) && dev_finite(o.w));
-      *reinterpret_cast<float4*>(out + r * d + c) = o;
+#pragma unroll
+    for (int i = 0; i < G; ++i) {
+      float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int p = 0; p < PAIRS; ++p) {
+        if (p < pairs) {
+          const unsigned int z = static_cast<unsigned int>(__builtin_amdgcn_readlane(static_cast<int>(zv[i]), p));
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[e] = gate_join_dot(z, wp[p][e], acc[e]);
+        }
+      }
+      if (live && rg + i < r1) {
+        float4 o = make_float4(a[i][0] + acc[0], a[i][1] + acc[1], a[i][2] + acc[2], a[i][3] + acc[3]);
+        bad |= !(dev_finite(o.x) && dev_finite(o.y) && dev_finite(o.z) && dev_finite(o.w));
+        *reinterpret_cast<float4*>(out + (rg + i) * d + c) = o;
+      }
     }
   }
   if (bad) dev_raise_fault(fault, tag);
@@ -739,10 +771,11 @@ int32_t omx_per_head_sigmoid_gate_input_grad_add(omx_ctx* ctx, const void* gz, c
                        (add_dtype == OMX_BF16 || (reinterpret_cast<uintptr_t>(add_in) & 15u) == 0);
   if (operand_dtype == OMX_BF16 && d_model % 4 == 0 && d_model <= 1024 && heads <= GATE_JOIN_HEADS && aligned) {
     const int rows_per_block = 8;
+    const unsigned threads = static_cast<unsigned>((d_model / 4 + 63) / 64 * 64);
     const unsigned long long tag = omx_tag(ctx, F_GATE_BACKWARD);
     dim3 grid(static_cast<unsigned>((rows + rows_per_block - 1) / rows_per_block));
 #define GATE_JOIN(TA_)                                                                                        \
-  hipLaunchKernelGGL(gate_input_grad_add_kernel<TA_>, grid, dim3(256), 0, ctx->stream,                        \
+  hipLaunchKernelGGL(gate_input_grad_add_kernel<TA_>, grid, dim3(threads), 0, ctx->stream,                    \
                      static_cast<const unsigned short*>(gz), static_cast<const unsigned short*>(weight),      \
                      static_cast<const TA_*>(add_in), static_cast<float*>(out), rows, static_cast<int>(d_model), \
                      static_cast<int>(heads), rows_per_block, ctx->fault, tag)
