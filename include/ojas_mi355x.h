@@ -285,7 +285,8 @@ int32_t omx_rms_norm_backward(omx_ctx* ctx, const void* x, int32_t x_dtype, cons
  *     (ojas-model/src/block.rs:247-249; sum is f32);
  *   gx = residual_grad + rms_norm_backward(x, w, gy).gx, the gradient fan-in at
  *     a residual (ojas-autograd/src/tape.rs:2565-2591); gx is f32, gx_bf16
- *     (may be null) receives the same values rounded to bf16. */
+ *     (may be null) receives the same values rounded to bf16; gw_f32 may be null for a
+ *     frozen weight, whose gradient is then not formed. */
 int32_t omx_residual_add_rms_norm_forward(omx_ctx* ctx, const void* x, int32_t x_dtype,
                                           const void* y, int32_t y_dtype, const void* w_f32,
                                           void* sum_f32, void* normed, int32_t normed_dtype,

@@ -522,11 +522,13 @@ class MiBackend:
             self._p(normed), C.c_int32(od), C.c_uint64(x.numel // dim), C.c_uint64(dim), C.c_float(eps)))
         return total, normed
 
-    def rms_norm_backward_residual(self, x, w, gy, residual_grad, eps: float = 1e-6, want_bf16: bool = False):
+    def rms_norm_backward_residual(self, x, w, gy, residual_grad, eps: float = 1e-6, want_bf16: bool = False,
+                                   want_weight_grad: bool = True):
         """`rms_norm_backward` whose input gradient is added to `residual_grad` (f32):
-        returns (gx f32, gx bf16 or None, gw)."""
+        returns (gx f32, gx bf16 or None, gw; gw is None and not formed with `want_weight_grad=False`,
+        for a frozen weight)."""
         dim = x.shape[-1]
-        gx, gw = self.empty(x.shape, F32), self.empty((dim,), F32)
+        gx, gw = self.empty(x.shape, F32), (self.empty((dim,), F32) if want_weight_grad else None)
         gx16 = self.empty(x.shape, BF16) if want_bf16 else None
         self._check(self._lib.omx_rms_norm_backward_residual(
             self._ctx, self._p(x), C.c_int32(x.dtype), self._p(w), self._p(gy), C.c_int32(gy.dtype),

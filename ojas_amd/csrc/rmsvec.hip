@@ -106,6 +106,7 @@ __global__ __launch_bounds__(RV_THREADS) void rms_bwd_vec_kernel(
     const TX* __restrict__ x, const float* __restrict__ w, const TG* __restrict__ gy, const float* __restrict__ add_in,
     TO* __restrict__ gx, unsigned short* __restrict__ gx16, float* __restrict__ partial, size_t rows, int dim,
     float eps, int rows_per_block, OmxFaultWord* fault, unsigned long long tag) {
+  const bool want_w = partial != nullptr;  // a frozen weight: no column sums
   extern __shared__ float lds[];  // [4][dim]
   const unsigned lane = threadIdx.x & 63;
   const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -118,7 +119,7 @@ __global__ __launch_bounds__(RV_THREADS) void rms_bwd_vec_kernel(
   for (int j = 0; j < NCH; ++j) {
     const unsigned c = j * 256 + lane * 4;
     if constexpr (WIDE) {
-      if (FULL || c < udim) *reinterpret_cast<float4*>(mine + c) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      if (want_w && (FULL || c < udim)) *reinterpret_cast<float4*>(mine + c) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     } else {
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -223,26 +224,30 @@ __global__ __launch_bounds__(RV_THREADS) void rms_bwd_vec_kernel(
       for (int e = 0; e < 4; ++e) bad |= !dev_finite(out[e]);
       if (FULL || c < udim) {
         if constexpr (WIDE) {
-          float4 a = *reinterpret_cast<const float4*>(mine + c);
-          a.x += aw[0]; a.y += aw[1]; a.z += aw[2]; a.w += aw[3];
-          *reinterpret_cast<float4*>(mine + c) = a;
+          if (want_w) {
+            float4 a = *reinterpret_cast<const float4*>(mine + c);
+            a.x += aw[0]; a.y += aw[1]; a.z += aw[2]; a.w += aw[3];
+            *reinterpret_cast<float4*>(mine + c) = a;
+          }
         }
         dev_store4<TO>(outr, c, out);
         if (gx16) dev_store4<unsigned short>(out16r, c, out);
       }
     }
   }
-  if constexpr (!WIDE) {
+  if (want_w) {  // uniform over the grid
+    if constexpr (!WIDE) {
 #pragma unroll
-    for (int j = 0; j < NCH; ++j) {
-      const unsigned c = j * 256 + lane * 4;
-      if (FULL || c < udim) dev_store4<float>(mine, c, accw[j]);
+      for (int j = 0; j < NCH; ++j) {
+        const unsigned c = j * 256 + lane * 4;
+        if (FULL || c < udim) dev_store4<float>(mine, c, accw[j]);
+      }
     }
-  }
-  __syncthreads();
-  for (unsigned c = threadIdx.x; c < udim; c += RV_THREADS) {
-    float s = ((lds[c] + lds[udim + c]) + lds[2 * udim + c]) + lds[3 * udim + c];
-    partial[static_cast<size_t>(blockIdx.x) * udim + c] = s;
+    __syncthreads();
+    for (unsigned c = threadIdx.x; c < udim; c += RV_THREADS) {
+      float s = ((lds[c] + lds[udim + c]) + lds[2 * udim + c]) + lds[3 * udim + c];
+      partial[static_cast<size_t>(blockIdx.x) * udim + c] = s;
+    }
   }
   if (bad) dev_raise_fault(fault, tag);
 }
@@ -309,11 +314,15 @@ int32_t omx_rms_backward_vec(omx_ctx* ctx, const void* x, int32_t x_dtype, const
   int rows_per_block = 8;
   while (rows_per_block < (dim > 1024 ? 16 : 32) && rows / rows_per_block > 512) rows_per_block *= 2;
   const uint64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
-  void* ws = nullptr;
-  int32_t rc = omx_workspace(ctx, (blocks + OMX_COLUMN_SUM_GROUPS) * dim * sizeof(float), &ws);
-  if (rc != OMX_OK) return rc;
-  float* partial = static_cast<float*>(ws);
-  float* scratch = partial + blocks * dim;
+  // A null gw: the weight is frozen, its gradient is not formed (no partial sums, no second launch).
+  float *partial = nullptr, *scratch = nullptr;
+  if (gw) {
+    void* ws = nullptr;
+    int32_t rc = omx_workspace(ctx, (blocks + OMX_COLUMN_SUM_GROUPS) * dim * sizeof(float), &ws);
+    if (rc != OMX_OK) return rc;
+    partial = static_cast<float*>(ws);
+    scratch = partial + blocks * dim;
+  }
   dim3 grid(static_cast<unsigned>(blocks)), block(RV_THREADS);
   const size_t smem = 4 * dim * sizeof(float);
   const int nch = static_cast<int>((dim + 255) / 256);
@@ -329,12 +338,12 @@ int32_t omx_rms_backward_vec(omx_ctx* ctx, const void* x, int32_t x_dtype, const
   do {                                                                                                               \
     if (full)                                                                                                        \
       omx_launch_timed(ctx, rms_bwd_vec_kernel<TX, TG, TO, N, (N > 4), true>, grid, block, smem, timer.start(),      \
-                       nullptr, static_cast<const TX*>(x), w, static_cast<const TG*>(gy), add_in,                    \
+                       gw ? nullptr : timer.stop(), static_cast<const TX*>(x), w, static_cast<const TG*>(gy), add_in,                    \
                        static_cast<TO*>(gx), static_cast<h16*>(gx16), partial, static_cast<size_t>(rows),            \
                        static_cast<int>(dim), eps, rows_per_block, ctx->fault, tag);                                 \
     else                                                                                                             \
       omx_launch_timed(ctx, rms_bwd_vec_kernel<TX, TG, TO, N, (N > 4), false>, grid, block, smem, timer.start(),     \
-                       nullptr, static_cast<const TX*>(x), w, static_cast<const TG*>(gy), add_in,                    \
+                       gw ? nullptr : timer.stop(), static_cast<const TX*>(x), w, static_cast<const TG*>(gy), add_in,                    \
                        static_cast<TO*>(gx), static_cast<h16*>(gx16), partial, static_cast<size_t>(rows),            \
                        static_cast<int>(dim), eps, rows_per_block, ctx->fault, tag);                                 \
   } while (0)
@@ -363,6 +372,7 @@ int32_t omx_rms_backward_vec(omx_ctx* ctx, const void* x, int32_t x_dtype, const
 #undef RV_BWD_N
 #undef RV_BWD
   OMX_LAUNCH_CHECK(ctx, "rms_bwd_vec_kernel");
+  if (!gw) return OMX_OK;
   return omx_column_sum(ctx, partial, gw, blocks, dim, tag, scratch, timer.stop());
 }
 
@@ -391,11 +401,16 @@ int32_t omx_rms_norm_backward_residual(omx_ctx* ctx, const void* x, int32_t x_dt
                                        uint64_t rows, uint64_t dim, float eps) {
   OMX_REQUIRE_CTX(ctx);
   const char* op = "rms_norm_backward_residual";
-  if (!x || !w || !gy || !residual_grad || !gx || !gw) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  if (!x || !w || !gy || !residual_grad || !gx) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
   if (!omx_valid_float_dtype(x_dtype) || !omx_valid_float_dtype(gy_dtype))
     return omx_fail(ctx, OMX_DTYPE, "%s: dtype must be f32 or bf16", op);
   if (rows == 0 || dim == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
   if (!(eps == eps) || eps == INFINITY || eps == -INFINITY) return omx_fail(ctx, OMX_NON_FINITE, "%s", op);
+  if (!gw && !omx_rms_vec_eligible(dim, {x, w, gy, residual_grad, gx, gx_bf16})) {
+    // The separate kernels below always form the weight gradient: it goes to scratch.
+    int32_t wrc = omx_workspace(ctx, dim * sizeof(float), &gw, 1);
+    if (wrc != OMX_OK) return wrc;
+  }
   if (omx_rms_vec_eligible(dim, {x, w, gy, residual_grad, gx, gx_bf16, gw}))
     return omx_rms_backward_vec(ctx, x, x_dtype, static_cast<const float*>(w), gy, gy_dtype,
                                 static_cast<const float*>(residual_grad), gx, OMX_F32, gx_bf16,

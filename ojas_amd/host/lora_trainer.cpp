@@ -205,7 +205,7 @@ int32_t backward(olora* t) {
     uint16_t* gqkv = off16(t->gqkv_all, l * N * 3 * d);
     uint16_t* gh = off16(t->gh_all, l * N * 4 * r);
     TRY(omx_rms_norm_backward_residual(ctx, A.x1, OMX_F32, t->norm(l, 1), t->t_a, OMX_BF16, t->gres, t->gres1, gy_mid,
-                                       t->dummy_gw, N, d, eps));
+                                       nullptr, N, d, eps));  // the norms are frozen: no weight gradient
     // x1 = x + lora_linear(ap; Wo, Ao, Bo). With gy the gradient of the site's output:
     //   gh = gy B_eff [N, r];  dB_eff = gy^T h;  dA = gh^T x;  gx = gy W + gh A.
     TRY(omx_gemm_pitched(ctx, gy_mid, d, 1, t->b16(l, 3), r, 1, OMX_BF16, off16(gh, 3 * r), OMX_BF16, 4 * r, N, d, r, 0));
@@ -223,7 +223,7 @@ int32_t backward(olora* t) {
     omx_low_rank lr_qkv{gh, t->at(l), 4 * r, 4 * r, 3 * r, 0};
     TRY(q8_backward(t, A.qkv, gqkv, &lr_qkv, t->t_b));
     TRY(omx_rms_norm_backward_residual(ctx, A.x, OMX_F32, t->norm(l, 0), t->t_b, OMX_BF16, t->gres1, t->gres, t->gy16,
-                                       t->dummy_gw, N, d, eps));
+                                       nullptr, N, d, eps));
   }
   // The adapters' weight gradients, every layer's in one launch per site: dB_eff = gy^T h for q, k,
   // v and o; dA = gh^T x for [Aq; Ak; Av] (adjacent in the arena: one product) and for Ao.

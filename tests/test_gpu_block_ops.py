@@ -424,6 +424,10 @@ def test_fused_residual_rms_norm_equals_the_separate_ops(be, rows, dim, bf16):
         # f32 gradients: the fused sum is the separate kernels' f32 add of the same two values.
         sep = be.residual_add_forward(dres, gx_plain, F32)
         assert np.array_equal(be.download(gx), be.download(sep))
+    # A frozen weight: the same input gradient (and its bf16 copy) without the weight gradient.
+    gx_f, gx16_f, none = be.rms_norm_backward_residual(dx, dw, dgy, dres, 1e-6, want_bf16=True, want_weight_grad=False)
+    assert none is None
+    assert np.array_equal(be.download(gx_f), be.download(gx)) and np.array_equal(be.download(gx16_f), be.download(gx16))
 
 
 def test_fused_gelu_side_tensor_off_the_vector_boundary(be):
