@@ -258,6 +258,61 @@ __global__ __launch_bounds__(1024) void scan_counts_kernel(const unsigned int* _
   if (threadIdx.x == 0) offsets[vocab] = carry;
 }
 
+// The same scan over many blocks, for tables of more than a few thousand rows (one block walks
+// 50304 counts in 55 us): every block of 1024 counts leaves its total, then every block adds up the
+// totals before it (at most SCAN_MAX_BLOCKS of them) and scans its own counts behind that.
+constexpr int SCAN_MAX_BLOCKS = 1024;
+__device__ __forceinline__ unsigned int scan_block_1024(unsigned int v, unsigned int* wave_tot, unsigned int* total) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  unsigned int incl = v;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    unsigned int t = __shfl_up(incl, off, 64);
+    if (lane >= off) incl += t;
+  }
+  if (lane == 63) wave_tot[wave] = incl;
+  __syncthreads();
+  unsigned int before = 0, all = 0;
+  for (int wv = 0; wv < 16; ++wv) {
+    if (wv < wave) before += wave_tot[wv];
+    all += wave_tot[wv];
+  }
+  *total = all;
+  return before + incl - v;  // exclusive, within the block
+}
+__global__ __launch_bounds__(1024) void scan_totals_kernel(const unsigned int* __restrict__ counts,
+                                                           unsigned int* __restrict__ totals, size_t vocab) {
+  __shared__ unsigned int wave_tot[16];
+  const size_t i = static_cast<size_t>(blockIdx.x) * 1024 + threadIdx.x;
+  unsigned int total;
+  scan_block_1024(i < vocab ? counts[i] : 0u, wave_tot, &total);
+  if (threadIdx.x == 0) totals[blockIdx.x] = total;
+}
+__global__ __launch_bounds__(1024) void scan_blocks_kernel(const unsigned int* __restrict__ counts,
+                                                           const unsigned int* __restrict__ totals,
+                                                           unsigned int* __restrict__ offsets,
+                                                           unsigned int* __restrict__ cursor, size_t vocab) {
+  __shared__ unsigned int wave_tot[16];
+  __shared__ unsigned int lead_tot[16];
+  // The totals of the blocks before this one: thread t takes block t's.
+  unsigned int mine = threadIdx.x < blockIdx.x ? totals[threadIdx.x] : 0u;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) mine += __shfl_xor(mine, off, 64);
+  if ((threadIdx.x & 63) == 0) lead_tot[threadIdx.x >> 6] = mine;
+  __syncthreads();
+  unsigned int lead = 0;
+  for (int wv = 0; wv < 16; ++wv) lead += lead_tot[wv];
+  const size_t i = static_cast<size_t>(blockIdx.x) * 1024 + threadIdx.x;
+  const unsigned int v = i < vocab ? counts[i] : 0u;
+  unsigned int total;
+  const unsigned int excl = lead + scan_block_1024(v, wave_tot, &total);
+  if (i < vocab) {
+    offsets[i] = excl;
+    cursor[i] = excl;
+  }
+  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) offsets[vocab] = lead + total;
+}
+
 __global__ void fill_positions_kernel(const unsigned int* __restrict__ ids, unsigned int* __restrict__ cursor,
                                       unsigned int* __restrict__ positions, size_t tokens, size_t vocab) {
   size_t n = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
@@ -738,7 +793,8 @@ static int32_t embedding_backward_impl(omx_ctx* ctx, const void* ids, const void
     return omx_fail(ctx, OMX_OUT_OF_RANGE, "%s: axis does not fit in u32", op);
   // Workspace: counts[V], offsets[V+1], cursor[V], positions[N], sorted[N], the count of rows with
   // more than 64 tokens (one word, padded to four) and their list (at most N / 65 of them).
-  uint64_t words = vocab + (vocab + 1) + vocab + tokens + tokens + 4 + (tokens / 64 + 1);
+  const uint64_t scan_blocks = (vocab + 1023) / 1024;
+  uint64_t words = vocab + (vocab + 1) + vocab + tokens + tokens + 4 + (tokens / 64 + 1) + scan_blocks + 4;
   void* ws = nullptr;
   int32_t rc = omx_workspace(ctx, words * 4, &ws);
   if (rc != OMX_OK) return rc;
@@ -749,6 +805,7 @@ static int32_t embedding_backward_impl(omx_ctx* ctx, const void* ids, const void
   unsigned int* sorted = positions + tokens;
   unsigned int* long_count = sorted + tokens;
   unsigned int* long_rows = long_count + 4;
+  unsigned int* scan_totals = long_rows + (tokens / 64 + 1);
   unsigned long long tag = omx_tag(ctx, F_EMBEDDING_BACKWARD);
   rc = omx_fill_zero(ctx, counts, vocab * 4);
   if (rc != OMX_OK) return rc;
@@ -765,8 +822,16 @@ static int32_t embedding_backward_impl(omx_ctx* ctx, const void* ids, const void
   omx_launch_timed(ctx, count_ids_kernel, tgrid, dim3(256), 0, timer.start(), nullptr, idp, counts, tokens, vocab,
                    ctx->fault, tag);
   OMX_LAUNCH_CHECK(ctx, "count_ids_kernel");
-  hipLaunchKernelGGL(scan_counts_kernel, dim3(1), dim3(1024), 0, ctx->stream, counts, offsets, cursor, vocab);
-  OMX_LAUNCH_CHECK(ctx, "scan_counts_kernel");
+  if (scan_blocks > 4 && scan_blocks <= SCAN_MAX_BLOCKS) {
+    const dim3 sgrid(static_cast<unsigned>(scan_blocks));
+    hipLaunchKernelGGL(scan_totals_kernel, sgrid, dim3(1024), 0, ctx->stream, counts, scan_totals, vocab);
+    OMX_LAUNCH_CHECK(ctx, "scan_totals_kernel");
+    hipLaunchKernelGGL(scan_blocks_kernel, sgrid, dim3(1024), 0, ctx->stream, counts, scan_totals, offsets, cursor, vocab);
+    OMX_LAUNCH_CHECK(ctx, "scan_blocks_kernel");
+  } else {
+    hipLaunchKernelGGL(scan_counts_kernel, dim3(1), dim3(1024), 0, ctx->stream, counts, offsets, cursor, vocab);
+    OMX_LAUNCH_CHECK(ctx, "scan_counts_kernel");
+  }
   hipLaunchKernelGGL(fill_positions_kernel, tgrid, dim3(256), 0, ctx->stream, idp, cursor, positions, tokens, vocab);
   OMX_LAUNCH_CHECK(ctx, "fill_positions_kernel");
   dim3 vgrid(static_cast<unsigned>((vocab + 3) / 4));
