@@ -48,6 +48,7 @@ struct ogpt {
   std::vector<void*> owned;
 
   float *p32 = nullptr, *g32 = nullptr, *m1 = nullptr, *m2 = nullptr;
+  uint64_t adamw_end = 0;  // the tables and the norm weights are arena elements [0, adamw_end)
   void* p16 = nullptr;
   uint32_t *ids = nullptr, *targets = nullptr, *positions = nullptr;
   float* loss = nullptr;
@@ -264,7 +265,7 @@ int32_t backward(ogpt* t) {
     // gw[l](o, j) = sum_r gy[l][r, o] * x[l][r, j] for every layer l in one launch per weight:
     // 4 x layers long reductions with small outputs become four products with enough tiles to fill
     // the chip without splitting K.
-    const uint64_t layers = c.layers, per_layer = t->slots[t->li(1, 0)].offset - t->slots[t->li(0, 0)].offset;
+    const uint64_t layers = c.layers, per_layer = t->slots[t->li(1, 1)].offset - t->slots[t->li(0, 1)].offset;
     struct Deferred {
       const void *gy, *x;
       uint64_t which, out, in;
@@ -301,10 +302,10 @@ int32_t ogpt_create(omx_ctx* ctx, const ogpt_config* config, ogpt** out) {
   t->AD = c.bf16 ? OMX_BF16 : OMX_F32;
   t->asz = c.bf16 ? 2 : 4;
   const uint64_t d = c.d_model, M = c.mlp, N = t->N;
-  auto push = [&](uint64_t len) {
-    t->slots.push_back({t->P, len});
-    t->P += (len + kAlign - 1) / kAlign * kAlign;
-  };
+  // Slots in the parameter order of the header; places in the arena: the two tables, then every
+  // norm weight, then the layers' matrices (a layer's six together, layers at a fixed stride), so
+  // that what AdamW owns under the hybrid step is one range and takes one launch.
+  auto push = [&](uint64_t len) { t->slots.push_back({0, len}); };
   push(static_cast<uint64_t>(c.vocab) * d);
   push(static_cast<uint64_t>(c.ctx) * d);
   for (uint32_t l = 0; l < c.layers; ++l) {
@@ -315,6 +316,20 @@ int32_t ogpt_create(omx_ctx* ctx, const ogpt_config* config, ogpt** out) {
     push(d * M);
   }
   push(d);
+  auto place = [&](uint64_t i) {
+    t->slots[i].offset = t->P;
+    t->P += (t->slots[i].len + kAlign - 1) / kAlign * kAlign;
+  };
+  place(0);
+  place(1);
+  for (uint64_t l = 0; l < c.layers; ++l) {
+    place(t->li(l, 0));
+    place(t->li(l, 5));
+  }
+  place(t->nf());
+  t->adamw_end = t->P;  // [0, adamw_end): tables and norm weights
+  for (uint64_t l = 0; l < c.layers; ++l)
+    for (uint64_t w : {1, 2, 3, 4, 6, 7}) place(t->li(l, w));
   // wq, wk, wv sit back to back when d*d needs no padding.
   t->fused_qkv = c.bf16 && c.head_dim == 64 && (d * d) % kAlign == 0;
   auto fail = [&](int32_t rc) {
@@ -569,11 +584,6 @@ int32_t ogpt_step_hybrid(ogpt* t, const omx_muon_config* muon, const omx_adamw_c
   int32_t bounded = 0;
   TRY(adamw_inputs_bounded(t, ogpt::kHybrid, norm, &bounded));
   t->tracked = ogpt::kNone;  // until the readback at the end has seen this step through
-  auto adam = [&](uint64_t first, uint64_t last) -> int32_t {  // slots [first, last] are adjacent in the arena
-    const uint64_t at = t->slots[first].offset, n = t->slots[last].offset + t->slots[last].len - at;
-    return omx_adamw_step_bounded(t->ctx, t->p32 + at, t->g32 + at, t->m1 + at, t->m2 + at, n, t->steps, adamw,
-                                  mirror ? mirror + at : nullptr, bounded, t->unbounded);
-  };
   const uint64_t d = t->c.d_model, mlp = t->c.mlp;
   // Matrices of one shape go through Newton-Schulz together: three batched calls per step.
   struct Group {
@@ -589,15 +599,15 @@ int32_t ogpt_step_hybrid(ogpt* t, const omx_muon_config* muon, const omx_adamw_c
     grp.m.push_back(t->m1 + at);
     grp.p16.push_back(mirror ? mirror + at : nullptr);
   };
-  TRY(adam(0, 1));  // token and position tables
+  // The tables and every norm weight lie together at the front of the arena (padding between
+  // them holds zeros in all four arenas and stays zero): one AdamW launch.
+  TRY(omx_adamw_step_bounded(t->ctx, t->p32, t->g32, t->m1, t->m2, t->adamw_end, t->steps, adamw, mirror, bounded,
+                             t->unbounded));
   for (uint64_t l = 0; l < t->c.layers; ++l) {
-    TRY(adam(t->li(l, 0), t->li(l, 0)));
     for (uint64_t w = 1; w <= 4; ++w) add(groups[0], t->li(l, w));
-    TRY(adam(t->li(l, 5), t->li(l, 5)));
     add(groups[1], t->li(l, 6));
     add(groups[2], t->li(l, 7));
   }
-  TRY(adam(t->nf(), t->nf()));
   for (Group& grp : groups)
     TRY(omx_muon_ns5_step_batched(t->ctx, grp.p.data(), grp.g.data(), grp.m.data(), mirror ? grp.p16.data() : nullptr,
                                   grp.p.size(), grp.rows, grp.cols, muon));
