@@ -228,12 +228,13 @@ def kv_decode(args) -> int:
 
 def attention(args) -> int:
     """Secondary workload: the training step's attention alone, forward + backward of one block's
-    causal attention at the headline shape (batch 16, 12 heads, 1024 tokens, head_dim 64, bf16)
-    through `causal_sdpa_forward` / `causal_sdpa_backward`. `value` is causal-counted TFLOP/s over
-    both passes (forward 2 B H T^2 D, backward 5 B H T^2 D)."""
+    causal attention at the headline shape (batch 16, 12 heads, 1024 tokens, head_dim 64, bf16;
+    `--attention-batch 8` is the isolated attention case of the baseline's configs) through
+    `causal_sdpa_forward` / `causal_sdpa_backward`. `value` is causal-counted TFLOP/s over both
+    passes (forward 2 B H T^2 D, backward 5 B H T^2 D)."""
     from ojas_amd.backend import BF16, MiBackend
 
-    b, h, t, d = 16, 12, 1024, 64
+    b, h, t, d = args.attention_batch, 12, 1024, 64
     be = MiBackend(0)
     r = np.random.default_rng(0)
     q, k, v, gy = (be.upload(r.standard_normal((b, h, t, d)).astype(np.float32), BF16) for _ in range(4))
@@ -253,11 +254,11 @@ def attention(args) -> int:
     flops = {"forward": unit, "backward": 2.5 * unit}
     total = sum(times.values())
     line = {
-        "metric": "causal attention forward + backward (B16 H12 T1024 D64 bf16): causal-counted TFLOP/s",
+        "metric": f"causal attention forward + backward (B{b} H12 T1024 D64 bf16): causal-counted TFLOP/s",
         "value": sum(flops.values()) / total / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": total * 1e3, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "causal_sdpa_forward + causal_sdpa_backward: q, k, v [16,12,1024,64] bf16",
+        "config": {"workload": f"causal_sdpa_forward + causal_sdpa_backward: q, k, v [{b},12,1024,64] bf16",
                    "tokens_per_step": b * t},
         "roofline": {"bound": "mfma", "kernel": "flash_fwd_kernel; flash_key_mean_kernel + flash_bwd_dq_kernel + "
                                                 "flash_bwd_dkv_kernel",
@@ -552,6 +553,7 @@ def main() -> int:
     ap.add_argument("--optimizer", default="adamw", choices=["adamw", "muon"],
                     help="adamw: BASELINE configs[2], the headline (default); muon: configs[3], Muon-NS5 (bf16 "
                          "iteration, lr 0.02, momentum 0.95) on the hidden matrices and AdamW on tables and norms")
+    ap.add_argument("--attention-batch", type=int, default=16, help="batch of --workload attention")
     ap.add_argument("--workload", default="train_step", choices=["train_step", "kv_decode", "attention"],
                     help="train_step: the headline metric (default); kv_decode: the decode attention op alone; "
                          "attention: the step's causal attention alone, forward + backward")
