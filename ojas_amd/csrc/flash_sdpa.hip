@@ -44,6 +44,10 @@ struct FlashStrides {
 };
 struct FlashShape {
   int batch, heads, kv_heads, time, window, rep;
+  // One 128-row block per workgroup instead of a mirrored pair, heaviest blocks first (query side:
+  // forward and dQ; key side: dK/dV). Chosen by the host when the pairs would leave workgroup
+  // places empty (few planes) or, on the key side, need a half-empty second round.
+  int q_single, kv_single;
   float scale;
   FlashStrides q, kv, o;  // q and grad_q; k, v and their gradients; out and grad_out
 };
@@ -241,8 +245,13 @@ __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_fwd_kernel(const un
   const int q_blocks = (T + 127) / 128;
   int pair;
   long plane;
-  flash_block_of((q_blocks + 1) / 2, s.batch * s.heads, &pair, &plane);
-  for (int pass = 0; pass < 2; ++pass) {
+  if (s.q_single) {  // block rank (0 = the last, heaviest block) in the high part of the index
+    pair = static_cast<int>(blockIdx.x) / (s.batch * s.heads);
+    plane = static_cast<int>(blockIdx.x) % (s.batch * s.heads);
+  } else {
+    flash_block_of((q_blocks + 1) / 2, s.batch * s.heads, &pair, &plane);
+  }
+  for (int pass = 0; pass < (s.q_single ? 1 : 2); ++pass) {
     const int qb = pass == 0 ? q_blocks - 1 - pair : pair;
     if (pass == 1 && qb >= q_blocks - 1 - pair) break;
     const int h = static_cast<int>(plane % s.heads), b = static_cast<int>(plane / s.heads);
@@ -546,10 +555,15 @@ __global__ __launch_bounds__(FT, 2) void flash_bwd_dkv_kernel(
   const int k_blocks = (s.time + 127) / 128;
   int pair;
   long kv_plane;
-  flash_block_of((k_blocks + 1) / 2, s.batch * s.kv_heads, &pair, &kv_plane);
+  if (s.kv_single) {  // block index (0 = the first, heaviest block) in the high part of the index
+    pair = static_cast<int>(blockIdx.x) / (s.batch * s.kv_heads);
+    kv_plane = static_cast<int>(blockIdx.x) % (s.batch * s.kv_heads);
+  } else {
+    flash_block_of((k_blocks + 1) / 2, s.batch * s.kv_heads, &pair, &kv_plane);
+  }
   const int gidx = static_cast<int>(kv_plane % s.kv_heads), b = static_cast<int>(kv_plane / s.kv_heads);
   bool bad = false;
-  for (int pass = 0; pass < 2; ++pass) {
+  for (int pass = 0; pass < (s.kv_single ? 1 : 2); ++pass) {
     const int kb = pass == 0 ? pair : k_blocks - 1 - pair;
     if (pass == 1 && kb <= pair) break;
     if constexpr (D == 64) {
@@ -613,8 +627,13 @@ __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_bwd_dq_kernel(
   const int q_blocks = (T + 127) / 128;
   int pair;
   long plane;
-  flash_block_of((q_blocks + 1) / 2, s.batch * s.heads, &pair, &plane);
-  for (int pass = 0; pass < 2; ++pass) {
+  if (s.q_single) {  // block rank (0 = the last, heaviest block) in the high part of the index
+    pair = static_cast<int>(blockIdx.x) / (s.batch * s.heads);
+    plane = static_cast<int>(blockIdx.x) % (s.batch * s.heads);
+  } else {
+    flash_block_of((q_blocks + 1) / 2, s.batch * s.heads, &pair, &plane);
+  }
+  for (int pass = 0; pass < (s.q_single ? 1 : 2); ++pass) {
     const int qb = pass == 0 ? q_blocks - 1 - pair : pair;
     if (pass == 1 && qb >= q_blocks - 1 - pair) break;
     const int h = static_cast<int>(plane % s.heads), b = static_cast<int>(plane / s.heads);
@@ -775,15 +794,30 @@ FlashShape make_shape(uint64_t batch, uint64_t heads, uint64_t kv_heads, uint64_
   s.time = static_cast<int>(time);
   s.window = static_cast<int>(window);
   s.rep = static_cast<int>(heads / kv_heads);
+  s.q_single = s.kv_single = 0;
   s.scale = scale;
   return s;
 }
 
+// Whether a pass takes one block per workgroup: when the mirrored pairs are fewer than the chip's
+// workgroup places (`per_cu` per compute unit), twice as many workgroups fill them; `also_rounds`:
+// also when the pairs need more than one round, whose last would run part empty (the blocks go out
+// heaviest first, so the light ones fill the end).
+int flash_single(omx_ctx* ctx, unsigned pair_groups, int per_cu, bool also_rounds) {
+  const unsigned places = static_cast<unsigned>(ctx->cu_count > 0 ? ctx->cu_count : 256) * per_cu;
+  if (pair_groups < places) return 1;
+  return also_rounds && pair_groups > places ? 1 : 0;
+}
+
 template <int D>
 void launch_forward(omx_ctx* ctx, const unsigned short* q, const unsigned short* k, const unsigned short* v, void* out,
-                    int32_t out_dtype, void* out_residual, float* lse, const FlashShape& s, unsigned long long tag) {
-  // Two 128-row query blocks per workgroup (see the kernel).
-  dim3 grid(static_cast<unsigned>((s.time + 127) / 128 + 1) / 2 * s.batch * s.heads), block(FT);
+                    int32_t out_dtype, void* out_residual, float* lse, const FlashShape& shape, unsigned long long tag) {
+  FlashShape s = shape;
+  // Two 128-row query blocks per workgroup (see the kernel), or one when the pairs would not fill
+  // the chip's workgroup places.
+  const unsigned q_blocks = static_cast<unsigned>((s.time + 127) / 128), planes = static_cast<unsigned>(s.batch * s.heads);
+  s.q_single = flash_single(ctx, (q_blocks + 1) / 2 * planes, D == 64 ? 3 : 2, false);
+  dim3 grid((s.q_single ? q_blocks : (q_blocks + 1) / 2) * planes), block(FT);
   // Causal-counted work: half of the 4 B H T^2 D of the two full products.
   OmxKernelTimer timer(ctx, OMX_K_FLASH_FWD, 2.0 * s.batch * s.heads * static_cast<double>(s.time) * s.time * D);
   if (out_dtype == OMX_BF16)
@@ -799,7 +833,8 @@ template <int D>
 void launch_backward(omx_ctx* ctx, const unsigned short* q, const unsigned short* k, const unsigned short* v,
                      const unsigned short* out, const unsigned short* resid, const float* lse, float* delta,
                      float* key_mean, const unsigned short* gy, void* gq, void* gk, void* gv, int32_t grad_dtype,
-                     const FlashShape& s, unsigned long long tag) {
+                     const FlashShape& shape, unsigned long long tag) {
+  FlashShape s = shape;
   // Five causal-counted products (S and dP twice each way, dV, dQ, dK) of B H T^2 D each.
   OmxKernelTimer timer(ctx, OMX_K_FLASH_BWD, 5.0 * s.batch * s.heads * static_cast<double>(s.time) * s.time * D);
   omx_launch_timed(ctx, flash_key_mean_kernel<D>, dim3(static_cast<unsigned>(s.batch * s.kv_heads)), dim3(256), 0,
@@ -807,8 +842,12 @@ void launch_backward(omx_ctx* ctx, const unsigned short* q, const unsigned short
   // dQ first: it also leaves delta = dO . O per row for the dK/dV pass.
   dim3 block(FT);
   const unsigned pairs = static_cast<unsigned>((s.time + 127) / 128 + 1) / 2;  // two 128-row blocks per workgroup
-  dim3 kv_grid(pairs * static_cast<unsigned>(s.batch * s.kv_heads));
-  dim3 q_grid(pairs * static_cast<unsigned>(s.batch * s.heads));
+  const unsigned blocks = static_cast<unsigned>((s.time + 127) / 128);
+  const unsigned kv_planes = static_cast<unsigned>(s.batch * s.kv_heads), q_planes = static_cast<unsigned>(s.batch * s.heads);
+  s.q_single = flash_single(ctx, pairs * q_planes, D == 64 ? 3 : 2, false);
+  s.kv_single = flash_single(ctx, pairs * kv_planes, 2, true);
+  dim3 kv_grid((s.kv_single ? blocks : pairs) * kv_planes);
+  dim3 q_grid((s.q_single ? blocks : pairs) * q_planes);
   if (grad_dtype == OMX_BF16) {
     hipLaunchKernelGGL((flash_bwd_dq_kernel<D, unsigned short>), q_grid, block, 0, ctx->stream, q, k, v, out, resid,
                        lse, delta, key_mean, gy, static_cast<unsigned short*>(gq), s, ctx->fault, tag);
