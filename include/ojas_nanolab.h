@@ -56,6 +56,21 @@ uint64_t onano_steps(onano* t);
  * generator (synthetic weights for benchmarks; the reference's init streams are not restated). */
 int32_t onano_init(onano* t, uint64_t seed);
 
+/* The reference's fresh init, `init_params` (ojas-model/src/init.rs:67-114): parameter `name` draws
+ * from SplitMix64(seed ^ fnv1a(name)) through Box-Muller in f64 (:35-59), `(std * z) as f32` with
+ * std the f32 0.02 widened to f64; norm weights exactly one; o_proj, ffn.down, the gate's bias and
+ * vr_lambda exactly zero (ojas-model/src/names.rs:188-300). Optimizer state and the step count are
+ * cleared. The logarithm, sine and cosine are the C library's, as the reference's are Rust std's. */
+int32_t onano_init_reference(onano* t, uint64_t seed);
+/* Row `index` of the parameter table's name (names.rs:188-300), NUL-terminated. */
+int32_t onano_param_name(onano* t, uint64_t index, char* out, uint64_t capacity);
+/* `init_param` (init.rs:75-112) for one parameter on the host: no device involved. A std that is
+ * not positive and finite is OMX_OUT_OF_RANGE (:101-106). */
+enum { ONANO_INIT_ZEROS = 0, ONANO_INIT_ONES = 1, ONANO_INIT_NORMAL = 2 };
+int32_t onano_reference_init_values(const char* name, uint64_t len, int32_t init, float std_dev, uint64_t seed, float* out);
+/* 64-bit FNV-1a of `len` bytes (init.rs:15-29). */
+uint64_t onano_fnv1a(const char* bytes, uint64_t len);
+
 /* One micro-batch ([batch, seq] ids and targets): forward and backward with the backward started
  * from `loss_seed` (Tape::backward_seeded, trainer.rs:1089-1119). first != 0 starts a step (the
  * accumulated gradient and loss are replaced), otherwise they are added to. `loss_scale` multiplies

@@ -12,6 +12,7 @@
 // Newton-Schulz call); the bf16 tier keeps a bf16 mirror of the parameters that the optimizers
 // refresh. The gate and up projections are adjacent in the arena, so on the bf16 tier they are one
 // [2 hidden, n_embd] matrix whose product feeds the fused SwiGLU.
+#include <cstdio>
 #include <cstdlib>
 #include <cmath>
 #include <cstdint>
@@ -688,6 +689,115 @@ int32_t onano_init(onano* t, uint64_t seed) {
       else if (i != 0 && which == LAMBDA) v = 0.5f;
       else v = 1.0f;
     }
+    TRY(onano_set_param(t, i, host.data()));
+  }
+  TRY(omx_fill_zero(t->ctx, t->m1, t->P * 4));
+  TRY(omx_fill_zero(t->ctx, t->m2, t->P * 4));
+  t->steps = 0;
+  t->tracked = false;
+  return omx_sync(t->ctx);
+}
+
+// ---------------------------------------------------------------------------------------------
+// The reference's fresh init (ojas-model/src/init.rs:55-114): every parameter draws from its own
+// SplitMix64 stream seeded with seed ^ fnv1a(name), through Box-Muller in f64, so a parameter's
+// values depend on the seed and its name alone.
+namespace {
+
+// 64-bit FNV-1a (init.rs:15-29).
+uint64_t fnv1a_64(const char* bytes, size_t n) {
+  uint64_t h = 0xcbf29ce484222325ull;
+  for (size_t i = 0; i < n; ++i) h = (h ^ static_cast<unsigned char>(bytes[i])) * 0x00000100000001b3ull;
+  return h;
+}
+
+// SplitMix64 (ojas-kernels/src/rng.rs; CounterRng of ojas-data/src/rng.rs:10).
+struct CounterStream {
+  uint64_t state;
+  uint64_t next() {
+    state += 0x9e3779b97f4a7c15ull;
+    uint64_t z = state;
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+    return z ^ (z >> 31);
+  }
+};
+
+// Standard normal values in pairs (init.rs:35-59): u1 in (0, 1], u2 in [0, 1) from the top 53 bits
+// of two draws; the cosine branch is returned first, the sine branch kept for the next call.
+struct NormalStream {
+  CounterStream rng;
+  bool has_spare = false;
+  double spare = 0.0;
+  double next() {
+    if (has_spare) {
+      has_spare = false;
+      return spare;
+    }
+    constexpr double ulp53 = 1.0 / 9007199254740992.0;
+    const double u1 = static_cast<double>((rng.next() >> 11) + 1) * ulp53;
+    const double u2 = static_cast<double>(rng.next() >> 11) * ulp53;
+    const double radius = std::sqrt(-2.0 * std::log(u1));
+    const double angle = 6.283185307179586476925286766559 * u2;
+    spare = radius * std::sin(angle);
+    has_spare = true;
+    return radius * std::cos(angle);
+  }
+};
+
+const char* const kBlockNames[kPerBlock] = {
+    "norm1.weight",        "mixer.q_proj.weight", "mixer.k_proj.weight", "mixer.v_proj.weight", "mixer.o_proj.weight",
+    "mixer.q_norm.weight", "mixer.k_norm.weight", "mixer.gate.weight",   "mixer.gate.bias",     "mixer.vr_lambda",
+    "norm2.weight",        "ffn.gate.weight",     "ffn.up.weight",       "ffn.down.weight"};
+// The init rule of each row of the parameter table (ojas-model/src/names.rs:188-300): the output
+// projections o_proj and ffn.down start at zero (:236-243, :290-296), norm weights at one, the
+// gate's bias and vr_lambda at zero, every other matrix at N(0, 0.02).
+const int kBlockInit[kPerBlock] = {ONANO_INIT_ONES,   ONANO_INIT_NORMAL, ONANO_INIT_NORMAL, ONANO_INIT_NORMAL, ONANO_INIT_ZEROS,
+                                   ONANO_INIT_ONES,   ONANO_INIT_ONES,   ONANO_INIT_NORMAL, ONANO_INIT_ZEROS,  ONANO_INIT_ZEROS,
+                                   ONANO_INIT_ONES,   ONANO_INIT_NORMAL, ONANO_INIT_NORMAL, ONANO_INIT_ZEROS};
+
+}  // namespace
+
+uint64_t onano_fnv1a(const char* bytes, uint64_t len) { return bytes || len == 0 ? fnv1a_64(bytes, len) : 0; }
+
+int32_t onano_reference_init_values(const char* name, uint64_t len, int32_t init, float std_dev, uint64_t seed, float* out) {
+  if (!name || (!out && len != 0)) return OMX_PLACEMENT;
+  if (init == ONANO_INIT_ZEROS) {
+    for (uint64_t i = 0; i < len; ++i) out[i] = 0.0f;
+  } else if (init == ONANO_INIT_ONES) {
+    for (uint64_t i = 0; i < len; ++i) out[i] = 1.0f;
+  } else if (init == ONANO_INIT_NORMAL) {
+    if (!(std::isfinite(std_dev) && std_dev > 0.0f)) return OMX_OUT_OF_RANGE;  // init.rs:101-106
+    NormalStream normal{CounterStream{seed ^ fnv1a_64(name, std::strlen(name))}};
+    const double sd = static_cast<double>(std_dev);  // the f32 constant widened, not the decimal 0.02
+    for (uint64_t i = 0; i < len; ++i) out[i] = static_cast<float>(sd * normal.next());
+  } else {
+    return OMX_OUT_OF_RANGE;
+  }
+  return OMX_OK;
+}
+
+int32_t onano_param_name(onano* t, uint64_t index, char* out, uint64_t capacity) {
+  if (!t || !out || index >= t->slots.size()) return OMX_SHAPE;
+  char text[96];
+  if (index == 0) std::snprintf(text, sizeof text, "tok_emb.weight");
+  else if (index == t->nf()) std::snprintf(text, sizeof text, "norm_f.weight");
+  else std::snprintf(text, sizeof text, "blocks.%llu.%s", static_cast<unsigned long long>((index - 1) / kPerBlock), kBlockNames[(index - 1) % kPerBlock]);
+  if (std::strlen(text) + 1 > capacity) return OMX_CAPACITY_EXCEEDED;
+  std::memcpy(out, text, std::strlen(text) + 1);
+  return OMX_OK;
+}
+
+int32_t onano_init_reference(onano* t, uint64_t seed) {
+  if (!t) return OMX_BACKEND;
+  std::vector<float> host;
+  char name[96];
+  for (uint64_t i = 0; i < t->slots.size(); ++i) {
+    const Slot& s = t->slots[i];
+    host.resize(s.len);
+    TRY(onano_param_name(t, i, name, sizeof name));
+    const int32_t init = i == 0 ? ONANO_INIT_NORMAL : i == t->nf() ? ONANO_INIT_ONES : kBlockInit[(i - 1) % kPerBlock];
+    TRY(onano_reference_init_values(name, s.len, init, 0.02f, seed, host.data()));
     TRY(onano_set_param(t, i, host.data()));
   }
   TRY(omx_fill_zero(t->ctx, t->m1, t->P * 4));

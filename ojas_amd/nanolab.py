@@ -338,6 +338,18 @@ class NativeNanolabTrainer:
     def init(self, seed: int):
         self.be._check(self._lib.onano_init(self._h, C.c_uint64(seed)))
 
+    def init_reference(self, seed: int):
+        """`init_params` (ojas-model/src/init.rs:114): the reference's per-name streams."""
+        self.be._check(self._lib.onano_init_reference(self._h, C.c_uint64(seed)))
+
+    def native_param_names(self) -> List[str]:
+        out = []
+        buf = C.create_string_buffer(96)
+        for i in range(len(self.names)):
+            self.be._check(self._lib.onano_param_name(self._h, C.c_uint64(i), buf, C.c_uint64(96)))
+            out.append(buf.value.decode())
+        return out
+
     def set_params(self, host_params: Dict[str, np.ndarray]):
         for i, n in enumerate(self.names):
             a = np.ascontiguousarray(host_params[n], np.float32).reshape(-1)

@@ -203,3 +203,39 @@ def test_steps_follow_the_torch_trace(be, bf16):
     print(f"  worst |bf16 - f32| {gap.max():.2e} at step {int(gap.argmax()) + 1} (bound {bound:.2e})", flush=True)
     assert np.any(gap > 0) and np.all(gap <= bound), (int(gap.argmax()), float(gap.max()))
     assert losses16[39] <= np.log(spec.vocab) - tf.CURVE_MIN_DROP_NATS
+
+
+def test_reference_init_on_the_device(be):
+    """`onano_init_reference`: the parameters on the device are the reference's per-name streams
+    (ojas-model/src/init.rs:67-114) bit for bit, as the oracle's Python restatement draws them;
+    optimizer state zero, no steps taken; both tiers (the bf16 tier keeps f32 masters)."""
+    import sys
+    from pathlib import Path
+
+    sys.path.insert(0, str(Path(__file__).resolve().parent.parent / "oracle"))
+    import init_exact as ie
+    from ojas_amd.nanolab import NanolabSpec, NativeNanolabTrainer
+
+    print("native nanolab: reference init", flush=True)
+    spec = NanolabSpec(n_layer=2, n_embd=128, n_head=2, n_kv_head=1, head_dim=64, hidden=256, vocab=96)
+    table = ie.param_table(spec.n_layer, spec.n_embd, spec.n_head, spec.n_kv_head, spec.head_dim, spec.hidden, spec.vocab)
+    for bf16 in (False, True):
+        tr = NativeNanolabTrainer(be, spec, 2, 64, bf16=bf16)
+        assert tr.native_param_names() == [n for n, _, _ in table] == spec.param_names()
+        for seed in (0, 0xC0FFEE):
+            tr.init_reference(seed)
+            got = tr.download_params()
+            for name, shape, init in table:
+                want = ie.init_values(name, int(np.prod(shape)), init, seed).reshape(shape)
+                assert got[name].shape == tuple(shape)
+                assert (got[name].view(np.uint32) == want.view(np.uint32)).all(), name
+            assert tr.step == 0
+            assert all(not a.any() for slot in (0, 1) for a in tr.state(slot).values())
+        # The zero-initialised output projections make every block the identity at init: the loss
+        # is that of the tied head on the normalised embedding alone, within a nat of ln V.
+        r = orc.SplitMix64(3)
+        ids = np.array([r.below(spec.vocab) for _ in range(2 * 64)], np.uint32)
+        loss, grads = tr.loss_and_grads(ids, np.roll(ids, -1))
+        assert abs(loss - np.log(spec.vocab)) < 1.0
+        assert grads["blocks.1.mixer.o_proj.weight"].any() and not grads["blocks.1.mixer.q_proj.weight"].any()
+        tr.close()
