@@ -79,6 +79,10 @@ int32_t omx_free(omx_ctx* ctx, void* ptr);
 uint64_t omx_budget_live(omx_ctx* ctx);
 uint64_t omx_budget_peak(omx_ctx* ctx);
 uint64_t omx_budget_limit(omx_ctx* ctx);
+/* Bytes of freed blocks the context keeps parked for reuse (at most 4 GiB, blocks of at most
+ * 256 MiB; returned to the driver when an allocation fails and at close). The limit and `live`
+ * count what callers hold; parked blocks are on top of that. */
+uint64_t omx_budget_pooled(omx_ctx* ctx);
 void omx_budget_reset_peak(omx_ctx* ctx);
 
 int32_t omx_upload(omx_ctx* ctx, void* dst, uint64_t dst_offset, const void* host_src,
@@ -305,7 +309,9 @@ int32_t omx_cross_entropy_mean_forward(omx_ctx* ctx, const void* logits, int32_t
  * tight serving loops, harnesses that forbid hipMalloc). No counterpart in the reference. Same
  * arguments and result; the row state and the valid counter live in a file-scope device array
  * (786,688 bytes per device, held until the process ends) instead of the context's workspace,
- * so the call makes no hipMalloc / hipFree and grows nothing. At most 65536 rows: more is
+ * so the call makes no hipMalloc / hipFree and grows nothing; the array's device address is looked
+ * up by omx_open, so the call itself is kernel launches on the context's stream and nothing else.
+ * At most 65536 rows: more is
  * OMX_CAPACITY_EXCEEDED and nothing runs. Every call on a device shares that array: calls that
  * overlap on one device (two contexts, two streams) race; calls on one context are stream-ordered
  * and safe. */

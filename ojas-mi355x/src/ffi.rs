@@ -69,6 +69,7 @@ extern "C" {
     pub fn omx_budget_live(ctx: *mut OmxCtx) -> u64;
     pub fn omx_budget_peak(ctx: *mut OmxCtx) -> u64;
     pub fn omx_budget_limit(ctx: *mut OmxCtx) -> u64;
+    pub fn omx_budget_pooled(ctx: *mut OmxCtx) -> u64;
     pub fn omx_budget_reset_peak(ctx: *mut OmxCtx);
     pub fn omx_upload(ctx: *mut OmxCtx, dst: *mut c_void, dst_offset: u64, host_src: *const c_void, bytes: u64) -> i32;
     pub fn omx_download(ctx: *mut OmxCtx, host_dst: *mut c_void, src: *const c_void, src_offset: u64, bytes: u64) -> i32;

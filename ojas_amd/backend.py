@@ -76,7 +76,7 @@ def load_library() -> C.CDLL:
     lib = C.CDLL(str(LIB_PATH))
     lib.omx_last_error.restype = C.c_size_t
     lib.omx_device_name.restype = C.c_size_t
-    for name in ("omx_budget_live", "omx_budget_peak", "omx_budget_limit", "omx_muon_scratch_bytes"):
+    for name in ("omx_budget_live", "omx_budget_peak", "omx_budget_limit", "omx_budget_pooled", "omx_muon_scratch_bytes"):
         if hasattr(lib, name):
             getattr(lib, name).restype = C.c_uint64
     lib.omx_stream.restype = C.c_void_p
@@ -154,7 +154,8 @@ class MiBackend:
 
     def budget(self):
         return {"live": int(self._lib.omx_budget_live(self._ctx)), "peak": int(self._lib.omx_budget_peak(self._ctx)),
-                "limit": int(self._lib.omx_budget_limit(self._ctx))}
+                "limit": int(self._lib.omx_budget_limit(self._ctx)),
+                "pooled": int(self._lib.omx_budget_pooled(self._ctx))}
 
     def empty(self, shape, dtype: int = F32) -> DeviceTensor:
         shape = tuple(int(s) for s in (shape if isinstance(shape, (tuple, list)) else (shape,)))

@@ -114,6 +114,7 @@ int32_t omx_open(int32_t device, uint64_t budget_bytes, omx_ctx** out) {
     delete ctx;
     return OMX_BACKEND;
   }
+  ctx->ce_static_scratch = omx_ce_static_scratch_address();
   *out = ctx;
   return OMX_OK;
 }
@@ -224,6 +225,7 @@ int32_t omx_free(omx_ctx* ctx, void* ptr) {
 uint64_t omx_budget_live(omx_ctx* ctx) { return ctx ? ctx->budget_live : 0; }
 uint64_t omx_budget_peak(omx_ctx* ctx) { return ctx ? ctx->budget_peak : 0; }
 uint64_t omx_budget_limit(omx_ctx* ctx) { return ctx ? ctx->budget_limit : 0; }
+uint64_t omx_budget_pooled(omx_ctx* ctx) { return ctx ? ctx->pooled_bytes : 0; }
 void omx_budget_reset_peak(omx_ctx* ctx) {
   if (ctx) ctx->budget_peak = ctx->budget_live;
 }
@@ -293,8 +295,15 @@ int32_t omx_workspace(omx_ctx* ctx, uint64_t bytes, void** out, int slot) {
     return OMX_OK;
   }
   if (ctx->workspace[slot]) {
-    int32_t rc = omx_free(ctx, ctx->workspace[slot]);
-    if (rc != OMX_OK) return rc;
+    // An outgrown workspace goes back to the driver, not into the pool: its size (a multiple of
+    // 1 MiB that only this slot ever asked for) would match no later request and stay parked.
+    auto it = ctx->allocations.find(ctx->workspace[slot]);
+    if (it != ctx->allocations.end()) {
+      ctx->budget_live -= it->second;
+      ctx->allocations.erase(it);
+    }
+    OMX_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    OMX_HIP(ctx, hipFree(ctx->workspace[slot]));
     ctx->workspace[slot] = nullptr;
     ctx->workspace_bytes[slot] = 0;
   }

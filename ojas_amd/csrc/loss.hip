@@ -519,9 +519,15 @@ int32_t ce_forward_in(omx_ctx* ctx, const void* logits, int32_t logits_dtype, co
 // valid counter for up to CE_STATIC_MAX_ROWS rows, 786,688 bytes held by every device the library
 // runs on until the process ends. All calls on a device share it.
 constexpr uint64_t CE_STATIC_MAX_ROWS = 65536;
-constexpr int CE_STATIC_MAX_DEVICES = 64;
 static __device__ __align__(256) float g_ce_static_scratch[3 * CE_STATIC_MAX_ROWS + 64];
-static void* g_ce_static_ptr[CE_STATIC_MAX_DEVICES] = {};
+
+// The array's name is a host-side handle; each device holds its own copy at its own address.
+// omx_open calls this once per context with the context's device current and keeps the result.
+void* omx_ce_static_scratch_address() {
+  void* p = nullptr;
+  if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_ce_static_scratch)) != hipSuccess) return nullptr;
+  return p;
+}
 
 extern "C" {
 
@@ -550,19 +556,9 @@ int32_t omx_cross_entropy_mean_forward_static(omx_ctx* ctx, const void* logits, 
   if (rows > CE_STATIC_MAX_ROWS)
     return omx_fail(ctx, OMX_CAPACITY_EXCEEDED, "%s: %llu rows, the static scratch holds at most %llu", op,
                     (unsigned long long)rows, (unsigned long long)CE_STATIC_MAX_ROWS);
-  if (ctx->device < 0 || ctx->device >= CE_STATIC_MAX_DEVICES)
-    return omx_fail(ctx, OMX_UNSUPPORTED, "%s: device ordinal %d is outside 0..%d", op, ctx->device,
-                    CE_STATIC_MAX_DEVICES - 1);
-  // The array's name is a host-side handle; each device holds its own copy at its own address,
-  // looked up once per device with that device current.
-  void*& ws = g_ce_static_ptr[ctx->device];
-  if (!ws) {
-    OMX_HIP(ctx, hipSetDevice(ctx->device));
-    void* p = nullptr;
-    OMX_HIP(ctx, hipGetSymbolAddress(&p, HIP_SYMBOL(g_ce_static_scratch)));
-    if (!p) return omx_fail(ctx, OMX_BACKEND, "%s: the scratch symbol has no device address", op);
-    ws = p;
-  }
+  // Looked up when the context was opened: nothing here but launches on the context's stream.
+  void* ws = ctx->ce_static_scratch;
+  if (!ws) return omx_fail(ctx, OMX_BACKEND, "%s: the scratch symbol has no device address", op);
   return ce_forward_in(ctx, logits, logits_dtype, targets, rows, vocab, has_ignore, ignore_index, loss, ws);
 }
 

@@ -86,6 +86,9 @@ struct omx_ctx {
   void* workspace[3] = {nullptr, nullptr, nullptr};
   uint64_t workspace_bytes[3] = {0, 0, 0};
   int cu_count = 0;
+  // This device's copy of the static scratch of omx_cross_entropy_mean_forward_static, looked up
+  // when the context is opened (the lookup is not stream work and may load the code object).
+  void* ce_static_scratch = nullptr;
   // Optional per-launch timing of the GEMM kernel (benchmark only).
   // 0: 128x128 kernel only; 1: choose by shape; 2 / 3: force the 256x256 / 256x128 direct-to-LDS kernel where eligible.
   int gemm_dma_mode = 1;
@@ -123,6 +126,8 @@ inline void omx_launch_timed(omx_ctx* ctx, F kernel, dim3 grid, dim3 block, unsi
 
 int32_t omx_fail(omx_ctx* ctx, omx_status code, const char* fmt, ...);
 void omx_release_pool(omx_ctx* ctx);
+// The device address of the static cross-entropy scratch on the current device (loss.hip), or null.
+void* omx_ce_static_scratch_address();
 // Per-product timing for callers outside gemm.hip: takes a pair of events for the product about
 // to be launched (when omx_profile_gemm is on) and files them with its FLOP count afterwards.
 int32_t omx_timing_begin(omx_ctx* ctx, double flops, omx_ctx::TimedLaunch* timed);

@@ -692,8 +692,11 @@ __global__ __launch_bounds__(ST_THREADS) void sdpa_tiled_dkv_kernel(const float*
   if (bad) dev_raise_fault(fault, tag);
 }
 
-bool sdpa_tiled_supports(uint64_t dim, std::initializer_list<int32_t> dtypes, std::initializer_list<const void*> ptrs) {
+// The tiled kernels put the (batch, head) plane in grid.y, which holds at most 65535: more planes
+// than that (many short sequences) go to the row kernels, whose grids are one-dimensional.
+bool sdpa_tiled_supports(uint64_t dim, uint64_t planes, std::initializer_list<int32_t> dtypes, std::initializer_list<const void*> ptrs) {
   if (dim != 16 && dim != 32 && dim != 64 && dim != 128) return false;
+  if (planes > 65535) return false;
   for (int32_t d : dtypes)
     if (d != OMX_F32) return false;
   for (const void* p : ptrs)
@@ -742,7 +745,7 @@ int32_t omx_causal_sdpa_forward(omx_ctx* ctx, const void* q, const void* k, cons
   if (omx_flash_sdpa_supports(head_dim, operand_dtype))
     return omx_flash_sdpa_forward(ctx, q, k, v, out, out_dtype, nullptr, static_cast<float*>(lse), batch, heads,
                                   kv_heads, time, head_dim, s.window, s.scale, tag, nullptr);
-  if (ctx->sdpa_tiled && sdpa_tiled_supports(head_dim, {operand_dtype, out_dtype}, {q, k, v, out})) {
+  if (ctx->sdpa_tiled && sdpa_tiled_supports(head_dim, batch * heads, {operand_dtype, out_dtype}, {q, k, v, out})) {
     dim3 tgrid(static_cast<unsigned>((time + 63) / 64), static_cast<unsigned>(batch * heads));
 #define SDPA_TILED_FWD(D_)                                                                                      \
   hipLaunchKernelGGL((sdpa_tiled_fwd_kernel<D_>), tgrid, dim3(ST_THREADS), 0, ctx->stream,                      \
@@ -843,7 +846,7 @@ int32_t omx_causal_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, con
     if (rc != OMX_OK) return rc;
     gy = conv;
   }
-  if (ctx->sdpa_tiled && sdpa_tiled_supports(head_dim, {operand_dtype, grad_dtype}, {q, k, v, gy, gq, gk, gv})) {
+  if (ctx->sdpa_tiled && sdpa_tiled_supports(head_dim, batch * heads, {operand_dtype, grad_dtype}, {q, k, v, gy, gq, gk, gv})) {
     dim3 qgrid(static_cast<unsigned>((time + 63) / 64), static_cast<unsigned>(batch * heads));
     dim3 kgrid(static_cast<unsigned>((time + 63) / 64), static_cast<unsigned>(batch * kv_heads));
 #define SDPA_TILED_BWD(D_)                                                                                          \

@@ -415,6 +415,24 @@ def test_causal_sdpa_f32_tiled_kernels_agree_with_the_row_kernels(be, shape, hkv
             close(a, c, F32_TOL, "tiled against the oracle: " + name)
 
 
+def test_causal_sdpa_f32_with_more_planes_than_a_grid_axis_holds(be):
+    """65536 (batch, head) planes of a short sequence: above the 65535 a grid's second axis takes,
+    so the call goes to the row kernels (decided on the host) instead of failing at launch."""
+    b, h, hkv, t, d = 8192, 8, 8, 8, 16
+    print(f"sdpa f32 many planes {[b, h, t, d]}", flush=True)
+    r = orc.SplitMix64(77)
+    q, k, v, gy = (r.vec(b * h * t * d, 0.5).reshape(b, h, t, d) for _ in range(4))
+    orc.set_threads(8)
+    oy, olse = orc.causal_sdpa_forward(q, k, v, 0)
+    ogq, ogk, ogv = orc.causal_sdpa_backward(q, k, v, oy, olse, gy, 0)
+    dq, dk, dv, dgy = be.upload(q), be.upload(k), be.upload(v), be.upload(gy)
+    y, lse = be.causal_sdpa_forward(dq, dk, dv, None)
+    gq, gk, gv = be.causal_sdpa_backward(dq, dk, dv, y, lse, dgy, None)
+    be.sync()
+    for name, a, c in zip(("out", "lse", "gq", "gk", "gv"), (y, lse, gq, gk, gv), (oy, olse, ogq, ogk, ogv)):
+        close(be.download(a), c, F32_TOL, "many planes: " + name)
+
+
 def test_adamw_matches_fast_f32_contract_bitwise_and_exact_within_1e6(be):
     from ojas_amd.backend import AdamWConfig
 

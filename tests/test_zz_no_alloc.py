@@ -16,6 +16,16 @@ pytestmark = pytest.mark.gpu
 F32_TOL = 1e-5
 
 
+def device_free_bytes() -> int:
+    """hipMemGetInfo's free bytes on the current device, read from the HIP runtime directly."""
+    import ctypes as C
+
+    hip = C.CDLL("libamdhip64.so")
+    free, total = C.c_size_t(), C.c_size_t()
+    assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+    return int(free.value)
+
+
 def test_cross_entropy_forward_static_matches_workspace_form():
     from ojas_amd.backend import BF16, CAPACITY_EXCEEDED, F32, MiBackend, OjasError
 
@@ -31,10 +41,19 @@ def test_cross_entropy_forward_static_matches_workspace_form():
                 logits = orc.round_bf16(logits)
             targets = np.array([(ignore or 0) if i % 9 == 2 else r.below(vocab) for i in range(rows)], np.uint32)
             dl, dt = be.upload(logits, dtype), be.upload(targets)
-            live = be.budget()["live"]
-            got = be.download(be.cross_entropy_mean_forward_static(dl, dt, loss_static, ignore))[0]
-            assert be.budget()["live"] == live, "the static form must not take memory from the budget"
+            # The workspace form first: it loads the kernels and grows the workspace, so that whatever
+            # moves during the static call below is the static call's own doing.
             ref = be.download(be.cross_entropy_mean_forward(dl, dt, ignore))[0]
+            budget = be.budget()
+            be.sync()
+            free_before = device_free_bytes()
+            result = be.cross_entropy_mean_forward_static(dl, dt, loss_static, ignore)
+            be.sync()
+            # Neither the context's ledger (held and parked bytes) nor the device's own count of
+            # free memory moves: the call reached no allocator.
+            assert device_free_bytes() == free_before, "the static form must not allocate device memory"
+            assert be.budget() == budget, "the static form must not take memory from the budget or the pool"
+            got = be.download(result)[0]
             assert got.tobytes() == ref.tobytes(), (call, got, ref)
             want = float(orc.cross_entropy_mean_forward(logits, targets, ignore))
             tol = F32_TOL if dtype == F32 else 1e-3
