@@ -155,8 +155,10 @@ int32_t omx_gemm_pitched_strided_batch(omx_ctx* ctx, const void* a, uint64_t a_r
  * dequantise -> linear_forward (ojas-autograd/src/tape.rs:1514-1518, backend.rs:2586); these two
  * entry points serve that pair of calls for a frozen base, forward and input gradient (a frozen
  * weight has no gradient, ojas-model/src/lora.rs:4-8).
- * x, y, gy, gx, add: bf16. `add` (optional, the output's shape) is added to the product before the
- * rounding: the place of the adapter's term in lora_linear (lora.rs:332-344).
+ * x, gy, gx, add: bf16; the forward's y is bf16 or f32 (`y_dtype`: f32 keeps the product unrounded
+ * for a pointwise op that follows, so the activation is rounded once, as the next product's
+ * operand). `add` (optional, the output's shape) is added to the product before the rounding: the
+ * place of the adapter's term in lora_linear (lora.rs:332-344).
  * forward needs k_in % 32 == 0 and n_out % 4 == 0; the input gradient k_in % 32 == 0 and n_out % 32 == 0.
  * `layout`: OMX_I8_ROW_MAJOR (codes [n_out, k_in], scales [n_out, k_in / 32]) or OMX_I8_BLOCKED, the
  * form omx_pack_i8_group writes (same bytes, reordered so that both products read whole cache
@@ -179,7 +181,7 @@ typedef struct {
 int32_t omx_linear_i8_group_forward(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* codes_i8,
                                     const void* scales_f32, uint64_t group, int32_t layout,
                                     const void* add, const omx_low_rank* low_rank, void* y,
-                                    uint64_t rows, uint64_t k_in, uint64_t n_out);
+                                    int32_t y_dtype, uint64_t rows, uint64_t k_in, uint64_t n_out);
 int32_t omx_linear_i8_group_backward_input(omx_ctx* ctx, const void* codes_i8, const void* scales_f32,
                                            uint64_t group, int32_t layout, const void* gy,
                                            int32_t gy_dtype, const void* add,
@@ -494,10 +496,20 @@ int32_t omx_rope_half_split_backward(omx_ctx* ctx, const void* gy, const void* c
 int32_t omx_rope_half_split_inplace(omx_ctx* ctx, void* x, int32_t dtype, uint64_t pitch,
                                     const void* cos_f32, const void* sin_f32, uint64_t tokens,
                                     uint64_t time, uint64_t heads, uint64_t dim, int32_t backward);
+/* The forward of the same out of place, from a projection output kept in f32 (or bf16) to the
+ * bf16 tensor attention reads: the first `heads` heads of every token row are rotated, the
+ * `plain_heads` that follow (the value heads) are converted as they are; both tensors share the
+ * pitch. One rounding per value where the in-place form on a bf16 output makes two. */
+int32_t omx_rope_half_split_pitched(omx_ctx* ctx, const void* x, int32_t x_dtype, void* out_bf16,
+                                    uint64_t pitch, const void* cos_f32, const void* sin_f32,
+                                    uint64_t tokens, uint64_t time, uint64_t heads,
+                                    uint64_t plain_heads, uint64_t dim);
 /* silu_forward then mul_forward (backend.rs:1151-1163; ojas-model/src/block.rs:248-262) on a fused
- * gate | up projection output: gate_up is bf16 [rows, 2 hidden] with the gate columns first,
- * out[r, c] = silu(gate[r, c]) * up[r, c]. The backward writes the gradient of gate_up in the
- * same layout from gy [rows, hidden] (mul_backward then silu_backward). bf16, hidden % 8 == 0. */
+ * gate | up projection output: gate_up is [rows, 2 hidden] with the gate columns first, of
+ * `dtype` (bf16, or f32: the product's output kept unrounded, so that the activation is rounded
+ * once, as the next product's operand); out[r, c] = silu(gate[r, c]) * up[r, c], bf16. The backward
+ * writes the gradient of gate_up (bf16, same layout) from gy [rows, hidden] bf16 (mul_backward
+ * then silu_backward). hidden % 8 == 0. */
 int32_t omx_swiglu_forward(omx_ctx* ctx, const void* gate_up, void* out, int32_t dtype, uint64_t rows,
                            uint64_t hidden);
 int32_t omx_swiglu_backward(omx_ctx* ctx, const void* gate_up, const void* gy, void* g_gate_up,
@@ -577,22 +589,23 @@ int32_t omx_value_residual_blend_backward(omx_ctx* ctx, const void* value, const
 
 /* rms_qk_norm_forward, rope_half_split_forward and value_residual_blend_forward (backend.rs:1674-1699,
  * 1907-1920; the sequence of ojas-model/src/block.rs:225-240) in one pass over a fused q | k | v
- * projection output: bf16 [tokens, pitch] whose token rows hold the query heads, then the key heads,
- * then the value heads. q and k heads are normed (weights f32 [head_dim]) and rotated (cos / sin f32
+ * projection output: [tokens, pitch] of `lin_dtype` (bf16, or f32: the product's output kept
+ * unrounded, so q, k and v reach attention with one rounding) whose token rows hold the query heads,
+ * then the key heads, then the value heads; the prepared tensor and both gradients are bf16. q and k heads are normed (weights f32 [head_dim]) and rotated (cos / sin f32
  * [time, head_dim], row r uses table row r % time); the normed row is not rounded to bf16 in
  * between, where the separate calls round. The value heads are blended with those of `value0`
- * (block 0's projection output: same layout and pitch; lambda f32 [1]), or copied when value0 is
+ * (block 0's projection output: same layout, pitch and dtype; lambda f32 [1]), or copied when value0 is
  * NULL. head_dim 64 or 128. The backward takes the gradient of the prepared tensor in the same
  * layout and writes that of the projection output; what the blend sends to block 0's value is
  * written to (value0_grad_first != 0) or added to value0_grad_f32 [tokens, kv_heads * head_dim];
  * add_value_grad_f32 (same shape; the block without a blend) is added to the value's gradient.
  * No counterpart in the trait: a fusion of three of its calls. */
-int32_t omx_qkv_prepare_forward(omx_ctx* ctx, const void* qkv_lin, void* qkv_out, uint64_t pitch,
+int32_t omx_qkv_prepare_forward(omx_ctx* ctx, const void* qkv_lin, int32_t lin_dtype, void* qkv_out, uint64_t pitch,
                                 const void* q_weight_f32, const void* k_weight_f32, const void* cos_f32,
                                 const void* sin_f32, const void* value0, const void* lambda_f32,
                                 uint64_t tokens, uint64_t time, uint64_t heads, uint64_t kv_heads,
                                 uint64_t head_dim, float eps);
-int32_t omx_qkv_prepare_backward(omx_ctx* ctx, const void* qkv_lin, const void* g_qkv, void* g_qkv_lin,
+int32_t omx_qkv_prepare_backward(omx_ctx* ctx, const void* qkv_lin, int32_t lin_dtype, const void* g_qkv, void* g_qkv_lin,
                                  uint64_t pitch, const void* q_weight_f32, const void* k_weight_f32,
                                  const void* cos_f32, const void* sin_f32, const void* value0,
                                  const void* lambda_f32, void* value0_grad_f32, int32_t value0_grad_first,

@@ -86,7 +86,7 @@ extern "C" {
     pub fn omx_gemm_pitched(ctx: *mut OmxCtx, a: *const c_void, a_rs: u64, a_cs: u64, b: *const c_void, b_rs: u64, b_cs: u64, operand_dtype: i32, c: *mut c_void, c_dtype: i32, ldc: u64, m: u64, k: u64, n: u64, accumulate: i32) -> i32;
     pub fn omx_gemm_strided_batch(ctx: *mut OmxCtx, a: *const c_void, a_rs: u64, a_cs: u64, b: *const c_void, b_rs: u64, b_cs: u64, operand_dtype: i32, c: *mut c_void, c_dtype: i32, m: u64, k: u64, n: u64, accumulate: i32, count: u64, stride_a: u64, stride_b: u64, stride_c: u64) -> i32;
     pub fn omx_gemm_pitched_strided_batch(ctx: *mut OmxCtx, a: *const c_void, a_rs: u64, a_cs: u64, b: *const c_void, b_rs: u64, b_cs: u64, operand_dtype: i32, c: *mut c_void, c_dtype: i32, ldc: u64, m: u64, k: u64, n: u64, accumulate: i32, count: u64, stride_a: u64, stride_b: u64, stride_c: u64) -> i32;
-    pub fn omx_linear_i8_group_forward(ctx: *mut OmxCtx, x: *const c_void, x_dtype: i32, codes_i8: *const c_void, scales_f32: *const c_void, group: u64, layout: i32, add: *const c_void, low_rank: *const OmxLowRank, y: *mut c_void, rows: u64, k_in: u64, n_out: u64) -> i32;
+    pub fn omx_linear_i8_group_forward(ctx: *mut OmxCtx, x: *const c_void, x_dtype: i32, codes_i8: *const c_void, scales_f32: *const c_void, group: u64, layout: i32, add: *const c_void, low_rank: *const OmxLowRank, y: *mut c_void, y_dtype: i32, rows: u64, k_in: u64, n_out: u64) -> i32;
     pub fn omx_linear_i8_group_backward_input(ctx: *mut OmxCtx, codes_i8: *const c_void, scales_f32: *const c_void, group: u64, layout: i32, gy: *const c_void, gy_dtype: i32, add: *const c_void, low_rank: *const OmxLowRank, gx: *mut c_void, rows: u64, k_in: u64, n_out: u64) -> i32;
     pub fn omx_pack_i8_group(ctx: *mut OmxCtx, codes_i8: *const c_void, scales_f32: *const c_void, blocked_codes: *mut c_void, blocked_scales: *mut c_void, n_out: u64, k_in: u64, group: u64, unpack: i32) -> i32;
     pub fn omx_causal_sdpa_forward(ctx: *mut OmxCtx, q: *const c_void, k: *const c_void, v: *const c_void, operand_dtype: i32, out: *mut c_void, out_dtype: i32, lse: *mut c_void, batch: u64, heads: u64, kv_heads: u64, time: u64, head_dim: u64, window: u64) -> i32;
@@ -131,6 +131,7 @@ extern "C" {
     pub fn omx_rope_half_split_forward(ctx: *mut OmxCtx, x: *const c_void, cos_f32: *const c_void, sin_f32: *const c_void, y: *mut c_void, dtype: i32, rows: u64, dim: u64, time: u64, heads: u64) -> i32;
     pub fn omx_rope_half_split_backward(ctx: *mut OmxCtx, gy: *const c_void, cos_f32: *const c_void, sin_f32: *const c_void, gx: *mut c_void, dtype: i32, rows: u64, dim: u64, time: u64, heads: u64) -> i32;
     pub fn omx_rope_half_split_inplace(ctx: *mut OmxCtx, x: *mut c_void, dtype: i32, pitch: u64, cos_f32: *const c_void, sin_f32: *const c_void, tokens: u64, time: u64, heads: u64, dim: u64, backward: i32) -> i32;
+    pub fn omx_rope_half_split_pitched(ctx: *mut OmxCtx, x: *const c_void, x_dtype: i32, out_bf16: *mut c_void, pitch: u64, cos_f32: *const c_void, sin_f32: *const c_void, tokens: u64, time: u64, heads: u64, plain_heads: u64, dim: u64) -> i32;
     pub fn omx_swiglu_forward(ctx: *mut OmxCtx, gate_up: *const c_void, out: *mut c_void, dtype: i32, rows: u64, hidden: u64) -> i32;
     pub fn omx_swiglu_backward(ctx: *mut OmxCtx, gate_up: *const c_void, gy: *const c_void, g_gate_up: *mut c_void, dtype: i32, rows: u64, hidden: u64) -> i32;
     pub fn omx_init_normal(ctx: *mut OmxCtx, dst: *mut c_void, dtype: i32, n: u64, seed: u64, std: f32) -> i32;
@@ -143,8 +144,8 @@ extern "C" {
     pub fn omx_per_head_sigmoid_gate_input_grad_add(ctx: *mut OmxCtx, gz: *const c_void, weight: *const c_void, operand_dtype: i32, add_in: *const c_void, add_dtype: i32, out_f32: *mut c_void, rows: u64, d_model: u64, heads: u64) -> i32;
     pub fn omx_value_residual_blend_forward(ctx: *mut OmxCtx, value: *const c_void, value0: *const c_void, lambda_f32: *const c_void, out: *mut c_void, dtype: i32, n: u64) -> i32;
     pub fn omx_value_residual_blend_backward(ctx: *mut OmxCtx, value: *const c_void, value0: *const c_void, lambda_f32: *const c_void, gy: *const c_void, g_value: *mut c_void, g_value0: *mut c_void, dtype: i32, g_lambda_f32: *mut c_void, n: u64) -> i32;
-    pub fn omx_qkv_prepare_forward(ctx: *mut OmxCtx, qkv_lin: *const c_void, qkv_out: *mut c_void, pitch: u64, q_weight_f32: *const c_void, k_weight_f32: *const c_void, cos_f32: *const c_void, sin_f32: *const c_void, value0: *const c_void, lambda_f32: *const c_void, tokens: u64, time: u64, heads: u64, kv_heads: u64, head_dim: u64, eps: f32) -> i32;
-    pub fn omx_qkv_prepare_backward(ctx: *mut OmxCtx, qkv_lin: *const c_void, g_qkv: *const c_void, g_qkv_lin: *mut c_void, pitch: u64, q_weight_f32: *const c_void, k_weight_f32: *const c_void, cos_f32: *const c_void, sin_f32: *const c_void, value0: *const c_void, lambda_f32: *const c_void, value0_grad_f32: *mut c_void, value0_grad_first: i32, add_value_grad_f32: *const c_void, g_q_weight_f32: *mut c_void, g_k_weight_f32: *mut c_void, g_lambda_f32: *mut c_void, tokens: u64, time: u64, heads: u64, kv_heads: u64, head_dim: u64, eps: f32) -> i32;
+    pub fn omx_qkv_prepare_forward(ctx: *mut OmxCtx, qkv_lin: *const c_void, lin_dtype: i32, qkv_out: *mut c_void, pitch: u64, q_weight_f32: *const c_void, k_weight_f32: *const c_void, cos_f32: *const c_void, sin_f32: *const c_void, value0: *const c_void, lambda_f32: *const c_void, tokens: u64, time: u64, heads: u64, kv_heads: u64, head_dim: u64, eps: f32) -> i32;
+    pub fn omx_qkv_prepare_backward(ctx: *mut OmxCtx, qkv_lin: *const c_void, lin_dtype: i32, g_qkv: *const c_void, g_qkv_lin: *mut c_void, pitch: u64, q_weight_f32: *const c_void, k_weight_f32: *const c_void, cos_f32: *const c_void, sin_f32: *const c_void, value0: *const c_void, lambda_f32: *const c_void, value0_grad_f32: *mut c_void, value0_grad_first: i32, add_value_grad_f32: *const c_void, g_q_weight_f32: *mut c_void, g_k_weight_f32: *mut c_void, g_lambda_f32: *mut c_void, tokens: u64, time: u64, heads: u64, kv_heads: u64, head_dim: u64, eps: f32) -> i32;
     pub fn omx_argmax_rows(ctx: *mut OmxCtx, x_f32: *const c_void, rows: u64, cols: u64, out_u32: *mut c_void) -> i32;
     pub fn omx_topk_rows(ctx: *mut OmxCtx, x_f32: *const c_void, rows: u64, cols: u64, k: u64, values_f32: *mut c_void, ids_u32: *mut c_void) -> i32;
     pub fn omx_read_scalar_f32(ctx: *mut OmxCtx, src: *const c_void, out: *mut f32) -> i32;

@@ -275,16 +275,25 @@ class MiBackend:
             C.c_uint64(tokens), C.c_uint64(time), C.c_uint64(heads), C.c_uint64(dim), C.c_int32(1 if backward else 0)))
         return x
 
+    def rope_half_split_pitched(self, x, cos, sin, tokens, time, heads, plain_heads, dim):
+        """The rotation out of place: x [tokens, pitch] f32 or bf16 -> bf16, `heads` rotated heads then
+        `plain_heads` converted as they are (`omx_rope_half_split_pitched`)."""
+        out = self.empty(x.shape, BF16)
+        self._check(self._lib.omx_rope_half_split_pitched(
+            self._ctx, self._p(x), C.c_int32(x.dtype), self._p(out), C.c_uint64(x.shape[-1]), self._p(cos), self._p(sin),
+            C.c_uint64(tokens), C.c_uint64(time), C.c_uint64(heads), C.c_uint64(plain_heads), C.c_uint64(dim)))
+        return out
+
     def swiglu_forward(self, gate_up):
         rows, two_h = gate_up.shape
-        out = self.empty((rows, two_h // 2), gate_up.dtype)
+        out = self.empty((rows, two_h // 2), BF16)
         self._check(self._lib.omx_swiglu_forward(self._ctx, self._p(gate_up), self._p(out), C.c_int32(gate_up.dtype),
                                                  C.c_uint64(rows), C.c_uint64(two_h // 2)))
         return out
 
     def swiglu_backward(self, gate_up, gy):
         rows, two_h = gate_up.shape
-        g = self.empty(gate_up.shape, gate_up.dtype)
+        g = self.empty(gate_up.shape, BF16)
         self._check(self._lib.omx_swiglu_backward(self._ctx, self._p(gate_up), self._p(gy), self._p(g),
                                                   C.c_int32(gate_up.dtype), C.c_uint64(rows), C.c_uint64(two_h // 2)))
         return g
@@ -313,16 +322,18 @@ class MiBackend:
         h, w, block_cols = low_rank
         return C.byref(LowRank(h.ptr, w.ptr, h.shape[-1], w.shape[-1], w.shape[-1], block_cols))
 
-    def linear_i8_group_forward(self, x, codes, scales, add=None, group=32, blocked=False, low_rank=None):
+    def linear_i8_group_forward(self, x, codes, scales, add=None, group=32, blocked=False, low_rank=None,
+                                out_dtype=BF16):
         """y = x W^T (+ add) for a frozen weight held as int8 codes [out, in] and f32 group scales
-        [out, in / group] (value = code * scale); bf16 in, bf16 out."""
+        [out, in / group] (value = code * scale); bf16 in, bf16 (or f32) out."""
         rows, kin, nout = x.numel // x.shape[-1], x.shape[-1], codes.shape[0]
         if codes.shape != (nout, kin) or scales.shape != (nout, kin // group) or codes.dtype != I8 or scales.dtype != F32:
             raise OjasError(SHAPE, f"linear_i8_group_forward: input {x.shape} codes {codes.shape} scales {scales.shape}")
-        y = self.empty(x.shape[:-1] + (nout,), BF16)
+        y = self.empty(x.shape[:-1] + (nout,), out_dtype)
         self._check(self._lib.omx_linear_i8_group_forward(
             self._ctx, self._p(x), C.c_int32(x.dtype), self._p(codes), self._p(scales), C.c_uint64(group),
-            C.c_int32(1 if blocked else 0), self._p(add), self._low_rank(low_rank), self._p(y), C.c_uint64(rows), C.c_uint64(kin), C.c_uint64(nout)))
+            C.c_int32(1 if blocked else 0), self._p(add), self._low_rank(low_rank), self._p(y), C.c_int32(out_dtype),
+            C.c_uint64(rows), C.c_uint64(kin), C.c_uint64(nout)))
         return y
 
     def linear_i8_group_backward_input(self, codes, scales, gy, add=None, group=32, blocked=False, low_rank=None):
@@ -884,11 +895,13 @@ class MiBackend:
     def qkv_prepare_forward(self, qkv_lin, q_weight, k_weight, cos, sin, heads, kv_heads, head_dim, value0=None, lam=None,
                             eps: float = 1e-6):
         """QK-norm, RoPE and the value blend over a fused q | k | v projection output (`omx_qkv_prepare_forward`):
-        bf16 [batch, time, (heads + 2 kv_heads) head_dim]."""
+        [batch, time, (heads + 2 kv_heads) head_dim], bf16 or f32; the result is bf16."""
         b, t, pitch = qkv_lin.shape
+        if value0 is not None and value0.dtype != qkv_lin.dtype:
+            raise OjasError(DTYPE, "qkv_prepare_forward: value0 has the projection output's dtype")
         out = self.empty(qkv_lin.shape, BF16)
         self._check(self._lib.omx_qkv_prepare_forward(
-            self._ctx, self._p(qkv_lin), self._p(out), C.c_uint64(pitch), self._p(q_weight), self._p(k_weight),
+            self._ctx, self._p(qkv_lin), C.c_int32(qkv_lin.dtype), self._p(out), C.c_uint64(pitch), self._p(q_weight), self._p(k_weight),
             self._p(cos), self._p(sin), self._p(value0), self._p(lam), C.c_uint64(b * t), C.c_uint64(t), C.c_uint64(heads),
             C.c_uint64(kv_heads), C.c_uint64(head_dim), C.c_float(eps)))
         return out
@@ -898,11 +911,13 @@ class MiBackend:
         """Returns (g_qkv_lin, g_q_weight, g_k_weight, g_lambda or None); `value0_grad` (f32
         [batch, time, kv_heads head_dim]) is written or added to in place."""
         b, t, pitch = qkv_lin.shape
+        if value0 is not None and value0.dtype != qkv_lin.dtype:
+            raise OjasError(DTYPE, "qkv_prepare_backward: value0 has the projection output's dtype")
         g_lin = self.empty(qkv_lin.shape, BF16)
         gqw, gkw = self.empty((head_dim,), F32), self.empty((head_dim,), F32)
         g_lam = self.empty((1,), F32) if value0 is not None else None
         self._check(self._lib.omx_qkv_prepare_backward(
-            self._ctx, self._p(qkv_lin), self._p(g_qkv), self._p(g_lin), C.c_uint64(pitch), self._p(q_weight),
+            self._ctx, self._p(qkv_lin), C.c_int32(qkv_lin.dtype), self._p(g_qkv), self._p(g_lin), C.c_uint64(pitch), self._p(q_weight),
             self._p(k_weight), self._p(cos), self._p(sin), self._p(value0), self._p(lam), self._p(value0_grad),
             C.c_int32(1 if value0_grad_first else 0), self._p(add_value_grad), self._p(gqw), self._p(gkw), self._p(g_lam),
             C.c_uint64(b * t), C.c_uint64(t), C.c_uint64(heads), C.c_uint64(kv_heads), C.c_uint64(head_dim), C.c_float(eps)))

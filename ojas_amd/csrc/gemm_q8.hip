@@ -32,8 +32,9 @@ struct Q8Args {
   const signed char* codes;  // [nout][kin]
   const float* scales;       // [nout][kin / 32]
   long kin;
-  unsigned short* c;  // [M][N] bf16
+  unsigned short* c;  // [M][N] bf16, or f32 when c_f32 (the pointer is then a float*)
   long ldc;
+  int c_f32;
   const unsigned short* add;  // optional [M][N] bf16 with C's pitch, added before the rounding
   int M, N, K;
   int tiles_m, tiles_n;
@@ -351,8 +352,9 @@ __global__ __launch_bounds__(512, 4) void gemm_q8_kernel(Q8Args g) {
           val.w += __uint_as_float(addv[it].y & 0xffff0000u);
         }
         bad |= !(dev_finite(val.x) && dev_finite(val.y) && dev_finite(val.z) && dev_finite(val.w));
-        *reinterpret_cast<uint2*>(g.c + static_cast<long>(grow0 + row) * g.ldc + gcol0 + piece * 4) =
-            make_uint2(q8_pack2(val.x, val.y), q8_pack2(val.z, val.w));
+        const long at = static_cast<long>(grow0 + row) * g.ldc + gcol0 + piece * 4;
+        if (g.c_f32) *reinterpret_cast<float4*>(reinterpret_cast<float*>(g.c) + at) = val;
+        else *reinterpret_cast<uint2*>(g.c + at) = make_uint2(q8_pack2(val.x, val.y), q8_pack2(val.z, val.w));
       }
     } else {
 #pragma unroll 1
@@ -365,7 +367,8 @@ __global__ __launch_bounds__(512, 4) void gemm_q8_kernel(Q8Args g) {
           float v = cs[row * CPW + piece * 4 + e];
           if (g.add) v += dev_bf16_bits_to_f32(g.add[off]);
           bad |= !dev_finite(v);
-          g.c[off] = dev_f32_to_bf16_bits(v);
+          if (g.c_f32) reinterpret_cast<float*>(g.c)[off] = v;
+          else g.c[off] = dev_f32_to_bf16_bits(v);
         }
       }
     }
@@ -464,12 +467,13 @@ extern "C" {
 
 int32_t omx_linear_i8_group_forward(omx_ctx* ctx, const void* x, int32_t x_dtype, const void* codes_i8,
                                     const void* scales_f32, uint64_t group, int32_t layout, const void* add,
-                                    const omx_low_rank* low_rank, void* y, uint64_t rows, uint64_t kin,
-                                    uint64_t nout) {
+                                    const omx_low_rank* low_rank, void* y, int32_t y_dtype, uint64_t rows,
+                                    uint64_t kin, uint64_t nout) {
   OMX_REQUIRE_CTX(ctx);
   const char* op = "linear_i8_group_forward";
   int32_t rc = check_q8(ctx, op, x, codes_i8, scales_f32, y, add, rows, kin, nout, group, x_dtype, layout);
   if (rc != OMX_OK) return rc;
+  if (!omx_valid_float_dtype(y_dtype)) return omx_fail(ctx, OMX_DTYPE, "%s: the output must be f32 or bf16", op);
   if (nout % 4 != 0) return omx_fail(ctx, OMX_SHAPE, "%s: n_out %llu is not a multiple of 4", op, (unsigned long long)nout);
   Q8Args g{};
   g.a = static_cast<const unsigned short*>(x);
@@ -478,6 +482,7 @@ int32_t omx_linear_i8_group_forward(omx_ctx* ctx, const void* x, int32_t x_dtype
   g.scales = static_cast<const float*>(scales_f32);
   g.kin = static_cast<long>(kin);
   g.c = static_cast<unsigned short*>(y);
+  g.c_f32 = y_dtype == OMX_F32;
   g.ldc = static_cast<long>(nout);
   g.add = static_cast<const unsigned short*>(add);
   g.M = static_cast<int>(rows);

@@ -65,16 +65,67 @@ __global__ void rope_pitched_kernel(unsigned short* __restrict__ x, long pitch, 
 
 __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + __expf(-x)); }
 
-// gate_up: [rows][2 * hidden] (gate columns first). out[r][c] = silu(gate[r][c]) * up[r][c].
-__global__ void swiglu_fwd_kernel(const unsigned short* __restrict__ gate_up, unsigned short* __restrict__ out,
+// Eight consecutive values of a bf16 or an f32 tensor as floats (16-byte accesses).
+__device__ __forceinline__ void load8(const unsigned short* p, float (&v)[8]) { unpack8(*reinterpret_cast<const uint4*>(p), v); }
+__device__ __forceinline__ void load8(const float* p, float (&v)[8]) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
+}
+
+// The forward rotation out of place, x (bf16 or f32) -> bf16 out at the same pitch: a thread takes
+// elements [c, c + 8) and [c + dim/2, c + dim/2 + 8) of one head, rotates them when the head is one
+// of the first `heads` and converts them as they are for the `plain` heads behind those.
+template <typename TIN>
+__global__ void rope_pitched_out_kernel(const TIN* __restrict__ x, unsigned short* __restrict__ out, long pitch,
+                                        const float* __restrict__ cos_t, const float* __restrict__ sin_t, long tokens,
+                                        int time, int heads, int plain, int dim, OmxFaultWord* fault,
+                                        unsigned long long tag) {
+  const int half = dim / 2, per_head = half / 8, all = heads + plain;
+  const long total = tokens * all * per_head;
+  const long i = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int piece = static_cast<int>(i % per_head);
+  const int head = static_cast<int>((i / per_head) % all);
+  const long token = i / (static_cast<long>(per_head) * all);
+  const long at = token * pitch + static_cast<long>(head) * dim + piece * 8;
+  float lo[8], hi[8], ylo[8], yhi[8];
+  load8(x + at, lo);
+  load8(x + at + half, hi);
+  bool bad = false;
+  if (head < heads) {
+    const int t = static_cast<int>(token % time);
+    float c[8], s[8];
+    load8(cos_t + static_cast<long>(t) * dim + piece * 8, c);
+    load8(sin_t + static_cast<long>(t) * dim + piece * 8, s);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      ylo[e] = lo[e] * c[e] - hi[e] * s[e];
+      yhi[e] = hi[e] * c[e] + lo[e] * s[e];
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ylo[e] = lo[e], yhi[e] = hi[e];
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) bad |= !(dev_finite(ylo[e]) && dev_finite(yhi[e]));
+  *reinterpret_cast<uint4*>(out + at) = pack8(ylo);
+  *reinterpret_cast<uint4*>(out + at + half) = pack8(yhi);
+  if (bad) dev_raise_fault(fault, tag);
+}
+
+// gate_up: [rows][2 * hidden] (gate columns first), bf16 or f32 (the projection's output as its
+// product left it, so the activation is rounded once, when it is stored as the next product's
+// operand). out[r][c] = silu(gate[r][c]) * up[r][c], bf16.
+template <typename GU>
+__global__ void swiglu_fwd_kernel(const GU* __restrict__ gate_up, unsigned short* __restrict__ out,
                                   long rows, long hidden, OmxFaultWord* fault, unsigned long long tag) {
   const long per_row = hidden / 8, total = rows * per_row;
   const long i = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (i >= total) return;
   const long r = i / per_row, c = (i % per_row) * 8;
   float g[8], u[8], y[8];
-  unpack8(*reinterpret_cast<const uint4*>(gate_up + r * 2 * hidden + c), g);
-  unpack8(*reinterpret_cast<const uint4*>(gate_up + r * 2 * hidden + hidden + c), u);
+  load8(gate_up + r * 2 * hidden + c, g);
+  load8(gate_up + r * 2 * hidden + hidden + c, u);
   bool bad = false;
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
@@ -86,7 +137,8 @@ __global__ void swiglu_fwd_kernel(const unsigned short* __restrict__ gate_up, un
 }
 
 // g_gate = gm * up * silu'(gate), g_up = gm * silu(gate); silu'(x) = s (1 + x (1 - s)), s = sigmoid(x).
-__global__ void swiglu_bwd_kernel(const unsigned short* __restrict__ gate_up, const unsigned short* __restrict__ gm,
+template <typename GU>
+__global__ void swiglu_bwd_kernel(const GU* __restrict__ gate_up, const unsigned short* __restrict__ gm,
                                   unsigned short* __restrict__ g_gate_up, long rows, long hidden, OmxFaultWord* fault,
                                   unsigned long long tag) {
   const long per_row = hidden / 8, total = rows * per_row;
@@ -94,8 +146,8 @@ __global__ void swiglu_bwd_kernel(const unsigned short* __restrict__ gate_up, co
   if (i >= total) return;
   const long r = i / per_row, c = (i % per_row) * 8;
   float g[8], u[8], d[8], gg[8], gu[8];
-  unpack8(*reinterpret_cast<const uint4*>(gate_up + r * 2 * hidden + c), g);
-  unpack8(*reinterpret_cast<const uint4*>(gate_up + r * 2 * hidden + hidden + c), u);
+  load8(gate_up + r * 2 * hidden + c, g);
+  load8(gate_up + r * 2 * hidden + hidden + c, u);
   unpack8(*reinterpret_cast<const uint4*>(gm + r * hidden + c), d);
   bool bad = false;
 #pragma unroll
@@ -203,6 +255,40 @@ int32_t omx_rope_half_split_inplace(omx_ctx* ctx, void* x, int32_t dtype, uint64
   return OMX_OK;
 }
 
+int32_t omx_rope_half_split_pitched(omx_ctx* ctx, const void* x, int32_t x_dtype, void* out, uint64_t pitch,
+                                    const void* cos_f32, const void* sin_f32, uint64_t tokens, uint64_t time,
+                                    uint64_t heads, uint64_t plain_heads, uint64_t dim) {
+  OMX_REQUIRE_CTX(ctx);
+  const char* op = "rope_half_split_forward";
+  if (!x || !out || !cos_f32 || !sin_f32) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
+  if (!omx_valid_float_dtype(x_dtype)) return omx_fail(ctx, OMX_DTYPE, "%s: the input must be f32 or bf16", op);
+  if (tokens == 0 || time == 0 || heads + plain_heads == 0 || dim == 0)
+    return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
+  if (dim % 16 != 0) return omx_fail(ctx, OMX_SHAPE, "%s: head_dim %llu is not a multiple of 16", op, (unsigned long long)dim);
+  if (pitch < (heads + plain_heads) * dim || pitch % 8 != 0 || !aligned16(x) || !aligned16(out) || !aligned16(cos_f32) ||
+      !aligned16(sin_f32))
+    return omx_fail(ctx, OMX_SHAPE, "%s: pitch %llu does not hold %llu heads of %llu in 16-byte pieces", op,
+                    (unsigned long long)pitch, (unsigned long long)(heads + plain_heads), (unsigned long long)dim);
+  if (tokens > 0x7fffffffull || (heads + plain_heads) * dim > 0x7fffffffull)
+    return omx_fail(ctx, OMX_OUT_OF_RANGE, "%s: axis does not fit in i32", op);
+  const long total = static_cast<long>(tokens * (heads + plain_heads) * (dim / 16));
+  const dim3 grid(static_cast<unsigned>((total + 255) / 256));
+  const unsigned long long tag = omx_tag(ctx, F_ROPE_FORWARD);
+  if (x_dtype == OMX_BF16)
+    hipLaunchKernelGGL(rope_pitched_out_kernel<unsigned short>, grid, dim3(256), 0, ctx->stream,
+                       static_cast<const unsigned short*>(x), static_cast<unsigned short*>(out), static_cast<long>(pitch),
+                       static_cast<const float*>(cos_f32), static_cast<const float*>(sin_f32), static_cast<long>(tokens),
+                       static_cast<int>(time), static_cast<int>(heads), static_cast<int>(plain_heads),
+                       static_cast<int>(dim), ctx->fault, tag);
+  else
+    hipLaunchKernelGGL(rope_pitched_out_kernel<float>, grid, dim3(256), 0, ctx->stream, static_cast<const float*>(x),
+                       static_cast<unsigned short*>(out), static_cast<long>(pitch), static_cast<const float*>(cos_f32),
+                       static_cast<const float*>(sin_f32), static_cast<long>(tokens), static_cast<int>(time),
+                       static_cast<int>(heads), static_cast<int>(plain_heads), static_cast<int>(dim), ctx->fault, tag);
+  OMX_LAUNCH_CHECK(ctx, "rope_pitched_out_kernel");
+  return OMX_OK;
+}
+
 int32_t omx_init_normal(omx_ctx* ctx, void* dst, int32_t dtype, uint64_t n, uint64_t seed, float std) {
   OMX_REQUIRE_CTX(ctx);
   if (!dst) return omx_fail(ctx, OMX_PLACEMENT, "init_normal: null device pointer");
@@ -240,15 +326,21 @@ int32_t omx_swiglu_forward(omx_ctx* ctx, const void* gate_up, void* out, int32_t
   OMX_REQUIRE_CTX(ctx);
   const char* op = "swiglu_forward";
   if (!gate_up || !out) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
-  if (dtype != OMX_BF16) return omx_fail(ctx, OMX_DTYPE, "%s: bf16 only", op);
+  if (!omx_valid_float_dtype(dtype)) return omx_fail(ctx, OMX_DTYPE, "%s: gate_up must be f32 or bf16", op);
   if (rows == 0 || hidden == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
   if (hidden % 8 != 0 || !aligned16(gate_up) || !aligned16(out))
     return omx_fail(ctx, OMX_SHAPE, "%s: hidden %llu must be a multiple of 8 and the tensors 16-byte aligned", op,
                     (unsigned long long)hidden);
   const long total = static_cast<long>(rows * (hidden / 8));
-  hipLaunchKernelGGL(swiglu_fwd_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, ctx->stream,
-                     static_cast<const unsigned short*>(gate_up), static_cast<unsigned short*>(out),
-                     static_cast<long>(rows), static_cast<long>(hidden), ctx->fault, omx_tag(ctx, F_MUL_FORWARD));
+  const unsigned long long tag = omx_tag(ctx, F_MUL_FORWARD);
+  if (dtype == OMX_BF16)
+    hipLaunchKernelGGL(swiglu_fwd_kernel<unsigned short>, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0,
+                       ctx->stream, static_cast<const unsigned short*>(gate_up), static_cast<unsigned short*>(out),
+                       static_cast<long>(rows), static_cast<long>(hidden), ctx->fault, tag);
+  else
+    hipLaunchKernelGGL(swiglu_fwd_kernel<float>, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0,
+                       ctx->stream, static_cast<const float*>(gate_up), static_cast<unsigned short*>(out),
+                       static_cast<long>(rows), static_cast<long>(hidden), ctx->fault, tag);
   OMX_LAUNCH_CHECK(ctx, "swiglu_fwd_kernel");
   return OMX_OK;
 }
@@ -258,16 +350,23 @@ int32_t omx_swiglu_backward(omx_ctx* ctx, const void* gate_up, const void* gy, v
   OMX_REQUIRE_CTX(ctx);
   const char* op = "swiglu_backward";
   if (!gate_up || !gy || !g_gate_up) return omx_fail(ctx, OMX_PLACEMENT, "%s: null device pointer", op);
-  if (dtype != OMX_BF16) return omx_fail(ctx, OMX_DTYPE, "%s: bf16 only", op);
+  if (!omx_valid_float_dtype(dtype)) return omx_fail(ctx, OMX_DTYPE, "%s: gate_up must be f32 or bf16", op);
   if (rows == 0 || hidden == 0) return omx_fail(ctx, OMX_SHAPE, "%s: zero-sized axis", op);
   if (hidden % 8 != 0 || !aligned16(gate_up) || !aligned16(gy) || !aligned16(g_gate_up))
     return omx_fail(ctx, OMX_SHAPE, "%s: hidden %llu must be a multiple of 8 and the tensors 16-byte aligned", op,
                     (unsigned long long)hidden);
   const long total = static_cast<long>(rows * (hidden / 8));
-  hipLaunchKernelGGL(swiglu_bwd_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, ctx->stream,
-                     static_cast<const unsigned short*>(gate_up), static_cast<const unsigned short*>(gy),
-                     static_cast<unsigned short*>(g_gate_up), static_cast<long>(rows), static_cast<long>(hidden),
-                     ctx->fault, omx_tag(ctx, F_MUL_BACKWARD));
+  const unsigned long long tag = omx_tag(ctx, F_MUL_BACKWARD);
+  if (dtype == OMX_BF16)
+    hipLaunchKernelGGL(swiglu_bwd_kernel<unsigned short>, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0,
+                       ctx->stream, static_cast<const unsigned short*>(gate_up), static_cast<const unsigned short*>(gy),
+                       static_cast<unsigned short*>(g_gate_up), static_cast<long>(rows), static_cast<long>(hidden),
+                       ctx->fault, tag);
+  else
+    hipLaunchKernelGGL(swiglu_bwd_kernel<float>, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0,
+                       ctx->stream, static_cast<const float*>(gate_up), static_cast<const unsigned short*>(gy),
+                       static_cast<unsigned short*>(g_gate_up), static_cast<long>(rows), static_cast<long>(hidden),
+                       ctx->fault, tag);
   OMX_LAUNCH_CHECK(ctx, "swiglu_bwd_kernel");
   return OMX_OK;
 }

@@ -1,9 +1,11 @@
 // What the nanolab block does to a fused q | k | v projection output before attention, in one pass
 // over HBM each way: per-head RMSNorm of q and k (rms_qk_norm, ojas-cpu/src/norm.rs:60-180), the
 // half-split rotary embedding on the result (norm.rs:271-347), and the value-residual blend on v
-// (ojas-cpu/src/pointwise.rs:2031-2148); the graph is ojas-model/src/block.rs:225-240. bf16 tensors
+// (ojas-cpu/src/pointwise.rs:2031-2148); the graph is ojas-model/src/block.rs:225-240. Tensors
 // whose token rows are `pitch` elements apart and hold, per token, the query heads, then the key
-// heads, then the value heads.
+// heads, then the value heads. The prepared q | k | v and the gradients are bf16 (operands of the
+// attention products and of the projection's backward); the projection output itself (and block
+// 0's, for the blend) is bf16 or f32: kept in f32 it reaches attention with one rounding.
 //
 // A head row (64 or 128 values) is held by head_dim / 8 adjacent lanes, 8 values (one 16-byte
 // access) each: the row's sum of squares is a shuffle reduction over those lanes and the rotary
@@ -36,6 +38,12 @@ __device__ __forceinline__ uint4 pack8(const float (&v)[8]) {
     w[i] = dev_pack_bf16_pair(v[2 * i], v[2 * i + 1]);
   return make_uint4(w[0], w[1], w[2], w[3]);
 }
+__device__ __forceinline__ void load8f(const float* __restrict__ p, float (&v)[8]);
+// Eight consecutive values of a projection output stored as bf16 or as f32.
+__device__ __forceinline__ void load_lin(const unsigned short* __restrict__ p, float (&v)[8]) {
+  unpack8(*reinterpret_cast<const uint4*>(p), v);
+}
+__device__ __forceinline__ void load_lin(const float* __restrict__ p, float (&v)[8]) { load8f(p, v); }
 __device__ __forceinline__ void load8f(const float* __restrict__ p, float (&v)[8]) {
   const float4 a = reinterpret_cast<const float4*>(p)[0], b = reinterpret_cast<const float4*>(p)[1];
   v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
@@ -58,11 +66,11 @@ __device__ __forceinline__ void sigmoid_both(float u, float* s, float* rest) {
 
 // Row r of the launch is (token, slot): slot < heads is a query head, the next kv_heads are key
 // heads, the rest value heads.
-template <int D>
+template <int D, typename LIN>
 __global__ __launch_bounds__(QP_THREADS) void qkv_prepare_fwd_kernel(
-    const unsigned short* __restrict__ lin, unsigned short* __restrict__ out, const float* __restrict__ q_weight,
+    const LIN* __restrict__ lin, unsigned short* __restrict__ out, const float* __restrict__ q_weight,
     const float* __restrict__ k_weight, const float* __restrict__ cos, const float* __restrict__ sin,
-    const unsigned short* __restrict__ v0, const float* __restrict__ lambda, QkvShape s, OmxFaultWord* fault,
+    const LIN* __restrict__ v0, const float* __restrict__ lambda, QkvShape s, OmxFaultWord* fault,
     unsigned long long tag) {
   constexpr int LPR = D / 8, ROWS = QP_THREADS / LPR;
   const int slots = s.heads + 2 * s.kv_heads;
@@ -80,11 +88,11 @@ __global__ __launch_bounds__(QP_THREADS) void qkv_prepare_fwd_kernel(
     const int slot = static_cast<int>(r % slots);
     const long at = token * s.pitch + static_cast<long>(slot) * D + col;
     float x[8], y[8];
-    unpack8(*reinterpret_cast<const uint4*>(lin + at), x);
+    load_lin(lin + at, x);
     if (slot >= s.heads + s.kv_heads) {
       if (v0) {
         float b[8];
-        unpack8(*reinterpret_cast<const uint4*>(v0 + at), b);
+        load_lin(v0 + at, b);
 #pragma unroll
         for (int i = 0; i < 8; ++i) y[i] = blend_rest * x[i] + blend_s * b[i];
       } else {
@@ -124,11 +132,11 @@ __global__ __launch_bounds__(QP_THREADS) void qkv_prepare_fwd_kernel(
 // (partial_w: [blocks][2][D], q then k) and the blend's as one partial per workgroup; v0_acc
 // (f32 [tokens, kv_heads * D]) collects what the blends send to block 0's value, written when
 // `v0_first` and added to otherwise; `add_v` (block 0 only, no blend) is added to the value's gradient.
-template <int D>
+template <int D, typename LIN>
 __global__ __launch_bounds__(QP_THREADS) void qkv_prepare_bwd_kernel(
-    const unsigned short* __restrict__ lin, const unsigned short* __restrict__ g, unsigned short* __restrict__ g_lin,
+    const LIN* __restrict__ lin, const unsigned short* __restrict__ g, unsigned short* __restrict__ g_lin,
     const float* __restrict__ q_weight, const float* __restrict__ k_weight, const float* __restrict__ cos,
-    const float* __restrict__ sin, const unsigned short* __restrict__ v0, const float* __restrict__ lambda,
+    const float* __restrict__ sin, const LIN* __restrict__ v0, const float* __restrict__ lambda,
     float* __restrict__ v0_acc, int v0_first, const float* __restrict__ add_v, float* __restrict__ partial_w,
     float* __restrict__ partial_lambda, QkvShape s, OmxFaultWord* fault, unsigned long long tag) {
   constexpr int LPR = D / 8, ROWS = QP_THREADS / LPR;
@@ -154,13 +162,13 @@ __global__ __launch_bounds__(QP_THREADS) void qkv_prepare_bwd_kernel(
     const int slot = static_cast<int>(r % slots);
     const long at = token * s.pitch + static_cast<long>(slot) * D + col;
     float x[8], gy[8], out[8];
-    unpack8(*reinterpret_cast<const uint4*>(lin + at), x);
+    load_lin(lin + at, x);
     unpack8(*reinterpret_cast<const uint4*>(g + at), gy);
     if (slot >= s.heads + s.kv_heads) {
       const long vat = token * kv_cols + static_cast<long>(slot - s.heads - s.kv_heads) * D + col;
       if (v0) {
         float b[8];
-        unpack8(*reinterpret_cast<const uint4*>(v0 + at), b);
+        load_lin(v0 + at, b);
         float* acc = v0_acc + vat;
         float keep[8];
         if (!v0_first) load8f(acc, keep);
@@ -286,12 +294,13 @@ unsigned grid_for(const omx_ctx* ctx, uint64_t rows, int rows_per_block) {
 
 extern "C" {
 
-int32_t omx_qkv_prepare_forward(omx_ctx* ctx, const void* qkv_lin, void* qkv_out, uint64_t pitch, const void* q_weight,
+int32_t omx_qkv_prepare_forward(omx_ctx* ctx, const void* qkv_lin, int32_t lin_dtype, void* qkv_out, uint64_t pitch, const void* q_weight,
                                 const void* k_weight, const void* cos, const void* sin, const void* value0,
                                 const void* lambda, uint64_t tokens, uint64_t time, uint64_t heads, uint64_t kv_heads,
                                 uint64_t head_dim, float eps) {
   OMX_REQUIRE_CTX(ctx);
   const char* op = "qkv_prepare_forward";
+  if (!omx_valid_float_dtype(lin_dtype)) return omx_fail(ctx, OMX_DTYPE, "%s: the projection output must be f32 or bf16", op);
   int32_t rc = check(ctx, op, pitch, tokens, time, heads, kv_heads, head_dim, eps, {qkv_lin, qkv_out, q_weight, k_weight, cos, sin});
   if (rc != OMX_OK) return rc;
   if ((value0 != nullptr) != (lambda != nullptr)) return omx_fail(ctx, OMX_PLACEMENT, "%s: value0 and lambda come together", op);
@@ -300,20 +309,25 @@ int32_t omx_qkv_prepare_forward(omx_ctx* ctx, const void* qkv_lin, void* qkv_out
              static_cast<int>(kv_heads), static_cast<int>(head_dim), eps};
   const uint64_t rows = tokens * (heads + 2 * kv_heads);
   const unsigned long long tag = omx_tag(ctx, F_RMS_FORWARD);
-#define QP_FWD(D_)                                                                                                    \
-  hipLaunchKernelGGL((qkv_prepare_fwd_kernel<D_>), dim3(grid_for(ctx, rows, QP_THREADS / (D_ / 8))), dim3(QP_THREADS), \
-                     0, ctx->stream, static_cast<const unsigned short*>(qkv_lin), static_cast<unsigned short*>(qkv_out), \
-                     static_cast<const float*>(q_weight), static_cast<const float*>(k_weight),                        \
-                     static_cast<const float*>(cos), static_cast<const float*>(sin),                                  \
-                     static_cast<const unsigned short*>(value0), static_cast<const float*>(lambda), s, ctx->fault, tag)
-  if (head_dim == 64) QP_FWD(64);
-  else QP_FWD(128);
+#define QP_FWD(D_, LIN_)                                                                                           \
+  hipLaunchKernelGGL((qkv_prepare_fwd_kernel<D_, LIN_>), dim3(grid_for(ctx, rows, QP_THREADS / (D_ / 8))),             \
+                     dim3(QP_THREADS), 0, ctx->stream, static_cast<const LIN_*>(qkv_lin),                              \
+                     static_cast<unsigned short*>(qkv_out), static_cast<const float*>(q_weight),                       \
+                     static_cast<const float*>(k_weight), static_cast<const float*>(cos), static_cast<const float*>(sin), \
+                     static_cast<const LIN_*>(value0), static_cast<const float*>(lambda), s, ctx->fault, tag)
+  if (lin_dtype == OMX_BF16) {
+    if (head_dim == 64) QP_FWD(64, unsigned short);
+    else QP_FWD(128, unsigned short);
+  } else {
+    if (head_dim == 64) QP_FWD(64, float);
+    else QP_FWD(128, float);
+  }
 #undef QP_FWD
   OMX_LAUNCH_CHECK(ctx, "qkv_prepare_fwd_kernel");
   return OMX_OK;
 }
 
-int32_t omx_qkv_prepare_backward(omx_ctx* ctx, const void* qkv_lin, const void* g_qkv, void* g_qkv_lin, uint64_t pitch,
+int32_t omx_qkv_prepare_backward(omx_ctx* ctx, const void* qkv_lin, int32_t lin_dtype, const void* g_qkv, void* g_qkv_lin, uint64_t pitch,
                                  const void* q_weight, const void* k_weight, const void* cos, const void* sin,
                                  const void* value0, const void* lambda, void* value0_grad_f32, int32_t value0_grad_first,
                                  const void* add_value_grad_f32, void* g_q_weight, void* g_k_weight, void* g_lambda,
@@ -321,6 +335,7 @@ int32_t omx_qkv_prepare_backward(omx_ctx* ctx, const void* qkv_lin, const void* 
                                  float eps) {
   OMX_REQUIRE_CTX(ctx);
   const char* op = "qkv_prepare_backward";
+  if (!omx_valid_float_dtype(lin_dtype)) return omx_fail(ctx, OMX_DTYPE, "%s: the projection output must be f32 or bf16", op);
   int32_t rc = check(ctx, op, pitch, tokens, time, heads, kv_heads, head_dim, eps,
                      {qkv_lin, g_qkv, g_qkv_lin, q_weight, k_weight, cos, sin, g_q_weight, g_k_weight});
   if (rc != OMX_OK) return rc;
@@ -345,16 +360,21 @@ int32_t omx_qkv_prepare_backward(omx_ctx* ctx, const void* qkv_lin, const void* 
   float* stage = summed + 2 * head_dim;          // the column sum's first stage
   float* partial_lambda = stage + OMX_COLUMN_SUM_GROUPS * 2 * head_dim;
   const unsigned long long tag = omx_tag(ctx, F_RMS_BACKWARD);
-#define QP_BWD(D_)                                                                                                     \
-  hipLaunchKernelGGL((qkv_prepare_bwd_kernel<D_>), dim3(blocks), dim3(QP_THREADS), 0, ctx->stream,                     \
-                     static_cast<const unsigned short*>(qkv_lin), static_cast<const unsigned short*>(g_qkv),           \
+#define QP_BWD(D_, LIN_)                                                                                               \
+  hipLaunchKernelGGL((qkv_prepare_bwd_kernel<D_, LIN_>), dim3(blocks), dim3(QP_THREADS), 0, ctx->stream,               \
+                     static_cast<const LIN_*>(qkv_lin), static_cast<const unsigned short*>(g_qkv),                     \
                      static_cast<unsigned short*>(g_qkv_lin), static_cast<const float*>(q_weight),                     \
                      static_cast<const float*>(k_weight), static_cast<const float*>(cos), static_cast<const float*>(sin), \
-                     static_cast<const unsigned short*>(value0), static_cast<const float*>(lambda),                    \
+                     static_cast<const LIN_*>(value0), static_cast<const float*>(lambda),                              \
                      static_cast<float*>(value0_grad_f32), value0_grad_first, static_cast<const float*>(add_value_grad_f32), \
                      partial_w, partial_lambda, s, ctx->fault, tag)
-  if (head_dim == 64) QP_BWD(64);
-  else QP_BWD(128);
+  if (lin_dtype == OMX_BF16) {
+    if (head_dim == 64) QP_BWD(64, unsigned short);
+    else QP_BWD(128, unsigned short);
+  } else {
+    if (head_dim == 64) QP_BWD(64, float);
+    else QP_BWD(128, float);
+  }
 #undef QP_BWD
   OMX_LAUNCH_CHECK(ctx, "qkv_prepare_bwd_kernel");
   // partial_w is [blocks][2 D]: one column sum gives both weights' gradients side by side.

@@ -56,7 +56,8 @@ struct olora {
   struct Layer {
     QMat qkv, o, gu, dn;
     float *x = nullptr, *x1 = nullptr;  // residual stream before / inside the block (f32)
-    void *h1 = nullptr, *ha = nullptr, *qkv_out = nullptr, *ap = nullptr, *apr = nullptr, *gu_out = nullptr;  // bf16
+    void *h1 = nullptr, *ha = nullptr, *qkv_out = nullptr, *ap = nullptr, *apr = nullptr;  // bf16
+    void* gu_out = nullptr;  // [N, 2 hidden] f32: the gate | up projection's output, read again by the backward
     float* lse = nullptr;
   };
   std::vector<Layer> layers;
@@ -77,6 +78,7 @@ struct olora {
   float *loss = nullptr, *cos_t = nullptr, *sin_t = nullptr, *dummy_gw = nullptr;
   // Scratch.
   float *x_final = nullptr, *gres = nullptr, *gres1 = nullptr;
+  void *t_f = nullptr, *qkv32 = nullptr;  // f32 scratch: a [N, d] product output, the q | k | v projection's [N, 3d]
   void *hf = nullptr, *h2 = nullptr, *m = nullptr, *t_a = nullptr, *t_b = nullptr, *gy16 = nullptr, *gm = nullptr,
        *ggu = nullptr, *ga = nullptr, *ghf = nullptr;
 
@@ -137,9 +139,12 @@ int32_t refresh_operands(olora* t) {
   return omx_permute_0213(t->ctx, t->p16, t->at16, OMX_BF16, L, 4 * r, d, 1);
 }
 
-int32_t q8_forward(olora* t, const void* x, const QMat& w, const omx_low_rank* lr, void* y) {
-  return omx_linear_i8_group_forward(t->ctx, x, OMX_BF16, w.codes, w.scales, 32, OMX_I8_BLOCKED, nullptr, lr, y, t->N,
-                                     w.kin, w.nout);
+// The forward's products leave their outputs in f32: what follows each (the rotation, the residual
+// add and norm, SwiGLU) reads them unrounded, so an activation is rounded to bf16 once, where it
+// becomes the next product's operand.
+int32_t q8_forward(olora* t, const void* x, const QMat& w, const omx_low_rank* lr, void* y_f32) {
+  return omx_linear_i8_group_forward(t->ctx, x, OMX_BF16, w.codes, w.scales, 32, OMX_I8_BLOCKED, nullptr, lr, y_f32,
+                                     OMX_F32, t->N, w.kin, w.nout);
 }
 int32_t q8_backward(olora* t, const QMat& w, const void* gy, const omx_low_rank* lr, void* gx) {
   return omx_linear_i8_group_backward_input(t->ctx, w.codes, w.scales, 32, OMX_I8_BLOCKED, gy, OMX_BF16, nullptr, lr, gx,
@@ -159,24 +164,24 @@ int32_t forward(olora* t) {
     // h A^T for the three sites at once: [N, 3r] in the first columns of ha.
     TRY(omx_gemm_pitched(ctx, A.h1, d, 1, t->a16(l, 0), 1, d, OMX_BF16, A.ha, OMX_BF16, 4 * r, N, d, 3 * r, 0));
     omx_low_rank lr_qkv{A.ha, t->b16(l, 0), 4 * r, r, r, d};
-    TRY(q8_forward(t, A.h1, A.qkv, &lr_qkv, A.qkv_out));
-    TRY(omx_rope_half_split_inplace(ctx, A.qkv_out, OMX_BF16, 3 * d, t->cos_t, t->sin_t, N, T, 2 * H, D, 0));
+    TRY(q8_forward(t, A.h1, A.qkv, &lr_qkv, t->qkv32));
+    TRY(omx_rope_half_split_pitched(ctx, t->qkv32, OMX_F32, A.qkv_out, 3 * d, t->cos_t, t->sin_t, N, T, 2 * H, H, D));
     // The output's rounding residual is kept for the backward's row term, as the reference keeps
     // its saved output unrounded (ojas-core/src/autocast.rs:177-186).
     TRY(omx_causal_attention_forward_saving(ctx, A.qkv_out, 3 * d, off16(A.qkv_out, d), off16(A.qkv_out, 2 * d), 3 * d,
                                             OMX_BF16, A.ap, A.apr, d, OMX_BF16, A.lse, B, T, H, H, D, 0));
     TRY(omx_gemm_pitched(ctx, A.ap, d, 1, t->a16(l, 3), 1, d, OMX_BF16, off16(A.ha, 3 * r), OMX_BF16, 4 * r, N, d, r, 0));
     omx_low_rank lr_o{off16(A.ha, 3 * r), t->b16(l, 3), 4 * r, r, r, 0};
-    TRY(q8_forward(t, A.ap, A.o, &lr_o, t->t_a));
-    TRY(omx_residual_add_rms_norm_forward(ctx, A.x, OMX_F32, t->t_a, OMX_BF16, t->norm(l, 1), A.x1, t->h2, OMX_BF16, N, d,
+    TRY(q8_forward(t, A.ap, A.o, &lr_o, t->t_f));
+    TRY(omx_residual_add_rms_norm_forward(ctx, A.x, OMX_F32, t->t_f, OMX_F32, t->norm(l, 1), A.x1, t->h2, OMX_BF16, N, d,
                                           eps));
     TRY(q8_forward(t, t->h2, A.gu, nullptr, A.gu_out));
-    TRY(omx_swiglu_forward(ctx, A.gu_out, t->m, OMX_BF16, N, Hd));
-    TRY(q8_forward(t, t->m, A.dn, nullptr, t->t_a));
+    TRY(omx_swiglu_forward(ctx, A.gu_out, t->m, OMX_F32, N, Hd));
+    TRY(q8_forward(t, t->m, A.dn, nullptr, t->t_f));
     float* x_next = last ? t->x_final : t->layers[l + 1].x;
     void* h_next = last ? t->hf : t->layers[l + 1].h1;
     const float* next_norm = last ? t->final_norm() : t->norm(l + 1, 0);
-    TRY(omx_residual_add_rms_norm_forward(ctx, A.x1, OMX_F32, t->t_a, OMX_BF16, next_norm, x_next, h_next, OMX_BF16, N, d,
+    TRY(omx_residual_add_rms_norm_forward(ctx, A.x1, OMX_F32, t->t_f, OMX_F32, next_norm, x_next, h_next, OMX_BF16, N, d,
                                           eps));
   }
   return OMX_OK;
@@ -197,7 +202,7 @@ int32_t backward(olora* t) {
     olora::Layer& A = t->layers[l];
     // x_next = x1 + down(silu(gate) * up)
     TRY(q8_backward(t, A.dn, t->gy16, nullptr, t->gm));
-    TRY(omx_swiglu_backward(ctx, A.gu_out, t->gm, t->ggu, OMX_BF16, N, Hd));
+    TRY(omx_swiglu_backward(ctx, A.gu_out, t->gm, t->ggu, OMX_F32, N, Hd));
     TRY(q8_backward(t, A.gu, t->ggu, nullptr, t->t_a));
     // Fan-in at x1: the residual branch first, then the norm branch. The bf16 copy is this layer's
     // own: the o site's weight gradients read it after the loop.
@@ -338,7 +343,7 @@ int32_t olora_create(omx_ctx* ctx, const olora_config* config, olora** out) {
     ++layer_index;
     CREATE_TRY(alloc16(t, N * 3 * d, &A.qkv_out));
     CREATE_TRY(alloc16(t, N * d, &A.apr));
-    CREATE_TRY(alloc16(t, N * 2 * h, &A.gu_out));
+    CREATE_TRY(alloc(t, N * 2 * h * 4, &A.gu_out));
     CREATE_TRY(alloc_t(t, static_cast<uint64_t>(c.batch) * c.heads * c.seq, &A.lse));
   }
   CREATE_TRY(alloc_t(t, t->P, &t->p32));
@@ -379,6 +384,8 @@ int32_t olora_create(omx_ctx* ctx, const olora_config* config, olora** out) {
   CREATE_TRY(alloc16(t, N * d, &t->h2));
   CREATE_TRY(alloc16(t, N * h, &t->m));
   CREATE_TRY(alloc16(t, N * d, &t->t_a));
+  CREATE_TRY(alloc(t, N * d * 4, &t->t_f));
+  CREATE_TRY(alloc(t, N * 3 * d * 4, &t->qkv32));
   CREATE_TRY(alloc16(t, N * d, &t->t_b));
   CREATE_TRY(alloc16(t, N * d, &t->gy16));
   CREATE_TRY(alloc16(t, N * h, &t->gm));

@@ -52,6 +52,13 @@ struct onano {
   // the arena: one [(heads + 2 kv_heads) head_dim, n_embd] matrix), QK-norm, RoPE and the value blend
   // are one pass over its output, and attention reads q, k and v where that pass left them.
   bool fused_qkv = false;
+  // bf16 tier, fused paths: the forward's product outputs (the q | k | v, o, gate | up and down
+  // projections) and the attention output the gate reads stay f32, so every activation is rounded
+  // to bf16 once, where it becomes a product's operand, and not a second time where a product
+  // left it. `LD` is the dtype of those outputs, `lsz` its size.
+  bool keep_f32 = false;
+  int32_t LD = OMX_F32;
+  uint64_t lsz = 4;
   uint64_t steps = 0;
   uint64_t device_bytes = 0;
   std::vector<void*> owned;
@@ -82,6 +89,8 @@ struct onano {
   // Scratch.
   void *t_q = nullptr, *t_k = nullptr;   // [N, H D], [N, KV D] AD
   void *t_a = nullptr;                   // [N, max(d, H D)] AD
+  void *t_f = nullptr;                   // [N, d] LD: the o and down projections' outputs on the forward
+  float *ap32 = nullptr;                 // [N, H D] f32: the attention output and its rounding residual, summed (keep_f32)
   void *gm = nullptr, *ggu = nullptr, *g_gact = nullptr, *g_up = nullptr;  // MLP gradients AD
   void *gyy = nullptr, *gap = nullptr, *gq = nullptr, *gk = nullptr, *gv = nullptr, *g_raw_v = nullptr, *part_v0 = nullptr;
   void *g_v0 = nullptr;                  // [N, KV D] AD: what the later blocks' blends send to block 0's v
@@ -152,7 +161,7 @@ int32_t forward(onano* t) {
   const uint64_t N = t->N, d = c.n_embd, B = c.batch, T = c.seq, H = c.heads, KV = c.kv_heads, D = c.head_dim,
                  Hd = c.hidden, W = c.window;
   const uint64_t qd = H * D, kd = KV * D;
-  const int32_t AD = t->AD;
+  const int32_t AD = t->AD, LD = t->LD;
   const float eps = c.rms_eps;
   // x = tok_emb[ids], then norm1 of block 0 (or the final norm of a model without blocks).
   {
@@ -170,18 +179,18 @@ int32_t forward(onano* t) {
     if (t->fused_qkv) {
       const uint64_t P3 = qd + 2 * kd;
       char* prepared = static_cast<char*>(A.qkv);
-      TRY(omx_linear_forward(ctx, A.h, AD, t->w(t->li(l, WQ)), AD, A.qkv_lin, AD, N, d, P3));
+      TRY(omx_linear_forward(ctx, A.h, AD, t->w(t->li(l, WQ)), AD, A.qkv_lin, LD, N, d, P3));
       // Block 0 has no earlier value to blend with (block.rs:232-238).
-      TRY(omx_qkv_prepare_forward(ctx, A.qkv_lin, A.qkv, P3, t->w32(t->li(l, QNORM)), t->w32(t->li(l, KNORM)), t->cos_t,
+      TRY(omx_qkv_prepare_forward(ctx, A.qkv_lin, LD, A.qkv, P3, t->w32(t->li(l, QNORM)), t->w32(t->li(l, KNORM)), t->cos_t,
                                   t->sin_t, l > 0 ? t->layers[0].qkv_lin : nullptr,
                                   l > 0 ? t->w32(t->li(l, LAMBDA)) : nullptr, N, T, H, KV, D, eps));
       TRY(omx_causal_attention_forward_saving(ctx, prepared, P3, prepared + qd * 2, prepared + (qd + kd) * 2, P3, AD, A.ap,
                                               A.apr, qd, AD, A.lse, B, T, H, KV, D, W));
     } else {
-    TRY(omx_linear_forward(ctx, A.h, AD, t->w(t->li(l, WQ)), AD, A.q_lin, AD, N, d, qd));
-    TRY(omx_linear_forward(ctx, A.h, AD, t->w(t->li(l, WK)), AD, A.k_lin, AD, N, d, kd));
+    TRY(omx_linear_forward(ctx, A.h, AD, t->w(t->li(l, WQ)), AD, A.q_lin, LD, N, d, qd));
+    TRY(omx_linear_forward(ctx, A.h, AD, t->w(t->li(l, WK)), AD, A.k_lin, LD, N, d, kd));
     TRY(omx_linear_forward(ctx, A.h, AD, t->w(t->li(l, WV)), AD, A.raw_v, AD, N, d, kd));
-    TRY(omx_rms_qk_norm_forward(ctx, A.q_lin, A.k_lin, AD, t->w32(t->li(l, QNORM)), t->w32(t->li(l, KNORM)), t->t_q,
+    TRY(omx_rms_qk_norm_forward(ctx, A.q_lin, A.k_lin, LD, t->w32(t->li(l, QNORM)), t->w32(t->li(l, KNORM)), t->t_q,
                                 t->t_k, AD, N * H, N * KV, D, eps));
     TRY(omx_rope_half_split_forward(ctx, t->t_q, t->cos_t, t->sin_t, A.q, AD, N * H, D, T, H));
     TRY(omx_rope_half_split_forward(ctx, t->t_k, t->cos_t, t->sin_t, A.k, AD, N * KV, D, T, KV));
@@ -201,22 +210,29 @@ int32_t forward(onano* t) {
       TRY(omx_permute_0213(ctx, A.att, A.ap, AD, B, H, T, D));
     }
     }
-    TRY(omx_per_head_sigmoid_gate_forward(ctx, A.h, t->w(t->li(l, GATE_W)), AD, t->w32(t->li(l, GATE_B)), A.ap, AD, A.y,
-                                          AD, A.gates, N, d, H, D));
-    TRY(omx_linear_forward(ctx, A.y, AD, t->w(t->li(l, WO)), AD, t->t_a, AD, N, qd, d));
-    TRY(omx_residual_add_rms_norm_forward(ctx, A.x, OMX_F32, t->t_a, AD, t->w32(t->li(l, NORM2)), A.x1, A.h2, AD, N, d,
+    // The row-kernel attention keeps no rounding residual: the gate then reads what was stored.
+    const bool gate_f32 = t->keep_f32 && t->flash;
+    const void* attn = A.ap;
+    if (gate_f32) {  // the gate reads the attention output at 16 bits of mantissa: what was stored plus what that dropped
+      TRY(omx_residual_add(ctx, A.ap, AD, A.apr, AD, t->ap32, OMX_F32, N * qd));
+      attn = t->ap32;
+    }
+    TRY(omx_per_head_sigmoid_gate_forward(ctx, A.h, t->w(t->li(l, GATE_W)), AD, t->w32(t->li(l, GATE_B)), attn,
+                                          gate_f32 ? OMX_F32 : AD, A.y, AD, A.gates, N, d, H, D));
+    TRY(omx_linear_forward(ctx, A.y, AD, t->w(t->li(l, WO)), AD, t->t_f, LD, N, qd, d));
+    TRY(omx_residual_add_rms_norm_forward(ctx, A.x, OMX_F32, t->t_f, LD, t->w32(t->li(l, NORM2)), A.x1, A.h2, AD, N, d,
                                           eps));
     if (t->fused_mlp) {
-      TRY(omx_linear_forward(ctx, A.h2, AD, t->w(t->li(l, FFN_GATE)), AD, A.gu, AD, N, d, 2 * Hd));
-      TRY(omx_swiglu_forward(ctx, A.gu, A.m, AD, N, Hd));
+      TRY(omx_linear_forward(ctx, A.h2, AD, t->w(t->li(l, FFN_GATE)), AD, A.gu, LD, N, d, 2 * Hd));
+      TRY(omx_swiglu_forward(ctx, A.gu, A.m, LD, N, Hd));
     } else {
       TRY(omx_linear_forward(ctx, A.h2, AD, t->w(t->li(l, FFN_GATE)), AD, A.g_lin, AD, N, d, Hd));
       TRY(omx_silu_forward(ctx, A.g_lin, A.g_act, AD, N * Hd));
       TRY(omx_linear_forward(ctx, A.h2, AD, t->w(t->li(l, FFN_UP)), AD, A.up, AD, N, d, Hd));
       TRY(omx_mul_forward(ctx, A.g_act, A.up, A.m, AD, N * Hd));
     }
-    TRY(omx_linear_forward(ctx, A.m, AD, t->w(t->li(l, FFN_DOWN)), AD, t->t_a, AD, N, Hd, d));
-    TRY(omx_residual_add_rms_norm_forward(ctx, A.x1, OMX_F32, t->t_a, AD, next_norm, x_next, h_next, AD, N, d, eps));
+    TRY(omx_linear_forward(ctx, A.m, AD, t->w(t->li(l, FFN_DOWN)), AD, t->t_f, LD, N, Hd, d));
+    TRY(omx_residual_add_rms_norm_forward(ctx, A.x1, OMX_F32, t->t_f, LD, next_norm, x_next, h_next, AD, N, d, eps));
   }
   return OMX_OK;
 }
@@ -227,7 +243,7 @@ int32_t backward(onano* t, float loss_seed) {
   const uint64_t N = t->N, d = c.n_embd, B = c.batch, T = c.seq, H = c.heads, KV = c.kv_heads, D = c.head_dim,
                  Hd = c.hidden, W = c.window;
   const uint64_t qd = H * D, kd = KV * D;
-  const int32_t AD = t->AD;
+  const int32_t AD = t->AD, LD = t->LD;
   const float eps = c.rms_eps;
   const uint64_t chunk_rows = N < 16384 ? N : 16384;
   TRY(omx_linear_cross_entropy_mean(ctx, t->hf, t->w(0), AD, t->targets, N, d, c.vocab, 0, 0, chunk_rows, c.vocab,
@@ -269,7 +285,7 @@ int32_t backward(onano* t, float loss_seed) {
     // x_next = x1 + down(silu(gate(h2)) * up(h2))
     TRY(omx_linear_backward(ctx, A.m, t->w(t->li(l, FFN_DOWN)), gy, AD, t->gm, AD, gw(FFN_DOWN), OMX_F32, N, Hd, d));
     if (t->fused_mlp) {
-      TRY(omx_swiglu_backward(ctx, A.gu, t->gm, ggu, AD, N, Hd));
+      TRY(omx_swiglu_backward(ctx, A.gu, t->gm, ggu, LD, N, Hd));
       // One product for both projections: their input gradients add in its f32 accumulators.
       TRY(omx_linear_backward(ctx, A.h2, t->w(t->li(l, FFN_GATE)), ggu, AD, t->t_a, AD, gw(FFN_GATE), OMX_F32, N, d,
                               2 * Hd));
@@ -289,15 +305,24 @@ int32_t backward(onano* t, float loss_seed) {
     }
     gy = AD == OMX_BF16 ? static_cast<const void*>(t->fused_mlp ? copy_o : copy16) : static_cast<const void*>(t->gres1);
     // x1 = x + o(gate(h) * attention)
-    TRY(omx_linear_backward(ctx, A.y, t->w(t->li(l, WO)), gy, AD, t->gyy, AD, gw(WO), OMX_F32, N, qd, d));
+    // The gate's backward takes the attention output and the gradient of its own output in one
+    // dtype: both f32 when the forward kept the output's dropped bits.
+    const bool gate_f32 = t->keep_f32 && t->flash;
+    const int32_t GD = gate_f32 ? OMX_F32 : AD;
+    const void* attn = A.ap;
+    if (gate_f32) {
+      TRY(omx_residual_add(ctx, A.ap, AD, A.apr, AD, t->ap32, OMX_F32, N * qd));
+      attn = t->ap32;
+    }
+    TRY(omx_linear_backward(ctx, A.y, t->w(t->li(l, WO)), gy, AD, t->gyy, GD, gw(WO), OMX_F32, N, qd, d));
     if (defer && t->gz_all)  // the gate's weight gradient waits for the batched product below
-      TRY(omx_per_head_sigmoid_gate_backward_deferred(ctx, A.h, t->w(t->li(l, GATE_W)), AD, t->w32(t->li(l, GATE_B)), A.ap,
-                                                      AD, t->gyy, AD, A.gates, t->fused_qkv ? nullptr : t->gh, OMX_F32,
+      TRY(omx_per_head_sigmoid_gate_backward_deferred(ctx, A.h, t->w(t->li(l, GATE_W)), AD, t->w32(t->li(l, GATE_B)), attn,
+                                                      GD, t->gyy, GD, A.gates, t->fused_qkv ? nullptr : t->gh, OMX_F32,
                                                       slice(t->gz_all, l, N * H),
                                                       t->g(t->li(l, GATE_B)), t->gap, AD, N, d, H, D));
     else
-      TRY(omx_per_head_sigmoid_gate_backward(ctx, A.h, t->w(t->li(l, GATE_W)), AD, t->w32(t->li(l, GATE_B)), A.ap, AD,
-                                             t->gyy, AD, A.gates, t->gh, OMX_F32, t->g(t->li(l, GATE_W)),
+      TRY(omx_per_head_sigmoid_gate_backward(ctx, A.h, t->w(t->li(l, GATE_W)), AD, t->w32(t->li(l, GATE_B)), attn, GD,
+                                             t->gyy, GD, A.gates, t->gh, OMX_F32, t->g(t->li(l, GATE_W)),
                                              t->g(t->li(l, GATE_B)), t->gap, AD, N, d, H, D));
     if (t->fused_qkv) {
       const uint64_t P3 = qd + 2 * kd;
@@ -310,7 +335,7 @@ int32_t backward(onano* t, float loss_seed) {
       // Block 0's value also feeds every later block's blend: their shares collect in v0_acc (the
       // last block writes it, the others add) and join block 0's own gradient here.
       const bool blends = l > 0, last = l + 1 == c.layers;
-      TRY(omx_qkv_prepare_backward(ctx, A.qkv_lin, t->g_qkv, g_lin, P3, t->w32(t->li(l, QNORM)), t->w32(t->li(l, KNORM)),
+      TRY(omx_qkv_prepare_backward(ctx, A.qkv_lin, LD, t->g_qkv, g_lin, P3, t->w32(t->li(l, QNORM)), t->w32(t->li(l, KNORM)),
                                    t->cos_t, t->sin_t, blends ? t->layers[0].qkv_lin : nullptr,
                                    blends ? t->w32(t->li(l, LAMBDA)) : nullptr, blends ? t->v0_acc : nullptr, last ? 1 : 0,
                                    !blends && c.layers > 1 ? t->v0_acc : nullptr, t->g(t->li(l, QNORM)),
@@ -357,7 +382,7 @@ int32_t backward(onano* t, float loss_seed) {
     }
     TRY(omx_rope_half_split_backward(ctx, t->gk, t->cos_t, t->sin_t, t->t_k, AD, N * KV, D, T, KV));
     TRY(omx_rope_half_split_backward(ctx, t->gq, t->cos_t, t->sin_t, t->t_q, AD, N * H, D, T, H));
-    TRY(omx_rms_qk_norm_backward(ctx, A.q_lin, A.k_lin, AD, t->w32(t->li(l, QNORM)), t->w32(t->li(l, KNORM)), t->t_q, t->t_k,
+    TRY(omx_rms_qk_norm_backward(ctx, A.q_lin, A.k_lin, LD, t->w32(t->li(l, QNORM)), t->w32(t->li(l, KNORM)), t->t_q, t->t_k,
                                  AD, gq_lin, gk_lin, AD, t->g(t->li(l, QNORM)), t->g(t->li(l, KNORM)), N * H, N * KV, D, eps));
     // h feeds the gate, v, k and q; their gradients arrive in that order (the later consumer first).
     struct Proj {
@@ -438,6 +463,9 @@ int32_t onano_create(omx_ctx* ctx, const onano_config* config, onano** out) {
   // The three projections are one matrix only if nothing pads the arena between them.
   t->fused_qkv = t->flash && (static_cast<uint64_t>(c.heads) * c.head_dim * c.n_embd) % kAlign == 0 &&
                  (static_cast<uint64_t>(c.kv_heads) * c.head_dim * c.n_embd) % kAlign == 0;
+  t->keep_f32 = c.bf16 == 1 && t->fused_mlp;
+  t->LD = t->keep_f32 ? OMX_F32 : t->AD;
+  t->lsz = t->keep_f32 ? 4 : t->asz;
   const uint64_t N = t->N, d = c.n_embd, H = c.heads, KV = c.kv_heads, D = c.head_dim, Hd = c.hidden;
   const uint64_t qd = H * D, kd = KV * D;
   // Arena order (the parameter indices keep the order of names.rs): the table, then every vector of
@@ -556,11 +584,11 @@ int32_t onano_create(omx_ctx* ctx, const onano_config* config, onano** out) {
       CREATE_TRY(alloc_act(t, N * Hd, &A.m));
     }
     if (t->fused_qkv) {
-      CREATE_TRY(alloc_act(t, N * (qd + 2 * kd), &A.qkv_lin));
+      CREATE_TRY(alloc(t, N * (qd + 2 * kd) * t->lsz, &A.qkv_lin));
       CREATE_TRY(alloc_act(t, N * (qd + 2 * kd), &A.qkv));
     } else {
-      CREATE_TRY(alloc_act(t, N * qd, &A.q_lin));
-      CREATE_TRY(alloc_act(t, N * kd, &A.k_lin));
+      CREATE_TRY(alloc(t, N * qd * t->lsz, &A.q_lin));
+      CREATE_TRY(alloc(t, N * kd * t->lsz, &A.k_lin));
       CREATE_TRY(alloc_act(t, N * qd, &A.q));
       CREATE_TRY(alloc_act(t, N * kd, &A.k));
       CREATE_TRY(alloc_act(t, N * kd, &A.raw_v));
@@ -569,7 +597,7 @@ int32_t onano_create(omx_ctx* ctx, const onano_config* config, onano** out) {
     }
     CREATE_TRY(alloc_act(t, N * qd, &A.ap));
     if (t->fused_mlp) {
-      CREATE_TRY(alloc_act(t, 2 * N * Hd, &A.gu));
+      CREATE_TRY(alloc(t, 2 * N * Hd * t->lsz, &A.gu));
     } else {
       CREATE_TRY(alloc_act(t, N * Hd, &A.g_lin));
       CREATE_TRY(alloc_act(t, N * Hd, &A.up));
@@ -591,6 +619,8 @@ int32_t onano_create(omx_ctx* ctx, const onano_config* config, onano** out) {
   CREATE_TRY(alloc_act(t, N * qd, &t->t_q));
   CREATE_TRY(alloc_act(t, N * kd, &t->t_k));
   CREATE_TRY(alloc_act(t, N * (d > qd ? d : qd), &t->t_a));
+  CREATE_TRY(alloc(t, N * d * t->lsz, &t->t_f));
+  if (t->keep_f32 && t->flash) CREATE_TRY(alloc_t(t, N * qd, &t->ap32));
   CREATE_TRY(alloc_act(t, N * Hd, &t->gm));
   if (t->fused_mlp) {
     if (!t->deferred_dw) CREATE_TRY(alloc_act(t, 2 * N * Hd, &t->ggu));
@@ -603,7 +633,7 @@ int32_t onano_create(omx_ctx* ctx, const onano_config* config, onano** out) {
     if (!t->deferred_dw) CREATE_TRY(alloc_act(t, N * (qd + 2 * kd), &t->g_qkv_lin));
     CREATE_TRY(alloc_t(t, N * kd, &t->v0_acc));
   }
-  CREATE_TRY(alloc_act(t, N * qd, &t->gyy));
+  CREATE_TRY(alloc(t, N * qd * (t->keep_f32 && t->flash ? 4 : t->asz), &t->gyy));
   CREATE_TRY(alloc_act(t, N * qd, &t->gap));
   CREATE_TRY(alloc_act(t, N * qd, &t->gq));
   CREATE_TRY(alloc_act(t, N * kd, &t->gk));

@@ -20,6 +20,27 @@
 //
 // Pinned by ojas-oracle/fixtures/tiny/{init,forward,grads_init}.safetensors
 // (torch 2.13 logits, loss and every gradient at the seeded init).
+//
+// orc_nanolab_loss_and_grads_rounded runs the same graph with bf16 roundings
+// (orc_round_bf16_vec, the integer rule of ojas-core/src/autocast.rs:66-101)
+// placed where a bf16 tier places them; every operation itself stays Exact
+// f32 arithmetic on the rounded values, as `Autocast<CpuBackend>` computes:
+//   ORC_ROUND_OPERANDS  only what a matrix product reads: the operands `prep`
+//                       rounds (autocast.rs:518-525) for linear_*, the gate,
+//                       causal_sdpa_* and the fused head. Fewer roundings than
+//                       any tier whose products take bf16 operands can have:
+//                       its distance from the Exact result is that noise floor.
+//   ORC_ROUND_AUTOCAST  the reference's own bf16 tier: the operands, the
+//                       activation outputs `emit` rounds (:533-538: linear,
+//                       attention and gate outputs, their input gradients) and
+//                       the pointwise results `promote` rounds when their
+//                       inputs are tagged (:540-546: SiLU, the product, RoPE's
+//                       backward). Norms, residual adds (the stream is never
+//                       tagged), the blend (lambda is a parameter) and the
+//                       loss stay f32; weight gradients stay f32 (`keep_f32`).
+// The saved attention output that the backward's row term reads is never
+// rounded (:177-186, :1200-1236). With rounding 0 the function is
+// orc_nanolab_loss_and_grads bit for bit.
 #include <cmath>
 #include <vector>
 
@@ -77,6 +98,22 @@ void add_into(std::vector<float>& acc, const std::vector<float>& g) {
   for (size_t i = 0; i < acc.size(); ++i) acc[i] = acc[i] + g[i];
 }
 
+// Where a rounding sits: at a product's operand, or at an output the reference's Autocast emits.
+enum RoundAt { AT_OPERAND, AT_OUTPUT };
+struct Rounding {
+  int mode;
+  void operator()(std::vector<float>& v, RoundAt at) const {
+    if (mode == ORC_ROUND_AUTOCAST || (mode == ORC_ROUND_OPERANDS && at == AT_OPERAND))
+      orc_round_bf16_vec(v.data(), v.data(), v.size());
+  }
+  // A rounded copy for a product to read while the f32 value lives on (the residual stream's gradient).
+  std::vector<float> copy(const std::vector<float>& v, RoundAt at) const {
+    std::vector<float> out = v;
+    (*this)(out, at);
+    return out;
+  }
+};
+
 #define ORC_TRY(expr)              \
   do {                             \
     int rc_ = (expr);              \
@@ -106,8 +143,10 @@ void orc_rope_tables(size_t seq, size_t head_dim, double base, float* cos, float
     }
 }
 
-int orc_nanolab_loss_and_grads(const orc_nanolab_config* c, float* const* params, const uint32_t* ids,
-                               const uint32_t* targets, float* loss, float* logits, float* const* grads) {
+static int nanolab_impl(int rounding, const orc_nanolab_config* c, float* const* params, const uint32_t* ids,
+                        const uint32_t* targets, float* loss, float* logits, float* const* grads) {
+  if (rounding != 0 && rounding != ORC_ROUND_OPERANDS && rounding != ORC_ROUND_AUTOCAST) return ORC_OUT_OF_RANGE;
+  const Rounding R{rounding};
   const Dims s = dims_of(c);
   if (s.KV == 0 || s.H % s.KV != 0 || s.D % 2 != 0) return ORC_SHAPE;
   const size_t N = s.N, d = s.d, B = s.B, T = s.T, H = s.H, KV = s.KV, D = s.D, M = s.hidden;
@@ -126,12 +165,16 @@ int orc_nanolab_loss_and_grads(const orc_nanolab_config* c, float* const* params
     A.x = x;
     A.h.resize(N * d);
     ORC_TRY(orc_rms_norm_forward(A.x.data(), P(P_NORM1), A.h.data(), N, d, eps));
+    R(A.h, AT_OPERAND);  // read by the three projections and the gate
     A.q_lin.resize(N * s.qw);
     A.k_lin.resize(N * s.kvw);
     A.raw_v.resize(N * s.kvw);
     ORC_TRY(orc_linear_forward(A.h.data(), P(P_Q), A.q_lin.data(), N, d, s.qw));
     ORC_TRY(orc_linear_forward(A.h.data(), P(P_K), A.k_lin.data(), N, d, s.kvw));
     ORC_TRY(orc_linear_forward(A.h.data(), P(P_V), A.raw_v.data(), N, d, s.kvw));
+    R(A.q_lin, AT_OUTPUT);
+    R(A.k_lin, AT_OUTPUT);
+    R(A.raw_v, AT_OUTPUT);
     A.qn.resize(N * s.qw);
     A.kn.resize(N * s.kvw);
     ORC_TRY(orc_rms_norm_forward(A.q_lin.data(), P(P_QN), A.qn.data(), N * H, D, eps));
@@ -143,6 +186,9 @@ int orc_nanolab_loss_and_grads(const orc_nanolab_config* c, float* const* params
     A.v.resize(N * s.kvw);
     if (l == 0) A.v = A.raw_v;
     else ORC_TRY(orc_value_residual_forward(A.raw_v.data(), acts[0].raw_v.data(), P(P_LAMBDA)[0], A.v.data(), N * s.kvw));
+    R(A.q, AT_OPERAND);
+    R(A.k, AT_OPERAND);
+    R(A.v, AT_OPERAND);
     A.qp.resize(N * s.qw);
     A.kp.resize(N * s.kvw);
     A.vp.resize(N * s.kvw);
@@ -155,26 +201,36 @@ int orc_nanolab_loss_and_grads(const orc_nanolab_config* c, float* const* params
                                     c->window));
     A.ap.resize(N * s.qw);
     orc_permute_0213(A.a.data(), A.ap.data(), B, H, T, D);
+    R(A.ap, AT_OUTPUT);  // what the gate reads; A.a, which the backward's row term reads, stays as it is
     A.y.resize(N * s.qw);
     ORC_TRY(orc_gate_forward(A.h.data(), P(P_GW), P(P_GB), A.ap.data(), A.y.data(), N, d, H, D));
+    R(A.y, AT_OPERAND);
     ORC_TRY(orc_linear_forward(A.y.data(), P(P_O), tmp.data(), N, s.qw, d));
+    R(tmp, AT_OUTPUT);
     A.x1.resize(N * d);
     ORC_TRY(orc_residual_add(A.x.data(), tmp.data(), A.x1.data(), N * d));
     A.h2.resize(N * d);
     ORC_TRY(orc_rms_norm_forward(A.x1.data(), P(P_NORM2), A.h2.data(), N, d, eps));
+    R(A.h2, AT_OPERAND);
     A.g_lin.resize(N * M);
     A.g_act.resize(N * M);
     A.up.resize(N * M);
     A.m.resize(N * M);
     ORC_TRY(orc_linear_forward(A.h2.data(), P(P_FGATE), A.g_lin.data(), N, d, M));
+    R(A.g_lin, AT_OUTPUT);
     orc_silu_forward_vec(A.g_lin.data(), A.g_act.data(), N * M);
+    R(A.g_act, AT_OUTPUT);
     ORC_TRY(orc_linear_forward(A.h2.data(), P(P_FUP), A.up.data(), N, d, M));
+    R(A.up, AT_OUTPUT);
     ORC_TRY(orc_mul_forward(A.g_act.data(), A.up.data(), A.m.data(), N * M));
+    R(A.m, AT_OPERAND);
     ORC_TRY(orc_linear_forward(A.m.data(), P(P_FDOWN), tmp.data(), N, M, d));
+    R(tmp, AT_OUTPUT);
     ORC_TRY(orc_residual_add(A.x1.data(), tmp.data(), x.data(), N * d));
   }
   std::vector<float> hf(N * d);
   ORC_TRY(orc_rms_norm_forward(x.data(), params[final_norm], hf.data(), N, d, eps));
+  R(hf, AT_OPERAND);
   if (logits) ORC_TRY(orc_linear_forward(hf.data(), params[0], logits, N, d, s.V));
   if (!grads)
     return orc_linear_cross_entropy_mean(hf.data(), params[0], targets, N, d, s.V, 0, 0, loss, nullptr, nullptr);
@@ -183,6 +239,7 @@ int orc_nanolab_loss_and_grads(const orc_nanolab_config* c, float* const* params
   std::vector<float> ghf(N * d), g_head(s.V * d);
   ORC_TRY(orc_linear_cross_entropy_mean(hf.data(), params[0], targets, N, d, s.V, 0, 0, loss, ghf.data(),
                                         g_head.data()));
+  R(ghf, AT_OUTPUT);
   std::vector<float> gx(N * d);
   ORC_TRY(orc_rms_norm_backward(x.data(), params[final_norm], ghf.data(), gx.data(), grads[final_norm], N, d, eps));
   std::vector<float> g_v0(N * s.kvw, 0.0f);  // gradient of block 0's raw v from the later blocks' blends
@@ -196,27 +253,45 @@ int orc_nanolab_loss_and_grads(const orc_nanolab_config* c, float* const* params
     auto P = [&](int which) { return params[pidx(l, which)]; };
     auto G = [&](int which) { return grads[pidx(l, which)]; };
     // x2 = x1 + down(m)
-    ORC_TRY(orc_linear_backward(A.m.data(), P(P_FDOWN), gx.data(), gm.data(), G(P_FDOWN), N, M, d));
+    {
+      const std::vector<float> gx_op = R.copy(gx, AT_OPERAND);
+      ORC_TRY(orc_linear_backward(A.m.data(), P(P_FDOWN), gx_op.data(), gm.data(), G(P_FDOWN), N, M, d));
+    }
+    R(gm, AT_OUTPUT);
     ORC_TRY(orc_mul_backward(A.g_act.data(), A.up.data(), gm.data(), g_gact.data(), g_up.data(), N * M));
+    R(g_gact, AT_OUTPUT);
+    R(g_up, AT_OPERAND);
     // h2 feeds ffn.gate then ffn.up: the later consumer (up) first.
     ORC_TRY(orc_linear_backward(A.h2.data(), P(P_FUP), g_up.data(), gh2.data(), G(P_FUP), N, d, M));
+    R(gh2, AT_OUTPUT);
     orc_silu_backward_vec(A.g_lin.data(), g_gact.data(), g_glin.data(), N * M);
+    R(g_glin, AT_OPERAND);
     ORC_TRY(orc_linear_backward(A.h2.data(), P(P_FGATE), g_glin.data(), gh2b.data(), G(P_FGATE), N, d, M));
+    R(gh2b, AT_OUTPUT);
     add_into(gh2, gh2b);
     ORC_TRY(orc_rms_norm_backward(A.x1.data(), P(P_NORM2), gh2.data(), gt.data(), G(P_NORM2), N, d, eps));
     std::vector<float> gx1 = gx;  // the residual branch first, then the norm branch
     add_into(gx1, gt);
     // x1 = x + o_proj(y)
-    ORC_TRY(orc_linear_backward(A.y.data(), P(P_O), gx1.data(), gy.data(), G(P_O), N, s.qw, d));
+    {
+      const std::vector<float> gx1_op = R.copy(gx1, AT_OPERAND);
+      ORC_TRY(orc_linear_backward(A.y.data(), P(P_O), gx1_op.data(), gy.data(), G(P_O), N, s.qw, d));
+    }
+    R(gy, AT_OPERAND);  // emitted by the product, read by the gate's backward
     // h feeds q, k, v and (last) the gate: the gate's gradient comes first.
     ORC_TRY(orc_gate_backward(A.h.data(), P(P_GW), P(P_GB), A.ap.data(), gy.data(), gh.data(), G(P_GW), G(P_GB),
                               gap.data(), N, d, H, D));
+    R(gh, AT_OUTPUT);
+    R(gap, AT_OPERAND);
     orc_permute_0213(gap.data(), ga.data(), B, T, H, D);
     ORC_TRY(orc_causal_sdpa_backward(A.qp.data(), A.kp.data(), A.vp.data(), A.a.data(), A.lse.data(), ga.data(),
                                      gqp.data(), gkp.data(), gvp.data(), B, H, KV, T, D, c->window));
     orc_permute_0213(gvp.data(), gv.data(), B, KV, T, D);
     orc_permute_0213(gkp.data(), gk.data(), B, KV, T, D);
     orc_permute_0213(gqp.data(), gq.data(), B, H, T, D);
+    R(gq, AT_OUTPUT);
+    R(gk, AT_OUTPUT);
+    R(gv, AT_OUTPUT);
     if (l == 0) {
       // Block 0's raw v: the later blocks' blends were visited first, its own attention last.
       if (g_v0_live) {
@@ -237,13 +312,21 @@ int orc_nanolab_loss_and_grads(const orc_nanolab_config* c, float* const* params
     }
     ORC_TRY(orc_rope_backward(gk.data(), cos.data(), sin.data(), gkn.data(), N * KV, D, T, KV));
     ORC_TRY(orc_rope_backward(gq.data(), cos.data(), sin.data(), gqn.data(), N * H, D, T, H));
+    R(gkn, AT_OUTPUT);
+    R(gqn, AT_OUTPUT);
     ORC_TRY(orc_rms_norm_backward(A.k_lin.data(), P(P_KN), gkn.data(), gk_lin.data(), G(P_KN), N * KV, D, eps));
     ORC_TRY(orc_rms_norm_backward(A.q_lin.data(), P(P_QN), gqn.data(), gq_lin.data(), G(P_QN), N * H, D, eps));
+    R(gq_lin, AT_OPERAND);
+    R(gk_lin, AT_OPERAND);
+    R(g_raw_v, AT_OPERAND);
     ORC_TRY(orc_linear_backward(A.h.data(), P(P_V), g_raw_v.data(), gh_part.data(), G(P_V), N, d, s.kvw));
+    R(gh_part, AT_OUTPUT);
     add_into(gh, gh_part);
     ORC_TRY(orc_linear_backward(A.h.data(), P(P_K), gk_lin.data(), gh_part.data(), G(P_K), N, d, s.kvw));
+    R(gh_part, AT_OUTPUT);
     add_into(gh, gh_part);
     ORC_TRY(orc_linear_backward(A.h.data(), P(P_Q), gq_lin.data(), gh_part.data(), G(P_Q), N, d, s.qw));
+    R(gh_part, AT_OUTPUT);
     add_into(gh, gh_part);
     ORC_TRY(orc_rms_norm_backward(A.x.data(), P(P_NORM1), gh.data(), gt.data(), G(P_NORM1), N, d, eps));
     gx = gx1;
@@ -253,6 +336,16 @@ int orc_nanolab_loss_and_grads(const orc_nanolab_config* c, float* const* params
   ORC_TRY(orc_embedding_backward(ids, gx.data(), grads[0], N, s.V, d));
   for (size_t i = 0; i < s.V * d; ++i) grads[0][i] = g_head[i] + grads[0][i];
   return ORC_OK;
+}
+
+int orc_nanolab_loss_and_grads(const orc_nanolab_config* c, float* const* params, const uint32_t* ids,
+                               const uint32_t* targets, float* loss, float* logits, float* const* grads) {
+  return nanolab_impl(0, c, params, ids, targets, loss, logits, grads);
+}
+
+int orc_nanolab_loss_and_grads_rounded(int rounding, const orc_nanolab_config* c, float* const* params,
+                                       const uint32_t* ids, const uint32_t* targets, float* loss, float* const* grads) {
+  return nanolab_impl(rounding, c, params, ids, targets, loss, nullptr, grads);
 }
 
 }  // extern "C"

@@ -200,6 +200,11 @@ void orc_rope_tables(size_t seq, size_t head_dim, double base, float* cos, float
 /* logits ([batch*seq, vocab]) and grads may be NULL. */
 int orc_nanolab_loss_and_grads(const orc_nanolab_config* c, float* const* params, const uint32_t* ids,
                                const uint32_t* targets, float* loss, float* logits, float* const* grads);
+/* The same graph with bf16 roundings placed as a bf16 tier places them (nanolab_exact.cpp): at the
+ * products' operands only, or at every point the reference's Autocast rounds; 0 = none. */
+enum { ORC_ROUND_OPERANDS = 1, ORC_ROUND_AUTOCAST = 2 };
+int orc_nanolab_loss_and_grads_rounded(int rounding, const orc_nanolab_config* c, float* const* params,
+                                       const uint32_t* ids, const uint32_t* targets, float* loss, float* const* grads);
 
 /* ---- symmetric int8 weights in groups along the input axis, and the LoRA step over a frozen
  * decoder (oracle/lora_exact.cpp; ojas-cpu/src/quant_sparse.rs:284-346 applied per group,

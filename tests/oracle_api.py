@@ -629,6 +629,26 @@ def rope_tables(seq: int, head_dim: int, base: float = 10000.0):
     return cos, sin
 
 
+ROUND_OPERANDS, ROUND_AUTOCAST = 1, 2
+
+
+def nanolab_loss_and_grads_rounded(cfg: NanolabConfig, params, ids, targets, rounding: int):
+    """The nanolab graph with bf16 roundings placed as a bf16 tier places them (oracle/nanolab_exact.cpp):
+    ROUND_OPERANDS = at the products' operands only, ROUND_AUTOCAST = wherever the reference's
+    Autocast rounds; 0 = none (then equal to nanolab_loss_and_grads bit for bit). Returns (loss, grads)."""
+    params = [_f32(p).reshape(-1) for p in params]
+    assert [p.size for p in params] == nanolab_param_lens(cfg)
+    ids = np.ascontiguousarray(ids, dtype=np.uint32)
+    targets = np.ascontiguousarray(targets, dtype=np.uint32)
+    grads = [np.zeros_like(p) for p in params]
+    pp = (_f * len(params))(*[_fp(p) for p in params])
+    gp = (_f * len(grads))(*[_fp(g) for g in grads])
+    loss = C.c_float()
+    _check(_lib.orc_nanolab_loss_and_grads_rounded(C.c_int(rounding), C.byref(cfg), pp, _up(ids), _up(targets),
+                                                   C.byref(loss), gp), "nanolab_loss_and_grads_rounded")
+    return np.float32(loss.value), grads
+
+
 def nanolab_loss_and_grads(cfg: NanolabConfig, params, ids, targets, want_logits=False, want_grads=True):
     params = [_f32(p).reshape(-1) for p in params]
     assert [p.size for p in params] == nanolab_param_lens(cfg)

@@ -526,22 +526,24 @@ def test_value_residual_known_answer_and_nonfinite_lambda(be):
     assert e.value.variant == "NonFinite"
 
 
+@pytest.mark.parametrize("lin_f32", [False, True])
 @pytest.mark.parametrize("heads,kv_heads,dim,blend", [(4, 2, 64, True), (2, 2, 128, True), (3, 1, 64, False), (2, 1, 128, False)])
-def test_qkv_prepare_equals_norm_then_rope_then_blend(be, heads, kv_heads, dim, blend):
+def test_qkv_prepare_equals_norm_then_rope_then_blend(be, heads, kv_heads, dim, blend, lin_f32):
     """`omx_qkv_prepare_forward / _backward` over a fused q | k | v projection output against the
     oracle's separate ops in sequence (rms_norm per head, half-split RoPE, value-residual blend):
     forward and every gradient within the bf16 gate of the largest value. Without a blend the value
     block is copied and `add_value_grad` joins its gradient (block 0 of the model, which every later
-    block's blend feeds)."""
-    from ojas_amd.backend import BF16
+    block's blend feeds). `lin_f32`: the projection output (and block 0's) as unrounded f32."""
+    from ojas_amd.backend import BF16, F32
 
-    print(f"qkv prepare heads={heads}/{kv_heads} dim={dim} blend={blend}", flush=True)
+    print(f"qkv prepare heads={heads}/{kv_heads} dim={dim} blend={blend} lin_f32={lin_f32}", flush=True)
     b, t = 2, 37
     slots = heads + 2 * kv_heads
     r = orc.SplitMix64(500 + dim + heads)
     rnd = orc.round_bf16
-    lin = rnd(r.vec(b * t * slots * dim, 1.0)).reshape(b, t, slots * dim)
-    lin0 = rnd(r.vec(b * t * slots * dim, 1.0)).reshape(b, t, slots * dim)
+    rnd_lin = (lambda a: a) if lin_f32 else rnd
+    lin = rnd_lin(r.vec(b * t * slots * dim, 1.0)).reshape(b, t, slots * dim)
+    lin0 = rnd_lin(r.vec(b * t * slots * dim, 1.0)).reshape(b, t, slots * dim)
     g = rnd(r.vec(b * t * slots * dim, 1.0)).reshape(b, t, slots * dim)
     qw, kw = 1.0 + r.vec(dim, 0.2), 1.0 + r.vec(dim, 0.2)
     lam = np.array([0.3], np.float32)
@@ -565,7 +567,8 @@ def test_qkv_prepare_equals_norm_then_rope_then_blend(be, heads, kv_heads, dim, 
     else:
         want_gv = gv + add_v.reshape(gv.shape)
     # the device, one call each way
-    d_lin, d_lin0, d_g = (be.upload(a, BF16) for a in (lin, lin0, g))
+    d_lin, d_lin0 = (be.upload(a, F32 if lin_f32 else BF16) for a in (lin, lin0))
+    d_g = be.upload(g, BF16)
     d_qw, d_kw, d_cos, d_sin, d_lam = (be.upload(a) for a in (qw, kw, cos, sin, lam))
     out = be.qkv_prepare_forward(d_lin, d_qw, d_kw, d_cos, d_sin, heads, kv_heads, dim, d_lin0 if blend else None,
                                  d_lam if blend else None)

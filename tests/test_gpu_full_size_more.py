@@ -184,17 +184,11 @@ def test_lora_full_width_two_blocks_match_the_oracle(be):
     normwise = [float(np.linalg.norm(g - og) / np.linalg.norm(og)) for g, og in zip(grads, ograds)]
     print("  worst element / largest:", " ".join(f"{e:.4f}" for e in elementwise), flush=True)
     print("  normwise:", " ".join(f"{e:.4f}" for e in normwise), flush=True)
-    # The stated gate (2e-2 of the tensor's largest value) holds on 14 of the 16 adapters, at 0.9e-2
-    # to 1.6e-2, and the worst of the last block's query and key adapters measure 2.0e-2 and 2.2e-2
-    # (2.1e-2 normwise). The step keeps activations and their gradients in bf16 where the reference
-    # keeps f32 between operations, about 1e-2 by the time the backward pass reaches the last block's
-    # attention; dS = P (dO . (V - out)) there sees only the part of dO inside the span of the value
-    # rows' differences, and after one block the value rows share a large common component, so the
-    # same absolute error is a larger share of dQ and dK than of dV. The attention kernels on their
-    # own stay at 2.4e-3 on such inputs (test_gpu_parity_ops.py). Gate: 2.5e-2, stated here.
-    assert max(elementwise) <= 2.5e-2, elementwise
-    assert max(normwise) <= 2.5e-2, normwise
-    assert sorted(elementwise)[-3] <= 2e-2 and sorted(normwise)[-5] <= 2e-2
+    # 2e-2 of each tensor's largest value per element, and normwise (measured at most 1.9e-2 on the
+    # last block's query and key adapters and 0.9e-2 to 1.6e-2 elsewhere): the forward's product
+    # outputs stay f32, so every activation is rounded to bf16 once.
+    assert max(elementwise) <= 2e-2, elementwise
+    assert max(normwise) <= 2e-2, normwise
 
 
 @pytest.mark.parametrize("kin,nout", [(2048, 6144), (2048, 16384), (8192, 2048)])
@@ -271,70 +265,128 @@ def test_lora_step_at_full_size(be):
 
 
 # ------------------------------------------------------------------ the nanolab graph at the 124M size
+def _nanolab_124m_params(spec, rng, bf16_exact=True):
+    """N(0, 0.02) matrices and table (bf16-exact by default: both tiers then multiply the same
+    weights), norm weights one, a gate that is not flat and value residuals that are not at their
+    start."""
+    params = {}
+    for name, shape in spec.param_shapes().items():
+        if len(shape) == 2:
+            w = rng.normal(0, 0.02, shape).astype(np.float32)
+            params[name] = orc.round_bf16(w) if bf16_exact else w
+        elif name.endswith("vr_lambda"):
+            params[name] = rng.uniform(0.2, 0.8, shape).astype(np.float32)
+        elif name.endswith("gate.bias"):
+            params[name] = rng.normal(0, 0.5, shape).astype(np.float32)
+        else:
+            params[name] = np.ones(shape, np.float32)
+    return params
+
+
+def _matrix_distances(got, want, shapes):
+    """(worst normwise, worst element / largest) over the matrices and the table."""
+    normwise = elementwise = 0.0
+    for name, ref in want.items():
+        if len(shapes[name]) != 2:
+            continue
+        ref = ref.reshape(-1).astype(np.float64)
+        diff = got[name].reshape(-1).astype(np.float64) - ref
+        normwise = max(normwise, float(np.linalg.norm(diff) / np.linalg.norm(ref)))
+        elementwise = max(elementwise, float(np.max(np.abs(diff)) / np.max(np.abs(ref))))
+    return normwise, elementwise
+
+
+def test_nanolab_124m_against_the_oracle_at_full_depth_and_width(be):
+    """`ModelSpec::nanolab_124m` (ojas-model/src/spec.rs:74-91: 12 blocks, 768 wide, 12 heads of 64,
+    SwiGLU 2048, vocabulary 50304) on one 256-token sequence, which the oracle finishes in seconds.
+    f32 tier: loss 1e-5 relative, every gradient 1e-4 normwise (the reference's gate for a device,
+    ojas-oracle/src/parity.rs:28-40). bf16 tier: loss 1e-3 relative. Its gradients cannot be inside
+    2e-2 at this depth: the oracle's own Exact arithmetic with nothing but the products' operands
+    rounded to bf16 (`ROUND_OPERANDS`, the least rounding a tier with bf16 products can do) is
+    about 3e-2 from its unrounded self here, normwise and per element (1e-2 per sqrt(block),
+    tests/test_oracle_bf16_floor.py), and the reference's own rounding points (`ROUND_AUTOCAST`) 4e-2.
+    The device's tier is held to that floor: within 1.25 x of it, and below the reference's tier."""
+    from ojas_amd.nanolab import NativeNanolabTrainer, spec_nanolab_124m
+    from test_gpu_nanolab_native import oracle_step
+
+    spec = spec_nanolab_124m()
+    shapes = spec.param_shapes()
+    rng = np.random.default_rng(77)
+    params = _nanolab_124m_params(spec, rng)
+    window = rng.integers(0, spec.vocab, (1, 257)).astype(np.uint32)
+    ids, targets = np.ascontiguousarray(window[:, :-1]), np.ascontiguousarray(window[:, 1:])
+    print("nanolab 124M, 1 x 256 tokens: oracle (exact, operands-only, autocast points)", flush=True)
+    orc.set_threads(16)
+    o_loss, exact = oracle_step(spec, params, ids, targets, 1, 256)
+    _, floor = oracle_step(spec, params, ids, targets, 1, 256, rounding=orc.ROUND_OPERANDS)
+    _, autocast = oracle_step(spec, params, ids, targets, 1, 256, rounding=orc.ROUND_AUTOCAST)
+    floor_n, floor_e = _matrix_distances(floor, exact, shapes)
+    auto_n, auto_e = _matrix_distances(autocast, exact, shapes)
+    print(f"  oracle operands-only: {floor_n:.4f} normwise, {floor_e:.4f} per element; autocast points: {auto_n:.4f}, {auto_e:.4f}",
+          flush=True)
+    assert 2e-2 < floor_n < auto_n < 6e-2
+    for bf16 in (False, True):
+        tr = NativeNanolabTrainer(be, spec, 1, 256, params, bf16=bf16)
+        try:
+            loss, grads = tr.loss_and_grads(ids, targets)
+        finally:
+            tr.close()
+        normwise, elementwise = _matrix_distances(grads, exact, shapes)
+        print(f"  device bf16={bf16}: loss {loss:.6f} (oracle {o_loss:.6f}), matrices {normwise:.2e} normwise, "
+              f"{elementwise:.2e} per element", flush=True)
+        if not bf16:
+            assert abs(loss - o_loss) <= 1e-5 * abs(o_loss)
+            for name, ref in exact.items():
+                if np.any(ref):
+                    got = grads[name].astype(np.float64)
+                    assert np.linalg.norm(got - ref.reshape(-1)) <= 1e-4 * np.linalg.norm(ref), name
+            continue
+        assert abs(loss - o_loss) <= 1e-3 * abs(o_loss)
+        assert normwise <= 1.25 * floor_n and elementwise <= 1.25 * floor_e, (normwise, floor_n, elementwise, floor_e)
+        assert normwise < auto_n
+
+
 def test_nanolab_124m_step_at_full_size(be):
     """The native nanolab driver at `ModelSpec::nanolab_124m` (ojas-model/src/spec.rs:74-91), 16 x 1024
     tokens, bf16 tier: the paths only this size takes (MFMA attention on the fused q | k | v output,
     the weight gradients as strided batches after the backward, one AdamW pass over the table and
-    the vectors). The f32 tier, which the oracle pins at small sizes, gives the same gradients at
-    4 x 1024 tokens; the gradient predicts the change of the loss along itself; two half-weighted
-    micro-batches add up to the whole one; six hybrid steps on one batch lower the loss."""
+    the vectors). The two tiers agree on the loss and, at 4 x 1024 tokens, on every matrix gradient
+    as closely as 12 blocks of bf16 operands allow (the test above measures that floor against
+    the oracle: about 3e-2; the gate here is 4e-2 normwise); the gradient predicts the change of the
+    loss along itself; two half-weighted micro-batches add up to the whole one; six hybrid steps on
+    one batch lower the loss."""
     from ojas_amd.nanolab import NativeNanolabTrainer, spec_nanolab_124m
 
     spec = spec_nanolab_124m()
     rng = np.random.default_rng(31)
     print("nanolab 124M: tiers at 4 x 1024", flush=True)
     small = rng.integers(0, spec.vocab, (4, 1025)).astype(np.uint32)
+    params = _nanolab_124m_params(spec, rng)
     tier = {}
-    params = None
     for bf16 in (True, False):
-        tr = NativeNanolabTrainer(be, spec, 4, 1024, bf16=bf16)
+        tr = NativeNanolabTrainer(be, spec, 4, 1024, params, bf16=bf16)
         try:
-            if params is None:
-                tr.init(17)
-                params = tr.download_params()
-                # a gate that is not flat and value residuals that are not at their start
-                for name in params:
-                    if name.endswith("vr_lambda"):
-                        params[name] = rng.uniform(0.2, 0.8, params[name].shape).astype(np.float32)
-                    if name.endswith("gate.bias"):
-                        params[name] = rng.normal(0, 0.5, params[name].shape).astype(np.float32)
-            tr.set_params(params)
             tier[bf16] = tr.loss_and_grads(small[:, :-1], small[:, 1:])
         finally:
             tr.close()
     (loss16, g16), (loss32, g32) = tier[True], tier[False]
     print(f"loss bf16 {loss16:.5f} f32 {loss32:.5f}", flush=True)
     assert abs(loss32 - np.log(spec.vocab)) < 1.0 and abs(loss16 - loss32) <= 1e-3 * abs(loss32)
-    table = []
-    for name, want in g32.items():
-        if name == "blocks.0.mixer.vr_lambda":
-            assert not np.any(want) and not np.any(g16[name])  # block 0 blends with itself: no gradient
-            continue
-        scale = float(np.linalg.norm(want.astype(np.float64)))
-        assert scale > 0, name
-        diff = g16[name].astype(np.float64) - want
-        table.append((float(np.linalg.norm(diff)) / scale, float(np.max(np.abs(diff)) / np.max(np.abs(want))), name,
-                      want.size))
-    table.sort(reverse=True)
-    for row in table[:6]:
-        print("tier distance (normwise, worst element / largest, name, size)", row, flush=True)
-    # Every bf16 rounding of a block (ten stored activations each way) adds its share in quadrature:
-    # measured at this width the distance of every matrix gradient, first block or last, is about
-    # 0.9e-2 x sqrt(blocks) (1 block 0.7-1.1e-2, 2: 1.1-2.0, 4: 1.7-2.8, 8: 2.4-4.0, 12: 2.8-4.9,
-    # the q and k projections at the top of each range: their path runs through the softmax at
-    # scores of order one, which QK-norm gives from the first step). At 12 blocks: matrices at most
-    # 4.9e-2 normwise, the 64-element QK-norm weights 5.7e-2. A lambda's gradient is one number, a
-    # sum over every value element with both signs; one of them alone reads 6e-2 to 1.8e-1 from run
-    # to run of the kernels' summation orders, so the eleven are held as one vector.
-    for normwise, _, name, size in table:
-        if size > 1:
-            assert normwise <= (6e-2 if size >= spec.n_embd * spec.n_head else 8e-2), (name, normwise)
+    assert not np.any(g32["blocks.0.mixer.vr_lambda"]) and not np.any(g16["blocks.0.mixer.vr_lambda"])
+    normwise, elementwise = _matrix_distances(g16, g32, spec.param_shapes())
+    print(f"tier distance over the matrices: {normwise:.4f} normwise, {elementwise:.4f} per element", flush=True)
+    assert normwise <= 4e-2, normwise
     lam = [n for n in g32 if n.endswith("vr_lambda") and n != "blocks.0.mixer.vr_lambda"]
     want = np.array([g32[n][0] for n in lam], np.float64)
     got = np.array([g16[n][0] for n in lam], np.float64)
+    # A lambda's gradient is one number, a sum over every value element with both signs: the eleven
+    # are held as one vector.
     print("lambda gradients: distance", float(np.linalg.norm(got - want) / np.linalg.norm(want)), flush=True)
     assert np.linalg.norm(got - want) <= 8e-2 * np.linalg.norm(want), (got, want)
     print("nanolab 124M: 16 x 1024", flush=True)
+    # Weights between bf16 values from here on: a step along the gradient is far smaller than the
+    # spacing of bf16 numbers, and from bf16-exact weights the tier's operand copies would not move.
+    params = _nanolab_124m_params(spec, rng, bf16_exact=False)
     window = rng.integers(0, spec.vocab, (16, 1025)).astype(np.uint32)
     ids, targets = window[:, :-1], window[:, 1:]
     tr = NativeNanolabTrainer(be, spec, 16, 1024, bf16=True, adam_lr=1e-3, matrix_lr=0.02)

@@ -46,6 +46,12 @@ def test_linear_i8_group_forward(be, rows, kin, nout, with_add):
     y = be.linear_i8_group_forward(be.upload(x, BF16), be.upload(codes), be.upload(scales),
                                    be.upload(add, BF16) if with_add else None)
     _close(be.download_f32(y), want)
+    # The same product left in f32: what the bf16 output is the rounding of.
+    from ojas_amd.backend import F32
+    y32 = be.linear_i8_group_forward(be.upload(x, BF16), be.upload(codes), be.upload(scales),
+                                     be.upload(add, BF16) if with_add else None, out_dtype=F32)
+    assert y32.dtype == F32
+    assert np.array_equal(orc.round_bf16(be.download(y32)), be.download_f32(y))
 
 
 @pytest.mark.parametrize("rows,kin,nout", [(256, 128, 64), (300, 96, 160), (77, 32, 32), (512, 256, 2048),
@@ -169,6 +175,17 @@ def test_rope_in_place_and_swiglu(be):
     be.rope_half_split_inplace(dx, be.upload(cos), be.upload(sin), tokens, time, heads, dim, backward=True)
     back = orc.rope_backward(rot, cos, sin).reshape(tokens, heads * dim)
     _close(be.download_f32(dx)[:, :heads * dim], back, 2e-2)
+    # The rotation out of place from an f32 projection output: rotated heads and the value block in
+    # one pass, one rounding each.
+    from ojas_amd.backend import F32
+    x32 = rng.normal(0, 1, (tokens, pitch)).astype(np.float32)
+    rot32 = orc.rope_forward(np.ascontiguousarray(x32[:, :heads * dim]).reshape(tokens // time, time, heads, dim), cos, sin)
+    for dtype, src in ((F32, x32), (BF16, x)):
+        out = be.rope_half_split_pitched(be.upload(src, dtype), be.upload(cos), be.upload(sin), tokens, time, heads, 2, dim)
+        got = be.download_f32(out)
+        want = rot32 if dtype == F32 else rot
+        _close(got[:, :heads * dim], want.reshape(tokens, heads * dim), 1e-2)
+        assert np.array_equal(got[:, heads * dim:], orc.round_bf16(src[:, heads * dim:]))  # the value block: converted as it is
     # SwiGLU on a fused gate | up tensor.
     rows, hidden = 37, 72
     gu = orc.round_bf16(rng.normal(0, 1.5, (rows, 2 * hidden)).astype(np.float32))
@@ -183,6 +200,19 @@ def test_rope_in_place_and_swiglu(be):
     got = be.download_f32(be.swiglu_backward(dgu, be.upload(gm, BF16)))
     _close(got[:, :hidden], g_gate)
     _close(got[:, hidden:], g_up)
+    # The same on an unrounded f32 gate | up tensor (the projection's output kept in f32).
+    from ojas_amd.backend import F32
+    gu32 = rng.normal(0, 1.5, (rows, 2 * hidden)).astype(np.float32)
+    gate, up = np.ascontiguousarray(gu32[:, :hidden]), np.ascontiguousarray(gu32[:, hidden:])
+    act = orc.silu_forward(gate)
+    dgu = be.upload(gu32, F32)
+    out = be.swiglu_forward(dgu)
+    assert out.dtype == BF16
+    _close(be.download_f32(out), orc.mul_forward(act, up))
+    g_act, g_up = orc.mul_backward(act, up, gm)
+    got = be.download_f32(be.swiglu_backward(dgu, be.upload(gm, BF16)))
+    _close(got[:, :hidden], orc.silu_backward(gate, g_act))
+    _close(got[:, hidden:], g_up)
 
 
 def test_linear_i8_group_refusals(be):
@@ -193,17 +223,17 @@ def test_linear_i8_group_refusals(be):
     scales = be.upload(np.zeros((32, 1), np.float32))
     with pytest.raises(OjasError) as e:  # k_in is not a multiple of the group
         be._check(be._lib.omx_linear_i8_group_forward(be._ctx, be._p(x), C.c_int32(1), be._p(codes), be._p(scales),
-                                                      C.c_uint64(32), C.c_int32(0), None, None, be._p(x), C.c_uint64(8), C.c_uint64(48),
+                                                      C.c_uint64(32), C.c_int32(0), None, None, be._p(x), C.c_int32(1), C.c_uint64(8), C.c_uint64(48),
                                                       C.c_uint64(32)))
     assert e.value.code == SHAPE
     with pytest.raises(OjasError) as e:
         be._check(be._lib.omx_linear_i8_group_forward(be._ctx, be._p(x), C.c_int32(1), be._p(codes), be._p(scales),
-                                                      C.c_uint64(64), C.c_int32(0), None, None, be._p(x), C.c_uint64(8), C.c_uint64(64),
+                                                      C.c_uint64(64), C.c_int32(0), None, None, be._p(x), C.c_int32(1), C.c_uint64(8), C.c_uint64(64),
                                                       C.c_uint64(32)))
     assert e.value.code == UNSUPPORTED
     with pytest.raises(OjasError) as e:
         be._check(be._lib.omx_linear_i8_group_forward(be._ctx, be._p(x), C.c_int32(0), be._p(codes), be._p(scales),
-                                                      C.c_uint64(32), C.c_int32(0), None, None, be._p(x), C.c_uint64(8), C.c_uint64(64),
+                                                      C.c_uint64(32), C.c_int32(0), None, None, be._p(x), C.c_int32(1), C.c_uint64(8), C.c_uint64(64),
                                                       C.c_uint64(32)))
     assert e.value.code == DTYPE
 

@@ -71,12 +71,15 @@ def random_model(spec, seed):
     return host, r
 
 
-def oracle_step(spec, host, ids, targets, B, T):
+def oracle_step(spec, host, ids, targets, B, T, rounding=0):
     cfg = orc.NanolabConfig(layers=spec.n_layer, n_embd=spec.n_embd, n_head=spec.n_head, n_kv_head=spec.n_kv_head,
                             head_dim=spec.head_dim, hidden=spec.hidden, vocab=spec.vocab, batch=B, seq=T,
                             window=spec.window or 0, rms_eps=spec.rms_eps, rope_base=spec.rope_base)
     names = spec.param_names()
-    loss, _, grads = orc.nanolab_loss_and_grads(cfg, [host[n] for n in names], ids, targets)
+    if rounding:
+        loss, grads = orc.nanolab_loss_and_grads_rounded(cfg, [host[n] for n in names], ids, targets, rounding)
+    else:
+        loss, _, grads = orc.nanolab_loss_and_grads(cfg, [host[n] for n in names], ids, targets)
     return float(loss), dict(zip(names, grads))
 
 
@@ -116,8 +119,13 @@ def test_f32_tier_every_gradient_against_the_oracle(be, kv_heads, window):
                                         window=40),
                                    dict(n_layer=2, n_embd=128, n_head=4, n_kv_head=2, head_dim=32, hidden=136, vocab=64)])
 def test_bf16_tier_against_the_oracle(be, shape):
-    """bf16 storage: MFMA attention at head_dim 64 / 128 (row kernels at 32), the gate | up product
-    with the fused SwiGLU. Parameters are bf16-exact so that both sides multiply the same weights."""
+    """The bf16 tier (bf16 operands, every activation rounded once: the forward's product outputs
+    stay f32): MFMA attention at head_dim 64 / 128 (row kernels at 32), the gate | up product with
+    the fused SwiGLU. Parameters are bf16-exact so that both sides multiply the same weights.
+    Against the Exact oracle: loss 1e-3 relative; every matrix and the table within 2e-2 of its
+    largest value per element and 2e-2 normwise; norm weights within 2e-2, or within 1.25 x what the
+    oracle itself moves them when nothing but its products' operands are rounded to bf16, where that
+    floor lies higher; the one- to four-element vectors by the bound argued below."""
     from ojas_amd.nanolab import NanolabSpec, NativeNanolabTrainer
 
     print(f"native nanolab bf16 vs oracle {shape}", flush=True)
@@ -131,34 +139,31 @@ def test_bf16_tier_against_the_oracle(be, shape):
     loss, grads = tr.loss_and_grads(ids, targets)
     tr.close()
     o_loss, o_grads = oracle_step(spec, host, ids, targets, B, T)
+    _, floor_grads = oracle_step(spec, host, ids, targets, B, T, rounding=orc.ROUND_OPERANDS)
     assert abs(loss - o_loss) <= 1e-3 * abs(o_loss), (loss, o_loss)
-    worst = {"matrix": 0.0, "vector": 0.0, "normwise": 0.0}
-    vectors = []
     shapes = spec.param_shapes()
+    worst = {"matrix": 0.0, "normwise": 0.0, "norm weight": 0.0, "tiny vector": 0.0}
     for name, ref in o_grads.items():
         got = grads[name].astype(np.float64)
         if name == "blocks.0.mixer.vr_lambda":
             assert not np.any(got)
             continue
-        kind = "matrix" if len(shapes[name]) == 2 else "vector"
-        worst[kind] = max(worst[kind], float(np.max(np.abs(got - ref))) / float(np.max(np.abs(ref))))
-        if kind == "vector":
-            vectors.append((float(np.max(np.abs(got - ref))) / float(np.max(np.abs(ref))), name))
-        if kind == "matrix":
-            worst["normwise"] = max(worst["normwise"], float(np.linalg.norm(got - ref) / np.linalg.norm(ref)))
-    print(f"  worst element / largest: matrices {worst['matrix']:.2e} (normwise {worst['normwise']:.2e}), "
-          f"vectors {worst['vector']:.2e}", flush=True)
-    print("  largest vector distances:", ", ".join(f"{n} {e:.1e}" for e, n in sorted(vectors, reverse=True)[:4]), flush=True)
-    # The oracle keeps f32 between operations and rounds operands only (the reference's Autocast); this
-    # tier stores activations and their gradients in bf16, which the reference holds to its loss
-    # curve alone (the trace test below). Against the oracle's gradients the matrices and the table
-    # measured at most 1.9e-2, 2.4e-2 and 1.6e-2 of their largest value on these three models (the
-    # second, with three blocks, head_dim 128 and a window, has k_proj above 2e-2), normwise at most
-    # 2.3e-2. The vectors with 64 to 256 values (norm weights) measured up to 3.4e-2; the ones with one
-    # or two values (vr_lambda, the gate bias of two heads: each a sum of some 10^4 signed terms, where
-    # "of the largest value" is the relative error of that one sum) up to 9.3e-2.
-    assert worst["matrix"] <= 3e-2 and worst["normwise"] <= 3e-2 and worst["vector"] <= 1.2e-1, worst
-    assert all(e <= 4e-2 for e, n in vectors if "norm" in n), vectors
+        elementwise = float(np.max(np.abs(got - ref))) / float(np.max(np.abs(ref)))
+        floor = float(np.max(np.abs(floor_grads[name] - ref))) / float(np.max(np.abs(ref)))
+        if len(shapes[name]) == 2:
+            normwise = float(np.linalg.norm(got - ref) / np.linalg.norm(ref))
+            worst["matrix"], worst["normwise"] = max(worst["matrix"], elementwise), max(worst["normwise"], normwise)
+            assert elementwise <= 2e-2 and normwise <= 2e-2, (name, elementwise, normwise)
+        elif ref.size > 4:
+            worst["norm weight"] = max(worst["norm weight"], elementwise)
+            assert elementwise <= max(2e-2, 1.25 * floor), (name, elementwise, floor)
+        else:
+            # vr_lambda, the gate's bias per head: one number each, a sum of some 10^4 signed terms,
+            # so "of the largest value" is the relative error of that one sum. The oracle's own
+            # operands-only run moves these by up to 6e-2 on these models.
+            worst["tiny vector"] = max(worst["tiny vector"], elementwise)
+            assert elementwise <= 1.2e-1, (name, elementwise, floor)
+    print("  worst distances:", ", ".join(f"{k} {v:.2e}" for k, v in worst.items()), flush=True)
 
 
 @pytest.mark.parametrize("bf16", [False, True])
