@@ -463,7 +463,7 @@ int32_t onano_create(omx_ctx* ctx, const onano_config* config, onano** out) {
   // The three projections are one matrix only if nothing pads the arena between them.
   t->fused_qkv = t->flash && (static_cast<uint64_t>(c.heads) * c.head_dim * c.n_embd) % kAlign == 0 &&
                  (static_cast<uint64_t>(c.kv_heads) * c.head_dim * c.n_embd) % kAlign == 0;
-  t->keep_f32 = c.bf16 == 1 && t->fused_mlp;
+  t->keep_f32 = c.bf16 && t->fused_mlp;
   t->LD = t->keep_f32 ? OMX_F32 : t->AD;
   t->lsz = t->keep_f32 ? 4 : t->asz;
   const uint64_t N = t->N, d = c.n_embd, H = c.heads, KV = c.kv_heads, D = c.head_dim, Hd = c.hidden;
