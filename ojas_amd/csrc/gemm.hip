@@ -496,7 +496,18 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
       // (916 against 1121 us), the others on 256 x 128.
       const bool unbatched = g.batches == 1;
       const long outputs = static_cast<long>(g.M) * g.N;
-      if (unbatched && a_km && b_km && g.K >= 4096 && outputs <= (1l << 22)) dma_variant = 6;
+      // The alternating 256 x 256 kernel (one workgroup per compute unit) where its tiles fill the
+      // chip several times over, or twice over a long reduction: the head's forward product
+      // (12608 tiles over K = 768: 1463 against 1636 us) and weight gradient (591 tiles over
+      // K = 16384: 1223 against 1295 us), square products of 8192 (945 against 1230 us). With
+      // fewer rounds of tiles what a tile costs outside its K steps (first loads, store pass)
+      // is not hidden by a second workgroup and the 256 x 128 form is ahead (576 tiles over
+      // K = 768: 84 against 73 us).
+      const long tiles256 = static_cast<long>((g.M + 255) / 256) * ((g.N + 255) / 256);
+      const long cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
+      if (unbatched && !(epi && epi->mode != OMX_EPI_NONE) && (tiles256 >= 4 * cus || (tiles256 >= 2 * cus && g.K >= 4096)))
+        dma_variant = 8;
+      else if (unbatched && a_km && b_km && g.K >= 4096 && outputs <= (1l << 22)) dma_variant = 6;
       else if (!unbatched && a_km && b_km && g.K >= 4096 && g.M >= 3072 && g.N <= 1024) dma_variant = 0;
       else if (outputs * g.batches <= (1l << 20)) dma_variant = -1;
       else if (unbatched && !a_km && b_km && g.N <= 1024 && g.K <= 4096) dma_variant = 6;
@@ -506,6 +517,7 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
     else if (mode == 2) dma_variant = 0;
     else if (mode == 3) dma_variant = 3;
     else if (mode == 4) dma_variant = 6;
+    else if (mode == 8) dma_variant = 8;
   }
   int BM = 128, BN = 128;
   if (dma_variant >= 0) omx_gemm_dma_tile(dma_variant, &BM, &BN);
@@ -662,7 +674,7 @@ int32_t omx_set_option(omx_ctx* ctx, const char* name, int64_t value) {
     return OMX_OK;
   }
   if (name && strcmp(name, "gemm_dma") == 0) {
-    if (value < 0 || value > 4) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: gemm_dma takes 0..4");
+    if (value < 0 || (value > 4 && value != 8)) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: gemm_dma takes 0..4 or 8");
     ctx->gemm_dma_mode = static_cast<int>(value);
     return OMX_OK;
   }

@@ -3,6 +3,7 @@
 // holds the description of the kernels and chooses among the four.
 #pragma once
 #include "gemm_tiles.h"
+#include "gemm_pp_impl.h"
 
 namespace {
 
@@ -636,6 +637,7 @@ int32_t launch_dma(omx_ctx* ctx, const GemmArgs& g) {
 // stages, two workgroups per compute unit); 6: 128 x 128 with four waves (three per compute unit).
 template <bool A_KM, bool B_KM>
 int32_t launch_variant(omx_ctx* ctx, const GemmArgs& g, int variant) {
+  if (variant == 8) return launch_pp<A_KM, B_KM>(ctx, g);
   if (variant == 0) return launch_dma<A_KM, B_KM, 2, 4, 4, 2, 64, 2>(ctx, g);
   if (variant == 6) return launch_dma<A_KM, B_KM, 2, 2, 2, 2, 32, 3>(ctx, g);
   return launch_dma<A_KM, B_KM, 4, 2, 2, 2, 32, 3>(ctx, g);

@@ -65,6 +65,20 @@ struct TileLoads {
       src[i] += step;
     }
   }
+  // The same for the loads named in MASK only (bit i: this wave's load i, which fills KiB
+  // wave + NW i of the tile): a part of the tile is refilled as soon as it has been read.
+  template <unsigned MASK>
+  __device__ __forceinline__ void issue_some(unsigned tile, int wave) {
+    static_assert(EVEN, "every wave holds every load slot");
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      if (!((MASK >> i) & 1u)) continue;
+      asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src[i]),
+                   "s"(tile + (wave + NW * i) * 1024)
+                   : "memory");
+      src[i] += step;
+    }
+  }
 };
 
 // The same loads with one scalar base address per operand and a 32-bit byte offset per lane and
