@@ -804,6 +804,7 @@ FlashShape make_shape(uint64_t batch, uint64_t heads, uint64_t kv_heads, uint64_
 // also when the pairs need more than one round, whose last would run part empty (the blocks go out
 // heaviest first, so the light ones fill the end).
 int flash_single(omx_ctx* ctx, unsigned pair_groups, int per_cu, bool also_rounds) {
+  if (ctx->flash_schedule != 0) return ctx->flash_schedule == 1 ? 1 : 0;  // forced (tests cover both)
   const unsigned places = static_cast<unsigned>(ctx->cu_count > 0 ? ctx->cu_count : 256) * per_cu;
   if (pair_groups < places) return 1;
   return also_rounds && pair_groups > places ? 1 : 0;

@@ -477,42 +477,47 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
   if (!thin && operand_dtype == OMX_BF16 && omx_gemm_dma_eligible(g, a_km, b_km)) {
     const int mode = ctx->gemm_dma_mode;
     if (mode == 1) {
-      // Measured on the GPT shapes: small outputs (the d x d weight gradients, the
-      // Newton-Schulz squares) stay on the 128 x 128 kernel; everything else takes 256 x 128
-      // tiles in 32-column K steps, three stages in 72 KiB, so two workgroups share a compute
-      // unit and one's output stores, first loads and barrier waits overlap the other's
-      // products. The 64-column forms fetch whole cache lines but run alone on their compute
-      // unit; they win only on long reductions with large outputs (8192^3: 1.09 against
-      // 0.95 PFLOP/s for 256 x 256) and lose on every GPT shape.
-      // 128 x 128 tiles with four waves (48 KiB, three workgroups per compute unit) give the
-      // layers' input-gradient products with up to 1024 output columns three tiles per compute
-      // unit instead of one and a half (K = 3072: 94 against 104 us), and are 3 to 20 % ahead on
-      // the layers' weight-gradient products (both operands K-major, K = tokens), d x d included.
-      // The head's products (K or M = vocabulary) are faster on the larger tile, and its input
-      // gradient (16384 x 768 outputs over K = 50304) on 256 x 256 in whole-line steps: one
-      // workgroup per compute unit, but 2095 steps to amortise that over (1610 against 1824 us).
-      // A batch of weight gradients over stacked layers (K = tokens) has tiles enough without
-      // splitting K; its tall form (3072 x 768 outputs, twelve layers) is faster on 256 x 256
-      // (916 against 1121 us), the others on 256 x 128.
+      // Four tilings, chosen by how many tiles the output makes per compute unit and how many K
+      // steps a tile runs, not by a model's dimensions (measured over GPT-124M's shapes and over
+      // d = 1024 / 2048 / 4096 with 8192 tokens; tests/test_gpu_gemm_kernels.py holds the choice
+      // to within 10 % of the best forced tiling):
+      //   3  256 x 128, 32-column steps, two workgroups per compute unit: one's first loads and
+      //      store pass run under the other's products, so it is the form for short reductions
+      //      and for outputs of a round or two of tiles. The default.
+      //   6  128 x 128, four waves, three workgroups per compute unit: weight gradients (both
+      //      operands k-major, K = tokens) whose output is under one tile per compute unit, with
+      //      the reduction split (3 to 20 % ahead of 256 x 128 there).
+      //   0  256 x 256, whole-line 64-column steps, one workgroup per compute unit: k-contiguous
+      //      A (forward and input-gradient products) over at least 32 steps when the tiles fill
+      //      the chip (K = 8192, 8192 x 2048 outputs: 233 against 282 us for 256 x 128), and the
+      //      tall weight-gradient batches.
+      //   8  the alternating 256 x 256 kernel: k-major products over long reductions when the
+      //      tiles fill the chip (4096 x 4096 over K = 8192: 225 against 241 us), and outputs of
+      //      four rounds of tiles or more over a short reduction (the head's forward product,
+      //      12608 tiles over K = 768: 1554 against 1642 us), where 0 pays its exposed first
+      //      loads once per 12 steps (1881 us).
       const bool unbatched = g.batches == 1;
+      const bool plain = !(epi && epi->mode != OMX_EPI_NONE);
       const long outputs = static_cast<long>(g.M) * g.N;
-      // The alternating 256 x 256 kernel (one workgroup per compute unit) where its tiles fill the
-      // chip several times over, or twice over a long reduction: the head's forward product
-      // (12608 tiles over K = 768: 1463 against 1636 us) and weight gradient (591 tiles over
-      // K = 16384: 1223 against 1295 us), square products of 8192 (945 against 1230 us). With
-      // fewer rounds of tiles what a tile costs outside its K steps (first loads, store pass)
-      // is not hidden by a second workgroup and the 256 x 128 form is ahead (576 tiles over
-      // K = 768: 84 against 73 us).
-      const long tiles256 = static_cast<long>((g.M + 255) / 256) * ((g.N + 255) / 256);
       const long cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
-      if (unbatched && !(epi && epi->mode != OMX_EPI_NONE) && (tiles256 >= 4 * cus || (tiles256 >= 2 * cus && g.K >= 4096)))
-        dma_variant = 8;
-      else if (unbatched && a_km && b_km && g.K >= 4096 && outputs <= (1l << 22)) dma_variant = 6;
-      else if (!unbatched && a_km && b_km && g.K >= 4096 && g.M >= 3072 && g.N <= 1024) dma_variant = 0;
-      else if (outputs * g.batches <= (1l << 20)) dma_variant = -1;
-      else if (unbatched && !a_km && b_km && g.N <= 1024 && g.K <= 4096) dma_variant = 6;
-      else if (unbatched && !a_km && b_km && g.N <= 1024 && g.K >= 32768 && g.M >= 8192) dma_variant = 0;
-      else dma_variant = 3;
+      const long tiles256 = static_cast<long>((g.M + 255) / 256) * ((g.N + 255) / 256);
+      const long tiles128 = static_cast<long>((g.M + 127) / 128) * ((g.N + 127) / 128);
+      const long ksteps64 = g.K / 64;
+      if (a_km && b_km && unbatched && ksteps64 >= 64 && tiles128 < cus) {
+        dma_variant = 6;
+      } else if (outputs * g.batches <= (1l << 20)) {
+        dma_variant = -1;  // a handful of tiles: the register-staged kernel, which splits K freely
+      } else if (a_km && b_km) {
+        if (unbatched && plain && tiles256 >= cus && ksteps64 >= 64) dma_variant = 8;
+        else if (!unbatched && ksteps64 >= 64 && g.M >= 12 * 256 && g.N <= 4 * 256) dma_variant = 0;
+        else dma_variant = 3;
+      } else if (!a_km) {
+        if (unbatched && plain && tiles256 >= 4 * cus && ksteps64 < 32) dma_variant = 8;
+        else if (unbatched && plain && ((tiles256 >= cus && ksteps64 >= 32) || ksteps64 >= 512)) dma_variant = 0;
+        else dma_variant = 3;
+      } else {
+        dma_variant = 3;
+      }
     }
     else if (mode == 2) dma_variant = 0;
     else if (mode == 3) dma_variant = 3;
@@ -660,22 +665,18 @@ extern "C" {
 
 int32_t omx_set_option(omx_ctx* ctx, const char* name, int64_t value) {
   OMX_REQUIRE_CTX(ctx);
-  if (name && strcmp(name, "gemm_persistent_min_steps") == 0) {
-    if (value < 2) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: gemm_persistent_min_steps is at least 2");
-    ctx->gemm_persistent_min_steps = static_cast<int>(value);
-    return OMX_OK;
-  }
   if (name && strcmp(name, "gemm_thin") == 0) {
     ctx->gemm_thin = value != 0;
-    return OMX_OK;
-  }
-  if (name && strcmp(name, "gemm_persistent") == 0) {
-    ctx->gemm_persistent = static_cast<int>(value) & 15;
     return OMX_OK;
   }
   if (name && strcmp(name, "gemm_dma") == 0) {
     if (value < 0 || (value > 4 && value != 8)) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: gemm_dma takes 0..4 or 8");
     ctx->gemm_dma_mode = static_cast<int>(value);
+    return OMX_OK;
+  }
+  if (name && strcmp(name, "flash_schedule") == 0) {
+    if (value < 0 || value > 2) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: flash_schedule takes 0..2");
+    ctx->flash_schedule = static_cast<int>(value);
     return OMX_OK;
   }
   if (name && strcmp(name, "ce_fused") == 0) {

@@ -587,6 +587,9 @@ gemm_dma_persistent_kernel(GemmArgs g) {
   }
 }
 
+// The persistent form pays for its longer code and parked offsets from 64 K steps on (K >= 2048).
+constexpr int kPersistentMinSteps = 64;
+
 template <bool A_KM, bool B_KM, int WGM, int WGN, int TM, int TN, int DBK, int NST>
 int32_t launch_dma(omx_ctx* ctx, const GemmArgs& g) {
   constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
@@ -594,7 +597,7 @@ int32_t launch_dma(omx_ctx* ctx, const GemmArgs& g) {
   if constexpr (NST == 3 && TM * TN <= 4 && ((BM + BN) * DBK * 2) % (1024 * WGM * WGN) == 0) {
     // Tiles wholly inside both operands (the persistent form never clamps a row).
     const long tiles_all = static_cast<long>(g.tiles_m) * g.tiles_n * g.batches;
-    if (g.splits == 1 && (ctx->gemm_persistent >> ((A_KM ? 2 : 0) + (B_KM ? 1 : 0)) & 1) && g.M % BM == 0 && g.N % BN == 0 && g.K / DBK >= ctx->gemm_persistent_min_steps &&
+    if (g.splits == 1 && g.M % BM == 0 && g.N % BN == 0 && g.K / DBK >= kPersistentMinSteps &&
         (!g.c_bf16 || g.c_vec) &&
         g.tiles_n * 4 < 65536 && tiles_all * (g.K / DBK) < (1l << 30)) {
       GemmArgs gp = g;

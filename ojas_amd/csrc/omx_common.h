@@ -92,10 +92,8 @@ struct omx_ctx {
   // Optional per-launch timing of the GEMM kernel (benchmark only).
   // 0: 128x128 kernel only; 1: choose by shape; 2 / 3: force the 256x256 / 256x128 direct-to-LDS kernel where eligible.
   int gemm_dma_mode = 1;
-  // Which operand layouts take the persistent form of the direct-to-LDS kernel: bit (2 A_k-major + B_k-major).
   int gemm_thin = 1;         // outputs of at most 64 columns over many rows take gemm_thin_kernel
-  int gemm_persistent = 15;
-  int gemm_persistent_min_steps = 64;  // ... and only for reductions of at least this many 32-column steps
+  int flash_schedule = 0;     // 0: by the chip's workgroup places; 1: one 128-row block per workgroup; 2: mirrored pairs
   int kv_attention_mode = 0;  // 1: cached attention always takes the LDS-tiled kernel
   int adamw_trust = 1;        // 0: omx_adamw_step_bounded always runs its checking pass
   int ce_fused = 1;           // 0: linear-CE always takes the separate statistics and gradient kernels

@@ -730,14 +730,22 @@ def test_causal_sdpa_bf16_scores_that_keep_growing(be, per_key):
     close(be.download(gv), ogv, BF16_TOL, "growing scores: gv")
 
 
+@pytest.fixture(params=["one block per workgroup", "mirrored pairs"])
+def flash_schedule(request, be):
+    """Both block schedules of the flash kernels, whichever the chip's size would pick by itself."""
+    be.set_option("flash_schedule", 1 if request.param == "one block per workgroup" else 2)
+    yield request.param
+    be.set_option("flash_schedule", 0)
+
+
 @pytest.mark.parametrize("shape,hkv,window", FLASH_SHAPES)
-def test_causal_sdpa_bf16_mfma(be, shape, hkv, window):
+def test_causal_sdpa_bf16_mfma(be, shape, hkv, window, flash_schedule):
     """head_dim 64 or 128 with bf16 operands takes the MFMA flash kernels. Inputs are
     bf16-exact on both sides; the GPU additionally rounds P and dS to bf16 for
     the second product, so the gate is the bf16 one (2e-2 of the largest value)."""
     from ojas_amd.backend import BF16, F32
 
-    print(f"sdpa bf16 {shape} hkv {hkv} window {window}", flush=True)
+    print(f"sdpa bf16 {shape} hkv {hkv} window {window} schedule: {flash_schedule}", flush=True)
     b, h, t, d = shape
     r = orc.SplitMix64(900 + t)
     mk = lambda n, sh: orc.round_bf16(r.vec(n, 1.0)).reshape(sh)
