@@ -17,7 +17,7 @@ bandwidth), each from the dispatch timestamps of its own launches in the same
 timed steps. `cpu_baseline` times the CPU oracle (a C++ restatement of the
 reference's CPU Exact arithmetic; the Rust reference cannot be built without
 cargo) on the host cores, on a bounded sample of the same workload, with all
-cores and with one thread, three repeats each.
+cores and with one thread, five repeats each (minimum, median and spread reported).
 """
 import argparse
 import ctypes as C
@@ -86,20 +86,34 @@ def cpu_model() -> str:
     return "unknown"
 
 
-def repeat_timed(fn, repeats: int = 3):
-    """fn() -> seconds of the part it times itself; returns the sorted list of `repeats` runs."""
+def repeat_timed(fn, repeats: int = 5):
+    """fn() -> seconds of the part it times itself; one untimed run first (page faults, thread
+    start-up), then the sorted list of `repeats` runs."""
+    fn()
     return sorted(fn() for _ in range(repeats))
+
+
+def median_of(runs):
+    return runs[len(runs) // 2]
+
+
+def spread_of(runs):
+    """(max - min) / median of sorted timings."""
+    return (runs[-1] - runs[0]) / median_of(runs)
 
 
 def cpu_baseline(cfg, threads: int):
     """Times the oracle on a bounded sample of the same model and scales it to the step.
 
     Sequences share nothing but the weights and blocks cost the same, so the step's time is
-    tokens x (rest + layers x block) / sample tokens + the optimizer pass, with `block` and `rest`
-    from the model at one and at two blocks on one short sequence, and the optimizer (clip +
-    AdamW) timed on one block's parameters and scaled by the parameter count. A configuration small
-    enough (the tiny one) is timed whole instead. All cores and one thread, three repeats each;
-    `value` is the median of the all-cores runs."""
+    tokens x (rest + layers x block) / sample tokens + the optimizer pass. `block` comes from the
+    model at one and at three blocks over a 256-entry vocabulary (the head is then a negligible part
+    of both timings, so their difference is two blocks and little else), `rest` (embedding, final
+    norm, the head over the real vocabulary) from the one-block model at the real vocabulary minus a
+    block, and the optimizer (clip + AdamW) from one block's parameters scaled by the parameter
+    count. A configuration small enough (the tiny one) is timed whole instead. All cores (the
+    thread count is set explicitly) and one thread, one untimed run then five timed ones each;
+    `value` is the median of the all-cores runs, `spread` their (max - min) / median."""
     sys.path.insert(0, str(ROOT / "tests"))
     import oracle_api as orc
     from ojas_amd.trainer import GptConfig, synthetic_batch
@@ -108,9 +122,10 @@ def cpu_baseline(cfg, threads: int):
     whole = tokens * cfg.layers * cfg.d_model * cfg.d_model < 3e9  # the tiny configuration: 0.5e9
     rng = np.random.default_rng(0)
 
-    def model(layers, batch, ctx):
-        sample = GptConfig(layers, cfg.d_model, cfg.heads, cfg.head_dim, cfg.mlp, ctx, cfg.vocab, batch, cfg.gelu_tanh, 0)
-        ocfg = orc.GptConfig(layers, cfg.d_model, cfg.heads, cfg.head_dim, cfg.mlp, ctx, cfg.vocab, batch, cfg.gelu_tanh)
+    def model(layers, batch, ctx, vocab=None):
+        vocab = vocab or cfg.vocab
+        sample = GptConfig(layers, cfg.d_model, cfg.heads, cfg.head_dim, cfg.mlp, ctx, vocab, batch, cfg.gelu_tanh, 0)
+        ocfg = orc.GptConfig(layers, cfg.d_model, cfg.heads, cfg.head_dim, cfg.mlp, ctx, vocab, batch, cfg.gelu_tanh)
         params = [np.ones(n, np.float32) if n == cfg.d_model else rng.normal(0, 0.02, n).astype(np.float32)
                   for n in orc.gpt_param_lens(ocfg)]
         ids, targets = synthetic_batch(sample, 1)
@@ -136,35 +151,38 @@ def cpu_baseline(cfg, threads: int):
 
             runs = repeat_timed(once)
             return runs, f"the whole step ({cfg.batch}x{cfg.ctx} tokens)"
-        one, two = model(1, 1, sample_ctx), model(2, 1, sample_ctx)
+        one, small_one, small_three = model(1, 1, sample_ctx), model(1, 1, sample_ctx, 256), model(3, 1, sample_ctx, 256)
         n_params = sum(orc.gpt_param_lens(orc.GptConfig(cfg.layers, cfg.d_model, cfg.heads, cfg.head_dim, cfg.mlp,
                                                         cfg.ctx, cfg.vocab, cfg.batch, cfg.gelu_tanh)))
         block_params = [p for p in one[1][2:-1]]  # the block's eight tensors
 
         def once():
             t = []
-            for ocfg, params, ids, targets in (one, two):
+            for ocfg, params, ids, targets in (small_one, small_three, one):
                 t0 = time.perf_counter()
                 orc.gpt_loss_and_grads(ocfg, params, ids, targets)
                 t.append(time.perf_counter() - t0)
-            block = max(t[1] - t[0], 1e-9)
-            rest = max(t[0] - block, 0.0)
+            block = max((t[1] - t[0]) / 2, 1e-9)
+            rest = max(t[2] - block, 0.0)
             opt = optimizer_seconds(block_params, [np.full_like(p, 1e-3) for p in block_params])
             opt *= n_params / sum(p.size for p in block_params)
             return tokens * (rest + cfg.layers * block) / sample_ctx + opt
 
         runs = repeat_timed(once)
-        return runs, (f"one and two blocks on 1x{sample_ctx} tokens (block and rest), clip + AdamW on one block's "
-                      f"parameters, scaled to {cfg.layers} blocks, {tokens} tokens and {n_params} parameters")
+        return runs, (f"one and three blocks over a 256-entry vocabulary (a block) and one block over the real one "
+                      f"(the rest) on 1x{sample_ctx} tokens, clip + AdamW on one block's parameters, scaled to "
+                      f"{cfg.layers} blocks, {tokens} tokens and {n_params} parameters")
 
-    all_runs, how = measure(threads, 256)
+    all_runs, how = measure(threads, 512)
     one_runs, how_one = measure(1, 64)
     note = ("" if whole else " Attention grows with the sequence: at these sample lengths it is a smaller share than at "
             f"{cfg.ctx}, so the estimate favours the CPU by up to its 8 % of the step's work.")
-    return {"value": tokens / all_runs[1], "unit": "tokens/s", "cores": threads, "kind": "port",
-            "cpu_model": cpu_model(), "repeats": 3, "step_seconds_min": all_runs[0], "step_seconds_median": all_runs[1],
-            "single_thread": {"value": tokens / one_runs[1], "cores": 1, "step_seconds_min": one_runs[0],
-                              "step_seconds_median": one_runs[1], "sample": how_one},
+    median, spread = median_of, spread_of
+    return {"value": tokens / median(all_runs), "unit": "tokens/s", "cores": threads, "kind": "port",
+            "cpu_model": cpu_model(), "repeats": len(all_runs), "step_seconds_min": all_runs[0],
+            "step_seconds_median": median(all_runs), "spread": spread(all_runs),
+            "single_thread": {"value": tokens / median(one_runs), "cores": 1, "step_seconds_min": one_runs[0],
+                              "step_seconds_median": median(one_runs), "spread": spread(one_runs), "sample": how_one},
             "sample": f"same model (L{cfg.layers} d{cfg.d_model} vocab{cfg.vocab}) in f32 Exact arithmetic: {how}."
                       f"{note} C++ restatement of ojas-cpu, not the Rust binary"}
 
@@ -277,7 +295,7 @@ def lora_cpu_baseline(cfg, threads: int):
     sequence, once with one block and once with two; the difference is a block's time, the rest the
     table, final norm and head; the step is tokens x (rest + layers x block) / sample tokens plus
     clip + AdamW on the adapters (timed on the two-block model's, scaled by their count). All cores
-    and one thread, three repeats each; `value` is the median of the all-cores runs."""
+    and one thread, five repeats each; `value` is the median of the all-cores runs."""
     sys.path.insert(0, str(ROOT / "tests"))
     import oracle_api as orc
 
@@ -327,10 +345,11 @@ def lora_cpu_baseline(cfg, threads: int):
 
     all_runs = measure(threads, 128)
     one_runs = measure(1, 32)
-    return {"value": tokens / all_runs[1], "unit": "tokens/s", "cores": threads, "kind": "port",
-            "cpu_model": cpu_model(), "repeats": 3, "step_seconds_min": all_runs[0], "step_seconds_median": all_runs[1],
-            "single_thread": {"value": tokens / one_runs[1], "cores": 1, "step_seconds_min": one_runs[0],
-                              "step_seconds_median": one_runs[1], "sample": "as below on 1x32 tokens"},
+    return {"value": tokens / median_of(all_runs), "unit": "tokens/s", "cores": threads, "kind": "port",
+            "cpu_model": cpu_model(), "repeats": len(all_runs), "step_seconds_min": all_runs[0],
+            "step_seconds_median": median_of(all_runs), "spread": spread_of(all_runs),
+            "single_thread": {"value": tokens / median_of(one_runs), "cores": 1, "step_seconds_min": one_runs[0],
+                              "step_seconds_median": median_of(one_runs), "spread": spread_of(one_runs), "sample": "as below on 1x32 tokens"},
             "sample": f"same model at full width in f32 Exact arithmetic on dequantised weights: one and two blocks on "
                       f"1x128 tokens (block and rest), clip + AdamW on two blocks' adapters, scaled to {cfg.layers} "
                       f"blocks and {tokens} tokens. Attention grows with the sequence: at this sample length it is a "
@@ -410,7 +429,7 @@ def nanolab_cpu_baseline(spec, batch, seq, threads: int):
     """The oracle's nanolab step on a bounded sample: one and two blocks on one short sequence give a
     block's time and the rest (table, final norm, head); clip + Muon-NS5 (f32 iteration) on one
     block's matrices and AdamW on its vectors and on the table give the optimizer's. Scaled to the
-    model's blocks and the step's tokens. All cores and one thread, three repeats each."""
+    model's blocks and the step's tokens. All cores and one thread, five repeats each."""
     sys.path.insert(0, str(ROOT / "tests"))
     import oracle_api as orc
     from ojas_amd.nanolab import NanolabSpec
@@ -464,10 +483,11 @@ def nanolab_cpu_baseline(spec, batch, seq, threads: int):
 
     all_runs = measure(threads, 128)
     one_runs = measure(1, 32)
-    return {"value": tokens / all_runs[1], "unit": "tokens/s", "cores": threads, "kind": "port",
-            "cpu_model": cpu_model(), "repeats": 3, "step_seconds_min": all_runs[0], "step_seconds_median": all_runs[1],
-            "single_thread": {"value": tokens / one_runs[1], "cores": 1, "step_seconds_min": one_runs[0],
-                              "step_seconds_median": one_runs[1], "sample": "as below on 1x32 tokens"},
+    return {"value": tokens / median_of(all_runs), "unit": "tokens/s", "cores": threads, "kind": "port",
+            "cpu_model": cpu_model(), "repeats": len(all_runs), "step_seconds_min": all_runs[0],
+            "step_seconds_median": median_of(all_runs), "spread": spread_of(all_runs),
+            "single_thread": {"value": tokens / median_of(one_runs), "cores": 1, "step_seconds_min": one_runs[0],
+                              "step_seconds_median": median_of(one_runs), "spread": spread_of(one_runs), "sample": "as below on 1x32 tokens"},
             "sample": f"same model in f32 Exact arithmetic: one and two blocks on 1x128 tokens (block and rest), Muon-NS5 "
                       f"and AdamW on one block's parameters and the table, scaled to {spec.n_layer} blocks and {tokens} "
                       f"tokens. Attention grows with the sequence: at this sample length it is a smaller share than at "
