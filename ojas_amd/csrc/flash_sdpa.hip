@@ -23,6 +23,7 @@
 //     keeps its k index in the matching order (bits 2 and 3 of the index
 //     swapped), so one 16-byte LDS read fetches exactly those rows.
 #include "omx_common.h"
+#include <type_traits>
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
@@ -120,6 +121,51 @@ __device__ __forceinline__ void tile_store_rows(char* lds, const u32x4 (&r)[D / 
   const int row = t / CPR, kc = t % CPR;
 #pragma unroll
   for (int i = 0; i < D / 32; ++i) *reinterpret_cast<u32x4*>(lds + (row + i * RPP) * fpitch(D) + kc * 16) = r[i];
+}
+// The same loads with the per-thread part of the address formed once. A tile that ends inside the
+// sequence is fetched from a wave-uniform base (plane + row0 rows) plus the thread's fixed 32-bit byte
+// offset: no address arithmetic and no bounds test per load. Only the last, ragged tile takes the
+// checked path. The host refuses row strides for which the offset would not fit.
+template <int D>
+struct TileFetch {
+  static constexpr int CPR = D / 8, RPP = FT / CPR;
+  unsigned off;  // bytes from a tile's first element to this thread's first chunk
+  long rs;
+  int time;
+  __device__ __forceinline__ TileFetch(long row_stride, int t_end) : rs(row_stride), time(t_end) {
+    const int t = threadIdx.x;
+    off = static_cast<unsigned>((t / CPR) * row_stride + (t % CPR) * 8) * 2u;
+  }
+  __device__ __forceinline__ void load(const unsigned short* __restrict__ plane, int row0, u32x4 (&r)[D / 32]) const {
+    if (row0 + 64 <= time) {
+      const char* base = reinterpret_cast<const char*>(plane + static_cast<long>(row0) * rs);
+#pragma unroll
+      for (int i = 0; i < D / 32; ++i) r[i] = *reinterpret_cast<const u32x4*>(base + static_cast<long>(i * RPP) * rs * 2 + off);
+    } else {
+      tile_load<D>(plane, rs, row0, time, r);
+    }
+  }
+};
+constexpr long FLASH_MAX_ROW_STRIDE = 1L << 24;  // elements: 31 rows of it, in bytes, stay below 2^32
+
+// The wave's index as a scalar, so that what depends on it (which tiles the wave takes, which of
+// them the diagonal cuts) is decided by scalar branches.
+__device__ __forceinline__ int wave_index() { return __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6)); }
+
+// x combined with the value lane ^ 32 holds: v_permlane32_swap exchanges the upper half of one
+// register with the lower half of another, so swapping x with a copy of itself leaves (x of the lower
+// lane, x of the upper lane) in the register pair of both lanes. One VALU instruction, no LDS round trip.
+__device__ __forceinline__ float halves_max(float x) {
+  const unsigned int u = __float_as_uint(x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  float m;
+  asm("v_max_f32 %0, %1, %2" : "=v"(m) : "v"(__uint_as_float(r[0])), "v"(__uint_as_float(r[1])));
+  return m;
+}
+__device__ __forceinline__ float halves_sum(float x) {
+  const unsigned int u = __float_as_uint(x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 // A operand from a [row][d] tile: rows sub*32 + lane%32, d-slab kk.
 template <int D>
@@ -227,7 +273,117 @@ __device__ __forceinline__ void flash_block_of(int pairs, int planes, int* pair,
 }
 
 // ------------------------------------------------------------------ forward
-template <int D, typename TO>
+// One 32-query x 64-key tile of one wave: scores, online softmax, weights times values.
+//   NSUB      32-key halves of the tile that hold a visible key (the second half of a tile whose
+//             first key is the wave's first query is hidden from all 32 rows and is left out);
+//   MASK_SUB  the half the causal diagonal cuts (its keys start at the wave's first query), or -1;
+//   GENERAL   the tile crosses the sequence end or a window edge: every element is tested.
+// `m` is the running maximum of the raw scores; the scale joins inside the fma. `lsum` sums the
+// weights as computed, `wsum` their bf16 copies (this lane's half of the keys).
+template <int D, int NSUB, int MASK_SUB, bool GENERAL>
+__device__ __forceinline__ void flash_fwd_tile(const char* k_rows, const char* v_rows, const u32x4 (&qf)[D / 16],
+                                               floatx16 (&o)[D / 32], float& m, float& lsum, float& wsum,
+                                               float scale_log2, int key0, int q_row, int T, int window, int lane) {
+  constexpr int KK = D / 16, MT = D / 32;
+  const int l32 = lane & 31, lg = lane >> 5;
+  floatx16 sc[NSUB];
+  // The SIMD serves its oldest wave first, and matrix and vector instructions of different waves
+  // barely overlap (measured: three waves of 16 MFMAs + 160 FMAs take 0.88 of the sum of both alone).
+  // A wave in its vector phase therefore holds up the others' products for the whole phase; raised
+  // priority for the two short product phases keeps the matrix units fed (7 % on the forward pass).
+  __builtin_amdgcn_s_setprio(2);
+#pragma unroll
+  for (int sub = 0; sub < NSUB; ++sub) {
+    sc[sub] = zero16();
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) sc[sub] = mfma(frag_rows<D>(k_rows, sub, kk, l32, lg), qf[kk], sc[sub]);
+  }
+  __builtin_amdgcn_s_setprio(0);
+  if constexpr (GENERAL) {
+#pragma unroll
+    for (int sub = 0; sub < NSUB; ++sub)
+#pragma unroll
+      for (int vv = 0; vv < 16; ++vv) {
+        const int key = key0 + sub * 32 + acc_row(vv, lg);
+        const bool masked = key > q_row || key >= T || (window > 0 && key + window <= q_row);
+        sc[sub][vv] = masked ? -INFINITY : sc[sub][vv];
+      }
+  } else if constexpr (MASK_SUB >= 0) {
+    // Key 4 lg + acc_row(v, 0) of the half against query l32 of the wave: a constant against one
+    // value that never changes (kept opaque: hoisted out of the tile loop, the sixteen compare
+    // results would occupy 32 scalar registers for the whole kernel).
+    int tri = l32 - 4 * lg;
+    asm volatile("" : "+v"(tri));
+#pragma unroll
+    for (int vv = 0; vv < 16; ++vv) sc[MASK_SUB][vv] = acc_row(vv, 0) > tri ? -INFINITY : sc[MASK_SUB][vv];
+  }
+  // Two chains, so that neither waits on the other's result.
+  float tmax, tmax2;
+  if constexpr (NSUB == 2) {
+    tmax = fmaxf(sc[0][0], sc[1][0]);
+    tmax2 = fmaxf(sc[0][1], sc[1][1]);
+#pragma unroll
+    for (int vv = 2; vv < 16; vv += 2) {
+      tmax = max3(tmax, sc[0][vv], sc[1][vv]);
+      tmax2 = max3(tmax2, sc[0][vv + 1], sc[1][vv + 1]);
+    }
+  } else {
+    tmax = fmaxf(sc[0][0], sc[0][1]);
+    tmax2 = fmaxf(sc[0][2], sc[0][3]);
+#pragma unroll
+    for (int vv = 4; vv < 16; vv += 4) {
+      tmax = max3(tmax, sc[0][vv], sc[0][vv + 1]);
+      tmax2 = max3(tmax2, sc[0][vv + 2], sc[0][vv + 3]);
+    }
+  }
+  tmax = halves_max(fmaxf(tmax, tmax2));
+  // The reference point of the exponents moves only when a row's maximum grew by more than 8
+  // binary orders (always on a row's first tile, where m is -inf): below that the weights of
+  // this tile are at most 2^8, well inside f32 and bf16, and the accumulators need no rescaling.
+  // The quotient at the end and the log-sum-exp use the same reference, so both stay exact.
+  const bool grow = (tmax - m) * scale_log2 > 8.0f;
+  const float new_m = grow ? tmax : m;
+  const float m_safe = new_m == -INFINITY ? 0.0f : new_m;
+  const float neg_m = -m_safe * scale_log2;
+  float psum = 0.0f;
+#pragma unroll
+  for (int sub = 0; sub < NSUB; ++sub)
+#pragma unroll
+    for (int vv = 0; vv < 16; ++vv) {
+      float p = __builtin_amdgcn_exp2f(fmaf(sc[sub][vv], scale_log2, neg_m));
+      sc[sub][vv] = p;
+      psum += p;
+    }
+  psum = halves_sum(psum);
+  if (__any(grow)) {
+    // Some row's reference moved: rescale what is accumulated so far (by exactly 1 in the
+    // rows that keep theirs).
+    const float alpha = __builtin_amdgcn_exp2f(fmaf(m, scale_log2, neg_m));
+    lsum *= alpha;
+    wsum *= alpha;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int vv = 0; vv < 16; ++vv) o[mt][vv] *= alpha;
+  }
+  lsum += psum;
+  m = new_m;
+  __builtin_amdgcn_s_setprio(2);
+#pragma unroll
+  for (int sub = 0; sub < NSUB; ++sub)
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const u32x4 pb = pack8(sc[sub], c);
+      wsum = sum_pairs(pb.x, sum_pairs(pb.y, sum_pairs(pb.z, sum_pairs(pb.w, wsum))));
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) o[mt] = mfma(frag_tr<D>(v_rows, mt, sub, c, lane), pb, o[mt]);
+    }
+  __builtin_amdgcn_s_setprio(0);
+}
+
+// WIN: the sliding-window form (every tile tested element by element), compiled apart so that the
+// plain causal kernel carries neither its code nor its registers.
+template <int D, typename TO, bool WIN>
 __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_fwd_kernel(const unsigned short* __restrict__ q,
                                                        const unsigned short* __restrict__ k,
                                                        const unsigned short* __restrict__ v, TO* __restrict__ out,
@@ -237,8 +393,9 @@ __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_fwd_kernel(const un
   // Two key / value tile pairs: the next tile is stored while this one is multiplied, so a tile
   // costs one barrier.
   __shared__ __attribute__((aligned(16))) char smem[4 * ftile(D)];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lg = lane >> 5;
+  const int lane = threadIdx.x & 63, wave = wave_index(), l32 = lane & 31, lg = lane >> 5;
   const int T = s.time;
+  const TileFetch<D> fetch(s.kv.rs, T);
   // Query block j sees j / 2 + 1 key tiles (causal): a workgroup takes a late block and then
   // its mirror image from the front, so every workgroup does the same amount of work and the
   // grid ends without a tail of half-empty compute units.
@@ -279,104 +436,65 @@ __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_fwd_kernel(const un
     const int kt_last = block_q1 / 64;
     // The next tile's global loads are in flight while the current one is multiplied.
     u32x4 rk[NL], rv[NL];
-    tile_load<D>(kp, s.kv.rs, kt_first * 64, T, rk);
-    tile_load<D>(vp, s.kv.rs, kt_first * 64, T, rv);
+    fetch.load(kp, kt_first * 64, rk);
+    fetch.load(vp, kt_first * 64, rv);
     __syncthreads();  // the previous pass's reads of the first pair are done
     tile_store_rows<D>(smem, rk);
     tile_store_rows<D>(smem + ftile(D), rv);
     if (kt_first < kt_last) {
-      tile_load<D>(kp, s.kv.rs, kt_first * 64 + 64, T, rk);
-      tile_load<D>(vp, s.kv.rs, kt_first * 64 + 64, T, rv);
+      fetch.load(kp, kt_first * 64 + 64, rk);
+      fetch.load(vp, kt_first * 64 + 64, rv);
     }
-    for (int kt = kt_first; kt <= kt_last; ++kt) {
-      const int key0 = kt * 64;
+    // One step of the tile pipeline, taken by every wave for every tile of the block: wait for tile
+    // kt's pair, store tile kt + 1 into the other pair, start the loads of tile kt + 2.
+    const char* k_rows;
+    const char* v_rows;
+    auto advance = [&](int kt) {
       const int cur = (kt - kt_first) & 1;
-      char* k_rows = smem + cur * 2 * ftile(D);
-      char* v_rows = k_rows + ftile(D);
+      k_rows = smem + cur * 2 * ftile(D);
+      v_rows = k_rows + ftile(D);
       __syncthreads();  // this pair is complete, and every wave is done with the other one
       if (kt < kt_last) {
         char* next = smem + (cur ^ 1) * 2 * ftile(D);
         tile_store_rows<D>(next, rk);
         tile_store_rows<D>(next + ftile(D), rv);
         if (kt + 1 < kt_last) {
-          tile_load<D>(kp, s.kv.rs, key0 + 128, T, rk);
-          tile_load<D>(vp, s.kv.rs, key0 + 128, T, rv);
+          fetch.load(kp, kt * 64 + 128, rk);
+          fetch.load(vp, kt * 64 + 128, rv);
         }
       }
-      const bool active = key0 <= wave_q0 + 31 && (s.window == 0 || key0 + 63 + s.window > wave_q0);
-      if (!active) continue;
-      floatx16 sc[2] = {zero16(), zero16()};
-#pragma unroll
-      for (int sub = 0; sub < 2; ++sub)
-#pragma unroll
-        for (int kk = 0; kk < KK; ++kk) sc[sub] = mfma(frag_rows<D>(k_rows, sub, kk, l32, lg), qf[kk], sc[sub]);
-      // Only a tile that crosses the diagonal, the sequence end or the window edge needs the mask
-      // (wave-uniform). `m` is the running maximum of the raw scores; the scale joins inside the fma.
-      if (s.window == 0 && key0 + 63 < T) {
-        // The diagonal alone: key > q_row is one compare of a constant with the lane's offset.
-        if (key0 + 63 > wave_q0) {
-          const int rel = q_row - key0 - 4 * lg;
-#pragma unroll
-          for (int sub = 0; sub < 2; ++sub)
-#pragma unroll
-            for (int vv = 0; vv < 16; ++vv) sc[sub][vv] = sub * 32 + acc_row(vv, 0) > rel ? -INFINITY : sc[sub][vv];
-        }
-      } else if (key0 + 63 > wave_q0 || key0 + 63 >= T || s.window > 0) {
-#pragma unroll
-        for (int sub = 0; sub < 2; ++sub)
-#pragma unroll
-          for (int vv = 0; vv < 16; ++vv) {
-            const int key = key0 + sub * 32 + acc_row(vv, lg);
-            const bool masked = key > q_row || key >= T || (s.window > 0 && key + s.window <= q_row);
-            sc[sub][vv] = masked ? -INFINITY : sc[sub][vv];
-          }
+    };
+    int kt = kt_first;
+    if constexpr (WIN) {
+      for (; kt <= kt_last; ++kt) {
+        advance(kt);
+        const int key0 = kt * 64;
+        if (key0 <= wave_q0 + 31 && key0 + 63 + s.window > wave_q0)
+          flash_fwd_tile<D, 2, -1, true>(k_rows, v_rows, qf, o, m, lsum, wsum, scale_log2, key0, q_row, T, s.window, lane);
       }
-      float tmax = fmaxf(sc[0][0], sc[1][0]);
-#pragma unroll
-      for (int vv = 1; vv < 16; ++vv) tmax = max3(tmax, sc[0][vv], sc[1][vv]);
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-      // The reference point of the exponents moves only when a row's maximum grew by more than 8
-      // binary orders (always on a row's first tile, where m is -inf): below that the weights of
-      // this tile are at most 2^8, well inside f32 and bf16, and the accumulators need no rescaling.
-      // The quotient at the end and the log-sum-exp use the same reference, so both stay exact.
-      const bool grow = (tmax - m) * scale_log2 > 8.0f;
-      const float new_m = grow ? tmax : m;
-      const float m_safe = new_m == -INFINITY ? 0.0f : new_m;
-      const float neg_m = -m_safe * scale_log2;
-      float psum = 0.0f;
-#pragma unroll
-      for (int sub = 0; sub < 2; ++sub)
-#pragma unroll
-        for (int vv = 0; vv < 16; ++vv) {
-          float p = __builtin_amdgcn_exp2f(fmaf(sc[sub][vv], scale_log2, neg_m));
-          sc[sub][vv] = p;
-          psum += p;
-        }
-      psum += __shfl_xor(psum, 32, 64);
-      if (__any(grow)) {
-        // Some row's reference moved: rescale what is accumulated so far (by exactly 1 in the
-        // rows that keep theirs).
-        const float alpha = __builtin_amdgcn_exp2f(fmaf(m, scale_log2, neg_m));
-        lsum *= alpha;
-        wsum *= alpha;
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-          for (int vv = 0; vv < 16; ++vv) o[mt][vv] *= alpha;
+    } else if (wave_q0 < T) {  // (a wave whose rows all lie past the sequence end only keeps the barriers)
+      // The wave's first query is a multiple of 32 and a tile's first key a multiple of 64, so the
+      // diagonal cuts exactly one 32 x 32 half of one tile, the wave's last: the first half of the tile
+      // that starts at the wave's first query (whose second half no row sees), or the second half of
+      // the tile that starts 32 keys earlier. The tiles before it need no mask, and their loop holds
+      // nothing else: one body, so the accumulators stay in the registers the matrix units update.
+      const int diag_kt = wave_q0 / 64;
+      for (; kt < diag_kt; ++kt) {
+        advance(kt);
+        flash_fwd_tile<D, 2, -1, false>(k_rows, v_rows, qf, o, m, lsum, wsum, scale_log2, kt * 64, q_row, T, 0, lane);
       }
-      lsum += psum;
-      m = new_m;
-#pragma unroll
-      for (int sub = 0; sub < 2; ++sub)
-#pragma unroll
-        for (int c = 0; c < 2; ++c) {
-          const u32x4 pb = pack8(sc[sub], c);
-          wsum = sum_pairs(pb.x, sum_pairs(pb.y, sum_pairs(pb.z, sum_pairs(pb.w, wsum))));
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt) o[mt] = mfma(frag_tr<D>(v_rows, mt, sub, c, lane), pb, o[mt]);
-        }
+      advance(kt);
+      const int key0 = kt * 64;
+      if (D > 64 || key0 + 63 >= T)  // (at head_dim 128 the two cut-tile forms cost registers the kernel does not have)
+        flash_fwd_tile<D, 2, -1, true>(k_rows, v_rows, qf, o, m, lsum, wsum, scale_log2, key0, q_row, T, 0, lane);
+      else if (key0 == wave_q0)
+        flash_fwd_tile<D, 1, 0, false>(k_rows, v_rows, qf, o, m, lsum, wsum, scale_log2, key0, q_row, T, 0, lane);
+      else
+        flash_fwd_tile<D, 2, 1, false>(k_rows, v_rows, qf, o, m, lsum, wsum, scale_log2, key0, q_row, T, 0, lane);
+      ++kt;
     }
-    wsum += __shfl_xor(wsum, 32, 64);
+    for (; kt <= kt_last; ++kt) advance(kt);  // tiles of the block's later waves (same barrier count for all)
+    wsum = halves_sum(wsum);
     bool bad = false;
     if (q_row < T) {
       bad |= !(dev_finite(lsum) && lsum > 0.0f && wsum > 0.0f);
@@ -394,12 +512,74 @@ __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_fwd_kernel(const un
 }
 
 // ------------------------------------------------------------------ backward: dK, dV
+// One 64-query x 32-key tile of one wave in the dK/dV pass. GENERAL: the tile crosses the diagonal,
+// the sequence end or a window edge and every element is tested (as in the dQ pass, the cheaper
+// forms of the cut tile would push the kernel past its registers).
+template <int D, bool WANT_DK, bool WANT_DV, bool GENERAL>
+__device__ __forceinline__ void flash_dkv_tile(const char* q_rows, const char* g_rows, const float* lse_s,
+                                               const float* del_s, const u32x4 (&kf)[D / 16],
+                                               const u32x4 (&vf)[WANT_DK ? D / 16 : 1], floatx16 (&dk)[WANT_DK ? D / 32 : 1],
+                                               floatx16 (&dv)[WANT_DV ? D / 32 : 1], float scale_log2, int q0, int key_row,
+                                               int T, int window, int lane) {
+  constexpr int KK = D / 16, MT = D / 32;
+  const int l32 = lane & 31, lg = lane >> 5;
+#pragma unroll
+  for (int sub = 0; sub < 2; ++sub) {
+    floatx16 sc = zero16(), dp = zero16();
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      sc = mfma(frag_rows<D>(q_rows, sub, kk, l32, lg), kf[kk], sc);
+      if constexpr (WANT_DK) dp = mfma(frag_rows<D>(g_rows, sub, kk, l32, lg), vf[kk], dp);
+    }
+    if constexpr (GENERAL) {
+#pragma unroll
+      for (int vv = 0; vv < 16; ++vv) {
+        const int qi = q0 + sub * 32 + acc_row(vv, lg);
+        const bool masked = key_row > qi || qi >= T || key_row >= T || (window > 0 && key_row + window <= qi);
+        sc[vv] = masked ? -INFINITY : sc[vv];
+      }
+    }
+    // P = 2^(s * scale * log2e - lse * log2e); dS / scale = P (dP - delta): the scale joins dK at the end.
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      const float4 l4 = *reinterpret_cast<const float4*>(lse_s + sub * 32 + 8 * q4 + 4 * lg);
+      const float lv[4] = {l4.x, l4.y, l4.z, l4.w};
+      float dl[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+      if constexpr (WANT_DK) {
+        const float4 d4 = *reinterpret_cast<const float4*>(del_s + sub * 32 + 8 * q4 + 4 * lg);
+        dl[0] = d4.x;
+        dl[1] = d4.y;
+        dl[2] = d4.z;
+        dl[3] = d4.w;
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int vv = 4 * q4 + j;
+        const float p = __builtin_amdgcn_exp2f(fmaf(sc[vv], scale_log2, -lv[j]));
+        if constexpr (WANT_DK) dp[vv] = p * (dp[vv] - dl[j]);
+        sc[vv] = p;
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      u32x4 pb = u32x4{0u, 0u, 0u, 0u}, dsb = u32x4{0u, 0u, 0u, 0u};
+      if constexpr (WANT_DV) pb = pack8(sc, c);
+      if constexpr (WANT_DK) dsb = pack8(dp, c);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        if constexpr (WANT_DV) dv[mt] = mfma(frag_tr<D>(g_rows, mt, sub, c, lane), pb, dv[mt]);
+        if constexpr (WANT_DK) dk[mt] = mfma(frag_tr<D>(q_rows, mt, sub, c, lane), dsb, dk[mt]);
+      }
+    }
+  }
+}
+
 // One key block of one KV head: the loop over the query tiles that see it, accumulating dK
 // (WANT_DK) and / or dV (WANT_DV) for the wave's 32 keys, then their stores. head_dim 64 runs it
 // once for both. At head_dim 128 the two accumulator sets (128 registers), both key / value
 // fragments (64) and the score tiles do not fit the 256 registers of two waves per SIMD, so the
 // block is walked twice, once per gradient; the second walk recomputes the scores.
-template <int D, typename TO, bool WANT_DK, bool WANT_DV>
+template <int D, typename TO, bool WANT_DK, bool WANT_DV, bool WIN>
 __device__ __forceinline__ bool flash_dkv_block(const unsigned short* __restrict__ q,
                                                 const unsigned short* __restrict__ k,
                                                 const unsigned short* __restrict__ v, const float* __restrict__ lse,
@@ -408,8 +588,9 @@ __device__ __forceinline__ bool flash_dkv_block(const unsigned short* __restrict
                                                 int kb, int b, int gidx) {
   constexpr int KK = D / 16, MT = D / 32, NL = D / 32;
   constexpr int SET = 2 * ftile(D) + 2 * 64 * 4;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lg = lane >> 5;
+  const int lane = threadIdx.x & 63, wave = wave_index(), l32 = lane & 31, lg = lane >> 5;
   const int T = s.time;
+  const TileFetch<D> fetch_q(s.q.rs, T), fetch_g(s.o.rs, T);
   const long kv_off = b * s.kv.bs + gidx * s.kv.hs;
   const int wave_k0 = kb * 128 + wave * 32;
   const int key_row = wave_k0 + l32;
@@ -426,14 +607,14 @@ __device__ __forceinline__ bool flash_dkv_block(const unsigned short* __restrict
   const int qt_first = block_k0 / 64;
   const int qt_last = (s.window > 0 ? min(T - 1, block_k1 + s.window - 1) : T - 1) / 64;
   bool bad = false;
-  // One flat loop over (query head of the group, query tile), ascending, so the
+  // One flat sequence of (query head of the group, query tile), ascending, so the
   // next tile's global loads can be in flight while the current one is multiplied.
   const int nq = qt_last - qt_first + 1;
   const int steps = s.rep * nq;
   u32x4 rq[NL], rg[NL];
   float row_lse = 0.0f, row_del = 0.0f;
-  // (head of the group, query tile) of the tile being fetched / being multiplied.
-  int fetch_r = 0, fetch_qt = qt_first, cur_qt = qt_first;
+  // (head of the group, query tile) of the tile being fetched.
+  int fetch_r = 0, fetch_qt = qt_first;
   auto fetch = [&]() {
     const int r = fetch_r, q0 = fetch_qt * 64;
     if (++fetch_qt > qt_last) {
@@ -442,8 +623,8 @@ __device__ __forceinline__ bool flash_dkv_block(const unsigned short* __restrict
     }
     const long q_plane = static_cast<long>(b) * s.heads + static_cast<long>(gidx) * s.rep + r;
     const long head = static_cast<long>(gidx) * s.rep + r;
-    tile_load<D>(q + b * s.q.bs + head * s.q.hs, s.q.rs, q0, T, rq);
-    tile_load<D>(gy + b * s.o.bs + head * s.o.hs, s.o.rs, q0, T, rg);
+    fetch_q.load(q + b * s.q.bs + head * s.q.hs, q0, rq);
+    fetch_g.load(gy + b * s.o.bs + head * s.o.hs, q0, rg);
     row_lse = 0.0f;
     row_del = 0.0f;
     if (threadIdx.x < 64 && q0 + static_cast<int>(threadIdx.x) < T) {
@@ -465,84 +646,64 @@ __device__ __forceinline__ bool flash_dkv_block(const unsigned short* __restrict
   __syncthreads();  // an earlier walk's reads of the first set are done
   store_set(smem);
   if (steps > 1) fetch();
-  for (int idx = 0; idx < steps; ++idx) {
-    const int q0 = cur_qt * 64;
-    if (++cur_qt > qt_last) cur_qt = qt_first;
-    char* q_rows = smem + (idx & 1) * SET;
-    char* g_rows = q_rows + ftile(D);
-    const float* lse_s = reinterpret_cast<const float*>(q_rows + 2 * ftile(D));
-    const float* del_s = lse_s + 64;
+  // One step of the tile pipeline, taken by every wave for every tile: wait for set idx, store the
+  // next one into the other set, start the loads of the one after.
+  int idx = 0;
+  const char* q_rows;
+  const char* g_rows;
+  const float* lse_s;
+  const float* del_s;
+  auto advance = [&]() {
+    q_rows = smem + (idx & 1) * SET;
+    g_rows = q_rows + ftile(D);
+    lse_s = reinterpret_cast<const float*>(q_rows + 2 * ftile(D));
+    del_s = lse_s + 64;
     __syncthreads();  // this set is complete, and every wave is done with the other one
     if (idx + 1 < steps) {
       store_set(smem + ((idx & 1) ^ 1) * SET);
       if (idx + 2 < steps) fetch();
     }
-    const bool active = q0 + 63 >= wave_k0 && (s.window == 0 || q0 < wave_k0 + 31 + s.window);
-    if (!active) continue;
-    // Wave-uniform: a tile whose queries all come after the wave's keys and end inside the sequence has no mask.
-    const bool needs_mask = q0 < wave_k0 + 31 || q0 + 63 >= T || s.window > 0;
-    // Wave-uniform: the tile and the wave's keys end inside the sequence and only the diagonal cuts it.
-    const bool diagonal_only = needs_mask && s.window == 0 && q0 + 63 < T && wave_k0 + 31 < T;
-#pragma unroll
-    for (int sub = 0; sub < 2; ++sub) {
-      floatx16 sc = zero16(), dp = zero16();
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk) {
-        sc = mfma(frag_rows<D>(q_rows, sub, kk, l32, lg), kf[kk], sc);
-        if constexpr (WANT_DK) dp = mfma(frag_rows<D>(g_rows, sub, kk, l32, lg), vf[kk], dp);
+    ++idx;
+  };
+  auto tile = [&](auto general, int q0) {
+    flash_dkv_tile<D, WANT_DK, WANT_DV, decltype(general)::value>(q_rows, g_rows, lse_s, del_s, kf, vf, dk, dv, scale_log2, q0,
+                                                                 key_row, T, s.window, lane);
+  };
+  for (int r = 0; r < s.rep; ++r) {
+    int qt = qt_first;
+    if constexpr (WIN) {
+      for (; qt <= qt_last; ++qt) {
+        advance();
+        const int q0 = qt * 64;
+        if (q0 + 63 >= wave_k0 && q0 < wave_k0 + 31 + s.window) tile(std::true_type{}, q0);
       }
-      if (diagonal_only) {
-        const int rel = key_row - q0 - 4 * lg;  // key_row > query: a constant against the lane's offset
-#pragma unroll
-        for (int vv = 0; vv < 16; ++vv) sc[vv] = sub * 32 + acc_row(vv, 0) < rel ? -INFINITY : sc[vv];
-      } else if (needs_mask) {
-#pragma unroll
-        for (int vv = 0; vv < 16; ++vv) {
-          const int qi = q0 + sub * 32 + acc_row(vv, lg);
-          const bool masked = key_row > qi || qi >= T || key_row >= T || (s.window > 0 && key_row + s.window <= qi);
-          sc[vv] = masked ? -INFINITY : sc[vv];
-        }
+    } else if (wave_k0 < T) {  // (a wave whose keys all lie past the sequence end only keeps the barriers)
+      // The wave's first key is a multiple of 32 and a tile's first query a multiple of 64, so the
+      // diagonal cuts one tile, the first the wave takes. The tiles after it need no mask until the
+      // sequence ends inside one, or inside the wave's keys; their loop holds nothing else.
+      const int diag_qt = wave_k0 / 64;
+      for (; qt < diag_qt; ++qt) advance();  // tiles of the block's earlier waves
+      advance();
+      tile(std::true_type{}, qt * 64);
+      ++qt;
+      const int plain_last = wave_k0 + 31 >= T ? qt - 1 : (T / 64) - 1;  // the last tile that ends inside the sequence
+      for (; qt <= min(plain_last, qt_last); ++qt) {
+        advance();
+        tile(std::false_type{}, qt * 64);
       }
-      // P = 2^(s * scale * log2e - lse * log2e); dS / scale = P (dP - delta): the scale joins dK at the end.
-#pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        const float4 l4 = *reinterpret_cast<const float4*>(lse_s + sub * 32 + 8 * q4 + 4 * lg);
-        const float lv[4] = {l4.x, l4.y, l4.z, l4.w};
-        float dl[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        if constexpr (WANT_DK) {
-          const float4 d4 = *reinterpret_cast<const float4*>(del_s + sub * 32 + 8 * q4 + 4 * lg);
-          dl[0] = d4.x;
-          dl[1] = d4.y;
-          dl[2] = d4.z;
-          dl[3] = d4.w;
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int vv = 4 * q4 + j;
-          const float p = __builtin_amdgcn_exp2f(fmaf(sc[vv], scale_log2, -lv[j]));
-          if constexpr (WANT_DK) dp[vv] = p * (dp[vv] - dl[j]);
-          sc[vv] = p;
-        }
-      }
-#pragma unroll
-      for (int c = 0; c < 2; ++c) {
-        u32x4 pb = u32x4{0u, 0u, 0u, 0u}, dsb = u32x4{0u, 0u, 0u, 0u};
-        if constexpr (WANT_DV) pb = pack8(sc, c);
-        if constexpr (WANT_DK) dsb = pack8(dp, c);
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          if constexpr (WANT_DV) dv[mt] = mfma(frag_tr<D>(g_rows, mt, sub, c, lane), pb, dv[mt]);
-          if constexpr (WANT_DK) dk[mt] = mfma(frag_tr<D>(q_rows, mt, sub, c, lane), dsb, dk[mt]);
-        }
+      for (; qt <= qt_last; ++qt) {
+        advance();
+        tile(std::true_type{}, qt * 64);
       }
     }
+    for (; qt <= qt_last; ++qt) advance();
   }
   if constexpr (WANT_DK) bad |= store_transposed_acc<D, TO>(gk + kv_off, s.kv.rs, key_row, T, lg, dk, s.scale);
   if constexpr (WANT_DV) bad |= store_transposed_acc<D, TO>(gv + kv_off, s.kv.rs, key_row, T, lg, dv, 1.0f);
   return bad;
 }
 
-template <int D, typename TO>
+template <int D, typename TO, bool WIN>
 __global__ __launch_bounds__(FT, 2) void flash_bwd_dkv_kernel(
     const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
     const float* __restrict__ lse, const float* __restrict__ delta, const unsigned short* __restrict__ gy,
@@ -567,10 +728,10 @@ __global__ __launch_bounds__(FT, 2) void flash_bwd_dkv_kernel(
     const int kb = pass == 0 ? pair : k_blocks - 1 - pair;
     if (pass == 1 && kb <= pair) break;
     if constexpr (D == 64) {
-      bad |= flash_dkv_block<D, TO, true, true>(q, k, v, lse, delta, gy, gk, gv, s, smem, kb, b, gidx);
+      bad |= flash_dkv_block<D, TO, true, true, WIN>(q, k, v, lse, delta, gy, gk, gv, s, smem, kb, b, gidx);
     } else {
-      bad |= flash_dkv_block<D, TO, false, true>(q, k, v, lse, delta, gy, gk, gv, s, smem, kb, b, gidx);
-      bad |= flash_dkv_block<D, TO, true, false>(q, k, v, lse, delta, gy, gk, gv, s, smem, kb, b, gidx);
+      bad |= flash_dkv_block<D, TO, false, true, WIN>(q, k, v, lse, delta, gy, gk, gv, s, smem, kb, b, gidx);
+      bad |= flash_dkv_block<D, TO, true, false, WIN>(q, k, v, lse, delta, gy, gk, gv, s, smem, kb, b, gidx);
     }
   }
   if (bad) dev_raise_fault(fault, tag);
@@ -612,7 +773,50 @@ __global__ __launch_bounds__(256) void flash_key_mean_kernel(const unsigned shor
 }
 
 // ------------------------------------------------------------------ backward: dQ
-template <int D, typename TO>
+// One 32-query x 64-key tile of one wave in the dQ pass. GENERAL: the tile crosses the diagonal,
+// the sequence end or a window edge and every element is tested (the forward's cheaper forms of
+// the cut tile cost registers this kernel does not have: with them it spills, and runs 11 % slower).
+// dS / scale = P (dP - delta) goes into dQ^T through the matrix units, and `ds_sum` collects this
+// lane's share of the row sum of its bf16 copy.
+template <int D, bool GENERAL>
+__device__ __forceinline__ void flash_dq_tile(const char* k_rows, const char* v_rows, const u32x4 (&qf)[D / 16],
+                                              const u32x4 (&gf)[D / 16], floatx16 (&dq)[D / 32], float& ds_sum,
+                                              float scale_log2, float neg_lse, float row_del, int key0, int q_row, int T,
+                                              int window, int lane) {
+  constexpr int KK = D / 16, MT = D / 32;
+  const int l32 = lane & 31, lg = lane >> 5;
+#pragma unroll
+  for (int sub = 0; sub < 2; ++sub) {
+    floatx16 sc = zero16(), dp = zero16();
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      sc = mfma(frag_rows<D>(k_rows, sub, kk, l32, lg), qf[kk], sc);
+      dp = mfma(frag_rows<D>(v_rows, sub, kk, l32, lg), gf[kk], dp);
+    }
+    if constexpr (GENERAL) {
+#pragma unroll
+      for (int vv = 0; vv < 16; ++vv) {
+        const int key = key0 + sub * 32 + acc_row(vv, lg);
+        const bool masked = key > q_row || key >= T || q_row >= T || (window > 0 && key + window <= q_row);
+        sc[vv] = masked ? -INFINITY : sc[vv];
+      }
+    }
+#pragma unroll
+    for (int vv = 0; vv < 16; ++vv) {
+      const float p = __builtin_amdgcn_exp2f(fmaf(sc[vv], scale_log2, neg_lse));
+      dp[vv] = p * (dp[vv] - row_del);  // dS / scale: the scale joins dQ at the end
+    }
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const u32x4 dsb = pack8(dp, c);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) dq[mt] = mfma(frag_tr<D>(k_rows, mt, sub, c, lane), dsb, dq[mt]);
+      ds_sum = sum_pairs(dsb.x, sum_pairs(dsb.y, sum_pairs(dsb.z, sum_pairs(dsb.w, ds_sum))));
+    }
+  }
+}
+
+template <int D, typename TO, bool WIN>
 __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_bwd_dq_kernel(
     const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
     const unsigned short* __restrict__ out, const unsigned short* __restrict__ resid, const float* __restrict__ lse,
@@ -621,8 +825,9 @@ __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_bwd_dq_kernel(
   constexpr int KK = D / 16, MT = D / 32, NL = D / 32;
   // Two key / value tile pairs, as in the forward: one barrier per tile.
   __shared__ __attribute__((aligned(16))) char smem[4 * ftile(D)];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lg = lane >> 5;
+  const int lane = threadIdx.x & 63, wave = wave_index(), l32 = lane & 31, lg = lane >> 5;
   const int T = s.time;
+  const TileFetch<D> fetch(s.kv.rs, T);
   // A late query block, then its mirror image from the front (see the forward kernel).
   const int q_blocks = (T + 127) / 128;
   int pair;
@@ -668,7 +873,7 @@ __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_bwd_dq_kernel(
       };
       row_del = dot_rows(out);
       if (resid) row_del += dot_rows(resid);
-      row_del += __shfl_xor(row_del, 32, 64);
+      row_del = halves_sum(row_del);
     }
     float row_lse = 0.0f;
     bool bad = false;
@@ -692,72 +897,57 @@ __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_bwd_dq_kernel(
     const int kt_first = s.window > 0 ? max(0, block_q0 + 1 - s.window) / 64 : 0;
     const int kt_last = block_q1 / 64;
     u32x4 rk[NL], rv[NL];
-    tile_load<D>(kp, s.kv.rs, kt_first * 64, T, rk);
-    tile_load<D>(vp, s.kv.rs, kt_first * 64, T, rv);
+    fetch.load(kp, kt_first * 64, rk);
+    fetch.load(vp, kt_first * 64, rv);
     __syncthreads();  // the previous pass's reads of the first pair are done
     tile_store_rows<D>(smem, rk);
     tile_store_rows<D>(smem + ftile(D), rv);
     if (kt_first < kt_last) {
-      tile_load<D>(kp, s.kv.rs, kt_first * 64 + 64, T, rk);
-      tile_load<D>(vp, s.kv.rs, kt_first * 64 + 64, T, rv);
+      fetch.load(kp, kt_first * 64 + 64, rk);
+      fetch.load(vp, kt_first * 64 + 64, rv);
     }
-    for (int kt = kt_first; kt <= kt_last; ++kt) {
-      const int key0 = kt * 64;
+    // The tile pipeline and the split into unmasked tiles, the wave's diagonal tile and the other
+    // waves' tiles are the forward kernel's.
+    const char* k_rows;
+    const char* v_rows;
+    auto advance = [&](int kt) {
       const int cur = (kt - kt_first) & 1;
-      char* k_rows = smem + cur * 2 * ftile(D);
-      char* v_rows = k_rows + ftile(D);
+      k_rows = smem + cur * 2 * ftile(D);
+      v_rows = k_rows + ftile(D);
       __syncthreads();  // this pair is complete, and every wave is done with the other one
       if (kt < kt_last) {
         char* next = smem + (cur ^ 1) * 2 * ftile(D);
         tile_store_rows<D>(next, rk);
         tile_store_rows<D>(next + ftile(D), rv);
         if (kt + 1 < kt_last) {
-          tile_load<D>(kp, s.kv.rs, key0 + 128, T, rk);
-          tile_load<D>(vp, s.kv.rs, key0 + 128, T, rv);
+          fetch.load(kp, kt * 64 + 128, rk);
+          fetch.load(vp, kt * 64 + 128, rv);
         }
       }
-      const bool active = key0 <= wave_q0 + 31 && (s.window == 0 || key0 + 63 + s.window > wave_q0);
-      if (!active) continue;
-      const bool needs_mask = key0 + 63 > wave_q0 || key0 + 63 >= T || s.window > 0;
-      // Wave-uniform: the tile and the wave's rows end inside the sequence and only the diagonal cuts it.
-      const bool diagonal_only = needs_mask && s.window == 0 && key0 + 63 < T && wave_q0 + 31 < T;
-#pragma unroll
-      for (int sub = 0; sub < 2; ++sub) {
-        floatx16 sc = zero16(), dp = zero16();
-#pragma unroll
-        for (int kk = 0; kk < KK; ++kk) {
-          sc = mfma(frag_rows<D>(k_rows, sub, kk, l32, lg), qf[kk], sc);
-          dp = mfma(frag_rows<D>(v_rows, sub, kk, l32, lg), gf[kk], dp);
-        }
-        if (diagonal_only) {
-          const int rel = q_row - key0 - 4 * lg;  // key > q_row: a constant against the lane's offset
-#pragma unroll
-          for (int vv = 0; vv < 16; ++vv) sc[vv] = sub * 32 + acc_row(vv, 0) > rel ? -INFINITY : sc[vv];
-        } else if (needs_mask) {
-#pragma unroll
-          for (int vv = 0; vv < 16; ++vv) {
-            const int key = key0 + sub * 32 + acc_row(vv, lg);
-            const bool masked = key > q_row || key >= T || q_row >= T || (s.window > 0 && key + s.window <= q_row);
-            sc[vv] = masked ? -INFINITY : sc[vv];
-          }
-        }
-#pragma unroll
-        for (int vv = 0; vv < 16; ++vv) {
-          const float p = __builtin_amdgcn_exp2f(fmaf(sc[vv], scale_log2, neg_lse));
-          dp[vv] = p * (dp[vv] - row_del);  // dS / scale: the scale joins dQ at the end
-        }
-#pragma unroll
-        for (int c = 0; c < 2; ++c) {
-          const u32x4 dsb = pack8(dp, c);
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt) dq[mt] = mfma(frag_tr<D>(k_rows, mt, sub, c, lane), dsb, dq[mt]);
-          ds_sum = sum_pairs(dsb.x, sum_pairs(dsb.y, sum_pairs(dsb.z, sum_pairs(dsb.w, ds_sum))));
-        }
+    };
+    int kt = kt_first;
+    if constexpr (WIN) {
+      for (; kt <= kt_last; ++kt) {
+        advance(kt);
+        const int key0 = kt * 64;
+        if (key0 <= wave_q0 + 31 && key0 + 63 + s.window > wave_q0)
+          flash_dq_tile<D, true>(k_rows, v_rows, qf, gf, dq, ds_sum, scale_log2, neg_lse, row_del, key0, q_row, T, s.window,
+                                 lane);
       }
+    } else if (wave_q0 < T) {
+      const int diag_kt = wave_q0 / 64;
+      for (; kt < diag_kt; ++kt) {
+        advance(kt);
+        flash_dq_tile<D, false>(k_rows, v_rows, qf, gf, dq, ds_sum, scale_log2, neg_lse, row_del, kt * 64, q_row, T, 0, lane);
+      }
+      advance(kt);
+      flash_dq_tile<D, true>(k_rows, v_rows, qf, gf, dq, ds_sum, scale_log2, neg_lse, row_del, kt * 64, q_row, T, 0, lane);
+      ++kt;
     }
+    for (; kt <= kt_last; ++kt) advance(kt);  // tiles of the block's later waves (same barrier count for all)
     {
       const float* mean = key_mean + (static_cast<long>(b) * s.kv_heads + kvh) * D;
-      const float row_sum = ds_sum + __shfl_xor(ds_sum, 32, 64);  // the two half-waves hold half the keys each
+      const float row_sum = halves_sum(ds_sum);  // the two half-waves hold half the keys each
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -821,13 +1011,18 @@ void launch_forward(omx_ctx* ctx, const unsigned short* q, const unsigned short*
   dim3 grid((s.q_single ? q_blocks : (q_blocks + 1) / 2) * planes), block(FT);
   // Causal-counted work: half of the 4 B H T^2 D of the two full products.
   OmxKernelTimer timer(ctx, OMX_K_FLASH_FWD, 2.0 * s.batch * s.heads * static_cast<double>(s.time) * s.time * D);
-  if (out_dtype == OMX_BF16)
-    omx_launch_timed(ctx, flash_fwd_kernel<D, unsigned short>, grid, block, 0, timer.start(), timer.stop(), q, k, v,
-                     static_cast<unsigned short*>(out), static_cast<unsigned short*>(out_residual), lse, s, ctx->fault,
-                     tag);
-  else
-    omx_launch_timed(ctx, flash_fwd_kernel<D, float>, grid, block, 0, timer.start(), timer.stop(), q, k, v,
-                     static_cast<float*>(out), static_cast<unsigned short*>(nullptr), lse, s, ctx->fault, tag);
+  auto go = [&](auto kernel, auto* out_ptr, unsigned short* resid_ptr) {
+    omx_launch_timed(ctx, kernel, grid, block, 0, timer.start(), timer.stop(), q, k, v, out_ptr, resid_ptr, lse, s,
+                     ctx->fault, tag);
+  };
+  unsigned short* resid = static_cast<unsigned short*>(out_residual);
+  if (out_dtype == OMX_BF16) {
+    if (s.window > 0) go(flash_fwd_kernel<D, unsigned short, true>, static_cast<unsigned short*>(out), resid);
+    else go(flash_fwd_kernel<D, unsigned short, false>, static_cast<unsigned short*>(out), resid);
+  } else {
+    if (s.window > 0) go(flash_fwd_kernel<D, float, true>, static_cast<float*>(out), static_cast<unsigned short*>(nullptr));
+    else go(flash_fwd_kernel<D, float, false>, static_cast<float*>(out), static_cast<unsigned short*>(nullptr));
+  }
 }
 
 template <int D>
@@ -849,18 +1044,36 @@ void launch_backward(omx_ctx* ctx, const unsigned short* q, const unsigned short
   s.kv_single = flash_single(ctx, pairs * kv_planes, 2, true);
   dim3 kv_grid((s.kv_single ? blocks : pairs) * kv_planes);
   dim3 q_grid((s.q_single ? blocks : pairs) * q_planes);
+  auto go = [&](auto dq_kernel, auto dkv_kernel, auto* gq_ptr, auto* gk_ptr, auto* gv_ptr) {
+    hipLaunchKernelGGL(dq_kernel, q_grid, block, 0, ctx->stream, q, k, v, out, resid, lse, delta, key_mean, gy, gq_ptr, s,
+                       ctx->fault, tag);
+    omx_launch_timed(ctx, dkv_kernel, kv_grid, block, 0, nullptr, timer.stop(), q, k, v, lse, delta, gy, gk_ptr, gv_ptr, s,
+                     ctx->fault, tag);
+  };
   if (grad_dtype == OMX_BF16) {
-    hipLaunchKernelGGL((flash_bwd_dq_kernel<D, unsigned short>), q_grid, block, 0, ctx->stream, q, k, v, out, resid,
-                       lse, delta, key_mean, gy, static_cast<unsigned short*>(gq), s, ctx->fault, tag);
-    omx_launch_timed(ctx, flash_bwd_dkv_kernel<D, unsigned short>, kv_grid, block, 0, nullptr, timer.stop(), q, k, v,
-                     lse, delta, gy, static_cast<unsigned short*>(gk), static_cast<unsigned short*>(gv), s, ctx->fault,
-                     tag);
+    typedef unsigned short T16;
+    if (s.window > 0)
+      go(flash_bwd_dq_kernel<D, T16, true>, flash_bwd_dkv_kernel<D, T16, true>, static_cast<T16*>(gq), static_cast<T16*>(gk),
+         static_cast<T16*>(gv));
+    else
+      go(flash_bwd_dq_kernel<D, T16, false>, flash_bwd_dkv_kernel<D, T16, false>, static_cast<T16*>(gq),
+         static_cast<T16*>(gk), static_cast<T16*>(gv));
   } else {
-    hipLaunchKernelGGL((flash_bwd_dq_kernel<D, float>), q_grid, block, 0, ctx->stream, q, k, v, out, resid, lse, delta,
-                       key_mean, gy, static_cast<float*>(gq), s, ctx->fault, tag);
-    omx_launch_timed(ctx, flash_bwd_dkv_kernel<D, float>, kv_grid, block, 0, nullptr, timer.stop(), q, k, v, lse, delta,
-                     gy, static_cast<float*>(gk), static_cast<float*>(gv), s, ctx->fault, tag);
+    if (s.window > 0)
+      go(flash_bwd_dq_kernel<D, float, true>, flash_bwd_dkv_kernel<D, float, true>, static_cast<float*>(gq),
+         static_cast<float*>(gk), static_cast<float*>(gv));
+    else
+      go(flash_bwd_dq_kernel<D, float, false>, flash_bwd_dkv_kernel<D, float, false>, static_cast<float*>(gq),
+         static_cast<float*>(gk), static_cast<float*>(gv));
   }
+}
+
+// The tile loads add a thread's rows as a 32-bit byte offset to a scalar base.
+int32_t check_row_strides(omx_ctx* ctx, const FlashShape& s) {
+  for (long rs : {s.q.rs, s.kv.rs, s.o.rs})
+    if (rs < 1 || rs > FLASH_MAX_ROW_STRIDE)
+      return omx_fail(ctx, OMX_SHAPE, "flash attention: row stride %ld outside 1..%ld elements", rs, FLASH_MAX_ROW_STRIDE);
+  return OMX_OK;
 }
 
 }  // namespace
@@ -877,6 +1090,7 @@ int32_t omx_flash_sdpa_forward(omx_ctx* ctx, const void* q, const void* k, const
     return omx_fail(ctx, OMX_UNSUPPORTED_HEAD_DIM, "head_dim %llu: the MFMA kernels take 64 and 128",
                     (unsigned long long)dim);
   FlashShape s = make_shape(batch, heads, kv_heads, time, dim, window, scale, strides);
+  if (int32_t rc = check_row_strides(ctx, s); rc != OMX_OK) return rc;
   const unsigned short* qs = static_cast<const unsigned short*>(q);
   const unsigned short* ks = static_cast<const unsigned short*>(k);
   const unsigned short* vs = static_cast<const unsigned short*>(v);
@@ -895,6 +1109,7 @@ int32_t omx_flash_sdpa_backward(omx_ctx* ctx, const void* q, const void* k, cons
     return omx_fail(ctx, OMX_UNSUPPORTED_HEAD_DIM, "head_dim %llu: the MFMA kernels take 64 and 128",
                     (unsigned long long)dim);
   FlashShape s = make_shape(batch, heads, kv_heads, time, dim, window, scale, strides);
+  if (int32_t rc = check_row_strides(ctx, s); rc != OMX_OK) return rc;
   const long rows = static_cast<long>(batch * heads * time);
   void* ws = nullptr;
   const long rows4 = (rows + 3) & ~3L;  // the mean key rows are read four values at a time
