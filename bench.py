@@ -97,6 +97,17 @@ def median_of(runs):
     return runs[len(runs) // 2]
 
 
+def timed(fn, inner: int = 1):
+    """(median seconds of `inner` calls of fn, its last result). The host is shared: a single timing of
+    a one-second piece is off by 10-20 % now and then, the median of three rarely."""
+    ts, result = [], None
+    for _ in range(inner):
+        t0 = time.perf_counter()
+        result = fn()
+        ts.append(time.perf_counter() - t0)
+    return median_of(sorted(ts)), result
+
+
 def spread_of(runs):
     """(max - min) / median of sorted timings."""
     return (runs[-1] - runs[0]) / median_of(runs)
@@ -112,8 +123,9 @@ def cpu_baseline(cfg, threads: int):
     norm, the head over the real vocabulary) from the one-block model at the real vocabulary minus a
     block, and the optimizer (clip + AdamW) from one block's parameters scaled by the parameter
     count. A configuration small enough (the tiny one) is timed whole instead. All cores (the
-    thread count is set explicitly) and one thread, one untimed run then five timed ones each;
-    `value` is the median of the all-cores runs, `spread` their (max - min) / median."""
+    thread count is set explicitly) and one thread, one untimed run then five timed ones each; in the
+    all-cores runs every model's time is itself the median of three calls. `value` is the median of
+    the all-cores runs, `spread` their (max - min) / median."""
     sys.path.insert(0, str(ROOT / "tests"))
     import oracle_api as orc
     from ojas_amd.trainer import GptConfig, synthetic_batch
@@ -139,7 +151,7 @@ def cpu_baseline(cfg, threads: int):
             orc.adamw_step(p, g, m, v, 0, 3e-4, 0.9, 0.95, 1e-8, 0.1, exact=True)
         return time.perf_counter() - t0
 
-    def measure(n_threads, sample_ctx):
+    def measure(n_threads, sample_ctx, inner):
         orc.set_threads(n_threads)
         if whole:
             ocfg, params, ids, targets = model(cfg.layers, cfg.batch, cfg.ctx)
@@ -157,11 +169,7 @@ def cpu_baseline(cfg, threads: int):
         block_params = [p for p in one[1][2:-1]]  # the block's eight tensors
 
         def once():
-            t = []
-            for ocfg, params, ids, targets in (small_one, small_three, one):
-                t0 = time.perf_counter()
-                orc.gpt_loss_and_grads(ocfg, params, ids, targets)
-                t.append(time.perf_counter() - t0)
+            t = [timed(lambda m=m: orc.gpt_loss_and_grads(*m), inner)[0] for m in (small_one, small_three, one)]
             block = max((t[1] - t[0]) / 2, 1e-9)
             rest = max(t[2] - block, 0.0)
             opt = optimizer_seconds(block_params, [np.full_like(p, 1e-3) for p in block_params])
@@ -173,8 +181,8 @@ def cpu_baseline(cfg, threads: int):
                       f"(the rest) on 1x{sample_ctx} tokens, clip + AdamW on one block's parameters, scaled to "
                       f"{cfg.layers} blocks, {tokens} tokens and {n_params} parameters")
 
-    all_runs, how = measure(threads, 512)
-    one_runs, how_one = measure(1, 64)
+    all_runs, how = measure(threads, 512, 3)
+    one_runs, how_one = measure(1, 64, 1)
     note = ("" if whole else " Attention grows with the sequence: at these sample lengths it is a smaller share than at "
             f"{cfg.ctx}, so the estimate favours the CPU by up to its 8 % of the step's work.")
     median, spread = median_of, spread_of
@@ -294,64 +302,68 @@ def lora_cpu_baseline(cfg, threads: int):
     """Times the oracle's LoRA step on a bounded sample of the same model at full width: one short
     sequence, once with one block and once with two; the difference is a block's time, the rest the
     table, final norm and head; the step is tokens x (rest + layers x block) / sample tokens plus
-    clip + AdamW on the adapters (timed on the two-block model's, scaled by their count). All cores
-    and one thread, five repeats each; `value` is the median of the all-cores runs."""
+    clip + AdamW on the adapters (timed on one block's, scaled by their count). The block's time comes
+    from a small-vocabulary pair of models, as in `cpu_baseline`. All cores and one thread, one
+    untimed run then five timed ones each; `value` is the median of the all-cores runs."""
     sys.path.insert(0, str(ROOT / "tests"))
     import oracle_api as orc
 
     tokens = cfg.batch * cfg.seq
     rng = np.random.default_rng(0)
 
-    def model(layers, seq):
-        ocfg = orc.LoraConfig(layers, cfg.d_model, cfg.heads, cfg.head_dim, cfg.hidden, cfg.vocab, 1, seq, cfg.rank,
+    def model(layers, seq, vocab):
+        ocfg = orc.LoraConfig(layers, cfg.d_model, cfg.heads, cfg.head_dim, cfg.hidden, vocab, 1, seq, cfg.rank,
                               cfg.rms_eps, cfg.lora_scale, cfg.rope_base)
         frozen = []
         for shape in orc.lora_frozen_shapes(ocfg):
             if len(shape) == 1:
                 frozen.append(np.ones(shape, np.float32))
-            elif shape[0] == cfg.vocab:
+            elif shape[0] == vocab:
                 frozen.append(rng.normal(0, 0.02, shape).astype(np.float32))
             else:  # codes and scales drawn directly: the values a quantised N(0, 0.02) matrix dequantises to
                 codes = rng.integers(-127, 128, shape).astype(np.int8)
                 scales = np.full((shape[0], shape[1] // 32), 0.05 / 127, np.float32)
                 frozen.append(orc.dequant_i8_group(codes, scales, 32))
         adapters = [rng.normal(0, 0.02, sh).astype(np.float32) for sh in orc.lora_adapter_shapes(ocfg)]
-        ids = rng.integers(0, cfg.vocab, seq).astype(np.uint32)
-        targets = rng.integers(0, cfg.vocab, seq).astype(np.uint32)
+        ids = rng.integers(0, vocab, seq).astype(np.uint32)
+        targets = rng.integers(0, vocab, seq).astype(np.uint32)
         return ocfg, frozen, adapters, ids, targets
 
-    def measure(n_threads, seq):
+    def measure(n_threads, seq, inner):
         orc.set_threads(n_threads)
-        one, two = model(1, seq), model(2, seq)
+        # A block's time from one and three blocks over a 256-entry vocabulary (the head is then a
+        # negligible part of both timings); the rest from one block over the real vocabulary. Every
+        # model's time is the median of `inner` calls.
+        small_one, small_three, one = model(1, seq, 256), model(3, seq, 256), model(1, seq, cfg.vocab)
 
         def once():
             t = []
-            for ocfg, frozen, adapters, ids, targets in (one, two):
-                t0 = time.perf_counter()
-                _, grads = orc.lora_loss_and_grads(ocfg, frozen, adapters, ids, targets)
-                t.append(time.perf_counter() - t0)
-            flat = [a.reshape(-1).copy() for a in two[2]]
+            for m in (small_one, small_three, one):
+                dt, (_, grads) = timed(lambda m=m: orc.lora_loss_and_grads(*m), inner)
+                t.append(dt)
+            flat = [a.reshape(-1).copy() for a in one[2]]
             moments = [(np.zeros_like(p), np.zeros_like(p)) for p in flat]
             t0 = time.perf_counter()
             _, clipped = orc.clip_grad_norm(grads, 1.0)
             for p, g, (m, v) in zip(flat, clipped, moments):
                 orc.adamw_step(p, g, m, v, 0, 1e-4, 0.9, 0.95, 1e-8, 0.0, exact=True)
-            opt = (time.perf_counter() - t0) * cfg.layers / 2
-            block = max(t[1] - t[0], 1e-9)
-            rest = max(t[0] - block, 0.0)
+            opt = (time.perf_counter() - t0) * cfg.layers
+            block = max((t[1] - t[0]) / 2, 1e-9)
+            rest = max(t[2] - block, 0.0)
             return tokens * (rest + cfg.layers * block) / seq + opt
 
-        return repeat_timed(once)
+        return repeat_timed(once, 5 if n_threads > 1 else 3)
 
-    all_runs = measure(threads, 128)
-    one_runs = measure(1, 32)
+    all_runs = measure(threads, 128, 3)
+    one_runs = measure(1, 32, 1)
     return {"value": tokens / median_of(all_runs), "unit": "tokens/s", "cores": threads, "kind": "port",
             "cpu_model": cpu_model(), "repeats": len(all_runs), "step_seconds_min": all_runs[0],
             "step_seconds_median": median_of(all_runs), "spread": spread_of(all_runs),
             "single_thread": {"value": tokens / median_of(one_runs), "cores": 1, "step_seconds_min": one_runs[0],
                               "step_seconds_median": median_of(one_runs), "spread": spread_of(one_runs), "sample": "as below on 1x32 tokens"},
-            "sample": f"same model at full width in f32 Exact arithmetic on dequantised weights: one and two blocks on "
-                      f"1x128 tokens (block and rest), clip + AdamW on two blocks' adapters, scaled to {cfg.layers} "
+            "sample": f"same model at full width in f32 Exact arithmetic on dequantised weights: one and three blocks over a "
+                      f"256-entry vocabulary (a block) and one block over the real one (the rest) on 1x128 tokens, one "
+                      f"untimed run then five timed ones, clip + AdamW on one block's adapters, scaled to {cfg.layers} "
                       f"blocks and {tokens} tokens. Attention grows with the sequence: at this sample length it is a "
                       f"smaller share than at {cfg.seq}, so the estimate favours the CPU by up to its 9 % of the step's "
                       f"work. C++ restatement of ojas-cpu, not the Rust binary"}
@@ -426,10 +438,11 @@ def lora_step(args) -> int:
 
 
 def nanolab_cpu_baseline(spec, batch, seq, threads: int):
-    """The oracle's nanolab step on a bounded sample: one and two blocks on one short sequence give a
-    block's time and the rest (table, final norm, head); clip + Muon-NS5 (f32 iteration) on one
-    block's matrices and AdamW on its vectors and on the table give the optimizer's. Scaled to the
-    model's blocks and the step's tokens. All cores and one thread, five repeats each."""
+    """The oracle's nanolab step on a bounded sample: one and three blocks over a small vocabulary
+    give a block's time, one block over the real vocabulary the rest (table, final norm, head), all on
+    one short sequence; clip + Muon-NS5 (f32 iteration) on one block's matrices and AdamW on its
+    vectors and on the table give the optimizer's. Scaled to the model's blocks and the step's
+    tokens. All cores and one thread, one untimed run then five timed ones each."""
     sys.path.insert(0, str(ROOT / "tests"))
     import oracle_api as orc
     from ojas_amd.nanolab import NanolabSpec
@@ -437,8 +450,8 @@ def nanolab_cpu_baseline(spec, batch, seq, threads: int):
     tokens = batch * seq
     rng = np.random.default_rng(0)
 
-    def model(layers, sample_seq):
-        sp = NanolabSpec(**{**spec.__dict__, "n_layer": layers})
+    def model(layers, sample_seq, vocab):
+        sp = NanolabSpec(**{**spec.__dict__, "n_layer": layers, "vocab": vocab})
         cfg = orc.NanolabConfig(layers=layers, n_embd=sp.n_embd, n_head=sp.n_head, n_kv_head=sp.n_kv_head,
                                 head_dim=sp.head_dim, hidden=sp.hidden, vocab=sp.vocab, batch=1, seq=sample_seq, window=0,
                                 rms_eps=sp.rms_eps, rope_base=sp.rope_base)
@@ -448,47 +461,48 @@ def nanolab_cpu_baseline(spec, batch, seq, threads: int):
         ids = rng.integers(0, sp.vocab, (1, sample_seq)).astype(np.uint32)
         return sp, cfg, params, ids
 
-    def measure(n_threads, sample_seq):
+    def measure(n_threads, sample_seq, inner):
         orc.set_threads(n_threads)
-        one, two = model(1, sample_seq), model(2, sample_seq)
+        # A block's time from one and three blocks over a 256-entry vocabulary (the head is then a
+        # negligible part of both timings); the rest from one block over the real vocabulary. Every
+        # model's time is the median of `inner` calls (the optimizer, a twentieth of the step, is timed once).
+        small_one, small_three, one = model(1, sample_seq, 256), model(3, sample_seq, 256), model(1, sample_seq, spec.vocab)
         shapes = one[0].param_shapes()
         names = one[0].param_names()
 
         def once():
-            t = []
-            for sp, cfg, params, ids in (one, two):
-                t0 = time.perf_counter()
-                _, _, grads = orc.nanolab_loss_and_grads(cfg, params, ids, ids)
-                t.append(time.perf_counter() - t0)
-            block = max(t[1] - t[0], 1e-9)
-            rest = max(t[0] - block, 0.0)
+            t = [timed(lambda m=m: orc.nanolab_loss_and_grads(m[1], m[2], m[3], m[3]), inner)[0]
+                 for m in (small_one, small_three, one)]
+            block = max((t[1] - t[0]) / 2, 1e-9)
+            rest = max(t[2] - block, 0.0)
             # optimizer on the one-block model: the table and final norm once, the block's tensors per block
             t_table, t_block = 0.0, 0.0
             for n, p in zip(names, one[2]):
                 g = np.full_like(p, 1e-3)
-                t0 = time.perf_counter()
                 if len(shapes[n]) == 2 and n != "tok_emb.weight":
-                    orc.muon_ns5_step(p.reshape(shapes[n]).copy(), g.reshape(shapes[n]), np.zeros(shapes[n], np.float32),
-                                      lr=0.025, momentum=0.99, weight_decay=0.1, nesterov=True, bf16=False)
+                    w, g2, mom = p.reshape(shapes[n]).copy(), g.reshape(shapes[n]), np.zeros(shapes[n], np.float32)
+                    dt = timed(lambda: orc.muon_ns5_step(w, g2, mom, lr=0.025, momentum=0.99, weight_decay=0.1,
+                                                         nesterov=True, bf16=False))[0]
                 else:
-                    orc.adamw_step(p.copy(), g, np.zeros_like(p), np.zeros_like(p), 0, 6e-4, 0.9, 0.95, 1e-8, 0.0, exact=True)
-                dt = time.perf_counter() - t0
+                    w, m1, m2 = p.copy(), np.zeros_like(p), np.zeros_like(p)
+                    dt = timed(lambda: orc.adamw_step(w, g, m1, m2, 0, 6e-4, 0.9, 0.95, 1e-8, 0.0, exact=True))[0]
                 if n.startswith("blocks."):
                     t_block += dt
                 else:
                     t_table += dt
             return tokens * (rest + spec.n_layer * block) / sample_seq + t_table + spec.n_layer * t_block
 
-        return repeat_timed(once)
+        return repeat_timed(once, 5 if n_threads > 1 else 3)
 
-    all_runs = measure(threads, 128)
-    one_runs = measure(1, 32)
+    all_runs = measure(threads, 128, 3)
+    one_runs = measure(1, 32, 1)
     return {"value": tokens / median_of(all_runs), "unit": "tokens/s", "cores": threads, "kind": "port",
             "cpu_model": cpu_model(), "repeats": len(all_runs), "step_seconds_min": all_runs[0],
             "step_seconds_median": median_of(all_runs), "spread": spread_of(all_runs),
             "single_thread": {"value": tokens / median_of(one_runs), "cores": 1, "step_seconds_min": one_runs[0],
                               "step_seconds_median": median_of(one_runs), "spread": spread_of(one_runs), "sample": "as below on 1x32 tokens"},
-            "sample": f"same model in f32 Exact arithmetic: one and two blocks on 1x128 tokens (block and rest), Muon-NS5 "
+            "sample": f"same model in f32 Exact arithmetic: one and three blocks over a 256-entry vocabulary (a block) and one "
+                      f"block over the real one (the rest) on 1x128 tokens, one untimed run then five timed ones, Muon-NS5 "
                       f"and AdamW on one block's parameters and the table, scaled to {spec.n_layer} blocks and {tokens} "
                       f"tokens. Attention grows with the sequence: at this sample length it is a smaller share than at "
                       f"{seq}, so the estimate favours the CPU by up to its 8 % of the step's work. C++ restatement of "
