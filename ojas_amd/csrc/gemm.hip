@@ -486,7 +486,9 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
       //      and for outputs of a round or two of tiles. The default.
       //   6  128 x 128, four waves, three workgroups per compute unit: weight gradients (both
       //      operands k-major, K = tokens) whose output is under one tile per compute unit, with
-      //      the reduction split (3 to 20 % ahead of 256 x 128 there).
+      //      the reduction split (3 to 20 % ahead of 256 x 128 there), and input gradients whose
+      //      256 x 128 tiles would leave compute units empty, over at least 32 steps (8192 x 768
+      //      over K = 3072: 52 against 66 us).
       //   0  256 x 256, whole-line 64-column steps, one workgroup per compute unit: k-contiguous
       //      A (forward and input-gradient products) over at least 32 steps when the tiles fill
       //      the chip (K = 8192, 8192 x 2048 outputs: 233 against 282 us for 256 x 128), and the
@@ -512,8 +514,14 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
         else if (!unbatched && ksteps64 >= 64 && g.M >= 12 * 256 && g.N <= 4 * 256) dma_variant = 0;
         else dma_variant = 3;
       } else if (!a_km) {
+        // One workgroup per compute unit: a last round of 256 x 256 tiles that is under 7/8 full
+        // costs more than the tile saves (384 tiles on 256 units: 141 against 117 us for 256 x 128).
+        const long rounds256 = (tiles256 + cus - 1) / cus;
+        const bool fills256 = tiles256 * 8 >= rounds256 * cus * 7;
+        const long tiles256x128 = static_cast<long>((g.M + 255) / 256) * ((g.N + 127) / 128);
         if (unbatched && plain && tiles256 >= 4 * cus && ksteps64 < 32) dma_variant = 8;
-        else if (unbatched && plain && ((tiles256 >= cus && ksteps64 >= 32) || ksteps64 >= 512)) dma_variant = 0;
+        else if (unbatched && plain && ((tiles256 >= cus && fills256 && ksteps64 >= 32) || ksteps64 >= 512)) dma_variant = 0;
+        else if (unbatched && plain && b_km && tiles256x128 < cus && ksteps64 >= 32) dma_variant = 6;
         else dma_variant = 3;
       } else {
         dma_variant = 3;

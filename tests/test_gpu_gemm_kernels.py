@@ -63,7 +63,8 @@ def test_linear_bf16_under_each_kernel(be, mode, rows, kin, nout):
 
 @pytest.mark.parametrize("layout,m,k,n", [
     ("NN", 8192, 1024, 3072), ("NN", 8192, 8192, 2048), ("NN", 8192, 4096, 4096), ("NN", 4096, 768, 32000),
-    ("NT", 8192, 8192, 2048), ("NT", 8192, 3072, 1024), ("NT", 8192, 16384, 4096),
+    ("NT", 8192, 8192, 2048), ("NT", 8192, 3072, 1024), ("NT", 8192, 16384, 4096), ("NT", 8192, 3072, 768),
+    ("NT", 16384, 3072, 1536),
     ("TT", 4096, 8192, 1024), ("TT", 4096, 8192, 4096), ("TT", 1024, 8192, 1024), ("TT", 6144, 8192, 2048)])
 def test_the_dispatcher_picks_a_tiling_within_a_tenth_of_the_best(be, layout, m, k, n):
     """Shapes of other models (d = 1024 / 2048 / 4096, 8192 tokens): the tiling the shape rule
