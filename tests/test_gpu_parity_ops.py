@@ -687,6 +687,10 @@ FLASH_SHAPES = [([1, 1, 1, 64], 1, None), ([1, 2, 17, 64], 2, None), ([2, 3, 64,
                 ([1, 2, 128, 64], 2, None), ([1, 2, 129, 64], 1, None), ([1, 4, 300, 64], 2, None),
                 ([2, 2, 257, 64], 2, 40), ([1, 2, 200, 64], 2, 1), ([1, 1, 1024, 64], 1, None),
                 ([1, 2, 520, 64], 2, 130),
+                # sequence ends at every position inside a 128-row block's waves, tiles and half tiles
+                ([1, 1, 33, 64], 1, None), ([1, 1, 65, 64], 1, None), ([1, 2, 96, 64], 1, None),
+                ([1, 1, 160, 64], 1, None), ([1, 1, 192, 64], 1, None), ([1, 2, 448, 64], 2, None),
+                ([1, 1, 96, 128], 1, None), ([1, 1, 192, 128], 1, None),
                 # head_dim 128 (the dK / dV pass walks a key block once per gradient)
                 ([1, 1, 1, 128], 1, None), ([1, 2, 33, 128], 2, None), ([2, 2, 128, 128], 2, None),
                 ([1, 4, 300, 128], 2, None), ([1, 2, 257, 128], 1, 40), ([1, 1, 1024, 128], 1, None),
