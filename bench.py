@@ -41,7 +41,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor figure
 # (profiles/gemm_hbm_traffic_all_workloads.txt holds the runs and the tables for each workload).
 # The algorithmic figure of the gpt124m step (every operand read once, every output written once)
 # is 2.258e8 per op.
-GEMM_HBM_BYTES_PER_LAUNCH = {"gpt124m": 3.93e8, "gpt124m-muon": 3.13e8, "lora1b": 3.84e8, "nanolab124m": 2.55e8}
+GEMM_HBM_BYTES_PER_LAUNCH = {"gpt124m": 3.80e8, "gpt124m-muon": 3.02e8, "lora1b": 4.01e8, "nanolab124m": 2.77e8}
 
 
 # Kernel classes of omx_profile_kernels beyond the GEMM products: (bit, key, kernels, roofline).
