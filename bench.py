@@ -257,7 +257,7 @@ def attention(args) -> int:
     causal attention at the headline shape (batch 16, 12 heads, 1024 tokens, head_dim 64, bf16;
     `--attention-batch 8` is the isolated attention case of the baseline's configs) through
     `causal_sdpa_forward` / `causal_sdpa_backward`. `value` is causal-counted TFLOP/s over both
-    passes (forward 2 B H T^2 D, backward 5 B H T^2 D)."""
+    passes (forward 2 B H T^2 D, backward 5 B H T^2 D), from the median of five timed runs of each."""
     from ojas_amd.backend import BF16, MiBackend
 
     b, h, t, d = args.attention_batch, 12, 1024, 64
@@ -265,17 +265,24 @@ def attention(args) -> int:
     r = np.random.default_rng(0)
     q, k, v, gy = (be.upload(r.standard_normal((b, h, t, d)).astype(np.float32), BF16) for _ in range(4))
     out, lse = be.causal_sdpa_forward(q, k, v, None, BF16)
-    times = {}
+    times, fastest = {}, {}
     for name, fn in (("forward", lambda: be.causal_sdpa_forward(q, k, v, None, BF16)),
                      ("backward", lambda: be.causal_sdpa_backward(q, k, v, out, lse, gy, None, BF16))):
-        for _ in range(args.warmup):
-            fn()
-        be.sync()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            fn()
-        be.sync()
-        times[name] = (time.perf_counter() - t0) / args.steps
+        # Five timed runs of `steps` calls each, `warmup` untimed calls before every one: a run of 50
+        # calls is a few milliseconds, shorter than the clock takes to settle after an idle stretch,
+        # so single runs differ by 10 %. `us` is the median run, `us_min` the fastest.
+        runs = []
+        for _ in range(5):
+            for _ in range(args.warmup):
+                fn()
+            be.sync()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                fn()
+            be.sync()
+            runs.append((time.perf_counter() - t0) / args.steps)
+        runs.sort()
+        times[name], fastest[name] = runs[2], runs[0]
     unit = 2.0 * b * h * t * t * d
     flops = {"forward": unit, "backward": 2.5 * unit}
     total = sum(times.values())
@@ -291,6 +298,7 @@ def attention(args) -> int:
                      "achieved": sum(flops.values()) / total / 1e12, "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": sum(flops.values()) / total / 1e12 / BF16_MFMA_PEAK_TFLOPS, "traffic": None},
         "us": {name: dt * 1e6 for name, dt in times.items()},
+        "us_min": {name: dt * 1e6 for name, dt in fastest.items()},
         "tflops": {name: flops[name] / dt / 1e12 for name, dt in times.items()},
     }
     be.close()
