@@ -624,12 +624,13 @@ int32_t omx_topk_rows(omx_ctx* ctx, const void* x_f32, uint64_t rows, uint64_t c
 int32_t omx_read_scalar_f32(omx_ctx* ctx, const void* src, float* out);
 
 /* Tuning knobs (no counterpart in the reference). "gemm_dma": 0 = register-staged 128x128 GEMM
- * kernel only, 1 = choose by shape (default), 2 / 3 / 4 = force the 256x256 (64-column steps) /
- * 256x128 (32-column steps) / 128x128 four-wave direct-to-LDS kernel wherever the operands are
- * eligible. "gemm_persistent": bit mask over operand layouts (bit 2 * A k-major + B k-major) that
- * take the persistent form of the direct-to-LDS kernel (default 15), and
- * "gemm_persistent_min_steps": only for reductions of at least this many 32-column steps
- * (default 64). "gemm_thin": 0 = bf16 products with at most 64 output columns over 1024 rows or
+ * kernel only, 1 = choose a tiling by the output's tiles per compute unit and the K steps per
+ * tile (default), 2 / 3 / 4 / 8 = force the 256x256 (64-column steps) / 256x128 (32-column
+ * steps) / 128x128 four-wave / alternating 256x256 direct-to-LDS kernel wherever the operands
+ * are eligible (tests and measurements). "flash_schedule": 0 = the bf16 attention kernels choose
+ * between one 128-row block per workgroup and a mirrored pair by how the pairs fill the chip
+ * (default), 1 / 2 = always one block / always the pair (the parity tests run both).
+ * "gemm_thin": 0 = bf16 products with at most 64 output columns over 1024 rows or
  * more go through the tiled kernels and their split-K reduce instead of the one-pass kernel for
  * thin outputs (default 1). "kv_attention": 0 = choose by head_dim (default), 1 = always the
  * LDS-tiled kernel. "ce_fused": 0 = the fused linear-cross-entropy always takes its separate
