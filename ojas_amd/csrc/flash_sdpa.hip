@@ -418,14 +418,6 @@ __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_fwd_kernel(const un
     const unsigned short* vp = v + b * s.kv.bs + kvh * s.kv.hs;
     const int wave_q0 = qb * 128 + wave * 32;
     const int q_row = wave_q0 + l32;
-    const int block_q0 = qb * 128, block_q1 = min(T - 1, qb * 128 + 127);
-    const int kt_first = s.window > 0 ? max(0, block_q0 + 1 - s.window) / 64 : 0;
-    const int kt_last = block_q1 / 64;
-    // The first tile's loads go out before the row's own, so that their latencies run side by side.
-    // The next tile's global loads are then in flight while the current one is multiplied.
-    u32x4 rk[NL], rv[NL];
-    fetch.load(kp, kt_first * 64, rk);
-    fetch.load(vp, kt_first * 64, rv);
     u32x4 qf[KK];
     row_frags<D>(qp, s.q.rs, q_row, T, lg, qf);
     floatx16 o[MT];
@@ -439,6 +431,13 @@ __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_fwd_kernel(const un
     // come through scaled by (sum of rounded weights) / (sum of weights).
     float m = -INFINITY, lsum = 0.0f, wsum = 0.0f;
     const float scale_log2 = s.scale * LOG2E;
+    const int block_q0 = qb * 128, block_q1 = min(T - 1, qb * 128 + 127);
+    const int kt_first = s.window > 0 ? max(0, block_q0 + 1 - s.window) / 64 : 0;
+    const int kt_last = block_q1 / 64;
+    // The next tile's global loads are in flight while the current one is multiplied.
+    u32x4 rk[NL], rv[NL];
+    fetch.load(kp, kt_first * 64, rk);
+    fetch.load(vp, kt_first * 64, rv);
     __syncthreads();  // the previous pass's reads of the first pair are done
     tile_store_rows<D>(smem, rk);
     tile_store_rows<D>(smem + ftile(D), rv);
@@ -596,6 +595,8 @@ __device__ __forceinline__ bool flash_dkv_block(const unsigned short* __restrict
   const int wave_k0 = kb * 128 + wave * 32;
   const int key_row = wave_k0 + l32;
   u32x4 kf[KK], vf[WANT_DK ? KK : 1];
+  row_frags<D>(k + kv_off, s.kv.rs, key_row, T, lg, kf);
+  if constexpr (WANT_DK) row_frags<D>(v + kv_off, s.kv.rs, key_row, T, lg, vf);
   floatx16 dk[WANT_DK ? MT : 1], dv[WANT_DV ? MT : 1];
 #pragma unroll
   for (int mt = 0; mt < (WANT_DK ? MT : 1); ++mt) dk[mt] = zero16();
@@ -642,9 +643,6 @@ __device__ __forceinline__ bool flash_dkv_block(const unsigned short* __restrict
     }
   };
   fetch();
-  // (the first tile's loads go out before the rows' own, so that their latencies run side by side)
-  row_frags<D>(k + kv_off, s.kv.rs, key_row, T, lg, kf);
-  if constexpr (WANT_DK) row_frags<D>(v + kv_off, s.kv.rs, key_row, T, lg, vf);
   __syncthreads();  // an earlier walk's reads of the first set are done
   store_set(smem);
   if (steps > 1) fetch();
@@ -849,13 +847,6 @@ __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_bwd_dq_kernel(
     const unsigned short* vp = v + b * s.kv.bs + kvh * s.kv.hs;
     const int wave_q0 = qb * 128 + wave * 32;
     const int q_row = wave_q0 + l32;
-    const int block_q0 = qb * 128, block_q1 = min(T - 1, qb * 128 + 127);
-    const int kt_first = s.window > 0 ? max(0, block_q0 + 1 - s.window) / 64 : 0;
-    const int kt_last = block_q1 / 64;
-    // The first tile's loads go out before the row's own, so that their latencies run side by side.
-    u32x4 rk[NL], rv[NL];
-    fetch.load(kp, kt_first * 64, rk);
-    fetch.load(vp, kt_first * 64, rv);
     u32x4 qf[KK], gf[KK];
     row_frags<D>(q + b * s.q.bs + h * s.q.hs, s.q.rs, q_row, T, lg, qf);
     row_frags<D>(gy + b * s.o.bs + h * s.o.hs, s.o.rs, q_row, T, lg, gf);
@@ -902,6 +893,12 @@ __global__ __launch_bounds__(FT, D == 64 ? 3 : 2) void flash_bwd_dq_kernel(
     // lane's share of the row sum of the rounded dS; the end takes (row sum) x (mean key) off.
     float ds_sum = 0.0f;
     const float scale_log2 = s.scale * LOG2E;
+    const int block_q0 = qb * 128, block_q1 = min(T - 1, qb * 128 + 127);
+    const int kt_first = s.window > 0 ? max(0, block_q0 + 1 - s.window) / 64 : 0;
+    const int kt_last = block_q1 / 64;
+    u32x4 rk[NL], rv[NL];
+    fetch.load(kp, kt_first * 64, rk);
+    fetch.load(vp, kt_first * 64, rv);
     __syncthreads();  // the previous pass's reads of the first pair are done
     tile_store_rows<D>(smem, rk);
     tile_store_rows<D>(smem + ftile(D), rv);
