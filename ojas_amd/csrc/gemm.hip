@@ -559,6 +559,24 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
         int p2 = 1;
         while (p2 * 2 <= splits + splits / 4) p2 *= 2;  // 7..9 -> 8, 10..12 -> 8, 13..16 -> 16
         splits = p2;
+        if (dma_variant == 0 || dma_variant == 8) {
+          // One workgroup per compute unit: what counts is how full the last round of workgroups is
+          // (192 tiles split in two are 384 workgroups on 256 units, a round and a half; split in
+          // four they are three full rounds of half the length). More splits only for a chip at
+          // least a tenth fuller: each costs a slice of partial sums and of the reduce pass.
+          const long units = ctx->cu_count > 0 ? ctx->cu_count : 256;
+          int best = 1;
+          double best_fill = 0.0;
+          for (int s2 = 1; s2 <= 16 && ksteps / s2 >= min_steps; s2 *= 2) {
+            const long groups = all_tiles * s2;
+            const double fill = static_cast<double>(groups) / static_cast<double>((groups + units - 1) / units * units);
+            if (fill > best_fill + 0.1) {
+              best = s2;
+              best_fill = fill;
+            }
+          }
+          splits = best;
+        }
       }
     }
     g.ksteps_per_split = (ksteps + splits - 1) / splits;
