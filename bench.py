@@ -157,9 +157,8 @@ def cpu_baseline(cfg, threads: int):
             ocfg, params, ids, targets = model(cfg.layers, cfg.batch, cfg.ctx)
 
             def once():
-                t0 = time.perf_counter()
-                _, grads = orc.gpt_loss_and_grads(ocfg, params, ids, targets)
-                return time.perf_counter() - t0 + optimizer_seconds(params, grads)
+                dt, (_, grads) = timed(lambda: orc.gpt_loss_and_grads(ocfg, params, ids, targets), inner)
+                return dt + optimizer_seconds(params, grads)
 
             runs = repeat_timed(once)
             return runs, f"the whole step ({cfg.batch}x{cfg.ctx} tokens)"
