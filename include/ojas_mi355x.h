@@ -632,7 +632,9 @@ int32_t omx_read_scalar_f32(omx_ctx* ctx, const void* src, float* out);
  * (default), 1 / 2 = always one block / always the pair (the parity tests run both).
  * "gemm_thin": 0 = bf16 products with at most 64 output columns over 1024 rows or
  * more go through the tiled kernels and their split-K reduce instead of the one-pass kernel for
- * thin outputs (default 1). "kv_attention": 0 = choose by head_dim (default), 1 = always the
+ * thin outputs (default 1). "gemm_row_split": 0 = a product on 256x256 tiles whose last round
+ * of tiles fills under 2/5 of the compute units is not cut into two launches by rows (default 1:
+ * the rows of the whole rounds keep the tiling, the rest choose their own). "kv_attention": 0 = choose by head_dim (default), 1 = always the
  * LDS-tiled kernel. "ce_fused": 0 = the fused linear-cross-entropy always takes its separate
  * statistics and gradient kernels (default 1: one kernel when a tile holds the whole
  * vocabulary). "adamw_trust": 0 = omx_adamw_step_bounded always runs its checking pass

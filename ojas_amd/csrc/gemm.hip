@@ -476,7 +476,9 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
   int dma_variant = -1;
   if (!thin && operand_dtype == OMX_BF16 && omx_gemm_dma_eligible(g, a_km, b_km)) {
     const int mode = ctx->gemm_dma_mode;
-    if (mode == 1) {
+    if (mode == 1 && ctx->gemm_forced_tiling >= 0) {
+      dma_variant = ctx->gemm_forced_tiling;
+    } else if (mode == 1) {
       // Four tilings, chosen by how many tiles the output makes per compute unit and how many K
       // steps a tile runs, not by a model's dimensions (measured over GPT-124M's shapes and over
       // d = 1024 / 2048 / 4096 with 8192 tokens; tests/test_gpu_gemm_kernels.py holds the choice
@@ -531,6 +533,31 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
     else if (mode == 3) dma_variant = 3;
     else if (mode == 4) dma_variant = 6;
     else if (mode == 8) dma_variant = 8;
+  }
+  // One 256 x 256 workgroup per compute unit: when the last round of tiles fills under 2/5 of the
+  // chip (the head's weight gradient: 591 tiles on 256 units), the rows of the whole rounds go to
+  // this tiling and the rest to a launch of their own, which picks a smaller tile (1222 -> 1040 us).
+  if ((dma_variant == 0 || dma_variant == 8) && ctx->gemm_dma_mode == 1 && ctx->gemm_row_split &&
+      !ctx->gemm_in_row_split && batches == 1 && !(epi && epi->mode != OMX_EPI_NONE)) {
+    const long cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
+    const long tm = (g.M + 255) / 256, tn = (g.N + 255) / 256;
+    const long rounds = tm * tn / cus, rest = tm * tn % cus;
+    const long head_tm = rounds * cus / tn;
+    if (rounds >= 1 && rounds <= 6 && rest > 0 && rest * 5 < cus * 2 && head_tm >= 1 && head_tm < tm) {
+      const uint64_t m0 = static_cast<uint64_t>(head_tm) * 256;
+      const uint64_t esz = 2, csz = c_dtype == OMX_BF16 ? 2 : 4;
+      ctx->gemm_in_row_split = true;
+      ctx->gemm_forced_tiling = dma_variant;
+      int32_t rc = omx_gemm_impl(ctx, fault_op, a, a_rs, a_cs, b, b_rs, b_cs, operand_dtype, c, c_dtype, ldc, m0, k, n,
+                                 accumulate, epi, nullptr);
+      ctx->gemm_forced_tiling = -1;
+      if (rc == OMX_OK)
+        rc = omx_gemm_impl(ctx, fault_op, static_cast<const char*>(a) + m0 * a_rs * esz, a_rs, a_cs, b, b_rs, b_cs,
+                           operand_dtype, static_cast<char*>(c) + m0 * ldc * csz, c_dtype, ldc, m - m0, k, n,
+                           accumulate, epi, nullptr);
+      ctx->gemm_in_row_split = false;
+      return rc;
+    }
   }
   int BM = 128, BN = 128;
   if (dma_variant >= 0) omx_gemm_dma_tile(dma_variant, &BM, &BN);
@@ -698,6 +725,10 @@ int32_t omx_set_option(omx_ctx* ctx, const char* name, int64_t value) {
   if (name && strcmp(name, "gemm_dma") == 0) {
     if (value < 0 || (value > 4 && value != 8)) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: gemm_dma takes 0..4 or 8");
     ctx->gemm_dma_mode = static_cast<int>(value);
+    return OMX_OK;
+  }
+  if (name && strcmp(name, "gemm_row_split") == 0) {
+    ctx->gemm_row_split = value != 0;
     return OMX_OK;
   }
   if (name && strcmp(name, "flash_schedule") == 0) {

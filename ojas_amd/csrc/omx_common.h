@@ -92,6 +92,9 @@ struct omx_ctx {
   // Optional per-launch timing of the GEMM kernel (benchmark only).
   // 0: 128x128 kernel only; 1: choose by shape; 2 / 3: force the 256x256 / 256x128 direct-to-LDS kernel where eligible.
   int gemm_dma_mode = 1;
+  int gemm_row_split = 1;    // 0: a product whose last round of 256 x 256 tiles is mostly empty is not cut by rows
+  bool gemm_in_row_split = false;  // set while omx_gemm_impl runs the two halves of a cut product
+  int gemm_forced_tiling = -1;     // the tiling the first half keeps, whatever its own tile count says
   int gemm_thin = 1;         // outputs of at most 64 columns over many rows take gemm_thin_kernel
   int flash_schedule = 0;     // 0: by the chip's workgroup places; 1: one 128-row block per workgroup; 2: mirrored pairs
   int kv_attention_mode = 0;  // 1: cached attention always takes the LDS-tiled kernel

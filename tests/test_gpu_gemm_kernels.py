@@ -1,6 +1,5 @@
 """Every GEMM kernel variant against the oracle: the 128x128 kernel and the
-direct-to-LDS kernels (256x256, 256x128, 128x128 and 128x192, 32- and 64-column steps, eight, six
-and four waves),
+direct-to-LDS kernels (256x256 whole-line and alternating, 256x128 and 128x128 four-wave),
 forced through `omx_set_option`, on
 shapes with ragged M and N (rows past the edge are fetched from a clamped
 address and must never be stored), every operand layout, split-K, bf16 and f32
@@ -112,6 +111,62 @@ def test_the_dispatcher_picks_a_tiling_within_a_tenth_of_the_best(be, layout, m,
     fastest = min(forced.values())
     print("  us: chosen %.1f, forced %s" % (chosen * 1e6, {mode: round(t * 1e6, 1) for mode, t in forced.items()}), flush=True)
     assert chosen <= 1.10 * fastest, (chosen, forced)
+
+
+def test_a_mostly_empty_last_round_is_cut_by_rows(be):
+    """65 x 16 tiles of 256 x 256 are four rounds of the 256 compute units and 16 tiles more: the
+    first 64 tile rows keep the tiling, the last goes to a launch of its own. Checked against the
+    oracle (ragged M and N), and the rows of the first launch against the uncut product bit for bit."""
+    from ojas_amd.backend import BF16
+
+    m, k, n = 16616, 128, 4088
+    print(f"gemm row split NT {m}x{k}x{n}", flush=True)
+    r = orc.SplitMix64(77)
+    a = orc.round_bf16(r.vec(m * k, 0.5)).reshape(m, k)
+    b = orc.round_bf16(r.vec(k * n, 0.5)).reshape(k, n)
+    orc.set_threads(8)
+    want = orc.linear_forward(a, np.ascontiguousarray(b.T))
+    da, db = be.upload(a, BF16), be.upload(b, BF16)
+    be.set_option("gemm_dma", 1)
+    try:
+        cut = be.download(be.gemm(da, (k, 1), db, (n, 1), m, k, n))
+        be.set_option("gemm_row_split", 0)
+        whole = be.download(be.gemm(da, (k, 1), db, (n, 1), m, k, n))
+    finally:
+        be.set_option("gemm_row_split", 1)
+    scale = max(1.0, float(np.max(np.abs(want))))
+    assert float(np.max(np.abs(cut.astype(np.float64) - want))) <= 1e-5 * scale
+    assert float(np.max(np.abs(whole.astype(np.float64) - want))) <= 1e-5 * scale
+    assert np.array_equal(cut[:64 * 256], whole[:64 * 256])
+
+
+def test_a_cut_weight_gradient_matches_the_uncut_one(be):
+    """Both operands k-major over 4096 rows (a head's weight gradient in small): 86 x 3 tiles are one
+    round and two tiles; the cut product accumulates into C like the uncut one."""
+    from ojas_amd.backend import BF16, F32
+
+    m, k, n = 22016, 4096, 768
+    print(f"gemm row split TT {m}x{k}x{n}", flush=True)
+    a = be.empty((k * m,), BF16)
+    b = be.empty((k * n,), BF16)
+    for t, seed in ((a, 3), (b, 4)):
+        be._check(be._lib.omx_init_normal(be._ctx, be._p(t), C.c_int32(BF16), C.c_uint64(t.numel), C.c_uint64(seed),
+                                          C.c_float(0.05)))
+    c0 = np.full((m, n), 0.25, np.float32)
+    be.set_option("gemm_dma", 1)
+    try:
+        cut = be.upload(c0)
+        be.gemm(a, (1, m), b, (n, 1), m, k, n, c=cut)
+        be.set_option("gemm_row_split", 0)
+        whole = be.upload(c0)
+        be.gemm(a, (1, m), b, (n, 1), m, k, n, c=whole)
+    finally:
+        be.set_option("gemm_row_split", 1)
+    got, ref = be.download(cut), be.download(whole)
+    assert np.array_equal(got[:85 * 256], ref[:85 * 256])
+    # The last 256 rows take another tiling and split K: the same sums in another order.
+    assert float(np.max(np.abs(got[85 * 256:] - ref[85 * 256:]))) <= 1e-5 * max(1.0, float(np.max(np.abs(ref))))
+    assert float(np.max(np.abs(ref - 0.25))) > 0.1
 
 
 def test_unknown_option_is_refused(be):
