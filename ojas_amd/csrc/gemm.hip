@@ -507,22 +507,22 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
       const long tiles256 = static_cast<long>((g.M + 255) / 256) * ((g.N + 255) / 256);
       const long tiles128 = static_cast<long>((g.M + 127) / 128) * ((g.N + 127) / 128);
       const long ksteps64 = g.K / 64;
+      // How full the last round of 256 x 256 tiles is, one workgroup per compute unit.
+      const long all256 = tiles256 * g.batches;
+      const long rounds256 = (all256 + cus - 1) / cus;
+      const bool fills256 = all256 * 8 >= rounds256 * cus * 7;
       if (a_km && b_km && unbatched && ksteps64 >= 64 && tiles128 < cus) {
         dma_variant = 6;
       } else if (outputs * g.batches <= (1l << 20)) {
         dma_variant = -1;  // a handful of tiles: the register-staged kernel, which splits K freely
       } else if (a_km && b_km) {
-        if (unbatched && plain && tiles256 >= cus && ksteps64 >= 64) dma_variant = 8;
-        else if (!unbatched && ksteps64 >= 64 && g.M >= 12 * 256 && g.N <= 4 * 256) dma_variant = 0;
+        // Weight gradients (K = tokens). An unbatched product with a poor last round is cut by rows below.
+        if (plain && ksteps64 >= 64 && all256 >= cus && (unbatched || all256 * 5 >= rounds256 * cus * 4)) dma_variant = 9;
         else dma_variant = 3;
       } else if (!a_km) {
-        // One workgroup per compute unit: a last round of 256 x 256 tiles that is under 7/8 full
-        // costs more than the tile saves (384 tiles on 256 units: 141 against 117 us for 256 x 128).
-        const long rounds256 = (tiles256 + cus - 1) / cus;
-        const bool fills256 = tiles256 * 8 >= rounds256 * cus * 7;
         const long tiles256x128 = static_cast<long>((g.M + 255) / 256) * ((g.N + 127) / 128);
-        if (unbatched && plain && tiles256 >= 4 * cus && ksteps64 < 32) dma_variant = 8;
-        else if (unbatched && plain && ((tiles256 >= cus && fills256 && ksteps64 >= 32) || ksteps64 >= 512)) dma_variant = 0;
+        if (unbatched && plain && tiles256 >= 4 * cus && ksteps64 < 32) dma_variant = 9;
+        else if (unbatched && plain && ((tiles256 >= cus && fills256 && ksteps64 >= 32) || ksteps64 >= 512)) dma_variant = 9;
         else if (unbatched && plain && b_km && tiles256x128 < cus && ksteps64 >= 32) dma_variant = 6;
         else dma_variant = 3;
       } else {
@@ -533,11 +533,12 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
     else if (mode == 3) dma_variant = 3;
     else if (mode == 4) dma_variant = 6;
     else if (mode == 8) dma_variant = 8;
+    else if (mode == 9) dma_variant = 9;
   }
   // One 256 x 256 workgroup per compute unit: when the last round of tiles fills under 2/5 of the
   // chip (the head's weight gradient: 591 tiles on 256 units), the rows of the whole rounds go to
   // this tiling and the rest to a launch of their own, which picks a smaller tile (1222 -> 1040 us).
-  if ((dma_variant == 0 || dma_variant == 8) && ctx->gemm_dma_mode == 1 && ctx->gemm_row_split &&
+  if ((dma_variant == 0 || dma_variant >= 8) && ctx->gemm_dma_mode == 1 && ctx->gemm_row_split &&
       !ctx->gemm_in_row_split && batches == 1 && !(epi && epi->mode != OMX_EPI_NONE)) {
     const long cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
     const long tm = (g.M + 255) / 256, tn = (g.N + 255) / 256;
@@ -586,7 +587,7 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
         int p2 = 1;
         while (p2 * 2 <= splits + splits / 4) p2 *= 2;  // 7..9 -> 8, 10..12 -> 8, 13..16 -> 16
         splits = p2;
-        if (dma_variant == 0 || dma_variant == 8) {
+        if (dma_variant == 0 || dma_variant >= 8) {
           // One workgroup per compute unit: what counts is how full the last round of workgroups is
           // (192 tiles split in two are 384 workgroups on 256 units, a round and a half; split in
           // four they are three full rounds of half the length). More splits only for a chip at
@@ -723,7 +724,7 @@ int32_t omx_set_option(omx_ctx* ctx, const char* name, int64_t value) {
     return OMX_OK;
   }
   if (name && strcmp(name, "gemm_dma") == 0) {
-    if (value < 0 || (value > 4 && value != 8)) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: gemm_dma takes 0..4 or 8");
+    if (value < 0 || (value > 4 && value != 8 && value != 9)) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: gemm_dma takes 0..4 or 8");
     ctx->gemm_dma_mode = static_cast<int>(value);
     return OMX_OK;
   }

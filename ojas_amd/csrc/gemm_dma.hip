@@ -45,7 +45,7 @@ bool omx_gemm_dma_eligible(const GemmArgs& g, bool a_km, bool b_km) {
 
 void omx_gemm_dma_tile(int variant, int* bm, int* bn) {
   *bm = variant == 6 ? 128 : 256;
-  *bn = variant == 0 || variant == 8 ? 256 : 128;
+  *bn = variant == 0 || variant == 8 || variant == 9 ? 256 : 128;
 }
 
 

@@ -4,6 +4,7 @@
 #pragma once
 #include "gemm_tiles.h"
 #include "gemm_pp_impl.h"
+#include "gemm_w4_impl.h"
 
 namespace {
 
@@ -640,6 +641,12 @@ int32_t launch_dma(omx_ctx* ctx, const GemmArgs& g) {
 // stages, two workgroups per compute unit); 6: 128 x 128 with four waves (three per compute unit).
 template <bool A_KM, bool B_KM>
 int32_t launch_variant(omx_ctx* ctx, const GemmArgs& g, int variant) {
+  if (variant == 9) {
+    if constexpr (!A_KM || B_KM) {
+      if (w4_offsets_fit(g)) return launch_w4<A_KM, B_KM>(ctx, g);
+    }
+    return launch_pp<A_KM, B_KM>(ctx, g);
+  }
   if (variant == 8) return launch_pp<A_KM, B_KM>(ctx, g);
   if (variant == 0) return launch_dma<A_KM, B_KM, 2, 4, 4, 2, 64, 2>(ctx, g);
   if (variant == 6) return launch_dma<A_KM, B_KM, 2, 2, 2, 2, 32, 3>(ctx, g);

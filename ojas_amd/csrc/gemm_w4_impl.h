@@ -1,0 +1,446 @@
+// The bf16 GEMM with one wave per SIMD: a 256 x 256 output tile per workgroup, one workgroup per
+// compute unit, four waves of 128 x 128 each (16 accumulator blocks of 32 x 32: 256 of the wave's
+// 512 registers). A wave interleaves its own LDS reads and global -> LDS loads between its own
+// matrix products, in an order fixed in the source: per product a wave reads two thirds of the
+// fragment bytes that eight waves of 128 x 64 read, and no other wave on the SIMD takes issue
+// slots from the products.
+//
+//   K steps of 64 columns, two LDS stages per operand (A0 A1 B0 B1, 32 KiB each). A step is 64
+//   products per wave in two halves of 32, and a stage is refilled in two parts, each as soon as
+//   every wave has read it:
+//     A k-contiguous (a load covers 8 rows x 64 columns): half 0 is the wave's row blocks 0-1 over
+//       the step's four K slabs against all of B, half 1 its row blocks 2-3 against the same B
+//       fragments, which stay in registers. Part 0 = B and the A rows of half 0 (12 loads per
+//       wave), part 1 = the A rows of half 1 (4 loads).
+//     A and B k-major (a load covers 2 K rows x 256 rows): half h is K slabs 2h, 2h + 1 of every
+//       block; part h = K rows 32h .. 32h + 31 of both operands (8 loads per wave).
+//   During half 1 of step j the wave reads part 0 of step j + 1, during half 0 part 1 of step j.
+//   Two barriers per step: B0, after the first 8 products of half 0, says that every wave has read
+//   part 0 of this step, and publishes part 1; part 0 of step j + 2 is loaded behind it. B1,
+//   between the halves, says that part 1 has been read and publishes part 0 of step j + 1; part 1
+//   of step j + 2 is loaded behind it. Every load has more than a step to land.
+//   The K loop is one body for every step (the stage is a register, the last steps skip their
+//   loads by scalar branches): with copies of the body for the last steps the compiler permutes
+//   the 256 accumulator registers between the copies through scratch memory.
+#pragma once
+#include "gemm_tiles.h"
+
+namespace {
+
+constexpr int W4_BM = 256, W4_BN = 256, W4_BK = 64;
+constexpr int W4_OPERAND = W4_BM * W4_BK * 2;  // one stage of one operand
+constexpr int W4_SMEM = 4 * W4_OPERAND;
+constexpr int W4_B0 = 2 * W4_OPERAND;  // LDS byte offset of B's first stage
+
+// Loads of one operand: a wave-uniform base address (the tile's first element at the current K
+// step) and a 32-bit byte offset per lane and load, so a K step advances one scalar.
+template <bool KM>
+struct W4Loads {
+  static constexpr int N = 8;  // 32 loads of 1 KiB per step, four waves
+  unsigned off[N];
+  const char* base;
+  long step;
+  __device__ __forceinline__ void init(const unsigned short* __restrict__ p, long ld, int row0, int rows, int k0,
+                                       int wave, int lane) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int q = wave + 4 * i;
+      if constexpr (!KM) {
+        const int r = q * 8 + (lane >> 3);
+        const int kc = (lane & 7) ^ ((r >> 1) & 7);
+        int gr = row0 + r;
+        gr = gr < rows ? gr : rows - 1;
+        off[i] = static_cast<unsigned>(gr - row0) * static_cast<unsigned>(ld * 2) + kc * 16;
+      } else {
+        const int idx = q * 64 + lane;
+        const int kr = idx >> 5, slot = idx & 31;
+        const int mc = slot ^ ((kr & 3) * 4);
+        int gm = mc * 8;
+        gm = row0 + gm + 8 <= rows ? gm : 0;
+        off[i] = static_cast<unsigned>(kr) * static_cast<unsigned>(ld * 2) + gm * 2;
+      }
+    }
+    base = reinterpret_cast<const char*>(p) +
+           (KM ? static_cast<long>(k0) * ld + row0 : static_cast<long>(row0) * ld + k0) * 2;
+    step = (KM ? W4_BK * ld : W4_BK) * 2;
+  }
+  // Load I of this wave into LDS byte `lds_wave` + LDS_IMM.
+  template <int I, int LDS_IMM>
+  __device__ __forceinline__ void issue(unsigned lds_wave) const {
+    asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off[I]), "s"(base),
+                 "s"(lds_wave), "n"(LDS_IMM)
+                 : "memory", "scc");
+  }
+};
+
+// Fragment addresses of one operand in one stage: four registers; the block and the K slab are
+// immediates. flip() moves them to the other stage.
+template <bool KM>
+struct W4Frags {
+  int b[4];
+  __device__ __forceinline__ void init(int first) {
+#pragma unroll
+    for (int x = 0; x < 4; ++x) b[x] = KM ? first ^ (x << 6) : first ^ (x << 5);
+  }
+  __device__ __forceinline__ void flip() {
+#pragma unroll
+    for (int x = 0; x < 4; ++x) b[x] ^= W4_OPERAND;
+  }
+  template <int T, int KK>
+  __device__ __forceinline__ u32x4 read(const char* smem) const {
+    if constexpr (!KM) {
+      return *reinterpret_cast<const u32x4*>(smem + b[KK] + T * 32 * W4_BK * 2);
+    } else {
+      return frag_at<true, 256>(smem + b[T] + KK * 16 * 256 * 2);
+    }
+  }
+};
+
+template <bool A_KM, bool B_KM, int EPI>
+__global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
+  static_assert(!A_KM || B_KM, "a k-major A goes with a k-major B");
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  constexpr int TM = 4, TN = 4, NW = 4;
+  // Tile order: as gemm_dma_kernel.
+  const int total = g.tiles_m * g.tiles_n;
+  int split = 0, id = blockIdx.x, product = blockIdx.y;
+  if (g.batches > 1 && g.splits == 1 && ((total * g.batches) & 7) == 0) {
+    const int linear = blockIdx.y * total + blockIdx.x;
+    const int r = (linear & 7) * ((total * g.batches) >> 3) + (linear >> 3);
+    product = r / total;
+    id = r - product * total;
+  } else if (g.splits > 1) {
+    split = blockIdx.x % g.splits;
+    id = blockIdx.x / g.splits;
+  } else if (total % 8 == 0) {
+    id = (id & 7) * (total >> 3) + (id >> 3);
+  }
+  const int band = 4;
+  const int tiles_per_band = band * g.tiles_n;
+  const int band_id = id / tiles_per_band;
+  const int first_m = band_id * band;
+  const int band_rows = min(band, g.tiles_m - first_m);
+  const int in_band = id - band_id * tiles_per_band;
+  const int tile_m = first_m + in_band % band_rows;
+  const int tile_n = in_band / band_rows;
+  // (the divisions above run on the vector unit: back to scalars, which the loads' bases need)
+  const int m0 = __builtin_amdgcn_readfirstlane(tile_m * W4_BM), n0 = __builtin_amdgcn_readfirstlane(tile_n * W4_BN);
+  product = __builtin_amdgcn_readfirstlane(product);
+  split = __builtin_amdgcn_readfirstlane(split);
+  gemm_select_batch(g, product);
+  const unsigned short* __restrict__ A = static_cast<const unsigned short*>(g.a);
+  const unsigned short* __restrict__ B = static_cast<const unsigned short*>(g.b);
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int l32 = lane & 31, lg = lane >> 5;
+
+  floatx16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  const int ks_begin = split * g.ksteps_per_split;
+  const int ks_end = min(g.K / W4_BK, ks_begin + g.ksteps_per_split);
+  const int steps = ks_end - ks_begin;
+  W4Loads<A_KM> la;
+  W4Loads<B_KM> lb;
+  la.init(A, g.lda, m0, g.M, ks_begin * W4_BK, wave, lane);
+  lb.init(B, g.ldb, n0, g.N, ks_begin * W4_BK, wave, lane);
+  const unsigned lds_wave =
+      __builtin_amdgcn_readfirstlane(static_cast<unsigned>(reinterpret_cast<uintptr_t>(smem))) + wave * 1024;
+  constexpr int NO_WAIT = 64;
+  auto wait_loads = [&](int n) {
+    if (n >= NO_WAIT) return;
+    if (n >= 16) __builtin_amdgcn_s_waitcnt(vmcnt_only(16));
+    else if (n >= 8) __builtin_amdgcn_s_waitcnt(vmcnt_only(8));
+    else if (n >= 4) __builtin_amdgcn_s_waitcnt(vmcnt_only(4));
+    else __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+  };
+  auto publish = [&](int in_flight) {
+    __builtin_amdgcn_sched_barrier(0);
+    wait_loads(in_flight);
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt == 0: this wave's fragment reads have returned
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto product_of = [&](floatx16& c, const u32x4& a, const u32x4& b) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  };
+  unsigned lds_here = lds_wave;  // where this wave's loads into the current stage go
+  if constexpr (!A_KM) {
+    // `here`: the stage of the step being multiplied, `there`: the other one. B is only ever read a
+    // step ahead.
+    W4Frags<false> a_here, a_there;
+    W4Frags<B_KM> b_there;
+    a_here.init(frag_offset<false, W4_BM, W4_BK>(wm * 128, 0, lane));
+    a_there.init(frag_offset<false, W4_BM, W4_BK>(wm * 128, 0, lane));
+    b_there.init(W4_B0 + frag_offset<B_KM, W4_BN, W4_BK>(wn * 128, 0, lane));
+    a_there.flip();  // the loop starts in stage 0 (b_there follows once step 0's fragments are read)
+
+    // Part 0 of a stage: all of B and A's loads 0, 1, 4, 5 (rows 0-63 and 128-191 of the tile);
+    // part 1: A's loads 2, 3, 6, 7. `n` counts the part's loads.
+    auto issue_p0 = [&](unsigned lds, auto n_index) {
+      constexpr int n = decltype(n_index)::value;
+      if constexpr (n < 8) {
+        lb.template issue<n, W4_B0 + NW * n * 1024>(lds);
+      } else {
+        constexpr int i = n == 8 ? 0 : n == 9 ? 1 : n == 10 ? 4 : 5;
+        la.template issue<i, NW * i * 1024>(lds);
+      }
+    };
+    auto issue_p1 = [&](unsigned lds, auto n_index) {
+      constexpr int n = decltype(n_index)::value;
+      constexpr int i = n == 0 ? 2 : n == 1 ? 3 : n == 2 ? 6 : 7;
+      la.template issue<i, NW * i * 1024>(lds);
+    };
+    // fa0[t][k]: row blocks 0-1, fa1[t][k]: row blocks 2-3, fb[u][k]: column blocks, K slab k.
+    u32x4 fa0[2][4], fa1[2][4], fb[4][4];
+    // Fragment n (0..5) of K slab k of part 0 of the stage `a` and `b` point at: four of B, two of A.
+    auto read_p0 = [&](const W4Frags<false>& a, const W4Frags<B_KM>& b, auto k_index, auto n_index) {
+      constexpr int k = decltype(k_index)::value, n = decltype(n_index)::value;
+      if constexpr (n < 4) fb[n][k] = b.template read<n, k>(smem);
+      else fa0[n - 4][k] = a.template read<n - 4, k>(smem);
+    };
+    // Fragment n (0..7) of part 1 of the current stage: K slab n / 2, row block 2 + n % 2.
+    auto read_p1 = [&](auto n_index) {
+      constexpr int n = decltype(n_index)::value;
+      fa1[n % 2][n / 2] = a_here.template read<2 + n % 2, n / 2>(smem);
+    };
+    // Both stages' loads, part 0 of step 0 published, its fragments read.
+    static_for<0, 12>([&](auto n_index) { issue_p0(lds_wave, n_index); });
+    static_for<0, 4>([&](auto n_index) { issue_p1(lds_wave, n_index); });
+    la.base += la.step;
+    lb.base += lb.step;
+    if (steps > 1) {
+      static_for<0, 12>([&](auto n_index) { issue_p0(lds_wave + W4_OPERAND, n_index); });
+      static_for<0, 4>([&](auto n_index) { issue_p1(lds_wave + W4_OPERAND, n_index); });
+      la.base += la.step;
+      lb.base += lb.step;
+    }
+    wait_loads(4 + (steps > 1 ? 16 : 0));
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<0, 4>([&](auto k_index) {
+      static_for<0, 6>([&](auto n_index) { read_p0(a_here, b_there, k_index, n_index); });
+    });
+    b_there.flip();
+    __builtin_amdgcn_sched_barrier(0);
+
+    // One K step per turn: the same code for every step, so the accumulators stay where they are.
+    // `next`: another step follows; `loads`: two more follow (the loads of the second start here).
+    // The fragment reads "of the next step" also run in the last step, on stale data nobody uses.
+  #pragma unroll 1
+    for (int j = 0; j < steps; ++j) {
+      const bool next = j + 1 < steps, loads = j + 2 < steps;
+      // Half 0.
+      static_for<0, 32>([&](auto n_index) {
+        constexpr int n = decltype(n_index)::value, k = n / 8, t = (n % 8) / 4, u = n % 4;
+        product_of(acc[t][u], fa0[t][k], fb[u][k]);
+        if constexpr (n == 7) {
+          // B0. In flight behind part 1 of this step: both parts of the next.
+          publish(next ? 16 : 0);
+        } else {
+          if constexpr (n >= 8 && n % 2 == 0) {
+            if (loads) issue_p0(lds_here, std::integral_constant<int, (n - 8) / 2>{});
+          }
+          if constexpr (n >= 9 && n < 24 && n % 2 == 1) read_p1(std::integral_constant<int, (n - 9) / 2>{});
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      });
+      if (loads) lb.base += lb.step;
+      // B1. In flight behind part 0 of the next step: its part 1 and part 0 of the one after.
+      publish(loads ? 16 : 4);
+      // Half 1.
+      static_for<0, 32>([&](auto n_index) {
+        constexpr int n = decltype(n_index)::value, k = n / 8, t = (n % 8) / 4, u = n % 4;
+        product_of(acc[2 + t][u], fa1[t][k], fb[u][k]);
+        if constexpr (n < 8 && n % 2 == 0) {
+          if (loads) issue_p1(lds_here, std::integral_constant<int, n / 2>{});
+        }
+        // The next step's fragments of slab k - 1 go where this step's have just been used.
+        if constexpr (n >= 8 && n % 8 < 6)
+          read_p0(a_there, b_there, std::integral_constant<int, n / 8 - 1>{}, std::integral_constant<int, n % 8>{});
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      if (loads) la.base += la.step;
+      static_for<0, 6>([&](auto n_index) { read_p0(a_there, b_there, std::integral_constant<int, 3>{}, n_index); });
+      a_here.flip();
+      a_there.flip();
+      b_there.flip();
+      lds_here = lds_wave + ((j + 1) & 1) * W4_OPERAND;
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  } else {
+    // `here`: the stage of the step being multiplied, `there`: the other one.
+    W4Frags<true> a_here, a_there, b_here, b_there;
+    a_here.init(frag_offset<true, W4_BM, W4_BK>(wm * 128, 0, lane));
+    b_here.init(W4_B0 + frag_offset<true, W4_BN, W4_BK>(wn * 128, 0, lane));
+    a_there = a_here;
+    b_there = b_here;
+    a_there.flip();
+    b_there.flip();
+    // Part h of a stage: this wave's loads 4h .. 4h + 3 of A, then of B.
+    auto issue_part = [&](unsigned lds, auto h_index, auto n_index) {
+      constexpr int h = decltype(h_index)::value, n = decltype(n_index)::value;
+      constexpr int i = 4 * h + n % 4;
+      if constexpr (n < 4) la.template issue<i, NW * i * 1024>(lds);
+      else lb.template issue<i, W4_B0 + NW * i * 1024>(lds);
+    };
+    // fa[h][t][s]: row block t, K slab 2h + s; fb[h][u][s] likewise.
+    u32x4 fa[2][4][2], fb[2][4][2];
+    // Fragment n (0..15) of half h out of the stage `a` and `b` point at.
+    auto read_half = [&](auto h_index, const W4Frags<true>& a, const W4Frags<true>& b, auto n_index) {
+      constexpr int h = decltype(h_index)::value, n = decltype(n_index)::value;
+      constexpr int block = (n % 8) / 2, s = n % 2;
+      if constexpr (n < 8) fa[h][block][s] = a.template read<block, 2 * h + s>(smem);
+      else fb[h][block][s] = b.template read<block, 2 * h + s>(smem);
+    };
+    const std::integral_constant<int, 0> H0{};
+    const std::integral_constant<int, 1> H1{};
+
+    static_for<0, 8>([&](auto n_index) { issue_part(lds_wave, H0, n_index); });
+    static_for<0, 8>([&](auto n_index) { issue_part(lds_wave, H1, n_index); });
+    la.base += la.step;
+    lb.base += lb.step;
+    if (steps > 1) {
+      static_for<0, 8>([&](auto n_index) { issue_part(lds_wave + W4_OPERAND, H0, n_index); });
+      static_for<0, 8>([&](auto n_index) { issue_part(lds_wave + W4_OPERAND, H1, n_index); });
+      la.base += la.step;
+      lb.base += lb.step;
+    }
+    wait_loads(8 + (steps > 1 ? 16 : 0));
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<0, 16>([&](auto n_index) { read_half(H0, a_here, b_here, n_index); });
+    __builtin_amdgcn_sched_barrier(0);
+
+#pragma unroll 1
+    for (int j = 0; j < steps; ++j) {
+      const bool next = j + 1 < steps, loads = j + 2 < steps;
+      // Half 0.
+      static_for<0, 32>([&](auto n_index) {
+        constexpr int n = decltype(n_index)::value, s = n / 16, t = (n % 16) / 4, u = n % 4;
+        product_of(acc[t][u], fa[0][t][s], fb[0][u][s]);
+        if constexpr (n == 7) {
+          // B0. In flight behind part 1 of this step: both parts of the next.
+          publish(next ? 16 : 0);
+        } else {
+          if constexpr (n >= 8 && n < 24) {
+            if constexpr (n % 2 == 0) {
+              if (loads) issue_part(lds_here, H0, std::integral_constant<int, (n - 8) / 2>{});
+            }
+            read_half(H1, a_here, b_here, std::integral_constant<int, n - 8>{});
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      });
+      // B1. In flight behind part 0 of the next step: its part 1 and part 0 of the one after.
+      publish(loads ? 16 : 8);
+      // Half 1.
+      static_for<0, 32>([&](auto n_index) {
+        constexpr int n = decltype(n_index)::value, s = n / 16, t = (n % 16) / 4, u = n % 4;
+        product_of(acc[t][u], fa[1][t][s], fb[1][u][s]);
+        if constexpr (n < 16) {
+          if constexpr (n % 2 == 0) {
+            if (loads) issue_part(lds_here, H1, std::integral_constant<int, n / 2>{});
+          }
+          read_half(H0, a_there, b_there, n_index);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      if (loads) {
+        la.base += la.step;
+        lb.base += lb.step;
+      }
+      a_here.flip();
+      a_there.flip();
+      b_here.flip();
+      b_there.flip();
+      lds_here = lds_wave + ((j + 1) & 1) * W4_OPERAND;
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  // Every wave has read its last fragments before the stages are reused for the store pass.
+  __builtin_amdgcn_s_waitcnt(vmcnt_only(0) & 0xC07F);
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+
+  // Store pass: each wave stages 32 rows of its tile at a time through its own LDS region and
+  // writes whole 4-column pieces.
+  constexpr int CPW = TN * 32 + 4;
+  static_assert(NW * 32 * CPW * 4 <= W4_SMEM, "staging fits");
+  float* cs = reinterpret_cast<float*>(smem) + wave * (32 * CPW);
+  bool bad = false;
+  static_for<0, TM>([&](auto tm_index) {
+    constexpr int tm = decltype(tm_index)::value;
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) cs[(8 * (v >> 2) + 4 * lg + (v & 3)) * CPW + tn * 32 + l32] = acc[tm][tn][v];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    constexpr int PPR = TN * 8;  // 4-column pieces per row
+    const int grow0 = m0 + (wm * TM + tm) * 32, gcol0 = n0 + wn * TN * 32;
+    const bool interior = grow0 + 32 <= g.M && gcol0 + TN * 32 <= g.N;
+    bool stored = false;
+    if constexpr (EPI == OMX_EPI_NONE) {
+      if (interior && (g.splits > 1 ? (g.N & 3) == 0 : g.c_vec != 0)) {
+        if (g.splits > 1) bad |= gemm_store_block<0, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
+        else if (g.c_bf16) bad |= gemm_store_block<1, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
+        else if (!g.accumulate) bad |= gemm_store_block<2, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
+        else bad |= gemm_store_block<3, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
+        stored = true;
+      }
+    } else if constexpr (EPI == OMX_EPI_AXPBY) {
+      if (interior && g.c_vec != 0) {
+        bad |= gemm_epilogue_block<OMX_EPI_AXPBY, false, PPR>(g, cs, CPW, grow0, gcol0, lane);
+        stored = true;
+      }
+    } else {
+      if (interior && g.c_vec != 0) {
+        bad |= g.epi_tanh ? gemm_epilogue_block<EPI, true, PPR>(g, cs, CPW, grow0, gcol0, lane)
+                          : gemm_epilogue_block<EPI, false, PPR>(g, cs, CPW, grow0, gcol0, lane);
+        stored = true;
+      }
+    }
+    if (!stored) {
+#pragma unroll 1
+      for (int c = lane; c < 32 * PPR; c += 64) {
+        const int row = c / PPR, piece = c % PPR;
+        const int grow = grow0 + row, gcol = gcol0 + piece * 4;
+        if (grow < g.M && gcol < g.N) {
+          const float4 val = *reinterpret_cast<const float4*>(cs + row * CPW + piece * 4);
+          bad |= g.epi == OMX_EPI_NONE ? gemm_store4(g, split, grow, gcol, val.x, val.y, val.z, val.w)
+                                       : gemm_store4_epi(g, split, grow, gcol, val.x, val.y, val.z, val.w);
+        }
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  });
+  if (bad) dev_raise_fault(g.fault, g.tag);
+}
+
+// The leading dimensions whose 256-row lane offsets fit in 32 bits.
+inline bool w4_offsets_fit(const GemmArgs& g) { return g.lda < (1l << 22) && g.ldb < (1l << 22); }
+
+template <bool A_KM, bool B_KM>
+int32_t launch_w4(omx_ctx* ctx, const GemmArgs& g) {
+  auto kernel = g.epi == OMX_EPI_GELU_FWD   ? &gemm_w4_kernel<A_KM, B_KM, OMX_EPI_GELU_FWD>
+                : g.epi == OMX_EPI_GELU_BWD ? &gemm_w4_kernel<A_KM, B_KM, OMX_EPI_GELU_BWD>
+                : g.epi == OMX_EPI_AXPBY    ? &gemm_w4_kernel<A_KM, B_KM, OMX_EPI_AXPBY>
+                                            : &gemm_w4_kernel<A_KM, B_KM, OMX_EPI_NONE>;
+  OMX_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   W4_SMEM));
+  omx_launch_timed(ctx, kernel, dim3(g.tiles_m * g.tiles_n * g.splits, g.batches), dim3(256), W4_SMEM, ctx->timing_start,
+                   g.splits > 1 ? nullptr : ctx->timing_stop, g);
+  OMX_LAUNCH_CHECK(ctx, "gemm_w4_kernel");
+  return OMX_OK;
+}
+
+}  // namespace
