@@ -479,7 +479,7 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
     if (mode == 1 && ctx->gemm_forced_tiling >= 0) {
       dma_variant = ctx->gemm_forced_tiling;
     } else if (mode == 1) {
-      // Four tilings, chosen by how many tiles the output makes per compute unit and how many K
+      // Three tilings, chosen by how many tiles the output makes per compute unit and how many K
       // steps a tile runs, not by a model's dimensions (measured over GPT-124M's shapes and over
       // d = 1024 / 2048 / 4096 with 8192 tokens; tests/test_gpu_gemm_kernels.py holds the choice
       // to within 10 % of the best forced tiling):
@@ -491,15 +491,12 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
       //      the reduction split (3 to 20 % ahead of 256 x 128 there), and input gradients whose
       //      256 x 128 tiles would leave compute units empty, over at least 32 steps (8192 x 768
       //      over K = 3072: 52 against 66 us).
-      //   0  256 x 256, whole-line 64-column steps, one workgroup per compute unit: k-contiguous
-      //      A (forward and input-gradient products) over at least 32 steps when the tiles fill
-      //      the chip (K = 8192, 8192 x 2048 outputs: 233 against 282 us for 256 x 128), and the
-      //      tall weight-gradient batches.
-      //   8  the alternating 256 x 256 kernel: k-major products over long reductions when the
-      //      tiles fill the chip (4096 x 4096 over K = 8192: 225 against 241 us), and outputs of
-      //      four rounds of tiles or more over a short reduction (the head's forward product,
-      //      12608 tiles over K = 768: 1554 against 1642 us), where 0 pays its exposed first
-      //      loads once per 12 steps (1881 us).
+      //   9  256 x 256, one wave per SIMD, one workgroup per compute unit: nothing hides its first
+      //      loads and its store pass, so it takes long reductions whose tiles fill the chip
+      //      (K = 8192, 8192 x 2048 outputs: 203 against 276 us for 256 x 128; the weight-gradient
+      //      batches) and outputs of four rounds of tiles or more (the head's forward product). On
+      //      K = 768 with a round or three of tiles it is ahead when timed alone and behind inside
+      //      the training step (forward o 36.8 against 30.9 us).
       const bool unbatched = g.batches == 1;
       const bool plain = !(epi && epi->mode != OMX_EPI_NONE);
       const long outputs = static_cast<long>(g.M) * g.N;
@@ -529,16 +526,15 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
         dma_variant = 3;
       }
     }
-    else if (mode == 2) dma_variant = 0;
     else if (mode == 3) dma_variant = 3;
     else if (mode == 4) dma_variant = 6;
-    else if (mode == 8) dma_variant = 8;
     else if (mode == 9) dma_variant = 9;
+    if (dma_variant == 9 && !omx_gemm_w4_eligible(g, a_km, b_km)) dma_variant = 3;
   }
   // One 256 x 256 workgroup per compute unit: when the last round of tiles fills under 2/5 of the
   // chip (the head's weight gradient: 591 tiles on 256 units), the rows of the whole rounds go to
-  // this tiling and the rest to a launch of their own, which picks a smaller tile (1222 -> 1040 us).
-  if ((dma_variant == 0 || dma_variant >= 8) && ctx->gemm_dma_mode == 1 && ctx->gemm_row_split &&
+  // this tiling and the rest to a launch of their own, which picks a smaller tile (1181 -> 1034 us).
+  if (dma_variant == 9 && ctx->gemm_dma_mode == 1 && ctx->gemm_row_split &&
       !ctx->gemm_in_row_split && batches == 1 && !(epi && epi->mode != OMX_EPI_NONE)) {
     const long cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
     const long tm = (g.M + 255) / 256, tn = (g.N + 255) / 256;
@@ -587,7 +583,7 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
         int p2 = 1;
         while (p2 * 2 <= splits + splits / 4) p2 *= 2;  // 7..9 -> 8, 10..12 -> 8, 13..16 -> 16
         splits = p2;
-        if (dma_variant == 0 || dma_variant >= 8) {
+        if (dma_variant == 9) {
           // One workgroup per compute unit: what counts is how full the last round of workgroups is
           // (192 tiles split in two are 384 workgroups on 256 units, a round and a half; split in
           // four they are three full rounds of half the length). More splits only for a chip at
@@ -724,7 +720,8 @@ int32_t omx_set_option(omx_ctx* ctx, const char* name, int64_t value) {
     return OMX_OK;
   }
   if (name && strcmp(name, "gemm_dma") == 0) {
-    if (value < 0 || (value > 4 && value != 8 && value != 9)) return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: gemm_dma takes 0..4 or 8");
+    if (value != 0 && value != 1 && value != 3 && value != 4 && value != 9)
+      return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: gemm_dma takes 0, 1, 3, 4 or 9");
     ctx->gemm_dma_mode = static_cast<int>(value);
     return OMX_OK;
   }

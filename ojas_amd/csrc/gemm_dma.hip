@@ -43,9 +43,15 @@ bool omx_gemm_dma_eligible(const GemmArgs& g, bool a_km, bool b_km) {
   return true;
 }
 
+// The one-wave-per-SIMD kernel (variant 9) also needs a k-major B with a k-major A, and leading
+// dimensions whose 256-row lane offsets fit in 32 bits.
+bool omx_gemm_w4_eligible(const GemmArgs& g, bool a_km, bool b_km) {
+  return (!a_km || b_km) && g.lda < (1l << 22) && g.ldb < (1l << 22);
+}
+
 void omx_gemm_dma_tile(int variant, int* bm, int* bn) {
   *bm = variant == 6 ? 128 : 256;
-  *bn = variant == 0 || variant == 8 || variant == 9 ? 256 : 128;
+  *bn = variant == 9 ? 256 : 128;
 }
 
 

@@ -3,7 +3,6 @@
 // holds the description of the kernels and chooses among the four.
 #pragma once
 #include "gemm_tiles.h"
-#include "gemm_pp_impl.h"
 #include "gemm_w4_impl.h"
 
 namespace {
@@ -636,19 +635,16 @@ int32_t launch_dma(omx_ctx* ctx, const GemmArgs& g) {
   return OMX_OK;
 }
 
-// The three tilings the dispatcher chooses among: 0: 256 x 256 in 64-column steps (whole cache
-// lines, two stages, one workgroup per compute unit); 3: 256 x 128 in 32-column steps (three
-// stages, two workgroups per compute unit); 6: 128 x 128 with four waves (three per compute unit).
+// The tilings the dispatcher chooses among: 9: 256 x 256, one wave per SIMD, one workgroup per
+// compute unit (gemm_w4_impl.h); 3: 256 x 128 in 32-column steps (three stages, two workgroups per
+// compute unit); 6: 128 x 128 with four waves (three per compute unit).
 template <bool A_KM, bool B_KM>
 int32_t launch_variant(omx_ctx* ctx, const GemmArgs& g, int variant) {
   if (variant == 9) {
-    if constexpr (!A_KM || B_KM) {
-      if (w4_offsets_fit(g)) return launch_w4<A_KM, B_KM>(ctx, g);
-    }
-    return launch_pp<A_KM, B_KM>(ctx, g);
+    // (the caller has asked omx_gemm_w4_eligible: a k-major A comes with a k-major B)
+    if constexpr (!A_KM || B_KM) return launch_w4<A_KM, B_KM>(ctx, g);
+    else return omx_fail(ctx, OMX_SHAPE, "gemm: no one-wave-per-SIMD kernel for this operand layout");
   }
-  if (variant == 8) return launch_pp<A_KM, B_KM>(ctx, g);
-  if (variant == 0) return launch_dma<A_KM, B_KM, 2, 4, 4, 2, 64, 2>(ctx, g);
   if (variant == 6) return launch_dma<A_KM, B_KM, 2, 2, 2, 2, 32, 3>(ctx, g);
   return launch_dma<A_KM, B_KM, 4, 2, 2, 2, 32, 3>(ctx, g);
 }

@@ -426,9 +426,6 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
   if (bad) dev_raise_fault(g.fault, g.tag);
 }
 
-// The leading dimensions whose 256-row lane offsets fit in 32 bits.
-inline bool w4_offsets_fit(const GemmArgs& g) { return g.lda < (1l << 22) && g.ldb < (1l << 22); }
-
 template <bool A_KM, bool B_KM>
 int32_t launch_w4(omx_ctx* ctx, const GemmArgs& g) {
   auto kernel = g.epi == OMX_EPI_GELU_FWD   ? &gemm_w4_kernel<A_KM, B_KM, OMX_EPI_GELU_FWD>
