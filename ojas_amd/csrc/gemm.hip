@@ -515,6 +515,7 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
       } else if (a_km && b_km) {
         // Weight gradients (K = tokens). An unbatched product with a poor last round is cut by rows below.
         if (plain && ksteps64 >= 64 && all256 >= cus && (unbatched || all256 * 5 >= rounds256 * cus * 4)) dma_variant = 9;
+        else if (plain && !unbatched && ksteps64 >= 128 && all256 < cus && all256 * 8 >= cus) dma_variant = 9;  // with K split
         else dma_variant = 3;
       } else if (!a_km) {
         const long tiles256x128 = static_cast<long>((g.M + 255) / 256) * ((g.N + 127) / 128);
@@ -571,10 +572,12 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
     int splits = 1;
     // An f32 step is 64 MFMAs per wave (1.7 us): two of them already pay for a split.
     const int min_steps = operand_dtype == OMX_BF16 ? 8 : 2;
-    // A strided batch splits only on the register-staged kernel (thin outputs over a long
-    // reduction: 16 products of 16 tiles each leave three quarters of the chip's wave slots empty).
+    // A strided batch splits on the register-staged kernel (thin outputs over a long reduction: 16
+    // products of 16 tiles each leave three quarters of the chip's wave slots empty) and on the
+    // 256 x 256 kernel when its tiles do not fill one round (12 products of 768 x 768).
     const long all_tiles = tiles * g.batches;
-    const bool may_split = !thin && (g.batches == 1 ? tiles < 256 : (dma_variant < 0 && all_tiles < 512));
+    const bool may_split =
+        !thin && (g.batches == 1 ? tiles < 256 : ((dma_variant < 0 && all_tiles < 512) || (dma_variant == 9 && all_tiles < 256)));
     if (may_split && ksteps >= 4 * min_steps && !(epi && epi->mode != OMX_EPI_NONE)) {
       splits = static_cast<int>(((g.batches == 1 ? 512 : 1024) + all_tiles - 1) / all_tiles);
       if (splits > ksteps / min_steps) splits = ksteps / min_steps;
@@ -586,12 +589,12 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
         if (dma_variant == 9) {
           // One workgroup per compute unit: what counts is how full the last round of workgroups is
           // (192 tiles split in two are 384 workgroups on 256 units, a round and a half; split in
-          // four they are three full rounds of half the length). More splits only for a chip at
-          // least a tenth fuller: each costs a slice of partial sums and of the reduce pass.
+          // four they are three full rounds of half the length). More splits, four at most, only for a
+          // chip at least a tenth fuller: each costs a slice of partial sums and of the reduce pass.
           const long units = ctx->cu_count > 0 ? ctx->cu_count : 256;
           int best = 1;
           double best_fill = 0.0;
-          for (int s2 = 1; s2 <= 16 && ksteps / s2 >= min_steps; s2 *= 2) {
+          for (int s2 = 1; s2 <= 4 && ksteps / s2 >= 4 * min_steps; s2 *= 2) {
             const long groups = all_tiles * s2;
             const double fill = static_cast<double>(groups) / static_cast<double>((groups + units - 1) / units * units);
             if (fill > best_fill + 0.1) {
