@@ -507,7 +507,6 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
       // How full the last round of 256 x 256 tiles is, one workgroup per compute unit.
       const long all256 = tiles256 * g.batches;
       const long rounds256 = (all256 + cus - 1) / cus;
-      const bool fills256 = all256 * 8 >= rounds256 * cus * 7;
       if (a_km && b_km && unbatched && ksteps64 >= 64 && tiles128 < cus) {
         dma_variant = 6;
       } else if (outputs * g.batches <= (1l << 20)) {
@@ -515,12 +514,11 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
       } else if (a_km && b_km) {
         // Weight gradients (K = tokens). An unbatched product with a poor last round is cut by rows below.
         if (plain && ksteps64 >= 64 && all256 >= cus && (unbatched || all256 * 5 >= rounds256 * cus * 4)) dma_variant = 9;
-        else if (plain && !unbatched && ksteps64 >= 128 && all256 < cus && all256 * 8 >= cus) dma_variant = 9;  // with K split
+        else if (plain && !unbatched && ksteps64 >= 128 && all256 * 8 >= cus) dma_variant = 9;  // with K split
         else dma_variant = 3;
       } else if (!a_km) {
         const long tiles256x128 = static_cast<long>((g.M + 255) / 256) * ((g.N + 127) / 128);
-        if (unbatched && plain && tiles256 >= 4 * cus && ksteps64 < 32) dma_variant = 9;
-        else if (unbatched && plain && ((tiles256 >= cus && fills256 && ksteps64 >= 32) || ksteps64 >= 512)) dma_variant = 9;
+        if (unbatched && plain && tiles256 * 2 >= cus) dma_variant = 9;
         else if (unbatched && plain && b_km && tiles256x128 < cus && ksteps64 >= 32) dma_variant = 6;
         else dma_variant = 3;
       } else {
@@ -574,10 +572,11 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
     const int min_steps = operand_dtype == OMX_BF16 ? 8 : 2;
     // A strided batch splits on the register-staged kernel (thin outputs over a long reduction: 16
     // products of 16 tiles each leave three quarters of the chip's wave slots empty) and on the
-    // 256 x 256 kernel when its tiles do not fill one round (12 products of 768 x 768).
+    // 256 x 256 kernel when that fills its last round of tiles better (12 products of 768 x 768 are
+    // 108 tiles: two splits; of 2304 x 768, 324 tiles: two splits make three rounds of half the length).
     const long all_tiles = tiles * g.batches;
     const bool may_split =
-        !thin && (g.batches == 1 ? tiles < 256 : ((dma_variant < 0 && all_tiles < 512) || (dma_variant == 9 && all_tiles < 256)));
+        !thin && (g.batches == 1 ? tiles < 256 : ((dma_variant < 0 && all_tiles < 512) || dma_variant == 9));
     if (may_split && ksteps >= 4 * min_steps && !(epi && epi->mode != OMX_EPI_NONE)) {
       splits = static_cast<int>(((g.batches == 1 ? 512 : 1024) + all_tiles - 1) / all_tiles);
       if (splits > ksteps / min_steps) splits = ksteps / min_steps;
@@ -590,14 +589,14 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
           // One workgroup per compute unit: what counts is how full the last round of workgroups is
           // (192 tiles split in two are 384 workgroups on 256 units, a round and a half; split in
           // four they are three full rounds of half the length). More splits, four at most, only for a
-          // chip at least a tenth fuller: each costs a slice of partial sums and of the reduce pass.
+          // chip fuller by 0.15 of its units: each costs a slice of partial sums and of the reduce pass.
           const long units = ctx->cu_count > 0 ? ctx->cu_count : 256;
           int best = 1;
           double best_fill = 0.0;
           for (int s2 = 1; s2 <= 4 && ksteps / s2 >= 4 * min_steps; s2 *= 2) {
             const long groups = all_tiles * s2;
             const double fill = static_cast<double>(groups) / static_cast<double>((groups + units - 1) / units * units);
-            if (fill > best_fill + 0.1) {
+            if (fill > best_fill + 0.15) {
               best = s2;
               best_fill = fill;
             }

@@ -25,6 +25,12 @@
 #pragma once
 #include "gemm_tiles.h"
 
+#ifdef W4_TRACE
+__device__ long long* w4_trace_buf;
+#define W4_STAMP(i) do { if (w4_trace_buf && threadIdx.x == 0 && blockIdx.y == 0) { w4_trace_buf[blockIdx.x * 16 + (i)] = wall_clock64(); w4_trace_buf[blockIdx.x * 16 + 8 + (i)] = clock64(); } } while (0)
+#else
+#define W4_STAMP(i)
+#endif
 namespace {
 
 constexpr int W4_BM = 256, W4_BN = 256, W4_BK = 64;
@@ -100,6 +106,7 @@ template <bool A_KM, bool B_KM, int EPI>
 __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
   static_assert(!A_KM || B_KM, "a k-major A goes with a k-major B");
   extern __shared__ __attribute__((aligned(1024))) char smem[];
+  W4_STAMP(0);
   constexpr int TM = 4, TN = 4, NW = 4;
   // Tile order: as gemm_dma_kernel.
   const int total = g.tiles_m * g.tiles_n;
@@ -137,12 +144,17 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
   const int l32 = lane & 31, lg = lane >> 5;
 
   floatx16 acc[TM][TN];
+  // Cleared once the first loads are on their way (256 register writes).
+  auto clear_acc = [&]() {
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
+      for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+    __builtin_amdgcn_sched_barrier(0);
+  };
 
   const int ks_begin = split * g.ksteps_per_split;
   const int ks_end = min(g.K / W4_BK, ks_begin + g.ksteps_per_split);
@@ -168,8 +180,16 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
   };
+  // The plain kernel multiplies with the operands exchanged: a lane then holds, for ONE output row
+  // (block row l32), four consecutive columns per register quad (8 (v / 4) + 4 lg + v % 4), which
+  // the store pass packs and stages 8 or 16 bytes at a time. With an activation in the store pass
+  // a lane holds one column and 16 rows, the layout gemm_epilogue_block's staging expects.
+  constexpr bool ROW_LANES = EPI == OMX_EPI_NONE;
   auto product_of = [&](floatx16& c, const u32x4& a, const u32x4& b) {
-    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    if constexpr (ROW_LANES)
+      c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, b), __builtin_bit_cast(bf16x8, a), c, 0, 0, 0);
+    else
+      c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
   };
   unsigned lds_here = lds_wave;  // where this wave's loads into the current stage go
   if constexpr (!A_KM) {
@@ -222,14 +242,21 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
       la.base += la.step;
       lb.base += lb.step;
     }
+    W4_STAMP(1);
+    clear_acc();
     wait_loads(4 + (steps > 1 ? 16 : 0));
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
+    W4_STAMP(2);
     static_for<0, 4>([&](auto k_index) {
       static_for<0, 6>([&](auto n_index) { read_p0(a_here, b_there, k_index, n_index); });
     });
     b_there.flip();
     __builtin_amdgcn_sched_barrier(0);
+#ifdef W4_TRACE
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    W4_STAMP(3);
+#endif
 
     // One K step per turn: the same code for every step, so the accumulators stay where they are.
     // `next`: another step follows; `loads`: two more follow (the loads of the second start here).
@@ -313,6 +340,7 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
       la.base += la.step;
       lb.base += lb.step;
     }
+    clear_acc();
     wait_loads(8 + (steps > 1 ? 16 : 0));
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
@@ -369,60 +397,123 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
   __builtin_amdgcn_s_waitcnt(vmcnt_only(0) & 0xC07F);
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_sched_barrier(0);
+  W4_STAMP(4);
 
   // Store pass: each wave stages 32 rows of its tile at a time through its own LDS region and
-  // writes whole 4-column pieces.
+  // writes whole pieces of rows.
   constexpr int CPW = TN * 32 + 4;
   static_assert(NW * 32 * CPW * 4 <= W4_SMEM, "staging fits");
   float* cs = reinterpret_cast<float*>(smem) + wave * (32 * CPW);
   bool bad = false;
-  static_for<0, TM>([&](auto tm_index) {
-    constexpr int tm = decltype(tm_index)::value;
+  constexpr int PPR = TN * 8;  // 4-column pieces per row
+  const int gcol0 = n0 + wn * TN * 32;
+  if constexpr (ROW_LANES) {
+    const bool packed = g.splits == 1 && g.c_bf16 && g.c_vec != 0 && (g.ldc & 7) == 0 &&
+                        (reinterpret_cast<uintptr_t>(g.c) & 15) == 0;
+    constexpr int HP = TN * 32 * 2 + 16;  // bytes per staged bf16 row
+    char* hs = reinterpret_cast<char*>(cs);
+    unsigned flags = 0;  // bit 15 or 31 set: a stored bf16 has an all-ones exponent
+    static_for<0, TM>([&](auto tm_index) {
+      constexpr int tm = decltype(tm_index)::value;
+      const int grow0 = m0 + (wm * TM + tm) * 32;
+      const bool interior = grow0 + 32 <= g.M && gcol0 + TN * 32 <= g.N;
+      if (packed && interior) {
+        // bf16: rounded in registers, staged 8 bytes at a time, stored 16 bytes per lane (a wave
+        // instruction writes four rows of 256 bytes).
 #pragma unroll
-    for (int tn = 0; tn < TN; ++tn)
+        for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) cs[(8 * (v >> 2) + 4 * lg + (v & 3)) * CPW + tn * 32 + l32] = acc[tm][tn][v];
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    constexpr int PPR = TN * 8;  // 4-column pieces per row
-    const int grow0 = m0 + (wm * TM + tm) * 32, gcol0 = n0 + wn * TN * 32;
-    const bool interior = grow0 + 32 <= g.M && gcol0 + TN * 32 <= g.N;
-    bool stored = false;
-    if constexpr (EPI == OMX_EPI_NONE) {
-      if (interior && (g.splits > 1 ? (g.N & 3) == 0 : g.c_vec != 0)) {
-        if (g.splits > 1) bad |= gemm_store_block<0, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
-        else if (g.c_bf16) bad |= gemm_store_block<1, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
-        else if (!g.accumulate) bad |= gemm_store_block<2, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
-        else bad |= gemm_store_block<3, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
-        stored = true;
-      }
-    } else if constexpr (EPI == OMX_EPI_AXPBY) {
-      if (interior && g.c_vec != 0) {
-        bad |= gemm_epilogue_block<OMX_EPI_AXPBY, false, PPR>(g, cs, CPW, grow0, gcol0, lane);
-        stored = true;
-      }
-    } else {
-      if (interior && g.c_vec != 0) {
-        bad |= g.epi_tanh ? gemm_epilogue_block<EPI, true, PPR>(g, cs, CPW, grow0, gcol0, lane)
-                          : gemm_epilogue_block<EPI, false, PPR>(g, cs, CPW, grow0, gcol0, lane);
-        stored = true;
-      }
-    }
-    if (!stored) {
+          for (int q = 0; q < 4; ++q) {
+            const floatx16& c = acc[tm][tn];
+            uint2 w;
+            w.x = dev_pack_bf16_pair(c[4 * q], c[4 * q + 1]);
+            w.y = dev_pack_bf16_pair(c[4 * q + 2], c[4 * q + 3]);
+            flags |= ((w.x & 0x7F807F80u) + 0x00800080u) | ((w.y & 0x7F807F80u) + 0x00800080u);
+            *reinterpret_cast<uint2*>(hs + l32 * HP + (tn * 32 + 8 * q + 4 * lg) * 2) = w;
+          }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        unsigned short* crow = static_cast<unsigned short*>(g.c) + static_cast<long>(grow0 + (lane >> 4)) * g.ldc + gcol0 +
+                               (lane & 15) * 8;
+        const long four_rows = 4 * g.ldc;
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+          const uint4 v = *reinterpret_cast<const uint4*>(hs + (it * 4 + (lane >> 4)) * HP + (lane & 15) * 16);
+          *reinterpret_cast<uint4*>(crow + it * four_rows) = v;
+        }
+      } else {
+        // f32 results, split-K partials, ragged edges: staged as f32 rows.
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const floatx16& c = acc[tm][tn];
+            *reinterpret_cast<float4*>(cs + l32 * CPW + tn * 32 + 8 * q + 4 * lg) =
+                make_float4(c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]);
+          }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        if (interior && (g.splits > 1 ? (g.N & 3) == 0 : g.c_vec != 0)) {
+          if (g.splits > 1) bad |= gemm_store_block<0, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
+          else if (g.c_bf16) bad |= gemm_store_block<1, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
+          else if (!g.accumulate) bad |= gemm_store_block<2, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
+          else bad |= gemm_store_block<3, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
+        } else {
 #pragma unroll 1
-      for (int c = lane; c < 32 * PPR; c += 64) {
-        const int row = c / PPR, piece = c % PPR;
-        const int grow = grow0 + row, gcol = gcol0 + piece * 4;
-        if (grow < g.M && gcol < g.N) {
-          const float4 val = *reinterpret_cast<const float4*>(cs + row * CPW + piece * 4);
-          bad |= g.epi == OMX_EPI_NONE ? gemm_store4(g, split, grow, gcol, val.x, val.y, val.z, val.w)
-                                       : gemm_store4_epi(g, split, grow, gcol, val.x, val.y, val.z, val.w);
+          for (int c = lane; c < 32 * PPR; c += 64) {
+            const int row = c / PPR, piece = c % PPR;
+            const int grow = grow0 + row, gcol = gcol0 + piece * 4;
+            if (grow < g.M && gcol < g.N) {
+              const float4 val = *reinterpret_cast<const float4*>(cs + row * CPW + piece * 4);
+              bad |= gemm_store4(g, split, grow, gcol, val.x, val.y, val.z, val.w);
+            }
+          }
         }
       }
-    }
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-  });
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    });
+    bad |= (flags & 0x80008000u) != 0;
+  } else {
+    static_for<0, TM>([&](auto tm_index) {
+      constexpr int tm = decltype(tm_index)::value;
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) cs[(8 * (v >> 2) + 4 * lg + (v & 3)) * CPW + tn * 32 + l32] = acc[tm][tn][v];
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      const int grow0 = m0 + (wm * TM + tm) * 32;
+      const bool interior = grow0 + 32 <= g.M && gcol0 + TN * 32 <= g.N;
+      bool stored = false;
+      if constexpr (EPI == OMX_EPI_AXPBY) {
+        if (interior && g.c_vec != 0) {
+          bad |= gemm_epilogue_block<OMX_EPI_AXPBY, false, PPR>(g, cs, CPW, grow0, gcol0, lane);
+          stored = true;
+        }
+      } else {
+        if (interior && g.c_vec != 0) {
+          bad |= g.epi_tanh ? gemm_epilogue_block<EPI, true, PPR>(g, cs, CPW, grow0, gcol0, lane)
+                            : gemm_epilogue_block<EPI, false, PPR>(g, cs, CPW, grow0, gcol0, lane);
+          stored = true;
+        }
+      }
+      if (!stored) {
+#pragma unroll 1
+        for (int c = lane; c < 32 * PPR; c += 64) {
+          const int row = c / PPR, piece = c % PPR;
+          const int grow = grow0 + row, gcol = gcol0 + piece * 4;
+          if (grow < g.M && gcol < g.N) {
+            const float4 val = *reinterpret_cast<const float4*>(cs + row * CPW + piece * 4);
+            bad |= gemm_store4_epi(g, split, grow, gcol, val.x, val.y, val.z, val.w);
+          }
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    });
+  }
+  W4_STAMP(5);
   if (bad) dev_raise_fault(g.fault, g.tag);
 }
 
