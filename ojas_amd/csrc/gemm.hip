@@ -514,11 +514,11 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
       } else if (a_km && b_km) {
         // Weight gradients (K = tokens). An unbatched product with a poor last round is cut by rows below.
         if (plain && ksteps64 >= 64 && all256 >= cus && (unbatched || all256 * 5 >= rounds256 * cus * 4)) dma_variant = 9;
-        else if (plain && !unbatched && ksteps64 >= 128 && all256 * 8 >= cus) dma_variant = 9;  // with K split
+        else if (plain && ksteps64 >= 128 && all256 * 8 >= cus) dma_variant = 9;  // with K split
         else dma_variant = 3;
       } else if (!a_km) {
         const long tiles256x128 = static_cast<long>((g.M + 255) / 256) * ((g.N + 127) / 128);
-        if (unbatched && plain && tiles256 * 2 >= cus) dma_variant = 9;
+        if (unbatched && plain && tiles256 * 4 >= cus * 3) dma_variant = 9;
         else if (unbatched && plain && b_km && tiles256x128 < cus && ksteps64 >= 32) dma_variant = 6;
         else dma_variant = 3;
       } else {
@@ -588,15 +588,16 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
         if (dma_variant == 9) {
           // One workgroup per compute unit: what counts is how full the last round of workgroups is
           // (192 tiles split in two are 384 workgroups on 256 units, a round and a half; split in
-          // four they are three full rounds of half the length). More splits, four at most, only for a
-          // chip fuller by 0.15 of its units: each costs a slice of partial sums and of the reduce pass.
+          // four they are three full rounds of half the length). A split's partial sums cost 8 bytes
+          // of traffic per output element against 2 K operations: at 4 TB/s and 1 PFLOP/s that is
+          // 1000 / K of the product's time per split, which the fuller chip has to pay back.
           const long units = ctx->cu_count > 0 ? ctx->cu_count : 256;
           int best = 1;
           double best_fill = 0.0;
           for (int s2 = 1; s2 <= 4 && ksteps / s2 >= 4 * min_steps; s2 *= 2) {
             const long groups = all_tiles * s2;
             const double fill = static_cast<double>(groups) / static_cast<double>((groups + units - 1) / units * units);
-            if (fill > best_fill + 0.15) {
+            if (fill > best_fill * (1.0 + 1000.0 * s2 / static_cast<double>(g.K)) + 0.05) {
               best = s2;
               best_fill = fill;
             }
@@ -606,6 +607,7 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
       }
     }
     g.ksteps_per_split = (ksteps + splits - 1) / splits;
+    if (dma_variant == 9) g.ksteps_per_split += g.ksteps_per_split & 1;  // its K loop takes steps in pairs
     g.splits = (ksteps + g.ksteps_per_split - 1) / g.ksteps_per_split;
     g.partial = nullptr;
     if (g.splits > 1) {

@@ -19,18 +19,13 @@
 //   part 0 of this step, and publishes part 1; part 0 of step j + 2 is loaded behind it. B1,
 //   between the halves, says that part 1 has been read and publishes part 0 of step j + 1; part 1
 //   of step j + 2 is loaded behind it. Every load has more than a step to land.
-//   The K loop is one body for every step (the stage is a register, the last steps skip their
-//   loads by scalar branches): with copies of the body for the last steps the compiler permutes
-//   the 256 accumulator registers between the copies through scratch memory.
+//   The K loop holds one copy of the step per stage and nothing else: the last steps skip their
+//   loads by scalar branches, and the step count is even (K a multiple of 128, an even number of
+//   steps per split). With further copies of the step, or a branch around the second one, the
+//   compiler permutes the 256 accumulator registers between the copies through scratch memory.
 #pragma once
 #include "gemm_tiles.h"
 
-#ifdef W4_TRACE
-__device__ long long* w4_trace_buf;
-#define W4_STAMP(i) do { if (w4_trace_buf && threadIdx.x == 0 && blockIdx.y == 0) { w4_trace_buf[blockIdx.x * 16 + (i)] = wall_clock64(); w4_trace_buf[blockIdx.x * 16 + 8 + (i)] = clock64(); } } while (0)
-#else
-#define W4_STAMP(i)
-#endif
 namespace {
 
 constexpr int W4_BM = 256, W4_BN = 256, W4_BK = 64;
@@ -79,25 +74,32 @@ struct W4Loads {
   }
 };
 
-// Fragment addresses of one operand in one stage: four registers; the block and the K slab are
-// immediates. flip() moves them to the other stage.
+// Fragment addresses of one operand: four registers holding LDS byte addresses in stage 0; the
+// block, the K slab and the stage are immediates of the read.
 template <bool KM>
 struct W4Frags {
-  int b[4];
-  __device__ __forceinline__ void init(int first) {
+  unsigned b[4];
+  __device__ __forceinline__ void init(unsigned first) {
 #pragma unroll
-    for (int x = 0; x < 4; ++x) b[x] = KM ? first ^ (x << 6) : first ^ (x << 5);
+    for (int x = 0; x < 4; ++x) {
+      b[x] = KM ? first ^ (x << 6) : first ^ (x << 5);
+      // Held as it is: re-derived from its parts, a read would pay an addition for what the
+      // instruction's offset field carries for nothing.
+      asm volatile("" : "+v"(b[x]));
+    }
   }
-  __device__ __forceinline__ void flip() {
-#pragma unroll
-    for (int x = 0; x < 4; ++x) b[x] ^= W4_OPERAND;
-  }
-  template <int T, int KK>
-  __device__ __forceinline__ u32x4 read(const char* smem) const {
+  template <int T, int KK, int STAGE>
+  __device__ __forceinline__ u32x4 read() const {
     if constexpr (!KM) {
-      return *reinterpret_cast<const u32x4*>(smem + b[KK] + T * 32 * W4_BK * 2);
+      typedef const u32x4 __attribute__((address_space(3))) * lds_ptr;
+      return *reinterpret_cast<lds_ptr>(static_cast<uintptr_t>(b[KK] + (T * 32 * W4_BK * 2 + STAGE * W4_OPERAND)));
     } else {
-      return frag_at<true, 256>(smem + b[T] + KK * 16 * 256 * 2);
+      typedef short4v __attribute__((address_space(3))) * lds_ptr;
+      const unsigned p = b[T] + (KK * 16 * 256 * 2 + STAGE * W4_OPERAND);
+      short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<lds_ptr>(static_cast<uintptr_t>(p)));
+      short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<lds_ptr>(static_cast<uintptr_t>(p + 4 * 256 * 2)));
+      u32x2 x = __builtin_bit_cast(u32x2, lo), y = __builtin_bit_cast(u32x2, hi);
+      return u32x4{x.x, x.y, y.x, y.y};
     }
   }
 };
@@ -106,7 +108,6 @@ template <bool A_KM, bool B_KM, int EPI>
 __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
   static_assert(!A_KM || B_KM, "a k-major A goes with a k-major B");
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  W4_STAMP(0);
   constexpr int TM = 4, TN = 4, NW = 4;
   // Tile order: as gemm_dma_kernel.
   const int total = g.tiles_m * g.tiles_n;
@@ -191,79 +192,72 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
     else
       c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
   };
-  unsigned lds_here = lds_wave;  // where this wave's loads into the current stage go
+  const unsigned lds0 = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(reinterpret_cast<uintptr_t>(smem)));
+  const std::integral_constant<int, 0> S0{};
+  const std::integral_constant<int, 1> S1{};
   if constexpr (!A_KM) {
-    // `here`: the stage of the step being multiplied, `there`: the other one. B is only ever read a
-    // step ahead.
-    W4Frags<false> a_here, a_there;
-    W4Frags<B_KM> b_there;
-    a_here.init(frag_offset<false, W4_BM, W4_BK>(wm * 128, 0, lane));
-    a_there.init(frag_offset<false, W4_BM, W4_BK>(wm * 128, 0, lane));
-    b_there.init(W4_B0 + frag_offset<B_KM, W4_BN, W4_BK>(wn * 128, 0, lane));
-    a_there.flip();  // the loop starts in stage 0 (b_there follows once step 0's fragments are read)
+    W4Frags<false> ra;
+    W4Frags<B_KM> rb;
+    ra.init(lds0 + frag_offset<false, W4_BM, W4_BK>(wm * 128, 0, lane));
+    rb.init(lds0 + W4_B0 + frag_offset<B_KM, W4_BN, W4_BK>(wn * 128, 0, lane));
 
     // Part 0 of a stage: all of B and A's loads 0, 1, 4, 5 (rows 0-63 and 128-191 of the tile);
     // part 1: A's loads 2, 3, 6, 7. `n` counts the part's loads.
-    auto issue_p0 = [&](unsigned lds, auto n_index) {
-      constexpr int n = decltype(n_index)::value;
+    auto issue_p0 = [&](auto stage_index, auto n_index) {
+      constexpr int stage = decltype(stage_index)::value, n = decltype(n_index)::value;
       if constexpr (n < 8) {
-        lb.template issue<n, W4_B0 + NW * n * 1024>(lds);
+        lb.template issue<n, W4_B0 + stage * W4_OPERAND + NW * n * 1024>(lds_wave);
       } else {
         constexpr int i = n == 8 ? 0 : n == 9 ? 1 : n == 10 ? 4 : 5;
-        la.template issue<i, NW * i * 1024>(lds);
+        la.template issue<i, stage * W4_OPERAND + NW * i * 1024>(lds_wave);
       }
     };
-    auto issue_p1 = [&](unsigned lds, auto n_index) {
-      constexpr int n = decltype(n_index)::value;
+    auto issue_p1 = [&](auto stage_index, auto n_index) {
+      constexpr int stage = decltype(stage_index)::value, n = decltype(n_index)::value;
       constexpr int i = n == 0 ? 2 : n == 1 ? 3 : n == 2 ? 6 : 7;
-      la.template issue<i, NW * i * 1024>(lds);
+      la.template issue<i, stage * W4_OPERAND + NW * i * 1024>(lds_wave);
     };
     // fa0[t][k]: row blocks 0-1, fa1[t][k]: row blocks 2-3, fb[u][k]: column blocks, K slab k.
     u32x4 fa0[2][4], fa1[2][4], fb[4][4];
-    // Fragment n (0..5) of K slab k of part 0 of the stage `a` and `b` point at: four of B, two of A.
-    auto read_p0 = [&](const W4Frags<false>& a, const W4Frags<B_KM>& b, auto k_index, auto n_index) {
-      constexpr int k = decltype(k_index)::value, n = decltype(n_index)::value;
-      if constexpr (n < 4) fb[n][k] = b.template read<n, k>(smem);
-      else fa0[n - 4][k] = a.template read<n - 4, k>(smem);
+    // Fragment n (0..5) of K slab k of part 0 of a stage: four of B, two of A.
+    auto read_p0 = [&](auto stage_index, auto k_index, auto n_index) {
+      constexpr int stage = decltype(stage_index)::value, k = decltype(k_index)::value, n = decltype(n_index)::value;
+      if constexpr (n < 4) fb[n][k] = rb.template read<n, k, stage>();
+      else fa0[n - 4][k] = ra.template read<n - 4, k, stage>();
     };
-    // Fragment n (0..7) of part 1 of the current stage: K slab n / 2, row block 2 + n % 2.
-    auto read_p1 = [&](auto n_index) {
-      constexpr int n = decltype(n_index)::value;
-      fa1[n % 2][n / 2] = a_here.template read<2 + n % 2, n / 2>(smem);
+    // Fragment n (0..7) of part 1 of a stage: K slab n / 2, row block 2 + n % 2.
+    auto read_p1 = [&](auto stage_index, auto n_index) {
+      constexpr int stage = decltype(stage_index)::value, n = decltype(n_index)::value;
+      fa1[n % 2][n / 2] = ra.template read<2 + n % 2, n / 2, stage>();
     };
     // Both stages' loads, part 0 of step 0 published, its fragments read.
-    static_for<0, 12>([&](auto n_index) { issue_p0(lds_wave, n_index); });
-    static_for<0, 4>([&](auto n_index) { issue_p1(lds_wave, n_index); });
+    static_for<0, 12>([&](auto n_index) { issue_p0(S0, n_index); });
+    static_for<0, 4>([&](auto n_index) { issue_p1(S0, n_index); });
     la.base += la.step;
     lb.base += lb.step;
     if (steps > 1) {
-      static_for<0, 12>([&](auto n_index) { issue_p0(lds_wave + W4_OPERAND, n_index); });
-      static_for<0, 4>([&](auto n_index) { issue_p1(lds_wave + W4_OPERAND, n_index); });
+      static_for<0, 12>([&](auto n_index) { issue_p0(S1, n_index); });
+      static_for<0, 4>([&](auto n_index) { issue_p1(S1, n_index); });
       la.base += la.step;
       lb.base += lb.step;
     }
-    W4_STAMP(1);
     clear_acc();
     wait_loads(4 + (steps > 1 ? 16 : 0));
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
-    W4_STAMP(2);
     static_for<0, 4>([&](auto k_index) {
-      static_for<0, 6>([&](auto n_index) { read_p0(a_here, b_there, k_index, n_index); });
+      static_for<0, 6>([&](auto n_index) { read_p0(S0, k_index, n_index); });
     });
-    b_there.flip();
     __builtin_amdgcn_sched_barrier(0);
-#ifdef W4_TRACE
-    __builtin_amdgcn_s_waitcnt(0xC07F);
-    W4_STAMP(3);
-#endif
 
-    // One K step per turn: the same code for every step, so the accumulators stay where they are.
-    // `next`: another step follows; `loads`: two more follow (the loads of the second start here).
-    // The fragment reads "of the next step" also run in the last step, on stale data nobody uses.
-  #pragma unroll 1
-    for (int j = 0; j < steps; ++j) {
-      const bool next = j + 1 < steps, loads = j + 2 < steps;
+    // One K step out of stage STAGE. `next`: another step follows; `loads`: two more follow (the
+    // loads of the second start here). The fragment reads "of the next step" also run in the last
+    // step, on stale data nobody uses. The K loop holds one copy of this per stage and nothing
+    // else, so the accumulators stay where they are.
+    auto step = [&](auto stage_index, bool next, bool loads) {
+      constexpr int STAGE = decltype(stage_index)::value;
+      const std::integral_constant<int, STAGE> HERE{};
+      const std::integral_constant<int, STAGE ^ 1> THERE{};
       // Half 0.
       static_for<0, 32>([&](auto n_index) {
         constexpr int n = decltype(n_index)::value, k = n / 8, t = (n % 8) / 4, u = n % 4;
@@ -273,9 +267,9 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
           publish(next ? 16 : 0);
         } else {
           if constexpr (n >= 8 && n % 2 == 0) {
-            if (loads) issue_p0(lds_here, std::integral_constant<int, (n - 8) / 2>{});
+            if (loads) issue_p0(HERE, std::integral_constant<int, (n - 8) / 2>{});
           }
-          if constexpr (n >= 9 && n < 24 && n % 2 == 1) read_p1(std::integral_constant<int, (n - 9) / 2>{});
+          if constexpr (n >= 9 && n < 24 && n % 2 == 1) read_p1(HERE, std::integral_constant<int, (n - 9) / 2>{});
           __builtin_amdgcn_sched_barrier(0);
         }
       });
@@ -287,56 +281,52 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
         constexpr int n = decltype(n_index)::value, k = n / 8, t = (n % 8) / 4, u = n % 4;
         product_of(acc[2 + t][u], fa1[t][k], fb[u][k]);
         if constexpr (n < 8 && n % 2 == 0) {
-          if (loads) issue_p1(lds_here, std::integral_constant<int, n / 2>{});
+          if (loads) issue_p1(HERE, std::integral_constant<int, n / 2>{});
         }
         // The next step's fragments of slab k - 1 go where this step's have just been used.
         if constexpr (n >= 8 && n % 8 < 6)
-          read_p0(a_there, b_there, std::integral_constant<int, n / 8 - 1>{}, std::integral_constant<int, n % 8>{});
+          read_p0(THERE, std::integral_constant<int, n / 8 - 1>{}, std::integral_constant<int, n % 8>{});
         __builtin_amdgcn_sched_barrier(0);
       });
       if (loads) la.base += la.step;
-      static_for<0, 6>([&](auto n_index) { read_p0(a_there, b_there, std::integral_constant<int, 3>{}, n_index); });
-      a_here.flip();
-      a_there.flip();
-      b_there.flip();
-      lds_here = lds_wave + ((j + 1) & 1) * W4_OPERAND;
+      static_for<0, 6>([&](auto n_index) { read_p0(THERE, std::integral_constant<int, 3>{}, n_index); });
       __builtin_amdgcn_sched_barrier(0);
+    };
+#pragma unroll 1
+    for (int j = 0; j < steps; j += 2) {  // the host keeps the step count even
+      step(S0, true, j + 2 < steps);
+      step(S1, j + 2 < steps, j + 3 < steps);
     }
   } else {
-    // `here`: the stage of the step being multiplied, `there`: the other one.
-    W4Frags<true> a_here, a_there, b_here, b_there;
-    a_here.init(frag_offset<true, W4_BM, W4_BK>(wm * 128, 0, lane));
-    b_here.init(W4_B0 + frag_offset<true, W4_BN, W4_BK>(wn * 128, 0, lane));
-    a_there = a_here;
-    b_there = b_here;
-    a_there.flip();
-    b_there.flip();
+    W4Frags<true> ra, rb;
+    ra.init(lds0 + frag_offset<true, W4_BM, W4_BK>(wm * 128, 0, lane));
+    rb.init(lds0 + W4_B0 + frag_offset<true, W4_BN, W4_BK>(wn * 128, 0, lane));
     // Part h of a stage: this wave's loads 4h .. 4h + 3 of A, then of B.
-    auto issue_part = [&](unsigned lds, auto h_index, auto n_index) {
-      constexpr int h = decltype(h_index)::value, n = decltype(n_index)::value;
+    auto issue_part = [&](auto stage_index, auto h_index, auto n_index) {
+      constexpr int stage = decltype(stage_index)::value, h = decltype(h_index)::value, n = decltype(n_index)::value;
       constexpr int i = 4 * h + n % 4;
-      if constexpr (n < 4) la.template issue<i, NW * i * 1024>(lds);
-      else lb.template issue<i, W4_B0 + NW * i * 1024>(lds);
+      if constexpr (n < 4) la.template issue<i, stage * W4_OPERAND + NW * i * 1024>(lds_wave);
+      else lb.template issue<i, W4_B0 + stage * W4_OPERAND + NW * i * 1024>(lds_wave);
     };
     // fa[h][t][s]: row block t, K slab 2h + s; fb[h][u][s] likewise.
     u32x4 fa[2][4][2], fb[2][4][2];
-    // Fragment n (0..15) of half h out of the stage `a` and `b` point at.
-    auto read_half = [&](auto h_index, const W4Frags<true>& a, const W4Frags<true>& b, auto n_index) {
-      constexpr int h = decltype(h_index)::value, n = decltype(n_index)::value;
-      constexpr int block = (n % 8) / 2, s = n % 2;
-      if constexpr (n < 8) fa[h][block][s] = a.template read<block, 2 * h + s>(smem);
-      else fb[h][block][s] = b.template read<block, 2 * h + s>(smem);
+    // Fragment n (0..15) of half h of a stage.
+    auto read_half = [&](auto stage_index, auto h_index, auto n_index) {
+      constexpr int stage = decltype(stage_index)::value, h = decltype(h_index)::value, n = decltype(n_index)::value;
+      constexpr int block = (n % 8) / 2, sl = n % 2;
+      if constexpr (n < 8) fa[h][block][sl] = ra.template read<block, 2 * h + sl, stage>();
+      else fb[h][block][sl] = rb.template read<block, 2 * h + sl, stage>();
     };
     const std::integral_constant<int, 0> H0{};
     const std::integral_constant<int, 1> H1{};
 
-    static_for<0, 8>([&](auto n_index) { issue_part(lds_wave, H0, n_index); });
-    static_for<0, 8>([&](auto n_index) { issue_part(lds_wave, H1, n_index); });
+    static_for<0, 8>([&](auto n_index) { issue_part(S0, H0, n_index); });
+    static_for<0, 8>([&](auto n_index) { issue_part(S0, H1, n_index); });
     la.base += la.step;
     lb.base += lb.step;
     if (steps > 1) {
-      static_for<0, 8>([&](auto n_index) { issue_part(lds_wave + W4_OPERAND, H0, n_index); });
-      static_for<0, 8>([&](auto n_index) { issue_part(lds_wave + W4_OPERAND, H1, n_index); });
+      static_for<0, 8>([&](auto n_index) { issue_part(S1, H0, n_index); });
+      static_for<0, 8>([&](auto n_index) { issue_part(S1, H1, n_index); });
       la.base += la.step;
       lb.base += lb.step;
     }
@@ -344,25 +334,26 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
     wait_loads(8 + (steps > 1 ? 16 : 0));
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
-    static_for<0, 16>([&](auto n_index) { read_half(H0, a_here, b_here, n_index); });
+    static_for<0, 16>([&](auto n_index) { read_half(S0, H0, n_index); });
     __builtin_amdgcn_sched_barrier(0);
 
-#pragma unroll 1
-    for (int j = 0; j < steps; ++j) {
-      const bool next = j + 1 < steps, loads = j + 2 < steps;
+    auto step = [&](auto stage_index, bool next, bool loads) {
+      constexpr int STAGE = decltype(stage_index)::value;
+      const std::integral_constant<int, STAGE> HERE{};
+      const std::integral_constant<int, STAGE ^ 1> THERE{};
       // Half 0.
       static_for<0, 32>([&](auto n_index) {
-        constexpr int n = decltype(n_index)::value, s = n / 16, t = (n % 16) / 4, u = n % 4;
-        product_of(acc[t][u], fa[0][t][s], fb[0][u][s]);
+        constexpr int n = decltype(n_index)::value, sl = n / 16, t = (n % 16) / 4, u = n % 4;
+        product_of(acc[t][u], fa[0][t][sl], fb[0][u][sl]);
         if constexpr (n == 7) {
           // B0. In flight behind part 1 of this step: both parts of the next.
           publish(next ? 16 : 0);
         } else {
           if constexpr (n >= 8 && n < 24) {
             if constexpr (n % 2 == 0) {
-              if (loads) issue_part(lds_here, H0, std::integral_constant<int, (n - 8) / 2>{});
+              if (loads) issue_part(HERE, H0, std::integral_constant<int, (n - 8) / 2>{});
             }
-            read_half(H1, a_here, b_here, std::integral_constant<int, n - 8>{});
+            read_half(HERE, H1, std::integral_constant<int, n - 8>{});
           }
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -371,13 +362,13 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
       publish(loads ? 16 : 8);
       // Half 1.
       static_for<0, 32>([&](auto n_index) {
-        constexpr int n = decltype(n_index)::value, s = n / 16, t = (n % 16) / 4, u = n % 4;
-        product_of(acc[t][u], fa[1][t][s], fb[1][u][s]);
+        constexpr int n = decltype(n_index)::value, sl = n / 16, t = (n % 16) / 4, u = n % 4;
+        product_of(acc[t][u], fa[1][t][sl], fb[1][u][sl]);
         if constexpr (n < 16) {
           if constexpr (n % 2 == 0) {
-            if (loads) issue_part(lds_here, H1, std::integral_constant<int, n / 2>{});
+            if (loads) issue_part(HERE, H1, std::integral_constant<int, n / 2>{});
           }
-          read_half(H0, a_there, b_there, n_index);
+          read_half(THERE, H0, n_index);
         }
         __builtin_amdgcn_sched_barrier(0);
       });
@@ -385,19 +376,18 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
         la.base += la.step;
         lb.base += lb.step;
       }
-      a_here.flip();
-      a_there.flip();
-      b_here.flip();
-      b_there.flip();
-      lds_here = lds_wave + ((j + 1) & 1) * W4_OPERAND;
       __builtin_amdgcn_sched_barrier(0);
+    };
+#pragma unroll 1
+    for (int j = 0; j < steps; j += 2) {  // the host keeps the step count even
+      step(S0, true, j + 2 < steps);
+      step(S1, j + 2 < steps, j + 3 < steps);
     }
   }
   // Every wave has read its last fragments before the stages are reused for the store pass.
   __builtin_amdgcn_s_waitcnt(vmcnt_only(0) & 0xC07F);
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_sched_barrier(0);
-  W4_STAMP(4);
 
   // Store pass: each wave stages 32 rows of its tile at a time through its own LDS region and
   // writes whole pieces of rows.
@@ -513,7 +503,6 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
       __builtin_amdgcn_wave_barrier();
     });
   }
-  W4_STAMP(5);
   if (bad) dev_raise_fault(g.fault, g.tag);
 }
 
