@@ -528,7 +528,7 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
     else if (mode == 3) dma_variant = 3;
     else if (mode == 4) dma_variant = 6;
     else if (mode == 9) dma_variant = 9;
-    if (dma_variant == 9 && !omx_gemm_w4_eligible(g, a_km, b_km)) dma_variant = 3;
+    if (dma_variant == 9 && !omx_gemm_w4_eligible(g, a_km, b_km, !(epi && epi->mode != OMX_EPI_NONE))) dma_variant = 3;
   }
   // One 256 x 256 workgroup per compute unit: when the last round of tiles fills under 2/5 of the
   // chip (the head's weight gradient: 591 tiles on 256 units), the rows of the whole rounds go to

@@ -267,7 +267,7 @@ __device__ __forceinline__ bool gemm_store_block(const GemmArgs& g, int split, c
 // 128 x 128 (variant 6) workgroup tile. Needs K % 64 == 0, 16-byte aligned
 // operands, and row counts that are multiples of 8 for k-major operands.
 bool omx_gemm_dma_eligible(const GemmArgs& g, bool a_km, bool b_km);
-bool omx_gemm_w4_eligible(const GemmArgs& g, bool a_km, bool b_km);
+bool omx_gemm_w4_eligible(const GemmArgs& g, bool a_km, bool b_km, bool plain);
 void omx_gemm_dma_tile(int variant, int* bm, int* bn);
 int32_t omx_gemm_dma_launch(omx_ctx* ctx, const GemmArgs& g, bool a_km, bool b_km, int variant);
 

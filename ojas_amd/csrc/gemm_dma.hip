@@ -44,9 +44,10 @@ bool omx_gemm_dma_eligible(const GemmArgs& g, bool a_km, bool b_km) {
 }
 
 // The one-wave-per-SIMD kernel (variant 9) also needs a k-major B with a k-major A, leading
-// dimensions whose 256-row lane offsets fit in 32 bits, and an even number of 64-column K steps.
-bool omx_gemm_w4_eligible(const GemmArgs& g, bool a_km, bool b_km) {
-  return (!a_km || b_km) && g.lda < (1l << 22) && g.ldb < (1l << 22) && g.K % 128 == 0;
+// dimensions whose 256-row lane offsets fit in 32 bits, an even number of 64-column K steps, and a
+// store pass without an activation.
+bool omx_gemm_w4_eligible(const GemmArgs& g, bool a_km, bool b_km, bool plain) {
+  return plain && (!a_km || b_km) && g.lda < (1l << 22) && g.ldb < (1l << 22) && g.K % 128 == 0;
 }
 
 void omx_gemm_dma_tile(int variant, int* bm, int* bn) {

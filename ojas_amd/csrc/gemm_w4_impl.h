@@ -104,7 +104,7 @@ struct W4Frags {
   }
 };
 
-template <bool A_KM, bool B_KM, int EPI>
+template <bool A_KM, bool B_KM>
 __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
   static_assert(!A_KM || B_KM, "a k-major A goes with a k-major B");
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -181,16 +181,11 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
   };
-  // The plain kernel multiplies with the operands exchanged: a lane then holds, for ONE output row
-  // (block row l32), four consecutive columns per register quad (8 (v / 4) + 4 lg + v % 4), which
-  // the store pass packs and stages 8 or 16 bytes at a time. With an activation in the store pass
-  // a lane holds one column and 16 rows, the layout gemm_epilogue_block's staging expects.
-  constexpr bool ROW_LANES = EPI == OMX_EPI_NONE;
+  // The products are taken with the operands exchanged: a lane then holds, for ONE output row (block
+  // row l32), four consecutive columns per register quad (8 (v / 4) + 4 lg + v % 4), which the
+  // store pass packs and stages 8 or 16 bytes at a time.
   auto product_of = [&](floatx16& c, const u32x4& a, const u32x4& b) {
-    if constexpr (ROW_LANES)
-      c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, b), __builtin_bit_cast(bf16x8, a), c, 0, 0, 0);
-    else
-      c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, b), __builtin_bit_cast(bf16x8, a), c, 0, 0, 0);
   };
   const unsigned lds0 = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(reinterpret_cast<uintptr_t>(smem)));
   const std::integral_constant<int, 0> S0{};
@@ -397,121 +392,78 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
   bool bad = false;
   constexpr int PPR = TN * 8;  // 4-column pieces per row
   const int gcol0 = n0 + wn * TN * 32;
-  if constexpr (ROW_LANES) {
-    const bool packed = g.splits == 1 && g.c_bf16 && g.c_vec != 0 && (g.ldc & 7) == 0 &&
-                        (reinterpret_cast<uintptr_t>(g.c) & 15) == 0;
-    constexpr int HP = TN * 32 * 2 + 16;  // bytes per staged bf16 row
-    char* hs = reinterpret_cast<char*>(cs);
-    unsigned flags = 0;  // bit 15 or 31 set: a stored bf16 has an all-ones exponent
-    static_for<0, TM>([&](auto tm_index) {
-      constexpr int tm = decltype(tm_index)::value;
-      const int grow0 = m0 + (wm * TM + tm) * 32;
-      const bool interior = grow0 + 32 <= g.M && gcol0 + TN * 32 <= g.N;
-      if (packed && interior) {
-        // bf16: rounded in registers, staged 8 bytes at a time, stored 16 bytes per lane (a wave
-        // instruction writes four rows of 256 bytes).
-#pragma unroll
-        for (int tn = 0; tn < TN; ++tn)
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const floatx16& c = acc[tm][tn];
-            uint2 w;
-            w.x = dev_pack_bf16_pair(c[4 * q], c[4 * q + 1]);
-            w.y = dev_pack_bf16_pair(c[4 * q + 2], c[4 * q + 3]);
-            flags |= ((w.x & 0x7F807F80u) + 0x00800080u) | ((w.y & 0x7F807F80u) + 0x00800080u);
-            *reinterpret_cast<uint2*>(hs + l32 * HP + (tn * 32 + 8 * q + 4 * lg) * 2) = w;
-          }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        unsigned short* crow = static_cast<unsigned short*>(g.c) + static_cast<long>(grow0 + (lane >> 4)) * g.ldc + gcol0 +
-                               (lane & 15) * 8;
-        const long four_rows = 4 * g.ldc;
-#pragma unroll
-        for (int it = 0; it < 8; ++it) {
-          const uint4 v = *reinterpret_cast<const uint4*>(hs + (it * 4 + (lane >> 4)) * HP + (lane & 15) * 16);
-          *reinterpret_cast<uint4*>(crow + it * four_rows) = v;
-        }
-      } else {
-        // f32 results, split-K partials, ragged edges: staged as f32 rows.
-#pragma unroll
-        for (int tn = 0; tn < TN; ++tn)
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const floatx16& c = acc[tm][tn];
-            *reinterpret_cast<float4*>(cs + l32 * CPW + tn * 32 + 8 * q + 4 * lg) =
-                make_float4(c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]);
-          }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        if (interior && (g.splits > 1 ? (g.N & 3) == 0 : g.c_vec != 0)) {
-          if (g.splits > 1) bad |= gemm_store_block<0, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
-          else if (g.c_bf16) bad |= gemm_store_block<1, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
-          else if (!g.accumulate) bad |= gemm_store_block<2, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
-          else bad |= gemm_store_block<3, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
-        } else {
-#pragma unroll 1
-          for (int c = lane; c < 32 * PPR; c += 64) {
-            const int row = c / PPR, piece = c % PPR;
-            const int grow = grow0 + row, gcol = gcol0 + piece * 4;
-            if (grow < g.M && gcol < g.N) {
-              const float4 val = *reinterpret_cast<const float4*>(cs + row * CPW + piece * 4);
-              bad |= gemm_store4(g, split, grow, gcol, val.x, val.y, val.z, val.w);
-            }
-          }
-        }
-      }
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-    });
-    bad |= (flags & 0x80008000u) != 0;
-  } else {
-    static_for<0, TM>([&](auto tm_index) {
-      constexpr int tm = decltype(tm_index)::value;
+  const bool packed = g.splits == 1 && g.c_bf16 && g.c_vec != 0 && (g.ldc & 7) == 0 &&
+                      (reinterpret_cast<uintptr_t>(g.c) & 15) == 0;
+  constexpr int HP = TN * 32 * 2 + 16;  // bytes per staged bf16 row
+  char* hs = reinterpret_cast<char*>(cs);
+  unsigned flags = 0;  // bit 15 or 31 set: a stored bf16 has an all-ones exponent
+  static_for<0, TM>([&](auto tm_index) {
+    constexpr int tm = decltype(tm_index)::value;
+    const int grow0 = m0 + (wm * TM + tm) * 32;
+    const bool interior = grow0 + 32 <= g.M && gcol0 + TN * 32 <= g.N;
+    if (packed && interior) {
+      // bf16: rounded in registers, staged 8 bytes at a time, stored 16 bytes per lane (a wave
+      // instruction writes four rows of 256 bytes).
 #pragma unroll
       for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) cs[(8 * (v >> 2) + 4 * lg + (v & 3)) * CPW + tn * 32 + l32] = acc[tm][tn][v];
+        for (int q = 0; q < 4; ++q) {
+          const floatx16& c = acc[tm][tn];
+          uint2 w;
+          w.x = dev_pack_bf16_pair(c[4 * q], c[4 * q + 1]);
+          w.y = dev_pack_bf16_pair(c[4 * q + 2], c[4 * q + 3]);
+          flags |= ((w.x & 0x7F807F80u) + 0x00800080u) | ((w.y & 0x7F807F80u) + 0x00800080u);
+          *reinterpret_cast<uint2*>(hs + l32 * HP + (tn * 32 + 8 * q + 4 * lg) * 2) = w;
+        }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
-      const int grow0 = m0 + (wm * TM + tm) * 32;
-      const bool interior = grow0 + 32 <= g.M && gcol0 + TN * 32 <= g.N;
-      bool stored = false;
-      if constexpr (EPI == OMX_EPI_AXPBY) {
-        if (interior && g.c_vec != 0) {
-          bad |= gemm_epilogue_block<OMX_EPI_AXPBY, false, PPR>(g, cs, CPW, grow0, gcol0, lane);
-          stored = true;
-        }
-      } else {
-        if (interior && g.c_vec != 0) {
-          bad |= g.epi_tanh ? gemm_epilogue_block<EPI, true, PPR>(g, cs, CPW, grow0, gcol0, lane)
-                            : gemm_epilogue_block<EPI, false, PPR>(g, cs, CPW, grow0, gcol0, lane);
-          stored = true;
-        }
+      unsigned short* crow = static_cast<unsigned short*>(g.c) + static_cast<long>(grow0 + (lane >> 4)) * g.ldc + gcol0 +
+                             (lane & 15) * 8;
+      const long four_rows = 4 * g.ldc;
+#pragma unroll
+      for (int it = 0; it < 8; ++it) {
+        const uint4 v = *reinterpret_cast<const uint4*>(hs + (it * 4 + (lane >> 4)) * HP + (lane & 15) * 16);
+        *reinterpret_cast<uint4*>(crow + it * four_rows) = v;
       }
-      if (!stored) {
+    } else {
+      // f32 results, split-K partials, ragged edges: staged as f32 rows.
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const floatx16& c = acc[tm][tn];
+          *reinterpret_cast<float4*>(cs + l32 * CPW + tn * 32 + 8 * q + 4 * lg) =
+              make_float4(c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]);
+        }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      if (interior && (g.splits > 1 ? (g.N & 3) == 0 : g.c_vec != 0)) {
+        if (g.splits > 1) bad |= gemm_store_block<0, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
+        else if (g.c_bf16) bad |= gemm_store_block<1, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
+        else if (!g.accumulate) bad |= gemm_store_block<2, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
+        else bad |= gemm_store_block<3, PPR>(g, split, cs, CPW, grow0, gcol0, lane);
+      } else {
 #pragma unroll 1
         for (int c = lane; c < 32 * PPR; c += 64) {
           const int row = c / PPR, piece = c % PPR;
           const int grow = grow0 + row, gcol = gcol0 + piece * 4;
           if (grow < g.M && gcol < g.N) {
             const float4 val = *reinterpret_cast<const float4*>(cs + row * CPW + piece * 4);
-            bad |= gemm_store4_epi(g, split, grow, gcol, val.x, val.y, val.z, val.w);
+            bad |= gemm_store4(g, split, grow, gcol, val.x, val.y, val.z, val.w);
           }
         }
       }
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-    });
-  }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  });
+  bad |= (flags & 0x80008000u) != 0;
   if (bad) dev_raise_fault(g.fault, g.tag);
 }
 
 template <bool A_KM, bool B_KM>
 int32_t launch_w4(omx_ctx* ctx, const GemmArgs& g) {
-  auto kernel = g.epi == OMX_EPI_GELU_FWD   ? &gemm_w4_kernel<A_KM, B_KM, OMX_EPI_GELU_FWD>
-                : g.epi == OMX_EPI_GELU_BWD ? &gemm_w4_kernel<A_KM, B_KM, OMX_EPI_GELU_BWD>
-                : g.epi == OMX_EPI_AXPBY    ? &gemm_w4_kernel<A_KM, B_KM, OMX_EPI_AXPBY>
-                                            : &gemm_w4_kernel<A_KM, B_KM, OMX_EPI_NONE>;
+  auto kernel = &gemm_w4_kernel<A_KM, B_KM>;
   OMX_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    W4_SMEM));
   omx_launch_timed(ctx, kernel, dim3(g.tiles_m * g.tiles_n * g.splits, g.batches), dim3(256), W4_SMEM, ctx->timing_start,
