@@ -40,8 +40,9 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor figure
 # dispatch, scaled by what the same counters read for the AdamW pass, whose traffic is known
 # (profiles/gemm_hbm_traffic_all_workloads.txt holds the runs and the tables for each workload).
 # The algorithmic figure of the gpt124m step (every operand read once, every output written once)
-# is 2.258e8 per op.
-GEMM_HBM_BYTES_PER_LAUNCH = {"gpt124m": 3.80e8, "gpt124m-muon": 3.02e8, "lora1b": 4.01e8, "nanolab124m": 2.77e8}
+# is 2.326e10 bytes per step: 2.258e8 per product, 2.005e8 per launch (its 103 products run as 116
+# launches: the 12 q|k|v forward products and the head's weight gradient are cut by rows into two each).
+GEMM_HBM_BYTES_PER_LAUNCH = {"gpt124m": 3.17e8, "gpt124m-muon": 2.64e8, "lora1b": 4.02e8, "nanolab124m": 2.65e8}
 
 
 # Kernel classes of omx_profile_kernels beyond the GEMM products: (bit, key, kernels, roofline).
@@ -568,7 +569,7 @@ def nanolab_step(args) -> int:
         "step_tflops": flops / (ms_per_step * 1e-3) / 1e12,
         "pct_bf16_mfma_peak": 100.0 * flops / (ms_per_step * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS,
         "loss_first": losses[0], "loss_last": losses[-1],
-        "roofline": {"bound": "mfma", "kernel": "gemm_dma_kernel / gemm_kernel (bf16 MFMA GEMM, all operand layouts)",
+        "roofline": {"bound": "mfma", "kernel": "gemm_w4_kernel / gemm_dma_kernel / gemm_kernel (bf16 MFMA GEMM, all operand layouts)",
                      "achieved": achieved, "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / BF16_MFMA_PEAK_TFLOPS, "traffic": GEMM_HBM_BYTES_PER_LAUNCH["nanolab124m"],
                      "launches": int(launches.value),
@@ -689,7 +690,7 @@ def main() -> int:
         "pct_bf16_mfma_peak": 100.0 * flops / (ms_per_step * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS if cfg.bf16 else None,
         "loss_first": losses[0], "loss_last": losses[-1],
         "roofline": {"bound": "mfma",
-                     "kernel": "gemm_dma_kernel / gemm_kernel (bf16 MFMA GEMM, all operand layouts)" if cfg.bf16
+                     "kernel": "gemm_w4_kernel / gemm_dma_kernel / gemm_kernel (bf16 MFMA GEMM, all operand layouts)" if cfg.bf16
                                else "gemm_kernel<float> (f32 MFMA GEMM, all operand layouts)",
                      "achieved": achieved, "peak": gemm_peak, "unit": "TFLOP/s", "frac": achieved / gemm_peak,
                      "traffic": GEMM_HBM_BYTES_PER_LAUNCH.get(
