@@ -585,6 +585,65 @@ def nanolab_step(args) -> int:
     return 0
 
 
+def gemm(args) -> int:
+    """Secondary workload: one bf16 product through `omx_gemm`, `--gemm-shape M,K,N` in layout
+    `--gemm-layout` (NN: A [M,K] and B^T [N,K] both k-contiguous, a forward product; NT: B [K,N], an
+    input gradient; TT: A^T [K,M] too, a weight gradient), bf16 output (f32 for TT), the tiling
+    chosen by the library unless `--gemm-tiling` forces one. `value` is 2 M N K over the median of
+    five timed runs of `--steps` launches."""
+    import ctypes as C
+
+    from ojas_amd.backend import BF16, F32, MiBackend
+
+    m, k, n = (int(v) for v in args.gemm_shape.split(","))
+    layout = args.gemm_layout
+    be = MiBackend(0)
+    lib = be._lib
+    a = be.empty((m * k,), BF16)
+    b = be.empty((k * n,), BF16)
+    for t, seed in ((a, 1), (b, 2)):
+        be._check(lib.omx_init_normal(be._ctx, be._p(t), C.c_int32(BF16), C.c_uint64(t.numel), C.c_uint64(seed),
+                                      C.c_float(0.05)))
+    out_dtype = F32 if layout == "TT" else BF16
+    c = be.empty((m, n), out_dtype)
+    a_strides = (1, m) if layout == "TT" else (k, 1)
+    b_strides = (1, k) if layout == "NN" else (n, 1)
+    be.set_option("gemm_dma", args.gemm_tiling)
+
+    def launch():
+        be._check(lib.omx_gemm(be._ctx, be._p(a), C.c_uint64(a_strides[0]), C.c_uint64(a_strides[1]), be._p(b),
+                               C.c_uint64(b_strides[0]), C.c_uint64(b_strides[1]), C.c_int32(BF16), be._p(c),
+                               C.c_int32(out_dtype), C.c_uint64(m), C.c_uint64(k), C.c_uint64(n), C.c_int32(0)))
+
+    runs = []
+    for _ in range(5):
+        for _ in range(args.warmup):
+            launch()
+        be.sync()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            launch()
+        be.sync()
+        runs.append((time.perf_counter() - t0) / args.steps)
+    runs.sort()
+    flops = 2.0 * m * n * k
+    nbytes = 2.0 * (m * k + k * n) + (4.0 if out_dtype == F32 else 2.0) * m * n
+    line = {
+        "metric": f"bf16 GEMM {layout} {m}x{k}x{n}: TFLOP/s", "value": flops / runs[2] / 1e12, "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": runs[2] * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"omx_gemm {layout}: A [{m},{k}], B [{k},{n}] bf16, tiling option {args.gemm_tiling}"},
+        "roofline": {"bound": "mfma", "kernel": "gemm_w4_kernel / gemm_dma_kernel / gemm_kernel",
+                     "achieved": flops / runs[2] / 1e12, "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": flops / runs[2] / 1e12 / BF16_MFMA_PEAK_TFLOPS, "traffic": None,
+                     "algorithmic_bytes_per_launch": nbytes},
+        "us": runs[2] * 1e6, "us_min": runs[0] * 1e6,
+    }
+    be.close()
+    print(json.dumps(line))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -596,9 +655,13 @@ def main() -> int:
                     help="adamw: BASELINE configs[2], the headline (default); muon: configs[3], Muon-NS5 (bf16 "
                          "iteration, lr 0.02, momentum 0.95) on the hidden matrices and AdamW on tables and norms")
     ap.add_argument("--attention-batch", type=int, default=16, help="batch of --workload attention")
-    ap.add_argument("--workload", default="train_step", choices=["train_step", "kv_decode", "attention"],
+    ap.add_argument("--gemm-shape", default="8192,8192,8192", help="M,K,N of --workload gemm")
+    ap.add_argument("--gemm-layout", default="NN", choices=["NN", "NT", "TT"], help="operand layout of --workload gemm")
+    ap.add_argument("--gemm-tiling", type=int, default=1, choices=[0, 1, 3, 4, 9],
+                    help="the library's gemm_dma option for --workload gemm (1: chosen by shape)")
+    ap.add_argument("--workload", default="train_step", choices=["train_step", "kv_decode", "attention", "gemm"],
                     help="train_step: the headline metric (default); kv_decode: the decode attention op alone; "
-                         "attention: the step's causal attention alone, forward + backward")
+                         "attention: the step's causal attention alone, forward + backward; gemm: one bf16 product")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).", file=sys.stderr)
@@ -607,6 +670,8 @@ def main() -> int:
         return kv_decode(args)
     if args.workload == "attention":
         return attention(args)
+    if args.workload == "gemm":
+        return gemm(args)
     if args.config == "lora1b":
         return lora_step(args)
     if args.config == "nanolab124m":
