@@ -657,7 +657,7 @@ def main() -> int:
     ap.add_argument("--attention-batch", type=int, default=16, help="batch of --workload attention")
     ap.add_argument("--gemm-shape", default="8192,8192,8192", help="M,K,N of --workload gemm")
     ap.add_argument("--gemm-layout", default="NN", choices=["NN", "NT", "TT"], help="operand layout of --workload gemm")
-    ap.add_argument("--gemm-tiling", type=int, default=1, choices=[0, 1, 3, 4, 9],
+    ap.add_argument("--gemm-tiling", type=int, default=1, choices=[0, 1, 3, 4, 9, 10],
                     help="the library's gemm_dma option for --workload gemm (1: chosen by shape)")
     ap.add_argument("--workload", default="train_step", choices=["train_step", "kv_decode", "attention", "gemm"],
                     help="train_step: the headline metric (default); kv_decode: the decode attention op alone; "

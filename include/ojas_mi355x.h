@@ -625,9 +625,9 @@ int32_t omx_read_scalar_f32(omx_ctx* ctx, const void* src, float* out);
 
 /* Tuning knobs (no counterpart in the reference). "gemm_dma": 0 = register-staged 128x128 GEMM
  * kernel only, 1 = choose a tiling by the output's tiles per compute unit and the K steps per
- * tile (default), 3 / 4 / 9 = force the 256x128 (32-column steps) / 128x128 four-wave / 256x256
- * one-wave-per-SIMD direct-to-LDS kernel wherever the operands are eligible (tests and
- * measurements). "flash_schedule": 0 = the bf16 attention kernels choose
+ * tile (default), 3 / 4 / 9 / 10 = force the 256x128 (32-column steps) / 128x128 four-wave /
+ * 256x256 / 256x192 one-wave-per-SIMD direct-to-LDS kernel wherever the operands are eligible
+ * (tests and measurements). "flash_schedule": 0 = the bf16 attention kernels choose
  * between one 128-row block per workgroup and a mirrored pair by how the pairs fill the chip
  * (default), 1 / 2 = always one block / always the pair (the parity tests run both).
  * "gemm_thin": 0 = bf16 products with at most 64 output columns over 1024 rows or

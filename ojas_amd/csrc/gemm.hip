@@ -518,7 +518,19 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
         else dma_variant = 3;
       } else if (!a_km) {
         const long tiles256x128 = static_cast<long>((g.M + 255) / 256) * ((g.N + 127) / 128);
-        if (unbatched && plain && tiles256 * 4 >= cus * 3) dma_variant = 9;
+        if (unbatched && plain && tiles256 * 4 >= cus * 3) {
+          // 256 x 256 or 256 x 192 tiles, by rounds of tiles x what a tile costs: 4 or 3 units per K step
+          // and 18 outside the steps (first loads, store pass: about four and a half steps' worth).
+          // 768 output columns are 3 x 256 or 4 x 192: 16384 rows make 192 tiles (a round three
+          // quarters full) or 256 (a full one of tiles a quarter shorter).
+          dma_variant = 9;
+          if (g.N % 192 == 0) {
+            const long tiles192 = static_cast<long>((g.M + 255) / 256) * (g.N / 192);
+            const long cost256 = (tiles256 + cus - 1) / cus * (4 * ksteps64 + 18);
+            const long cost192 = (tiles192 + cus - 1) / cus * (3 * ksteps64 + 18);
+            if (cost192 < cost256) dma_variant = 10;
+          }
+        }
         else if (unbatched && plain && b_km && tiles256x128 < cus && ksteps64 >= 32) dma_variant = 6;
         else dma_variant = 3;
       } else {
@@ -528,7 +540,9 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
     else if (mode == 3) dma_variant = 3;
     else if (mode == 4) dma_variant = 6;
     else if (mode == 9) dma_variant = 9;
-    if (dma_variant == 9 && !omx_gemm_w4_eligible(g, a_km, b_km, !(epi && epi->mode != OMX_EPI_NONE))) dma_variant = 3;
+    else if (mode == 10) dma_variant = 10;
+    if (dma_variant == 10 && a_km) dma_variant = 9;  // 256 x 192 tiles for a k-contiguous A only
+    if (dma_variant >= 9 && !omx_gemm_w4_eligible(g, a_km, b_km, !(epi && epi->mode != OMX_EPI_NONE))) dma_variant = 3;
   }
   // One 256 x 256 workgroup per compute unit: when the last round of tiles fills under 2/5 of the
   // chip (the head's weight gradient: 591 tiles on 256 units), the rows of the whole rounds go to
@@ -576,7 +590,7 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
     // 108 tiles: two splits; of 2304 x 768, 324 tiles: two splits make three rounds of half the length).
     const long all_tiles = tiles * g.batches;
     const bool may_split =
-        !thin && (g.batches == 1 ? tiles < 256 : ((dma_variant < 0 && all_tiles < 512) || dma_variant == 9));
+        !thin && (g.batches == 1 ? tiles < 256 : ((dma_variant < 0 && all_tiles < 512) || dma_variant >= 9));
     if (may_split && ksteps >= 4 * min_steps && !(epi && epi->mode != OMX_EPI_NONE)) {
       splits = static_cast<int>(((g.batches == 1 ? 512 : 1024) + all_tiles - 1) / all_tiles);
       if (splits > ksteps / min_steps) splits = ksteps / min_steps;
@@ -585,7 +599,7 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
         int p2 = 1;
         while (p2 * 2 <= splits + splits / 4) p2 *= 2;  // 7..9 -> 8, 10..12 -> 8, 13..16 -> 16
         splits = p2;
-        if (dma_variant == 9) {
+        if (dma_variant >= 9) {
           // One workgroup per compute unit: what counts is how full the last round of workgroups is
           // (192 tiles split in two are 384 workgroups on 256 units, a round and a half; split in
           // four they are three full rounds of half the length). A split's partial sums cost 8 bytes
@@ -607,7 +621,7 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
       }
     }
     g.ksteps_per_split = (ksteps + splits - 1) / splits;
-    if (dma_variant == 9) g.ksteps_per_split += g.ksteps_per_split & 1;  // its K loop takes steps in pairs
+    if (dma_variant >= 9) g.ksteps_per_split += g.ksteps_per_split & 1;  // its K loop takes steps in pairs
     g.splits = (ksteps + g.ksteps_per_split - 1) / g.ksteps_per_split;
     g.partial = nullptr;
     if (g.splits > 1) {
@@ -724,8 +738,8 @@ int32_t omx_set_option(omx_ctx* ctx, const char* name, int64_t value) {
     return OMX_OK;
   }
   if (name && strcmp(name, "gemm_dma") == 0) {
-    if (value != 0 && value != 1 && value != 3 && value != 4 && value != 9)
-      return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: gemm_dma takes 0, 1, 3, 4 or 9");
+    if (value != 0 && value != 1 && value != 3 && value != 4 && value != 9 && value != 10)
+      return omx_fail(ctx, OMX_OUT_OF_RANGE, "set_option: gemm_dma takes 0, 1, 3, 4, 9 or 10");
     ctx->gemm_dma_mode = static_cast<int>(value);
     return OMX_OK;
   }

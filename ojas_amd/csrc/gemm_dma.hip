@@ -52,7 +52,7 @@ bool omx_gemm_w4_eligible(const GemmArgs& g, bool a_km, bool b_km, bool plain) {
 
 void omx_gemm_dma_tile(int variant, int* bm, int* bn) {
   *bm = variant == 6 ? 128 : 256;
-  *bn = variant == 9 ? 256 : 128;
+  *bn = variant == 9 ? 256 : variant == 10 ? 192 : 128;
 }
 
 

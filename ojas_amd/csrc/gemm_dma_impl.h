@@ -635,15 +635,19 @@ int32_t launch_dma(omx_ctx* ctx, const GemmArgs& g) {
   return OMX_OK;
 }
 
-// The tilings the dispatcher chooses among: 9: 256 x 256, one wave per SIMD, one workgroup per
-// compute unit (gemm_w4_impl.h); 3: 256 x 128 in 32-column steps (three stages, two workgroups per
+// The tilings the dispatcher chooses among: 9 and 10: 256 x 256 and 256 x 192, one wave per SIMD, one
+// workgroup per compute unit (gemm_w4_impl.h); 3: 256 x 128 in 32-column steps (three stages, two workgroups per
 // compute unit); 6: 128 x 128 with four waves (three per compute unit).
 template <bool A_KM, bool B_KM>
 int32_t launch_variant(omx_ctx* ctx, const GemmArgs& g, int variant) {
-  if (variant == 9) {
-    // (the caller has asked omx_gemm_w4_eligible: a k-major A comes with a k-major B)
-    if constexpr (!A_KM || B_KM) return launch_w4<A_KM, B_KM>(ctx, g);
-    else return omx_fail(ctx, OMX_SHAPE, "gemm: no one-wave-per-SIMD kernel for this operand layout");
+  if (variant == 9 || variant == 10) {
+    // (the caller has asked omx_gemm_w4_eligible: a k-major A comes with a k-major B and 256 x 256 tiles)
+    if constexpr (!A_KM) {
+      return variant == 10 ? launch_w4<A_KM, B_KM, 3>(ctx, g) : launch_w4<A_KM, B_KM, 4>(ctx, g);
+    } else if constexpr (B_KM) {
+      if (variant == 9) return launch_w4<A_KM, B_KM, 4>(ctx, g);
+    }
+    return omx_fail(ctx, OMX_SHAPE, "gemm: no one-wave-per-SIMD kernel for this operand layout");
   }
   if (variant == 6) return launch_dma<A_KM, B_KM, 2, 2, 2, 2, 32, 3>(ctx, g);
   return launch_dma<A_KM, B_KM, 4, 2, 2, 2, 32, 3>(ctx, g);

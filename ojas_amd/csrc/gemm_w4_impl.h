@@ -1,6 +1,8 @@
 // The bf16 GEMM with one wave per SIMD: a 256 x 256 output tile per workgroup, one workgroup per
 // compute unit, four waves of 128 x 128 each (16 accumulator blocks of 32 x 32: 256 of the wave's
-// 512 registers). A wave interleaves its own LDS reads and global -> LDS loads between its own
+// 512 registers); with TN = 3 the tile is 256 x 192 and a wave's part 128 x 96 (768 output columns
+// are four such tiles: 16384 rows then make 256 tiles, one per compute unit, where 256 x 256 tiles
+// make 192). A wave interleaves its own LDS reads and global -> LDS loads between its own
 // matrix products, in an order fixed in the source: per product a wave reads two thirds of the
 // fragment bytes that eight waves of 128 x 64 read, and no other wave on the SIMD takes issue
 // slots from the products.
@@ -28,16 +30,24 @@
 
 namespace {
 
-constexpr int W4_BM = 256, W4_BN = 256, W4_BK = 64;
+constexpr int W4_BM = 256, W4_BK = 64;  // the tile is 256 rows by 64 TN columns (TN = 4, or 3: 192 columns)
 constexpr int W4_OPERAND = W4_BM * W4_BK * 2;  // one stage of one operand
 constexpr int W4_SMEM = 4 * W4_OPERAND;
 constexpr int W4_B0 = 2 * W4_OPERAND;  // LDS byte offset of B's first stage
 
 // Loads of one operand: a wave-uniform base address (the tile's first element at the current K
 // step) and a 32-bit byte offset per lane and load, so a K step advances one scalar.
-template <bool KM>
+// The chunk swizzle of a k-major tile row (kr) of ROWS columns: 16-byte chunks moved by multiples of 64 bytes so that
+// the four K rows a transposing read touches per clock fall into different banks (rows of 512 bytes all start in
+// bank 0: four shifts; rows of 384 bytes alternate between banks 0 and 32: one shift for every second pair).
+template <int ROWS>
+__device__ __forceinline__ int w4_km_swizzle(int kr) {
+  return ROWS == 256 ? (kr & 3) * 4 : ((kr >> 1) & 1) * 4;
+}
+
+template <bool KM, int ROWS>
 struct W4Loads {
-  static constexpr int N = 8;  // 32 loads of 1 KiB per step, four waves
+  static constexpr int N = ROWS / 32;  // ROWS / 8 loads of 1 KiB per step, four waves
   unsigned off[N];
   const char* base;
   long step;
@@ -53,9 +63,10 @@ struct W4Loads {
         gr = gr < rows ? gr : rows - 1;
         off[i] = static_cast<unsigned>(gr - row0) * static_cast<unsigned>(ld * 2) + kc * 16;
       } else {
+        constexpr int CPR = ROWS / 8;  // 16-byte chunks per K row
         const int idx = q * 64 + lane;
-        const int kr = idx >> 5, slot = idx & 31;
-        const int mc = slot ^ ((kr & 3) * 4);
+        const int kr = idx / CPR, slot = idx % CPR;
+        const int mc = slot ^ w4_km_swizzle<ROWS>(kr);
         int gm = mc * 8;
         gm = row0 + gm + 8 <= rows ? gm : 0;
         off[i] = static_cast<unsigned>(kr) * static_cast<unsigned>(ld * 2) + gm * 2;
@@ -74,15 +85,27 @@ struct W4Loads {
   }
 };
 
-// Fragment addresses of one operand: four registers holding LDS byte addresses in stage 0; the
-// block, the K slab and the stage are immediates of the read.
-template <bool KM>
+// Fragment addresses of one operand tile of ROWS rows: four registers holding LDS byte addresses in stage 0; the
+// block, the K slab and the stage are immediates of the read. `tile` is the tile's LDS address, `row_base` the first
+// of the wave's rows in it.
+template <bool KM, int ROWS>
 struct W4Frags {
   unsigned b[4];
-  __device__ __forceinline__ void init(unsigned first) {
+  __device__ __forceinline__ void init(unsigned tile, int row_base, int lane) {
 #pragma unroll
     for (int x = 0; x < 4; ++x) {
-      b[x] = KM ? first ^ (x << 6) : first ^ (x << 5);
+      if constexpr (!KM) {
+        // [row][8 chunks of 16 bytes], chunk c of row r in slot c ^ ((r >> 1) & 7); x is the K slab.
+        const int r = row_base + (lane & 31);
+        const int kc = x * 2 + (lane >> 5);
+        b[x] = tile + r * (W4_BK * 2) + ((kc ^ ((r >> 1) & 7)) << 4);
+      } else {
+        // [K row][ROWS / 8 chunks]; x is the 32-column block; the first of the two transposing reads.
+        const int s16 = lane & 15, half = (lane >> 4) & 1, g = lane >> 5;
+        const int kr = g * 8 + (s16 >> 2);
+        const int col = row_base + x * 32 + half * 16 + (s16 & 3) * 4;
+        b[x] = tile + kr * (ROWS * 2) + (((col >> 3) ^ w4_km_swizzle<ROWS>(kr)) << 4) + (col & 7) * 2;
+      }
       // Held as it is: re-derived from its parts, a read would pay an addition for what the
       // instruction's offset field carries for nothing.
       asm volatile("" : "+v"(b[x]));
@@ -95,20 +118,21 @@ struct W4Frags {
       return *reinterpret_cast<lds_ptr>(static_cast<uintptr_t>(b[KK] + (T * 32 * W4_BK * 2 + STAGE * W4_OPERAND)));
     } else {
       typedef short4v __attribute__((address_space(3))) * lds_ptr;
-      const unsigned p = b[T] + (KK * 16 * 256 * 2 + STAGE * W4_OPERAND);
+      const unsigned p = b[T] + (KK * 16 * ROWS * 2 + STAGE * W4_OPERAND);
       short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<lds_ptr>(static_cast<uintptr_t>(p)));
-      short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<lds_ptr>(static_cast<uintptr_t>(p + 4 * 256 * 2)));
+      short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<lds_ptr>(static_cast<uintptr_t>(p + 4 * ROWS * 2)));
       u32x2 x = __builtin_bit_cast(u32x2, lo), y = __builtin_bit_cast(u32x2, hi);
       return u32x4{x.x, x.y, y.x, y.y};
     }
   }
 };
 
-template <bool A_KM, bool B_KM>
+template <bool A_KM, bool B_KM, int TN>
 __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
   static_assert(!A_KM || B_KM, "a k-major A goes with a k-major B");
+  static_assert(TN == 4 || (TN == 3 && !A_KM), "256 x 192 tiles for a k-contiguous A only");
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  constexpr int TM = 4, TN = 4, NW = 4;
+  constexpr int TM = 4, NW = 4, W4_BN = TN * 64;
   // Tile order: as gemm_dma_kernel.
   const int total = g.tiles_m * g.tiles_n;
   int split = 0, id = blockIdx.x, product = blockIdx.y;
@@ -141,7 +165,7 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave >> 1, wn = wave & 1;  // the wave's 128 rows and 32 TN columns of the tile
   const int l32 = lane & 31, lg = lane >> 5;
 
   floatx16 acc[TM][TN];
@@ -160,27 +184,25 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
   const int ks_begin = split * g.ksteps_per_split;
   const int ks_end = min(g.K / W4_BK, ks_begin + g.ksteps_per_split);
   const int steps = ks_end - ks_begin;
-  W4Loads<A_KM> la;
-  W4Loads<B_KM> lb;
+  W4Loads<A_KM, W4_BM> la;
+  W4Loads<B_KM, W4_BN> lb;
   la.init(A, g.lda, m0, g.M, ks_begin * W4_BK, wave, lane);
   lb.init(B, g.ldb, n0, g.N, ks_begin * W4_BK, wave, lane);
   const unsigned lds_wave =
       __builtin_amdgcn_readfirstlane(static_cast<unsigned>(reinterpret_cast<uintptr_t>(smem))) + wave * 1024;
-  constexpr int NO_WAIT = 64;
-  auto wait_loads = [&](int n) {
-    if (n >= NO_WAIT) return;
-    if (n >= 16) __builtin_amdgcn_s_waitcnt(vmcnt_only(16));
-    else if (n >= 8) __builtin_amdgcn_s_waitcnt(vmcnt_only(8));
-    else if (n >= 4) __builtin_amdgcn_s_waitcnt(vmcnt_only(4));
-    else __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+  // Waits until at most YES (if `which`) or NO of this wave's loads, the most recently issued, are in flight.
+  auto wait_loads = [&](bool which, auto yes_count, auto no_count) {
+    if (which) __builtin_amdgcn_s_waitcnt(vmcnt_only(decltype(yes_count)::value));
+    else __builtin_amdgcn_s_waitcnt(vmcnt_only(decltype(no_count)::value));
   };
-  auto publish = [&](int in_flight) {
+  auto publish = [&](bool which, auto yes_count, auto no_count) {
     __builtin_amdgcn_sched_barrier(0);
-    wait_loads(in_flight);
+    wait_loads(which, yes_count, no_count);
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt == 0: this wave's fragment reads have returned
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
   };
+
   // The products are taken with the operands exchanged: a lane then holds, for ONE output row (block
   // row l32), four consecutive columns per register quad (8 (v / 4) + 4 lg + v % 4), which the
   // store pass packs and stages 8 or 16 bytes at a time.
@@ -191,19 +213,25 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
   const std::integral_constant<int, 0> S0{};
   const std::integral_constant<int, 1> S1{};
   if constexpr (!A_KM) {
-    W4Frags<false> ra;
-    W4Frags<B_KM> rb;
-    ra.init(lds0 + frag_offset<false, W4_BM, W4_BK>(wm * 128, 0, lane));
-    rb.init(lds0 + W4_B0 + frag_offset<B_KM, W4_BN, W4_BK>(wn * 128, 0, lane));
+    W4Frags<false, W4_BM> ra;
+    W4Frags<B_KM, W4_BN> rb;
+    ra.init(lds0, wm * 128, lane);
+    rb.init(lds0 + W4_B0, wn * TN * 32, lane);
 
-    // Part 0 of a stage: all of B and A's loads 0, 1, 4, 5 (rows 0-63 and 128-191 of the tile);
-    // part 1: A's loads 2, 3, 6, 7. `n` counts the part's loads.
+    // Part 0 of a stage: all of B (2 TN loads per wave) and A's loads 0, 1, 4, 5 (rows 0-63 and 128-191 of the
+    // tile); part 1: A's loads 2, 3, 6, 7. `n` counts the part's loads.
+    constexpr int NB = 2 * TN, NP0 = NB + 4, NSTEP = NP0 + 4;
+    constexpr int SL = 2 * TN, HL = 4 * SL;  // products per K slab of a half, per half
+    typedef std::integral_constant<int, 0> C0;
+    typedef std::integral_constant<int, 4> C4;
+    typedef std::integral_constant<int, NSTEP> CSTEP;
+    typedef std::integral_constant<int, 4 + NP0> C4P0;
     auto issue_p0 = [&](auto stage_index, auto n_index) {
       constexpr int stage = decltype(stage_index)::value, n = decltype(n_index)::value;
-      if constexpr (n < 8) {
+      if constexpr (n < NB) {
         lb.template issue<n, W4_B0 + stage * W4_OPERAND + NW * n * 1024>(lds_wave);
       } else {
-        constexpr int i = n == 8 ? 0 : n == 9 ? 1 : n == 10 ? 4 : 5;
+        constexpr int i = n == NB ? 0 : n == NB + 1 ? 1 : n == NB + 2 ? 4 : 5;
         la.template issue<i, stage * W4_OPERAND + NW * i * 1024>(lds_wave);
       }
     };
@@ -213,12 +241,12 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
       la.template issue<i, stage * W4_OPERAND + NW * i * 1024>(lds_wave);
     };
     // fa0[t][k]: row blocks 0-1, fa1[t][k]: row blocks 2-3, fb[u][k]: column blocks, K slab k.
-    u32x4 fa0[2][4], fa1[2][4], fb[4][4];
-    // Fragment n (0..5) of K slab k of part 0 of a stage: four of B, two of A.
+    u32x4 fa0[2][4], fa1[2][4], fb[TN][4];
+    // Fragment n (0 .. TN + 1) of K slab k of part 0 of a stage: TN of B, two of A.
     auto read_p0 = [&](auto stage_index, auto k_index, auto n_index) {
       constexpr int stage = decltype(stage_index)::value, k = decltype(k_index)::value, n = decltype(n_index)::value;
-      if constexpr (n < 4) fb[n][k] = rb.template read<n, k, stage>();
-      else fa0[n - 4][k] = ra.template read<n - 4, k, stage>();
+      if constexpr (n < TN) fb[n][k] = rb.template read<n, k, stage>();
+      else fa0[n - TN][k] = ra.template read<n - TN, k, stage>();
     };
     // Fragment n (0..7) of part 1 of a stage: K slab n / 2, row block 2 + n % 2.
     auto read_p1 = [&](auto stage_index, auto n_index) {
@@ -226,22 +254,22 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
       fa1[n % 2][n / 2] = ra.template read<2 + n % 2, n / 2, stage>();
     };
     // Both stages' loads, part 0 of step 0 published, its fragments read.
-    static_for<0, 12>([&](auto n_index) { issue_p0(S0, n_index); });
+    static_for<0, NP0>([&](auto n_index) { issue_p0(S0, n_index); });
     static_for<0, 4>([&](auto n_index) { issue_p1(S0, n_index); });
     la.base += la.step;
     lb.base += lb.step;
     if (steps > 1) {
-      static_for<0, 12>([&](auto n_index) { issue_p0(S1, n_index); });
+      static_for<0, NP0>([&](auto n_index) { issue_p0(S1, n_index); });
       static_for<0, 4>([&](auto n_index) { issue_p1(S1, n_index); });
       la.base += la.step;
       lb.base += lb.step;
     }
     clear_acc();
-    wait_loads(4 + (steps > 1 ? 16 : 0));
+    wait_loads(steps > 1, std::integral_constant<int, 4 + NSTEP>{}, C4{});
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
     static_for<0, 4>([&](auto k_index) {
-      static_for<0, 6>([&](auto n_index) { read_p0(S0, k_index, n_index); });
+      static_for<0, TN + 2>([&](auto n_index) { read_p0(S0, k_index, n_index); });
     });
     __builtin_amdgcn_sched_barrier(0);
 
@@ -249,42 +277,47 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
     // loads of the second start here). The fragment reads "of the next step" also run in the last
     // step, on stale data nobody uses. The K loop holds one copy of this per stage and nothing
     // else, so the accumulators stay where they are.
+    // Part 0's load i goes out after product P0_AT(i) of half 0: spread over the products behind B0.
     auto step = [&](auto stage_index, bool next, bool loads) {
       constexpr int STAGE = decltype(stage_index)::value;
       const std::integral_constant<int, STAGE> HERE{};
       const std::integral_constant<int, STAGE ^ 1> THERE{};
       // Half 0.
-      static_for<0, 32>([&](auto n_index) {
-        constexpr int n = decltype(n_index)::value, k = n / 8, t = (n % 8) / 4, u = n % 4;
+      static_for<0, HL>([&](auto n_index) {
+        constexpr int n = decltype(n_index)::value, k = n / SL, t = (n % SL) / TN, u = n % TN;
         product_of(acc[t][u], fa0[t][k], fb[u][k]);
-        if constexpr (n == 7) {
+        if constexpr (n == SL - 1) {
           // B0. In flight behind part 1 of this step: both parts of the next.
-          publish(next ? 16 : 0);
+          publish(next, CSTEP{}, C0{});
         } else {
-          if constexpr (n >= 8 && n % 2 == 0) {
-            if (loads) issue_p0(HERE, std::integral_constant<int, (n - 8) / 2>{});
+          if constexpr (n >= SL) {
+            // load i after product SL + i (HL - SL) / NP0 (TN = 4: every second product)
+            constexpr int lo = ((n - SL) * NP0 + (HL - SL) - 1) / (HL - SL);  // first i with its place >= n
+            if constexpr (lo < NP0 && SL + lo * (HL - SL) / NP0 == n) {
+              if (loads) issue_p0(HERE, std::integral_constant<int, lo>{});
+            }
           }
-          if constexpr (n >= 9 && n < 24 && n % 2 == 1) read_p1(HERE, std::integral_constant<int, (n - 9) / 2>{});
+          if constexpr (n > SL && n < SL + 17 && (n - SL) % 2 == 1) read_p1(HERE, std::integral_constant<int, (n - SL - 1) / 2>{});
           __builtin_amdgcn_sched_barrier(0);
         }
       });
       if (loads) lb.base += lb.step;
       // B1. In flight behind part 0 of the next step: its part 1 and part 0 of the one after.
-      publish(loads ? 16 : 4);
+      publish(loads, C4P0{}, C4{});
       // Half 1.
-      static_for<0, 32>([&](auto n_index) {
-        constexpr int n = decltype(n_index)::value, k = n / 8, t = (n % 8) / 4, u = n % 4;
+      static_for<0, HL>([&](auto n_index) {
+        constexpr int n = decltype(n_index)::value, k = n / SL, t = (n % SL) / TN, u = n % TN;
         product_of(acc[2 + t][u], fa1[t][k], fb[u][k]);
         if constexpr (n < 8 && n % 2 == 0) {
           if (loads) issue_p1(HERE, std::integral_constant<int, n / 2>{});
         }
         // The next step's fragments of slab k - 1 go where this step's have just been used.
-        if constexpr (n >= 8 && n % 8 < 6)
-          read_p0(THERE, std::integral_constant<int, n / 8 - 1>{}, std::integral_constant<int, n % 8>{});
+        if constexpr (n >= SL && n % SL < TN + 2)
+          read_p0(THERE, std::integral_constant<int, n / SL - 1>{}, std::integral_constant<int, n % SL>{});
         __builtin_amdgcn_sched_barrier(0);
       });
       if (loads) la.base += la.step;
-      static_for<0, 6>([&](auto n_index) { read_p0(THERE, std::integral_constant<int, 3>{}, n_index); });
+      static_for<0, TN + 2>([&](auto n_index) { read_p0(THERE, std::integral_constant<int, 3>{}, n_index); });
       __builtin_amdgcn_sched_barrier(0);
     };
 #pragma unroll 1
@@ -293,9 +326,14 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
       step(S1, j + 2 < steps, j + 3 < steps);
     }
   } else {
-    W4Frags<true> ra, rb;
-    ra.init(lds0 + frag_offset<true, W4_BM, W4_BK>(wm * 128, 0, lane));
-    rb.init(lds0 + W4_B0 + frag_offset<true, W4_BN, W4_BK>(wn * 128, 0, lane));
+    W4Frags<true, W4_BM> ra;
+    W4Frags<true, W4_BN> rb;
+    ra.init(lds0, wm * 128, lane);
+    rb.init(lds0 + W4_B0, wn * 128, lane);
+    typedef std::integral_constant<int, 0> C0;
+    typedef std::integral_constant<int, 8> C8;
+    typedef std::integral_constant<int, 16> C16;
+    typedef std::integral_constant<int, 24> C24;
     // Part h of a stage: this wave's loads 4h .. 4h + 3 of A, then of B.
     auto issue_part = [&](auto stage_index, auto h_index, auto n_index) {
       constexpr int stage = decltype(stage_index)::value, h = decltype(h_index)::value, n = decltype(n_index)::value;
@@ -326,7 +364,7 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
       lb.base += lb.step;
     }
     clear_acc();
-    wait_loads(8 + (steps > 1 ? 16 : 0));
+    wait_loads(steps > 1, C24{}, C8{});
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
     static_for<0, 16>([&](auto n_index) { read_half(S0, H0, n_index); });
@@ -342,7 +380,7 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
         product_of(acc[t][u], fa[0][t][sl], fb[0][u][sl]);
         if constexpr (n == 7) {
           // B0. In flight behind part 1 of this step: both parts of the next.
-          publish(next ? 16 : 0);
+          publish(next, C16{}, C0{});
         } else {
           if constexpr (n >= 8 && n < 24) {
             if constexpr (n % 2 == 0) {
@@ -354,7 +392,7 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
         }
       });
       // B1. In flight behind part 0 of the next step: its part 1 and part 0 of the one after.
-      publish(loads ? 16 : 8);
+      publish(loads, C16{}, C8{});
       // Half 1.
       static_for<0, 32>([&](auto n_index) {
         constexpr int n = decltype(n_index)::value, sl = n / 16, t = (n % 16) / 4, u = n % 4;
@@ -403,7 +441,7 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
     const bool interior = grow0 + 32 <= g.M && gcol0 + TN * 32 <= g.N;
     if (packed && interior) {
       // bf16: rounded in registers, staged 8 bytes at a time, stored 16 bytes per lane (a wave
-      // instruction writes four rows of 256 bytes).
+      // instruction writes four rows of 64 TN bytes; with TN = 3 four lanes in 16 sit out).
 #pragma unroll
       for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
@@ -420,10 +458,12 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
       unsigned short* crow = static_cast<unsigned short*>(g.c) + static_cast<long>(grow0 + (lane >> 4)) * g.ldc + gcol0 +
                              (lane & 15) * 8;
       const long four_rows = 4 * g.ldc;
+      if ((lane & 15) < TN * 4) {
 #pragma unroll
-      for (int it = 0; it < 8; ++it) {
-        const uint4 v = *reinterpret_cast<const uint4*>(hs + (it * 4 + (lane >> 4)) * HP + (lane & 15) * 16);
-        *reinterpret_cast<uint4*>(crow + it * four_rows) = v;
+        for (int it = 0; it < 8; ++it) {
+          const uint4 v = *reinterpret_cast<const uint4*>(hs + (it * 4 + (lane >> 4)) * HP + (lane & 15) * 16);
+          *reinterpret_cast<uint4*>(crow + it * four_rows) = v;
+        }
       }
     } else {
       // f32 results, split-K partials, ragged edges: staged as f32 rows.
@@ -461,9 +501,9 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
   if (bad) dev_raise_fault(g.fault, g.tag);
 }
 
-template <bool A_KM, bool B_KM>
+template <bool A_KM, bool B_KM, int TN>
 int32_t launch_w4(omx_ctx* ctx, const GemmArgs& g) {
-  auto kernel = &gemm_w4_kernel<A_KM, B_KM>;
+  auto kernel = &gemm_w4_kernel<A_KM, B_KM, TN>;
   OMX_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    W4_SMEM));
   omx_launch_timed(ctx, kernel, dim3(g.tiles_m * g.tiles_n * g.splits, g.batches), dim3(256), W4_SMEM, ctx->timing_start,

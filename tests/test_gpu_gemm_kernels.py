@@ -28,7 +28,7 @@ SHAPES = [(256, 64, 256), (300, 128, 520), (64, 192, 96), (513, 256, 257), (1024
           (4160, 136, 264)]  # the last: a weight gradient over 4160 rows, split along K
 
 
-@pytest.mark.parametrize("mode", [0, 1, 3, 4, 9])
+@pytest.mark.parametrize("mode", [0, 1, 3, 4, 9, 10])
 @pytest.mark.parametrize("rows,kin,nout", SHAPES)
 def test_linear_bf16_under_each_kernel(be, mode, rows, kin, nout):
     from ojas_amd.backend import BF16, F32
@@ -104,7 +104,7 @@ def test_the_dispatcher_picks_a_tiling_within_a_tenth_of_the_best(be, layout, m,
         return best
 
     try:
-        forced = {mode: seconds(mode) for mode in (3, 4, 9)}
+        forced = {mode: seconds(mode) for mode in (3, 4, 9, 10)}
         chosen = seconds(1)
     finally:
         be.set_option("gemm_dma", 1)
@@ -209,7 +209,7 @@ def test_unknown_option_is_refused(be):
     assert be._lib.omx_set_option(be._ctx, b"gemm_dma", C.c_int64(5)) == 3
 
 
-@pytest.mark.parametrize("mode", [0, 1, 3, 4, 9])
+@pytest.mark.parametrize("mode", [0, 1, 3, 4, 9, 10])
 @pytest.mark.parametrize("layers", [3, 4])  # 4: a tile count divisible by 8, which takes the XCD-ordered mapping
 @pytest.mark.parametrize("rows,kin,nout", [(1088, 136, 264), (2048, 768, 256)])
 def test_strided_batch_of_weight_gradients(be, mode, rows, kin, nout, layers):
