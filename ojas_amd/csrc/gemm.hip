@@ -516,6 +516,21 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
         if (plain && ksteps64 >= 64 && all256 >= cus && (unbatched || all256 * 5 >= rounds256 * cus * 4)) dma_variant = 9;
         else if (plain && ksteps64 >= 128 && all256 * 8 >= cus) dma_variant = 9;  // with K split
         else dma_variant = 3;
+        // 256 x 192 tiles where their rounds cost less: rounds of tiles x (4 or 3 units per K step + 18 per
+        // tile), over the split counts the 256 x 256 tiling may take (a split pays 1000 / K of the product
+        // for its partial sums). 12 products of 2304 x 768 are 324 tiles of 256 x 256 (two splits: three
+        // rounds of half the length and a reduce pass) or 432 of 256 x 192 (two rounds, unsplit).
+        if (dma_variant == 9 && !unbatched && g.N % 192 == 0) {
+          const long all192 = static_cast<long>((g.M + 255) / 256) * (g.N / 192) * g.batches;
+          double cost256 = 1e30;
+          for (int s2 = 1; s2 <= 4 && ksteps64 / s2 >= 32; s2 *= 2) {
+            const double c = static_cast<double>((all256 * s2 + cus - 1) / cus) * (4.0 * ksteps64 / s2 + 18.0) *
+                             (s2 > 1 ? 1.0 + 1000.0 * s2 / static_cast<double>(g.K) : 1.0);
+            if (c < cost256) cost256 = c;
+          }
+          const double cost192 = static_cast<double>((all192 + cus - 1) / cus) * (3.0 * ksteps64 + 18.0);
+          if (cost192 < cost256) dma_variant = 10;
+        }
       } else if (!a_km) {
         const long tiles256x128 = static_cast<long>((g.M + 255) / 256) * ((g.N + 127) / 128);
         if (unbatched && plain && tiles256 * 4 >= cus * 3) {
@@ -541,7 +556,6 @@ int32_t omx_gemm_impl(omx_ctx* ctx, uint32_t fault_op, const void* a, uint64_t a
     else if (mode == 4) dma_variant = 6;
     else if (mode == 9) dma_variant = 9;
     else if (mode == 10) dma_variant = 10;
-    if (dma_variant == 10 && a_km) dma_variant = 9;  // 256 x 192 tiles for a k-contiguous A only
     if (dma_variant >= 9 && !omx_gemm_w4_eligible(g, a_km, b_km, !(epi && epi->mode != OMX_EPI_NONE))) dma_variant = 3;
   }
   // One 256 x 256 workgroup per compute unit: when the last round of tiles fills under 2/5 of the

@@ -642,10 +642,8 @@ template <bool A_KM, bool B_KM>
 int32_t launch_variant(omx_ctx* ctx, const GemmArgs& g, int variant) {
   if (variant == 9 || variant == 10) {
     // (the caller has asked omx_gemm_w4_eligible: a k-major A comes with a k-major B and 256 x 256 tiles)
-    if constexpr (!A_KM) {
+    if constexpr (!A_KM || B_KM) {
       return variant == 10 ? launch_w4<A_KM, B_KM, 3>(ctx, g) : launch_w4<A_KM, B_KM, 4>(ctx, g);
-    } else if constexpr (B_KM) {
-      if (variant == 9) return launch_w4<A_KM, B_KM, 4>(ctx, g);
     }
     return omx_fail(ctx, OMX_SHAPE, "gemm: no one-wave-per-SIMD kernel for this operand layout");
   }

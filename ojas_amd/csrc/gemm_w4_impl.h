@@ -130,7 +130,7 @@ struct W4Frags {
 template <bool A_KM, bool B_KM, int TN>
 __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
   static_assert(!A_KM || B_KM, "a k-major A goes with a k-major B");
-  static_assert(TN == 4 || (TN == 3 && !A_KM), "256 x 192 tiles for a k-contiguous A only");
+  static_assert(TN == 4 || TN == 3, "256 x 256 or 256 x 192 tiles");
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   constexpr int TM = 4, NW = 4, W4_BN = TN * 64;
   // Tile order: as gemm_dma_kernel.
@@ -329,45 +329,50 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
     W4Frags<true, W4_BM> ra;
     W4Frags<true, W4_BN> rb;
     ra.init(lds0, wm * 128, lane);
-    rb.init(lds0 + W4_B0, wn * 128, lane);
+    rb.init(lds0 + W4_B0, wn * TN * 32, lane);
+    // Part h of a stage: this wave's loads 4h .. 4h + 3 of A, then TN h .. TN h + TN - 1 of B.
+    constexpr int NPART = 4 + TN, NF = 2 * NPART;  // loads per part and wave; fragments per half
+    constexpr int SLAB = 4 * TN, HL = 2 * SLAB;   // products per K slab, per half
     typedef std::integral_constant<int, 0> C0;
-    typedef std::integral_constant<int, 8> C8;
-    typedef std::integral_constant<int, 16> C16;
-    typedef std::integral_constant<int, 24> C24;
-    // Part h of a stage: this wave's loads 4h .. 4h + 3 of A, then of B.
+    typedef std::integral_constant<int, NPART> C1P;
+    typedef std::integral_constant<int, 2 * NPART> C2P;
+    typedef std::integral_constant<int, 3 * NPART> C3P;
     auto issue_part = [&](auto stage_index, auto h_index, auto n_index) {
       constexpr int stage = decltype(stage_index)::value, h = decltype(h_index)::value, n = decltype(n_index)::value;
-      constexpr int i = 4 * h + n % 4;
-      if constexpr (n < 4) la.template issue<i, stage * W4_OPERAND + NW * i * 1024>(lds_wave);
-      else lb.template issue<i, W4_B0 + stage * W4_OPERAND + NW * i * 1024>(lds_wave);
+      if constexpr (n < 4) {
+        constexpr int i = 4 * h + n;
+        la.template issue<i, stage * W4_OPERAND + NW * i * 1024>(lds_wave);
+      } else {
+        constexpr int i = TN * h + (n - 4);
+        lb.template issue<i, W4_B0 + stage * W4_OPERAND + NW * i * 1024>(lds_wave);
+      }
     };
     // fa[h][t][s]: row block t, K slab 2h + s; fb[h][u][s] likewise.
-    u32x4 fa[2][4][2], fb[2][4][2];
-    // Fragment n (0..15) of half h of a stage.
+    u32x4 fa[2][4][2], fb[2][TN][2];
+    // Fragment n (0 .. NF - 1) of half h of a stage: eight of A, then 2 TN of B.
     auto read_half = [&](auto stage_index, auto h_index, auto n_index) {
       constexpr int stage = decltype(stage_index)::value, h = decltype(h_index)::value, n = decltype(n_index)::value;
-      constexpr int block = (n % 8) / 2, sl = n % 2;
-      if constexpr (n < 8) fa[h][block][sl] = ra.template read<block, 2 * h + sl, stage>();
-      else fb[h][block][sl] = rb.template read<block, 2 * h + sl, stage>();
+      if constexpr (n < 8) fa[h][n / 2][n % 2] = ra.template read<n / 2, 2 * h + n % 2, stage>();
+      else fb[h][(n - 8) / 2][n % 2] = rb.template read<(n - 8) / 2, 2 * h + n % 2, stage>();
     };
     const std::integral_constant<int, 0> H0{};
     const std::integral_constant<int, 1> H1{};
 
-    static_for<0, 8>([&](auto n_index) { issue_part(S0, H0, n_index); });
-    static_for<0, 8>([&](auto n_index) { issue_part(S0, H1, n_index); });
+    static_for<0, NPART>([&](auto n_index) { issue_part(S0, H0, n_index); });
+    static_for<0, NPART>([&](auto n_index) { issue_part(S0, H1, n_index); });
     la.base += la.step;
     lb.base += lb.step;
     if (steps > 1) {
-      static_for<0, 8>([&](auto n_index) { issue_part(S1, H0, n_index); });
-      static_for<0, 8>([&](auto n_index) { issue_part(S1, H1, n_index); });
+      static_for<0, NPART>([&](auto n_index) { issue_part(S1, H0, n_index); });
+      static_for<0, NPART>([&](auto n_index) { issue_part(S1, H1, n_index); });
       la.base += la.step;
       lb.base += lb.step;
     }
     clear_acc();
-    wait_loads(steps > 1, C24{}, C8{});
+    wait_loads(steps > 1, C3P{}, C1P{});
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
-    static_for<0, 16>([&](auto n_index) { read_half(S0, H0, n_index); });
+    static_for<0, NF>([&](auto n_index) { read_half(S0, H0, n_index); });
     __builtin_amdgcn_sched_barrier(0);
 
     auto step = [&](auto stage_index, bool next, bool loads) {
@@ -375,15 +380,15 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
       const std::integral_constant<int, STAGE> HERE{};
       const std::integral_constant<int, STAGE ^ 1> THERE{};
       // Half 0.
-      static_for<0, 32>([&](auto n_index) {
-        constexpr int n = decltype(n_index)::value, sl = n / 16, t = (n % 16) / 4, u = n % 4;
+      static_for<0, HL>([&](auto n_index) {
+        constexpr int n = decltype(n_index)::value, sl = n / SLAB, t = (n % SLAB) / TN, u = n % TN;
         product_of(acc[t][u], fa[0][t][sl], fb[0][u][sl]);
         if constexpr (n == 7) {
           // B0. In flight behind part 1 of this step: both parts of the next.
-          publish(next, C16{}, C0{});
+          publish(next, C2P{}, C0{});
         } else {
-          if constexpr (n >= 8 && n < 24) {
-            if constexpr (n % 2 == 0) {
+          if constexpr (n >= 8 && n < 8 + NF) {
+            if constexpr (n % 2 == 0 && (n - 8) / 2 < NPART) {
               if (loads) issue_part(HERE, H0, std::integral_constant<int, (n - 8) / 2>{});
             }
             read_half(HERE, H1, std::integral_constant<int, n - 8>{});
@@ -392,13 +397,13 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(GemmArgs g) {
         }
       });
       // B1. In flight behind part 0 of the next step: its part 1 and part 0 of the one after.
-      publish(loads, C16{}, C8{});
+      publish(loads, C2P{}, C1P{});
       // Half 1.
-      static_for<0, 32>([&](auto n_index) {
-        constexpr int n = decltype(n_index)::value, sl = n / 16, t = (n % 16) / 4, u = n % 4;
+      static_for<0, HL>([&](auto n_index) {
+        constexpr int n = decltype(n_index)::value, sl = n / SLAB, t = (n % SLAB) / TN, u = n % TN;
         product_of(acc[t][u], fa[1][t][sl], fb[1][u][sl]);
-        if constexpr (n < 16) {
-          if constexpr (n % 2 == 0) {
+        if constexpr (n < NF) {
+          if constexpr (n % 2 == 0 && n / 2 < NPART) {
             if (loads) issue_part(HERE, H1, std::integral_constant<int, n / 2>{});
           }
           read_half(THERE, H0, n_index);
