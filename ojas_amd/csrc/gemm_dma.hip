@@ -38,16 +38,16 @@ int32_t omx_gemm_dma_launch_tt(omx_ctx* ctx, const GemmArgs& g, int variant);
 
 bool omx_gemm_dma_eligible(const GemmArgs& g, bool a_km, bool b_km) {
   if (g.K % 64 != 0 || !g.a_vec || !g.b_vec) return false;
+  if (g.lda >= (1l << 22) || g.ldb >= (1l << 22)) return false;  // a tile's lane offsets are 32 bits of bytes
   if (a_km && g.M % 8 != 0) return false;
   if (b_km && g.N % 8 != 0) return false;
   return true;
 }
 
-// The one-wave-per-SIMD kernel (variant 9) also needs a k-major B with a k-major A, leading
-// dimensions whose 256-row lane offsets fit in 32 bits, an even number of 64-column K steps, and a
-// store pass without an activation.
+// The one-wave-per-SIMD kernel (variants 9 and 10) also needs a k-major B with a k-major A, an even
+// number of 64-column K steps, and a store pass without an activation.
 bool omx_gemm_w4_eligible(const GemmArgs& g, bool a_km, bool b_km, bool plain) {
-  return plain && (!a_km || b_km) && g.lda < (1l << 22) && g.ldb < (1l << 22) && g.K % 128 == 0;
+  return plain && (!a_km || b_km) && g.K % 128 == 0;
 }
 
 void omx_gemm_dma_tile(int variant, int* bm, int* bn) {

@@ -78,8 +78,10 @@ gemm_dma_kernel(GemmArgs g) {
   // Everything a K step needs is computed here, once per tile: the loads' global addresses and
   // the fragments' LDS offsets. Inside the loop the stage is a compile-time constant (the loop
   // body is unrolled over the stages), so a step is loads, LDS reads and MFMAs and little else.
-  TileLoads<A_KM, BM, DBK, NW> la;
-  TileLoads<B_KM, BN, DBK, NW> lb;
+  // (scalar base + lane offsets where every wave issues the same number of loads of each operand)
+  constexpr bool EVEN_LOADS = (BM * DBK * 2 / 1024) % NW == 0 && (BN * DBK * 2 / 1024) % NW == 0;
+  std::conditional_t<EVEN_LOADS, TileLoadsOff<A_KM, BM, DBK, NW>, TileLoads<A_KM, BM, DBK, NW>> la;
+  std::conditional_t<EVEN_LOADS, TileLoadsOff<B_KM, BN, DBK, NW>, TileLoads<B_KM, BN, DBK, NW>> lb;
   la.init(A, g.lda, m0, g.M, ks_begin * DBK, wave, lane);
   lb.init(B, g.ldb, n0, g.N, ks_begin * DBK, wave, lane);
   const unsigned lds0 = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(reinterpret_cast<uintptr_t>(smem)));
@@ -110,14 +112,18 @@ gemm_dma_kernel(GemmArgs g) {
   // The fragments of the next 16-column slab are read while the current slab is multiplied; the
   // first slab of the next step is read right after the barrier that publishes its stage, ahead
   // of the last slab's products, so neither the LDS latency nor the barrier drains the MFMA pipe.
-  u32x4 af[TM], bf[TN];
+  // Two sets of fragment registers that take turns (a step has an even number of slabs, so slab 0 of every step
+  // finds its fragments in set 0): no copies, and no wait for the next slab's fragments before this slab's
+  // products have been issued.
+  static_assert(KK % 2 == 0, "the fragment sets alternate by slab");
+  u32x4 af[2][TM], bf[2][TN];
   auto read_frags = [&](const char* stage, int kk, u32x4(&a)[TM], u32x4(&b)[TN]) {
 #pragma unroll
     for (int t = 0; t < TM; ++t) a[t] = frag_at<A_KM, BM>(stage + a_off[t][kk]);
 #pragma unroll
     for (int t = 0; t < TN; ++t) b[t] = frag_at<B_KM, BN>(stage + b_off[t][kk]);
   };
-  read_frags(smem, 0, af, bf);
+  read_frags(smem, 0, af[0], bf[0]);
   // One K step: the loads of step ks + NST - 1, then the slabs of stage `stage` (fragments one slab
   // ahead), the wait + barrier before the last slab's products, and the first slab of `next`.
   auto k_step = [&](int ks, unsigned fill_stage, const char* stage, const char* next) {
@@ -125,22 +131,17 @@ gemm_dma_kernel(GemmArgs g) {
       la.issue(lds0 + fill_stage * STAGE, wave);
       lb.issue(lds0 + fill_stage * STAGE + A_BYTES, wave);
     }
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-      u32x4 an[TM], bn[TN];
-#pragma unroll
-      for (int t = 0; t < TM; ++t) an[t] = af[t];
-#pragma unroll
-      for (int t = 0; t < TN; ++t) bn[t] = bf[t];
-      if (kk + 1 < KK) {
-        read_frags(stage, kk + 1, an, bn);
+    static_for<0, KK>([&](auto kk_index) {
+      constexpr int kk = decltype(kk_index)::value, cur = kk % 2, nxt = cur ^ 1;
+      if constexpr (kk + 1 < KK) {
+        read_frags(stage, kk + 1, af[nxt], bf[nxt]);
       } else {
         // Step ks + 1 must have landed (this wave's share, then everyone's); later steps may
         // still be in flight. Every wave has its last fragments of this stage in registers by
         // now, so the barrier also releases the stage for the loads of step ks + NST.
         wait_groups(min(NST - 2, ks_end - ks - 2));
         __syncthreads();
-        if (ks + 1 < ks_end) read_frags(next, 0, an, bn);
+        if (ks + 1 < ks_end) read_frags(next, 0, af[nxt], bf[nxt]);
       }
       // Keeps the reads above the products: the scheduler would otherwise sink them to their
       // first use to save registers, which puts the LDS latency back in front of every slab.
@@ -149,15 +150,11 @@ gemm_dma_kernel(GemmArgs g) {
       for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn)
-          acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[tm]),
-                                                                __builtin_bit_cast(bf16x8, bf[tn]), acc[tm][tn], 0, 0,
-                                                                0);
+          acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[cur][tm]),
+                                                                __builtin_bit_cast(bf16x8, bf[cur][tn]), acc[tm][tn], 0,
+                                                                0, 0);
       __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int t = 0; t < TM; ++t) af[t] = an[t];
-#pragma unroll
-      for (int t = 0; t < TN; ++t) bf[t] = bn[t];
-    }
+    });
   };
   if constexpr (TM * TN <= 4) {
     // Unrolled over the stages, so every LDS address is the precomputed offset plus a constant.

@@ -81,6 +81,61 @@ struct TileLoads {
   }
 };
 
+// TileLoads with a wave-uniform base address (the tile's first element at the current K step, a scalar pair) and a
+// 32-bit byte offset per lane and load that never changes: a K step advances one scalar instead of every lane's
+// pointer (the 64-bit vector additions would take issue slots from the matrix instructions). Rows past the end are
+// clamped in the offset, so edge tiles take this form too. Needs 255 rows of the leading dimension to fit 32 bits
+// of bytes, and the same number of loads in every wave.
+template <bool KM, int ROWS, int BK, int NW>
+struct TileLoadsOff {
+  static constexpr int TOTAL = ROWS * BK * 2 / 1024;
+  static constexpr int N = TOTAL / NW;
+  static_assert(TOTAL % NW == 0, "the same number of loads in every wave");
+  unsigned off[N];
+  const char* base;
+  long step;  // bytes between consecutive K steps
+
+  __device__ __forceinline__ void init(const unsigned short* __restrict__ p, long ld, int row0, int rows, int k0,
+                                       int wave, int lane) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int q = wave + NW * i;
+      if constexpr (!KM) {
+        constexpr int LPR = BK / 8;
+        const int r = q * (64 / LPR) + lane / LPR;
+        const int kc = (lane % LPR) ^ (BK == 32 ? (r >> 2) & 3 : (r >> 1) & 7);
+        int gr = row0 + r;
+        gr = gr < rows ? gr : rows - 1;
+        off[i] = static_cast<unsigned>(gr - row0) * static_cast<unsigned>(ld * 2) + kc * 16;
+      } else {
+        constexpr int CPR = ROWS / 8;
+        const int idx = q * 64 + lane;
+        const int kr = idx / CPR, slot = idx % CPR;
+        const int mc = slot ^ ((kr & 3) * 4);
+        int gm = mc * 8;
+        gm = row0 + gm + 8 <= rows ? gm : 0;
+        off[i] = static_cast<unsigned>(kr) * static_cast<unsigned>(ld * 2) + gm * 2;
+      }
+    }
+    const long first = KM ? static_cast<long>(k0) * ld + row0 : static_cast<long>(row0) * ld + k0;
+    const unsigned long long addr = reinterpret_cast<unsigned long long>(p) + static_cast<unsigned long long>(first) * 2;
+    // (tile coordinates come out of vector divisions: back to scalars)
+    const unsigned lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(addr));
+    const unsigned hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(addr >> 32));
+    base = reinterpret_cast<const char*>((static_cast<unsigned long long>(hi) << 32) | lo);
+    step = (KM ? BK * ld : BK) * 2;
+  }
+  __device__ __forceinline__ void issue(unsigned tile, int wave) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off[i]), "s"(base),
+                   "s"(tile + (wave + NW * i) * 1024)
+                   : "memory");
+    }
+    base += step;
+  }
+};
+
 // The same loads with one scalar base address per operand and a 32-bit byte offset per lane and
 // load, taken from the tile's first element: the offsets do not depend on the tile, so a
 // workgroup that walks several tiles only moves the scalar base (no per-lane address is ever
