@@ -218,14 +218,17 @@ __global__ __launch_bounds__(512, 4) void gemm_q8_kernel(Q8Args g) {
   if (feeds_b) widen(0, smem + Q_OFF_B16);
   __syncthreads();
 
-  u32x4 af[TM], bf[TN];
+  // Two sets of fragment registers that take turns (an even number of slabs per step: slab 0 always finds its
+  // fragments in set 0): no copies, no wait for the next slab's fragments before this slab's products are issued.
+  static_assert(KK % 2 == 0, "the fragment sets alternate by slab");
+  u32x4 af[2][TM], bf[2][TN];
   auto read_frags = [&](const char* a_stage, const char* b_buf, int kk, u32x4(&a)[TM], u32x4(&b)[TN]) {
 #pragma unroll
     for (int t = 0; t < TM; ++t) a[t] = frag_at<false, QBM>(a_stage + a_off[t][kk]);
 #pragma unroll
     for (int t = 0; t < TN; ++t) b[t] = frag_at<B_KM, QBN>(b_buf + b_off[t][kk]);
   };
-  read_frags(smem, smem, 0, af, bf);
+  read_frags(smem, smem, 0, af[0], bf[0]);
   // Step ks reads activation stage sa = ks % 3 and widened buffer sb = ks % 2.
   auto k_step = [&](int ks, int sa, int sb, int raw_slot_next, int raw_slot_fill) {
     const char* a_stage = smem + sa * Q_A_STAGE;
@@ -244,34 +247,25 @@ __global__ __launch_bounds__(512, 4) void gemm_q8_kernel(Q8Args g) {
       la.issue(lds0 + ((sa + 2) % 3) * Q_A_STAGE, wave);
       newer += 2;
     }
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-      u32x4 an[TM], bn[TN];
-#pragma unroll
-      for (int t = 0; t < TM; ++t) an[t] = af[t];
-#pragma unroll
-      for (int t = 0; t < TN; ++t) bn[t] = bf[t];
-      if (kk + 1 < KK) {
-        read_frags(a_stage, b_buf, kk + 1, an, bn);
+    static_for<0, KK>([&](auto kk_index) {
+      constexpr int kk = decltype(kk_index)::value, cur = kk % 2, nxt = cur ^ 1;
+      if constexpr (kk + 1 < KK) {
+        read_frags(a_stage, b_buf, kk + 1, af[nxt], bf[nxt]);
       } else {
         q8_wait_newer(newer);  // A(ks + 1) has landed (this wave's share, then everyone's)
         __syncthreads();
-        if (ks + 1 < steps) read_frags(a_next, b_next, 0, an, bn);
+        if (ks + 1 < steps) read_frags(a_next, b_next, 0, af[nxt], bf[nxt]);
       }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn)
-          acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[tm]),
-                                                                __builtin_bit_cast(bf16x8, bf[tn]), acc[tm][tn], 0, 0,
-                                                                0);
+          acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[cur][tm]),
+                                                                __builtin_bit_cast(bf16x8, bf[cur][tn]), acc[tm][tn], 0,
+                                                                0, 0);
       __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int t = 0; t < TM; ++t) af[t] = an[t];
-#pragma unroll
-      for (int t = 0; t < TN; ++t) bf[t] = bn[t];
-    }
+    });
   };
   // Unrolled over the six (stage, buffer) combinations so every LDS address is a precomputed
   // offset plus a constant.
