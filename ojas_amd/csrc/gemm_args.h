@@ -173,7 +173,12 @@ __device__ __forceinline__ bool gemm_epilogue_block(const GemmArgs& g, const flo
                                                     int gcol0, int lane) {
   constexpr int ITERS = 32 * PPR / 64;
   unsigned short* cbase = static_cast<unsigned short*>(g.c);
-  bool bad = false;
+  // Non-finite values are found in the packed words that get stored: a bf16 is infinite or NaN
+  // when its eight exponent bits are all set, and adding one at the exponent's lowest bit then
+  // carries into the half's top bit. (GELU of a finite value is finite, so the forward tests the
+  // pre-activation words only.)
+  unsigned int flags = 0;
+  auto note = [&](unsigned int w) { flags |= (w & 0x7F807F80u) + 0x00800080u; };
   long off[ITERS];
   uint2 aux[ITERS];
 #pragma unroll
@@ -198,10 +203,9 @@ __device__ __forceinline__ bool gemm_epilogue_block(const GemmArgs& g, const flo
                           __uint_as_float(w23 & 0xffff0000u)};
       float a[4];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        a[e] = TANH ? dev_gelu_tanh_fast(u[e]) : dev_gelu_erf_fast(u[e]);
-        bad |= !(dev_finite(x[e]) && dev_finite(a[e]));
-      }
+      for (int e = 0; e < 4; ++e) a[e] = TANH ? dev_gelu_tanh_fast(u[e]) : dev_gelu_erf_fast(u[e]);
+      note(w01);
+      note(w23);
       *reinterpret_cast<uint2*>(cbase + off[it]) = make_uint2(w01, w23);
       *reinterpret_cast<uint2*>(g.aux_out + off[it]) = make_uint2(pack(a[0], a[1]), pack(a[2], a[3]));
     } else {
@@ -211,12 +215,14 @@ __device__ __forceinline__ bool gemm_epilogue_block(const GemmArgs& g, const flo
       for (int e = 0; e < 4; ++e) {
         if constexpr (EPI == OMX_EPI_AXPBY) x[e] = gemm_axpby(g, u[e], x[e]);
         else x[e] = dev_round_bf16(x[e]) * (TANH ? dev_gelu_tanh_grad_fast(u[e]) : dev_gelu_erf_grad_fast(u[e]));
-        bad |= !dev_finite(x[e]);
       }
-      *reinterpret_cast<uint2*>(cbase + off[it]) = make_uint2(pack(x[0], x[1]), pack(x[2], x[3]));
+      const unsigned int w01 = pack(x[0], x[1]), w23 = pack(x[2], x[3]);
+      note(w01);
+      note(w23);
+      *reinterpret_cast<uint2*>(cbase + off[it]) = make_uint2(w01, w23);
     }
   }
-  return bad;
+  return (flags & 0x80008000u) != 0;
 }
 
 // The plain store of a 32-row block that lies wholly inside the output, in the same straight-line

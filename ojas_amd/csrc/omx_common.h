@@ -360,27 +360,30 @@ __device__ __forceinline__ float dev_gelu_tanh_grad(float x) {
 // (1 ulp) and a few fmas. erf: Abramowitz & Stegun 7.1.26, |error| <= 1.5e-7, evaluated as erfc so
 // the negative tail x * Phi(x) has no cancellation; exp(-z^2) doubles as the density in the
 // derivative.
-__device__ __forceinline__ void dev_normal_cdf_pdf_fast(float x, float* cdf, float* pdf) {
-  const float z = fabsf(x) * 0.70710678118654752f;
-  const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, z, 1.0f));
-  const float e = __builtin_amdgcn_exp2f(x * x * -0.72134752044448170f);  // exp(-x^2 / 2)
-  float poly = fmaf(t, 1.061405429f, -1.453152027f);
-  poly = fmaf(t, poly, 1.421413741f);
-  poly = fmaf(t, poly, -0.284496736f);
-  poly = fmaf(t, poly, 0.254829592f);
-  const float tail = 0.5f * (poly * t) * e;  // Phi(-|x|)
-  *cdf = x >= 0.0f ? 1.0f - tail : tail;
-  *pdf = 0.3989422804014327f * e;
+// tail = Phi(-|x|) and e = exp(-x^2 / 2). With w = |x| sqrt(log2(e) / 2): e = exp2(-w^2), and the
+// series' argument |x| / sqrt 2 is w / sqrt(log2 e), so its constant folds into the fma that feeds
+// the reciprocal; the 1/2 of erfc / 2 is folded into the coefficients.
+__device__ __forceinline__ void dev_normal_tail_fast(float x, float* tail, float* e) {
+  const float w = fabsf(x) * 0.84932180028801904f;
+  const float t = __builtin_amdgcn_rcpf(fmaf(0.27273748087922250f, w, 1.0f));
+  *e = __builtin_amdgcn_exp2f(-(w * w));
+  float poly = fmaf(t, 0.5307027145f, -0.7265760135f);
+  poly = fmaf(t, poly, 0.7107068705f);
+  poly = fmaf(t, poly, -0.142248368f);
+  poly = fmaf(t, poly, 0.127414796f);
+  *tail = (poly * t) * *e;
 }
+// x Phi(x) = max(x, 0) - |x| Phi(-|x|): no branch on the sign and no 1 - tail.
 __device__ __forceinline__ float dev_gelu_erf_fast(float x) {
-  float cdf, pdf;
-  dev_normal_cdf_pdf_fast(x, &cdf, &pdf);
-  return x * cdf;
+  float tail, e;
+  dev_normal_tail_fast(x, &tail, &e);
+  return fmaf(-fabsf(x), tail, fmaxf(x, 0.0f));
 }
 __device__ __forceinline__ float dev_gelu_erf_grad_fast(float x) {
-  float cdf, pdf;
-  dev_normal_cdf_pdf_fast(x, &cdf, &pdf);
-  return fmaf(x, pdf, cdf);
+  float tail, e;
+  dev_normal_tail_fast(x, &tail, &e);
+  const float cdf = x >= 0.0f ? 1.0f - tail : tail;
+  return fmaf(x, 0.3989422804014327f * e, cdf);
 }
 __device__ __forceinline__ void dev_sigmoid_pair_fast(float u, float* s, float* slope) {
   const float e = __builtin_amdgcn_exp2f(fabsf(u) * -1.4426950408889634f);
@@ -388,18 +391,22 @@ __device__ __forceinline__ void dev_sigmoid_pair_fast(float u, float* s, float* 
   *s = u >= 0.0f ? r : e * r;
   *slope = e * r * r;
 }
+// 2 sqrt(2/pi) (x + 0.044715 x^3) as x (c0 + c1 x^2).
+__device__ __forceinline__ float dev_gelu_tanh_arg_fast(float x) {
+  return x * fmaf(0.07135481627260025f, x * x, 1.5957691216057308f);
+}
 __device__ __forceinline__ float dev_gelu_tanh_fast(float x) {
-  const float u = 2.0f * 0.7978845608028654f * (x + 0.044715f * x * x * x);
+  const float u = dev_gelu_tanh_arg_fast(x);
   float s, slope;
   dev_sigmoid_pair_fast(u, &s, &slope);
   return x * s;
 }
 __device__ __forceinline__ float dev_gelu_tanh_grad_fast(float x) {
-  const float u = 2.0f * 0.7978845608028654f * (x + 0.044715f * x * x * x);
+  const float u = dev_gelu_tanh_arg_fast(x);
   float s, slope;
   dev_sigmoid_pair_fast(u, &s, &slope);
-  const float du = 2.0f * 0.7978845608028654f * (1.0f + 3.0f * 0.044715f * x * x);
-  return s + x * slope * du;
+  const float du = fmaf(0.21406444881780074f, x * x, 1.5957691216057308f);
+  return fmaf(x * slope, du, s);
 }
 // GELU of a value whose storage type is T: exact for f32, the fast forms for bf16.
 template <typename T, bool TANH>
