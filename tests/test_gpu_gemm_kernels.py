@@ -25,7 +25,8 @@ def be():
 
 
 SHAPES = [(256, 64, 256), (300, 128, 520), (64, 192, 96), (513, 256, 257), (1024, 768, 768), (264, 1024, 136),
-          (4160, 136, 264)]  # the last: a weight gradient over 4160 rows, split along K
+          (4160, 136, 264),  # a weight gradient over 4160 rows, split along K
+          (520, 256, 400), (256, 1280, 192), (768, 384, 576)]  # one-wave tiles: ragged both ways, one exact 256 x 192 tile, six steps
 
 
 @pytest.mark.parametrize("mode", [0, 1, 3, 4, 9, 10])
@@ -212,7 +213,7 @@ def test_unknown_option_is_refused(be):
 
 @pytest.mark.parametrize("mode", [0, 1, 3, 4, 9, 10])
 @pytest.mark.parametrize("layers", [3, 4])  # 4: a tile count divisible by 8, which takes the XCD-ordered mapping
-@pytest.mark.parametrize("rows,kin,nout", [(1088, 136, 264), (2048, 768, 256)])
+@pytest.mark.parametrize("rows,kin,nout", [(1088, 136, 264), (2048, 768, 256), (2048, 200, 328)])
 def test_strided_batch_of_weight_gradients(be, mode, rows, kin, nout, layers):
     """`omx_gemm_strided_batch` as the step driver uses it: gw[l] = gy[l]^T x[l] for three stacked
     layers in one launch, outputs at a padded stride; each equals the oracle's `linear_backward`
