@@ -25,7 +25,6 @@ struct GemmArgs {
   // product y - 1's. batches == 1 for a single product.
   int batches;
   long batch_a, batch_b, batch_c;
-  int band_rows;  // persistent kernel: tile rows per band (divides tiles_m)
 };
 
 // The arguments of product `product` of a strided batch.
