@@ -118,14 +118,15 @@ __global__ __launch_bounds__(512, 4) void gemm_q8_kernel(Q8Args g) {
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
   const int steps = g.K / QBK;
-  TileLoads<false, QBM, QBK, QNW> la;
+  TileLoadsOff<false, QBM, QBK, QNW> la;  // a scalar base that advances by the step and fixed lane offsets
   la.init(g.a, g.lda, m0, g.M, 0, wave, lane);
   const unsigned lds0 = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(reinterpret_cast<uintptr_t>(smem)));
 
-  // This lane's 16 codes of a step, its scale, and where their 16 bf16 go in the widened tile.
-  const signed char* code_src;
-  const float* scale_src;
-  long code_step, scale_step;
+  // This lane's 16 codes of a step, its scale, and where their 16 bf16 go in the widened tile. The
+  // loads take a scalar base, which advances by the step, and a lane offset in bytes that never
+  // changes (the host keeps the weight under 2 GiB), so no vector instruction forms an address in the K loop.
+  unsigned code_off, scale_off;
+  long code_step, scale_step;  // bytes
   int w_off0, w_off1;  // byte offsets of the two 16-byte chunks inside a widened buffer
   const long groups = g.kin / 32;
   if constexpr (!B_KM) {
@@ -133,15 +134,15 @@ __global__ __launch_bounds__(512, 4) void gemm_q8_kernel(Q8Args g) {
     int gr = n0 + r;
     gr = gr < g.N ? gr : g.N - 1;
     if (g.packed) {
-      code_src = g.codes + q8_packed_code_offset(gr, 0, g.kin) + h * 16;
-      scale_src = g.scales + q8_packed_scale_index(gr, 0, g.kin);
+      code_off = static_cast<unsigned>(q8_packed_code_offset(gr, 0, g.kin) + h * 16);
+      scale_off = static_cast<unsigned>(q8_packed_scale_index(gr, 0, g.kin) * 4);
       code_step = 256;
-      scale_step = 8;
+      scale_step = 8 * 4;
     } else {
-      code_src = g.codes + static_cast<long>(gr) * g.kin + h * 16;
-      scale_src = g.scales + static_cast<long>(gr) * groups;
+      code_off = static_cast<unsigned>(static_cast<long>(gr) * g.kin + h * 16);
+      scale_off = static_cast<unsigned>(static_cast<long>(gr) * groups * 4);
       code_step = QBK;
-      scale_step = 1;
+      scale_step = 4;
     }
     const int x = (r >> 2) & 3;
     w_off0 = r * 64 + (((2 * h) ^ x) << 4);
@@ -151,29 +152,31 @@ __global__ __launch_bounds__(512, 4) void gemm_q8_kernel(Q8Args g) {
     int gc = n0 + j * 16;
     gc = gc + 16 <= g.N ? gc : 0;
     if (g.packed) {
-      code_src = g.codes + q8_packed_code_offset(kr, gc / 32, g.kin) + (j & 1) * 16;
-      scale_src = g.scales + q8_packed_scale_index(kr, gc / 32, g.kin);
+      code_off = static_cast<unsigned>(q8_packed_code_offset(kr, gc / 32, g.kin) + (j & 1) * 16);
+      scale_off = static_cast<unsigned>(q8_packed_scale_index(kr, gc / 32, g.kin) * 4);
     } else {
-      code_src = g.codes + static_cast<long>(kr) * g.kin + gc;
-      scale_src = g.scales + static_cast<long>(kr) * groups + gc / 32;
+      code_off = static_cast<unsigned>(static_cast<long>(kr) * g.kin + gc);
+      scale_off = static_cast<unsigned>((static_cast<long>(kr) * groups + gc / 32) * 4);
     }
     code_step = QBK * g.kin;
-    scale_step = QBK * groups;
+    scale_step = QBK * groups * 4;
     const int x = (kr & 3) * 4;
     w_off0 = kr * 256 + (((2 * j) ^ x) << 4);
     w_off1 = kr * 256 + (((2 * j + 1) ^ x) << 4);
   }
   const unsigned raw_lds = lds0 + Q_OFF_RAW + wave * 1024;  // + slot * 4096
   const unsigned scl_lds = lds0 + Q_OFF_SCL + wave * 256;   // + slot * 1024
+  const char* code_base = reinterpret_cast<const char*>(g.codes);
+  const char* scale_base = reinterpret_cast<const char*>(g.scales);
   auto issue_raw = [&](int slot) {
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(code_src),
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(code_off), "s"(code_base),
                  "s"(raw_lds + slot * 4096)
                  : "memory");
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(scale_src),
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(scale_off), "s"(scale_base),
                  "s"(scl_lds + slot * 1024)
                  : "memory");
-    code_src += code_step;
-    scale_src += scale_step;
+    code_base += code_step;
+    scale_base += scale_step;
   };
   // Reads this lane's own 16 codes and scale back from slot `slot` and writes 16 bf16 into `dst`.
   auto widen = [&](int slot, char* dst) {
@@ -420,6 +423,9 @@ int32_t check_q8(omx_ctx* ctx, const char* op, const void* act, const void* code
     return omx_fail(ctx, OMX_SHAPE, "%s: the blocked layout needs k_in %% 128 == 0 and n_out %% 8 == 0", op);
   if (rows > 0x7fffffffull || kin > 0x7fffffffull || nout > 0x7fffffffull)
     return omx_fail(ctx, OMX_OUT_OF_RANGE, "%s: axis does not fit in i32", op);
+  // The kernel's loads address a lane's bytes with 32 bits beside a 64-bit base.
+  if (kin >= (1ull << 22) || nout * kin >= (1ull << 31))
+    return omx_fail(ctx, OMX_OUT_OF_RANGE, "%s: a weight of 2 GiB or more, or k_in of 4 Mi or more", op);
   if (!aligned16(act) || !aligned16(codes) || !aligned16(out) || (add && !aligned16(add)) ||
       (reinterpret_cast<uintptr_t>(scales) & 3u))
     return omx_fail(ctx, OMX_SHAPE, "%s: operands must be 16-byte aligned", op);
