@@ -42,7 +42,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor figure
 # The algorithmic figure of the gpt124m step (every operand read once, every output written once)
 # is 2.326e10 bytes per step: 2.258e8 per product, 2.237e8 per launch (its 103 products run as 104
 # launches: the head's weight gradient is cut by rows into two).
-GEMM_HBM_BYTES_PER_LAUNCH = {"gpt124m": 3.42e8, "gpt124m-muon": 2.77e8, "lora1b": 4.07e8, "nanolab124m": 2.68e8}
+GEMM_HBM_BYTES_PER_LAUNCH = {"gpt124m": 3.42e8, "gpt124m-muon": 2.75e8, "lora1b": 4.13e8, "nanolab124m": 2.68e8}
 
 
 # Kernel classes of omx_profile_kernels beyond the GEMM products: (bit, key, kernels, roofline).
