@@ -394,7 +394,7 @@ def lora_step(args) -> int:
     losses = [tr.step(adamw, 1.0)[0] for _ in range(args.warmup)]
     be.sync()
     lib = be._lib
-    timed_every = 4
+    timed_every = max(1, args.timed_every)
     step_ms = []
     t0 = time.perf_counter()
     for i in range(args.steps):
@@ -535,7 +535,7 @@ def nanolab_step(args) -> int:
     losses = [tr.run_resident(1.0).loss for _ in range(args.warmup)]
     be.sync()
     lib = be._lib
-    timed_every = 4
+    timed_every = max(1, args.timed_every)
     step_ms = []
     t0 = time.perf_counter()
     for i in range(args.steps):
@@ -648,6 +648,8 @@ def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--timed-every", type=int, default=10,
+                    help="the kernels of every N-th timed step carry events for the roofline figures")
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--config", default="gpt124m", choices=["gpt124m", "tiny", "lora1b", "nanolab124m"])
@@ -698,12 +700,12 @@ def main() -> int:
         losses.append(one_step())
     be.sync()
     lib = be._lib
-    # The kernels of every fourth timed step carry HIP events on their dispatches (begin and end
-    # timestamps of the kernels themselves): the GEMM products and the classes of KERNEL_CLASSES.
-    # All steps would cost about a millisecond per step on the number being measured (the timed
-    # launch path is slower: 103 products and some 80 other launches per step); a quarter of them
-    # is 515 timed products in the default run.
-    timed_every = 4
+    # The kernels of every tenth timed step (--timed-every) carry HIP events on their dispatches
+    # (begin and end timestamps of the kernels themselves): the GEMM products and the classes of
+    # KERNEL_CLASSES. All steps would cost about a millisecond per step on the number being measured
+    # (the timed launch path is slower: 104 GEMM launches and some 80 others per step); two steps of
+    # the default run's twenty are 208 timed GEMM launches.
+    timed_every = max(1, args.timed_every)
     step_ms = []
     t0 = time.perf_counter()
     for i in range(args.steps):
