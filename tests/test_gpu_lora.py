@@ -216,7 +216,7 @@ def test_rope_in_place_and_swiglu(be):
 
 
 def test_linear_i8_group_refusals(be):
-    from ojas_amd.backend import BF16, DTYPE, SHAPE, UNSUPPORTED, OjasError
+    from ojas_amd.backend import BF16, DTYPE, OUT_OF_RANGE, SHAPE, UNSUPPORTED, OjasError
 
     x = be.upload(np.zeros((8, 48), np.float32), BF16)
     codes = be.upload(np.zeros((32, 48), np.int8))
@@ -236,6 +236,14 @@ def test_linear_i8_group_refusals(be):
                                                       C.c_uint64(32), C.c_int32(0), None, None, be._p(x), C.c_int32(1), C.c_uint64(8), C.c_uint64(64),
                                                       C.c_uint64(32)))
     assert e.value.code == DTYPE
+    # The kernel addresses a lane's bytes with 32 bits beside a 64-bit base: weights of 2 GiB or more and
+    # k_in of 4 Mi or more are refused before anything is launched.
+    for kin, nout in ((1 << 22, 32), (1 << 16, 1 << 15)):
+        with pytest.raises(OjasError) as e:
+            be._check(be._lib.omx_linear_i8_group_forward(be._ctx, be._p(x), C.c_int32(1), be._p(codes), be._p(scales),
+                                                          C.c_uint64(32), C.c_int32(0), None, None, be._p(x), C.c_int32(1), C.c_uint64(8),
+                                                          C.c_uint64(kin), C.c_uint64(nout)))
+        assert e.value.code == OUT_OF_RANGE, (kin, nout)
 
 
 # ---- the step: reduced shapes against the oracle ----
