@@ -171,7 +171,9 @@ int32_t omx_gemm_pitched_strided_batch(omx_ctx* ctx, const void* a, uint64_t a_r
  * is a multiple of 16. block_cols > 0: column c reads h at
  * off = (c / block_cols) * rank, so one h [rows, 3 rank] serves a fused q / k / v projection
  * whose three up matrices are stacked in w (block_cols = d; a multiple of 128). For the forward,
- * h = x A^T and w = scale * B; for the input gradient, h = gy (scale * B) and w = A^T. */
+ * h = x A^T and w = scale * B; for the input gradient, h = gy (scale * B) and w = A^T.
+ * A weight of 2 GiB or more (n_out * k_in >= 2^31) or k_in >= 2^22 is refused with
+ * OMX_OUT_OF_RANGE: the kernel addresses a lane's bytes with 32 bits beside a 64-bit base. */
 enum { OMX_I8_ROW_MAJOR = 0, OMX_I8_BLOCKED = 1 };
 typedef struct {
   const void* h;
